@@ -1,0 +1,195 @@
+/*
+ * hipnx.h -- C ABI of libhipnx, the MI355X (gfx950) device library underneath HipNx.Backend.
+ *
+ * This is the drop-in boundary for the eager tensor path of Nx: every entry point is what a NIF
+ * for one `Nx.Backend` callback (reference: nx/lib/nx/backend.ex:46-144) binds.  The structural
+ * model is the reference's Torchx NIF (torchx/c_src/torchx.cpp, one native function per
+ * callback) with LibTorch replaced by hand-written HIP kernels.
+ *
+ * Conventions
+ *  - Plain C: opaque handles, pointers and sizes only.
+ *  - Every function returns an int status (HIPNX_OK = 0).  On failure a message is kept per
+ *    calling thread and can be fetched with hipnx_last_error().  Nothing aborts the process.
+ *  - A context owns one device and one HIP stream.  Compute entry points only enqueue work on
+ *    that stream and return; hipnx_d2h() and hipnx_sync() wait.  Contexts may be used from any
+ *    thread (NIFs run on arbitrary dirty-scheduler threads): each entry selects the device and
+ *    serialises enqueueing with a short mutex.
+ *  - Device buffers are flat, untyped byte ranges.  Shape, element type and strides always come
+ *    from the caller (the `Nx.Tensor` struct), never from the handle -- `Nx.reshape`, `rename`,
+ *    `vectorize` rewrite them without calling the backend (nx/lib/nx.ex:5354-5405, 3058-3060).
+ *  - Inputs are immutable; every op writes a buffer the caller allocated for `out`.
+ *  - Before any launch the host side checks that every operand buffer is live and large enough
+ *    for the shape it is claimed to hold.
+ */
+#ifndef HIPNX_H
+#define HIPNX_H
+#include <stddef.h>
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct hipnx_ctx hipnx_ctx;
+typedef struct hipnx_buf hipnx_buf;
+
+/* status codes */
+enum {
+  HIPNX_OK = 0,
+  HIPNX_ALREADY_FREED = 1, /* hipnx_buf_free on a freed buffer (-> :already_deallocated) */
+  HIPNX_EINVAL = 2,        /* malformed call: bad code, rank, size mismatch (-> ArgumentError) */
+  HIPNX_EFREED = 3,        /* an operand buffer was deallocated before use */
+  HIPNX_ENOMEM = 4,        /* device allocation failed */
+  HIPNX_EHIP = 5,          /* a HIP runtime call failed */
+  HIPNX_EINDEX = 6,        /* gather/take index out of bounds (-> ArgumentError, reference text) */
+  HIPNX_EUNSUPPORTED = 7   /* type combination not implemented natively */
+};
+
+/* element types, Nx.Type tuples {:u,8} .. {:f,64} (nx/lib/nx/type.ex:27-48) */
+enum {
+  HIPNX_U8 = 0, HIPNX_U16 = 1, HIPNX_U32 = 2, HIPNX_U64 = 3,
+  HIPNX_S8 = 4, HIPNX_S16 = 5, HIPNX_S32 = 6, HIPNX_S64 = 7,
+  HIPNX_F16 = 8, HIPNX_BF16 = 9, HIPNX_F32 = 10, HIPNX_F64 = 11, HIPNX_NTYPES = 12
+};
+
+/* element-wise binary callbacks, in the order of nx/lib/nx/binary_backend.ex:649-653 */
+enum {
+  HIPNX_ADD = 0, HIPNX_SUBTRACT, HIPNX_MULTIPLY, HIPNX_DIVIDE, HIPNX_POW, HIPNX_REMAINDER,
+  HIPNX_ATAN2, HIPNX_MIN, HIPNX_MAX, HIPNX_QUOTIENT, HIPNX_BITWISE_AND, HIPNX_BITWISE_OR,
+  HIPNX_BITWISE_XOR, HIPNX_LEFT_SHIFT, HIPNX_RIGHT_SHIFT, HIPNX_EQUAL, HIPNX_NOT_EQUAL,
+  HIPNX_GREATER, HIPNX_LESS, HIPNX_GREATER_EQUAL, HIPNX_LESS_EQUAL, HIPNX_LOGICAL_AND,
+  HIPNX_LOGICAL_OR, HIPNX_LOGICAL_XOR, HIPNX_NBINARY
+};
+
+/* element-wise unary callbacks: the 23 math functions of nx/lib/nx/shared.ex:311-376 in that
+ * order, then nx/lib/nx/backend.ex:125-132 */
+enum {
+  HIPNX_EXP = 0, HIPNX_EXPM1, HIPNX_LOG, HIPNX_LOG1P, HIPNX_SIGMOID, HIPNX_COS, HIPNX_SIN,
+  HIPNX_TAN, HIPNX_COSH, HIPNX_SINH, HIPNX_TANH, HIPNX_ACOS, HIPNX_ASIN, HIPNX_ATAN,
+  HIPNX_ACOSH, HIPNX_ASINH, HIPNX_ATANH, HIPNX_SQRT, HIPNX_RSQRT, HIPNX_CBRT, HIPNX_ERF,
+  HIPNX_ERFC, HIPNX_ERF_INV, HIPNX_ABS, HIPNX_BITWISE_NOT, HIPNX_CEIL, HIPNX_FLOOR,
+  HIPNX_NEGATE, HIPNX_ROUND, HIPNX_SIGN, HIPNX_CLZ, HIPNX_POPCOUNT, HIPNX_IS_NAN,
+  HIPNX_IS_INFINITY, HIPNX_NUNARY
+};
+
+enum { HIPNX_RED_SUM = 0, HIPNX_RED_MAX = 1, HIPNX_RED_MIN = 2, HIPNX_RED_PRODUCT = 3 };
+enum { HIPNX_ARGMAX = 0, HIPNX_ARGMIN = 1 };
+enum { HIPNX_TIE_LOW = 0, HIPNX_TIE_HIGH = 1 };
+
+/* operand layouts of hipnx_dot: which of the two non-batch axes is contiguous */
+enum {
+  HIPNX_K_INNER = 0, /* [batch, M or N, K]: the contracted axis is the last (unit stride) */
+  HIPNX_K_OUTER = 1  /* [batch, K, M or N]: the contracted axis comes first */
+};
+
+/* out-of-bounds index policy of hipnx_gather */
+enum {
+  HIPNX_OOB_RAISE = 0, /* Nx.BinaryBackend: raise (binary_backend.ex:1949-1952); waits for the kernel */
+  HIPNX_OOB_CLAMP = 1  /* EXLA / Torchx behaviour: clamp into range; stays asynchronous */
+};
+
+/* ---- context, errors ---------------------------------------------------------------------
+ * replaces: backend `init/1` + per-backend client/device selection
+ * (nx/lib/nx/backend.ex:46; torchx/lib/torchx/backend.ex:49-52; exla/lib/exla/client.ex:20-55) */
+int hipnx_device_count(int *count);
+int hipnx_ctx_create(int device, hipnx_ctx **out);
+int hipnx_ctx_destroy(hipnx_ctx *ctx);
+int hipnx_sync(hipnx_ctx *ctx);
+/* copies the calling thread's last error message (NUL-terminated, truncated to cap) */
+int hipnx_last_error(char *dst, size_t cap);
+/* live / peak / pooled device bytes of this context (cf. EXLA client memory statistics,
+ * exla/c_src/exla/exla_client.cc:597-631) */
+int hipnx_mem_stats(hipnx_ctx *ctx, uint64_t *live, uint64_t *peak, uint64_t *pooled);
+/* returns pooled (cached, unused) device memory to the driver */
+int hipnx_trim(hipnx_ctx *ctx);
+
+/* HIP-event stopwatch on the context's stream (device-side timing for benchmarks) */
+int hipnx_timer_start(hipnx_ctx *ctx);
+int hipnx_timer_stop(hipnx_ctx *ctx, float *elapsed_ms);
+
+/* ---- buffers -------------------------------------------------------------------------------
+ * replaces: from_binary / to_binary / backend_copy / backend_transfer / backend_deallocate
+ * (nx/lib/nx/backend.ex:50-57; torchx/c_src/torchx.cpp:100-185 from_blob, to_blob,
+ * delete_tensor; exla/c_src/exla/exla.cc:439-475) */
+int hipnx_buf_alloc(hipnx_ctx *ctx, size_t bytes, hipnx_buf **out);
+/* explicit deallocation; idempotent: HIPNX_OK the first time, HIPNX_ALREADY_FREED afterwards.
+ * The handle itself stays valid until hipnx_buf_destroy (the BEAM resource destructor). */
+int hipnx_buf_free(hipnx_buf *buf);
+/* releases the handle (and the device memory if still live) */
+int hipnx_buf_destroy(hipnx_buf *buf);
+int hipnx_buf_size(const hipnx_buf *buf, size_t *bytes);
+/* raw device pointer, for interop and profiling harnesses; NULL once freed */
+void *hipnx_buf_device_ptr(const hipnx_buf *buf);
+int hipnx_h2d(hipnx_ctx *ctx, hipnx_buf *dst, size_t dst_offset, const void *src, size_t bytes);
+/* waits for all work enqueued so far, then copies */
+int hipnx_d2h(hipnx_ctx *ctx, const hipnx_buf *src, size_t src_offset, void *dst, size_t bytes);
+int hipnx_d2d(hipnx_ctx *ctx, hipnx_buf *dst, size_t dst_offset, const hipnx_buf *src,
+              size_t src_offset, size_t bytes);
+/* replaces: constant/3 (nx/lib/nx/backend.ex:49): n copies of one element (elem_bytes <= 8) */
+int hipnx_fill(hipnx_ctx *ctx, hipnx_buf *dst, int elem_bytes, const void *elem, int64_t n);
+
+/* ---- element-wise --------------------------------------------------------------------------
+ * replaces: the 24 binary callbacks (nx/lib/nx/backend.ex:115-123; oracle
+ * nx/lib/nx/binary_backend.ex:649-823; torchx/c_src/torchx.cpp:737-769).
+ * out[i] = op(l[bcast i], r[bcast i]) over the row-major index space `out_dims[rank]`;
+ * strides are in elements, 0 marks a broadcast axis (numpy-style, nx/lib/nx/shape.ex:316-376). */
+int hipnx_binary(hipnx_ctx *ctx, int op, int l_dt, int r_dt, int out_dt, int rank,
+                 const int64_t *out_dims, const int64_t *l_strides, const int64_t *r_strides,
+                 const hipnx_buf *l, const hipnx_buf *r, hipnx_buf *out);
+
+/* replaces: the unary callbacks (nx/lib/nx/backend.ex:125-132; oracle binary_backend.ex:827-1005;
+ * torchx/c_src/torchx.cpp:777-828) */
+int hipnx_unary(hipnx_ctx *ctx, int op, int in_dt, int out_dt, int64_t n, const hipnx_buf *in,
+                hipnx_buf *out);
+
+/* replaces: as_type/2 (nx/lib/nx/backend.ex:68; oracle binary_backend.ex:2031-2076).
+ * float->bf16 truncates, float->int truncates toward zero then wraps, NaN->0, +-Inf->max/min. */
+int hipnx_as_type(hipnx_ctx *ctx, int in_dt, int out_dt, int64_t n, const hipnx_buf *in,
+                  hipnx_buf *out);
+
+/* ---- reductions ----------------------------------------------------------------------------
+ * replaces: sum / product / reduce_max / reduce_min (nx/lib/nx/backend.ex:89-92; oracle
+ * binary_backend.ex:1315-1375).  The input is viewed as [outer, red, inner] (the caller
+ * collapses axes, transposing first when the reduced axes are not adjacent); out is
+ * [outer, inner]. */
+int hipnx_reduce(hipnx_ctx *ctx, int op, int in_dt, int out_dt, int64_t outer, int64_t red,
+                 int64_t inner, const hipnx_buf *in, hipnx_buf *out);
+
+/* replaces: argmax / argmin (nx/lib/nx/backend.ex:93-94; oracle binary_backend.ex:1393-1431).
+ * Same view.  tie LOW = first index of the extreme, HIGH = last; any NaN wins and the last
+ * NaN's index is returned.  out_dt is an integer type. */
+int hipnx_argreduce(hipnx_ctx *ctx, int op, int tie, int in_dt, int out_dt, int64_t outer,
+                    int64_t red, int64_t inner, const hipnx_buf *in, hipnx_buf *out);
+
+/* ---- contraction ---------------------------------------------------------------------------
+ * replaces: dot/7 (nx/lib/nx/backend.ex:77; oracle binary_backend.ex:476-599, 2362-2385;
+ * torchx/c_src/torchx.cpp:844-890 tensordot).
+ * out[b, m, n] = sum_k l[b, m, k] * r[b, n, k]; l is [batch, M, K] (HIPNX_K_INNER) or
+ * [batch, K, M] (HIPNX_K_OUTER), r is [batch, N, K] or [batch, K, N]; out is [batch, M, N] in
+ * out_dt (f32 accumulation for f16/bf16/f32 operands, exact s32 for s8, then one encode). */
+int hipnx_dot(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batch, int64_t M, int64_t N,
+              int64_t K, int l_layout, int r_layout, const hipnx_buf *l, const hipnx_buf *r,
+              hipnx_buf *out);
+
+/* ---- data movement -------------------------------------------------------------------------
+ * replaces: transpose/3 (nx/lib/nx/backend.ex:74; oracle binary_backend.ex:280-319) */
+int hipnx_transpose(hipnx_ctx *ctx, int elem_bytes, int rank, const int64_t *in_dims,
+                    const int *perm, const hipnx_buf *in, hipnx_buf *out);
+
+/* replaces: broadcast/4 (nx/lib/nx/backend.ex:75; oracle binary_backend.ex:215-276);
+ * in_strides in elements per output axis, 0 = broadcast */
+int hipnx_broadcast(hipnx_ctx *ctx, int elem_bytes, int rank, const int64_t *out_dims,
+                    const int64_t *in_strides, const hipnx_buf *in, hipnx_buf *out);
+
+/* replaces: gather/4 and block(%Nx.Block.Take{}) (nx/lib/nx/backend.ex:81,144; oracle
+ * binary_backend.ex:1902-1959; nx/lib/nx.ex:14807-14819).  The tensor `t_dims[rank]` has its
+ * indexed axes leading; each of the n_tuples index tuples (idx is [n_tuples, depth], integer
+ * type idx_dt) addresses the first `depth` axes and the trailing slice is copied.  `take` along
+ * axis 0 is depth = 1. */
+int hipnx_gather(hipnx_ctx *ctx, int elem_bytes, int rank, const int64_t *t_dims, int idx_dt,
+                 int64_t n_tuples, int depth, int oob_policy, const hipnx_buf *t,
+                 const hipnx_buf *idx, hipnx_buf *out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

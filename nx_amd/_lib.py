@@ -1,0 +1,100 @@
+"""ctypes binding of libhipnx.so -- the same C ABI the Elixir NIF shim binds (include/hipnx.h).
+
+There is no fallback: if the shared library is missing the import of this module fails, and if
+no GPU is present every compute entry point fails with HipNxError.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.environ.get("HIPNX_LIB", os.path.join(_HERE, "lib", "libhipnx.so"))
+
+# status codes of include/hipnx.h
+OK, ALREADY_FREED, EINVAL, EFREED, ENOMEM, EHIP, EINDEX, EUNSUPPORTED = range(8)
+
+
+class HipNxError(RuntimeError):
+    """A failed libhipnx call; `.status` is the HIPNX_E* code."""
+
+    def __init__(self, status: int, message: str):
+        super().__init__(f"HipNx: {message}")
+        self.status = status
+
+
+class HipNxArgumentError(HipNxError, ValueError):
+    """Status codes the Elixir side maps to ArgumentError (EINVAL, EINDEX)."""
+
+
+if not os.path.exists(LIB_PATH):
+    raise ImportError(
+        f"libhipnx.so not found at {LIB_PATH}: build it first "
+        "(python -c 'import __graft_entry__ as g; g.build()' or make -C nx_amd/csrc)")
+
+lib = C.CDLL(LIB_PATH)
+
+_ctx_p, _buf_p = C.c_void_p, C.c_void_p
+_i64p, _intp = C.POINTER(C.c_int64), C.POINTER(C.c_int)
+
+# name -> argtypes, in the order of include/hipnx.h; every function returns int except
+# hipnx_buf_device_ptr
+PROTOTYPES = {
+    "hipnx_device_count": [_intp],
+    "hipnx_ctx_create": [C.c_int, C.POINTER(_ctx_p)],
+    "hipnx_ctx_destroy": [_ctx_p],
+    "hipnx_sync": [_ctx_p],
+    "hipnx_last_error": [C.c_char_p, C.c_size_t],
+    "hipnx_mem_stats": [_ctx_p, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)],
+    "hipnx_trim": [_ctx_p],
+    "hipnx_timer_start": [_ctx_p],
+    "hipnx_timer_stop": [_ctx_p, C.POINTER(C.c_float)],
+    "hipnx_buf_alloc": [_ctx_p, C.c_size_t, C.POINTER(_buf_p)],
+    "hipnx_buf_free": [_buf_p],
+    "hipnx_buf_destroy": [_buf_p],
+    "hipnx_buf_size": [_buf_p, C.POINTER(C.c_size_t)],
+    "hipnx_buf_device_ptr": [_buf_p],
+    "hipnx_h2d": [_ctx_p, _buf_p, C.c_size_t, C.c_void_p, C.c_size_t],
+    "hipnx_d2h": [_ctx_p, _buf_p, C.c_size_t, C.c_void_p, C.c_size_t],
+    "hipnx_d2d": [_ctx_p, _buf_p, C.c_size_t, _buf_p, C.c_size_t, C.c_size_t],
+    "hipnx_fill": [_ctx_p, _buf_p, C.c_int, C.c_void_p, C.c_int64],
+    "hipnx_binary": [_ctx_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _i64p, _i64p, _i64p, _buf_p, _buf_p, _buf_p],
+    "hipnx_unary": [_ctx_p, C.c_int, C.c_int, C.c_int, C.c_int64, _buf_p, _buf_p],
+    "hipnx_as_type": [_ctx_p, C.c_int, C.c_int, C.c_int64, _buf_p, _buf_p],
+    "hipnx_reduce": [_ctx_p, C.c_int, C.c_int, C.c_int, C.c_int64, C.c_int64, C.c_int64, _buf_p, _buf_p],
+    "hipnx_argreduce": [_ctx_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int64, C.c_int64, C.c_int64, _buf_p, _buf_p],
+    "hipnx_dot": [_ctx_p, C.c_int, C.c_int, C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_int,
+                  _buf_p, _buf_p, _buf_p],
+    "hipnx_transpose": [_ctx_p, C.c_int, C.c_int, _i64p, _intp, _buf_p, _buf_p],
+    "hipnx_broadcast": [_ctx_p, C.c_int, C.c_int, _i64p, _i64p, _buf_p, _buf_p],
+    "hipnx_gather": [_ctx_p, C.c_int, C.c_int, _i64p, C.c_int, C.c_int64, C.c_int, C.c_int, _buf_p, _buf_p, _buf_p],
+}
+
+for _name, _args in PROTOTYPES.items():
+    _fn = getattr(lib, _name)  # AttributeError here = the library lacks a declared symbol
+    _fn.argtypes = _args
+    _fn.restype = C.c_void_p if _name == "hipnx_buf_device_ptr" else C.c_int
+
+
+def last_error() -> str:
+    buf = C.create_string_buffer(512)
+    lib.hipnx_last_error(buf, 512)
+    return buf.value.decode("utf-8", "replace")
+
+
+def check(status: int) -> int:
+    """Raises on every status except OK and ALREADY_FREED (which the caller interprets)."""
+    if status in (OK, ALREADY_FREED):
+        return status
+    cls = HipNxArgumentError if status in (EINVAL, EINDEX) else HipNxError
+    raise cls(status, last_error())
+
+
+def i64_array(values):
+    values = list(values)
+    return (C.c_int64 * max(len(values), 1))(*values)
+
+
+def int_array(values):
+    values = list(values)
+    return (C.c_int * max(len(values), 1))(*values)

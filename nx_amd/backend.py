@@ -1,0 +1,487 @@
+"""HipNx.Backend -- the `Nx.Backend` behaviour (reference: nx/lib/nx/backend.ex:46-144) over
+libhipnx, for the eager tensor path on one MI355X.
+
+This is the Python twin of `lib/hipnx/backend.ex`: the same callbacks, with the same argument
+meaning (`op(out_template, args...) -> tensor`) and the same error behaviour, calling the same C
+ABI the NIF shim binds.  The structural model is the reference's Torchx backend
+(torchx/lib/torchx/backend.ex): one native call per callback, operands that live on another
+backend are transferred on entry (`from_nx/1`, torchx/lib/torchx/backend.ex:2040-2041),
+callbacks outside the device path raise (torchx/lib/torchx/backend.ex:2199-2210).
+
+A device tensor's `data` is `HipNxBackend(ref, device)`: `ref` owns a flat untyped device buffer;
+type, shape and strides always come from the `Tensor` structs passed to the callback.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import threading
+from math import prod
+
+import numpy as np
+
+from . import _lib as L
+from . import shape as S
+from . import types as T
+from .tensor import Tensor, number_to_binary
+
+BINARY_OPS = ["add", "subtract", "multiply", "divide", "pow", "remainder", "atan2", "min", "max", "quotient",
+              "bitwise_and", "bitwise_or", "bitwise_xor", "left_shift", "right_shift", "equal", "not_equal",
+              "greater", "less", "greater_equal", "less_equal", "logical_and", "logical_or", "logical_xor"]
+UNARY_OPS = ["exp", "expm1", "log", "log1p", "sigmoid", "cos", "sin", "tan", "cosh", "sinh", "tanh", "acos", "asin",
+             "atan", "acosh", "asinh", "atanh", "sqrt", "rsqrt", "cbrt", "erf", "erfc", "erf_inv", "abs",
+             "bitwise_not", "ceil", "floor", "negate", "round", "sign", "count_leading_zeros", "population_count",
+             "is_nan", "is_infinity"]
+RED_SUM, RED_MAX, RED_MIN, RED_PRODUCT = 0, 1, 2, 3
+K_INNER, K_OUTER = 0, 1
+OOB_RAISE, OOB_CLAMP = 0, 1
+
+# callbacks of the behaviour that are not on the device path (nx/lib/nx/backend.ex:58-144)
+UNSUPPORTED = ["iota", "eye", "to_batched", "from_pointer", "to_pointer", "slice", "put_slice", "pad", "reverse",
+               "concatenate", "stack", "select", "clip", "conv", "all", "any", "window_sum", "window_product",
+               "window_max", "window_min", "reduce", "window_reduce", "window_scatter_max", "window_scatter_min",
+               "indexed_add", "indexed_put", "sort", "argsort", "fft", "ifft", "fft2", "ifft2", "triangular_solve",
+               "conjugate", "real", "imag"]
+
+
+class _Context:
+    """One libhipnx context per device, created on first use and kept for the process
+    (cf. the client registry of exla/lib/exla/client.ex:20-55)."""
+
+    _lock = threading.Lock()
+    _by_device = {}
+
+    @classmethod
+    def get(cls, device: int):
+        with cls._lock:
+            ctx = cls._by_device.get(device)
+            if ctx is None:
+                handle = C.c_void_p()
+                L.check(L.lib.hipnx_ctx_create(device, C.byref(handle)))
+                ctx = cls._by_device[device] = handle
+            return ctx
+
+
+class _Ref:
+    """Owns one device buffer.  Metadata-only callbacks (reshape / squeeze / bitcast) share it;
+    it is deallocated when the last sharer is, or by the garbage collector."""
+
+    def __init__(self, ctx, nbytes: int):
+        self.ctx = ctx
+        self.handle = C.c_void_p()
+        self.nbytes = nbytes
+        self.sharers = 1
+        L.check(L.lib.hipnx_buf_alloc(ctx, nbytes, C.byref(self.handle)))
+
+    def __del__(self):
+        if getattr(self, "handle", None) and self.handle.value:
+            try:
+                L.lib.hipnx_buf_destroy(self.handle)
+            except Exception:  # interpreter shutdown
+                pass
+            self.handle = None
+
+
+class HipNxBackend:
+    """Backend struct: `%HipNx.Backend{ref, device}`."""
+
+    def __init__(self, ref: _Ref, device: int):
+        self.ref = ref
+        self.device = device
+        self.released = False
+
+    def __repr__(self):
+        return f"HipNxBackend(device={self.device}, bytes={self.ref.nbytes})"
+
+    # ---- options / plumbing -------------------------------------------------------------
+    @staticmethod
+    def init(opts):
+        """init/1 (backend.ex:46): validates the backend options, cf. torchx backend.ex:49-52."""
+        opts = dict(opts or {})
+        unknown = set(opts) - {"device"}
+        if unknown:
+            raise ValueError(f"unknown keys {sorted(unknown)!r} in {opts!r}, the allowed keys are: ['device']")
+        opts.setdefault("device", 0)
+        return opts
+
+    @staticmethod
+    def _ctx(device):
+        return _Context.get(device)
+
+    @classmethod
+    def _alloc(cls, out: Tensor, device: int) -> Tensor:
+        nbytes = out.size * T.size_bytes(out.type)
+        return out.with_(data=cls(_Ref(cls._ctx(device), nbytes), device))
+
+    @classmethod
+    def _handle(cls, t: Tensor):
+        d = t.data
+        if d.released:
+            raise L.HipNxError(L.EFREED, "tensor has been deallocated")
+        return d.ref.handle
+
+    @classmethod
+    def _from_nx(cls, t: Tensor, device: int) -> Tensor:
+        """Operands that live on another backend are copied in on entry."""
+        if isinstance(t.data, HipNxBackend):
+            return t
+        binary = t.data.__class__.to_binary(t, t.size)
+        return cls.from_binary(t, binary, {"device": device})
+
+    @staticmethod
+    def _device_of(*tensors) -> int:
+        for t in tensors:
+            if isinstance(t.data, HipNxBackend):
+                return t.data.device
+        return 0
+
+    # ---- creation / transfer -------------------------------------------------------------
+    @classmethod
+    def from_binary(cls, out: Tensor, binary, opts=None) -> Tensor:
+        """from_binary/3 (backend.ex:50); rejects a binary shorter than the shape needs
+        (torchx/c_src/torchx.cpp:119-123)."""
+        opts = cls.init(opts)
+        binary = bytes(binary) if not isinstance(binary, (bytes, bytearray, memoryview)) else binary
+        need = out.size * T.size_bytes(out.type)
+        if len(binary) < need:
+            raise ValueError("binary size is too small for the requested shape")
+        res = cls._alloc(out, opts["device"])
+        if need:
+            src = (C.c_char * need).from_buffer_copy(memoryview(binary)[:need])
+            L.check(L.lib.hipnx_h2d(res.data.ref.ctx, res.data.ref.handle, 0, src, need))
+        return res
+
+    @classmethod
+    def from_numpy(cls, out: Tensor, array: np.ndarray, opts=None) -> Tensor:
+        """Zero-staging variant of from_binary for harnesses: uploads straight from the array."""
+        opts = cls.init(opts)
+        array = np.ascontiguousarray(array)
+        need = out.size * T.size_bytes(out.type)
+        if array.nbytes < need:
+            raise ValueError("binary size is too small for the requested shape")
+        res = cls._alloc(out, opts["device"])
+        if need:
+            L.check(L.lib.hipnx_h2d(res.data.ref.ctx, res.data.ref.handle, 0, array.ctypes.data_as(C.c_void_p), need))
+        return res
+
+    @classmethod
+    def to_binary(cls, t: Tensor, limit: int) -> bytes:
+        """to_binary/2 (backend.ex:57): `limit` counts elements."""
+        n = min(int(limit), t.size) * T.size_bytes(t.type)
+        buf = C.create_string_buffer(max(n, 1))
+        L.check(L.lib.hipnx_d2h(t.data.ref.ctx, cls._handle(t), 0, buf, n))
+        return buf.raw[:n]
+
+    @classmethod
+    def to_numpy(cls, t: Tensor) -> np.ndarray:
+        arr = np.empty(t.shape, dtype=T.numpy_dtype(t.type))
+        L.check(L.lib.hipnx_d2h(t.data.ref.ctx, cls._handle(t), 0, arr.ctypes.data_as(C.c_void_p), arr.nbytes))
+        return arr
+
+    @classmethod
+    def constant(cls, out: Tensor, number, opts=None) -> Tensor:
+        """constant/3 (backend.ex:49; oracle binary_backend.ex:42-46)."""
+        opts = cls.init(opts)
+        res = cls._alloc(out, opts["device"])
+        elem = number_to_binary(number, out.type)
+        L.check(L.lib.hipnx_fill(res.data.ref.ctx, res.data.ref.handle, len(elem), elem, out.size))
+        return res
+
+    @classmethod
+    def backend_copy(cls, t: Tensor, backend, opts=None) -> Tensor:
+        """backend_copy/3 (backend.ex:52)."""
+        if backend is HipNxBackend:
+            opts = cls.init(opts)
+            if opts["device"] == t.data.device:
+                res = cls._alloc(t, opts["device"])
+                L.check(L.lib.hipnx_d2d(res.data.ref.ctx, res.data.ref.handle, 0, cls._handle(t), 0, res.data.ref.nbytes))
+                return res
+        return backend.from_binary(t, cls.to_binary(t, t.size), opts)
+
+    @classmethod
+    def backend_transfer(cls, t: Tensor, backend, opts=None) -> Tensor:
+        """backend_transfer/3 (backend.ex:51): copy, then deallocate the source."""
+        if backend is HipNxBackend and cls.init(opts)["device"] == t.data.device:
+            return t
+        res = cls.backend_copy(t, backend, opts)
+        cls.backend_deallocate(t)
+        return res
+
+    @classmethod
+    def backend_deallocate(cls, t: Tensor) -> str:
+        """backend_deallocate/1 (backend.ex:53): "ok" the first time, "already_deallocated" after
+        (torchx/test/torchx/device_test.exs:30-37)."""
+        d = t.data
+        if d.released:
+            return "already_deallocated"
+        d.released = True
+        d.ref.sharers -= 1
+        if d.ref.sharers > 0:
+            return "ok"
+        st = L.check(L.lib.hipnx_buf_free(d.ref.handle))
+        return "ok" if st == L.OK else "already_deallocated"
+
+    @classmethod
+    def inspect(cls, t: Tensor, limit: int = 50) -> str:
+        """inspect/2 (backend.ex:56): reads limit+1 elements like torchx backend.ex:2013-2035."""
+        from .tensor import to_float64, binary_to_numpy
+        binary = cls.to_binary(t, min(t.size, limit + 1))
+        n = len(binary) // T.size_bytes(t.type)
+        vals = to_float64(binary, t.type) if T.is_float(t.type) else binary_to_numpy(binary, t.type)
+        body = ", ".join(str(v) for v in vals[:limit]) + (", ..." if n > limit else "")
+        dims = "".join(f"[{d}]" for d in t.shape)
+        return f"#Nx.Tensor<\n  {T.name(t.type)}{dims}\n  HipNx.Backend({t.data.device})\n  [{body}]\n>"
+
+    # ---- metadata-only: the buffer is immutable, so these share it ------------------------
+    @classmethod
+    def _alias(cls, out: Tensor, t: Tensor) -> Tensor:
+        cls._handle(t)
+        t.data.ref.sharers += 1
+        return out.with_(data=cls(t.data.ref, t.data.device))
+
+    @classmethod
+    def reshape(cls, out, t):
+        return cls._alias(out, cls._from_nx(t, 0))
+
+    @classmethod
+    def squeeze(cls, out, t, axes):
+        return cls._alias(out, cls._from_nx(t, 0))
+
+    @classmethod
+    def bitcast(cls, out, t):
+        return cls._alias(out, cls._from_nx(t, 0))
+
+    # ---- element-wise ----------------------------------------------------------------------
+    @classmethod
+    def _binary(cls, op: int, out: Tensor, l: Tensor, r: Tensor) -> Tensor:
+        dev = cls._device_of(l, r)
+        l, r = cls._from_nx(l, dev), cls._from_nx(r, dev)
+        res = cls._alloc(out, dev)
+        rank = len(out.shape)
+        L.check(L.lib.hipnx_binary(
+            res.data.ref.ctx, op, T.code(l.type), T.code(r.type), T.code(out.type), rank, L.i64_array(out.shape),
+            L.i64_array(S.broadcast_strides(l.shape, out.shape)), L.i64_array(S.broadcast_strides(r.shape, out.shape)),
+            cls._handle(l), cls._handle(r), res.data.ref.handle))
+        return res
+
+    @classmethod
+    def _unary(cls, op: int, out: Tensor, t: Tensor) -> Tensor:
+        dev = cls._device_of(t)
+        t = cls._from_nx(t, dev)
+        res = cls._alloc(out, dev)
+        L.check(L.lib.hipnx_unary(res.data.ref.ctx, op, T.code(t.type), T.code(out.type), out.size, cls._handle(t),
+                                  res.data.ref.handle))
+        return res
+
+    @classmethod
+    def as_type(cls, out: Tensor, t: Tensor) -> Tensor:
+        """as_type/2 (backend.ex:68; oracle binary_backend.ex:2031-2076)."""
+        dev = cls._device_of(t)
+        t = cls._from_nx(t, dev)
+        if t.type == out.type:
+            return t
+        res = cls._alloc(out, dev)
+        L.check(L.lib.hipnx_as_type(res.data.ref.ctx, T.code(t.type), T.code(out.type), out.size, cls._handle(t),
+                                    res.data.ref.handle))
+        return res
+
+    # ---- reductions ------------------------------------------------------------------------
+    @classmethod
+    def _view_for_axes(cls, t: Tensor, axes):
+        """Collapses `t` to [outer, red, inner] for a reduction over `axes` (all axes if None).
+        Non-adjacent axes are brought together by a device transpose to kept ++ reduced, which
+        keeps the row-major order of the reduced axes (binary_backend.ex:2469-2512)."""
+        rank = len(t.shape)
+        if axes is None:
+            return t, 1, t.size, 1
+        axes = sorted(axes)
+        if not axes:
+            return t, t.size, 1, 1
+        if axes == list(range(axes[0], axes[-1] + 1)):
+            return t, prod(t.shape[:axes[0]]), prod(t.shape[axes[0]:axes[-1] + 1]), prod(t.shape[axes[-1] + 1:])
+        kept = [a for a in range(rank) if a not in axes]
+        perm = kept + axes
+        tt = cls.transpose(t.with_(shape=S.transpose(t.shape, perm)), t, perm)
+        return tt, prod(t.shape[a] for a in kept), prod(t.shape[a] for a in axes), 1
+
+    @classmethod
+    def _reduce(cls, op: int, out: Tensor, t: Tensor, opts) -> Tensor:
+        dev = cls._device_of(t)
+        t = cls._from_nx(t, dev)
+        view, outer, red, inner = cls._view_for_axes(t, opts.get("axes"))
+        res = cls._alloc(out, dev)
+        L.check(L.lib.hipnx_reduce(res.data.ref.ctx, op, T.code(t.type), T.code(out.type), outer, red, inner,
+                                   cls._handle(view), res.data.ref.handle))
+        return res
+
+    @classmethod
+    def sum(cls, out, t, opts):
+        return cls._reduce(RED_SUM, out, t, opts)
+
+    @classmethod
+    def product(cls, out, t, opts):
+        return cls._reduce(RED_PRODUCT, out, t, opts)
+
+    @classmethod
+    def reduce_max(cls, out, t, opts):
+        return cls._reduce(RED_MAX, out, t, opts)
+
+    @classmethod
+    def reduce_min(cls, out, t, opts):
+        return cls._reduce(RED_MIN, out, t, opts)
+
+    @classmethod
+    def _argreduce(cls, op: int, out: Tensor, t: Tensor, opts) -> Tensor:
+        dev = cls._device_of(t)
+        t = cls._from_nx(t, dev)
+        axis = opts.get("axis")
+        tie = {"low": 0, "high": 1}[opts.get("tie_break", "low")]
+        view, outer, red, inner = cls._view_for_axes(t, None if axis is None else [axis])
+        res = cls._alloc(out, dev)
+        L.check(L.lib.hipnx_argreduce(res.data.ref.ctx, op, tie, T.code(t.type), T.code(out.type), outer, red, inner,
+                                      cls._handle(view), res.data.ref.handle))
+        return res
+
+    @classmethod
+    def argmax(cls, out, t, opts):
+        return cls._argreduce(0, out, t, opts)
+
+    @classmethod
+    def argmin(cls, out, t, opts):
+        return cls._argreduce(1, out, t, opts)
+
+    # ---- contraction -----------------------------------------------------------------------
+    @classmethod
+    def _dot_operand(cls, t: Tensor, contract, nbatch: int):
+        """Returns (tensor, layout, kept_size): the operand as [batch, rows, K] (K_INNER) or
+        [batch, K, rows] (K_OUTER) without a copy when the axes already sit that way, else
+        transposed on the device to [batch, kept, contract] as binary_backend.ex:561-599 does."""
+        rank = len(t.shape)
+        batch = list(range(nbatch))
+        kept = [a for a in range(nbatch, rank) if a not in contract]
+        rows = prod(t.shape[a] for a in kept)
+        if batch + kept + list(contract) == list(range(rank)):
+            return t, K_INNER, rows
+        if batch + list(contract) + kept == list(range(rank)):
+            return t, K_OUTER, rows
+        perm = batch + kept + list(contract)
+        return cls.transpose(t.with_(shape=S.transpose(t.shape, perm)), t, perm), K_INNER, rows
+
+    @classmethod
+    def dot(cls, out: Tensor, l: Tensor, c1, b1, r: Tensor, c2, b2) -> Tensor:
+        """dot/7 (backend.ex:77; oracle binary_backend.ex:476-599).  Contraction axes are paired
+        in the given order; the pairs are walked in increasing left-axis order so that the left
+        operand needs no copy whenever its contracted axes are adjacent."""
+        dev = cls._device_of(l, r)
+        l, r = cls._from_nx(l, dev), cls._from_nx(r, dev)
+        pairs = sorted(zip(c1, c2))
+        c1s, c2s = [p[0] for p in pairs], [p[1] for p in pairs]
+        nb = len(b1)
+        K = prod(l.shape[a] for a in c1s)
+        batch = prod(l.shape[a] for a in b1)
+        lt, l_layout, M = cls._dot_operand(l, c1s, nb)
+        rt, r_layout, N = cls._dot_operand(r, c2s, nb)
+        res = cls._alloc(out, dev)
+        L.check(L.lib.hipnx_dot(res.data.ref.ctx, T.code(l.type), T.code(r.type), T.code(out.type), batch, M, N, K,
+                                l_layout, r_layout, cls._handle(lt), cls._handle(rt), res.data.ref.handle))
+        return res
+
+    # ---- data movement ---------------------------------------------------------------------
+    @classmethod
+    def transpose(cls, out: Tensor, t: Tensor, axes) -> Tensor:
+        """transpose/3 (backend.ex:74; oracle binary_backend.ex:280-306)."""
+        dev = cls._device_of(t)
+        t = cls._from_nx(t, dev)
+        res = cls._alloc(out, dev)
+        L.check(L.lib.hipnx_transpose(res.data.ref.ctx, T.size_bytes(t.type), len(t.shape), L.i64_array(t.shape),
+                                      L.int_array(axes), cls._handle(t), res.data.ref.handle))
+        return res
+
+    @classmethod
+    def broadcast(cls, out: Tensor, t: Tensor, shape, axes) -> Tensor:
+        """broadcast/4 (backend.ex:75; oracle binary_backend.ex:215-276): input axis i maps to
+        output axis axes[i]; size-1 input axes and unmapped output axes repeat."""
+        dev = cls._device_of(t)
+        t = cls._from_nx(t, dev)
+        strides = [0] * len(shape)
+        s = 1
+        for pos in range(len(t.shape) - 1, -1, -1):
+            if t.shape[pos] != 1:
+                strides[axes[pos]] = s
+            s *= t.shape[pos]
+        res = cls._alloc(out, dev)
+        L.check(L.lib.hipnx_broadcast(res.data.ref.ctx, T.size_bytes(t.type), len(shape), L.i64_array(shape),
+                                      L.i64_array(strides), cls._handle(t), res.data.ref.handle))
+        return res
+
+    @classmethod
+    def gather(cls, out: Tensor, t: Tensor, indices: Tensor, opts) -> Tensor:
+        """gather/4 (backend.ex:81; oracle binary_backend.ex:1902-1959): out-of-bounds indices
+        raise, with the reference's message."""
+        dev = cls._device_of(t, indices)
+        t, indices = cls._from_nx(t, dev), cls._from_nx(indices, dev)
+        axes = list(opts["axes"])
+        rank = len(t.shape)
+        if list(range(rank))[:len(axes)] != axes:
+            perm = axes + [a for a in range(rank) if a not in axes]
+            t = cls.transpose(t.with_(shape=S.transpose(t.shape, perm)), t, perm)
+        depth = indices.shape[-1]
+        n_tuples = prod(indices.shape[:-1])
+        res = cls._alloc(out, dev)
+        L.check(L.lib.hipnx_gather(res.data.ref.ctx, T.size_bytes(t.type), rank, L.i64_array(t.shape),
+                                   T.code(indices.type), n_tuples, depth, opts.get("oob_policy", OOB_RAISE),
+                                   cls._handle(t), cls._handle(indices), res.data.ref.handle))
+        return res
+
+    @classmethod
+    def block(cls, struct, out: Tensor, args, fun):
+        """block/4 (backend.ex:144): `Nx.Block.Take` along axis 0 is one row-copy kernel; other
+        blocks run their default implementation on this backend's callbacks."""
+        from .nx import BlockTake
+        if isinstance(struct, BlockTake) and struct.axis == 0:
+            t, indices = args
+            idx = indices.with_(shape=(indices.size, 1))
+            return cls.gather(out, t, idx, {"axes": [0]})
+        return fun(struct, *args)
+
+
+def _install():
+    for code, name in enumerate(BINARY_OPS):
+        def binary(cls, out, l, r, _code=code):
+            return cls._binary(_code, out, l, r)
+        binary.__name__ = name
+        binary.__doc__ = f"{name}/3 (backend.ex:115-123; oracle binary_backend.ex:649-823)."
+        setattr(HipNxBackend, name, classmethod(binary))
+    for code, name in enumerate(UNARY_OPS):
+        def unary(cls, out, t, _code=code):
+            return cls._unary(_code, out, t)
+        unary.__name__ = name
+        unary.__doc__ = f"{name}/2 (backend.ex:125-132; oracle binary_backend.ex:827-1005)."
+        setattr(HipNxBackend, name, classmethod(unary))
+    for name in UNSUPPORTED:
+        def unsupported(cls, *args, _name=name, **kw):
+            raise NotImplementedError(f"HipNx.Backend.{_name} is not on the device path")
+        unsupported.__name__ = name
+        setattr(HipNxBackend, name, classmethod(unsupported))
+
+
+_install()
+
+
+def sync(device: int = 0) -> None:
+    L.check(L.lib.hipnx_sync(_Context.get(device)))
+
+
+def timer_start(device: int = 0) -> None:
+    L.check(L.lib.hipnx_timer_start(_Context.get(device)))
+
+
+def timer_stop(device: int = 0) -> float:
+    ms = C.c_float()
+    L.check(L.lib.hipnx_timer_stop(_Context.get(device), C.byref(ms)))
+    return ms.value
+
+
+def mem_stats(device: int = 0):
+    live, peak, pooled = C.c_uint64(), C.c_uint64(), C.c_uint64()
+    L.check(L.lib.hipnx_mem_stats(_Context.get(device), C.byref(live), C.byref(peak), C.byref(pooled)))
+    return {"live": live.value, "peak": peak.value, "pooled": pooled.value}

@@ -1,0 +1,303 @@
+// Context, device buffers and transfers of libhipnx (host code only, no kernels).
+//
+// The buffer life-cycle follows what the reference's device backends expose to Elixir:
+// explicit, idempotent deallocation that reports :ok / :already_deallocated
+// (torchx/c_src/torchx_nif_util.h:66-111, torchx/test/torchx/device_test.exs:30-37) and a
+// use-after-free that is an error, not a crash (exla/test/exla/backend_test.exs:48-50).
+#include <cstdlib>
+#include <cstring>
+
+#include "internal.h"
+
+namespace hipnx {
+
+static thread_local char g_err[512] = "";
+
+int set_error(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof g_err, fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int hip_fail(hipError_t e, const char *what) {
+  (void)hipGetLastError();  // clear the sticky error so later calls report their own
+  return set_error(e == hipErrorOutOfMemory ? HIPNX_ENOMEM : HIPNX_EHIP, "HIP error %d (%s) in %s",
+                   (int)e, hipGetErrorString(e), what);
+}
+
+int check_buf(const hipnx_ctx *ctx, const hipnx_buf *b, uint64_t need_bytes, const char *name) {
+  if (!b) return set_error(HIPNX_EINVAL, "%s: null buffer handle", name);
+  if (b->freed.load()) return set_error(HIPNX_EFREED, "%s: buffer has been deallocated", name);
+  if (b->ctx != ctx) return set_error(HIPNX_EINVAL, "%s: buffer belongs to another context", name);
+  if (b->bytes < need_bytes)
+    return set_error(HIPNX_EINVAL, "%s: buffer holds %zu bytes, the shape needs %llu", name, b->bytes,
+                     (unsigned long long)need_bytes);
+  return HIPNX_OK;
+}
+
+Enter::Enter(hipnx_ctx *ctx) : status(HIPNX_OK) {
+  if (!ctx) {
+    status = set_error(HIPNX_EINVAL, "null context");
+    return;
+  }
+  lk = std::unique_lock<std::mutex>(ctx->mu);
+  hipError_t e = hipSetDevice(ctx->device);
+  if (e != hipSuccess) status = hip_fail(e, "hipSetDevice");
+}
+
+static uint64_t pool_cap_bytes() {
+  static uint64_t cap = [] {
+    const char *s = getenv("HIPNX_POOL_MAX_MB");
+    uint64_t mb = s ? strtoull(s, nullptr, 10) : 32768ull;
+    return mb << 20;
+  }();
+  return cap;
+}
+
+static size_t round_capacity(size_t bytes) {
+  if (bytes == 0) bytes = 1;
+  if (bytes <= (1u << 20)) return (bytes + 255) & ~size_t(255);
+  return (bytes + ((1u << 20) - 1)) & ~size_t((1u << 20) - 1);
+}
+
+// Both run with the context mutex held.
+int pool_alloc(hipnx_ctx *ctx, size_t bytes, void **ptr_out, size_t *cap_out) {
+  size_t cap = round_capacity(bytes);
+  void *ptr = nullptr;
+  auto it = ctx->pool.lower_bound(cap);
+  if (it != ctx->pool.end() && it->first <= cap + cap / 4) {
+    ptr = it->second;
+    cap = it->first;
+    ctx->pooled -= cap;
+    ctx->pool.erase(it);
+  } else {
+    hipError_t e = hipMalloc(&ptr, cap);
+    if (e != hipSuccess && !ctx->pool.empty()) {
+      // give cached blocks back and retry once
+      (void)hipGetLastError();
+      (void)hipStreamSynchronize(ctx->stream);
+      for (auto &kv : ctx->pool) (void)hipFree(kv.second);
+      ctx->pool.clear();
+      ctx->pooled = 0;
+      e = hipMalloc(&ptr, cap);
+    }
+    if (e != hipSuccess) return hip_fail(e, "hipMalloc");
+  }
+  ctx->live += cap;
+  if (ctx->live > ctx->peak) ctx->peak = ctx->live;
+  *ptr_out = ptr;
+  *cap_out = cap;
+  return HIPNX_OK;
+}
+
+int pool_free(hipnx_ctx *ctx, void *ptr, size_t cap) {
+  ctx->live -= cap;
+  if (ctx->pooled + cap <= pool_cap_bytes()) {
+    // reuse without a device wait is safe: all work of this context is ordered on one stream
+    ctx->pool.emplace(cap, ptr);
+    ctx->pooled += cap;
+    return HIPNX_OK;
+  }
+  HIPNX_HIP(hipStreamSynchronize(ctx->stream));
+  HIPNX_HIP(hipFree(ptr));
+  return HIPNX_OK;
+}
+
+}  // namespace hipnx
+
+using namespace hipnx;
+
+extern "C" {
+
+int hipnx_last_error(char *dst, size_t cap) {
+  if (!dst || cap == 0) return HIPNX_EINVAL;
+  snprintf(dst, cap, "%s", g_err);
+  return HIPNX_OK;
+}
+
+int hipnx_device_count(int *count) {
+  if (!count) return set_error(HIPNX_EINVAL, "null count");
+  int n = 0;
+  hipError_t e = hipGetDeviceCount(&n);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    n = 0;
+  }
+  *count = n;
+  return HIPNX_OK;
+}
+
+int hipnx_ctx_create(int device, hipnx_ctx **out) {
+  if (!out) return set_error(HIPNX_EINVAL, "null out");
+  int n = 0;
+  hipError_t e = hipGetDeviceCount(&n);
+  if (e != hipSuccess || n == 0) {
+    (void)hipGetLastError();
+    return set_error(HIPNX_EHIP, "no HIP device available");
+  }
+  if (device < 0 || device >= n) return set_error(HIPNX_EINVAL, "device %d out of range (0..%d)", device, n - 1);
+  HIPNX_HIP(hipSetDevice(device));
+  hipnx_ctx *ctx = new hipnx_ctx;
+  ctx->device = device;
+  hipDeviceProp_t prop;
+  if (hipGetDeviceProperties(&prop, device) == hipSuccess) ctx->num_cus = prop.multiProcessorCount;
+  hipError_t e1 = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
+  hipError_t e2 = hipEventCreate(&ctx->ev_start);
+  hipError_t e3 = hipEventCreate(&ctx->ev_stop);
+  hipError_t e4 = hipMalloc(&ctx->flag, 256);
+  hipError_t e5 = hipHostMalloc(&ctx->flag_host, 256, hipHostMallocDefault);
+  if (e1 != hipSuccess || e2 != hipSuccess || e3 != hipSuccess || e4 != hipSuccess || e5 != hipSuccess) {
+    hipnx_ctx_destroy(ctx);
+    return hip_fail(e1 != hipSuccess ? e1 : e2 != hipSuccess ? e2 : e3 != hipSuccess ? e3 : e4 != hipSuccess ? e4 : e5,
+                    "context set-up");
+  }
+  *out = ctx;
+  return HIPNX_OK;
+}
+
+int hipnx_ctx_destroy(hipnx_ctx *ctx) {
+  if (!ctx) return set_error(HIPNX_EINVAL, "null context");
+  (void)hipSetDevice(ctx->device);
+  if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+  for (auto &kv : ctx->pool) (void)hipFree(kv.second);
+  ctx->pool.clear();
+  if (ctx->flag) (void)hipFree(ctx->flag);
+  if (ctx->flag_host) (void)hipHostFree(ctx->flag_host);
+  if (ctx->ev_start) (void)hipEventDestroy(ctx->ev_start);
+  if (ctx->ev_stop) (void)hipEventDestroy(ctx->ev_stop);
+  if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
+  delete ctx;
+  return HIPNX_OK;
+}
+
+int hipnx_sync(hipnx_ctx *ctx) {
+  Enter in(ctx);
+  if (in.status) return in.status;
+  HIPNX_HIP(hipStreamSynchronize(ctx->stream));
+  return HIPNX_OK;
+}
+
+int hipnx_mem_stats(hipnx_ctx *ctx, uint64_t *live, uint64_t *peak, uint64_t *pooled) {
+  Enter in(ctx);
+  if (in.status) return in.status;
+  if (live) *live = ctx->live;
+  if (peak) *peak = ctx->peak;
+  if (pooled) *pooled = ctx->pooled;
+  return HIPNX_OK;
+}
+
+int hipnx_trim(hipnx_ctx *ctx) {
+  Enter in(ctx);
+  if (in.status) return in.status;
+  HIPNX_HIP(hipStreamSynchronize(ctx->stream));
+  for (auto &kv : ctx->pool) (void)hipFree(kv.second);
+  ctx->pool.clear();
+  ctx->pooled = 0;
+  return HIPNX_OK;
+}
+
+int hipnx_timer_start(hipnx_ctx *ctx) {
+  Enter in(ctx);
+  if (in.status) return in.status;
+  HIPNX_HIP(hipEventRecord(ctx->ev_start, ctx->stream));
+  return HIPNX_OK;
+}
+
+int hipnx_timer_stop(hipnx_ctx *ctx, float *elapsed_ms) {
+  Enter in(ctx);
+  if (in.status) return in.status;
+  if (!elapsed_ms) return set_error(HIPNX_EINVAL, "null elapsed_ms");
+  HIPNX_HIP(hipEventRecord(ctx->ev_stop, ctx->stream));
+  HIPNX_HIP(hipEventSynchronize(ctx->ev_stop));
+  HIPNX_HIP(hipEventElapsedTime(elapsed_ms, ctx->ev_start, ctx->ev_stop));
+  return HIPNX_OK;
+}
+
+int hipnx_buf_alloc(hipnx_ctx *ctx, size_t bytes, hipnx_buf **out) {
+  Enter in(ctx);
+  if (in.status) return in.status;
+  if (!out) return set_error(HIPNX_EINVAL, "null out");
+  void *ptr = nullptr;
+  size_t cap = 0;
+  if (int st = pool_alloc(ctx, bytes, &ptr, &cap)) return st;
+  hipnx_buf *b = new hipnx_buf;
+  b->ctx = ctx;
+  b->ptr = ptr;
+  b->bytes = bytes;
+  b->capacity = cap;
+  *out = b;
+  return HIPNX_OK;
+}
+
+int hipnx_buf_free(hipnx_buf *buf) {
+  if (!buf) return set_error(HIPNX_EINVAL, "null buffer handle");
+  int expected = 0;
+  if (!buf->freed.compare_exchange_strong(expected, 1)) return HIPNX_ALREADY_FREED;
+  hipnx_ctx *ctx = buf->ctx;
+  Enter in(ctx);
+  if (in.status) return in.status;
+  int st = pool_free(ctx, buf->ptr, buf->capacity);
+  buf->ptr = nullptr;
+  return st;
+}
+
+int hipnx_buf_destroy(hipnx_buf *buf) {
+  if (!buf) return set_error(HIPNX_EINVAL, "null buffer handle");
+  int st = hipnx_buf_free(buf);
+  delete buf;
+  return st == HIPNX_ALREADY_FREED ? HIPNX_OK : st;
+}
+
+int hipnx_buf_size(const hipnx_buf *buf, size_t *bytes) {
+  if (!buf || !bytes) return set_error(HIPNX_EINVAL, "null argument");
+  if (buf->freed.load()) return set_error(HIPNX_EFREED, "buffer has been deallocated");
+  *bytes = buf->bytes;
+  return HIPNX_OK;
+}
+
+void *hipnx_buf_device_ptr(const hipnx_buf *buf) {
+  if (!buf || buf->freed.load()) return nullptr;
+  return buf->ptr;
+}
+
+int hipnx_h2d(hipnx_ctx *ctx, hipnx_buf *dst, size_t dst_offset, const void *src, size_t bytes) {
+  Enter in(ctx);
+  if (in.status) return in.status;
+  if (int st = check_buf(ctx, dst, (uint64_t)dst_offset + bytes, "h2d dst")) return st;
+  if (bytes == 0) return HIPNX_OK;
+  if (!src) return set_error(HIPNX_EINVAL, "h2d: null source");
+  HIPNX_HIP(hipMemcpyAsync((char *)dst->ptr + dst_offset, src, bytes, hipMemcpyHostToDevice, ctx->stream));
+  // the source is caller-owned host memory (an Erlang binary): it must be consumed on return
+  HIPNX_HIP(hipStreamSynchronize(ctx->stream));
+  return HIPNX_OK;
+}
+
+int hipnx_d2h(hipnx_ctx *ctx, const hipnx_buf *src, size_t src_offset, void *dst, size_t bytes) {
+  Enter in(ctx);
+  if (in.status) return in.status;
+  if (int st = check_buf(ctx, src, (uint64_t)src_offset + bytes, "d2h src")) return st;
+  if (bytes == 0) {
+    HIPNX_HIP(hipStreamSynchronize(ctx->stream));
+    return HIPNX_OK;
+  }
+  if (!dst) return set_error(HIPNX_EINVAL, "d2h: null destination");
+  HIPNX_HIP(hipMemcpyAsync(dst, (const char *)src->ptr + src_offset, bytes, hipMemcpyDeviceToHost, ctx->stream));
+  HIPNX_HIP(hipStreamSynchronize(ctx->stream));
+  return HIPNX_OK;
+}
+
+int hipnx_d2d(hipnx_ctx *ctx, hipnx_buf *dst, size_t dst_offset, const hipnx_buf *src, size_t src_offset,
+              size_t bytes) {
+  Enter in(ctx);
+  if (in.status) return in.status;
+  if (int st = check_buf(ctx, dst, (uint64_t)dst_offset + bytes, "d2d dst")) return st;
+  if (int st = check_buf(ctx, src, (uint64_t)src_offset + bytes, "d2d src")) return st;
+  if (bytes == 0) return HIPNX_OK;
+  HIPNX_HIP(hipMemcpyAsync((char *)dst->ptr + dst_offset, (const char *)src->ptr + src_offset, bytes,
+                           hipMemcpyDeviceToDevice, ctx->stream));
+  return HIPNX_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,381 @@
+// Broadcasting element-wise binary / unary kernels and as_type: HBM streaming kernels.
+//
+// Each lane owns E = 8 consecutive output elements and moves them with 16-byte accesses.  A
+// binary op first has its index space collapsed on the host (unit axes dropped, axes merged
+// where both operands stay contiguous or both broadcast); whatever collapses to [rows, cols]
+// with per-operand strides (row stride, column stride in {0, 1}) -- same shape, scalar operand,
+// trailing row vector, keep-dims column -- runs on the vector kernel, the rest on a generic
+// rank-N kernel.  Algorithmic traffic is exactly bytes(l) + bytes(r) + bytes(out).
+#include "elementwise_ops.cuh"
+#include "internal.h"
+
+namespace hipnx {
+
+constexpr int E = 8;
+constexpr int BLOCK = 256;
+constexpr int MAXR = 8;
+
+struct NdIndex {
+  int rank;
+  int64_t dims[MAXR], ls[MAXR], rs[MAXR];
+};
+
+template <int OP, typename CT, bool UNS>
+__global__ void __launch_bounds__(BLOCK)
+binary_vec_kernel(const void *__restrict__ l, const void *__restrict__ r, void *__restrict__ out, int ldt, int rdt,
+                  int odt, int64_t cols, int64_t vecs_per_row, int64_t nvec, int64_t ls0, int ls1, int64_t rs0,
+                  int rs1) {
+  for (int64_t v = (int64_t)blockIdx.x * BLOCK + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * BLOCK) {
+    int64_t row = v / vecs_per_row;
+    int64_t col = (v - row * vecs_per_row) * E;
+    int64_t lo = row * ls0 + col * ls1, ro = row * rs0 + col * rs1, oo = row * cols + col;
+    CT a[E], b[E], c[E];
+    if (col + E <= cols) {
+      if (ls1) load_vec<CT, E>(l, ldt, lo, a);
+      else {
+        CT s = load_one<CT>(l, ldt, lo);
+#pragma unroll
+        for (int i = 0; i < E; i++) a[i] = s;
+      }
+      if (rs1) load_vec<CT, E>(r, rdt, ro, b);
+      else {
+        CT s = load_one<CT>(r, rdt, ro);
+#pragma unroll
+        for (int i = 0; i < E; i++) b[i] = s;
+      }
+#pragma unroll
+      for (int i = 0; i < E; i++) c[i] = binary_apply<OP, CT, UNS>(a[i], b[i]);
+      store_vec<CT, E>(out, odt, oo, c);
+    } else {  // ragged tail of a row
+      for (int i = 0; col + i < cols; i++) {
+        CT x = load_one<CT>(l, ldt, lo + i * ls1), y = load_one<CT>(r, rdt, ro + i * rs1);
+        store_one<CT>(out, odt, oo + i, binary_apply<OP, CT, UNS>(x, y));
+      }
+    }
+  }
+}
+
+template <typename CT, bool UNS>
+__device__ __forceinline__ CT binary_switch(int op, CT a, CT b) {
+  switch (op) {
+#define C(O) case O: return binary_apply<O, CT, UNS>(a, b);
+    C(0) C(1) C(2) C(3) C(4) C(5) C(6) C(7) C(8) C(9) C(10) C(11) C(12) C(13) C(14) C(15) C(16) C(17) C(18) C(19)
+    C(20) C(21) C(22) C(23)
+#undef C
+  }
+  return (CT)0;
+}
+
+// any rank, any strides: one element per lane per step
+template <typename CT, bool UNS>
+__global__ void __launch_bounds__(BLOCK)
+binary_nd_kernel(const void *__restrict__ l, const void *__restrict__ r, void *__restrict__ out, int op, int ldt,
+                 int rdt, int odt, int64_t n, NdIndex ix) {
+  for (int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x; i < n; i += (int64_t)gridDim.x * BLOCK) {
+    int64_t rem = i, lo = 0, ro = 0;
+    for (int a = ix.rank - 1; a >= 0; a--) {
+      int64_t q = rem / ix.dims[a], c = rem - q * ix.dims[a];
+      rem = q;
+      lo += c * ix.ls[a];
+      ro += c * ix.rs[a];
+    }
+    CT x = load_one<CT>(l, ldt, lo), y = load_one<CT>(r, rdt, ro);
+    store_one<CT>(out, odt, i, binary_switch<CT, UNS>(op, x, y));
+  }
+}
+
+template <int OP, typename CT>
+__global__ void __launch_bounds__(BLOCK)
+unary_vec_kernel(const void *__restrict__ in, void *__restrict__ out, int idt, int odt, int bits, int64_t n) {
+  int64_t nvec = (n + E - 1) / E;
+  for (int64_t v = (int64_t)blockIdx.x * BLOCK + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * BLOCK) {
+    int64_t o = v * E;
+    if (o + E <= n) {
+      CT a[E], c[E];
+      load_vec<CT, E>(in, idt, o, a);
+#pragma unroll
+      for (int i = 0; i < E; i++) c[i] = unary_apply<OP, CT>(a[i], bits);
+      store_vec<CT, E>(out, odt, o, c);
+    } else {
+      for (int i = 0; o + i < n; i++)
+        store_one<CT>(out, odt, o + i, unary_apply<OP, CT>(load_one<CT>(in, idt, o + i), bits));
+    }
+  }
+}
+
+// as_type: CT is the decode type of the input; float -> integer goes through the wrap rule
+template <typename CT>
+__global__ void __launch_bounds__(BLOCK)
+as_type_kernel(const void *__restrict__ in, void *__restrict__ out, int idt, int odt, int64_t n, int64_t tmax,
+               int64_t tmin) {
+  const bool to_int = odt < HIPNX_F16;
+  int64_t nvec = (n + E - 1) / E;
+  for (int64_t v = (int64_t)blockIdx.x * BLOCK + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * BLOCK) {
+    int64_t o = v * E;
+    if (o + E <= n) {
+      CT a[E];
+      load_vec<CT, E>(in, idt, o, a);
+      if constexpr (is_fp<CT>::value) {
+        if (to_int) {
+          int64_t c[E];
+#pragma unroll
+          for (int i = 0; i < E; i++) c[i] = float_to_int_wrap((double)a[i], tmax, tmin);
+          store_vec<int64_t, E>(out, odt, o, c);
+          continue;
+        }
+      }
+      store_vec<CT, E>(out, odt, o, a);
+    } else {
+      for (int i = 0; o + i < n; i++) {
+        CT x = load_one<CT>(in, idt, o + i);
+        if constexpr (is_fp<CT>::value) {
+          if (to_int) {
+            store_one<int64_t>(out, odt, o + i, float_to_int_wrap((double)x, tmax, tmin));
+            continue;
+          }
+        }
+        store_one<CT>(out, odt, o + i, x);
+      }
+    }
+  }
+}
+
+// ---- host side ------------------------------------------------------------------------------
+
+enum { CLS_F32 = 0, CLS_F64 = 1, CLS_I64 = 2, CLS_U64 = 3 };
+
+static int grid_for(const hipnx_ctx *ctx, int64_t work_items) {
+  int64_t blocks = (work_items + BLOCK - 1) / BLOCK;
+  int64_t cap = (int64_t)ctx->num_cus * 16;
+  if (blocks < 1) blocks = 1;
+  return (int)(blocks < cap ? blocks : cap);
+}
+
+struct BinArgs {
+  const void *l, *r;
+  void *out;
+  int ldt, rdt, odt;
+  int64_t cols, vecs_per_row, nvec, ls0, rs0;
+  int ls1, rs1;
+};
+
+template <int OP, typename CT, bool UNS>
+static void launch_bvec(const hipnx_ctx *ctx, const BinArgs &a) {
+  hipLaunchKernelGGL((binary_vec_kernel<OP, CT, UNS>), dim3(grid_for(ctx, a.nvec)), dim3(BLOCK), 0, ctx->stream, a.l,
+                     a.r, a.out, a.ldt, a.rdt, a.odt, a.cols, a.vecs_per_row, a.nvec, a.ls0, a.ls1, a.rs0, a.rs1);
+}
+
+template <int OP>
+static int launch_bvec_cls(const hipnx_ctx *ctx, int cls, const BinArgs &a) {
+  if constexpr (!binary_int_only(OP)) {
+    if (cls == CLS_F32) { launch_bvec<OP, float, false>(ctx, a); return HIPNX_OK; }
+    if (cls == CLS_F64) { launch_bvec<OP, double, false>(ctx, a); return HIPNX_OK; }
+  }
+  if constexpr (!binary_float_only(OP)) {
+    if (cls == CLS_I64) { launch_bvec<OP, int64_t, false>(ctx, a); return HIPNX_OK; }
+    if (cls == CLS_U64) {
+      if constexpr (binary_sign_matters(OP)) launch_bvec<OP, int64_t, true>(ctx, a);
+      else launch_bvec<OP, int64_t, false>(ctx, a);
+      return HIPNX_OK;
+    }
+  }
+  return set_error(HIPNX_EINVAL, "binary op %d is not defined for these operand types", OP);
+}
+
+template <int... OPS>
+static int launch_bvec_op(std::integer_sequence<int, OPS...>, const hipnx_ctx *ctx, int op, int cls,
+                          const BinArgs &a) {
+  int st = HIPNX_EINVAL;
+  (void)((op == OPS ? (st = launch_bvec_cls<OPS>(ctx, cls, a), true) : false) || ...);
+  return st;
+}
+
+static int binary_class(int op, int l_dt, int r_dt, int out_dt) {
+  bool any_float = is_float(l_dt) || is_float(r_dt) || is_float(out_dt);
+  if (any_float) {
+    bool wide = is_wide(l_dt) || is_wide(r_dt) || out_dt == HIPNX_F64;
+    return wide ? CLS_F64 : CLS_F32;
+  }
+  bool uns = is_unsigned(l_dt) && is_unsigned(r_dt) && (l_dt == HIPNX_U64 || r_dt == HIPNX_U64);
+  return uns ? CLS_U64 : CLS_I64;
+}
+
+}  // namespace hipnx
+
+using namespace hipnx;
+
+extern "C" int hipnx_binary(hipnx_ctx *ctx, int op, int l_dt, int r_dt, int out_dt, int rank,
+                            const int64_t *out_dims, const int64_t *l_strides, const int64_t *r_strides,
+                            const hipnx_buf *l, const hipnx_buf *r, hipnx_buf *out) {
+  Enter in(ctx);
+  if (in.status) return in.status;
+  if (op < 0 || op >= HIPNX_NBINARY) return set_error(HIPNX_EINVAL, "binary: unknown op %d", op);
+  if (dtype_size(l_dt) < 0 || dtype_size(r_dt) < 0 || dtype_size(out_dt) < 0)
+    return set_error(HIPNX_EINVAL, "binary: unknown element type");
+  if (rank < 0 || rank > 64 || (rank > 0 && (!out_dims || !l_strides || !r_strides)))
+    return set_error(HIPNX_EINVAL, "binary: bad rank / null shape");
+  // extent of each operand = 1 + sum (dim-1)*stride
+  int64_t n = 1, l_ext = 1, r_ext = 1;
+  for (int a = 0; a < rank; a++) {
+    if (out_dims[a] < 0 || l_strides[a] < 0 || r_strides[a] < 0)
+      return set_error(HIPNX_EINVAL, "binary: negative dimension or stride");
+    n *= out_dims[a];
+  }
+  if (n > 0)
+    for (int a = 0; a < rank; a++) {
+      l_ext += (out_dims[a] - 1) * l_strides[a];
+      r_ext += (out_dims[a] - 1) * r_strides[a];
+    }
+  if (int st = check_buf(ctx, l, n > 0 ? (uint64_t)l_ext * dtype_size(l_dt) : 0, "binary lhs")) return st;
+  if (int st = check_buf(ctx, r, n > 0 ? (uint64_t)r_ext * dtype_size(r_dt) : 0, "binary rhs")) return st;
+  if (int st = check_buf(ctx, out, (uint64_t)n * dtype_size(out_dt), "binary out")) return st;
+  if (n == 0) return HIPNX_OK;
+
+  bool any_float_in = is_float(l_dt) || is_float(r_dt);
+  if (binary_int_only(op) && (any_float_in || is_float(out_dt)))
+    return set_error(HIPNX_EINVAL, "binary: op %d needs integer operands", op);
+  int cls = binary_class(op, l_dt, r_dt, out_dt);
+
+  // collapse: drop unit axes, merge neighbours that stay contiguous (or broadcast) in both operands
+  NdIndex ix;
+  ix.rank = 0;
+  int64_t dims[64], ls[64], rs[64];
+  int m = 0;
+  for (int a = 0; a < rank; a++) {
+    if (out_dims[a] == 1) continue;
+    int64_t d = out_dims[a], s1 = l_strides[a], s2 = r_strides[a];
+    if (m > 0 && ls[m - 1] == s1 * d && rs[m - 1] == s2 * d) {
+      dims[m - 1] *= d;
+      ls[m - 1] = s1;
+      rs[m - 1] = s2;
+    } else {
+      dims[m] = d; ls[m] = s1; rs[m] = s2;
+      m++;
+    }
+  }
+  if (m == 0) { dims[0] = 1; ls[0] = 0; rs[0] = 0; m = 1; }
+
+  bool vec_ok = false;
+  BinArgs a{};
+  if (m <= 2) {
+    int64_t rows = m == 2 ? dims[0] : 1, cols = dims[m - 1];
+    int64_t l0 = m == 2 ? ls[0] : 0, r0 = m == 2 ? rs[0] : 0, l1 = ls[m - 1], r1 = rs[m - 1];
+    bool aligned = rows == 1 || (cols % E == 0 && l0 % E == 0 && r0 % E == 0) ||
+                   (cols % E == 0 && (l1 == 0 || l0 % E == 0) && (r1 == 0 || r0 % E == 0));
+    if ((l1 == 0 || l1 == 1) && (r1 == 0 || r1 == 1) && aligned) {
+      vec_ok = true;
+      a.l = l->ptr; a.r = r->ptr; a.out = out->ptr;
+      a.ldt = l_dt; a.rdt = r_dt; a.odt = out_dt;
+      a.cols = cols;
+      a.vecs_per_row = (cols + E - 1) / E;
+      a.nvec = rows * a.vecs_per_row;
+      a.ls0 = l0; a.rs0 = r0; a.ls1 = (int)l1; a.rs1 = (int)r1;
+    }
+  }
+  if (vec_ok) {
+    int st = launch_bvec_op(std::make_integer_sequence<int, HIPNX_NBINARY>{}, ctx, op, cls, a);
+    if (st) return st;
+  } else {
+    if (m > MAXR) return set_error(HIPNX_EUNSUPPORTED, "binary: more than %d non-collapsible axes", MAXR);
+    if (binary_float_only(op) && cls >= CLS_I64) return set_error(HIPNX_EINVAL, "binary: op %d yields a float", op);
+    ix.rank = m;
+    for (int q = 0; q < m; q++) { ix.dims[q] = dims[q]; ix.ls[q] = ls[q]; ix.rs[q] = rs[q]; }
+    dim3 grid(grid_for(ctx, n)), block(BLOCK);
+    switch (cls) {
+      case CLS_F32:
+        hipLaunchKernelGGL((binary_nd_kernel<float, false>), grid, block, 0, ctx->stream, l->ptr, r->ptr, out->ptr, op,
+                           l_dt, r_dt, out_dt, n, ix);
+        break;
+      case CLS_F64:
+        hipLaunchKernelGGL((binary_nd_kernel<double, false>), grid, block, 0, ctx->stream, l->ptr, r->ptr, out->ptr, op,
+                           l_dt, r_dt, out_dt, n, ix);
+        break;
+      case CLS_I64:
+        hipLaunchKernelGGL((binary_nd_kernel<int64_t, false>), grid, block, 0, ctx->stream, l->ptr, r->ptr, out->ptr,
+                           op, l_dt, r_dt, out_dt, n, ix);
+        break;
+      default:
+        hipLaunchKernelGGL((binary_nd_kernel<int64_t, true>), grid, block, 0, ctx->stream, l->ptr, r->ptr, out->ptr, op,
+                           l_dt, r_dt, out_dt, n, ix);
+        break;
+    }
+  }
+  HIPNX_HIP(hipGetLastError());
+  return HIPNX_OK;
+}
+
+namespace hipnx {
+
+template <int OP, typename CT>
+static void launch_uvec(const hipnx_ctx *ctx, const void *in, void *out, int idt, int odt, int bits, int64_t n) {
+  hipLaunchKernelGGL((unary_vec_kernel<OP, CT>), dim3(grid_for(ctx, (n + E - 1) / E)), dim3(BLOCK), 0, ctx->stream, in,
+                     out, idt, odt, bits, n);
+}
+
+template <int OP>
+static int launch_uvec_cls(const hipnx_ctx *ctx, int cls, const void *in, void *out, int idt, int odt, int bits,
+                           int64_t n) {
+  if constexpr (!unary_int_only(OP)) {
+    if (cls == CLS_F32) { launch_uvec<OP, float>(ctx, in, out, idt, odt, bits, n); return HIPNX_OK; }
+    if (cls == CLS_F64) { launch_uvec<OP, double>(ctx, in, out, idt, odt, bits, n); return HIPNX_OK; }
+  }
+  if constexpr (!unary_is_math(OP)) {
+    if (cls >= CLS_I64) { launch_uvec<OP, int64_t>(ctx, in, out, idt, odt, bits, n); return HIPNX_OK; }
+  }
+  return set_error(HIPNX_EINVAL, "unary op %d is not defined for this operand type", OP);
+}
+
+template <int... OPS>
+static int launch_uvec_op(std::integer_sequence<int, OPS...>, const hipnx_ctx *ctx, int op, int cls, const void *in,
+                          void *out, int idt, int odt, int bits, int64_t n) {
+  int st = HIPNX_EINVAL;
+  (void)((op == OPS ? (st = launch_uvec_cls<OPS>(ctx, cls, in, out, idt, odt, bits, n), true) : false) || ...);
+  return st;
+}
+
+}  // namespace hipnx
+
+extern "C" int hipnx_unary(hipnx_ctx *ctx, int op, int in_dt, int out_dt, int64_t n, const hipnx_buf *inb,
+                           hipnx_buf *out) {
+  Enter in(ctx);
+  if (in.status) return in.status;
+  if (op < 0 || op >= HIPNX_NUNARY) return set_error(HIPNX_EINVAL, "unary: unknown op %d", op);
+  if (dtype_size(in_dt) < 0 || dtype_size(out_dt) < 0 || n < 0)
+    return set_error(HIPNX_EINVAL, "unary: unknown element type or negative size");
+  if (int st = check_buf(ctx, inb, (uint64_t)n * dtype_size(in_dt), "unary in")) return st;
+  if (int st = check_buf(ctx, out, (uint64_t)n * dtype_size(out_dt), "unary out")) return st;
+  if (n == 0) return HIPNX_OK;
+  int cls;
+  if (is_float(in_dt) || is_float(out_dt)) cls = (is_wide(in_dt) || out_dt == HIPNX_F64) ? CLS_F64 : CLS_F32;
+  else cls = CLS_I64;
+  if (unary_int_only(op) && cls < CLS_I64) return set_error(HIPNX_EINVAL, "unary: op %d needs an integer operand", op);
+  int st = launch_uvec_op(std::make_integer_sequence<int, HIPNX_NUNARY>{}, ctx, op, cls, inb->ptr, out->ptr, in_dt,
+                          out_dt, 8 * dtype_size(in_dt), n);
+  if (st) return st;
+  HIPNX_HIP(hipGetLastError());
+  return HIPNX_OK;
+}
+
+extern "C" int hipnx_as_type(hipnx_ctx *ctx, int in_dt, int out_dt, int64_t n, const hipnx_buf *inb,
+                             hipnx_buf *out) {
+  Enter in(ctx);
+  if (in.status) return in.status;
+  if (dtype_size(in_dt) < 0 || dtype_size(out_dt) < 0 || n < 0)
+    return set_error(HIPNX_EINVAL, "as_type: unknown element type or negative size");
+  if (int st = check_buf(ctx, inb, (uint64_t)n * dtype_size(in_dt), "as_type in")) return st;
+  if (int st = check_buf(ctx, out, (uint64_t)n * dtype_size(out_dt), "as_type out")) return st;
+  if (n == 0) return HIPNX_OK;
+  static const int64_t tmax[8] = {0xFF, 0xFFFF, 0xFFFFFFFFll, -1ll /* u64 max */, 0x7F, 0x7FFF, 0x7FFFFFFFll,
+                                  0x7FFFFFFFFFFFFFFFll};
+  static const int64_t tmin[8] = {0, 0, 0, 0, -0x80, -0x8000, -0x80000000ll, (int64_t)0x8000000000000000ull};
+  int64_t mx = out_dt < HIPNX_F16 ? tmax[out_dt] : 0, mn = out_dt < HIPNX_F16 ? tmin[out_dt] : 0;
+  dim3 grid(grid_for(ctx, (n + E - 1) / E)), block(BLOCK);
+  if (!is_float(in_dt))
+    hipLaunchKernelGGL((as_type_kernel<int64_t>), grid, block, 0, ctx->stream, inb->ptr, out->ptr, in_dt, out_dt, n, mx, mn);
+  else if (in_dt == HIPNX_F64 || out_dt == HIPNX_F64 || out_dt == HIPNX_F16)
+    hipLaunchKernelGGL((as_type_kernel<double>), grid, block, 0, ctx->stream, inb->ptr, out->ptr, in_dt, out_dt, n, mx, mn);
+  else
+    hipLaunchKernelGGL((as_type_kernel<float>), grid, block, 0, ctx->stream, inb->ptr, out->ptr, in_dt, out_dt, n, mx, mn);
+  HIPNX_HIP(hipGetLastError());
+  return HIPNX_OK;
+}

@@ -1,0 +1,178 @@
+// Scalar semantics of the element-wise callbacks, shared by the streaming kernels.
+//
+// Compute classes.  The reference decodes every element to an Erlang number (IEEE double or
+// unbounded integer), applies the operation and encodes once (nx/lib/nx/binary_backend.ex:
+// 662-706, 2432-2438).  The same value is obtained on the device with
+//   float   when every operand is exactly representable in f32 and the output is f32/bf16/f16
+//           (a correctly rounded f32 + - * / equals the f64 operation rounded to f32);
+//   double  for every other combination that involves a float;
+//   int64_t (two's-complement wrap) when operands and output are integers.
+#pragma once
+#include <type_traits>
+#include <utility>
+
+#include "dtypes.cuh"
+
+namespace hipnx {
+
+template <typename T> struct is_fp { static constexpr bool value = false; };
+template <> struct is_fp<float> { static constexpr bool value = true; };
+template <> struct is_fp<double> { static constexpr bool value = true; };
+
+constexpr bool binary_int_only(int op) {
+  return op == HIPNX_QUOTIENT || (op >= HIPNX_BITWISE_AND && op <= HIPNX_RIGHT_SHIFT);
+}
+constexpr bool binary_float_only(int op) { return op == HIPNX_DIVIDE || op == HIPNX_ATAN2; }
+// ops whose integer result depends on reading the operands as signed or unsigned 64-bit
+constexpr bool binary_sign_matters(int op) {
+  return op == HIPNX_REMAINDER || op == HIPNX_QUOTIENT || op == HIPNX_MIN || op == HIPNX_MAX ||
+         op == HIPNX_RIGHT_SHIFT || (op >= HIPNX_GREATER && op <= HIPNX_LESS_EQUAL) || op == HIPNX_POW;
+}
+
+__device__ __forceinline__ int64_t ipow_wrap(int64_t base, uint64_t e) {
+  uint64_t r = 1, b = (uint64_t)base;
+  while (e) {
+    if (e & 1) r *= b;
+    b *= b;
+    e >>= 1;
+  }
+  return (int64_t)r;
+}
+
+// element_* of nx/lib/nx/binary_backend.ex:708-816
+template <int OP, typename CT, bool UNS>
+__device__ __forceinline__ CT binary_apply(CT a, CT b) {
+  if constexpr (is_fp<CT>::value) {
+    if constexpr (OP == HIPNX_ADD) return a + b;
+    else if constexpr (OP == HIPNX_SUBTRACT) return a - b;
+    else if constexpr (OP == HIPNX_MULTIPLY) return a * b;
+    else if constexpr (OP == HIPNX_DIVIDE) return a / b;
+    else if constexpr (OP == HIPNX_POW) return pow(a, b);
+    else if constexpr (OP == HIPNX_REMAINDER) return fmod(a, b);
+    else if constexpr (OP == HIPNX_ATAN2) return atan2(a, b);
+    else if constexpr (OP == HIPNX_MAX) return (a != a || b != b) ? (CT)NAN : (b > a ? b : a);
+    else if constexpr (OP == HIPNX_MIN) return (a != a || b != b) ? (CT)NAN : (b < a ? b : a);
+    else if constexpr (OP == HIPNX_EQUAL) return (CT)(a == b);
+    else if constexpr (OP == HIPNX_NOT_EQUAL) return (CT)(a != b);
+    else if constexpr (OP == HIPNX_GREATER) return (CT)(a > b);
+    else if constexpr (OP == HIPNX_LESS) return (CT)(a < b);
+    else if constexpr (OP == HIPNX_GREATER_EQUAL) return (CT)(a >= b);
+    else if constexpr (OP == HIPNX_LESS_EQUAL) return (CT)(a <= b);
+    else if constexpr (OP == HIPNX_LOGICAL_AND) return (CT)((a != 0) && (b != 0));
+    else if constexpr (OP == HIPNX_LOGICAL_OR) return (CT)((a != 0) || (b != 0));
+    else if constexpr (OP == HIPNX_LOGICAL_XOR) return (CT)((a != 0) != (b != 0));
+    else return (CT)0;  // integer-only ops never reach a float class
+  } else {
+    typedef typename std::conditional<UNS, uint64_t, int64_t>::type S;
+    const uint64_t ua = (uint64_t)a, ub = (uint64_t)b;
+    const S sa = (S)a, sb = (S)b;
+    if constexpr (OP == HIPNX_ADD) return (int64_t)(ua + ub);
+    else if constexpr (OP == HIPNX_SUBTRACT) return (int64_t)(ua - ub);
+    else if constexpr (OP == HIPNX_MULTIPLY) return (int64_t)(ua * ub);
+    else if constexpr (OP == HIPNX_POW) return (!UNS && b < 0) ? 0 : ipow_wrap(a, ub);
+    else if constexpr (OP == HIPNX_REMAINDER) {
+      if (sb == 0) return 0;  // the reference raises ArithmeticError
+      if (!UNS && b == -1) return 0;
+      return (int64_t)(sa % sb);
+    } else if constexpr (OP == HIPNX_QUOTIENT) {
+      if (sb == 0) return 0;  // the reference raises ArithmeticError
+      if (!UNS && b == -1) return (int64_t)(0 - ua);
+      return (int64_t)(sa / sb);
+    } else if constexpr (OP == HIPNX_MAX) return sb > sa ? b : a;
+    else if constexpr (OP == HIPNX_MIN) return sb < sa ? b : a;
+    else if constexpr (OP == HIPNX_BITWISE_AND) return a & b;
+    else if constexpr (OP == HIPNX_BITWISE_OR) return a | b;
+    else if constexpr (OP == HIPNX_BITWISE_XOR) return a ^ b;
+    else if constexpr (OP == HIPNX_LEFT_SHIFT) return (b < 0 || b >= 64) ? 0 : (int64_t)(ua << b);
+    else if constexpr (OP == HIPNX_RIGHT_SHIFT) {
+      if (b < 0) return 0;  // the reference raises ArgumentError
+      if (b >= 64) return (!UNS && a < 0) ? -1 : 0;
+      return (int64_t)(sa >> b);
+    } else if constexpr (OP == HIPNX_EQUAL) return a == b;
+    else if constexpr (OP == HIPNX_NOT_EQUAL) return a != b;
+    else if constexpr (OP == HIPNX_GREATER) return sa > sb;
+    else if constexpr (OP == HIPNX_LESS) return sa < sb;
+    else if constexpr (OP == HIPNX_GREATER_EQUAL) return sa >= sb;
+    else if constexpr (OP == HIPNX_LESS_EQUAL) return sa <= sb;
+    else if constexpr (OP == HIPNX_LOGICAL_AND) return (a != 0) && (b != 0);
+    else if constexpr (OP == HIPNX_LOGICAL_OR) return (a != 0) || (b != 0);
+    else if constexpr (OP == HIPNX_LOGICAL_XOR) return (a != 0) != (b != 0);
+    else return 0;  // float-only ops never reach the integer class
+  }
+}
+
+constexpr bool unary_int_only(int op) {
+  return op == HIPNX_BITWISE_NOT || op == HIPNX_CLZ || op == HIPNX_POPCOUNT;
+}
+constexpr bool unary_is_math(int op) { return op <= HIPNX_ERF_INV; }
+
+// nx/lib/nx/shared.ex:311-376 (formulas, e.g. expm1 = exp(x) - 1 and log1p = log(x + 1) exactly
+// as written there) and nx/lib/nx/binary_backend.ex:834-1003.  `bits` is the input width.
+template <int OP, typename CT>
+__device__ __forceinline__ CT unary_apply(CT x, int bits) {
+  if constexpr (is_fp<CT>::value) {
+    if constexpr (OP == HIPNX_EXP) return exp(x);
+    // the cancellation in these three is part of the reference result: follow it in f64
+    else if constexpr (OP == HIPNX_EXPM1) return (CT)(exp((double)x) - 1.0);
+    else if constexpr (OP == HIPNX_LOG1P) return (CT)log((double)x + 1.0);
+    else if constexpr (OP == HIPNX_SIGMOID) return (CT)(1.0 / (exp(-(double)x) + 1.0));
+    else if constexpr (OP == HIPNX_LOG) return log(x);
+    else if constexpr (OP == HIPNX_COS) return cos(x);
+    else if constexpr (OP == HIPNX_SIN) return sin(x);
+    else if constexpr (OP == HIPNX_TAN) return tan(x);
+    else if constexpr (OP == HIPNX_COSH) return cosh(x);
+    else if constexpr (OP == HIPNX_SINH) return sinh(x);
+    else if constexpr (OP == HIPNX_TANH) return tanh(x);
+    else if constexpr (OP == HIPNX_ACOS) return acos(x);
+    else if constexpr (OP == HIPNX_ASIN) return asin(x);
+    else if constexpr (OP == HIPNX_ATAN) return atan(x);
+    else if constexpr (OP == HIPNX_ACOSH) return acosh(x);
+    else if constexpr (OP == HIPNX_ASINH) return asinh(x);
+    else if constexpr (OP == HIPNX_ATANH) return atanh(x);
+    else if constexpr (OP == HIPNX_SQRT) return sqrt(x);
+    else if constexpr (OP == HIPNX_RSQRT) return (CT)1 / sqrt(x);
+    else if constexpr (OP == HIPNX_CBRT) return cbrt(x);
+    else if constexpr (OP == HIPNX_ERF) return erf(x);
+    else if constexpr (OP == HIPNX_ERFC) return erfc(x);
+    else if constexpr (OP == HIPNX_ERF_INV) return erfinv(x);
+    else if constexpr (OP == HIPNX_ABS) return fabs(x);
+    else if constexpr (OP == HIPNX_CEIL) return ceil(x);
+    else if constexpr (OP == HIPNX_FLOOR) return floor(x);
+    else if constexpr (OP == HIPNX_NEGATE) return -x;
+    else if constexpr (OP == HIPNX_ROUND) return round(x);  // half away from zero
+    else if constexpr (OP == HIPNX_SIGN) {
+      // guards `n < 0` / `n > 0` run in Erlang term order, where the atoms :nan, :infinity and
+      // :neg_infinity all sort above every number: each of them yields 1
+      if (x != x || isinf(x)) return (CT)1;
+      return x < 0 ? (CT)-1 : (x > 0 ? (CT)1 : x);
+    } else if constexpr (OP == HIPNX_IS_NAN) return (CT)(x != x);
+    else if constexpr (OP == HIPNX_IS_INFINITY) return (CT)(isinf(x) ? 1 : 0);
+    else return (CT)0;
+  } else {
+    uint64_t u = (uint64_t)x;
+    if (bits < 64) u &= (1ull << bits) - 1;
+    if constexpr (OP == HIPNX_ABS) return x < 0 ? (int64_t)(0 - (uint64_t)x) : x;
+    else if constexpr (OP == HIPNX_NEGATE) return (int64_t)(0 - (uint64_t)x);
+    else if constexpr (OP == HIPNX_BITWISE_NOT) return ~x;
+    else if constexpr (OP == HIPNX_SIGN) return x < 0 ? -1 : (x > 0 ? 1 : 0);
+    else if constexpr (OP == HIPNX_CLZ) return u == 0 ? bits : (int64_t)(__clzll((long long)u) - (64 - bits));
+    else if constexpr (OP == HIPNX_POPCOUNT) return (int64_t)__popcll(u);
+    else if constexpr (OP == HIPNX_CEIL || OP == HIPNX_FLOOR || OP == HIPNX_ROUND) return x;
+    else return 0;  // is_nan / is_infinity of an integer
+  }
+}
+
+// as_type float -> integer (nx/lib/nx/binary_backend.ex:2049-2069): trunc toward zero as an
+// unbounded integer whose low bits are kept; NaN -> 0, +Inf -> max, -Inf -> min of the type.
+__device__ __forceinline__ int64_t float_to_int_wrap(double d, int64_t tmax, int64_t tmin) {
+  if (d != d) return 0;
+  if (isinf(d)) return d > 0 ? tmax : tmin;
+  double t = trunc(d);
+  if (fabs(t) < 9.2e18) return (int64_t)t;
+  double m = fmod(t, 18446744073709551616.0);  // exact, in (-2^64, 2^64)
+  if (m < 0) m += 18446744073709551616.0;     // exact: both are multiples of the same ulp
+  uint64_t u = m >= 9223372036854775808.0 ? ((uint64_t)(m - 9223372036854775808.0) | (1ull << 63)) : (uint64_t)m;
+  return (int64_t)u;
+}
+
+}  // namespace hipnx

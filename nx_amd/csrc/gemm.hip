@@ -1,0 +1,285 @@
+// Nx.dot as a dense batched contraction  out[b, m, n] = sum_k l[b, m, k] * r[b, n, k].
+//
+// MFMA path (bf16 / f16 / f32 operands with f32 accumulation, s8 with s32 accumulation): both
+// operands K-contiguous.  A K-outer operand is first re-laid by the tiled transpose.
+// Everything else (f64, wide integers, mixed operand types) runs on a plain tiled kernel that
+// accumulates in f64 or wrapping 64-bit integers.
+//
+// MFMA kernel.  A 256-lane block (4 wavefronts, 2 x 2) owns a 128 x 128 output tile; each
+// wavefront owns 64 x 64 = 2 x 2 MFMA tiles of 32 x 32.  The K axis is walked in slabs of
+// 128 bytes per row (64 bf16 / 128 s8 / 32 f32).  Slabs are staged through LDS with 16-byte
+// accesses; the 16-byte chunk index is XOR-swizzled with the row so that the 64 lanes of a
+// fragment read hit distinct banks.  For all four element types a lane's MFMA operand
+// fragment for one 32-byte K-step is the 16-byte chunk (2*step + lane/32) of row (lane%32):
+// bf16/f16/s8 feed it to one 32x32x16 / 32x32x32 MFMA; f32 feeds its four floats to four
+// 32x32x2 MFMAs (both operands use the same k <-> slot map, so the sum covers the same 8 k).
+//
+// Algorithmic work: 2*B*M*N*K flop; minimum traffic bytes(l) + bytes(r) + bytes(out).
+#include <type_traits>
+
+#include "dtypes.cuh"
+#include "internal.h"
+
+namespace hipnx {
+
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+
+constexpr int GEMM_BLOCK = 256;
+constexpr int BM = 128, BN = 128;
+constexpr int SLAB = 128;            // bytes of K per row per slab
+constexpr int CHUNKS = SLAB / 16;    // 16-byte chunks per row
+
+template <int DT> struct Mma;
+template <> struct Mma<HIPNX_BF16> {
+  typedef v16f acc_t; typedef float scalar_t;
+  static __device__ __forceinline__ void step(acc_t &c, const v4i &a, const v4i &b) {
+    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
+  }
+};
+template <> struct Mma<HIPNX_F16> {
+  typedef v16f acc_t; typedef float scalar_t;
+  static __device__ __forceinline__ void step(acc_t &c, const v4i &a, const v4i &b) {
+    c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0, 0, 0);
+  }
+};
+template <> struct Mma<HIPNX_S8> {
+  typedef v16i acc_t; typedef int scalar_t;
+  static __device__ __forceinline__ void step(acc_t &c, const v4i &a, const v4i &b) {
+    c = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct Mma<HIPNX_F32> {
+  typedef v16f acc_t; typedef float scalar_t;
+  static __device__ __forceinline__ void step(acc_t &c, const v4i &a, const v4i &b) {
+#pragma unroll
+    for (int s = 0; s < 4; s++)
+      c = __builtin_amdgcn_mfma_f32_32x32x2f32(__int_as_float(a[s]), __int_as_float(b[s]), c, 0, 0, 0);
+  }
+};
+
+// l: [batch, M, Kb bytes], r: [batch, N, Kb bytes]  (Kb = K * element size, multiple of 16)
+template <int DT>
+__global__ void __launch_bounds__(GEMM_BLOCK)
+gemm_kinner_kernel(const unsigned char *__restrict__ l, const unsigned char *__restrict__ r, void *__restrict__ out,
+                   int odt, int64_t M, int64_t N, int64_t Kb, int tiles_m, int tiles_n) {
+  typedef typename Mma<DT>::acc_t acc_t;
+  typedef typename Mma<DT>::scalar_t scalar_t;
+  __shared__ __attribute__((aligned(16))) unsigned char sA[BM * SLAB];
+  __shared__ __attribute__((aligned(16))) unsigned char sB[BN * SLAB];
+
+  const int tile = blockIdx.x;
+  const int tm = tile / tiles_n, tn = tile % tiles_n;
+  const int64_t b = blockIdx.y;
+  const unsigned char *lb = l + b * M * Kb;
+  const unsigned char *rb = r + b * N * Kb;
+  const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+
+  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  const int wm = (wave / 2) * 64, wn = (wave % 2) * 64;
+
+  acc_t acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int q = 0; q < 16; q++) acc[i][j][q] = 0;
+
+  // global -> LDS assignment: 128 rows x 8 chunks = 1024 chunks per operand, 4 per lane
+  const int ld_chunk = tid % CHUNKS;  // 0..7
+  const int ld_row = tid / CHUNKS;    // 0..31, +32 per pass
+
+  for (int64_t k0 = 0; k0 < Kb; k0 += SLAB) {
+    v4i ra[4], rbv[4];
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+      const int row = ld_row + 32 * p;
+      const int64_t kb = k0 + ld_chunk * 16;
+      int64_t gm = m0 + row, gn = n0 + row;
+      gm = gm < M ? gm : M - 1;  // rows past the edge are loaded (clamped) and never stored
+      gn = gn < N ? gn : N - 1;
+      if (kb < Kb) {
+        ra[p] = *reinterpret_cast<const v4i *>(lb + gm * Kb + kb);
+        rbv[p] = *reinterpret_cast<const v4i *>(rb + gn * Kb + kb);
+      } else {
+        ra[p] = v4i{0, 0, 0, 0};  // K tail: zero contributes nothing
+        rbv[p] = v4i{0, 0, 0, 0};
+      }
+    }
+    __syncthreads();  // previous slab fully consumed
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+      const int row = ld_row + 32 * p;
+      const int sw = (ld_chunk ^ (row & 7)) * 16;
+      *reinterpret_cast<v4i *>(sA + row * SLAB + sw) = ra[p];
+      *reinterpret_cast<v4i *>(sB + row * SLAB + sw) = rbv[p];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int ks = 0; ks < SLAB / 32; ks++) {
+      v4i fa[2], fb[2];
+      const int chunk = 2 * ks + lane / 32;
+#pragma unroll
+      for (int i = 0; i < 2; i++) {
+        const int rowa = wm + 32 * i + lane % 32;
+        fa[i] = *reinterpret_cast<const v4i *>(sA + rowa * SLAB + ((chunk ^ (rowa & 7)) * 16));
+        const int rowb = wn + 32 * i + lane % 32;
+        fb[i] = *reinterpret_cast<const v4i *>(sB + rowb * SLAB + ((chunk ^ (rowb & 7)) * 16));
+      }
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) Mma<DT>::step(acc[i][j], fa[i], fb[j]);
+    }
+  }
+
+  // epilogue: D[i][j] of a 32x32 MFMA tile sits in lane (j + 32*((i/4)%2)), register 4*(i/8)+i%4
+  unsigned char *ob = (unsigned char *)out;
+  const int64_t obase = b * M * N;
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int q = 0; q < 16; q++) {
+        const int64_t gm = m0 + wm + 32 * i + 8 * (q / 4) + 4 * (lane / 32) + (q % 4);
+        const int64_t gn = n0 + wn + 32 * j + lane % 32;
+        if (gm < M && gn < N) {
+          if constexpr (DT == HIPNX_S8) store_one<int64_t>(ob, odt, obase + gm * N + gn, (int64_t)(scalar_t)acc[i][j][q]);
+          else store_one<float>(ob, odt, obase + gm * N + gn, (float)acc[i][j][q]);
+        }
+      }
+}
+
+// Plain tiled contraction for every other type combination.  16 x 16 outputs per block, K
+// walked in slabs of 16 through LDS; operands are decoded to CT (double or wrapping int64).
+// lk / rk: 1 when the operand is K-inner ([rows, K]), 0 when K-outer ([K, rows]).
+template <typename CT>
+__global__ void __launch_bounds__(256)
+dot_generic_kernel(const void *__restrict__ l, const void *__restrict__ r, void *__restrict__ out, int ldt, int rdt,
+                   int odt, int64_t M, int64_t N, int64_t K, int lk, int rk) {
+  constexpr int T = 16;
+  __shared__ CT sA[T][T + 1], sB[T][T + 1];
+  const int tx = threadIdx.x % T, ty = threadIdx.x / T;
+  const int64_t b = blockIdx.z;
+  const int64_t m = (int64_t)blockIdx.y * T + ty, n = (int64_t)blockIdx.x * T + tx;
+  const int64_t lbase = b * M * K, rbase = b * N * K;
+  CT acc = 0;
+  for (int64_t k0 = 0; k0 < K; k0 += T) {
+    {  // sA[ty][tx] = l[m, k0 + tx]; sB[ty][tx] = r[n0 + ty, k0 + tx]
+      const int64_t k = k0 + tx;
+      const int64_t mm = (int64_t)blockIdx.y * T + ty, nn = (int64_t)blockIdx.x * T + ty;
+      sA[ty][tx] = (mm < M && k < K) ? load_one<CT>(l, ldt, lbase + (lk ? mm * K + k : k * M + mm)) : (CT)0;
+      sB[ty][tx] = (nn < N && k < K) ? load_one<CT>(r, rdt, rbase + (rk ? nn * K + k : k * N + nn)) : (CT)0;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < T; kk++) {
+      if constexpr (std::is_same<CT, double>::value) acc = sA[ty][kk] * sB[tx][kk] + acc;
+      else acc = (int64_t)((uint64_t)sA[ty][kk] * (uint64_t)sB[tx][kk] + (uint64_t)acc);
+    }
+    __syncthreads();
+  }
+  if (m < M && n < N) store_one<CT>(out, odt, b * M * N + m * N + n, acc);
+}
+
+template <int DT>
+static void launch_mfma(const hipnx_ctx *ctx, const void *l, const void *r, void *out, int odt, int64_t batch,
+                        int64_t M, int64_t N, int64_t Kb) {
+  int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
+  dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)batch);
+  hipLaunchKernelGGL((gemm_kinner_kernel<DT>), grid, dim3(GEMM_BLOCK), 0, ctx->stream, (const unsigned char *)l,
+                     (const unsigned char *)r, out, odt, M, N, Kb, tiles_m, tiles_n);
+}
+
+}  // namespace hipnx
+
+using namespace hipnx;
+
+// defined in move.hip
+extern "C" int hipnx_transpose(hipnx_ctx *ctx, int elem_bytes, int rank, const int64_t *in_dims, const int *perm,
+                               const hipnx_buf *inb, hipnx_buf *out);
+
+extern "C" int hipnx_dot(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batch, int64_t M, int64_t N,
+                         int64_t K, int l_layout, int r_layout, const hipnx_buf *l, const hipnx_buf *r,
+                         hipnx_buf *out) {
+  int64_t Kb = 0;
+  bool mfma = false;
+  {
+    Enter in(ctx);
+    if (in.status) return in.status;
+    if (dtype_size(l_dt) < 0 || dtype_size(r_dt) < 0 || dtype_size(out_dt) < 0)
+      return set_error(HIPNX_EINVAL, "dot: unknown element type");
+    if (batch < 0 || M < 0 || N < 0 || K < 0) return set_error(HIPNX_EINVAL, "dot: negative extent");
+    if ((l_layout != HIPNX_K_INNER && l_layout != HIPNX_K_OUTER) || (r_layout != HIPNX_K_INNER && r_layout != HIPNX_K_OUTER))
+      return set_error(HIPNX_EINVAL, "dot: unknown operand layout");
+    if (int st = check_buf(ctx, l, (uint64_t)batch * M * K * dtype_size(l_dt), "dot lhs")) return st;
+    if (int st = check_buf(ctx, r, (uint64_t)batch * N * K * dtype_size(r_dt), "dot rhs")) return st;
+    if (int st = check_buf(ctx, out, (uint64_t)batch * M * N * dtype_size(out_dt), "dot out")) return st;
+    if (batch * M * N == 0) return HIPNX_OK;
+    if (batch > 65535) return set_error(HIPNX_EUNSUPPORTED, "dot: more than 65535 batch items");
+
+    Kb = K * dtype_size(l_dt);
+    const bool float_pair = l_dt == r_dt && (l_dt == HIPNX_BF16 || l_dt == HIPNX_F16 || l_dt == HIPNX_F32) && is_float(out_dt);
+    const bool int8_pair = l_dt == HIPNX_S8 && r_dt == HIPNX_S8 && !is_float(out_dt) && K <= (1ll << 16);
+    mfma = (float_pair || int8_pair) && K > 0 && Kb % 16 == 0 && M * N >= 256;
+
+    if (!mfma) {
+      const bool any_float = is_float(l_dt) || is_float(r_dt);
+      if (!any_float && is_float(out_dt)) return set_error(HIPNX_EUNSUPPORTED, "dot: integer operands with a float output");
+      dim3 grid((unsigned)((N + 15) / 16), (unsigned)((M + 15) / 16), (unsigned)batch), block(256);
+      if (grid.y > 65535) return set_error(HIPNX_EUNSUPPORTED, "dot: M too large for the generic kernel");
+      const int lk = l_layout == HIPNX_K_INNER, rk = r_layout == HIPNX_K_INNER;
+      if (any_float)
+        hipLaunchKernelGGL((dot_generic_kernel<double>), grid, block, 0, ctx->stream, l->ptr, r->ptr, out->ptr, l_dt, r_dt, out_dt, M, N, K, lk, rk);
+      else
+        hipLaunchKernelGGL((dot_generic_kernel<int64_t>), grid, block, 0, ctx->stream, l->ptr, r->ptr, out->ptr, l_dt, r_dt, out_dt, M, N, K, lk, rk);
+      HIPNX_HIP(hipGetLastError());
+      return HIPNX_OK;
+    }
+  }
+
+  // MFMA path: bring K-outer operands to K-inner through the tiled transpose (pool workspace)
+  const int esz = dtype_size(l_dt);
+  hipnx_buf *lt = nullptr, *rt = nullptr;
+  int st = HIPNX_OK;
+  if (l_layout == HIPNX_K_OUTER) {
+    st = hipnx_buf_alloc(ctx, (size_t)(batch * M * K * esz), &lt);
+    if (!st) {
+      int64_t dims[3] = {batch, K, M};
+      int perm[3] = {0, 2, 1};
+      st = hipnx_transpose(ctx, esz, 3, dims, perm, l, lt);
+    }
+  }
+  if (!st && r_layout == HIPNX_K_OUTER) {
+    st = hipnx_buf_alloc(ctx, (size_t)(batch * N * K * esz), &rt);
+    if (!st) {
+      int64_t dims[3] = {batch, K, N};
+      int perm[3] = {0, 2, 1};
+      st = hipnx_transpose(ctx, esz, 3, dims, perm, r, rt);
+    }
+  }
+  if (!st) {
+    Enter in(ctx);
+    st = in.status;
+    if (!st) {
+      const void *lp = lt ? lt->ptr : l->ptr, *rp = rt ? rt->ptr : r->ptr;
+      switch (l_dt) {
+        case HIPNX_BF16: launch_mfma<HIPNX_BF16>(ctx, lp, rp, out->ptr, out_dt, batch, M, N, Kb); break;
+        case HIPNX_F16: launch_mfma<HIPNX_F16>(ctx, lp, rp, out->ptr, out_dt, batch, M, N, Kb); break;
+        case HIPNX_F32: launch_mfma<HIPNX_F32>(ctx, lp, rp, out->ptr, out_dt, batch, M, N, Kb); break;
+        default: launch_mfma<HIPNX_S8>(ctx, lp, rp, out->ptr, out_dt, batch, M, N, Kb); break;
+      }
+      hipError_t e = hipGetLastError();
+      if (e != hipSuccess) st = hip_fail(e, "gemm launch");
+    }
+  }
+  // handing the workspaces back to the pool is safe: later work is ordered on the same stream
+  if (lt) hipnx_buf_destroy(lt);
+  if (rt) hipnx_buf_destroy(rt);
+  return st;
+}

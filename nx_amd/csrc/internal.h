@@ -1,0 +1,72 @@
+// Host-side internals of libhipnx: context, buffer handles, argument checks.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <map>
+#include <mutex>
+#include <vector>
+
+#include "../../include/hipnx.h"
+
+struct hipnx_ctx {
+  int device = 0;
+  hipStream_t stream = nullptr;
+  hipEvent_t ev_start = nullptr, ev_stop = nullptr;
+  std::mutex mu;  // serialises enqueueing and the pool
+  // size-bucketed cache of freed device blocks; reuse is safe without a device wait because
+  // every kernel of this context runs on the one stream, in order
+  std::multimap<size_t, void *> pool;
+  uint64_t live = 0, peak = 0, pooled = 0;
+  int num_cus = 256;
+  void *flag = nullptr;       // 32-byte device scratch for the gather bounds report
+  void *flag_host = nullptr;  // pinned mirror
+};
+
+struct hipnx_buf {
+  hipnx_ctx *ctx = nullptr;
+  void *ptr = nullptr;
+  size_t bytes = 0;     // what the caller asked for
+  size_t capacity = 0;  // what the pool block holds
+  std::atomic<int> freed{0};
+};
+
+namespace hipnx {
+
+int set_error(int code, const char *fmt, ...);
+int hip_fail(hipError_t e, const char *what);
+
+#define HIPNX_HIP(call)                                         \
+  do {                                                          \
+    hipError_t e__ = (call);                                    \
+    if (e__ != hipSuccess) return hipnx::hip_fail(e__, #call);  \
+  } while (0)
+
+inline int dtype_size(int dt) {
+  static const int sz[HIPNX_NTYPES] = {1, 2, 4, 8, 1, 2, 4, 8, 2, 2, 4, 8};
+  return (dt >= 0 && dt < HIPNX_NTYPES) ? sz[dt] : -1;
+}
+inline bool is_float(int dt) { return dt >= HIPNX_F16; }
+inline bool is_unsigned(int dt) { return dt >= 0 && dt <= HIPNX_U64; }
+inline bool is_wide(int dt) {  // not exactly representable in f32
+  return dt == HIPNX_U32 || dt == HIPNX_U64 || dt == HIPNX_S32 || dt == HIPNX_S64 || dt == HIPNX_F64;
+}
+
+// operand checks shared by every entry point: live handle, same context, enough bytes
+int check_buf(const hipnx_ctx *ctx, const hipnx_buf *b, uint64_t need_bytes, const char *name);
+
+// pooled device memory; both expect the context mutex to be held (i.e. inside an Enter scope)
+int pool_alloc(hipnx_ctx *ctx, size_t bytes, void **ptr_out, size_t *cap_out);
+int pool_free(hipnx_ctx *ctx, void *ptr, size_t cap);
+
+// RAII: select the device and take the context mutex for the duration of an entry point
+struct Enter {
+  std::unique_lock<std::mutex> lk;
+  int status;
+  explicit Enter(hipnx_ctx *ctx);
+};
+
+}  // namespace hipnx

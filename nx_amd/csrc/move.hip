@@ -1,0 +1,335 @@
+// Data movement: fill (constant), transpose, broadcast, gather / take.  Pure byte copies -- the
+// bit patterns of the source survive unchanged (NaN payloads included), as in the reference,
+// where these callbacks only slice and concatenate binaries
+// (nx/lib/nx/binary_backend.ex:215-319, 1902-1959).
+#include <cstring>
+
+#include "dtypes.cuh"
+#include "internal.h"
+
+namespace hipnx {
+
+constexpr int BLOCK = 256;
+constexpr int MAXR = 8;
+
+template <typename T>
+__global__ void __launch_bounds__(BLOCK) fill_kernel(T *__restrict__ out, T value, int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x; i < n; i += (int64_t)gridDim.x * BLOCK) out[i] = value;
+}
+
+struct Strided {
+  int rank;
+  int64_t dims[MAXR];     // output extents
+  int64_t strides[MAXR];  // input stride (elements) per output axis
+};
+
+// out[i] = in[sum c_a * stride_a]; one element per lane per step
+template <typename T>
+__global__ void __launch_bounds__(BLOCK)
+strided_copy_kernel(const T *__restrict__ in, T *__restrict__ out, int64_t n, Strided s) {
+  for (int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x; i < n; i += (int64_t)gridDim.x * BLOCK) {
+    int64_t rem = i, off = 0;
+    for (int a = s.rank - 1; a >= 0; a--) {
+      int64_t q = rem / s.dims[a];
+      off += (rem - q * s.dims[a]) * s.strides[a];
+      rem = q;
+    }
+    out[i] = in[off];
+  }
+}
+
+// batched 2-D transpose through an LDS tile: in [B, R, C] -> out [B, C, R].  The 64x64 tile is
+// read with lanes along C and written with lanes along R, so both sides are coalesced; the
+// +1 padding keeps the transposed LDS reads off a single bank.
+template <typename T>
+__global__ void __launch_bounds__(BLOCK)
+transpose2d_kernel(const T *__restrict__ in, T *__restrict__ out, int64_t R, int64_t C, int64_t tiles_r,
+                   int64_t tiles_c) {
+  constexpr int TILE = 64;
+  __shared__ T tile[TILE][TILE + 1];
+  int64_t t = blockIdx.x;
+  const int64_t tc = t % tiles_c;
+  t /= tiles_c;
+  const int64_t tr = t % tiles_r, b = t / tiles_r;
+  const T *src = in + b * R * C;
+  T *dst = out + b * R * C;
+  const int tx = threadIdx.x % TILE, ty = threadIdx.x / TILE;  // 64 x 4
+  for (int j = ty; j < TILE; j += BLOCK / TILE) {
+    int64_t r = tr * TILE + j, c = tc * TILE + tx;
+    if (r < R && c < C) tile[j][tx] = src[r * C + c];
+  }
+  __syncthreads();
+  for (int j = ty; j < TILE; j += BLOCK / TILE) {
+    int64_t c = tc * TILE + j, r = tr * TILE + tx;
+    if (r < R && c < C) dst[c * R + r] = tile[tx][j];
+  }
+}
+
+// gather: tuple i of `idx` ([n_tuples, depth]) selects a slice of `slice_bytes` bytes.
+// One block-row of lanes copies a slice with 16-byte (VEC) or 1-byte accesses.
+// flag[0] receives the smallest (tuple * depth + axis) whose index is out of range.
+template <bool VEC>
+__global__ void __launch_bounds__(BLOCK)
+gather_kernel(const unsigned char *__restrict__ t, const void *__restrict__ idx, unsigned char *__restrict__ out,
+              int idx_dt, int64_t n_tuples, int depth, Strided tdims /* dims = leading extents, strides = bytes */,
+              int64_t slice_bytes, int clamp, unsigned long long *__restrict__ flag) {
+  constexpr int W = VEC ? 16 : 1;
+  const int64_t chunks = slice_bytes / W;
+  // lanes_per_row: enough lanes to cover a slice, at most the block
+  int lpr = BLOCK;
+  while (lpr > 1 && lpr / 2 >= chunks) lpr >>= 1;
+  const int rpb = BLOCK / lpr;
+  const int sub = threadIdx.x / lpr, lane = threadIdx.x % lpr;
+  for (int64_t row = (int64_t)blockIdx.x * rpb + sub; row < n_tuples; row += (int64_t)gridDim.x * rpb) {
+    int64_t off = 0;
+    bool ok = true;
+    for (int a = 0; a < depth; a++) {
+      int64_t v = load_one<int64_t>(idx, idx_dt, row * depth + a);
+      const int64_t dim = tdims.dims[a];
+      bool oob = v < 0 || v >= dim || (idx_dt == HIPNX_U64 && (uint64_t)v >= (uint64_t)dim);
+      if (oob) {
+        if (clamp) v = (v < 0 && idx_dt != HIPNX_U64) ? 0 : dim - 1;
+        else {
+          ok = false;
+          if (lane == 0) atomicMin(flag, (unsigned long long)(row * depth + a));
+          break;
+        }
+      }
+      off += v * tdims.strides[a];
+    }
+    if (!ok) continue;
+    const unsigned char *src = t + off;
+    unsigned char *dst = out + row * slice_bytes;
+    for (int64_t c = lane; c < chunks; c += lpr)
+      *reinterpret_cast<raw_vec<W> *>(dst + c * W) = *reinterpret_cast<const raw_vec<W> *>(src + c * W);
+  }
+}
+
+static int grid_for(const hipnx_ctx *ctx, int64_t items, int per_block) {
+  int64_t blocks = (items + per_block - 1) / per_block;
+  int64_t cap = (int64_t)ctx->num_cus * 16;
+  if (blocks < 1) blocks = 1;
+  return (int)(blocks < cap ? blocks : cap);
+}
+
+template <typename T>
+static void launch_strided(const hipnx_ctx *ctx, const void *in, void *out, int64_t n, const Strided &s) {
+  hipLaunchKernelGGL((strided_copy_kernel<T>), dim3(grid_for(ctx, n, BLOCK)), dim3(BLOCK), 0, ctx->stream,
+                     (const T *)in, (T *)out, n, s);
+}
+
+static int strided_copy(const hipnx_ctx *ctx, int elem_bytes, const void *in, void *out, int64_t n, const Strided &s) {
+  switch (elem_bytes) {
+    case 1: launch_strided<uint8_t>(ctx, in, out, n, s); break;
+    case 2: launch_strided<uint16_t>(ctx, in, out, n, s); break;
+    case 4: launch_strided<uint32_t>(ctx, in, out, n, s); break;
+    case 8: launch_strided<uint64_t>(ctx, in, out, n, s); break;
+    default: return set_error(HIPNX_EINVAL, "element size %d is not 1, 2, 4 or 8", elem_bytes);
+  }
+  return HIPNX_OK;
+}
+
+template <typename T>
+static void launch_t2d(const hipnx_ctx *ctx, const void *in, void *out, int64_t B, int64_t R, int64_t C) {
+  int64_t tr = (R + 63) / 64, tc = (C + 63) / 64;
+  hipLaunchKernelGGL((transpose2d_kernel<T>), dim3((unsigned)(B * tr * tc)), dim3(BLOCK), 0, ctx->stream,
+                     (const T *)in, (T *)out, R, C, tr, tc);
+}
+
+}  // namespace hipnx
+
+using namespace hipnx;
+
+extern "C" int hipnx_fill(hipnx_ctx *ctx, hipnx_buf *dst, int elem_bytes, const void *elem, int64_t n) {
+  Enter in(ctx);
+  if (in.status) return in.status;
+  if (!elem || n < 0) return set_error(HIPNX_EINVAL, "fill: null element or negative count");
+  if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4 && elem_bytes != 8)
+    return set_error(HIPNX_EINVAL, "fill: element size %d is not 1, 2, 4 or 8", elem_bytes);
+  if (int st = check_buf(ctx, dst, (uint64_t)n * elem_bytes, "fill dst")) return st;
+  if (n == 0) return HIPNX_OK;
+  dim3 grid(grid_for(ctx, n, BLOCK)), block(BLOCK);
+  switch (elem_bytes) {
+    case 1: hipLaunchKernelGGL((fill_kernel<uint8_t>), grid, block, 0, ctx->stream, (uint8_t *)dst->ptr, *(const uint8_t *)elem, n); break;
+    case 2: { uint16_t v; std::memcpy(&v, elem, 2); hipLaunchKernelGGL((fill_kernel<uint16_t>), grid, block, 0, ctx->stream, (uint16_t *)dst->ptr, v, n); break; }
+    case 4: { uint32_t v; std::memcpy(&v, elem, 4); hipLaunchKernelGGL((fill_kernel<uint32_t>), grid, block, 0, ctx->stream, (uint32_t *)dst->ptr, v, n); break; }
+    default: { uint64_t v; std::memcpy(&v, elem, 8); hipLaunchKernelGGL((fill_kernel<uint64_t>), grid, block, 0, ctx->stream, (uint64_t *)dst->ptr, v, n); break; }
+  }
+  HIPNX_HIP(hipGetLastError());
+  return HIPNX_OK;
+}
+
+extern "C" int hipnx_transpose(hipnx_ctx *ctx, int elem_bytes, int rank, const int64_t *in_dims, const int *perm,
+                               const hipnx_buf *inb, hipnx_buf *out) {
+  Enter in(ctx);
+  if (in.status) return in.status;
+  if (rank < 0 || rank > 64 || (rank > 0 && (!in_dims || !perm))) return set_error(HIPNX_EINVAL, "transpose: bad rank");
+  if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4 && elem_bytes != 8)
+    return set_error(HIPNX_EINVAL, "transpose: element size %d is not 1, 2, 4 or 8", elem_bytes);
+  int64_t n = 1;
+  uint64_t seen = 0;
+  for (int a = 0; a < rank; a++) {
+    if (in_dims[a] < 0) return set_error(HIPNX_EINVAL, "transpose: negative dimension");
+    if (perm[a] < 0 || perm[a] >= rank || (seen >> perm[a] & 1)) return set_error(HIPNX_EINVAL, "transpose: not a permutation");
+    seen |= 1ull << perm[a];
+    n *= in_dims[a];
+  }
+  if (int st = check_buf(ctx, inb, (uint64_t)n * elem_bytes, "transpose in")) return st;
+  if (int st = check_buf(ctx, out, (uint64_t)n * elem_bytes, "transpose out")) return st;
+  if (n == 0) return HIPNX_OK;
+  // input strides, then walk the output axes: drop unit axes, merge output neighbours that are
+  // also neighbours (in order) in the input
+  int64_t in_str[64];
+  int64_t s = 1;
+  for (int a = rank - 1; a >= 0; a--) { in_str[a] = s; s *= in_dims[a]; }
+  int64_t dims[64], str[64];
+  int m = 0;
+  for (int a = 0; a < rank; a++) {
+    int64_t d = in_dims[perm[a]], st = in_str[perm[a]];
+    if (d == 1) continue;
+    if (m > 0 && str[m - 1] == st * d) { dims[m - 1] *= d; str[m - 1] = st; }
+    else { dims[m] = d; str[m] = st; m++; }
+  }
+  if (m <= 1) {  // the permutation moves nothing in memory
+    HIPNX_HIP(hipMemcpyAsync(out->ptr, inb->ptr, (size_t)n * elem_bytes, hipMemcpyDeviceToDevice, ctx->stream));
+    return HIPNX_OK;
+  }
+  // [B, R, C] -> [B, C, R] : out axes (B?, C, R) with strides (R*C, 1, C)
+  bool two_d = (m == 2 && str[0] == 1 && str[1] == dims[0]) ||
+               (m == 3 && str[1] == 1 && str[2] == dims[1] && str[0] == dims[1] * dims[2]);
+  if (two_d) {
+    int64_t B = m == 3 ? dims[0] : 1, C = dims[m - 2], R = dims[m - 1];
+    if (B * ((R + 63) / 64) * ((C + 63) / 64) < (1ll << 31)) {
+      switch (elem_bytes) {
+        case 1: launch_t2d<uint8_t>(ctx, inb->ptr, out->ptr, B, R, C); break;
+        case 2: launch_t2d<uint16_t>(ctx, inb->ptr, out->ptr, B, R, C); break;
+        case 4: launch_t2d<uint32_t>(ctx, inb->ptr, out->ptr, B, R, C); break;
+        default: launch_t2d<uint64_t>(ctx, inb->ptr, out->ptr, B, R, C); break;
+      }
+      HIPNX_HIP(hipGetLastError());
+      return HIPNX_OK;
+    }
+  }
+  if (m > MAXR) return set_error(HIPNX_EUNSUPPORTED, "transpose: more than %d non-collapsible axes", MAXR);
+  Strided sd;
+  sd.rank = m;
+  for (int q = 0; q < m; q++) { sd.dims[q] = dims[q]; sd.strides[q] = str[q]; }
+  if (int st = strided_copy(ctx, elem_bytes, inb->ptr, out->ptr, n, sd)) return st;
+  HIPNX_HIP(hipGetLastError());
+  return HIPNX_OK;
+}
+
+extern "C" int hipnx_broadcast(hipnx_ctx *ctx, int elem_bytes, int rank, const int64_t *out_dims,
+                               const int64_t *in_strides, const hipnx_buf *inb, hipnx_buf *out) {
+  Enter in(ctx);
+  if (in.status) return in.status;
+  if (rank < 0 || rank > 64 || (rank > 0 && (!out_dims || !in_strides))) return set_error(HIPNX_EINVAL, "broadcast: bad rank");
+  int64_t n = 1, ext = 1;
+  for (int a = 0; a < rank; a++) {
+    if (out_dims[a] < 0 || in_strides[a] < 0) return set_error(HIPNX_EINVAL, "broadcast: negative dimension or stride");
+    n *= out_dims[a];
+  }
+  if (n > 0)
+    for (int a = 0; a < rank; a++) ext += (out_dims[a] - 1) * in_strides[a];
+  if (int st = check_buf(ctx, inb, n > 0 ? (uint64_t)ext * elem_bytes : 0, "broadcast in")) return st;
+  if (int st = check_buf(ctx, out, (uint64_t)n * elem_bytes, "broadcast out")) return st;
+  if (n == 0) return HIPNX_OK;
+  int64_t dims[64], str[64];
+  int m = 0;
+  for (int a = 0; a < rank; a++) {
+    int64_t d = out_dims[a], st = in_strides[a];
+    if (d == 1) continue;
+    if (m > 0 && str[m - 1] == st * d) { dims[m - 1] *= d; str[m - 1] = st; }
+    else { dims[m] = d; str[m] = st; m++; }
+  }
+  if (m == 0) { dims[0] = 1; str[0] = 0; m = 1; }
+  if (m > MAXR) return set_error(HIPNX_EUNSUPPORTED, "broadcast: more than %d non-collapsible axes", MAXR);
+  Strided sd;
+  sd.rank = m;
+  for (int q = 0; q < m; q++) { sd.dims[q] = dims[q]; sd.strides[q] = str[q]; }
+  if (int st = strided_copy(ctx, elem_bytes, inb->ptr, out->ptr, n, sd)) return st;
+  HIPNX_HIP(hipGetLastError());
+  return HIPNX_OK;
+}
+
+extern "C" int hipnx_gather(hipnx_ctx *ctx, int elem_bytes, int rank, const int64_t *t_dims, int idx_dt,
+                            int64_t n_tuples, int depth, int oob_policy, const hipnx_buf *t, const hipnx_buf *idx,
+                            hipnx_buf *out) {
+  Enter in(ctx);
+  if (in.status) return in.status;
+  if (rank < 0 || rank > 64 || depth < 0 || depth > rank || depth > MAXR || n_tuples < 0 || (rank > 0 && !t_dims))
+    return set_error(HIPNX_EINVAL, "gather: bad rank / depth");
+  if (elem_bytes <= 0 || dtype_size(idx_dt) < 0 || is_float(idx_dt))
+    return set_error(HIPNX_EINVAL, "gather: indices must be an integer type");
+  if (oob_policy != HIPNX_OOB_RAISE && oob_policy != HIPNX_OOB_CLAMP) return set_error(HIPNX_EINVAL, "gather: bad policy");
+  int64_t total = 1, slice = 1;
+  for (int a = 0; a < rank; a++) {
+    if (t_dims[a] < 0) return set_error(HIPNX_EINVAL, "gather: negative dimension");
+    total *= t_dims[a];
+    if (a >= depth) slice *= t_dims[a];
+  }
+  const int64_t slice_bytes = slice * elem_bytes;
+  if (int st = check_buf(ctx, t, (uint64_t)total * elem_bytes, "gather tensor")) return st;
+  if (int st = check_buf(ctx, idx, (uint64_t)n_tuples * depth * dtype_size(idx_dt), "gather indices")) return st;
+  if (int st = check_buf(ctx, out, (uint64_t)n_tuples * slice_bytes, "gather out")) return st;
+  if (n_tuples == 0 || slice_bytes == 0) return HIPNX_OK;
+  if (total == 0) {
+    if (oob_policy == HIPNX_OOB_CLAMP) return set_error(HIPNX_EINVAL, "gather: cannot clamp into an empty tensor");
+    return set_error(HIPNX_EINDEX, "gather: index into an empty tensor");
+  }
+  Strided td;
+  td.rank = depth;
+  {
+    int64_t s = slice_bytes;
+    for (int a = depth - 1; a >= 0; a--) { td.dims[a] = t_dims[a]; td.strides[a] = s; s *= t_dims[a]; }
+  }
+  unsigned long long *flag = (unsigned long long *)ctx->flag;
+  if (oob_policy == HIPNX_OOB_RAISE)
+    hipLaunchKernelGGL((fill_kernel<unsigned long long>), dim3(1), dim3(BLOCK), 0, ctx->stream, flag, ~0ull, (int64_t)1);
+  const bool vec = slice_bytes % 16 == 0;
+  int64_t chunks = vec ? slice_bytes / 16 : slice_bytes;
+  int lpr = BLOCK;
+  while (lpr > 1 && lpr / 2 >= chunks) lpr >>= 1;
+  dim3 grid(grid_for(ctx, n_tuples, BLOCK / lpr)), block(BLOCK);
+  if (vec)
+    hipLaunchKernelGGL((gather_kernel<true>), grid, block, 0, ctx->stream, (const unsigned char *)t->ptr, idx->ptr,
+                       (unsigned char *)out->ptr, idx_dt, n_tuples, depth, td, slice_bytes, (int)(oob_policy == HIPNX_OOB_CLAMP), flag);
+  else
+    hipLaunchKernelGGL((gather_kernel<false>), grid, block, 0, ctx->stream, (const unsigned char *)t->ptr, idx->ptr,
+                       (unsigned char *)out->ptr, idx_dt, n_tuples, depth, td, slice_bytes, (int)(oob_policy == HIPNX_OOB_CLAMP), flag);
+  HIPNX_HIP(hipGetLastError());
+  if (oob_policy == HIPNX_OOB_RAISE) {
+    // the reference raises on the first offending index: wait, then report it the same way
+    unsigned long long *host = (unsigned long long *)ctx->flag_host;
+    HIPNX_HIP(hipMemcpyAsync(host, flag, 8, hipMemcpyDeviceToHost, ctx->stream));
+    HIPNX_HIP(hipStreamSynchronize(ctx->stream));
+    if (host[0] != ~0ull) {
+      const int64_t pos = (int64_t)host[0];
+      const int axis = (int)(pos % depth);
+      unsigned char raw[8] = {0};
+      const int isz = dtype_size(idx_dt);
+      HIPNX_HIP(hipMemcpy(raw, (const char *)idx->ptr + pos * isz, isz, hipMemcpyDeviceToHost));
+      long long v = 0;
+      switch (idx_dt) {
+        case HIPNX_U8: v = *(uint8_t *)raw; break;
+        case HIPNX_U16: { uint16_t x; std::memcpy(&x, raw, 2); v = x; break; }
+        case HIPNX_U32: { uint32_t x; std::memcpy(&x, raw, 4); v = x; break; }
+        case HIPNX_S8: v = *(int8_t *)raw; break;
+        case HIPNX_S16: { int16_t x; std::memcpy(&x, raw, 2); v = x; break; }
+        case HIPNX_S32: { int32_t x; std::memcpy(&x, raw, 4); v = x; break; }
+        default: { int64_t x; std::memcpy(&x, raw, 8); v = x; break; }
+      }
+      char shape[256] = "{";
+      for (int q = 0; q < rank; q++) {
+        char one[32];
+        snprintf(one, sizeof one, q ? ", %lld" : "%lld", (long long)t_dims[q]);
+        strncat(shape, one, sizeof shape - strlen(shape) - 2);
+      }
+      strcat(shape, "}");
+      if (idx_dt == HIPNX_U64)
+        return set_error(HIPNX_EINDEX, "index %llu is out of bounds for axis %d in shape %s", (unsigned long long)v, axis, shape);
+      return set_error(HIPNX_EINDEX, "index %lld is out of bounds for axis %d in shape %s", v, axis, shape);
+    }
+  }
+  return HIPNX_OK;
+}

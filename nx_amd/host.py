@@ -1,0 +1,83 @@
+"""HostBinary -- a tensor that is just bytes in host memory.
+
+It plays the part `Nx.BinaryBackend` plays for the *plumbing* of the reference (it is the backend
+`Nx.tensor/2` builds literals and scalar constants on when no other default is set,
+nx/lib/nx.ex:849-883, 2152-2157) and nothing more: it stores, returns and transfers a binary.
+Every compute callback raises, like the reference's own storage-only test backend
+(nx/test/support/backends.ex).  When a HostBinary tensor meets a device tensor in an operation
+the device backend wins the dispatch and copies it in (nx/lib/nx/shared.ex:449-473).
+"""
+from __future__ import annotations
+
+from . import types as T
+from .tensor import Tensor, number_to_binary
+
+
+class HostBinary:
+    def __init__(self, state: bytes):
+        self.state = state
+        self.released = False
+
+    @staticmethod
+    def init(opts):
+        if opts:
+            raise ValueError("HostBinary accepts no options")
+        return {}
+
+    @classmethod
+    def from_binary(cls, out: Tensor, binary, opts=None) -> Tensor:
+        need = out.size * T.size_bytes(out.type)
+        if len(binary) < need:
+            raise ValueError("binary size is too small for the requested shape")
+        return out.with_(data=cls(bytes(binary[:need])))
+
+    @classmethod
+    def constant(cls, out: Tensor, number, opts=None) -> Tensor:
+        return out.with_(data=cls(number_to_binary(number, out.type) * out.size))
+
+    @classmethod
+    def to_binary(cls, t: Tensor, limit: int) -> bytes:
+        if t.data.released:
+            raise RuntimeError("tensor has been deallocated")
+        return t.data.state[: min(int(limit), t.size) * T.size_bytes(t.type)]
+
+    @classmethod
+    def backend_copy(cls, t: Tensor, backend, opts=None) -> Tensor:
+        return backend.from_binary(t, cls.to_binary(t, t.size), opts)
+
+    @classmethod
+    def backend_transfer(cls, t: Tensor, backend, opts=None) -> Tensor:
+        if backend is HostBinary:
+            return t
+        res = cls.backend_copy(t, backend, opts)
+        cls.backend_deallocate(t)
+        return res
+
+    @classmethod
+    def backend_deallocate(cls, t: Tensor) -> str:
+        if t.data.released:
+            return "already_deallocated"
+        t.data.released = True
+        t.data.state = b""
+        return "ok"
+
+    @classmethod
+    def reshape(cls, out, t):
+        return out.with_(data=t.data)
+
+    squeeze = classmethod(lambda cls, out, t, axes: out.with_(data=t.data))
+    bitcast = classmethod(lambda cls, out, t: out.with_(data=t.data))
+
+    def __getattr__(self, name):
+        raise AttributeError(name)
+
+
+def _raise(name):
+    def fn(cls, *a, **k):
+        raise NotImplementedError(f"HostBinary only stores data; {name} needs a compute backend")
+    return classmethod(fn)
+
+
+for _n in ["add", "subtract", "multiply", "divide", "exp", "sum", "reduce_max", "reduce_min", "argmax", "argmin",
+           "dot", "gather", "transpose", "broadcast", "as_type", "block"]:
+    setattr(HostBinary, _n, _raise(_n))

@@ -1,0 +1,426 @@
+"""The slice of the `Nx` front end that sits above the device path (reference: nx/lib/nx.ex).
+
+Each function does what its namesake does before it reaches a backend: converts numbers to
+tensors, infers the output type and shape, builds the output template and dispatches to the
+backend chosen from the operands (`impl!/1,2`, nx/lib/nx/shared.ex:449-473).  It exists so that
+callers -- and the parity tests, which read like the reference's own -- can switch backend and
+run unchanged.  Vectorisation and axis names are not modelled.
+"""
+from __future__ import annotations
+
+import threading
+from dataclasses import dataclass
+from math import prod
+
+import numpy as np
+
+from . import shape as S
+from . import types as T
+from .host import HostBinary
+from .tensor import Tensor, binary_to_numpy, list_to_binary, template, to_float64
+
+_state = threading.local()
+_global_default = [(HostBinary, {})]
+
+
+def default_backend(backend=None, opts=None):
+    """Nx.default_backend/0,1 (nx.ex:5006-5049): per-thread override, `init/1` validates opts."""
+    if backend is None:
+        return getattr(_state, "backend", None) or _global_default[0]
+    previous = default_backend()
+    _state.backend = (backend, backend.init(opts or {}))
+    return previous
+
+
+def global_default_backend(backend, opts=None):
+    previous = _global_default[0]
+    _global_default[0] = (backend, backend.init(opts or {}))
+    return previous
+
+
+def _impl(*tensors):
+    """impl!/1,2 (shared.ex:449-473): HostBinary loses to any other backend; two different
+    compute backends cannot be mixed."""
+    chosen = None
+    for t in tensors:
+        b = type(t.data)
+        if b is HostBinary:
+            continue
+        if chosen is None:
+            chosen = b
+        elif chosen is not b:
+            raise ValueError(f"cannot invoke Nx function because it relies on two incompatible tensor "
+                             f"implementations: {chosen.__name__} and {b.__name__}")
+    return chosen or HostBinary
+
+
+# ---- creation / conversion ---------------------------------------------------------------
+
+def _infer_list_type(arr: np.ndarray):
+    return ("f", 32) if arr.dtype.kind == "f" else ("u", 8) if arr.dtype.kind == "b" else ("s", 32)
+
+
+def tensor(value, type=None, backend=None) -> Tensor:
+    """Nx.tensor/2 (nx.ex:774-883): nested lists / numbers -> tensor on the default backend."""
+    if isinstance(value, Tensor):
+        return value if type is None else as_type(value, type)
+    if isinstance(value, np.ndarray) and value.dtype.kind in "iuf" and type is None and value.dtype != np.float16:
+        arr = value
+        ty = {"i": "s", "u": "u", "f": "f"}[arr.dtype.kind], arr.dtype.itemsize * 8
+        binary = np.ascontiguousarray(arr).tobytes()
+    else:
+        arr = np.asarray(value)
+        if arr.dtype == object:
+            arr = np.asarray(value, dtype=np.float64)
+        ty = T.normalize(type) if type is not None else _infer_list_type(arr)
+        binary = list_to_binary(arr, ty)
+    mod, opts = (backend, {}) if backend is not None and not isinstance(backend, tuple) else (backend or default_backend())
+    return mod.from_binary(template(ty, arr.shape), binary, opts)
+
+
+def from_binary(binary, type, backend=None) -> Tensor:
+    """Nx.from_binary/3 (nx.ex:2051-2066): a flat tensor over the bytes."""
+    ty = T.normalize(type)
+    size = T.size_bytes(ty)
+    if len(binary) == 0 or len(binary) % size:
+        raise ValueError("binary has incompatible number of bits, expected a multiple of the type size")
+    mod, opts = (backend, {}) if backend is not None and not isinstance(backend, tuple) else (backend or default_backend())
+    return mod.from_binary(template(ty, (len(binary) // size,)), binary, opts)
+
+
+def to_tensor(value) -> Tensor:
+    """Nx.to_tensor/1 (nx.ex:2149-2157): numbers become rank-0 constants on the default backend."""
+    if isinstance(value, Tensor):
+        return value
+    if isinstance(value, (bool, int, float, np.integer, np.floating)):
+        mod, opts = default_backend()
+        v = value.item() if isinstance(value, np.generic) else value
+        return mod.constant(template(T.infer(v), ()), v, opts)
+    return tensor(value)
+
+
+def to_binary(t: Tensor, limit=None) -> bytes:
+    """Nx.to_binary/2 (nx.ex:2121-2133); `limit` counts elements."""
+    limit = t.size if limit is None else min(limit, t.size)
+    return type(t.data).to_binary(t, limit)
+
+
+def to_numpy(t: Tensor) -> np.ndarray:
+    """Raw element array (bf16 as uint16 bit patterns)."""
+    return binary_to_numpy(to_binary(t), t.type, t.shape).copy()
+
+
+def to_float64(t: Tensor) -> np.ndarray:
+    from .tensor import to_float64 as f
+    return f(to_binary(t), t.type, t.shape)
+
+
+def to_flat_list(t: Tensor):
+    return to_float64(t).ravel().tolist() if T.is_float(t.type) else to_numpy(t).ravel().tolist()
+
+
+def backend_copy(t: Tensor, backend=None, opts=None) -> Tensor:
+    mod, o = (backend, opts or {}) if backend is not None else default_backend()
+    return type(t.data).backend_copy(t, mod, o)
+
+
+def backend_transfer(t: Tensor, backend=None, opts=None) -> Tensor:
+    mod, o = (backend, opts or {}) if backend is not None else default_backend()
+    return type(t.data).backend_transfer(t, mod, o)
+
+
+def backend_deallocate(t: Tensor) -> str:
+    return type(t.data).backend_deallocate(t)
+
+
+def shape(t) -> tuple:
+    return to_tensor(t).shape
+
+
+def type_of(t):
+    return to_tensor(t).type
+
+
+# ---- element-wise ------------------------------------------------------------------------
+
+_ARITH = ["add", "subtract", "multiply", "pow", "remainder", "min", "max"]
+_INT_ONLY = ["quotient", "bitwise_and", "bitwise_or", "bitwise_xor", "left_shift", "right_shift"]
+_FLOAT_OUT = ["divide", "atan2"]
+_PRED = ["equal", "not_equal", "greater", "less", "greater_equal", "less_equal", "logical_and", "logical_or",
+         "logical_xor"]
+
+
+def _number_or_type(x):
+    return x if isinstance(x, (int, float)) and not isinstance(x, bool) else to_tensor(x).type
+
+
+def _binary(name, left, right, out_type_fun):
+    ty = T.binary_type(_number_or_type(left), _number_or_type(right))
+    l, r = to_tensor(left), to_tensor(right)
+    out = template(out_type_fun(ty), S.binary_broadcast(l.shape, r.shape))
+    return getattr(_impl(l, r), name)(out, l, r)
+
+
+def _def_binary():
+    g = globals()
+    for name in _ARITH:
+        g[name] = (lambda n: lambda left, right: _binary(n, left, right, lambda ty: ty))(name)
+    for name in _INT_ONLY:
+        def int_only(left, right, _n=name):
+            def check(ty):
+                if not T.is_integer(ty):
+                    raise ValueError(f"{_n} expects integer tensors as inputs and outputs an integer tensor, "
+                                     f"got: {ty!r}")
+                return ty
+            return _binary(_n, left, right, check)
+        g[name] = int_only
+    for name in _FLOAT_OUT:  # element_wise_bin_op with to_floating (nx.ex:6544, 6639)
+        g[name] = (lambda n: lambda left, right: _binary(n, left, right, T.to_floating))(name)
+    for name in _PRED:  # element_wise_pred_op: u8 output (nx.ex:6037-6050)
+        g[name] = (lambda n: lambda left, right: _binary(n, left, right, lambda ty: ("u", 8)))(name)
+
+
+_def_binary()
+
+_MATH = ["exp", "expm1", "log", "log1p", "sigmoid", "cos", "sin", "tan", "cosh", "sinh", "tanh", "acos", "asin",
+         "atan", "acosh", "asinh", "atanh", "sqrt", "rsqrt", "cbrt", "erf", "erfc", "erf_inv"]
+
+
+def _def_unary():
+    g = globals()
+    for name in _MATH:  # nx.ex:8592-8598: out type = to_floating
+        def math_fun(t, _n=name):
+            t = to_tensor(t)
+            return getattr(_impl(t), _n)(t.with_(data=None, type=T.to_floating(t.type)), t)
+        g[name] = math_fun
+    for name in ["negate", "sign"]:  # nx.ex:8703-8731
+        g[name] = (lambda n: lambda t: getattr(_impl(to_tensor(t)), n)(to_tensor(t).with_(data=None), to_tensor(t)))(name)
+    for name in ["floor", "ceil", "round"]:  # nx.ex:9095-9133: integers are returned as they are
+        def rounding(t, _n=name):
+            t = to_tensor(t)
+            return t if T.is_integer(t.type) else getattr(_impl(t), _n)(t.with_(data=None), t)
+        g[name] = rounding
+    for name in ["bitwise_not", "population_count", "count_leading_zeros"]:  # nx.ex:8979-9091
+        def bit_fun(t, _n=name):
+            t = to_tensor(t)
+            if not T.is_integer(t.type):
+                raise ValueError(f"{_n} expects integer tensors as inputs and outputs an integer tensor, "
+                                 f"got: {t.type!r}")
+            return getattr(_impl(t), _n)(t.with_(data=None), t)
+        g[name] = bit_fun
+    for name in ["is_nan", "is_infinity"]:  # nx.ex:8628-8690: u8 output
+        g[name] = (lambda n: lambda t: getattr(_impl(to_tensor(t)), n)(to_tensor(t).with_(data=None, type=("u", 8)), to_tensor(t)))(name)
+
+
+_def_unary()
+
+
+def abs(t):  # noqa: A001 - mirrors Nx.abs/1 (nx.ex:8746-8754): unsigned tensors are returned as-is
+    t = to_tensor(t)
+    return t if t.type[0] == "u" else _impl(t).abs(t.with_(data=None), t)
+
+
+def as_type(t, type) -> Tensor:
+    """Nx.as_type/2 (nx.ex:2863-2876): a no-op when the type already matches."""
+    t = to_tensor(t)
+    ty = T.normalize(type)
+    return t if t.type == ty else _impl(t).as_type(t.with_(data=None, type=ty), t)
+
+
+# ---- reductions ----------------------------------------------------------------------------
+
+def _aggregate(t, op, out_type, axes=None, keep_axes=False):
+    """aggregate_axes_op/4 (nx.ex:10594-10649)."""
+    t = to_tensor(t)
+    if axes is not None:
+        axes = S.normalize_axes(t.shape, axes)
+        shape_ = S.contract(t.shape, axes, keep_axes)
+    elif keep_axes:
+        shape_, axes = (1,) * len(t.shape), list(range(len(t.shape)))
+    else:
+        shape_ = ()
+    if axes == []:
+        return as_type(t, out_type)
+    return getattr(_impl(t), op)(template(out_type, shape_), t, {"axes": axes, "keep_axes": keep_axes})
+
+
+def sum(t, axes=None, keep_axes=False):  # noqa: A001 - Nx.sum/2 (nx.ex:9622-9626)
+    t = to_tensor(t)
+    return _aggregate(t, "sum", T.to_aggregate(t.type), axes, keep_axes)
+
+
+def product(t, axes=None, keep_axes=False):
+    t = to_tensor(t)
+    return _aggregate(t, "product", T.to_aggregate(t.type), axes, keep_axes)
+
+
+def reduce_max(t, axes=None, keep_axes=False):
+    """Nx.reduce_max/2 (nx.ex:10496-10500): output type = input type."""
+    t = to_tensor(t)
+    return _aggregate(t, "reduce_max", t.type, axes, keep_axes)
+
+
+def reduce_min(t, axes=None, keep_axes=False):
+    t = to_tensor(t)
+    return _aggregate(t, "reduce_min", t.type, axes, keep_axes)
+
+
+def _argmin_or_max(t, op, axis=None, tie_break="low", keep_axis=False, type=("s", 32)):
+    """argmin_or_max/3 (nx.ex:10948-11005)."""
+    if tie_break not in ("low", "high"):
+        raise ValueError(f"unknown value for :tie_break, expected :high or :low, got: {tie_break!r}")
+    t = to_tensor(t)
+    if axis is not None:
+        axis = S.normalize_axis(t.shape, axis)
+        shape_ = S.contract(t.shape, [axis], keep_axis)
+    else:
+        shape_ = ()
+    out = template(T.normalize(type), shape_)
+    return getattr(_impl(t), op)(out, t, {"tie_break": tie_break, "axis": axis, "keep_axis": keep_axis})
+
+
+def argmax(t, **opts):
+    return _argmin_or_max(t, "argmax", **opts)
+
+
+def argmin(t, **opts):
+    return _argmin_or_max(t, "argmin", **opts)
+
+
+# ---- contraction ---------------------------------------------------------------------------
+
+def dot(t1, *args, out_type=None):
+    """Nx.dot/2, /4 and /6 (nx.ex:12836-12847, 12918-12920, 13123-13161).
+
+    `out_type` is not part of the reference's front end: it sets the template type handed to the
+    `dot` callback (both reference backends honour `out.type` whatever the operand types,
+    binary_backend.ex:549-559) and is how a s8 x s8 -> s32 contraction is requested."""
+    if len(args) == 1:
+        t1, t2 = to_tensor(t1), to_tensor(args[0])
+        n, m = len(t1.shape), len(t2.shape)
+        if n == 0 or m == 0:
+            return globals()["multiply"](t1, t2)
+        if m == 1:
+            return dot(t1, [n - 1], [], t2, [0], [], out_type=out_type)
+        if n == 1:
+            return dot(t1, [0], [], t2, [m - 2], [], out_type=out_type)
+        return dot(t1, [n - 1], [], t2, [m - 2], [], out_type=out_type)
+    if len(args) == 3:
+        c1, t2, c2 = args
+        return dot(t1, c1, [], t2, c2, [], out_type=out_type)
+    c1, b1, t2, c2, b2 = args
+    t1, t2 = to_tensor(t1), to_tensor(t2)
+    ty = T.normalize(out_type) if out_type is not None else T.binary_type(t1.type, t2.type)
+    c1, c2 = S.normalize_axes(t1.shape, c1), S.normalize_axes(t2.shape, c2)
+    b1, b2 = S.normalize_axes(t1.shape, b1), S.normalize_axes(t2.shape, b2)
+    out = template(ty, S.dot(t1.shape, c1, b1, t2.shape, c2, b2))
+    return _impl(t1, t2).dot(out, t1, c1, b1, t2, c2, b2)
+
+
+# ---- shape / data movement -----------------------------------------------------------------
+
+def reshape(t, new_shape):
+    """Nx.reshape/2 (nx.ex:3010-3065), with one `"auto"` dimension allowed."""
+    t = to_tensor(t)
+    new_shape = list(new_shape)
+    if "auto" in new_shape:
+        i = new_shape.index("auto")
+        rest = prod(d for d in new_shape if d != "auto")
+        new_shape[i] = t.size // rest if rest else 0
+    if prod(new_shape) != t.size:
+        raise ValueError(f"cannot reshape, current shape {S.fmt(t.shape)} is not compatible with "
+                         f"new shape {S.fmt(tuple(new_shape))}")
+    if tuple(new_shape) == t.shape:
+        return t
+    return _impl(t).reshape(t.with_(data=None, shape=tuple(new_shape)), t)
+
+
+def new_axis(t, axis):
+    t = to_tensor(t)
+    rank = len(t.shape)
+    axis = axis + rank + 1 if axis < 0 else axis
+    return reshape(t, t.shape[:axis] + (1,) + t.shape[axis:])
+
+
+def squeeze(t, axes=None):
+    t = to_tensor(t)
+    axes = [i for i, d in enumerate(t.shape) if d == 1] if axes is None else S.normalize_axes(t.shape, axes)
+    if not axes:
+        return t
+    return _impl(t).squeeze(t.with_(data=None, shape=S.squeeze(t.shape, axes)), t, axes)
+
+
+def bitcast(t, type):
+    t = to_tensor(t)
+    ty = T.normalize(type)
+    if ty[1] != t.type[1]:
+        raise ValueError("input type width must match new type width")
+    return _impl(t).bitcast(t.with_(data=None, type=ty), t)
+
+
+def transpose(t, axes=None):
+    """Nx.transpose/2 (nx.ex:3440-3465): identity permutations return the tensor."""
+    t = to_tensor(t)
+    rank = len(t.shape)
+    axes = list(range(rank - 1, -1, -1)) if axes is None else S.normalize_axes(t.shape, axes)
+    if axes == list(range(rank)):
+        return t
+    return _impl(t).transpose(t.with_(data=None, shape=S.transpose(t.shape, axes)), t, axes)
+
+
+def broadcast(t, new_shape, axes=None):
+    """Nx.broadcast/3 (nx.ex:3180-3215)."""
+    t = to_tensor(t)
+    new_shape = tuple(new_shape)
+    axes = S.broadcast_axes(t.shape, new_shape) if axes is None else S.normalize_axes(new_shape, axes)
+    S.broadcast(t.shape, new_shape, axes)
+    if t.shape == new_shape and axes == list(range(len(new_shape))):
+        return t
+    return _impl(t).broadcast(t.with_(data=None, shape=new_shape), t, new_shape, axes)
+
+
+@dataclass(frozen=True)
+class BlockTake:
+    """%Nx.Block.Take{axis} (nx/lib/nx/block.ex:57-59)."""
+    axis: int
+
+
+def block(struct, args, out, fun):
+    """Nx.block/4 (nx.ex:7370-7380): lets the backend replace a composite op."""
+    return _impl(*args).block(struct, out, list(args), fun)
+
+
+def gather(t, indices, axes=None, **backend_opts):
+    """Nx.gather/3 (nx.ex:15160-15203)."""
+    t, indices = to_tensor(t), to_tensor(indices)
+    if len(indices.shape) == 0:
+        raise ValueError("expected indices rank to be at least 1, got: 0")
+    if not T.is_integer(indices.type):
+        raise ValueError(f"indices must be an integer tensor, got {indices.type!r}")
+    depth = indices.shape[-1]
+    axes = list(range(depth)) if axes is None else S.normalize_axes(t.shape, axes)
+    if len(axes) != depth:
+        raise ValueError(f"expected the last indices dimension size ({depth}) to match the number of axes")
+    out = t.with_(data=None, shape=S.gather(t.shape, indices.shape, axes))
+    return _impl(t, indices).gather(out, t, indices, dict(axes=axes, **backend_opts))
+
+
+def take(t, indices, axis=0):
+    """Nx.take/3 (nx.ex:14732-14821), non-vectorised path: wraps the default gather-based
+    implementation in a `Nx.Block.Take` so a backend can do it natively."""
+    t, indices = to_tensor(t), to_tensor(indices)
+    if not T.is_integer(indices.type):
+        raise ValueError(f"indices must be an integer tensor, got {indices.type!r}")
+    axis = S.normalize_axis(t.shape, axis)
+    inner_shape = S.take(t.shape, indices.shape, axis)
+    out = t.with_(data=None, shape=inner_shape)
+
+    def default(_struct, tensor_, indices_):
+        gather_indices = new_axis(indices_, len(indices_.shape))
+        n_idx = len(indices_.shape)
+        all_axes = list(range(len(inner_shape)))
+        indices_axes, tensor_axes = all_axes[:n_idx], all_axes[n_idx:]
+        leading, trailing = tensor_axes[:axis], tensor_axes[axis:]
+        return transpose(gather(tensor_, gather_indices, axes=[axis]), leading + indices_axes + trailing)
+
+    return block(BlockTake(axis), [t, indices], out, default)

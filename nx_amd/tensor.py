@@ -1,0 +1,126 @@
+"""The tensor struct and host-side number <-> binary codecs.
+
+`Tensor` mirrors `%Nx.Tensor{data, type, shape, names}` (reference: nx/lib/nx/tensor.ex:41-42):
+`data` holds a backend struct, everything else is metadata owned by the front end.  A backend
+fills `out.data` and never changes type / shape / names (nx/lib/nx/backend.ex:5-8).
+"""
+from __future__ import annotations
+
+import math
+import struct
+from dataclasses import dataclass, replace
+from typing import Any, Optional, Tuple
+
+import numpy as np
+
+from . import types as T
+
+
+@dataclass(frozen=True)
+class Tensor:
+    data: Any
+    type: Tuple[str, int]
+    shape: Tuple[int, ...]
+    names: Tuple[Optional[str], ...] = ()
+
+    def __post_init__(self):
+        object.__setattr__(self, "type", T.normalize(self.type))
+        object.__setattr__(self, "shape", tuple(int(d) for d in self.shape))
+        if len(self.names) != len(self.shape):
+            object.__setattr__(self, "names", (None,) * len(self.shape))
+
+    @property
+    def size(self) -> int:
+        return math.prod(self.shape)
+
+    @property
+    def rank(self) -> int:
+        return len(self.shape)
+
+    def with_(self, **kw) -> "Tensor":
+        if "shape" in kw and "names" not in kw:
+            kw["names"] = (None,) * len(kw["shape"])
+        return replace(self, **kw)
+
+
+def template(type, shape) -> Tensor:
+    """An output template: a tensor without data, as passed as the first callback argument."""
+    return Tensor(None, T.normalize(type), tuple(shape))
+
+
+# ---- number -> binary, following the reference's write path ---------------------------------
+# nx/lib/nx/shared.ex:136-194: integers keep the low bits, floats round to nearest even,
+# bf16 = the f32 encoding without its low 16 bits; type.ex:128-158 for the non-finite patterns.
+
+_NAN = {16: 0x7E00, 32: 0x7FC00000, 64: 0x7FF8000000000000}
+
+
+def number_to_binary(number, type) -> bytes:
+    kind, bits = T.normalize(type)
+    if kind in ("u", "s"):
+        if isinstance(number, float):
+            if number != number or math.isinf(number):
+                raise ValueError(f"cannot encode {number!r} as an integer")
+            if number != int(number):
+                raise ValueError(f"cannot encode the float {number!r} as an integer type")
+            number = int(number)
+        return (int(number) & ((1 << bits) - 1)).to_bytes(bits // 8, "little")
+    x = float(number)
+    if kind == "bf":
+        if x != x:
+            return (0x7FC0).to_bytes(2, "little")
+        with np.errstate(over="ignore"):
+            f = np.float32(x)
+        if np.isinf(f) and not math.isinf(x):
+            raise OverflowError(f"{number!r} does not fit a 32-bit float")
+        return (int(f.view(np.uint32)) >> 16).to_bytes(2, "little")
+    if x != x:
+        return _NAN[bits].to_bytes(bits // 8, "little")
+    if bits == 64:
+        return struct.pack("<d", x)
+    with np.errstate(over="ignore"):
+        v = np.float32(x) if bits == 32 else np.float16(x)
+    if np.isinf(v) and not math.isinf(x):
+        raise OverflowError(f"{number!r} does not fit a {bits}-bit float")
+    return v.tobytes()
+
+
+def list_to_binary(values, type) -> bytes:
+    """Flat list of Python numbers -> binary (Nx.tensor/2's flattening, nx/lib/nx.ex:774-883)."""
+    kind, bits = T.normalize(type)
+    arr = np.asarray(values)
+    if kind in ("u", "s"):
+        if arr.dtype.kind == "f":
+            raise ValueError("cannot build an integer tensor from floats")
+        if arr.dtype == object:
+            return b"".join(number_to_binary(v, type) for v in arr.ravel())
+        return arr.astype(np.int64).astype(T.numpy_dtype(type)).tobytes()
+    if kind == "bf":
+        f = np.asarray(values, dtype=np.float64).astype(np.float32).ravel()
+        out = (f.view(np.uint32) >> 16).astype(np.uint16)
+        out[np.isnan(f)] = 0x7FC0
+        return out.tobytes()
+    f = np.asarray(values, dtype=np.float64).astype(T.numpy_dtype(type)).ravel()
+    if np.isnan(f).any():
+        raw = f.view({16: np.uint16, 32: np.uint32, 64: np.uint64}[bits]).copy()
+        raw[np.isnan(f)] = _NAN[bits]
+        return raw.tobytes()
+    return f.tobytes()
+
+
+def binary_to_numpy(binary: bytes, type, shape=None) -> np.ndarray:
+    """Raw view of a tensor binary; bf16 comes back as uint16 bit patterns."""
+    arr = np.frombuffer(binary, dtype=T.numpy_dtype(type))
+    return arr.reshape(shape) if shape is not None else arr
+
+
+def bf16_bits_to_float32(bits: np.ndarray) -> np.ndarray:
+    return (bits.astype(np.uint32) << 16).view(np.float32)
+
+
+def to_float64(binary: bytes, type, shape=None) -> np.ndarray:
+    """Decoded values as float64 (exact for every type but 64-bit integers above 2^53)."""
+    raw = binary_to_numpy(binary, type, shape)
+    if T.normalize(type) == ("bf", 16):
+        return bf16_bits_to_float32(raw).astype(np.float64)
+    return raw.astype(np.float64)

@@ -1,0 +1,318 @@
+"""BinaryBackend -- the parity oracle: `Nx.BinaryBackend`'s callbacks over the C restatement.
+
+TEST INFRASTRUCTURE ONLY.  Tests, the smoke check and the CPU-baseline leg of the benchmark use
+it as the checker; nothing in the product imports it.
+
+It implements the same callback interface as the device backend (reference:
+nx/lib/nx/backend.ex:46-144), each callback following the cited lines of
+nx/lib/nx/binary_backend.ex through `libhipnx_ref.so` (oracle/hipnx_ref.c), so that the same
+front-end call can be run on either backend and compared -- the pattern of the reference's own
+cross-backend suite (torchx/test/torchx/nx_test.exs:25-50).
+
+Where the reference raises, this raises: `ReferenceRaises` carries the message.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+from math import prod
+
+import numpy as np
+
+from nx_amd import shape as S
+from nx_amd import types as T
+from nx_amd.tensor import Tensor, number_to_binary
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libhipnx_ref.so")
+
+
+def build(force: bool = False) -> str:
+    """Compiles the C restatement with gcc (seconds)."""
+    src = os.path.join(_HERE, "hipnx_ref.c")
+    if force or not os.path.exists(LIB_PATH) or os.path.getmtime(LIB_PATH) < os.path.getmtime(src):
+        subprocess.check_call(["make", "-C", _HERE, "-B", "libhipnx_ref.so"], stdout=subprocess.DEVNULL)
+    return LIB_PATH
+
+
+def _load():
+    if not os.path.exists(LIB_PATH):
+        build()
+    lib = C.CDLL(LIB_PATH)
+    i64p, intp, vp = C.POINTER(C.c_int64), C.POINTER(C.c_int), C.c_void_p
+    lib.ref_last_error.restype = C.c_char_p
+    lib.ref_set_threads.argtypes = [C.c_int]
+    lib.ref_binary.argtypes = [C.c_int] * 5 + [i64p, i64p, i64p, vp, vp, vp]
+    lib.ref_unary.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int64, vp, vp]
+    lib.ref_as_type.argtypes = [C.c_int, C.c_int, C.c_int64, vp, vp]
+    lib.ref_reduce.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int64, C.c_int64, C.c_int64, vp, vp]
+    lib.ref_argreduce.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int64, C.c_int64, C.c_int64, vp, vp]
+    lib.ref_dot.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int64, vp, vp, vp]
+    lib.ref_transpose.argtypes = [C.c_int, C.c_int, i64p, intp, vp, vp]
+    lib.ref_broadcast.argtypes = [C.c_int, C.c_int, i64p, i64p, vp, vp]
+    lib.ref_gather.argtypes = [C.c_int, C.c_int, i64p, C.c_int, C.c_int64, C.c_int, vp, vp, vp]
+    return lib
+
+
+lib = _load()
+
+
+class ReferenceRaises(Exception):
+    """The reference raises here (ArgumentError / ArithmeticError); `.code` is the REF_E* status."""
+
+    def __init__(self, code, message):
+        super().__init__(message)
+        self.code = code
+
+
+def _check(status):
+    if status:
+        raise ReferenceRaises(status, lib.ref_last_error().decode())
+
+
+def set_threads(n: int) -> None:
+    lib.ref_set_threads(n)
+
+
+def _i64(v):
+    v = list(v)
+    return (C.c_int64 * max(len(v), 1))(*v)
+
+
+def _ints(v):
+    v = list(v)
+    return (C.c_int * max(len(v), 1))(*v)
+
+
+BINARY_OPS = ["add", "subtract", "multiply", "divide", "pow", "remainder", "atan2", "min", "max", "quotient",
+              "bitwise_and", "bitwise_or", "bitwise_xor", "left_shift", "right_shift", "equal", "not_equal",
+              "greater", "less", "greater_equal", "less_equal", "logical_and", "logical_or", "logical_xor"]
+UNARY_OPS = ["exp", "expm1", "log", "log1p", "sigmoid", "cos", "sin", "tan", "cosh", "sinh", "tanh", "acos", "asin",
+             "atan", "acosh", "asinh", "atanh", "sqrt", "rsqrt", "cbrt", "erf", "erfc", "erf_inv", "abs",
+             "bitwise_not", "ceil", "floor", "negate", "round", "sign", "count_leading_zeros", "population_count",
+             "is_nan", "is_infinity"]
+
+
+class BinaryBackend:
+    """Backend struct: `%Nx.BinaryBackend{state: binary}` (binary_backend.ex:14-15)."""
+
+    def __init__(self, state: bytearray):
+        self.state = state
+
+    @staticmethod
+    def init(opts):  # binary_backend.ex:26-33
+        if opts:
+            raise ValueError("Nx.BinaryBackend accepts no options")
+        return {}
+
+    # -- helpers
+    @staticmethod
+    def _ptr(buf):
+        return (C.c_char * max(len(buf), 1)).from_buffer(buf) if len(buf) else (C.c_char * 1)()
+
+    @classmethod
+    def _bin(cls, t: Tensor) -> bytearray:
+        if isinstance(t.data, BinaryBackend):
+            return t.data.state
+        return bytearray(type(t.data).to_binary(t, t.size))
+
+    @classmethod
+    def _new(cls, out: Tensor):
+        buf = bytearray(out.size * T.size_bytes(out.type))
+        return buf, out.with_(data=cls(buf))
+
+    # -- plumbing (binary_backend.ex:42-46, 114-165)
+    @classmethod
+    def from_binary(cls, out, binary, opts=None):
+        need = out.size * T.size_bytes(out.type)
+        if len(binary) < need:
+            raise ValueError("binary size is too small for the requested shape")
+        return out.with_(data=cls(bytearray(binary[:need])))
+
+    @classmethod
+    def to_binary(cls, t, limit):
+        return bytes(t.data.state[: min(int(limit), t.size) * T.size_bytes(t.type)])
+
+    @classmethod
+    def constant(cls, out, number, opts=None):
+        return out.with_(data=cls(bytearray(number_to_binary(number, out.type) * out.size)))
+
+    @classmethod
+    def backend_copy(cls, t, backend, opts=None):
+        return backend.from_binary(t, cls.to_binary(t, t.size), opts)
+
+    backend_transfer = backend_copy
+
+    @classmethod
+    def backend_deallocate(cls, t):
+        return "ok"
+
+    @classmethod
+    def reshape(cls, out, t):
+        return out.with_(data=cls(cls._bin(t)))
+
+    @classmethod
+    def squeeze(cls, out, t, axes):
+        return out.with_(data=cls(cls._bin(t)))
+
+    @classmethod
+    def bitcast(cls, out, t):
+        return out.with_(data=cls(cls._bin(t)))
+
+    @classmethod
+    def block(cls, struct, out, args, fun):  # binary_backend.ex:36-38
+        return fun(struct, *args)
+
+    # -- element-wise (binary_backend.ex:649-706, 827-832, 957-960)
+    @classmethod
+    def _binary(cls, op, out, l, r):
+        lb, rb = cls._bin(l), cls._bin(r)
+        buf, res = cls._new(out)
+        _check(lib.ref_binary(op, T.code(l.type), T.code(r.type), T.code(out.type), len(out.shape), _i64(out.shape),
+                              _i64(S.broadcast_strides(l.shape, out.shape)),
+                              _i64(S.broadcast_strides(r.shape, out.shape)), cls._ptr(lb), cls._ptr(rb), cls._ptr(buf)))
+        return res
+
+    @classmethod
+    def _unary(cls, op, out, t):
+        tb = cls._bin(t)
+        buf, res = cls._new(out)
+        _check(lib.ref_unary(op, T.code(t.type), T.code(out.type), out.size, cls._ptr(tb), cls._ptr(buf)))
+        return res
+
+    @classmethod
+    def as_type(cls, out, t):  # binary_backend.ex:2031-2076
+        if t.type == out.type:
+            return t
+        tb = cls._bin(t)
+        buf, res = cls._new(out)
+        _check(lib.ref_as_type(T.code(t.type), T.code(out.type), out.size, cls._ptr(tb), cls._ptr(buf)))
+        return res
+
+    # -- data movement (binary_backend.ex:215-319, 1902-1959)
+    @classmethod
+    def transpose(cls, out, t, axes):
+        tb = cls._bin(t)
+        buf, res = cls._new(out)
+        _check(lib.ref_transpose(T.size_bytes(t.type), len(t.shape), _i64(t.shape), _ints(axes), cls._ptr(tb),
+                                 cls._ptr(buf)))
+        return res
+
+    @classmethod
+    def broadcast(cls, out, t, shape, axes):
+        strides, s = [0] * len(shape), 1
+        for pos in range(len(t.shape) - 1, -1, -1):
+            if t.shape[pos] != 1:
+                strides[axes[pos]] = s
+            s *= t.shape[pos]
+        tb = cls._bin(t)
+        buf, res = cls._new(out)
+        _check(lib.ref_broadcast(T.size_bytes(t.type), len(shape), _i64(shape), _i64(strides), cls._ptr(tb),
+                                 cls._ptr(buf)))
+        return res
+
+    @classmethod
+    def gather(cls, out, t, indices, opts):
+        axes = list(opts["axes"])
+        rank = len(t.shape)
+        if list(range(rank))[: len(axes)] != axes:  # binary_backend.ex:1907-1913
+            perm = axes + [a for a in range(rank) if a not in axes]
+            t = cls.transpose(t.with_(data=None, shape=S.transpose(t.shape, perm)), t, perm)
+        tb, ib = cls._bin(t), cls._bin(indices)
+        buf, res = cls._new(out)
+        _check(lib.ref_gather(T.size_bytes(t.type), rank, _i64(t.shape), T.code(indices.type),
+                              prod(indices.shape[:-1]), indices.shape[-1], cls._ptr(tb), cls._ptr(ib), cls._ptr(buf)))
+        return res
+
+    # -- reductions (binary_backend.ex:1315-1431, 2342-2360, 2469-2512)
+    @classmethod
+    def _view(cls, t, axes):
+        """[kept..., reduced...] in sorted axis order: the traversal order of aggregate_axes."""
+        rank = len(t.shape)
+        if axes is None:
+            return t, 1, t.size, 1
+        axes = sorted(axes)
+        kept = [a for a in range(rank) if a not in axes]
+        perm = kept + axes
+        if perm != list(range(rank)):
+            t = cls.transpose(t.with_(data=None, shape=S.transpose(t.shape, perm)), t, perm)
+        return t, prod(t.shape[: len(kept)]), prod(t.shape[len(kept):]), 1
+
+    @classmethod
+    def _reduce(cls, op, out, t, opts):
+        view, outer, red, inner = cls._view(t, opts.get("axes"))
+        tb = cls._bin(view)
+        buf, res = cls._new(out)
+        _check(lib.ref_reduce(op, T.code(t.type), T.code(out.type), outer, red, inner, cls._ptr(tb), cls._ptr(buf)))
+        return res
+
+    @classmethod
+    def sum(cls, out, t, opts):
+        return cls._reduce(0, out, t, opts)
+
+    @classmethod
+    def reduce_max(cls, out, t, opts):
+        return cls._reduce(1, out, t, opts)
+
+    @classmethod
+    def reduce_min(cls, out, t, opts):
+        return cls._reduce(2, out, t, opts)
+
+    @classmethod
+    def product(cls, out, t, opts):
+        return cls._reduce(3, out, t, opts)
+
+    @classmethod
+    def _arg(cls, op, out, t, opts):
+        axis = opts.get("axis")
+        view, outer, red, inner = cls._view(t, None if axis is None else [axis])
+        tie = {"low": 0, "high": 1}[opts.get("tie_break", "low")]
+        tb = cls._bin(view)
+        buf, res = cls._new(out)
+        _check(lib.ref_argreduce(op, tie, T.code(t.type), T.code(out.type), outer, red, inner, cls._ptr(tb),
+                                 cls._ptr(buf)))
+        return res
+
+    @classmethod
+    def argmax(cls, out, t, opts):
+        return cls._arg(0, out, t, opts)
+
+    @classmethod
+    def argmin(cls, out, t, opts):
+        return cls._arg(1, out, t, opts)
+
+    # -- dot (binary_backend.ex:476-599)
+    @classmethod
+    def _contract_last(cls, t, contract, nbatch):
+        """bin_dot_transpose_contract_axes/2: [batch, kept, contract in the given order]."""
+        rank = len(t.shape)
+        kept = [a for a in range(nbatch, rank) if a not in contract]
+        perm = list(range(nbatch)) + kept + list(contract)
+        rows = prod(t.shape[a] for a in kept)
+        if perm != list(range(rank)):
+            t = cls.transpose(t.with_(data=None, shape=S.transpose(t.shape, perm)), t, perm)
+        return t, rows
+
+    @classmethod
+    def dot(cls, out, l, c1, b1, r, c2, b2):
+        nb = len(b1)
+        K = prod(l.shape[a] for a in c1)
+        batch = prod(l.shape[a] for a in b1)
+        lt, M = cls._contract_last(l, c1, nb)
+        rt, N = cls._contract_last(r, c2, nb)
+        lb, rb = cls._bin(lt), cls._bin(rt)
+        buf, res = cls._new(out)
+        _check(lib.ref_dot(T.code(l.type), T.code(r.type), T.code(out.type), batch, M, N, K, cls._ptr(lb),
+                           cls._ptr(rb), cls._ptr(buf)))
+        return res
+
+
+def _install():
+    for code, name in enumerate(BINARY_OPS):
+        setattr(BinaryBackend, name, classmethod(lambda cls, out, l, r, _c=code: cls._binary(_c, out, l, r)))
+    for code, name in enumerate(UNARY_OPS):
+        setattr(BinaryBackend, name, classmethod(lambda cls, out, t, _c=code: cls._unary(_c, out, t)))
+
+
+_install()

@@ -1,0 +1,743 @@
+/*
+ * hipnx_ref.c -- CPU restatement of Nx.BinaryBackend (reference: nx/lib/nx/binary_backend.ex)
+ * for the eager tensor hot path: broadcasting element-wise ops, as_type, sum / reduce_max /
+ * reduce_min / argmax / argmin, dot, transpose, broadcast, gather.
+ *
+ * TEST INFRASTRUCTURE ONLY: this is the parity checker, never a product code path.
+ *
+ * Numeric model (binary_backend.ex:2415-2438, shared.ex:57-194, 240-283, floating.ex:26-68):
+ * every element is decoded into an "Erlang number" -- an unbounded integer (held here in
+ * __int128, enough for every case exercised), an IEEE double, or one of the atoms
+ * :nan / :infinity / :neg_infinity -- the operation runs on those, and the result is encoded
+ * once into the output type: integers keep the low `size` bits (wrap), f64 -> f32/f16 rounds to
+ * nearest even and *raises* when a finite value overflows, bf16 is the f32 encoding with the
+ * low 16 bits dropped, atoms become canonical bit patterns (type.ex:128-158).
+ *
+ * Parity pinning status of the pieces (what independent evidence fixes them) is recorded in
+ * the test-suite next to the golden vectors; functions whose last-bit behaviour lives in the
+ * un-vendored `complex` 0.7.0 package (erf, erfc, erf_inv, cbrt, pow/atan2/divide on
+ * non-finite or zero operands, fmod corner cases) are "parity unpinned": they follow IEEE /
+ * libm here.
+ *
+ * Build: gcc -O2 -ffp-contract=off -fopenmp -shared -fPIC hipnx_ref.c -lm
+ * (-ffp-contract=off is required: the reference multiplies and adds in two roundings.)
+ */
+#include "hipnx_ref.h"
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+typedef __int128 i128;
+typedef unsigned __int128 u128;
+
+static __thread char g_err[256];
+static int g_threads = 0;
+
+const char *ref_last_error(void) { return g_err; }
+void ref_set_threads(int n) { g_threads = n; }
+static int nthreads(void) {
+#ifdef _OPENMP
+  return g_threads > 0 ? g_threads : omp_get_num_procs();
+#else
+  return 1;
+#endif
+}
+
+static int fail(int code, const char *msg) {
+  snprintf(g_err, sizeof g_err, "%s", msg);
+  return code;
+}
+
+int ref_dtype_size(int dt) {
+  static const int sz[REF_NTYPES] = {1, 2, 4, 8, 1, 2, 4, 8, 2, 2, 4, 8};
+  return (dt >= 0 && dt < REF_NTYPES) ? sz[dt] : -1;
+}
+static int is_float_dt(int dt) { return dt >= REF_F16; }
+static int is_unsigned_dt(int dt) { return dt <= REF_U64; }
+
+/* ---- the Erlang-number model ------------------------------------------------------------ */
+
+enum { K_INT = 0, K_FLT = 1, K_NAN = 2, K_INF = 3, K_NINF = 4 };
+typedef struct {
+  int k;
+  i128 i;
+  double f;
+} num;
+
+static num mk_int(i128 v) { num n = {K_INT, v, 0.0}; return n; }
+static num mk_atom(int k) { num n = {k, 0, 0.0}; return n; }
+static num from_double(double d) {
+  num n = {K_FLT, 0, d};
+  if (isnan(d)) n.k = K_NAN;
+  else if (isinf(d)) n.k = d > 0 ? K_INF : K_NINF;
+  return n;
+}
+static double to_double(num n) {
+  switch (n.k) {
+    case K_INT: return (double)n.i;
+    case K_FLT: return n.f;
+    case K_INF: return INFINITY;
+    case K_NINF: return -INFINITY;
+    default: return NAN;
+  }
+}
+static int is_atom(num n) { return n.k >= K_NAN; }
+
+static double half_to_double(uint16_t h) {
+  int s = h >> 15, e = (h >> 10) & 31, m = h & 1023;
+  double v;
+  if (e == 0) v = ldexp((double)m, -24);
+  else if (e == 31) v = m ? NAN : INFINITY;
+  else v = ldexp((double)(m + 1024), e - 25);
+  return s ? -v : v;
+}
+
+/* round-to-nearest-even f64 -> f16 bits; *ovf set when a finite value becomes infinite */
+static uint16_t double_to_half(double d, int *ovf) {
+  uint16_t s = signbit(d) ? 0x8000 : 0;
+  double a = fabs(d);
+  if (isnan(d)) return 0x7E00;
+  if (isinf(d)) return s | 0x7C00;
+  if (a == 0.0) return s;
+  int e;
+  double fr = frexp(a, &e); /* a = fr * 2^e, fr in [0.5,1) */
+  int ue = e - 1;           /* unbiased exponent of 1.xxx form */
+  double scaled;
+  if (ue < -14) scaled = ldexp(a, 24);            /* subnormal: units of 2^-24 */
+  else scaled = ldexp(a, 10 - ue);                 /* 1024..2047.x */
+  (void)fr;
+  double r = nearbyint(scaled);                    /* RNE (default rounding mode) */
+  if (ue < -14) {
+    uint32_t m = (uint32_t)r;                      /* may carry into the normal range: fine */
+    return s | (uint16_t)m;
+  }
+  uint32_t m = (uint32_t)r;
+  if (m == 2048) { m = 1024; ue += 1; }
+  if (ue > 15) { *ovf = 1; return s | 0x7C00; }
+  return s | (uint16_t)(((ue + 15) << 10) | (m - 1024));
+}
+
+/* shared.ex:123-131 (floats), 240-270 (non-finite atoms), floating.ex:26-35 (bf16) */
+static num read_num(int dt, const void *p, int64_t idx) {
+  switch (dt) {
+    case REF_U8: return mk_int(((const uint8_t *)p)[idx]);
+    case REF_U16: return mk_int(((const uint16_t *)p)[idx]);
+    case REF_U32: return mk_int(((const uint32_t *)p)[idx]);
+    case REF_U64: return mk_int((i128)((const uint64_t *)p)[idx]);
+    case REF_S8: return mk_int(((const int8_t *)p)[idx]);
+    case REF_S16: return mk_int(((const int16_t *)p)[idx]);
+    case REF_S32: return mk_int(((const int32_t *)p)[idx]);
+    case REF_S64: return mk_int(((const int64_t *)p)[idx]);
+    case REF_F16: return from_double(half_to_double(((const uint16_t *)p)[idx]));
+    case REF_BF16: {
+      uint32_t b = (uint32_t)((const uint16_t *)p)[idx] << 16;
+      float f;
+      memcpy(&f, &b, 4);
+      return from_double((double)f);
+    }
+    case REF_F32: return from_double((double)((const float *)p)[idx]);
+    default: return from_double(((const double *)p)[idx]);
+  }
+}
+
+/* shared.ex:136-194 (write!), type.ex:128-158 (canonical non-finite patterns) */
+static int write_num(int dt, num n, void *p, int64_t idx) {
+  if (!is_float_dt(dt)) {
+    if (n.k != K_INT)
+      return fail(REF_ERAISE, "ArgumentError: cannot encode a float or non-finite value as an integer");
+    uint64_t low = (uint64_t)(u128)n.i; /* two's-complement low bits: wrap */
+    switch (dt) {
+      case REF_U8: case REF_S8: ((uint8_t *)p)[idx] = (uint8_t)low; break;
+      case REF_U16: case REF_S16: ((uint16_t *)p)[idx] = (uint16_t)low; break;
+      case REF_U32: case REF_S32: ((uint32_t *)p)[idx] = (uint32_t)low; break;
+      default: ((uint64_t *)p)[idx] = low; break;
+    }
+    return REF_OK;
+  }
+  double d = to_double(n);
+  switch (dt) {
+    case REF_F64: {
+      uint64_t b;
+      if (n.k == K_NAN) b = 0x7FF8000000000000ull;
+      else memcpy(&b, &d, 8);
+      ((uint64_t *)p)[idx] = b;
+      return REF_OK;
+    }
+    case REF_F32:
+    case REF_BF16: {
+      uint32_t b;
+      if (n.k == K_NAN) b = 0x7FC00000u;
+      else {
+        float f = (float)d; /* RNE */
+        if (isinf(f) && !is_atom(n))
+          return fail(REF_EOVERFLOW, "ArgumentError: finite value overflows the 32-bit float encoding");
+        memcpy(&b, &f, 4);
+      }
+      if (dt == REF_F32) ((uint32_t *)p)[idx] = b;
+      else ((uint16_t *)p)[idx] = (uint16_t)(b >> 16); /* floating.ex:60-64: drop low 16 bits */
+      return REF_OK;
+    }
+    default: { /* f16 */
+      int ovf = 0;
+      uint16_t h = double_to_half(d, &ovf);
+      if (ovf && !is_atom(n))
+        return fail(REF_EOVERFLOW, "ArgumentError: finite value overflows the 16-bit float encoding");
+      ((uint16_t *)p)[idx] = h;
+      return REF_OK;
+    }
+  }
+}
+
+/* ---- element-wise binary (binary_backend.ex:708-823) ------------------------------------ */
+
+static int both_int(num a, num b) { return a.k == K_INT && b.k == K_INT; }
+static i128 wrap_mul(i128 a, i128 b) { return (i128)((u128)a * (u128)b); }
+
+static i128 ipow(i128 base, i128 e) { /* Integer.pow then wrap == modular square-and-multiply */
+  i128 r = 1;
+  while (e > 0) {
+    if (e & 1) r = wrap_mul(r, base);
+    base = wrap_mul(base, base);
+    e >>= 1;
+  }
+  return r;
+}
+
+/* numeric comparison of two Erlang numbers that are not atoms */
+static int num_cmp(num a, num b) {
+  if (both_int(a, b)) return a.i < b.i ? -1 : (a.i > b.i ? 1 : 0);
+  double x = to_double(a), y = to_double(b);
+  return x < y ? -1 : (x > y ? 1 : 0);
+}
+static int as_boolean(num a) { /* binary_backend.ex:818-820: only a numeric zero is false */
+  if (a.k == K_INT) return a.i != 0;
+  if (a.k == K_FLT) return a.f != 0.0;
+  return 1;
+}
+
+static int bin_elem(int op, num a, num b, num *out) {
+  switch (op) {
+    case REF_ADD:
+      *out = both_int(a, b) ? mk_int(a.i + b.i) : from_double(to_double(a) + to_double(b));
+      return REF_OK;
+    case REF_SUBTRACT:
+      *out = both_int(a, b) ? mk_int(a.i - b.i) : from_double(to_double(a) - to_double(b));
+      return REF_OK;
+    case REF_MULTIPLY:
+      *out = both_int(a, b) ? mk_int(wrap_mul(a.i, b.i)) : from_double(to_double(a) * to_double(b));
+      return REF_OK;
+    case REF_DIVIDE: /* always a float result (nx.ex:6544) */
+      *out = from_double(to_double(a) / to_double(b));
+      return REF_OK;
+    case REF_POW:
+      if (both_int(a, b)) {
+        if (b.i < 0) return fail(REF_ERAISE, "ArithmeticError: negative exponent in Integer.pow");
+        *out = mk_int(ipow(a.i, b.i));
+      } else *out = from_double(pow(to_double(a), to_double(b)));
+      return REF_OK;
+    case REF_REMAINDER:
+      if (both_int(a, b)) {
+        if (b.i == 0) return fail(REF_ERAISE, "ArithmeticError: bad argument in arithmetic expression");
+        *out = mk_int(a.i % b.i); /* C99 %: sign of the dividend, like rem/2 */
+      } else *out = from_double(fmod(to_double(a), to_double(b)));
+      return REF_OK;
+    case REF_QUOTIENT:
+      if (!both_int(a, b)) return fail(REF_ERAISE, "ArithmeticError: div/2 needs integers");
+      if (b.i == 0) return fail(REF_ERAISE, "ArithmeticError: bad argument in arithmetic expression");
+      *out = mk_int(a.i / b.i); /* truncating, like div/2 */
+      return REF_OK;
+    case REF_ATAN2:
+      *out = from_double(atan2(to_double(a), to_double(b)));
+      return REF_OK;
+    case REF_MAX: /* binary_backend.ex:719-725 */
+      if (a.k == K_NAN || b.k == K_NAN) *out = mk_atom(K_NAN);
+      else if (a.k == K_INF || b.k == K_INF) *out = mk_atom(K_INF);
+      else if (a.k == K_NINF) *out = b;
+      else if (b.k == K_NINF) *out = a;
+      else *out = num_cmp(b, a) > 0 ? b : a; /* Kernel.max keeps the first when equal */
+      return REF_OK;
+    case REF_MIN: /* binary_backend.ex:727-733 */
+      if (a.k == K_NAN || b.k == K_NAN) *out = mk_atom(K_NAN);
+      else if (a.k == K_INF) *out = b;
+      else if (b.k == K_INF) *out = a;
+      else if (a.k == K_NINF || b.k == K_NINF) *out = mk_atom(K_NINF);
+      else *out = num_cmp(b, a) < 0 ? b : a;
+      return REF_OK;
+    case REF_BITWISE_AND: *out = mk_int(a.i & b.i); return REF_OK;
+    case REF_BITWISE_OR: *out = mk_int(a.i | b.i); return REF_OK;
+    case REF_BITWISE_XOR: *out = mk_int(a.i ^ b.i); return REF_OK;
+    case REF_LEFT_SHIFT:
+      if (b.i < 0) return fail(REF_ERAISE, "ArgumentError: cannot left shift by a negative count");
+      *out = mk_int(b.i >= 127 ? 0 : (i128)((u128)a.i << (int)b.i));
+      return REF_OK;
+    case REF_RIGHT_SHIFT:
+      if (b.i < 0) return fail(REF_ERAISE, "ArgumentError: cannot right shift by a negative count");
+      *out = mk_int(b.i >= 127 ? (a.i < 0 ? -1 : 0) : (a.i >> (int)b.i));
+      return REF_OK;
+    case REF_EQUAL:
+    case REF_NOT_EQUAL: {
+      int eq;
+      if (a.k == K_NAN || b.k == K_NAN) eq = 0;
+      else if (is_atom(a) || is_atom(b)) eq = (a.k == b.k);
+      else eq = num_cmp(a, b) == 0;
+      *out = mk_int(op == REF_EQUAL ? eq : 1 - eq);
+      return REF_OK;
+    }
+    case REF_GREATER:
+    case REF_LESS:
+    case REF_GREATER_EQUAL:
+    case REF_LESS_EQUAL: {
+      int r;
+      if (a.k == K_NAN || b.k == K_NAN) r = 0;
+      else {
+        /* the clause tables at binary_backend.ex:774-816 order -inf < every number < +inf,
+         * and an atom compared with itself is "equal" */
+        int ca = a.k == K_INF ? 1 : (a.k == K_NINF ? -1 : 0);
+        int cb = b.k == K_INF ? 1 : (b.k == K_NINF ? -1 : 0);
+        int c = ca != cb ? (ca < cb ? -1 : 1) : (ca == 0 ? num_cmp(a, b) : 0);
+        r = op == REF_GREATER ? c > 0 : op == REF_LESS ? c < 0 : op == REF_GREATER_EQUAL ? c >= 0 : c <= 0;
+      }
+      *out = mk_int(r);
+      return REF_OK;
+    }
+    case REF_LOGICAL_AND: *out = mk_int(as_boolean(a) && as_boolean(b)); return REF_OK;
+    case REF_LOGICAL_OR: *out = mk_int(as_boolean(a) || as_boolean(b)); return REF_OK;
+    case REF_LOGICAL_XOR: *out = mk_int(as_boolean(a) != as_boolean(b)); return REF_OK;
+  }
+  return fail(REF_EARG, "unknown binary op");
+}
+
+int ref_binary(int op, int l_dt, int r_dt, int out_dt, int rank, const int64_t *out_dims,
+               const int64_t *l_strides, const int64_t *r_strides, const void *l, const void *r,
+               void *out) {
+  if (op < 0 || op >= REF_NBINARY || ref_dtype_size(l_dt) < 0 || ref_dtype_size(r_dt) < 0 ||
+      ref_dtype_size(out_dt) < 0 || rank < 0 || rank > 16)
+    return fail(REF_EARG, "bad argument");
+  int64_t n = 1;
+  for (int a = 0; a < rank; a++) n *= out_dims[a];
+  int status = REF_OK;
+#pragma omp parallel for num_threads(nthreads()) schedule(static) if (n > 65536)
+  for (int64_t i = 0; i < n; i++) {
+    int64_t rem = i, lo = 0, ro = 0;
+    for (int a = rank - 1; a >= 0; a--) {
+      int64_t c = rem % out_dims[a];
+      rem /= out_dims[a];
+      lo += c * l_strides[a];
+      ro += c * r_strides[a];
+    }
+    num res;
+    int st = bin_elem(op, read_num(l_dt, l, lo), read_num(r_dt, r, ro), &res);
+    if (st == REF_OK) st = write_num(out_dt, res, out, i);
+    if (st != REF_OK) {
+#pragma omp critical
+      status = st;
+    }
+  }
+  return status;
+}
+
+/* ---- element-wise unary (shared.ex:311-376, binary_backend.ex:834-1005) ----------------- */
+
+/* Inverse error function: Newton steps on erf from a closed-form start.  The reference calls
+ * Complex.erf_inv (complex 0.7.0, not vendored): parity unpinned beyond ~1e-15 relative. */
+static double erf_inv_d(double y) {
+  if (isnan(y) || y < -1 || y > 1) return NAN;
+  if (y == 1) return INFINITY;
+  if (y == -1) return -INFINITY;
+  if (y == 0) return y;
+  double a = 0.147, ln = log(1 - y * y), t = 2 / (M_PI * a) + ln / 2;
+  double x = copysign(sqrt(sqrt(t * t - ln / a) - t), y);
+  for (int it = 0; it < 4; it++) {
+    double e = erf(x) - y;
+    x -= e / (2 / sqrt(M_PI) * exp(-x * x));
+  }
+  return x;
+}
+
+static int un_elem(int op, num x, int in_bits, num *out) {
+  double d = to_double(x);
+  switch (op) {
+    case REF_EXP: *out = from_double(exp(d)); return REF_OK;
+    case REF_EXPM1: *out = from_double(exp(d) - 1); return REF_OK;          /* exp |> subtract(1) */
+    case REF_LOG: *out = from_double(log(d)); return REF_OK;
+    case REF_LOG1P: *out = from_double(log(d + 1)); return REF_OK;          /* log(add(x, 1)) */
+    case REF_SIGMOID: *out = from_double(1 / (exp(-d) + 1)); return REF_OK; /* 1 / (exp(-x) + 1) */
+    case REF_COS: *out = from_double(cos(d)); return REF_OK;
+    case REF_SIN: *out = from_double(sin(d)); return REF_OK;
+    case REF_TAN: *out = from_double(tan(d)); return REF_OK;
+    case REF_COSH: *out = from_double(cosh(d)); return REF_OK;
+    case REF_SINH: *out = from_double(sinh(d)); return REF_OK;
+    case REF_TANH: *out = from_double(tanh(d)); return REF_OK;
+    case REF_ACOS: *out = from_double(acos(d)); return REF_OK;
+    case REF_ASIN: *out = from_double(asin(d)); return REF_OK;
+    case REF_ATAN: *out = from_double(atan(d)); return REF_OK;
+    case REF_ACOSH: *out = from_double(acosh(d)); return REF_OK;
+    case REF_ASINH: *out = from_double(asinh(d)); return REF_OK;
+    case REF_ATANH: *out = from_double(atanh(d)); return REF_OK;
+    case REF_SQRT: *out = from_double(sqrt(d)); return REF_OK;
+    case REF_RSQRT: *out = from_double(1 / sqrt(d)); return REF_OK;         /* divide(1, sqrt(x)) */
+    case REF_CBRT: *out = from_double(cbrt(d)); return REF_OK;
+    case REF_ERF: *out = from_double(erf(d)); return REF_OK;
+    case REF_ERFC: *out = from_double(erfc(d)); return REF_OK;
+    case REF_ERF_INV: *out = from_double(erf_inv_d(d)); return REF_OK;
+    case REF_ABS:
+      *out = x.k == K_INT ? mk_int(x.i < 0 ? -x.i : x.i) : from_double(fabs(d));
+      return REF_OK;
+    case REF_NEGATE:
+      *out = x.k == K_INT ? mk_int(-x.i) : from_double(-d);
+      return REF_OK;
+    case REF_BITWISE_NOT:
+      if (x.k != K_INT) return fail(REF_ERAISE, "ArithmeticError: bnot/1 needs an integer");
+      *out = mk_int(-x.i - 1);
+      return REF_OK;
+    case REF_CEIL: *out = x.k == K_INT ? x : from_double(ceil(d)); return REF_OK;
+    case REF_FLOOR: *out = x.k == K_INT ? x : from_double(floor(d)); return REF_OK;
+    case REF_ROUND: /* :erlang.round/1: half away from zero (binary_backend.ex:940) */
+      *out = x.k == K_INT ? x : from_double(round(d));
+      return REF_OK;
+    case REF_SIGN: /* binary_backend.ex:945-947: n<0 -> -1, n>0 -> 1, else n itself */
+      if (x.k == K_INT) *out = mk_int(x.i < 0 ? -1 : (x.i > 0 ? 1 : 0));
+      else if (is_atom(x)) *out = mk_int(1); /* guards use Erlang term order: any atom > 0 */
+      else if (d < 0) *out = mk_int(-1);
+      else if (d > 0) *out = mk_int(1);
+      else *out = x;
+      return REF_OK;
+    case REF_CLZ: { /* binary_backend.ex:962-1003, on the unsigned view of the element */
+      uint64_t v = (uint64_t)(u128)x.i;
+      if (in_bits < 64) v &= ((1ull << in_bits) - 1);
+      int c = 0;
+      for (int b = in_bits - 1; b >= 0 && !((v >> b) & 1); b--) c++;
+      *out = mk_int(c);
+      return REF_OK;
+    }
+    case REF_POPCOUNT: {
+      uint64_t v = (uint64_t)(u128)x.i;
+      if (in_bits < 64) v &= ((1ull << in_bits) - 1);
+      *out = mk_int(__builtin_popcountll(v));
+      return REF_OK;
+    }
+    case REF_IS_NAN: *out = mk_int(x.k == K_NAN); return REF_OK;
+    case REF_IS_INFINITY: *out = mk_int(x.k == K_INF || x.k == K_NINF); return REF_OK;
+  }
+  return fail(REF_EARG, "unknown unary op");
+}
+
+int ref_unary(int op, int in_dt, int out_dt, int64_t n, const void *in, void *out) {
+  if (op < 0 || op >= REF_NUNARY || ref_dtype_size(in_dt) < 0 || ref_dtype_size(out_dt) < 0)
+    return fail(REF_EARG, "bad argument");
+  int in_bits = 8 * ref_dtype_size(in_dt);
+  int status = REF_OK;
+#pragma omp parallel for num_threads(nthreads()) schedule(static) if (n > 65536)
+  for (int64_t i = 0; i < n; i++) {
+    num res;
+    int st = un_elem(op, read_num(in_dt, in, i), in_bits, &res);
+    /* a whole-number float result written to an integer type only happens for sign():
+     * the reference returns the integers -1 / 1 there, which a float output re-encodes */
+    if (st == REF_OK) st = write_num(out_dt, res, out, i);
+    if (st != REF_OK) {
+#pragma omp critical
+      status = st;
+    }
+  }
+  return status;
+}
+
+/* ---- as_type (binary_backend.ex:2031-2076) ---------------------------------------------- */
+
+static const uint64_t k_int_max[8] = {0xFFull, 0xFFFFull, 0xFFFFFFFFull, 0xFFFFFFFFFFFFFFFFull,
+                                      0x7Full, 0x7FFFull, 0x7FFFFFFFull, 0x7FFFFFFFFFFFFFFFull};
+
+int ref_as_type(int in_dt, int out_dt, int64_t n, const void *in, void *out) {
+  if (ref_dtype_size(in_dt) < 0 || ref_dtype_size(out_dt) < 0) return fail(REF_EARG, "bad dtype");
+  int status = REF_OK;
+  int fout = is_float_dt(out_dt);
+#pragma omp parallel for num_threads(nthreads()) schedule(static) if (n > 65536)
+  for (int64_t i = 0; i < n; i++) {
+    num x = read_num(in_dt, in, i), res;
+    if (fout) res = x;                                   /* number_to_binary(x, float type) */
+    else if (x.k == K_INT) res = x;                      /* trunc(int) = int, then wrap */
+    else if (x.k == K_FLT) {
+      /* trunc/1 gives an unbounded integer; only its low 64 bits can reach the output, and
+       * every double >= 2^64 in magnitude is a multiple of 2^11 * 2^53-ish: reduce mod 2^64 */
+      double t = trunc(x.f);
+      double m = fmod(t, 18446744073709551616.0); /* exact */
+      res = mk_int((i128)m);
+    } else if (x.k == K_NAN) res = mk_int(0);
+    else if (x.k == K_INF) res = mk_int((i128)k_int_max[out_dt]);       /* max_finite_binary */
+    else res = mk_int(is_unsigned_dt(out_dt) ? 0 : -(i128)k_int_max[out_dt] - 1); /* min_finite */
+    int st = write_num(out_dt, res, out, i);
+    if (st != REF_OK) {
+#pragma omp critical
+      status = st;
+    }
+  }
+  return status;
+}
+
+/* ---- reductions (binary_backend.ex:1315-1375, 2342-2360) -------------------------------- */
+
+static num nf_max(num a, num v) { /* non_finite_max/2, binary_backend.ex:1349-1355 */
+  if (a.k == K_NAN || v.k == K_NAN) return mk_atom(K_NAN);
+  if (a.k == K_INF || v.k == K_INF) return mk_atom(K_INF);
+  if (a.k == K_NINF) return v;
+  if (v.k == K_NINF) return a;
+  return num_cmp(v, a) > 0 ? v : a;
+}
+static num nf_min(num a, num v) { /* non_finite_min/2, binary_backend.ex:1369-1375 */
+  if (a.k == K_NAN || v.k == K_NAN) return mk_atom(K_NAN);
+  if (a.k == K_INF) return v;
+  if (v.k == K_INF) return a;
+  if (a.k == K_NINF || v.k == K_NINF) return mk_atom(K_NINF);
+  return num_cmp(v, a) < 0 ? v : a;
+}
+
+int ref_reduce(int op, int in_dt, int out_dt, int64_t outer, int64_t red, int64_t inner,
+               const void *in, void *out) {
+  if (ref_dtype_size(in_dt) < 0 || ref_dtype_size(out_dt) < 0 || op < 0 || op > REF_RED_PRODUCT)
+    return fail(REF_EARG, "bad argument");
+  if ((op == REF_RED_MAX || op == REF_RED_MIN) && red == 0)
+    return fail(REF_ERAISE, "cannot encode :first -- empty reduction");
+  int status = REF_OK;
+  int64_t nout = outer * inner;
+#pragma omp parallel for num_threads(nthreads()) schedule(static) if (nout * red > 65536 && nout > 1)
+  for (int64_t o = 0; o < nout; o++) {
+    int64_t ou = o / inner, iv = o % inner;
+    int64_t base = ou * red * inner + iv;
+    num acc;
+    if (op == REF_RED_SUM && is_float_dt(in_dt)) {
+      /* fast path, same arithmetic: acc = x + acc in IEEE double, starting from integer 0 */
+      double a = 0.0;
+      for (int64_t k = 0; k < red; k++) a = to_double(read_num(in_dt, in, base + k * inner)) + a;
+      acc = red == 0 ? mk_int(0) : from_double(a);
+    } else if (op == REF_RED_SUM || op == REF_RED_PRODUCT) {
+      acc = mk_int(op == REF_RED_SUM ? 0 : 1);
+      for (int64_t k = 0; k < red; k++) {
+        num x = read_num(in_dt, in, base + k * inner);
+        if (op == REF_RED_SUM)
+          acc = both_int(x, acc) ? mk_int(x.i + acc.i) : from_double(to_double(x) + to_double(acc));
+        else
+          acc = both_int(x, acc) ? mk_int(wrap_mul(x.i, acc.i))
+                                 : from_double(to_double(x) * to_double(acc));
+      }
+    } else {
+      acc = read_num(in_dt, in, base);
+      for (int64_t k = 1; k < red; k++) {
+        num x = read_num(in_dt, in, base + k * inner);
+        acc = op == REF_RED_MAX ? nf_max(acc, x) : nf_min(acc, x);
+      }
+    }
+    int st = write_num(out_dt, acc, out, o);
+    if (st != REF_OK) {
+#pragma omp critical
+      status = st;
+    }
+  }
+  return status;
+}
+
+/* non_finite_gt / non_finite_lt, binary_backend.ex:1377-1391 */
+static int nf_gt(num x, num y) {
+  if (x.k == K_NAN || y.k == K_NAN) return 0;
+  if (y.k == K_INF) return 0;
+  if (x.k == K_INF) return 1;
+  if (x.k == K_NINF) return 0;
+  if (y.k == K_NINF) return 1;
+  return num_cmp(x, y) > 0;
+}
+static int nf_lt(num x, num y) {
+  if (x.k == K_NAN || y.k == K_NAN) return 0;
+  if (x.k == K_INF) return 0;
+  if (y.k == K_INF) return 1;
+  if (y.k == K_NINF) return 0;
+  if (x.k == K_NINF) return 1;
+  return num_cmp(x, y) < 0;
+}
+static int nf_same(num x, num y) { /* `&1 == &2` on Erlang terms of the tie_break: :high clause */
+  if (is_atom(x) || is_atom(y)) return x.k == y.k;
+  return num_cmp(x, y) == 0;
+}
+
+int ref_argreduce(int op, int tie, int in_dt, int out_dt, int64_t outer, int64_t red,
+                  int64_t inner, const void *in, void *out) {
+  if (ref_dtype_size(in_dt) < 0 || ref_dtype_size(out_dt) < 0 || is_float_dt(out_dt))
+    return fail(REF_EARG, "bad argument");
+  int status = REF_OK;
+  int64_t nout = outer * inner;
+#pragma omp parallel for num_threads(nthreads()) schedule(static) if (nout * red > 65536 && nout > 1)
+  for (int64_t o = 0; o < nout; o++) {
+    int64_t ou = o / inner, iv = o % inner;
+    int64_t base = ou * red * inner + iv;
+    num cur = mk_int(0);
+    int64_t cur_i = -1; /* {0, :first, -1} */
+    for (int64_t k = 0; k < red; k++) {
+      num x = read_num(in_dt, in, base + k * inner);
+      int take;
+      if (cur_i < 0 || x.k == K_NAN) take = 1; /* any NaN replaces: the last NaN wins */
+      else {
+        int strict = op == REF_ARGMAX ? nf_gt(x, cur) : nf_lt(x, cur);
+        take = strict || (tie == REF_TIE_HIGH && nf_same(x, cur));
+      }
+      if (take) { cur = x; cur_i = k; }
+    }
+    int st = write_num(out_dt, mk_int(cur_i), out, o);
+    if (st != REF_OK) {
+#pragma omp critical
+      status = st;
+    }
+  }
+  return status;
+}
+
+/* ---- dot (binary_backend.ex:549-559, 2362-2385) ----------------------------------------- */
+
+static void to_double_array(int dt, const void *p, int64_t n, double *dst) {
+#pragma omp parallel for num_threads(nthreads()) schedule(static) if (n > 65536)
+  for (int64_t i = 0; i < n; i++) dst[i] = to_double(read_num(dt, p, i));
+}
+
+int ref_dot(int l_dt, int r_dt, int out_dt, int64_t batch, int64_t M, int64_t N, int64_t K,
+            const void *l, const void *r, void *out) {
+  if (ref_dtype_size(l_dt) < 0 || ref_dtype_size(r_dt) < 0 || ref_dtype_size(out_dt) < 0)
+    return fail(REF_EARG, "bad dtype");
+  int status = REF_OK;
+  int any_float = is_float_dt(l_dt) || is_float_dt(r_dt);
+  if (!any_float) {
+    /* integers: res = x * y + acc on unbounded integers from 0; encode once.  The sum is kept
+     * in __int128 (exact while |sum| < 2^127, i.e. for every operand narrower than 64 bits). */
+#pragma omp parallel for num_threads(nthreads()) schedule(static) collapse(2) if (batch * M * N * K > 65536)
+    for (int64_t b = 0; b < batch; b++)
+      for (int64_t i = 0; i < M; i++)
+        for (int64_t j = 0; j < N; j++) {
+          i128 acc = 0;
+          for (int64_t k = 0; k < K; k++) {
+            num x = read_num(l_dt, l, (b * M + i) * K + k), y = read_num(r_dt, r, (b * N + j) * K + k);
+            acc = (i128)((u128)wrap_mul(x.i, y.i) + (u128)acc);
+          }
+          int st = write_num(out_dt, mk_int(acc), out, (b * M + i) * N + j);
+          if (st != REF_OK) {
+#pragma omp critical
+            status = st;
+          }
+        }
+    return status;
+  }
+  /* floats (or mixed): every step is `x * y + acc` in IEEE double -- two roundings, no FMA --
+   * sequential over k for each output; IEEE arithmetic on inf/nan stands in for the atom
+   * clauses of Complex.multiply/add.  Outputs are independent, so the loop nest may run them
+   * side by side (vectorised over j) without changing any output's own operation order. */
+  double *ld = malloc(sizeof(double) * (size_t)(batch * M * K > 0 ? batch * M * K : 1));
+  double *rt = malloc(sizeof(double) * (size_t)(batch * N * K > 0 ? batch * N * K : 1));
+  if (!ld || !rt) { free(ld); free(rt); return fail(REF_EARG, "out of memory"); }
+  to_double_array(l_dt, l, batch * M * K, ld);
+  {
+    double *tmp = malloc(sizeof(double) * (size_t)(batch * N * K > 0 ? batch * N * K : 1));
+    if (!tmp) { free(ld); free(rt); return fail(REF_EARG, "out of memory"); }
+    to_double_array(r_dt, r, batch * N * K, tmp);
+    /* [b][j][k] -> [b][k][j] so the j loop is unit stride */
+#pragma omp parallel for num_threads(nthreads()) schedule(static) collapse(2) if (batch * N * K > 65536)
+    for (int64_t b = 0; b < batch; b++)
+      for (int64_t j = 0; j < N; j++)
+        for (int64_t k = 0; k < K; k++) rt[(b * K + k) * N + j] = tmp[(b * N + j) * K + k];
+    free(tmp);
+  }
+#pragma omp parallel num_threads(nthreads()) if (batch * M * N * K > 65536)
+  {
+    double *acc = malloc(sizeof(double) * (size_t)(N > 0 ? N : 1));
+#pragma omp for schedule(static) collapse(2)
+    for (int64_t b = 0; b < batch; b++)
+      for (int64_t i = 0; i < M; i++) {
+        for (int64_t j = 0; j < N; j++) acc[j] = 0.0;
+        const double *lrow = ld + (b * M + i) * K;
+        for (int64_t k = 0; k < K; k++) {
+          double x = lrow[k];
+          const double *rrow = rt + (b * K + k) * N;
+          for (int64_t j = 0; j < N; j++) acc[j] = x * rrow[j] + acc[j];
+        }
+        for (int64_t j = 0; j < N; j++) {
+          int st = write_num(out_dt, K == 0 ? mk_int(0) : from_double(acc[j]), out, (b * M + i) * N + j);
+          if (st != REF_OK) {
+#pragma omp critical
+            status = st;
+          }
+        }
+      }
+    free(acc);
+  }
+  free(ld);
+  free(rt);
+  return status;
+}
+
+/* ---- data movement ---------------------------------------------------------------------- */
+
+int ref_transpose(int elem_bytes, int rank, const int64_t *in_dims, const int *perm,
+                  const void *in, void *out) {
+  if (rank < 0 || rank > 16 || elem_bytes <= 0) return fail(REF_EARG, "bad argument");
+  int64_t in_str[16], out_dims[16], n = 1;
+  int64_t s = 1;
+  for (int a = rank - 1; a >= 0; a--) { in_str[a] = s; s *= in_dims[a]; }
+  for (int a = 0; a < rank; a++) { out_dims[a] = in_dims[perm[a]]; n *= out_dims[a]; }
+  for (int64_t i = 0; i < n; i++) {
+    int64_t rem = i, off = 0;
+    for (int a = rank - 1; a >= 0; a--) {
+      off += (rem % out_dims[a]) * in_str[perm[a]];
+      rem /= out_dims[a];
+    }
+    memcpy((char *)out + i * elem_bytes, (const char *)in + off * elem_bytes, (size_t)elem_bytes);
+  }
+  return REF_OK;
+}
+
+int ref_broadcast(int elem_bytes, int rank, const int64_t *out_dims, const int64_t *in_strides,
+                  const void *in, void *out) {
+  if (rank < 0 || rank > 16 || elem_bytes <= 0) return fail(REF_EARG, "bad argument");
+  int64_t n = 1;
+  for (int a = 0; a < rank; a++) n *= out_dims[a];
+  for (int64_t i = 0; i < n; i++) {
+    int64_t rem = i, off = 0;
+    for (int a = rank - 1; a >= 0; a--) {
+      off += (rem % out_dims[a]) * in_strides[a];
+      rem /= out_dims[a];
+    }
+    memcpy((char *)out + i * elem_bytes, (const char *)in + off * elem_bytes, (size_t)elem_bytes);
+  }
+  return REF_OK;
+}
+
+int ref_gather(int elem_bytes, int rank, const int64_t *t_dims, int idx_dt, int64_t n_tuples,
+               int depth, const void *t, const void *idx, void *out) {
+  if (rank < 0 || rank > 16 || depth < 0 || depth > rank || elem_bytes <= 0 ||
+      ref_dtype_size(idx_dt) < 0 || is_float_dt(idx_dt))
+    return fail(REF_EARG, "bad argument");
+  int64_t slice = 1;
+  for (int a = depth; a < rank; a++) slice *= t_dims[a];
+  for (int64_t i = 0; i < n_tuples; i++) {
+    int64_t off = 0;
+    /* index_to_binary_offset/2, binary_backend.ex:1942-1959 */
+    for (int a = 0; a < depth; a++) {
+      i128 v = read_num(idx_dt, idx, i * depth + a).i;
+      if (v < 0 || v >= t_dims[a]) {
+        char shape[128] = "{";
+        for (int q = 0; q < rank; q++) {
+          char one[32];
+          snprintf(one, sizeof one, q ? ", %lld" : "%lld", (long long)t_dims[q]);
+          strncat(shape, one, sizeof shape - strlen(shape) - 2);
+        }
+        strcat(shape, "}");
+        snprintf(g_err, sizeof g_err, "index %lld is out of bounds for axis %d in shape %s",
+                 (long long)v, a, shape);
+        return REF_ERAISE;
+      }
+      int64_t rest = 1;
+      for (int q = a + 1; q < rank; q++) rest *= t_dims[q];
+      off += (int64_t)v * rest;
+    }
+    memcpy((char *)out + i * slice * elem_bytes, (const char *)t + off * elem_bytes,
+           (size_t)(slice * elem_bytes));
+  }
+  return REF_OK;
+}
