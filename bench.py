@@ -1,0 +1,178 @@
+#!/usr/bin/env python3
+"""Benchmark of the HipNx hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-suite] [--no-cpu]
+
+Headline workload (the configuration the metric is quoted on): `Nx.dot` of bf16 {4096,4096} x
+{4096,4096}, f32 accumulation on MFMA, bf16 output -- one step = one `dot` callback through the
+C ABI, inputs resident in HBM.  Prints ONE JSON line; `value` is TFLOP/s over K timed steps
+(wall clock between two device synchronisations).  `roofline` is measured live with HIP events on
+the stream the kernels are launched on.  `suite` carries the other configurations (GB/s or
+TFLOP/s and their roofline fractions), `cpu_baseline` the CPU restatement of the reference on a
+bounded sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_HBM_GBS = 8000.0
+PEAK = {"bf16": 2500.0, "f16": 2500.0, "s8": 5000.0, "f32": 157.3}  # dense MFMA TFLOP/s (TOP/s)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-suite", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this build runs on exactly one GPU (no sharding, no collectives); use --gpus 1")
+
+    from nx_amd import nx as Nx
+    from nx_amd import workloads as W
+    from nx_amd import backend as B
+    from nx_amd.backend import HipNxBackend as H
+    from nx_amd.tensor import template
+
+    def put(arr, ty):
+        return H.from_numpy(template(ty, arr.shape), arr)
+
+    def timed(fn, steps, warmup):
+        """(wall ms per step, device ms per step): K calls between two synchronisations, with a
+        HIP-event pair recorded on the context's stream around the same region."""
+        for _ in range(warmup):
+            keep = fn()
+        B.sync()
+        t0 = time.perf_counter()
+        B.timer_start()
+        for _ in range(steps):
+            keep = fn()  # noqa: F841 - results are dropped (returned to the pool) as a caller would
+        dev_ms = B.timer_stop()
+        B.sync()
+        wall_ms = (time.perf_counter() - t0) * 1e3
+        return wall_ms / steps, dev_ms / steps
+
+    # ---- headline: config 2, dense bf16 GEMM ------------------------------------------------
+    n = 4096
+    a_np, b_np = W.dense_gemm_bf16(n=n)
+    a, b = put(a_np, "bf16"), put(b_np, "bf16")
+    flop = 2.0 * n * n * n
+    wall_ms, dev_ms = timed(lambda: Nx.dot(a, b), args.steps, args.warmup)
+    value = flop / (wall_ms * 1e-3) / 1e12
+    achieved = flop / (dev_ms * 1e-3) / 1e12
+
+    result = {
+        "metric": "Nx.dot TFLOP/s (bf16, s8->s32) + elementwise/reduce GB/s, % of MI355X peak",
+        "value": round(value, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "dense GEMM: Nx.dot bf16 {4096,4096} x {4096,4096}, f32 accumulate, bf16 output "
+                               "(BASELINE configs[1])", "seed": 2},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK["bf16"], "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK["bf16"], 4), "traffic": None,
+                     "kernel": "dot callback (gemm kernel + operand re-layout, if any), HIP events on the launch stream"},
+    }
+
+    # ---- the other configurations -----------------------------------------------------------
+    if not args.no_suite:
+        suite = {}
+        steps, warm = max(args.steps // 2, 10), 5
+
+        def entry(name, work, unit, ms, peak, bound):
+            rate = work / (ms * 1e-3) / (1e12 if unit == "TFLOP/s" or unit == "TOP/s" else 1e9)
+            suite[name] = {"ms": round(ms, 5), "achieved": round(rate, 2), "unit": unit, "bound": bound,
+                           "peak": peak, "frac": round(rate / peak, 4)}
+
+        # K-inner operands: the gemm kernel alone (no re-layout pass)
+        bt = Nx.transpose(b)
+        _, ms = timed(lambda: Nx.dot(a, [1], bt, [1]), steps, warm)
+        entry("dot_bf16_4096_kinner", flop, "TFLOP/s", ms, PEAK["bf16"], "mfma")
+        fa, fb = W.dense_gemm_f32()
+        fa, fb = put(fa, "f32"), put(fb, "f32")
+        _, ms = timed(lambda: Nx.dot(fa, fb), steps, warm)
+        entry("dot_f32_2048", 2.0 * 2048 ** 3, "TFLOP/s", ms, PEAK["f32"], "mfma")
+        sa, sb = W.dense_gemm_s8()
+        sa, sb = put(sa, "s8"), put(sb, "s8")
+        _, ms = timed(lambda: Nx.dot(sa, sb, out_type="s32"), steps, warm)
+        entry("dot_s8_4096_s32", flop, "TOP/s", ms, PEAK["s8"], "mfma")
+        del fa, fb, sa, sb, bt
+
+        # config 1 (and a HBM-resident scale of it)
+        for nn in (1024, 16384):
+            x, y = W.elementwise_reduce(n=nn)
+            x, y = put(x, "f32"), put(y, "f32")
+            N = nn * nn
+            _, ms = timed(lambda: Nx.add(x, y), steps, warm)
+            entry(f"add_f32_{nn}", 12.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+            _, ms = timed(lambda: Nx.multiply(x, 0.5), steps, warm)
+            entry(f"multiply_scalar_f32_{nn}", 8.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+            _, ms = timed(lambda: Nx.exp(x), steps, warm)
+            entry(f"exp_f32_{nn}", 8.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+            _, ms = timed(lambda: Nx.sum(x, axes=[1]), steps, warm)
+            entry(f"sum_rows_f32_{nn}", 4.0 * N + 4.0 * nn, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+            del x, y
+
+        # config 3: attention scores + softmax chain
+        q, k = W.attention_scores()
+        q, k = put(q, "bf16"), put(k, "bf16")
+        _, ms = timed(lambda: Nx.dot(q, [2], [0], k, [2], [0]), steps, warm)
+        entry("dot_qk_bf16_32x512x64", 20971520.0, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+        s = Nx.dot(q, [2], [0], k, [2], [0])
+
+        def softmax():
+            z = Nx.multiply(Nx.as_type(s, "f32"), 0.125)
+            e = Nx.exp(Nx.subtract(z, Nx.reduce_max(z, axes=[2], keep_axes=True)))
+            return Nx.divide(e, Nx.sum(e, axes=[2], keep_axes=True))
+        _, ms = timed(softmax, steps, warm)
+        entry("softmax_chain_32x512x512", 386138112.0, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+        del q, k, s
+
+        # config 4: int8 weight-only linear
+        w, xq, sc = W.int8_linear()
+        w, xq, sc = put(w, "s8"), put(xq, "s8"), put(sc, "f32")
+        _, ms = timed(lambda: Nx.dot(xq, [1], w, [1], out_type="s32"), steps, warm)
+        entry("dot_s8_w8_64x11008x4096", 48168960.0, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+        suite["dot_s8_w8_64x11008x4096"]["tops"] = round(5771362304.0 / (ms * 1e-3) / 1e12, 2)
+        del w, xq, sc
+
+        # config 5: argmax + take
+        logits, table, _ = W.logits_and_table()
+        logits, table = put(logits, "f32"), put(table, "bf16")
+        _, ms = timed(lambda: Nx.argmax(logits, axis=1, type="u32"), steps, warm)
+        entry("argmax_f32_8192x32000", 1048608768.0, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+        idx = Nx.argmax(logits, axis=1, type="u32")
+        _, ms = timed(lambda: Nx.take(table, idx), steps, warm)
+        entry("take_bf16_8192_of_32000x4096", 134250496.0, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+        del logits, table, idx
+        result["suite"] = suite
+
+    # ---- CPU baseline: the reference-semantics restatement on a bounded sample -----------------
+    if not args.no_cpu:
+        from oracle import binary_backend as O
+        threads = min(os.cpu_count() or 1, 16)
+        O.set_threads(threads)
+        rows = 2048
+        oa = O.BinaryBackend.from_binary(template("bf16", (rows, n)), a_np[:rows].tobytes())
+        ob = O.BinaryBackend.from_binary(template("bf16", (n, n)), b_np.tobytes())
+        t0 = time.perf_counter()
+        Nx.dot(oa, ob)
+        dt = time.perf_counter() - t0
+        result["cpu_baseline"] = {
+            "value": round(2.0 * rows * n * n / dt / 1e12, 6), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": f"first {rows} of 4096 output rows of the same bf16 GEMM (f64 sequential accumulation, "
+                      f"reference semantics), {dt:.1f} s"}
+
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -24,13 +24,8 @@ from . import shape as S
 from . import types as T
 from .tensor import Tensor, number_to_binary
 
-BINARY_OPS = ["add", "subtract", "multiply", "divide", "pow", "remainder", "atan2", "min", "max", "quotient",
-              "bitwise_and", "bitwise_or", "bitwise_xor", "left_shift", "right_shift", "equal", "not_equal",
-              "greater", "less", "greater_equal", "less_equal", "logical_and", "logical_or", "logical_xor"]
-UNARY_OPS = ["exp", "expm1", "log", "log1p", "sigmoid", "cos", "sin", "tan", "cosh", "sinh", "tanh", "acos", "asin",
-             "atan", "acosh", "asinh", "atanh", "sqrt", "rsqrt", "cbrt", "erf", "erfc", "erf_inv", "abs",
-             "bitwise_not", "ceil", "floor", "negate", "round", "sign", "count_leading_zeros", "population_count",
-             "is_nan", "is_infinity"]
+from .backend_names import BINARY_OPS, UNARY_OPS  # noqa: E402
+
 RED_SUM, RED_MAX, RED_MIN, RED_PRODUCT = 0, 1, 2, 3
 K_INNER, K_OUTER = 0, 1
 OOB_RAISE, OOB_CLAMP = 0, 1

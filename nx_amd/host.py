@@ -78,6 +78,11 @@ def _raise(name):
     return classmethod(fn)
 
 
-for _n in ["add", "subtract", "multiply", "divide", "exp", "sum", "reduce_max", "reduce_min", "argmax", "argmin",
-           "dot", "gather", "transpose", "broadcast", "as_type", "block"]:
-    setattr(HostBinary, _n, _raise(_n))
+def _install():
+    from .backend_names import BINARY_OPS, UNARY_OPS
+    for _n in BINARY_OPS + UNARY_OPS + ["sum", "product", "reduce_max", "reduce_min", "argmax", "argmin", "dot",
+                                        "gather", "transpose", "broadcast", "as_type", "block"]:
+        setattr(HostBinary, _n, _raise(_n))
+
+
+_install()

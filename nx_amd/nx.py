@@ -8,6 +8,7 @@ run unchanged.  Vectorisation and axis names are not modelled.
 """
 from __future__ import annotations
 
+import builtins
 import threading
 from dataclasses import dataclass
 from math import prod
@@ -101,7 +102,7 @@ def to_tensor(value) -> Tensor:
 
 def to_binary(t: Tensor, limit=None) -> bytes:
     """Nx.to_binary/2 (nx.ex:2121-2133); `limit` counts elements."""
-    limit = t.size if limit is None else min(limit, t.size)
+    limit = t.size if limit is None else builtins.min(limit, t.size)
     return type(t.data).to_binary(t, limit)
 
 

@@ -14,6 +14,12 @@ from nx_amd.tensor import Tensor, binary_to_numpy, list_to_binary, template, to_
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 
 
+def seed_of(*parts) -> int:
+    """Deterministic seed from test parameters (Python's hash() of strings changes per process)."""
+    import zlib
+    return zlib.crc32(repr(parts).encode())
+
+
 def load_cases(name="nx_known_answers.json"):
     with open(os.path.join(GOLDEN, name)) as f:
         return json.load(f)["cases"]

@@ -1,0 +1,125 @@
+"""Device Nx.dot against the CPU oracle.
+
+Bar: integer results bit-exact (s8 x s8 -> s32 / s8 on MFMA, everything else on the plain
+kernel); float results within the K-scaled bound
+    |d| <= 2K * 2^-24 * sum_k |a_k b_k|  +  1 ulp(out type) * |ref|
+(the device accumulates in f32 on MFMA, the reference sequentially in f64), and for f64 operands
+within 1e-13 relative to sum|a_k b_k|."""
+import numpy as np
+import pytest
+
+from nx_amd import nx as Nx
+from nx_amd import types as T
+from support import assert_bits_equal, from_numpy, seed_of, values
+from test_gpu_elementwise import both, rand_raw
+
+pytestmark = pytest.mark.gpu
+
+ULP = {("bf", 16): 2.0 ** -7, ("f", 16): 2.0 ** -10, ("f", 32): 2.0 ** -23, ("f", 64): 2.0 ** -52}
+
+
+def check_float_dot(got, want, a64, b64, eq, K, what):
+    """a64/b64: decoded operands; eq: einsum spec producing the output from |a|, |b|."""
+    assert got.type == want.type and got.shape == want.shape, what
+    mag = np.einsum(eq, np.abs(a64), np.abs(b64)).reshape(got.shape)
+    ref = values(want)
+    acc = 2.0 ** -24 if got.type != ("f", 64) and True else 2.0 ** -50
+    bound = 2 * max(K, 1) * acc * mag + ULP[got.type] * np.abs(ref) + 1e-30
+    err = np.abs(values(got) - ref)
+    assert (err <= bound).all(), f"{what}: max err/bound {np.max(err / bound):.3f}"
+
+
+MNK = [(128, 128, 64), (256, 256, 256), (130, 70, 136), (1, 1, 8), (17, 300, 1000), (512, 64, 2048), (64, 11008 // 8, 4096),
+       (33, 33, 40), (200, 129, 8), (5, 7, 3), (64, 64, 7)]
+
+
+@pytest.mark.parametrize("M,N,K", MNK)
+@pytest.mark.parametrize("ty", ["bf16", "f16", "f32", "f64"])
+@pytest.mark.parametrize("layout", ["nn", "nt", "tn", "tt"])
+def test_float_matmul_layouts(M, N, K, ty, layout, hip, oracle):
+    if ty == "f64" and M * N * K > 5_000_000:
+        pytest.skip("plain-kernel path: covered at smaller sizes")
+    rng = np.random.default_rng(seed_of(M, N, K, ty))
+    a_shape = (M, K) if layout[0] == "n" else (K, M)
+    b_shape = (K, N) if layout[1] == "n" else (N, K)
+    a, b = rand_raw(rng, ty, a_shape, lo=-1, hi=1), rand_raw(rng, ty, b_shape, lo=-1, hi=1)
+    ha, oa = both(a, ty, hip, oracle)
+    hb, ob = both(b, ty, hip, oracle)
+    c1 = [1] if layout[0] == "n" else [0]
+    c2 = [0] if layout[1] == "n" else [1]
+    got, want = Nx.dot(ha, c1, hb, c2), Nx.dot(oa, c1, ob, c2)
+    eq = ("mk" if layout[0] == "n" else "km") + "," + ("kn" if layout[1] == "n" else "nk") + "->mn"
+    check_float_dot(got, want, values(oa), values(ob), eq, K, f"dot {ty} {layout} {M}x{N}x{K}")
+
+
+@pytest.mark.parametrize("M,N,K", [(64, 344, 4096), (128, 128, 128), (7, 9, 16), (130, 70, 1024), (64, 64, 48), (3, 5, 7)])
+@pytest.mark.parametrize("out_type", ["s32", "s8", "s64"])
+def test_int8_dot_is_bit_exact(M, N, K, out_type, hip, oracle):
+    rng = np.random.default_rng(seed_of(M, N, K))
+    x = rng.integers(-127, 128, size=(M, K)).astype(np.int8)
+    w = rng.integers(-127, 128, size=(N, K)).astype(np.int8)
+    hx, ox = both(x, "s8", hip, oracle)
+    hw, ow = both(w, "s8", hip, oracle)
+    ot = None if out_type == "s8" else out_type  # s8 is what the public API infers (wraps)
+    assert_bits_equal(Nx.dot(hx, [1], hw, [1], out_type=ot), Nx.dot(ox, [1], ow, [1], out_type=ot), f"s8 dot -> {out_type}")
+    # exact closed form as an independent check of both
+    exact = x.astype(np.int64) @ w.astype(np.int64).T
+    got = hip.to_numpy(Nx.dot(hx, [1], hw, [1], out_type="s32"))
+    assert np.array_equal(got, exact.astype(np.int32))
+
+
+@pytest.mark.parametrize("lt,rt", [("s32", "s32"), ("u8", "u8"), ("s16", "s64"), ("u32", "s8"), ("s64", "s64"), ("u8", "s8")])
+def test_integer_dot_is_bit_exact(lt, rt, hip, oracle):
+    rng = np.random.default_rng(seed_of(lt, rt))
+    a, b = rand_raw(rng, lt, (19, 45)), rand_raw(rng, rt, (45, 23))
+    ha, oa = both(a, lt, hip, oracle)
+    hb, ob = both(b, rt, hip, oracle)
+    assert_bits_equal(Nx.dot(ha, hb), Nx.dot(oa, ob), f"dot {lt} {rt}")
+
+
+@pytest.mark.parametrize("lt,rt", [("f32", "bf16"), ("s8", "f32"), ("f16", "f32"), ("f64", "f32")])
+def test_mixed_type_dot(lt, rt, hip, oracle):
+    rng = np.random.default_rng(seed_of(lt, rt))
+    a, b = rand_raw(rng, lt, (40, 64), lo=-1, hi=1), rand_raw(rng, rt, (64, 24), lo=-1, hi=1)
+    ha, oa = both(a, lt, hip, oracle)
+    hb, ob = both(b, rt, hip, oracle)
+    check_float_dot(Nx.dot(ha, hb), Nx.dot(oa, ob), values(oa), values(ob), "mk,kn->mn", 64, f"dot {lt} {rt}")
+
+
+BATCHED = [((32, 64, 64), [2], [0], (32, 48, 64), [2], [0], "bmk,bnk->bmn"),
+           ((4, 16, 40), [1], [0], (4, 16, 24), [1], [0], "bkm,bkn->bmn"),
+           ((3, 5, 32, 8), [3], [0, 1], (3, 5, 8, 16), [2], [0, 1], "abmk,abkn->abmn"),
+           ((2, 8, 16, 4), [1, 3], [0], (2, 4, 8, 6), [2, 1], [0], "bkml,blkn->bmn"),
+           ((6, 10), [0, 1], [], (10, 6), [1, 0], [], "ab,ba->"),
+           ((4, 6, 5), [1], [], (3, 6, 2), [1], [], "amb,cmd->abcd"),
+           ((8, 3), [], [], (2, 5), [], [], "ab,cd->abcd")]
+
+
+@pytest.mark.parametrize("case", BATCHED, ids=[c[-1] for c in BATCHED])
+@pytest.mark.parametrize("ty", ["bf16", "f32", "s32", "s8"])
+def test_general_contraction_and_batch_axes(case, ty, hip, oracle):
+    ls, c1, b1, rs, c2, b2, eq = case
+    rng = np.random.default_rng(seed_of(eq, ty))
+    a, b = rand_raw(rng, ty, ls, lo=-1, hi=1), rand_raw(rng, ty, rs, lo=-1, hi=1)
+    ha, oa = both(a, ty, hip, oracle)
+    hb, ob = both(b, ty, hip, oracle)
+    got, want = Nx.dot(ha, c1, b1, hb, c2, b2), Nx.dot(oa, c1, b1, ob, c2, b2)
+    if T.is_integer(T.normalize(ty)):
+        assert_bits_equal(got, want, f"dot {eq} {ty}")
+    else:
+        K = int(np.prod([ls[x] for x in c1])) if c1 else 1
+        check_float_dot(got, want, values(oa), values(ob), eq, K, f"dot {eq} {ty}")
+
+
+def test_dot_matches_closed_form_on_small_integers_in_bf16(hip):
+    """Small-integer operands make every partial sum exact in f32: the MFMA result must equal the
+    integer matrix product exactly, whatever the accumulation order."""
+    rng = np.random.default_rng(2)
+    a = rng.integers(-4, 5, size=(256, 512))
+    b = rng.integers(-4, 5, size=(512, 384))
+    bits = lambda m: (m.astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    ha, hb = from_numpy(bits(a), "bf16", hip), from_numpy(bits(b), "bf16", hip)
+    got = values(Nx.dot(Nx.as_type(ha, "f32"), Nx.as_type(hb, "f32")))
+    assert np.array_equal(got, (a @ b).astype(np.float64))
+    got_bf = values(Nx.dot(ha, hb, out_type="f32"))
+    assert np.array_equal(got_bf, (a @ b).astype(np.float64))

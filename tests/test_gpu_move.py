@@ -1,0 +1,98 @@
+"""Device take / gather / transpose / broadcast against the CPU oracle: pure copies, bit-exact."""
+import numpy as np
+import pytest
+
+from nx_amd import nx as Nx
+from support import assert_bits_equal, from_numpy, seed_of
+from test_gpu_elementwise import both, rand_raw
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("shape,perm", [((64, 48), [1, 0]), ((5, 64, 48), [0, 2, 1]), ((3, 4, 5, 6), [3, 1, 0, 2]),
+                                         ((2, 3, 4), [1, 0, 2]), ((1, 7, 1, 9), [3, 2, 1, 0]), ((130, 70), [1, 0]),
+                                         ((2, 2, 2, 2, 2, 2, 3), [6, 0, 5, 1, 4, 2, 3]), ((4096, 33), [1, 0])])
+@pytest.mark.parametrize("ty", ["u8", "bf16", "f32", "s64"])
+def test_transpose(shape, perm, ty, hip, oracle):
+    rng = np.random.default_rng(seed_of(shape, perm, ty))
+    x = rand_raw(rng, ty, shape)
+    hx, ox = both(x, ty, hip, oracle)
+    assert_bits_equal(Nx.transpose(hx, perm), Nx.transpose(ox, perm), f"transpose {shape} {perm}")
+
+
+@pytest.mark.parametrize("shape,new,axes", [((3,), (4, 3), None), ((3, 1), (3, 5), None), ((2,), (2, 6), [0]),
+                                             ((), (7, 3), None), ((1, 4, 1), (5, 4, 9), None), ((4, 2), (4, 3, 2), [0, 2])])
+def test_broadcast(shape, new, axes, hip, oracle):
+    rng = np.random.default_rng(seed_of(shape, new))
+    x = rand_raw(rng, "f32", shape)
+    hx, ox = both(x, "f32", hip, oracle)
+    assert_bits_equal(Nx.broadcast(hx, new, axes), Nx.broadcast(ox, new, axes), f"broadcast {shape}->{new}")
+
+
+@pytest.mark.parametrize("rows,cols,ty", [(1000, 64, "bf16"), (1000, 4096, "bf16"), (77, 3, "f32"), (500, 1, "u8"),
+                                           (300, 17, "s64"), (32000, 128, "bf16"), (50, 1000, "f32")])
+@pytest.mark.parametrize("idx_ty", ["u32", "s32", "s64", "u8"])
+def test_take_rows(rows, cols, ty, idx_ty, hip, oracle):
+    rng = np.random.default_rng(seed_of(rows, cols, ty, idx_ty))
+    table = rand_raw(rng, ty, (rows, cols))
+    hi = min(rows, 256 if idx_ty == "u8" else rows)
+    idx = rng.integers(0, hi, size=(4, 333)).astype(np.dtype({"u32": np.uint32, "s32": np.int32, "s64": np.int64, "u8": np.uint8}[idx_ty]))
+    ht, ot = both(table, ty, hip, oracle)
+    hi_, oi = both(idx, idx_ty, hip, oracle)
+    got, want = Nx.take(ht, hi_), Nx.take(ot, oi)
+    assert_bits_equal(got, want, f"take {rows}x{cols} {ty} idx {idx_ty}")
+    assert np.array_equal(hip.to_numpy(got), table[idx.astype(np.int64)])  # closed form
+
+
+@pytest.mark.parametrize("axis", [0, 1, 2, -1])
+def test_take_other_axes(axis, hip, oracle):
+    rng = np.random.default_rng(axis + 10)
+    t = rand_raw(rng, "f32", (6, 7, 8))
+    idx = rng.integers(0, 6, size=(3, 2)).astype(np.int32)
+    ht, ot = both(t, "f32", hip, oracle)
+    hi_, oi = both(idx, "s32", hip, oracle)
+    got = Nx.take(ht, hi_, axis=axis)
+    assert_bits_equal(got, Nx.take(ot, oi, axis=axis), f"take axis {axis}")
+    assert np.array_equal(hip.to_numpy(got), np.take(t, idx, axis=axis))
+
+
+@pytest.mark.parametrize("axes", [None, [0], [1], [0, 2], [2, 0], [1, 2]])
+def test_gather(axes, hip, oracle):
+    rng = np.random.default_rng(7)
+    t = rand_raw(rng, "s32", (5, 6, 7))
+    depth = 3 if axes is None else len(axes)
+    dims = [5, 6, 7] if axes is None else [[5, 6, 7][a] for a in axes]
+    idx = np.stack([rng.integers(0, d, size=(4, 9)) for d in dims], axis=-1).astype(np.int64)
+    ht, ot = both(t, "s32", hip, oracle)
+    hi_, oi = both(idx, "s64", hip, oracle)
+    assert_bits_equal(Nx.gather(ht, hi_, axes=axes), Nx.gather(ot, oi, axes=axes), f"gather axes={axes}")
+
+
+def test_gather_out_of_bounds_raises_like_the_reference(hip, oracle):
+    from nx_amd._lib import HipNxArgumentError
+    from oracle.binary_backend import ReferenceRaises
+    t = np.arange(12, dtype=np.int32).reshape(3, 4)
+    for bad in ([[0, 0], [3, 1], [9, 9]], [[2, -1]], [[0, 4]], [[-7, 0]]):
+        idx = np.array(bad, dtype=np.int32)
+        ht, ot = both(t, "s32", hip, oracle)
+        hi_, oi = both(idx, "s32", hip, oracle)
+        with pytest.raises(ReferenceRaises) as want:
+            Nx.gather(ot, oi)
+        with pytest.raises(HipNxArgumentError) as got:
+            Nx.gather(ht, hi_)
+        assert str(want.value) in str(got.value)
+    # and the first offender in index order is the one reported
+    idx = np.zeros((5000, 1), dtype=np.int32)
+    idx[4000], idx[1234], idx[4999] = 77, -5, 99
+    ht = from_numpy(t, "s32", hip)
+    with pytest.raises(HipNxArgumentError, match="index -5 is out of bounds for axis 0 in shape \\{3, 4\\}"):
+        Nx.gather(ht, from_numpy(idx, "s32", hip))
+
+
+def test_gather_clamp_policy_matches_the_compiled_backends(hip):
+    """EXLA clamps out-of-range indices (exla/test/exla/defn/expr_test.exs:3478-3481):
+    gather([[1,2],[3,4]], [[-1,-1],[10,11],[-1,10]]) -> [1, 4, 2]."""
+    t = from_numpy(np.array([[1, 2], [3, 4]], dtype=np.int32), "s32", hip)
+    idx = from_numpy(np.array([[-1, -1], [10, 11], [-1, 10]], dtype=np.int32), "s32", hip)
+    from nx_amd.backend import OOB_CLAMP
+    assert hip.to_numpy(Nx.gather(t, idx, oob_policy=OOB_CLAMP)).tolist() == [1, 4, 2]

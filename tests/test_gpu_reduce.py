@@ -1,0 +1,121 @@
+"""Device reductions (sum / product / reduce_max / reduce_min / argmax / argmin) against the CPU
+oracle.  Integer and index results bit-exact; float sums within K * 2^-24 * sum|x| + 1 ulp (the
+device folds in f64 in tree order, the reference in f64 sequentially); max/min exact bits."""
+import numpy as np
+import pytest
+
+from nx_amd import nx as Nx
+from nx_amd import types as T
+from support import assert_bits_equal, from_numpy, seed_of, values
+from test_gpu_elementwise import both, rand_raw
+
+pytestmark = pytest.mark.gpu
+
+SHAPES_AXES = [((1024, 1024), [1]), ((1024, 1024), [0]), ((1024, 1024), None), ((32, 512, 64), [2]),
+               ((32, 512, 64), [1]), ((32, 512, 64), [0]), ((32, 512, 64), [0, 2]), ((32, 512, 64), [1, 2]),
+               ((7, 13), [1]), ((7, 13), [0]), ((5, 3, 9, 2), [1, 3]), ((3, 70001), [1]), ((2, 4097, 3), [1]),
+               ((1, 1), [0]), ((9,), None), ((2, 300000), [1]), ((1500000,), None), ((6, 1, 5), [1])]
+
+
+def sum_bound(x64, axes, out_bits):
+    """K * 2^-24 * sum|x| (+ an ulp of the output type) for the given reduction."""
+    ax = tuple(range(x64.ndim)) if axes is None else tuple(axes)
+    k = int(np.prod([x64.shape[a] for a in ax]))
+    s = np.abs(x64).sum(axis=ax)
+    eps = {64: 2.0 ** -52, 32: 2.0 ** -23, 16: 2.0 ** -7}[out_bits]
+    return k * 2.0 ** -24 * s * (1 if out_bits < 64 else 2.0 ** -29) + eps * np.abs(x64.sum(axis=ax)) + 1e-30
+
+
+@pytest.mark.parametrize("shape,axes", SHAPES_AXES, ids=[f"{s}-{a}" for s, a in SHAPES_AXES])
+@pytest.mark.parametrize("ty", ["f32", "bf16", "f64", "s32", "u8", "s8", "s64"])
+@pytest.mark.parametrize("keep", [False, True])
+def test_sum(shape, axes, ty, keep, hip, oracle):
+    if keep and ty not in ("f32", "s32"):
+        pytest.skip("keep_axes only changes the output shape")
+    rng = np.random.default_rng(seed_of(shape, axes, ty))
+    x = rand_raw(rng, ty, shape, lo=-1, hi=1)
+    hx, ox = both(x, ty, hip, oracle)
+    got, want = Nx.sum(hx, axes=axes, keep_axes=keep), Nx.sum(ox, axes=axes, keep_axes=keep)
+    if T.is_integer(T.normalize(ty)):
+        assert_bits_equal(got, want, f"sum {ty} {shape} {axes}")
+        return
+    assert got.type == want.type and got.shape == want.shape
+    x64 = values(ox)
+    bound = sum_bound(x64, axes, got.type[1] if got.type[0] == "f" else 16).reshape(got.shape)
+    err = np.abs(values(got) - values(want))
+    assert (err <= bound).all(), f"sum {ty} {shape} {axes}: max err {err.max():.3e}"
+    if ty == "f32":  # f64 accumulation on the device: expect the very same rounded f32 almost always
+        same = (hip.to_numpy(got).view(np.uint32) == oracle_raw(want).view(np.uint32)).mean()
+        assert same >= 0.99, f"only {same:.4f} of f32 sums are bit-identical"
+
+
+def oracle_raw(t):
+    from support import raw
+    return raw(t)
+
+
+@pytest.mark.parametrize("shape,axes", SHAPES_AXES[:14], ids=[f"{s}-{a}" for s, a in SHAPES_AXES[:14]])
+@pytest.mark.parametrize("ty", ["f32", "bf16", "f16", "f64", "s32", "u8", "u64", "s64"])
+@pytest.mark.parametrize("op", ["reduce_max", "reduce_min"])
+def test_reduce_max_min_exact(shape, axes, ty, op, hip, oracle):
+    rng = np.random.default_rng(seed_of(shape, axes, ty, op))
+    x = rand_raw(rng, ty, shape, lo=-100, hi=100)
+    if ty == "f32" and x.size > 100:  # NaN is sticky, infinities are ordered
+        flat = x.reshape(-1)
+        flat[rng.integers(0, flat.size, 5)] = np.nan
+        flat[rng.integers(0, flat.size, 5)] = np.inf
+        flat[rng.integers(0, flat.size, 5)] = -np.inf
+    hx, ox = both(x, ty, hip, oracle)
+    assert_bits_equal(getattr(Nx, op)(hx, axes=axes), getattr(Nx, op)(ox, axes=axes), f"{op} {ty} {shape} {axes}")
+
+
+def test_product(hip, oracle):
+    rng = np.random.default_rng(3)
+    x = rng.integers(-3, 4, size=(64, 9)).astype(np.int32)
+    hx, ox = both(x, "s32", hip, oracle)
+    assert_bits_equal(Nx.product(hx, axes=[1]), Nx.product(ox, axes=[1]), "product s32")
+    f = rng.uniform(0.5, 1.5, size=(50, 40)).astype(np.float32)
+    hf, of = both(f, "f32", hip, oracle)
+    from support import assert_all_close
+    assert_all_close(Nx.product(hf, axes=[0]), Nx.product(of, axes=[0]), 1e-5, 0, "product f32")
+
+
+ARG_SHAPES = [((64, 1000), 1), ((64, 1000), 0), ((64, 1000), None), ((4, 33, 7), 1), ((4, 33, 7), 2), ((4, 33, 7), 0),
+              ((3, 70001), 1), ((1300001,), None), ((5, 8), -1), ((1, 1), 0), ((2, 40000, 2), 1)]
+
+
+@pytest.mark.parametrize("shape,axis", ARG_SHAPES, ids=[f"{s}-{a}" for s, a in ARG_SHAPES])
+@pytest.mark.parametrize("ty", ["f32", "bf16", "s32", "u8", "f64"])
+@pytest.mark.parametrize("op", ["argmax", "argmin"])
+@pytest.mark.parametrize("tie", ["low", "high"])
+def test_argreduce_is_bit_exact(shape, axis, ty, op, tie, hip, oracle):
+    rng = np.random.default_rng(seed_of(shape, axis, ty, op))
+    # few distinct values => many exact ties along every axis
+    if T.is_float(T.normalize(ty)):
+        x = rng.integers(-6, 7, size=shape).astype(np.float64) / 2
+        x = (x.astype(np.float32).view(np.uint32) >> 16).astype(np.uint16) if ty == "bf16" else x.astype(T.numpy_dtype(T.normalize(ty)))
+    else:
+        x = rng.integers(0 if ty == "u8" else -6, 7, size=shape).astype(T.numpy_dtype(T.normalize(ty)))
+    hx, ox = both(x, ty, hip, oracle)
+    for out_type in ("s32", "u32") if tie == "low" else ("s64",):
+        got = getattr(Nx, op)(hx, axis=axis, tie_break=tie, type=out_type)
+        want = getattr(Nx, op)(ox, axis=axis, tie_break=tie, type=out_type)
+        assert_bits_equal(got, want, f"{op} {ty} {shape} axis={axis} tie={tie}")
+
+
+@pytest.mark.parametrize("op", ["argmax", "argmin"])
+def test_argreduce_nan_and_infinities(op, hip, oracle):
+    """Any NaN wins and the last NaN's index is returned (nx/test/nx_test.exs:1746-1798)."""
+    rng = np.random.default_rng(11)
+    x = rng.normal(size=(257, 5000)).astype(np.float32)
+    for r in range(0, 257, 3):
+        cols = rng.integers(0, 5000, size=rng.integers(1, 5))
+        x[r, cols] = np.nan
+    for r in range(1, 257, 3):
+        x[r, rng.integers(0, 5000, size=3)] = np.inf
+        x[r, rng.integers(0, 5000, size=3)] = -np.inf
+    hx, ox = both(x, "f32", hip, oracle)
+    for tie in ("low", "high"):
+        assert_bits_equal(getattr(Nx, op)(hx, axis=1, tie_break=tie), getattr(Nx, op)(ox, axis=1, tie_break=tie), op)
+        assert_bits_equal(getattr(Nx, op)(hx, axis=0, tie_break=tie), getattr(Nx, op)(ox, axis=0, tie_break=tie), op)
+    assert_bits_equal(getattr(Nx, op)(hx), getattr(Nx, op)(ox), f"{op} flat")
