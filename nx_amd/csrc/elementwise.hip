@@ -370,9 +370,10 @@ extern "C" int hipnx_as_type(hipnx_ctx *ctx, int in_dt, int out_dt, int64_t n, c
   static const int64_t tmin[8] = {0, 0, 0, 0, -0x80, -0x8000, -0x80000000ll, (int64_t)0x8000000000000000ull};
   int64_t mx = out_dt < HIPNX_F16 ? tmax[out_dt] : 0, mn = out_dt < HIPNX_F16 ? tmin[out_dt] : 0;
   dim3 grid(grid_for(ctx, (n + E - 1) / E)), block(BLOCK);
-  if (!is_float(in_dt))
+  if (!is_float(in_dt) && !is_float(out_dt))  // integer -> integer: keep the low bits
     hipLaunchKernelGGL((as_type_kernel<int64_t>), grid, block, 0, ctx->stream, inb->ptr, out->ptr, in_dt, out_dt, n, mx, mn);
-  else if (in_dt == HIPNX_F64 || out_dt == HIPNX_F64 || out_dt == HIPNX_F16)
+  else if (!is_float(in_dt) || in_dt == HIPNX_F64 || out_dt == HIPNX_F64 || out_dt == HIPNX_F16)
+    // integer -> float decodes to f64 (exact below 2^53, u64 read as unsigned), then one rounding
     hipLaunchKernelGGL((as_type_kernel<double>), grid, block, 0, ctx->stream, inb->ptr, out->ptr, in_dt, out_dt, n, mx, mn);
   else
     hipLaunchKernelGGL((as_type_kernel<float>), grid, block, 0, ctx->stream, inb->ptr, out->ptr, in_dt, out_dt, n, mx, mn);
