@@ -1,65 +1,24 @@
-// Nx.dot as a dense batched contraction  out[b, m, n] = sum_k l[b, m, k] * r[b, n, k].
+// Nx.dot as a dense batched contraction  out[b, m, n] = sum_k l[b, m, k] * r[b, n, k]:
+// argument checks and the choice of kernel.
 //
-// MFMA path (bf16 / f16 / f32 operands with f32 accumulation, s8 with s32 accumulation): both
-// operands K-contiguous.  A K-outer operand is first re-laid by the tiled transpose.
-// Everything else (f64, wide integers, mixed operand types) runs on a plain tiled kernel that
-// accumulates in f64 or wrapping 64-bit integers.
-//
-// MFMA kernel.  A 256-lane block (4 wavefronts, 2 x 2) owns a 128 x 128 output tile; each
-// wavefront owns 64 x 64 = 2 x 2 MFMA tiles of 32 x 32.  The K axis is walked in slabs of
-// 128 bytes per row (64 bf16 / 128 s8 / 32 f32).  Slabs are staged through LDS with 16-byte
-// accesses; the 16-byte chunk index is XOR-swizzled with the row so that the 64 lanes of a
-// fragment read hit distinct banks.  For all four element types a lane's MFMA operand
-// fragment for one 32-byte K-step is the 16-byte chunk (2*step + lane/32) of row (lane%32):
-// bf16/f16/s8 feed it to one 32x32x16 / 32x32x32 MFMA; f32 feeds its four floats to four
-// 32x32x2 MFMAs (both operands use the same k <-> slot map, so the sum covers the same 8 k).
+//   bf16 / f16 / f32 operand pairs (f32 accumulation) and s8 pairs (exact s32 accumulation):
+//     K a multiple of 128 bytes  -> the pipelined MFMA kernel (gemm_mfma.cuh).  bf16 / f16 take
+//       both operand layouts directly; K-outer f32 / s8 operands (and ragged 2-byte ones) are
+//       first re-laid by the tiled transpose.
+//     K a multiple of 16 bytes   -> gemm_kinner_kernel below: same MFMA fragments, single LDS
+//       stage, register-staged loads, zero-filled K tail.
+//   everything else (f64, wide integers, mixed operand types, tiny problems): dot_generic_kernel,
+//     a plain tiled kernel accumulating in f64 or wrapping 64-bit integers.
 //
 // Algorithmic work: 2*B*M*N*K flop; minimum traffic bytes(l) + bytes(r) + bytes(out).
 #include <type_traits>
 
-#include "dtypes.cuh"
-#include "internal.h"
+#include "gemm_launch.cuh"
 
 namespace hipnx {
 
-typedef float v16f __attribute__((ext_vector_type(16)));
-typedef int v16i __attribute__((ext_vector_type(16)));
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
-typedef _Float16 v8h __attribute__((ext_vector_type(8)));
-
 constexpr int GEMM_BLOCK = 256;
 constexpr int BM = 128, BN = 128;
-constexpr int SLAB = 128;            // bytes of K per row per slab
-constexpr int CHUNKS = SLAB / 16;    // 16-byte chunks per row
-
-template <int DT> struct Mma;
-template <> struct Mma<HIPNX_BF16> {
-  typedef v16f acc_t; typedef float scalar_t;
-  static __device__ __forceinline__ void step(acc_t &c, const v4i &a, const v4i &b) {
-    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
-  }
-};
-template <> struct Mma<HIPNX_F16> {
-  typedef v16f acc_t; typedef float scalar_t;
-  static __device__ __forceinline__ void step(acc_t &c, const v4i &a, const v4i &b) {
-    c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0, 0, 0);
-  }
-};
-template <> struct Mma<HIPNX_S8> {
-  typedef v16i acc_t; typedef int scalar_t;
-  static __device__ __forceinline__ void step(acc_t &c, const v4i &a, const v4i &b) {
-    c = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
-  }
-};
-template <> struct Mma<HIPNX_F32> {
-  typedef v16f acc_t; typedef float scalar_t;
-  static __device__ __forceinline__ void step(acc_t &c, const v4i &a, const v4i &b) {
-#pragma unroll
-    for (int s = 0; s < 4; s++)
-      c = __builtin_amdgcn_mfma_f32_32x32x2f32(__int_as_float(a[s]), __int_as_float(b[s]), c, 0, 0, 0);
-  }
-};
 
 // l: [batch, M, Kb bytes], r: [batch, N, Kb bytes]  (Kb = K * element size, multiple of 16)
 template <int DT>
@@ -67,8 +26,7 @@ __global__ void __launch_bounds__(GEMM_BLOCK)
 gemm_kinner_kernel(const unsigned char *__restrict__ l, const unsigned char *__restrict__ r, void *__restrict__ out,
                    int odt, int64_t M, int64_t N, int64_t Kb, int tiles_m, int tiles_n) {
   typedef typename Mma<DT>::acc_t acc_t;
-  typedef typename Mma<DT>::scalar_t scalar_t;
-  __shared__ __attribute__((aligned(16))) unsigned char sA[BM * SLAB];
+    __shared__ __attribute__((aligned(16))) unsigned char sA[BM * SLAB];
   __shared__ __attribute__((aligned(16))) unsigned char sB[BN * SLAB];
 
   const int tile = blockIdx.x;
@@ -149,7 +107,7 @@ gemm_kinner_kernel(const unsigned char *__restrict__ l, const unsigned char *__r
         const int64_t gm = m0 + wm + 32 * i + 8 * (q / 4) + 4 * (lane / 32) + (q % 4);
         const int64_t gn = n0 + wn + 32 * j + lane % 32;
         if (gm < M && gn < N) {
-          if constexpr (DT == HIPNX_S8) store_one<int64_t>(ob, odt, obase + gm * N + gn, (int64_t)(scalar_t)acc[i][j][q]);
+          if constexpr (DT == HIPNX_S8) store_one<int64_t>(ob, odt, obase + gm * N + gn, (int64_t)acc[i][j][q]);
           else store_one<float>(ob, odt, obase + gm * N + gn, (float)acc[i][j][q]);
         }
       }
@@ -243,11 +201,15 @@ extern "C" int hipnx_dot(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t
     }
   }
 
-  // MFMA path: bring K-outer operands to K-inner through the tiled transpose (pool workspace)
+  // MFMA path.  Which operands need the tiled transpose to become K-inner first?
   const int esz = dtype_size(l_dt);
+  const bool pipelined = Kb % SLAB == 0;
+  const bool native_kouter = pipelined && esz == 2;  // the pipelined kernel transposes 2-byte operands itself
+  const bool l_relay = l_layout == HIPNX_K_OUTER && !(native_kouter && M % 8 == 0);
+  const bool r_relay = r_layout == HIPNX_K_OUTER && !(native_kouter && N % 8 == 0);
   hipnx_buf *lt = nullptr, *rt = nullptr;
   int st = HIPNX_OK;
-  if (l_layout == HIPNX_K_OUTER) {
+  if (l_relay) {
     st = hipnx_buf_alloc(ctx, (size_t)(batch * M * K * esz), &lt);
     if (!st) {
       int64_t dims[3] = {batch, K, M};
@@ -255,7 +217,7 @@ extern "C" int hipnx_dot(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t
       st = hipnx_transpose(ctx, esz, 3, dims, perm, l, lt);
     }
   }
-  if (!st && r_layout == HIPNX_K_OUTER) {
+  if (!st && r_relay) {
     st = hipnx_buf_alloc(ctx, (size_t)(batch * N * K * esz), &rt);
     if (!st) {
       int64_t dims[3] = {batch, K, N};
@@ -268,14 +230,41 @@ extern "C" int hipnx_dot(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t
     st = in.status;
     if (!st) {
       const void *lp = lt ? lt->ptr : l->ptr, *rp = rt ? rt->ptr : r->ptr;
-      switch (l_dt) {
-        case HIPNX_BF16: launch_mfma<HIPNX_BF16>(ctx, lp, rp, out->ptr, out_dt, batch, M, N, Kb); break;
-        case HIPNX_F16: launch_mfma<HIPNX_F16>(ctx, lp, rp, out->ptr, out_dt, batch, M, N, Kb); break;
-        case HIPNX_F32: launch_mfma<HIPNX_F32>(ctx, lp, rp, out->ptr, out_dt, batch, M, N, Kb); break;
-        default: launch_mfma<HIPNX_S8>(ctx, lp, rp, out->ptr, out_dt, batch, M, N, Kb); break;
+      if (pipelined) {
+        const bool l_kin = l_layout == HIPNX_K_INNER || l_relay, r_kin = r_layout == HIPNX_K_INNER || r_relay;
+        GemmArgs a{};
+        a.l = (const unsigned char *)lp;
+        a.r = (const unsigned char *)rp;
+        a.out = out->ptr;
+        a.odt = out_dt;
+        a.M = M; a.N = N; a.Kb = Kb;
+        a.ld_l = l_kin ? Kb : M * esz;
+        a.ld_r = r_kin ? Kb : N * esz;
+        a.bs_l = M * Kb;
+        a.bs_r = N * Kb;
+        // tile choice: the largest tile that still gives every CU work; few rows against a long
+        // weight matrix stream the weights with many small tiles
+        const int64_t t256 = ((M + 255) / 256) * ((N + 255) / 256) * batch;
+        int cfg;
+        if (M <= 64) cfg = GEMM_CFG_64x32;
+        else if (t256 * 4 >= (int64_t)ctx->num_cus * 3 && M >= 192 && N >= 192) cfg = GEMM_CFG_256;
+        else cfg = GEMM_CFG_128;
+        switch (l_dt) {
+          case HIPNX_BF16: st = launch_gemm_bf16(ctx, cfg, l_kin, r_kin, a, batch); break;
+          case HIPNX_F16: st = launch_gemm_f16(ctx, cfg, l_kin, r_kin, a, batch); break;
+          case HIPNX_F32: st = launch_gemm_f32(ctx, cfg, a, batch); break;
+          default: st = launch_gemm_s8(ctx, cfg, a, batch); break;
+        }
+      } else {
+        switch (l_dt) {
+          case HIPNX_BF16: launch_mfma<HIPNX_BF16>(ctx, lp, rp, out->ptr, out_dt, batch, M, N, Kb); break;
+          case HIPNX_F16: launch_mfma<HIPNX_F16>(ctx, lp, rp, out->ptr, out_dt, batch, M, N, Kb); break;
+          case HIPNX_F32: launch_mfma<HIPNX_F32>(ctx, lp, rp, out->ptr, out_dt, batch, M, N, Kb); break;
+          default: launch_mfma<HIPNX_S8>(ctx, lp, rp, out->ptr, out_dt, batch, M, N, Kb); break;
+        }
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) st = hip_fail(e, "gemm launch");
       }
-      hipError_t e = hipGetLastError();
-      if (e != hipSuccess) st = hip_fail(e, "gemm launch");
     }
   }
   // handing the workspaces back to the pool is safe: later work is ordered on the same stream

@@ -1,0 +1,56 @@
+// Launcher shared by the per-type translation units of the pipelined MFMA kernel (one unit per
+// operand type keeps the build parallel).
+#pragma once
+#include "gemm_mfma.cuh"
+#include "internal.h"
+
+namespace hipnx {
+
+// tile configurations of gemm_pipelined_kernel<DT, WM, WN, TM, TN, ...>
+enum {
+  GEMM_CFG_256 = 0,  // 256 x 256, 8 waves (4 x 2, each 64 x 128): large square-ish problems
+  GEMM_CFG_128 = 1,  // 128 x 128, 4 waves (2 x 2, each 64 x 64): mid-size and batched problems
+  GEMM_CFG_64x32 = 2 // 64 x 32, 2 waves: few rows against a long weight matrix (HBM streaming)
+};
+
+int launch_gemm_bf16(const hipnx_ctx *ctx, int cfg, bool l_kin, bool r_kin, GemmArgs a, int64_t batch);
+int launch_gemm_f16(const hipnx_ctx *ctx, int cfg, bool l_kin, bool r_kin, GemmArgs a, int64_t batch);
+int launch_gemm_f32(const hipnx_ctx *ctx, int cfg, GemmArgs a, int64_t batch);
+int launch_gemm_s8(const hipnx_ctx *ctx, int cfg, GemmArgs a, int64_t batch);
+
+template <int DT, int WM, int WN, int TM, int TN, bool LK, bool RK>
+static int launch_one(const hipnx_ctx *ctx, GemmArgs a, int64_t batch) {
+  constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
+  constexpr int smem = 2 * (BM + BN) * SLAB;
+  auto kern = gemm_pipelined_kernel<DT, WM, WN, TM, TN, LK, RK>;
+  static bool configured = false;  // per instantiation; racing writers store the same value
+  if (!configured) {
+    HIPNX_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
+    configured = true;
+  }
+  a.tiles_m = (int)((a.M + BM - 1) / BM);
+  a.tiles_n = (int)((a.N + BN - 1) / BN);
+  dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)batch), block(WM * WN * 64);
+  hipLaunchKernelGGL(kern, grid, block, smem, ctx->stream, a);
+  HIPNX_HIP(hipGetLastError());
+  return HIPNX_OK;
+}
+
+template <int DT, bool LK, bool RK>
+static int launch_cfg(const hipnx_ctx *ctx, int cfg, const GemmArgs &a, int64_t batch) {
+  switch (cfg) {
+    case GEMM_CFG_256: return launch_one<DT, 4, 2, 2, 4, LK, RK>(ctx, a, batch);
+    case GEMM_CFG_128: return launch_one<DT, 2, 2, 2, 2, LK, RK>(ctx, a, batch);
+    default: return launch_one<DT, 2, 1, 1, 1, LK, RK>(ctx, a, batch);
+  }
+}
+
+template <int DT>
+static int launch_layouts(const hipnx_ctx *ctx, int cfg, bool l_kin, bool r_kin, const GemmArgs &a, int64_t batch) {
+  if (l_kin && r_kin) return launch_cfg<DT, true, true>(ctx, cfg, a, batch);
+  if (l_kin) return launch_cfg<DT, true, false>(ctx, cfg, a, batch);
+  if (r_kin) return launch_cfg<DT, false, true>(ctx, cfg, a, batch);
+  return launch_cfg<DT, false, false>(ctx, cfg, a, batch);
+}
+
+}  // namespace hipnx

@@ -1,0 +1,324 @@
+// Pipelined MFMA contraction kernel  out[b, m, n] = sum_k l[b, m, k] * r[b, n, k]  for gfx950.
+//
+// Work-group tile BM x BN = (WM*TM*32) x (WN*TN*32): WM x WN wavefronts, each owning TM x TN MFMA
+// tiles of 32 x 32 whose accumulators stay in registers for the whole K walk.
+//
+// K is walked in slabs of 128 bytes per row (64 bf16/f16, 128 s8, 32 f32): one full cache line
+// per row, the granularity at which a CU ingests L2-resident data fastest (half lines halve it).
+// LDS holds a ring of NUNIT "units"; a unit is one operand's share of one slab (BM or BN rows x
+// 128 B).  Slab s is units 2s (l rows) and 2s+1 (r rows).  While the MFMAs consume slab s, the
+// r unit of slab s+1 and the l unit of slab s+2 are in flight (the l unit of slab s+1 was issued a
+// slab earlier), so the data needed next has had between one and two slab times to arrive; the
+// wait before the per-slab barrier uses vmcnt(n) and leaves the youngest unit outstanding.
+//   K-inner operand ([rows, K], K contiguous): `global_load_lds_dwordx4` -- each lane moves 16 B
+//     straight from global memory into LDS, no VGPR round trip.  A wave instruction fills 1 KiB of
+//     LDS (8 rows x 8 chunks); the lane picks the *global* chunk that belongs at its LDS slot.
+//   K-outer operand ([K, rows], rows contiguous; 2-byte types): each lane loads an 8(k) x 8(row)
+//     block with eight 16-byte row loads, transposes it in registers with byte permutes and
+//     writes eight 16-byte K-runs to LDS -- the slab arrives in the same [row][k] LDS layout.
+// LDS layout of a unit: row-major, 128 B per row, the 16-byte chunk index XOR-ed with
+// ((row ^ row>>3) & 7): conflict-free for the fragment reads (32 consecutive rows, one chunk) and
+// for the transposed writes (rows 8 apart, one chunk).
+// Fragments: for one 32-byte K-step a lane's MFMA operand is chunk (2*step + lane/32) of row
+// (lane%32) -- 8 bf16/f16, 16 s8 or 4 f32 (fed to four 32x32x2 MFMAs; both operands use the same
+// k <-> slot map).  The MFMA is issued with the r-fragment as its first operand so that a lane ends
+// up with 4 consecutive n per accumulator quad: the epilogue stores 4 outputs at a time.
+#pragma once
+#include <type_traits>
+
+#include "dtypes.cuh"
+
+namespace hipnx {
+
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+
+constexpr int SLAB = 128;          // bytes of K per row per slab
+constexpr int CHUNKS = SLAB / 16;  // 16-byte chunks per row
+
+template <int DT> struct Mma;
+template <> struct Mma<HIPNX_BF16> {
+  typedef v16f acc_t;
+  static __device__ __forceinline__ void step(acc_t &c, const v4i &a, const v4i &b) {
+    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
+  }
+};
+template <> struct Mma<HIPNX_F16> {
+  typedef v16f acc_t;
+  static __device__ __forceinline__ void step(acc_t &c, const v4i &a, const v4i &b) {
+    c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0, 0, 0);
+  }
+};
+template <> struct Mma<HIPNX_S8> {
+  typedef v16i acc_t;
+  static __device__ __forceinline__ void step(acc_t &c, const v4i &a, const v4i &b) {
+    c = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct Mma<HIPNX_F32> {
+  typedef v16f acc_t;
+  static __device__ __forceinline__ void step(acc_t &c, const v4i &a, const v4i &b) {
+#pragma unroll
+    for (int s = 0; s < 4; s++)
+      c = __builtin_amdgcn_mfma_f32_32x32x2f32(__int_as_float(a[s]), __int_as_float(b[s]), c, 0, 0, 0);
+  }
+};
+
+__device__ __forceinline__ int lds_slot(int row, int chunk) { return chunk ^ ((row ^ (row >> 3)) & 7); }
+
+typedef const __attribute__((address_space(1))) void *gptr_t;
+typedef __attribute__((address_space(3))) void *lptr_t;
+
+// K-inner slab loader: ROWS x 128 B, direct to LDS.  The per-lane source pointers (row clamp,
+// row * stride, swizzled chunk) are computed once; per slab only the K offset moves.
+// Rows past `rows_valid` are clamped (loaded from the last valid row; their results are never
+// stored).
+template <int ROWS, int NWAVES>
+struct KInnerLoader {
+  static constexpr int INSTR = ROWS / 8;  // wave instructions per slab (1 KiB of LDS each)
+  static constexpr int PER = INSTR / NWAVES;
+  static_assert(INSTR % NWAVES == 0, "slab rows must split evenly over the waves");
+  const unsigned char *src[PER];
+  int lds_off[PER];
+
+  __device__ __forceinline__ void init(const unsigned char *__restrict__ g, int64_t ld, int64_t row0, int64_t rows_valid,
+                                       int wave, int lane) {
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+      const int t = wave + NWAVES * i;
+      const int r = t * 8 + (lane >> 3);
+      const int chunk = lds_slot(r, lane & 7);  // the XOR map is an involution: slot -> chunk
+      int64_t gr = row0 + r;
+      gr = gr < rows_valid ? gr : rows_valid - 1;
+      src[i] = g + gr * ld + chunk * 16;
+      lds_off[i] = t * 1024;
+    }
+  }
+  __device__ __forceinline__ void issue(int64_t kbyte0, unsigned char *lds) const {
+#pragma unroll
+    for (int i = 0; i < PER; i++)
+      __builtin_amdgcn_global_load_lds((gptr_t)(src[i] + kbyte0), (lptr_t)(lds + lds_off[i]), 16, 0, 0);
+  }
+};
+
+// 8 x 8 transpose of 16-bit elements held as rows[k] = 8 consecutive `row` values at one k:
+// out[i] = the 8 consecutive k values of row i.
+__device__ __forceinline__ void transpose8x8_b16(const v4i (&in)[8], v4i (&out)[8]) {
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      // out[i] dword j = { in[2j] half i , in[2j+1] half i }
+      const unsigned lo = (unsigned)in[2 * j][i >> 1], hi = (unsigned)in[2 * j + 1][i >> 1];
+      out[i][j] = (int)__builtin_amdgcn_perm(hi, lo, (i & 1) ? 0x07060302u : 0x05040100u);
+    }
+  }
+}
+
+// K-outer slab of a 2-byte type: g is [K, rows] (row stride ld bytes per k); the slab covers
+// 64 k x ROWS rows.  ROWS*8/8 = ROWS blocks of 8 x 8, one or more per lane.
+template <int ROWS, int NTHREADS>
+struct KOuterRegs {
+  static constexpr int BLOCKS = (ROWS / 8) * 8;  // (ROWS/8 row-blocks) x (8 k-blocks)
+  static constexpr int PER = (BLOCKS + NTHREADS - 1) / NTHREADS;
+  v4i v[PER][8];
+};
+
+template <int ROWS, int NTHREADS>
+__device__ __forceinline__ void fetch_slab_kouter16(KOuterRegs<ROWS, NTHREADS> &regs, const unsigned char *__restrict__ g,
+                                                    int64_t ld, int64_t row0, int64_t rows_valid, int64_t k0,
+                                                    int64_t k_valid, int tid) {
+  constexpr int RB = ROWS / 8;
+#pragma unroll
+  for (int p = 0; p < KOuterRegs<ROWS, NTHREADS>::PER; p++) {
+    const int blk = tid + p * NTHREADS;
+    if (blk >= KOuterRegs<ROWS, NTHREADS>::BLOCKS) break;
+    const int rb = blk % RB, kb = blk / RB;
+    int64_t col = row0 + rb * 8;
+    // whole 16-byte run must be inside the row; a ragged edge re-reads the last full run
+    col = col + 8 <= rows_valid ? col : (rows_valid >= 8 ? rows_valid - 8 : 0);
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      int64_t k = k0 + kb * 8 + j;
+      k = k < k_valid ? k : k_valid - 1;
+      regs.v[p][j] = *reinterpret_cast<const v4i *>(g + k * ld + col * 2);
+    }
+  }
+}
+
+template <int ROWS, int NTHREADS>
+__device__ __forceinline__ void store_slab_kouter16(const KOuterRegs<ROWS, NTHREADS> &regs, unsigned char *lds, int tid) {
+  constexpr int RB = ROWS / 8;
+#pragma unroll
+  for (int p = 0; p < KOuterRegs<ROWS, NTHREADS>::PER; p++) {
+    const int blk = tid + p * NTHREADS;
+    if (blk >= KOuterRegs<ROWS, NTHREADS>::BLOCKS) break;
+    const int rb = blk % RB, kb = blk / RB;
+    v4i t[8];
+    transpose8x8_b16(regs.v[p], t);
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const int r = rb * 8 + i;
+      *reinterpret_cast<v4i *>(lds + r * SLAB + lds_slot(r, kb) * 16) = t[i];
+    }
+  }
+}
+
+struct GemmArgs {
+  const unsigned char *l, *r;
+  void *out;
+  int odt;
+  int64_t M, N, Kb;      // Kb = K in bytes (a multiple of 128 for this kernel)
+  int64_t ld_l, ld_r;    // bytes between consecutive rows (K-inner) or consecutive k (K-outer)
+  int64_t bs_l, bs_r;    // bytes between batch items
+  int tiles_m, tiles_n;
+};
+
+// Epilogue of one wave: lane holds m = lane%32 and, per accumulator quad qq of tile (i, j),
+// n = 32*j + 8*qq + 4*(lane/32) + 0..3.  ODT is a compile-time constant here, so the typed
+// stores fold to plain vector stores; every accumulator index is a constant (the accumulators
+// must never be addressed dynamically, or they leave the register file).
+template <int DT, int ODT, int TM, int TN>
+__device__ __forceinline__ void gemm_epilogue(typename Mma<DT>::acc_t (&acc)[TM][TN], void *out, int64_t obase,
+                                              int64_t M, int64_t N, int64_t row0, int64_t col0, int lane) {
+  constexpr bool int_acc = DT == HIPNX_S8;
+  constexpr bool int_out = ODT < HIPNX_F16;
+  if constexpr (int_acc != int_out) return;  // the host never pairs them
+  else {
+    typedef typename std::conditional<int_acc, int64_t, float>::type S;
+    const bool vec_ok = (N % 4) == 0;
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+      const int64_t gm = row0 + 32 * i + (lane & 31);
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+#pragma unroll
+        for (int qq = 0; qq < 4; qq++) {
+          const int64_t gn = col0 + 32 * j + 8 * qq + 4 * (lane >> 5);
+          S v[4];
+#pragma unroll
+          for (int e = 0; e < 4; e++) v[e] = (S)acc[i][j][4 * qq + e];
+          const int64_t idx = obase + gm * N + gn;
+          if (gm < M) {
+            if (vec_ok && gn + 4 <= N) store_vec<S, 4>(out, ODT, idx, v);
+            else {
+#pragma unroll
+              for (int e = 0; e < 4; e++)
+                if (gn + e < N) store_one<S>(out, ODT, idx + e, v[e]);
+            }
+          }
+        }
+    }
+  }
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {  // s_waitcnt vmcnt(N), other counters untouched
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
+}
+
+template <int DT, int WM, int WN, int TM, int TN, bool L_KIN, bool R_KIN>
+__global__ void __launch_bounds__(WM *WN * 64)
+gemm_pipelined_kernel(GemmArgs a) {
+  typedef typename Mma<DT>::acc_t acc_t;
+  constexpr int NW = WM * WN, NT = NW * 64;
+  constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
+  constexpr int STAGE = (BM + BN) * SLAB;
+  constexpr int KSTEPS = SLAB / 32;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+
+  // tile order: consecutive block ids go to different XCDs (id % 8); give each XCD a compact
+  // band of tiles so that the operand panels it streams are shared through its own L2
+  int tile = blockIdx.x;
+  {
+    const int total = a.tiles_m * a.tiles_n;
+    if (total % 8 == 0) tile = (blockIdx.x % 8) * (total / 8) + blockIdx.x / 8;
+  }
+  const int tm = tile / a.tiles_n, tn = tile % a.tiles_n;
+  const int64_t b = blockIdx.y;
+  const unsigned char *lb = a.l + b * a.bs_l;
+  const unsigned char *rb = a.r + b * a.bs_r;
+  const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = (wave / WN) * (TM * 32), wn = (wave % WN) * (TN * 32);
+
+  acc_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int q = 0; q < 16; q++) acc[i][j][q] = 0;
+
+  KInnerLoader<BM, NW> lload;
+  KInnerLoader<BN, NW> rload;
+  if constexpr (L_KIN) lload.init(lb, a.ld_l, m0, a.M, wave, lane);
+  if constexpr (R_KIN) rload.init(rb, a.ld_r, n0, a.N, wave, lane);
+  KOuterRegs<BM, NT> lregs;
+  KOuterRegs<BN, NT> rregs;
+  const int64_t K_elems = a.Kb / 2;  // only used by the 2-byte K-outer path
+
+  auto issue = [&](int stage, int64_t kbyte0) {
+    unsigned char *sA = smem + stage * STAGE, *sB = sA + BM * SLAB;
+    if constexpr (L_KIN) lload.issue(kbyte0, sA);
+    else fetch_slab_kouter16<BM, NT>(lregs, lb, a.ld_l, m0, a.M, kbyte0 / 2, K_elems, tid);
+    if constexpr (R_KIN) rload.issue(kbyte0, sB);
+    else fetch_slab_kouter16<BN, NT>(rregs, rb, a.ld_r, n0, a.N, kbyte0 / 2, K_elems, tid);
+  };
+  auto commit = [&](int stage) {  // K-outer operands: registers -> transposed LDS writes
+    unsigned char *sA = smem + stage * STAGE, *sB = sA + BM * SLAB;
+    if constexpr (!L_KIN) store_slab_kouter16<BM, NT>(lregs, sA, tid);
+    if constexpr (!R_KIN) store_slab_kouter16<BN, NT>(rregs, sB, tid);
+  };
+
+  const int nslab = (int)(a.Kb / SLAB);
+  issue(0, 0);
+  commit(0);
+  wait_vmcnt<0>();  // my direct-to-LDS loads have landed
+  __syncthreads();
+
+  for (int s = 0; s < nslab; s++) {
+    const int cur = s & 1;
+    if (s + 1 < nslab) issue(cur ^ 1, (int64_t)(s + 1) * SLAB);
+    const unsigned char *sA = smem + cur * STAGE, *sB = sA + BM * SLAB;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ks++) {
+      v4i fa[TM], fb[TN];
+      const int chunk = 2 * ks + (lane >> 5);
+#pragma unroll
+      for (int i = 0; i < TM; i++) {
+        const int row = wm + 32 * i + (lane & 31);
+        fa[i] = *reinterpret_cast<const v4i *>(sA + row * SLAB + lds_slot(row, chunk) * 16);
+      }
+#pragma unroll
+      for (int j = 0; j < TN; j++) {
+        const int row = wn + 32 * j + (lane & 31);
+        fb[j] = *reinterpret_cast<const v4i *>(sB + row * SLAB + lds_slot(row, chunk) * 16);
+      }
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) Mma<DT>::step(acc[i][j], fb[j], fa[i]);
+    }
+    if (s + 1 < nslab) commit(cur ^ 1);
+    wait_vmcnt<0>();
+    __syncthreads();
+  }
+
+  // epilogue: the output type is wave-uniform; branch once, then every store is straight-line
+  const int64_t obase = b * a.M * a.N;
+  switch (a.odt) {
+#define HIPNX_EPI(T) case T: gemm_epilogue<DT, T, TM, TN>(acc, a.out, obase, a.M, a.N, m0 + wm, n0 + wn, lane); break;
+    HIPNX_EPI(HIPNX_BF16) HIPNX_EPI(HIPNX_F16) HIPNX_EPI(HIPNX_F32) HIPNX_EPI(HIPNX_F64)
+    HIPNX_EPI(HIPNX_S8) HIPNX_EPI(HIPNX_U8) HIPNX_EPI(HIPNX_S16) HIPNX_EPI(HIPNX_U16)
+    HIPNX_EPI(HIPNX_S32) HIPNX_EPI(HIPNX_U32) HIPNX_EPI(HIPNX_S64) HIPNX_EPI(HIPNX_U64)
+#undef HIPNX_EPI
+  }
+}
+
+}  // namespace hipnx
