@@ -1,0 +1,401 @@
+defmodule HipNx.Backend do
+  @moduledoc """
+  An `Nx.Backend` for one AMD Instinct MI355X over `libhipnx` (hand-written gfx950 kernels).
+
+      Nx.default_backend({HipNx.Backend, device: 0})
+
+  Native callbacks: the element-wise binary and unary ops, `as_type`, `sum`, `product`,
+  `reduce_max`, `reduce_min`, `argmax`, `argmin`, `dot`, `gather`, `take` (through
+  `Nx.Block.Take`), `transpose`, `broadcast`, and the plumbing (`from_binary`, `to_binary`,
+  `constant`, transfers, `reshape`/`squeeze`/`bitcast`, `inspect`).  Every other callback of the
+  behaviour runs on `Nx.BinaryBackend` after a device-to-host copy and comes back with
+  `from_binary` -- the same escape hatch `EXLA.Backend` uses for `concatenate`/`stack`.
+
+  Results follow `Nx.BinaryBackend` (integers, indices and argmax bit-exact; see the repository's
+  DESIGN.md for the float tolerances and the documented divergences).
+
+  This module cannot be compiled in the repository's build container (no BEAM); its Python twin
+  `nx_amd/backend.py` exercises the same C ABI with the same lowering and is what the test-suite
+  runs.
+  """
+  @behaviour Nx.Backend
+
+  @enforce_keys [:ref, :device]
+  defstruct [:ref, :device]
+
+  alias Nx.Tensor, as: T
+  alias HipNx.NIF
+
+  @binary_ops ~w(add subtract multiply divide pow remainder atan2 min max quotient bitwise_and
+                 bitwise_or bitwise_xor left_shift right_shift equal not_equal greater less
+                 greater_equal less_equal logical_and logical_or logical_xor)a
+  @unary_ops ~w(exp expm1 log log1p sigmoid cos sin tan cosh sinh tanh acos asin atan acosh asinh
+                atanh sqrt rsqrt cbrt erf erfc erf_inv abs bitwise_not ceil floor negate round sign
+                count_leading_zeros population_count is_nan is_infinity)a
+  @dtypes %{{:u, 8} => 0, {:u, 16} => 1, {:u, 32} => 2, {:u, 64} => 3, {:s, 8} => 4, {:s, 16} => 5,
+            {:s, 32} => 6, {:s, 64} => 7, {:f, 16} => 8, {:bf, 16} => 9, {:f, 32} => 10, {:f, 64} => 11}
+
+  ## Options and context
+
+  @impl true
+  def init(opts), do: Keyword.validate!(opts, device: 0)
+
+  defp ctx(device) do
+    key = {__MODULE__, :ctx, device}
+
+    case :persistent_term.get(key, nil) do
+      nil ->
+        ctx = unwrap!(NIF.ctx_create(device))
+        :persistent_term.put(key, ctx)
+        ctx
+
+      ctx ->
+        ctx
+    end
+  end
+
+  defp unwrap!({:ok, value}), do: value
+  defp unwrap!({:error, {status, msg}}) when status in [2, 6], do: raise(ArgumentError, List.to_string(msg))
+  defp unwrap!({:error, {_status, msg}}), do: raise(RuntimeError, "HipNx: " <> List.to_string(msg))
+
+  defp dt(type), do: Map.get(@dtypes, type) || raise(ArgumentError, "HipNx does not support type #{inspect(type)}")
+  defp bytes(%T{type: {_, bits}, shape: shape}), do: div(bits, 8) * Nx.size(shape)
+  defp to_nx(ref, device, %T{} = out), do: %{out | data: %__MODULE__{ref: ref, device: device}}
+
+  # operands living on another backend are copied in on entry (cf. Torchx.Backend.from_nx/1)
+  defp from_nx(%T{data: %__MODULE__{ref: ref, device: device}}, _), do: {ref, device}
+
+  defp from_nx(%T{} = t, device) do
+    %T{data: %__MODULE__{ref: ref}} = Nx.backend_transfer(t, {__MODULE__, device: device})
+    {ref, device}
+  end
+
+  defp device_of(tensors) do
+    Enum.find_value(tensors, 0, fn
+      %T{data: %__MODULE__{device: d}} -> d
+      _ -> nil
+    end)
+  end
+
+  ## Creation and transfer
+
+  @impl true
+  def from_binary(%T{} = out, binary, opts) do
+    device = init(opts)[:device]
+    to_nx(unwrap!(NIF.from_binary(ctx(device), IO.iodata_to_binary(binary), bytes(out))), device, out)
+  end
+
+  @impl true
+  def to_binary(%T{data: %__MODULE__{ref: ref, device: device}, type: {_, bits}} = t, limit) do
+    n = min(limit, Nx.size(t))
+    unwrap!(NIF.to_binary(ctx(device), ref, n * div(bits, 8)))
+  end
+
+  @impl true
+  def constant(%T{type: type} = out, number, opts) do
+    device = init(opts)[:device]
+    %T{data: %Nx.BinaryBackend{state: elem}} = Nx.BinaryBackend.constant(%{out | shape: {}, names: []}, number, [])
+    _ = type
+    to_nx(unwrap!(NIF.fill(ctx(device), elem, Nx.size(out))), device, out)
+  end
+
+  @impl true
+  def backend_copy(%T{data: %__MODULE__{ref: ref, device: device}} = t, __MODULE__, opts) do
+    if init(opts)[:device] == device do
+      to_nx(unwrap!(NIF.copy(ctx(device), ref, bytes(t))), device, t)
+    else
+      from_binary(t, to_binary(t, Nx.size(t)), opts)
+    end
+  end
+
+  def backend_copy(t, backend, opts), do: backend.from_binary(t, to_binary(t, Nx.size(t)), opts)
+
+  @impl true
+  def backend_transfer(%T{data: %__MODULE__{device: device}} = t, __MODULE__, opts) do
+    if init(opts)[:device] == device do
+      t
+    else
+      copy = backend_copy(t, __MODULE__, opts)
+      backend_deallocate(t)
+      copy
+    end
+  end
+
+  def backend_transfer(t, backend, opts) do
+    copy = backend_copy(t, backend, opts)
+    backend_deallocate(t)
+    copy
+  end
+
+  @impl true
+  def backend_deallocate(%T{data: %__MODULE__{ref: ref}}) do
+    case NIF.deallocate(ref) do
+      :ok -> :ok
+      :already_deallocated -> :already_deallocated
+      other -> unwrap!(other)
+    end
+  end
+
+  @impl true
+  def inspect(%T{} = t, inspect_opts) do
+    limit = if inspect_opts.limit == :infinity, do: :infinity, else: inspect_opts.limit + 1
+    t |> to_binary(min(limit, Nx.size(t))) |> then(&Nx.Backend.inspect(t, &1, inspect_opts))
+  end
+
+  ## Metadata-only callbacks: buffers are immutable, so the handle is shared
+
+  @impl true
+  def reshape(out, %T{} = t), do: share(out, t)
+  @impl true
+  def squeeze(out, %T{} = t, _axes), do: share(out, t)
+  @impl true
+  def bitcast(out, %T{} = t), do: share(out, t)
+
+  defp share(out, t) do
+    device = device_of([t])
+    {ref, _} = from_nx(t, device)
+    # a second owner of the same device memory: copy on the device keeps deallocation simple
+    to_nx(unwrap!(NIF.copy(ctx(device), ref, bytes(out))), device, out)
+  end
+
+  ## Element-wise
+
+  for {op, code} <- Enum.with_index(@binary_ops) do
+    @impl true
+    def unquote(op)(out, l, r), do: binary(unquote(code), out, l, r)
+  end
+
+  defp binary(code, %T{shape: shape} = out, %T{} = l, %T{} = r) do
+    device = device_of([l, r])
+    {lref, _} = from_nx(l, device)
+    {rref, _} = from_nx(r, device)
+    dims = Tuple.to_list(shape)
+
+    ref =
+      NIF.binary(ctx(device), code, dt(l.type), dt(r.type), dt(out.type), dims,
+        broadcast_strides(l.shape, shape), broadcast_strides(r.shape, shape), lref, rref, bytes(out))
+
+    to_nx(unwrap!(ref), device, out)
+  end
+
+  # element strides of `shape` viewed in `out_shape` (right-aligned), 0 on broadcast axes
+  defp broadcast_strides(shape, out_shape) do
+    rank = tuple_size(out_shape)
+    padded = List.duplicate(1, rank - tuple_size(shape)) ++ Tuple.to_list(shape)
+
+    {strides, _} =
+      padded
+      |> Enum.reverse()
+      |> Enum.map_reduce(1, fn dim, acc -> {if(dim == 1, do: 0, else: acc), acc * dim} end)
+
+    Enum.reverse(strides)
+  end
+
+  for {op, code} <- Enum.with_index(@unary_ops) do
+    @impl true
+    def unquote(op)(out, t), do: unary(unquote(code), out, t)
+  end
+
+  defp unary(code, out, %T{} = t) do
+    device = device_of([t])
+    {ref, _} = from_nx(t, device)
+    to_nx(unwrap!(NIF.unary(ctx(device), code, dt(t.type), dt(out.type), Nx.size(out), ref, bytes(out))), device, out)
+  end
+
+  @impl true
+  def as_type(%T{type: type}, %T{type: type} = t), do: t
+  def as_type(out, t), do: unary(-1, out, t)
+
+  ## Reductions
+
+  @impl true
+  def sum(out, t, opts), do: reduce_op(0, out, t, opts)
+  @impl true
+  def reduce_max(out, t, opts), do: reduce_op(1, out, t, opts)
+  @impl true
+  def reduce_min(out, t, opts), do: reduce_op(2, out, t, opts)
+  @impl true
+  def product(out, t, opts), do: reduce_op(3, out, t, opts)
+
+  defp reduce_op(code, out, %T{} = t, opts) do
+    device = device_of([t])
+    {view, outer, red, inner} = view_for_axes(t, opts[:axes], device)
+    {ref, _} = from_nx(view, device)
+    to_nx(unwrap!(NIF.reduce(ctx(device), code, dt(t.type), dt(out.type), outer, red, inner, ref, bytes(out))), device, out)
+  end
+
+  @impl true
+  def argmax(out, t, opts), do: arg_op(0, out, t, opts)
+  @impl true
+  def argmin(out, t, opts), do: arg_op(1, out, t, opts)
+
+  defp arg_op(code, out, %T{} = t, opts) do
+    device = device_of([t])
+    tie = if opts[:tie_break] == :high, do: 1, else: 0
+    axes = if opts[:axis], do: [opts[:axis]], else: nil
+    {view, outer, red, inner} = view_for_axes(t, axes, device)
+    {ref, _} = from_nx(view, device)
+
+    to_nx(unwrap!(NIF.argreduce(ctx(device), code, tie, dt(t.type), dt(out.type), outer, red, inner, ref, bytes(out))),
+      device, out)
+  end
+
+  # collapses to [outer, red, inner]; non-adjacent axes are brought together by a device
+  # transpose to kept ++ reduced, which keeps the row-major order of the reduced axes
+  defp view_for_axes(t, nil, _device), do: {t, 1, Nx.size(t), 1}
+
+  defp view_for_axes(%T{shape: shape} = t, axes, _device) do
+    axes = Enum.sort(axes)
+    dims = Tuple.to_list(shape)
+    first = hd(axes)
+    last = List.last(axes)
+
+    if axes == Enum.to_list(first..last) do
+      {t, prod(Enum.take(dims, first)), prod(Enum.slice(dims, first..last)), prod(Enum.drop(dims, last + 1))}
+    else
+      kept = Nx.axes(t) -- axes
+      perm = kept ++ axes
+      tt = transpose(%{t | shape: permute(shape, perm), names: permute_names(t.names, perm)}, t, perm)
+      {tt, prod(Enum.map(kept, &elem(shape, &1))), prod(Enum.map(axes, &elem(shape, &1))), 1}
+    end
+  end
+
+  defp prod(list), do: Enum.product(list)
+  defp permute(shape, perm), do: perm |> Enum.map(&elem(shape, &1)) |> List.to_tuple()
+  defp permute_names(names, perm), do: Enum.map(perm, &Enum.at(names, &1))
+
+  ## Contraction
+
+  @impl true
+  def dot(out, %T{} = l, c1, b1, %T{} = r, c2, b2) do
+    device = device_of([l, r])
+    # walk the contraction pairs in increasing left-axis order: no copy of the left operand
+    # whenever its contracted axes are adjacent (the pairing itself is kept)
+    {c1, c2} = Enum.zip(c1, c2) |> Enum.sort() |> Enum.unzip()
+    nb = length(b1)
+    k = prod(Enum.map(c1, &elem(l.shape, &1)))
+    batch = prod(Enum.map(b1, &elem(l.shape, &1)))
+    {lt, l_layout, m} = dot_operand(l, c1, nb)
+    {rt, r_layout, n} = dot_operand(r, c2, nb)
+    {lref, _} = from_nx(lt, device)
+    {rref, _} = from_nx(rt, device)
+
+    ref =
+      NIF.dot(ctx(device), dt(l.type), dt(r.type), dt(out.type), batch, m, n, k, l_layout, r_layout, lref, rref, bytes(out))
+
+    to_nx(unwrap!(ref), device, out)
+  end
+
+  # [batch, rows, K] (layout 0) or [batch, K, rows] (layout 1) in place when the axes already
+  # sit that way, else transposed to [batch, kept, contract] as Nx.BinaryBackend does
+  defp dot_operand(%T{shape: shape} = t, contract, nb) do
+    rank = tuple_size(shape)
+    batch = Enum.to_list(0..(nb - 1)//1)
+    kept = Enum.to_list(nb..(rank - 1)//1) -- contract
+    rows = prod(Enum.map(kept, &elem(shape, &1)))
+    identity = Enum.to_list(0..(rank - 1)//1)
+
+    cond do
+      batch ++ kept ++ contract == identity -> {t, 0, rows}
+      batch ++ contract ++ kept == identity -> {t, 1, rows}
+      true ->
+        perm = batch ++ kept ++ contract
+        {transpose(%{t | shape: permute(shape, perm), names: permute_names(t.names, perm)}, t, perm), 0, rows}
+    end
+  end
+
+  ## Data movement
+
+  @impl true
+  def transpose(out, %T{type: {_, bits}} = t, axes) do
+    device = device_of([t])
+    {ref, _} = from_nx(t, device)
+    to_nx(unwrap!(NIF.transpose(ctx(device), div(bits, 8), Tuple.to_list(t.shape), axes, ref, bytes(out))), device, out)
+  end
+
+  @impl true
+  def broadcast(out, %T{type: {_, bits}} = t, shape, axes) do
+    device = device_of([t])
+    {ref, _} = from_nx(t, device)
+    in_dims = Tuple.to_list(t.shape)
+
+    {pairs, _} =
+      Enum.zip(in_dims, axes)
+      |> Enum.reverse()
+      |> Enum.map_reduce(1, fn {dim, axis}, acc -> {{axis, if(dim == 1, do: 0, else: acc)}, acc * dim} end)
+
+    by_axis = Map.new(pairs)
+    strides = for a <- 0..(tuple_size(shape) - 1)//1, do: Map.get(by_axis, a, 0)
+    to_nx(unwrap!(NIF.broadcast(ctx(device), div(bits, 8), Tuple.to_list(shape), strides, ref, bytes(out))), device, out)
+  end
+
+  @impl true
+  def gather(out, %T{type: {_, bits}} = t, %T{} = indices, opts) do
+    device = device_of([t, indices])
+    axes = opts[:axes]
+    t_axes = Nx.axes(t)
+
+    t =
+      if List.starts_with?(t_axes, axes) do
+        t
+      else
+        perm = axes ++ (t_axes -- axes)
+        transpose(%{t | shape: permute(t.shape, perm), names: permute_names(t.names, perm)}, t, perm)
+      end
+
+    {tref, _} = from_nx(t, device)
+    {iref, _} = from_nx(indices, device)
+    depth = elem(indices.shape, tuple_size(indices.shape) - 1)
+    n_tuples = div(Nx.size(indices), depth)
+
+    ref =
+      NIF.gather(ctx(device), div(bits, 8), Tuple.to_list(t.shape), dt(indices.type), n_tuples, depth, 0, tref, iref, bytes(out))
+
+    to_nx(unwrap!(ref), device, out)
+  end
+
+  @impl true
+  def block(%Nx.Block.Take{axis: 0}, out, [t, indices], _fun) do
+    gather(out, t, %{indices | shape: {Nx.size(indices), 1}, names: [nil, nil]}, axes: [0])
+  end
+
+  def block(struct, _out, args, fun), do: apply(fun, [struct | args])
+
+  ## Everything else: round trip through Nx.BinaryBackend
+
+  fallbacks =
+    Nx.Backend.behaviour_info(:callbacks) --
+      (Module.definitions_in(__MODULE__, :def) ++ [from_pointer: 5, to_pointer: 2])
+
+  for {name, arity} <- fallbacks do
+    args = Macro.generate_arguments(arity, __MODULE__)
+
+    @impl true
+    def unquote(name)(unquote_splicing(args)) do
+      device = device_of(Enum.filter(unquote(args), &is_struct(&1, T)))
+
+      host = fn
+        %T{data: %__MODULE__{}} = t -> Nx.backend_copy(t, Nx.BinaryBackend)
+        list when is_list(list) -> Enum.map(list, &if(is_struct(&1, T), do: Nx.backend_copy(&1, Nx.BinaryBackend), else: &1))
+        other -> other
+      end
+
+      result = apply(Nx.BinaryBackend, unquote(name), Enum.map(unquote(args), host))
+
+      back = fn
+        %T{data: %Nx.BinaryBackend{}} = t -> Nx.backend_transfer(t, {__MODULE__, device: device})
+        other -> other
+      end
+
+      case result do
+        list when is_list(list) -> Enum.map(list, back)
+        other -> back.(other)
+      end
+    end
+  end
+
+  @impl true
+  def from_pointer(_, _, _, _, _), do: raise(ArgumentError, "HipNx.Backend does not support pointers")
+  @impl true
+  def to_pointer(_, _), do: raise(ArgumentError, "HipNx.Backend does not support pointers")
+end

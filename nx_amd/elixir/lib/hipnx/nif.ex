@@ -1,0 +1,30 @@
+defmodule HipNx.NIF do
+  @moduledoc false
+  # Stubs replaced by c_src/hipnx_nif.c at load time (same scheme as torchx/lib/torchx/nif.ex).
+  @on_load :__on_load__
+
+  def __on_load__ do
+    path = :filename.join(:code.priv_dir(:hipnx), ~c"hipnx_nif")
+    :erlang.load_nif(path, 0)
+  end
+
+  def device_count, do: err()
+  def ctx_create(_device), do: err()
+  def from_binary(_ctx, _binary, _nbytes), do: err()
+  def to_binary(_ctx, _buf, _nbytes), do: err()
+  def alloc(_ctx, _nbytes), do: err()
+  def deallocate(_buf), do: err()
+  def copy(_ctx, _buf, _nbytes), do: err()
+  def fill(_ctx, _elem, _count), do: err()
+  def binary(_ctx, _op, _l_dt, _r_dt, _out_dt, _dims, _l_strides, _r_strides, _l, _r, _out_bytes), do: err()
+  def unary(_ctx, _op, _in_dt, _out_dt, _n, _in, _out_bytes), do: err()
+  def reduce(_ctx, _op, _in_dt, _out_dt, _outer, _red, _inner, _in, _out_bytes), do: err()
+  def argreduce(_ctx, _op, _tie, _in_dt, _out_dt, _outer, _red, _inner, _in, _out_bytes), do: err()
+  def dot(_ctx, _l_dt, _r_dt, _out_dt, _batch, _m, _n, _k, _l_layout, _r_layout, _l, _r, _out_bytes), do: err()
+  def transpose(_ctx, _elem_bytes, _dims, _perm, _in, _out_bytes), do: err()
+  def broadcast(_ctx, _elem_bytes, _dims, _strides, _in, _out_bytes), do: err()
+  def gather(_ctx, _elem_bytes, _dims, _idx_dt, _n_tuples, _depth, _policy, _t, _idx, _out_bytes), do: err()
+  def sync(_ctx), do: err()
+
+  defp err, do: :erlang.nif_error(:undef)
+end
