@@ -148,6 +148,7 @@ int hipnx_ctx_create(int device, hipnx_ctx **out) {
   hipError_t e3 = hipEventCreate(&ctx->ev_stop);
   hipError_t e4 = hipMalloc(&ctx->flag, 256);
   hipError_t e5 = hipHostMalloc(&ctx->flag_host, 256, hipHostMallocDefault);
+  if (e4 == hipSuccess) e4 = hipMemset(ctx->flag, 0xFF, 256);  // gather bounds word: all-ones = no bad index
   if (e1 != hipSuccess || e2 != hipSuccess || e3 != hipSuccess || e4 != hipSuccess || e5 != hipSuccess) {
     hipnx_ctx_destroy(ctx);
     return hip_fail(e1 != hipSuccess ? e1 : e2 != hipSuccess ? e2 : e3 != hipSuccess ? e3 : e4 != hipSuccess ? e4 : e5,

@@ -221,7 +221,7 @@ __device__ __forceinline__ void wait_vmcnt() {  // s_waitcnt vmcnt(N), other cou
   __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
 }
 
-template <int DT, int WM, int WN, int TM, int TN, bool L_KIN, bool R_KIN>
+template <int DT, int WM, int WN, int TM, int TN, bool L_KIN, bool R_KIN, int NSTAGE = 2>
 __global__ void __launch_bounds__(WM *WN * 64)
 gemm_pipelined_kernel(GemmArgs a) {
   typedef typename Mma<DT>::acc_t acc_t;
@@ -276,16 +276,27 @@ gemm_pipelined_kernel(GemmArgs a) {
     if constexpr (!R_KIN) store_slab_kouter16<BN, NT>(rregs, sB, tid);
   };
 
+  // NSTAGE LDS stages, slab s lives in stage s % NSTAGE, NSTAGE-1 slabs are requested ahead.
+  // Per slab: wait until my own loads of slab s have landed (younger ones may still fly: loads
+  // complete in issue order), barrier (everyone's loads of slab s are in, everyone is done
+  // reading slab s-1), refill the stage slab s-1 occupied with slab s+NSTAGE-1, then compute.
   const int nslab = (int)(a.Kb / SLAB);
-  issue(0, 0);
+  constexpr int AHEAD = NSTAGE - 1;
+  constexpr int OPS = (L_KIN ? KInnerLoader<BM, NW>::PER : 0) + (R_KIN ? KInnerLoader<BN, NW>::PER : 0);
+  static_assert(NSTAGE == 2 || (L_KIN && R_KIN), "deep pipelines are for K-inner operands");
+  static_assert(OPS * (AHEAD - 1) < 64, "vmcnt is a 6-bit counter");
+#pragma unroll
+  for (int p = 0; p < AHEAD; p++)
+    if (p < nslab) issue(p, (int64_t)p * SLAB);
   commit(0);
-  wait_vmcnt<0>();  // my direct-to-LDS loads have landed
-  __syncthreads();
 
   for (int s = 0; s < nslab; s++) {
-    const int cur = s & 1;
-    if (s + 1 < nslab) issue(cur ^ 1, (int64_t)(s + 1) * SLAB);
-    const unsigned char *sA = smem + cur * STAGE, *sB = sA + BM * SLAB;
+    // slabs s+1 .. s+AHEAD-1 may stay in flight, unless the walk is about to end
+    if (s + AHEAD - 1 < nslab) wait_vmcnt<OPS *(AHEAD - 1)>();
+    else wait_vmcnt<0>();
+    __syncthreads();
+    if (s + AHEAD < nslab) issue((s + AHEAD) % NSTAGE, (int64_t)(s + AHEAD) * SLAB);
+    const unsigned char *sA = smem + (s % NSTAGE) * STAGE, *sB = sA + BM * SLAB;
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ks++) {
       v4i fa[TM], fb[TN];
@@ -305,9 +316,8 @@ gemm_pipelined_kernel(GemmArgs a) {
 #pragma unroll
         for (int j = 0; j < TN; j++) Mma<DT>::step(acc[i][j], fb[j], fa[i]);
     }
-    if (s + 1 < nslab) commit(cur ^ 1);
-    wait_vmcnt<0>();
-    __syncthreads();
+    // K-outer operands (NSTAGE == 2): the registers fetched above go to the other stage now
+    if (s + AHEAD < nslab) commit((s + AHEAD) % NSTAGE);
   }
 
   // epilogue: the output type is wave-uniform; branch once, then every store is straight-line

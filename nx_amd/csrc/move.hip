@@ -66,18 +66,18 @@ transpose2d_kernel(const T *__restrict__ in, T *__restrict__ out, int64_t R, int
 }
 
 // gather: tuple i of `idx` ([n_tuples, depth]) selects a slice of `slice_bytes` bytes.
-// One block-row of lanes copies a slice with 16-byte (VEC) or 1-byte accesses.
-// flag[0] receives the smallest (tuple * depth + axis) whose index is out of range.
+// LPR lanes (a power of two, at most one wavefront) copy one slice with 16-byte (VEC) or 1-byte
+// accesses, four independent accesses in flight per lane; a 256-lane block works on 256/LPR
+// slices at once so that the index -> address -> data dependency of one slice overlaps with the
+// others'.  flag[0] receives the smallest (tuple * depth + axis) whose index is out of range.
 template <bool VEC>
 __global__ void __launch_bounds__(BLOCK)
 gather_kernel(const unsigned char *__restrict__ t, const void *__restrict__ idx, unsigned char *__restrict__ out,
               int idx_dt, int64_t n_tuples, int depth, Strided tdims /* dims = leading extents, strides = bytes */,
-              int64_t slice_bytes, int clamp, unsigned long long *__restrict__ flag) {
+              int64_t slice_bytes, int lpr, int clamp, unsigned long long *__restrict__ flag) {
   constexpr int W = VEC ? 16 : 1;
+  typedef raw_vec<W> vec_t;
   const int64_t chunks = slice_bytes / W;
-  // lanes_per_row: enough lanes to cover a slice, at most the block
-  int lpr = BLOCK;
-  while (lpr > 1 && lpr / 2 >= chunks) lpr >>= 1;
   const int rpb = BLOCK / lpr;
   const int sub = threadIdx.x / lpr, lane = threadIdx.x % lpr;
   for (int64_t row = (int64_t)blockIdx.x * rpb + sub; row < n_tuples; row += (int64_t)gridDim.x * rpb) {
@@ -98,16 +98,21 @@ gather_kernel(const unsigned char *__restrict__ t, const void *__restrict__ idx,
       off += v * tdims.strides[a];
     }
     if (!ok) continue;
-    const unsigned char *src = t + off;
-    unsigned char *dst = out + row * slice_bytes;
-    for (int64_t c = lane; c < chunks; c += lpr)
-      *reinterpret_cast<raw_vec<W> *>(dst + c * W) = *reinterpret_cast<const raw_vec<W> *>(src + c * W);
+    const vec_t *src = reinterpret_cast<const vec_t *>(t + off);
+    vec_t *dst = reinterpret_cast<vec_t *>(out + row * slice_bytes);
+    int64_t c = lane;
+    for (; c + 3 * (int64_t)lpr < chunks; c += 4 * (int64_t)lpr) {
+      vec_t v0 = src[c], v1 = src[c + lpr], v2 = src[c + 2 * lpr], v3 = src[c + 3 * lpr];
+      dst[c] = v0; dst[c + lpr] = v1; dst[c + 2 * lpr] = v2; dst[c + 3 * lpr] = v3;
+    }
+    for (; c < chunks; c += lpr) dst[c] = src[c];
   }
 }
 
 static int grid_for(const hipnx_ctx *ctx, int64_t items, int per_block) {
   int64_t blocks = (items + per_block - 1) / per_block;
-  int64_t cap = (int64_t)ctx->num_cus * 16;
+  (void)ctx;
+  int64_t cap = 1ll << 30;  // cover the whole index space: faster here than a resident grid that loops
   if (blocks < 1) blocks = 1;
   return (int)(blocks < cap ? blocks : cap);
 }
@@ -283,28 +288,30 @@ extern "C" int hipnx_gather(hipnx_ctx *ctx, int elem_bytes, int rank, const int6
     int64_t s = slice_bytes;
     for (int a = depth - 1; a >= 0; a--) { td.dims[a] = t_dims[a]; td.strides[a] = s; s *= t_dims[a]; }
   }
+  // bounds report: a device word that stays all-ones until a kernel finds a bad index (it is set
+  // when the context is created and re-armed below after a failure), so the common path needs
+  // no launch to clear it
   unsigned long long *flag = (unsigned long long *)ctx->flag;
-  if (oob_policy == HIPNX_OOB_RAISE)
-    hipLaunchKernelGGL((fill_kernel<unsigned long long>), dim3(1), dim3(BLOCK), 0, ctx->stream, flag, ~0ull, (int64_t)1);
   const bool vec = slice_bytes % 16 == 0;
   int64_t chunks = vec ? slice_bytes / 16 : slice_bytes;
-  int lpr = BLOCK;
+  int lpr = 64;  // lanes per slice: at most one wavefront, fewer for short slices
   while (lpr > 1 && lpr / 2 >= chunks) lpr >>= 1;
   dim3 grid(grid_for(ctx, n_tuples, BLOCK / lpr)), block(BLOCK);
   if (vec)
     hipLaunchKernelGGL((gather_kernel<true>), grid, block, 0, ctx->stream, (const unsigned char *)t->ptr, idx->ptr,
-                       (unsigned char *)out->ptr, idx_dt, n_tuples, depth, td, slice_bytes, (int)(oob_policy == HIPNX_OOB_CLAMP), flag);
+                       (unsigned char *)out->ptr, idx_dt, n_tuples, depth, td, slice_bytes, lpr, (int)(oob_policy == HIPNX_OOB_CLAMP), flag);
   else
     hipLaunchKernelGGL((gather_kernel<false>), grid, block, 0, ctx->stream, (const unsigned char *)t->ptr, idx->ptr,
-                       (unsigned char *)out->ptr, idx_dt, n_tuples, depth, td, slice_bytes, (int)(oob_policy == HIPNX_OOB_CLAMP), flag);
+                       (unsigned char *)out->ptr, idx_dt, n_tuples, depth, td, slice_bytes, lpr, (int)(oob_policy == HIPNX_OOB_CLAMP), flag);
   HIPNX_HIP(hipGetLastError());
   if (oob_policy == HIPNX_OOB_RAISE) {
     // the reference raises on the first offending index: wait, then report it the same way
-    unsigned long long *host = (unsigned long long *)ctx->flag_host;
-    HIPNX_HIP(hipMemcpyAsync(host, flag, 8, hipMemcpyDeviceToHost, ctx->stream));
+    volatile unsigned long long *host = (volatile unsigned long long *)ctx->flag_host;
+    HIPNX_HIP(hipMemcpyAsync((void *)host, flag, 8, hipMemcpyDeviceToHost, ctx->stream));
     HIPNX_HIP(hipStreamSynchronize(ctx->stream));
     if (host[0] != ~0ull) {
       const int64_t pos = (int64_t)host[0];
+      HIPNX_HIP(hipMemsetAsync(flag, 0xFF, 8, ctx->stream));  // re-arm
       const int axis = (int)(pos % depth);
       unsigned char raw[8] = {0};
       const int isz = dtype_size(idx_dt);

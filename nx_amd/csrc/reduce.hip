@@ -37,16 +37,16 @@ struct PlainReducer {
   static __device__ __forceinline__ acc_t init() {
     if constexpr (OP == HIPNX_RED_SUM) return (CT)0;
     else if constexpr (OP == HIPNX_RED_PRODUCT) return (CT)1;
-    else if constexpr (std::is_same<CT, double>::value) return OP == HIPNX_RED_MAX ? -INFINITY : INFINITY;
+    else if constexpr (std::is_floating_point<CT>::value) return OP == HIPNX_RED_MAX ? (CT)-INFINITY : (CT)INFINITY;
     else if constexpr (UNS) return OP == HIPNX_RED_MAX ? (int64_t)0 : (int64_t)-1;
     else return OP == HIPNX_RED_MAX ? INT64_MIN : INT64_MAX;
   }
   static __device__ __forceinline__ acc_t combine(acc_t a, acc_t b) {
-    if constexpr (std::is_same<CT, double>::value) {
+    if constexpr (std::is_floating_point<CT>::value) {
       if constexpr (OP == HIPNX_RED_SUM) return a + b;
       else if constexpr (OP == HIPNX_RED_PRODUCT) return a * b;
-      else if constexpr (OP == HIPNX_RED_MAX) return (a != a || b != b) ? (double)NAN : (b > a ? b : a);
-      else return (a != a || b != b) ? (double)NAN : (b < a ? b : a);
+      else if constexpr (OP == HIPNX_RED_MAX) return (a != a || b != b) ? (CT)NAN : (b > a ? b : a);
+      else return (a != a || b != b) ? (CT)NAN : (b < a ? b : a);
     } else {
       if constexpr (OP == HIPNX_RED_SUM) return (int64_t)((uint64_t)a + (uint64_t)b);
       else if constexpr (OP == HIPNX_RED_PRODUCT) return (int64_t)((uint64_t)a * (uint64_t)b);
@@ -59,6 +59,7 @@ struct PlainReducer {
       }
     }
   }
+  static __device__ __forceinline__ acc_t seed(acc_t a, int64_t) { return a; }
   static __device__ __forceinline__ acc_t accumulate(acc_t a, CT x, int64_t) { return combine(a, x); }
   static __device__ __forceinline__ acc_t shfl_xor(acc_t a, int m) { return __shfl_xor(a, m, WAVE); }
 };
@@ -66,41 +67,58 @@ struct PlainReducer {
 template <typename CT>
 struct ArgAcc {
   CT v;
-  int64_t i;  // -1 = empty
-  int nan;
+  int i;  // position along the reduced axis (extents below 2^31); -1 = empty
 };
 
 template <typename CT, int OP, int TIE, bool UNS>
 struct ArgReducer {
   typedef ArgAcc<CT> acc_t;
-  static __device__ __forceinline__ acc_t init() { return acc_t{(CT)0, -1, 0}; }
+  static constexpr bool FP = std::is_floating_point<CT>::value;
+  // the worst possible value: nothing is worse, so a lane seeded with {worst, first index} is
+  // already the right answer for "no better element seen yet"
+  static __device__ __forceinline__ acc_t init() {
+    if constexpr (FP) return acc_t{OP == HIPNX_ARGMAX ? (CT)-INFINITY : (CT)INFINITY, -1};
+    else if constexpr (UNS) return acc_t{OP == HIPNX_ARGMAX ? (CT)0 : (CT)-1, -1};
+    else return acc_t{OP == HIPNX_ARGMAX ? (CT)INT64_MIN : (CT)INT64_MAX, -1};
+  }
+  static __device__ __forceinline__ acc_t seed(acc_t a, int64_t first) { a.i = (int)first; return a; }
   static __device__ __forceinline__ bool better(CT x, CT y) {  // x strictly better than y
     if constexpr (std::is_same<CT, int64_t>::value && UNS)
       return OP == HIPNX_ARGMAX ? (uint64_t)x > (uint64_t)y : (uint64_t)x < (uint64_t)y;
     else return OP == HIPNX_ARGMAX ? x > y : x < y;
   }
+  static __device__ __forceinline__ bool better_or_equal(CT x, CT y) {
+    if constexpr (std::is_same<CT, int64_t>::value && UNS)
+      return OP == HIPNX_ARGMAX ? (uint64_t)x >= (uint64_t)y : (uint64_t)x <= (uint64_t)y;
+    else return OP == HIPNX_ARGMAX ? x >= y : x <= y;
+  }
+  // any order (cross-lane tree, partials): NaN beats numbers, the larger index wins among NaNs
   static __device__ __forceinline__ acc_t combine(acc_t a, acc_t b) {
     if (b.i < 0) return a;
     if (a.i < 0) return b;
-    if (a.nan | b.nan) {
-      if (a.nan && b.nan) return a.i > b.i ? a : b;
-      return a.nan ? a : b;
+    if constexpr (FP) {
+      const bool an = a.v != a.v, bn = b.v != b.v;
+      if (an | bn) {
+        if (an && bn) return a.i > b.i ? a : b;
+        return an ? a : b;
+      }
     }
     if (better(b.v, a.v)) return b;
     if (better(a.v, b.v)) return a;
     if constexpr (TIE == HIPNX_TIE_LOW) return a.i < b.i ? a : b;
     else return a.i > b.i ? a : b;
   }
+  // streaming step of a seeded lane: indices only grow, so a tie resolves by position, and a
+  // NaN extreme is sticky by itself (every comparison with it is false)
   static __device__ __forceinline__ acc_t accumulate(acc_t a, CT x, int64_t idx) {
-    int isnan = 0;
-    if constexpr (std::is_same<CT, double>::value) isnan = x != x;
-    return combine(a, acc_t{x, idx, isnan});
+    bool take = TIE == HIPNX_TIE_LOW ? better(x, a.v) : better_or_equal(x, a.v);
+    if constexpr (FP) take |= x != x;
+    return take ? acc_t{x, (int)idx} : a;
   }
   static __device__ __forceinline__ acc_t shfl_xor(acc_t a, int m) {
     acc_t r;
     r.v = __shfl_xor(a.v, m, WAVE);
     r.i = __shfl_xor(a.i, m, WAVE);
-    r.nan = __shfl_xor(a.nan, m, WAVE);
     return r;
   }
 };
@@ -116,7 +134,7 @@ template <typename CT>
 __device__ __forceinline__ void finalize(void *out, int odt, int64_t o, CT v) { store_one<CT>(out, odt, o, v); }
 template <typename CT>
 __device__ __forceinline__ void finalize(void *out, int odt, int64_t o, ArgAcc<CT> a) {
-  store_one<int64_t>(out, odt, o, a.i);
+  store_one<int64_t>(out, odt, o, (int64_t)a.i);
 }
 
 // ---- rows: inner == 1 -----------------------------------------------------------------------
@@ -138,13 +156,27 @@ reduce_rows_kernel(const void *__restrict__ in, void *__restrict__ out, typename
     const int64_t k1 = k0 + seg_len < red ? k0 + seg_len : red;
     const int64_t base = row * red;
     if constexpr (VEC) {  // red % E == 0 and seg_len % E == 0: every vector is aligned
-      for (int64_t k = k0 + (int64_t)lane * E; k < k1; k += (int64_t)TPR * E) {
+      // two (then one) 8-element vectors per step: both loads are issued before either is folded
+      int64_t k = k0 + (int64_t)lane * E;
+      if (k < k1) acc = R::seed(acc, k);
+      const int64_t step = (int64_t)TPR * E;
+      for (; k + step < k1; k += 2 * step) {
+        CT v[E], w[E];
+        load_vec<CT, E>(in, idt, base + k, v);
+        load_vec<CT, E>(in, idt, base + k + step, w);
+#pragma unroll
+        for (int i = 0; i < E; i++) acc = R::accumulate(acc, v[i], k + i);
+#pragma unroll
+        for (int i = 0; i < E; i++) acc = R::accumulate(acc, w[i], k + step + i);
+      }
+      for (; k < k1; k += step) {
         CT v[E];
         load_vec<CT, E>(in, idt, base + k, v);
 #pragma unroll
         for (int i = 0; i < E; i++) acc = R::accumulate(acc, v[i], k + i);
       }
     } else {
+      if (k0 + lane < k1) acc = R::seed(acc, k0 + lane);
       for (int64_t k = k0 + lane; k < k1; k += TPR) acc = R::accumulate(acc, load_one<CT>(in, idt, base + k), k);
     }
   }
@@ -196,9 +228,24 @@ reduce_cols_kernel(const void *__restrict__ in, void *__restrict__ out, typename
     const int64_t k0 = (int64_t)seg * seg_len, k1 = k0 + seg_len < red ? k0 + seg_len : red;
     typename R::acc_t acc[W];
 #pragma unroll
-    for (int i = 0; i < W; i++) acc[i] = R::init();
+    for (int i = 0; i < W; i++) acc[i] = k0 < k1 ? R::seed(R::init(), k0) : R::init();
     const int64_t base = o * red * inner + iv * W;
-    for (int64_t k = k0; k < k1; k++) {
+    int64_t k = k0;
+    for (; k + 3 < k1; k += 4) {  // four independent row loads in flight per lane
+      CT v0[W], v1[W], v2[W], v3[W];
+      load_vec<CT, W>(in, idt, base + k * inner, v0);
+      load_vec<CT, W>(in, idt, base + (k + 1) * inner, v1);
+      load_vec<CT, W>(in, idt, base + (k + 2) * inner, v2);
+      load_vec<CT, W>(in, idt, base + (k + 3) * inner, v3);
+#pragma unroll
+      for (int i = 0; i < W; i++) {
+        acc[i] = R::accumulate(acc[i], v0[i], k);
+        acc[i] = R::accumulate(acc[i], v1[i], k + 1);
+        acc[i] = R::accumulate(acc[i], v2[i], k + 2);
+        acc[i] = R::accumulate(acc[i], v3[i], k + 3);
+      }
+    }
+    for (; k < k1; k++) {
       CT v[W];
       load_vec<CT, W>(in, idt, base + k * inner, v);
 #pragma unroll
@@ -299,7 +346,7 @@ static int run_reduce(hipnx_ctx *ctx, int idt, int odt, int64_t outer, int64_t r
     }
     int64_t total = lanes * nseg;
     int64_t blocks = (total + BLOCK - 1) / BLOCK;
-    int64_t cap = (int64_t)ctx->num_cus * 32;
+    int64_t cap = 1ll << 30;
     dim3 grid((unsigned)(blocks < 1 ? 1 : (blocks < cap ? blocks : cap))), block(BLOCK);
     if (total > 0) {
       if (vec) hipLaunchKernelGGL((reduce_cols_kernel<R, CT, true>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, outer, red, inner, seg_len, nseg);
@@ -319,6 +366,9 @@ static int run_reduce(hipnx_ctx *ctx, int idt, int odt, int64_t outer, int64_t r
 template <int OP>
 static int reduce_op(hipnx_ctx *ctx, int idt, int odt, int64_t outer, int64_t red, int64_t inner, const void *in,
                      void *out) {
+  // selection (max / min) is exact in the element's own precision: f32 covers f32, bf16 and f16
+  if (is_float(idt) && idt != HIPNX_F64 && (OP == HIPNX_RED_MAX || OP == HIPNX_RED_MIN))
+    return run_reduce<PlainReducer<float, OP, false>, float>(ctx, idt, odt, outer, red, inner, in, out);
   if (is_float(idt)) return run_reduce<PlainReducer<double, OP, false>, double>(ctx, idt, odt, outer, red, inner, in, out);
   if (idt == HIPNX_U64 && (OP == HIPNX_RED_MAX || OP == HIPNX_RED_MIN))
     return run_reduce<PlainReducer<int64_t, OP, true>, int64_t>(ctx, idt, odt, outer, red, inner, in, out);
@@ -328,6 +378,8 @@ static int reduce_op(hipnx_ctx *ctx, int idt, int odt, int64_t outer, int64_t re
 template <int OP, int TIE>
 static int argreduce_op(hipnx_ctx *ctx, int idt, int odt, int64_t outer, int64_t red, int64_t inner, const void *in,
                         void *out) {
+  if (is_float(idt) && idt != HIPNX_F64)
+    return run_reduce<ArgReducer<float, OP, TIE, false>, float>(ctx, idt, odt, outer, red, inner, in, out);
   if (is_float(idt)) return run_reduce<ArgReducer<double, OP, TIE, false>, double>(ctx, idt, odt, outer, red, inner, in, out);
   if (idt == HIPNX_U64) return run_reduce<ArgReducer<int64_t, OP, TIE, true>, int64_t>(ctx, idt, odt, outer, red, inner, in, out);
   return run_reduce<ArgReducer<int64_t, OP, TIE, false>, int64_t>(ctx, idt, odt, outer, red, inner, in, out);
@@ -372,6 +424,7 @@ extern "C" int hipnx_argreduce(hipnx_ctx *ctx, int op, int tie, int in_dt, int o
     return set_error(HIPNX_EINVAL, "argreduce: bad element type (the output must be an integer type)");
   if (int st = check_view(outer, red, inner)) return st;
   if (red == 0 && outer * inner > 0) return set_error(HIPNX_EINVAL, "argreduce: empty axis");
+  if (red > 0x7FFFFFFF) return set_error(HIPNX_EUNSUPPORTED, "argreduce: more than 2^31 - 1 elements along the reduced axis");
   if (int st = check_buf(ctx, inb, (uint64_t)outer * red * inner * dtype_size(in_dt), "argreduce in")) return st;
   if (int st = check_buf(ctx, out, (uint64_t)outer * inner * dtype_size(out_dt), "argreduce out")) return st;
   if (outer * inner == 0) return HIPNX_OK;
