@@ -2,9 +2,10 @@
 // argument checks and the choice of kernel.
 //
 //   bf16 / f16 / f32 operand pairs (f32 accumulation) and s8 pairs (exact s32 accumulation):
-//     K a multiple of 128 bytes  -> the pipelined MFMA kernel (gemm_mfma.cuh).  bf16 / f16 take
-//       both operand layouts directly; K-outer f32 / s8 operands (and ragged 2-byte ones) are
-//       first re-laid by the tiled transpose.
+//     K a multiple of 128 bytes  -> the pipelined MFMA kernel (gemm_mfma.cuh), which takes both
+//       operand layouts directly; only a K-outer operand whose row count is not a multiple of
+//       its transpose block (16 s8 / 8 bf16,f16 / 4 f32 rows) is first re-laid by the tiled
+//       transpose.
 //     K a multiple of 16 bytes   -> gemm_kinner_kernel below: same MFMA fragments, single LDS
 //       stage, register-staged loads, zero-filled K tail.
 //   everything else (f64, wide integers, mixed operand types, tiny problems): dot_generic_kernel,
@@ -204,9 +205,10 @@ extern "C" int hipnx_dot(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t
   // MFMA path.  Which operands need the tiled transpose to become K-inner first?
   const int esz = dtype_size(l_dt);
   const bool pipelined = Kb % SLAB == 0;
-  const bool native_kouter = pipelined && esz == 2;  // the pipelined kernel transposes 2-byte operands itself
-  const bool l_relay = l_layout == HIPNX_K_OUTER && !(native_kouter && M % 8 == 0);
-  const bool r_relay = r_layout == HIPNX_K_OUTER && !(native_kouter && N % 8 == 0);
+  // the pipelined kernel transposes K-outer operands itself when the rows come in whole blocks
+  const int row_block = esz == 1 ? 16 : (esz == 2 ? 8 : 4);
+  const bool l_relay = l_layout == HIPNX_K_OUTER && !(pipelined && M % row_block == 0);
+  const bool r_relay = r_layout == HIPNX_K_OUTER && !(pipelined && N % row_block == 0);
   hipnx_buf *lt = nullptr, *rt = nullptr;
   int st = HIPNX_OK;
   if (l_relay) {
@@ -252,8 +254,8 @@ extern "C" int hipnx_dot(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t
         switch (l_dt) {
           case HIPNX_BF16: st = launch_gemm_bf16(ctx, cfg, l_kin, r_kin, a, batch); break;
           case HIPNX_F16: st = launch_gemm_f16(ctx, cfg, l_kin, r_kin, a, batch); break;
-          case HIPNX_F32: st = launch_gemm_f32(ctx, cfg, a, batch); break;
-          default: st = launch_gemm_s8(ctx, cfg, a, batch); break;
+          case HIPNX_F32: st = launch_gemm_f32(ctx, cfg, l_kin, r_kin, a, batch); break;
+          default: st = launch_gemm_s8(ctx, cfg, l_kin, r_kin, a, batch); break;
         }
       } else {
         switch (l_dt) {

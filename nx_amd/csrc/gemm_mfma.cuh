@@ -13,9 +13,10 @@
 //   K-inner operand ([rows, K], K contiguous): `global_load_lds_dwordx4` -- each lane moves 16 B
 //     straight from global memory into LDS, no VGPR round trip.  A wave instruction fills 1 KiB of
 //     LDS (8 rows x 8 chunks); the lane picks the *global* chunk that belongs at its LDS slot.
-//   K-outer operand ([K, rows], rows contiguous; 2-byte types): each lane loads an 8(k) x 8(row)
-//     block with eight 16-byte row loads, transposes it in registers with byte permutes and
-//     writes eight 16-byte K-runs to LDS -- the slab arrives in the same [row][k] LDS layout.
+//   K-outer operand ([K, rows], rows contiguous): each lane loads a small k x rows block with
+//     16-byte row loads, transposes it in registers (byte permutes) and writes K-runs to LDS --
+//     the slab arrives in the same [row][k] LDS layout, so a plain `Nx.dot(a, b)` needs no
+//     re-layout pass.
 // LDS layout of a unit: row-major, 128 B per row, the 16-byte chunk index XOR-ed with
 // ((row ^ row>>3) & 7): conflict-free for the fragment reads (32 consecutive rows, one chunk) and
 // for the transposed writes (rows 8 apart, one chunk).
@@ -104,67 +105,150 @@ struct KInnerLoader {
   }
 };
 
-// 8 x 8 transpose of 16-bit elements held as rows[k] = 8 consecutive `row` values at one k:
-// out[i] = the 8 consecutive k values of row i.
-__device__ __forceinline__ void transpose8x8_b16(const v4i (&in)[8], v4i (&out)[8]) {
+// ---- K-outer operands: g is [K, rows] (rows contiguous).  A lane loads a small block of
+// 16-byte row runs at consecutive k, transposes it in registers and writes K-runs into the same
+// [row][k] LDS layout the K-inner loader produces.  Block shape per element size ES:
+//   ES = 2:  8 k x  8 rows -> eight 16-byte K-runs (v_perm_b32 pairs halves)
+//   ES = 4:  4 k x  4 rows -> four 16-byte K-runs (pure register renaming)
+//   ES = 1:  4 k x 16 rows -> sixteen 4-byte K-runs (4 x 4 byte transposes with v_perm_b32)
+// `rows_valid` must be a multiple of the block's row count (the host falls back to a transpose
+// pass otherwise); k never runs past K because K*ES is a multiple of the slab.
+template <int ES> struct KOuterShape;
+template <> struct KOuterShape<2> { static constexpr int KB = 8, RB = 8; };
+template <> struct KOuterShape<4> { static constexpr int KB = 4, RB = 4; };
+template <> struct KOuterShape<1> { static constexpr int KB = 4, RB = 16; };
+
+template <int ES, int ROWS, int NTHREADS>
+struct KOuterStage {
+  static constexpr int KB = KOuterShape<ES>::KB, RB = KOuterShape<ES>::RB;
+  static constexpr int KSLAB = SLAB / ES;                       // k values per slab
+  static constexpr int BLOCKS = (ROWS / RB) * (KSLAB / KB);
+  static constexpr int PER = (BLOCKS + NTHREADS - 1) / NTHREADS;
+  static constexpr int LOADS = PER * KB;                        // vector-memory ops per slab per lane
+  v4i v[PER][KB];
+
+  __device__ __forceinline__ void fetch(const unsigned char *__restrict__ g, int64_t ld, int64_t row0, int64_t rows_valid,
+                                        int64_t k0, int tid) {
 #pragma unroll
-  for (int i = 0; i < 8; i++) {
+    for (int p = 0; p < PER; p++) {
+      const int blk = tid + p * NTHREADS;
+      if (blk >= BLOCKS) break;
+      const int rb = blk % (ROWS / RB), kb = blk / (ROWS / RB);
+      int64_t col = row0 + rb * RB;
+      col = col + RB <= rows_valid ? col : rows_valid - RB;  // tile rows past the edge: any valid run
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-      // out[i] dword j = { in[2j] half i , in[2j+1] half i }
-      const unsigned lo = (unsigned)in[2 * j][i >> 1], hi = (unsigned)in[2 * j + 1][i >> 1];
-      out[i][j] = (int)__builtin_amdgcn_perm(hi, lo, (i & 1) ? 0x07060302u : 0x05040100u);
+      for (int j = 0; j < KB; j++)
+        v[p][j] = *reinterpret_cast<const v4i *>(g + (k0 + kb * KB + j) * ld + col * ES);
     }
   }
-}
 
-// K-outer slab of a 2-byte type: g is [K, rows] (row stride ld bytes per k); the slab covers
-// 64 k x ROWS rows.  ROWS*8/8 = ROWS blocks of 8 x 8, one or more per lane.
-template <int ROWS, int NTHREADS>
-struct KOuterRegs {
-  static constexpr int BLOCKS = (ROWS / 8) * 8;  // (ROWS/8 row-blocks) x (8 k-blocks)
-  static constexpr int PER = (BLOCKS + NTHREADS - 1) / NTHREADS;
-  v4i v[PER][8];
+  __device__ __forceinline__ void store(unsigned char *lds, int tid) const {
+#pragma unroll
+    for (int p = 0; p < PER; p++) {
+      const int blk = tid + p * NTHREADS;
+      if (blk >= BLOCKS) break;
+      const int rb = blk % (ROWS / RB), kb = blk / (ROWS / RB);
+      if constexpr (ES == 2) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {  // row i: dword j = { k = 2j , k = 2j+1 }
+          v4i t;
+#pragma unroll
+          for (int j = 0; j < 4; j++) {
+            const unsigned lo = (unsigned)v[p][2 * j][i >> 1], hi = (unsigned)v[p][2 * j + 1][i >> 1];
+            t[j] = (int)__builtin_amdgcn_perm(hi, lo, (i & 1) ? 0x07060302u : 0x05040100u);
+          }
+          const int r = rb * 8 + i;
+          *reinterpret_cast<v4i *>(lds + r * SLAB + lds_slot(r, kb) * 16) = t;
+        }
+      } else if constexpr (ES == 4) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const v4i t = {v[p][0][i], v[p][1][i], v[p][2][i], v[p][3][i]};
+          const int r = rb * 4 + i;
+          *reinterpret_cast<v4i *>(lds + r * SLAB + lds_slot(r, kb) * 16) = t;
+        }
+      } else {
+#pragma unroll
+        for (int c = 0; c < 4; c++) {  // dword column c holds rows 4c .. 4c+3 of the four k
+          const unsigned w0 = (unsigned)v[p][0][c], w1 = (unsigned)v[p][1][c], w2 = (unsigned)v[p][2][c], w3 = (unsigned)v[p][3][c];
+          const unsigned a01 = __builtin_amdgcn_perm(w1, w0, 0x05010400u), b01 = __builtin_amdgcn_perm(w1, w0, 0x07030602u);
+          const unsigned a23 = __builtin_amdgcn_perm(w3, w2, 0x05010400u), b23 = __builtin_amdgcn_perm(w3, w2, 0x07030602u);
+          const unsigned o[4] = {__builtin_amdgcn_perm(a23, a01, 0x05040100u), __builtin_amdgcn_perm(a23, a01, 0x07060302u),
+                                 __builtin_amdgcn_perm(b23, b01, 0x05040100u), __builtin_amdgcn_perm(b23, b01, 0x07060302u)};
+#pragma unroll
+          for (int i = 0; i < 4; i++) {  // row 4c+i: its four k bytes are dword (kb % 4) of chunk (kb / 4)
+            const int r = rb * 16 + 4 * c + i;
+            *reinterpret_cast<unsigned *>(lds + r * SLAB + lds_slot(r, kb >> 2) * 16 + (kb & 3) * 4) = o[i];
+          }
+        }
+      }
+    }
+  }
 };
 
-template <int ROWS, int NTHREADS>
-__device__ __forceinline__ void fetch_slab_kouter16(KOuterRegs<ROWS, NTHREADS> &regs, const unsigned char *__restrict__ g,
-                                                    int64_t ld, int64_t row0, int64_t rows_valid, int64_t k0,
-                                                    int64_t k_valid, int tid) {
-  constexpr int RB = ROWS / 8;
-#pragma unroll
-  for (int p = 0; p < KOuterRegs<ROWS, NTHREADS>::PER; p++) {
-    const int blk = tid + p * NTHREADS;
-    if (blk >= KOuterRegs<ROWS, NTHREADS>::BLOCKS) break;
-    const int rb = blk % RB, kb = blk / RB;
-    int64_t col = row0 + rb * 8;
-    // whole 16-byte run must be inside the row; a ragged edge re-reads the last full run
-    col = col + 8 <= rows_valid ? col : (rows_valid >= 8 ? rows_valid - 8 : 0);
-#pragma unroll
-    for (int j = 0; j < 8; j++) {
-      int64_t k = k0 + kb * 8 + j;
-      k = k < k_valid ? k : k_valid - 1;
-      regs.v[p][j] = *reinterpret_cast<const v4i *>(g + k * ld + col * 2);
-    }
-  }
-}
+// ---- K-outer 2-byte operands of the big tiles: no register staging at all.  The slab is copied
+// as it lies in memory -- [64 k][ROWS] , ROWS*2 bytes per k -- straight into LDS, and the MFMA
+// fragments are fetched with the transposing LDS read of gfx950, `ds_read_b64_tr_b16`: within
+// each group of 16 lanes, lane i supplies the address of a run of four 16-bit elements and lane j
+// receives element j%4 of the runs of lanes j/4, j/4+4, j/4+8, j/4+12 (measured on the part).
+// With lane i pointing at (k0 + i/4, n0 + 4*(i%4)) lane j therefore receives
+// [k0 .. k0+3][n0 + j]: four consecutive k of one row -- half an MFMA operand.
+// LDS layout: k-major, the 16-byte chunk index of a k-row XOR-ed with 4*(k&3): the 32 lanes served
+// per clock touch four k-rows x 64 contiguous bytes, which this spreads over all 64 banks
+// (SQ_LDS_BANK_CONFLICT = 0; with 2*(k&3) every such read took a second pass).
+typedef short v4s __attribute__((ext_vector_type(4)));
 
-template <int ROWS, int NTHREADS>
-__device__ __forceinline__ void store_slab_kouter16(const KOuterRegs<ROWS, NTHREADS> &regs, unsigned char *lds, int tid) {
-  constexpr int RB = ROWS / 8;
+__device__ __forceinline__ int tr_slot(int k, int chunk) { return chunk ^ ((k & 3) << 2); }
+
+template <int ROWS, int NWAVES>
+struct KOuterDmaLoader {
+  static constexpr int RBYTES = ROWS * 2;      // bytes per k-row of the slab
+  static constexpr int INSTR = ROWS / 8;       // 64 k-rows * RBYTES / 1 KiB
+  static constexpr int PER = INSTR / NWAVES;
+  static_assert(RBYTES >= 256 && INSTR % NWAVES == 0, "needs at least 16 chunks per k-row");
+  const unsigned char *src[PER];
+  int lds_off[PER];
+
+  // g: [K, cols] with `ld` bytes per k; the tile covers columns col0 .. col0+ROWS-1, of which
+  // cols_valid (a multiple of 8) exist: chunks past the edge re-read the last valid chunk
+  __device__ __forceinline__ void init(const unsigned char *__restrict__ g, int64_t ld, int64_t col0, int64_t cols_valid,
+                                       int wave, int lane) {
 #pragma unroll
-  for (int p = 0; p < KOuterRegs<ROWS, NTHREADS>::PER; p++) {
-    const int blk = tid + p * NTHREADS;
-    if (blk >= KOuterRegs<ROWS, NTHREADS>::BLOCKS) break;
-    const int rb = blk % RB, kb = blk / RB;
-    v4i t[8];
-    transpose8x8_b16(regs.v[p], t);
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-      const int r = rb * 8 + i;
-      *reinterpret_cast<v4i *>(lds + r * SLAB + lds_slot(r, kb) * 16) = t[i];
+    for (int i = 0; i < PER; i++) {
+      const int t = wave + NWAVES * i;
+      const int o = t * 1024 + lane * 16;
+      const int k = o / RBYTES, slot = (o % RBYTES) / 16;
+      int64_t byte = col0 * 2 + tr_slot(k, slot) * 16;
+      const int64_t last = cols_valid * 2 - 16;
+      byte = byte <= last ? byte : last;
+      src[i] = g + (int64_t)k * ld + byte;
+      lds_off[i] = t * 1024;
     }
   }
+  __device__ __forceinline__ void issue(int64_t k0, int64_t ld, unsigned char *lds) const {
+#pragma unroll
+    for (int i = 0; i < PER; i++)
+      __builtin_amdgcn_global_load_lds((gptr_t)(src[i] + k0 * ld), (lptr_t)(lds + lds_off[i]), 16, 0, 0);
+  }
+};
+
+// MFMA operand fragment of rows row0 .. row0+31 for K step `ks` out of a k-major slab
+template <int ROWS>
+__device__ __forceinline__ v4i read_fragment_tr(const unsigned char *slab, int row0, int ks, int lane) {
+  const int i16 = lane & 15;
+  const int n = row0 + ((lane >> 4) & 1) * 16 + 4 * (i16 & 3);  // first of the 4 elements this lane points at
+  const int kbase = 16 * ks + 8 * (lane >> 5) + (i16 >> 2);
+  v4i out;
+#pragma unroll
+  for (int h = 0; h < 2; h++) {
+    const int k = kbase + 4 * h;
+    const unsigned char *p = slab + k * (ROWS * 2) + tr_slot(k, n >> 3) * 16 + (n & 7) * 2;
+    const v4s r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s *)p);
+    const int2 w = __builtin_bit_cast(int2, r);
+    out[2 * h] = w.x;
+    out[2 * h + 1] = w.y;
+  }
+  return out;
 }
 
 struct GemmArgs {
@@ -259,21 +343,30 @@ gemm_pipelined_kernel(GemmArgs a) {
   KInnerLoader<BN, NW> rload;
   if constexpr (L_KIN) lload.init(lb, a.ld_l, m0, a.M, wave, lane);
   if constexpr (R_KIN) rload.init(rb, a.ld_r, n0, a.N, wave, lane);
-  KOuterRegs<BM, NT> lregs;
-  KOuterRegs<BN, NT> rregs;
-  const int64_t K_elems = a.Kb / 2;  // only used by the 2-byte K-outer path
+  constexpr int ES = (DT == HIPNX_S8) ? 1 : (DT == HIPNX_F32 ? 4 : 2);
+  // K-outer 2-byte operands of tiles with at least a cache line per k-row: DMA + transposing reads
+  constexpr bool L_TR = !L_KIN && ES == 2 && BM >= 128 && (BM / 8) % NW == 0;
+  constexpr bool R_TR = !R_KIN && ES == 2 && BN >= 128 && (BN / 8) % NW == 0;
+  KOuterDmaLoader<L_TR ? BM : 128 * NW, NW> ltr;
+  KOuterDmaLoader<R_TR ? BN : 128 * NW, NW> rtr;
+  if constexpr (L_TR) ltr.init(lb, a.ld_l, m0, a.M, wave, lane);
+  if constexpr (R_TR) rtr.init(rb, a.ld_r, n0, a.N, wave, lane);
+  KOuterStage<ES, BM, NT> lregs;
+  KOuterStage<ES, BN, NT> rregs;
 
   auto issue = [&](int stage, int64_t kbyte0) {
     unsigned char *sA = smem + stage * STAGE, *sB = sA + BM * SLAB;
     if constexpr (L_KIN) lload.issue(kbyte0, sA);
-    else fetch_slab_kouter16<BM, NT>(lregs, lb, a.ld_l, m0, a.M, kbyte0 / 2, K_elems, tid);
+    else if constexpr (L_TR) ltr.issue(kbyte0 / ES, a.ld_l, sA);
+    else lregs.fetch(lb, a.ld_l, m0, a.M, kbyte0 / ES, tid);
     if constexpr (R_KIN) rload.issue(kbyte0, sB);
-    else fetch_slab_kouter16<BN, NT>(rregs, rb, a.ld_r, n0, a.N, kbyte0 / 2, K_elems, tid);
+    else if constexpr (R_TR) rtr.issue(kbyte0 / ES, a.ld_r, sB);
+    else rregs.fetch(rb, a.ld_r, n0, a.N, kbyte0 / ES, tid);
   };
-  auto commit = [&](int stage) {  // K-outer operands: registers -> transposed LDS writes
+  auto commit = [&](int stage) {  // register-staged K-outer operands: transposed LDS writes
     unsigned char *sA = smem + stage * STAGE, *sB = sA + BM * SLAB;
-    if constexpr (!L_KIN) store_slab_kouter16<BM, NT>(lregs, sA, tid);
-    if constexpr (!R_KIN) store_slab_kouter16<BN, NT>(rregs, sB, tid);
+    if constexpr (!L_KIN && !L_TR) lregs.store(sA, tid);
+    if constexpr (!R_KIN && !R_TR) rregs.store(sB, tid);
   };
 
   // NSTAGE LDS stages, slab s lives in stage s % NSTAGE, NSTAGE-1 slabs are requested ahead.
@@ -304,12 +397,14 @@ gemm_pipelined_kernel(GemmArgs a) {
 #pragma unroll
       for (int i = 0; i < TM; i++) {
         const int row = wm + 32 * i + (lane & 31);
-        fa[i] = *reinterpret_cast<const v4i *>(sA + row * SLAB + lds_slot(row, chunk) * 16);
+        if constexpr (L_TR) fa[i] = read_fragment_tr<BM>(sA, wm + 32 * i, ks, lane);
+        else fa[i] = *reinterpret_cast<const v4i *>(sA + row * SLAB + lds_slot(row, chunk) * 16);
       }
 #pragma unroll
       for (int j = 0; j < TN; j++) {
         const int row = wn + 32 * j + (lane & 31);
-        fb[j] = *reinterpret_cast<const v4i *>(sB + row * SLAB + lds_slot(row, chunk) * 16);
+        if constexpr (R_TR) fb[j] = read_fragment_tr<BN>(sB, wn + 32 * j, ks, lane);
+        else fb[j] = *reinterpret_cast<const v4i *>(sB + row * SLAB + lds_slot(row, chunk) * 16);
       }
 #pragma unroll
       for (int i = 0; i < TM; i++)

@@ -123,3 +123,37 @@ def test_dot_matches_closed_form_on_small_integers_in_bf16(hip):
     assert np.array_equal(got, (a @ b).astype(np.float64))
     got_bf = values(Nx.dot(ha, hb, out_type="f32"))
     assert np.array_equal(got_bf, (a @ b).astype(np.float64))
+
+
+@pytest.mark.parametrize("M,N,K", [(256, 256, 256), (64, 48, 128), (130, 72, 256), (512, 528, 384), (16, 4096, 128)])
+@pytest.mark.parametrize("layout", ["nn", "nt", "tn", "tt"])
+def test_int8_dot_every_operand_layout_is_bit_exact(M, N, K, layout, hip, oracle):
+    """K-outer s8 operands are transposed inside the MFMA kernel (or by a pass when the row count
+    is ragged): all four layouts must give the exact integer product."""
+    rng = np.random.default_rng(seed_of(M, N, K, layout))
+    a = rng.integers(-128, 128, size=(M, K) if layout[0] == "n" else (K, M)).astype(np.int8)
+    b = rng.integers(-128, 128, size=(K, N) if layout[1] == "n" else (N, K)).astype(np.int8)
+    c1 = [1] if layout[0] == "n" else [0]
+    c2 = [0] if layout[1] == "n" else [1]
+    got = hip.to_numpy(Nx.dot(from_numpy(a, "s8", hip), c1, from_numpy(b, "s8", hip), c2, out_type="s32"))
+    am = a if layout[0] == "n" else a.T
+    bm = b if layout[1] == "n" else b.T
+    exact = (am.astype(np.float64) @ bm.astype(np.float64)).astype(np.int64)  # exact: |sum| < 2^53
+    assert np.array_equal(got, exact.astype(np.int32))
+    want = Nx.dot(from_numpy(a, "s8", oracle), c1, from_numpy(b, "s8", oracle), c2, out_type="s32")
+    assert np.array_equal(got, np.frombuffer(Nx.to_binary(want), dtype=np.int32).reshape(M, N))
+
+
+@pytest.mark.parametrize("ty,M,N,K", [("f32", 128, 128, 64), ("f32", 100, 36, 96), ("f32", 102, 38, 96), ("bf16", 136, 72, 128),
+                                      ("f16", 264, 200, 192), ("bf16", 132, 76, 64), ("f32", 300, 260, 2048)])
+@pytest.mark.parametrize("layout", ["nn", "nt", "tn", "tt"])
+def test_float_dot_pipelined_kernel_layouts(ty, M, N, K, layout, hip, oracle):
+    rng = np.random.default_rng(seed_of(ty, M, N, K, layout))
+    a = rand_raw(rng, ty, (M, K) if layout[0] == "n" else (K, M), lo=-1, hi=1)
+    b = rand_raw(rng, ty, (K, N) if layout[1] == "n" else (N, K), lo=-1, hi=1)
+    ha, oa = both(a, ty, hip, oracle)
+    hb, ob = both(b, ty, hip, oracle)
+    c1 = [1] if layout[0] == "n" else [0]
+    c2 = [0] if layout[1] == "n" else [1]
+    eq = ("mk" if layout[0] == "n" else "km") + "," + ("kn" if layout[1] == "n" else "nk") + "->mn"
+    check_float_dot(Nx.dot(ha, c1, hb, c2), Nx.dot(oa, c1, ob, c2), values(oa), values(ob), eq, K, f"{ty} {layout} {M}x{N}x{K}")
