@@ -30,6 +30,7 @@ static int launch_one(const hipnx_ctx *ctx, GemmArgs a, int64_t batch) {
   }
   a.tiles_m = (int)((a.M + BM - 1) / BM);
   a.tiles_n = (int)((a.N + BN - 1) / BN);
+  a.group_m = gemm_group_m(a.tiles_m, a.tiles_n);
   dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)batch), block(WM * WN * 64);
   hipLaunchKernelGGL(kern, grid, block, smem, ctx->stream, a);
   HIPNX_HIP(hipGetLastError());

@@ -259,6 +259,7 @@ struct GemmArgs {
   int64_t ld_l, ld_r;    // bytes between consecutive rows (K-inner) or consecutive k (K-outer)
   int64_t bs_l, bs_r;    // bytes between batch items
   int tiles_m, tiles_n;
+  int group_m;  // tile rows per group of the tile order (see gemm_group_m)
 };
 
 // Epilogue of one wave: lane holds m = lane%32 and, per accumulator quad qq of tile (i, j),
@@ -299,6 +300,16 @@ __device__ __forceinline__ void gemm_epilogue(typename Mma<DT>::acc_t (&acc)[TM]
   }
 }
 
+// Rows per group of the tile order: the largest power of two not above the square root of the
+// number of tiles one XCD works on at a time.
+inline int gemm_group_m(int tiles_m, int tiles_n) {
+  int per_xcd = (tiles_m * tiles_n + 7) / 8;
+  if (per_xcd > 64) per_xcd = 64;
+  int g = 1;
+  while ((2 * g) * (2 * g) <= per_xcd && 2 * g <= tiles_m) g *= 2;
+  return g;
+}
+
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {  // s_waitcnt vmcnt(N), other counters untouched
   static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
@@ -315,14 +326,24 @@ gemm_pipelined_kernel(GemmArgs a) {
   constexpr int KSTEPS = SLAB / 32;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
-  // tile order: consecutive block ids go to different XCDs (id % 8); give each XCD a compact
-  // band of tiles so that the operand panels it streams are shared through its own L2
+  // tile order: consecutive block ids go to different XCDs (id % 8), so each XCD takes a run of
+  // total/8 consecutive positions of the order below; the order walks groups of `group_m` tile
+  // rows column by column, which makes such a run a compact rectangle of tiles whose operand
+  // panels are shared through the XCD's own L2
   int tile = blockIdx.x;
   {
     const int total = a.tiles_m * a.tiles_n;
     if (total % 8 == 0) tile = (blockIdx.x % 8) * (total / 8) + blockIdx.x / 8;
   }
-  const int tm = tile / a.tiles_n, tn = tile % a.tiles_n;
+  int tm, tn;
+  {
+    const int per_group = a.group_m * a.tiles_n;
+    const int first = (tile / per_group) * a.group_m;
+    const int rows = min(a.group_m, a.tiles_m - first);
+    const int in = tile % per_group;
+    tm = first + in % rows;
+    tn = in / rows;
+  }
   const int64_t b = blockIdx.y;
   const unsigned char *lb = a.l + b * a.bs_l;
   const unsigned char *rb = a.r + b * a.bs_r;
