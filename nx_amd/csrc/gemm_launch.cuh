@@ -18,11 +18,11 @@ int launch_gemm_f16(const hipnx_ctx *ctx, int cfg, bool l_kin, bool r_kin, GemmA
 int launch_gemm_f32(const hipnx_ctx *ctx, int cfg, bool l_kin, bool r_kin, GemmArgs a, int64_t batch);
 int launch_gemm_s8(const hipnx_ctx *ctx, int cfg, bool l_kin, bool r_kin, GemmArgs a, int64_t batch);
 
-template <int DT, int WM, int WN, int TM, int TN, bool LK, bool RK, int NSTAGE = 2>
+template <int DT, int WM, int WN, int TM, int TN, bool LK, bool RK>
 static int launch_one(const hipnx_ctx *ctx, GemmArgs a, int64_t batch) {
   constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
-  constexpr int smem = NSTAGE * (BM + BN) * SLAB;
-  auto kern = gemm_pipelined_kernel<DT, WM, WN, TM, TN, LK, RK, NSTAGE>;
+  constexpr int smem = 2 * (BM + BN) * SLAB;
+  auto kern = gemm_pipelined_kernel<DT, WM, WN, TM, TN, LK, RK>;
   static bool configured = false;  // per instantiation; racing writers store the same value
   if (!configured) {
     HIPNX_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem));

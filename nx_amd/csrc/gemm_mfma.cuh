@@ -1,29 +1,29 @@
 // Pipelined MFMA contraction kernel  out[b, m, n] = sum_k l[b, m, k] * r[b, n, k]  for gfx950.
 //
-// Work-group tile BM x BN = (WM*TM*32) x (WN*TN*32): WM x WN wavefronts, each owning TM x TN MFMA
-// tiles of 32 x 32 whose accumulators stay in registers for the whole K walk.
+// Work-group tile BM x BN = (WM*TM*32) x (WN*TN*32): WM x WN wavefronts, each owning
+// 2TM x 2TN MFMA tiles of 16 x 16 whose accumulators stay in registers for the whole K walk.
+// (Under the power cap the 16x16 MFMA shapes sustain 10-20 % more than the 32x32 ones with the
+// same operands, and the f32 16x16x4 form almost 1.5x the 32x32x2 form.)
 //
 // K is walked in slabs of 128 bytes per row (64 bf16/f16, 128 s8, 32 f32): one full cache line
 // per row, the granularity at which a CU ingests L2-resident data fastest (half lines halve it).
-// LDS holds a ring of NUNIT "units"; a unit is one operand's share of one slab (BM or BN rows x
-// 128 B).  Slab s is units 2s (l rows) and 2s+1 (r rows).  While the MFMAs consume slab s, the
-// r unit of slab s+1 and the l unit of slab s+2 are in flight (the l unit of slab s+1 was issued a
-// slab earlier), so the data needed next has had between one and two slab times to arrive; the
-// wait before the per-slab barrier uses vmcnt(n) and leaves the youngest unit outstanding.
+// LDS holds NSTAGE stages of one slab each (BM + BN rows x 128 B).
 //   K-inner operand ([rows, K], K contiguous): `global_load_lds_dwordx4` -- each lane moves 16 B
 //     straight from global memory into LDS, no VGPR round trip.  A wave instruction fills 1 KiB of
 //     LDS (8 rows x 8 chunks); the lane picks the *global* chunk that belongs at its LDS slot.
-//   K-outer operand ([K, rows], rows contiguous): each lane loads a small k x rows block with
-//     16-byte row loads, transposes it in registers (byte permutes) and writes K-runs to LDS --
-//     the slab arrives in the same [row][k] LDS layout, so a plain `Nx.dot(a, b)` needs no
-//     re-layout pass.
-// LDS layout of a unit: row-major, 128 B per row, the 16-byte chunk index XOR-ed with
-// ((row ^ row>>3) & 7): conflict-free for the fragment reads (32 consecutive rows, one chunk) and
-// for the transposed writes (rows 8 apart, one chunk).
-// Fragments: for one 32-byte K-step a lane's MFMA operand is chunk (2*step + lane/32) of row
-// (lane%32) -- 8 bf16/f16, 16 s8 or 4 f32 (fed to four 32x32x2 MFMAs; both operands use the same
-// k <-> slot map).  The MFMA is issued with the r-fragment as its first operand so that a lane ends
-// up with 4 consecutive n per accumulator quad: the epilogue stores 4 outputs at a time.
+//     LDS layout: row-major, 128 B per row, the 16-byte chunk index XOR-ed with
+//     ((row ^ row>>3) & 7): conflict-free for the fragment reads (16 consecutive rows, one chunk)
+//     and for the transposed writes below (rows 8 apart, one chunk).
+//   K-outer operand ([K, rows], rows contiguous), 2-byte elements, tiles of 128 rows or more: the
+//     slab is copied k-major with the same direct-to-LDS loads and the fragment is built by the
+//     transposing LDS read `ds_read_b64_tr_b16`.
+//   K-outer operand otherwise: each lane loads a small k x rows block with 16-byte row loads,
+//     transposes it in registers (byte permutes) and writes K-runs into the K-inner LDS layout.
+//   Either way a plain `Nx.dot(a, b)` needs no re-layout pass.
+// Fragments: for one 64-byte K-step a lane's MFMA operand is chunk (4*step + lane/16) of row
+// (lane%16) -- 8 bf16/f16, 16 s8 or 4 f32 (fed to four 16x16x4 MFMAs; both operands use the same
+// k <-> slot map).  The MFMA is issued with the r-fragment as its first operand so that a lane
+// ends up with 4 consecutive n per accumulator: the epilogue stores 4 outputs at a time.
 #pragma once
 #include <type_traits>
 
@@ -68,10 +68,58 @@ template <> struct Mma<HIPNX_F32> {
   }
 };
 
-__device__ __forceinline__ int lds_slot(int row, int chunk) { return chunk ^ ((row ^ (row >> 3)) & 7); }
+typedef float v4f __attribute__((ext_vector_type(4)));
 
-typedef const __attribute__((address_space(1))) void *gptr_t;
+// 16x16 MFMA forms used by the pipelined kernel (one 16-byte operand chunk per lane and step)
+template <int DT> struct Mma16;
+template <> struct Mma16<HIPNX_BF16> {
+  typedef v4f acc_t;
+  static __device__ __forceinline__ void step(acc_t &c, const v4i &a, const v4i &b) {
+    c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
+  }
+};
+template <> struct Mma16<HIPNX_F16> {
+  typedef v4f acc_t;
+  static __device__ __forceinline__ void step(acc_t &c, const v4i &a, const v4i &b) {
+    c = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0, 0, 0);
+  }
+};
+template <> struct Mma16<HIPNX_S8> {
+  typedef v4i acc_t;
+  static __device__ __forceinline__ void step(acc_t &c, const v4i &a, const v4i &b) {
+    c = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct Mma16<HIPNX_F32> {
+  typedef v4f acc_t;
+  static __device__ __forceinline__ void step(acc_t &c, const v4i &a, const v4i &b) {
+#pragma unroll
+    for (int s = 0; s < 4; s++)
+      c = __builtin_amdgcn_mfma_f32_16x16x4f32(__int_as_float(a[s]), __int_as_float(b[s]), c, 0, 0, 0);
+  }
+};
+
+// Swizzle of the [row][k] LDS layout: 16-byte chunk index XOR a 3-bit function of the row.  The
+// function (bit0 = r0^r2, bit1 = r1^r2, bit2 = r2^r3 of the row index) is one of the maps a sweep
+// over all linear maps of the low four row bits measured as conflict-free for the fragment read
+// (16 consecutive rows x 4 chunks per ds_read_b128: 4 clocks per instruction instead of 8).
+__device__ __forceinline__ int lds_slot(int row, int chunk) {
+  return chunk ^ (((row ^ (row >> 2)) & 1) | ((((row >> 1) ^ (row >> 2)) & 1) << 1) | ((((row >> 2) ^ (row >> 3)) & 1) << 2));
+}
+
 typedef __attribute__((address_space(3))) void *lptr_t;
+
+// One direct-to-LDS load: every lane moves 16 bytes from its global address to
+// LDS[lds_base + 16 * lane] (lds_base wave-uniform, carried in M0).  Written as inline assembly
+// rather than through the compiler's builtin on purpose: after the builtin the compiler no
+// longer trusts the in-order return of LDS reads and turns every partial lgkmcnt(n) wait of the
+// fragment pipeline into lgkmcnt(0).  The compiler therefore does not count these loads: the
+// kernel waits for them itself (wait_vmcnt) before the barrier that publishes a slab; the
+// compiler's own vmcnt waits only become stricter by loads it does not know of.
+__device__ __forceinline__ void lds_dma16(const unsigned char *g, unsigned char *lds) {
+  const unsigned base = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(lptr_t)lds);
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(base) : "memory", "m0");
+}
 
 // K-inner slab loader: ROWS x 128 B, direct to LDS.  The per-lane source pointers (row clamp,
 // row * stride, swizzled chunk) are computed once; per slab only the K offset moves.
@@ -101,7 +149,14 @@ struct KInnerLoader {
   __device__ __forceinline__ void issue(int64_t kbyte0, unsigned char *lds) const {
 #pragma unroll
     for (int i = 0; i < PER; i++)
-      __builtin_amdgcn_global_load_lds((gptr_t)(src[i] + kbyte0), (lptr_t)(lds + lds_off[i]), 16, 0, 0);
+      lds_dma16(src[i] + kbyte0, lds + lds_off[i]);
+  }
+  // instruction i of the slab goes out at step i * spread / PER + phase (+ skew, which may be a
+  // run-time value); with t, spread and phase known after unrolling the tests fold away
+  __device__ __forceinline__ void issue_at(int t, int spread, int phase, int skew, int64_t kbyte0, unsigned char *lds) const {
+#pragma unroll
+    for (int i = 0; i < PER; i++)
+      if (t == i * spread / PER + phase + skew) lds_dma16(src[i] + kbyte0, lds + lds_off[i]);
   }
 };
 
@@ -198,7 +253,7 @@ struct KOuterStage {
 // (SQ_LDS_BANK_CONFLICT = 0; with 2*(k&3) every such read took a second pass).
 typedef short v4s __attribute__((ext_vector_type(4)));
 
-__device__ __forceinline__ int tr_slot(int k, int chunk) { return chunk ^ ((k & 3) << 2); }
+__device__ __forceinline__ int tr_slot(int k, int chunk) { return chunk ^ ((k & 3) << 2) ^ (((k >> 3) & 1) << 1); }
 
 template <int ROWS, int NWAVES>
 struct KOuterDmaLoader {
@@ -228,16 +283,24 @@ struct KOuterDmaLoader {
   __device__ __forceinline__ void issue(int64_t k0, int64_t ld, unsigned char *lds) const {
 #pragma unroll
     for (int i = 0; i < PER; i++)
-      __builtin_amdgcn_global_load_lds((gptr_t)(src[i] + k0 * ld), (lptr_t)(lds + lds_off[i]), 16, 0, 0);
+      lds_dma16(src[i] + k0 * ld, lds + lds_off[i]);
+  }
+  __device__ __forceinline__ void issue_at(int t, int spread, int phase, int skew, int64_t k0, int64_t ld, unsigned char *lds) const {
+#pragma unroll
+    for (int i = 0; i < PER; i++)
+      if (t == i * spread / PER + phase + skew) lds_dma16(src[i] + k0 * ld, lds + lds_off[i]);
   }
 };
 
-// MFMA operand fragment of rows row0 .. row0+31 for K step `ks` out of a k-major slab
+// MFMA operand fragment of rows row0 .. row0+15 for K step `ks` (32 elements) out of a k-major
+// slab.  `ds_read_b64_tr_b16`: within a group of 16 lanes, lane j receives element j%4 of the
+// 8-byte runs addressed by lanes j/4, j/4+4, j/4+8 and j/4+12 -- so lane i points at row block
+// i%4 of k-row i/4, and lane j ends up with row j at four consecutive k.
 template <int ROWS>
 __device__ __forceinline__ v4i read_fragment_tr(const unsigned char *slab, int row0, int ks, int lane) {
   const int i16 = lane & 15;
-  const int n = row0 + ((lane >> 4) & 1) * 16 + 4 * (i16 & 3);  // first of the 4 elements this lane points at
-  const int kbase = 16 * ks + 8 * (lane >> 5) + (i16 >> 2);
+  const int n = row0 + 4 * (i16 & 3);
+  const int kbase = 32 * ks + 8 * (lane >> 4) + (i16 >> 2);
   v4i out;
 #pragma unroll
   for (int h = 0; h < 2; h++) {
@@ -262,12 +325,12 @@ struct GemmArgs {
   int group_m;  // tile rows per group of the tile order (see gemm_group_m)
 };
 
-// Epilogue of one wave: lane holds m = lane%32 and, per accumulator quad qq of tile (i, j),
-// n = 32*j + 8*qq + 4*(lane/32) + 0..3.  ODT is a compile-time constant here, so the typed
-// stores fold to plain vector stores; every accumulator index is a constant (the accumulators
-// must never be addressed dynamically, or they leave the register file).
+// Epilogue of one wave: for 16x16 tile (i, j) a lane holds m = 16*i + lane%16 and
+// n = 16*j + 4*(lane/16) + 0..3.  ODT is a compile-time constant here, so the typed stores fold
+// to plain vector stores; every accumulator index is a constant (the accumulators must never be
+// addressed dynamically, or they leave the register file).
 template <int DT, int ODT, int TM, int TN>
-__device__ __forceinline__ void gemm_epilogue(typename Mma<DT>::acc_t (&acc)[TM][TN], void *out, int64_t obase,
+__device__ __forceinline__ void gemm_epilogue(typename Mma16<DT>::acc_t (&acc)[TM][TN], void *out, int64_t obase,
                                               int64_t M, int64_t N, int64_t row0, int64_t col0, int lane) {
   constexpr bool int_acc = DT == HIPNX_S8;
   constexpr bool int_out = ODT < HIPNX_F16;
@@ -277,25 +340,23 @@ __device__ __forceinline__ void gemm_epilogue(typename Mma<DT>::acc_t (&acc)[TM]
     const bool vec_ok = (N % 4) == 0;
 #pragma unroll
     for (int i = 0; i < TM; i++) {
-      const int64_t gm = row0 + 32 * i + (lane & 31);
+      const int64_t gm = row0 + 16 * i + (lane & 15);
 #pragma unroll
-      for (int j = 0; j < TN; j++)
+      for (int j = 0; j < TN; j++) {
+        const int64_t gn = col0 + 16 * j + 4 * (lane >> 4);
+        S v[4];
 #pragma unroll
-        for (int qq = 0; qq < 4; qq++) {
-          const int64_t gn = col0 + 32 * j + 8 * qq + 4 * (lane >> 5);
-          S v[4];
+        for (int e = 0; e < 4; e++) v[e] = (S)acc[i][j][e];
+        const int64_t idx = obase + gm * N + gn;
+        if (gm < M) {
+          if (vec_ok && gn + 4 <= N) store_vec<S, 4>(out, ODT, idx, v);
+          else {
 #pragma unroll
-          for (int e = 0; e < 4; e++) v[e] = (S)acc[i][j][4 * qq + e];
-          const int64_t idx = obase + gm * N + gn;
-          if (gm < M) {
-            if (vec_ok && gn + 4 <= N) store_vec<S, 4>(out, ODT, idx, v);
-            else {
-#pragma unroll
-              for (int e = 0; e < 4; e++)
-                if (gn + e < N) store_one<S>(out, ODT, idx + e, v[e]);
-            }
+            for (int e = 0; e < 4; e++)
+              if (gn + e < N) store_one<S>(out, ODT, idx + e, v[e]);
           }
         }
+      }
     }
   }
 }
@@ -316,14 +377,15 @@ __device__ __forceinline__ void wait_vmcnt() {  // s_waitcnt vmcnt(N), other cou
   __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
 }
 
-template <int DT, int WM, int WN, int TM, int TN, bool L_KIN, bool R_KIN, int NSTAGE = 2>
+template <int DT, int WM, int WN, int TM, int TN, bool L_KIN, bool R_KIN>
 __global__ void __launch_bounds__(WM *WN * 64)
 gemm_pipelined_kernel(GemmArgs a) {
-  typedef typename Mma<DT>::acc_t acc_t;
+  typedef typename Mma16<DT>::acc_t acc_t;
   constexpr int NW = WM * WN, NT = NW * 64;
+  constexpr int TM16 = 2 * TM, TN16 = 2 * TN;  // 16x16 MFMA tiles per wave
   constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
   constexpr int STAGE = (BM + BN) * SLAB;
-  constexpr int KSTEPS = SLAB / 32;
+  constexpr int KSTEPS = SLAB / 64;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
   // tile order: consecutive block ids go to different XCDs (id % 8), so each XCD takes a run of
@@ -352,13 +414,13 @@ gemm_pipelined_kernel(GemmArgs a) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = (wave / WN) * (TM * 32), wn = (wave % WN) * (TN * 32);
 
-  acc_t acc[TM][TN];
+  acc_t acc[TM16][TN16];
 #pragma unroll
-  for (int i = 0; i < TM; i++)
+  for (int i = 0; i < TM16; i++)
 #pragma unroll
-    for (int j = 0; j < TN; j++)
+    for (int j = 0; j < TN16; j++)
 #pragma unroll
-      for (int q = 0; q < 16; q++) acc[i][j][q] = 0;
+      for (int q = 0; q < 4; q++) acc[i][j][q] = 0;
 
   KInnerLoader<BM, NW> lload;
   KInnerLoader<BN, NW> rload;
@@ -390,56 +452,96 @@ gemm_pipelined_kernel(GemmArgs a) {
     if constexpr (!R_KIN && !R_TR) rregs.store(sB, tid);
   };
 
-  // NSTAGE LDS stages, slab s lives in stage s % NSTAGE, NSTAGE-1 slabs are requested ahead.
-  // Per slab: wait until my own loads of slab s have landed (younger ones may still fly: loads
-  // complete in issue order), barrier (everyone's loads of slab s are in, everyone is done
-  // reading slab s-1), refill the stage slab s-1 occupied with slab s+NSTAGE-1, then compute.
+  // ---- the K walk.  Two LDS stages; slab s lives in stage s % 2.
+  // One step = one column of 16x16 tiles (TM16 MFMAs) of one K step; a slab is STEPS steps.
+  // Fragment reads run DIST steps ahead of the MFMAs that use them (r fragments in a ring of
+  // four, l fragments of the next K step fetched during the last steps of the current one), and
+  // the waits in between are partial (lgkmcnt(n): LDS reads return in order).
+  // The one barrier per slab sits after step BAR = STEPS-DIST-1, by which a wave has issued every
+  // read of the slab.  Before it the wave drains its reads (so the stage may be overwritten) and
+  // its direct-to-LDS loads of the next slab (so that slab may be read); after it the remaining
+  // DIST steps of MFMAs run on fragments already in registers while the first fragments of the
+  // next slab are fetched -- no wave sits idle behind the barrier waiting for LDS.
+  // The next slab's global requests go out one instruction at a time during the steps before
+  // BAR (l and r in alternate steps): a wave that issues a slab's loads back to back sits in
+  // the issue stage until the address unit has taken them all and feeds no MFMA meanwhile.
+  constexpr int STEPS = KSTEPS * TN16;
+  constexpr int DIST = STEPS >= 8 ? 3 : 2;
+  constexpr int RING = 4;
+  constexpr int BAR = STEPS - DIST - 1;
+  constexpr int SPREAD = BAR * 3 / 4 > 0 ? BAR * 3 / 4 : 1;
+  static_assert(KSTEPS == 2 && TN16 >= TM16 && STEPS % RING == 0 && BAR >= 1 && BAR >= TN16 - 1 && SPREAD <= BAR,
+                "wave tile shape does not fit the fragment pipeline");
+  auto issue_step = [&](int t, int stage, int64_t kbyte0) {
+    unsigned char *sA = smem + stage * STAGE, *sB = sA + BM * SLAB;
+    if constexpr (L_KIN) lload.issue_at(t, SPREAD, 0, 0, kbyte0, sA);
+    else if constexpr (L_TR) ltr.issue_at(t, SPREAD, 0, 0, kbyte0 / ES, a.ld_l, sA);
+    else if (t == 0) lregs.fetch(lb, a.ld_l, m0, a.M, kbyte0 / ES, tid);
+    if constexpr (R_KIN) rload.issue_at(t, SPREAD, 1, 0, kbyte0, sB);
+    else if constexpr (R_TR) rtr.issue_at(t, SPREAD, 1, 0, kbyte0 / ES, a.ld_r, sB);
+    else if (t == 0) rregs.fetch(rb, a.ld_r, n0, a.N, kbyte0 / ES, tid);
+  };
+  auto read_l = [&](const unsigned char *st, int ks, int i) -> v4i {
+    const int row = wm + 16 * i + (lane & 15);
+    if constexpr (L_TR) return read_fragment_tr<BM>(st, wm + 16 * i, ks, lane);
+    else return *reinterpret_cast<const v4i *>(st + row * SLAB + lds_slot(row, 4 * ks + (lane >> 4)) * 16);
+  };
+  auto read_r = [&](const unsigned char *st, int t) -> v4i {  // step t = (K step, column tile)
+    const int ks = t / TN16, j = t % TN16;
+    const int row = wn + 16 * j + (lane & 15);
+    const unsigned char *sB = st + BM * SLAB;
+    if constexpr (R_TR) return read_fragment_tr<BN>(sB, wn + 16 * j, ks, lane);
+    else return *reinterpret_cast<const v4i *>(sB + row * SLAB + lds_slot(row, 4 * ks + (lane >> 4)) * 16);
+  };
+
   const int nslab = (int)(a.Kb / SLAB);
-  constexpr int AHEAD = NSTAGE - 1;
-  constexpr int OPS = (L_KIN ? KInnerLoader<BM, NW>::PER : 0) + (R_KIN ? KInnerLoader<BN, NW>::PER : 0);
-  static_assert(NSTAGE == 2 || (L_KIN && R_KIN), "deep pipelines are for K-inner operands");
-  static_assert(OPS * (AHEAD - 1) < 64, "vmcnt is a 6-bit counter");
-#pragma unroll
-  for (int p = 0; p < AHEAD; p++)
-    if (p < nslab) issue(p, (int64_t)p * SLAB);
+  issue(0, 0);
   commit(0);
+  wait_vmcnt<0>();
+  __syncthreads();
+  v4i fa[2][TM16], fb[RING];
+#pragma unroll
+  for (int i = 0; i < TM16; i++) fa[0][i] = read_l(smem, 0, i);
+#pragma unroll
+  for (int d = 0; d < DIST; d++) fb[d] = read_r(smem, d);
 
   for (int s = 0; s < nslab; s++) {
-    // slabs s+1 .. s+AHEAD-1 may stay in flight, unless the walk is about to end
-    if (s + AHEAD - 1 < nslab) wait_vmcnt<OPS *(AHEAD - 1)>();
-    else wait_vmcnt<0>();
-    __syncthreads();
-    if (s + AHEAD < nslab) issue((s + AHEAD) % NSTAGE, (int64_t)(s + AHEAD) * SLAB);
-    const unsigned char *sA = smem + (s % NSTAGE) * STAGE, *sB = sA + BM * SLAB;
+    const unsigned char *cur = smem + (s & 1) * STAGE, *nxt = smem + ((s + 1) & 1) * STAGE;
+    const bool more = s + 1 < nslab;
+    const int64_t next_kbyte = (int64_t)(s + 1) * SLAB;
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ks++) {
-      v4i fa[TM], fb[TN];
-      const int chunk = 2 * ks + (lane >> 5);
+    for (int t = 0; t < STEPS; t++) {
+      const int ks = t / TN16, j = t % TN16;
+      // r fragment of step t + DIST (of the next slab once past the end of this one)
+      if (t + DIST < STEPS) fb[(t + DIST) % RING] = read_r(cur, t + DIST);
+      else if (more) fb[(t + DIST) % RING] = read_r(nxt, t + DIST - STEPS);
+      // l fragments of the next K step: within the slab during the last TM16 steps of this K
+      // step, across the slab boundary spread over the DIST steps behind the barrier
+      if (ks + 1 < KSTEPS) {
+        if (j >= TN16 - TM16) fa[(ks + 1) & 1][j - (TN16 - TM16)] = read_l(cur, ks + 1, j - (TN16 - TM16));
+      } else if (more && t >= STEPS - DIST) {
+        const int d = t - (STEPS - DIST);
 #pragma unroll
-      for (int i = 0; i < TM; i++) {
-        const int row = wm + 32 * i + (lane & 31);
-        if constexpr (L_TR) fa[i] = read_fragment_tr<BM>(sA, wm + 32 * i, ks, lane);
-        else fa[i] = *reinterpret_cast<const v4i *>(sA + row * SLAB + lds_slot(row, chunk) * 16);
+        for (int i = 0; i < TM16; i++)
+          if (i >= d * TM16 / DIST && i < (d + 1) * TM16 / DIST) fa[0][i] = read_l(nxt, 0, i);
       }
+      if (more && t <= BAR) issue_step(t, (s + 1) & 1, next_kbyte);
 #pragma unroll
-      for (int j = 0; j < TN; j++) {
-        const int row = wn + 32 * j + (lane & 31);
-        if constexpr (R_TR) fb[j] = read_fragment_tr<BN>(sB, wn + 32 * j, ks, lane);
-        else fb[j] = *reinterpret_cast<const v4i *>(sB + row * SLAB + lds_slot(row, chunk) * 16);
+      for (int i = 0; i < TM16; i++) Mma16<DT>::step(acc[i][j], fb[t % RING], fa[ks & 1][i]);
+      if (t == BAR && more) {
+        commit((s + 1) & 1);
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): my reads of this slab have returned
+        wait_vmcnt<0>();                     // my loads of the next slab have landed
+        __syncthreads();
       }
-#pragma unroll
-      for (int i = 0; i < TM; i++)
-#pragma unroll
-        for (int j = 0; j < TN; j++) Mma<DT>::step(acc[i][j], fb[j], fa[i]);
+      __builtin_amdgcn_sched_barrier(0);
     }
-    // K-outer operands (NSTAGE == 2): the registers fetched above go to the other stage now
-    if (s + AHEAD < nslab) commit((s + AHEAD) % NSTAGE);
   }
 
   // epilogue: the output type is wave-uniform; branch once, then every store is straight-line
   const int64_t obase = b * a.M * a.N;
   switch (a.odt) {
-#define HIPNX_EPI(T) case T: gemm_epilogue<DT, T, TM, TN>(acc, a.out, obase, a.M, a.N, m0 + wm, n0 + wn, lane); break;
+#define HIPNX_EPI(T) case T: gemm_epilogue<DT, T, TM16, TN16>(acc, a.out, obase, a.M, a.N, m0 + wm, n0 + wn, lane); break;
     HIPNX_EPI(HIPNX_BF16) HIPNX_EPI(HIPNX_F16) HIPNX_EPI(HIPNX_F32) HIPNX_EPI(HIPNX_F64)
     HIPNX_EPI(HIPNX_S8) HIPNX_EPI(HIPNX_U8) HIPNX_EPI(HIPNX_S16) HIPNX_EPI(HIPNX_U16)
     HIPNX_EPI(HIPNX_S32) HIPNX_EPI(HIPNX_U32) HIPNX_EPI(HIPNX_S64) HIPNX_EPI(HIPNX_U64)
