@@ -99,12 +99,15 @@ template <> struct Mma16<HIPNX_F32> {
   }
 };
 
-// Swizzle of the [row][k] LDS layout: 16-byte chunk index XOR a 3-bit function of the row.  The
-// function (bit0 = r0^r2, bit1 = r1^r2, bit2 = r2^r3 of the row index) is one of the maps a sweep
-// over all linear maps of the low four row bits measured as conflict-free for the fragment read
-// (16 consecutive rows x 4 chunks per ds_read_b128: 4 clocks per instruction instead of 8).
+// Swizzle of the [row][k] LDS layout: 16-byte chunk index XOR a 3-bit function of the row.  Its
+// part in the low four row bits (bit0 = r0^r2, bit1 = r1^r2, bit2 = r2^r3) is one of the maps a
+// sweep over all linear maps of those bits measured as conflict-free for the fragment read
+// (16 consecutive rows x 4 chunks per ds_read_b128: 4 clocks per instruction instead of 8); row
+// bits 4..6 are constant within a fragment and are mixed in for the transposed writes of the
+// register-staged operands, whose lanes hold rows 4, 8 or 16 apart.
 __device__ __forceinline__ int lds_slot(int row, int chunk) {
-  return chunk ^ (((row ^ (row >> 2)) & 1) | ((((row >> 1) ^ (row >> 2)) & 1) << 1) | ((((row >> 2) ^ (row >> 3)) & 1) << 2));
+  const int low = ((row ^ (row >> 2)) & 1) | ((((row >> 1) ^ (row >> 2)) & 1) << 1) | ((((row >> 2) ^ (row >> 3)) & 1) << 2);
+  return chunk ^ low ^ ((row >> 4) & 7);
 }
 
 typedef __attribute__((address_space(3))) void *lptr_t;
@@ -241,31 +244,40 @@ struct KOuterStage {
   }
 };
 
-// ---- K-outer 2-byte operands of the big tiles: no register staging at all.  The slab is copied
-// as it lies in memory -- [64 k][ROWS] , ROWS*2 bytes per k -- straight into LDS, and the MFMA
-// fragments are fetched with the transposing LDS read of gfx950, `ds_read_b64_tr_b16`: within
-// each group of 16 lanes, lane i supplies the address of a run of four 16-bit elements and lane j
-// receives element j%4 of the runs of lanes j/4, j/4+4, j/4+8, j/4+12 (measured on the part).
-// With lane i pointing at (k0 + i/4, n0 + 4*(i%4)) lane j therefore receives
-// [k0 .. k0+3][n0 + j]: four consecutive k of one row -- half an MFMA operand.
-// LDS layout: k-major, the 16-byte chunk index of a k-row XOR-ed with 4*(k&3): the 32 lanes served
-// per clock touch four k-rows x 64 contiguous bytes, which this spreads over all 64 banks
-// (SQ_LDS_BANK_CONFLICT = 0; with 2*(k&3) every such read took a second pass).
+// ---- K-outer 1- and 2-byte operands of the big tiles: no register staging at all.  The slab is
+// copied as it lies in memory -- [k][ROWS], ROWS*ES bytes per k -- straight into LDS, and the MFMA
+// fragments are fetched with the transposing LDS reads of gfx950 (semantics measured on the part).
+// Within each group of 16 lanes every lane supplies the address of an 8-byte run, and
+//   ds_read_b64_tr_b16: lane j receives element j%4 of the runs of lanes j/4 + {0, 4, 8, 12};
+//     with lane i pointing at (k0 + i/4, n0 + 4*(i%4)) lane j receives [k0..k0+3][n0 + j];
+//   ds_read_b64_tr_b8:  lane j receives byte j%8 of the runs of lanes j/8 + {0, 2, .., 14};
+//     with lane i pointing at (k0 + i/2, n0 + 8*(i%2)) lane j receives [k0..k0+7][n0 + j]
+// -- in both cases half an MFMA operand (8 bytes of consecutive k of one row).
+// LDS layout: k-major, the 16-byte chunk index of a k-row XOR-ed with a function of k chosen so
+// that the 32 lanes served per clock (lanes 0..31, then 32..63) cover all 64 banks
+// (SQ_LDS_BANK_CONFLICT = 0): per clock the 16-bit form touches 8 k-rows x 32 bytes
+// (k = 8g + 4h + 0..3 for lane groups g and g+1), the 8-bit form 16 k-rows x 16 bytes
+// (k = 16g + 8h + 0..7).  A k-row must span all banks, i.e. at least 256 bytes.
 typedef short v4s __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
 
-__device__ __forceinline__ int tr_slot(int k, int chunk) { return chunk ^ ((k & 3) << 2) ^ (((k >> 3) & 1) << 1); }
+template <int ES>
+__device__ __forceinline__ int tr_slot(int k, int chunk) {
+  if constexpr (ES == 2) return chunk ^ ((k & 3) << 2) ^ (((k >> 3) & 1) << 1);
+  else return chunk ^ (k & 7) ^ (((k >> 4) & 1) << 3);
+}
 
-template <int ROWS, int NWAVES>
+template <int ES, int ROWS, int NWAVES>
 struct KOuterDmaLoader {
-  static constexpr int RBYTES = ROWS * 2;      // bytes per k-row of the slab
-  static constexpr int INSTR = ROWS / 8;       // 64 k-rows * RBYTES / 1 KiB
+  static constexpr int RBYTES = ROWS * ES;     // bytes per k-row of the slab
+  static constexpr int INSTR = ROWS / 8;       // (128 / ES) k-rows * RBYTES / 1 KiB
   static constexpr int PER = INSTR / NWAVES;
   static_assert(RBYTES >= 256 && INSTR % NWAVES == 0, "needs at least 16 chunks per k-row");
   const unsigned char *src[PER];
   int lds_off[PER];
 
   // g: [K, cols] with `ld` bytes per k; the tile covers columns col0 .. col0+ROWS-1, of which
-  // cols_valid (a multiple of 8) exist: chunks past the edge re-read the last valid chunk
+  // cols_valid (a multiple of 16 bytes' worth) exist: chunks past the edge re-read the last valid one
   __device__ __forceinline__ void init(const unsigned char *__restrict__ g, int64_t ld, int64_t col0, int64_t cols_valid,
                                        int wave, int lane) {
 #pragma unroll
@@ -273,8 +285,8 @@ struct KOuterDmaLoader {
       const int t = wave + NWAVES * i;
       const int o = t * 1024 + lane * 16;
       const int k = o / RBYTES, slot = (o % RBYTES) / 16;
-      int64_t byte = col0 * 2 + tr_slot(k, slot) * 16;
-      const int64_t last = cols_valid * 2 - 16;
+      int64_t byte = col0 * ES + tr_slot<ES>(k, slot) * 16;
+      const int64_t last = cols_valid * ES - 16;
       byte = byte <= last ? byte : last;
       src[i] = g + (int64_t)k * ld + byte;
       lds_off[i] = t * 1024;
@@ -292,24 +304,35 @@ struct KOuterDmaLoader {
   }
 };
 
-// MFMA operand fragment of rows row0 .. row0+15 for K step `ks` (32 elements) out of a k-major
-// slab.  `ds_read_b64_tr_b16`: within a group of 16 lanes, lane j receives element j%4 of the
-// 8-byte runs addressed by lanes j/4, j/4+4, j/4+8 and j/4+12 -- so lane i points at row block
-// i%4 of k-row i/4, and lane j ends up with row j at four consecutive k.
-template <int ROWS>
+// MFMA operand fragment (16 bytes of consecutive k per lane) of rows row0 .. row0+15 for K step
+// `ks` (64 bytes of k) out of a k-major slab: two transposing reads.
+template <int ES, int ROWS>
 __device__ __forceinline__ v4i read_fragment_tr(const unsigned char *slab, int row0, int ks, int lane) {
   const int i16 = lane & 15;
-  const int n = row0 + 4 * (i16 & 3);
-  const int kbase = 32 * ks + 8 * (lane >> 4) + (i16 >> 2);
   v4i out;
+  if constexpr (ES == 2) {
+    const int n = row0 + 4 * (i16 & 3);
+    const int kbase = 32 * ks + 8 * (lane >> 4) + (i16 >> 2);
 #pragma unroll
-  for (int h = 0; h < 2; h++) {
-    const int k = kbase + 4 * h;
-    const unsigned char *p = slab + k * (ROWS * 2) + tr_slot(k, n >> 3) * 16 + (n & 7) * 2;
-    const v4s r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s *)p);
-    const int2 w = __builtin_bit_cast(int2, r);
-    out[2 * h] = w.x;
-    out[2 * h + 1] = w.y;
+    for (int h = 0; h < 2; h++) {
+      const int k = kbase + 4 * h;
+      const unsigned char *p = slab + k * (ROWS * 2) + tr_slot<2>(k, n >> 3) * 16 + (n & 7) * 2;
+      const v4s r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s *)p);
+      const int2 w = __builtin_bit_cast(int2, r);
+      out[2 * h] = w.x;
+      out[2 * h + 1] = w.y;
+    }
+  } else {
+    const int n = row0 + 8 * (i16 & 1);
+    const int kbase = 64 * ks + 16 * (lane >> 4) + (i16 >> 1);
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      const int k = kbase + 8 * h;
+      const unsigned char *p = slab + k * ROWS + tr_slot<1>(k, n >> 4) * 16 + (n & 15);
+      const v2i r = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i *)p);
+      out[2 * h] = r[0];
+      out[2 * h + 1] = r[1];
+    }
   }
   return out;
 }
@@ -427,11 +450,12 @@ gemm_pipelined_kernel(GemmArgs a) {
   if constexpr (L_KIN) lload.init(lb, a.ld_l, m0, a.M, wave, lane);
   if constexpr (R_KIN) rload.init(rb, a.ld_r, n0, a.N, wave, lane);
   constexpr int ES = (DT == HIPNX_S8) ? 1 : (DT == HIPNX_F32 ? 4 : 2);
-  // K-outer 2-byte operands of tiles with at least a cache line per k-row: DMA + transposing reads
-  constexpr bool L_TR = !L_KIN && ES == 2 && BM >= 128 && (BM / 8) % NW == 0;
-  constexpr bool R_TR = !R_KIN && ES == 2 && BN >= 128 && (BN / 8) % NW == 0;
-  KOuterDmaLoader<L_TR ? BM : 128 * NW, NW> ltr;
-  KOuterDmaLoader<R_TR ? BN : 128 * NW, NW> rtr;
+  // K-outer 1- and 2-byte operands of tiles whose k-rows span all LDS banks: DMA + transposing reads
+  constexpr bool L_TR = !L_KIN && ES <= 2 && BM * ES >= 256 && (BM / 8) % NW == 0;
+  constexpr bool R_TR = !R_KIN && ES <= 2 && BN * ES >= 256 && (BN / 8) % NW == 0;
+  constexpr int TR_ES = ES <= 2 ? ES : 2;
+  KOuterDmaLoader<TR_ES, L_TR ? BM : 256 * NW, NW> ltr;
+  KOuterDmaLoader<TR_ES, R_TR ? BN : 256 * NW, NW> rtr;
   if constexpr (L_TR) ltr.init(lb, a.ld_l, m0, a.M, wave, lane);
   if constexpr (R_TR) rtr.init(rb, a.ld_r, n0, a.N, wave, lane);
   KOuterStage<ES, BM, NT> lregs;
@@ -483,14 +507,14 @@ gemm_pipelined_kernel(GemmArgs a) {
   };
   auto read_l = [&](const unsigned char *st, int ks, int i) -> v4i {
     const int row = wm + 16 * i + (lane & 15);
-    if constexpr (L_TR) return read_fragment_tr<BM>(st, wm + 16 * i, ks, lane);
+    if constexpr (L_TR) return read_fragment_tr<TR_ES, BM>(st, wm + 16 * i, ks, lane);
     else return *reinterpret_cast<const v4i *>(st + row * SLAB + lds_slot(row, 4 * ks + (lane >> 4)) * 16);
   };
   auto read_r = [&](const unsigned char *st, int t) -> v4i {  // step t = (K step, column tile)
     const int ks = t / TN16, j = t % TN16;
     const int row = wn + 16 * j + (lane & 15);
     const unsigned char *sB = st + BM * SLAB;
-    if constexpr (R_TR) return read_fragment_tr<BN>(sB, wn + 16 * j, ks, lane);
+    if constexpr (R_TR) return read_fragment_tr<TR_ES, BN>(sB, wn + 16 * j, ks, lane);
     else return *reinterpret_cast<const v4i *>(sB + row * SLAB + lds_slot(row, 4 * ks + (lane >> 4)) * 16);
   };
 
