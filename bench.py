@@ -31,7 +31,7 @@ PEAK = {"bf16": 2500.0, "f16": 2500.0, "s8": 5000.0, "f32": 157.3}  # dense MFMA
 # (`rocprofv3 --pmc FETCH_SIZE`, then `--pmc WRITE_SIZE`, with --calibrate): KiB per dispatch of the
 # gemm kernel, each scaled by what the same counter read for the 1 GiB + 1 GiB calibration kernel.
 # The figures and the commands are in profiles/dot_bf16_4096_hbm_traffic.md.
-HEADLINE_TRAFFIC_BYTES = 244290161  # 98468 KiB x 2.0 fetched + 41628 KiB x 1.0 written; algorithmic 100663296
+HEADLINE_TRAFFIC_BYTES = 235345715  # 98467 KiB x 2.0 fetched + 32895 KiB x 1.0 written; algorithmic 100663296
 
 
 def main():

@@ -18,11 +18,11 @@ int launch_gemm_f16(const hipnx_ctx *ctx, int cfg, bool l_kin, bool r_kin, GemmA
 int launch_gemm_f32(const hipnx_ctx *ctx, int cfg, bool l_kin, bool r_kin, GemmArgs a, int64_t batch);
 int launch_gemm_s8(const hipnx_ctx *ctx, int cfg, bool l_kin, bool r_kin, GemmArgs a, int64_t batch);
 
-template <int DT, int WM, int WN, int TM, int TN, bool LK, bool RK>
+template <int DT, int WM, int WN, int TM, int TN, bool LK, bool RK, int NSTAGE = 2>
 static int launch_one(const hipnx_ctx *ctx, GemmArgs a, int64_t batch) {
   constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
-  constexpr int smem = 2 * (BM + BN) * SLAB;
-  auto kern = gemm_pipelined_kernel<DT, WM, WN, TM, TN, LK, RK>;
+  constexpr int smem = NSTAGE * (BM + BN) * SLAB;
+  auto kern = gemm_pipelined_kernel<DT, WM, WN, TM, TN, LK, RK, NSTAGE>;
   static bool configured = false;  // per instantiation; racing writers store the same value
   if (!configured) {
     HIPNX_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
@@ -42,7 +42,12 @@ static int launch_cfg(const hipnx_ctx *ctx, int cfg, const GemmArgs &a, int64_t 
   switch (cfg) {
     case GEMM_CFG_256: return launch_one<DT, 4, 2, 2, 4, LK, RK>(ctx, a, batch);
     case GEMM_CFG_128: return launch_one<DT, 2, 2, 2, 2, LK, RK>(ctx, a, batch);
-    default: return launch_one<DT, 2, 1, 1, 1, LK, RK>(ctx, a, batch);
+    default:
+      // streaming a long weight matrix past a few rows is bound by the bytes in flight: six
+      // stages (five slabs of 12 KiB requested ahead per work-group) when both operands are copied
+      // straight into LDS
+      if constexpr (LK && RK) return launch_one<DT, 2, 1, 1, 1, LK, RK, 6>(ctx, a, batch);
+      else return launch_one<DT, 2, 1, 1, 1, LK, RK>(ctx, a, batch);
   }
 }
 

@@ -400,7 +400,7 @@ __device__ __forceinline__ void wait_vmcnt() {  // s_waitcnt vmcnt(N), other cou
   __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
 }
 
-template <int DT, int WM, int WN, int TM, int TN, bool L_KIN, bool R_KIN>
+template <int DT, int WM, int WN, int TM, int TN, bool L_KIN, bool R_KIN, int NSTAGE = 2>
 __global__ void __launch_bounds__(WM *WN * 64)
 gemm_pipelined_kernel(GemmArgs a) {
   typedef typename Mma16<DT>::acc_t acc_t;
@@ -476,7 +476,10 @@ gemm_pipelined_kernel(GemmArgs a) {
     if constexpr (!R_KIN && !R_TR) rregs.store(sB, tid);
   };
 
-  // ---- the K walk.  Two LDS stages; slab s lives in stage s % 2.
+  // ---- the K walk.  NSTAGE LDS stages; slab s lives in stage s % NSTAGE and the requests for
+  // slab s+NSTAGE-1 go out while slab s is computed (more than two stages only when every
+  // operand arrives by direct-to-LDS loads: these are counted by hand, vmcnt(n) leaves the
+  // younger slabs in flight).
   // One step = one column of 16x16 tiles (TM16 MFMAs) of one K step; a slab is STEPS steps.
   // Fragment reads run DIST steps ahead of the MFMAs that use them (r fragments in a ring of
   // four, l fragments of the next K step fetched during the last steps of the current one), and
@@ -518,10 +521,19 @@ gemm_pipelined_kernel(GemmArgs a) {
     else return *reinterpret_cast<const v4i *>(sB + row * SLAB + lds_slot(row, 4 * ks + (lane >> 4)) * 16);
   };
 
+  constexpr bool ALL_DMA = (L_KIN || L_TR) && (R_KIN || R_TR);
+  static_assert(NSTAGE == 2 || ALL_DMA, "register-staged operands need the two-stage walk");
+  constexpr int OPS = (L_KIN ? KInnerLoader<BM, NW>::PER : L_TR ? KOuterDmaLoader<TR_ES, L_TR ? BM : 256 * NW, NW>::PER : 0) +
+                      (R_KIN ? KInnerLoader<BN, NW>::PER : R_TR ? KOuterDmaLoader<TR_ES, R_TR ? BN : 256 * NW, NW>::PER : 0);
+  constexpr int INFLIGHT = OPS * (NSTAGE - 2);  // requests of younger slabs that may stay outstanding
+  static_assert(INFLIGHT < 64, "vmcnt is a 6-bit counter");
   const int nslab = (int)(a.Kb / SLAB);
-  issue(0, 0);
+#pragma unroll
+  for (int p = 0; p < NSTAGE - 1; p++)
+    if (p < nslab) issue(p, (int64_t)p * SLAB);
   commit(0);
-  wait_vmcnt<0>();
+  if (nslab >= NSTAGE - 1) wait_vmcnt<INFLIGHT>();
+  else wait_vmcnt<0>();
   __syncthreads();
   v4i fa[2][TM16], fb[RING];
 #pragma unroll
@@ -530,9 +542,11 @@ gemm_pipelined_kernel(GemmArgs a) {
   for (int d = 0; d < DIST; d++) fb[d] = read_r(smem, d);
 
   for (int s = 0; s < nslab; s++) {
-    const unsigned char *cur = smem + (s & 1) * STAGE, *nxt = smem + ((s + 1) & 1) * STAGE;
-    const bool more = s + 1 < nslab;
-    const int64_t next_kbyte = (int64_t)(s + 1) * SLAB;
+    const unsigned char *cur = smem + (s % NSTAGE) * STAGE, *nxt = smem + ((s + 1) % NSTAGE) * STAGE;
+    const bool more = s + 1 < nslab;                  // another slab to compute after this one
+    const bool request = s + NSTAGE - 1 < nslab;      // another slab to request during this one
+    const int req_stage = (s + NSTAGE - 1) % NSTAGE;
+    const int64_t req_kbyte = (int64_t)(s + NSTAGE - 1) * SLAB;
 #pragma unroll
     for (int t = 0; t < STEPS; t++) {
       const int ks = t / TN16, j = t % TN16;
@@ -549,13 +563,14 @@ gemm_pipelined_kernel(GemmArgs a) {
         for (int i = 0; i < TM16; i++)
           if (i >= d * TM16 / DIST && i < (d + 1) * TM16 / DIST) fa[0][i] = read_l(nxt, 0, i);
       }
-      if (more && t <= BAR) issue_step(t, (s + 1) & 1, next_kbyte);
+      if (request && t <= BAR) issue_step(t, req_stage, req_kbyte);
 #pragma unroll
       for (int i = 0; i < TM16; i++) Mma16<DT>::step(acc[i][j], fb[t % RING], fa[ks & 1][i]);
       if (t == BAR && more) {
-        commit((s + 1) & 1);
+        commit(req_stage);                   // (two stages: the slab requested is the next one)
         __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): my reads of this slab have returned
-        wait_vmcnt<0>();                     // my loads of the next slab have landed
+        if (request) wait_vmcnt<INFLIGHT>(); // my loads of the next slab have landed
+        else wait_vmcnt<0>();
         __syncthreads();
       }
       __builtin_amdgcn_sched_barrier(0);
