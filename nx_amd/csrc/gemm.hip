@@ -14,6 +14,8 @@
 // Algorithmic work: 2*B*M*N*K flop; minimum traffic bytes(l) + bytes(r) + bytes(out).
 #include <type_traits>
 
+#include <algorithm>
+
 #include "gemm_launch.cuh"
 
 namespace hipnx {
@@ -251,6 +253,9 @@ extern "C" int hipnx_dot(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t
         if (M <= 64) cfg = GEMM_CFG_64x32;
         else if (t256 * 4 >= (int64_t)ctx->num_cus * 3 && M >= 192 && N >= 192) cfg = GEMM_CFG_256;
         else cfg = GEMM_CFG_128;
+        if (M <= 64 && l_kin && r_kin && Kb % 4096 == 0 && N >= 256) {
+          st = launch_gemm_rows(ctx, l_dt, a, batch);  // weights streamed once, never through LDS
+        } else
         switch (l_dt) {
           case HIPNX_BF16: st = launch_gemm_bf16(ctx, cfg, l_kin, r_kin, a, batch); break;
           case HIPNX_F16: st = launch_gemm_f16(ctx, cfg, l_kin, r_kin, a, batch); break;

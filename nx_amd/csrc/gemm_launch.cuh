@@ -17,6 +17,8 @@ int launch_gemm_bf16(const hipnx_ctx *ctx, int cfg, bool l_kin, bool r_kin, Gemm
 int launch_gemm_f16(const hipnx_ctx *ctx, int cfg, bool l_kin, bool r_kin, GemmArgs a, int64_t batch);
 int launch_gemm_f32(const hipnx_ctx *ctx, int cfg, bool l_kin, bool r_kin, GemmArgs a, int64_t batch);
 int launch_gemm_s8(const hipnx_ctx *ctx, int cfg, bool l_kin, bool r_kin, GemmArgs a, int64_t batch);
+// few rows (M <= 64) against a long K-inner matrix, Kb a multiple of 4096: gemm_rows.hip
+int launch_gemm_rows(const hipnx_ctx *ctx, int dt, GemmArgs a, int64_t batch);
 
 template <int DT, int WM, int WN, int TM, int TN, bool LK, bool RK, int NSTAGE = 2>
 static int launch_one(const hipnx_ctx *ctx, GemmArgs a, int64_t batch) {

@@ -121,7 +121,12 @@ typedef __attribute__((address_space(3))) void *lptr_t;
 // compiler's own vmcnt waits only become stricter by loads it does not know of.
 __device__ __forceinline__ void lds_dma16(const unsigned char *g, unsigned char *lds) {
   const unsigned base = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(lptr_t)lds);
+  // (M0 is named as clobbered so that the compiler re-initialises it for its own uses; the
+  // diagnostic about reserved registers in a clobber list is expected)
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(base) : "memory", "m0");
+#pragma clang diagnostic pop
 }
 
 // K-inner slab loader: ROWS x 128 B, direct to LDS.  The per-lane source pointers (row clamp,

@@ -157,3 +157,37 @@ def test_float_dot_pipelined_kernel_layouts(ty, M, N, K, layout, hip, oracle):
     c2 = [0] if layout[1] == "n" else [1]
     eq = ("mk" if layout[0] == "n" else "km") + "," + ("kn" if layout[1] == "n" else "nk") + "->mn"
     check_float_dot(Nx.dot(ha, c1, hb, c2), Nx.dot(oa, c1, ob, c2), values(oa), values(ob), eq, K, f"{ty} {layout} {M}x{N}x{K}")
+
+
+# Few rows against a long K-inner matrix (M <= 64, K a multiple of 4096 bytes, N >= 256) take
+# the weight-streaming kernel: ragged row counts, a column count that is not a multiple of the
+# 64 columns of a work-group, every MFMA element type, and a batch.
+@pytest.mark.parametrize("M", [1, 16, 33, 64])
+@pytest.mark.parametrize("ty,N,K", [("s8", 300, 4096), ("s8", 1000, 8192), ("bf16", 264, 2048), ("f16", 257, 4096),
+                                    ("f32", 320, 1024), ("bf16", 1024, 4096)])
+def test_few_rows_against_long_matrix(M, ty, N, K, hip, oracle):
+    rng = np.random.default_rng(seed_of(M, ty, N, K))
+    if ty == "s8":
+        x = rng.integers(-127, 128, size=(M, K)).astype(np.int8)
+        w = rng.integers(-127, 128, size=(N, K)).astype(np.int8)
+        hx, ox = both(x, ty, hip, oracle)
+        hw, ow = both(w, ty, hip, oracle)
+        got, want = Nx.dot(hx, [1], hw, [1], out_type="s32"), Nx.dot(ox, [1], ow, [1], out_type="s32")
+        assert_bits_equal(got, want, f"few rows s8 {M}x{N}x{K}")
+    else:
+        x, w = rand_raw(rng, ty, (M, K), lo=-1, hi=1), rand_raw(rng, ty, (N, K), lo=-1, hi=1)
+        hx, ox = both(x, ty, hip, oracle)
+        hw, ow = both(w, ty, hip, oracle)
+        got, want = Nx.dot(hx, [1], hw, [1]), Nx.dot(ox, [1], ow, [1])
+        check_float_dot(got, want, values(ox), values(ow), "mk,nk->mn", K, f"few rows {ty} {M}x{N}x{K}")
+
+
+def test_few_rows_against_long_matrix_batched(hip, oracle):
+    rng = np.random.default_rng(7)
+    x = rng.integers(-127, 128, size=(3, 20, 4096)).astype(np.int8)
+    w = rng.integers(-127, 128, size=(3, 272, 4096)).astype(np.int8)
+    hx, ox = both(x, "s8", hip, oracle)
+    hw, ow = both(w, "s8", hip, oracle)
+    got = Nx.dot(hx, [2], [0], hw, [2], [0], out_type="s32")
+    want = Nx.dot(ox, [2], [0], ow, [2], [0], out_type="s32")
+    assert_bits_equal(got, want, "few rows s8 batched")
