@@ -6,6 +6,7 @@ no GPU is present every compute entry point fails with HipNxError.
 from __future__ import annotations
 
 import ctypes as C
+import functools
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
@@ -90,9 +91,14 @@ def check(status: int) -> int:
     raise cls(status, last_error())
 
 
-def i64_array(values):
-    values = list(values)
+@functools.lru_cache(maxsize=4096)
+def _i64_array_cached(values: tuple):
     return (C.c_int64 * max(len(values), 1))(*values)
+
+
+def i64_array(values):
+    """A C array of int64 for dims / strides (read-only on the C side, so equal tuples share one)."""
+    return _i64_array_cached(tuple(values))
 
 
 def int_array(values):

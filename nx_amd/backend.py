@@ -172,12 +172,28 @@ class HipNxBackend:
         L.check(L.lib.hipnx_d2h(t.data.ref.ctx, cls._handle(t), 0, arr.ctypes.data_as(C.c_void_p), arr.nbytes))
         return arr
 
+    _scalar_cache = {}  # (device, type, encoded element) -> _Ref of a rank-0 constant
+
     @classmethod
     def constant(cls, out: Tensor, number, opts=None) -> Tensor:
-        """constant/3 (backend.ex:49; oracle binary_backend.ex:42-46)."""
+        """constant/3 (backend.ex:49; oracle binary_backend.ex:42-46).  Rank-0 constants -- what
+        `Nx.multiply(t, 0.5)` turns its number into -- are kept per device and shared: tensors are
+        immutable, and the cache holds its own share of the buffer, so deallocating one user
+        never frees it."""
         opts = cls.init(opts)
-        res = cls._alloc(out, opts["device"])
         elem = number_to_binary(number, out.type)
+        if out.shape == ():
+            key = (opts["device"], out.type, elem)
+            ref = cls._scalar_cache.get(key)
+            if ref is None:
+                if len(cls._scalar_cache) >= 1024:
+                    cls._scalar_cache.clear()
+                res = cls._alloc(out, opts["device"])
+                L.check(L.lib.hipnx_fill(res.data.ref.ctx, res.data.ref.handle, len(elem), elem, 1))
+                ref = cls._scalar_cache[key] = res.data.ref
+            ref.sharers += 1
+            return out.with_(data=cls(ref, opts["device"]))
+        res = cls._alloc(out, opts["device"])
         L.check(L.lib.hipnx_fill(res.data.ref.ctx, res.data.ref.handle, len(elem), elem, out.size))
         return res
 

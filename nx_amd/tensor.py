@@ -8,7 +8,7 @@ from __future__ import annotations
 
 import math
 import struct
-from dataclasses import dataclass, replace
+from dataclasses import dataclass
 from typing import Any, Optional, Tuple
 
 import numpy as np
@@ -38,9 +38,21 @@ class Tensor:
         return len(self.shape)
 
     def with_(self, **kw) -> "Tensor":
-        if "shape" in kw and "names" not in kw:
-            kw["names"] = (None,) * len(kw["shape"])
-        return replace(self, **kw)
+        """A copy with some fields replaced (the hot path of every callback: no re-validation of
+        the fields that are carried over)."""
+        t = object.__new__(Tensor)
+        set_ = object.__setattr__
+        set_(t, "data", kw["data"] if "data" in kw else self.data)
+        set_(t, "type", T.normalize(kw["type"]) if "type" in kw else self.type)
+        if "shape" in kw:
+            shape = tuple(int(d) for d in kw["shape"])
+            set_(t, "shape", shape)
+            names = kw.get("names", ())
+            set_(t, "names", tuple(names) if len(names) == len(shape) else (None,) * len(shape))
+        else:
+            set_(t, "shape", self.shape)
+            set_(t, "names", tuple(kw["names"]) if "names" in kw and len(kw["names"]) == len(self.shape) else self.names)
+        return t
 
 
 def template(type, shape) -> Tensor:

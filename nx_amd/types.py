@@ -31,6 +31,8 @@ _NUMPY = {
 
 def normalize(t):
     """Nx.Type.normalize!/1 (type.ex:190-230): accepts ("f", 32) or the short atom name "f32"."""
+    if t.__class__ is tuple and t in _CODES:  # already normal: the common case
+        return t
     if isinstance(t, str):
         if t not in _NAMES:
             raise ValueError(f"invalid numerical type: {t!r}")
