@@ -147,7 +147,11 @@ int hipnx_ctx_create(int device, hipnx_ctx **out) {
   hipError_t e2 = hipEventCreate(&ctx->ev_start);
   hipError_t e3 = hipEventCreate(&ctx->ev_stop);
   hipError_t e4 = hipMalloc(&ctx->flag, 256);
-  hipError_t e5 = hipHostMalloc(&ctx->flag_host, 256, hipHostMallocDefault);
+  hipError_t e5 = hipHostMalloc(&ctx->flag_host, 256, hipHostMallocMapped);
+  if (e5 == hipSuccess) {
+    std::memset(ctx->flag_host, 0, 256);
+    e5 = hipHostGetDevicePointer(&ctx->flag_host_dev, ctx->flag_host, 0);
+  }
   if (e4 == hipSuccess) e4 = hipMemset(ctx->flag, 0xFF, 256);  // gather bounds word: all-ones = no bad index
   if (e1 != hipSuccess || e2 != hipSuccess || e3 != hipSuccess || e4 != hipSuccess || e5 != hipSuccess) {
     hipnx_ctx_destroy(ctx);

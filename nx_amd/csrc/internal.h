@@ -23,7 +23,8 @@ struct hipnx_ctx {
   uint64_t live = 0, peak = 0, pooled = 0;
   int num_cus = 256;
   void *flag = nullptr;       // 32-byte device scratch for the gather bounds report
-  void *flag_host = nullptr;  // pinned mirror
+  void *flag_host = nullptr;  // pinned host word, mapped into the device: non-zero once a kernel saw a bad index
+  void *flag_host_dev = nullptr;  // its device address
 };
 
 struct hipnx_buf {

@@ -69,12 +69,14 @@ transpose2d_kernel(const T *__restrict__ in, T *__restrict__ out, int64_t R, int
 // LPR lanes (a power of two, at most one wavefront) copy one slice with 16-byte (VEC) or 1-byte
 // accesses, four independent accesses in flight per lane; a 256-lane block works on 256/LPR
 // slices at once so that the index -> address -> data dependency of one slice overlaps with the
-// others'.  flag[0] receives the smallest (tuple * depth + axis) whose index is out of range.
+// others'.  flag[0] receives the smallest (tuple * depth + axis) whose index is out of range, and the
+// pinned host word `host_seen` is set so that the host learns of it without a copy.
 template <bool VEC>
 __global__ void __launch_bounds__(BLOCK)
 gather_kernel(const unsigned char *__restrict__ t, const void *__restrict__ idx, unsigned char *__restrict__ out,
               int idx_dt, int64_t n_tuples, int depth, Strided tdims /* dims = leading extents, strides = bytes */,
-              int64_t slice_bytes, int lpr, int clamp, unsigned long long *__restrict__ flag) {
+              int64_t slice_bytes, int lpr, int clamp, unsigned long long *__restrict__ flag,
+              unsigned int *__restrict__ host_seen) {
   constexpr int W = VEC ? 16 : 1;
   typedef raw_vec<W> vec_t;
   const int64_t chunks = slice_bytes / W;
@@ -91,7 +93,10 @@ gather_kernel(const unsigned char *__restrict__ t, const void *__restrict__ idx,
         if (clamp) v = (v < 0 && idx_dt != HIPNX_U64) ? 0 : dim - 1;
         else {
           ok = false;
-          if (lane == 0) atomicMin(flag, (unsigned long long)(row * depth + a));
+          if (lane == 0) {
+            atomicMin(flag, (unsigned long long)(row * depth + a));
+            __hip_atomic_store(host_seen, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);  // pinned host word
+          }
           break;
         }
       }
@@ -299,18 +304,21 @@ extern "C" int hipnx_gather(hipnx_ctx *ctx, int elem_bytes, int rank, const int6
   dim3 grid(grid_for(ctx, n_tuples, BLOCK / lpr)), block(BLOCK);
   if (vec)
     hipLaunchKernelGGL((gather_kernel<true>), grid, block, 0, ctx->stream, (const unsigned char *)t->ptr, idx->ptr,
-                       (unsigned char *)out->ptr, idx_dt, n_tuples, depth, td, slice_bytes, lpr, (int)(oob_policy == HIPNX_OOB_CLAMP), flag);
+                       (unsigned char *)out->ptr, idx_dt, n_tuples, depth, td, slice_bytes, lpr, (int)(oob_policy == HIPNX_OOB_CLAMP), flag, (unsigned int *)ctx->flag_host_dev);
   else
     hipLaunchKernelGGL((gather_kernel<false>), grid, block, 0, ctx->stream, (const unsigned char *)t->ptr, idx->ptr,
-                       (unsigned char *)out->ptr, idx_dt, n_tuples, depth, td, slice_bytes, lpr, (int)(oob_policy == HIPNX_OOB_CLAMP), flag);
+                       (unsigned char *)out->ptr, idx_dt, n_tuples, depth, td, slice_bytes, lpr, (int)(oob_policy == HIPNX_OOB_CLAMP), flag, (unsigned int *)ctx->flag_host_dev);
   HIPNX_HIP(hipGetLastError());
   if (oob_policy == HIPNX_OOB_RAISE) {
-    // the reference raises on the first offending index: wait, then report it the same way
-    volatile unsigned long long *host = (volatile unsigned long long *)ctx->flag_host;
-    HIPNX_HIP(hipMemcpyAsync((void *)host, flag, 8, hipMemcpyDeviceToHost, ctx->stream));
+    // the reference raises on the first offending index: wait, then report it the same way.
+    // The kernel marks a pinned host word when it meets one, so the good path costs the wait only.
+    volatile unsigned int *seen = (volatile unsigned int *)ctx->flag_host;
     HIPNX_HIP(hipStreamSynchronize(ctx->stream));
-    if (host[0] != ~0ull) {
-      const int64_t pos = (int64_t)host[0];
+    if (seen[0] != 0) {
+      unsigned long long first = ~0ull;
+      HIPNX_HIP(hipMemcpy(&first, flag, 8, hipMemcpyDeviceToHost));
+      const int64_t pos = (int64_t)first;
+      seen[0] = 0;
       HIPNX_HIP(hipMemsetAsync(flag, 0xFF, 8, ctx->stream));  // re-arm
       const int axis = (int)(pos % depth);
       unsigned char raw[8] = {0};
