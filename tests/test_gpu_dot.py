@@ -191,3 +191,33 @@ def test_few_rows_against_long_matrix_batched(hip, oracle):
     got = Nx.dot(hx, [2], [0], hw, [2], [0], out_type="s32")
     want = Nx.dot(ox, [2], [0], ow, [2], [0], out_type="s32")
     assert_bits_equal(got, want, "few rows s8 batched")
+
+
+# Shapes large enough for the 256 x 256 tile (at least 192 of them), ragged at both edges, in every
+# operand layout: covers the transposing-read staging of K-outer bf16 and s8 operands on both
+# sides.  The oracle runs on a sample of output rows.
+@pytest.mark.parametrize("ty", ["bf16", "s8"])
+@pytest.mark.parametrize("layout", ["nn", "nt", "tn", "tt"])
+def test_large_ragged_dot_on_the_big_tile(ty, layout, hip, oracle):
+    M, N, K = 2064, 6160, 256
+    rng = np.random.default_rng(seed_of(ty, layout, "big tile"))
+    if ty == "s8":
+        a = rng.integers(-127, 128, size=(M, K)).astype(np.int8)
+        b = rng.integers(-127, 128, size=(K, N)).astype(np.int8)
+    else:
+        a, b = rand_raw(rng, ty, (M, K), lo=-1, hi=1), rand_raw(rng, ty, (K, N), lo=-1, hi=1)
+    la = a if layout[0] == "n" else np.ascontiguousarray(a.T)
+    lb = b if layout[1] == "n" else np.ascontiguousarray(b.T)
+    c1 = [1] if layout[0] == "n" else [0]
+    c2 = [0] if layout[1] == "n" else [1]
+    kw = {"out_type": "s32"} if ty == "s8" else {}
+    got = Nx.dot(from_numpy(la, ty, hip), c1, from_numpy(lb, ty, hip), c2, **kw)
+    assert got.shape == (M, N)
+    rows = np.unique(np.concatenate([[0, 255, 256, M - 1], rng.integers(0, M, size=24)]))
+    oa, ob = from_numpy(np.ascontiguousarray(a[rows]), ty, oracle), from_numpy(b, ty, oracle)
+    want = Nx.dot(oa, ob, **kw)
+    got_rows = from_numpy(np.ascontiguousarray(hip.to_numpy(got)[rows]), "s32" if ty == "s8" else ty, oracle)
+    if ty == "s8":
+        assert_bits_equal(got_rows, want, f"big tile s8 {layout}")
+    else:
+        check_float_dot(got_rows, want, values(oa), values(ob), "mk,kn->mn", K, f"big tile {ty} {layout}")
