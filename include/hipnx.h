@@ -71,7 +71,7 @@ enum {
   HIPNX_IS_INFINITY, HIPNX_NUNARY
 };
 
-enum { HIPNX_RED_SUM = 0, HIPNX_RED_MAX = 1, HIPNX_RED_MIN = 2, HIPNX_RED_PRODUCT = 3 };
+enum { HIPNX_RED_SUM = 0, HIPNX_RED_MAX = 1, HIPNX_RED_MIN = 2, HIPNX_RED_PRODUCT = 3, HIPNX_RED_ALL = 4, HIPNX_RED_ANY = 5 };
 enum { HIPNX_ARGMAX = 0, HIPNX_ARGMIN = 1 };
 enum { HIPNX_TIE_LOW = 0, HIPNX_TIE_HIGH = 1 };
 
@@ -147,8 +147,8 @@ int hipnx_as_type(hipnx_ctx *ctx, int in_dt, int out_dt, int64_t n, const hipnx_
                   hipnx_buf *out);
 
 /* ---- reductions ----------------------------------------------------------------------------
- * replaces: sum / product / reduce_max / reduce_min (nx/lib/nx/backend.ex:89-92; oracle
- * binary_backend.ex:1315-1375).  The input is viewed as [outer, red, inner] (the caller
+ * replaces: sum / product / reduce_max / reduce_min / all / any (nx/lib/nx/backend.ex:87-92; oracle
+ * binary_backend.ex:1293-1375; all / any: 1 unless / if an element differs from 0, u8 output).  The input is viewed as [outer, red, inner] (the caller
  * collapses axes, transposing first when the reduced axes are not adjacent); out is
  * [outer, inner]. */
 int hipnx_reduce(hipnx_ctx *ctx, int op, int in_dt, int out_dt, int64_t outer, int64_t red,
@@ -188,6 +188,36 @@ int hipnx_broadcast(hipnx_ctx *ctx, int elem_bytes, int rank, const int64_t *out
 int hipnx_gather(hipnx_ctx *ctx, int elem_bytes, int rank, const int64_t *t_dims, int idx_dt,
                  int64_t n_tuples, int depth, int oob_policy, const hipnx_buf *t,
                  const hipnx_buf *idx, hipnx_buf *out);
+
+/* ---- callbacks one step off the hot path (callers: Nx.LinAlg, Nx.Random, grad code) ----------
+ * replaces: select/4 (nx/lib/nx/backend.ex:84; oracle binary_backend.ex:604-648).
+ * out[i] = pred[i] != 0 ? on_true[i] : on_false[i]; the three operands are broadcast to out_dims
+ * by per-axis strides in elements (0 = repeat), values are converted to out_dt. */
+int hipnx_select(hipnx_ctx *ctx, int pred_dt, int true_dt, int false_dt, int out_dt, int rank,
+                 const int64_t *out_dims, const int64_t *pred_strides, const int64_t *true_strides,
+                 const int64_t *false_strides, const hipnx_buf *pred, const hipnx_buf *on_true,
+                 const hipnx_buf *on_false, hipnx_buf *out);
+
+/* replaces: clip/4 (nx/lib/nx/backend.ex:78; oracle binary_backend.ex:1788-1811); min and max
+ * are one-element buffers of their own types, read on the device */
+int hipnx_clip(hipnx_ctx *ctx, int in_dt, int min_dt, int max_dt, int out_dt, int64_t n,
+               const hipnx_buf *in, const hipnx_buf *min, const hipnx_buf *max, hipnx_buf *out);
+
+/* replaces: slice/5, concatenate/3, stack/3 (nx/lib/nx/backend.ex:79,82-83; oracle
+ * binary_backend.ex:1813-1863, 1962-2030) -- one copy over the index space `dims` with element
+ * strides and offsets on both sides: a slice reads strided and writes dense, a concatenation
+ * writes each operand into its window of the output */
+int hipnx_strided_copy(hipnx_ctx *ctx, int elem_bytes, int rank, const int64_t *dims,
+                       const int64_t *in_strides, int64_t in_offset, const int64_t *out_strides,
+                       int64_t out_offset, const hipnx_buf *in, hipnx_buf *out);
+
+/* replaces: iota/3 (nx/lib/nx/backend.ex:51; oracle binary_backend.ex:49-87):
+ * out[i] = (i / inner) % dim; the flat iota is dim = n, inner = 1 */
+int hipnx_iota(hipnx_ctx *ctx, int out_dt, int64_t n, int64_t dim, int64_t inner, hipnx_buf *out);
+
+/* replaces: eye/2 (nx/lib/nx/backend.ex:50; oracle binary_backend.ex:90-110): n elements of
+ * stacked rows x cols identity matrices */
+int hipnx_eye(hipnx_ctx *ctx, int out_dt, int64_t n, int64_t rows, int64_t cols, hipnx_buf *out);
 
 #ifdef __cplusplus
 }

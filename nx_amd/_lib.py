@@ -69,6 +69,12 @@ PROTOTYPES = {
     "hipnx_transpose": [_ctx_p, C.c_int, C.c_int, _i64p, _intp, _buf_p, _buf_p],
     "hipnx_broadcast": [_ctx_p, C.c_int, C.c_int, _i64p, _i64p, _buf_p, _buf_p],
     "hipnx_gather": [_ctx_p, C.c_int, C.c_int, _i64p, C.c_int, C.c_int64, C.c_int, C.c_int, _buf_p, _buf_p, _buf_p],
+    "hipnx_select": [_ctx_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _i64p, _i64p, _i64p, _i64p, _buf_p, _buf_p,
+                     _buf_p, _buf_p],
+    "hipnx_clip": [_ctx_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int64, _buf_p, _buf_p, _buf_p, _buf_p],
+    "hipnx_strided_copy": [_ctx_p, C.c_int, C.c_int, _i64p, _i64p, C.c_int64, _i64p, C.c_int64, _buf_p, _buf_p],
+    "hipnx_iota": [_ctx_p, C.c_int, C.c_int64, C.c_int64, C.c_int64, _buf_p],
+    "hipnx_eye": [_ctx_p, C.c_int, C.c_int64, C.c_int64, C.c_int64, _buf_p],
 }
 
 for _name, _args in PROTOTYPES.items():

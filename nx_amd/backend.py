@@ -26,13 +26,13 @@ from .tensor import Tensor, number_to_binary
 
 from .backend_names import BINARY_OPS, UNARY_OPS  # noqa: E402
 
-RED_SUM, RED_MAX, RED_MIN, RED_PRODUCT = 0, 1, 2, 3
+RED_SUM, RED_MAX, RED_MIN, RED_PRODUCT, RED_ALL, RED_ANY = 0, 1, 2, 3, 4, 5
 K_INNER, K_OUTER = 0, 1
 OOB_RAISE, OOB_CLAMP = 0, 1
 
 # callbacks of the behaviour that are not on the device path (nx/lib/nx/backend.ex:58-144)
-UNSUPPORTED = ["iota", "eye", "to_batched", "from_pointer", "to_pointer", "slice", "put_slice", "pad", "reverse",
-               "concatenate", "stack", "select", "clip", "conv", "all", "any", "window_sum", "window_product",
+UNSUPPORTED = ["to_batched", "from_pointer", "to_pointer", "put_slice", "pad", "reverse",
+               "conv", "window_sum", "window_product",
                "window_max", "window_min", "reduce", "window_reduce", "window_scatter_max", "window_scatter_min",
                "indexed_add", "indexed_put", "sort", "argsort", "fft", "ifft", "fft2", "ifft2", "triangular_solve",
                "conjugate", "real", "imag"]
@@ -341,6 +341,16 @@ class HipNxBackend:
         return cls._reduce(RED_MIN, out, t, opts)
 
     @classmethod
+    def all(cls, out, t, opts):
+        """all/3 (backend.ex:87; oracle binary_backend.ex:1293-1302): 1 unless an element is 0."""
+        return cls._reduce(RED_ALL, out, t, opts)
+
+    @classmethod
+    def any(cls, out, t, opts):
+        """any/3 (backend.ex:88; oracle binary_backend.ex:1305-1314): 1 if an element is not 0."""
+        return cls._reduce(RED_ANY, out, t, opts)
+
+    @classmethod
     def _argreduce(cls, op: int, out: Tensor, t: Tensor, opts) -> Tensor:
         dev = cls._device_of(t)
         t = cls._from_nx(t, dev)
@@ -442,6 +452,107 @@ class HipNxBackend:
                                    T.code(indices.type), n_tuples, depth, opts.get("oob_policy", OOB_RAISE),
                                    cls._handle(t), cls._handle(indices), res.data.ref.handle))
         return res
+
+    # ---- one step off the hot path: creation, selection, windows of memory -----------------------
+    @classmethod
+    def iota(cls, out: Tensor, axis, opts=None) -> Tensor:
+        """iota/3 (backend.ex:51; oracle binary_backend.ex:49-87): the index along `axis`, or the flat
+        index when `axis` is None."""
+        opts = cls.init(opts)
+        res = cls._alloc(out, opts["device"])
+        if axis is None:
+            dim, inner = max(out.size, 1), 1
+        else:
+            dim, inner = out.shape[axis], prod(out.shape[axis + 1:])
+        L.check(L.lib.hipnx_iota(res.data.ref.ctx, T.code(out.type), out.size, dim, inner, res.data.ref.handle))
+        return res
+
+    @classmethod
+    def eye(cls, out: Tensor, opts=None) -> Tensor:
+        """eye/2 (backend.ex:50; oracle binary_backend.ex:90-110): identity in the last two axes."""
+        opts = cls.init(opts)
+        res = cls._alloc(out, opts["device"])
+        L.check(L.lib.hipnx_eye(res.data.ref.ctx, T.code(out.type), out.size, out.shape[-2], out.shape[-1],
+                                res.data.ref.handle))
+        return res
+
+    @classmethod
+    def select(cls, out: Tensor, pred: Tensor, on_true: Tensor, on_false: Tensor) -> Tensor:
+        """select/4 (backend.ex:84; oracle binary_backend.ex:604-648)."""
+        dev = cls._device_of(pred, on_true, on_false)
+        pred, on_true, on_false = (cls._from_nx(x, dev) for x in (pred, on_true, on_false))
+        res = cls._alloc(out, dev)
+        L.check(L.lib.hipnx_select(
+            res.data.ref.ctx, T.code(pred.type), T.code(on_true.type), T.code(on_false.type), T.code(out.type),
+            len(out.shape), L.i64_array(out.shape), L.i64_array(S.broadcast_strides(pred.shape, out.shape)),
+            L.i64_array(S.broadcast_strides(on_true.shape, out.shape)),
+            L.i64_array(S.broadcast_strides(on_false.shape, out.shape)),
+            cls._handle(pred), cls._handle(on_true), cls._handle(on_false), res.data.ref.handle))
+        return res
+
+    @classmethod
+    def clip(cls, out: Tensor, t: Tensor, min_t: Tensor, max_t: Tensor) -> Tensor:
+        """clip/4 (backend.ex:78; oracle binary_backend.ex:1788-1811)."""
+        dev = cls._device_of(t, min_t, max_t)
+        t, min_t, max_t = (cls._from_nx(x, dev) for x in (t, min_t, max_t))
+        res = cls._alloc(out, dev)
+        L.check(L.lib.hipnx_clip(res.data.ref.ctx, T.code(t.type), T.code(min_t.type), T.code(max_t.type),
+                                 T.code(out.type), out.size, cls._handle(t), cls._handle(min_t), cls._handle(max_t),
+                                 res.data.ref.handle))
+        return res
+
+    @staticmethod
+    def _dense_strides(shape):
+        strides, s = [0] * len(shape), 1
+        for a in range(len(shape) - 1, -1, -1):
+            strides[a] = s
+            s *= shape[a]
+        return strides
+
+    @classmethod
+    def slice(cls, out: Tensor, t: Tensor, start_indices, lengths, strides) -> Tensor:
+        """slice/5 (backend.ex:79; oracle binary_backend.ex:1813-1863): start indices are numbers or
+        rank-0 tensors (read back when on the device) and are clamped so the window fits."""
+        dev = cls._device_of(t)
+        t = cls._from_nx(t, dev)
+        starts = []
+        for dim, idx, length in zip(t.shape, start_indices, lengths):
+            if isinstance(idx, Tensor):
+                idx = int(np.frombuffer(type(idx.data).to_binary(idx, 1), dtype=T.numpy_dtype(idx.type))[0])
+            starts.append(min(max(int(idx), 0), dim - length))
+        dense = cls._dense_strides(t.shape)
+        res = cls._alloc(out, dev)
+        L.check(L.lib.hipnx_strided_copy(
+            res.data.ref.ctx, T.size_bytes(t.type), len(out.shape), L.i64_array(out.shape),
+            L.i64_array([d * s for d, s in zip(dense, strides)]), sum(d * s for d, s in zip(dense, starts)),
+            L.i64_array(cls._dense_strides(out.shape)), 0, cls._handle(t), res.data.ref.handle))
+        return res
+
+    @classmethod
+    def concatenate(cls, out: Tensor, tensors, axis: int) -> Tensor:
+        """concatenate/3 (backend.ex:82; oracle binary_backend.ex:1975-1986): every operand is
+        converted to the output type and copied into its window along `axis`."""
+        dev = cls._device_of(*tensors)
+        res = cls._alloc(out, dev)
+        out_strides = cls._dense_strides(out.shape)
+        offset = 0
+        for t in tensors:
+            t = cls._from_nx(t, dev)
+            if t.type != out.type:
+                t = cls.as_type(t.with_(data=None, type=out.type), t)
+            L.check(L.lib.hipnx_strided_copy(
+                res.data.ref.ctx, T.size_bytes(out.type), len(t.shape), L.i64_array(t.shape),
+                L.i64_array(cls._dense_strides(t.shape)), 0, L.i64_array(out_strides), offset * out_strides[axis],
+                cls._handle(t), res.data.ref.handle))
+            offset += t.shape[axis]
+        return res
+
+    @classmethod
+    def stack(cls, out: Tensor, tensors, axis: int) -> Tensor:
+        """stack/3 (backend.ex:83; oracle binary_backend.ex:1962-1972): concatenation of the operands
+        with a unit axis inserted at `axis`."""
+        widened = [t.with_(shape=t.shape[:axis] + (1,) + t.shape[axis:]) for t in tensors]
+        return cls.concatenate(out, widened, axis)
 
     @classmethod
     def block(cls, struct, out: Tensor, args, fun):

@@ -35,14 +35,17 @@ template <typename CT, int OP, bool UNS>
 struct PlainReducer {
   typedef CT acc_t;
   static __device__ __forceinline__ acc_t init() {
-    if constexpr (OP == HIPNX_RED_SUM) return (CT)0;
-    else if constexpr (OP == HIPNX_RED_PRODUCT) return (CT)1;
+    if constexpr (OP == HIPNX_RED_SUM || OP == HIPNX_RED_ANY) return (CT)0;
+    else if constexpr (OP == HIPNX_RED_PRODUCT || OP == HIPNX_RED_ALL) return (CT)1;
     else if constexpr (std::is_floating_point<CT>::value) return OP == HIPNX_RED_MAX ? (CT)-INFINITY : (CT)INFINITY;
     else if constexpr (UNS) return OP == HIPNX_RED_MAX ? (int64_t)0 : (int64_t)-1;
     else return OP == HIPNX_RED_MAX ? INT64_MIN : INT64_MAX;
   }
   static __device__ __forceinline__ acc_t combine(acc_t a, acc_t b) {
-    if constexpr (std::is_floating_point<CT>::value) {
+    // all / any work on truth values 0 / 1 (see accumulate)
+    if constexpr (OP == HIPNX_RED_ALL) return (a != (CT)0 && b != (CT)0) ? (CT)1 : (CT)0;
+    else if constexpr (OP == HIPNX_RED_ANY) return (a != (CT)0 || b != (CT)0) ? (CT)1 : (CT)0;
+    else if constexpr (std::is_floating_point<CT>::value) {
       if constexpr (OP == HIPNX_RED_SUM) return a + b;
       else if constexpr (OP == HIPNX_RED_PRODUCT) return a * b;
       else if constexpr (OP == HIPNX_RED_MAX) return (a != a || b != b) ? (CT)NAN : (b > a ? b : a);
@@ -60,6 +63,8 @@ struct PlainReducer {
     }
   }
   static __device__ __forceinline__ acc_t seed(acc_t a, int64_t) { return a; }
+  // (for all / any an element counts as true unless it equals 0 -- NaN included,
+  // binary_backend.ex:1293-1314)
   static __device__ __forceinline__ acc_t accumulate(acc_t a, CT x, int64_t) { return combine(a, x); }
   static __device__ __forceinline__ acc_t shfl_xor(acc_t a, int m) { return __shfl_xor(a, m, WAVE); }
 };
@@ -367,7 +372,7 @@ template <int OP>
 static int reduce_op(hipnx_ctx *ctx, int idt, int odt, int64_t outer, int64_t red, int64_t inner, const void *in,
                      void *out) {
   // selection (max / min) is exact in the element's own precision: f32 covers f32, bf16 and f16
-  if (is_float(idt) && idt != HIPNX_F64 && (OP == HIPNX_RED_MAX || OP == HIPNX_RED_MIN))
+  if (is_float(idt) && idt != HIPNX_F64 && (OP == HIPNX_RED_MAX || OP == HIPNX_RED_MIN || OP == HIPNX_RED_ALL || OP == HIPNX_RED_ANY))
     return run_reduce<PlainReducer<float, OP, false>, float>(ctx, idt, odt, outer, red, inner, in, out);
   if (is_float(idt)) return run_reduce<PlainReducer<double, OP, false>, double>(ctx, idt, odt, outer, red, inner, in, out);
   if (idt == HIPNX_U64 && (OP == HIPNX_RED_MAX || OP == HIPNX_RED_MIN))
@@ -398,7 +403,7 @@ extern "C" int hipnx_reduce(hipnx_ctx *ctx, int op, int in_dt, int out_dt, int64
                             int64_t inner, const hipnx_buf *inb, hipnx_buf *out) {
   Enter in(ctx);
   if (in.status) return in.status;
-  if (op < 0 || op > HIPNX_RED_PRODUCT) return set_error(HIPNX_EINVAL, "reduce: unknown op %d", op);
+  if (op < 0 || op > HIPNX_RED_ANY) return set_error(HIPNX_EINVAL, "reduce: unknown op %d", op);
   if (dtype_size(in_dt) < 0 || dtype_size(out_dt) < 0) return set_error(HIPNX_EINVAL, "reduce: unknown element type");
   if (int st = check_view(outer, red, inner)) return st;
   if ((op == HIPNX_RED_MAX || op == HIPNX_RED_MIN) && red == 0 && outer * inner > 0)
@@ -410,7 +415,9 @@ extern "C" int hipnx_reduce(hipnx_ctx *ctx, int op, int in_dt, int out_dt, int64
     case HIPNX_RED_SUM: return reduce_op<HIPNX_RED_SUM>(ctx, in_dt, out_dt, outer, red, inner, inb->ptr, out->ptr);
     case HIPNX_RED_MAX: return reduce_op<HIPNX_RED_MAX>(ctx, in_dt, out_dt, outer, red, inner, inb->ptr, out->ptr);
     case HIPNX_RED_MIN: return reduce_op<HIPNX_RED_MIN>(ctx, in_dt, out_dt, outer, red, inner, inb->ptr, out->ptr);
-    default: return reduce_op<HIPNX_RED_PRODUCT>(ctx, in_dt, out_dt, outer, red, inner, inb->ptr, out->ptr);
+    case HIPNX_RED_PRODUCT: return reduce_op<HIPNX_RED_PRODUCT>(ctx, in_dt, out_dt, outer, red, inner, inb->ptr, out->ptr);
+    case HIPNX_RED_ALL: return reduce_op<HIPNX_RED_ALL>(ctx, in_dt, out_dt, outer, red, inner, inb->ptr, out->ptr);
+    default: return reduce_op<HIPNX_RED_ANY>(ctx, in_dt, out_dt, outer, red, inner, inb->ptr, out->ptr);
   }
 }
 

@@ -1,0 +1,357 @@
+// Callbacks one step off the hot path, native so that chains stay on the device:
+// select, clip, slice / concatenate / stack (one strided copy), iota, eye.
+// Reference semantics: nx/lib/nx/binary_backend.ex:49-112 (iota, eye), 604-648 (select),
+// 1788-1811 (clip), 1813-1863 (slice), 1962-2030 (stack, concatenate).
+#include <cstring>
+
+#include "dtypes.cuh"
+#include "internal.h"
+
+namespace hipnx {
+
+constexpr int BLOCK = 256;
+constexpr int MAXR = 8;
+constexpr int E = 8;  // elements per lane per step of the vector kernels
+
+static int grid_for(int64_t items) {
+  int64_t blocks = (items + BLOCK - 1) / BLOCK;
+  if (blocks < 1) blocks = 1;
+  return (int)(blocks < (1ll << 30) ? blocks : (1ll << 30));
+}
+
+// ---- select ---------------------------------------------------------------------------------
+// out[i] = pred[i] != 0 ? on_true[i] : on_false[i], each operand broadcast by strides (0 = repeat).
+// CT: double when the output is a float type, int64 otherwise (both value operands are integers
+// then; u64 travels as its bit pattern and the store keeps the low bits).
+struct Sel {
+  int rank;
+  int64_t dims[MAXR], ps[MAXR], ts[MAXR], fs[MAXR];
+};
+
+template <typename CT>
+__device__ __forceinline__ bool truthy(const void *p, int dt, int64_t i) {
+  if (dt >= HIPNX_F16) {
+    const double v = load_one<double>(p, dt, i);
+    return v != 0;  // NaN is true, as in the reference (as_boolean: everything but 0)
+  }
+  return load_one<int64_t>(p, dt, i) != 0;
+}
+
+template <typename CT>
+__global__ void __launch_bounds__(BLOCK)
+select_nd_kernel(const void *__restrict__ p, const void *__restrict__ t, const void *__restrict__ f, void *__restrict__ out,
+                 int pdt, int tdt, int fdt, int odt, int64_t n, Sel s) {
+  for (int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x; i < n; i += (int64_t)gridDim.x * BLOCK) {
+    int64_t rem = i, po = 0, to = 0, fo = 0;
+    for (int a = s.rank - 1; a >= 0; a--) {
+      const int64_t q = rem / s.dims[a], c = rem - q * s.dims[a];
+      po += c * s.ps[a]; to += c * s.ts[a]; fo += c * s.fs[a];
+      rem = q;
+    }
+    const CT v = truthy<CT>(p, pdt, po) ? load_one<CT>(t, tdt, to) : load_one<CT>(f, fdt, fo);
+    store_one<CT>(out, odt, i, v);
+  }
+}
+
+// all three operands dense (step 1) or a single element (step 0)
+template <typename CT>
+__global__ void __launch_bounds__(BLOCK)
+select_vec_kernel(const void *__restrict__ p, const void *__restrict__ t, const void *__restrict__ f, void *__restrict__ out,
+                  int pdt, int tdt, int fdt, int odt, int64_t n, int pstep, int tstep, int fstep) {
+  const int64_t nvec = (n + E - 1) / E;
+  for (int64_t v = (int64_t)blockIdx.x * BLOCK + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * BLOCK) {
+    const int64_t i0 = v * E;
+    if (i0 + E <= n) {
+      CT a[E], b[E], c[E];
+      double pd[E];
+      int64_t pi[E];
+      const bool pf = pdt >= HIPNX_F16;
+      if (pstep) { if (pf) load_vec<double, E>(p, pdt, i0, pd); else load_vec<int64_t, E>(p, pdt, i0, pi); }
+      else {
+        const bool one = truthy<CT>(p, pdt, 0);
+#pragma unroll
+        for (int e = 0; e < E; e++) { pd[e] = one; pi[e] = one; }
+      }
+      if (tstep) load_vec<CT, E>(t, tdt, i0, a);
+      else { const CT x = load_one<CT>(t, tdt, 0);
+#pragma unroll
+        for (int e = 0; e < E; e++) a[e] = x; }
+      if (fstep) load_vec<CT, E>(f, fdt, i0, b);
+      else { const CT x = load_one<CT>(f, fdt, 0);
+#pragma unroll
+        for (int e = 0; e < E; e++) b[e] = x; }
+#pragma unroll
+      for (int e = 0; e < E; e++) c[e] = (pf ? pd[e] != 0 : pi[e] != 0) ? a[e] : b[e];
+      store_vec<CT, E>(out, odt, i0, c);
+    } else {
+      for (int64_t i = i0; i < n; i++) {
+        const CT x = truthy<CT>(p, pdt, i * pstep) ? load_one<CT>(t, tdt, i * tstep) : load_one<CT>(f, fdt, i * fstep);
+        store_one<CT>(out, odt, i, x);
+      }
+    }
+  }
+}
+
+// ---- clip -----------------------------------------------------------------------------------
+// c = x > min ? x : min;  out = c < max ? c : max  (so a NaN element becomes min, a NaN bound wins
+// the way the reference's comparisons make it: binary_backend.ex:1794-1806)
+// Integers are compared as the unbounded numbers the reference decodes them to: a value is the
+// 64 bits plus whether they came from a u64 (then a set top bit means 2^63 or more, above every
+// signed value).
+struct Wide {
+  int64_t bits;
+  bool uns;
+};
+__device__ inline bool wide_gt(Wide a, Wide b) {
+  const bool a_huge = a.uns && a.bits < 0, b_huge = b.uns && b.bits < 0;
+  if (a_huge || b_huge) return a_huge && (!b_huge || (uint64_t)a.bits > (uint64_t)b.bits);
+  return a.bits > b.bits;
+}
+template <typename CT>
+__device__ inline CT clip_one(CT x, CT lo, CT hi, bool xu, bool lou, bool hiu) {
+  if constexpr (std::is_same<CT, int64_t>::value) {
+    const Wide X{x, xu}, LO{lo, lou}, HI{hi, hiu};
+    const Wide c = wide_gt(X, LO) ? X : LO;
+    return wide_gt(HI, c) ? c.bits : HI.bits;
+  } else {
+    const CT c = x > lo ? x : lo;  // element_greater(x, min) == 1 ? x : min   (NaN compares false)
+    return c < hi ? c : hi;        // element_less(clipped, max) == 1 ? clipped : max
+  }
+}
+
+template <typename CT>
+__global__ void __launch_bounds__(BLOCK)
+clip_kernel(const void *__restrict__ in, const void *__restrict__ mn, const void *__restrict__ mx, void *__restrict__ out,
+            int idt, int mndt, int mxdt, int odt, int64_t n) {
+  const CT lo = load_one<CT>(mn, mndt, 0), hi = load_one<CT>(mx, mxdt, 0);
+  const bool xu = idt == HIPNX_U64, lou = mndt == HIPNX_U64, hiu = mxdt == HIPNX_U64;
+  const int64_t nvec = (n + E - 1) / E;
+  for (int64_t v = (int64_t)blockIdx.x * BLOCK + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * BLOCK) {
+    const int64_t i0 = v * E;
+    if (i0 + E <= n) {
+      CT x[E];
+      load_vec<CT, E>(in, idt, i0, x);
+#pragma unroll
+      for (int e = 0; e < E; e++) x[e] = clip_one<CT>(x[e], lo, hi, xu, lou, hiu);
+      store_vec<CT, E>(out, odt, i0, x);
+    } else {
+      for (int64_t i = i0; i < n; i++) store_one<CT>(out, odt, i, clip_one<CT>(load_one<CT>(in, idt, i), lo, hi, xu, lou, hiu));
+    }
+  }
+}
+
+// ---- strided copy: out[out_off + sum c_a * os_a] = in[in_off + sum c_a * is_a] -------------
+struct Copy {
+  int rank;
+  int64_t dims[MAXR], is[MAXR], os[MAXR];
+};
+
+template <typename T>
+__global__ void __launch_bounds__(BLOCK)
+copy_nd_kernel(const T *__restrict__ in, T *__restrict__ out, int64_t n, Copy c) {
+  for (int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x; i < n; i += (int64_t)gridDim.x * BLOCK) {
+    int64_t rem = i, io = 0, oo = 0;
+    for (int a = c.rank - 1; a >= 0; a--) {
+      const int64_t q = rem / c.dims[a], k = rem - q * c.dims[a];
+      io += k * c.is[a]; oo += k * c.os[a];
+      rem = q;
+    }
+    out[oo] = in[io];
+  }
+}
+
+// ---- iota / eye -----------------------------------------------------------------------------
+// mode 0: out[i] = (i / inner) % dim (iota along an axis; the flat iota is inner = 1, dim = n)
+// mode 1: out[i] = 1 where (i / inner) % dim == i % inner  (eye: dim = rows, inner = columns)
+template <typename CT>
+__global__ void __launch_bounds__(BLOCK)
+iota_kernel(void *__restrict__ out, int odt, int64_t n, int64_t dim, int64_t inner, int mode) {
+  const int64_t nvec = (n + E - 1) / E;
+  for (int64_t v = (int64_t)blockIdx.x * BLOCK + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * BLOCK) {
+    const int64_t i0 = v * E;
+    CT x[E];
+#pragma unroll
+    for (int e = 0; e < E; e++) {
+      const int64_t i = i0 + e, r = (i / inner) % dim;
+      x[e] = mode == 0 ? (CT)r : (CT)(r == i % inner ? 1 : 0);
+    }
+    if (i0 + E <= n) store_vec<CT, E>(out, odt, i0, x);
+    else
+      for (int e = 0; i0 + e < n; e++) store_one<CT>(out, odt, i0 + e, x[e]);
+  }
+}
+
+}  // namespace hipnx
+
+using namespace hipnx;
+
+extern "C" int hipnx_select(hipnx_ctx *ctx, int pred_dt, int true_dt, int false_dt, int out_dt, int rank,
+                            const int64_t *out_dims, const int64_t *pred_strides, const int64_t *true_strides,
+                            const int64_t *false_strides, const hipnx_buf *pred, const hipnx_buf *on_true,
+                            const hipnx_buf *on_false, hipnx_buf *out) {
+  Enter in(ctx);
+  if (in.status) return in.status;
+  if (dtype_size(pred_dt) < 0 || dtype_size(true_dt) < 0 || dtype_size(false_dt) < 0 || dtype_size(out_dt) < 0)
+    return set_error(HIPNX_EINVAL, "select: unknown element type");
+  if (rank < 0 || rank > 64 || (rank > 0 && (!out_dims || !pred_strides || !true_strides || !false_strides)))
+    return set_error(HIPNX_EINVAL, "select: bad rank");
+  if (!is_float(out_dt) && (is_float(true_dt) || is_float(false_dt)))
+    return set_error(HIPNX_EINVAL, "select: float operands with an integer output");
+  int64_t n = 1, pe = 1, te = 1, fe = 1;
+  for (int a = 0; a < rank; a++) {
+    if (out_dims[a] < 0 || pred_strides[a] < 0 || true_strides[a] < 0 || false_strides[a] < 0)
+      return set_error(HIPNX_EINVAL, "select: negative dimension or stride");
+    n *= out_dims[a];
+  }
+  if (n > 0)
+    for (int a = 0; a < rank; a++) {
+      pe += (out_dims[a] - 1) * pred_strides[a]; te += (out_dims[a] - 1) * true_strides[a]; fe += (out_dims[a] - 1) * false_strides[a];
+    }
+  if (int st = check_buf(ctx, pred, n > 0 ? (uint64_t)pe * dtype_size(pred_dt) : 0, "select pred")) return st;
+  if (int st = check_buf(ctx, on_true, n > 0 ? (uint64_t)te * dtype_size(true_dt) : 0, "select on_true")) return st;
+  if (int st = check_buf(ctx, on_false, n > 0 ? (uint64_t)fe * dtype_size(false_dt) : 0, "select on_false")) return st;
+  if (int st = check_buf(ctx, out, (uint64_t)n * dtype_size(out_dt), "select out")) return st;
+  if (n == 0) return HIPNX_OK;
+  // collapse: drop extent-1 axes, merge neighbours that are contiguous for all three operands
+  Sel s;
+  int m = 0;
+  for (int a = 0; a < rank; a++) {
+    const int64_t d = out_dims[a];
+    if (d == 1) continue;
+    if (m > 0 && s.ps[m - 1] == pred_strides[a] * d && s.ts[m - 1] == true_strides[a] * d && s.fs[m - 1] == false_strides[a] * d) {
+      s.dims[m - 1] *= d; s.ps[m - 1] = pred_strides[a]; s.ts[m - 1] = true_strides[a]; s.fs[m - 1] = false_strides[a];
+    } else {
+      if (m == MAXR) return set_error(HIPNX_EUNSUPPORTED, "select: more than %d non-collapsible axes", MAXR);
+      s.dims[m] = d; s.ps[m] = pred_strides[a]; s.ts[m] = true_strides[a]; s.fs[m] = false_strides[a]; m++;
+    }
+  }
+  if (m == 0) { s.dims[0] = 1; s.ps[0] = s.ts[0] = s.fs[0] = 0; m = 1; }
+  s.rank = m;
+  const bool fl = is_float(out_dt);
+  if (m == 1 && s.ps[0] <= 1 && s.ts[0] <= 1 && s.fs[0] <= 1) {
+    dim3 grid(grid_for((n + E - 1) / E)), block(BLOCK);
+    if (fl) hipLaunchKernelGGL((select_vec_kernel<double>), grid, block, 0, ctx->stream, pred->ptr, on_true->ptr, on_false->ptr, out->ptr,
+                               pred_dt, true_dt, false_dt, out_dt, n, (int)s.ps[0], (int)s.ts[0], (int)s.fs[0]);
+    else hipLaunchKernelGGL((select_vec_kernel<int64_t>), grid, block, 0, ctx->stream, pred->ptr, on_true->ptr, on_false->ptr, out->ptr,
+                            pred_dt, true_dt, false_dt, out_dt, n, (int)s.ps[0], (int)s.ts[0], (int)s.fs[0]);
+  } else {
+    dim3 grid(grid_for(n)), block(BLOCK);
+    if (fl) hipLaunchKernelGGL((select_nd_kernel<double>), grid, block, 0, ctx->stream, pred->ptr, on_true->ptr, on_false->ptr, out->ptr,
+                               pred_dt, true_dt, false_dt, out_dt, n, s);
+    else hipLaunchKernelGGL((select_nd_kernel<int64_t>), grid, block, 0, ctx->stream, pred->ptr, on_true->ptr, on_false->ptr, out->ptr,
+                            pred_dt, true_dt, false_dt, out_dt, n, s);
+  }
+  HIPNX_HIP(hipGetLastError());
+  return HIPNX_OK;
+}
+
+extern "C" int hipnx_clip(hipnx_ctx *ctx, int in_dt, int min_dt, int max_dt, int out_dt, int64_t n,
+                          const hipnx_buf *inb, const hipnx_buf *min, const hipnx_buf *max, hipnx_buf *out) {
+  Enter in(ctx);
+  if (in.status) return in.status;
+  if (dtype_size(in_dt) < 0 || dtype_size(min_dt) < 0 || dtype_size(max_dt) < 0 || dtype_size(out_dt) < 0)
+    return set_error(HIPNX_EINVAL, "clip: unknown element type");
+  if (n < 0) return set_error(HIPNX_EINVAL, "clip: negative size");
+  if (!is_float(out_dt) && (is_float(in_dt) || is_float(min_dt) || is_float(max_dt)))
+    return set_error(HIPNX_EINVAL, "clip: float operands with an integer output");
+  if (int st = check_buf(ctx, inb, (uint64_t)n * dtype_size(in_dt), "clip in")) return st;
+  if (int st = check_buf(ctx, min, dtype_size(min_dt), "clip min")) return st;
+  if (int st = check_buf(ctx, max, dtype_size(max_dt), "clip max")) return st;
+  if (int st = check_buf(ctx, out, (uint64_t)n * dtype_size(out_dt), "clip out")) return st;
+  if (n == 0) return HIPNX_OK;
+  dim3 grid(grid_for((n + E - 1) / E)), block(BLOCK);
+  if (is_float(out_dt))
+    hipLaunchKernelGGL((clip_kernel<double>), grid, block, 0, ctx->stream, inb->ptr, min->ptr, max->ptr, out->ptr, in_dt, min_dt, max_dt, out_dt, n);
+  else
+    hipLaunchKernelGGL((clip_kernel<int64_t>), grid, block, 0, ctx->stream, inb->ptr, min->ptr, max->ptr, out->ptr, in_dt, min_dt, max_dt, out_dt, n);
+  HIPNX_HIP(hipGetLastError());
+  return HIPNX_OK;
+}
+
+namespace {
+template <typename T>
+void launch_copy(const hipnx_ctx *ctx, const void *in, void *out, int64_t n, const Copy &c) {
+  hipLaunchKernelGGL((copy_nd_kernel<T>), dim3(grid_for(n)), dim3(BLOCK), 0, ctx->stream, (const T *)in, (T *)out, n, c);
+}
+}  // namespace
+
+extern "C" int hipnx_strided_copy(hipnx_ctx *ctx, int elem_bytes, int rank, const int64_t *dims,
+                                  const int64_t *in_strides, int64_t in_offset, const int64_t *out_strides,
+                                  int64_t out_offset, const hipnx_buf *inb, hipnx_buf *out) {
+  Enter in(ctx);
+  if (in.status) return in.status;
+  if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4 && elem_bytes != 8)
+    return set_error(HIPNX_EINVAL, "strided_copy: element size %d is not 1, 2, 4 or 8", elem_bytes);
+  if (rank < 0 || rank > 64 || (rank > 0 && (!dims || !in_strides || !out_strides))) return set_error(HIPNX_EINVAL, "strided_copy: bad rank");
+  if (in_offset < 0 || out_offset < 0) return set_error(HIPNX_EINVAL, "strided_copy: negative offset");
+  int64_t n = 1, ie = in_offset + 1, oe = out_offset + 1;
+  for (int a = 0; a < rank; a++) {
+    if (dims[a] < 0 || in_strides[a] < 0 || out_strides[a] < 0) return set_error(HIPNX_EINVAL, "strided_copy: negative dimension or stride");
+    n *= dims[a];
+  }
+  if (n > 0)
+    for (int a = 0; a < rank; a++) { ie += (dims[a] - 1) * in_strides[a]; oe += (dims[a] - 1) * out_strides[a]; }
+  if (int st = check_buf(ctx, inb, n > 0 ? (uint64_t)ie * elem_bytes : 0, "strided_copy in")) return st;
+  if (int st = check_buf(ctx, out, n > 0 ? (uint64_t)oe * elem_bytes : 0, "strided_copy out")) return st;
+  if (n == 0) return HIPNX_OK;
+  Copy c;
+  int m = 0;
+  for (int a = 0; a < rank; a++) {
+    const int64_t d = dims[a];
+    if (d == 1) continue;
+    if (m > 0 && c.is[m - 1] == in_strides[a] * d && c.os[m - 1] == out_strides[a] * d) {
+      c.dims[m - 1] *= d; c.is[m - 1] = in_strides[a]; c.os[m - 1] = out_strides[a];
+    } else {
+      if (m == MAXR) return set_error(HIPNX_EUNSUPPORTED, "strided_copy: more than %d non-collapsible axes", MAXR);
+      c.dims[m] = d; c.is[m] = in_strides[a]; c.os[m] = out_strides[a]; m++;
+    }
+  }
+  if (m == 0) { c.dims[0] = 1; c.is[0] = c.os[0] = 0; m = 1; }
+  c.rank = m;
+  // widen: when the innermost axis is dense on both sides and everything else sits on 16-byte
+  // boundaries, move 16 bytes per lane instead of one element
+  int eb = elem_bytes;
+  int64_t io = in_offset, oo = out_offset;
+  const int per = 16 / elem_bytes;
+  bool wide = c.is[m - 1] == 1 && c.os[m - 1] == 1 && c.dims[m - 1] % per == 0 && io % per == 0 && oo % per == 0 &&
+              ((uintptr_t)inb->ptr % 16 == 0) && ((uintptr_t)out->ptr % 16 == 0);
+  for (int a = 0; a + 1 < m && wide; a++) wide = c.is[a] % per == 0 && c.os[a] % per == 0;
+  if (wide && per > 1) {
+    c.dims[m - 1] /= per;
+    for (int a = 0; a + 1 < m; a++) { c.is[a] /= per; c.os[a] /= per; }
+    io /= per; oo /= per; n /= per; eb = 16;
+  }
+  const char *src = (const char *)inb->ptr + io * eb;
+  char *dst = (char *)out->ptr + oo * eb;
+  switch (eb) {
+    case 1: launch_copy<uint8_t>(ctx, src, dst, n, c); break;
+    case 2: launch_copy<uint16_t>(ctx, src, dst, n, c); break;
+    case 4: launch_copy<uint32_t>(ctx, src, dst, n, c); break;
+    case 8: launch_copy<uint64_t>(ctx, src, dst, n, c); break;
+    default: launch_copy<uint4>(ctx, src, dst, n, c); break;
+  }
+  HIPNX_HIP(hipGetLastError());
+  return HIPNX_OK;
+}
+
+static int iota_like(hipnx_ctx *ctx, int out_dt, int64_t n, int64_t dim, int64_t inner, int mode, hipnx_buf *out, const char *what) {
+  Enter in(ctx);
+  if (in.status) return in.status;
+  if (dtype_size(out_dt) < 0) return set_error(HIPNX_EINVAL, "%s: unknown element type", what);
+  if (n < 0 || dim < 1 || inner < 1) return set_error(HIPNX_EINVAL, "%s: bad extents", what);
+  if (int st = check_buf(ctx, out, (uint64_t)n * dtype_size(out_dt), what)) return st;
+  if (n == 0) return HIPNX_OK;
+  dim3 grid(grid_for((n + E - 1) / E)), block(BLOCK);
+  if (is_float(out_dt)) hipLaunchKernelGGL((iota_kernel<double>), grid, block, 0, ctx->stream, out->ptr, out_dt, n, dim, inner, mode);
+  else hipLaunchKernelGGL((iota_kernel<int64_t>), grid, block, 0, ctx->stream, out->ptr, out_dt, n, dim, inner, mode);
+  HIPNX_HIP(hipGetLastError());
+  return HIPNX_OK;
+}
+
+extern "C" int hipnx_iota(hipnx_ctx *ctx, int out_dt, int64_t n, int64_t dim, int64_t inner, hipnx_buf *out) {
+  return iota_like(ctx, out_dt, n, dim, inner, 0, out, "iota");
+}
+
+extern "C" int hipnx_eye(hipnx_ctx *ctx, int out_dt, int64_t n, int64_t rows, int64_t cols, hipnx_buf *out) {
+  return iota_like(ctx, out_dt, n, rows, cols, 1, out, "eye");
+}

@@ -265,6 +265,84 @@ static ERL_NIF_TERM nif_gather(ErlNifEnv *env, int argc, const ERL_NIF_TERM argv
   return ok(env, make_buf(env, out));
 }
 
+/* select(ctx, pred_dt, true_dt, false_dt, out_dt, out_dims, pred_strides, true_strides, false_strides, pred, on_true, on_false, out_bytes) */
+static ERL_NIF_TERM nif_select(ErlNifEnv *env, int argc, const ERL_NIF_TERM argv[]) {
+  (void)argc;
+  GET_CTX(0, ctx); GET_INT(1, pdt); GET_INT(2, tdt); GET_INT(3, fdt); GET_INT(4, odt);
+  int64_t dims[64], ps[64], ts[64], fs[64];
+  int rank, n1, n2, n3;
+  if (!get_i64_list(env, argv[5], dims, 64, &rank) || !get_i64_list(env, argv[6], ps, 64, &n1) ||
+      !get_i64_list(env, argv[7], ts, 64, &n2) || !get_i64_list(env, argv[8], fs, 64, &n3) || n1 != rank || n2 != rank ||
+      n3 != rank)
+    return enif_make_badarg(env);
+  GET_BUF(9, pred); GET_BUF(10, on_true); GET_BUF(11, on_false); GET_I64(12, out_bytes);
+  hipnx_buf *out;
+  CHECK(hipnx_buf_alloc(ctx, (size_t)out_bytes, &out));
+  int st = hipnx_select(ctx, pdt, tdt, fdt, odt, rank, dims, ps, ts, fs, pred, on_true, on_false, out);
+  if (st != HIPNX_OK) { hipnx_buf_destroy(out); return error_from_status(env, st); }
+  return ok(env, make_buf(env, out));
+}
+
+/* clip(ctx, in_dt, min_dt, max_dt, out_dt, n, in, min, max, out_bytes) */
+static ERL_NIF_TERM nif_clip(ErlNifEnv *env, int argc, const ERL_NIF_TERM argv[]) {
+  (void)argc;
+  GET_CTX(0, ctx); GET_INT(1, idt); GET_INT(2, mndt); GET_INT(3, mxdt); GET_INT(4, odt); GET_I64(5, n);
+  GET_BUF(6, in); GET_BUF(7, mn); GET_BUF(8, mx); GET_I64(9, out_bytes);
+  hipnx_buf *out;
+  CHECK(hipnx_buf_alloc(ctx, (size_t)out_bytes, &out));
+  int st = hipnx_clip(ctx, idt, mndt, mxdt, odt, n, in, mn, mx, out);
+  if (st != HIPNX_OK) { hipnx_buf_destroy(out); return error_from_status(env, st); }
+  return ok(env, make_buf(env, out));
+}
+
+/* strided_copy(ctx, elem_bytes, dims, in_strides, in_offset, out_strides, out_offset, in, out | out_bytes):
+ * the last argument is either a buffer to write into (a concatenation fills one output window
+ * by window; buffers are only ever written before they are published as a tensor) or the size
+ * of a fresh one */
+static ERL_NIF_TERM nif_strided_copy(ErlNifEnv *env, int argc, const ERL_NIF_TERM argv[]) {
+  (void)argc;
+  GET_CTX(0, ctx); GET_INT(1, esz);
+  int64_t dims[64], is[64], os[64];
+  int rank, n1, n2;
+  if (!get_i64_list(env, argv[2], dims, 64, &rank) || !get_i64_list(env, argv[3], is, 64, &n1) ||
+      !get_i64_list(env, argv[5], os, 64, &n2) || n1 != rank || n2 != rank)
+    return enif_make_badarg(env);
+  GET_I64(4, in_off); GET_I64(6, out_off); GET_BUF(7, in);
+  buf_res *dst;
+  if (enif_get_resource(env, argv[8], BUF_TYPE, (void **)&dst)) {
+    CHECK(hipnx_strided_copy(ctx, esz, rank, dims, is, in_off, os, out_off, in, dst->buf));
+    return ok(env, argv[8]);
+  }
+  GET_I64(8, out_bytes);
+  hipnx_buf *out;
+  CHECK(hipnx_buf_alloc(ctx, (size_t)out_bytes, &out));
+  int st = hipnx_strided_copy(ctx, esz, rank, dims, is, in_off, os, out_off, in, out);
+  if (st != HIPNX_OK) { hipnx_buf_destroy(out); return error_from_status(env, st); }
+  return ok(env, make_buf(env, out));
+}
+
+/* iota(ctx, out_dt, n, dim, inner, out_bytes) */
+static ERL_NIF_TERM nif_iota(ErlNifEnv *env, int argc, const ERL_NIF_TERM argv[]) {
+  (void)argc;
+  GET_CTX(0, ctx); GET_INT(1, odt); GET_I64(2, n); GET_I64(3, dim); GET_I64(4, inner); GET_I64(5, out_bytes);
+  hipnx_buf *out;
+  CHECK(hipnx_buf_alloc(ctx, (size_t)out_bytes, &out));
+  int st = hipnx_iota(ctx, odt, n, dim, inner, out);
+  if (st != HIPNX_OK) { hipnx_buf_destroy(out); return error_from_status(env, st); }
+  return ok(env, make_buf(env, out));
+}
+
+/* eye(ctx, out_dt, n, rows, cols, out_bytes) */
+static ERL_NIF_TERM nif_eye(ErlNifEnv *env, int argc, const ERL_NIF_TERM argv[]) {
+  (void)argc;
+  GET_CTX(0, ctx); GET_INT(1, odt); GET_I64(2, n); GET_I64(3, rows); GET_I64(4, cols); GET_I64(5, out_bytes);
+  hipnx_buf *out;
+  CHECK(hipnx_buf_alloc(ctx, (size_t)out_bytes, &out));
+  int st = hipnx_eye(ctx, odt, n, rows, cols, out);
+  if (st != HIPNX_OK) { hipnx_buf_destroy(out); return error_from_status(env, st); }
+  return ok(env, make_buf(env, out));
+}
+
 static ERL_NIF_TERM nif_sync(ErlNifEnv *env, int argc, const ERL_NIF_TERM argv[]) {
   (void)argc;
   GET_CTX(0, ctx);
@@ -289,6 +367,8 @@ static ErlNifFunc funcs[] = {
     {"reduce", 9, nif_reduce, IO},              {"argreduce", 10, nif_argreduce, IO},
     {"dot", 13, nif_dot, IO},                   {"transpose", 6, nif_transpose, IO},
     {"broadcast", 6, nif_broadcast, IO},        {"gather", 10, nif_gather, IO},
-    {"sync", 1, nif_sync, IO}};
+    {"select", 13, nif_select, IO},             {"clip", 10, nif_clip, IO},
+    {"strided_copy", 9, nif_strided_copy, IO},  {"iota", 6, nif_iota, IO},
+    {"eye", 6, nif_eye, IO},                    {"sync", 1, nif_sync, IO}};
 
 ERL_NIF_INIT(Elixir.HipNx.NIF, funcs, on_load, NULL, NULL, NULL)

@@ -216,6 +216,10 @@ defmodule HipNx.Backend do
   def reduce_min(out, t, opts), do: reduce_op(2, out, t, opts)
   @impl true
   def product(out, t, opts), do: reduce_op(3, out, t, opts)
+  @impl true
+  def all(out, t, opts), do: reduce_op(4, out, t, opts)
+  @impl true
+  def any(out, t, opts), do: reduce_op(5, out, t, opts)
 
   defp reduce_op(code, out, %T{} = t, opts) do
     device = device_of([t])
@@ -360,6 +364,114 @@ defmodule HipNx.Backend do
   end
 
   def block(struct, _out, args, fun), do: apply(fun, [struct | args])
+
+  ## Selection, windows and creation
+
+  @impl true
+  def select(%T{shape: shape} = out, %T{} = pred, %T{} = on_true, %T{} = on_false) do
+    device = device_of([pred, on_true, on_false])
+    {pref, _} = from_nx(pred, device)
+    {tref, _} = from_nx(on_true, device)
+    {fref, _} = from_nx(on_false, device)
+
+    ref =
+      NIF.select(ctx(device), dt(pred.type), dt(on_true.type), dt(on_false.type), dt(out.type), Tuple.to_list(shape),
+        broadcast_strides(pred.shape, shape), broadcast_strides(on_true.shape, shape),
+        broadcast_strides(on_false.shape, shape), pref, tref, fref, bytes(out))
+
+    to_nx(unwrap!(ref), device, out)
+  end
+
+  @impl true
+  def clip(out, %T{} = t, %T{} = min, %T{} = max) do
+    device = device_of([t, min, max])
+    {ref, _} = from_nx(t, device)
+    {mn, _} = from_nx(min, device)
+    {mx, _} = from_nx(max, device)
+
+    to_nx(unwrap!(NIF.clip(ctx(device), dt(t.type), dt(min.type), dt(max.type), dt(out.type), Nx.size(out), ref, mn, mx,
+      bytes(out))), device, out)
+  end
+
+  @impl true
+  def slice(%T{shape: out_shape, type: {_, bits}} = out, %T{shape: shape} = t, start_indices, lengths, strides) do
+    device = device_of([t])
+    {ref, _} = from_nx(t, device)
+    dense = dense_strides(shape)
+
+    # dynamic starts are read back and clamped as binary_backend.ex:1813-1863 does
+    starts =
+      [start_indices, Tuple.to_list(shape), lengths]
+      |> Enum.zip_with(fn [idx, dim, len] ->
+        idx = if is_struct(idx, T), do: Nx.to_number(idx), else: idx
+        idx |> max(0) |> min(dim - len)
+      end)
+
+    offset = Enum.zip_with(starts, dense, &(&1 * &2)) |> Enum.sum()
+    in_strides = Enum.zip_with(strides, dense, &(&1 * &2))
+
+    ref =
+      NIF.strided_copy(ctx(device), div(bits, 8), Tuple.to_list(out_shape), in_strides, offset, dense_strides(out_shape), 0,
+        ref, bytes(out))
+
+    to_nx(unwrap!(ref), device, out)
+  end
+
+  @impl true
+  def concatenate(%T{shape: out_shape, type: {_, bits} = type} = out, tensors, axis) do
+    device = device_of(tensors)
+    out_strides = dense_strides(out_shape)
+    step = Enum.at(out_strides, axis)
+    buf = unwrap!(NIF.alloc(ctx(device), bytes(out)))
+
+    Enum.reduce(tensors, 0, fn %T{shape: shape} = t, at ->
+      t = if t.type == type, do: t, else: as_type(%{t | type: type}, t)
+      {ref, _} = from_nx(t, device)
+
+      unwrap!(
+        NIF.strided_copy(ctx(device), div(bits, 8), Tuple.to_list(shape), dense_strides(shape), 0, out_strides, at * step,
+          ref, buf)
+      )
+
+      at + elem(shape, axis)
+    end)
+
+    to_nx(buf, device, out)
+  end
+
+  @impl true
+  def stack(out, tensors, axis) do
+    widened = Enum.map(tensors, fn %T{shape: shape, names: names} = t ->
+      %{t | shape: Tuple.insert_at(shape, axis, 1), names: List.insert_at(names, axis, nil)}
+    end)
+
+    concatenate(out, widened, axis)
+  end
+
+  @impl true
+  def iota(%T{shape: shape} = out, axis, opts) do
+    device = opts[:device] || 0
+    n = Nx.size(shape)
+
+    {dim, inner} =
+      if axis, do: {elem(shape, axis), shape |> Tuple.to_list() |> Enum.drop(axis + 1) |> prod()}, else: {max(n, 1), 1}
+
+    to_nx(unwrap!(NIF.iota(ctx(device), dt(out.type), n, dim, inner, bytes(out))), device, out)
+  end
+
+  @impl true
+  def eye(%T{shape: shape} = out, opts) do
+    device = opts[:device] || 0
+    rank = tuple_size(shape)
+
+    to_nx(unwrap!(NIF.eye(ctx(device), dt(out.type), Nx.size(shape), elem(shape, rank - 2), elem(shape, rank - 1),
+      bytes(out))), device, out)
+  end
+
+  defp dense_strides(shape) do
+    {strides, _} = shape |> Tuple.to_list() |> Enum.reverse() |> Enum.map_reduce(1, fn dim, acc -> {acc, acc * dim} end)
+    Enum.reverse(strides)
+  end
 
   ## Everything else: round trip through Nx.BinaryBackend
 

@@ -24,6 +24,11 @@ defmodule HipNx.NIF do
   def transpose(_ctx, _elem_bytes, _dims, _perm, _in, _out_bytes), do: err()
   def broadcast(_ctx, _elem_bytes, _dims, _strides, _in, _out_bytes), do: err()
   def gather(_ctx, _elem_bytes, _dims, _idx_dt, _n_tuples, _depth, _policy, _t, _idx, _out_bytes), do: err()
+  def select(_ctx, _p_dt, _t_dt, _f_dt, _out_dt, _dims, _p_strides, _t_strides, _f_strides, _p, _t, _f, _out_bytes), do: err()
+  def clip(_ctx, _in_dt, _min_dt, _max_dt, _out_dt, _n, _in, _min, _max, _out_bytes), do: err()
+  def strided_copy(_ctx, _elem_bytes, _dims, _in_strides, _in_offset, _out_strides, _out_offset, _in, _out_or_bytes), do: err()
+  def iota(_ctx, _out_dt, _n, _dim, _inner, _out_bytes), do: err()
+  def eye(_ctx, _out_dt, _n, _rows, _cols, _out_bytes), do: err()
   def sync(_ctx), do: err()
 
   defp err, do: :erlang.nif_error(:undef)

@@ -425,3 +425,131 @@ def take(t, indices, axis=0):
         return transpose(gather(tensor_, gather_indices, axes=[axis]), leading + indices_axes + trailing)
 
     return block(BlockTake(axis), [t, indices], out, default)
+
+
+# ---- one step off the hot path: creation, selection, windows (SURVEY "next" rows) --------------
+
+def all(t, axes=None, keep_axes=False):  # noqa: A001 - Nx.all/2 (nx.ex:9207-9209): u8 output
+    return _aggregate(to_tensor(t), "all", ("u", 8), axes, keep_axes)
+
+
+def any(t, axes=None, keep_axes=False):  # noqa: A001 - Nx.any/2 (nx.ex:9272-9274)
+    return _aggregate(to_tensor(t), "any", ("u", 8), axes, keep_axes)
+
+
+def iota(shape, type="s32", axis=None, backend=None):
+    """Nx.iota/2 (nx.ex:1213-1260): counts along `axis`, or over the flattened tensor."""
+    shape = tuple(shape)
+    mod, opts = (backend, {}) if backend is not None and not isinstance(backend, tuple) else (backend or default_backend())
+    if axis is not None:
+        axis = S.normalize_axis(shape, axis)
+    return mod.iota(template(type, shape), axis, opts)
+
+
+def eye(n_or_shape, type="s32", backend=None):
+    """Nx.eye/2 (nx.ex:1363-1420): identity matrices in the last two axes."""
+    shape = (n_or_shape, n_or_shape) if isinstance(n_or_shape, int) else tuple(n_or_shape)
+    if len(shape) < 2:
+        raise ValueError(f"eye/2 expects a shape with at least 2 dimensions or an integer, got: {shape!r}")
+    mod, opts = (backend, {}) if backend is not None and not isinstance(backend, tuple) else (backend or default_backend())
+    return mod.eye(template(type, shape), opts)
+
+
+def select(pred, on_true, on_false):
+    """Nx.select/3 (nx.ex:7782-7830): the output takes the predicate's shape unless the predicate
+    is a scalar, and the merged type of the two value operands."""
+    pred, on_true, on_false = to_tensor(pred), to_tensor(on_true), to_tensor(on_false)
+    out_type = T.binary_type(on_true.type, on_false.type)
+    out_shape = S.binary_broadcast(on_true.shape, on_false.shape) if pred.shape == () else pred.shape
+    for operand in (on_true, on_false):
+        S.broadcast(operand.shape, out_shape, S.broadcast_axes(operand.shape, out_shape))
+    return _impl(pred, on_true, on_false).select(template(out_type, out_shape), pred, on_true, on_false)
+
+
+def clip(t, min, max):  # noqa: A002 - Nx.clip/3 (nx.ex:13973-14000)
+    t, min, max = to_tensor(t), to_tensor(min), to_tensor(max)
+    if min.shape != ():
+        raise ValueError(f"min value must be a non-vectorized scalar shape, got shape {min.shape!r}")
+    if max.shape != ():
+        raise ValueError(f"max value must be a non-vectorized scalar shape, got shape {max.shape!r}")
+    out_type = T.merge(t.type, T.merge(min.type, max.type))
+    return _impl(t, min, max).clip(t.with_(data=None, type=out_type), t, min, max)
+
+
+def slice(t, start_indices, lengths, strides=1):  # noqa: A001 - Nx.slice/4 (nx.ex:14203-14290)
+    t = to_tensor(t)
+    start_indices, lengths = list(start_indices), list(lengths)
+    if t.shape == () and not start_indices and not lengths:
+        return t
+    rank = len(t.shape)
+    strides = [strides] * rank if isinstance(strides, int) else list(strides)
+    if len(strides) != rank:
+        raise ValueError(f"invalid strides rank for shape of rank {rank}")
+    if len(start_indices) != rank:
+        raise ValueError(f"invalid start indices rank for shape of rank {rank}")
+    if len(lengths) != rank:
+        raise ValueError(f"invalid limit indices rank for shape of rank {rank}")
+    out_shape, starts = [], []
+    for pos, (i, length, s) in enumerate(zip(start_indices, lengths, strides)):  # Nx.Shape.slice (shape.ex:1110-1164)
+        dim = t.shape[pos]
+        if not isinstance(length, int) or length < 1:
+            raise ValueError(f"length at axis {pos} must be greater than or equal to 1, got: {length!r}")
+        if not isinstance(s, int) or s < 1:
+            raise ValueError(f"stride at axis {pos} must be greater than or equal to 1, got: {s!r}")
+        if length > dim:
+            raise ValueError(f"length at axis {pos} must be less than axis size of {dim}, got: {length}")
+        out_shape.append(-(-length // s))
+        starts.append(builtins.min(i, dim - length) if isinstance(i, int) else i)
+    return _impl(t).slice(t.with_(data=None, shape=tuple(out_shape)), t, starts, lengths, strides)
+
+
+def slice_along_axis(t, start_index, length, axis=0, strides=1):
+    """Nx.slice_along_axis/4 (nx.ex:14391-14420)."""
+    t = to_tensor(t)
+    axis = S.normalize_axis(t.shape, axis)
+    rank = len(t.shape)
+    starts = [0] * rank
+    lengths = list(t.shape)
+    steps = [1] * rank
+    starts[axis], lengths[axis], steps[axis] = start_index, length, strides
+    return slice(t, starts, lengths, steps)
+
+
+def _concat_type_and_operands(tensors):
+    tensors = [to_tensor(t) for t in tensors]
+    if not tensors:
+        raise ValueError("no tensors were given to concatenate")
+    out_type = tensors[0].type
+    for t in tensors[1:]:
+        out_type = T.merge(out_type, t.type)
+    return out_type, tensors
+
+
+def concatenate(tensors, axis=0):
+    """Nx.concatenate/2 (nx.ex:15343-15362; Nx.Shape.concatenate shape.ex:1713-1760)."""
+    out_type, tensors = _concat_type_and_operands(tensors)
+    if len(tensors) == 1:
+        return tensors[0]
+    first = tensors[0].shape
+    axis = S.normalize_axis(first, axis)
+    total = 0
+    for t in tensors:
+        if len(t.shape) != len(first) or builtins.any(a != b for pos, (a, b) in enumerate(zip(t.shape, first)) if pos != axis):
+            raise ValueError("expected all shapes to match " + repr(first) + ", except for the axis of concatenation, got "
+                             "unmatching shape: " + repr(t.shape))
+        total += t.shape[axis]
+    out_shape = first[:axis] + (total,) + first[axis + 1:]
+    return _impl(*tensors).concatenate(template(out_type, out_shape), tensors, axis)
+
+
+def stack(tensors, axis=0):
+    """Nx.stack/2 (nx.ex:15502-15520; Nx.Shape.stack shape.ex:1689-1711): a new axis of the
+    operands' count at `axis`."""
+    out_type, tensors = _concat_type_and_operands(tensors)
+    first = tensors[0].shape
+    for t in tensors:
+        if t.shape != first:
+            raise ValueError(f"can only stack tensors of the same shape, got shapes {first!r} and {t.shape!r}")
+    axis = S.normalize_axis(first + (1,), axis)
+    out_shape = first[:axis] + (len(tensors),) + first[axis:]
+    return _impl(*tensors).stack(template(out_type, out_shape), tensors, axis)

@@ -308,6 +308,119 @@ class BinaryBackend:
         return res
 
 
+    # -- one step off the hot path ---------------------------------------------------------------
+    # numpy restatements of byte-level / integer rules; encodings go through ref_as_type so that
+    # every number reaches its binary the way number_to_binary writes it.
+    @classmethod
+    def _typed(cls, t):
+        """The tensor's elements as a numpy array of its storage type (bf16: raw uint16)."""
+        return np.frombuffer(bytes(cls._bin(t)), dtype=T.numpy_dtype(t.type)).reshape(t.shape)
+
+    @classmethod
+    def _from_array(cls, out, arr, src_type):
+        """Encodes `arr` (s64 / f64 numbers) into out.type as the reference's write path does."""
+        src = out.with_(data=cls(bytearray(np.ascontiguousarray(arr).tobytes())), type=T.normalize(src_type))
+        return cls.as_type(out, src) if src.type != out.type else src
+
+    @classmethod
+    def _numbers(cls, t):
+        """Decoded values: float64 for float types (bf16 widened), uint64 for u64, int64 otherwise."""
+        a = cls._typed(t)
+        if t.type == ("bf", 16):
+            return (a.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+        if t.type == ("u", 64):
+            return a
+        return a.astype(np.float64) if T.is_float(t.type) else a.astype(np.int64)
+
+    @classmethod
+    def iota(cls, out, axis, opts=None):  # binary_backend.ex:49-87
+        n = out.size
+        if axis is None:
+            idx = np.arange(n, dtype=np.int64)
+        else:
+            inner = prod(out.shape[axis + 1:])
+            idx = (np.arange(n, dtype=np.int64) // inner) % out.shape[axis]
+        return cls._from_array(out, idx, "s64")
+
+    @classmethod
+    def eye(cls, out, opts=None):  # binary_backend.ex:90-110
+        m, n = out.shape[-2], out.shape[-1]
+        one = np.eye(m, n, dtype=np.int64)
+        return cls._from_array(out, np.broadcast_to(one, out.shape), "s64")
+
+    @classmethod
+    def select(cls, out, pred, on_true, on_false):  # binary_backend.ex:604-648
+        truth = cls._numbers(pred) != 0  # as_boolean: everything but 0, NaN included
+        truth = np.broadcast_to(truth, out.shape)
+        sides = []
+        for side in (on_true, on_false):
+            full = cls.broadcast(side.with_(data=None, shape=out.shape), side, out.shape,
+                                 S.broadcast_axes(side.shape, out.shape)) if side.shape != out.shape else side
+            full = cls.as_type(full.with_(data=None, type=out.type), full)
+            sides.append(cls._typed(full))
+        buf, res = cls._new(out)
+        buf[:] = np.where(truth, sides[0], sides[1]).astype(sides[0].dtype).tobytes()
+        return res
+
+    @classmethod
+    def clip(cls, out, t, min_t, max_t):  # binary_backend.ex:1788-1811
+        x, lo, hi = cls._numbers(t), cls._numbers(min_t).reshape(()), cls._numbers(max_t).reshape(())
+        if T.is_float(out.type):
+            x, lo, hi = x.astype(np.float64), np.float64(lo), np.float64(hi)
+        elif np.uint64 in (x.dtype, lo.dtype, hi.dtype):  # unbounded integers, as the reference's numbers are
+            x, lo, hi = x.astype(object), int(lo), int(hi)
+            c = np.where(x > lo, x, lo)
+            r = np.where(c < hi, c, hi)
+            wrapped = np.array([int(v) & 0xFFFFFFFFFFFFFFFF for v in r.reshape(-1)], dtype=np.uint64).reshape(r.shape)
+            return cls._from_array(out, wrapped, "u64")
+        with np.errstate(invalid="ignore"):
+            c = np.where(x > lo, x, lo)      # element_greater(x, min) == 1 ? x : min
+            r = np.where(c < hi, c, hi)      # element_less(clipped, max) == 1 ? clipped : max
+        return cls._from_array(out, r, "f64" if T.is_float(out.type) else "s64")
+
+    @classmethod
+    def slice(cls, out, t, start_indices, lengths, strides):  # binary_backend.ex:1813-1863
+        a = cls._typed(t)
+        window = []
+        for dim, idx, length, step in zip(t.shape, start_indices, lengths, strides):
+            if isinstance(idx, Tensor):
+                idx = int(cls._numbers(idx).reshape(()))
+            start = min(max(int(idx), 0), dim - length)  # clamp_indices
+            window.append(np.s_[start:start + length:step])
+        buf, res = cls._new(out)
+        buf[:] = np.ascontiguousarray(a[tuple(window)]).tobytes()
+        return res
+
+    @classmethod
+    def concatenate(cls, out, tensors, axis):  # binary_backend.ex:1975-1986
+        parts = [cls._typed(cls.as_type(t.with_(data=None, type=out.type), t)) for t in tensors]
+        buf, res = cls._new(out)
+        buf[:] = np.concatenate(parts, axis=axis).tobytes()
+        return res
+
+    @classmethod
+    def stack(cls, out, tensors, axis):  # binary_backend.ex:1962-1972
+        parts = [cls._typed(cls.as_type(t.with_(data=None, type=out.type), t)) for t in tensors]
+        buf, res = cls._new(out)
+        buf[:] = np.stack(parts, axis=axis).tobytes()
+        return res
+
+    @classmethod
+    def _truth_reduce(cls, fn, out, t, opts):  # binary_backend.ex:1293-1314
+        axes = opts.get("axes")
+        truth = cls._numbers(t) != 0
+        r = fn(truth, axis=tuple(axes) if axes is not None else None)
+        return cls._from_array(out, np.asarray(r).astype(np.int64).reshape(out.shape), "s64")
+
+    @classmethod
+    def all(cls, out, t, opts):
+        return cls._truth_reduce(np.all, out, t, opts)
+
+    @classmethod
+    def any(cls, out, t, opts):
+        return cls._truth_reduce(np.any, out, t, opts)
+
+
 def _install():
     for code, name in enumerate(BINARY_OPS):
         setattr(BinaryBackend, name, classmethod(lambda cls, out, l, r, _c=code: cls._binary(_c, out, l, r)))

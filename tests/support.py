@@ -56,12 +56,20 @@ def spec_to_tensor(spec, backend):
 def from_numpy(arr, ty, backend):
     """Raw element array (bf16 as uint16 bits) -> tensor on `backend`."""
     ty = T.normalize(ty)
+    shape = np.shape(arr)  # ascontiguousarray turns a rank-0 array into {1}
     arr = np.ascontiguousarray(arr, dtype=T.numpy_dtype(ty))
-    return backend.from_binary(template(ty, arr.shape), arr.tobytes(), {})
+    return backend.from_binary(template(ty, shape), arr.tobytes(), {})
 
 
 def run_case(case, backend):
     op, opts = case["op"], dict(case.get("opts", {}))
+    if op in ("iota", "eye"):  # creation: the shape is a plain list, the backend is an option
+        return getattr(Nx, op)(case["args"][0], backend=backend, **opts)
+    if op in ("concatenate", "stack"):  # a list of operands
+        return getattr(Nx, op)([spec_to_tensor(a, backend) for a in case["args"][0]], **opts)
+    if op == "slice":  # start indices may be rank-0 tensors
+        t, starts, lengths = case["args"]
+        return Nx.slice(spec_to_tensor(t, backend), [spec_to_tensor(i, backend) for i in starts], lengths, **opts)
     args = [spec_to_tensor(a, backend) for a in case["args"]]
     if op in ("dot", "dot4", "dot6"):
         return Nx.dot(*args)
