@@ -205,6 +205,27 @@ def main():
         _, ms = timed(lambda: Nx.take(table, idx), steps, warm)
         entry("take_bf16_8192_of_32000x4096", 134250496.0, "GB/s", ms, PEAK_HBM_GBS, "hbm")
         del logits, table, idx
+
+        # selection, windows and creation at the HBM-resident size of config 1
+        nn = 16384
+        N = nn * nn
+        x, y = W.elementwise_reduce(n=nn)
+        x, y = put(x, "f32"), put(y, "f32")
+        pred = Nx.greater(x, y)
+        _, ms = timed(lambda: Nx.select(pred, x, y), steps, warm)
+        entry(f"select_f32_{nn}", 13.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+        _, ms = timed(lambda: Nx.clip(x, -0.5, 0.5), steps, warm)
+        entry(f"clip_f32_{nn}", 8.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+        _, ms = timed(lambda: Nx.slice(x, [64, 128], [nn - 128, nn - 256]), steps, warm)
+        entry(f"slice_f32_{nn}", 8.0 * (nn - 128) * (nn - 256), "GB/s", ms, PEAK_HBM_GBS, "hbm")
+        del pred
+        _, ms = timed(lambda: Nx.concatenate([x, y], axis=1), steps, warm)
+        entry(f"concatenate_axis1_f32_{nn}", 16.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+        _, ms = timed(lambda: Nx.all(x, axes=[1]), steps, warm)
+        entry(f"all_rows_f32_{nn}", 4.0 * N + nn, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+        _, ms = timed(lambda: Nx.iota((nn, nn), type="f32", axis=1, backend=H), steps, warm)
+        entry(f"iota_f32_{nn}", 4.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+        del x, y
         result["suite"] = suite
 
     # ---- CPU baseline: the reference-semantics restatement on a bounded sample -----------------

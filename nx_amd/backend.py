@@ -31,7 +31,7 @@ K_INNER, K_OUTER = 0, 1
 OOB_RAISE, OOB_CLAMP = 0, 1
 
 # callbacks of the behaviour that are not on the device path (nx/lib/nx/backend.ex:58-144)
-UNSUPPORTED = ["to_batched", "from_pointer", "to_pointer", "put_slice", "pad", "reverse",
+UNSUPPORTED = ["to_batched", "from_pointer", "to_pointer", "put_slice", "reverse",
                "conv", "window_sum", "window_product",
                "window_max", "window_min", "reduce", "window_reduce", "window_scatter_max", "window_scatter_min",
                "indexed_add", "indexed_put", "sort", "argsort", "fft", "ifft", "fft2", "ifft2", "triangular_solve",
@@ -409,7 +409,7 @@ class HipNxBackend:
     # ---- data movement ---------------------------------------------------------------------
     @classmethod
     def transpose(cls, out: Tensor, t: Tensor, axes) -> Tensor:
-        """transpose/3 (backend.ex:74; oracle binary_backend.ex:280-306)."""
+        """transpose/3 (backend.ex:73; oracle binary_backend.ex:280-306)."""
         dev = cls._device_of(t)
         t = cls._from_nx(t, dev)
         res = cls._alloc(out, dev)
@@ -419,7 +419,7 @@ class HipNxBackend:
 
     @classmethod
     def broadcast(cls, out: Tensor, t: Tensor, shape, axes) -> Tensor:
-        """broadcast/4 (backend.ex:75; oracle binary_backend.ex:215-276): input axis i maps to
+        """broadcast/4 (backend.ex:72; oracle binary_backend.ex:215-276): input axis i maps to
         output axis axes[i]; size-1 input axes and unmapped output axes repeat."""
         dev = cls._device_of(t)
         t = cls._from_nx(t, dev)
@@ -526,6 +526,45 @@ class HipNxBackend:
             res.data.ref.ctx, T.size_bytes(t.type), len(out.shape), L.i64_array(out.shape),
             L.i64_array([d * s for d, s in zip(dense, strides)]), sum(d * s for d, s in zip(dense, starts)),
             L.i64_array(cls._dense_strides(out.shape)), 0, cls._handle(t), res.data.ref.handle))
+        return res
+
+    @classmethod
+    def pad(cls, out: Tensor, t: Tensor, pad_value: Tensor, padding_config) -> Tensor:
+        """pad/4 (backend.ex:74; oracle binary_backend.ex:326-431): interior padding first, then the
+        edges, where a negative edge cuts into the interior-padded axis.  Element i of an axis lands
+        at low + i * (interior + 1); the ones that land inside the output are one strided copy into
+        a buffer filled with the pad value.  Operands are converted to out.type first (the oracle
+        splices the two encodings when they differ; EXLA and Torchx convert)."""
+        if t.shape == ():
+            return t  # as the oracle does, whatever out.type says
+        dev = cls._device_of(t, pad_value)
+        t, pad_value = cls._from_nx(t, dev), cls._from_nx(pad_value, dev)
+        if any(d < 0 for d in out.shape):
+            raise ValueError(f"padding configuration crops more than the tensor holds: output shape {out.shape!r}")
+        if t.type != out.type:
+            t = cls.as_type(t.with_(data=None, type=out.type), t)
+        if pad_value.type != out.type:
+            pad_value = cls.as_type(pad_value.with_(data=None, type=out.type), pad_value)
+        res = cls._alloc(out, dev)
+        rank = len(out.shape)
+        ctx, esz = res.data.ref.ctx, T.size_bytes(out.type)
+        L.check(L.lib.hipnx_broadcast(ctx, esz, rank, L.i64_array(out.shape), L.i64_array([0] * rank),
+                                      cls._handle(pad_value), res.data.ref.handle))
+        counts, first = [], []
+        for dim, odim, (low, _high, interior) in zip(t.shape, out.shape, padding_config):
+            step = interior + 1
+            lo = -(min(low, 0) // step)                      # first i with low + i * step >= 0
+            hi = min(dim - 1, (odim - 1 - low) // step) if odim > 0 else -1
+            counts.append(max(hi - lo + 1, 0))
+            first.append(lo)
+        if all(counts):
+            dense_in, dense_out = cls._dense_strides(t.shape), cls._dense_strides(out.shape)
+            steps = [c[2] + 1 for c in padding_config]
+            L.check(L.lib.hipnx_strided_copy(
+                ctx, esz, rank, L.i64_array(counts), L.i64_array(dense_in), sum(f * d for f, d in zip(first, dense_in)),
+                L.i64_array([s * d for s, d in zip(steps, dense_out)]),
+                sum((c[0] + f * s) * d for c, f, s, d in zip(padding_config, first, steps, dense_out)),
+                cls._handle(t), res.data.ref.handle))
         return res
 
     @classmethod

@@ -418,6 +418,41 @@ defmodule HipNx.Backend do
   end
 
   @impl true
+  def pad(_out, %T{shape: {}} = t, _pad_value, _config), do: t
+
+  def pad(%T{shape: out_shape, type: {_, bits} = type} = out, %T{shape: shape} = t, %T{} = pad_value, config) do
+    device = device_of([t, pad_value])
+    t = if t.type == type, do: t, else: as_type(%{t | type: type}, t)
+    pad_value = if pad_value.type == type, do: pad_value, else: as_type(%{pad_value | type: type}, pad_value)
+    {ref, _} = from_nx(t, device)
+    {vref, _} = from_nx(pad_value, device)
+    out_dims = Tuple.to_list(out_shape)
+    filled = unwrap!(NIF.broadcast(ctx(device), div(bits, 8), out_dims, List.duplicate(0, length(out_dims)), vref, bytes(out)))
+
+    # element i of an axis lands at low + i * (interior + 1); keep the ones that land inside
+    ranges =
+      [Tuple.to_list(shape), out_dims, config]
+      |> Enum.zip_with(fn [dim, odim, {low, _high, interior}] ->
+        step = interior + 1
+        lo = -Integer.floor_div(min(low, 0), step)
+        hi = if odim > 0, do: min(dim - 1, Integer.floor_div(odim - 1 - low, step)), else: -1
+        {lo, max(hi - lo + 1, 0), step, low}
+      end)
+
+    if Enum.all?(ranges, fn {_, count, _, _} -> count > 0 end) do
+      dense_in = dense_strides(shape)
+      dense_out = dense_strides(out_shape)
+      in_offset = Enum.zip_with(ranges, dense_in, fn {lo, _, _, _}, d -> lo * d end) |> Enum.sum()
+      out_offset = Enum.zip_with(ranges, dense_out, fn {lo, _, step, low}, d -> (low + lo * step) * d end) |> Enum.sum()
+      out_strides = Enum.zip_with(ranges, dense_out, fn {_, _, step, _}, d -> step * d end)
+      counts = Enum.map(ranges, &elem(&1, 1))
+      unwrap!(NIF.strided_copy(ctx(device), div(bits, 8), counts, dense_in, in_offset, out_strides, out_offset, ref, filled))
+    end
+
+    to_nx(filled, device, out)
+  end
+
+  @impl true
   def concatenate(%T{shape: out_shape, type: {_, bits} = type} = out, tensors, axis) do
     device = device_of(tensors)
     out_strides = dense_strides(out_shape)

@@ -476,6 +476,24 @@ def clip(t, min, max):  # noqa: A002 - Nx.clip/3 (nx.ex:13973-14000)
     return _impl(t, min, max).clip(t.with_(data=None, type=out_type), t, min, max)
 
 
+def pad(t, pad_value, padding_config):
+    """Nx.pad/3 (nx.ex:4233-4250; shape rule shape.ex:1038-1071): (low, high, interior) per axis;
+    negative edges crop, interior padding must be non-negative."""
+    t, pad_value = to_tensor(t), to_tensor(pad_value)
+    out_type = T.binary_type(t.type, pad_value.type)
+    if pad_value.shape != ():
+        raise ValueError("padding value must be a scalar and non-vectorized")
+    padding_config = [tuple(c) for c in padding_config]
+    if len(padding_config) != len(t.shape):
+        raise ValueError("invalid padding configuration, rank of padding configuration and shape must match")
+    dims = []
+    for dim, (low, high, interior) in zip(t.shape, padding_config):
+        if interior < 0:
+            raise ValueError("invalid padding configuration, interior padding must be non-negative")
+        dims.append(dim + (dim - 1) * interior + low + high)
+    return _impl(t, pad_value).pad(template(out_type, tuple(dims)), t, pad_value, padding_config)
+
+
 def slice(t, start_indices, lengths, strides=1):  # noqa: A001 - Nx.slice/4 (nx.ex:14203-14290)
     t = to_tensor(t)
     start_indices, lengths = list(start_indices), list(lengths)

@@ -379,6 +379,37 @@ class BinaryBackend:
         return cls._from_array(out, r, "f64" if T.is_float(out.type) else "s64")
 
     @classmethod
+    def pad(cls, out, t, pad_value, padding_config):  # binary_backend.ex:326-431
+        if t.shape == ():
+            return t  # the reference hands the scalar back untouched, whatever out.type says
+        if t.type != out.type:
+            # the reference splices pad bytes of out.type into the binary of t and labels the result
+            # with t's type (binary_backend.ex:327,352,418): not a behaviour to restate
+            raise NotImplementedError("pad: the reference mixes two encodings when the types differ")
+        value = cls._typed(cls.as_type(pad_value.with_(data=None, type=out.type), pad_value)).reshape(())
+        a = cls._typed(t)  # elements keep their bytes: the reference pads the binary of t as it is
+        for axis, (low, high, interior) in enumerate(padding_config):
+            a = np.moveaxis(a, axis, -1)
+            rows, n = a.shape[:-1], a.shape[-1]
+            # interior padding after every element, the last run dropped again
+            spread = np.full(rows + (n, interior + 1), value, dtype=a.dtype)
+            spread[..., 0] = a
+            seq = spread.reshape(rows + (n * (interior + 1),))[..., :max(n * (interior + 1) - interior, 0)]
+            # edges: positive ones add the value, negative ones cut into the interior-padded row
+            if low < 0:
+                seq = seq[..., -low:]
+            else:
+                seq = np.concatenate([np.full(rows + (low,), value, dtype=a.dtype), seq], axis=-1)
+            if high < 0:
+                seq = seq[..., :seq.shape[-1] + high]
+            else:
+                seq = np.concatenate([seq, np.full(rows + (high,), value, dtype=a.dtype)], axis=-1)
+            a = np.moveaxis(seq, -1, axis)
+        buf, res = cls._new(out)
+        buf[:] = np.ascontiguousarray(a).tobytes()
+        return res
+
+    @classmethod
     def slice(cls, out, t, start_indices, lengths, strides):  # binary_backend.ex:1813-1863
         a = cls._typed(t)
         window = []

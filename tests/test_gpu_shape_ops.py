@@ -175,3 +175,31 @@ def test_clip_compares_u64_as_unbounded_numbers(hip, oracle):
         Nx.default_backend(oracle)
     assert_bits_equal(got, want, "clip u64 with signed bounds")
     assert hip.to_numpy(got).tolist() == [3, 5, 1000, 1000, 1000, 999, 1000]
+
+
+PADS = [((10,), [(2, 1, 3)]), ((10,), [(-3, -2, 0)]), ((10,), [(-5, 2, 2)]), ((7, 9), [(1, 2, 0), (3, 0, 1)]), ((7, 9), [(-2, -1, 2), (-4, 5, 3)]),
+        ((4, 5, 6), [(0, 0, 0), (1, 1, 1), (-1, -1, 0)]), ((4, 5, 6), [(-1, 1, 1), (-2, 1, 1), (-2, 1, 1)]), ((3, 1, 8), [(0, 0, 2), (4, 4, 7), (0, 0, 0)]),
+        ((512, 384), [(16, 16, 0), (64, 64, 0)]), ((512, 384), [(0, 0, 1), (-8, -8, 0)]), ((6,), [(-3, -3, 0)]), ((6,), [(-20, 4, 3)]),
+        ((5, 4), [(0, 0, 0), (0, 0, 0)])]
+
+
+@pytest.mark.parametrize("ty", ["u8", "s16", "bf16", "f32", "s64", "f64"])
+@pytest.mark.parametrize("shape,config", PADS)
+def test_pad(ty, shape, config, hip, oracle):
+    rng = np.random.default_rng(seed_of(ty, shape, config))
+    ht, ot = pair(rng, ty, shape, hip, oracle, special=True)
+    hv, ov = pair(rng, ty, (), hip, oracle)
+    assert_bits_equal(Nx.pad(ht, hv, config), Nx.pad(ot, ov, config), f"pad {ty} {shape} {config}")
+
+
+@pytest.mark.parametrize("ty,vty", [("s32", "f32"), ("u8", "s16"), ("bf16", "f32"), ("f32", "s64"), ("s8", "u8")])
+def test_pad_converts_both_operands_to_the_merged_type(ty, vty, hip, oracle):
+    # the oracle follows the reference, which splices the two encodings when the types differ; the device
+    # converts first, as the compiled backends do: compare with the oracle applied after its own as_type
+    rng = np.random.default_rng(seed_of(ty, vty))
+    ht, ot = pair(rng, ty, (6, 11), hip, oracle, small=True)
+    hv, ov = pair(rng, vty, (), hip, oracle, small=True)
+    config = [(1, -1, 1), (-2, 3, 2)]
+    got = Nx.pad(ht, hv, config)
+    want = Nx.pad(Nx.as_type(ot, got.type), Nx.as_type(ov, got.type), config)
+    assert_bits_equal(got, want, f"pad {ty} with {vty}")
