@@ -13,6 +13,8 @@ constexpr int BLOCK = 256;
 constexpr int MAXR = 8;
 constexpr int E = 8;  // elements per lane per step of the vector kernels
 
+static bool narrow_float(int dt) { return dt == HIPNX_BF16 || dt == HIPNX_F16 || dt == HIPNX_F32; }
+
 static int grid_for(int64_t items) {
   int64_t blocks = (items + BLOCK - 1) / BLOCK;
   if (blocks < 1) blocks = 1;
@@ -63,14 +65,25 @@ select_vec_kernel(const void *__restrict__ p, const void *__restrict__ t, const 
     const int64_t i0 = v * E;
     if (i0 + E <= n) {
       CT a[E], b[E], c[E];
-      double pd[E];
-      int64_t pi[E];
-      const bool pf = pdt >= HIPNX_F16;
-      if (pstep) { if (pf) load_vec<double, E>(p, pdt, i0, pd); else load_vec<int64_t, E>(p, pdt, i0, pi); }
-      else {
+      bool pt[E];
+      if (!pstep) {
         const bool one = truthy<CT>(p, pdt, 0);
 #pragma unroll
-        for (int e = 0; e < E; e++) { pd[e] = one; pi[e] = one; }
+        for (int e = 0; e < E; e++) pt[e] = one;
+      } else if (pdt == HIPNX_U8 || pdt == HIPNX_S8) {  // what comparisons and logical ops produce
+        const uint2 w = *reinterpret_cast<const uint2 *>(static_cast<const unsigned char *>(p) + i0);
+#pragma unroll
+        for (int e = 0; e < E; e++) pt[e] = (((e < 4 ? w.x : w.y) >> (8 * (e & 3))) & 0xFF) != 0;
+      } else if (pdt >= HIPNX_F16) {
+        double pd[E];
+        load_vec<double, E>(p, pdt, i0, pd);
+#pragma unroll
+        for (int e = 0; e < E; e++) pt[e] = pd[e] != 0;
+      } else {
+        int64_t pi[E];
+        load_vec<int64_t, E>(p, pdt, i0, pi);
+#pragma unroll
+        for (int e = 0; e < E; e++) pt[e] = pi[e] != 0;
       }
       if (tstep) load_vec<CT, E>(t, tdt, i0, a);
       else { const CT x = load_one<CT>(t, tdt, 0);
@@ -81,7 +94,7 @@ select_vec_kernel(const void *__restrict__ p, const void *__restrict__ t, const 
 #pragma unroll
         for (int e = 0; e < E; e++) b[e] = x; }
 #pragma unroll
-      for (int e = 0; e < E; e++) c[e] = (pf ? pd[e] != 0 : pi[e] != 0) ? a[e] : b[e];
+      for (int e = 0; e < E; e++) c[e] = pt[e] ? a[e] : b[e];
       store_vec<CT, E>(out, odt, i0, c);
     } else {
       for (int64_t i = i0; i < n; i++) {
@@ -170,10 +183,15 @@ iota_kernel(void *__restrict__ out, int odt, int64_t n, int64_t dim, int64_t inn
   for (int64_t v = (int64_t)blockIdx.x * BLOCK + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * BLOCK) {
     const int64_t i0 = v * E;
     CT x[E];
+    // one division per vector, then count along: c = i % inner, r = (i / inner) % dim
+    int64_t q, c;
+    if (n <= 0xFFFFFFFFll) { q = (uint32_t)i0 / (uint32_t)inner; c = (uint32_t)i0 - (uint32_t)q * (uint32_t)inner; }
+    else { q = i0 / inner; c = i0 - q * inner; }
+    int64_t r = q < dim ? q : q % dim;
 #pragma unroll
     for (int e = 0; e < E; e++) {
-      const int64_t i = i0 + e, r = (i / inner) % dim;
-      x[e] = mode == 0 ? (CT)r : (CT)(r == i % inner ? 1 : 0);
+      x[e] = mode == 0 ? (CT)r : (CT)(r == c ? 1 : 0);
+      if (++c == inner) { c = 0; if (++r == dim) r = 0; }
     }
     if (i0 + E <= n) store_vec<CT, E>(out, odt, i0, x);
     else
@@ -228,9 +246,13 @@ extern "C" int hipnx_select(hipnx_ctx *ctx, int pred_dt, int true_dt, int false_
   if (m == 0) { s.dims[0] = 1; s.ps[0] = s.ts[0] = s.fs[0] = 0; m = 1; }
   s.rank = m;
   const bool fl = is_float(out_dt);
+  // values only pass through: f32 arithmetic holds every bf16 / f16 / f32 exactly
+  const bool narrow = narrow_float(true_dt) && narrow_float(false_dt) && narrow_float(out_dt);
   if (m == 1 && s.ps[0] <= 1 && s.ts[0] <= 1 && s.fs[0] <= 1) {
     dim3 grid(grid_for((n + E - 1) / E)), block(BLOCK);
-    if (fl) hipLaunchKernelGGL((select_vec_kernel<double>), grid, block, 0, ctx->stream, pred->ptr, on_true->ptr, on_false->ptr, out->ptr,
+    if (narrow) hipLaunchKernelGGL((select_vec_kernel<float>), grid, block, 0, ctx->stream, pred->ptr, on_true->ptr, on_false->ptr, out->ptr,
+                                   pred_dt, true_dt, false_dt, out_dt, n, (int)s.ps[0], (int)s.ts[0], (int)s.fs[0]);
+    else if (fl) hipLaunchKernelGGL((select_vec_kernel<double>), grid, block, 0, ctx->stream, pred->ptr, on_true->ptr, on_false->ptr, out->ptr,
                                pred_dt, true_dt, false_dt, out_dt, n, (int)s.ps[0], (int)s.ts[0], (int)s.fs[0]);
     else hipLaunchKernelGGL((select_vec_kernel<int64_t>), grid, block, 0, ctx->stream, pred->ptr, on_true->ptr, on_false->ptr, out->ptr,
                             pred_dt, true_dt, false_dt, out_dt, n, (int)s.ps[0], (int)s.ts[0], (int)s.fs[0]);
@@ -260,7 +282,9 @@ extern "C" int hipnx_clip(hipnx_ctx *ctx, int in_dt, int min_dt, int max_dt, int
   if (int st = check_buf(ctx, out, (uint64_t)n * dtype_size(out_dt), "clip out")) return st;
   if (n == 0) return HIPNX_OK;
   dim3 grid(grid_for((n + E - 1) / E)), block(BLOCK);
-  if (is_float(out_dt))
+  if (narrow_float(in_dt) && narrow_float(min_dt) && narrow_float(max_dt) && narrow_float(out_dt))
+    hipLaunchKernelGGL((clip_kernel<float>), grid, block, 0, ctx->stream, inb->ptr, min->ptr, max->ptr, out->ptr, in_dt, min_dt, max_dt, out_dt, n);
+  else if (is_float(out_dt))
     hipLaunchKernelGGL((clip_kernel<double>), grid, block, 0, ctx->stream, inb->ptr, min->ptr, max->ptr, out->ptr, in_dt, min_dt, max_dt, out_dt, n);
   else
     hipLaunchKernelGGL((clip_kernel<int64_t>), grid, block, 0, ctx->stream, inb->ptr, min->ptr, max->ptr, out->ptr, in_dt, min_dt, max_dt, out_dt, n);

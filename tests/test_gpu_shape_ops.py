@@ -66,6 +66,12 @@ def test_select_treats_nan_and_negative_zero_as_the_reference_does(hip, oracle):
     assert hip.to_numpy(got).tolist() == [0, -2, -3, 3, 4]
 
 
+def bound(number, backend):
+    """A clip bound as the front end would make it from a plain number: s32 or f32, rank 0."""
+    ty = "f32" if isinstance(number, float) else "s32"
+    return from_numpy(np.array(number, dtype=np.float32 if ty == "f32" else np.int32), ty, backend)
+
+
 @pytest.mark.parametrize("ty", TYPES)
 @pytest.mark.parametrize("lo,hi", [(-10, 10), (2.5, 7), (-3, 4.25), (5, -5)])
 @pytest.mark.parametrize("shape", [(1001,), (16, 64)])
@@ -74,13 +80,8 @@ def test_clip(ty, lo, hi, shape, hip, oracle):
         lo, hi = abs(lo), abs(hi)
     rng = np.random.default_rng(seed_of(ty, lo, hi, shape))
     ht, ot = pair(rng, ty, shape, hip, oracle, special=True)
-    Nx.default_backend(oracle)
-    want = Nx.clip(ot, lo, hi)
-    Nx.default_backend(hip)
-    try:
-        got = Nx.clip(ht, lo, hi)
-    finally:
-        Nx.default_backend(oracle)
+    got = Nx.clip(ht, bound(lo, hip), bound(hi, hip))
+    want = Nx.clip(ot, bound(lo, oracle), bound(hi, oracle))
     assert_bits_equal(got, want, f"clip {ty} [{lo}, {hi}] {shape}")
 
 
@@ -166,13 +167,8 @@ def test_all_any_count_nan_as_true(hip, oracle):
 def test_clip_compares_u64_as_unbounded_numbers(hip, oracle):
     # u64 against s32 bounds gives s64: 2^63 and above must land on the upper bound, not wrap below the lower one
     x = np.array([0, 5, 2**63 - 1, 2**63, 2**64 - 1, 999, 1001], dtype=np.uint64)
-    Nx.default_backend(oracle)
-    want = Nx.clip(from_numpy(x, "u64", oracle), 3, 1000)
-    Nx.default_backend(hip)
-    try:
-        got = Nx.clip(from_numpy(x, "u64", hip), 3, 1000)
-    finally:
-        Nx.default_backend(oracle)
+    want = Nx.clip(from_numpy(x, "u64", oracle), bound(3, oracle), bound(1000, oracle))
+    got = Nx.clip(from_numpy(x, "u64", hip), bound(3, hip), bound(1000, hip))
     assert_bits_equal(got, want, "clip u64 with signed bounds")
     assert hip.to_numpy(got).tolist() == [3, 5, 1000, 1000, 1000, 999, 1000]
 
