@@ -226,6 +226,18 @@ def main():
         _, ms = timed(lambda: Nx.iota((nn, nn), type="f32", axis=1, backend=H), steps, warm)
         entry(f"iota_f32_{nn}", 4.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
         del x, y
+
+        # Nx.Random on the device: 2^28 u32 words from one key (counter-based, write-only), and
+        # uniform f32 samples built on them by the reference's chain of element-wise callbacks
+        from nx_amd import random as Random
+        key = Random.key(1701, backend=H)
+        nw = 1 << 28
+        _, ms = timed(lambda: Random.random_bits(key, shape=(nw,)), steps, warm)
+        entry("random_bits_u32_2p28", 4.0 * nw, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+        _, ms = timed(lambda: Random.uniform_split(key, 0.0, 1.0, shape=(nw,)), steps, warm)
+        # bits out; shift, or, subtract, multiply, add, max each read and write the array once
+        entry("uniform_f32_2p28_unfused", 4.0 * nw * 13, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+        del key
         result["suite"] = suite
 
     # ---- CPU baseline: the reference-semantics restatement on a bounded sample -----------------

@@ -221,6 +221,14 @@ int hipnx_iota(hipnx_ctx *ctx, int out_dt, int64_t n, int64_t dim, int64_t inner
  * stacked rows x cols identity matrices */
 int hipnx_eye(hipnx_ctx *ctx, int out_dt, int64_t n, int64_t rows, int64_t cols, hipnx_buf *out);
 
+/* replaces: the callback composition behind threefry2x32/2 of Nx.Random (nx/lib/nx/random.ex:214-285;
+ * about 110 element-wise callbacks per call) with one kernel producing the same words: out[n] u32 is
+ * the Threefry-2x32-20 stream of key (u32[2]) over the counters 0 .. n-1, in the reference's
+ * order (pairs (i, ceil(n/2) + i), first words then second words, an odd n padded by one zero
+ * counter whose output is dropped).  Not a Nx.Backend callback: a binding calls it from its
+ * own random module when the key lives on the device. */
+int hipnx_threefry2x32(hipnx_ctx *ctx, const hipnx_buf *key, int64_t n, hipnx_buf *out);
+
 #ifdef __cplusplus
 }
 #endif

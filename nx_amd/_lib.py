@@ -75,6 +75,7 @@ PROTOTYPES = {
     "hipnx_strided_copy": [_ctx_p, C.c_int, C.c_int, _i64p, _i64p, C.c_int64, _i64p, C.c_int64, _buf_p, _buf_p],
     "hipnx_iota": [_ctx_p, C.c_int, C.c_int64, C.c_int64, C.c_int64, _buf_p],
     "hipnx_eye": [_ctx_p, C.c_int, C.c_int64, C.c_int64, C.c_int64, _buf_p],
+    "hipnx_threefry2x32": [_ctx_p, _buf_p, C.c_int64, _buf_p],
 }
 
 for _name, _args in PROTOTYPES.items():

@@ -594,6 +594,17 @@ class HipNxBackend:
         return cls.concatenate(out, widened, axis)
 
     @classmethod
+    def threefry2x32(cls, out: Tensor, key: Tensor) -> Tensor:
+        """The random words of Nx.Random's threefry2x32/2 (random.ex:214-285) for `out.size`
+        counters in one kernel; `out` is a u32 template.  Not a behaviour callback: the random
+        module asks the key's backend for it and composes the callbacks when it is absent."""
+        dev = cls._device_of(key)
+        key = cls._from_nx(key, dev)
+        res = cls._alloc(out, dev)
+        L.check(L.lib.hipnx_threefry2x32(res.data.ref.ctx, cls._handle(key), out.size, res.data.ref.handle))
+        return res
+
+    @classmethod
     def block(cls, struct, out: Tensor, args, fun):
         """block/4 (backend.ex:144): `Nx.Block.Take` along axis 0 is one row-copy kernel; other
         blocks run their default implementation on this backend's callbacks."""

@@ -343,6 +343,17 @@ static ERL_NIF_TERM nif_eye(ErlNifEnv *env, int argc, const ERL_NIF_TERM argv[])
   return ok(env, make_buf(env, out));
 }
 
+/* threefry2x32(ctx, key, n, out_bytes) */
+static ERL_NIF_TERM nif_threefry2x32(ErlNifEnv *env, int argc, const ERL_NIF_TERM argv[]) {
+  (void)argc;
+  GET_CTX(0, ctx); GET_BUF(1, key); GET_I64(2, n); GET_I64(3, out_bytes);
+  hipnx_buf *out;
+  CHECK(hipnx_buf_alloc(ctx, (size_t)out_bytes, &out));
+  int st = hipnx_threefry2x32(ctx, key, n, out);
+  if (st != HIPNX_OK) { hipnx_buf_destroy(out); return error_from_status(env, st); }
+  return ok(env, make_buf(env, out));
+}
+
 static ERL_NIF_TERM nif_sync(ErlNifEnv *env, int argc, const ERL_NIF_TERM argv[]) {
   (void)argc;
   GET_CTX(0, ctx);
@@ -369,6 +380,7 @@ static ErlNifFunc funcs[] = {
     {"broadcast", 6, nif_broadcast, IO},        {"gather", 10, nif_gather, IO},
     {"select", 13, nif_select, IO},             {"clip", 10, nif_clip, IO},
     {"strided_copy", 9, nif_strided_copy, IO},  {"iota", 6, nif_iota, IO},
-    {"eye", 6, nif_eye, IO},                    {"sync", 1, nif_sync, IO}};
+    {"eye", 6, nif_eye, IO},                    {"threefry2x32", 4, nif_threefry2x32, IO},
+    {"sync", 1, nif_sync, IO}};
 
 ERL_NIF_INIT(Elixir.HipNx.NIF, funcs, on_load, NULL, NULL, NULL)

@@ -503,6 +503,16 @@ defmodule HipNx.Backend do
       bytes(out))), device, out)
   end
 
+  @doc """
+  The words of `Nx.Random`'s `threefry2x32/2` for `Nx.size(out)` counters in one kernel
+  (`out` is a u32 template). Not a behaviour callback.
+  """
+  def threefry2x32(%T{} = out, %T{} = key) do
+    device = device_of([key])
+    {ref, _} = from_nx(key, device)
+    to_nx(unwrap!(NIF.threefry2x32(ctx(device), ref, Nx.size(out), bytes(out))), device, out)
+  end
+
   defp dense_strides(shape) do
     {strides, _} = shape |> Tuple.to_list() |> Enum.reverse() |> Enum.map_reduce(1, fn dim, acc -> {acc, acc * dim} end)
     Enum.reverse(strides)

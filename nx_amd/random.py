@@ -4,7 +4,9 @@
 Every function is the reference's composition of front-end calls, in the same order and with the
 same operand types, so the bits are the reference's on whichever backend the key lives: a key on
 the device keeps the whole computation there (u32 add / xor / shift / or, iota, concatenate,
-slice, as_type, bitcast are all native callbacks).  Keys are `u32[2]` tensors; functions are pure
+slice, as_type, bitcast are all native callbacks).  The one exception is an optimisation: when the
+key's backend has `threefry2x32(out, key)`, the cipher over the counter range is taken from it (the
+device computes the same words in one kernel instead of about 110 launches).  Keys are `u32[2]` tensors; functions are pure
 and return `(sample, new_key)` like the reference, the `*_split` variants take a key that has
 already been split.  Complex types and `shuffle`, `choice`, `gumbel`, `multivariate_normal` are
 not mirrored.
@@ -16,9 +18,18 @@ from math import prod
 
 from . import nx as Nx
 from . import types as T
-from .tensor import Tensor
+from .tensor import Tensor, template
 
 NBITS = 32
+_COMPOSE_ONLY = [False]
+
+
+def compose_only(flag: bool) -> bool:
+    """Forces threefry2x32 through the reference's composition of callbacks even when the key's
+    backend offers the words in one step (tests compare the two); returns the previous setting."""
+    previous, _COMPOSE_ONLY[0] = _COMPOSE_ONLY[0], bool(flag)
+    return previous
+
 _MANTISSA = {("bf", 16): 7, ("f", 16): 10, ("f", 32): 23, ("f", 64): 52}
 # Threefry-2x32 rotation schedule, two groups of four rounds (random.ex:216)
 _ROTATIONS = ((13, 15, 26, 6), (17, 29, 16, 24))
@@ -83,6 +94,9 @@ def threefry2x32(key: Tensor, shape) -> Tensor:
     shape = tuple(shape)
     size = prod(shape)
     backend = type(key.data)
+    fused = None if _COMPOSE_ONLY[0] else getattr(backend, "threefry2x32", None)
+    if fused is not None:  # a backend may produce the same words in one step
+        return fused(template(("u", 32), shape), key)
     if size % 2 == 0:
         xs = Nx.iota((2, size // 2), type="u32", backend=backend)
         return Nx.reshape(threefry2x32_20_concat(xs, key), shape)

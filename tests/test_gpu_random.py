@@ -87,3 +87,24 @@ def test_moments_of_a_large_sample_stay_on_the_device(hip):
     assert abs(r.mean() - 52.5) < 5.25 and abs(r.var() - 84 * 86 / 12) < 60.2
     n = hip.to_numpy(Random.normal_split(key, 10, 5, shape=(10000,))).astype(np.float64)
     assert abs(n.mean() - 10) < 1 and abs(n.std() - 5) < 0.5
+
+
+@pytest.mark.parametrize("shape", [(), (1,), (2,), (7,), (8,), (3, 5), (1001,), (64, 129), (1 << 20,), ((1 << 20) + 1,)])
+def test_fused_threefry_matches_the_composition(shape, hip):
+    key = Random.key(seed_of(shape), backend=hip)
+    fused = Random.threefry2x32(key, shape)
+    previous = Random.compose_only(True)
+    try:
+        composed = Random.threefry2x32(key, shape)
+    finally:
+        Random.compose_only(previous)
+    assert_bits_equal(fused, composed, f"threefry2x32 {shape}")
+
+
+def test_known_answers_hold_through_the_composition_too(hip):
+    previous = Random.compose_only(True)
+    try:
+        for case in CASES:
+            check_random_case(case, hip)
+    finally:
+        Random.compose_only(previous)
