@@ -596,8 +596,8 @@ class HipNxBackend:
     @classmethod
     def threefry2x32(cls, out: Tensor, key: Tensor) -> Tensor:
         """The random words of Nx.Random's threefry2x32/2 (random.ex:214-285) for `out.size`
-        counters in one kernel; `out` is a u32 template.  Not a behaviour callback: the random
-        module asks the key's backend for it and composes the callbacks when it is absent."""
+        counters in one kernel; `out` is a u32 template.  Reached through block/4 with a
+        `BlockThreefry`."""
         dev = cls._device_of(key)
         key = cls._from_nx(key, dev)
         res = cls._alloc(out, dev)
@@ -608,11 +608,13 @@ class HipNxBackend:
     def block(cls, struct, out: Tensor, args, fun):
         """block/4 (backend.ex:144): `Nx.Block.Take` along axis 0 is one row-copy kernel; other
         blocks run their default implementation on this backend's callbacks."""
-        from .nx import BlockTake
+        from .nx import BlockTake, BlockThreefry
         if isinstance(struct, BlockTake) and struct.axis == 0:
             t, indices = args
             idx = indices.with_(shape=(indices.size, 1))
             return cls.gather(out, t, idx, {"axes": [0]})
+        if isinstance(struct, BlockThreefry):
+            return cls.threefry2x32(out, args[0])
         return fun(struct, *args)
 
 

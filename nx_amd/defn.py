@@ -1,0 +1,687 @@
+"""Traced functions and their evaluator: the caller one step above the backend callbacks.
+
+Host-side mirror of `Nx.Defn.jit` with the default compiler (reference:
+nx/lib/nx/defn/compiler.ex:159-205, nx/lib/nx/defn/expr.ex, nx/lib/nx/defn/evaluator.ex).
+`jit(fun)` runs `fun` once on *expressions* -- tensors whose data is an `Expr` node, built by the
+`Expr` backend while the front end does its usual shape and type work -- and then walks the graph,
+calling the callbacks of the backend the arguments live on (`eval_apply`, evaluator.ex:363-388).
+
+Two things of the reference are kept because they change results or memory:
+  * the expression builder rewrites sums and products with constant operands and folds
+    operations on constants (expr.ex:889-984, 1597-1674).  Float arithmetic does not associate, so a
+    traced `c * (k * x)` really is `(c*k) * x` in the reference, and here.
+  * every node is evaluated once and dropped after its last use (reference counts per scope,
+    evaluator.ex:86-210, 213-262), so device buffers of intermediates return to the pool as the
+    walk proceeds.
+Control flow: `while_loop` and `cond` build `:while` / `:cond` nodes whose bodies are scopes of
+their own; outside a trace they run eagerly.
+"""
+from __future__ import annotations
+
+import itertools
+import operator
+import threading
+from typing import Any, Callable, Dict, List, Optional, Tuple
+
+import numpy as np
+
+from . import nx as Nx
+from . import types as T
+from .backend_names import BINARY_OPS, UNARY_OPS
+from .host import HostBinary
+from .tensor import Tensor, binary_to_numpy, template
+
+_ids = itertools.count(1)
+_trace = threading.local()  # .scopes: stack of scope tags of the trace in progress
+
+
+class _ExprMeta(type):
+    """Any callback name not written out below builds a plain node `op(out, *args)`."""
+
+    def __getattr__(cls, op):
+        if op.startswith("_"):
+            raise AttributeError(op)
+
+        def build(out, *args):
+            return cls._expr(out, op, [_to_expr_arg(a) for a in args])
+        build.__name__ = op
+        return build
+
+
+class Expr(metaclass=_ExprMeta):
+    """%Nx.Defn.Expr{id, op, args} (expr.ex:1-60) and, as a class, the backend that builds them."""
+
+    __slots__ = ("id", "op", "args", "scope")
+
+    def __init__(self, id, op, args, scope):  # noqa: A002
+        self.id, self.op, self.args, self.scope = id, op, args, scope
+
+    def __repr__(self):
+        return f"Expr<{self.op} #{self.id}>"
+
+    # ---- construction ------------------------------------------------------------------------
+    @classmethod
+    def init(cls, opts=None):
+        return {}
+
+    @classmethod
+    def _expr(cls, out: Tensor, op: str, args: list) -> Tensor:
+        scopes = getattr(_trace, "scopes", None)
+        if not scopes:
+            raise RuntimeError("expressions can only be built while a function is being traced")
+        return out.with_(data=Expr(next(_ids), op, args, scopes[-1]))
+
+    @classmethod
+    def _constant(cls, out: Tensor, number) -> Tensor:
+        # expr.ex:1553-1576: integers become floats in a float type; a non-integer has no integer form
+        if T.is_float(out.type):
+            number = float(number)
+        elif not isinstance(number, (int, np.integer)) or isinstance(number, bool):
+            raise ValueError(f"value {number!r} is not valid for constant of type {out.type!r}")
+        else:
+            number = int(number)
+        return out.with_(data=Expr(("c", repr(number), out.type, out.shape), "constant", [number], None))
+
+    # creation callbacks (expr.ex:851-871)
+    @classmethod
+    def constant(cls, out, number, opts=None):
+        return cls._constant(out, number)
+
+    @classmethod
+    def from_binary(cls, out, binary, opts=None):
+        return to_expr(HostBinary.from_binary(out, binary, {}))
+
+    @classmethod
+    def iota(cls, out, axis, opts=None):
+        return cls._expr(out, "iota", [axis])
+
+    @classmethod
+    def eye(cls, out, opts=None):
+        return cls._expr(out, "eye", [])
+
+    @classmethod
+    def to_binary(cls, t, limit):
+        raise ValueError("cannot read the value of a tensor expression: it has no data while the function is being traced")
+
+    @classmethod
+    def backend_transfer(cls, t, backend, opts=None):
+        raise ValueError("cannot transfer a tensor expression between backends")
+
+    backend_copy = backend_transfer
+
+    @classmethod
+    def backend_deallocate(cls, t):
+        return "already_deallocated"
+
+    # ---- rewrites of the arithmetic with constants (expr.ex:889-984) ---------------------------
+    @classmethod
+    def add(cls, out, t1, t2):
+        t1, t2 = to_expr(t1), to_expr(t2)
+        c1, c2 = _const(t1), _const(t2)
+        if c1 is not None and c1 == 0:
+            return _ensure_compatible(t2, out)
+        if c2 is not None and c2 == 0:
+            return _ensure_compatible(t1, out)
+        if c2 is not None:
+            return cls._commute(out, "add", operator.add, c2, t2, t1)
+        inner = _node(t2, "subtract")
+        if inner is not None and _const(inner[0]) is not None and _const(inner[0]) == 0:
+            return cls._binary_expr(out, "subtract", t1, inner[1])  # a + (0 - b) = a - b
+        return cls._commute(out, "add", operator.add, c1, t1, t2)
+
+    @classmethod
+    def subtract(cls, out, t1, t2):
+        t1, t2 = to_expr(t1), to_expr(t2)
+        c1, c2 = _const(t1), _const(t2)
+        if c2 is not None and c2 == 0:
+            return _ensure_compatible(t1, out)
+        if c1 is not None and c2 is not None:
+            return cls._constant(out, c1 - c2)
+        return cls._binary_expr(out, "subtract", t1, t2)
+
+    @classmethod
+    def multiply(cls, out, t1, t2):
+        t1, t2 = to_expr(t1), to_expr(t2)
+        c1, c2 = _const(t1), _const(t2)
+        if c1 is not None and c1 == 1:
+            return _ensure_compatible(t2, out)
+        if c2 is not None and c2 == 1:
+            return _ensure_compatible(t1, out)
+        if c2 is not None:
+            return cls._commute(out, "multiply", operator.mul, c2, t2, t1)
+        inner = _node(t2, "divide")
+        if inner is not None and _const(inner[0]) is not None and _const(inner[0]) == 1:
+            return cls._binary_expr(out, "divide", t1, inner[1])  # a * (1 / b) = a / b
+        return cls._commute(out, "multiply", operator.mul, c1, t1, t2)
+
+    @classmethod
+    def divide(cls, out, t1, t2):
+        t1, t2 = to_expr(t1), to_expr(t2)
+        c2 = _const(t2)
+        if c2 is not None and c2 == 1:
+            return _ensure_compatible(t1, out)
+        return cls._binary_expr(out, "divide", t1, t2)
+
+    @classmethod
+    def pow(cls, out, t1, t2):  # noqa: A003
+        t1, t2 = to_expr(t1), to_expr(t2)
+        c2 = _const(t2)
+        if c2 is not None and c2 == 1:
+            return _ensure_compatible(t1, out)
+        return cls._binary_expr(out, "pow", t1, t2)
+
+    @classmethod
+    def _commute(cls, out, op, fun, s1, t1, t2):
+        """expr.ex:1597-1621: the constant of a commutative chain moves to the left, two constants
+        merge (in host arithmetic, not rounded to the tensor type until the constant is used)."""
+        scalar = out.with_(data=None, shape=())
+        a1, a2 = t1, t2
+        inner2, inner1 = _node(t2, op), _node(t1, op)
+        if inner2 is not None and _const(inner2[0]) is not None:
+            s2, t3 = _const(inner2[0]), inner2[1]
+            if s1 is not None:
+                a1, a2 = cls._constant(scalar, fun(s1, s2)), Nx.broadcast(t3, out.shape)
+            else:
+                a1, a2 = cls._constant(scalar, s2), Nx.broadcast(getattr(Nx, op)(t1, t3), out.shape)
+        elif inner1 is not None and _const(inner1[0]) is not None:
+            a1, a2 = cls._constant(scalar, _const(inner1[0])), Nx.broadcast(getattr(Nx, op)(t2, inner1[1]), out.shape)
+        return cls._binary_expr(out, op, a1, a2)
+
+    @classmethod
+    def _binary_expr(cls, out, op, a1, a2):
+        c1, c2 = _const(a1), _const(a2)
+        if c1 is not None and c2 is not None:  # expr.ex:1628-1635: folded by a compute backend
+            backend, opts = _fold_backend()
+            scalar = out.with_(data=None, shape=())
+            left = backend.constant(template(a1.type, ()), c1, opts)
+            right = backend.constant(template(a2.type, ()), c2, opts)
+            return cls._constant(out, _to_number(getattr(backend, op)(scalar, left, right)))
+        if c1 is not None:
+            a1 = _upcast_float_constant(a1, out.type)
+        elif c2 is not None:
+            a2 = _upcast_float_constant(a2, out.type)
+        return cls._expr(out, op, [a1, a2])
+
+    @classmethod
+    def _unary_expr(cls, out, op, t):
+        t = to_expr(t)
+        c = _const(t)
+        if c is None:
+            return cls._expr(out, op, [t])
+        backend, opts = _fold_backend()  # expr.ex:1666-1674
+        value = backend.constant(template(t.type, ()), c, opts)
+        return cls._constant(out, _to_number(getattr(backend, op)(out.with_(data=None, shape=()), value)))
+
+    # ---- shape callbacks with their collapses (expr.ex:1088-1145) -------------------------------
+    @classmethod
+    def squeeze(cls, out, t, axes):
+        t = to_expr(t)
+        inner = _node(t, "squeeze")
+        if inner is not None:  # a squeeze of a squeeze is one squeeze (keeps `t[i][j]` one node)
+            return cls._expr(out, "squeeze", [inner[0], _merge_squeeze(sorted(inner[1]), sorted(axes), 0)])
+        return cls._expr(out, "squeeze", [t, list(axes)])
+
+    @classmethod
+    def broadcast(cls, out, t, shape, axes):
+        t = to_expr(t)
+        inner = _node(t, "broadcast")
+        if inner is not None:
+            inner_t, inner_shape, inner_axes = inner
+            first = _contiguous(inner_axes, 0) and _contiguous(axes, 0)
+            last = (_contiguous(inner_axes, len(inner_shape) - len(inner_t.shape))
+                    and _contiguous(axes, len(shape) - len(t.shape)))
+            if first or last:
+                return cls._expr(out, "broadcast", [inner_t, tuple(shape), list(inner_axes)])
+        c = _const(t)
+        if c is not None:
+            return cls._constant(out, c)
+        return cls._expr(out, "broadcast", [t, tuple(shape), list(axes)])
+
+    @classmethod
+    def block(cls, struct, out, args, fun):
+        # expr.ex:824-842, without re-tracing the default implementation: the evaluator hands the
+        # node to the backend's block/4, which runs `fun` on its own callbacks when it has no kernel
+        return cls._expr(out, "block", [struct, [to_expr(a) for a in args], fun])
+
+
+def _install():
+    for op in BINARY_OPS:
+        if op not in ("add", "subtract", "multiply", "divide", "pow"):
+            def binary(out, t1, t2, _op=op):
+                return Expr._binary_expr(out, _op, to_expr(t1), to_expr(t2))
+            binary.__name__ = op
+            setattr(Expr, op, staticmethod(binary))
+    for op in list(UNARY_OPS) + ["as_type", "bitcast"]:
+        def unary(out, t, _op=op):
+            return Expr._unary_expr(out, _op, t)
+        unary.__name__ = op
+        setattr(Expr, op, staticmethod(unary))
+
+
+_install()
+
+
+# ---- helpers of the builder ---------------------------------------------------------------------
+
+def _const(t) -> Optional[Any]:
+    return t.data.args[0] if isinstance(t, Tensor) and isinstance(t.data, Expr) and t.data.op == "constant" else None
+
+
+def _node(t, op) -> Optional[list]:
+    return t.data.args if isinstance(t, Tensor) and isinstance(t.data, Expr) and t.data.op == op else None
+
+
+def _contiguous(axes, start) -> bool:
+    return list(axes) == list(range(start, start + len(axes)))
+
+
+def _merge_squeeze(inner, axes, extra):  # expr.ex:1112-1121
+    if inner and axes and inner[0] <= axes[0] + extra:
+        return [inner[0]] + _merge_squeeze(inner[1:], axes, extra + 1)
+    if axes:
+        return [axes[0] + extra] + _merge_squeeze(inner, axes[1:], extra)
+    return []
+
+
+def _ensure_compatible(t, out):  # expr.ex:1589-1594
+    return Nx.broadcast(Nx.as_type(t, out.type), out.shape)
+
+
+def _upcast_float_constant(t, out_type):  # expr.ex:1648-1664
+    if T.is_float(t.type) and T.is_float(out_type):
+        return Expr._constant(t.with_(data=None, type=out_type), _const(t))
+    return t
+
+
+def _to_number(t: Tensor):
+    value = binary_to_numpy(Nx.to_binary(t), t.type, ())
+    if t.type == ("bf", 16):
+        value = (np.asarray(value, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+    return np.asarray(value).reshape(()).item()
+
+
+def _fold_backend():
+    """Where operations on constants are computed while tracing.  The reference folds on its host
+    backend; here the backend that was the default when the trace began does it, or the device when
+    that default only stores data."""
+    mod, opts = getattr(_trace, "fold", None) or (None, None)
+    if mod is None or mod is HostBinary or mod is Expr:
+        from .backend import HipNxBackend
+        return HipNxBackend, HipNxBackend.init({})
+    return mod, opts
+
+
+def to_expr(value) -> Tensor:
+    """expr.ex:1349-1376: expressions pass, host tensors become constants (rank 0) or literals,
+    numbers become constants; a tensor of a compute backend cannot be captured."""
+    if isinstance(value, Tensor):
+        if isinstance(value.data, Expr):
+            return value
+        if isinstance(value.data, HostBinary):
+            if value.shape == ():
+                return Expr._constant(value.with_(data=None), _to_number(value))
+            return Expr._expr(value.with_(data=None), "tensor", [value])
+        raise ValueError(
+            f"cannot convert tensor allocated on {type(value.data).__name__} to an expression. This may mean you "
+            "are passing a tensor to a traced function as a closure; pass it as an argument instead")
+    if isinstance(value, (bool, int, float, np.integer, np.floating)):
+        v = value.item() if isinstance(value, np.generic) else value
+        return Expr._constant(template(T.infer(v), ()), v)
+    raise ValueError(f"unable to build tensor expression, expected a tensor or a number, got: {value!r}")
+
+
+def _to_expr_arg(a):
+    if isinstance(a, Tensor):
+        return to_expr(a)
+    if isinstance(a, (list, tuple)) and any(isinstance(x, Tensor) for x in a):
+        return [to_expr(x) if isinstance(x, Tensor) else x for x in a]
+    return a
+
+
+# ---- composites -----------------------------------------------------------------------------------
+
+def _flatten(value, leaves: list):
+    """Nested tuples / lists / dicts of tensors -> a structure of leaf positions."""
+    if isinstance(value, (tuple, list)):
+        return type(value)(_flatten(v, leaves) for v in value)
+    if isinstance(value, dict):
+        return {k: _flatten(v, leaves) for k, v in value.items()}
+    leaves.append(value)
+    return _Leaf(len(leaves) - 1)
+
+
+class _Leaf:
+    __slots__ = ("index",)
+
+    def __init__(self, index):
+        self.index = index
+
+
+def _unflatten(structure, leaves):
+    if isinstance(structure, (tuple, list)):
+        return type(structure)(_unflatten(v, leaves) for v in structure)
+    if isinstance(structure, dict):
+        return {k: _unflatten(v, leaves) for k, v in structure.items()}
+    return leaves[structure.index]
+
+
+# ---- control flow ---------------------------------------------------------------------------------
+
+def _tracing() -> bool:
+    return bool(getattr(_trace, "scopes", None))
+
+
+def _push_scope():
+    tag = next(_ids)
+    _trace.scopes.append(tag)
+    return tag
+
+
+def while_loop(initial, condition: Callable, body: Callable):
+    """`while` of Nx.Defn.Kernel (expr.ex:306-420): `condition(state)` is a rank-0 tensor,
+    `body(state)` returns a state of the same structure, shapes and types.  Everything the two use
+    must come in through `state`."""
+    if not _tracing():
+        state = initial
+        while _to_number(Nx.to_tensor(condition(state))) != 0:
+            state = body(state)
+        return state
+    leaves: list = []
+    structure = _flatten(initial, leaves)
+    initial_exprs = [to_expr(Nx.to_tensor(v)) for v in leaves]
+    tag = _push_scope()
+    try:
+        params = [Expr._expr(t.with_(data=None), "parameter", [i]) for i, t in enumerate(initial_exprs)]
+        state = _unflatten(structure, params)
+        pred = to_expr(Nx.to_tensor(condition(state)))
+        if pred.shape != ():
+            raise ValueError(f"condition must be a scalar tensor, got shape {pred.shape!r}")
+        out_leaves: list = []
+        out_structure = _flatten(body(state), out_leaves)
+        out_exprs = [to_expr(Nx.to_tensor(v)) for v in out_leaves]
+    finally:
+        _trace.scopes.pop()
+    if len(out_exprs) != len(initial_exprs) or any(
+            (a.type, a.shape) != (b.type, b.shape) for a, b in zip(initial_exprs, out_exprs)):
+        raise ValueError("the body of while must return tensors with the same shape and type as the initial arguments")
+    del out_structure
+    node = Expr(next(_ids), "while", [initial_exprs, pred, out_exprs, tag], _trace.scopes[-1])
+    results = [Expr._expr(t.with_(data=None), "elem", [node, i]) for i, t in enumerate(initial_exprs)]
+    return _unflatten(structure, results)
+
+
+def cond(pred, on_true: Callable, on_false: Callable):
+    """`cond` / `if` of Nx.Defn.Kernel (expr.ex:139-300): only the chosen branch is evaluated.
+    The branches are thunks returning composites of the same structure, shapes and types."""
+    if not _tracing():
+        return on_true() if _to_number(Nx.to_tensor(pred)) != 0 else on_false()
+    pred = to_expr(Nx.to_tensor(pred))
+    if pred.shape != ():
+        raise ValueError(f"condition must be a scalar tensor, got shape {pred.shape!r}")
+    branches = []
+    for thunk in (on_true, on_false):
+        tag = _push_scope()
+        try:
+            leaves: list = []
+            structure = _flatten(thunk(), leaves)
+            branches.append((tag, structure, [to_expr(Nx.to_tensor(v)) for v in leaves]))
+        finally:
+            _trace.scopes.pop()
+    (_, structure, first), (_, _, second) = branches
+    if len(first) != len(second) or any((a.type, a.shape) != (b.type, b.shape) for a, b in zip(first, second)):
+        raise ValueError("cond expects all branches to return compatible tensor types")
+    node = Expr(next(_ids), "cond", [pred, [(tag, exprs) for tag, _, exprs in branches]], _trace.scopes[-1])
+    results = [Expr._expr(t.with_(data=None), "elem", [node, i]) for i, t in enumerate(first)]
+    return _unflatten(structure, results)
+
+
+# ---- the evaluator ----------------------------------------------------------------------------------
+
+CREATION_OPS = ("eye", "iota")           # evaluator.ex:26-28
+LIST_OPS = ("concatenate", "stack")
+INDICES_OPS = ("slice", "put_slice")
+
+
+def _children(node: Expr):
+    """The tensor expressions a node reads in its own scope (Tree.apply_args, tree.ex)."""
+    if node.op in ("constant", "tensor", "parameter"):
+        return
+    if node.op == "elem":
+        yield node.args[0]  # the scope node itself (an Expr, not a tensor)
+        return
+    if node.op == "while":
+        yield from node.args[0]
+        return
+    if node.op == "cond":
+        yield node.args[0]
+        return
+    for a in (node.args[1] if node.op == "block" else node.args):
+        if isinstance(a, Tensor):
+            yield a
+        elif isinstance(a, list):
+            for x in a:
+                if isinstance(x, Tensor):
+                    yield x
+
+
+def _expr_of(x) -> Expr:
+    return x.data if isinstance(x, Tensor) else x
+
+
+class _Plan:
+    """Reference counts of one scope: id -> uses inside the scope (evaluator.ex:86-128), the nodes of
+    enclosing scopes it reads, and the plans of the scopes nested in it."""
+
+    def __init__(self, roots, tag, plans):
+        self.tag = tag
+        self.counts: Dict[Any, int] = {}
+        self.outer: Dict[Any, Any] = {}  # id -> node (tensor or Expr) that belongs to an enclosing scope
+        for r in roots:
+            self._visit(r, plans)
+
+    def _visit(self, x, plans):
+        e = _expr_of(x)
+        if e.op in ("constant", "tensor"):
+            return
+        if e.scope != self.tag:
+            self.outer.setdefault(e.id, x)
+            return
+        if e.id in self.counts:
+            self.counts[e.id] += 1
+            return
+        self.counts[e.id] = 1
+        for child in _children(e):
+            self._visit(child, plans)
+        nested = []
+        if e.op == "while":
+            _, pred, body, tag = e.args
+            nested.append(_Plan([pred] + list(body), tag, plans))
+        elif e.op == "cond":
+            nested.extend(_Plan(exprs, tag, plans) for tag, exprs in e.args[1])
+        for plan in nested:
+            plans[plan.tag] = plan
+            for outer in plan.outer.values():  # one use per nested scope, released when the scope node is done
+                self._visit(outer, plans)
+
+
+class _Scope:
+    def __init__(self, plan: _Plan, parent: Optional["_Scope"], params):
+        self.plan, self.parent, self.params = plan, parent, params
+        self.counts = dict(plan.counts)
+        self.results: Dict[Any, Any] = {}
+
+
+class _Run:
+    def __init__(self, plans, backend):
+        self.plans, self.backend = plans, backend
+
+    def eval(self, x, scope: _Scope):  # noqa: A003
+        e = _expr_of(x)
+        if e.op == "tensor":
+            t = e.args[0]
+            mod, opts = self.backend
+            return t if mod is HostBinary else Nx.backend_transfer(t, mod, opts)
+        if e.op == "constant":
+            mod, opts = self.backend  # evaluator.ex:212-215
+            return mod.constant(x.with_(data=None), e.args[0], opts)
+        owner = scope
+        while owner is not None and e.id not in owner.counts:
+            owner = owner.parent
+        if owner is None:
+            raise RuntimeError(f"evaluator cache has expired for {e!r}")
+        if e.id in owner.results:
+            res = owner.results[e.id]
+        else:
+            res = self.apply(e, x, owner)
+            owner.results[e.id] = res
+        if owner is scope:  # a read from a nested scope is released by the scope node (evaluator.ex:231-236)
+            self.release(e.id, owner)
+        return res
+
+    def release(self, id_, owner: _Scope):
+        owner.counts[id_] -= 1
+        if owner.counts[id_] == 0:
+            owner.results.pop(id_, None)
+
+    def release_outer(self, plan: _Plan, scope: _Scope):
+        for id_ in plan.outer:
+            owner = scope
+            while owner is not None and id_ not in owner.counts:
+                owner = owner.parent
+            if owner is not None:
+                self.release(id_, owner)
+
+    def apply(self, e: Expr, x, scope: _Scope):
+        op = e.op
+        if op == "parameter":
+            return scope.params[e.args[0]]
+        if op == "elem":
+            return self.eval(e.args[0], scope)[e.args[1]]
+        if op == "while":
+            initial, pred, body, tag = e.args
+            state = [self.eval(t, scope) for t in initial]
+            plan = self.plans[tag]
+            while True:  # evaluator.ex:398-409: a fresh set of counts per trip
+                trip = _Scope(plan, scope, state)
+                if _to_number(self.eval(pred, trip)) == 0:
+                    break
+                state = [self.eval(t, trip) for t in body]
+            self.release_outer(plan, scope)
+            return state
+        if op == "cond":
+            pred, branches = e.args
+            chosen = 0 if _to_number(self.eval(pred, scope)) != 0 else 1
+            tag, exprs = branches[chosen]
+            branch = _Scope(self.plans[tag], scope, scope.params)
+            result = [self.eval(t, branch) for t in exprs]
+            for tag, _ in branches:
+                self.release_outer(self.plans[tag], scope)
+            return result
+        if op == "block":
+            struct, in_args, fun = e.args
+            args = [self.eval(a, scope) for a in in_args]
+            return self.pick(args).block(struct, x.with_(data=None), args, fun)
+        out = x.with_(data=None)
+        if op in CREATION_OPS:  # evaluator.ex:368-371
+            mod, opts = self.backend
+            return getattr(mod, op)(out, *e.args, opts)
+        args = []
+        for a in e.args:
+            if isinstance(a, Tensor):
+                args.append(self.eval(a, scope))
+            elif isinstance(a, list) and any(isinstance(v, Tensor) for v in a):
+                args.append([self.eval(v, scope) if isinstance(v, Tensor) else v for v in a])
+            else:
+                args.append(a)
+        if op in LIST_OPS:
+            mod = self.pick(args[0])
+        elif op in INDICES_OPS:
+            mod = self.pick([args[0]] + [i for i in args[1] if isinstance(i, Tensor)])
+        else:
+            mod = self.pick([a for a in args if isinstance(a, Tensor)])
+        return getattr(mod, op)(out, *args)
+
+    def pick(self, tensors):
+        """Nx.Shared.list_impl!/1 (shared.ex:459-472); operands that only store data follow the others,
+        or the default backend when nothing else is there."""
+        tensors = [t for t in tensors if isinstance(t, Tensor)]
+        mod = Nx._impl(*tensors) if tensors else HostBinary
+        return self.backend[0] if mod is HostBinary else mod
+
+
+class Compiled:
+    """A traced function: call it with arguments of the traced shapes and types."""
+
+    def __init__(self, roots, structure, n_params):
+        self.roots, self.structure, self.n_params = roots, structure, n_params
+        self.plans: Dict[Any, _Plan] = {}
+        self.plan = _Plan(roots, 0, self.plans)
+
+    def __call__(self, *args):
+        leaves: list = []
+        _flatten(list(args), leaves)
+        if len(leaves) != self.n_params:
+            raise ValueError(f"expected {self.n_params} tensor arguments, got {len(leaves)}")
+        params = [Nx.to_tensor(v) for v in leaves]
+        backend = _runtime_backend(params)
+        run = _Run(self.plans, backend)
+        root = _Scope(self.plan, None, params)
+        results = []
+        for r in self.roots:
+            value = run.eval(r, root)
+            # evaluator.ex:68-75: the output keeps the traced template, the data is the result's
+            results.append(r.with_(data=value.data))
+        return _unflatten(self.structure, results)
+
+
+def _runtime_backend(params):
+    """evaluator.ex:36-38 (`__to_backend__`): constants and created tensors go to the default
+    backend; when that one only stores data they go where the arguments live."""
+    mod, opts = Nx.default_backend()
+    if mod is HostBinary or mod is Expr:
+        for p in params:
+            b = type(p.data)
+            if b is not HostBinary and b is not Expr:
+                return b, b.init({})
+    return mod, opts
+
+
+def trace(fun: Callable, args, kwargs=None) -> Compiled:
+    """Runs `fun` on parameter expressions shaped like `args` (compiler.ex:184-205: the default
+    backend is the expression builder while the function runs)."""
+    leaves: list = []
+    structure = _flatten(list(args), leaves)
+    templates = [v if isinstance(v, Tensor) else Nx.to_tensor(v) for v in leaves]
+    if getattr(_trace, "scopes", None):
+        raise RuntimeError("a traced function cannot be traced again from inside a trace")
+    _trace.scopes = [0]
+    _trace.fold = Nx.default_backend()
+    previous = Nx.default_backend(Expr)
+    try:
+        params = [Expr._expr(t.with_(data=None), "parameter", [i]) for i, t in enumerate(templates)]
+        result = fun(*_unflatten(structure, params), **(kwargs or {}))
+        out_leaves: list = []
+        out_structure = _flatten(result, out_leaves)
+        roots = [to_expr(Nx.to_tensor(v)) for v in out_leaves]
+    finally:
+        Nx.default_backend(*previous)
+        _trace.scopes = []
+        _trace.fold = None
+    return Compiled(roots, out_structure, len(templates))
+
+
+def jit(fun: Callable = None, **static):
+    """Nx.Defn.jit/2 with the default compiler: traces on every call, like the reference's
+    evaluator (evaluator.ex:41-43), then evaluates.  Keyword arguments are static options."""
+    if fun is None:
+        return lambda f: jit(f, **static)
+
+    def call(*args, **kwargs):
+        return trace(fun, args, {**static, **kwargs})(*args)
+    call.__name__ = getattr(fun, "__name__", "jitted")
+    return call
+
+
+def compile(fun: Callable, *templates, **static) -> Compiled:  # noqa: A001 - Nx.Defn.compile/3
+    """Traces once for arguments shaped like `templates`; the result is called many times."""
+    return trace(fun, templates, static)

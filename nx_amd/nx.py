@@ -386,6 +386,14 @@ class BlockTake:
     axis: int
 
 
+@dataclass(frozen=True)
+class BlockThreefry:
+    """The Threefry-2x32 stream of a key over `size` counters (the body of threefry2x32/2,
+    nx/lib/nx/random.ex:214-229) as a block, so a backend can produce the words in one step.  The
+    reference composes it from callbacks without a block; the words are the same."""
+    shape: tuple
+
+
 def block(struct, args, out, fun):
     """Nx.block/4 (nx.ex:7370-7380): lets the backend replace a composite op."""
     return _impl(*args).block(struct, out, list(args), fun)
@@ -427,7 +435,7 @@ def take(t, indices, axis=0):
     return block(BlockTake(axis), [t, indices], out, default)
 
 
-# ---- one step off the hot path: creation, selection, windows (SURVEY "next" rows) --------------
+# ---- one step off the hot path: creation, selection, windows -------------------------------------
 
 def all(t, axes=None, keep_axes=False):  # noqa: A001 - Nx.all/2 (nx.ex:9207-9209): u8 output
     return _aggregate(to_tensor(t), "all", ("u", 8), axes, keep_axes)

@@ -4,9 +4,9 @@
 Every function is the reference's composition of front-end calls, in the same order and with the
 same operand types, so the bits are the reference's on whichever backend the key lives: a key on
 the device keeps the whole computation there (u32 add / xor / shift / or, iota, concatenate,
-slice, as_type, bitcast are all native callbacks).  The one exception is an optimisation: when the
-key's backend has `threefry2x32(out, key)`, the cipher over the counter range is taken from it (the
-device computes the same words in one kernel instead of about 110 launches).  Keys are `u32[2]` tensors; functions are pure
+slice, as_type, bitcast are all native callbacks).  The one exception is an optimisation: the cipher
+over a counter range is wrapped in a block (`Nx.BlockThreefry`), which the device backend answers
+with the same words from one kernel instead of about 110 launches.  Keys are `u32[2]` tensors; functions are pure
 and return `(sample, new_key)` like the reference, the `*_split` variants take a key that has
 already been split.  Complex types and `shuffle`, `choice`, `gumbel`, `multivariate_normal` are
 not mirrored.
@@ -90,13 +90,18 @@ def fold_in(key: Tensor, data) -> Tensor:
 
 def threefry2x32(key: Tensor, shape) -> Tensor:
     """random.ex:214-229: the block cipher over the counters 0 .. size-1, keyed by `key`; an odd
-    count is padded with one zero counter whose output is dropped."""
+    count is padded with one zero counter whose output is dropped.  Offered to the key's backend
+    as a block; the default is the reference's composition."""
     shape = tuple(shape)
+    if _COMPOSE_ONLY[0]:
+        return _threefry2x32_composed(key, shape)
+    return Nx.block(Nx.BlockThreefry(shape), [key], template(("u", 32), shape),
+                    lambda _struct, key_: _threefry2x32_composed(key_, shape))
+
+
+def _threefry2x32_composed(key: Tensor, shape) -> Tensor:
     size = prod(shape)
-    backend = type(key.data)
-    fused = None if _COMPOSE_ONLY[0] else getattr(backend, "threefry2x32", None)
-    if fused is not None:  # a backend may produce the same words in one step
-        return fused(template(("u", 32), shape), key)
+    backend = type(key.data)  # the expression builder while a function is traced
     if size % 2 == 0:
         xs = Nx.iota((2, size // 2), type="u32", backend=backend)
         return Nx.reshape(threefry2x32_20_concat(xs, key), shape)

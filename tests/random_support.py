@@ -15,7 +15,7 @@ CASES = load_cases("nx_random_known_answers.json")
 LOOSE_RTOL = {("bf", 16): 2.0 ** -7, ("f", 16): 2.0 ** -9, ("f", 32): 2.0 ** -21, ("f", 64): 2.0 ** -40}
 
 
-def run_random_case(case, backend):
+def run_random_case(case, backend, through=None):
     seed = zlib.adler32(case["seed_of_name"].encode()) if "seed_of_name" in case else case["seed"]
     key = Random.key(seed, backend=backend)
     fn = case["fn"]
@@ -25,12 +25,16 @@ def run_random_case(case, backend):
     opts = dict(case.get("opts", {}))
     if "shape" in opts:
         opts["shape"] = tuple(opts["shape"])
-    out = getattr(Random, fn)(key, *args, **opts)
+    fun = getattr(Random, fn)
+    if through is not None:  # e.g. defn.jit: the options are static, the key and operands are arguments
+        fun = through(fun, **opts)
+        opts = {}
+    out = fun(key, *args, **opts)
     return out[0] if isinstance(out, tuple) else out  # (sample, new_key) for the unsplit variants
 
 
-def check_random_case(case, backend):
-    result = run_random_case(case, backend)
+def check_random_case(case, backend, through=None):
+    result = run_random_case(case, backend, through)
     assert type(result.data) is backend, f"{case['name']}: result left the backend of the key"
     exp = case["expect"]
     ty = T.normalize(exp["t"])

@@ -1,0 +1,239 @@
+"""The traced-function layer (nx_amd/defn.py) on the CPU, with the oracle as the compute backend:
+the rewrites of the expression builder (they change float results, so they are part of parity), the
+evaluator against eager execution, scopes and reference counts, and `Nx.Random` through a trace
+against the reference's known answers."""
+import numpy as np
+import pytest
+
+from nx_amd import defn
+from nx_amd import nx as Nx
+from nx_amd import random as Random
+from nx_amd.defn import Expr
+from random_support import CASES, check_random_case
+from support import assert_bits_equal, from_numpy
+
+
+@pytest.fixture()
+def on_oracle(oracle):
+    previous = Nx.default_backend(oracle)
+    yield oracle
+    Nx.default_backend(*previous)
+
+
+def traced(fun, *args):
+    """The root expressions of `fun` traced on `args`."""
+    return defn.trace(fun, args).roots
+
+
+def f32(values, backend):
+    return from_numpy(np.asarray(values, dtype=np.float32), "f32", backend)
+
+
+# ---- the builder's rewrites (nx/lib/nx/defn/expr.ex:889-984, 1597-1674) -------------------------
+
+def test_constant_factors_merge_and_move_left(on_oracle):
+    x = f32([1, 2, 3], on_oracle)
+    (root,) = traced(lambda t: Nx.multiply(3.0, Nx.multiply(t, 5.0)), x)
+    assert root.data.op == "multiply"
+    const, rest = root.data.args
+    assert const.data.op == "constant" and const.data.args == [15.0] and rest.data.op == "parameter"
+
+
+def test_constant_of_an_inner_product_is_pulled_out(on_oracle):
+    # d * (c * e) with d not a constant becomes c * (d * e): the order the reference multiplies in
+    x = f32([1, 2, 3], on_oracle)
+    (root,) = traced(lambda t, d: Nx.multiply(d, Nx.multiply(1.5, t)), x, f32([4, 5, 6], on_oracle))
+    const, inner = root.data.args
+    assert const.data.args == [1.5] and inner.data.op == "multiply"
+    assert [a.data.op for a in inner.data.args] == ["parameter", "parameter"]
+
+
+def test_neutral_elements_vanish(on_oracle):
+    x = f32([1, 2, 3], on_oracle)
+    for fun in (lambda t: Nx.add(t, 0), lambda t: Nx.multiply(1, t), lambda t: Nx.subtract(t, 0.0),
+                lambda t: Nx.divide(t, 1), lambda t: Nx.pow(t, 1)):
+        (root,) = traced(fun, x)
+        assert root.data.op == "parameter"
+    (root,) = traced(lambda t: Nx.add(t, Nx.subtract(0, t)), x)
+    assert root.data.op == "subtract"
+    (root,) = traced(lambda t: Nx.multiply(t, Nx.divide(1, t)), x)
+    assert root.data.op == "divide"
+
+
+def test_operations_on_constants_fold(on_oracle):
+    x = f32([1, 2, 3], on_oracle)
+    (root,) = traced(lambda t: Nx.multiply(t, Nx.sqrt(Nx.tensor(2.0, type="f32"))), x)
+    const = root.data.args[0]
+    assert const.data.op == "constant" and const.data.args == [float(np.sqrt(np.float32(2.0)))]  # rounded to f32
+    (root,) = traced(lambda t: Nx.add(t, Nx.subtract(1.0, 0.25)), x)
+    assert root.data.args[0].data.args == [0.75]
+    (root,) = traced(lambda t: Nx.add(t, Nx.as_type(Nx.max(3, 4), "f32")), x)
+    assert root.data.args[0].data.args == [4.0]
+
+
+def test_squeezes_and_broadcasts_collapse(on_oracle):
+    x = from_numpy(np.zeros((1, 3, 1, 4), dtype=np.float32), "f32", on_oracle)
+    (root,) = traced(lambda t: Nx.squeeze(Nx.squeeze(t, axes=[0]), axes=[1]), x)
+    assert root.data.op == "squeeze" and root.data.args[1] == [0, 2] and root.data.args[0].data.op == "parameter"
+    v = f32([1, 2, 3], on_oracle)
+    (root,) = traced(lambda t: Nx.broadcast(Nx.broadcast(t, (2, 3)), (4, 2, 3)), v)
+    assert root.data.op == "broadcast" and root.data.args[0].data.op == "parameter" and root.shape == (4, 2, 3)
+    (root,) = traced(lambda t: Nx.add(t, Nx.broadcast(2.0, (3,))), v)
+    assert root.data.args[0].data.op == "constant"
+
+
+def test_captured_compute_tensor_is_refused(on_oracle):
+    outside = f32([1, 2, 3], on_oracle)
+    with pytest.raises(ValueError, match="incompatible tensor implementations"):
+        defn.jit(lambda t: Nx.add(t, outside))(f32([1, 2, 3], on_oracle))
+
+
+def test_expressions_have_no_value(on_oracle):
+    with pytest.raises(ValueError, match="cannot read the value"):
+        defn.jit(lambda t: Nx.to_binary(t))(f32([1.0], on_oracle))
+
+
+# ---- evaluation -----------------------------------------------------------------------------------
+
+def softmax(t):
+    z = Nx.multiply(Nx.as_type(t, "f32"), 0.125)
+    e = Nx.exp(Nx.subtract(z, Nx.reduce_max(z, axes=[-1], keep_axes=True)))
+    return Nx.divide(e, Nx.sum(e, axes=[-1], keep_axes=True))
+
+
+def elementwise_reduce(x, y):
+    return Nx.sum(Nx.exp(Nx.multiply(Nx.add(x, y), 0.5)), axes=[1])
+
+
+def linear_int8(xq, w, scales):
+    return Nx.multiply(Nx.as_type(Nx.dot(xq, [1], w, [1], out_type="s32"), "f32"), scales)
+
+
+def argmax_take(logits, table):
+    return Nx.take(table, Nx.argmax(logits, axis=1, type="u32"))
+
+
+def build_args(backend):
+    rng = np.random.default_rng(7)
+    return {
+        "softmax": (from_numpy((rng.standard_normal((4, 16, 16)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16), "bf16", backend),),
+        "elementwise_reduce": (f32(rng.standard_normal((33, 65)), backend), f32(rng.standard_normal((33, 65)), backend)),
+        "linear_int8": (from_numpy(rng.integers(-128, 128, (8, 64), dtype=np.int8), "s8", backend),
+                        from_numpy(rng.integers(-128, 128, (48, 64), dtype=np.int8), "s8", backend),
+                        f32(rng.uniform(0.01, 0.1, (48,)), backend)),
+        "argmax_take": (f32(rng.standard_normal((16, 100)), backend),
+                        from_numpy((rng.standard_normal((100, 24)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16), "bf16", backend)),
+    }
+
+
+CHAINS = {"softmax": softmax, "elementwise_reduce": elementwise_reduce, "linear_int8": linear_int8, "argmax_take": argmax_take}
+
+
+@pytest.mark.parametrize("name", sorted(CHAINS))
+def test_jitted_chain_equals_eager(name, on_oracle):
+    args = build_args(on_oracle)[name]
+    assert_bits_equal(defn.jit(CHAINS[name])(*args), CHAINS[name](*args), name)
+    compiled = defn.compile(CHAINS[name], *args)
+    assert_bits_equal(compiled(*args), CHAINS[name](*args), f"{name} compiled")
+    assert_bits_equal(compiled(*args), CHAINS[name](*args), f"{name} compiled, second call")
+
+
+def test_composite_arguments_and_results(on_oracle):
+    a, b = f32([1, 2, 3], on_oracle), f32([10, 20, 30], on_oracle)
+    out = defn.jit(lambda pair, scale: {"sum": Nx.add(pair[0], pair[1]), "scaled": (Nx.multiply(pair[0], scale),)})((a, b), 2.0)
+    assert Nx.to_numpy(out["sum"]).tolist() == [11, 22, 33] and Nx.to_numpy(out["scaled"][0]).tolist() == [2, 4, 6]
+
+
+def test_while_loop(on_oracle):
+    def power_iteration(m, v):
+        def body(state):
+            i, vec = state
+            w = Nx.dot(m, vec)
+            return Nx.add(i, 1), Nx.divide(w, Nx.sqrt(Nx.sum(Nx.multiply(w, w))))
+        _, vec = defn.while_loop((Nx.tensor(0), v), lambda s: Nx.less(s[0], 20), body)
+        return vec
+    m = f32([[2, 1], [1, 3]], on_oracle)
+    v = f32([1, 0], on_oracle)
+    assert_bits_equal(defn.jit(power_iteration)(m, v), power_iteration(m, v), "power iteration")
+
+
+def test_while_reads_the_enclosing_scope_without_consuming_it(on_oracle):
+    def fun(x):
+        shifted = Nx.add(x, 1.0)  # used inside the loop on every trip and after it
+        _, acc = defn.while_loop((Nx.tensor(0), shifted), lambda s: Nx.less(s[0], 3),
+                                 lambda s: (Nx.add(s[0], 1), Nx.add(s[1], s[1])))
+        return Nx.subtract(acc, shifted)
+    x = f32([1, 2], on_oracle)
+    assert Nx.to_numpy(defn.jit(fun)(x)).tolist() == [14.0, 21.0]
+
+
+def test_cond_evaluates_one_branch(on_oracle):
+    calls = []
+
+    class Counting(on_oracle):
+        @classmethod
+        def exp(cls, out, t):
+            calls.append("exp")
+            return super().exp(out, t)
+
+    def fun(x):
+        shared = Nx.multiply(x, 2.0)
+        return defn.cond(Nx.greater(Nx.sum(x), 0.0), lambda: Nx.add(shared, 1.0), lambda: Nx.exp(shared))
+    x = from_numpy(np.asarray([1, 2], dtype=np.float32), "f32", Counting)
+    previous = Nx.default_backend(Counting)
+    try:
+        assert Nx.to_numpy(defn.jit(fun)(x)).tolist() == [3.0, 5.0]
+        assert calls == []
+        y = from_numpy(np.asarray([-1, -2], dtype=np.float32), "f32", Counting)
+        assert np.allclose(Nx.to_numpy(defn.jit(fun)(y)), np.exp([-2.0, -4.0]))
+        assert calls == ["exp"]
+    finally:
+        Nx.default_backend(*previous)
+
+
+def test_results_are_dropped_after_their_last_use(on_oracle):
+    """Walks a chain and records how many intermediate results the evaluator still holds."""
+    held = []
+    original = defn._Run.apply
+
+    def spying(self, e, x, scope):
+        held.append(len(scope.results))
+        return original(self, e, x, scope)
+    defn._Run.apply = spying
+    try:
+        def chain(t):
+            for _ in range(10):
+                t = Nx.exp(Nx.negate(t))
+            return t
+        defn.jit(chain)(f32([0.5, 1.5], on_oracle))
+    finally:
+        defn._Run.apply = original
+    assert max(held) <= 1, held  # a straight chain never holds more than the operand in flight
+
+
+def test_shared_node_is_computed_once(on_oracle):
+    calls = []
+
+    class Counting(on_oracle):
+        @classmethod
+        def exp(cls, out, t):
+            calls.append(1)
+            return super().exp(out, t)
+
+    def fun(x):
+        e = Nx.exp(x)
+        return Nx.add(Nx.multiply(e, e), e)
+    x = from_numpy(np.asarray([0.0, 1.0], dtype=np.float32), "f32", Counting)
+    previous = Nx.default_backend(Counting)
+    try:
+        defn.jit(fun)(x)
+    finally:
+        Nx.default_backend(*previous)
+    assert len(calls) == 1
+
+
+# ---- Nx.Random as a traced function -----------------------------------------------------------------
+
+@pytest.mark.parametrize("case", [c for c in CASES if c["fn"] != "key"], ids=[c["name"] for c in CASES if c["fn"] != "key"])
+def test_random_known_answers_through_a_trace(case, on_oracle):
+    check_random_case(case, on_oracle, through=defn.jit)
