@@ -238,6 +238,49 @@ def main():
         # bits out; shift, or, subtract, multiply, add, max each read and write the array once
         entry("uniform_f32_2p28_unfused", 4.0 * nw * 13, "GB/s", ms, PEAK_HBM_GBS, "hbm")
         del key
+
+        # traced chains: one callback per node (the evaluator), and the same chain captured once and
+        # replayed as a device graph (one submission for all its kernels)
+        from nx_amd import defn
+
+        def chain1(a, b):
+            return Nx.sum(Nx.exp(Nx.multiply(Nx.add(a, b), 0.5)), axes=[1])
+
+        def chain3(scores):
+            z = Nx.multiply(Nx.as_type(scores, "f32"), 0.125)
+            e = Nx.exp(Nx.subtract(z, Nx.reduce_max(z, axes=[2], keep_axes=True)))
+            return Nx.divide(e, Nx.sum(e, axes=[2], keep_axes=True))
+
+        def chain4(xq_, w_, sc_):
+            return Nx.multiply(Nx.as_type(Nx.dot(xq_, [1], w_, [1], out_type="s32"), "f32"), sc_)
+        x, y = W.elementwise_reduce(n=1024)
+        q, k = W.attention_scores()
+        w, xq, sc = W.int8_linear()
+        q, k = put(q, "bf16"), put(k, "bf16")
+        cases = {"config1_chain_f32_1024": (chain1, (put(x, "f32"), put(y, "f32")), 32.0 * 1024 * 1024 + 4096.0),
+                 "softmax_chain_32x512x512": (chain3, (Nx.dot(q, [2], [0], k, [2], [0]),), 386138112.0),
+                 "config4_chain": (chain4, (put(xq, "s8"), put(w, "s8"), put(sc, "f32")), 48168960.0 + 5636096.0 + 5680128.0)}
+        for name, (fun, targs, nbytes) in cases.items():
+            compiled = defn.compile(fun, *targs)
+            _, ms = timed(lambda: compiled(*targs), steps, warm)
+            entry(name + "_traced", nbytes, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+            captured = compiled.capture(*targs)
+            held = captured.inputs  # arguments already in the captured buffers: no copies in
+            _, ms = timed(lambda: captured(*held), steps, warm)
+            entry(name + "_graph", nbytes, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+            captured.destroy()
+            fused = defn.compile(fun, *targs, fuse=True)
+            _, ms = timed(lambda: fused(*targs), steps, warm)
+            entry(name + "_fused", nbytes, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+        x, y = W.elementwise_reduce(n=16384)
+        big = (put(x, "f32"), put(y, "f32"))
+        fused = defn.compile(chain1, *big, fuse=True)
+        _, ms = timed(lambda: fused(*big), steps, warm)
+        # priced at the bytes of the node-by-node chain, like the unfused entry: above 1.0 means the fused
+        # pass beats what the reference's formulation can reach at all
+        entry("config1_chain_f32_16384_fused", 32.0 * 16384 * 16384 + 4.0 * 16384, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+        del big, x, y
+        del cases, q, k
         result["suite"] = suite
 
     # ---- CPU baseline: the reference-semantics restatement on a bounded sample -----------------

@@ -31,6 +31,7 @@ extern "C" {
 
 typedef struct hipnx_ctx hipnx_ctx;
 typedef struct hipnx_buf hipnx_buf;
+typedef struct hipnx_graph hipnx_graph;
 
 /* status codes */
 enum {
@@ -228,6 +229,52 @@ int hipnx_eye(hipnx_ctx *ctx, int out_dt, int64_t n, int64_t rows, int64_t cols,
  * counter whose output is dropped).  Not a Nx.Backend callback: a binding calls it from its
  * own random module when the key lives on the device. */
 int hipnx_threefry2x32(hipnx_ctx *ctx, const hipnx_buf *key, int64_t n, hipnx_buf *out);
+
+/* ---- fused element-wise chains ----------------------------------------------------------------
+ * replaces: a group of element-wise callbacks that the reference's evaluator issues one by one
+ * (nx/lib/nx/defn/evaluator.ex:363-388; the callbacks of nx/lib/nx/backend.ex:115-133) by one pass
+ * over memory.  The group is a register program: every instruction writes one of
+ * HIPNX_FUSED_REGS registers and rounds its value to `dt`, the type the node has in the
+ * graph, so the result is what the separate kernels would have produced.
+ * Input k starts out in register k (converted to f32; its element (row, col) is at
+ * row * row_stride + col * col_stride), so at most HIPNX_FUSED_REGS inputs.
+ *   CONST  dst = imm
+ *   UNARY  dst = op(reg a)        op: HIPNX_EXP ... (not the integer-only ones)
+ *   BINARY dst = op(reg a, reg b) op: HIPNX_ADD ... (not the integer-only ones)
+ *   SELECT dst = reg a != 0 ? reg b : reg c
+ *   AS_TYPE dst = reg a (rounded to dt)
+ * Types: bf16 / f16 / f32 values, u8 truth values; inputs of at most 4 bytes per element.  The
+ * index space is [rows, cols]; col strides are 1 or 0; with more than one row, cols and the row
+ * strides of dense inputs are multiples of 8 (otherwise HIPNX_EUNSUPPORTED: run the nodes one by one). */
+enum { HIPNX_FUSED_CONST = 1, HIPNX_FUSED_UNARY, HIPNX_FUSED_BINARY, HIPNX_FUSED_SELECT, HIPNX_FUSED_AS_TYPE };
+enum { HIPNX_FUSED_REGS = 8, HIPNX_FUSED_MAX_INSTR = 32, HIPNX_FUSED_MAX_INPUTS = 7 };
+typedef struct {
+  uint8_t kind, op, dst, a, b, c, dt, pad;
+  float imm;
+  uint32_t reserved;  /* 16 bytes: the interpreter fetches an instruction with one scalar load */
+} hipnx_fused_instr;
+int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_fused_instr *prog, int n_inputs,
+                            const hipnx_buf *const *inputs, const int *in_dts, const int64_t *in_row_strides,
+                            const int *in_col_strides, int64_t rows, int64_t cols, int out_reg, int out_dt,
+                            hipnx_buf *out);
+
+/* ---- captured sequences ---------------------------------------------------------------------
+ * The reference's evaluator (nx/lib/nx/defn/evaluator.ex:363-388) issues one callback per node
+ * on every call of a compiled function; the XLA-based backend compiles the function instead
+ * (exla/lib/exla/defn.ex).  This is the device-side middle: between capture_begin and
+ * capture_end the entry points of the context record their kernels instead of running them,
+ * capture_end turns the record into an executable graph, graph_launch replays it on the
+ * context's stream with one submission.  Every device block handed out while capturing stays
+ * with the graph until graph_destroy (a replay writes to the same addresses), so buffers
+ * allocated during the capture -- the results among them -- are overwritten by each replay.
+ * Entry points that wait for the device (h2d, d2h, sync, trim, the timer, gather with
+ * HIPNX_OOB_RAISE) return HIPNX_EUNSUPPORTED while capturing.  Run the sequence once before
+ * capturing it: kernel attributes are set and the pool holds its block sizes after that.  One
+ * thread drives a capture; graphs must be destroyed before their context. */
+int hipnx_capture_begin(hipnx_ctx *ctx);
+int hipnx_capture_end(hipnx_ctx *ctx, hipnx_graph **out);
+int hipnx_graph_launch(hipnx_graph *graph);
+int hipnx_graph_destroy(hipnx_graph *graph);
 
 #ifdef __cplusplus
 }

@@ -185,6 +185,11 @@ class HipNxBackend:
         if out.shape == ():
             key = (opts["device"], out.type, elem)
             ref = cls._scalar_cache.get(key)
+            if ref is None and opts["device"] in _capturing:
+                # written only when the captured graph replays: must not be shared with eager code
+                res = cls._alloc(out, opts["device"])
+                L.check(L.lib.hipnx_fill(res.data.ref.ctx, res.data.ref.handle, len(elem), elem, 1))
+                return res
             if ref is None:
                 if len(cls._scalar_cache) >= 1024:
                     cls._scalar_cache.clear()
@@ -594,6 +599,27 @@ class HipNxBackend:
         return cls.concatenate(out, widened, axis)
 
     @classmethod
+    def fused_elementwise(cls, out: Tensor, program, out_reg: int, inputs, layout) -> Tensor:
+        """A group of element-wise nodes in one kernel (the evaluator offers it groups it has found
+        in a traced function).  `program` is a list of (kind, op, dst, a, b, c, type, imm); `layout` is
+        (rows, cols, [(row_stride, col_stride) per input]).  Raises HipNxError with status
+        EUNSUPPORTED when the shapes do not vectorise: the caller then runs the nodes one by one."""
+        dev = cls._device_of(*inputs)
+        inputs = [cls._from_nx(t, dev) for t in inputs]
+        rows, cols, strides = layout
+        prog = (L.FusedInstr * len(program))()
+        for q, (kind, op, dst, a, b, c, ty, imm) in zip(prog, program):
+            q.kind, q.op, q.dst, q.a, q.b, q.c, q.dt, q.imm = kind, op, dst, a, b, c, T.code(ty), imm
+        res = cls._alloc(out, dev)
+        handles = (C.c_void_p * max(len(inputs), 1))(*[cls._handle(t) for t in inputs])
+        dts = (C.c_int * max(len(inputs), 1))(*[T.code(t.type) for t in inputs])
+        rs = (C.c_int64 * max(len(inputs), 1))(*[s[0] for s in strides])
+        cs = (C.c_int * max(len(inputs), 1))(*[s[1] for s in strides])
+        L.check(L.lib.hipnx_fused_elementwise(res.data.ref.ctx, len(program), C.cast(prog, C.c_void_p), len(inputs), handles,
+                                              dts, rs, cs, rows, cols, out_reg, T.code(out.type), res.data.ref.handle))
+        return res
+
+    @classmethod
     def threefry2x32(cls, out: Tensor, key: Tensor) -> Tensor:
         """The random words of Nx.Random's threefry2x32/2 (random.ex:214-285) for `out.size`
         counters in one kernel; `out` is a u32 template.  Reached through block/4 with a
@@ -653,6 +679,53 @@ def timer_stop(device: int = 0) -> float:
     ms = C.c_float()
     L.check(L.lib.hipnx_timer_stop(_Context.get(device), C.byref(ms)))
     return ms.value
+
+
+_capturing = set()  # devices whose context is recording instead of running
+
+
+class DeviceGraph:
+    """A captured sequence of device work (`hipnx_capture_begin` .. `hipnx_capture_end`): `launch`
+    replays it with one submission.  Buffers allocated while capturing belong to the graph; tensors
+    produced then are overwritten by every replay and die with the graph."""
+
+    def __init__(self, handle, device):
+        self.handle, self.device = handle, device
+
+    def launch(self):
+        if self.handle is None:
+            raise L.HipNxError(L.EINVAL, "the graph has been destroyed")
+        L.check(L.lib.hipnx_graph_launch(self.handle))
+
+    def destroy(self):
+        if self.handle is not None:
+            handle, self.handle = self.handle, None
+            L.check(L.lib.hipnx_graph_destroy(handle))
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:  # interpreter shutdown: the context may be gone already
+            pass
+
+
+def copy_into(dst: Tensor, src: Tensor) -> None:
+    """Overwrites the device memory of `dst` with `src` (same type and shape, same device)."""
+    if (dst.type, dst.shape) != (src.type, src.shape) or dst.data.device != src.data.device:
+        raise ValueError("copy_into needs two device tensors of one type, shape and device")
+    L.check(L.lib.hipnx_d2d(dst.data.ref.ctx, HipNxBackend._handle(dst), 0, HipNxBackend._handle(src), 0, dst.data.ref.nbytes))
+
+
+def capture_begin(device: int = 0) -> None:
+    L.check(L.lib.hipnx_capture_begin(_Context.get(device)))
+    _capturing.add(device)
+
+
+def capture_end(device: int = 0) -> DeviceGraph:
+    _capturing.discard(device)
+    handle = C.c_void_p()
+    L.check(L.lib.hipnx_capture_end(_Context.get(device), C.byref(handle)))
+    return DeviceGraph(handle, device)
 
 
 def mem_stats(device: int = 0):

@@ -66,6 +66,17 @@ static size_t round_capacity(size_t bytes) {
 int pool_alloc(hipnx_ctx *ctx, size_t bytes, void **ptr_out, size_t *cap_out) {
   size_t cap = round_capacity(bytes);
   void *ptr = nullptr;
+  if (ctx->capture) {  // blocks released earlier in this capture come first: they already belong to the graph
+    auto own = ctx->capture->parked.lower_bound(cap);
+    if (own != ctx->capture->parked.end() && own->first <= cap + cap / 4) {
+      *ptr_out = own->second;
+      *cap_out = own->first;
+      ctx->live += own->first;
+      if (ctx->live > ctx->peak) ctx->peak = ctx->live;
+      ctx->capture->parked.erase(own);
+      return HIPNX_OK;
+    }
+  }
   auto it = ctx->pool.lower_bound(cap);
   if (it != ctx->pool.end() && it->first <= cap + cap / 4) {
     ptr = it->second;
@@ -74,7 +85,7 @@ int pool_alloc(hipnx_ctx *ctx, size_t bytes, void **ptr_out, size_t *cap_out) {
     ctx->pool.erase(it);
   } else {
     hipError_t e = hipMalloc(&ptr, cap);
-    if (e != hipSuccess && !ctx->pool.empty()) {
+    if (e != hipSuccess && !ctx->pool.empty() && !ctx->capture) {
       // give cached blocks back and retry once
       (void)hipGetLastError();
       (void)hipStreamSynchronize(ctx->stream);
@@ -87,6 +98,10 @@ int pool_alloc(hipnx_ctx *ctx, size_t bytes, void **ptr_out, size_t *cap_out) {
   }
   ctx->live += cap;
   if (ctx->live > ctx->peak) ctx->peak = ctx->live;
+  if (ctx->capture) {
+    ctx->capture->owned.emplace_back(ptr, cap);
+    ctx->graph_blocks[ptr] = ctx->capture;
+  }
   *ptr_out = ptr;
   *cap_out = cap;
   return HIPNX_OK;
@@ -94,7 +109,12 @@ int pool_alloc(hipnx_ctx *ctx, size_t bytes, void **ptr_out, size_t *cap_out) {
 
 int pool_free(hipnx_ctx *ctx, void *ptr, size_t cap) {
   ctx->live -= cap;
-  if (ctx->pooled + cap <= pool_cap_bytes()) {
+  auto owner = ctx->graph_blocks.find(ptr);
+  if (owner != ctx->graph_blocks.end()) {  // stays with its graph, whenever it is released
+    owner->second->parked.emplace(cap, ptr);
+    return HIPNX_OK;
+  }
+  if (ctx->pooled + cap <= pool_cap_bytes() || ctx->capture) {
     // reuse without a device wait is safe: all work of this context is ordered on one stream
     ctx->pool.emplace(cap, ptr);
     ctx->pooled += cap;
@@ -166,6 +186,13 @@ int hipnx_ctx_destroy(hipnx_ctx *ctx) {
   if (!ctx) return set_error(HIPNX_EINVAL, "null context");
   (void)hipSetDevice(ctx->device);
   if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+  for (hipnx_graph *g : ctx->graphs) {  // handles to them are dead from here on, like buffer handles
+    if (g->exec) (void)hipGraphExecDestroy(g->exec);
+    if (g->graph) (void)hipGraphDestroy(g->graph);
+    for (auto &kv : g->parked) (void)hipFree(kv.second);
+    delete g;
+  }
+  ctx->graphs.clear();
   for (auto &kv : ctx->pool) (void)hipFree(kv.second);
   ctx->pool.clear();
   if (ctx->flag) (void)hipFree(ctx->flag);
@@ -180,6 +207,7 @@ int hipnx_ctx_destroy(hipnx_ctx *ctx) {
 int hipnx_sync(hipnx_ctx *ctx) {
   Enter in(ctx);
   if (in.status) return in.status;
+  HIPNX_NOT_CAPTURING(ctx, "sync");
   HIPNX_HIP(hipStreamSynchronize(ctx->stream));
   return HIPNX_OK;
 }
@@ -196,6 +224,7 @@ int hipnx_mem_stats(hipnx_ctx *ctx, uint64_t *live, uint64_t *peak, uint64_t *po
 int hipnx_trim(hipnx_ctx *ctx) {
   Enter in(ctx);
   if (in.status) return in.status;
+  HIPNX_NOT_CAPTURING(ctx, "trim");
   HIPNX_HIP(hipStreamSynchronize(ctx->stream));
   for (auto &kv : ctx->pool) (void)hipFree(kv.second);
   ctx->pool.clear();
@@ -206,6 +235,7 @@ int hipnx_trim(hipnx_ctx *ctx) {
 int hipnx_timer_start(hipnx_ctx *ctx) {
   Enter in(ctx);
   if (in.status) return in.status;
+  HIPNX_NOT_CAPTURING(ctx, "timer");
   HIPNX_HIP(hipEventRecord(ctx->ev_start, ctx->stream));
   return HIPNX_OK;
 }
@@ -214,9 +244,80 @@ int hipnx_timer_stop(hipnx_ctx *ctx, float *elapsed_ms) {
   Enter in(ctx);
   if (in.status) return in.status;
   if (!elapsed_ms) return set_error(HIPNX_EINVAL, "null elapsed_ms");
+  HIPNX_NOT_CAPTURING(ctx, "timer");
   HIPNX_HIP(hipEventRecord(ctx->ev_stop, ctx->stream));
   HIPNX_HIP(hipEventSynchronize(ctx->ev_stop));
   HIPNX_HIP(hipEventElapsedTime(elapsed_ms, ctx->ev_start, ctx->ev_stop));
+  return HIPNX_OK;
+}
+
+// ---- captured graphs -------------------------------------------------------------------------
+
+static void release_graph(hipnx_ctx *ctx, hipnx_graph *g) {
+  for (auto &blk : g->owned) ctx->graph_blocks.erase(blk.first);
+  for (auto &kv : g->parked) {  // blocks still held by buffers go to the pool when those are freed
+    ctx->pool.emplace(kv.first, kv.second);
+    ctx->pooled += kv.first;
+  }
+  for (size_t i = 0; i < ctx->graphs.size(); i++)
+    if (ctx->graphs[i] == g) { ctx->graphs.erase(ctx->graphs.begin() + i); break; }
+  if (g->exec) (void)hipGraphExecDestroy(g->exec);
+  if (g->graph) (void)hipGraphDestroy(g->graph);
+  delete g;
+}
+
+int hipnx_capture_begin(hipnx_ctx *ctx) {
+  Enter in(ctx);
+  if (in.status) return in.status;
+  if (ctx->capture) return set_error(HIPNX_EINVAL, "capture_begin: the context is already capturing");
+  hipnx_graph *g = new hipnx_graph;
+  g->ctx = ctx;
+  // relaxed: a pool miss may still call hipMalloc (run the sequence once before capturing it and there is none)
+  hipError_t e = hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed);
+  if (e != hipSuccess) {
+    delete g;
+    return hip_fail(e, "hipStreamBeginCapture");
+  }
+  ctx->capture = g;
+  ctx->graphs.push_back(g);
+  return HIPNX_OK;
+}
+
+int hipnx_capture_end(hipnx_ctx *ctx, hipnx_graph **out) {
+  Enter in(ctx);
+  if (in.status) return in.status;
+  if (!ctx->capture) return set_error(HIPNX_EINVAL, "capture_end: the context is not capturing");
+  hipnx_graph *g = ctx->capture;
+  ctx->capture = nullptr;
+  hipError_t e = hipStreamEndCapture(ctx->stream, &g->graph);
+  if (e == hipSuccess) e = hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0);
+  if (e != hipSuccess || !out) {
+    release_graph(ctx, g);
+    if (out) *out = nullptr;
+    return e != hipSuccess ? hip_fail(e, "ending the capture") : set_error(HIPNX_EINVAL, "capture_end: null out");
+  }
+  *out = g;
+  return HIPNX_OK;
+}
+
+int hipnx_graph_launch(hipnx_graph *g) {
+  if (!g) return set_error(HIPNX_EINVAL, "null graph");
+  hipnx_ctx *ctx = g->ctx;
+  Enter in(ctx);
+  if (in.status) return in.status;
+  if (ctx->capture) return set_error(HIPNX_EINVAL, "graph_launch: the context is capturing");
+  HIPNX_HIP(hipGraphLaunch(g->exec, ctx->stream));
+  return HIPNX_OK;
+}
+
+int hipnx_graph_destroy(hipnx_graph *g) {
+  if (!g) return set_error(HIPNX_EINVAL, "null graph");
+  hipnx_ctx *ctx = g->ctx;
+  Enter in(ctx);
+  if (in.status) return in.status;
+  if (ctx->capture == g) return set_error(HIPNX_EINVAL, "graph_destroy: this graph is still being captured");
+  if (!ctx->capture) HIPNX_HIP(hipStreamSynchronize(ctx->stream));  // a replay may be in flight
+  release_graph(ctx, g);
   return HIPNX_OK;
 }
 
@@ -271,6 +372,7 @@ int hipnx_h2d(hipnx_ctx *ctx, hipnx_buf *dst, size_t dst_offset, const void *src
   Enter in(ctx);
   if (in.status) return in.status;
   if (int st = check_buf(ctx, dst, (uint64_t)dst_offset + bytes, "h2d dst")) return st;
+  HIPNX_NOT_CAPTURING(ctx, "h2d");
   if (bytes == 0) return HIPNX_OK;
   if (!src) return set_error(HIPNX_EINVAL, "h2d: null source");
   HIPNX_HIP(hipMemcpyAsync((char *)dst->ptr + dst_offset, src, bytes, hipMemcpyHostToDevice, ctx->stream));
@@ -283,6 +385,7 @@ int hipnx_d2h(hipnx_ctx *ctx, const hipnx_buf *src, size_t src_offset, void *dst
   Enter in(ctx);
   if (in.status) return in.status;
   if (int st = check_buf(ctx, src, (uint64_t)src_offset + bytes, "d2h src")) return st;
+  HIPNX_NOT_CAPTURING(ctx, "d2h");
   if (bytes == 0) {
     HIPNX_HIP(hipStreamSynchronize(ctx->stream));
     return HIPNX_OK;

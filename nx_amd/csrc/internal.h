@@ -8,9 +8,24 @@
 #include <cstdio>
 #include <map>
 #include <mutex>
+#include <unordered_map>
 #include <vector>
 
 #include "../../include/hipnx.h"
+
+struct hipnx_ctx;
+
+// A captured sequence of this context's work (stream capture -> executable graph) together with
+// the device blocks it runs in.  Every block handed out while capturing belongs to the graph until
+// the graph is destroyed: a replay writes to the same addresses, so none of them may reach the
+// shared pool (and another owner) in between.
+struct hipnx_graph {
+  hipnx_ctx *ctx = nullptr;
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
+  std::vector<std::pair<void *, size_t>> owned;  // every block allocated during the capture
+  std::multimap<size_t, void *> parked;          // owned blocks that no buffer holds right now
+};
 
 struct hipnx_ctx {
   int device = 0;
@@ -25,6 +40,9 @@ struct hipnx_ctx {
   void *flag = nullptr;       // 32-byte device scratch for the gather bounds report
   void *flag_host = nullptr;  // pinned host word, mapped into the device: non-zero once a kernel saw a bad index
   void *flag_host_dev = nullptr;  // its device address
+  hipnx_graph *capture = nullptr;                        // non-null while the stream is capturing
+  std::unordered_map<void *, hipnx_graph *> graph_blocks;  // block -> the live graph that owns it
+  std::vector<hipnx_graph *> graphs;                     // live graphs of this context
 };
 
 struct hipnx_buf {
@@ -62,6 +80,13 @@ int check_buf(const hipnx_ctx *ctx, const hipnx_buf *b, uint64_t need_bytes, con
 // pooled device memory; both expect the context mutex to be held (i.e. inside an Enter scope)
 int pool_alloc(hipnx_ctx *ctx, size_t bytes, void **ptr_out, size_t *cap_out);
 int pool_free(hipnx_ctx *ctx, void *ptr, size_t cap);
+
+// entry points that wait for the device cannot run while the stream is capturing
+#define HIPNX_NOT_CAPTURING(ctx, what)                                                                 \
+  do {                                                                                                 \
+    if ((ctx)->capture)                                                                                \
+      return hipnx::set_error(HIPNX_EUNSUPPORTED, "%s waits for the device: not possible while capturing", what); \
+  } while (0)
 
 // RAII: select the device and take the context mutex for the duration of an entry point
 struct Enter {

@@ -267,6 +267,7 @@ extern "C" int hipnx_gather(hipnx_ctx *ctx, int elem_bytes, int rank, const int6
                             hipnx_buf *out) {
   Enter in(ctx);
   if (in.status) return in.status;
+  if (oob_policy == HIPNX_OOB_RAISE) HIPNX_NOT_CAPTURING(ctx, "gather with the raising bounds policy");
   if (rank < 0 || rank > 64 || depth < 0 || depth > rank || depth > MAXR || n_tuples < 0 || (rank > 0 && !t_dims))
     return set_error(HIPNX_EINVAL, "gather: bad rank / depth");
   if (elem_bytes <= 0 || dtype_size(idx_dt) < 0 || is_float(idx_dt))

@@ -21,6 +21,7 @@ from __future__ import annotations
 import itertools
 import operator
 import threading
+from math import prod
 from typing import Any, Callable, Dict, List, Optional, Tuple
 
 import numpy as np
@@ -435,6 +436,239 @@ def cond(pred, on_true: Callable, on_false: Callable):
     return _unflatten(structure, results)
 
 
+# ---- fusion of element-wise groups --------------------------------------------------------------------
+# The reference's evaluator knows one granularity: a callback per node.  A backend that offers
+# `fused_elementwise` is handed whole groups of element-wise nodes instead (one pass over memory,
+# intermediates in registers, each still rounded to its node's type: same bits as node by node).
+# Opt-in (`compile(..., fuse=True)`), root scope only; a group that does not fit the kernel's
+# limits, or a backend without the entry point, is evaluated node by node as before.
+
+_NARROW = (("bf", 16), ("f", 16), ("f", 32))
+_TRUTH = ("u", 8)
+_INT_ONLY_BINARY = ("quotient", "bitwise_and", "bitwise_or", "bitwise_xor", "left_shift", "right_shift")
+_INT_ONLY_UNARY = ("bitwise_not", "count_leading_zeros", "population_count")
+_COMPARE = ("equal", "not_equal", "greater", "less", "greater_equal", "less_equal")
+_LOGICAL = ("logical_and", "logical_or", "logical_xor")
+_EXACT_WITH_INT_CONSTANT = ("add", "subtract", "multiply", "divide", "min", "max") + _COMPARE
+_KIND = {"const": 1, "unary": 2, "binary": 3, "select": 4, "as_type": 5}
+_MAX_REGS, _MAX_INSTR, _MAX_INPUTS = 8, 32, 8
+
+
+def _fusable(t: Tensor) -> bool:
+    """Whether the node computes in the f32 class of the element-wise kernels with operands and a
+    result the fused kernel holds exactly."""
+    e = t.data
+    op, args = e.op, e.args
+
+    def value_ok(a, binary_op=None):
+        if _const(a) is not None:
+            if a.type in _NARROW:
+                return True
+            c = _const(a)
+            return binary_op in _EXACT_WITH_INT_CONSTANT and T.is_integer(a.type) and abs(c) <= 1 << 24
+        return a.type in _NARROW
+
+    if op in UNARY_OPS and op not in _INT_ONLY_UNARY:
+        out_ok = t.type == _TRUTH if op in ("is_nan", "is_infinity") else t.type in _NARROW
+        return out_ok and value_ok(args[0])
+    if op in BINARY_OPS and op not in _INT_ONLY_BINARY:
+        if op in _LOGICAL:
+            return t.type == _TRUTH and all(a.type in _NARROW or a.type == _TRUTH for a in args)
+        out_ok = t.type == _TRUTH if op in _COMPARE else t.type in _NARROW
+        return out_ok and all(value_ok(a, op) for a in args)
+    if op == "as_type":
+        src = args[0].type
+        return t.type in _NARROW and (src in _NARROW or (T.is_integer(src) and src[1] <= 32)) and _const(args[0]) is None
+    if op == "select":
+        pred, on_true, on_false = args
+        return (t.type in _NARROW and (pred.type in _NARROW or pred.type == _TRUTH) and _const(pred) is None
+                and value_ok(on_true) and value_ok(on_false))
+    return False
+
+
+def _layout(out_shape, in_shapes):
+    """The index space as [rows, cols] with a (row stride, column stride) per input, or None: an
+    input is the full shape, one value, one row shared by all rows, or one value per row."""
+    rank = len(out_shape)
+    padded = [(1,) * (rank - len(s)) + tuple(s) for s in in_shapes]
+    for p in range(rank + 1):
+        rows, cols = prod(out_shape[:p]), prod(out_shape[p:])
+        if cols % 8:  # the kernel works on whole vectors of 8 along a row
+            continue
+        strides = []
+        for s in padded:
+            outer, inner = s[:p], s[p:]
+            dense_inner, one_inner = inner == tuple(out_shape[p:]), all(d == 1 for d in inner)
+            dense_outer, one_outer = outer == tuple(out_shape[:p]), all(d == 1 for d in outer)
+            if not (dense_inner or one_inner) or not (dense_outer or one_outer):
+                break
+            cs = 1 if dense_inner and cols > 1 else 0
+            rs = (cols if cs else 1) if dense_outer and rows > 1 else 0
+            if cs and rows > 1 and rs % 8:
+                break
+            strides.append((rs, cs))
+        else:
+            return rows, cols, strides
+    return None
+
+
+class _Group:
+    """One fused group: the member nodes in evaluation order, its external inputs, and the register
+    program for them (None when the group does not fit the kernel)."""
+
+    def __init__(self, root: Tensor, members: List[Tensor], inputs: List[Tensor]):
+        self.root, self.members, self.inputs = root, members, inputs
+        self.program, self.out_reg = self._assemble()
+        self.layout = _layout(root.shape, [t.shape for t in inputs]) if self.program else None
+
+    def _assemble(self):
+        member_ids = {m.data.id: i for i, m in enumerate(self.members)}
+        input_ids = {t.data.id: k for k, t in enumerate(self.inputs)}
+        if len(self.inputs) >= _MAX_REGS:
+            return None, None
+
+        def key(a):
+            if _const(a) is not None:
+                return ("c", a.type, _const(a))
+            return ("m", a.data.id) if a.data.id in member_ids else ("i", input_ids[a.data.id])
+
+        last_use: Dict[Any, int] = {}
+        for i, m in enumerate(self.members):
+            for a in m.data.args:
+                if isinstance(a, Tensor):
+                    last_use[key(a)] = i
+        last_use[("m", self.root.data.id)] = len(self.members)
+        # input k starts out in register k; the others are handed out as values are born
+        where = {("i", k): k for k in range(len(self.inputs))}
+        free, program = list(range(len(self.inputs), _MAX_REGS)), []
+
+        def claim():
+            return free.pop(0) if free else None
+
+        for k in range(len(self.inputs)):  # an input nobody reads (cannot happen) would hold its register
+            if ("i", k) not in last_use:
+                free.append(where.pop(("i", k)))
+        for i, m in enumerate(self.members):
+            operands = [a for a in m.data.args if isinstance(a, Tensor)]
+            for a in operands:
+                k = key(a)
+                if k in where:
+                    continue
+                reg = claim()  # only constants are born here: inputs and earlier members have registers
+                if reg is None:
+                    return None, None
+                where[k] = reg
+                program.append((_KIND["const"], 0, reg, 0, 0, 0, a.type if a.type in _NARROW else ("f", 32), _imm(a)))
+            regs = [where[key(a)] for a in operands]
+            for a in operands:  # operands read for the last time free their registers for the result
+                k = key(a)
+                if last_use.get(k) == i and k in where:
+                    free.insert(0, where.pop(k))
+            dst = claim()
+            if dst is None:
+                return None, None
+            where[("m", m.data.id)] = dst
+            op = m.data.op
+            if op in UNARY_OPS:
+                program.append((_KIND["unary"], UNARY_OPS.index(op), dst, regs[0], 0, 0, m.type, 0.0))
+            elif op in BINARY_OPS:
+                program.append((_KIND["binary"], BINARY_OPS.index(op), dst, regs[0], regs[1], 0, m.type, 0.0))
+            elif op == "select":
+                program.append((_KIND["select"], 0, dst, regs[0], regs[1], regs[2], m.type, 0.0))
+            else:
+                program.append((_KIND["as_type"], 0, dst, regs[0], 0, 0, m.type, 0.0))
+            if len(program) > _MAX_INSTR:
+                return None, None
+        return program, where[("m", self.root.data.id)]
+
+    def run(self, run: "_Run", out: Tensor, values: List[Tensor]):
+        mod = run.pick(values)
+        fused = getattr(mod, "fused_elementwise", None) if self.program and self.layout else None
+        if fused is not None:
+            return fused(out, self.program, self.out_reg, values, self.layout)
+        # node by node, on the callbacks (a backend without the kernel, or a group that does not fit)
+        done = {t.data.id: v for t, v in zip(self.inputs, values)}
+        for m in self.members:
+            args = []
+            for a in m.data.args:
+                if isinstance(a, Tensor):
+                    args.append(done[a.data.id] if a.data.id in done else run.eval(a, None))
+                else:
+                    args.append(a)
+            done[m.data.id] = getattr(run.pick(args), m.data.op)(m.with_(data=None), *args)
+        return done[self.root.data.id]
+
+
+def _imm(a: Tensor) -> float:
+    """The constant as the f32 the kernels would load: encoded in its type, decoded again."""
+    from .tensor import number_to_binary
+    ty = a.type if a.type in _NARROW else ("f", 32)
+    raw = np.frombuffer(number_to_binary(_const(a), ty), dtype=T.numpy_dtype(ty))
+    if ty == ("bf", 16):
+        return float((raw.astype(np.uint32) << 16).view(np.float32)[0])
+    return float(raw.astype(np.float32)[0])
+
+
+def _fuse(roots: List[Tensor]) -> int:
+    """Rewrites element-wise groups of the root scope into `fused` nodes, in place; returns how
+    many groups were formed."""
+    order, uses, seen = [], {}, set()
+
+    def walk(t):
+        e = t.data
+        if e.op in ("constant", "tensor") or e.scope != 0:
+            return
+        uses[e.id] = uses.get(e.id, 0) + 1
+        if e.id in seen:
+            return
+        seen.add(e.id)
+        for child in _children(e):
+            if isinstance(child, Tensor):
+                walk(child)
+        order.append(t)
+
+    for r in roots:
+        walk(r)
+    taken, formed = set(), 0
+    for root in reversed(order):  # consumers first: a group grows from its last node upwards
+        if root.data.id in taken or not _fusable(root):
+            continue
+        members, inside = {root.data.id: root}, {}
+        changed = True
+        while changed:
+            changed = False
+            inside.clear()
+            for m in members.values():
+                for a in m.data.args:
+                    if isinstance(a, Tensor) and isinstance(a.data, Expr) and a.data.op != "constant":
+                        inside[a.data.id] = inside.get(a.data.id, 0) + 1
+            for m in list(members.values()):
+                for a in m.data.args:
+                    if (isinstance(a, Tensor) and isinstance(a.data, Expr) and a.data.id not in members
+                            and a.data.id not in taken and a.data.op not in ("constant", "tensor") and a.data.scope == 0
+                            and a.shape == root.shape and _fusable(a) and inside[a.data.id] == uses.get(a.data.id)):
+                        members[a.data.id] = a
+                        changed = True
+        if len(members) < 2:
+            continue
+        ordered = [t for t in order if t.data.id in members]
+        inputs, input_seen = [], set()
+        for m in ordered:
+            for a in m.data.args:
+                if (isinstance(a, Tensor) and _const(a) is None and a.data.id not in members
+                        and a.data.id not in input_seen):
+                    input_seen.add(a.data.id)
+                    inputs.append(a)
+        # the members keep their own nodes for the node-by-node path; the root becomes the group
+        inner_root = root.with_(data=Expr(next(_ids), root.data.op, root.data.args, 0))
+        ordered[-1] = inner_root
+        group = _Group(inner_root, ordered, inputs)
+        taken.update(members)
+        root.data.op, root.data.args = "fused", [group, inputs]
+        formed += 1
+    return formed
+
+
 # ---- the evaluator ----------------------------------------------------------------------------------
 
 CREATION_OPS = ("eye", "iota")           # evaluator.ex:26-28
@@ -577,6 +811,9 @@ class _Run:
             for tag, _ in branches:
                 self.release_outer(self.plans[tag], scope)
             return result
+        if op == "fused":
+            group, inputs = e.args
+            return group.run(self, x.with_(data=None), [self.eval(t, scope) for t in inputs])
         if op == "block":
             struct, in_args, fun = e.args
             args = [self.eval(a, scope) for a in in_args]
@@ -612,26 +849,85 @@ class _Run:
 class Compiled:
     """A traced function: call it with arguments of the traced shapes and types."""
 
-    def __init__(self, roots, structure, n_params):
-        self.roots, self.structure, self.n_params = roots, structure, n_params
+    def __init__(self, roots, structure, templates):
+        self.roots, self.structure, self.templates = roots, structure, templates
+        self.n_params = len(templates)
         self.plans: Dict[Any, _Plan] = {}
         self.plan = _Plan(roots, 0, self.plans)
 
-    def __call__(self, *args):
+    def _params(self, args):
         leaves: list = []
         _flatten(list(args), leaves)
         if len(leaves) != self.n_params:
             raise ValueError(f"expected {self.n_params} tensor arguments, got {len(leaves)}")
         params = [Nx.to_tensor(v) for v in leaves]
-        backend = _runtime_backend(params)
-        run = _Run(self.plans, backend)
+        for i, (p, t) in enumerate(zip(params, self.templates)):
+            if (p.type, p.shape) != (t.type, t.shape):
+                raise ValueError(f"argument {i} is {p.type!r}{p.shape!r}, the function was traced for {t.type!r}{t.shape!r}")
+        return params
+
+    def _evaluate(self, params):
+        run = _Run(self.plans, _runtime_backend(params))
         root = _Scope(self.plan, None, params)
         results = []
         for r in self.roots:
             value = run.eval(r, root)
             # evaluator.ex:68-75: the output keeps the traced template, the data is the result's
             results.append(r.with_(data=value.data))
-        return _unflatten(self.structure, results)
+        return results
+
+    def __call__(self, *args):
+        return _unflatten(self.structure, self._evaluate(self._params(args)))
+
+    def capture(self, *args) -> "Captured":
+        """Records one evaluation on the device as a graph: later calls replay all its kernels with
+        a single submission instead of one callback (and one launch) per node.  The function must
+        not need the host while it runs: no `while_loop` / `cond`, no bounds-checked `take`."""
+        return Captured(self, self._params(args))
+
+
+class Captured:
+    """A compiled function whose device work was captured once, on private copies of the arguments
+    (`inputs`).  Calling it copies the arguments into those (pass `inputs` themselves to skip the
+    copies), replays the graph and returns the captured result tensors: they are overwritten by the
+    next call and die with this object."""
+
+    def __init__(self, compiled: Compiled, params):
+        from . import backend as B
+        devices = {p.data.device for p in params if isinstance(p.data, B.HipNxBackend)}
+        if len(devices) != 1 or any(not isinstance(p.data, B.HipNxBackend) for p in params):
+            raise ValueError("capture needs every argument on one device")
+        (self.device,) = devices
+        self.compiled = compiled
+        self.params = [Nx.backend_copy(p, B.HipNxBackend, {"device": self.device}) for p in params]
+        compiled._evaluate(self.params)  # once for real: kernel attributes, pool block sizes, cached constants
+        B.capture_begin(self.device)
+        try:
+            self.results = compiled._evaluate(self.params)
+        except BaseException:
+            B.capture_end(self.device).destroy()
+            raise
+        self.graph = B.capture_end(self.device)
+
+    @property
+    def inputs(self):
+        return list(self.params)
+
+    def __call__(self, *args):
+        from . import backend as B
+        new = self.compiled._params(args)
+        for held, given in zip(self.params, new):
+            if given.data is held.data or getattr(given.data, "ref", None) is held.data.ref:
+                continue
+            if not isinstance(given.data, B.HipNxBackend):
+                given = Nx.backend_transfer(given, B.HipNxBackend, {"device": self.device})
+            B.copy_into(held, given)
+        self.graph.launch()
+        return _unflatten(self.compiled.structure, self.results)
+
+    def destroy(self):
+        self.graph.destroy()
+        self.results = []
 
 
 def _runtime_backend(params):
@@ -646,7 +942,7 @@ def _runtime_backend(params):
     return mod, opts
 
 
-def trace(fun: Callable, args, kwargs=None) -> Compiled:
+def trace(fun: Callable, args, kwargs=None, fuse: bool = False) -> Compiled:
     """Runs `fun` on parameter expressions shaped like `args` (compiler.ex:184-205: the default
     backend is the expression builder while the function runs)."""
     leaves: list = []
@@ -667,21 +963,25 @@ def trace(fun: Callable, args, kwargs=None) -> Compiled:
         Nx.default_backend(*previous)
         _trace.scopes = []
         _trace.fold = None
-    return Compiled(roots, out_structure, len(templates))
+    compiled_groups = _fuse(roots) if fuse else 0
+    compiled = Compiled(roots, out_structure, [t.with_(data=None) for t in templates])
+    compiled.fused_groups = compiled_groups
+    return compiled
 
 
-def jit(fun: Callable = None, **static):
+def jit(fun: Callable = None, fuse: bool = False, **static):
     """Nx.Defn.jit/2 with the default compiler: traces on every call, like the reference's
-    evaluator (evaluator.ex:41-43), then evaluates.  Keyword arguments are static options."""
+    evaluator (evaluator.ex:41-43), then evaluates.  Keyword arguments are static options; `fuse`
+    hands groups of element-wise nodes to the backend as one kernel each."""
     if fun is None:
-        return lambda f: jit(f, **static)
+        return lambda f: jit(f, fuse=fuse, **static)
 
     def call(*args, **kwargs):
-        return trace(fun, args, {**static, **kwargs})(*args)
+        return trace(fun, args, {**static, **kwargs}, fuse=fuse)(*args)
     call.__name__ = getattr(fun, "__name__", "jitted")
     return call
 
 
-def compile(fun: Callable, *templates, **static) -> Compiled:  # noqa: A001 - Nx.Defn.compile/3
+def compile(fun: Callable, *templates, fuse: bool = False, **static) -> Compiled:  # noqa: A001 - Nx.Defn.compile/3
     """Traces once for arguments shaped like `templates`; the result is called many times."""
-    return trace(fun, templates, static)
+    return trace(fun, templates, static, fuse=fuse)

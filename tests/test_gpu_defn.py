@@ -97,3 +97,158 @@ def test_traced_random_uses_the_one_kernel_cipher(hip):
     finally:
         Random.compose_only(previous)
     assert_bits_equal(traced, composed, "random_bits traced vs composed")
+
+
+# ---- captured graphs: one submission replays every kernel of a compiled function ------------------
+
+GRAPHABLE = ["softmax", "elementwise_reduce", "linear_int8"]  # argmax_take needs the bounds check of take: a host read
+
+
+@pytest.mark.parametrize("name", GRAPHABLE)
+def test_captured_chain_replays_with_new_inputs(name, hip):
+    from nx_amd.backend import sync
+    args = build_args(hip)[name]
+    compiled = defn.compile(CHAINS[name], *args)
+    eager = hip.to_numpy(compiled(*args)).copy()
+    captured = compiled.capture(*args)
+    try:
+        # replays between eager work and synchronisations, every one checked against the eager result
+        for _ in range(3):
+            out = captured(*args)
+            np.testing.assert_array_equal(hip.to_numpy(out), eager, f"{name}: replay with the captured tensors")
+            compiled(*args)
+            sync()
+        # new values in fresh tensors of the same shapes: copied in, same kernels
+        rng = np.random.default_rng(11)
+        fresh = []
+        for a in args:
+            raw = hip.to_numpy(a)
+            perm = rng.permutation(raw.size)
+            fresh.append(from_numpy(raw.reshape(-1)[perm].reshape(raw.shape), a.type, hip))
+        want = hip.to_numpy(compiled(*fresh)).copy()
+        np.testing.assert_array_equal(hip.to_numpy(captured(*fresh)), want, f"{name}: replay with new inputs")
+        np.testing.assert_array_equal(hip.to_numpy(captured(*args)), eager, f"{name}: and back")
+    finally:
+        captured.destroy()
+
+
+def test_capture_refuses_what_needs_the_host(hip):
+    from nx_amd._lib import HipNxError
+    args = build_args(hip)["argmax_take"]
+    compiled = defn.compile(CHAINS["argmax_take"], *args)
+    with pytest.raises(HipNxError, match="not possible while capturing"):
+        compiled.capture(*args)
+    # the failed capture leaves the context usable
+    assert_bits_equal(compiled(*args), CHAINS["argmax_take"](*args), "eager after a refused capture")
+
+
+def test_graph_blocks_do_not_leak_into_the_pool(hip):
+    n = 1 << 20
+    x = from_numpy(np.linspace(-1, 1, n, dtype=np.float32), "f32", hip)
+
+    def chain(t):
+        for _ in range(6):
+            t = Nx.exp(Nx.negate(t))
+        return t
+    compiled = defn.compile(chain, x)
+    want = hip.to_numpy(compiled(x)).copy()
+    captured = compiled.capture(x)
+    out = captured(x)
+    # eager work of the same sizes in between must not be handed the graph's blocks
+    others = [Nx.exp(x) for _ in range(8)]
+    np.testing.assert_array_equal(hip.to_numpy(captured(x)), want)
+    np.testing.assert_array_equal(hip.to_numpy(others[0]), hip.to_numpy(Nx.exp(x)))
+    del others, out
+    before = mem_stats()
+    captured.destroy()
+    after = mem_stats()
+    assert after["pooled"] >= before["pooled"]  # the graph's blocks return to the pool only now
+    np.testing.assert_array_equal(hip.to_numpy(compiled(x)), want)
+
+
+# ---- fused element-wise groups: one kernel per group, the same bits as node by node -----------------
+
+def gelu_like(x, bias):
+    h = Nx.add(x, bias)
+    return Nx.multiply(Nx.multiply(h, 0.5), Nx.add(1.0, Nx.tanh(Nx.multiply(0.7978845608, Nx.add(h, Nx.multiply(0.044715, Nx.pow(h, 3.0)))))))
+
+
+def relu_mask(x, y):
+    keep = Nx.logical_and(Nx.greater(x, 0.0), Nx.less_equal(y, 0.5))
+    return Nx.select(keep, Nx.sqrt(Nx.abs(x)), Nx.negate(y))
+
+
+def mixed_precision(a, b):
+    # every intermediate rounds to its own type: bf16 by truncation, f16 to nearest
+    h = Nx.multiply(a, b)                       # bf16 * f16 -> f16? no: merged float type
+    return Nx.as_type(Nx.exp(Nx.as_type(Nx.add(h, 0.25), "bf16")), "f16")
+
+
+def row_and_column_operands(x, row, col):
+    return Nx.divide(Nx.subtract(x, col), Nx.add(row, 1.5))
+
+
+def rand_float(rng, ty, shape, backend):
+    v = rng.standard_normal(shape).astype(np.float32)
+    if ty == "bf16":
+        return from_numpy((v.view(np.uint32) >> 16).astype(np.uint16), "bf16", backend)
+    return from_numpy(v.astype(np.float16 if ty == "f16" else np.float32), ty, backend)
+
+
+FUSED_CASES = {
+    "gelu_like": (gelu_like, lambda rng, b: (rand_float(rng, "f32", (64, 256), b), rand_float(rng, "f32", (256,), b))),
+    "gelu_like_bf16": (gelu_like, lambda rng, b: (rand_float(rng, "bf16", (8, 16, 128), b), rand_float(rng, "bf16", (128,), b))),
+    "relu_mask": (relu_mask, lambda rng, b: (rand_float(rng, "f32", (1000, 24), b), rand_float(rng, "f32", (1000, 24), b))),
+    "relu_mask_ragged": (relu_mask, lambda rng, b: (rand_float(rng, "f32", (37, 11), b), rand_float(rng, "f32", (37, 11), b))),
+    "mixed_precision": (mixed_precision, lambda rng, b: (rand_float(rng, "bf16", (33, 40), b), rand_float(rng, "f16", (33, 40), b))),
+    "row_and_column": (row_and_column_operands, lambda rng, b: (rand_float(rng, "f32", (48, 64), b), rand_float(rng, "f32", (64,), b),
+                                                                 rand_float(rng, "f32", (48, 1), b))),
+    "row_and_column_unaligned": (row_and_column_operands, lambda rng, b: (rand_float(rng, "f32", (5, 7), b), rand_float(rng, "f32", (7,), b),
+                                                                           rand_float(rng, "f32", (5, 1), b))),
+}
+
+
+@pytest.mark.parametrize("name", sorted(FUSED_CASES))
+def test_fused_group_is_bit_identical_to_node_by_node(name, hip):
+    fun, make = FUSED_CASES[name]
+    args = make(np.random.default_rng(3), hip)
+    fused = defn.compile(fun, *args, fuse=True)
+    assert fused.fused_groups >= 1
+    assert_bits_equal(fused(*args), defn.compile(fun, *args)(*args), name)
+
+
+@pytest.mark.parametrize("name", sorted(CHAINS))
+def test_fused_configuration_chains(name, hip):
+    args = build_args(hip)[name]
+    assert_bits_equal(defn.compile(CHAINS[name], *args, fuse=True)(*args), defn.compile(CHAINS[name], *args)(*args), name)
+
+
+def test_fused_kernel_is_the_path_taken(hip):
+    calls = []
+    original = hip.fused_elementwise.__func__
+
+    def counting(cls, *a, **k):
+        calls.append(1)
+        return original(cls, *a, **k)
+    hip.fused_elementwise = classmethod(counting)
+    try:
+        fun, make = FUSED_CASES["gelu_like"]
+        args = make(np.random.default_rng(5), hip)
+        defn.compile(fun, *args, fuse=True)(*args)
+    finally:
+        hip.fused_elementwise = classmethod(original)
+    assert calls == [1]  # the whole function is one group
+
+
+def test_fused_entry_point_validates_its_program(hip):
+    from nx_amd._lib import FUSED_BINARY, FUSED_UNARY, HipNxError
+    x = rand_float(np.random.default_rng(1), "f32", (16,), hip)
+    out = x.with_(data=None)
+    with pytest.raises(HipNxError, match="unwritten register"):
+        hip.fused_elementwise(out, [(FUSED_BINARY, 0, 1, 0, 2, 0, ("f", 32), 0.0)], 1, [x], (1, 16, [(0, 1)]))
+    with pytest.raises(HipNxError, match="binary op"):
+        hip.fused_elementwise(out, [(FUSED_BINARY, 9, 1, 0, 0, 0, ("f", 32), 0.0)], 1, [x], (1, 16, [(0, 1)]))
+    with pytest.raises(HipNxError, match="holds"):
+        hip.fused_elementwise(out.with_(shape=(32,)), [(FUSED_UNARY, 0, 1, 0, 0, 0, ("f", 32), 0.0)], 1, [x], (1, 32, [(0, 1)]))
+    got = hip.fused_elementwise(out, [(FUSED_UNARY, 27, 1, 0, 0, 0, ("f", 32), 0.0)], 1, [x], (1, 16, [(0, 1)]))  # negate
+    np.testing.assert_array_equal(hip.to_numpy(got), -hip.to_numpy(x))
