@@ -118,8 +118,15 @@ int hipnx_buf_free(hipnx_buf *buf);
 /* releases the handle (and the device memory if still live) */
 int hipnx_buf_destroy(hipnx_buf *buf);
 int hipnx_buf_size(const hipnx_buf *buf, size_t *bytes);
-/* raw device pointer, for interop and profiling harnesses; NULL once freed */
+/* replaces: to_pointer/2 with mode :local (nx/lib/nx/backend.ex:66; exla/lib/exla/backend.ex:86-131,
+ * exla/c_src/exla/exla.cc:327-385): the raw device address of a live buffer; NULL once freed */
 void *hipnx_buf_device_ptr(const hipnx_buf *buf);
+/* replaces: from_pointer/5 for a :local pointer (nx/lib/nx/backend.ex:59-65;
+ * exla/lib/exla/backend.ex:133-181, exla/c_src/exla/exla.cc:387-437): a handle over `bytes` of
+ * device memory of this context's device that someone else owns.  Freeing or destroying the
+ * handle never frees the memory; the owner keeps it alive while the handle is used.  The :ipc
+ * kind of pointer (a handle another process opens) is not built. */
+int hipnx_buf_wrap(hipnx_ctx *ctx, void *device_ptr, size_t bytes, hipnx_buf **out);
 int hipnx_h2d(hipnx_ctx *ctx, hipnx_buf *dst, size_t dst_offset, const void *src, size_t bytes);
 /* waits for all work enqueued so far, then copies */
 int hipnx_d2h(hipnx_ctx *ctx, const hipnx_buf *src, size_t src_offset, void *dst, size_t bytes);

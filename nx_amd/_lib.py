@@ -64,6 +64,7 @@ PROTOTYPES = {
     "hipnx_buf_destroy": [_buf_p],
     "hipnx_buf_size": [_buf_p, C.POINTER(C.c_size_t)],
     "hipnx_buf_device_ptr": [_buf_p],
+    "hipnx_buf_wrap": [_ctx_p, C.c_void_p, C.c_size_t, C.POINTER(_buf_p)],
     "hipnx_h2d": [_ctx_p, _buf_p, C.c_size_t, C.c_void_p, C.c_size_t],
     "hipnx_d2h": [_ctx_p, _buf_p, C.c_size_t, C.c_void_p, C.c_size_t],
     "hipnx_d2d": [_ctx_p, _buf_p, C.c_size_t, _buf_p, C.c_size_t, C.c_size_t],

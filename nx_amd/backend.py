@@ -31,7 +31,7 @@ K_INNER, K_OUTER = 0, 1
 OOB_RAISE, OOB_CLAMP = 0, 1
 
 # callbacks of the behaviour that are not on the device path (nx/lib/nx/backend.ex:58-144)
-UNSUPPORTED = ["to_batched", "from_pointer", "to_pointer", "put_slice", "reverse",
+UNSUPPORTED = ["to_batched", "put_slice", "reverse",
                "conv", "window_sum", "window_product",
                "window_max", "window_min", "reduce", "window_reduce", "window_scatter_max", "window_scatter_min",
                "indexed_add", "indexed_put", "sort", "argsort", "fft", "ifft", "fft2", "ifft2", "triangular_solve",
@@ -60,12 +60,16 @@ class _Ref:
     """Owns one device buffer.  Metadata-only callbacks (reshape / squeeze / bitcast) share it;
     it is deallocated when the last sharer is, or by the garbage collector."""
 
-    def __init__(self, ctx, nbytes: int):
+    def __init__(self, ctx, nbytes: int, address=None, keep=None):
         self.ctx = ctx
         self.handle = C.c_void_p()
         self.nbytes = nbytes
         self.sharers = 1
-        L.check(L.lib.hipnx_buf_alloc(ctx, nbytes, C.byref(self.handle)))
+        self.keep = keep  # the owner of borrowed memory, kept alive with the handle
+        if address is None:
+            L.check(L.lib.hipnx_buf_alloc(ctx, nbytes, C.byref(self.handle)))
+        else:  # someone else's device memory: the handle never frees it
+            L.check(L.lib.hipnx_buf_wrap(ctx, C.c_void_p(address), nbytes, C.byref(self.handle)))
 
     def __del__(self):
         if getattr(self, "handle", None) and self.handle.value:
@@ -597,6 +601,38 @@ class HipNxBackend:
         with a unit axis inserted at `axis`."""
         widened = [t.with_(shape=t.shape[:axis] + (1,) + t.shape[axis:]) for t in tensors]
         return cls.concatenate(out, widened, axis)
+
+    @classmethod
+    def to_pointer(cls, t: Tensor, opts=None):
+        """to_pointer/2 (backend.ex:66; semantics of exla/lib/exla/backend.ex:86-131): the device
+        address of the tensor's buffer as a `Pointer` of kind "local".  The "ipc" kind -- a handle
+        for another process -- is not built."""
+        opts = dict(opts or {})
+        mode = opts.pop("mode", "local")
+        if opts:
+            raise ValueError(f"unknown options {sorted(opts)!r}")
+        if mode == "ipc":
+            raise NotImplementedError("HipNx.Backend.to_pointer: the :ipc mode is not built, only :local")
+        if mode != "local":
+            raise ValueError(f"expected one of :local, :ipc, got: {mode!r}")
+        from .nx import Pointer
+        address = L.lib.hipnx_buf_device_ptr(cls._handle(t))
+        return Pointer(kind="local", address=int(address), data_size=t.size * T.size_bytes(t.type))
+
+    @classmethod
+    def from_pointer(cls, pointer, type, shape, backend_opts=None, opts=None) -> Tensor:  # noqa: A002
+        """from_pointer/5 (backend.ex:59-65; exla/lib/exla/backend.ex:133-181): a tensor over device
+        memory that someone else owns.  `opts["keep"]`, if given, is held for the tensor's lifetime
+        (the object that owns the memory)."""
+        backend_opts, opts = cls.init(backend_opts), dict(opts or {})
+        ty = T.normalize(type)
+        size = prod(shape) * T.size_bytes(ty)
+        if pointer.data_size != size:
+            raise ValueError(f"invalid pointer data_size for shape, expected: {size}, got: {pointer.data_size}")
+        if pointer.kind != "local":
+            raise NotImplementedError("HipNx.Backend.from_pointer: only pointers of kind :local are built")
+        ref = _Ref(_Context.get(backend_opts["device"]), size, address=pointer.address, keep=opts.get("keep"))
+        return Tensor(cls(ref, backend_opts["device"]), ty, tuple(shape), tuple(opts.get("names") or ()))
 
     @classmethod
     def fused_elementwise(cls, out: Tensor, program, out_reg: int, inputs, layout) -> Tensor:

@@ -344,9 +344,31 @@ int hipnx_buf_free(hipnx_buf *buf) {
   hipnx_ctx *ctx = buf->ctx;
   Enter in(ctx);
   if (in.status) return in.status;
-  int st = pool_free(ctx, buf->ptr, buf->capacity);
+  int st = buf->borrowed ? HIPNX_OK : pool_free(ctx, buf->ptr, buf->capacity);
   buf->ptr = nullptr;
   return st;
+}
+
+int hipnx_buf_wrap(hipnx_ctx *ctx, void *device_ptr, size_t bytes, hipnx_buf **out) {
+  Enter in(ctx);
+  if (in.status) return in.status;
+  if (!out || !device_ptr) return set_error(HIPNX_EINVAL, "buf_wrap: null argument");
+  hipPointerAttribute_t attr;
+  hipError_t e = hipPointerGetAttributes(&attr, device_ptr);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    return set_error(HIPNX_EINVAL, "buf_wrap: %p is not a pointer this process can use on a device", device_ptr);
+  }
+  if (attr.type != hipMemoryTypeDevice || attr.device != ctx->device)
+    return set_error(HIPNX_EINVAL, "buf_wrap: %p is not device memory of device %d", device_ptr, ctx->device);
+  hipnx_buf *b = new hipnx_buf;
+  b->ctx = ctx;
+  b->ptr = device_ptr;
+  b->bytes = bytes;
+  b->capacity = bytes;
+  b->borrowed = true;
+  *out = b;
+  return HIPNX_OK;
 }
 
 int hipnx_buf_destroy(hipnx_buf *buf) {

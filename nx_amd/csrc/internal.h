@@ -51,6 +51,7 @@ struct hipnx_buf {
   size_t bytes = 0;     // what the caller asked for
   size_t capacity = 0;  // what the pool block holds
   std::atomic<int> freed{0};
+  bool borrowed = false;  // wraps memory owned by someone else: never returned to the pool
 };
 
 namespace hipnx {

@@ -11,6 +11,7 @@ from __future__ import annotations
 import builtins
 import threading
 from dataclasses import dataclass
+from typing import Optional
 from math import prod
 
 import numpy as np
@@ -378,6 +379,27 @@ def broadcast(t, new_shape, axes=None):
     if t.shape == new_shape and axes == list(range(len(new_shape))):
         return t
     return _impl(t).broadcast(t.with_(data=None, shape=new_shape), t, new_shape, axes)
+
+
+@dataclass(frozen=True)
+class Pointer:
+    """%Nx.Pointer{kind, address, data_size, handle} (nx/lib/nx/pointer.ex:8-15)."""
+    kind: str
+    address: Optional[int] = None
+    data_size: int = 0
+    handle: Optional[bytes] = None
+
+
+def to_pointer(t, **opts) -> "Pointer":
+    """Nx.to_pointer/2 (nx.ex:17807-17810)."""
+    t = to_tensor(t)
+    return _impl(t).to_pointer(t, opts)
+
+
+def from_pointer(backend, pointer: "Pointer", type, shape, **opts) -> Tensor:  # noqa: A002
+    """Nx.from_pointer/5 (nx.ex:17762-17775): `backend` is a module or (module, options)."""
+    mod, backend_opts = backend if isinstance(backend, tuple) else (backend, {})
+    return mod.from_pointer(pointer, T.normalize(type), tuple(shape), backend_opts, opts)
 
 
 @dataclass(frozen=True)
