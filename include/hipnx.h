@@ -211,12 +211,13 @@ int hipnx_select(hipnx_ctx *ctx, int pred_dt, int true_dt, int false_dt, int out
 int hipnx_clip(hipnx_ctx *ctx, int in_dt, int min_dt, int max_dt, int out_dt, int64_t n,
                const hipnx_buf *in, const hipnx_buf *min, const hipnx_buf *max, hipnx_buf *out);
 
-/* replaces: slice/5, concatenate/3, stack/3, pad/4 (nx/lib/nx/backend.ex:79,82-83,74; oracle
- * binary_backend.ex:1813-1863, 1962-2030, 326-431) -- one copy over the index space `dims` with
+/* replaces: slice/5, concatenate/3, stack/3, pad/4, reverse/3, put_slice/4 (nx/lib/nx/backend.ex:79,82-83,
+ * 74-75,80; oracle binary_backend.ex:1813-1863, 1962-2030, 326-431, 434-474, 1865-1900) -- one copy over the index space `dims` with
  * element strides and offsets on both sides: a slice reads strided and writes dense, a
  * concatenation writes each operand into its window of the output, a pad writes the elements
  * that survive the cropping at their spread-out positions in an output filled with the pad
- * value (hipnx_broadcast with zero strides) */
+ * value (hipnx_broadcast with zero strides), a reverse reads an axis backwards (negative input
+ * stride, the offset on its last element), a put_slice writes the slice into its window of a copy */
 int hipnx_strided_copy(hipnx_ctx *ctx, int elem_bytes, int rank, const int64_t *dims,
                        const int64_t *in_strides, int64_t in_offset, const int64_t *out_strides,
                        int64_t out_offset, const hipnx_buf *in, hipnx_buf *out);

@@ -31,7 +31,7 @@ K_INNER, K_OUTER = 0, 1
 OOB_RAISE, OOB_CLAMP = 0, 1
 
 # callbacks of the behaviour that are not on the device path (nx/lib/nx/backend.ex:58-144)
-UNSUPPORTED = ["to_batched", "put_slice", "reverse",
+UNSUPPORTED = ["to_batched",
                "conv", "window_sum", "window_product",
                "window_max", "window_min", "reduce", "window_reduce", "window_scatter_max", "window_scatter_min",
                "indexed_add", "indexed_put", "sort", "argsort", "fft", "ifft", "fft2", "ifft2", "triangular_solve",
@@ -574,6 +574,46 @@ class HipNxBackend:
                 L.i64_array([s * d for s, d in zip(steps, dense_out)]),
                 sum((c[0] + f * s) * d for c, f, s, d in zip(padding_config, first, steps, dense_out)),
                 cls._handle(t), res.data.ref.handle))
+        return res
+
+    @classmethod
+    def reverse(cls, out: Tensor, t: Tensor, axes) -> Tensor:
+        """reverse/3 (backend.ex:75; oracle binary_backend.ex:434-474): one copy that reads the given
+        axes backwards."""
+        dev = cls._device_of(t)
+        t = cls._from_nx(t, dev)
+        dense = cls._dense_strides(t.shape)
+        strides = [-s if a in axes else s for a, s in enumerate(dense)]
+        offset = sum((t.shape[a] - 1) * dense[a] for a in axes)
+        res = cls._alloc(out, dev)
+        L.check(L.lib.hipnx_strided_copy(res.data.ref.ctx, T.size_bytes(t.type), len(t.shape), L.i64_array(t.shape),
+                                         L.i64_array(strides), offset, L.i64_array(dense), 0, cls._handle(t), res.data.ref.handle))
+        return res
+
+    @classmethod
+    def put_slice(cls, out: Tensor, t: Tensor, start_indices, slice_t: Tensor) -> Tensor:
+        """put_slice/4 (backend.ex:80; oracle binary_backend.ex:1865-1900): both operands in
+        out.type, start indices clamped so the slice fits, the slice written into a copy of `t`."""
+        dev = cls._device_of(t, slice_t)
+        t, slice_t = cls._from_nx(t, dev), cls._from_nx(slice_t, dev)
+        if t.type != out.type:
+            t = cls.as_type(t.with_(data=None, type=out.type), t)
+        if slice_t.type != out.type:
+            slice_t = cls.as_type(slice_t.with_(data=None, type=out.type), slice_t)
+        starts = []
+        for dim, idx, length in zip(t.shape, start_indices, slice_t.shape):
+            if isinstance(idx, Tensor):
+                idx = int(np.frombuffer(type(idx.data).to_binary(idx, 1), dtype=T.numpy_dtype(idx.type))[0])
+            starts.append(min(max(int(idx), 0), dim - length))
+        res = cls._alloc(out, dev)
+        ctx = res.data.ref.ctx
+        L.check(L.lib.hipnx_d2d(ctx, res.data.ref.handle, 0, cls._handle(t), 0, res.data.ref.nbytes))
+        if slice_t.size:
+            dense = cls._dense_strides(out.shape)
+            L.check(L.lib.hipnx_strided_copy(
+                ctx, T.size_bytes(out.type), len(slice_t.shape), L.i64_array(slice_t.shape),
+                L.i64_array(cls._dense_strides(slice_t.shape)), 0, L.i64_array(dense),
+                sum(s * d for s, d in zip(starts, dense)), cls._handle(slice_t), res.data.ref.handle))
         return res
 
     @classmethod

@@ -308,13 +308,19 @@ extern "C" int hipnx_strided_copy(hipnx_ctx *ctx, int elem_bytes, int rank, cons
     return set_error(HIPNX_EINVAL, "strided_copy: element size %d is not 1, 2, 4 or 8", elem_bytes);
   if (rank < 0 || rank > 64 || (rank > 0 && (!dims || !in_strides || !out_strides))) return set_error(HIPNX_EINVAL, "strided_copy: bad rank");
   if (in_offset < 0 || out_offset < 0) return set_error(HIPNX_EINVAL, "strided_copy: negative offset");
-  int64_t n = 1, ie = in_offset + 1, oe = out_offset + 1;
+  int64_t n = 1, ie = in_offset + 1, oe = out_offset + 1, ifirst = in_offset;
   for (int a = 0; a < rank; a++) {
-    if (dims[a] < 0 || in_strides[a] < 0 || out_strides[a] < 0) return set_error(HIPNX_EINVAL, "strided_copy: negative dimension or stride");
+    // the input may be walked backwards along an axis (reverse); the output never is
+    if (dims[a] < 0 || out_strides[a] < 0) return set_error(HIPNX_EINVAL, "strided_copy: negative dimension or output stride");
     n *= dims[a];
   }
   if (n > 0)
-    for (int a = 0; a < rank; a++) { ie += (dims[a] - 1) * in_strides[a]; oe += (dims[a] - 1) * out_strides[a]; }
+    for (int a = 0; a < rank; a++) {
+      if (in_strides[a] >= 0) ie += (dims[a] - 1) * in_strides[a];
+      else ifirst += (dims[a] - 1) * in_strides[a];
+      oe += (dims[a] - 1) * out_strides[a];
+    }
+  if (n > 0 && ifirst < 0) return set_error(HIPNX_EINVAL, "strided_copy: the input walk leaves the buffer at its start");
   if (int st = check_buf(ctx, inb, n > 0 ? (uint64_t)ie * elem_bytes : 0, "strided_copy in")) return st;
   if (int st = check_buf(ctx, out, n > 0 ? (uint64_t)oe * elem_bytes : 0, "strided_copy out")) return st;
   if (n == 0) return HIPNX_OK;

@@ -453,6 +453,44 @@ defmodule HipNx.Backend do
   end
 
   @impl true
+  def reverse(%T{type: {_, bits}} = out, %T{shape: shape} = t, axes) do
+    device = device_of([t])
+    {ref, _} = from_nx(t, device)
+    dense = dense_strides(shape)
+    strides = dense |> Enum.with_index() |> Enum.map(fn {s, a} -> if a in axes, do: -s, else: s end)
+    offset = axes |> Enum.map(&((elem(shape, &1) - 1) * Enum.at(dense, &1))) |> Enum.sum()
+
+    to_nx(unwrap!(NIF.strided_copy(ctx(device), div(bits, 8), Tuple.to_list(shape), strides, offset, dense, 0, ref, bytes(out))),
+      device, out)
+  end
+
+  @impl true
+  def put_slice(%T{shape: shape, type: {_, bits} = type} = out, %T{} = t, start_indices, %T{shape: slice_shape} = slice) do
+    device = device_of([t, slice])
+    t = if t.type == type, do: t, else: as_type(%{t | type: type}, t)
+    slice = if slice.type == type, do: slice, else: as_type(%{slice | type: type}, slice)
+    {ref, _} = from_nx(t, device)
+    {sref, _} = from_nx(slice, device)
+
+    starts =
+      [start_indices, Tuple.to_list(shape), Tuple.to_list(slice_shape)]
+      |> Enum.zip_with(fn [idx, dim, len] ->
+        idx = if is_struct(idx, T), do: Nx.to_number(idx), else: idx
+        idx |> max(0) |> min(dim - len)
+      end)
+
+    dense = dense_strides(shape)
+    buf = unwrap!(NIF.copy(ctx(device), ref, bytes(out)))
+
+    if Nx.size(slice_shape) > 0 do
+      at = Enum.zip_with(starts, dense, &(&1 * &2)) |> Enum.sum()
+      unwrap!(NIF.strided_copy(ctx(device), div(bits, 8), Tuple.to_list(slice_shape), dense_strides(slice_shape), 0, dense, at, sref, buf))
+    end
+
+    to_nx(buf, device, out)
+  end
+
+  @impl true
   def concatenate(%T{shape: out_shape, type: {_, bits} = type} = out, tensors, axis) do
     device = device_of(tensors)
     out_strides = dense_strides(out_shape)

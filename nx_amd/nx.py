@@ -551,6 +551,35 @@ def slice(t, start_indices, lengths, strides=1):  # noqa: A001 - Nx.slice/4 (nx.
     return _impl(t).slice(t.with_(data=None, shape=tuple(out_shape)), t, starts, lengths, strides)
 
 
+def reverse(t, axes=None):
+    """Nx.reverse/2 (nx.ex:13527-13543): all axes by default; no axes, no work."""
+    t = to_tensor(t)
+    axes = list(range(len(t.shape))) if axes is None else S.normalize_axes(t.shape, axes)
+    if not axes:
+        return t
+    return _impl(t).reverse(t.with_(data=None), t, sorted(axes))
+
+
+def put_slice(t, start_indices, slice_t):
+    """Nx.put_slice/3 (nx.ex:14491-14530; shape rule shape.ex:1304-1345): the slice has the rank of
+    the tensor and fits inside it; start indices are numbers or rank-0 integer tensors."""
+    t, slice_t = to_tensor(t), to_tensor(slice_t)
+    start_indices = list(start_indices)
+    rank = len(t.shape)
+    if len(start_indices) != rank:
+        raise ValueError(f"invalid start indices rank for shape of rank {rank}")
+    if len(slice_t.shape) != rank:
+        raise ValueError(f"invalid slice for put_slice, rank of slice must match {rank}, got: {len(slice_t.shape)}")
+    if builtins.any(s > d for s, d in zip(slice_t.shape, t.shape)):
+        raise ValueError(f"slice shape {S.fmt(slice_t.shape)} must be less than or equal to tensor shape {S.fmt(t.shape)}")
+    for i in start_indices:
+        if isinstance(i, Tensor) and (i.shape != () or not T.is_integer(i.type)):
+            raise ValueError("index must be an integer or a scalar integer tensor")
+    out = t.with_(data=None, type=T.binary_type(t.type, slice_t.type))
+    operands = [t, slice_t] + [i for i in start_indices if isinstance(i, Tensor)]
+    return _impl(*operands).put_slice(out, t, start_indices, slice_t)
+
+
 def slice_along_axis(t, start_index, length, axis=0, strides=1):
     """Nx.slice_along_axis/4 (nx.ex:14391-14420)."""
     t = to_tensor(t)

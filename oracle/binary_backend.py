@@ -423,6 +423,27 @@ class BinaryBackend:
         return res
 
     @classmethod
+    def reverse(cls, out, t, axes):  # binary_backend.ex:434-474
+        buf, res = cls._new(out)
+        buf[:] = np.ascontiguousarray(np.flip(cls._typed(t), axis=tuple(axes))).tobytes()
+        return res
+
+    @classmethod
+    def put_slice(cls, out, t, start_indices, slice_t):  # binary_backend.ex:1865-1900
+        base = cls._typed(cls.as_type(t.with_(data=None, type=out.type), t)).copy()
+        piece = cls._typed(cls.as_type(slice_t.with_(data=None, type=out.type), slice_t))
+        window = []
+        for dim, idx, length in zip(t.shape, start_indices, slice_t.shape):
+            if isinstance(idx, Tensor):
+                idx = int(cls._numbers(idx).reshape(()))
+            start = min(max(int(idx), 0), dim - length)  # clamp_indices
+            window.append(np.s_[start:start + length])
+        base[tuple(window)] = piece
+        buf, res = cls._new(out)
+        buf[:] = base.tobytes()
+        return res
+
+    @classmethod
     def concatenate(cls, out, tensors, axis):  # binary_backend.ex:1975-1986
         parts = [cls._typed(cls.as_type(t.with_(data=None, type=out.type), t)) for t in tensors]
         buf, res = cls._new(out)

@@ -70,6 +70,9 @@ def run_case(case, backend):
     if op == "slice":  # start indices may be rank-0 tensors
         t, starts, lengths = case["args"]
         return Nx.slice(spec_to_tensor(t, backend), [spec_to_tensor(i, backend) for i in starts], lengths, **opts)
+    if op == "put_slice":  # start indices are numbers or rank-0 tensors
+        t, starts, piece = case["args"]
+        return Nx.put_slice(spec_to_tensor(t, backend), [spec_to_tensor(i, backend) for i in starts], spec_to_tensor(piece, backend))
     if op == "pad":  # the padding configuration is a plain list of (low, high, interior)
         t, value, config = case["args"]
         return Nx.pad(spec_to_tensor(t, backend), spec_to_tensor(value, backend), config)

@@ -199,3 +199,36 @@ def test_pad_converts_both_operands_to_the_merged_type(ty, vty, hip, oracle):
     got = Nx.pad(ht, hv, config)
     want = Nx.pad(Nx.as_type(ot, got.type), Nx.as_type(ov, got.type), config)
     assert_bits_equal(got, want, f"pad {ty} with {vty}")
+
+
+@pytest.mark.parametrize("ty", ["u8", "bf16", "f32", "s64"])
+@pytest.mark.parametrize("shape,axes", [((10,), None), ((7, 9), [0]), ((7, 9), [1]), ((7, 9), None), ((4, 5, 6), [0, 2]), ((4, 5, 6), [1]),
+                                        ((3, 1, 8), [1]), ((256, 384), [1]), ((256, 384), [0]), ((1,), None)])
+def test_reverse(ty, shape, axes, hip, oracle):
+    rng = np.random.default_rng(seed_of(ty, shape, axes))
+    ht, ot = pair(rng, ty, shape, hip, oracle)
+    assert_bits_equal(Nx.reverse(ht, axes=axes), Nx.reverse(ot, axes=axes), f"reverse {ty} {shape} {axes}")
+
+
+PUTS = [((10,), (3,), [4]), ((10,), (10,), [0]), ((10,), (4,), [9]), ((6, 8), (2, 3), [1, 2]), ((6, 8), (6, 1), [0, -5]), ((4, 5, 6), (1, 5, 2), [3, 0, 100]),
+        ((256, 256), (64, 128), [32, 64]), ((5, 5), (0, 3), [1, 1])]
+
+
+@pytest.mark.parametrize("types", [("f32", "f32"), ("s32", "f32"), ("bf16", "s8"), ("u8", "s16"), ("s64", "s64")])
+@pytest.mark.parametrize("shape,piece,starts", PUTS)
+def test_put_slice(types, shape, piece, starts, hip, oracle):
+    rng = np.random.default_rng(seed_of(types, shape, piece, starts))
+    ht, ot = pair(rng, types[0], shape, hip, oracle, small=True)
+    hs, os_ = pair(rng, types[1], piece, hip, oracle, small=True)
+    assert_bits_equal(Nx.put_slice(ht, starts, hs), Nx.put_slice(ot, starts, os_), f"put_slice {types} {shape} {piece} {starts}")
+    # the operand is left as it was
+    assert_bits_equal(ht, ot, "put_slice operand")
+
+
+def test_put_slice_with_tensor_start_indices(hip, oracle):
+    rng = np.random.default_rng(9)
+    ht, ot = pair(rng, "f32", (12, 40), hip, oracle)
+    hs, os_ = pair(rng, "f32", (3, 8), hip, oracle)
+    hi = [from_numpy(np.array(7, dtype=np.int32), "s32", hip), from_numpy(np.array(100, dtype=np.int64), "s64", hip)]
+    oi = [from_numpy(np.array(7, dtype=np.int32), "s32", oracle), from_numpy(np.array(100, dtype=np.int64), "s64", oracle)]
+    assert_bits_equal(Nx.put_slice(ht, hi, hs), Nx.put_slice(ot, oi, os_), "put_slice with tensor starts")
