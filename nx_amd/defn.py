@@ -629,6 +629,8 @@ def _fuse(roots: List[Tensor]) -> int:
 
     for r in roots:
         walk(r)
+    if any(t.data.op in ("while", "cond", "elem") for t in order):
+        return 0  # bodies of nested scopes read root-scope nodes that the counts above do not see
     taken, formed = set(), 0
     for root in reversed(order):  # consumers first: a group grows from its last node upwards
         if root.data.id in taken or not _fusable(root):

@@ -237,3 +237,49 @@ def test_shared_node_is_computed_once(on_oracle):
 @pytest.mark.parametrize("case", [c for c in CASES if c["fn"] != "key"], ids=[c["name"] for c in CASES if c["fn"] != "key"])
 def test_random_known_answers_through_a_trace(case, on_oracle):
     check_random_case(case, on_oracle, through=defn.jit)
+
+
+# ---- fused groups: the planner (the kernel itself is tested on the device) ---------------------------
+
+def test_fusion_groups_and_their_fallback_on_a_backend_without_the_kernel(on_oracle):
+    for name, fun in CHAINS.items():
+        args = build_args(on_oracle)[name]
+        fused = defn.compile(fun, *args, fuse=True)
+        assert_bits_equal(fused(*args), fun(*args), name)
+    assert defn.compile(CHAINS["elementwise_reduce"], *build_args(on_oracle)["elementwise_reduce"], fuse=True).fused_groups == 1
+    assert defn.compile(CHAINS["softmax"], *build_args(on_oracle)["softmax"], fuse=True).fused_groups == 2
+    assert defn.compile(CHAINS["argmax_take"], *build_args(on_oracle)["argmax_take"], fuse=True).fused_groups == 0
+
+
+def test_fusion_leaves_shared_and_returned_nodes_alone(on_oracle):
+    x = f32(np.linspace(-1, 1, 64), on_oracle)
+
+    def fun(t):
+        e = Nx.exp(t)                       # returned and consumed: must stay a node of its own
+        return e, Nx.multiply(Nx.add(e, 1.0), 2.0)
+    compiled = defn.compile(fun, x, fuse=True)
+    e, y = compiled(x)
+    assert compiled.roots[0].data.op == "exp" and compiled.roots[1].data.op == "fused"
+    assert_bits_equal(e, Nx.exp(x), "returned intermediate")
+    assert_bits_equal(y, Nx.multiply(Nx.add(Nx.exp(x), 1.0), 2.0), "group above it")
+
+
+def test_fusion_is_skipped_when_the_function_has_control_flow(on_oracle):
+    x = f32([1.0, 2.0], on_oracle)
+
+    def fun(t):
+        doubled = Nx.multiply(Nx.add(t, 1.0), 2.0)
+        _, out = defn.while_loop((Nx.tensor(0), doubled), lambda s: Nx.less(s[0], 2), lambda s: (Nx.add(s[0], 1), Nx.add(s[1], doubled)))
+        return out
+    compiled = defn.compile(fun, x, fuse=True)
+    assert compiled.fused_groups == 0
+    assert Nx.to_numpy(compiled(x)).tolist() == [12.0, 18.0]
+
+
+def test_layout_of_a_group(on_oracle):
+    assert defn._layout((4, 16), [(4, 16), ()]) == (1, 64, [(0, 1), (0, 0)])
+    assert defn._layout((4, 16), [(4, 16), (16,)]) == (4, 16, [(16, 1), (0, 1)])
+    assert defn._layout((4, 16), [(4, 16), (4, 1)]) == (4, 16, [(16, 1), (1, 0)])
+    assert defn._layout((2, 3, 16), [(2, 3, 16), (2, 3, 1), (16,)]) == (6, 16, [(16, 1), (1, 0), (0, 1)])
+    assert defn._layout((5, 7), [(5, 7), (7,)]) is None            # rows are not whole vectors
+    assert defn._layout((4, 16), [(4, 16), (4, 1), (1, 16), (2, 1, 16)]) is None
