@@ -241,30 +241,34 @@ int hipnx_threefry2x32(hipnx_ctx *ctx, const hipnx_buf *key, int64_t n, hipnx_bu
 /* ---- fused element-wise chains ----------------------------------------------------------------
  * replaces: a group of element-wise callbacks that the reference's evaluator issues one by one
  * (nx/lib/nx/defn/evaluator.ex:363-388; the callbacks of nx/lib/nx/backend.ex:115-133) by one pass
- * over memory.  The group is a register program: every instruction writes one of
- * HIPNX_FUSED_REGS registers and rounds its value to `dt`, the type the node has in the
- * graph, so the result is what the separate kernels would have produced.
- * Input k starts out in register k (converted to f32; its element (row, col) is at
- * row * row_stride + col * col_stride), so at most HIPNX_FUSED_REGS inputs.
- *   CONST  dst = imm
- *   UNARY  dst = op(reg a)        op: HIPNX_EXP ... (not the integer-only ones)
- *   BINARY dst = op(reg a, reg b) op: HIPNX_ADD ... (not the integer-only ones)
- *   SELECT dst = reg a != 0 ? reg b : reg c
- *   AS_TYPE dst = reg a (rounded to dt)
- * Types: bf16 / f16 / f32 values, u8 truth values; inputs of at most 4 bytes per element.  The
- * index space is [rows, cols]; col strides are 1 or 0; with more than one row, cols and the row
- * strides of dense inputs are multiples of 8 (otherwise HIPNX_EUNSUPPORTED: run the nodes one by one). */
-enum { HIPNX_FUSED_CONST = 1, HIPNX_FUSED_UNARY, HIPNX_FUSED_BINARY, HIPNX_FUSED_SELECT, HIPNX_FUSED_AS_TYPE };
-enum { HIPNX_FUSED_REGS = 8, HIPNX_FUSED_MAX_INSTR = 32, HIPNX_FUSED_MAX_INPUTS = 7 };
+ * over memory.  The group is a program for an accumulator machine: the accumulator holds the
+ * value computed last, an instruction combines it with one other operand and rounds the result
+ * to `dt`, the type the node has in the graph, so the final value is what the separate kernels
+ * would have produced.
+ *   SET     acc = other
+ *   UNARY   acc = op(acc)                 op: HIPNX_EXP ... (not the integer-only ones)
+ *   BINARY  acc = op(acc, other)          op: HIPNX_ADD ... (not the integer-only ones);
+ *                                         flags bit 0: acc is the right operand, op(other, acc)
+ *   SELECT  acc = acc != 0 ? other : other2
+ *   AS_TYPE acc = acc (rounded to dt)
+ * `other` is (src, arg, imm): input number arg (converted to f32; its element (row, col) is at
+ * row * row_stride + col * col_stride), the constant imm, or saved slot arg; `other2` likewise
+ * with (src2, arg2, imm2).  flags bits 4..7: slot + 1 in which the result is also saved (0: none).
+ * The result of the last instruction is the output.  Types: bf16 / f16 / f32 values, u8 truth
+ * values; inputs of at most 4 bytes per element.  The index space is [rows, cols]; col strides
+ * are 1 or 0; cols, and with more than one row the row strides of dense inputs, are multiples
+ * of 8 (otherwise HIPNX_EUNSUPPORTED: run the nodes one by one). */
+enum { HIPNX_FUSED_SET = 0, HIPNX_FUSED_UNARY, HIPNX_FUSED_BINARY, HIPNX_FUSED_SELECT, HIPNX_FUSED_AS_TYPE };
+enum { HIPNX_FUSED_SRC_CONST = 0, HIPNX_FUSED_SRC_INPUT, HIPNX_FUSED_SRC_SAVED };
+enum { HIPNX_FUSED_SAVED = 3, HIPNX_FUSED_MAX_INSTR = 32, HIPNX_FUSED_MAX_INPUTS = 8 };
 typedef struct {
-  uint8_t kind, op, dst, a, b, c, dt, pad;
-  float imm;
-  uint32_t reserved;  /* 16 bytes: the interpreter fetches an instruction with one scalar load */
-} hipnx_fused_instr;
+  uint8_t kind, op, src, arg;
+  uint8_t src2, arg2, flags, dt;
+  float imm, imm2;
+} hipnx_fused_instr; /* 16 bytes: the interpreter fetches an instruction with one scalar load */
 int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_fused_instr *prog, int n_inputs,
                             const hipnx_buf *const *inputs, const int *in_dts, const int64_t *in_row_strides,
-                            const int *in_col_strides, int64_t rows, int64_t cols, int out_reg, int out_dt,
-                            hipnx_buf *out);
+                            const int *in_col_strides, int64_t rows, int64_t cols, int out_dt, hipnx_buf *out);
 
 /* ---- captured sequences ---------------------------------------------------------------------
  * The reference's evaluator (nx/lib/nx/defn/evaluator.ex:363-388) issues one callback per node

@@ -37,12 +37,13 @@ lib = C.CDLL(LIB_PATH)
 
 class FusedInstr(C.Structure):
     """hipnx_fused_instr of include/hipnx.h."""
-    _fields_ = [("kind", C.c_uint8), ("op", C.c_uint8), ("dst", C.c_uint8), ("a", C.c_uint8), ("b", C.c_uint8),
-                ("c", C.c_uint8), ("dt", C.c_uint8), ("pad", C.c_uint8), ("imm", C.c_float), ("reserved", C.c_uint32)]
+    _fields_ = [("kind", C.c_uint8), ("op", C.c_uint8), ("src", C.c_uint8), ("arg", C.c_uint8), ("src2", C.c_uint8),
+                ("arg2", C.c_uint8), ("flags", C.c_uint8), ("dt", C.c_uint8), ("imm", C.c_float), ("imm2", C.c_float)]
 
 
-FUSED_CONST, FUSED_UNARY, FUSED_BINARY, FUSED_SELECT, FUSED_AS_TYPE = range(1, 6)
-FUSED_REGS, FUSED_MAX_INSTR, FUSED_MAX_INPUTS = 8, 32, 7
+FUSED_SET, FUSED_UNARY, FUSED_BINARY, FUSED_SELECT, FUSED_AS_TYPE = range(5)
+FUSED_SRC_CONST, FUSED_SRC_INPUT, FUSED_SRC_SAVED = range(3)
+FUSED_SAVED, FUSED_MAX_INSTR, FUSED_MAX_INPUTS = 3, 32, 8
 
 _ctx_p, _buf_p = C.c_void_p, C.c_void_p
 _i64p, _intp = C.POINTER(C.c_int64), C.POINTER(C.c_int)
@@ -87,7 +88,7 @@ PROTOTYPES = {
     "hipnx_eye": [_ctx_p, C.c_int, C.c_int64, C.c_int64, C.c_int64, _buf_p],
     "hipnx_threefry2x32": [_ctx_p, _buf_p, C.c_int64, _buf_p],
     "hipnx_fused_elementwise": [_ctx_p, C.c_int, C.c_void_p, C.c_int, C.POINTER(C.c_void_p), _intp, _i64p, _intp, C.c_int64,
-                                C.c_int64, C.c_int, C.c_int, _buf_p],
+                                C.c_int64, C.c_int, _buf_p],
     "hipnx_capture_begin": [_ctx_p],
     "hipnx_capture_end": [_ctx_p, C.POINTER(C.c_void_p)],
     "hipnx_graph_launch": [C.c_void_p],

@@ -675,24 +675,28 @@ class HipNxBackend:
         return Tensor(cls(ref, backend_opts["device"]), ty, tuple(shape), tuple(opts.get("names") or ()))
 
     @classmethod
-    def fused_elementwise(cls, out: Tensor, program, out_reg: int, inputs, layout) -> Tensor:
+    def fused_elementwise(cls, out: Tensor, program, inputs, layout) -> Tensor:
         """A group of element-wise nodes in one kernel (the evaluator offers it groups it has found
-        in a traced function).  `program` is a list of (kind, op, dst, a, b, c, type, imm); `layout` is
-        (rows, cols, [(row_stride, col_stride) per input]).  Raises HipNxError with status
-        EUNSUPPORTED when the shapes do not vectorise: the caller then runs the nodes one by one."""
-        dev = cls._device_of(*inputs)
+        in a traced function).  `program` is a list of dicts with the fields of `hipnx_fused_instr`
+        (`dt` as a type tuple); `layout` is (rows, cols, [(row_stride, col_stride) per input]).
+        Raises HipNxError with status EUNSUPPORTED when the shapes do not vectorise: the caller then
+        runs the nodes one by one."""
+        dev = cls._device_of(*inputs) if inputs else 0
         inputs = [cls._from_nx(t, dev) for t in inputs]
         rows, cols, strides = layout
         prog = (L.FusedInstr * len(program))()
-        for q, (kind, op, dst, a, b, c, ty, imm) in zip(prog, program):
-            q.kind, q.op, q.dst, q.a, q.b, q.c, q.dt, q.imm = kind, op, dst, a, b, c, T.code(ty), imm
+        for q, ins in zip(prog, program):
+            q.kind, q.op, q.src, q.arg = ins["kind"], ins.get("op", 0), ins.get("src", 0), ins.get("arg", 0)
+            q.src2, q.arg2, q.flags, q.dt = ins.get("src2", 0), ins.get("arg2", 0), ins.get("flags", 0), T.code(ins["dt"])
+            q.imm, q.imm2 = ins.get("imm", 0.0), ins.get("imm2", 0.0)
         res = cls._alloc(out, dev)
-        handles = (C.c_void_p * max(len(inputs), 1))(*[cls._handle(t) for t in inputs])
-        dts = (C.c_int * max(len(inputs), 1))(*[T.code(t.type) for t in inputs])
-        rs = (C.c_int64 * max(len(inputs), 1))(*[s[0] for s in strides])
-        cs = (C.c_int * max(len(inputs), 1))(*[s[1] for s in strides])
+        n = max(len(inputs), 1)
+        handles = (C.c_void_p * n)(*[cls._handle(t) for t in inputs])
+        dts = (C.c_int * n)(*[T.code(t.type) for t in inputs])
+        rs = (C.c_int64 * n)(*[s[0] for s in strides])
+        cs = (C.c_int * n)(*[s[1] for s in strides])
         L.check(L.lib.hipnx_fused_elementwise(res.data.ref.ctx, len(program), C.cast(prog, C.c_void_p), len(inputs), handles,
-                                              dts, rs, cs, rows, cols, out_reg, T.code(out.type), res.data.ref.handle))
+                                              dts, rs, cs, rows, cols, T.code(out.type), res.data.ref.handle))
         return res
 
     @classmethod

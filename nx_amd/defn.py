@@ -450,8 +450,7 @@ _INT_ONLY_UNARY = ("bitwise_not", "count_leading_zeros", "population_count")
 _COMPARE = ("equal", "not_equal", "greater", "less", "greater_equal", "less_equal")
 _LOGICAL = ("logical_and", "logical_or", "logical_xor")
 _EXACT_WITH_INT_CONSTANT = ("add", "subtract", "multiply", "divide", "min", "max") + _COMPARE
-_KIND = {"const": 1, "unary": 2, "binary": 3, "select": 4, "as_type": 5}
-_MAX_REGS, _MAX_INSTR, _MAX_INPUTS = 8, 32, 8
+_SAVED_SLOTS, _MAX_INSTR, _MAX_INPUTS = 3, 32, 8
 
 
 def _fusable(t: Tensor) -> bool:
@@ -513,79 +512,109 @@ def _layout(out_shape, in_shapes):
 
 
 class _Group:
-    """One fused group: the member nodes in evaluation order, its external inputs, and the register
-    program for them (None when the group does not fit the kernel)."""
+    """One fused group: the member nodes in evaluation order, its external inputs, and the program
+    for the backend's accumulator machine (None when the group does not fit it)."""
 
     def __init__(self, root: Tensor, members: List[Tensor], inputs: List[Tensor]):
         self.root, self.members, self.inputs = root, members, inputs
-        self.program, self.out_reg = self._assemble()
+        self.program = self._assemble()
         self.layout = _layout(root.shape, [t.shape for t in inputs]) if self.program else None
 
     def _assemble(self):
+        """Linear code for the accumulator machine: each member combines the value computed just
+        before it (the accumulator) with one other operand; a value that is needed later than that
+        is saved in one of three slots, and fetched back (SET) when the accumulator holds
+        something else."""
         member_ids = {m.data.id: i for i, m in enumerate(self.members)}
         input_ids = {t.data.id: k for k, t in enumerate(self.inputs)}
-        if len(self.inputs) >= _MAX_REGS:
-            return None, None
-
-        def key(a):
-            if _const(a) is not None:
-                return ("c", a.type, _const(a))
-            return ("m", a.data.id) if a.data.id in member_ids else ("i", input_ids[a.data.id])
-
-        last_use: Dict[Any, int] = {}
+        if len(self.inputs) > _MAX_INPUTS:
+            return None
+        # where each member's value is read: (reader index, operand position)
+        readers: Dict[Any, List[int]] = {}
         for i, m in enumerate(self.members):
             for a in m.data.args:
-                if isinstance(a, Tensor):
-                    last_use[key(a)] = i
-        last_use[("m", self.root.data.id)] = len(self.members)
-        # input k starts out in register k; the others are handed out as values are born
-        where = {("i", k): k for k in range(len(self.inputs))}
-        free, program = list(range(len(self.inputs), _MAX_REGS)), []
+                if isinstance(a, Tensor) and a.data.id in member_ids:
+                    readers.setdefault(a.data.id, []).append(i)
+        slots: Dict[Any, int] = {}       # member id -> slot while it is saved
+        free = list(range(_SAVED_SLOTS))
+        program: List[dict] = []
 
-        def claim():
-            return free.pop(0) if free else None
+        def source(a):
+            """(src, arg, imm) of an operand that is not the accumulator."""
+            if _const(a) is not None:
+                return 0, 0, _imm(a)
+            if a.data.id in input_ids:
+                return 1, input_ids[a.data.id], 0.0
+            return 2, slots[a.data.id], 0.0
 
-        for k in range(len(self.inputs)):  # an input nobody reads (cannot happen) would hold its register
-            if ("i", k) not in last_use:
-                free.append(where.pop(("i", k)))
         for i, m in enumerate(self.members):
             operands = [a for a in m.data.args if isinstance(a, Tensor)]
-            for a in operands:
-                k = key(a)
-                if k in where:
-                    continue
-                reg = claim()  # only constants are born here: inputs and earlier members have registers
-                if reg is None:
-                    return None, None
-                where[k] = reg
-                program.append((_KIND["const"], 0, reg, 0, 0, 0, a.type if a.type in _NARROW else ("f", 32), _imm(a)))
-            regs = [where[key(a)] for a in operands]
-            for a in operands:  # operands read for the last time free their registers for the result
-                k = key(a)
-                if last_use.get(k) == i and k in where:
-                    free.insert(0, where.pop(k))
-            dst = claim()
-            if dst is None:
-                return None, None
-            where[("m", m.data.id)] = dst
+            prev = self.members[i - 1].data.id if i else None
+
+            def is_acc(a):
+                return prev is not None and _const(a) is None and a.data.id == prev
+
             op = m.data.op
-            if op in UNARY_OPS:
-                program.append((_KIND["unary"], UNARY_OPS.index(op), dst, regs[0], 0, 0, m.type, 0.0))
+            if op == "select":
+                want_acc = [0]           # the predicate
             elif op in BINARY_OPS:
-                program.append((_KIND["binary"], BINARY_OPS.index(op), dst, regs[0], regs[1], 0, m.type, 0.0))
-            elif op == "select":
-                program.append((_KIND["select"], 0, dst, regs[0], regs[1], regs[2], m.type, 0.0))
+                want_acc = [0, 1]
             else:
-                program.append((_KIND["as_type"], 0, dst, regs[0], 0, 0, m.type, 0.0))
+                want_acc = [0]
+            pos = next((p for p in want_acc if is_acc(operands[p])), None)
+            if pos is None:  # the accumulator holds something else: fetch the operand
+                pos = want_acc[0]
+                first = operands[pos]
+                if first.data.id in member_ids and _const(first) is None and first.data.id not in slots:
+                    return None          # cannot happen: a member read later than next is saved below
+                src, arg, imm = source(first)
+                program.append({"kind": 0, "src": src, "arg": arg, "imm": imm,
+                                "dt": first.type if first.type in _NARROW or first.type == _TRUTH else ("f", 32)})
+            others = [a for p, a in enumerate(operands) if p != pos]
+            if any(_const(o) is None and o.data.id in member_ids and o.data.id not in slots for o in others):
+                return None              # an operand that is neither the accumulator nor saved: cannot happen
+            ins = {"dt": m.type}
+            if op in UNARY_OPS:
+                ins.update(kind=1, op=UNARY_OPS.index(op))
+            elif op in BINARY_OPS:
+                src, arg, imm = source(others[0])
+                ins.update(kind=2, op=BINARY_OPS.index(op), src=src, arg=arg, imm=imm, flags=1 if pos == 1 else 0)
+            elif op == "select":
+                (s1, a1, i1), (s2, a2, i2) = source(others[0]), source(others[1])
+                ins.update(kind=3, src=s1, arg=a1, imm=i1, src2=s2, arg2=a2, imm2=i2)
+            else:
+                ins.update(kind=4)
+            # slots whose value was read for the last time here are free again
+            for a in operands:
+                if _const(a) is None and a.data.id in slots and max(readers[a.data.id]) == i:
+                    free.insert(0, slots.pop(a.data.id))
+            # does this result outlive the next instruction's accumulator read?
+            later = [r for r in readers.get(m.data.id, []) if r != i + 1]
+            next_reads = i + 1 < len(self.members) and (i + 1) in readers.get(m.data.id, [])
+            next_op = self.members[i + 1].data if i + 1 < len(self.members) else None
+            # the next member can only take it from the accumulator in an operand position it accepts
+            takes_acc = False
+            if next_reads:
+                nxt_operands = [a for a in next_op.args if isinstance(a, Tensor)]
+                accept = [0] if next_op.op == "select" or next_op.op not in BINARY_OPS else [0, 1]
+                hits = [p for p, a in enumerate(nxt_operands) if _const(a) is None and a.data.id == m.data.id]
+                takes_acc = len(hits) == 1 and hits[0] in accept
+            if later or (next_reads and not takes_acc):
+                if not free:
+                    return None
+                slot = free.pop(0)
+                slots[m.data.id] = slot
+                ins["flags"] = ins.get("flags", 0) | ((slot + 1) << 4)
+            program.append(ins)
             if len(program) > _MAX_INSTR:
-                return None, None
-        return program, where[("m", self.root.data.id)]
+                return None
+        return program
 
     def run(self, run: "_Run", out: Tensor, values: List[Tensor]):
         mod = run.pick(values)
         fused = getattr(mod, "fused_elementwise", None) if self.program and self.layout else None
         if fused is not None:
-            return fused(out, self.program, self.out_reg, values, self.layout)
+            return fused(out, self.program, values, self.layout)
         # node by node, on the callbacks (a backend without the kernel, or a group that does not fit)
         done = {t.data.id: v for t, v in zip(self.inputs, values)}
         for m in self.members:

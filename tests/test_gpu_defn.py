@@ -195,7 +195,14 @@ def rand_float(rng, ty, shape, backend):
     return from_numpy(v.astype(np.float16 if ty == "f16" else np.float32), ty, backend)
 
 
+def reuse_and_square(x, y):
+    s = Nx.add(x, y)
+    return Nx.multiply(Nx.multiply(s, s), Nx.subtract(s, x))   # op(s, s) and three reads of one value
+
+
 FUSED_CASES = {
+    "reuse_and_square": (reuse_and_square, lambda rng, b: (rand_float(rng, "f32", (40, 64), b), rand_float(rng, "f32", (40, 64), b))),
+    "long_rows_tail": (gelu_like, lambda rng, b: (rand_float(rng, "f32", (3, 4104), b), rand_float(rng, "f32", (4104,), b))),
     "gelu_like": (gelu_like, lambda rng, b: (rand_float(rng, "f32", (64, 256), b), rand_float(rng, "f32", (256,), b))),
     "gelu_like_bf16": (gelu_like, lambda rng, b: (rand_float(rng, "bf16", (8, 16, 128), b), rand_float(rng, "bf16", (128,), b))),
     "relu_mask": (relu_mask, lambda rng, b: (rand_float(rng, "f32", (1000, 24), b), rand_float(rng, "f32", (1000, 24), b))),
@@ -241,14 +248,20 @@ def test_fused_kernel_is_the_path_taken(hip):
 
 
 def test_fused_entry_point_validates_its_program(hip):
-    from nx_amd._lib import FUSED_BINARY, FUSED_UNARY, HipNxError
+    from nx_amd._lib import FUSED_BINARY, FUSED_SET, FUSED_SRC_INPUT, FUSED_SRC_SAVED, FUSED_UNARY, HipNxError
     x = rand_float(np.random.default_rng(1), "f32", (16,), hip)
     out = x.with_(data=None)
-    with pytest.raises(HipNxError, match="unwritten register"):
-        hip.fused_elementwise(out, [(FUSED_BINARY, 0, 1, 0, 2, 0, ("f", 32), 0.0)], 1, [x], (1, 16, [(0, 1)]))
+    flat = (1, 16, [(0, 1)])
+    load = {"kind": FUSED_SET, "src": FUSED_SRC_INPUT, "arg": 0, "dt": ("f", 32)}
+    with pytest.raises(HipNxError, match="before anything set it"):
+        hip.fused_elementwise(out, [{"kind": FUSED_UNARY, "op": 0, "dt": ("f", 32)}], [x], flat)
+    with pytest.raises(HipNxError, match="reads an input that is not there"):
+        hip.fused_elementwise(out, [dict(load, arg=3)], [x], flat)
+    with pytest.raises(HipNxError, match="reads an empty slot"):
+        hip.fused_elementwise(out, [load, {"kind": FUSED_BINARY, "op": 0, "src": FUSED_SRC_SAVED, "arg": 1, "dt": ("f", 32)}], [x], flat)
     with pytest.raises(HipNxError, match="binary op"):
-        hip.fused_elementwise(out, [(FUSED_BINARY, 9, 1, 0, 0, 0, ("f", 32), 0.0)], 1, [x], (1, 16, [(0, 1)]))
+        hip.fused_elementwise(out, [load, {"kind": FUSED_BINARY, "op": 9, "src": FUSED_SRC_INPUT, "arg": 0, "dt": ("f", 32)}], [x], flat)
     with pytest.raises(HipNxError, match="holds"):
-        hip.fused_elementwise(out.with_(shape=(32,)), [(FUSED_UNARY, 0, 1, 0, 0, 0, ("f", 32), 0.0)], 1, [x], (1, 32, [(0, 1)]))
-    got = hip.fused_elementwise(out, [(FUSED_UNARY, 27, 1, 0, 0, 0, ("f", 32), 0.0)], 1, [x], (1, 16, [(0, 1)]))  # negate
+        hip.fused_elementwise(out.with_(shape=(32,)), [load], [x], (1, 32, [(0, 1)]))
+    got = hip.fused_elementwise(out, [load, {"kind": FUSED_UNARY, "op": 27, "dt": ("f", 32)}], [x], flat)  # negate
     np.testing.assert_array_equal(hip.to_numpy(got), -hip.to_numpy(x))
