@@ -257,7 +257,10 @@ int hipnx_threefry2x32(hipnx_ctx *ctx, const hipnx_buf *key, int64_t n, hipnx_bu
  * The result of the last instruction is the output.  Types: bf16 / f16 / f32 values, u8 truth
  * values; inputs of at most 4 bytes per element.  The index space is [rows, cols]; col strides
  * are 1 or 0; cols, and with more than one row the row strides of dense inputs, are multiples
- * of 8 (otherwise HIPNX_EUNSUPPORTED: run the nodes one by one). */
+ * of 8 (otherwise HIPNX_EUNSUPPORTED: run the nodes one by one).
+ * reduce_op: -1, or HIPNX_RED_SUM / MAX / MIN to reduce the result along its rows without storing it
+ * (sum/4, reduce_max/4, reduce_min/4 over the last axis, nx/lib/nx/backend.ex:89-92): `out` then has
+ * `rows` elements, and equals the separate reduction kernel applied to the stored result. */
 enum { HIPNX_FUSED_SET = 0, HIPNX_FUSED_UNARY, HIPNX_FUSED_BINARY, HIPNX_FUSED_SELECT, HIPNX_FUSED_AS_TYPE };
 enum { HIPNX_FUSED_SRC_CONST = 0, HIPNX_FUSED_SRC_INPUT, HIPNX_FUSED_SRC_SAVED };
 enum { HIPNX_FUSED_SAVED = 3, HIPNX_FUSED_MAX_INSTR = 32, HIPNX_FUSED_MAX_INPUTS = 8 };
@@ -268,7 +271,8 @@ typedef struct {
 } hipnx_fused_instr; /* 16 bytes: the interpreter fetches an instruction with one scalar load */
 int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_fused_instr *prog, int n_inputs,
                             const hipnx_buf *const *inputs, const int *in_dts, const int64_t *in_row_strides,
-                            const int *in_col_strides, int64_t rows, int64_t cols, int out_dt, hipnx_buf *out);
+                            const int *in_col_strides, int64_t rows, int64_t cols, int reduce_op, int out_dt,
+                            hipnx_buf *out);
 
 /* ---- captured sequences ---------------------------------------------------------------------
  * The reference's evaluator (nx/lib/nx/defn/evaluator.ex:363-388) issues one callback per node

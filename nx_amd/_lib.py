@@ -88,7 +88,7 @@ PROTOTYPES = {
     "hipnx_eye": [_ctx_p, C.c_int, C.c_int64, C.c_int64, C.c_int64, _buf_p],
     "hipnx_threefry2x32": [_ctx_p, _buf_p, C.c_int64, _buf_p],
     "hipnx_fused_elementwise": [_ctx_p, C.c_int, C.c_void_p, C.c_int, C.POINTER(C.c_void_p), _intp, _i64p, _intp, C.c_int64,
-                                C.c_int64, C.c_int, _buf_p],
+                                C.c_int64, C.c_int, C.c_int, _buf_p],
     "hipnx_capture_begin": [_ctx_p],
     "hipnx_capture_end": [_ctx_p, C.POINTER(C.c_void_p)],
     "hipnx_graph_launch": [C.c_void_p],

@@ -675,12 +675,13 @@ class HipNxBackend:
         return Tensor(cls(ref, backend_opts["device"]), ty, tuple(shape), tuple(opts.get("names") or ()))
 
     @classmethod
-    def fused_elementwise(cls, out: Tensor, program, inputs, layout) -> Tensor:
+    def fused_elementwise(cls, out: Tensor, program, inputs, layout, reduce_op: int = -1) -> Tensor:
         """A group of element-wise nodes in one kernel (the evaluator offers it groups it has found
         in a traced function).  `program` is a list of dicts with the fields of `hipnx_fused_instr`
         (`dt` as a type tuple); `layout` is (rows, cols, [(row_stride, col_stride) per input]).
-        Raises HipNxError with status EUNSUPPORTED when the shapes do not vectorise: the caller then
-        runs the nodes one by one."""
+        `reduce_op` (RED_SUM / RED_MAX / RED_MIN) reduces the group's value along its rows without
+        storing it; `out` is then the reduction's template.  Raises HipNxError with status
+        EUNSUPPORTED when the shapes do not fit the kernel: the caller then runs the nodes one by one."""
         dev = cls._device_of(*inputs) if inputs else 0
         inputs = [cls._from_nx(t, dev) for t in inputs]
         rows, cols, strides = layout
@@ -696,7 +697,7 @@ class HipNxBackend:
         rs = (C.c_int64 * n)(*[s[0] for s in strides])
         cs = (C.c_int * n)(*[s[1] for s in strides])
         L.check(L.lib.hipnx_fused_elementwise(res.data.ref.ctx, len(program), C.cast(prog, C.c_void_p), len(inputs), handles,
-                                              dts, rs, cs, rows, cols, T.code(out.type), res.data.ref.handle))
+                                              dts, rs, cs, rows, cols, reduce_op, T.code(out.type), res.data.ref.handle))
         return res
 
     @classmethod

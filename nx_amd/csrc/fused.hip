@@ -21,6 +21,7 @@
 // Bound by HBM: bytes(inputs) + bytes(out).
 #include "elementwise_ops.cuh"
 #include "internal.h"
+#include "reduce_ops.cuh"
 
 namespace hipnx {
 
@@ -203,6 +204,52 @@ __device__ __forceinline__ void fetch(KernArgs a, const Saved &S, int src, int a
   }
 }
 
+// the program for the lane's vector at (row, col); the result is left in `acc`
+template <bool FULL>
+__device__ __forceinline__ void run_program(KernArgs a, int n_instr, const int64_t (&row)[FV], const int64_t (&col)[FV], Vecs &acc) {
+  typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+  typedef const __attribute__((address_space(4))) u32x4 *InstrWords;
+  Vecs y, z;
+  Saved S;
+  u32x4 next = *(InstrWords)&a->ins[0];
+  for (int pc = 0; pc < n_instr; pc++) {
+    // one 16-byte scalar load per instruction, requested one instruction ahead
+    const u32x4 q = next;
+    if (pc + 1 < n_instr) next = *(InstrWords)&a->ins[pc + 1];
+    const int kind = q.x & 0xFF, op = (q.x >> 8) & 0xFF, src = (q.x >> 16) & 0xFF, arg = q.x >> 24;
+    const int src2 = q.y & 0xFF, arg2 = (q.y >> 8) & 0xFF, flags = (q.y >> 16) & 0xFF, dt = q.y >> 24;
+    switch (kind) {
+      case HIPNX_FUSED_SET:
+        fetch(a, S, src, arg, __uint_as_float(q.z), row, col, acc);
+        break;
+      case HIPNX_FUSED_UNARY:
+        unary_all<FULL>(std::make_integer_sequence<int, HIPNX_NUNARY>{}, op, acc);
+        break;
+      case HIPNX_FUSED_BINARY:
+        fetch(a, S, src, arg, __uint_as_float(q.z), row, col, y);
+        binary_all<FULL>(std::make_integer_sequence<int, HIPNX_NBINARY>{}, op, acc, y, (flags & 1) != 0);
+        break;
+      case HIPNX_FUSED_SELECT:
+        fetch(a, S, src, arg, __uint_as_float(q.z), row, col, y);
+        fetch(a, S, src2, arg2, __uint_as_float(q.w), row, col, z);
+#pragma unroll
+        for (int u = 0; u < FV; u++)
+#pragma unroll
+          for (int e = 0; e < FE; e++) acc[u][e] = acc[u][e] != 0.0f ? y[u][e] : z[u][e];  // NaN is true
+        break;
+      default:  // HIPNX_FUSED_AS_TYPE: the rounding below is the conversion
+        break;
+    }
+    if (dt == HIPNX_BF16 || dt == HIPNX_F16) {
+#pragma unroll
+      for (int u = 0; u < FV; u++)
+#pragma unroll
+        for (int e = 0; e < FE; e++) acc[u][e] = round_to(acc[u][e], dt);
+    }
+    if (flags >> 4) write_saved(S, (flags >> 4) - 1, acc);
+  }
+}
+
 template <bool FULL>
 __global__ void __launch_bounds__(FBLOCK) fused_elementwise_kernel(FusedArgs by_value) {
   (void)by_value;
@@ -210,8 +257,6 @@ __global__ void __launch_bounds__(FBLOCK) fused_elementwise_kernel(FusedArgs by_
   const int64_t nvec = a->nvec, vecs_per_row = a->vecs_per_row, cols = a->cols;
   const int n_instr = a->n_instr;
   const int64_t stride = (int64_t)gridDim.x * FBLOCK;
-  typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-  typedef const __attribute__((address_space(4))) u32x4 *InstrWords;
   for (int64_t v0 = (int64_t)blockIdx.x * FBLOCK + threadIdx.x; v0 < nvec; v0 += stride * FV) {
     int64_t row[FV], col[FV];
     bool live[FV];
@@ -227,50 +272,62 @@ __global__ void __launch_bounds__(FBLOCK) fused_elementwise_kernel(FusedArgs by_
         col[u] = (v - row[u] * vecs_per_row) * FE;
       }
     }
-    Vecs acc, y, z;
-    Saved S;
-    u32x4 next = *(InstrWords)&a->ins[0];
-    for (int pc = 0; pc < n_instr; pc++) {
-      // one 16-byte scalar load per instruction, requested one instruction ahead
-      const u32x4 q = next;
-      if (pc + 1 < n_instr) next = *(InstrWords)&a->ins[pc + 1];
-      const int kind = q.x & 0xFF, op = (q.x >> 8) & 0xFF, src = (q.x >> 16) & 0xFF, arg = q.x >> 24;
-      const int src2 = q.y & 0xFF, arg2 = (q.y >> 8) & 0xFF, flags = (q.y >> 16) & 0xFF, dt = q.y >> 24;
-      switch (kind) {
-        case HIPNX_FUSED_SET:
-          fetch(a, S, src, arg, __uint_as_float(q.z), row, col, acc);
-          break;
-        case HIPNX_FUSED_UNARY:
-          unary_all<FULL>(std::make_integer_sequence<int, HIPNX_NUNARY>{}, op, acc);
-          break;
-        case HIPNX_FUSED_BINARY:
-          fetch(a, S, src, arg, __uint_as_float(q.z), row, col, y);
-          binary_all<FULL>(std::make_integer_sequence<int, HIPNX_NBINARY>{}, op, acc, y, (flags & 1) != 0);
-          break;
-        case HIPNX_FUSED_SELECT:
-          fetch(a, S, src, arg, __uint_as_float(q.z), row, col, y);
-          fetch(a, S, src2, arg2, __uint_as_float(q.w), row, col, z);
-#pragma unroll
-          for (int u = 0; u < FV; u++)
-#pragma unroll
-            for (int e = 0; e < FE; e++) acc[u][e] = acc[u][e] != 0.0f ? y[u][e] : z[u][e];  // NaN is true
-          break;
-        default:  // HIPNX_FUSED_AS_TYPE: the rounding below is the conversion
-          break;
-      }
-      if (dt == HIPNX_BF16 || dt == HIPNX_F16) {
-#pragma unroll
-        for (int u = 0; u < FV; u++)
-#pragma unroll
-          for (int e = 0; e < FE; e++) acc[u][e] = round_to(acc[u][e], dt);
-      }
-      if (flags >> 4) write_saved(S, (flags >> 4) - 1, acc);
-    }
+    Vecs acc;
+    run_program<FULL>(a, n_instr, row, col, acc);
     void *out = (void *)a->out;
     const int odt = a->out_dt;
 #pragma unroll
     for (int u = 0; u < FV; u++)
       if (live[u]) store_vec<float, FE>(out, odt, row[u] * cols + col[u], acc[u]);
+  }
+}
+
+// The group's result reduced along its rows without ever being stored: TPR lanes per row walk it
+// in the order of reduce_rows_kernel (lane l takes the vectors l, l + TPR, ... and folds their
+// elements in turn, then lanes combine by wave shuffles and the block's waves through LDS) with the
+// same reducer policy, so the value equals what the element-wise group followed by the separate
+// reduction kernel gives, bit for bit.
+template <typename R, typename CT, int TPR>
+__global__ void __launch_bounds__(FBLOCK) fused_reduce_rows_kernel(FusedArgs by_value) {
+  (void)by_value;
+  static_assert(FV == 1, "one vector per lane and step");
+  KernArgs a = (KernArgs)__builtin_amdgcn_kernarg_segment_ptr();
+  constexpr int RPB = FBLOCK / TPR;
+  const int sub = threadIdx.x / TPR, lane = threadIdx.x % TPR;
+  const int64_t rows = a->rows, red = a->cols;
+  const int n_instr = a->n_instr;
+  const int64_t r = (int64_t)blockIdx.x * RPB + sub;
+  typename R::acc_t acc = R::init();
+  if (r < rows) {
+    const int64_t step = (int64_t)TPR * FE;
+    for (int64_t k = (int64_t)lane * FE; k < red; k += step) {
+      const int64_t row[FV] = {r}, col[FV] = {k};
+      Vecs x;
+      run_program<false>(a, n_instr, row, col, x);
+#pragma unroll
+      for (int e = 0; e < FE; e++) acc = R::accumulate(acc, (CT)x[0][e], k + e);
+    }
+  }
+  acc = wave_reduce<R>(acc);
+  if constexpr (TPR > WAVE) {
+    __shared__ typename R::acc_t sm[FBLOCK / WAVE];
+    if (threadIdx.x % WAVE == 0) sm[threadIdx.x / WAVE] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+#pragma unroll
+      for (int w = 1; w < FBLOCK / WAVE; w++) acc = R::combine(acc, sm[w]);
+    }
+  }
+  if (lane == 0 && r < rows) finalize((void *)a->out, a->out_dt, r, acc);
+}
+
+template <typename R, typename CT>
+static void launch_fused_reduce(const hipnx_ctx *ctx, const FusedArgs &a) {
+  if (a.cols <= 4096) {
+    const int rpb = FBLOCK / WAVE;
+    hipLaunchKernelGGL((fused_reduce_rows_kernel<R, CT, WAVE>), dim3((unsigned)((a.rows + rpb - 1) / rpb)), dim3(FBLOCK), 0, ctx->stream, a);
+  } else {
+    hipLaunchKernelGGL((fused_reduce_rows_kernel<R, CT, FBLOCK>), dim3((unsigned)a.rows), dim3(FBLOCK), 0, ctx->stream, a);
   }
 }
 
@@ -282,7 +339,8 @@ using namespace hipnx;
 
 extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_fused_instr *prog, int n_inputs,
                                        const hipnx_buf *const *inputs, const int *in_dts, const int64_t *in_row_strides,
-                                       const int *in_col_strides, int64_t rows, int64_t cols, int out_dt, hipnx_buf *out) {
+                                       const int *in_col_strides, int64_t rows, int64_t cols, int reduce_op, int out_dt,
+                                       hipnx_buf *out) {
   Enter in(ctx);
   if (in.status) return in.status;
   if (n_instr < 1 || n_instr > HIPNX_FUSED_MAX_INSTR || !prog)
@@ -291,6 +349,8 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
     return set_error(HIPNX_EINVAL, "fused: 0 .. %d inputs", HIPNX_FUSED_MAX_INPUTS);
   if (rows < 0 || cols < 0) return set_error(HIPNX_EINVAL, "fused: negative extent");
   if (!narrow(out_dt) && out_dt != HIPNX_U8) return set_error(HIPNX_EUNSUPPORTED, "fused: result type %d", out_dt);
+  if (reduce_op != -1 && reduce_op != HIPNX_RED_SUM && reduce_op != HIPNX_RED_MAX && reduce_op != HIPNX_RED_MIN)
+    return set_error(HIPNX_EUNSUPPORTED, "fused: reduction %d (sum, max and min along the rows are built)", reduce_op);
   FusedArgs a{};
   a.n_instr = n_instr;
   a.n_inputs = n_inputs;
@@ -353,7 +413,14 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
     a.in_rs[k] = in_row_strides[k];
     a.in_cs[k] = in_col_strides[k];
   }
-  if (int st = check_buf(ctx, out, (uint64_t)n * dtype_size(out_dt), "fused out")) return st;
+  if (reduce_op != -1) {
+    if (full) return set_error(HIPNX_EUNSUPPORTED, "fused: a reduction after a program with pow, atan2, remainder, trigonometric or erf functions");
+    if (!narrow(prog[n_instr - 1].dt) || !narrow(out_dt)) return set_error(HIPNX_EUNSUPPORTED, "fused: a reduction of a non-float value");
+    if (cols == 0) return set_error(HIPNX_EUNSUPPORTED, "fused: a reduction over an empty axis");
+    // a few very long rows are split into segments by the separate reduction: not here
+    if (rows < (int64_t)ctx->num_cus * 8 && cols >= 2 * 16384) return set_error(HIPNX_EUNSUPPORTED, "fused: rows that the reduction would split");
+  }
+  if (int st = check_buf(ctx, out, (uint64_t)(reduce_op == -1 ? n : rows) * dtype_size(out_dt), "fused out")) return st;
   if (n == 0) return HIPNX_OK;
   a.out = out->ptr;
   a.out_dt = out_dt;
@@ -361,6 +428,13 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
   a.cols = cols;
   a.vecs_per_row = cols / FE;
   a.nvec = rows * a.vecs_per_row;
+  if (reduce_op == HIPNX_RED_SUM) launch_fused_reduce<PlainReducer<double, HIPNX_RED_SUM, false>, double>(ctx, a);
+  else if (reduce_op == HIPNX_RED_MAX) launch_fused_reduce<PlainReducer<float, HIPNX_RED_MAX, false>, float>(ctx, a);
+  else if (reduce_op == HIPNX_RED_MIN) launch_fused_reduce<PlainReducer<float, HIPNX_RED_MIN, false>, float>(ctx, a);
+  if (reduce_op != -1) {
+    HIPNX_HIP(hipGetLastError());
+    return HIPNX_OK;
+  }
   int64_t blocks = (a.nvec + (int64_t)FBLOCK * FV - 1) / ((int64_t)FBLOCK * FV);
   if (blocks > (1ll << 30)) blocks = 1ll << 30;
   if (full) hipLaunchKernelGGL((fused_elementwise_kernel<true>), dim3((unsigned)blocks), dim3(FBLOCK), 0, ctx->stream, a);

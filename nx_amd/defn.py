@@ -451,6 +451,8 @@ _COMPARE = ("equal", "not_equal", "greater", "less", "greater_equal", "less_equa
 _LOGICAL = ("logical_and", "logical_or", "logical_xor")
 _EXACT_WITH_INT_CONSTANT = ("add", "subtract", "multiply", "divide", "min", "max") + _COMPARE
 _SAVED_SLOTS, _MAX_INSTR, _MAX_INPUTS = 3, 32, 8
+_REDUCE_CODES = {"sum": 0, "reduce_max": 1, "reduce_min": 2}  # HIPNX_RED_SUM / MAX / MIN
+_EUNSUPPORTED = 7
 
 
 def _fusable(t: Tensor) -> bool:
@@ -485,12 +487,14 @@ def _fusable(t: Tensor) -> bool:
     return False
 
 
-def _layout(out_shape, in_shapes):
+def _layout(out_shape, in_shapes, split=None):
     """The index space as [rows, cols] with a (row stride, column stride) per input, or None: an
-    input is the full shape, one value, one row shared by all rows, or one value per row."""
+    input is the full shape, one value, one row shared by all rows, or one value per row.  `split`
+    fixes the axis where the columns begin (a reduction over the last axis needs the rows it
+    reduces)."""
     rank = len(out_shape)
     padded = [(1,) * (rank - len(s)) + tuple(s) for s in in_shapes]
-    for p in range(rank + 1):
+    for p in (range(rank + 1) if split is None else [split]):
         rows, cols = prod(out_shape[:p]), prod(out_shape[p:])
         if cols % 8:  # the kernel works on whole vectors of 8 along a row
             continue
@@ -519,6 +523,21 @@ class _Group:
         self.root, self.members, self.inputs = root, members, inputs
         self.program = self._assemble()
         self.layout = _layout(root.shape, [t.shape for t in inputs]) if self.program else None
+        self.reduce = None  # (callback name, opts, rows layout) when a reduction of the result is part of the group
+
+    def with_reduction(self, name: str, opts) -> Optional["_Group"]:
+        """This group followed by `name` over the last axis of its result, or None when the
+        backend kernel cannot take it (the reduction then stays a node of its own)."""
+        rank = len(self.root.shape)
+        if not self.program or rank == 0 or self.root.type not in _NARROW:
+            return None
+        rows_layout = _layout(self.root.shape, [t.shape for t in self.inputs], split=rank - 1)
+        if rows_layout is None or rows_layout[1] == 0:
+            return None
+        both = object.__new__(_Group)
+        both.__dict__.update(self.__dict__)
+        both.reduce = (name, dict(opts), rows_layout)
+        return both
 
     def _assemble(self):
         """Linear code for the accumulator machine: each member combines the value computed just
@@ -613,6 +632,19 @@ class _Group:
     def run(self, run: "_Run", out: Tensor, values: List[Tensor]):
         mod = run.pick(values)
         fused = getattr(mod, "fused_elementwise", None) if self.program and self.layout else None
+        if self.reduce is not None:
+            name, opts, rows_layout = self.reduce
+            if fused is not None:
+                try:
+                    return fused(out, self.program, values, rows_layout, _REDUCE_CODES[name])
+                except Exception as e:  # a shape the kernel leaves to the separate reduction
+                    if getattr(e, "status", None) != _EUNSUPPORTED:
+                        raise
+            plain = object.__new__(_Group)
+            plain.__dict__.update(self.__dict__)
+            plain.reduce = None
+            value = plain.run(run, self.root.with_(data=None), values)
+            return getattr(run.pick([value]), name)(out, value, opts)
         if fused is not None:
             return fused(out, self.program, values, self.layout)
         # node by node, on the callbacks (a backend without the kernel, or a group that does not fit)
@@ -697,6 +729,22 @@ def _fuse(roots: List[Tensor]) -> int:
         taken.update(members)
         root.data.op, root.data.args = "fused", [group, inputs]
         formed += 1
+    # a reduction over the last axis whose operand is a group nobody else reads joins that group
+    for node in order:
+        e = node.data
+        if e.op not in _REDUCE_CODES or not isinstance(e.args[0], Tensor):
+            continue
+        operand, opts = e.args[0], e.args[1]
+        inner = operand.data
+        if not isinstance(inner, Expr) or inner.op != "fused" or uses.get(inner.id) != 1:
+            continue
+        rank = len(operand.shape)
+        if list(opts.get("axes") or []) != [rank - 1]:
+            continue
+        both = inner.args[0].with_reduction(e.op, opts)
+        if both is None:
+            continue
+        e.op, e.args = "fused", [both, inner.args[1]]
     return formed
 
 

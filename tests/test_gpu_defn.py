@@ -10,7 +10,7 @@ from nx_amd import nx as Nx
 from nx_amd import random as Random
 from nx_amd.backend import mem_stats
 from random_support import CASES, check_random_case
-from support import assert_all_close, assert_bits_equal, from_numpy
+from support import assert_all_close, assert_bits_equal, from_numpy, seed_of
 from test_defn import CHAINS, build_args, f32
 
 pytestmark = pytest.mark.gpu
@@ -265,3 +265,55 @@ def test_fused_entry_point_validates_its_program(hip):
         hip.fused_elementwise(out.with_(shape=(32,)), [load], [x], (1, 32, [(0, 1)]))
     got = hip.fused_elementwise(out, [load, {"kind": FUSED_UNARY, "op": 27, "dt": ("f", 32)}], [x], flat)  # negate
     np.testing.assert_array_equal(hip.to_numpy(got), -hip.to_numpy(x))
+
+
+# ---- a reduction over the last axis joins the group that feeds it ----------------------------------------
+
+def sum_of_exp(a, b):
+    return Nx.sum(Nx.exp(Nx.multiply(Nx.add(a, b), 0.5)), axes=[1])
+
+
+def max_of_scaled(a, b):
+    return Nx.reduce_max(Nx.multiply(Nx.subtract(a, b), 0.125), axes=[-1], keep_axes=True)
+
+
+def min_of_bf16(a, b):
+    return Nx.reduce_min(Nx.as_type(Nx.add(a, b), "bf16"), axes=[1])
+
+
+REDUCED = {"sum_of_exp": sum_of_exp, "max_of_scaled": max_of_scaled, "min_of_bf16": min_of_bf16}
+
+
+@pytest.mark.parametrize("name", sorted(REDUCED))
+@pytest.mark.parametrize("shape", [(64, 256), (300, 4096), (16, 8192), (5, 40000), (4, 65536), (2049, 8), (3, 7, 512)])
+def test_group_with_its_row_reduction_is_bit_identical(name, shape, hip):
+    rng = np.random.default_rng(seed_of(name, shape))
+    if len(shape) == 3 and name == "sum_of_exp":
+        pytest.skip("this function reduces axis 1, which is the last axis only for matrices")
+    fun = REDUCED[name]
+    if len(shape) == 3 and name == "min_of_bf16":
+        fun = lambda a, b: Nx.reduce_min(Nx.as_type(Nx.add(a, b), "bf16"), axes=[2])  # noqa: E731
+    args = (rand_float(rng, "f32", shape, hip), rand_float(rng, "f32", shape, hip))
+    fused = defn.compile(fun, *args, fuse=True)
+    assert fused.fused_groups == 1 and fused.roots[0].data.op == "fused" and fused.roots[0].data.args[0].reduce is not None
+    assert_bits_equal(fused(*args), defn.compile(fun, *args)(*args), f"{name} {shape}")
+
+
+def test_reduction_stays_separate_when_its_operand_is_read_elsewhere(hip):
+    args = build_args(hip)["softmax"]
+    fused = defn.compile(CHAINS["softmax"], *args, fuse=True)
+    assert_bits_equal(fused(*args), defn.compile(CHAINS["softmax"], *args)(*args), "softmax")
+
+    def seen(t, acc):
+        e = t.data
+        if e.op == "fused":
+            acc.append(e.args[0])
+            for i in e.args[1]:
+                seen(i, acc)
+        elif e.op not in ("parameter", "constant", "tensor"):
+            for ch in defn._children(e):
+                if isinstance(ch, defn.Tensor):
+                    seen(ch, acc)
+    groups = []
+    seen(fused.roots[0], groups)
+    assert groups and all(g.reduce is None for g in groups)
