@@ -692,28 +692,60 @@ def _fuse(roots: List[Tensor]) -> int:
         walk(r)
     if any(t.data.op in ("while", "cond", "elem") for t in order):
         return 0  # bodies of nested scopes read root-scope nodes that the counts above do not see
-    taken, formed = set(), 0
-    for root in reversed(order):  # consumers first: a group grows from its last node upwards
-        if root.data.id in taken or not _fusable(root):
-            continue
-        members, inside = {root.data.id: root}, {}
+    def candidate(a, root):
+        return (isinstance(a, Tensor) and isinstance(a.data, Expr) and a.data.op not in ("constant", "tensor", "fused")
+                and a.data.scope == 0 and a.shape == root.shape and _fusable(a))
+
+    def cheap_to_recompute(a, root):
+        """A value read by several consumers may be computed again inside each group that reads it,
+        when that is cheaper than storing it once and loading it in each: a short subtree whose own
+        full-size inputs are no wider than the value."""
+        nodes, leaf_bytes, stack, visited = 0, 0, [a], set()
+        while stack:
+            t = stack.pop()
+            if t.data.id in visited:
+                continue
+            visited.add(t.data.id)
+            nodes += 1
+            for b in t.data.args:
+                if not isinstance(b, Tensor) or _const(b) is not None:
+                    continue
+                if candidate(b, root):
+                    stack.append(b)
+                elif b.data.id not in visited:
+                    visited.add(b.data.id)
+                    leaf_bytes += T.size_bytes(b.type) if b.shape == root.shape else 0
+        return nodes <= 6 and leaf_bytes <= T.size_bytes(a.type)
+
+    def grow(root, recompute):
+        """Members of the group under `root`.  A value all of whose readers are members that belong
+        to this group alone moves in for good; any other value may be computed again inside the
+        group (`shared`), and so may everything only reachable through it."""
+        members, shared, own_reads = {root.data.id: root}, set(), {}
         changed = True
         while changed:
             changed = False
-            inside.clear()
+            own_reads.clear()  # reads by members that are this group's alone
             for m in members.values():
+                if m.data.id in shared:
+                    continue
                 for a in m.data.args:
                     if isinstance(a, Tensor) and isinstance(a.data, Expr) and a.data.op != "constant":
-                        inside[a.data.id] = inside.get(a.data.id, 0) + 1
+                        own_reads[a.data.id] = own_reads.get(a.data.id, 0) + 1
             for m in list(members.values()):
                 for a in m.data.args:
-                    if (isinstance(a, Tensor) and isinstance(a.data, Expr) and a.data.id not in members
-                            and a.data.id not in taken and a.data.op not in ("constant", "tensor") and a.data.scope == 0
-                            and a.shape == root.shape and _fusable(a) and inside[a.data.id] == uses.get(a.data.id)):
+                    if not candidate(a, root) or a.data.id in members or a.data.id in taken:
+                        continue
+                    if own_reads.get(a.data.id, 0) == uses.get(a.data.id):
                         members[a.data.id] = a
                         changed = True
-        if len(members) < 2:
-            continue
+                    elif recompute and cheap_to_recompute(a, root):
+                        members[a.data.id] = a
+                        shared.add(a.data.id)
+                        changed = True
+        return members, shared, dict(own_reads)
+
+    def build(root, members):
         ordered = [t for t in order if t.data.id in members]
         inputs, input_seen = [], set()
         for m in ordered:
@@ -722,13 +754,42 @@ def _fuse(roots: List[Tensor]) -> int:
                         and a.data.id not in input_seen):
                     input_seen.add(a.data.id)
                     inputs.append(a)
-        # the members keep their own nodes for the node-by-node path; the root becomes the group
-        inner_root = root.with_(data=Expr(next(_ids), root.data.op, root.data.args, 0))
-        ordered[-1] = inner_root
-        group = _Group(inner_root, ordered, inputs)
-        taken.update(members)
+        # members are copies (same ids): the originals may become groups of their own later
+        ordered = [t.with_(data=Expr(t.data.id, t.data.op, t.data.args, 0)) for t in ordered]
+        ordered[-1] = root.with_(data=Expr(next(_ids), root.data.op, root.data.args, 0))
+        return _Group(ordered[-1], ordered, inputs), inputs
+
+    taken, formed = set(), 0
+    for root in reversed(order):  # consumers first: a group grows from its last node upwards
+        if root.data.id in taken or uses.get(root.data.id, 0) == 0 or not _fusable(root):
+            continue
+        members, shared, inside = grow(root, recompute=True)
+        group, inputs = build(root, members) if len(members) >= 2 else (None, None)
+        if group is not None and shared and (group.program is None or group.layout is None):
+            members, shared, inside = grow(root, recompute=False)  # too big with the recomputed parts: without them
+            group, inputs = build(root, members) if len(members) >= 2 else (None, None)
+        if group is None:
+            continue
+        taken.update(i for i in members if i not in shared)
+        for i in shared:  # this group no longer reads the shared values; a value nobody reads is dead
+            uses[i] -= inside.get(i, 0)
+        dead = [i for i in shared if uses[i] == 0]
+        while dead:  # the operands of a dead node lose a reader each
+            gone = dead.pop()
+            node = next(t for t in order if t.data.id == gone)
+            for a in node.data.args:
+                if isinstance(a, Tensor) and isinstance(a.data, Expr) and a.data.id in uses and _const(a) is None:
+                    uses[a.data.id] -= 1
+                    if uses[a.data.id] == 0:
+                        dead.append(a.data.id)
         root.data.op, root.data.args = "fused", [group, inputs]
         formed += 1
+    # recount the readers on the rewritten graph
+    uses.clear()
+    seen.clear()
+    del order[:]
+    for r in roots:
+        walk(r)
     # a reduction over the last axis whose operand is a group nobody else reads joins that group
     for node in order:
         e = node.data

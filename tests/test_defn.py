@@ -247,7 +247,9 @@ def test_fusion_groups_and_their_fallback_on_a_backend_without_the_kernel(on_ora
         fused = defn.compile(fun, *args, fuse=True)
         assert_bits_equal(fused(*args), fun(*args), name)
     assert defn.compile(CHAINS["elementwise_reduce"], *build_args(on_oracle)["elementwise_reduce"], fuse=True).fused_groups == 1
-    assert defn.compile(CHAINS["softmax"], *build_args(on_oracle)["softmax"], fuse=True).fused_groups == 2
+    # softmax: max-reduction group, sum-reduction group, final division -- the scaled scores and the
+    # exponentials are computed again inside each group instead of being stored
+    assert defn.compile(CHAINS["softmax"], *build_args(on_oracle)["softmax"], fuse=True).fused_groups == 3
     assert defn.compile(CHAINS["argmax_take"], *build_args(on_oracle)["argmax_take"], fuse=True).fused_groups == 0
 
 

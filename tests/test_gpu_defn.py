@@ -299,21 +299,54 @@ def test_group_with_its_row_reduction_is_bit_identical(name, shape, hip):
     assert_bits_equal(fused(*args), defn.compile(fun, *args)(*args), f"{name} {shape}")
 
 
-def test_reduction_stays_separate_when_its_operand_is_read_elsewhere(hip):
-    args = build_args(hip)["softmax"]
-    fused = defn.compile(CHAINS["softmax"], *args, fuse=True)
-    assert_bits_equal(fused(*args), defn.compile(CHAINS["softmax"], *args)(*args), "softmax")
+def fused_groups_of(compiled):
+    groups = []
 
-    def seen(t, acc):
+    def seen(t):
         e = t.data
         if e.op == "fused":
-            acc.append(e.args[0])
+            groups.append(e.args[0])
             for i in e.args[1]:
-                seen(i, acc)
+                seen(i)
         elif e.op not in ("parameter", "constant", "tensor"):
             for ch in defn._children(e):
                 if isinstance(ch, defn.Tensor):
-                    seen(ch, acc)
-    groups = []
-    seen(fused.roots[0], groups)
-    assert groups and all(g.reduce is None for g in groups)
+                    seen(ch)
+    for r in compiled.roots:
+        seen(r)
+    return groups
+
+
+def test_softmax_becomes_three_kernels(hip):
+    """The scaled scores feed the max and the subtraction, the exponentials feed the sum and the
+    division: both are cheap to compute again from the bf16 scores, so nothing but the two row
+    statistics and the result is ever stored."""
+    args = build_args(hip)["softmax"]
+    fused = defn.compile(CHAINS["softmax"], *args, fuse=True)
+    assert_bits_equal(fused(*args), defn.compile(CHAINS["softmax"], *args)(*args), "softmax")
+    groups = fused_groups_of(fused)
+    assert sorted(str(g.reduce and g.reduce[0]) for g in {id(g): g for g in groups}.values()) == ["None", "reduce_max", "sum"]
+    calls = []
+    original = hip.fused_elementwise.__func__
+
+    def counting(cls, *a, **k):
+        calls.append(1)
+        return original(cls, *a, **k)
+    hip.fused_elementwise = classmethod(counting)
+    try:
+        fused(*args)
+    finally:
+        hip.fused_elementwise = classmethod(original)
+    assert len(calls) == 3
+
+
+def test_value_with_an_outside_reader_is_still_stored_once(hip):
+    x = rand_float(np.random.default_rng(2), "f32", (32, 64), hip)
+
+    def fun(t):
+        h = Nx.tanh(Nx.multiply(t, 0.5))
+        return Nx.add(h, 1.0), Nx.dot(h, [1], h, [1])   # the dot is not element-wise: h must exist in memory
+    fused = defn.compile(fun, x, fuse=True)
+    plain = defn.compile(fun, x)
+    for got, want in zip(fused(x), plain(x)):
+        assert_bits_equal(got, want, "shared with a dot")
