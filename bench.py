@@ -279,9 +279,6 @@ def main():
         # priced at the bytes of the node-by-node chain, like the unfused entry: above 1.0 means the fused
         # pass beats what the reference's formulation can reach at all
         entry("config1_chain_f32_16384_fused", 32.0 * 16384 * 16384 + 4.0 * 16384, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-        fused1k = defn.compile(chain1, *cases["config1_chain_f32_1024"][1], fuse=True)
-        small = cases["config1_chain_f32_1024"][1]
-        _, ms = timed(lambda: fused1k(*small), steps, warm)
         del big, x, y
         del cases, q, k
         result["suite"] = suite
