@@ -176,18 +176,22 @@ copy_nd_kernel(const T *__restrict__ in, T *__restrict__ out, int64_t n, Copy c)
 // ---- iota / eye -----------------------------------------------------------------------------
 // mode 0: out[i] = (i / inner) % dim (iota along an axis; the flat iota is inner = 1, dim = n)
 // mode 1: out[i] = 1 where (i / inner) % dim == i % inner  (eye: dim = rows, inner = columns)
-template <typename CT>
+// IT is the type the coordinates are counted in: 32-bit when the tensor has fewer than 2^31 elements
+// (so the integer -> float conversion is one instruction and exact-or-nearest-even like the
+// reference's integer written as a float, nx/lib/nx/binary_backend.ex:49-75), 64-bit otherwise.
+template <typename CT, typename IT>
 __global__ void __launch_bounds__(BLOCK)
-iota_kernel(void *__restrict__ out, int odt, int64_t n, int64_t dim, int64_t inner, int mode) {
+iota_kernel(void *__restrict__ out, int odt, int64_t n, int64_t dim_, int64_t inner_, int mode) {
   const int64_t nvec = (n + E - 1) / E;
+  const IT dim = (IT)dim_, inner = (IT)inner_;
   for (int64_t v = (int64_t)blockIdx.x * BLOCK + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * BLOCK) {
     const int64_t i0 = v * E;
     CT x[E];
     // one division per vector, then count along: c = i % inner, r = (i / inner) % dim
-    int64_t q, c;
-    if (n <= 0xFFFFFFFFll) { q = (uint32_t)i0 / (uint32_t)inner; c = (uint32_t)i0 - (uint32_t)q * (uint32_t)inner; }
-    else { q = i0 / inner; c = i0 - q * inner; }
-    int64_t r = q < dim ? q : q % dim;
+    IT q, c;
+    if (sizeof(IT) == 4) { q = (IT)((uint32_t)i0 / (uint32_t)inner); c = (IT)((uint32_t)i0 - (uint32_t)q * (uint32_t)inner); }
+    else { q = (IT)(i0 / inner); c = (IT)(i0 - q * inner); }
+    IT r = q < dim ? q : q % dim;
 #pragma unroll
     for (int e = 0; e < E; e++) {
       x[e] = mode == 0 ? (CT)r : (CT)(r == c ? 1 : 0);
@@ -372,8 +376,18 @@ static int iota_like(hipnx_ctx *ctx, int out_dt, int64_t n, int64_t dim, int64_t
   if (int st = check_buf(ctx, out, (uint64_t)n * dtype_size(out_dt), what)) return st;
   if (n == 0) return HIPNX_OK;
   dim3 grid(grid_for((n + E - 1) / E)), block(BLOCK);
-  if (is_float(out_dt)) hipLaunchKernelGGL((iota_kernel<double>), grid, block, 0, ctx->stream, out->ptr, out_dt, n, dim, inner, mode);
-  else hipLaunchKernelGGL((iota_kernel<int64_t>), grid, block, 0, ctx->stream, out->ptr, out_dt, n, dim, inner, mode);
+  // an extent beyond the element count never wraps: clamp it so that it fits the counter type
+  if (dim > n) dim = n;
+  if (inner > n) inner = n;
+  const bool small = n < (1ll << 31);
+  if (small && is_float(out_dt) && out_dt != HIPNX_F64)
+    hipLaunchKernelGGL((iota_kernel<float, int32_t>), grid, block, 0, ctx->stream, out->ptr, out_dt, n, dim, inner, mode);
+  else if (is_float(out_dt))
+    hipLaunchKernelGGL((iota_kernel<double, int64_t>), grid, block, 0, ctx->stream, out->ptr, out_dt, n, dim, inner, mode);
+  else if (small)
+    hipLaunchKernelGGL((iota_kernel<int64_t, int32_t>), grid, block, 0, ctx->stream, out->ptr, out_dt, n, dim, inner, mode);
+  else
+    hipLaunchKernelGGL((iota_kernel<int64_t, int64_t>), grid, block, 0, ctx->stream, out->ptr, out_dt, n, dim, inner, mode);
   HIPNX_HIP(hipGetLastError());
   return HIPNX_OK;
 }
