@@ -230,6 +230,13 @@ int hipnx_iota(hipnx_ctx *ctx, int out_dt, int64_t n, int64_t dim, int64_t inner
  * stacked rows x cols identity matrices */
 int hipnx_eye(hipnx_ctx *ctx, int out_dt, int64_t n, int64_t rows, int64_t cols, hipnx_buf *out);
 
+/* replaces: the write of an integer result at a sub-byte width, `<<x::size(bits)>>` keeping the low
+ * bits (nx/lib/nx/shared.ex:190-194), for tensors of u2 / u4 / s2 / s4 held one element per byte as
+ * the reference's device backends hold them (exla/lib/exla/device_buffer.ex:24-34,
+ * torchx/lib/torchx/backend.ex:428-434): every byte of buf keeps its low `bits` bits (2 or 4), zero- or
+ * sign-extended to the byte.  In place: meant for the fresh output of a callback that computed at 8 bits */
+int hipnx_narrow_int(hipnx_ctx *ctx, hipnx_buf *buf, int64_t n, int bits, int is_signed);
+
 /* replaces: the callback composition behind threefry2x32/2 of Nx.Random (nx/lib/nx/random.ex:214-285;
  * about 110 element-wise callbacks per call) with one kernel producing the same words: out[n] u32 is
  * the Threefry-2x32-20 stream of key (u32[2]) over the counters 0 .. n-1, in the reference's

@@ -22,9 +22,11 @@ import numpy as np
 from . import _lib as L
 from . import shape as S
 from . import types as T
-from .tensor import Tensor, number_to_binary
+from .tensor import Tensor, number_to_binary, pack_sub_byte, unpack_sub_byte, wrap_to_type
 
 from .backend_names import BINARY_OPS, UNARY_OPS  # noqa: E402
+
+_BIT_COUNTS = (UNARY_OPS.index("count_leading_zeros"), UNARY_OPS.index("population_count"))
 
 RED_SUM, RED_MAX, RED_MIN, RED_PRODUCT, RED_ALL, RED_ANY = 0, 1, 2, 3, 4, 5
 K_INNER, K_OUTER = 0, 1
@@ -112,6 +114,15 @@ class HipNxBackend:
         return out.with_(data=cls(_Ref(cls._ctx(device), nbytes), device))
 
     @classmethod
+    def _narrow(cls, res: Tensor) -> Tensor:
+        """A sub-byte result was computed at 8 bits: keep its low bits, as the reference's write of
+        `<<x::size(bits)>>` does (shared.ex:190-194).  In place, on the callback's own fresh output."""
+        kind, bits = res.type
+        if bits < 8:
+            L.check(L.lib.hipnx_narrow_int(res.data.ref.ctx, res.data.ref.handle, res.size, bits, int(kind == "s")))
+        return res
+
+    @classmethod
     def _handle(cls, t: Tensor):
         d = t.data
         if d.released:
@@ -140,6 +151,10 @@ class HipNxBackend:
         (torchx/c_src/torchx.cpp:119-123)."""
         opts = cls.init(opts)
         binary = bytes(binary) if not isinstance(binary, (bytes, bytearray, memoryview)) else binary
+        if T.is_sub_byte(out.type):
+            # packed in the binary, one element per byte on the device, as the reference's device
+            # backends unpack them on entry (exla/lib/exla/device_buffer.ex:24-34)
+            binary = unpack_sub_byte(binary, out.type, out.size).tobytes()
         need = out.size * T.size_bytes(out.type)
         if len(binary) < need:
             raise ValueError("binary size is too small for the requested shape")
@@ -168,6 +183,8 @@ class HipNxBackend:
         n = min(int(limit), t.size) * T.size_bytes(t.type)
         buf = C.create_string_buffer(max(n, 1))
         L.check(L.lib.hipnx_d2h(t.data.ref.ctx, cls._handle(t), 0, buf, n))
+        if T.is_sub_byte(t.type):  # packed again on the way out (exla/lib/exla/device_buffer.ex:65-75)
+            return pack_sub_byte(np.frombuffer(buf.raw[:n], dtype=np.uint8), t.type)
         return buf.raw[:n]
 
     @classmethod
@@ -185,7 +202,11 @@ class HipNxBackend:
         immutable, and the cache holds its own share of the buffer, so deallocating one user
         never frees it."""
         opts = cls.init(opts)
-        elem = number_to_binary(number, out.type)
+        if T.is_sub_byte(out.type):
+            number_to_binary(number, out.type)  # the reference's argument checks
+            elem = wrap_to_type(np.array([int(number)]), out.type).tobytes()
+        else:
+            elem = number_to_binary(number, out.type)
         if out.shape == ():
             key = (opts["device"], out.type, elem)
             ref = cls._scalar_cache.get(key)
@@ -244,9 +265,9 @@ class HipNxBackend:
     def inspect(cls, t: Tensor, limit: int = 50) -> str:
         """inspect/2 (backend.ex:56): reads limit+1 elements like torchx backend.ex:2013-2035."""
         from .tensor import to_float64, binary_to_numpy
-        binary = cls.to_binary(t, min(t.size, limit + 1))
-        n = len(binary) // T.size_bytes(t.type)
-        vals = to_float64(binary, t.type) if T.is_float(t.type) else binary_to_numpy(binary, t.type)
+        n = min(t.size, limit + 1)
+        binary = cls.to_binary(t, n)
+        vals = to_float64(binary, t.type) if T.is_float(t.type) else binary_to_numpy(binary, t.type, (n,))
         body = ", ".join(str(v) for v in vals[:limit]) + (", ..." if n > limit else "")
         dims = "".join(f"[{d}]" for d in t.shape)
         return f"#Nx.Tensor<\n  {T.name(t.type)}{dims}\n  HipNx.Backend({t.data.device})\n  [{body}]\n>"
@@ -268,7 +289,14 @@ class HipNxBackend:
 
     @classmethod
     def bitcast(cls, out, t):
-        return cls._alias(out, cls._from_nx(t, 0))
+        t = cls._from_nx(t, 0)
+        if T.is_sub_byte(out.type) and t.type != out.type:
+            # same bits, the other signedness: the byte an element lives in is extended differently
+            res = cls._alloc(out, t.data.device)
+            L.check(L.lib.hipnx_as_type(res.data.ref.ctx, T.code(t.type), T.code(out.type), out.size, cls._handle(t),
+                                        res.data.ref.handle))
+            return cls._narrow(res)
+        return cls._alias(out, t)
 
     # ---- element-wise ----------------------------------------------------------------------
     @classmethod
@@ -281,16 +309,21 @@ class HipNxBackend:
             res.data.ref.ctx, op, T.code(l.type), T.code(r.type), T.code(out.type), rank, L.i64_array(out.shape),
             L.i64_array(S.broadcast_strides(l.shape, out.shape)), L.i64_array(S.broadcast_strides(r.shape, out.shape)),
             cls._handle(l), cls._handle(r), res.data.ref.handle))
-        return res
+        return cls._narrow(res) if out.type[1] < 8 else res
 
     @classmethod
     def _unary(cls, op: int, out: Tensor, t: Tensor) -> Tensor:
         dev = cls._device_of(t)
         t = cls._from_nx(t, dev)
+        if t.type[1] < 8 and op in _BIT_COUNTS:
+            if UNARY_OPS[op] == "count_leading_zeros":  # no clause in the reference either (binary_backend.ex:962-966)
+                raise NotImplementedError("count_leading_zeros of a sub-byte integer")
+            # population_count reads the element as an unsigned segment of its width (binary_backend.ex:844-850)
+            t = cls.bitcast(t.with_(type=("u", t.type[1])), t)
         res = cls._alloc(out, dev)
         L.check(L.lib.hipnx_unary(res.data.ref.ctx, op, T.code(t.type), T.code(out.type), out.size, cls._handle(t),
                                   res.data.ref.handle))
-        return res
+        return cls._narrow(res) if out.type[1] < 8 else res
 
     @classmethod
     def as_type(cls, out: Tensor, t: Tensor) -> Tensor:
@@ -302,6 +335,18 @@ class HipNxBackend:
         res = cls._alloc(out, dev)
         L.check(L.lib.hipnx_as_type(res.data.ref.ctx, T.code(t.type), T.code(out.type), out.size, cls._handle(t),
                                     res.data.ref.handle))
+        if out.type[1] < 8:
+            res = cls._narrow(res)
+            if T.is_float(t.type):
+                # an infinity becomes the narrow type's own extreme, not the low bits of the 8-bit one
+                # (binary_backend.ex:2062-2069)
+                kind, bits = out.type
+                lo, hi = (-(1 << (bits - 1)), (1 << (bits - 1)) - 1) if kind == "s" else (0, (1 << bits) - 1)
+                u8 = out.with_(type=("u", 8))
+                zero = cls.constant(t.with_(shape=()), 0.0, {"device": dev})
+                extreme = cls.select(out, cls.greater(u8, t, zero), cls.constant(out.with_(shape=()), hi, {"device": dev}),
+                                     cls.constant(out.with_(shape=()), lo, {"device": dev}))
+                res = cls.select(out, cls.is_infinity(u8, t), extreme, res)
         return res
 
     # ---- reductions ------------------------------------------------------------------------
@@ -413,7 +458,7 @@ class HipNxBackend:
         res = cls._alloc(out, dev)
         L.check(L.lib.hipnx_dot(res.data.ref.ctx, T.code(l.type), T.code(r.type), T.code(out.type), batch, M, N, K,
                                 l_layout, r_layout, cls._handle(lt), cls._handle(rt), res.data.ref.handle))
-        return res
+        return cls._narrow(res) if out.type[1] < 8 else res
 
     # ---- data movement ---------------------------------------------------------------------
     @classmethod
@@ -474,7 +519,7 @@ class HipNxBackend:
         else:
             dim, inner = out.shape[axis], prod(out.shape[axis + 1:])
         L.check(L.lib.hipnx_iota(res.data.ref.ctx, T.code(out.type), out.size, dim, inner, res.data.ref.handle))
-        return res
+        return cls._narrow(res) if out.type[1] < 8 else res
 
     @classmethod
     def eye(cls, out: Tensor, opts=None) -> Tensor:

@@ -203,9 +203,41 @@ iota_kernel(void *__restrict__ out, int odt, int64_t n, int64_t dim_, int64_t in
   }
 }
 
+// ---- sub-byte integers held one per byte: keep the low bits of each byte ------------------------
+__global__ void __launch_bounds__(BLOCK)
+narrow_int_kernel(unsigned char *__restrict__ p, int64_t n, int bits, int is_signed) {
+  const int sh = 8 - bits;
+  const int64_t nvec = n / 16;
+  for (int64_t v = (int64_t)blockIdx.x * BLOCK + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * BLOCK) {
+    raw_vec<16> r = *reinterpret_cast<raw_vec<16> *>(p + v * 16);
+#pragma unroll
+    for (int i = 0; i < 16; i++)
+      r.b[i] = is_signed ? (unsigned char)((signed char)(r.b[i] << sh) >> sh) : (unsigned char)(r.b[i] & (0xFF >> sh));
+    *reinterpret_cast<raw_vec<16> *>(p + v * 16) = r;
+  }
+  if (blockIdx.x == 0 && threadIdx.x < n - nvec * 16) {
+    const int64_t i = nvec * 16 + threadIdx.x;
+    p[i] = is_signed ? (unsigned char)((signed char)(p[i] << sh) >> sh) : (unsigned char)(p[i] & (0xFF >> sh));
+  }
+}
+
 }  // namespace hipnx
 
 using namespace hipnx;
+
+extern "C" int hipnx_narrow_int(hipnx_ctx *ctx, hipnx_buf *buf, int64_t n, int bits, int is_signed) {
+  Enter in(ctx);
+  if (in.status) return in.status;
+  if (bits != 2 && bits != 4) return set_error(HIPNX_EINVAL, "narrow_int: %d bits (2 or 4)", bits);
+  if (n < 0) return set_error(HIPNX_EINVAL, "narrow_int: negative size");
+  if (int st = check_buf(ctx, buf, (uint64_t)n, "narrow_int")) return st;
+  if (n == 0) return HIPNX_OK;
+  if ((uintptr_t)buf->ptr % 16) return set_error(HIPNX_EINVAL, "narrow_int: buffer not 16-byte aligned");
+  hipLaunchKernelGGL(narrow_int_kernel, dim3(grid_for(n / 16 + 1)), dim3(BLOCK), 0, ctx->stream,
+                     (unsigned char *)buf->ptr, n, bits, is_signed);
+  HIPNX_HIP(hipGetLastError());
+  return HIPNX_OK;
+}
 
 extern "C" int hipnx_select(hipnx_ctx *ctx, int pred_dt, int true_dt, int false_dt, int out_dt, int rank,
                             const int64_t *out_dims, const int64_t *pred_strides, const int64_t *true_strides,

@@ -354,6 +354,14 @@ static ERL_NIF_TERM nif_threefry2x32(ErlNifEnv *env, int argc, const ERL_NIF_TER
   return ok(env, make_buf(env, out));
 }
 
+/* narrow_int(ctx, buf, n, bits, signed): in place on a callback's fresh output; returns the same buffer */
+static ERL_NIF_TERM nif_narrow_int(ErlNifEnv *env, int argc, const ERL_NIF_TERM argv[]) {
+  (void)argc;
+  GET_CTX(0, ctx); GET_BUF(1, buf); GET_I64(2, n); GET_INT(3, bits); GET_INT(4, is_signed);
+  CHECK(hipnx_narrow_int(ctx, buf, n, bits, is_signed));
+  return ok(env, argv[1]);
+}
+
 static ERL_NIF_TERM nif_sync(ErlNifEnv *env, int argc, const ERL_NIF_TERM argv[]) {
   (void)argc;
   GET_CTX(0, ctx);
@@ -380,6 +388,7 @@ static ErlNifFunc funcs[] = {
     {"broadcast", 6, nif_broadcast, IO},        {"gather", 10, nif_gather, IO},
     {"select", 13, nif_select, IO},             {"clip", 10, nif_clip, IO},
     {"strided_copy", 9, nif_strided_copy, IO},  {"iota", 6, nif_iota, IO},
+    {"narrow_int", 5, nif_narrow_int, IO},
     {"eye", 6, nif_eye, IO},                    {"threefry2x32", 4, nif_threefry2x32, IO},
     {"sync", 1, nif_sync, IO}};
 

@@ -33,7 +33,9 @@ defmodule HipNx.Backend do
                 atanh sqrt rsqrt cbrt erf erfc erf_inv abs bitwise_not ceil floor negate round sign
                 count_leading_zeros population_count is_nan is_infinity)a
   @dtypes %{{:u, 8} => 0, {:u, 16} => 1, {:u, 32} => 2, {:u, 64} => 3, {:s, 8} => 4, {:s, 16} => 5,
-            {:s, 32} => 6, {:s, 64} => 7, {:f, 16} => 8, {:bf, 16} => 9, {:f, 32} => 10, {:f, 64} => 11}
+            {:s, 32} => 6, {:s, 64} => 7, {:f, 16} => 8, {:bf, 16} => 9, {:f, 32} => 10, {:f, 64} => 11,
+            # sub-byte integers live one per byte on the device, as in EXLA.DeviceBuffer: kernels see s8 / u8
+            {:u, 2} => 0, {:u, 4} => 0, {:s, 2} => 4, {:s, 4} => 4}
 
   ## Options and context
 
@@ -59,7 +61,14 @@ defmodule HipNx.Backend do
   defp unwrap!({:error, {_status, msg}}), do: raise(RuntimeError, "HipNx: " <> List.to_string(msg))
 
   defp dt(type), do: Map.get(@dtypes, type) || raise(ArgumentError, "HipNx does not support type #{inspect(type)}")
-  defp bytes(%T{type: {_, bits}, shape: shape}), do: div(bits, 8) * Nx.size(shape)
+  defp bytes(%T{type: {_, bits}, shape: shape}), do: max(div(bits, 8), 1) * Nx.size(shape)
+
+  # a result of a sub-byte type was computed at 8 bits: keep its low bits (Nx.Shared's `<<x::size(bits)>>`)
+  defp to_nx(ref, device, %T{type: {kind, bits}} = out) when bits < 8 do
+    ref = unwrap!(NIF.narrow_int(ctx(device), ref, Nx.size(out), bits, if(kind == :s, do: 1, else: 0)))
+    %{out | data: %__MODULE__{ref: ref, device: device}}
+  end
+
   defp to_nx(ref, device, %T{} = out), do: %{out | data: %__MODULE__{ref: ref, device: device}}
 
   # operands living on another backend are copied in on entry (cf. Torchx.Backend.from_nx/1)
@@ -82,21 +91,37 @@ defmodule HipNx.Backend do
   @impl true
   def from_binary(%T{} = out, binary, opts) do
     device = init(opts)[:device]
-    to_nx(unwrap!(NIF.from_binary(ctx(device), IO.iodata_to_binary(binary), bytes(out))), device, out)
+    to_nx(unwrap!(NIF.from_binary(ctx(device), unpack(binary, out.type), bytes(out))), device, out)
   end
+
+  # packed bitstring <-> one element per byte (cf. EXLA.DeviceBuffer.place_on_device/4 and read/2)
+  defp unpack(data, {:u, size}) when size in [2, 4],
+    do: for(<<x::native-size(size) <- data>>, into: <<>>, do: <<x::native-8>>)
+
+  defp unpack(data, {:s, size}) when size in [2, 4],
+    do: for(<<x::native-signed-size(size) <- data>>, into: <<>>, do: <<x::native-signed-8>>)
+
+  defp unpack(data, _type), do: IO.iodata_to_binary(data)
+
+  defp pack(data, {:u, size}) when size in [2, 4],
+    do: for(<<x::native-8 <- data>>, into: <<>>, do: <<x::native-size(size)>>)
+
+  defp pack(data, {:s, size}) when size in [2, 4],
+    do: for(<<x::native-signed-8 <- data>>, into: <<>>, do: <<x::native-signed-size(size)>>)
+
+  defp pack(data, _type), do: data
 
   @impl true
   def to_binary(%T{data: %__MODULE__{ref: ref, device: device}, type: {_, bits}} = t, limit) do
     n = min(limit, Nx.size(t))
-    unwrap!(NIF.to_binary(ctx(device), ref, n * div(bits, 8)))
+    pack(unwrap!(NIF.to_binary(ctx(device), ref, n * max(div(bits, 8), 1))), t.type)
   end
 
   @impl true
   def constant(%T{type: type} = out, number, opts) do
     device = init(opts)[:device]
     %T{data: %Nx.BinaryBackend{state: elem}} = Nx.BinaryBackend.constant(%{out | shape: {}, names: []}, number, [])
-    _ = type
-    to_nx(unwrap!(NIF.fill(ctx(device), elem, Nx.size(out))), device, out)
+    to_nx(unwrap!(NIF.fill(ctx(device), unpack(elem, type), Nx.size(out))), device, out)
   end
 
   @impl true

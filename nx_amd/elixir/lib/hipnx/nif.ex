@@ -29,6 +29,7 @@ defmodule HipNx.NIF do
   def strided_copy(_ctx, _elem_bytes, _dims, _in_strides, _in_offset, _out_strides, _out_offset, _in, _out_or_bytes), do: err()
   def iota(_ctx, _out_dt, _n, _dim, _inner, _out_bytes), do: err()
   def eye(_ctx, _out_dt, _n, _rows, _cols, _out_bytes), do: err()
+  def narrow_int(_ctx, _buf, _n, _bits, _signed), do: err()
   def threefry2x32(_ctx, _key, _n, _out_bytes), do: err()
   def sync(_ctx), do: err()
 

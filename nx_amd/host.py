@@ -10,7 +10,7 @@ the device backend wins the dispatch and copies it in (nx/lib/nx/shared.ex:449-4
 from __future__ import annotations
 
 from . import types as T
-from .tensor import Tensor, number_to_binary
+from .tensor import Tensor, binary_prefix, binary_size, list_to_binary, number_to_binary
 
 
 class HostBinary:
@@ -26,20 +26,21 @@ class HostBinary:
 
     @classmethod
     def from_binary(cls, out: Tensor, binary, opts=None) -> Tensor:
-        need = out.size * T.size_bytes(out.type)
-        if len(binary) < need:
+        if len(binary) < binary_size(out.type, out.size):
             raise ValueError("binary size is too small for the requested shape")
-        return out.with_(data=cls(bytes(binary[:need])))
+        return out.with_(data=cls(binary_prefix(binary, out.type, out.size)))
 
     @classmethod
     def constant(cls, out: Tensor, number, opts=None) -> Tensor:
+        if T.is_sub_byte(out.type):
+            return out.with_(data=cls(list_to_binary([int(number)] * out.size, out.type)))
         return out.with_(data=cls(number_to_binary(number, out.type) * out.size))
 
     @classmethod
     def to_binary(cls, t: Tensor, limit: int) -> bytes:
         if t.data.released:
             raise RuntimeError("tensor has been deallocated")
-        return t.data.state[: min(int(limit), t.size) * T.size_bytes(t.type)]
+        return binary_prefix(t.data.state, t.type, min(int(limit), t.size))
 
     @classmethod
     def backend_copy(cls, t: Tensor, backend, opts=None) -> Tensor:

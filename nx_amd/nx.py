@@ -80,14 +80,42 @@ def tensor(value, type=None, backend=None) -> Tensor:
     return mod.from_binary(template(ty, arr.shape), binary, opts)
 
 
-def from_binary(binary, type, backend=None) -> Tensor:
-    """Nx.from_binary/3 (nx.ex:2051-2066): a flat tensor over the bytes."""
+def from_binary(binary, type, backend=None, count=None) -> Tensor:
+    """Nx.from_binary/3 (nx.ex:2051-2066): a flat tensor over the bytes.  A packed sub-byte binary
+    whose last byte is only partly used needs `count` elements said (the reference reads it off
+    the bitstring's bit size)."""
     ty = T.normalize(type)
-    size = T.size_bytes(ty)
-    if len(binary) == 0 or len(binary) % size:
+    bits = T.bit_size(ty)
+    if len(binary) == 0:
+        raise ValueError("cannot build an empty tensor")
+    if (len(binary) * 8) % bits:
         raise ValueError("binary has incompatible number of bits, expected a multiple of the type size")
+    n = len(binary) * 8 // bits
+    if count is not None:
+        if not T.is_sub_byte(ty) or not n - 8 // bits < count <= n:
+            raise ValueError("count does not fit the binary")
+        n = count
     mod, opts = (backend, {}) if backend is not None and not isinstance(backend, tuple) else (backend or default_backend())
-    return mod.from_binary(template(ty, (len(binary) // size,)), binary, opts)
+    return mod.from_binary(template(ty, (n,)), binary, opts)
+
+
+def _def_typed_constructors():
+    # Nx.u2/1 .. Nx.f64/1 (nx.ex:974-984): aliases for Nx.tensor(value, type: t)
+    for name in ("u2", "u4", "u8", "u16", "u32", "u64", "s2", "s4", "s8", "s16", "s32", "s64", "bf16", "f16", "f32", "f64"):
+        globals()[name] = (lambda value, _t=name: tensor(value, type=_t))
+
+
+_def_typed_constructors()
+
+
+def bit_size(t: Tensor) -> int:
+    """Nx.bit_size/1 (nx.ex:4890-4915)."""
+    return t.size * T.bit_size(t.type)
+
+
+def byte_size(t: Tensor) -> int:
+    """Nx.byte_size/1 (nx.ex:4860-4888): whole bytes of the binary."""
+    return bit_size(t) // 8
 
 
 def to_tensor(value) -> Tensor:

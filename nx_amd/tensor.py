@@ -67,6 +67,69 @@ def template(type, shape) -> Tensor:
 _NAN = {16: 0x7E00, 32: 0x7FC00000, 64: 0x7FF8000000000000}
 
 
+# ---- sub-byte integers: packed in a binary, one byte per element in memory ------------------
+# The reference's binary is a bitstring with the first element in the highest bits
+# (`<<x::size(4)>>` segments, nx/lib/nx/shared.ex:190-194).  Python has no bitstrings: a packed
+# binary whose bit count is not a multiple of eight carries zero bits at the end of its last byte,
+# and the element count comes from the tensor's shape.
+
+def pack_sub_byte(values, type) -> bytes:
+    """One-per-byte elements (any integer array; only the low bits count) -> packed binary."""
+    bits = T.bit_size(type)
+    v = np.asarray(values).astype(np.int64).ravel() & ((1 << bits) - 1)
+    per = 8 // bits
+    pad = (-v.size) % per
+    if pad:
+        v = np.concatenate([v, np.zeros(pad, dtype=np.int64)])
+    v = v.reshape(-1, per)
+    out = np.zeros(v.shape[0], dtype=np.int64)
+    for k in range(per):
+        out |= v[:, k] << (8 - bits * (k + 1))
+    return out.astype(np.uint8).tobytes()
+
+
+def unpack_sub_byte(binary, type, count=None) -> np.ndarray:
+    """Packed binary -> one element per byte (int8 sign-extended, or uint8), `count` of them."""
+    kind, bits = T.normalize(type)
+    per = 8 // bits
+    raw = np.frombuffer(binary, dtype=np.uint8).astype(np.int64)
+    cols = [(raw >> (8 - bits * (k + 1))) & ((1 << bits) - 1) for k in range(per)]
+    v = np.stack(cols, axis=1).ravel()
+    if count is not None:
+        if count > v.size:
+            raise ValueError("binary size is too small for the requested shape")
+        v = v[:count]
+    if kind == "s":
+        v = np.where(v >= (1 << (bits - 1)), v - (1 << bits), v)
+        return v.astype(np.int8)
+    return v.astype(np.uint8)
+
+
+def binary_size(type, count: int) -> int:
+    """Bytes of the binary of `count` elements (a partly used last byte counts)."""
+    return (count * T.bit_size(type) + 7) // 8
+
+
+def binary_prefix(binary, type, count: int) -> bytes:
+    """The binary of the first `count` elements of a binary."""
+    if not T.is_sub_byte(type):
+        return bytes(binary[: count * T.size_bytes(type)])
+    if (count * T.bit_size(type)) % 8 == 0:
+        return bytes(binary[: binary_size(type, count)])
+    return pack_sub_byte(unpack_sub_byte(binary[: binary_size(type, count)], type, count), type)
+
+
+def wrap_to_type(values: np.ndarray, type) -> np.ndarray:
+    """Low bits of integers as elements of `type`, one per storage element (sub-byte included)."""
+    kind, bits = T.normalize(type)
+    if not T.is_sub_byte(type):
+        return values.astype(T.numpy_dtype(type))
+    v = values.astype(np.int64) & ((1 << bits) - 1)
+    if kind == "s":
+        v = np.where(v >= (1 << (bits - 1)), v - (1 << bits), v)
+    return v.astype(T.numpy_dtype(type))
+
+
 def number_to_binary(number, type) -> bytes:
     kind, bits = T.normalize(type)
     if kind in ("u", "s"):
@@ -76,6 +139,8 @@ def number_to_binary(number, type) -> bytes:
             if number != int(number):
                 raise ValueError(f"cannot encode the float {number!r} as an integer type")
             number = int(number)
+        if bits < 8:  # a one-element bitstring, zero bits after it
+            return bytes([((int(number) & ((1 << bits) - 1)) << (8 - bits))])
         return (int(number) & ((1 << bits) - 1)).to_bytes(bits // 8, "little")
     x = float(number)
     if kind == "bf":
@@ -104,6 +169,8 @@ def list_to_binary(values, type) -> bytes:
     if kind in ("u", "s"):
         if arr.dtype.kind == "f":
             raise ValueError("cannot build an integer tensor from floats")
+        if bits < 8:
+            return pack_sub_byte(arr.astype(np.int64), type)
         if arr.dtype == object:
             return b"".join(number_to_binary(v, type) for v in arr.ravel())
         return arr.astype(np.int64).astype(T.numpy_dtype(type)).tobytes()
@@ -121,7 +188,11 @@ def list_to_binary(values, type) -> bytes:
 
 
 def binary_to_numpy(binary: bytes, type, shape=None) -> np.ndarray:
-    """Raw view of a tensor binary; bf16 comes back as uint16 bit patterns."""
+    """Raw view of a tensor binary; bf16 comes back as uint16 bit patterns, sub-byte integers
+    unpacked to one per byte (as many as the shape holds, or as the binary's bytes hold)."""
+    if T.is_sub_byte(type):
+        arr = unpack_sub_byte(binary, type, math.prod(shape) if shape is not None else None)
+        return arr.reshape(shape) if shape is not None else arr
     arr = np.frombuffer(binary, dtype=T.numpy_dtype(type))
     return arr.reshape(shape) if shape is not None else arr
 

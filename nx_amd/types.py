@@ -1,8 +1,14 @@
 """Element types and the type-inference rules of Nx (reference: nx/lib/nx/type.ex).
 
 A type is a tuple ``(kind, bits)`` with kind in {"u", "s", "f", "bf"} -- the Python spelling of
-the reference's ``{:u, 8}`` .. ``{:f, 64}`` / ``{:bf, 16}`` (type.ex:27-48).  Complex, f8 and
-sub-byte integer types are outside the device path and are rejected by ``normalize``.
+the reference's ``{:u, 8}`` .. ``{:f, 64}`` / ``{:bf, 16}`` (type.ex:27-48).  Complex and f8 types
+are outside the device path and are rejected by ``normalize``.
+
+The sub-byte integers u2, u4, s2, s4 are packed only in a tensor's binary (the reference's
+bitstring: first element in the highest bits).  In memory -- on the device and in the host
+backends -- each element has a byte of its own, sign- or zero-extended, as the reference's device
+backends keep them (exla/lib/exla/device_buffer.ex:24-34, torchx/lib/torchx/backend.ex:428-434);
+kernels see them as s8 / u8 and the backend wraps results back to the narrow width.
 """
 from __future__ import annotations
 
@@ -21,6 +27,8 @@ _NAMES = {
     "s8": ("s", 8), "s16": ("s", 16), "s32": ("s", 32), "s64": ("s", 64),
     "f16": ("f", 16), "bf16": ("bf", 16), "f32": ("f", 32), "f64": ("f", 64),
 }
+_SUB_BYTE = {("u", 2): U8, ("u", 4): U8, ("s", 2): S8, ("s", 4): S8}  # type -> the code kernels see
+_NAMES.update({"u2": ("u", 2), "u4": ("u", 4), "s2": ("s", 2), "s4": ("s", 4)})
 # bf16 has no numpy dtype: it travels as raw uint16 bit patterns
 _NUMPY = {
     ("u", 8): np.uint8, ("u", 16): np.uint16, ("u", 32): np.uint32, ("u", 64): np.uint64,
@@ -38,13 +46,25 @@ def normalize(t):
             raise ValueError(f"invalid numerical type: {t!r}")
         return _NAMES[t]
     t = (t[0], int(t[1]))
-    if t not in _CODES:
+    if t not in _CODES and t not in _SUB_BYTE:
         raise ValueError(f"invalid numerical type: {t!r}")
     return t
 
 
+def is_sub_byte(t) -> bool:
+    return t in _SUB_BYTE or (t.__class__ is not tuple and normalize(t) in _SUB_BYTE)
+
+
 def code(t) -> int:
-    return _CODES[normalize(t)]
+    """The element type a kernel is told: sub-byte integers are held one per byte."""
+    t = normalize(t)
+    return _CODES[t] if t in _CODES else _SUB_BYTE[t]
+
+
+def storage(t):
+    """The type of a tensor's elements in memory: itself, or s8 / u8 for a sub-byte integer."""
+    t = normalize(t)
+    return (t[0], 8) if t in _SUB_BYTE else t
 
 
 def from_code(c: int):
@@ -60,11 +80,17 @@ def name(t) -> str:
 
 
 def size_bytes(t) -> int:
-    return normalize(t)[1] // 8
+    """Bytes per element in memory (one for a sub-byte integer; its binary is packed, see bit_size)."""
+    return max(normalize(t)[1] // 8, 1)
+
+
+def bit_size(t) -> int:
+    """Bits per element of a tensor's binary (Nx.Type's size; nx.ex:4890-4915 for Nx.bit_size/1)."""
+    return normalize(t)[1]
 
 
 def numpy_dtype(t):
-    return np.dtype(_NUMPY[normalize(t)])
+    return np.dtype(_NUMPY[storage(t)])
 
 
 def is_float(t) -> bool:
@@ -89,15 +115,14 @@ def merge(left, right):
     return b
 
 
-def _unsigned_size(x: int) -> int:
-    return 8 if x <= 0xFF else 16 if x <= 0xFFFF else 32 if x <= 0xFFFFFFFF else 64
+def _unsigned_size(x: int) -> int:  # type.ex:694-698
+    return 1 if x <= 1 else 8 if x <= 0xFF else 16 if x <= 0xFFFF else 32 if x <= 0xFFFFFFFF else 64
 
 
-def _signed_size(x: int) -> int:
-    for bits in (8, 16, 32):
-        if -(1 << (bits - 1)) <= x < (1 << (bits - 1)):
-            return bits
-    return 64
+def _signed_size(x: int) -> int:  # type.ex:700-705
+    if x < 0:
+        x = -x - 1
+    return 1 if x <= 1 else 8 if x <= 127 else 16 if x <= 32767 else 32 if x <= 2147483647 else 64
 
 
 def merge_number(t, number):

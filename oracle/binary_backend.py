@@ -22,7 +22,7 @@ import numpy as np
 
 from nx_amd import shape as S
 from nx_amd import types as T
-from nx_amd.tensor import Tensor, number_to_binary
+from nx_amd.tensor import Tensor, number_to_binary, pack_sub_byte, unpack_sub_byte
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libhipnx_ref.so")
@@ -123,8 +123,15 @@ class BinaryBackend:
         return buf, out.with_(data=cls(buf))
 
     # -- plumbing (binary_backend.ex:42-46, 114-165)
+    # Sub-byte integers (u2, u4, s2, s4): the reference's state is the packed bitstring and every
+    # callback reads `size`-bit segments and writes the low `size` bits (binary_backend.ex:2415-2438,
+    # shared.ex:190-194).  Here the state holds one element per byte, extended to s8 / u8, the C
+    # functions run on those, and `_narrow` keeps the low bits of what they wrote; from_binary
+    # and to_binary convert from and to the packed form (first element in the highest bits).
     @classmethod
     def from_binary(cls, out, binary, opts=None):
+        if T.is_sub_byte(out.type):
+            return out.with_(data=cls(bytearray(unpack_sub_byte(binary, out.type, out.size).tobytes())))
         need = out.size * T.size_bytes(out.type)
         if len(binary) < need:
             raise ValueError("binary size is too small for the requested shape")
@@ -132,11 +139,29 @@ class BinaryBackend:
 
     @classmethod
     def to_binary(cls, t, limit):
-        return bytes(t.data.state[: min(int(limit), t.size) * T.size_bytes(t.type)])
+        n = min(int(limit), t.size)
+        if T.is_sub_byte(t.type):
+            return pack_sub_byte(np.frombuffer(bytes(t.data.state[:n]), dtype=np.uint8), t.type)
+        return bytes(t.data.state[: n * T.size_bytes(t.type)])
 
     @classmethod
     def constant(cls, out, number, opts=None):
+        if T.is_sub_byte(out.type):
+            one = unpack_sub_byte(number_to_binary(number, out.type), out.type, 1).tobytes()
+            return out.with_(data=cls(bytearray(one * out.size)))
         return out.with_(data=cls(bytearray(number_to_binary(number, out.type) * out.size)))
+
+    @classmethod
+    def _narrow(cls, res):
+        """Keeps the low bits of a sub-byte result that was computed at 8 bits."""
+        if not T.is_sub_byte(res.type):
+            return res
+        kind, bits = res.type
+        v = np.frombuffer(bytes(res.data.state), dtype=np.uint8).astype(np.int64) & ((1 << bits) - 1)
+        if kind == "s":
+            v = np.where(v >= (1 << (bits - 1)), v - (1 << bits), v)
+        res.data.state[:] = v.astype(np.int8 if kind == "s" else np.uint8).tobytes()
+        return res
 
     @classmethod
     def backend_copy(cls, t, backend, opts=None):
@@ -158,6 +183,8 @@ class BinaryBackend:
 
     @classmethod
     def bitcast(cls, out, t):
+        if T.is_sub_byte(out.type):  # same bits, read with the other signedness
+            return cls._narrow(out.with_(data=cls(bytearray(cls._bin(t)))))
         return out.with_(data=cls(cls._bin(t)))
 
     @classmethod
@@ -172,23 +199,42 @@ class BinaryBackend:
         _check(lib.ref_binary(op, T.code(l.type), T.code(r.type), T.code(out.type), len(out.shape), _i64(out.shape),
                               _i64(S.broadcast_strides(l.shape, out.shape)),
                               _i64(S.broadcast_strides(r.shape, out.shape)), cls._ptr(lb), cls._ptr(rb), cls._ptr(buf)))
-        return res
+        return cls._narrow(res)
 
     @classmethod
     def _unary(cls, op, out, t):
         tb = cls._bin(t)
         buf, res = cls._new(out)
+        if T.is_sub_byte(t.type) and UNARY_OPS[op] == "count_leading_zeros":
+            raise NotImplementedError("count_leading_zeros of a sub-byte integer")  # binary_backend.ex:962-966: no clause
+        if T.is_sub_byte(t.type) and UNARY_OPS[op] == "population_count":
+            # binary_backend.ex:844-850 reads each element as an unsigned segment of the type's width
+            bits = np.frombuffer(bytes(tb), dtype=np.uint8) & ((1 << t.type[1]) - 1)
+            counts = np.array([bin(int(b)).count("1") for b in bits], dtype=np.int64).reshape(t.shape)
+            return cls._from_array(out, counts, "s64")
         _check(lib.ref_unary(op, T.code(t.type), T.code(out.type), out.size, cls._ptr(tb), cls._ptr(buf)))
-        return res
+        return cls._narrow(res)
 
     @classmethod
     def as_type(cls, out, t):  # binary_backend.ex:2031-2076
         if t.type == out.type:
             return t
+        if T.is_sub_byte(out.type) and T.is_float(t.type):
+            # binary_backend.ex:2056-2069: NaN -> 0, infinities -> the type's extremes, the rest
+            # truncated and written at the type's width
+            x = cls._numbers(t).ravel()
+            kind, bits = out.type
+            lo, hi = (-(1 << (bits - 1)), (1 << (bits - 1)) - 1) if kind == "s" else (0, (1 << bits) - 1)
+            finite = np.isfinite(x)
+            v = np.zeros(x.shape, dtype=np.int64)
+            v[finite] = np.trunc(x[finite]).astype(np.int64)
+            v[np.isposinf(x)] = hi
+            v[np.isneginf(x)] = lo
+            return cls._narrow(out.with_(data=cls(bytearray(v.astype(np.uint8).tobytes()))))
         tb = cls._bin(t)
         buf, res = cls._new(out)
         _check(lib.ref_as_type(T.code(t.type), T.code(out.type), out.size, cls._ptr(tb), cls._ptr(buf)))
-        return res
+        return cls._narrow(res)
 
     # -- data movement (binary_backend.ex:215-319, 1902-1959)
     @classmethod
@@ -305,7 +351,7 @@ class BinaryBackend:
         buf, res = cls._new(out)
         _check(lib.ref_dot(T.code(l.type), T.code(r.type), T.code(out.type), batch, M, N, K, cls._ptr(lb),
                            cls._ptr(rb), cls._ptr(buf)))
-        return res
+        return cls._narrow(res)
 
 
     # -- one step off the hot path ---------------------------------------------------------------
