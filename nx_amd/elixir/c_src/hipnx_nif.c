@@ -362,6 +362,27 @@ static ERL_NIF_TERM nif_narrow_int(ErlNifEnv *env, int argc, const ERL_NIF_TERM 
   return ok(env, argv[1]);
 }
 
+/* device_ptr(buf) -> {:ok, address}: the :local pointer of to_pointer/2 */
+static ERL_NIF_TERM nif_device_ptr(ErlNifEnv *env, int argc, const ERL_NIF_TERM argv[]) {
+  (void)argc;
+  GET_BUF(0, buf);
+  void *p = hipnx_buf_device_ptr(buf);
+  if (!p) return error_from_status(env, HIPNX_EFREED);
+  return ok(env, enif_make_uint64(env, (ErlNifUInt64)(uintptr_t)p));
+}
+
+/* wrap(ctx, address, nbytes): from_pointer/5 for a :local pointer; the memory stays with its owner */
+static ERL_NIF_TERM nif_wrap(ErlNifEnv *env, int argc, const ERL_NIF_TERM argv[]) {
+  (void)argc;
+  GET_CTX(0, ctx);
+  ErlNifUInt64 address;
+  if (!enif_get_uint64(env, argv[1], &address)) return enif_make_badarg(env);
+  GET_I64(2, nbytes);
+  hipnx_buf *buf;
+  CHECK(hipnx_buf_wrap(ctx, (void *)(uintptr_t)address, (size_t)nbytes, &buf));
+  return ok(env, make_buf(env, buf));
+}
+
 static ERL_NIF_TERM nif_sync(ErlNifEnv *env, int argc, const ERL_NIF_TERM argv[]) {
   (void)argc;
   GET_CTX(0, ctx);
@@ -388,7 +409,8 @@ static ErlNifFunc funcs[] = {
     {"broadcast", 6, nif_broadcast, IO},        {"gather", 10, nif_gather, IO},
     {"select", 13, nif_select, IO},             {"clip", 10, nif_clip, IO},
     {"strided_copy", 9, nif_strided_copy, IO},  {"iota", 6, nif_iota, IO},
-    {"narrow_int", 5, nif_narrow_int, IO},
+    {"narrow_int", 5, nif_narrow_int, IO},      {"device_ptr", 1, nif_device_ptr, 0},
+    {"wrap", 3, nif_wrap, 0},
     {"eye", 6, nif_eye, IO},                    {"threefry2x32", 4, nif_threefry2x32, IO},
     {"sync", 1, nif_sync, IO}};
 

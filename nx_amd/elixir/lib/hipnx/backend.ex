@@ -11,8 +11,9 @@ defmodule HipNx.Backend do
   behaviour runs on `Nx.BinaryBackend` after a device-to-host copy and comes back with
   `from_binary` -- the same escape hatch `EXLA.Backend` uses for `concatenate`/`stack`.
 
-  Results follow `Nx.BinaryBackend` (integers, indices and argmax bit-exact; see the repository's
-  DESIGN.md for the float tolerances and the documented divergences).
+  Results follow `Nx.BinaryBackend`: integers, indices and argmax bit-exact; `+ - * /`, comparisons,
+  `as_type` and selections bit-exact for floats too; libm-class functions within 1 ulp of the output
+  type; `dot` and `sum` over floats within the bound of an f32 accumulation of the same terms.
 
   This module cannot be compiled in the repository's build container (no BEAM); its Python twin
   `nx_amd/backend.py` exercises the same C ABI with the same lowering and is what the test-suite
@@ -614,8 +615,36 @@ defmodule HipNx.Backend do
     end
   end
 
+  ## Pointers (the :local kind; cf. EXLA.Backend.to_pointer/2 and from_pointer/5)
+
   @impl true
-  def from_pointer(_, _, _, _, _), do: raise(ArgumentError, "HipNx.Backend does not support pointers")
+  def to_pointer(%T{data: %__MODULE__{ref: ref}} = t, opts) do
+    opts = Keyword.validate!(opts, mode: :local)
+
+    case opts[:mode] do
+      :local -> %Nx.Pointer{kind: :local, address: unwrap!(NIF.device_ptr(ref)), data_size: bytes(t)}
+      :ipc -> raise ArgumentError, "HipNx.Backend.to_pointer/2: the :ipc mode is not built, only :local"
+      mode -> raise ArgumentError, "expected one of :local, :ipc, got: #{inspect(mode)}"
+    end
+  end
+
   @impl true
-  def to_pointer(_, _), do: raise(ArgumentError, "HipNx.Backend does not support pointers")
+  def from_pointer(%Nx.Pointer{} = pointer, type, dims, backend_opts, opts) do
+    device = init(backend_opts)[:device]
+    opts = Keyword.validate!(opts, [:names])
+    template = Nx.template(dims, type, names: opts[:names])
+    size = bytes(template)
+
+    case pointer do
+      %Nx.Pointer{data_size: other} when other != size ->
+        raise ArgumentError, "invalid pointer data_size for shape, expected: #{size}, got: #{other}"
+
+      %Nx.Pointer{kind: :local, address: address} ->
+        # the memory stays with its owner: deallocating this tensor never frees it
+        to_nx(unwrap!(NIF.wrap(ctx(device), address, size)), device, template)
+
+      %Nx.Pointer{kind: :ipc} ->
+        raise ArgumentError, "HipNx.Backend.from_pointer/5: only pointers of kind :local are built"
+    end
+  end
 end

@@ -30,6 +30,8 @@ defmodule HipNx.NIF do
   def iota(_ctx, _out_dt, _n, _dim, _inner, _out_bytes), do: err()
   def eye(_ctx, _out_dt, _n, _rows, _cols, _out_bytes), do: err()
   def narrow_int(_ctx, _buf, _n, _bits, _signed), do: err()
+  def device_ptr(_buf), do: err()
+  def wrap(_ctx, _address, _nbytes), do: err()
   def threefry2x32(_ctx, _key, _n, _out_bytes), do: err()
   def sync(_ctx), do: err()
 
