@@ -33,8 +33,7 @@ K_INNER, K_OUTER = 0, 1
 OOB_RAISE, OOB_CLAMP = 0, 1
 
 # callbacks of the behaviour that are not on the device path (nx/lib/nx/backend.ex:58-144)
-UNSUPPORTED = ["to_batched",
-               "conv", "window_sum", "window_product",
+UNSUPPORTED = ["conv", "window_sum", "window_product",
                "window_max", "window_min", "reduce", "window_reduce", "window_scatter_max", "window_scatter_min",
                "indexed_add", "indexed_put", "sort", "argsort", "fft", "ifft", "fft2", "ifft2", "triangular_solve",
                "conjugate", "real", "imag"]
@@ -581,6 +580,37 @@ class HipNxBackend:
             L.i64_array([d * s for d, s in zip(dense, strides)]), sum(d * s for d, s in zip(dense, starts)),
             L.i64_array(cls._dense_strides(out.shape)), 0, cls._handle(t), res.data.ref.handle))
         return res
+
+    @classmethod
+    def to_batched(cls, out: Tensor, t: Tensor, opts):
+        """to_batched/3 (backend.ex:58; oracle binary_backend.ex:178-211): a lazy sequence of
+        batches of out.shape[0] leading entries -- each one contiguous copy; with leftover "repeat"
+        a last, short batch is completed from the tensor's first entries (two copies into one
+        buffer)."""
+        dev = cls._device_of(t)
+        t = cls._from_nx(t, dev)
+        batch, total = out.shape[0], t.shape[0]
+        full, rest = divmod(total, batch)
+        row = prod(t.shape[1:]) * T.size_bytes(t.type)
+
+        def window(res, first, count, at):
+            # `count` leading entries starting at entry `first`, written from entry `at` of the batch
+            if count and row:
+                L.check(L.lib.hipnx_strided_copy(
+                    res.data.ref.ctx, 1, 1, L.i64_array([count * row]), L.i64_array([1]), first * row, L.i64_array([1]),
+                    at * row, cls._handle(t), res.data.ref.handle))
+
+        def batches():
+            for i in range(full + (1 if rest and opts.get("leftover", "repeat") == "repeat" else 0)):
+                res = cls._alloc(out, dev)
+                if i < full:
+                    window(res, i * batch, batch, 0)
+                else:
+                    window(res, full * batch, rest, 0)
+                    window(res, 0, batch - rest, rest)
+                yield res
+
+        return batches()
 
     @classmethod
     def pad(cls, out: Tensor, t: Tensor, pad_value: Tensor, padding_config) -> Tensor:

@@ -43,6 +43,24 @@ class HostBinary:
         return binary_prefix(t.data.state, t.type, min(int(limit), t.size))
 
     @classmethod
+    def to_batched(cls, out: Tensor, t: Tensor, opts):
+        """to_batched/3 (binary_backend.ex:178-211): byte ranges of the binary."""
+        if T.is_sub_byte(t.type):
+            raise NotImplementedError("HostBinary.to_batched of a sub-byte tensor needs a compute backend")
+        state = cls.to_binary(t, t.size)
+        size = out.size * T.size_bytes(out.type)
+        full, rest = divmod(t.shape[0], out.shape[0])
+        count = full + (1 if rest and opts.get("leftover", "repeat") == "repeat" else 0)
+
+        def one(i):
+            if i < full:
+                return out.with_(data=cls(state[i * size:(i + 1) * size]))
+            tail = state[full * size:]
+            return out.with_(data=cls(tail + state[:size - len(tail)]))
+
+        return (one(i) for i in range(count))
+
+    @classmethod
     def backend_copy(cls, t: Tensor, backend, opts=None) -> Tensor:
         return backend.from_binary(t, cls.to_binary(t, t.size), opts)
 

@@ -135,6 +135,23 @@ def to_binary(t: Tensor, limit=None) -> bytes:
     return type(t.data).to_binary(t, limit)
 
 
+def to_batched(t, batch_size: int, leftover="repeat"):
+    """Nx.to_batched/3 (nx.ex:2455-2666): a lazy sequence of tensors of `batch_size` leading
+    entries; a last, short batch is completed from the first entries ("repeat") or dropped
+    ("discard")."""
+    if not isinstance(batch_size, int) or batch_size < 1:
+        raise ValueError("batch_size must be a positive integer")
+    if leftover not in ("repeat", "discard"):
+        raise ValueError(f"expected :leftover to be :repeat or :discard, got: {leftover!r}")
+    t = to_tensor(t)
+    if t.shape == ():
+        raise ValueError("cannot batch non-vectorized scalar tensor")
+    if t.shape[0] < batch_size:
+        raise ValueError("cannot batch beyond original tensor")
+    out = t.with_(shape=(batch_size,) + t.shape[1:], names=t.names)
+    return _impl(t).to_batched(out, t, {"leftover": leftover})
+
+
 def to_numpy(t: Tensor) -> np.ndarray:
     """Raw element array (bf16 as uint16 bit patterns)."""
     return binary_to_numpy(to_binary(t), t.type, t.shape).copy()

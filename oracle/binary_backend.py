@@ -164,6 +164,22 @@ class BinaryBackend:
         return res
 
     @classmethod
+    def to_batched(cls, out, t, opts):  # binary_backend.ex:178-211
+        batch, total = out.shape[0], t.shape[0]
+        full, rest = divmod(total, batch)
+        state = bytes(cls._bin(t))
+        size = out.size * T.size_bytes(out.type)
+        count = full + (1 if rest and opts.get("leftover", "repeat") == "repeat" else 0)
+
+        def one(i):
+            if i < full:
+                return out.with_(data=cls(bytearray(state[i * size:(i + 1) * size])))
+            tail = state[full * size:]
+            return out.with_(data=cls(bytearray(tail + state[:size - len(tail)])))
+
+        return (one(i) for i in range(count))
+
+    @classmethod
     def backend_copy(cls, t, backend, opts=None):
         return backend.from_binary(t, cls.to_binary(t, t.size), opts)
 

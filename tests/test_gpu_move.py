@@ -96,3 +96,23 @@ def test_gather_clamp_policy_matches_the_compiled_backends(hip):
     idx = from_numpy(np.array([[-1, -1], [10, 11], [-1, 10]], dtype=np.int32), "s32", hip)
     from nx_amd.backend import OOB_CLAMP
     assert hip.to_numpy(Nx.gather(t, idx, oob_policy=OOB_CLAMP)).tolist() == [1, 4, 2]
+
+
+def test_to_batched_known_answers_and_cyclic_rows(hip):
+    from to_batched_support import check_counts, check_known_answers
+    check_known_answers(hip)
+    check_counts(hip)
+
+
+@pytest.mark.parametrize("ty", ["u8", "bf16", "f32", "s64", "u4"])
+@pytest.mark.parametrize("shape,batch", [((1000, 33), 64), ((7, 3, 5), 2), ((4096,), 1000)])
+def test_to_batched_against_the_oracle(ty, shape, batch, hip, oracle):
+    from nx_amd import nx as Nx
+    n = int(np.prod(shape))
+    values = (np.arange(n) % 7).reshape(shape)
+    h, o = Nx.tensor(values, type=ty, backend=hip), Nx.tensor(values, type=ty, backend=oracle)
+    for leftover in ("repeat", "discard"):
+        got, want = list(Nx.to_batched(h, batch, leftover=leftover)), list(Nx.to_batched(o, batch, leftover=leftover))
+        assert len(got) == len(want)
+        for g, w in zip(got, want):
+            assert g.type == w.type and g.shape == w.shape and Nx.to_binary(g) == Nx.to_binary(w)

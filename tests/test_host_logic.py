@@ -132,3 +132,11 @@ def test_front_end_runs_unchanged_on_the_oracle_backend(oracle):
     assert Nx.dot(Nx.as_type(t, "s8"), Nx.as_type(t, "s8")).type == ("s", 8)
     assert Nx.argmax(t, axis=0, type="u32").type == ("u", 32)
     assert Nx.exp(t).type == ("f", 32) and Nx.exp(Nx.as_type(t, "bf16")).type == ("bf", 16)
+
+
+def test_to_batched_known_answers_on_the_host_backend_and_the_oracle(oracle):
+    from nx_amd.host import HostBinary
+    from to_batched_support import check_counts, check_known_answers
+    for backend in (HostBinary, oracle):
+        check_known_answers(backend)
+        check_counts(backend)
