@@ -23,8 +23,10 @@
  */
 #ifndef HIPNX_H
 #define HIPNX_H
+#ifndef __HIPCC_RTC__ /* the run-time compiler brings its own fixed-width types and has no C headers */
 #include <stddef.h>
 #include <stdint.h>
+#endif
 #ifdef __cplusplus
 extern "C" {
 #endif
@@ -280,6 +282,18 @@ int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_fused_instr
                             const hipnx_buf *const *inputs, const int *in_dts, const int64_t *in_row_strides,
                             const int *in_col_strides, int64_t rows, int64_t cols, int reduce_op, int out_dt,
                             hipnx_buf *out);
+
+/* How hipnx_fused_elementwise runs a program on this context.  HIPNX_FUSED_INTERPRETED (the default):
+ * one pair of kernels decodes any program, instruction by instruction.  HIPNX_FUSED_COMPILED: each
+ * distinct program (instructions, input types and column strides, result type, reduction) is written
+ * out over the same device functions, compiled for the device once by the run-time compiler (a few
+ * hundred milliseconds) and kept with the context -- the role exla/lib/exla/defn.ex's compilation
+ * cache plays for a whole function, here for one element-wise group.  Results are bit-identical in
+ * both modes.  A program first met while the context is capturing runs interpreted in that capture.
+ * hipnx_fused_compiled_count reports how many programs the context holds compiled. */
+enum { HIPNX_FUSED_INTERPRETED = 0, HIPNX_FUSED_COMPILED = 1 };
+int hipnx_fused_set_mode(hipnx_ctx *ctx, int mode);
+int hipnx_fused_compiled_count(hipnx_ctx *ctx, int *count);
 
 /* ---- captured sequences ---------------------------------------------------------------------
  * The reference's evaluator (nx/lib/nx/defn/evaluator.ex:363-388) issues one callback per node

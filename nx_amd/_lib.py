@@ -44,6 +44,7 @@ class FusedInstr(C.Structure):
 FUSED_SET, FUSED_UNARY, FUSED_BINARY, FUSED_SELECT, FUSED_AS_TYPE = range(5)
 FUSED_SRC_CONST, FUSED_SRC_INPUT, FUSED_SRC_SAVED = range(3)
 FUSED_SAVED, FUSED_MAX_INSTR, FUSED_MAX_INPUTS = 3, 32, 8
+FUSED_INTERPRETED, FUSED_COMPILED = 0, 1
 
 _ctx_p, _buf_p = C.c_void_p, C.c_void_p
 _i64p, _intp = C.POINTER(C.c_int64), C.POINTER(C.c_int)
@@ -87,6 +88,8 @@ PROTOTYPES = {
     "hipnx_iota": [_ctx_p, C.c_int, C.c_int64, C.c_int64, C.c_int64, _buf_p],
     "hipnx_eye": [_ctx_p, C.c_int, C.c_int64, C.c_int64, C.c_int64, _buf_p],
     "hipnx_narrow_int": [_ctx_p, _buf_p, C.c_int64, C.c_int, C.c_int],
+    "hipnx_fused_set_mode": [_ctx_p, C.c_int],
+    "hipnx_fused_compiled_count": [_ctx_p, C.POINTER(C.c_int)],
     "hipnx_threefry2x32": [_ctx_p, _buf_p, C.c_int64, _buf_p],
     "hipnx_fused_elementwise": [_ctx_p, C.c_int, C.c_void_p, C.c_int, C.POINTER(C.c_void_p), _intp, _i64p, _intp, C.c_int64,
                                 C.c_int64, C.c_int, C.c_int, _buf_p],

@@ -760,11 +760,17 @@ class HipNxBackend:
         dev = cls._device_of(*inputs) if inputs else 0
         inputs = [cls._from_nx(t, dev) for t in inputs]
         rows, cols, strides = layout
-        prog = (L.FusedInstr * len(program))()
-        for q, ins in zip(prog, program):
-            q.kind, q.op, q.src, q.arg = ins["kind"], ins.get("op", 0), ins.get("src", 0), ins.get("arg", 0)
-            q.src2, q.arg2, q.flags, q.dt = ins.get("src2", 0), ins.get("arg2", 0), ins.get("flags", 0), T.code(ins["dt"])
-            q.imm, q.imm2 = ins.get("imm", 0.0), ins.get("imm2", 0.0)
+        prog = getattr(program, "packed", None)
+        if prog is None:
+            prog = (L.FusedInstr * len(program))()
+            for q, ins in zip(prog, program):
+                q.kind, q.op, q.src, q.arg = ins["kind"], ins.get("op", 0), ins.get("src", 0), ins.get("arg", 0)
+                q.src2, q.arg2, q.flags, q.dt = ins.get("src2", 0), ins.get("arg2", 0), ins.get("flags", 0), T.code(ins["dt"])
+                q.imm, q.imm2 = ins.get("imm", 0.0), ins.get("imm2", 0.0)
+            try:
+                program.packed = prog  # a caller's list type with room for the packed form keeps it
+            except AttributeError:
+                pass
         res = cls._alloc(out, dev)
         n = max(len(inputs), 1)
         handles = (C.c_void_p * n)(*[cls._handle(t) for t in inputs])
@@ -888,3 +894,19 @@ def mem_stats(device: int = 0):
     live, peak, pooled = C.c_uint64(), C.c_uint64(), C.c_uint64()
     L.check(L.lib.hipnx_mem_stats(_Context.get(device), C.byref(live), C.byref(peak), C.byref(pooled)))
     return {"live": live.value, "peak": peak.value, "pooled": pooled.value}
+
+
+def fused_mode(mode: str, device: int = 0) -> None:
+    """How fused groups run on the device from now on: "interpreted" (one pair of kernels decodes any
+    program; the default) or "compiled" (each distinct program is compiled for the device once, on
+    first use, and kept).  Results are bit-identical."""
+    codes = {"interpreted": L.FUSED_INTERPRETED, "compiled": L.FUSED_COMPILED}
+    if mode not in codes:
+        raise ValueError(f"expected one of {sorted(codes)!r}, got: {mode!r}")
+    L.check(L.lib.hipnx_fused_set_mode(_Context.get(device), codes[mode]))
+
+
+def fused_compiled_count(device: int = 0) -> int:
+    count = C.c_int()
+    L.check(L.lib.hipnx_fused_compiled_count(_Context.get(device), C.byref(count)))
+    return count.value

@@ -193,6 +193,8 @@ int hipnx_ctx_destroy(hipnx_ctx *ctx) {
     delete g;
   }
   ctx->graphs.clear();
+  for (auto &kv : ctx->fused_kernels) (void)hipModuleUnload(kv.second.first);
+  ctx->fused_kernels.clear();
   for (auto &kv : ctx->pool) (void)hipFree(kv.second);
   ctx->pool.clear();
   if (ctx->flag) (void)hipFree(ctx->flag);

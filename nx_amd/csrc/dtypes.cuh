@@ -7,10 +7,14 @@
 // f32/f16 round to nearest even, bf16 is the f32 encoding with the low 16 bits dropped, and a
 // NaN is always written as the canonical quiet NaN of the output type.
 #pragma once
+#ifndef __HIPCC_RTC__  // the run-time compiler has the device runtime built in and is given headers by name
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
 #include "../../include/hipnx.h"
+#else
+#include "hipnx.h"
+#endif
 
 namespace hipnx {
 

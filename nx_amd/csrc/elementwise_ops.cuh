@@ -8,8 +8,10 @@
 //   double  for every other combination that involves a float;
 //   int64_t (two's-complement wrap) when operands and output are integers.
 #pragma once
+#ifndef __HIPCC_RTC__
 #include <type_traits>
 #include <utility>
+#endif
 
 #include "dtypes.cuh"
 

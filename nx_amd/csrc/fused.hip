@@ -19,63 +19,10 @@
 // u8 truth values between comparisons / logical ops and select, and integer inputs of at most
 // 32 bits feeding an as_type (exact in f32 after one rounding, as the as_type kernel does it).
 // Bound by HBM: bytes(inputs) + bytes(out).
-#include "elementwise_ops.cuh"
+#include "fused_ops.cuh"
 #include "internal.h"
-#include "reduce_ops.cuh"
 
 namespace hipnx {
-
-constexpr int FBLOCK = 256;
-constexpr int FE = 8;  // elements per vector: two 16-byte accesses of f32, one of a 2-byte type
-constexpr int FV = 1;  // vectors per lane and trip (more were measured: the registers they take cost more in
-                       // waves per SIMD than the shared decoding saves: 276 / 303 / 402 us for 1 / 2 / 4)
-
-static_assert(sizeof(hipnx_fused_instr) == 16, "an instruction is one 16-byte scalar load");
-
-struct FusedArgs {
-  int n_instr, n_inputs;
-  int64_t pad_to_16;
-  hipnx_fused_instr ins[HIPNX_FUSED_MAX_INSTR];
-  const void *in[HIPNX_FUSED_MAX_INPUTS];
-  int in_dt[HIPNX_FUSED_MAX_INPUTS];
-  int64_t in_rs[HIPNX_FUSED_MAX_INPUTS];  // element stride between rows (0 = the same row for all)
-  int in_cs[HIPNX_FUSED_MAX_INPUTS];      // element stride along a row: 1, or 0 = one value per row
-  void *out;
-  int out_dt, unused;
-  int64_t rows, cols, vecs_per_row, nvec;
-};
-
-// The argument block is read where the launch put it (the kernel-argument segment, constant address
-// space) with wave-uniform indices: indexing the by-value copy would move it to per-lane scratch.
-typedef const __attribute__((address_space(4))) FusedArgs *KernArgs;
-typedef float Vecs[FV][FE];
-
-// what a store to `dt` followed by a load would give back
-__device__ __forceinline__ float round_to(float x, int dt) {
-  switch (dt) {
-    case HIPNX_BF16: return bf16_bits_to_f32(f32_to_bf16_bits_trunc(x));
-    case HIPNX_F16: return (float)bits_f16(f32_to_f16_bits(x));
-    default: return x;  // f32, and u8 truth values (0 / 1)
-  }
-}
-
-// one uniform dispatch per instruction, the loops over the vectors inside each case
-template <int OP>
-__device__ __forceinline__ void unary_vecs(Vecs &x) {
-#pragma unroll
-  for (int u = 0; u < FV; u++)
-#pragma unroll
-    for (int e = 0; e < FE; e++) x[u][e] = unary_apply<OP, float>(x[u][e], 32);
-}
-
-template <int OP>
-__device__ __forceinline__ void binary_vecs(Vecs &x, const Vecs &y, bool swap) {
-#pragma unroll
-  for (int u = 0; u < FV; u++)
-#pragma unroll
-    for (int e = 0; e < FE; e++)
-      x[u][e] = swap ? binary_apply<OP, float, false>(y[u][e], x[u][e]) : binary_apply<OP, float, false>(x[u][e], y[u][e]);
-}
 
 // The kernel comes in two sizes.  The registers a kernel needs are those of its hungriest path, and
 // the rarely used functions (pow, atan2, remainder, the trigonometric and hyperbolic families, erf,
@@ -97,79 +44,6 @@ template <bool FULL, int... OPS>
 __device__ __forceinline__ void binary_all(std::integer_sequence<int, OPS...>, int op, Vecs &x, const Vecs &y, bool swap) {
   (void)(((FULL || binary_light(OPS)) && op == OPS ? (binary_vecs<OPS>(x, y, swap), true) : false) || ...);
 }
-
-__device__ __forceinline__ float element_to_f32(uint32_t bits, int dt) {
-  switch (dt) {
-    case HIPNX_U8: case HIPNX_U16: case HIPNX_U32: return (float)bits;
-    case HIPNX_S8: return (float)(int32_t)(int8_t)bits;
-    case HIPNX_S16: return (float)(int32_t)(int16_t)bits;
-    case HIPNX_S32: return (float)(int32_t)bits;
-    case HIPNX_F16: return (float)bits_f16((uint16_t)bits);
-    case HIPNX_BF16: return bf16_bits_to_f32((uint16_t)bits);
-    default: return __uint_as_float(bits);
-  }
-}
-
-// input k for the lane's FV vectors: all loads are requested, then converted
-__device__ __forceinline__ void load_input(KernArgs a, int k, const int64_t (&row)[FV], const int64_t (&col)[FV], Vecs &dst) {
-  const int dt = a->in_dt[k], cs = a->in_cs[k];
-  const int esz = (dt == HIPNX_U8 || dt == HIPNX_S8) ? 1 : (dt == HIPNX_U32 || dt == HIPNX_S32 || dt == HIPNX_F32) ? 4 : 2;
-  const char *base = (const char *)a->in[k];
-  const int64_t rs = a->in_rs[k];
-  uint32_t w[FV][FE];  // raw words: 8 for 4-byte elements, 4 for 2-byte ones, 2 for bytes, 1 for a broadcast value
-#pragma unroll
-  for (int u = 0; u < FV; u++) {
-    const char *p = base + (row[u] * rs + col[u] * cs) * esz;
-    if (cs == 0) {
-      w[u][0] = esz == 4 ? *reinterpret_cast<const uint32_t *>(p)
-                : esz == 2 ? (uint32_t)*reinterpret_cast<const uint16_t *>(p)
-                           : (uint32_t)*reinterpret_cast<const uint8_t *>(p);
-    } else if (esz == 4) {
-      const uint4 lo = *reinterpret_cast<const uint4 *>(p), hi = *reinterpret_cast<const uint4 *>(p + 16);
-      w[u][0] = lo.x; w[u][1] = lo.y; w[u][2] = lo.z; w[u][3] = lo.w;
-      w[u][4] = hi.x; w[u][5] = hi.y; w[u][6] = hi.z; w[u][7] = hi.w;
-    } else if (esz == 2) {
-      const uint4 lo = *reinterpret_cast<const uint4 *>(p);
-      w[u][0] = lo.x; w[u][1] = lo.y; w[u][2] = lo.z; w[u][3] = lo.w;
-    } else {
-      const uint2 lo = *reinterpret_cast<const uint2 *>(p);
-      w[u][0] = lo.x; w[u][1] = lo.y;
-    }
-  }
-#pragma unroll
-  for (int u = 0; u < FV; u++) {
-    if (cs == 0) {
-      const float v = element_to_f32(w[u][0], dt);
-#pragma unroll
-      for (int e = 0; e < FE; e++) dst[u][e] = v;
-    } else if (esz == 4) {
-      if (dt == HIPNX_F32) {
-#pragma unroll
-        for (int e = 0; e < FE; e++) dst[u][e] = __uint_as_float(w[u][e]);
-      } else {
-#pragma unroll
-        for (int e = 0; e < FE; e++) dst[u][e] = element_to_f32(w[u][e], dt);
-      }
-    } else if (esz == 2) {
-#pragma unroll
-      for (int e = 0; e < FE; e++) dst[u][e] = element_to_f32((w[u][e / 2] >> (16 * (e & 1))) & 0xFFFFu, dt);
-    } else {
-#pragma unroll
-      for (int e = 0; e < FE; e++) dst[u][e] = element_to_f32((w[u][e / 4] >> (8 * (e & 3))) & 0xFFu, dt);
-    }
-  }
-}
-
-__device__ __forceinline__ void copy_vecs(Vecs &dst, const Vecs &src) {
-#pragma unroll
-  for (int u = 0; u < FV; u++)
-#pragma unroll
-    for (int e = 0; e < FE; e++) dst[u][e] = src[u][e];
-}
-
-struct Saved {
-  Vecs s[HIPNX_FUSED_SAVED];
-};
 
 // saved slots are numbered by wave-uniform run-time values: a switch keeps them in registers (the
 // empty asm differs from case to case so that the cases are not merged into one access through a
@@ -193,7 +67,7 @@ __device__ __forceinline__ void write_saved(Saved &S, int slot, const Vecs &src)
 __device__ __forceinline__ void fetch(KernArgs a, const Saved &S, int src, int arg, float imm, const int64_t (&row)[FV],
                                       const int64_t (&col)[FV], Vecs &dst) {
   switch (src) {
-    case HIPNX_FUSED_SRC_INPUT: load_input(a, arg, row, col, dst); break;
+    case HIPNX_FUSED_SRC_INPUT: load_input_as(a, arg, a->in_dt[arg], a->in_cs[arg], row, col, dst); break;
     case HIPNX_FUSED_SRC_SAVED: read_saved(S, arg, dst); break;
     default:
 #pragma unroll
@@ -251,74 +125,23 @@ __device__ __forceinline__ void run_program(KernArgs a, int n_instr, const int64
 }
 
 template <bool FULL>
+struct RunInterpreted {
+  static __device__ __forceinline__ void run(KernArgs a, const int64_t (&row)[FV], const int64_t (&col)[FV], Vecs &acc) {
+    run_program<FULL>(a, a->n_instr, row, col, acc);
+  }
+  static __device__ __forceinline__ int out_dt(KernArgs a) { return a->out_dt; }
+};
+
+template <bool FULL>
 __global__ void __launch_bounds__(FBLOCK) fused_elementwise_kernel(FusedArgs by_value) {
   (void)by_value;
-  KernArgs a = (KernArgs)__builtin_amdgcn_kernarg_segment_ptr();
-  const int64_t nvec = a->nvec, vecs_per_row = a->vecs_per_row, cols = a->cols;
-  const int n_instr = a->n_instr;
-  const int64_t stride = (int64_t)gridDim.x * FBLOCK;
-  for (int64_t v0 = (int64_t)blockIdx.x * FBLOCK + threadIdx.x; v0 < nvec; v0 += stride * FV) {
-    int64_t row[FV], col[FV];
-    bool live[FV];
-#pragma unroll
-    for (int u = 0; u < FV; u++) {
-      int64_t v = v0 + u * stride;
-      live[u] = v < nvec;
-      if (!live[u]) v = v0;  // a vector past the end repeats the lane's first one and is not stored
-      row[u] = 0;
-      col[u] = v * FE;
-      if (vecs_per_row != nvec) {  // more than one row
-        row[u] = nvec <= 0xFFFFFFFFll ? (int64_t)((uint32_t)v / (uint32_t)vecs_per_row) : v / vecs_per_row;
-        col[u] = (v - row[u] * vecs_per_row) * FE;
-      }
-    }
-    Vecs acc;
-    run_program<FULL>(a, n_instr, row, col, acc);
-    void *out = (void *)a->out;
-    const int odt = a->out_dt;
-#pragma unroll
-    for (int u = 0; u < FV; u++)
-      if (live[u]) store_vec<float, FE>(out, odt, row[u] * cols + col[u], acc[u]);
-  }
+  fused_elementwise_body<RunInterpreted<FULL>>();
 }
 
-// The group's result reduced along its rows without ever being stored: TPR lanes per row walk it
-// in the order of reduce_rows_kernel (lane l takes the vectors l, l + TPR, ... and folds their
-// elements in turn, then lanes combine by wave shuffles and the block's waves through LDS) with the
-// same reducer policy, so the value equals what the element-wise group followed by the separate
-// reduction kernel gives, bit for bit.
 template <typename R, typename CT, int TPR>
 __global__ void __launch_bounds__(FBLOCK) fused_reduce_rows_kernel(FusedArgs by_value) {
   (void)by_value;
-  static_assert(FV == 1, "one vector per lane and step");
-  KernArgs a = (KernArgs)__builtin_amdgcn_kernarg_segment_ptr();
-  constexpr int RPB = FBLOCK / TPR;
-  const int sub = threadIdx.x / TPR, lane = threadIdx.x % TPR;
-  const int64_t rows = a->rows, red = a->cols;
-  const int n_instr = a->n_instr;
-  const int64_t r = (int64_t)blockIdx.x * RPB + sub;
-  typename R::acc_t acc = R::init();
-  if (r < rows) {
-    const int64_t step = (int64_t)TPR * FE;
-    for (int64_t k = (int64_t)lane * FE; k < red; k += step) {
-      const int64_t row[FV] = {r}, col[FV] = {k};
-      Vecs x;
-      run_program<false>(a, n_instr, row, col, x);
-#pragma unroll
-      for (int e = 0; e < FE; e++) acc = R::accumulate(acc, (CT)x[0][e], k + e);
-    }
-  }
-  acc = wave_reduce<R>(acc);
-  if constexpr (TPR > WAVE) {
-    __shared__ typename R::acc_t sm[FBLOCK / WAVE];
-    if (threadIdx.x % WAVE == 0) sm[threadIdx.x / WAVE] = acc;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-#pragma unroll
-      for (int w = 1; w < FBLOCK / WAVE; w++) acc = R::combine(acc, sm[w]);
-    }
-  }
-  if (lane == 0 && r < rows) finalize((void *)a->out, a->out_dt, r, acc);
+  fused_reduce_rows_body<RunInterpreted<false>, R, CT, TPR>();
 }
 
 template <typename R, typename CT>
@@ -332,6 +155,9 @@ static void launch_fused_reduce(const hipnx_ctx *ctx, const FusedArgs &a) {
 }
 
 static bool narrow(int dt) { return dt == HIPNX_BF16 || dt == HIPNX_F16 || dt == HIPNX_F32; }
+
+// fused_rtc.hip
+int fused_launch_compiled(hipnx_ctx *ctx, const FusedArgs &a, int reduce_op, bool block_per_row, unsigned grid, bool *done);
 
 }  // namespace hipnx
 
@@ -428,6 +254,16 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
   a.cols = cols;
   a.vecs_per_row = cols / FE;
   a.nvec = rows * a.vecs_per_row;
+  if (ctx->fused_mode == HIPNX_FUSED_COMPILED) {
+    // the same grids as the interpreting kernels below
+    const bool block_per_row = reduce_op != -1 && a.cols > 4096;
+    int64_t grid = reduce_op == -1 ? (a.nvec + (int64_t)FBLOCK * FV - 1) / ((int64_t)FBLOCK * FV)
+                   : block_per_row ? a.rows : (a.rows + FBLOCK / WAVE - 1) / (FBLOCK / WAVE);
+    if (grid > (1ll << 30)) grid = 1ll << 30;
+    bool done = false;
+    if (int st = fused_launch_compiled(ctx, a, reduce_op, block_per_row, (unsigned)grid, &done)) return st;
+    if (done) return HIPNX_OK;
+  }
   if (reduce_op == HIPNX_RED_SUM) launch_fused_reduce<PlainReducer<double, HIPNX_RED_SUM, false>, double>(ctx, a);
   else if (reduce_op == HIPNX_RED_MAX) launch_fused_reduce<PlainReducer<float, HIPNX_RED_MAX, false>, float>(ctx, a);
   else if (reduce_op == HIPNX_RED_MIN) launch_fused_reduce<PlainReducer<float, HIPNX_RED_MIN, false>, float>(ctx, a);

@@ -1,0 +1,272 @@
+// The device side of the fused element-wise groups, shared by the interpreting kernels of
+// fused.hip and by the kernels compiled at run time for one program (fused_rtc.cpp): the lane's
+// vectors, the loads with their conversions, the rounding after every instruction, the kernel
+// bodies, and the program as compile-time constants.  Both forms call the same functions in the
+// same order on the same values, which is what makes their results bit-identical.
+// This header is also given to the run-time compiler, which has no host headers: keep it to
+// device code.
+#pragma once
+#include "elementwise_ops.cuh"
+#include "reduce_ops.cuh"
+
+namespace hipnx {
+
+
+constexpr int FBLOCK = 256;
+constexpr int FE = 8;  // elements per vector: two 16-byte accesses of f32, one of a 2-byte type
+constexpr int FV = 1;  // vectors per lane and trip (more were measured: the registers they take cost more in
+                       // waves per SIMD than the shared decoding saves: 276 / 303 / 402 us for 1 / 2 / 4)
+
+static_assert(sizeof(hipnx_fused_instr) == 16, "an instruction is one 16-byte scalar load");
+
+struct FusedArgs {
+  int n_instr, n_inputs;
+  int64_t pad_to_16;
+  hipnx_fused_instr ins[HIPNX_FUSED_MAX_INSTR];
+  const void *in[HIPNX_FUSED_MAX_INPUTS];
+  int in_dt[HIPNX_FUSED_MAX_INPUTS];
+  int64_t in_rs[HIPNX_FUSED_MAX_INPUTS];  // element stride between rows (0 = the same row for all)
+  int in_cs[HIPNX_FUSED_MAX_INPUTS];      // element stride along a row: 1, or 0 = one value per row
+  void *out;
+  int out_dt, unused;
+  int64_t rows, cols, vecs_per_row, nvec;
+};
+
+// The argument block is read where the launch put it (the kernel-argument segment, constant address
+// space) with wave-uniform indices: indexing the by-value copy would move it to per-lane scratch.
+typedef const __attribute__((address_space(4))) FusedArgs *KernArgs;
+typedef float Vecs[FV][FE];
+
+// what a store to `dt` followed by a load would give back
+__device__ __forceinline__ float round_to(float x, int dt) {
+  switch (dt) {
+    case HIPNX_BF16: return bf16_bits_to_f32(f32_to_bf16_bits_trunc(x));
+    case HIPNX_F16: return (float)bits_f16(f32_to_f16_bits(x));
+    default: return x;  // f32, and u8 truth values (0 / 1)
+  }
+}
+
+// one uniform dispatch per instruction, the loops over the vectors inside each case
+template <int OP>
+__device__ __forceinline__ void unary_vecs(Vecs &x) {
+#pragma unroll
+  for (int u = 0; u < FV; u++)
+#pragma unroll
+    for (int e = 0; e < FE; e++) x[u][e] = unary_apply<OP, float>(x[u][e], 32);
+}
+
+template <int OP>
+__device__ __forceinline__ void binary_vecs(Vecs &x, const Vecs &y, bool swap) {
+#pragma unroll
+  for (int u = 0; u < FV; u++)
+#pragma unroll
+    for (int e = 0; e < FE; e++)
+      x[u][e] = swap ? binary_apply<OP, float, false>(y[u][e], x[u][e]) : binary_apply<OP, float, false>(x[u][e], y[u][e]);
+}
+
+__device__ __forceinline__ float element_to_f32(uint32_t bits, int dt) {
+  switch (dt) {
+    case HIPNX_U8: case HIPNX_U16: case HIPNX_U32: return (float)bits;
+    case HIPNX_S8: return (float)(int32_t)(int8_t)bits;
+    case HIPNX_S16: return (float)(int32_t)(int16_t)bits;
+    case HIPNX_S32: return (float)(int32_t)bits;
+    case HIPNX_F16: return (float)bits_f16((uint16_t)bits);
+    case HIPNX_BF16: return bf16_bits_to_f32((uint16_t)bits);
+    default: return __uint_as_float(bits);
+  }
+}
+
+// input k (element type dt, column stride cs) for the lane's FV vectors: all loads are requested,
+// then converted
+__device__ __forceinline__ void load_input_as(KernArgs a, int k, int dt, int cs, const int64_t (&row)[FV],
+                                              const int64_t (&col)[FV], Vecs &dst) {
+  const int esz = (dt == HIPNX_U8 || dt == HIPNX_S8) ? 1 : (dt == HIPNX_U32 || dt == HIPNX_S32 || dt == HIPNX_F32) ? 4 : 2;
+  const char *base = (const char *)a->in[k];
+  const int64_t rs = a->in_rs[k];
+  uint32_t w[FV][FE];  // raw words: 8 for 4-byte elements, 4 for 2-byte ones, 2 for bytes, 1 for a broadcast value
+#pragma unroll
+  for (int u = 0; u < FV; u++) {
+    const char *p = base + (row[u] * rs + col[u] * cs) * esz;
+    if (cs == 0) {
+      w[u][0] = esz == 4 ? *reinterpret_cast<const uint32_t *>(p)
+                : esz == 2 ? (uint32_t)*reinterpret_cast<const uint16_t *>(p)
+                           : (uint32_t)*reinterpret_cast<const uint8_t *>(p);
+    } else if (esz == 4) {
+      const uint4 lo = *reinterpret_cast<const uint4 *>(p), hi = *reinterpret_cast<const uint4 *>(p + 16);
+      w[u][0] = lo.x; w[u][1] = lo.y; w[u][2] = lo.z; w[u][3] = lo.w;
+      w[u][4] = hi.x; w[u][5] = hi.y; w[u][6] = hi.z; w[u][7] = hi.w;
+    } else if (esz == 2) {
+      const uint4 lo = *reinterpret_cast<const uint4 *>(p);
+      w[u][0] = lo.x; w[u][1] = lo.y; w[u][2] = lo.z; w[u][3] = lo.w;
+    } else {
+      const uint2 lo = *reinterpret_cast<const uint2 *>(p);
+      w[u][0] = lo.x; w[u][1] = lo.y;
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < FV; u++) {
+    if (cs == 0) {
+      const float v = element_to_f32(w[u][0], dt);
+#pragma unroll
+      for (int e = 0; e < FE; e++) dst[u][e] = v;
+    } else if (esz == 4) {
+      if (dt == HIPNX_F32) {
+#pragma unroll
+        for (int e = 0; e < FE; e++) dst[u][e] = __uint_as_float(w[u][e]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < FE; e++) dst[u][e] = element_to_f32(w[u][e], dt);
+      }
+    } else if (esz == 2) {
+#pragma unroll
+      for (int e = 0; e < FE; e++) dst[u][e] = element_to_f32((w[u][e / 2] >> (16 * (e & 1))) & 0xFFFFu, dt);
+    } else {
+#pragma unroll
+      for (int e = 0; e < FE; e++) dst[u][e] = element_to_f32((w[u][e / 4] >> (8 * (e & 3))) & 0xFFu, dt);
+    }
+  }
+}
+
+__device__ __forceinline__ void copy_vecs(Vecs &dst, const Vecs &src) {
+#pragma unroll
+  for (int u = 0; u < FV; u++)
+#pragma unroll
+    for (int e = 0; e < FE; e++) dst[u][e] = src[u][e];
+}
+
+struct Saved {
+  Vecs s[HIPNX_FUSED_SAVED];
+};
+
+
+// ---- the program as compile-time constants ------------------------------------------------------
+// P holds the program one field per array (kind[], op[], src[], arg[], src2[], arg2[], flags[],
+// dt[], imm[] and imm2[] as f32 bit patterns), the inputs' element types and column strides, and
+// the result type.  Every branch the interpreter takes on an instruction field is taken by the
+// compiler here.
+template <typename P, int SRC, int ARG, unsigned IMM>
+__device__ __forceinline__ void fetch_static(KernArgs a, const Saved &S, const int64_t (&row)[FV], const int64_t (&col)[FV], Vecs &dst) {
+  if constexpr (SRC == HIPNX_FUSED_SRC_INPUT) {
+    load_input_as(a, ARG, P::in_dt[ARG], P::in_cs[ARG], row, col, dst);
+  } else if constexpr (SRC == HIPNX_FUSED_SRC_SAVED) {
+    copy_vecs(dst, S.s[ARG]);
+  } else {
+#pragma unroll
+    for (int u = 0; u < FV; u++)
+#pragma unroll
+      for (int e = 0; e < FE; e++) dst[u][e] = __uint_as_float(IMM);
+  }
+}
+
+template <typename P, int PC>
+__device__ __forceinline__ void static_steps(KernArgs a, const int64_t (&row)[FV], const int64_t (&col)[FV], Vecs &acc, Saved &S) {
+  if constexpr (PC < P::n_instr) {
+    constexpr int kind = P::kind[PC], op = P::op[PC], src = P::src[PC], arg = P::arg[PC];
+    constexpr int src2 = P::src2[PC], arg2 = P::arg2[PC], flags = P::flags[PC], dt = P::dt[PC];
+    constexpr unsigned imm = P::imm[PC], imm2 = P::imm2[PC];
+    if constexpr (kind == HIPNX_FUSED_SET) {
+      fetch_static<P, src, arg, imm>(a, S, row, col, acc);
+    } else if constexpr (kind == HIPNX_FUSED_UNARY) {
+      unary_vecs<op>(acc);
+    } else if constexpr (kind == HIPNX_FUSED_BINARY) {
+      Vecs y;
+      fetch_static<P, src, arg, imm>(a, S, row, col, y);
+      binary_vecs<op>(acc, y, (flags & 1) != 0);
+    } else if constexpr (kind == HIPNX_FUSED_SELECT) {
+      Vecs y, z;
+      fetch_static<P, src, arg, imm>(a, S, row, col, y);
+      fetch_static<P, src2, arg2, imm2>(a, S, row, col, z);
+#pragma unroll
+      for (int u = 0; u < FV; u++)
+#pragma unroll
+        for (int e = 0; e < FE; e++) acc[u][e] = acc[u][e] != 0.0f ? y[u][e] : z[u][e];  // NaN is true
+    }
+    if constexpr (dt == HIPNX_BF16 || dt == HIPNX_F16) {
+#pragma unroll
+      for (int u = 0; u < FV; u++)
+#pragma unroll
+        for (int e = 0; e < FE; e++) acc[u][e] = round_to(acc[u][e], dt);
+    }
+    if constexpr ((flags >> 4) != 0) copy_vecs(S.s[(flags >> 4) - 1], acc);
+    static_steps<P, PC + 1>(a, row, col, acc, S);
+  }
+}
+
+template <typename P>
+struct RunStatic {
+  static __device__ __forceinline__ void run(KernArgs a, const int64_t (&row)[FV], const int64_t (&col)[FV], Vecs &acc) {
+    Saved S;
+    static_steps<P, 0>(a, row, col, acc, S);
+  }
+  static __device__ __forceinline__ int out_dt(KernArgs) { return P::out_dt; }
+};
+
+// ---- kernel bodies: RUN is RunStatic<P> or the interpreter of fused.hip ---------------------------
+template <typename RUN>
+__device__ __forceinline__ void fused_elementwise_body() {
+  KernArgs a = (KernArgs)__builtin_amdgcn_kernarg_segment_ptr();
+  const int64_t nvec = a->nvec, vecs_per_row = a->vecs_per_row, cols = a->cols;
+  const int64_t stride = (int64_t)gridDim.x * FBLOCK;
+  for (int64_t v0 = (int64_t)blockIdx.x * FBLOCK + threadIdx.x; v0 < nvec; v0 += stride * FV) {
+    int64_t row[FV], col[FV];
+    bool live[FV];
+#pragma unroll
+    for (int u = 0; u < FV; u++) {
+      int64_t v = v0 + u * stride;
+      live[u] = v < nvec;
+      if (!live[u]) v = v0;  // a vector past the end repeats the lane's first one and is not stored
+      row[u] = 0;
+      col[u] = v * FE;
+      if (vecs_per_row != nvec) {  // more than one row
+        row[u] = nvec <= 0xFFFFFFFFll ? (int64_t)((uint32_t)v / (uint32_t)vecs_per_row) : v / vecs_per_row;
+        col[u] = (v - row[u] * vecs_per_row) * FE;
+      }
+    }
+    Vecs acc;
+    RUN::run(a, row, col, acc);
+    void *out = (void *)a->out;
+    const int odt = RUN::out_dt(a);
+#pragma unroll
+    for (int u = 0; u < FV; u++)
+      if (live[u]) store_vec<float, FE>(out, odt, row[u] * cols + col[u], acc[u]);
+  }
+}
+
+// The group's result reduced along its rows without ever being stored: TPR lanes per row walk it
+// in the order of reduce_rows_kernel (lane l takes the vectors l, l + TPR, ... and folds their
+// elements in turn, then lanes combine by wave shuffles and the block's waves through LDS) with the
+// same reducer policy, so the value equals what the element-wise group followed by the separate
+// reduction kernel gives, bit for bit.
+template <typename RUN, typename R, typename CT, int TPR>
+__device__ __forceinline__ void fused_reduce_rows_body() {
+  static_assert(FV == 1, "one vector per lane and step");
+  KernArgs a = (KernArgs)__builtin_amdgcn_kernarg_segment_ptr();
+  constexpr int RPB = FBLOCK / TPR;
+  const int sub = threadIdx.x / TPR, lane = threadIdx.x % TPR;
+  const int64_t rows = a->rows, red = a->cols;
+  const int64_t r = (int64_t)blockIdx.x * RPB + sub;
+  typename R::acc_t acc = R::init();
+  if (r < rows) {
+    const int64_t step = (int64_t)TPR * FE;
+    for (int64_t k = (int64_t)lane * FE; k < red; k += step) {
+      const int64_t row[FV] = {r}, col[FV] = {k};
+      Vecs x;
+      RUN::run(a, row, col, x);
+#pragma unroll
+      for (int e = 0; e < FE; e++) acc = R::accumulate(acc, (CT)x[0][e], k + e);
+    }
+  }
+  acc = wave_reduce<R>(acc);
+  if constexpr (TPR > WAVE) {
+    __shared__ typename R::acc_t sm[FBLOCK / WAVE];
+    if (threadIdx.x % WAVE == 0) sm[threadIdx.x / WAVE] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+#pragma unroll
+      for (int w = 1; w < FBLOCK / WAVE; w++) acc = R::combine(acc, sm[w]);
+    }
+  }
+  if (lane == 0 && r < rows) finalize((void *)a->out, a->out_dt, r, acc);
+}
+
+}  // namespace hipnx

@@ -8,6 +8,7 @@
 #include <cstdio>
 #include <map>
 #include <mutex>
+#include <string>
 #include <unordered_map>
 #include <vector>
 
@@ -43,6 +44,9 @@ struct hipnx_ctx {
   hipnx_graph *capture = nullptr;                        // non-null while the stream is capturing
   std::unordered_map<void *, hipnx_graph *> graph_blocks;  // block -> the live graph that owns it
   std::vector<hipnx_graph *> graphs;                     // live graphs of this context
+  // fused groups compiled at run time for one program each: program bytes -> loaded kernel
+  int fused_mode = 0;  // 0 = the interpreting kernels, 1 = compile each distinct program once
+  std::unordered_map<std::string, std::pair<hipModule_t, hipFunction_t>> fused_kernels;
 };
 
 struct hipnx_buf {

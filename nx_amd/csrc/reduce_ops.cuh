@@ -3,8 +3,10 @@
 // result is stored.  The kernels that use them fix the order of the folds; two kernels that walk a
 // row in the same order with the same policy give the same bits.
 #pragma once
+#ifndef __HIPCC_RTC__
 #include <type_traits>
 #include <utility>
+#endif
 
 #include "dtypes.cuh"
 

@@ -515,6 +515,11 @@ def _layout(out_shape, in_shapes, split=None):
     return None
 
 
+class _Program(list):
+    """A group's instructions; a backend may keep its packed form of them here after the first launch."""
+    packed = None
+
+
 class _Group:
     """One fused group: the member nodes in evaluation order, its external inputs, and the program
     for the backend's accumulator machine (None when the group does not fit it)."""
@@ -556,7 +561,7 @@ class _Group:
                     readers.setdefault(a.data.id, []).append(i)
         slots: Dict[Any, int] = {}       # member id -> slot while it is saved
         free = list(range(_SAVED_SLOTS))
-        program: List[dict] = []
+        program: List[dict] = _Program()
 
         def source(a):
             """(src, arg, imm) of an operand that is not the accumulator."""

@@ -215,8 +215,17 @@ FUSED_CASES = {
 }
 
 
+@pytest.fixture(params=["interpreted", "compiled"])
+def fused_mode(request, hip):
+    """Runs a test once with the interpreting kernels and once with each program compiled at run time."""
+    from nx_amd.backend import fused_mode as set_mode
+    set_mode(request.param)
+    yield request.param
+    set_mode("interpreted")
+
+
 @pytest.mark.parametrize("name", sorted(FUSED_CASES))
-def test_fused_group_is_bit_identical_to_node_by_node(name, hip):
+def test_fused_group_is_bit_identical_to_node_by_node(name, hip, fused_mode):
     fun, make = FUSED_CASES[name]
     args = make(np.random.default_rng(3), hip)
     fused = defn.compile(fun, *args, fuse=True)
@@ -225,7 +234,7 @@ def test_fused_group_is_bit_identical_to_node_by_node(name, hip):
 
 
 @pytest.mark.parametrize("name", sorted(CHAINS))
-def test_fused_configuration_chains(name, hip):
+def test_fused_configuration_chains(name, hip, fused_mode):
     args = build_args(hip)[name]
     assert_bits_equal(defn.compile(CHAINS[name], *args, fuse=True)(*args), defn.compile(CHAINS[name], *args)(*args), name)
 
@@ -267,6 +276,57 @@ def test_fused_entry_point_validates_its_program(hip):
     np.testing.assert_array_equal(hip.to_numpy(got), -hip.to_numpy(x))
 
 
+def test_each_distinct_program_is_compiled_once(hip):
+    from nx_amd.backend import fused_compiled_count, fused_mode as set_mode
+    fun, make = FUSED_CASES["relu_mask"]
+    args = make(np.random.default_rng(8), hip)
+    other = tuple(rand_float(np.random.default_rng(9), "f32", (16, 128), hip) for _ in range(2))
+    want = defn.compile(fun, *args)(*args)
+    set_mode("compiled")
+    try:
+        before = fused_compiled_count()
+        fused = defn.compile(fun, *args, fuse=True)
+        assert_bits_equal(fused(*args), want, "first call compiles")
+        after = fused_compiled_count()
+        assert after >= before  # `before + 1` unless an earlier test met the same program
+        assert_bits_equal(fused(*args), want, "second call reuses")
+        defn.compile(fun, *other, fuse=True)(*other)  # other shape, same program: the shape is not compiled in
+        assert fused_compiled_count() == after
+        set_mode("interpreted")
+        assert_bits_equal(fused(*args), want, "and back")
+    finally:
+        set_mode("interpreted")
+
+
+def test_program_first_met_during_a_capture_runs_interpreted(hip):
+    from nx_amd import backend as B
+
+    def fresh(x, y):  # a program no other test builds
+        return Nx.subtract(Nx.multiply(Nx.sigmoid(x), 1.25), Nx.floor(y))
+    args = tuple(rand_float(np.random.default_rng(10), "f32", (64, 64), hip) for _ in range(2))
+    want = defn.compile(fresh, *args)(*args)
+    fused = defn.compile(fresh, *args, fuse=True)
+    fused(*args)  # the run before a capture, as the capture rules ask -- interpreted, so nothing is compiled yet
+    B.fused_mode("compiled")
+    try:
+        before = B.fused_compiled_count()
+        B.capture_begin(0)
+        try:
+            out = fused(*args)
+        finally:
+            graph = B.capture_end(0)
+        assert B.fused_compiled_count() == before  # compiling and loading a module is no work to record
+        for _ in range(3):
+            graph.launch()
+            assert_bits_equal(out, want, "replay")
+        del out
+        graph.destroy()
+        assert_bits_equal(fused(*args), want, "compiled after the capture")
+        assert B.fused_compiled_count() == before + 1
+    finally:
+        B.fused_mode("interpreted")
+
+
 # ---- a reduction over the last axis joins the group that feeds it ----------------------------------------
 
 def sum_of_exp(a, b):
@@ -286,7 +346,7 @@ REDUCED = {"sum_of_exp": sum_of_exp, "max_of_scaled": max_of_scaled, "min_of_bf1
 
 @pytest.mark.parametrize("name", sorted(REDUCED))
 @pytest.mark.parametrize("shape", [(64, 256), (300, 4096), (16, 8192), (5, 40000), (4, 65536), (2049, 8), (3, 7, 512)])
-def test_group_with_its_row_reduction_is_bit_identical(name, shape, hip):
+def test_group_with_its_row_reduction_is_bit_identical(name, shape, hip, fused_mode):
     rng = np.random.default_rng(seed_of(name, shape))
     if len(shape) == 3 and name == "sum_of_exp":
         pytest.skip("this function reduces axis 1, which is the last axis only for matrices")
@@ -317,7 +377,7 @@ def fused_groups_of(compiled):
     return groups
 
 
-def test_softmax_becomes_three_kernels(hip):
+def test_softmax_becomes_three_kernels(hip, fused_mode):
     """The scaled scores feed the max and the subtraction, the exponentials feed the sum and the
     division: both are cheap to compute again from the bf16 scores, so nothing but the two row
     statistics and the result is ever stored."""
