@@ -237,7 +237,14 @@ def main():
         _, ms = timed(lambda: Random.uniform_split(key, 0.0, 1.0, shape=(nw,)), steps, warm)
         # bits out; shift, or, subtract, multiply, add, max each read and write the array once
         entry("uniform_f32_2p28_unfused", 4.0 * nw * 13, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-        del key
+        # the same function traced, its bits-to-floats chain (shift, or, bitcast, subtract, ..., max) planned as
+        # one group compiled for the device: the cipher writes the words, one more pass reads them and writes floats
+        from nx_amd import defn as _defn
+        uniform = _defn.compile(lambda k: Random.uniform_split(k, 0.0, 1.0, shape=(nw,)), key, fuse="compiled")
+        _, ms = timed(lambda: uniform(key), steps, warm)
+        entry("uniform_f32_2p28_fused_compiled", 4.0 * nw * 13, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+        entry("uniform_f32_2p28_fused_compiled_two_passes", 4.0 * nw * 3, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+        del key, uniform
 
         # traced chains: one callback per node (the evaluator), and the same chain captured once and
         # replayed as a device graph (one submission for all its kernels)

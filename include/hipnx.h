@@ -270,13 +270,21 @@ int hipnx_threefry2x32(hipnx_ctx *ctx, const hipnx_buf *key, int64_t n, hipnx_bu
  * reduce_op: -1, or HIPNX_RED_SUM / MAX / MIN to reduce the result along its rows without storing it
  * (sum/4, reduce_max/4, reduce_min/4 over the last axis, nx/lib/nx/backend.ex:89-92): `out` then has
  * `rows` elements, and equals the separate reduction kernel applied to the stored result. */
-enum { HIPNX_FUSED_SET = 0, HIPNX_FUSED_UNARY, HIPNX_FUSED_BINARY, HIPNX_FUSED_SELECT, HIPNX_FUSED_AS_TYPE };
+enum { HIPNX_FUSED_SET = 0, HIPNX_FUSED_UNARY, HIPNX_FUSED_BINARY, HIPNX_FUSED_SELECT, HIPNX_FUSED_AS_TYPE,
+       HIPNX_FUSED_BITCAST };
+/* flags bit 1: the instruction works on 32-bit integers (dt u32 / s32) kept as raw bits -- a SET loads the
+ * words of a 4-byte input, or the bits of imm, unconverted; a UNARY / BINARY computes like the integer
+ * class of the separate kernels (wrapping at 32 bits); an AS_TYPE converts the integer of type `op` (an
+ * element-type code) to the float dt; BITCAST (nx/lib/nx/backend.ex:69) relabels the bits.  These need
+ * HIPNX_FUSED_COMPILED: the interpreting kernels return HIPNX_EUNSUPPORTED for them. */
+enum { HIPNX_FUSED_FLAG_SWAP = 1, HIPNX_FUSED_FLAG_INT = 2 };
 enum { HIPNX_FUSED_SRC_CONST = 0, HIPNX_FUSED_SRC_INPUT, HIPNX_FUSED_SRC_SAVED };
 enum { HIPNX_FUSED_SAVED = 3, HIPNX_FUSED_MAX_INSTR = 32, HIPNX_FUSED_MAX_INPUTS = 8 };
 typedef struct {
   uint8_t kind, op, src, arg;
   uint8_t src2, arg2, flags, dt;
-  float imm, imm2;
+  union { float imm; uint32_t imm_bits; };
+  union { float imm2; uint32_t imm2_bits; };
 } hipnx_fused_instr; /* 16 bytes: the interpreter fetches an instruction with one scalar load */
 int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_fused_instr *prog, int n_inputs,
                             const hipnx_buf *const *inputs, const int *in_dts, const int64_t *in_row_strides,

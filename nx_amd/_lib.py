@@ -35,13 +35,18 @@ if not os.path.exists(LIB_PATH):
 
 lib = C.CDLL(LIB_PATH)
 
+class _Imm(C.Union):
+    _fields_ = [("f", C.c_float), ("bits", C.c_uint32)]
+
+
 class FusedInstr(C.Structure):
-    """hipnx_fused_instr of include/hipnx.h."""
+    """hipnx_fused_instr of include/hipnx.h (imm / imm2 as a float or as raw bits)."""
     _fields_ = [("kind", C.c_uint8), ("op", C.c_uint8), ("src", C.c_uint8), ("arg", C.c_uint8), ("src2", C.c_uint8),
-                ("arg2", C.c_uint8), ("flags", C.c_uint8), ("dt", C.c_uint8), ("imm", C.c_float), ("imm2", C.c_float)]
+                ("arg2", C.c_uint8), ("flags", C.c_uint8), ("dt", C.c_uint8), ("imm", _Imm), ("imm2", _Imm)]
 
 
-FUSED_SET, FUSED_UNARY, FUSED_BINARY, FUSED_SELECT, FUSED_AS_TYPE = range(5)
+FUSED_SET, FUSED_UNARY, FUSED_BINARY, FUSED_SELECT, FUSED_AS_TYPE, FUSED_BITCAST = range(6)
+FUSED_FLAG_SWAP, FUSED_FLAG_INT = 1, 2
 FUSED_SRC_CONST, FUSED_SRC_INPUT, FUSED_SRC_SAVED = range(3)
 FUSED_SAVED, FUSED_MAX_INSTR, FUSED_MAX_INPUTS = 3, 32, 8
 FUSED_INTERPRETED, FUSED_COMPILED = 0, 1

@@ -750,14 +750,22 @@ class HipNxBackend:
         return Tensor(cls(ref, backend_opts["device"]), ty, tuple(shape), tuple(opts.get("names") or ()))
 
     @classmethod
-    def fused_elementwise(cls, out: Tensor, program, inputs, layout, reduce_op: int = -1) -> Tensor:
+    def fused_elementwise(cls, out: Tensor, program, inputs, layout, reduce_op: int = -1, mode=None) -> Tensor:
         """A group of element-wise nodes in one kernel (the evaluator offers it groups it has found
         in a traced function).  `program` is a list of dicts with the fields of `hipnx_fused_instr`
         (`dt` as a type tuple); `layout` is (rows, cols, [(row_stride, col_stride) per input]).
         `reduce_op` (RED_SUM / RED_MAX / RED_MIN) reduces the group's value along its rows without
         storing it; `out` is then the reduction's template.  Raises HipNxError with status
-        EUNSUPPORTED when the shapes do not fit the kernel: the caller then runs the nodes one by one."""
+        EUNSUPPORTED when the shapes do not fit the kernel: the caller then runs the nodes one by one.
+        `mode` ("interpreted" / "compiled") runs this call in that mode whatever the device is set to."""
         dev = cls._device_of(*inputs) if inputs else 0
+        previous = _fused_modes.get(dev, "interpreted")
+        if mode is not None and previous != mode:
+            fused_mode(mode, dev)
+            try:
+                return cls.fused_elementwise(out, program, inputs, layout, reduce_op)
+            finally:
+                fused_mode(previous, dev)
         inputs = [cls._from_nx(t, dev) for t in inputs]
         rows, cols, strides = layout
         prog = getattr(program, "packed", None)
@@ -766,7 +774,9 @@ class HipNxBackend:
             for q, ins in zip(prog, program):
                 q.kind, q.op, q.src, q.arg = ins["kind"], ins.get("op", 0), ins.get("src", 0), ins.get("arg", 0)
                 q.src2, q.arg2, q.flags, q.dt = ins.get("src2", 0), ins.get("arg2", 0), ins.get("flags", 0), T.code(ins["dt"])
-                q.imm, q.imm2 = ins.get("imm", 0.0), ins.get("imm2", 0.0)
+                q.imm.f, q.imm2.f = ins.get("imm", 0.0), ins.get("imm2", 0.0)
+                if "imm_bits" in ins:  # the constant of an integer instruction, as the bits it is
+                    q.imm.bits = ins["imm_bits"]
             try:
                 program.packed = prog  # a caller's list type with room for the packed form keeps it
             except AttributeError:
@@ -904,6 +914,10 @@ def fused_mode(mode: str, device: int = 0) -> None:
     if mode not in codes:
         raise ValueError(f"expected one of {sorted(codes)!r}, got: {mode!r}")
     L.check(L.lib.hipnx_fused_set_mode(_Context.get(device), codes[mode]))
+    _fused_modes[device] = mode
+
+
+_fused_modes = {}  # device -> the mode last set here
 
 
 def fused_compiled_count(device: int = 0) -> int:

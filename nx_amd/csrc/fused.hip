@@ -130,6 +130,7 @@ struct RunInterpreted {
     run_program<FULL>(a, a->n_instr, row, col, acc);
   }
   static __device__ __forceinline__ int out_dt(KernArgs a) { return a->out_dt; }
+  static constexpr bool raw_out = false;
 };
 
 template <bool FULL>
@@ -174,14 +175,17 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
   if (n_inputs < 0 || n_inputs > HIPNX_FUSED_MAX_INPUTS || (n_inputs > 0 && (!inputs || !in_dts || !in_row_strides || !in_col_strides)))
     return set_error(HIPNX_EINVAL, "fused: 0 .. %d inputs", HIPNX_FUSED_MAX_INPUTS);
   if (rows < 0 || cols < 0) return set_error(HIPNX_EINVAL, "fused: negative extent");
-  if (!narrow(out_dt) && out_dt != HIPNX_U8) return set_error(HIPNX_EUNSUPPORTED, "fused: result type %d", out_dt);
+  const bool int_out = out_dt == HIPNX_U32 || out_dt == HIPNX_S32;
+  if (!narrow(out_dt) && out_dt != HIPNX_U8 && !int_out) return set_error(HIPNX_EUNSUPPORTED, "fused: result type %d", out_dt);
   if (reduce_op != -1 && reduce_op != HIPNX_RED_SUM && reduce_op != HIPNX_RED_MAX && reduce_op != HIPNX_RED_MIN)
     return set_error(HIPNX_EUNSUPPORTED, "fused: reduction %d (sum, max and min along the rows are built)", reduce_op);
   FusedArgs a{};
   a.n_instr = n_instr;
   a.n_inputs = n_inputs;
   unsigned saved = 0;  // slots that hold a value so far
-  bool have_acc = false, full = false;
+  unsigned raw_inputs = 0;  // inputs whose words are loaded unconverted
+  bool have_acc = false, full = false, needs_compiled = false;
+  auto int32 = [](int dt) { return dt == HIPNX_U32 || dt == HIPNX_S32; };
   auto source_ok = [&](int src, int arg, const char **why) {
     if (src == HIPNX_FUSED_SRC_INPUT && arg >= n_inputs) { *why = "reads an input that is not there"; return false; }
     if (src == HIPNX_FUSED_SRC_SAVED && (arg >= HIPNX_FUSED_SAVED || !(saved >> arg & 1))) { *why = "reads an empty slot"; return false; }
@@ -191,27 +195,48 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
   for (int i = 0; i < n_instr; i++) {
     const hipnx_fused_instr &q = prog[i];
     const char *why = nullptr;
-    if (!narrow(q.dt) && q.dt != HIPNX_U8) return set_error(HIPNX_EUNSUPPORTED, "fused: instruction %d has result type %d", i, q.dt);
+    const bool ints = (q.flags & HIPNX_FUSED_FLAG_INT) != 0;
+    needs_compiled |= ints || q.kind == HIPNX_FUSED_BITCAST;
+    if (ints && q.kind != HIPNX_FUSED_AS_TYPE && q.kind != HIPNX_FUSED_SET && !int32(q.dt))
+      return set_error(HIPNX_EINVAL, "fused: integer instruction %d has result type %d", i, q.dt);
+    if (!narrow(q.dt) && q.dt != HIPNX_U8 && !((ints || q.kind == HIPNX_FUSED_BITCAST) && int32(q.dt)))
+      return set_error(HIPNX_EUNSUPPORTED, "fused: instruction %d has result type %d", i, q.dt);
     if (q.kind != HIPNX_FUSED_SET && !have_acc) return set_error(HIPNX_EINVAL, "fused: instruction %d uses the accumulator before anything set it", i);
     switch (q.kind) {
       case HIPNX_FUSED_SET:
         if (!source_ok(q.src, q.arg, &why)) return set_error(HIPNX_EINVAL, "fused: instruction %d %s", i, why);
+        if (ints && q.src == HIPNX_FUSED_SRC_INPUT) raw_inputs |= 1u << q.arg;
         break;
       case HIPNX_FUSED_UNARY:
+        if (ints) {
+          if (q.op != HIPNX_NEGATE && q.op != HIPNX_BITWISE_NOT) return set_error(HIPNX_EUNSUPPORTED, "fused: integer unary op %d", q.op);
+          break;
+        }
         if (q.op >= HIPNX_NUNARY || q.op == HIPNX_BITWISE_NOT || q.op == HIPNX_CLZ || q.op == HIPNX_POPCOUNT)
           return set_error(HIPNX_EUNSUPPORTED, "fused: unary op %d", q.op);
         full |= !unary_light(q.op);
         break;
       case HIPNX_FUSED_BINARY:
-        if (q.op >= HIPNX_NBINARY || binary_int_only(q.op)) return set_error(HIPNX_EUNSUPPORTED, "fused: binary op %d", q.op);
         if (!source_ok(q.src, q.arg, &why)) return set_error(HIPNX_EINVAL, "fused: instruction %d %s", i, why);
+        if (ints) {
+          if (q.op != HIPNX_ADD && q.op != HIPNX_SUBTRACT && q.op != HIPNX_MULTIPLY && q.op != HIPNX_MIN && q.op != HIPNX_MAX &&
+              q.op != HIPNX_BITWISE_AND && q.op != HIPNX_BITWISE_OR && q.op != HIPNX_BITWISE_XOR &&
+              q.op != HIPNX_LEFT_SHIFT && q.op != HIPNX_RIGHT_SHIFT)
+            return set_error(HIPNX_EUNSUPPORTED, "fused: integer binary op %d", q.op);
+          if (q.src == HIPNX_FUSED_SRC_INPUT) raw_inputs |= 1u << q.arg;
+          break;
+        }
+        if (q.op >= HIPNX_NBINARY || binary_int_only(q.op)) return set_error(HIPNX_EUNSUPPORTED, "fused: binary op %d", q.op);
         full |= !binary_light(q.op);
         break;
+      case HIPNX_FUSED_BITCAST: break;
       case HIPNX_FUSED_SELECT:
         if (!source_ok(q.src, q.arg, &why) || !source_ok(q.src2, q.arg2, &why))
           return set_error(HIPNX_EINVAL, "fused: instruction %d %s", i, why);
         break;
-      case HIPNX_FUSED_AS_TYPE: break;
+      case HIPNX_FUSED_AS_TYPE:
+        if (ints && (!int32(q.op) || !narrow(q.dt))) return set_error(HIPNX_EINVAL, "fused: instruction %d converts type %d to %d", i, q.op, q.dt);
+        break;
       default: return set_error(HIPNX_EINVAL, "fused: instruction %d has kind %d", i, q.kind);
     }
     have_acc = true;
@@ -221,12 +246,16 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
     }
     a.ins[i] = q;
   }
+  if (int_out != int32(prog[n_instr - 1].dt)) return set_error(HIPNX_EINVAL, "fused: result type %d after a program that ends in type %d", out_dt, prog[n_instr - 1].dt);
+  if (needs_compiled && ctx->fused_mode != HIPNX_FUSED_COMPILED)
+    return set_error(HIPNX_EUNSUPPORTED, "fused: 32-bit integer instructions need the compiled mode");
   const int64_t n = rows * cols;
   if (cols % 8 != 0) return set_error(HIPNX_EUNSUPPORTED, "fused: the row length is not a multiple of 8");
   for (int k = 0; k < n_inputs; k++) {
     const int dt = in_dts[k];
     const int sz = dtype_size(dt);
     if (sz < 0 || sz > 4) return set_error(HIPNX_EUNSUPPORTED, "fused: input %d has type %d", k, dt);
+    if ((raw_inputs >> k & 1) && sz != 4) return set_error(HIPNX_EINVAL, "fused: input %d of type %d is read as 32-bit words", k, dt);
     if (in_row_strides[k] < 0 || (in_col_strides[k] != 0 && in_col_strides[k] != 1))
       return set_error(HIPNX_EINVAL, "fused: input %d has strides (%lld, %d)", k, (long long)in_row_strides[k], in_col_strides[k]);
     // rows of an operand read with vector loads must start on a vector boundary
@@ -264,6 +293,7 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
     if (int st = fused_launch_compiled(ctx, a, reduce_op, block_per_row, (unsigned)grid, &done)) return st;
     if (done) return HIPNX_OK;
   }
+  if (needs_compiled) return set_error(HIPNX_EUNSUPPORTED, "fused: a program with 32-bit integer instructions first met while capturing");
   if (reduce_op == HIPNX_RED_SUM) launch_fused_reduce<PlainReducer<double, HIPNX_RED_SUM, false>, double>(ctx, a);
   else if (reduce_op == HIPNX_RED_MAX) launch_fused_reduce<PlainReducer<float, HIPNX_RED_MAX, false>, float>(ctx, a);
   else if (reduce_op == HIPNX_RED_MIN) launch_fused_reduce<PlainReducer<float, HIPNX_RED_MIN, false>, float>(ctx, a);

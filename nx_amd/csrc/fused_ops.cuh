@@ -144,10 +144,11 @@ struct Saved {
 // dt[], imm[] and imm2[] as f32 bit patterns), the inputs' element types and column strides, and
 // the result type.  Every branch the interpreter takes on an instruction field is taken by the
 // compiler here.
-template <typename P, int SRC, int ARG, unsigned IMM>
+template <typename P, int SRC, int ARG, unsigned IMM, bool RAW>
 __device__ __forceinline__ void fetch_static(KernArgs a, const Saved &S, const int64_t (&row)[FV], const int64_t (&col)[FV], Vecs &dst) {
   if constexpr (SRC == HIPNX_FUSED_SRC_INPUT) {
-    load_input_as(a, ARG, P::in_dt[ARG], P::in_cs[ARG], row, col, dst);
+    // RAW: the words of a 4-byte input as they are (what the f32 path does with its bits)
+    load_input_as(a, ARG, RAW ? (int)HIPNX_F32 : P::in_dt[ARG], P::in_cs[ARG], row, col, dst);
   } else if constexpr (SRC == HIPNX_FUSED_SRC_SAVED) {
     copy_vecs(dst, S.s[ARG]);
   } else {
@@ -158,29 +159,64 @@ __device__ __forceinline__ void fetch_static(KernArgs a, const Saved &S, const i
   }
 }
 
+// 32-bit integers travel through the lane's vectors as raw bits; an operation on them widens to
+// the 64-bit integer class of the separate kernels and keeps the low word, as their stores do
+template <int OP, bool UNS>
+__device__ __forceinline__ float int_binary(float x, float y, bool swap) {
+  const uint32_t a = __float_as_uint(swap ? y : x), b = __float_as_uint(swap ? x : y);
+  const int64_t wa = UNS ? (int64_t)a : (int64_t)(int32_t)a, wb = UNS ? (int64_t)b : (int64_t)(int32_t)b;
+  return __uint_as_float((uint32_t)binary_apply<OP, int64_t, UNS>(wa, wb));
+}
+
+template <int OP, bool UNS>
+__device__ __forceinline__ float int_unary(float x) {
+  const uint32_t a = __float_as_uint(x);
+  return __uint_as_float((uint32_t)unary_apply<OP, int64_t>(UNS ? (int64_t)a : (int64_t)(int32_t)a, 32));
+}
+
 template <typename P, int PC>
 __device__ __forceinline__ void static_steps(KernArgs a, const int64_t (&row)[FV], const int64_t (&col)[FV], Vecs &acc, Saved &S) {
   if constexpr (PC < P::n_instr) {
     constexpr int kind = P::kind[PC], op = P::op[PC], src = P::src[PC], arg = P::arg[PC];
     constexpr int src2 = P::src2[PC], arg2 = P::arg2[PC], flags = P::flags[PC], dt = P::dt[PC];
     constexpr unsigned imm = P::imm[PC], imm2 = P::imm2[PC];
+    constexpr bool ints = (flags & HIPNX_FUSED_FLAG_INT) != 0, uns = dt == HIPNX_U32;
     if constexpr (kind == HIPNX_FUSED_SET) {
-      fetch_static<P, src, arg, imm>(a, S, row, col, acc);
+      fetch_static<P, src, arg, imm, ints>(a, S, row, col, acc);
     } else if constexpr (kind == HIPNX_FUSED_UNARY) {
-      unary_vecs<op>(acc);
+      if constexpr (ints) {
+#pragma unroll
+        for (int u = 0; u < FV; u++)
+#pragma unroll
+          for (int e = 0; e < FE; e++) acc[u][e] = int_unary<op, uns>(acc[u][e]);
+      } else {
+        unary_vecs<op>(acc);
+      }
     } else if constexpr (kind == HIPNX_FUSED_BINARY) {
       Vecs y;
-      fetch_static<P, src, arg, imm>(a, S, row, col, y);
-      binary_vecs<op>(acc, y, (flags & 1) != 0);
+      fetch_static<P, src, arg, imm, ints>(a, S, row, col, y);
+      if constexpr (ints) {
+#pragma unroll
+        for (int u = 0; u < FV; u++)
+#pragma unroll
+          for (int e = 0; e < FE; e++) acc[u][e] = int_binary<op, uns>(acc[u][e], y[u][e], (flags & 1) != 0);
+      } else {
+        binary_vecs<op>(acc, y, (flags & 1) != 0);
+      }
     } else if constexpr (kind == HIPNX_FUSED_SELECT) {
       Vecs y, z;
-      fetch_static<P, src, arg, imm>(a, S, row, col, y);
-      fetch_static<P, src2, arg2, imm2>(a, S, row, col, z);
+      fetch_static<P, src, arg, imm, false>(a, S, row, col, y);
+      fetch_static<P, src2, arg2, imm2, false>(a, S, row, col, z);
 #pragma unroll
       for (int u = 0; u < FV; u++)
 #pragma unroll
         for (int e = 0; e < FE; e++) acc[u][e] = acc[u][e] != 0.0f ? y[u][e] : z[u][e];  // NaN is true
-    }
+    } else if constexpr (kind == HIPNX_FUSED_AS_TYPE && ints) {  // the integer of type `op`, held as bits, to a float
+#pragma unroll
+      for (int u = 0; u < FV; u++)
+#pragma unroll
+        for (int e = 0; e < FE; e++) acc[u][e] = element_to_f32(__float_as_uint(acc[u][e]), op);
+    }  // a float AS_TYPE is the rounding below; a BITCAST changes nothing in the registers
     if constexpr (dt == HIPNX_BF16 || dt == HIPNX_F16) {
 #pragma unroll
       for (int u = 0; u < FV; u++)
@@ -198,7 +234,9 @@ struct RunStatic {
     Saved S;
     static_steps<P, 0>(a, row, col, acc, S);
   }
+  // a u32 / s32 result leaves as the bits it is held as
   static __device__ __forceinline__ int out_dt(KernArgs) { return P::out_dt; }
+  static constexpr bool raw_out = P::out_dt == HIPNX_U32 || P::out_dt == HIPNX_S32;
 };
 
 // ---- kernel bodies: RUN is RunStatic<P> or the interpreter of fused.hip ---------------------------
@@ -227,8 +265,16 @@ __device__ __forceinline__ void fused_elementwise_body() {
     void *out = (void *)a->out;
     const int odt = RUN::out_dt(a);
 #pragma unroll
-    for (int u = 0; u < FV; u++)
-      if (live[u]) store_vec<float, FE>(out, odt, row[u] * cols + col[u], acc[u]);
+    for (int u = 0; u < FV; u++) {
+      if (!live[u]) continue;
+      if constexpr (RUN::raw_out) {
+        uint4 *p = reinterpret_cast<uint4 *>((uint32_t *)out + row[u] * cols + col[u]);
+        p[0] = make_uint4(__float_as_uint(acc[u][0]), __float_as_uint(acc[u][1]), __float_as_uint(acc[u][2]), __float_as_uint(acc[u][3]));
+        p[1] = make_uint4(__float_as_uint(acc[u][4]), __float_as_uint(acc[u][5]), __float_as_uint(acc[u][6]), __float_as_uint(acc[u][7]));
+      } else {
+        store_vec<float, FE>(out, odt, row[u] * cols + col[u], acc[u]);
+      }
+    }
   }
 }
 

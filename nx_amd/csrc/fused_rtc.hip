@@ -45,12 +45,6 @@ static void list_of(std::string &s, const char *name, const char *type, int n, c
   s += "};\n";
 }
 
-static std::string bits_of(float x) {
-  uint32_t u;
-  memcpy(&u, &x, 4);
-  return std::to_string(u) + "u";
-}
-
 // everything a compiled kernel is specialised on, as bytes: the cache key
 static std::string make_key(const FusedArgs &a, int reduce_op, bool block_per_row) {
   std::string k;
@@ -76,8 +70,8 @@ static std::string make_source(const FusedArgs &a, int reduce_op, bool block_per
   list_of(s, "arg2", "int", a.n_instr, [&](int i) { return std::to_string((int)q[i].arg2); });
   list_of(s, "flags", "int", a.n_instr, [&](int i) { return std::to_string((int)q[i].flags); });
   list_of(s, "dt", "int", a.n_instr, [&](int i) { return std::to_string((int)q[i].dt); });
-  list_of(s, "imm", "unsigned", a.n_instr, [&](int i) { return bits_of(q[i].imm); });
-  list_of(s, "imm2", "unsigned", a.n_instr, [&](int i) { return bits_of(q[i].imm2); });
+  list_of(s, "imm", "unsigned", a.n_instr, [&](int i) { return std::to_string(q[i].imm_bits) + "u"; });
+  list_of(s, "imm2", "unsigned", a.n_instr, [&](int i) { return std::to_string(q[i].imm2_bits) + "u"; });
   list_of(s, "in_dt", "int", a.n_inputs, [&](int k) { return std::to_string(a.in_dt[k]); });
   list_of(s, "in_cs", "int", a.n_inputs, [&](int k) { return std::to_string(a.in_cs[k]); });
   s += "};\n}\nusing namespace hipnx;\nextern \"C\" __global__ void __launch_bounds__(FBLOCK) fused_group(FusedArgs by_value) {\n  (void)by_value;\n";

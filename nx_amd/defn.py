@@ -450,6 +450,14 @@ _INT_ONLY_UNARY = ("bitwise_not", "count_leading_zeros", "population_count")
 _COMPARE = ("equal", "not_equal", "greater", "less", "greater_equal", "less_equal")
 _LOGICAL = ("logical_and", "logical_or", "logical_xor")
 _EXACT_WITH_INT_CONSTANT = ("add", "subtract", "multiply", "divide", "min", "max") + _COMPARE
+_INT32 = (("u", 32), ("s", 32))
+_WORD = _INT32 + (("f", 32),)
+# with `fuse="compiled"` a group may also compute on 32-bit integers (held as raw bits, wrapping like
+# the integer kernels) and relabel 32-bit values: what Nx.Random's bits-to-floats chains are made of
+_INT_FUSED_BINARY = ("add", "subtract", "multiply", "bitwise_and", "bitwise_or", "bitwise_xor", "left_shift",
+                     "right_shift", "min", "max")
+_INT_FUSED_UNARY = ("negate", "bitwise_not")
+_plan = {"ints": False}
 _SAVED_SLOTS, _MAX_INSTR, _MAX_INPUTS = 3, 32, 8
 _REDUCE_CODES = {"sum": 0, "reduce_max": 1, "reduce_min": 2}  # HIPNX_RED_SUM / MAX / MIN
 _EUNSUPPORTED = 7
@@ -460,6 +468,18 @@ def _fusable(t: Tensor) -> bool:
     result the fused kernel holds exactly."""
     e = t.data
     op, args = e.op, e.args
+    if _plan["ints"]:
+        if op in _INT_FUSED_BINARY and t.type in _INT32:
+            def word_ok(a):
+                if _const(a) is None:
+                    return a.type == t.type
+                c = _const(a)
+                return T.is_integer(a.type) and float(c).is_integer() and (a.type == t.type or 0 <= c < 1 << 31)
+            return all(word_ok(a) for a in args)
+        if op in _INT_FUSED_UNARY and t.type in _INT32:
+            return args[0].type == t.type and _const(args[0]) is None
+        if op == "bitcast":
+            return t.type in _WORD and args[0].type in _WORD and _const(args[0]) is None
 
     def value_ok(a, binary_op=None):
         if _const(a) is not None:
@@ -526,6 +546,8 @@ class _Group:
 
     def __init__(self, root: Tensor, members: List[Tensor], inputs: List[Tensor]):
         self.root, self.members, self.inputs = root, members, inputs
+        # planned for compiled execution (integer instructions allowed): ask the backend for that mode
+        self.how = {"mode": "compiled"} if _plan["ints"] else {}
         self.program = self._assemble()
         self.layout = _layout(root.shape, [t.shape for t in inputs]) if self.program else None
         self.reduce = None  # (callback name, opts, rows layout) when a reduction of the result is part of the group
@@ -563,13 +585,21 @@ class _Group:
         free = list(range(_SAVED_SLOTS))
         program: List[dict] = _Program()
 
-        def source(a):
-            """(src, arg, imm) of an operand that is not the accumulator."""
+        def source(a, raw=False):
+            """(src, arg, imm) of an operand that is not the accumulator; `raw`: for an integer
+            instruction (a constant is then the bits of the integer, marked by a str)."""
             if _const(a) is not None:
-                return 0, 0, _imm(a)
+                return 0, 0, (str(int(_const(a)) & 0xFFFFFFFF) if raw else _imm(a))
             if a.data.id in input_ids:
                 return 1, input_ids[a.data.id], 0.0
             return 2, slots[a.data.id], 0.0
+
+        def with_imm(ins, imm):
+            if isinstance(imm, str):
+                ins["imm_bits"] = int(imm)
+            else:
+                ins["imm"] = imm
+            return ins
 
         for i, m in enumerate(self.members):
             operands = [a for a in m.data.args if isinstance(a, Tensor)]
@@ -579,6 +609,10 @@ class _Group:
                 return prev is not None and _const(a) is None and a.data.id == prev
 
             op = m.data.op
+            ints = m.type in _INT32 and (op in _INT_FUSED_BINARY or op in _INT_FUSED_UNARY)
+            # an integer held as bits that a conversion reads (an integer *input* is converted as it is loaded)
+            from_bits = op == "as_type" and operands[0].type in _INT32 and operands[0].data.id in member_ids
+            raw = ints or op == "bitcast" or from_bits
             if op == "select":
                 want_acc = [0]           # the predicate
             elif op in BINARY_OPS:
@@ -591,21 +625,27 @@ class _Group:
                 first = operands[pos]
                 if first.data.id in member_ids and _const(first) is None and first.data.id not in slots:
                     return None          # cannot happen: a member read later than next is saved below
-                src, arg, imm = source(first)
-                program.append({"kind": 0, "src": src, "arg": arg, "imm": imm,
-                                "dt": first.type if first.type in _NARROW or first.type == _TRUTH else ("f", 32)})
+                src, arg, imm = source(first, raw)
+                keeps = first.type in _NARROW or first.type == _TRUTH or (raw and first.type in _INT32)
+                program.append(with_imm({"kind": 0, "src": src, "arg": arg, "flags": 2 if raw else 0,
+                                         "dt": first.type if keeps else ("f", 32)}, imm))
             others = [a for p, a in enumerate(operands) if p != pos]
             if any(_const(o) is None and o.data.id in member_ids and o.data.id not in slots for o in others):
                 return None              # an operand that is neither the accumulator nor saved: cannot happen
             ins = {"dt": m.type}
-            if op in UNARY_OPS:
-                ins.update(kind=1, op=UNARY_OPS.index(op))
+            if op == "bitcast":
+                ins.update(kind=5)
+            elif op in UNARY_OPS:
+                ins.update(kind=1, op=UNARY_OPS.index(op), flags=2 if ints else 0)
             elif op in BINARY_OPS:
-                src, arg, imm = source(others[0])
-                ins.update(kind=2, op=BINARY_OPS.index(op), src=src, arg=arg, imm=imm, flags=1 if pos == 1 else 0)
+                src, arg, imm = source(others[0], ints)
+                with_imm(ins, imm).update(kind=2, op=BINARY_OPS.index(op), src=src, arg=arg,
+                                          flags=(1 if pos == 1 else 0) | (2 if ints else 0))
             elif op == "select":
                 (s1, a1, i1), (s2, a2, i2) = source(others[0]), source(others[1])
                 ins.update(kind=3, src=s1, arg=a1, imm=i1, src2=s2, arg2=a2, imm2=i2)
+            elif from_bits:
+                ins.update(kind=4, op=T.code(operands[0].type), flags=2)
             else:
                 ins.update(kind=4)
             # slots whose value was read for the last time here are free again
@@ -641,7 +681,7 @@ class _Group:
             name, opts, rows_layout = self.reduce
             if fused is not None:
                 try:
-                    return fused(out, self.program, values, rows_layout, _REDUCE_CODES[name])
+                    return fused(out, self.program, values, rows_layout, _REDUCE_CODES[name], **self.how)
                 except Exception as e:  # a shape the kernel leaves to the separate reduction
                     if getattr(e, "status", None) != _EUNSUPPORTED:
                         raise
@@ -651,7 +691,11 @@ class _Group:
             value = plain.run(run, self.root.with_(data=None), values)
             return getattr(run.pick([value]), name)(out, value, opts)
         if fused is not None:
-            return fused(out, self.program, values, self.layout)
+            try:
+                return fused(out, self.program, values, self.layout, **self.how)
+            except Exception as e:  # e.g. integer instructions met while the device is capturing
+                if getattr(e, "status", None) != _EUNSUPPORTED:
+                    raise
         # node by node, on the callbacks (a backend without the kernel, or a group that does not fit)
         done = {t.data.id: v for t, v in zip(self.inputs, values)}
         for m in self.members:
@@ -675,9 +719,18 @@ def _imm(a: Tensor) -> float:
     return float(raw.astype(np.float32)[0])
 
 
-def _fuse(roots: List[Tensor]) -> int:
+def _fuse(roots: List[Tensor], ints: bool = False) -> int:
     """Rewrites element-wise groups of the root scope into `fused` nodes, in place; returns how
-    many groups were formed."""
+    many groups were formed.  `ints`: plan for groups that are compiled for the device, which may
+    compute on 32-bit integers and relabel bits as well."""
+    _plan["ints"] = ints
+    try:
+        return _fuse_planned(roots)
+    finally:
+        _plan["ints"] = False
+
+
+def _fuse_planned(roots: List[Tensor]) -> int:
     order, uses, seen = [], {}, set()
 
     def walk(t):
@@ -1087,7 +1140,7 @@ def _runtime_backend(params):
     return mod, opts
 
 
-def trace(fun: Callable, args, kwargs=None, fuse: bool = False) -> Compiled:
+def trace(fun: Callable, args, kwargs=None, fuse=False) -> Compiled:
     """Runs `fun` on parameter expressions shaped like `args` (compiler.ex:184-205: the default
     backend is the expression builder while the function runs)."""
     leaves: list = []
@@ -1108,13 +1161,15 @@ def trace(fun: Callable, args, kwargs=None, fuse: bool = False) -> Compiled:
         Nx.default_backend(*previous)
         _trace.scopes = []
         _trace.fold = None
-    compiled_groups = _fuse(roots) if fuse else 0
+    if fuse not in (False, True, "compiled"):
+        raise ValueError(f"fuse is False, True or \"compiled\", got: {fuse!r}")
+    compiled_groups = _fuse(roots, ints=fuse == "compiled") if fuse else 0
     compiled = Compiled(roots, out_structure, [t.with_(data=None) for t in templates])
     compiled.fused_groups = compiled_groups
     return compiled
 
 
-def jit(fun: Callable = None, fuse: bool = False, **static):
+def jit(fun: Callable = None, fuse=False, **static):
     """Nx.Defn.jit/2 with the default compiler: traces on every call, like the reference's
     evaluator (evaluator.ex:41-43), then evaluates.  Keyword arguments are static options; `fuse`
     hands groups of element-wise nodes to the backend as one kernel each."""
@@ -1127,6 +1182,6 @@ def jit(fun: Callable = None, fuse: bool = False, **static):
     return call
 
 
-def compile(fun: Callable, *templates, fuse: bool = False, **static) -> Compiled:  # noqa: A001 - Nx.Defn.compile/3
+def compile(fun: Callable, *templates, fuse=False, **static) -> Compiled:  # noqa: A001 - Nx.Defn.compile/3
     """Traces once for arguments shaped like `templates`; the result is called many times."""
     return trace(fun, templates, static, fuse=fuse)

@@ -410,3 +410,92 @@ def test_value_with_an_outside_reader_is_still_stored_once(hip):
     plain = defn.compile(fun, x)
     for got, want in zip(fused(x), plain(x)):
         assert_bits_equal(got, want, "shared with a dot")
+
+
+# ---- groups planned for compilation: 32-bit integer work and bit relabelling join in --------------------
+
+def bits_to_unit_floats(bits):
+    # the core of Nx.Random.uniform for f32 (random.ex:424-470): mantissa bits under the exponent of 1.0
+    mantissa = Nx.bitwise_or(Nx.right_shift(bits, 9), 0x3F800000)
+    return Nx.subtract(Nx.bitcast(mantissa, "f32"), 1.0)
+
+
+def integer_mix(a, b):
+    x = Nx.bitwise_xor(Nx.add(a, b), Nx.left_shift(a, 3))
+    return Nx.multiply(Nx.subtract(x, 7), Nx.bitwise_not(b))
+
+
+def signed_shift_and_convert(a, b):
+    x = Nx.max(Nx.right_shift(Nx.negate(a), 2), Nx.min(b, 1000))
+    return Nx.multiply(Nx.as_type(x, "f32"), 0.5)
+
+
+def floats_to_bits_and_back(x):
+    sign_cleared = Nx.bitwise_and(Nx.bitcast(x, "u32"), 0x7FFFFFFF)
+    return Nx.sqrt(Nx.bitcast(sign_cleared, "f32"))
+
+
+def rand_words(rng, ty, shape, backend):
+    info = np.iinfo(np.uint32 if ty == "u32" else np.int32)
+    return from_numpy(rng.integers(info.min, info.max, size=shape, dtype=info.dtype, endpoint=True), ty, backend)
+
+
+INT_CASES = {
+    "bits_to_unit_floats": (bits_to_unit_floats, lambda rng, b: (rand_words(rng, "u32", (64, 256), b),)),
+    "integer_mix_u32": (integer_mix, lambda rng, b: (rand_words(rng, "u32", (33, 128), b), rand_words(rng, "u32", (33, 128), b))),
+    "integer_mix_s32": (integer_mix, lambda rng, b: (rand_words(rng, "s32", (8, 4096), b), rand_words(rng, "s32", (4096,), b))),
+    "signed_shift_and_convert": (signed_shift_and_convert, lambda rng, b: (rand_words(rng, "s32", (40, 64), b), rand_words(rng, "s32", (40, 64), b))),
+    "floats_to_bits_and_back": (floats_to_bits_and_back, lambda rng, b: (rand_float(rng, "f32", (1000, 8), b),)),
+}
+
+
+@pytest.mark.parametrize("name", sorted(INT_CASES))
+def test_compiled_group_with_integer_work_is_bit_identical(name, hip):
+    from nx_amd.backend import fused_mode as set_mode
+    fun, make = INT_CASES[name]
+    args = make(np.random.default_rng(seed_of(name)), hip)
+    want = defn.compile(fun, *args)(*args)
+    fused = defn.compile(fun, *args, fuse="compiled")
+    assert fused.fused_groups == 1 and fused.roots[0].data.op == "fused"  # the whole function is one kernel
+    assert_bits_equal(fused(*args), want, name)
+    # planned without the integer class, the same function still agrees (float parts fuse, the rest runs node by node)
+    assert_bits_equal(defn.compile(fun, *args, fuse=True)(*args), want, name + " float-only plan")
+    set_mode("compiled")
+    try:
+        assert_bits_equal(fused(*args), want, name + " in compiled mode")
+    finally:
+        set_mode("interpreted")
+
+
+def test_integer_program_is_refused_by_the_interpreting_kernels(hip):
+    from nx_amd._lib import FUSED_BINARY, FUSED_SET, FUSED_SRC_CONST, FUSED_SRC_INPUT, HipNxError
+    x = rand_words(np.random.default_rng(4), "u32", (64,), hip)
+    program = [{"kind": FUSED_SET, "src": FUSED_SRC_INPUT, "arg": 0, "flags": 2, "dt": ("u", 32)},
+               {"kind": FUSED_BINARY, "op": 14, "src": FUSED_SRC_CONST, "imm_bits": 9, "flags": 2, "dt": ("u", 32)}]  # right_shift
+    with pytest.raises(HipNxError, match="need the compiled mode"):
+        hip.fused_elementwise(x.with_(data=None), program, [x], (1, 64, [(0, 1)]))
+    got = hip.fused_elementwise(x.with_(data=None), program, [x], (1, 64, [(0, 1)]), mode="compiled")
+    np.testing.assert_array_equal(hip.to_numpy(got), hip.to_numpy(x) >> 9)
+
+
+@pytest.mark.parametrize("name", ["uniform", "normal"])
+def test_random_floats_from_one_compiled_group(name, hip):
+    from nx_amd import random as Random
+    key = Random.key(99, backend=hip)
+    fun = {"uniform": lambda k: Random.uniform_split(k, -2.0, 3.0, shape=(64, 1024)),
+           "normal": lambda k: Random.normal_split(k, 1.0, 2.0, shape=(64, 1024))}[name]
+    want = defn.compile(fun, key)(key)
+    fused = defn.compile(fun, key, fuse="compiled")
+    assert_bits_equal(fused(key), want, name)
+    calls = []
+    original = hip.fused_elementwise.__func__
+
+    def counting(cls, *a, **k):
+        calls.append(1)
+        return original(cls, *a, **k)
+    hip.fused_elementwise = classmethod(counting)
+    try:
+        fused(key)
+    finally:
+        hip.fused_elementwise = classmethod(original)
+    assert len(calls) >= 1 and fused.fused_groups == 1  # everything after the cipher is one group
