@@ -18,6 +18,8 @@
 // Scope: operands and results in bf16 / f16 / f32 (the f32 compute class of elementwise_ops.cuh),
 // u8 truth values between comparisons / logical ops and select, and integer inputs of at most
 // 32 bits feeding an as_type (exact in f32 after one rounding, as the as_type kernel does it).
+// Programs with 32-bit integer instructions or bitcasts (flags bit 1, HIPNX_FUSED_BITCAST) exist only
+// compiled (fused_rtc.hip); the kernels here refuse them.
 // Bound by HBM: bytes(inputs) + bytes(out).
 #include "fused_ops.cuh"
 #include "internal.h"
