@@ -271,7 +271,9 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
     a.in_cs[k] = in_col_strides[k];
   }
   if (reduce_op != -1) {
-    if (full) return set_error(HIPNX_EUNSUPPORTED, "fused: a reduction after a program with pow, atan2, remainder, trigonometric or erf functions");
+    // the interpreting reduction kernels exist in the light instantiation only (registers); a compiled one holds just its own program
+    if (full && ctx->fused_mode != HIPNX_FUSED_COMPILED)
+      return set_error(HIPNX_EUNSUPPORTED, "fused: a reduction after a program with pow, atan2, remainder, trigonometric or erf functions");
     if (!narrow(prog[n_instr - 1].dt) || !narrow(out_dt)) return set_error(HIPNX_EUNSUPPORTED, "fused: a reduction of a non-float value");
     if (cols == 0) return set_error(HIPNX_EUNSUPPORTED, "fused: a reduction over an empty axis");
     // a few very long rows are split into segments by the separate reduction: not here
@@ -295,7 +297,8 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
     if (int st = fused_launch_compiled(ctx, a, reduce_op, block_per_row, (unsigned)grid, &done)) return st;
     if (done) return HIPNX_OK;
   }
-  if (needs_compiled) return set_error(HIPNX_EUNSUPPORTED, "fused: a program with 32-bit integer instructions first met while capturing");
+  if (needs_compiled || (full && reduce_op != -1))
+    return set_error(HIPNX_EUNSUPPORTED, "fused: a program that exists only compiled, first met while capturing");
   if (reduce_op == HIPNX_RED_SUM) launch_fused_reduce<PlainReducer<double, HIPNX_RED_SUM, false>, double>(ctx, a);
   else if (reduce_op == HIPNX_RED_MAX) launch_fused_reduce<PlainReducer<float, HIPNX_RED_MAX, false>, float>(ctx, a);
   else if (reduce_op == HIPNX_RED_MIN) launch_fused_reduce<PlainReducer<float, HIPNX_RED_MIN, false>, float>(ctx, a);

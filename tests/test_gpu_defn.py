@@ -341,7 +341,36 @@ def min_of_bf16(a, b):
     return Nx.reduce_min(Nx.as_type(Nx.add(a, b), "bf16"), axes=[1])
 
 
+def sum_of_sines(a, b):  # sin is outside the light instantiation of the interpreting kernels
+    return Nx.sum(Nx.sin(Nx.add(a, b)), axes=[1])
+
+
 REDUCED = {"sum_of_exp": sum_of_exp, "max_of_scaled": max_of_scaled, "min_of_bf16": min_of_bf16}
+
+
+def test_compiled_reduction_takes_any_float_program(hip):
+    from nx_amd.backend import fused_mode as set_mode
+    rng = np.random.default_rng(21)
+    args = (rand_float(rng, "f32", (96, 512), hip), rand_float(rng, "f32", (96, 512), hip))
+    want = defn.compile(sum_of_sines, *args)(*args)
+    fused = defn.compile(sum_of_sines, *args, fuse=True)
+    calls = []
+    original = hip.fused_elementwise.__func__
+
+    def counting(cls, *a, **k):
+        calls.append(a[4] if len(a) > 4 else k.get("reduce_op", -1))
+        return original(cls, *a, **k)
+    hip.fused_elementwise = classmethod(counting)
+    try:
+        assert_bits_equal(fused(*args), want, "interpreted: the group, then the separate reduction")
+        assert calls == [0, -1]  # offered with the reduction, refused, run without it
+        del calls[:]
+        set_mode("compiled")
+        assert_bits_equal(fused(*args), want, "compiled: one kernel")
+        assert calls == [0]
+    finally:
+        set_mode("interpreted")
+        hip.fused_elementwise = classmethod(original)
 
 
 @pytest.mark.parametrize("name", sorted(REDUCED))
