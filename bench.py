@@ -277,6 +277,8 @@ def main():
             _, ms = timed(lambda: captured(*held), steps, warm)
             entry(name + "_graph", nbytes, "GB/s", ms, PEAK_HBM_GBS, "hbm")
             captured.destroy()
+            # (for configuration 4 the planner also finishes the layer on the dot's accumulators: dot, as_type and
+            # the multiplication by the scales are one kernel)
             # element-wise groups (with the row reduction that follows them) as one kernel each: decoded by
             # the interpreting kernels, then with each group's program compiled for the device on first use
             fused = defn.compile(fun, *targs, fuse=True)

@@ -180,6 +180,19 @@ int hipnx_dot(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batch, int
               int64_t K, int l_layout, int r_layout, const hipnx_buf *l, const hipnx_buf *r,
               hipnx_buf *out);
 
+/* replaces: the three callbacks of a quantised linear layer in one -- dot/7 with an s32 result, as_type/2
+ * to f32 and multiply/3 by the scales (nx/lib/nx/backend.ex:77, 68, 115), i.e.
+ * Nx.multiply(Nx.as_type(Nx.dot(x, w), :f32), scales) on s8 operands.  out[b, m, n] (f32) =
+ * (float)(sum_k l[b, m, k] * r[b, n, k] as s32) * scale, where scale (f32) is scale[n]
+ * (HIPNX_SCALE_PER_COLUMN), scale[m] (PER_ROW, batch = 1) or scale[0] (ONE): the conversion and the product
+ * are done on the accumulators and round exactly as the separate kernels do, so the result is
+ * bit-identical to the three calls.  s8 x s8 on the matrix-core kernels only (K <= 65536, K a multiple of
+ * 128); anything else is HIPNX_EUNSUPPORTED: make the three calls. */
+enum { HIPNX_SCALE_NONE = 0, HIPNX_SCALE_PER_COLUMN = 1, HIPNX_SCALE_PER_ROW = 2, HIPNX_SCALE_ONE = 3 };
+int hipnx_dot_scaled(hipnx_ctx *ctx, int l_dt, int r_dt, int64_t batch, int64_t M, int64_t N, int64_t K,
+                     int l_layout, int r_layout, const hipnx_buf *l, const hipnx_buf *r, int scale_mode,
+                     const hipnx_buf *scale, hipnx_buf *out);
+
 /* ---- data movement -------------------------------------------------------------------------
  * replaces: transpose/3 (nx/lib/nx/backend.ex:73; oracle binary_backend.ex:280-319) */
 int hipnx_transpose(hipnx_ctx *ctx, int elem_bytes, int rank, const int64_t *in_dims,

@@ -50,6 +50,7 @@ FUSED_FLAG_SWAP, FUSED_FLAG_INT = 1, 2
 FUSED_SRC_CONST, FUSED_SRC_INPUT, FUSED_SRC_SAVED = range(3)
 FUSED_SAVED, FUSED_MAX_INSTR, FUSED_MAX_INPUTS = 3, 32, 8
 FUSED_INTERPRETED, FUSED_COMPILED = 0, 1
+SCALE_NONE, SCALE_PER_COLUMN, SCALE_PER_ROW, SCALE_ONE = range(4)
 
 _ctx_p, _buf_p = C.c_void_p, C.c_void_p
 _i64p, _intp = C.POINTER(C.c_int64), C.POINTER(C.c_int)
@@ -83,6 +84,8 @@ PROTOTYPES = {
     "hipnx_argreduce": [_ctx_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int64, C.c_int64, C.c_int64, _buf_p, _buf_p],
     "hipnx_dot": [_ctx_p, C.c_int, C.c_int, C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_int,
                   _buf_p, _buf_p, _buf_p],
+    "hipnx_dot_scaled": [_ctx_p, C.c_int, C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_int,
+                         _buf_p, _buf_p, C.c_int, _buf_p, _buf_p],
     "hipnx_transpose": [_ctx_p, C.c_int, C.c_int, _i64p, _intp, _buf_p, _buf_p],
     "hipnx_broadcast": [_ctx_p, C.c_int, C.c_int, _i64p, _i64p, _buf_p, _buf_p],
     "hipnx_gather": [_ctx_p, C.c_int, C.c_int, _i64p, C.c_int, C.c_int64, C.c_int, C.c_int, _buf_p, _buf_p, _buf_p],

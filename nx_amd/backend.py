@@ -461,6 +461,29 @@ class HipNxBackend:
 
     # ---- data movement ---------------------------------------------------------------------
     @classmethod
+    def dot_scaled(cls, out: Tensor, l: Tensor, c1, b1, r: Tensor, c2, b2, scale: Tensor, mode: int) -> Tensor:
+        """`multiply(as_type(dot(l, r) with an s32 result, f32), scale)` in one kernel: the quantised
+        linear layer (the evaluator offers it when it finds that chain; backend.ex:77, 68, 115).
+        `mode`: SCALE_PER_COLUMN (one scale per entry of the right operand's free axes), SCALE_PER_ROW
+        or SCALE_ONE.  Raises HipNxError with status EUNSUPPORTED for what the kernel does not take:
+        the caller then makes the three calls."""
+        if l.type != ("s", 8) or r.type != ("s", 8) or scale.type != ("f", 32) or out.type != ("f", 32):
+            raise L.HipNxError(L.EUNSUPPORTED, "dot_scaled: s8 operands, f32 scales and result")
+        dev = cls._device_of(l, r, scale)
+        l, r, scale = cls._from_nx(l, dev), cls._from_nx(r, dev), cls._from_nx(scale, dev)
+        pairs = sorted(zip(c1, c2))
+        c1s, c2s = [p[0] for p in pairs], [p[1] for p in pairs]
+        nb = len(b1)
+        K = prod(l.shape[a] for a in c1s)
+        batch = prod(l.shape[a] for a in b1)
+        lt, l_layout, M = cls._dot_operand(l, c1s, nb)
+        rt, r_layout, N = cls._dot_operand(r, c2s, nb)
+        res = cls._alloc(out, dev)
+        L.check(L.lib.hipnx_dot_scaled(res.data.ref.ctx, T.code(l.type), T.code(r.type), batch, M, N, K, l_layout, r_layout,
+                                       cls._handle(lt), cls._handle(rt), mode, cls._handle(scale), res.data.ref.handle))
+        return res
+
+    @classmethod
     def transpose(cls, out: Tensor, t: Tensor, axes) -> Tensor:
         """transpose/3 (backend.ex:73; oracle binary_backend.ex:280-306)."""
         dev = cls._device_of(t)

@@ -165,9 +165,10 @@ using namespace hipnx;
 extern "C" int hipnx_transpose(hipnx_ctx *ctx, int elem_bytes, int rank, const int64_t *in_dims, const int *perm,
                                const hipnx_buf *inb, hipnx_buf *out);
 
-extern "C" int hipnx_dot(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batch, int64_t M, int64_t N,
-                         int64_t K, int l_layout, int r_layout, const hipnx_buf *l, const hipnx_buf *r,
-                         hipnx_buf *out) {
+// scale_mode != NONE: the scaled form (out_dt is then f32 over an s32 sum)
+static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batch, int64_t M, int64_t N,
+                    int64_t K, int l_layout, int r_layout, const hipnx_buf *l, const hipnx_buf *r,
+                    hipnx_buf *out, int scale_mode, const hipnx_buf *scale) {
   int64_t Kb = 0;
   bool mfma = false;
   {
@@ -186,8 +187,15 @@ extern "C" int hipnx_dot(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t
 
     Kb = K * dtype_size(l_dt);
     const bool float_pair = l_dt == r_dt && (l_dt == HIPNX_BF16 || l_dt == HIPNX_F16 || l_dt == HIPNX_F32) && is_float(out_dt);
-    const bool int8_pair = l_dt == HIPNX_S8 && r_dt == HIPNX_S8 && !is_float(out_dt) && K <= (1ll << 16);
+    const bool scaled = scale_mode != HIPNX_SCALE_NONE;
+    const bool int8_pair = l_dt == HIPNX_S8 && r_dt == HIPNX_S8 && (scaled || !is_float(out_dt)) && K <= (1ll << 16);
     mfma = (float_pair || int8_pair) && K > 0 && Kb % 16 == 0 && M * N >= 256;
+    if (scaled) {
+      if (!(int8_pair && mfma && Kb % SLAB == 0)) return set_error(HIPNX_EUNSUPPORTED, "dot_scaled: s8 x s8 with K a multiple of 128 and at most 65536, M * N >= 256");
+      if (scale_mode == HIPNX_SCALE_PER_ROW && batch != 1) return set_error(HIPNX_EUNSUPPORTED, "dot_scaled: a scale per row with more than one batch item");
+      const int64_t need = scale_mode == HIPNX_SCALE_PER_COLUMN ? N : scale_mode == HIPNX_SCALE_PER_ROW ? M : 1;
+      if (int st = check_buf(ctx, scale, (uint64_t)need * 4, "dot_scaled scale")) return st;
+    }
 
     if (!mfma) {
       const bool any_float = is_float(l_dt) || is_float(r_dt);
@@ -246,6 +254,8 @@ extern "C" int hipnx_dot(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t
         a.ld_r = r_kin ? Kb : N * esz;
         a.bs_l = M * Kb;
         a.bs_r = N * Kb;
+        a.scale = scale_mode != HIPNX_SCALE_NONE ? (const float *)scale->ptr : nullptr;
+        a.scale_mode = scale_mode;
         // tile choice: the largest tile that still gives every CU work; few rows against a long
         // weight matrix stream the weights with many small tiles
         const int64_t t256 = ((M + 255) / 256) * ((N + 255) / 256) * batch;
@@ -278,4 +288,18 @@ extern "C" int hipnx_dot(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t
   if (lt) hipnx_buf_destroy(lt);
   if (rt) hipnx_buf_destroy(rt);
   return st;
+}
+
+extern "C" int hipnx_dot(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batch, int64_t M, int64_t N,
+                         int64_t K, int l_layout, int r_layout, const hipnx_buf *l, const hipnx_buf *r,
+                         hipnx_buf *out) {
+  return dot_impl(ctx, l_dt, r_dt, out_dt, batch, M, N, K, l_layout, r_layout, l, r, out, HIPNX_SCALE_NONE, nullptr);
+}
+
+extern "C" int hipnx_dot_scaled(hipnx_ctx *ctx, int l_dt, int r_dt, int64_t batch, int64_t M, int64_t N, int64_t K,
+                                int l_layout, int r_layout, const hipnx_buf *l, const hipnx_buf *r, int scale_mode,
+                                const hipnx_buf *scale, hipnx_buf *out) {
+  if (scale_mode != HIPNX_SCALE_PER_COLUMN && scale_mode != HIPNX_SCALE_PER_ROW && scale_mode != HIPNX_SCALE_ONE)
+    return set_error(HIPNX_EINVAL, "dot_scaled: scale mode %d", scale_mode);
+  return dot_impl(ctx, l_dt, r_dt, HIPNX_F32, batch, M, N, K, l_layout, r_layout, l, r, out, scale_mode, scale);
 }

@@ -351,6 +351,10 @@ struct GemmArgs {
   int64_t bs_l, bs_r;    // bytes between batch items
   int tiles_m, tiles_n;
   int group_m;  // tile rows per group of the tile order (see gemm_group_m)
+  // s8 x s8 with an f32 output: out = (float)(the s32 sum) * scale -- the conversion and the
+  // multiplication that follow the contraction of a quantised linear layer, done on the accumulators
+  const float *scale;
+  int scale_mode;  // HIPNX_SCALE_NONE / PER_COLUMN (scale[n]) / PER_ROW (scale[m]) / ONE (scale[0])
 };
 
 // Epilogue of one wave: for 16x16 tile (i, j) a lane holds m = 16*i + lane%16 and
@@ -359,10 +363,40 @@ struct GemmArgs {
 // addressed dynamically, or they leave the register file).
 template <int DT, int ODT, int TM, int TN>
 __device__ __forceinline__ void gemm_epilogue(typename Mma16<DT>::acc_t (&acc)[TM][TN], void *out, int64_t obase,
-                                              int64_t M, int64_t N, int64_t row0, int64_t col0, int lane) {
+                                              int64_t M, int64_t N, int64_t row0, int64_t col0, int lane,
+                                              const float *scale = nullptr, int scale_mode = 0) {
   constexpr bool int_acc = DT == HIPNX_S8;
   constexpr bool int_out = ODT < HIPNX_F16;
-  if constexpr (int_acc != int_out) return;  // the host never pairs them
+  if constexpr (int_acc && ODT == HIPNX_F32) {
+    // as_type(s32 -> f32) then multiply, each rounding once, as the two separate kernels would
+    if (scale_mode == HIPNX_SCALE_NONE) return;  // the host pairs them only with a scale
+    const bool vec_ok = (N % 4) == 0;
+    const float one = scale_mode == HIPNX_SCALE_ONE ? scale[0] : 0.0f;
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+      const int64_t gm = row0 + 16 * i + (lane & 15);
+      const float per_row = scale_mode == HIPNX_SCALE_PER_ROW && gm < M ? scale[gm] : one;
+#pragma unroll
+      for (int j = 0; j < TN; j++) {
+        const int64_t gn = col0 + 16 * j + 4 * (lane >> 4);
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const float sc = scale_mode == HIPNX_SCALE_PER_COLUMN ? (gn + e < N ? scale[gn + e] : 0.0f) : per_row;
+          v[e] = (float)(int32_t)acc[i][j][e] * sc;
+        }
+        const int64_t idx = obase + gm * N + gn;
+        if (gm < M) {
+          if (vec_ok && gn + 4 <= N) store_vec<float, 4>(out, HIPNX_F32, idx, v);
+          else {
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+              if (gn + e < N) store_one<float>(out, HIPNX_F32, idx + e, v[e]);
+          }
+        }
+      }
+    }
+  } else if constexpr (int_acc != int_out) return;  // the host never pairs them
   else {
     typedef typename std::conditional<int_acc, int64_t, float>::type S;
     const bool vec_ok = (N % 4) == 0;
@@ -585,7 +619,7 @@ gemm_pipelined_kernel(GemmArgs a) {
   // epilogue: the output type is wave-uniform; branch once, then every store is straight-line
   const int64_t obase = b * a.M * a.N;
   switch (a.odt) {
-#define HIPNX_EPI(T) case T: gemm_epilogue<DT, T, TM16, TN16>(acc, a.out, obase, a.M, a.N, m0 + wm, n0 + wn, lane); break;
+#define HIPNX_EPI(T) case T: gemm_epilogue<DT, T, TM16, TN16>(acc, a.out, obase, a.M, a.N, m0 + wm, n0 + wn, lane, a.scale, a.scale_mode); break;
     HIPNX_EPI(HIPNX_BF16) HIPNX_EPI(HIPNX_F16) HIPNX_EPI(HIPNX_F32) HIPNX_EPI(HIPNX_F64)
     HIPNX_EPI(HIPNX_S8) HIPNX_EPI(HIPNX_U8) HIPNX_EPI(HIPNX_S16) HIPNX_EPI(HIPNX_U16)
     HIPNX_EPI(HIPNX_S32) HIPNX_EPI(HIPNX_U32) HIPNX_EPI(HIPNX_S64) HIPNX_EPI(HIPNX_U64)

@@ -730,6 +730,50 @@ def _fuse(roots: List[Tensor], ints: bool = False) -> int:
         _plan["ints"] = False
 
 
+def _scale_mode(scale: Tensor, out_shape, n_axes: int, batch_axes: int):
+    """How `scale` broadcasts over a contraction's result [batch..., rows..., columns...] (the last
+    `n_axes` axes are the right operand's free axes): one value, one per column, one per row, or None."""
+    if scale.size == 1:
+        return 3
+    rank = len(out_shape)
+    padded = (1,) * (rank - len(scale.shape)) + tuple(scale.shape)
+    if len(padded) != rank:
+        return None
+    if n_axes and padded == (1,) * (rank - n_axes) + tuple(out_shape[rank - n_axes:]):
+        return 1
+    if batch_axes == 0 and rank > n_axes and padded == tuple(out_shape[:rank - n_axes]) + (1,) * n_axes:
+        return 2
+    return None
+
+
+def _absorb_scales(order: List[Tensor], uses) -> int:
+    """multiply(as_type(dot(s8, s8) -> s32, f32), scales) becomes one `dot_scaled` node when nobody
+    else reads the sum or its conversion: the quantised linear layer, finished on the accumulators."""
+    found = 0
+    for node in order:
+        e = node.data
+        if e.op != "multiply" or node.type != ("f", 32):
+            continue
+        for x, scale in (e.args, e.args[::-1]):
+            if not (isinstance(x, Tensor) and isinstance(x.data, Expr) and x.data.op == "as_type" and uses.get(x.data.id) == 1):
+                continue
+            d = x.data.args[0]
+            if not (isinstance(d.data, Expr) and d.data.op == "dot" and uses.get(d.data.id) == 1 and d.type == ("s", 32)):
+                continue
+            l, c1, b1, r, c2, b2 = d.data.args
+            if l.type != ("s", 8) or r.type != ("s", 8) or not isinstance(scale, Tensor) or scale.type != ("f", 32):
+                continue
+            if x.shape != node.shape or d.shape != node.shape:
+                continue
+            mode = _scale_mode(scale, node.shape, len(r.shape) - len(c2) - len(b2), len(b1))
+            if mode is None:
+                continue
+            e.op, e.args = "dot_scaled", [l, list(c1), list(b1), r, list(c2), list(b2), scale, mode]
+            found += 1
+            break
+    return found
+
+
 def _fuse_planned(roots: List[Tensor]) -> int:
     order, uses, seen = [], {}, set()
 
@@ -750,6 +794,12 @@ def _fuse_planned(roots: List[Tensor]) -> int:
         walk(r)
     if any(t.data.op in ("while", "cond", "elem") for t in order):
         return 0  # bodies of nested scopes read root-scope nodes that the counts above do not see
+    if _absorb_scales(order, uses):
+        uses.clear()
+        seen.clear()
+        del order[:]
+        for r in roots:
+            walk(r)
     def candidate(a, root):
         return (isinstance(a, Tensor) and isinstance(a.data, Expr) and a.data.op not in ("constant", "tensor", "fused")
                 and a.data.scope == 0 and a.shape == root.shape and _fusable(a))
@@ -1012,6 +1062,19 @@ class _Run:
         if op == "fused":
             group, inputs = e.args
             return group.run(self, x.with_(data=None), [self.eval(t, scope) for t in inputs])
+        if op == "dot_scaled":
+            l, c1, b1, r, c2, b2, scale, mode = e.args
+            lv, rv, sv = self.eval(l, scope), self.eval(r, scope), self.eval(scale, scope)
+            mod, out = self.pick([lv, rv, sv]), x.with_(data=None)
+            one_call = getattr(mod, "dot_scaled", None)
+            if one_call is not None:
+                try:
+                    return one_call(out, lv, c1, b1, rv, c2, b2, sv, mode)
+                except Exception as err:  # a shape the kernel leaves to the separate callbacks
+                    if getattr(err, "status", None) != _EUNSUPPORTED:
+                        raise
+            summed = mod.dot(out.with_(type=("s", 32)), lv, c1, b1, rv, c2, b2)
+            return mod.multiply(out, mod.as_type(out, summed), sv)
         if op == "block":
             struct, in_args, fun = e.args
             args = [self.eval(a, scope) for a in in_args]

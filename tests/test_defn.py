@@ -285,3 +285,42 @@ def test_layout_of_a_group(on_oracle):
     assert defn._layout((2, 3, 16), [(2, 3, 16), (2, 3, 1), (16,)]) == (6, 16, [(16, 1), (1, 0), (0, 1)])
     assert defn._layout((5, 7), [(5, 7), (7,)]) is None            # rows are not whole vectors
     assert defn._layout((4, 16), [(4, 16), (4, 1), (1, 16), (2, 1, 16)]) is None
+
+
+# ---- the quantised linear layer: dot -> as_type -> multiply by the scales becomes one node ---------------
+
+def _roots_ops(compiled):
+    return [r.data.op for r in compiled.roots]
+
+
+def test_scales_after_an_int8_dot_are_absorbed_and_fall_back_without_the_kernel(on_oracle):
+    rng = np.random.default_rng(0)
+    x = from_numpy(rng.integers(-127, 128, size=(8, 256), dtype=np.int8), "s8", on_oracle)
+    w = from_numpy(rng.integers(-127, 128, size=(32, 256), dtype=np.int8), "s8", on_oracle)
+    per_column = f32(rng.uniform(1e-3, 1e-2, size=(32,)), on_oracle)
+    per_row = f32(rng.uniform(1e-3, 1e-2, size=(8, 1)), on_oracle)
+
+    def layer(xq, wq, sc):
+        return Nx.multiply(Nx.as_type(Nx.dot(xq, [1], wq, [1], out_type="s32"), "f32"), sc)
+
+    def layer_scale_first(xq, wq, sc):
+        return Nx.multiply(sc, Nx.as_type(Nx.dot(xq, [1], wq, [1], out_type="s32"), "f32"))
+
+    def layer_constant(xq, wq):
+        return Nx.multiply(Nx.as_type(Nx.dot(xq, [1], wq, [1], out_type="s32"), "f32"), 0.0078125)
+
+    for fun, args, mode in ((layer, (x, w, per_column), 1), (layer_scale_first, (x, w, per_column), 1),
+                            (layer, (x, w, per_row), 2), (layer_constant, (x, w), 3)):
+        planned = defn.compile(fun, *args, fuse=True)
+        assert _roots_ops(planned) == ["dot_scaled"] and planned.roots[0].data.args[-1] == mode
+        # the oracle has no such callback: the evaluator makes the three calls
+        assert_bits_equal(planned(*args), fun(*args), f"{fun.__name__} mode {mode}")
+
+    def sum_read_twice(xq, wq, sc):
+        d = Nx.dot(xq, [1], wq, [1], out_type="s32")
+        return Nx.multiply(Nx.as_type(d, "f32"), sc), d
+
+    assert "dot_scaled" not in _roots_ops(defn.compile(sum_read_twice, x, w, per_column, fuse=True))
+    odd = f32(rng.uniform(size=(8, 32)), on_oracle)  # a full matrix of scales is no scale vector
+    assert "dot_scaled" not in _roots_ops(defn.compile(layer, x, w, odd, fuse=True))
+    assert _roots_ops(defn.compile(layer, x, w, per_column)) == ["multiply"]  # only when fusing is asked for

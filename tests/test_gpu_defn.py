@@ -528,3 +528,75 @@ def test_random_floats_from_one_compiled_group(name, hip):
     finally:
         hip.fused_elementwise = classmethod(original)
     assert len(calls) >= 1 and fused.fused_groups == 1  # everything after the cipher is one group
+
+
+# ---- dot -> as_type -> multiply by the scales on the accumulators (the quantised linear layer) -----------
+
+def linear_scaled(xq, wq, sc):
+    return Nx.multiply(Nx.as_type(Nx.dot(xq, [1], wq, [1], out_type="s32"), "f32"), sc)
+
+
+def rand_s8(rng, shape, backend):
+    return from_numpy(rng.integers(-127, 128, size=shape, dtype=np.int8), "s8", backend)
+
+
+@pytest.mark.parametrize("m,n,k", [(64, 11008, 4096), (64, 256, 4096), (16, 512, 8192), (300, 520, 256), (256, 256, 128), (1024, 1024, 1024), (8, 40, 128)])
+@pytest.mark.parametrize("scales", ["per_column", "per_row", "one", "constant"])
+def test_scaled_int8_dot_is_bit_identical_to_the_three_callbacks(m, n, k, scales, hip):
+    rng = np.random.default_rng(seed_of(m, n, k, scales))
+    x, w = rand_s8(rng, (m, k), hip), rand_s8(rng, (n, k), hip)
+    if scales == "constant":
+        fun, args = (lambda xq, wq: linear_scaled(xq, wq, 0.0078125)), (x, w)
+    else:
+        shape = {"per_column": (n,), "per_row": (m, 1), "one": (1, 1)}[scales]
+        sc = from_numpy(rng.uniform(1e-3, 1e-2, size=shape).astype(np.float32), "f32", hip)
+        if scales == "per_column":  # a NaN and an infinity among the scales travel like in the multiply kernel
+            raw = hip.to_numpy(sc).copy()
+            raw[0], raw[-1] = np.nan, np.inf
+            sc = from_numpy(raw, "f32", hip)
+        fun, args = linear_scaled, (x, w, sc)
+    want = defn.compile(fun, *args)(*args)
+    planned = defn.compile(fun, *args, fuse=True)
+    assert planned.roots[0].data.op == "dot_scaled"
+    calls = []
+    original = hip.dot_scaled.__func__
+
+    def counting(cls, *a, **kw):
+        calls.append(1)
+        return original(cls, *a, **kw)
+    hip.dot_scaled = classmethod(counting)
+    try:
+        assert_bits_equal(planned(*args), want, f"{m}x{n}x{k} {scales}")
+    finally:
+        hip.dot_scaled = classmethod(original)
+    assert calls == [1]
+
+
+def test_scaled_dot_with_batches_and_with_the_weights_k_outer(hip):
+    rng = np.random.default_rng(77)
+    x, w = rand_s8(rng, (4, 48, 256), hip), rand_s8(rng, (4, 256, 80), hip)
+    sc = from_numpy(rng.uniform(1e-3, 1e-2, size=(80,)).astype(np.float32), "f32", hip)
+
+    def fun(xq, wq, s):  # batched, the right operand contracted on its middle axis
+        return Nx.multiply(Nx.as_type(Nx.dot(xq, [2], [0], wq, [1], [0], out_type="s32"), "f32"), s)
+    planned = defn.compile(fun, x, w, sc, fuse=True)
+    assert planned.roots[0].data.op == "dot_scaled"
+    assert_bits_equal(planned(x, w, sc), defn.compile(fun, x, w, sc)(x, w, sc), "batched")
+
+
+def test_scaled_dot_entry_point_refuses_what_it_does_not_take(hip):
+    from nx_amd._lib import EUNSUPPORTED, SCALE_PER_COLUMN, HipNxError
+    rng = np.random.default_rng(5)
+    x, w = rand_s8(rng, (8, 100), hip), rand_s8(rng, (40, 100), hip)  # K is not a multiple of 128
+    sc = from_numpy(np.ones(40, dtype=np.float32), "f32", hip)
+    out = sc.with_(data=None, shape=(8, 40))
+    with pytest.raises(HipNxError) as err:
+        hip.dot_scaled(out, x, [1], [], w, [1], [], sc, SCALE_PER_COLUMN)
+    assert err.value.status == EUNSUPPORTED
+    # through the evaluator the same shapes make the three calls instead
+    planned = defn.compile(linear_scaled, x, w, sc, fuse=True)
+    assert_bits_equal(planned(x, w, sc), defn.compile(linear_scaled, x, w, sc)(x, w, sc), "fallback")
+    short = from_numpy(np.ones(8, dtype=np.float32), "f32", hip)
+    x2, w2 = rand_s8(rng, (16, 128), hip), rand_s8(rng, (40, 128), hip)
+    with pytest.raises(HipNxError, match="holds"):
+        hip.dot_scaled(sc.with_(data=None, shape=(16, 40)), x2, [1], [], w2, [1], [], short, SCALE_PER_COLUMN)
