@@ -287,6 +287,11 @@ def main():
                 _, ms = timed(lambda: fused(*targs), steps, warm)
                 entry(name + tag, nbytes, "GB/s", ms, PEAK_HBM_GBS, "hbm")
             fused_mode("interpreted")
+            # planned for compiled kernels from the start: groups over the same rows become stages of one program
+            # (the softmax: row maximum, sum of exponentials and division in one kernel)
+            staged = defn.compile(fun, *targs, fuse="compiled")
+            _, ms = timed(lambda: staged(*targs), steps, warm)
+            entry(name + "_planned_compiled", nbytes, "GB/s", ms, PEAK_HBM_GBS, "hbm")
         x, y = W.elementwise_reduce(n=16384)
         big = (put(x, "f32"), put(y, "f32"))
         fused = defn.compile(chain1, *big, fuse=True)

@@ -187,10 +187,15 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
   unsigned saved = 0;  // slots that hold a value so far
   unsigned raw_inputs = 0;  // inputs whose words are loaded unconverted
   bool have_acc = false, full = false, needs_compiled = false;
+  int n_stats = 0;  // row statistics produced so far (HIPNX_FUSED_ROW_REDUCE markers)
   auto int32 = [](int dt) { return dt == HIPNX_U32 || dt == HIPNX_S32; };
   auto source_ok = [&](int src, int arg, const char **why) {
     if (src == HIPNX_FUSED_SRC_INPUT && arg >= n_inputs) { *why = "reads an input that is not there"; return false; }
     if (src == HIPNX_FUSED_SRC_SAVED && (arg >= HIPNX_FUSED_SAVED || !(saved >> arg & 1))) { *why = "reads an empty slot"; return false; }
+    if (src == HIPNX_FUSED_SRC_ROWSTAT) {
+      if (arg >= n_stats) { *why = "reads a row statistic that no stage has produced yet"; return false; }
+      return true;
+    }
     if (src != HIPNX_FUSED_SRC_INPUT && src != HIPNX_FUSED_SRC_SAVED && src != HIPNX_FUSED_SRC_CONST) { *why = "has an unknown operand source"; return false; }
     return true;
   };
@@ -232,6 +237,15 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
         full |= !binary_light(q.op);
         break;
       case HIPNX_FUSED_BITCAST: break;
+      case HIPNX_FUSED_ROW_REDUCE:
+        if (q.op != HIPNX_RED_SUM && q.op != HIPNX_RED_MAX && q.op != HIPNX_RED_MIN) return set_error(HIPNX_EUNSUPPORTED, "fused: stage reduction %d", q.op);
+        if (n_stats >= HIPNX_FUSED_STATS || q.arg != n_stats) return set_error(HIPNX_EINVAL, "fused: instruction %d is row statistic %d of at most %d, in order", i, q.arg, HIPNX_FUSED_STATS);
+        if (!narrow(q.dt) || i == 0 || !narrow(prog[i - 1].dt) || i == n_instr - 1)
+          return set_error(HIPNX_EINVAL, "fused: instruction %d reduces a non-float value, or nothing follows it", i);
+        if (q.flags) return set_error(HIPNX_EINVAL, "fused: instruction %d: a stage reduction takes no flags", i);
+        n_stats++;
+        needs_compiled = true;
+        break;
       case HIPNX_FUSED_SELECT:
         if (!source_ok(q.src, q.arg, &why) || !source_ok(q.src2, q.arg2, &why))
           return set_error(HIPNX_EINVAL, "fused: instruction %d %s", i, why);
@@ -241,7 +255,8 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
         break;
       default: return set_error(HIPNX_EINVAL, "fused: instruction %d has kind %d", i, q.kind);
     }
-    have_acc = true;
+    have_acc = q.kind != HIPNX_FUSED_ROW_REDUCE;  // the next stage starts from nothing
+    if (q.kind == HIPNX_FUSED_ROW_REDUCE) saved = 0;
     if (q.flags >> 4) {
       if ((q.flags >> 4) > HIPNX_FUSED_SAVED) return set_error(HIPNX_EINVAL, "fused: instruction %d saves to slot %d", i, (q.flags >> 4) - 1);
       saved |= 1u << ((q.flags >> 4) - 1);
@@ -250,7 +265,9 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
   }
   if (int_out != int32(prog[n_instr - 1].dt)) return set_error(HIPNX_EINVAL, "fused: result type %d after a program that ends in type %d", out_dt, prog[n_instr - 1].dt);
   if (needs_compiled && ctx->fused_mode != HIPNX_FUSED_COMPILED)
-    return set_error(HIPNX_EUNSUPPORTED, "fused: 32-bit integer instructions need the compiled mode");
+    return set_error(HIPNX_EUNSUPPORTED, "fused: 32-bit integer instructions and stages need the compiled mode");
+  if (n_stats && (reduce_op != -1 || cols > 4096 || cols == 0))
+    return set_error(HIPNX_EUNSUPPORTED, "fused: stages take rows of 1 .. 4096 elements and no reduction of the result");
   const int64_t n = rows * cols;
   if (cols % 8 != 0) return set_error(HIPNX_EUNSUPPORTED, "fused: the row length is not a multiple of 8");
   for (int k = 0; k < n_inputs; k++) {
@@ -290,7 +307,8 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
   if (ctx->fused_mode == HIPNX_FUSED_COMPILED) {
     // the same grids as the interpreting kernels below
     const bool block_per_row = reduce_op != -1 && a.cols > 4096;
-    int64_t grid = reduce_op == -1 ? (a.nvec + (int64_t)FBLOCK * FV - 1) / ((int64_t)FBLOCK * FV)
+    int64_t grid = n_stats ? (a.rows + FBLOCK / WAVE - 1) / (FBLOCK / WAVE)  // a wave per row
+                   : reduce_op == -1 ? (a.nvec + (int64_t)FBLOCK * FV - 1) / ((int64_t)FBLOCK * FV)
                    : block_per_row ? a.rows : (a.rows + FBLOCK / WAVE - 1) / (FBLOCK / WAVE);
     if (grid > (1ll << 30)) grid = 1ll << 30;
     bool done = false;

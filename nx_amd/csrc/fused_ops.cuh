@@ -144,9 +144,17 @@ struct Saved {
 // dt[], imm[] and imm2[] as f32 bit patterns), the inputs' element types and column strides, and
 // the result type.  Every branch the interpreter takes on an instruction field is taken by the
 // compiler here.
+typedef float RowStats[HIPNX_FUSED_STATS];  // results of the row reductions of earlier stages (fused_row_stages_body)
+
 template <typename P, int SRC, int ARG, unsigned IMM, bool RAW>
-__device__ __forceinline__ void fetch_static(KernArgs a, const Saved &S, const int64_t (&row)[FV], const int64_t (&col)[FV], Vecs &dst) {
-  if constexpr (SRC == HIPNX_FUSED_SRC_INPUT) {
+__device__ __forceinline__ void fetch_static(KernArgs a, const Saved &S, const RowStats &stats, const int64_t (&row)[FV],
+                                             const int64_t (&col)[FV], Vecs &dst) {
+  if constexpr (SRC == HIPNX_FUSED_SRC_ROWSTAT) {
+#pragma unroll
+    for (int u = 0; u < FV; u++)
+#pragma unroll
+      for (int e = 0; e < FE; e++) dst[u][e] = stats[ARG];
+  } else if constexpr (SRC == HIPNX_FUSED_SRC_INPUT) {
     // RAW: the words of a 4-byte input as they are (what the f32 path does with its bits)
     load_input_as(a, ARG, RAW ? (int)HIPNX_F32 : P::in_dt[ARG], P::in_cs[ARG], row, col, dst);
   } else if constexpr (SRC == HIPNX_FUSED_SRC_SAVED) {
@@ -174,15 +182,17 @@ __device__ __forceinline__ float int_unary(float x) {
   return __uint_as_float((uint32_t)unary_apply<OP, int64_t>(UNS ? (int64_t)a : (int64_t)(int32_t)a, 32));
 }
 
-template <typename P, int PC>
-__device__ __forceinline__ void static_steps(KernArgs a, const int64_t (&row)[FV], const int64_t (&col)[FV], Vecs &acc, Saved &S) {
-  if constexpr (PC < P::n_instr) {
+// instructions PC .. END-1
+template <typename P, int PC, int END>
+__device__ __forceinline__ void static_steps(KernArgs a, const int64_t (&row)[FV], const int64_t (&col)[FV], Vecs &acc, Saved &S,
+                                             const RowStats &stats) {
+  if constexpr (PC < END) {
     constexpr int kind = P::kind[PC], op = P::op[PC], src = P::src[PC], arg = P::arg[PC];
     constexpr int src2 = P::src2[PC], arg2 = P::arg2[PC], flags = P::flags[PC], dt = P::dt[PC];
     constexpr unsigned imm = P::imm[PC], imm2 = P::imm2[PC];
     constexpr bool ints = (flags & HIPNX_FUSED_FLAG_INT) != 0, uns = dt == HIPNX_U32;
     if constexpr (kind == HIPNX_FUSED_SET) {
-      fetch_static<P, src, arg, imm, ints>(a, S, row, col, acc);
+      fetch_static<P, src, arg, imm, ints>(a, S, stats, row, col, acc);
     } else if constexpr (kind == HIPNX_FUSED_UNARY) {
       if constexpr (ints) {
 #pragma unroll
@@ -194,7 +204,7 @@ __device__ __forceinline__ void static_steps(KernArgs a, const int64_t (&row)[FV
       }
     } else if constexpr (kind == HIPNX_FUSED_BINARY) {
       Vecs y;
-      fetch_static<P, src, arg, imm, ints>(a, S, row, col, y);
+      fetch_static<P, src, arg, imm, ints>(a, S, stats, row, col, y);
       if constexpr (ints) {
 #pragma unroll
         for (int u = 0; u < FV; u++)
@@ -205,8 +215,8 @@ __device__ __forceinline__ void static_steps(KernArgs a, const int64_t (&row)[FV
       }
     } else if constexpr (kind == HIPNX_FUSED_SELECT) {
       Vecs y, z;
-      fetch_static<P, src, arg, imm, false>(a, S, row, col, y);
-      fetch_static<P, src2, arg2, imm2, false>(a, S, row, col, z);
+      fetch_static<P, src, arg, imm, false>(a, S, stats, row, col, y);
+      fetch_static<P, src2, arg2, imm2, false>(a, S, stats, row, col, z);
 #pragma unroll
       for (int u = 0; u < FV; u++)
 #pragma unroll
@@ -224,7 +234,7 @@ __device__ __forceinline__ void static_steps(KernArgs a, const int64_t (&row)[FV
         for (int e = 0; e < FE; e++) acc[u][e] = round_to(acc[u][e], dt);
     }
     if constexpr ((flags >> 4) != 0) copy_vecs(S.s[(flags >> 4) - 1], acc);
-    static_steps<P, PC + 1>(a, row, col, acc, S);
+    static_steps<P, PC + 1, END>(a, row, col, acc, S, stats);
   }
 }
 
@@ -232,7 +242,8 @@ template <typename P>
 struct RunStatic {
   static __device__ __forceinline__ void run(KernArgs a, const int64_t (&row)[FV], const int64_t (&col)[FV], Vecs &acc) {
     Saved S;
-    static_steps<P, 0>(a, row, col, acc, S);
+    const RowStats none = {};
+    static_steps<P, 0, P::n_instr>(a, row, col, acc, S, none);
   }
   // a u32 / s32 result leaves as the bits it is held as
   static __device__ __forceinline__ int out_dt(KernArgs) { return P::out_dt; }
@@ -313,6 +324,72 @@ __device__ __forceinline__ void fused_reduce_rows_body() {
     }
   }
   if (lane == 0 && r < rows) finalize((void *)a->out, a->out_dt, r, acc);
+}
+
+// ---- several stages over the same rows in one kernel ------------------------------------------------
+// A program with HIPNX_FUSED_ROW_REDUCE markers is a sequence of stages: each stage but the last
+// ends in a reduction of its value along the row, and later stages read that row statistic as an
+// operand (softmax: the row maximum, then the sum of the exponentials, then the division).  One wave
+// takes a row through all stages; a stage walks the row exactly as fused_reduce_rows_body does with
+// TPR = WAVE (same lanes, same order, same reducer), and a statistic is carried on as the value a
+// store to its type and a load would give -- so the result equals the separate kernels', bit for bit.
+// The row is read again by every stage, from the caches: one wave has just read it.
+template <typename CT>
+__device__ __forceinline__ float as_stored(CT v, int dt) {
+  switch (dt) {
+    case HIPNX_BF16: return bf16_bits_to_f32(conv<CT>::to_bf16(v));
+    case HIPNX_F16: return (float)bits_f16(conv<CT>::to_f16(v));
+    default: return __uint_as_float(conv<CT>::to_f32(v));
+  }
+}
+
+template <typename P, int SEG>
+__device__ __forceinline__ void row_stage(KernArgs a, int64_t r, int lane, RowStats &stats) {
+  constexpr int begin = SEG == 0 ? 0 : P::seg_end[SEG - 1] + 1;  // past the previous stage's marker
+  constexpr int end = P::seg_end[SEG];
+  constexpr int red = P::seg_red[SEG];
+  const int64_t cols = a->cols, step = (int64_t)WAVE * FE;
+  if constexpr (red < 0) {  // the last stage: its value is the result
+    void *out = (void *)a->out;
+    for (int64_t k = (int64_t)lane * FE; k < cols; k += step) {
+      const int64_t row[FV] = {r}, col[FV] = {k};
+      Vecs x;
+      Saved S;
+      static_steps<P, begin, end>(a, row, col, x, S, stats);
+      if constexpr (P::out_dt == HIPNX_U32 || P::out_dt == HIPNX_S32) {
+        uint4 *p = reinterpret_cast<uint4 *>((uint32_t *)out + r * cols + k);
+        p[0] = make_uint4(__float_as_uint(x[0][0]), __float_as_uint(x[0][1]), __float_as_uint(x[0][2]), __float_as_uint(x[0][3]));
+        p[1] = make_uint4(__float_as_uint(x[0][4]), __float_as_uint(x[0][5]), __float_as_uint(x[0][6]), __float_as_uint(x[0][7]));
+      } else {
+        store_vec<float, FE>(out, P::out_dt, r * cols + k, x[0]);
+      }
+    }
+  } else {
+    typedef typename std::conditional<red == HIPNX_RED_SUM, double, float>::type CT;
+    typedef PlainReducer<CT, red, false> R;
+    typename R::acc_t acc = R::init();
+    for (int64_t k = (int64_t)lane * FE; k < cols; k += step) {
+      const int64_t row[FV] = {r}, col[FV] = {k};
+      Vecs x;
+      Saved S;
+      static_steps<P, begin, end>(a, row, col, x, S, stats);
+#pragma unroll
+      for (int e = 0; e < FE; e++) acc = R::accumulate(acc, (CT)x[0][e], k + e);
+    }
+    acc = wave_reduce<R>(acc);  // the butterfly leaves the same value in every lane
+    stats[SEG] = as_stored<CT>(acc, P::seg_dt[SEG]);
+    row_stage<P, SEG + 1>(a, r, lane, stats);
+  }
+}
+
+template <typename P>
+__device__ __forceinline__ void fused_row_stages_body() {
+  static_assert(FV == 1, "one vector per lane and step");
+  KernArgs a = (KernArgs)__builtin_amdgcn_kernarg_segment_ptr();
+  const int64_t r = (int64_t)blockIdx.x * (FBLOCK / WAVE) + threadIdx.x / WAVE;
+  if (r >= a->rows) return;
+  RowStats stats = {};
+  row_stage<P, 0>(a, r, threadIdx.x % WAVE, stats);
 }
 
 }  // namespace hipnx

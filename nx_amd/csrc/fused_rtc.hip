@@ -11,6 +11,7 @@
 #include <cstring>
 #include <functional>
 #include <string>
+#include <vector>
 
 #include "fused_ops.cuh"
 #include "internal.h"
@@ -74,9 +75,19 @@ static std::string make_source(const FusedArgs &a, int reduce_op, bool block_per
   list_of(s, "imm2", "unsigned", a.n_instr, [&](int i) { return std::to_string(q[i].imm2_bits) + "u"; });
   list_of(s, "in_dt", "int", a.n_inputs, [&](int k) { return std::to_string(a.in_dt[k]); });
   list_of(s, "in_cs", "int", a.n_inputs, [&](int k) { return std::to_string(a.in_cs[k]); });
+  // stages: where each ends (its marker, or the end of the program), what it reduces with, the statistic's type
+  std::vector<int> seg_end, seg_red, seg_dt;
+  for (int i = 0; i < a.n_instr; i++)
+    if (q[i].kind == HIPNX_FUSED_ROW_REDUCE) { seg_end.push_back(i); seg_red.push_back(q[i].op); seg_dt.push_back(q[i].dt); }
+  const bool stages = !seg_end.empty();
+  seg_end.push_back(a.n_instr); seg_red.push_back(-1); seg_dt.push_back(a.out_dt);
+  list_of(s, "seg_end", "int", (int)seg_end.size(), [&](int k) { return std::to_string(seg_end[k]); });
+  list_of(s, "seg_red", "int", (int)seg_red.size(), [&](int k) { return std::to_string(seg_red[k]); });
+  list_of(s, "seg_dt", "int", (int)seg_dt.size(), [&](int k) { return std::to_string(seg_dt[k]); });
   s += "};\n}\nusing namespace hipnx;\nextern \"C\" __global__ void __launch_bounds__(FBLOCK) fused_group(FusedArgs by_value) {\n  (void)by_value;\n";
   const char *tpr = block_per_row ? "FBLOCK" : "WAVE";
-  switch (reduce_op) {
+  if (stages) s += "  fused_row_stages_body<P>();\n";
+  else switch (reduce_op) {
     case HIPNX_RED_SUM: s += std::string("  fused_reduce_rows_body<RunStatic<P>, PlainReducer<double, HIPNX_RED_SUM, false>, double, ") + tpr + ">();\n"; break;
     case HIPNX_RED_MAX: s += std::string("  fused_reduce_rows_body<RunStatic<P>, PlainReducer<float, HIPNX_RED_MAX, false>, float, ") + tpr + ">();\n"; break;
     case HIPNX_RED_MIN: s += std::string("  fused_reduce_rows_body<RunStatic<P>, PlainReducer<float, HIPNX_RED_MIN, false>, float, ") + tpr + ">();\n"; break;

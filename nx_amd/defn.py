@@ -914,6 +914,133 @@ def _fuse_planned(roots: List[Tensor]) -> int:
         if both is None:
             continue
         e.op, e.args = "fused", [both, inner.args[1]]
+    if _plan["ints"]:  # planned for compiled kernels: groups over the same rows become stages of one
+        _cluster_rows(roots)
+    return formed
+
+
+class _RowCluster:
+    """Fused groups over the same rows as stages of one program: every group but the last ends in a
+    reduction along the row, later groups read its result (`stages` are (node, group, inputs) in
+    evaluation order, `final` the element-wise group that produces the result).  A backend that
+    cannot run the program gets the groups one by one."""
+
+    reduce = None
+    how = {"mode": "compiled"}
+
+    def __init__(self, stages, final, inputs, program, layout):
+        self.stages, self.final, self.inputs, self.program, self.layout = stages, final, inputs, program, layout
+        self.root = final[0]
+
+    def run(self, run: "_Run", out: Tensor, values: List[Tensor]):
+        fused = getattr(run.pick(values), "fused_elementwise", None)
+        if fused is not None:
+            try:
+                return fused(out, self.program, values, self.layout, **self.how)
+            except Exception as e:
+                if getattr(e, "status", None) != _EUNSUPPORTED:
+                    raise
+        known = {t.data.id: v for t, v in zip(self.inputs, values)}
+        for node, group, inputs in self.stages + [self.final]:
+            known[node.data.id] = group.run(run, node.with_(data=None), [known[t.data.id] for t in inputs])
+        return known[self.root.data.id]
+
+
+def _cluster_rows(roots: List[Tensor]) -> int:
+    """Rewrites an element-wise fused node together with the row-reducing fused nodes that only it
+    (and each other) read into one node holding a _RowCluster.  Rows of at most 4096 elements:
+    the width at which the separate reduction gives a row to one wave, whose order the stages keep."""
+    order, readers, seen = [], {}, set()
+
+    def walk(t):
+        e = t.data
+        if e.op in ("constant", "tensor") or e.scope != 0:
+            return
+        if e.id in seen:
+            return
+        seen.add(e.id)
+        for child in _children(e):
+            if isinstance(child, Tensor):
+                readers.setdefault(child.data.id, set()).add(e.id)
+                walk(child)
+        order.append(t)
+
+    for r in roots:
+        readers.setdefault(r.data.id, set()).add("result")
+        walk(r)
+    position = {t.data.id: i for i, t in enumerate(order)}
+    formed = 0
+    for root in order:
+        e = root.data
+        if e.op != "fused" or not isinstance(e.args[0], _Group):
+            continue
+        group, inputs = e.args
+        rank = len(root.shape)
+        if group.reduce is not None or not group.program or rank == 0:
+            continue
+        cols, rows = root.shape[-1], prod(root.shape[:-1])
+        if cols > 4096 or cols % 8:
+            continue
+        members = {e.id: root}
+
+        per_row = tuple(root.shape[:-1]) + (1,)
+
+        def stage_of(t):
+            """The group behind `t` if it reduces a value of the root's shape along its rows and `t`
+            broadcasts against that shape as one value per row."""
+            g = t.data.args[0] if isinstance(t.data, Expr) and t.data.op == "fused" else None
+            ok = (isinstance(g, _Group) and g.reduce is not None and g.program and g.root.shape == root.shape
+                  and g.reduce[2][0] == rows and g.reduce[2][1] == cols and t.type in _NARROW
+                  and (1,) * (rank - len(t.shape)) + tuple(t.shape) == per_row)
+            return g if ok else None
+
+        changed = True
+        while changed:
+            changed = False
+            for m in list(members.values()):
+                for t in m.data.args[1]:
+                    if t.data.id in members or stage_of(t) is None:
+                        continue
+                    if readers.get(t.data.id, set()) <= set(members):
+                        members[t.data.id] = t
+                        changed = True
+        if len(members) < 2 or len(members) - 1 > 3:
+            continue
+        stage_nodes = sorted((t for i, t in members.items() if i != e.id), key=lambda t: position[t.data.id])
+        number = {t.data.id: k for k, t in enumerate(stage_nodes)}
+        union, index = [], {}
+
+        def remap(ins, key_src, key_arg, own_inputs):
+            if ins.get(key_src, 0) != 1:
+                return
+            t = own_inputs[ins.get(key_arg, 0)]
+            if t.data.id in number:
+                ins[key_src], ins[key_arg] = 3, number[t.data.id]
+            else:
+                if t.data.id not in index:
+                    index[t.data.id] = len(union)
+                    union.append(t)
+                ins[key_arg] = index[t.data.id]
+
+        program = _Program()
+        for t in stage_nodes + [root]:
+            g, own = t.data.args
+            for ins in g.program:
+                ins = dict(ins)
+                remap(ins, "src", "arg", own)
+                if ins["kind"] == 3:
+                    remap(ins, "src2", "arg2", own)
+                program.append(ins)
+            if t is not root:
+                program.append({"kind": 6, "op": _REDUCE_CODES[g.reduce[0]], "arg": number[t.data.id], "dt": t.type})
+        layout = _layout(root.shape, [t.shape for t in union], split=rank - 1)
+        if layout is None or len(program) > _MAX_INSTR or len(union) > _MAX_INPUTS:
+            continue
+        # the pieces keep their own nodes (copies) for a backend that runs them one by one
+        stages = [(t.with_(data=Expr(t.data.id, "fused", t.data.args, 0)), t.data.args[0], t.data.args[1]) for t in stage_nodes]
+        final = (root.with_(data=Expr(e.id, "fused", e.args, 0)), group, inputs)
+        e.args = [_RowCluster(stages, final, union, program, layout), union]
+        formed += 1
     return formed
 
 

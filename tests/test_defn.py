@@ -324,3 +324,42 @@ def test_scales_after_an_int8_dot_are_absorbed_and_fall_back_without_the_kernel(
     odd = f32(rng.uniform(size=(8, 32)), on_oracle)  # a full matrix of scales is no scale vector
     assert "dot_scaled" not in _roots_ops(defn.compile(layer, x, w, odd, fuse=True))
     assert _roots_ops(defn.compile(layer, x, w, per_column)) == ["multiply"]  # only when fusing is asked for
+
+
+# ---- groups over the same rows as stages of one program (planned for compiled kernels) -------------------
+
+def test_softmax_is_one_node_with_three_stages_and_falls_back_group_by_group(on_oracle):
+    args = build_args(on_oracle)["softmax"]
+    planned = defn.compile(CHAINS["softmax"], *args, fuse="compiled")
+    cluster = planned.roots[0].data.args[0]
+    assert type(cluster).__name__ == "_RowCluster" and len(cluster.stages) == 2
+    kinds = [ins["kind"] for ins in cluster.program]
+    assert kinds.count(6) == 2 and kinds[-1] != 6          # two stage reductions, then the division
+    assert [ins["op"] for ins in cluster.program if ins["kind"] == 6] == [1, 0]  # the maximum, then the sum
+    assert any(ins.get("src") == 3 for ins in cluster.program)                   # later stages read the row statistics
+    assert len(cluster.inputs) == 1                                              # only the scores come from memory
+    assert_bits_equal(planned(*args), CHAINS["softmax"](*args), "softmax, group by group on a backend without the kernel")
+
+
+def test_row_statistics_with_outside_readers_or_another_broadcast_stay_groups(on_oracle):
+    x = f32(np.random.default_rng(3).standard_normal((16, 64)), on_oracle)
+
+    def stat_is_returned(t):
+        m = Nx.reduce_max(Nx.multiply(t, 2.0), axes=[1], keep_axes=True)
+        return Nx.subtract(Nx.multiply(t, 2.0), m), m
+
+    planned = defn.compile(stat_is_returned, x, fuse="compiled")
+    assert all(type(r.data.args[0]).__name__ != "_RowCluster" for r in planned.roots if r.data.op == "fused")
+    got, want = planned(x), stat_is_returned(x)
+    assert_bits_equal(got[0], want[0], "value")
+    assert_bits_equal(got[1], want[1], "statistic")
+
+    sq = f32(np.random.default_rng(4).standard_normal((64, 64)), on_oracle)
+
+    def stat_read_along_columns(t):     # {64} against {64, 64}: one value per column, not per row
+        m = Nx.reduce_max(Nx.multiply(t, 2.0), axes=[1])
+        return Nx.subtract(Nx.multiply(t, 2.0), m)
+
+    planned = defn.compile(stat_read_along_columns, sq, fuse="compiled")
+    assert type(planned.roots[0].data.args[0]).__name__ != "_RowCluster"
+    assert_bits_equal(planned(sq), stat_read_along_columns(sq), "per column")

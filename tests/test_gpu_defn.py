@@ -600,3 +600,70 @@ def test_scaled_dot_entry_point_refuses_what_it_does_not_take(hip):
     x2, w2 = rand_s8(rng, (16, 128), hip), rand_s8(rng, (40, 128), hip)
     with pytest.raises(HipNxError, match="holds"):
         hip.dot_scaled(sc.with_(data=None, shape=(16, 40)), x2, [1], [], w2, [1], [], short, SCALE_PER_COLUMN)
+
+
+# ---- stages over the same rows in one kernel (planned for compiled kernels) ------------------------------
+
+def softmax_rows(x):
+    z = Nx.multiply(x, 0.125)
+    e = Nx.exp(Nx.subtract(z, Nx.reduce_max(z, axes=[-1], keep_axes=True)))
+    return Nx.divide(e, Nx.sum(e, axes=[-1], keep_axes=True))
+
+
+def centred_and_scaled(x, gain):  # layer-norm-like: mean, then mean of squares of the centred values
+    n = x.shape[-1]
+    mean = Nx.divide(Nx.sum(x, axes=[-1], keep_axes=True), float(n))
+    c = Nx.subtract(x, mean)
+    var = Nx.divide(Nx.sum(Nx.multiply(c, c), axes=[-1], keep_axes=True), float(n))
+    return Nx.multiply(Nx.multiply(c, Nx.rsqrt(Nx.add(var, 1e-5))), gain)
+
+
+def range_normalised(x):          # three statistics: minimum, maximum, and the sum of the result's numerator
+    lo = Nx.reduce_min(x, axes=[-1], keep_axes=True)
+    hi = Nx.reduce_max(x, axes=[-1], keep_axes=True)
+    u = Nx.divide(Nx.subtract(x, lo), Nx.subtract(hi, lo))
+    return Nx.divide(u, Nx.sum(u, axes=[-1], keep_axes=True))
+
+
+@pytest.mark.parametrize("ty", ["f32", "bf16"])
+@pytest.mark.parametrize("shape", [(32, 512, 512), (100, 64), (7, 4096), (3, 5, 8), (1, 1024), (2049, 40)])
+@pytest.mark.parametrize("name", ["softmax_rows", "centred_and_scaled", "range_normalised"])
+def test_row_stages_are_bit_identical_to_node_by_node(name, shape, ty, hip):
+    rng = np.random.default_rng(seed_of(name, shape, ty))
+    x = rand_float(rng, ty, shape, hip)
+    args = (x, rand_float(rng, ty, (shape[-1],), hip)) if name == "centred_and_scaled" else (x,)
+    fun = {"softmax_rows": softmax_rows, "centred_and_scaled": centred_and_scaled, "range_normalised": range_normalised}[name]
+    want = defn.compile(fun, *args)(*args)
+    planned = defn.compile(fun, *args, fuse="compiled")
+    # statistics that are worked on before they are used (the mean and the variance of the second function are
+    # divided by n first) keep their groups apart; statistics used as they are become stages of one program
+    staged = name != "centred_and_scaled"
+    assert (type(planned.roots[0].data.args[0]).__name__ == "_RowCluster") == staged
+    calls = []
+    original = hip.fused_elementwise.__func__
+
+    def counting(cls, *a, **k):
+        if "mode" in k:
+            calls.append(1)
+        return original(cls, *a, **k)
+    hip.fused_elementwise = classmethod(counting)
+    try:
+        assert_bits_equal(planned(*args), want, f"{name} {shape} {ty}")
+    finally:
+        hip.fused_elementwise = classmethod(original)
+    if staged:
+        assert calls == [1]  # one launch for all stages
+
+
+def test_rows_longer_than_a_wave_takes_stay_separate_groups(hip):
+    x = rand_float(np.random.default_rng(6), "f32", (8, 8192), hip)
+    planned = defn.compile(softmax_rows, x, fuse="compiled")
+    assert type(planned.roots[0].data.args[0]).__name__ != "_RowCluster"
+    assert_bits_equal(planned(x), defn.compile(softmax_rows, x)(x), "long rows")
+
+
+def test_configuration_3_softmax_in_one_kernel(hip):
+    args = build_args(hip)["softmax"]
+    planned = defn.compile(CHAINS["softmax"], *args, fuse="compiled")
+    assert type(planned.roots[0].data.args[0]).__name__ == "_RowCluster"
+    assert_bits_equal(planned(*args), defn.compile(CHAINS["softmax"], *args)(*args), "softmax of the scores")
