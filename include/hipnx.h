@@ -284,7 +284,7 @@ int hipnx_threefry2x32(hipnx_ctx *ctx, const hipnx_buf *key, int64_t n, hipnx_bu
  * (sum/4, reduce_max/4, reduce_min/4 over the last axis, nx/lib/nx/backend.ex:89-92): `out` then has
  * `rows` elements, and equals the separate reduction kernel applied to the stored result. */
 enum { HIPNX_FUSED_SET = 0, HIPNX_FUSED_UNARY, HIPNX_FUSED_BINARY, HIPNX_FUSED_SELECT, HIPNX_FUSED_AS_TYPE,
-       HIPNX_FUSED_BITCAST, HIPNX_FUSED_ROW_REDUCE };
+       HIPNX_FUSED_BITCAST, HIPNX_FUSED_ROW_REDUCE, HIPNX_FUSED_ROW_STAT };
 /* flags bit 1: the instruction works on 32-bit integers (dt u32 / s32) kept as raw bits -- a SET loads the
  * words of a 4-byte input, or the bits of imm, unconverted; a UNARY / BINARY computes like the integer
  * class of the separate kernels (wrapping at 32 bits); an AS_TYPE converts the integer of type `op` (an
@@ -292,12 +292,15 @@ enum { HIPNX_FUSED_SET = 0, HIPNX_FUSED_UNARY, HIPNX_FUSED_BINARY, HIPNX_FUSED_S
  * HIPNX_FUSED_COMPILED: the interpreting kernels return HIPNX_EUNSUPPORTED for them. */
 enum { HIPNX_FUSED_FLAG_SWAP = 1, HIPNX_FUSED_FLAG_INT = 2 };
 enum { HIPNX_FUSED_SRC_CONST = 0, HIPNX_FUSED_SRC_INPUT, HIPNX_FUSED_SRC_SAVED, HIPNX_FUSED_SRC_ROWSTAT };
-/* HIPNX_FUSED_ROW_REDUCE ends a stage: the accumulator is reduced along the row (op = HIPNX_RED_SUM / MAX /
- * MIN, as the reduction of the separate entry point would, stored in type dt) and becomes row statistic
- * number `arg` (counted from 0 in program order), which later instructions read as an operand with source
- * HIPNX_FUSED_SRC_ROWSTAT; the next stage starts with a SET and empty slots.  The last stage's value is the
- * result: softmax over rows is three stages of one program.  Rows of at most 4096 elements, reduce_op = -1,
- * HIPNX_FUSED_COMPILED only (HIPNX_EUNSUPPORTED otherwise). */
+/* Stages over the same rows.  HIPNX_FUSED_ROW_REDUCE reduces the accumulator along the row (op =
+ * HIPNX_RED_SUM / MAX / MIN, exactly as the reduction of the separate entry point would, the result stored
+ * in type dt) and leaves that one value per row in the accumulator; the instructions that follow work on
+ * it (a sum divided by the row length, an rsqrt of a variance, ...; operands are constants or earlier row
+ * statistics) until HIPNX_FUSED_ROW_STAT ends the stage: the accumulator becomes row statistic number `arg`
+ * (counted from 0 in program order), which later instructions read with source HIPNX_FUSED_SRC_ROWSTAT.
+ * The next stage starts with a SET and empty slots; the last stage's value is the result.  Softmax over
+ * rows is three stages of one program, a layer normalisation three as well.  Rows of at most 4096
+ * elements, reduce_op = -1, HIPNX_FUSED_COMPILED only (HIPNX_EUNSUPPORTED otherwise). */
 enum { HIPNX_FUSED_SAVED = 3, HIPNX_FUSED_MAX_INSTR = 32, HIPNX_FUSED_MAX_INPUTS = 8, HIPNX_FUSED_STATS = 3 };
 typedef struct {
   uint8_t kind, op, src, arg;

@@ -187,7 +187,8 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
   unsigned saved = 0;  // slots that hold a value so far
   unsigned raw_inputs = 0;  // inputs whose words are loaded unconverted
   bool have_acc = false, full = false, needs_compiled = false;
-  int n_stats = 0;  // row statistics produced so far (HIPNX_FUSED_ROW_REDUCE markers)
+  int n_stats = 0;       // row statistics kept so far (HIPNX_FUSED_ROW_STAT)
+  bool on_stat = false;  // between a stage's reduction and its ROW_STAT
   auto int32 = [](int dt) { return dt == HIPNX_U32 || dt == HIPNX_S32; };
   auto source_ok = [&](int src, int arg, const char **why) {
     if (src == HIPNX_FUSED_SRC_INPUT && arg >= n_inputs) { *why = "reads an input that is not there"; return false; }
@@ -239,12 +240,16 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
       case HIPNX_FUSED_BITCAST: break;
       case HIPNX_FUSED_ROW_REDUCE:
         if (q.op != HIPNX_RED_SUM && q.op != HIPNX_RED_MAX && q.op != HIPNX_RED_MIN) return set_error(HIPNX_EUNSUPPORTED, "fused: stage reduction %d", q.op);
-        if (n_stats >= HIPNX_FUSED_STATS || q.arg != n_stats) return set_error(HIPNX_EINVAL, "fused: instruction %d is row statistic %d of at most %d, in order", i, q.arg, HIPNX_FUSED_STATS);
-        if (!narrow(q.dt) || i == 0 || !narrow(prog[i - 1].dt) || i == n_instr - 1)
-          return set_error(HIPNX_EINVAL, "fused: instruction %d reduces a non-float value, or nothing follows it", i);
+        if (on_stat || !narrow(q.dt) || i == 0 || !narrow(prog[i - 1].dt))
+          return set_error(HIPNX_EINVAL, "fused: instruction %d reduces a non-float value, or a row statistic", i);
         if (q.flags) return set_error(HIPNX_EINVAL, "fused: instruction %d: a stage reduction takes no flags", i);
-        n_stats++;
+        on_stat = true;  // until the ROW_STAT that keeps it, instructions work on one value per row
         needs_compiled = true;
+        break;
+      case HIPNX_FUSED_ROW_STAT:
+        if (!on_stat || n_stats >= HIPNX_FUSED_STATS || q.arg != n_stats || i == n_instr - 1 || !narrow(prog[i - 1].dt))
+          return set_error(HIPNX_EINVAL, "fused: instruction %d keeps row statistic %d: at most %d, in order, after a stage reduction, and a last stage follows", i, q.arg, HIPNX_FUSED_STATS);
+        if (q.flags) return set_error(HIPNX_EINVAL, "fused: instruction %d: keeping a row statistic takes no flags", i);
         break;
       case HIPNX_FUSED_SELECT:
         if (!source_ok(q.src, q.arg, &why) || !source_ok(q.src2, q.arg2, &why))
@@ -255,8 +260,16 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
         break;
       default: return set_error(HIPNX_EINVAL, "fused: instruction %d has kind %d", i, q.kind);
     }
-    have_acc = q.kind != HIPNX_FUSED_ROW_REDUCE;  // the next stage starts from nothing
-    if (q.kind == HIPNX_FUSED_ROW_REDUCE) saved = 0;
+    if (on_stat && q.kind != HIPNX_FUSED_ROW_REDUCE && q.kind != HIPNX_FUSED_ROW_STAT) {
+      // work on the statistic: nothing is loaded per element here, and nothing is set aside
+      const bool reads_input = (q.kind == HIPNX_FUSED_BINARY || q.kind == HIPNX_FUSED_SELECT || q.kind == HIPNX_FUSED_SET) &&
+                               (q.src == HIPNX_FUSED_SRC_INPUT || q.src == HIPNX_FUSED_SRC_SAVED ||
+                                (q.kind == HIPNX_FUSED_SELECT && (q.src2 == HIPNX_FUSED_SRC_INPUT || q.src2 == HIPNX_FUSED_SRC_SAVED)));
+      if (reads_input || q.kind == HIPNX_FUSED_SET || (q.flags >> 4) || ints)
+        return set_error(HIPNX_EINVAL, "fused: instruction %d works on a row statistic with something other than constants and earlier statistics", i);
+    }
+    have_acc = q.kind != HIPNX_FUSED_ROW_STAT;  // the next stage starts from nothing
+    if (q.kind == HIPNX_FUSED_ROW_STAT) { saved = 0; on_stat = false; n_stats++; }
     if (q.flags >> 4) {
       if ((q.flags >> 4) > HIPNX_FUSED_SAVED) return set_error(HIPNX_EINVAL, "fused: instruction %d saves to slot %d", i, (q.flags >> 4) - 1);
       saved |= 1u << ((q.flags >> 4) - 1);
@@ -266,6 +279,7 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
   if (int_out != int32(prog[n_instr - 1].dt)) return set_error(HIPNX_EINVAL, "fused: result type %d after a program that ends in type %d", out_dt, prog[n_instr - 1].dt);
   if (needs_compiled && ctx->fused_mode != HIPNX_FUSED_COMPILED)
     return set_error(HIPNX_EUNSUPPORTED, "fused: 32-bit integer instructions and stages need the compiled mode");
+  if (on_stat) return set_error(HIPNX_EINVAL, "fused: the program ends inside a stage's work on its statistic");
   if (n_stats && (reduce_op != -1 || cols > 4096 || cols == 0))
     return set_error(HIPNX_EUNSUPPORTED, "fused: stages take rows of 1 .. 4096 elements and no reduction of the result");
   const int64_t n = rows * cols;

@@ -345,9 +345,10 @@ __device__ __forceinline__ float as_stored(CT v, int dt) {
 
 template <typename P, int SEG>
 __device__ __forceinline__ void row_stage(KernArgs a, int64_t r, int lane, RowStats &stats) {
-  constexpr int begin = SEG == 0 ? 0 : P::seg_end[SEG - 1] + 1;  // past the previous stage's marker
-  constexpr int end = P::seg_end[SEG];
-  constexpr int red = P::seg_red[SEG];
+  // stage SEG: instructions [begin, red) on the row's elements, the reduction at `red`, instructions
+  // (red, save) on the statistic, which is kept at `save`; the last stage is [begin, n_instr)
+  constexpr int begin = SEG == 0 ? 0 : P::seg_save[SEG - 1] + 1;
+  constexpr int red = P::seg_red[SEG], save = P::seg_save[SEG];
   const int64_t cols = a->cols, step = (int64_t)WAVE * FE;
   if constexpr (red < 0) {  // the last stage: its value is the result
     void *out = (void *)a->out;
@@ -355,7 +356,7 @@ __device__ __forceinline__ void row_stage(KernArgs a, int64_t r, int lane, RowSt
       const int64_t row[FV] = {r}, col[FV] = {k};
       Vecs x;
       Saved S;
-      static_steps<P, begin, end>(a, row, col, x, S, stats);
+      static_steps<P, begin, P::n_instr>(a, row, col, x, S, stats);
       if constexpr (P::out_dt == HIPNX_U32 || P::out_dt == HIPNX_S32) {
         uint4 *p = reinterpret_cast<uint4 *>((uint32_t *)out + r * cols + k);
         p[0] = make_uint4(__float_as_uint(x[0][0]), __float_as_uint(x[0][1]), __float_as_uint(x[0][2]), __float_as_uint(x[0][3]));
@@ -365,19 +366,27 @@ __device__ __forceinline__ void row_stage(KernArgs a, int64_t r, int lane, RowSt
       }
     }
   } else {
-    typedef typename std::conditional<red == HIPNX_RED_SUM, double, float>::type CT;
-    typedef PlainReducer<CT, red, false> R;
+    constexpr int op = P::op[red];
+    typedef typename std::conditional<op == HIPNX_RED_SUM, double, float>::type CT;
+    typedef PlainReducer<CT, op, false> R;
     typename R::acc_t acc = R::init();
     for (int64_t k = (int64_t)lane * FE; k < cols; k += step) {
       const int64_t row[FV] = {r}, col[FV] = {k};
       Vecs x;
       Saved S;
-      static_steps<P, begin, end>(a, row, col, x, S, stats);
+      static_steps<P, begin, red>(a, row, col, x, S, stats);
 #pragma unroll
       for (int e = 0; e < FE; e++) acc = R::accumulate(acc, (CT)x[0][e], k + e);
     }
     acc = wave_reduce<R>(acc);  // the butterfly leaves the same value in every lane
-    stats[SEG] = as_stored<CT>(acc, P::seg_dt[SEG]);
+    // the work on the statistic: the same instructions on a vector that holds it eight times
+    const int64_t row[FV] = {r}, col[FV] = {0};
+    Vecs x;
+    Saved S;
+#pragma unroll
+    for (int e = 0; e < FE; e++) x[0][e] = as_stored<CT>(acc, P::dt[red]);
+    static_steps<P, red + 1, save>(a, row, col, x, S, stats);
+    stats[P::arg[save]] = x[0][0];
     row_stage<P, SEG + 1>(a, r, lane, stats);
   }
 }

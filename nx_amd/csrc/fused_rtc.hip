@@ -75,15 +75,16 @@ static std::string make_source(const FusedArgs &a, int reduce_op, bool block_per
   list_of(s, "imm2", "unsigned", a.n_instr, [&](int i) { return std::to_string(q[i].imm2_bits) + "u"; });
   list_of(s, "in_dt", "int", a.n_inputs, [&](int k) { return std::to_string(a.in_dt[k]); });
   list_of(s, "in_cs", "int", a.n_inputs, [&](int k) { return std::to_string(a.in_cs[k]); });
-  // stages: where each ends (its marker, or the end of the program), what it reduces with, the statistic's type
-  std::vector<int> seg_end, seg_red, seg_dt;
-  for (int i = 0; i < a.n_instr; i++)
-    if (q[i].kind == HIPNX_FUSED_ROW_REDUCE) { seg_end.push_back(i); seg_red.push_back(q[i].op); seg_dt.push_back(q[i].dt); }
-  const bool stages = !seg_end.empty();
-  seg_end.push_back(a.n_instr); seg_red.push_back(-1); seg_dt.push_back(a.out_dt);
-  list_of(s, "seg_end", "int", (int)seg_end.size(), [&](int k) { return std::to_string(seg_end[k]); });
+  // stages: where each one's reduction and the end of its work on the statistic are (-1, n_instr for the last)
+  std::vector<int> seg_red, seg_save;
+  for (int i = 0; i < a.n_instr; i++) {
+    if (q[i].kind == HIPNX_FUSED_ROW_REDUCE) seg_red.push_back(i);
+    if (q[i].kind == HIPNX_FUSED_ROW_STAT) seg_save.push_back(i);
+  }
+  const bool stages = !seg_red.empty();
+  seg_red.push_back(-1); seg_save.push_back(a.n_instr);
   list_of(s, "seg_red", "int", (int)seg_red.size(), [&](int k) { return std::to_string(seg_red[k]); });
-  list_of(s, "seg_dt", "int", (int)seg_dt.size(), [&](int k) { return std::to_string(seg_dt[k]); });
+  list_of(s, "seg_save", "int", (int)seg_save.size(), [&](int k) { return std::to_string(seg_save[k]); });
   s += "};\n}\nusing namespace hipnx;\nextern \"C\" __global__ void __launch_bounds__(FBLOCK) fused_group(FusedArgs by_value) {\n  (void)by_value;\n";
   const char *tpr = block_per_row ? "FBLOCK" : "WAVE";
   if (stages) s += "  fused_row_stages_body<P>();\n";

@@ -775,7 +775,7 @@ def _absorb_scales(order: List[Tensor], uses) -> int:
 
 
 def _fuse_planned(roots: List[Tensor]) -> int:
-    order, uses, seen = [], {}, set()
+    order, uses, seen, parents = [], {}, set(), {}
 
     def walk(t):
         e = t.data
@@ -787,8 +787,18 @@ def _fuse_planned(roots: List[Tensor]) -> int:
         seen.add(e.id)
         for child in _children(e):
             if isinstance(child, Tensor):
+                parents.setdefault(child.data.id, []).append(t)
                 walk(child)
         order.append(t)
+
+    def feeds_a_row_reduction(t):
+        """Whether the only reader of `t` reduces it over its last axis: one node and that reduction
+        are worth a kernel of their own (the node's value is never stored)."""
+        readers = parents.get(t.data.id, [])
+        if len(readers) != 1 or uses.get(t.data.id) != 1 or len(t.shape) == 0:
+            return False
+        r = readers[0].data
+        return (r.op in _REDUCE_CODES and isinstance(r.args[0], Tensor) and r.args[0].data.id == t.data.id and list(r.args[1].get("axes") or []) == [len(t.shape) - 1])
 
     for r in roots:
         walk(r)
@@ -797,6 +807,7 @@ def _fuse_planned(roots: List[Tensor]) -> int:
     if _absorb_scales(order, uses):
         uses.clear()
         seen.clear()
+        parents.clear()
         del order[:]
         for r in roots:
             walk(r)
@@ -871,11 +882,18 @@ def _fuse_planned(roots: List[Tensor]) -> int:
     for root in reversed(order):  # consumers first: a group grows from its last node upwards
         if root.data.id in taken or uses.get(root.data.id, 0) == 0 or not _fusable(root):
             continue
+        if _plan["ints"] and len(root.shape) >= 2 and root.shape[-1] == 1:
+            continue  # work on one value per row: left as nodes, so that it can join the stage that makes the value
         members, shared, inside = grow(root, recompute=True)
-        group, inputs = build(root, members) if len(members) >= 2 else (None, None)
+        # a single node is no group -- unless the plan may join it to the stages that make its per-row operands
+        least = 1 if _plan["ints"] and any(isinstance(a, Tensor) and _const(a) is None and len(a.shape) >= 2
+                                           and a.shape[-1] == 1 for a in root.data.args) else 2
+        if feeds_a_row_reduction(root):
+            least = 1
+        group, inputs = build(root, members) if len(members) >= least else (None, None)
         if group is not None and shared and (group.program is None or group.layout is None):
             members, shared, inside = grow(root, recompute=False)  # too big with the recomputed parts: without them
-            group, inputs = build(root, members) if len(members) >= 2 else (None, None)
+            group, inputs = build(root, members) if len(members) >= least else (None, None)
         if group is None:
             continue
         taken.update(i for i in members if i not in shared)
@@ -920,17 +938,18 @@ def _fuse_planned(roots: List[Tensor]) -> int:
 
 
 class _RowCluster:
-    """Fused groups over the same rows as stages of one program: every group but the last ends in a
-    reduction along the row, later groups read its result (`stages` are (node, group, inputs) in
-    evaluation order, `final` the element-wise group that produces the result).  A backend that
-    cannot run the program gets the groups one by one."""
+    """Fused groups over the same rows as stages of one program.  Every stage but the last reduces
+    its value along the row, may work on that one value per row (a sum divided by the row length),
+    and keeps it as a row statistic that later stages read.  `steps` are the original nodes in
+    evaluation order, the last one the element-wise group that produces the result: a backend
+    that cannot run the program gets them one by one."""
 
     reduce = None
     how = {"mode": "compiled"}
 
-    def __init__(self, stages, final, inputs, program, layout):
-        self.stages, self.final, self.inputs, self.program, self.layout = stages, final, inputs, program, layout
-        self.root = final[0]
+    def __init__(self, steps, inputs, program, layout, n_stages):
+        self.steps, self.inputs, self.program, self.layout, self.n_stages = steps, inputs, program, layout, n_stages
+        self.root = steps[-1]
 
     def run(self, run: "_Run", out: Tensor, values: List[Tensor]):
         fused = getattr(run.pick(values), "fused_elementwise", None)
@@ -941,15 +960,24 @@ class _RowCluster:
                 if getattr(e, "status", None) != _EUNSUPPORTED:
                     raise
         known = {t.data.id: v for t, v in zip(self.inputs, values)}
-        for node, group, inputs in self.stages + [self.final]:
-            known[node.data.id] = group.run(run, node.with_(data=None), [known[t.data.id] for t in inputs])
+        for node in self.steps:
+            e = node.data
+            if e.op == "fused":
+                group, inputs = e.args
+                known[e.id] = group.run(run, node.with_(data=None), [known[t.data.id] for t in inputs])
+                continue
+            args = [(known[a.data.id] if a.data.id in known else run.eval(a, None)) if isinstance(a, Tensor) else a
+                    for a in e.args]
+            known[e.id] = getattr(run.pick(args), e.op)(node.with_(data=None), *args)
         return known[self.root.data.id]
 
 
 def _cluster_rows(roots: List[Tensor]) -> int:
-    """Rewrites an element-wise fused node together with the row-reducing fused nodes that only it
-    (and each other) read into one node holding a _RowCluster.  Rows of at most 4096 elements:
-    the width at which the separate reduction gives a row to one wave, whose order the stages keep."""
+    """Rewrites an element-wise fused node, together with what makes the per-row values only it
+    (and they themselves) read, into one node holding a _RowCluster.  A per-row value is a *stage*:
+    a reduction over the last axis -- of a fused group's value or of a tensor as it is -- followed
+    by a chain of element-wise nodes on the one value per row.  Rows of at most 4096 elements: the
+    width at which the separate reduction gives a row to one wave, whose order the stages keep."""
     order, readers, seen = [], {}, set()
 
     def walk(t):
@@ -981,65 +1009,151 @@ def _cluster_rows(roots: List[Tensor]) -> int:
         cols, rows = root.shape[-1], prod(root.shape[:-1])
         if cols > 4096 or cols % 8:
             continue
-        members = {e.id: root}
-
         per_row = tuple(root.shape[:-1]) + (1,)
 
-        def stage_of(t):
-            """The group behind `t` if it reduces a value of the root's shape along its rows and `t`
-            broadcasts against that shape as one value per row."""
-            g = t.data.args[0] if isinstance(t.data, Expr) and t.data.op == "fused" else None
-            ok = (isinstance(g, _Group) and g.reduce is not None and g.program and g.root.shape == root.shape
-                  and g.reduce[2][0] == rows and g.reduce[2][1] == cols and t.type in _NARROW
-                  and (1,) * (rank - len(t.shape)) + tuple(t.shape) == per_row)
-            return g if ok else None
+        def is_per_row(t):
+            return (isinstance(t, Tensor) and isinstance(t.data, Expr) and _const(t) is None and t.type in _NARROW
+                    and (1,) * (rank - len(t.shape)) + tuple(t.shape) == per_row)
 
+        def base_of(t):
+            """"group" / "reduce" when `t` is the reduction along the rows of a value of the root's shape."""
+            d = t.data
+            if d.op == "fused" and isinstance(d.args[0], _Group):
+                g = d.args[0]
+                if (g.reduce is not None and g.program and g.root.shape == root.shape and g.reduce[2][0] == rows
+                        and g.reduce[2][1] == cols):
+                    return "group"
+            if d.op in _REDUCE_CODES and isinstance(d.args[0], Tensor):
+                x, opts = d.args[0], d.args[1]
+                if (x.shape == root.shape and x.type in _NARROW and _const(x) is None
+                        and list(opts.get("axes") or []) == [rank - 1]):
+                    return "reduce"
+            return None
+
+        stages = {}  # id of the kept value -> (base node, [links from the base towards the kept value])
+
+        def stage_ending_at(t, inside):
+            """Registers the stage whose kept value is `t` (and the stages it reads), or returns False.
+            `inside`: ids of the readers the cluster already has."""
+            if t.data.id in stages:
+                return True
+            if not is_per_row(t) or not readers.get(t.data.id, set()) <= inside:
+                return False
+            links, cur = [], t
+            while base_of(cur) is None:
+                d = cur.data
+                if d.op not in UNARY_OPS and d.op not in BINARY_OPS and d.op != "as_type":
+                    return False
+                if not _fusable(cur):
+                    return False
+                operands = [a for a in d.args if isinstance(a, Tensor) and _const(a) is None]
+                if not operands or not all(is_per_row(a) for a in operands):
+                    return False
+                # the chain continues through the operand computed last; any other one is a kept value of another stage
+                chain = max(operands, key=lambda a: position.get(a.data.id, -1))
+                if readers.get(chain.data.id, set()) != {d.id} and chain.data.id not in stages:
+                    return False
+                if chain.data.id in stages:  # a chain that starts from a kept value, not from a reduction
+                    return False
+                links.append(cur)
+                cur = chain
+            links.reverse()
+            chain_ids = {cur.data.id} | {l.data.id for l in links}
+            # operands of the links that are not the chain itself, and per-row inputs of the base group
+            needs = [a for l in links for a in l.data.args
+                     if isinstance(a, Tensor) and _const(a) is None and a.data.id not in chain_ids]
+            if cur.data.op == "fused":
+                needs += [a for a in cur.data.args[1] if is_per_row(a)]
+            stages[t.data.id] = (cur, links)
+            for a in needs:
+                if a.data.id in stages:
+                    continue
+                if not stage_ending_at(a, inside | chain_ids):
+                    if any(a is x for l in links for x in l.data.args):
+                        del stages[t.data.id]  # a link's other operand must be a kept value
+                        return False
+            return True
+
+        # grow: per-row inputs of the root, then of the stages' groups, until nothing new is internal
         changed = True
         while changed:
             changed = False
-            for m in list(members.values()):
-                for t in m.data.args[1]:
-                    if t.data.id in members or stage_of(t) is None:
-                        continue
-                    if readers.get(t.data.id, set()) <= set(members):
-                        members[t.data.id] = t
-                        changed = True
-        if len(members) < 2 or len(members) - 1 > 3:
+            inside = {e.id} | {b.data.id for b, _ in stages.values()} | {l.data.id for _, ls in stages.values() for l in ls}
+            for t in [a for a in inputs if is_per_row(a)] + [a for b, _ in stages.values() if b.data.op == "fused"
+                                                             for a in b.data.args[1] if is_per_row(a)]:
+                if t.data.id not in stages and stage_ending_at(t, inside):
+                    changed = True
+        if not stages or len(stages) > 3:
             continue
-        stage_nodes = sorted((t for i, t in members.items() if i != e.id), key=lambda t: position[t.data.id])
-        number = {t.data.id: k for k, t in enumerate(stage_nodes)}
+        kept = sorted(stages, key=lambda i: position[stages[i][0].data.id])
+        slot = {i: k for k, i in enumerate(kept)}
         union, index = [], {}
+
+        def external(t):
+            if t.data.id not in index:
+                index[t.data.id] = len(union)
+                union.append(t)
+            return index[t.data.id]
 
         def remap(ins, key_src, key_arg, own_inputs):
             if ins.get(key_src, 0) != 1:
                 return
             t = own_inputs[ins.get(key_arg, 0)]
-            if t.data.id in number:
-                ins[key_src], ins[key_arg] = 3, number[t.data.id]
+            if t.data.id in slot:
+                ins[key_src], ins[key_arg] = 3, slot[t.data.id]
             else:
-                if t.data.id not in index:
-                    index[t.data.id] = len(union)
-                    union.append(t)
-                ins[key_arg] = index[t.data.id]
+                ins[key_arg] = external(t)
 
-        program = _Program()
-        for t in stage_nodes + [root]:
-            g, own = t.data.args
+        def group_program(node):
+            g, own = node.data.args
             for ins in g.program:
                 ins = dict(ins)
                 remap(ins, "src", "arg", own)
                 if ins["kind"] == 3:
                     remap(ins, "src2", "arg2", own)
                 program.append(ins)
-            if t is not root:
-                program.append({"kind": 6, "op": _REDUCE_CODES[g.reduce[0]], "arg": number[t.data.id], "dt": t.type})
+
+        program, steps, fits = _Program(), [], True
+        for i in kept:
+            base, links = stages[i]
+            if base.data.op == "fused":
+                group_program(base)
+                code = _REDUCE_CODES[base.data.args[0].reduce[0]]
+            else:
+                x = base.data.args[0]
+                program.append({"kind": 0, "src": 1, "arg": external(x), "dt": x.type})
+                code = _REDUCE_CODES[base.data.op]
+            program.append({"kind": 6, "op": code, "dt": base.type})
+            steps.append(base)
+            chain = base
+            for l in links:
+                d = l.data
+                ins = {"dt": l.type}
+                if d.op in UNARY_OPS:
+                    ins.update(kind=1, op=UNARY_OPS.index(d.op))
+                elif d.op == "as_type":
+                    ins.update(kind=4)
+                else:
+                    pos = next(p for p, a in enumerate(d.args) if isinstance(a, Tensor) and a.data.id == chain.data.id)
+                    other = d.args[1 - pos]
+                    ins.update(kind=2, op=BINARY_OPS.index(d.op), flags=1 if pos == 1 else 0)
+                    if _const(other) is not None:
+                        ins.update(src=0, imm=_imm(other))
+                    elif other.data.id in slot and slot[other.data.id] < slot[i]:
+                        ins.update(src=3, arg=slot[other.data.id])
+                    else:
+                        fits = False
+                program.append(ins)
+                steps.append(l)
+                chain = l
+            program.append({"kind": 7, "arg": slot[i], "dt": chain.type})
+        group_program(root)
         layout = _layout(root.shape, [t.shape for t in union], split=rank - 1)
-        if layout is None or len(program) > _MAX_INSTR or len(union) > _MAX_INPUTS:
+        if not fits or layout is None or len(program) > _MAX_INSTR or len(union) > _MAX_INPUTS:
             continue
-        # the pieces keep their own nodes (copies) for a backend that runs them one by one
-        stages = [(t.with_(data=Expr(t.data.id, "fused", t.data.args, 0)), t.data.args[0], t.data.args[1]) for t in stage_nodes]
-        final = (root.with_(data=Expr(e.id, "fused", e.args, 0)), group, inputs)
-        e.args = [_RowCluster(stages, final, union, program, layout), union]
+        # the root's own node is rewritten below: the steps keep a copy of it for a backend that runs them one by one
+        steps.append(root.with_(data=Expr(e.id, "fused", e.args, 0)))
+        e.args = [_RowCluster(steps, union, program, layout, len(kept)), union]
         formed += 1
     return formed
 

@@ -332,9 +332,9 @@ def test_softmax_is_one_node_with_three_stages_and_falls_back_group_by_group(on_
     args = build_args(on_oracle)["softmax"]
     planned = defn.compile(CHAINS["softmax"], *args, fuse="compiled")
     cluster = planned.roots[0].data.args[0]
-    assert type(cluster).__name__ == "_RowCluster" and len(cluster.stages) == 2
+    assert type(cluster).__name__ == "_RowCluster" and cluster.n_stages == 2
     kinds = [ins["kind"] for ins in cluster.program]
-    assert kinds.count(6) == 2 and kinds[-1] != 6          # two stage reductions, then the division
+    assert kinds.count(6) == 2 and kinds.count(7) == 2 and kinds[-1] not in (6, 7)  # two stages, then the division
     assert [ins["op"] for ins in cluster.program if ins["kind"] == 6] == [1, 0]  # the maximum, then the sum
     assert any(ins.get("src") == 3 for ins in cluster.program)                   # later stages read the row statistics
     assert len(cluster.inputs) == 1                                              # only the scores come from memory
@@ -363,3 +363,36 @@ def test_row_statistics_with_outside_readers_or_another_broadcast_stay_groups(on
     planned = defn.compile(stat_read_along_columns, sq, fuse="compiled")
     assert type(planned.roots[0].data.args[0]).__name__ != "_RowCluster"
     assert_bits_equal(planned(sq), stat_read_along_columns(sq), "per column")
+
+
+def test_statistics_that_are_worked_on_become_part_of_their_stage(on_oracle):
+    rng = np.random.default_rng(5)
+    x, gain = f32(rng.standard_normal((12, 64)), on_oracle), f32(rng.standard_normal((64,)), on_oracle)
+
+    def layer_norm(t, g):
+        n = t.shape[-1]
+        mean = Nx.divide(Nx.sum(t, axes=[-1], keep_axes=True), float(n))
+        c = Nx.subtract(t, mean)
+        var = Nx.divide(Nx.sum(Nx.multiply(c, c), axes=[-1], keep_axes=True), float(n))
+        return Nx.multiply(Nx.multiply(c, Nx.rsqrt(Nx.add(var, 1e-5))), g)
+
+    planned = defn.compile(layer_norm, x, gain, fuse="compiled")
+    cluster = planned.roots[0].data.args[0]
+    assert type(cluster).__name__ == "_RowCluster" and cluster.n_stages == 2
+    kinds = [ins["kind"] for ins in cluster.program]
+    first_red, first_keep = kinds.index(6), kinds.index(7)
+    assert kinds[:first_red] == [0]                       # the mean's stage reduces the tensor as it is
+    assert kinds[first_red + 1:first_keep] == [2]         # ... and divides the sum by the row length before keeping it
+    second_red, second_keep = kinds.index(6, first_keep), kinds.index(7, first_keep + 1)
+    assert kinds[second_red + 1:second_keep] == [2, 2, 1]  # / n, + eps, rsqrt
+    assert {t.data.op for t in cluster.inputs} == {"parameter"} and len(cluster.inputs) == 2
+    assert_bits_equal(planned(x, gain), layer_norm(x, gain), "layer norm, step by step on a backend without the kernel")
+
+    def log_softmax(t):    # the logarithm of the sum is work on the statistic too
+        z = Nx.subtract(t, Nx.reduce_max(t, axes=[-1], keep_axes=True))
+        return Nx.subtract(z, Nx.log(Nx.sum(Nx.exp(z), axes=[-1], keep_axes=True)))
+
+    planned = defn.compile(log_softmax, x, fuse="compiled")
+    cluster = planned.roots[0].data.args[0]
+    assert type(cluster).__name__ == "_RowCluster" and cluster.n_stages == 2
+    assert_bits_equal(planned(x), log_softmax(x), "log softmax")

@@ -625,19 +625,31 @@ def range_normalised(x):          # three statistics: minimum, maximum, and the 
     return Nx.divide(u, Nx.sum(u, axes=[-1], keep_axes=True))
 
 
+def log_softmax_rows(x):
+    z = Nx.subtract(x, Nx.reduce_max(x, axes=[-1], keep_axes=True))
+    return Nx.subtract(z, Nx.log(Nx.sum(Nx.exp(z), axes=[-1], keep_axes=True)))
+
+
+def rms_scaled(x):                # one statistic, worked on with two constants and a square root; bf16 rounds at every node
+    n = x.shape[-1]
+    ms = Nx.divide(Nx.sum(Nx.multiply(x, x), axes=[-1], keep_axes=True), float(n))
+    return Nx.divide(x, Nx.sqrt(Nx.add(ms, 1e-6)))
+
+
 @pytest.mark.parametrize("ty", ["f32", "bf16"])
 @pytest.mark.parametrize("shape", [(32, 512, 512), (100, 64), (7, 4096), (3, 5, 8), (1, 1024), (2049, 40)])
-@pytest.mark.parametrize("name", ["softmax_rows", "centred_and_scaled", "range_normalised"])
+@pytest.mark.parametrize("name", ["softmax_rows", "centred_and_scaled", "range_normalised", "log_softmax_rows", "rms_scaled"])
 def test_row_stages_are_bit_identical_to_node_by_node(name, shape, ty, hip):
     rng = np.random.default_rng(seed_of(name, shape, ty))
     x = rand_float(rng, ty, shape, hip)
     args = (x, rand_float(rng, ty, (shape[-1],), hip)) if name == "centred_and_scaled" else (x,)
-    fun = {"softmax_rows": softmax_rows, "centred_and_scaled": centred_and_scaled, "range_normalised": range_normalised}[name]
+    fun = {"softmax_rows": softmax_rows, "centred_and_scaled": centred_and_scaled, "range_normalised": range_normalised,
+           "log_softmax_rows": log_softmax_rows, "rms_scaled": rms_scaled}[name]
     want = defn.compile(fun, *args)(*args)
     planned = defn.compile(fun, *args, fuse="compiled")
-    # statistics that are worked on before they are used (the mean and the variance of the second function are
-    # divided by n first) keep their groups apart; statistics used as they are become stages of one program
-    staged = name != "centred_and_scaled"
+    # work on a statistic before it is used (the mean and the variance of the second function are divided by n,
+    # the variance goes through an rsqrt) belongs to the stage that makes it
+    staged = True
     assert (type(planned.roots[0].data.args[0]).__name__ == "_RowCluster") == staged
     calls = []
     original = hip.fused_elementwise.__func__
