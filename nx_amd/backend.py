@@ -807,9 +807,15 @@ class HipNxBackend:
         res = cls._alloc(out, dev)
         n = max(len(inputs), 1)
         handles = (C.c_void_p * n)(*[cls._handle(t) for t in inputs])
-        dts = (C.c_int * n)(*[T.code(t.type) for t in inputs])
-        rs = (C.c_int64 * n)(*[s[0] for s in strides])
-        cs = (C.c_int * n)(*[s[1] for s in strides])
+        # types and strides repeat from call to call of a traced function: kept with the layout they belong to
+        key = (id(layout), tuple(t.type for t in inputs))
+        cached = _fused_arrays.get(key)
+        if cached is None or cached[0] is not layout:
+            if len(_fused_arrays) > 4096:
+                _fused_arrays.clear()
+            cached = _fused_arrays[key] = (layout, (C.c_int * n)(*[T.code(t.type) for t in inputs]),
+                                           (C.c_int64 * n)(*[s[0] for s in strides]), (C.c_int * n)(*[s[1] for s in strides]))
+        _, dts, rs, cs = cached
         L.check(L.lib.hipnx_fused_elementwise(res.data.ref.ctx, len(program), C.cast(prog, C.c_void_p), len(inputs), handles,
                                               dts, rs, cs, rows, cols, reduce_op, T.code(out.type), res.data.ref.handle))
         return res
@@ -941,6 +947,7 @@ def fused_mode(mode: str, device: int = 0) -> None:
 
 
 _fused_modes = {}  # device -> the mode last set here
+_fused_arrays = {}  # (id of a layout, input types) -> (the layout itself, so the id stays its own; C arrays of types and strides)
 
 
 def fused_compiled_count(device: int = 0) -> int:
