@@ -232,3 +232,16 @@ def test_put_slice_with_tensor_start_indices(hip, oracle):
     hi = [from_numpy(np.array(7, dtype=np.int32), "s32", hip), from_numpy(np.array(100, dtype=np.int64), "s64", hip)]
     oi = [from_numpy(np.array(7, dtype=np.int32), "s32", oracle), from_numpy(np.array(100, dtype=np.int64), "s64", oracle)]
     assert_bits_equal(Nx.put_slice(ht, hi, hs), Nx.put_slice(ot, oi, os_), "put_slice with tensor starts")
+
+
+@pytest.mark.parametrize("ty", ["f32", "bf16"])  # f16 overflows here: the reference raises, the device writes infinities
+def test_iota_beyond_the_exact_integers_of_f32(ty, hip, oracle):
+    # above 2^24 the integer -> float conversion rounds: to nearest even, once (binary_backend.ex:49-75 writes the
+    # integer as a float of the type)
+    n = (1 << 25) + 24
+    got = Nx.iota((n,), type=ty, backend=hip)
+    if ty == "f32":
+        np.testing.assert_array_equal(hip.to_numpy(got), np.arange(n, dtype=np.int64).astype(np.float32))
+    tail = Nx.slice(got, [n - 4096], [4096])
+    want = Nx.slice(Nx.iota((n,), type=ty, backend=oracle), [n - 4096], [4096])
+    assert_bits_equal(tail, want, f"iota {ty} tail")
