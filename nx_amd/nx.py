@@ -296,6 +296,13 @@ def sum(t, axes=None, keep_axes=False):  # noqa: A001 - Nx.sum/2 (nx.ex:9622-962
     return _aggregate(t, "sum", T.to_aggregate(t.type), axes, keep_axes)
 
 
+def mean(t, axes=None, keep_axes=False):
+    """Nx.mean/2 (nx.ex:9745-9761): the sum divided by the number of reduced entries."""
+    t = to_tensor(t)
+    count = t.size if axes is None else prod(t.shape[a] for a in S.normalize_axes(t.shape, axes))
+    return divide(sum(t, axes=axes, keep_axes=keep_axes), count)
+
+
 def product(t, axes=None, keep_axes=False):
     t = to_tensor(t)
     return _aggregate(t, "product", T.to_aggregate(t.type), axes, keep_axes)
@@ -459,6 +466,36 @@ class BlockThreefry:
     nx/lib/nx/random.ex:214-229) as a block, so a backend can produce the words in one step.  The
     reference composes it from callbacks without a block; the words are the same."""
     shape: tuple
+
+
+@dataclass(frozen=True)
+class BlockAllClose:
+    """%Nx.Block.AllClose{equal_nan, rtol, atol} (nx/lib/nx/block.ex:37-39)."""
+    equal_nan: bool = False
+    rtol: float = 1.0e-5
+    atol: float = 1.0e-8
+
+
+def all_close(a, b, equal_nan=False, rtol=1.0e-5, atol=1.0e-8):
+    """Nx.all_close/3 (nx.ex:9401-9452): |a - b| <= atol + rtol * |b| everywhere, infinities equal to
+    themselves only, NaNs equal to each other on request.  Runs on the backend of its arguments,
+    through block/4 like the reference."""
+    a, b = to_tensor(a), to_tensor(b)
+
+    def compose(o, x, y):
+        both_int = T.is_integer(x.type) and T.is_integer(y.type)
+        # abs of the lowest signed value overflows in its own width: widen first (nx.ex:9423-9427)
+        abs_y = abs(as_type(y, "f64")) if both_int else abs(y)
+        finite = less_equal(abs(subtract(x, y)), add(o.atol, multiply(o.rtol, abs_y)))
+        if both_int:
+            return all(finite)
+        # inf - inf is a NaN, yet the two are equal: equal entries are checked as such
+        entries = select(logical_or(is_infinity(x), is_infinity(y)), equal(x, y), finite)
+        if o.equal_nan:
+            entries = select(logical_and(is_nan(x), is_nan(y)), 1, entries)
+        return all(entries)
+
+    return block(BlockAllClose(equal_nan, rtol, atol), [a, b], template(("u", 8), ()), compose)
 
 
 def block(struct, args, out, fun):
