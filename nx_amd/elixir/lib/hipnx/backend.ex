@@ -444,6 +444,39 @@ defmodule HipNx.Backend do
   end
 
   @impl true
+  def to_batched(%T{shape: out_shape} = out, %T{shape: shape} = t, opts) do
+    # byte windows of the leading axis, lazily; a short last batch wraps to the first entries
+    # (binary_backend.ex:178-211)
+    device = device_of([t])
+    {ref, _} = from_nx(t, device)
+    batch = elem(out_shape, 0)
+    total = elem(shape, 0)
+    row = div(bytes(t), max(total, 1))
+    full = div(total, batch)
+    rest = rem(total, batch)
+    last = if rest != 0 and opts[:leftover] == :repeat, do: full, else: full - 1
+
+    window = fn buf, first, count, at ->
+      if count * row > 0 do
+        unwrap!(NIF.strided_copy(ctx(device), 1, [count * row], [1], first * row, [1], at * row, ref, buf))
+      end
+    end
+
+    Stream.map(0..last//1, fn i ->
+      buf = unwrap!(NIF.alloc(ctx(device), bytes(out)))
+
+      if i < full do
+        window.(buf, i * batch, batch, 0)
+      else
+        window.(buf, full * batch, rest, 0)
+        window.(buf, 0, batch - rest, rest)
+      end
+
+      to_nx(buf, device, out)
+    end)
+  end
+
+  @impl true
   def pad(_out, %T{shape: {}} = t, _pad_value, _config), do: t
 
   def pad(%T{shape: out_shape, type: {_, bits} = type} = out, %T{shape: shape} = t, %T{} = pad_value, config) do
