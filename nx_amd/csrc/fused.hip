@@ -189,6 +189,7 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
   bool have_acc = false, full = false, needs_compiled = false;
   int n_stats = 0;       // row statistics kept so far (HIPNX_FUSED_ROW_STAT)
   bool on_stat = false;  // between a stage's reduction and its ROW_STAT
+  bool row_result = false;  // the program ends in a ROW_STAT that is the result: one value per row
   auto int32 = [](int dt) { return dt == HIPNX_U32 || dt == HIPNX_S32; };
   auto source_ok = [&](int src, int arg, const char **why) {
     if (src == HIPNX_FUSED_SRC_INPUT && arg >= n_inputs) { *why = "reads an input that is not there"; return false; }
@@ -247,9 +248,15 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
         needs_compiled = true;
         break;
       case HIPNX_FUSED_ROW_STAT:
+        if (q.flags == HIPNX_FUSED_FLAG_RESULT) {  // the value per row is the result: nothing follows
+          if (!on_stat || i != n_instr - 1 || !narrow(prog[i - 1].dt) || q.dt != out_dt)
+            return set_error(HIPNX_EINVAL, "fused: instruction %d: a row result ends the program, after a stage reduction, in the result's type", i);
+          row_result = true;
+          break;
+        }
         if (!on_stat || n_stats >= HIPNX_FUSED_STATS || q.arg != n_stats || i == n_instr - 1 || !narrow(prog[i - 1].dt))
           return set_error(HIPNX_EINVAL, "fused: instruction %d keeps row statistic %d: at most %d, in order, after a stage reduction, and a last stage follows", i, q.arg, HIPNX_FUSED_STATS);
-        if (q.flags) return set_error(HIPNX_EINVAL, "fused: instruction %d: keeping a row statistic takes no flags", i);
+        if (q.flags) return set_error(HIPNX_EINVAL, "fused: instruction %d: keeping a row statistic takes no flags but the result mark", i);
         break;
       case HIPNX_FUSED_SELECT:
         if (!source_ok(q.src, q.arg, &why) || !source_ok(q.src2, q.arg2, &why))
@@ -269,7 +276,7 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
         return set_error(HIPNX_EINVAL, "fused: instruction %d works on a row statistic with something other than constants and earlier statistics", i);
     }
     have_acc = q.kind != HIPNX_FUSED_ROW_STAT;  // the next stage starts from nothing
-    if (q.kind == HIPNX_FUSED_ROW_STAT) { saved = 0; on_stat = false; n_stats++; }
+    if (q.kind == HIPNX_FUSED_ROW_STAT) { saved = 0; on_stat = false; n_stats++; }  // (a row result counts as a stage too)
     if (q.flags >> 4) {
       if ((q.flags >> 4) > HIPNX_FUSED_SAVED) return set_error(HIPNX_EINVAL, "fused: instruction %d saves to slot %d", i, (q.flags >> 4) - 1);
       saved |= 1u << ((q.flags >> 4) - 1);
@@ -310,7 +317,7 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
     // a few very long rows are split into segments by the separate reduction: not here
     if (rows < (int64_t)ctx->num_cus * 8 && cols >= 2 * 16384) return set_error(HIPNX_EUNSUPPORTED, "fused: rows that the reduction would split");
   }
-  if (int st = check_buf(ctx, out, (uint64_t)(reduce_op == -1 ? n : rows) * dtype_size(out_dt), "fused out")) return st;
+  if (int st = check_buf(ctx, out, (uint64_t)(reduce_op == -1 && !row_result ? n : rows) * dtype_size(out_dt), "fused out")) return st;
   if (n == 0) return HIPNX_OK;
   a.out = out->ptr;
   a.out_dt = out_dt;

@@ -386,8 +386,12 @@ __device__ __forceinline__ void row_stage(KernArgs a, int64_t r, int lane, RowSt
 #pragma unroll
     for (int e = 0; e < FE; e++) x[0][e] = as_stored<CT>(acc, P::dt[red]);
     static_steps<P, red + 1, save>(a, row, col, x, S, stats);
-    stats[P::arg[save]] = x[0][0];
-    row_stage<P, SEG + 1>(a, r, lane, stats);
+    if constexpr ((P::flags[save] & HIPNX_FUSED_FLAG_RESULT) != 0) {  // this one value per row is the result
+      if (lane == 0) store_one<float>((void *)a->out, P::out_dt, r, x[0][0]);
+    } else {
+      stats[P::arg[save]] = x[0][0];
+      row_stage<P, SEG + 1>(a, r, lane, stats);
+    }
   }
 }
 

@@ -82,7 +82,10 @@ static std::string make_source(const FusedArgs &a, int reduce_op, bool block_per
     if (q[i].kind == HIPNX_FUSED_ROW_STAT) seg_save.push_back(i);
   }
   const bool stages = !seg_red.empty();
-  seg_red.push_back(-1); seg_save.push_back(a.n_instr);
+  if (seg_save.size() < seg_red.size() || seg_save.empty() || seg_save.back() != a.n_instr - 1) {  // a last, element-wise stage
+    seg_red.push_back(-1);
+    seg_save.push_back(a.n_instr);
+  }
   list_of(s, "seg_red", "int", (int)seg_red.size(), [&](int k) { return std::to_string(seg_red[k]); });
   list_of(s, "seg_save", "int", (int)seg_save.size(), [&](int k) { return std::to_string(seg_save[k]); });
   s += "};\n}\nusing namespace hipnx;\nextern \"C\" __global__ void __launch_bounds__(FBLOCK) fused_group(FusedArgs by_value) {\n  (void)by_value;\n";

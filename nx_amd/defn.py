@@ -973,11 +973,13 @@ class _RowCluster:
 
 
 def _cluster_rows(roots: List[Tensor]) -> int:
-    """Rewrites an element-wise fused node, together with what makes the per-row values only it
-    (and they themselves) read, into one node holding a _RowCluster.  A per-row value is a *stage*:
-    a reduction over the last axis -- of a fused group's value or of a tensor as it is -- followed
-    by a chain of element-wise nodes on the one value per row.  Rows of at most 4096 elements: the
-    width at which the separate reduction gives a row to one wave, whose order the stages keep."""
+    """Rewrites a node, together with what makes the per-row values only it (and they themselves)
+    read, into one node holding a _RowCluster.  A per-row value is a *stage*: a reduction over the
+    last axis -- of a fused group's value or of a tensor as it is -- followed by a chain of
+    element-wise nodes on the one value per row.  The node that is rewritten is an element-wise fused
+    group over the full shape (a softmax, a layer normalisation), or itself such a per-row value
+    (a log-sum-exp).  Rows of at most 4096 elements: the width at which the separate reduction
+    gives a row to one wave, whose order the stages keep."""
     order, readers, seen = [], {}, set()
 
     def walk(t):
@@ -997,96 +999,111 @@ def _cluster_rows(roots: List[Tensor]) -> int:
         readers.setdefault(r.data.id, set()).add("result")
         walk(r)
     position = {t.data.id: i for i, t in enumerate(order)}
-    formed = 0
-    for root in order:
-        e = root.data
-        if e.op != "fused" or not isinstance(e.args[0], _Group):
-            continue
-        group, inputs = e.args
-        rank = len(root.shape)
-        if group.reduce is not None or not group.program or rank == 0:
-            continue
-        cols, rows = root.shape[-1], prod(root.shape[:-1])
-        if cols > 4096 or cols % 8:
-            continue
-        per_row = tuple(root.shape[:-1]) + (1,)
+    absorbed = set()  # nodes that have become part of a cluster
 
-        def is_per_row(t):
-            return (isinstance(t, Tensor) and isinstance(t.data, Expr) and _const(t) is None and t.type in _NARROW
-                    and (1,) * (rank - len(t.shape)) + tuple(t.shape) == per_row)
+    def reduced_shape(t):
+        """The full shape whose rows `t` reduces, when `t` is such a reduction."""
+        d = t.data
+        if d.op == "fused" and isinstance(d.args[0], _Group) and d.args[0].reduce is not None and d.args[0].program:
+            return tuple(d.args[0].root.shape)
+        if d.op in _REDUCE_CODES and isinstance(d.args[0], Tensor):
+            x, opts = d.args[0], d.args[1]
+            if x.type in _NARROW and _const(x) is None and list(opts.get("axes") or []) == [len(x.shape) - 1]:
+                return tuple(x.shape)
+        return None
+
+    def attempt(final, full_shape, row_valued):
+        e = final.data
+        rank = len(full_shape)
+        if rank == 0:
+            return False
+        cols, rows = full_shape[-1], prod(full_shape[:-1])
+        if cols > 4096 or cols % 8:
+            return False
+        per_row = tuple(full_shape[:-1]) + (1,)
+
+        def is_per_row(t, flat_too=False):
+            if not (isinstance(t, Tensor) and isinstance(t.data, Expr) and _const(t) is None and t.type in _NARROW):
+                return False
+            padded = (1,) * (rank - len(t.shape)) + tuple(t.shape)
+            return padded == per_row or (flat_too and tuple(t.shape) == tuple(full_shape[:-1]) and t.size == rows)
 
         def base_of(t):
-            """"group" / "reduce" when `t` is the reduction along the rows of a value of the root's shape."""
-            d = t.data
-            if d.op == "fused" and isinstance(d.args[0], _Group):
-                g = d.args[0]
-                if (g.reduce is not None and g.program and g.root.shape == root.shape and g.reduce[2][0] == rows
-                        and g.reduce[2][1] == cols):
-                    return "group"
-            if d.op in _REDUCE_CODES and isinstance(d.args[0], Tensor):
-                x, opts = d.args[0], d.args[1]
-                if (x.shape == root.shape and x.type in _NARROW and _const(x) is None
-                        and list(opts.get("axes") or []) == [rank - 1]):
-                    return "reduce"
-            return None
+            shape = reduced_shape(t)
+            if shape != tuple(full_shape):
+                return None
+            if t.data.op == "fused":
+                g = t.data.args[0]
+                return "group" if g.reduce[2][0] == rows and g.reduce[2][1] == cols else None
+            return "reduce"
 
         stages = {}  # id of the kept value -> (base node, [links from the base towards the kept value])
 
-        def stage_ending_at(t, inside):
+        def stage_ending_at(t, inside, is_final=False):
             """Registers the stage whose kept value is `t` (and the stages it reads), or returns False.
-            `inside`: ids of the readers the cluster already has."""
+            `inside`: ids of the readers the cluster already has (the final value may have any readers)."""
             if t.data.id in stages:
                 return True
-            if not is_per_row(t) or not readers.get(t.data.id, set()) <= inside:
+            if t.data.id in absorbed or not is_per_row(t, flat_too=is_final):
+                return False
+            if not is_final and not readers.get(t.data.id, set()) <= inside:
                 return False
             links, cur = [], t
             while base_of(cur) is None:
                 d = cur.data
-                if d.op not in UNARY_OPS and d.op not in BINARY_OPS and d.op != "as_type":
-                    return False
-                if not _fusable(cur):
+                if (d.op not in UNARY_OPS and d.op not in BINARY_OPS and d.op != "as_type") or not _fusable(cur):
                     return False
                 operands = [a for a in d.args if isinstance(a, Tensor) and _const(a) is None]
-                if not operands or not all(is_per_row(a) for a in operands):
+                if not operands or not all(is_per_row(a, flat_too=is_final) for a in operands):
                     return False
                 # the chain continues through the operand computed last; any other one is a kept value of another stage
                 chain = max(operands, key=lambda a: position.get(a.data.id, -1))
-                if readers.get(chain.data.id, set()) != {d.id} and chain.data.id not in stages:
-                    return False
-                if chain.data.id in stages:  # a chain that starts from a kept value, not from a reduction
+                if chain.data.id in stages or chain.data.id in absorbed or readers.get(chain.data.id, set()) != {d.id}:
                     return False
                 links.append(cur)
                 cur = chain
+                if len(links) > 12:
+                    return False
             links.reverse()
             chain_ids = {cur.data.id} | {l.data.id for l in links}
-            # operands of the links that are not the chain itself, and per-row inputs of the base group
-            needs = [a for l in links for a in l.data.args
-                     if isinstance(a, Tensor) and _const(a) is None and a.data.id not in chain_ids]
-            if cur.data.op == "fused":
-                needs += [a for a in cur.data.args[1] if is_per_row(a)]
+            others = [a for l in links for a in l.data.args
+                      if isinstance(a, Tensor) and _const(a) is None and a.data.id not in chain_ids]
             stages[t.data.id] = (cur, links)
-            for a in needs:
-                if a.data.id in stages:
-                    continue
+            for a in others:  # a link's other operand must be a kept value of a stage of this cluster
                 if not stage_ending_at(a, inside | chain_ids):
-                    if any(a is x for l in links for x in l.data.args):
-                        del stages[t.data.id]  # a link's other operand must be a kept value
-                        return False
+                    del stages[t.data.id]
+                    return False
+            if cur.data.op == "fused":  # per-row inputs of the base group join if they can (or stay inputs from memory)
+                for a in cur.data.args[1]:
+                    if is_per_row(a):
+                        stage_ending_at(a, inside | chain_ids)
             return True
 
-        # grow: per-row inputs of the root, then of the stages' groups, until nothing new is internal
+        if row_valued:
+            if not stage_ending_at(final, set(), is_final=True):
+                return False
+        # grow: per-row inputs of the final group, then of the stages' groups, until nothing new is internal
         changed = True
         while changed:
             changed = False
-            inside = {e.id} | {b.data.id for b, _ in stages.values()} | {l.data.id for _, ls in stages.values() for l in ls}
-            for t in [a for a in inputs if is_per_row(a)] + [a for b, _ in stages.values() if b.data.op == "fused"
-                                                             for a in b.data.args[1] if is_per_row(a)]:
+            inside = {b.data.id for b, _ in stages.values()} | {l.data.id for _, ls in stages.values() for l in ls}
+            pending = [a for b, _ in stages.values() if b.data.op == "fused" for a in b.data.args[1] if is_per_row(a)]
+            if not row_valued:
+                inside.add(e.id)
+                pending += [a for a in e.args[1] if is_per_row(a)]
+            for t in pending:
                 if t.data.id not in stages and stage_ending_at(t, inside):
                     changed = True
-        if not stages or len(stages) > 3:
-            continue
-        kept = sorted(stages, key=lambda i: position[stages[i][0].data.id])
+        if not stages or len(stages) > 3 + (1 if row_valued else 0):
+            return False
+        if row_valued and len(stages) < 2 and not stages[e.id][1]:
+            return False  # a lone reduction is what it already is
+        kept = sorted((i for i in stages if not (row_valued and i == e.id)), key=lambda i: position[stages[i][0].data.id])
+        if len(kept) > 3:
+            return False
         slot = {i: k for k, i in enumerate(kept)}
+        if row_valued:
+            kept.append(e.id)  # last, and not a statistic anyone reads: the result
         union, index = [], {}
 
         def external(t):
@@ -1139,22 +1156,49 @@ def _cluster_rows(roots: List[Tensor]) -> int:
                     ins.update(kind=2, op=BINARY_OPS.index(d.op), flags=1 if pos == 1 else 0)
                     if _const(other) is not None:
                         ins.update(src=0, imm=_imm(other))
-                    elif other.data.id in slot and slot[other.data.id] < slot[i]:
+                    elif other.data.id in slot and (i not in slot or slot[other.data.id] < slot[i]):
                         ins.update(src=3, arg=slot[other.data.id])
                     else:
                         fits = False
                 program.append(ins)
                 steps.append(l)
                 chain = l
-            program.append({"kind": 7, "arg": slot[i], "dt": chain.type})
-        group_program(root)
-        layout = _layout(root.shape, [t.shape for t in union], split=rank - 1)
+            if i in slot:
+                program.append({"kind": 7, "arg": slot[i], "dt": chain.type})
+            else:
+                program.append({"kind": 7, "arg": 0, "flags": 1, "dt": chain.type})  # the value per row is the result
+        if not row_valued:
+            group_program(final)
+        layout = _layout(full_shape, [t.shape for t in union], split=rank - 1)
         if not fits or layout is None or len(program) > _MAX_INSTR or len(union) > _MAX_INPUTS:
+            return False
+        if row_valued:
+            steps[-1] = steps[-1].with_(data=Expr(e.id, e.op, e.args, 0))  # (the final node is rewritten below)
+        else:
+            steps.append(final.with_(data=Expr(e.id, "fused", e.args, 0)))
+        for node in steps[:-1]:
+            absorbed.add(node.data.id)
+        absorbed.add(e.id)
+        e.op, e.args = "fused", [_RowCluster(steps, union, program, layout, len(kept)), union]
+        return True
+
+    formed = 0
+    for node in reversed(order):  # consumers first: the longest chain that ends in a value takes it
+        e = node.data
+        if e.id in absorbed:
             continue
-        # the root's own node is rewritten below: the steps keep a copy of it for a backend that runs them one by one
-        steps.append(root.with_(data=Expr(e.id, "fused", e.args, 0)))
-        e.args = [_RowCluster(steps, union, program, layout, len(kept)), union]
-        formed += 1
+        if e.op == "fused" and isinstance(e.args[0], _Group) and e.args[0].reduce is None and e.args[0].program:
+            formed += attempt(node, tuple(node.shape), False)
+            continue
+        # a per-row value: follow its chain down to the reduction it starts from
+        cur, depth = node, 0
+        while cur is not None and reduced_shape(cur) is None and depth < 12:
+            d = cur.data
+            operands = [a for a in d.args if isinstance(a, Tensor) and _const(a) is None] if d.op in UNARY_OPS or d.op in BINARY_OPS or d.op == "as_type" else []
+            cur = max(operands, key=lambda a: position.get(a.data.id, -1)) if operands else None
+            depth += 1
+        if cur is not None and reduced_shape(cur) is not None and node.type in _NARROW:
+            formed += attempt(node, reduced_shape(cur), True)
     return formed
 
 

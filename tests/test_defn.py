@@ -396,3 +396,30 @@ def test_statistics_that_are_worked_on_become_part_of_their_stage(on_oracle):
     cluster = planned.roots[0].data.args[0]
     assert type(cluster).__name__ == "_RowCluster" and cluster.n_stages == 2
     assert_bits_equal(planned(x), log_softmax(x), "log softmax")
+
+
+def test_a_per_row_result_is_a_cluster_too(on_oracle):
+    x = f32(np.random.default_rng(8).standard_normal((12, 64)), on_oracle)
+
+    def log_sum_exp(t):
+        m = Nx.reduce_max(t, axes=[-1], keep_axes=True)
+        return Nx.add(Nx.log(Nx.sum(Nx.exp(Nx.subtract(t, m)), axes=[-1], keep_axes=True)), m)
+
+    planned = defn.compile(log_sum_exp, x, fuse="compiled")
+    cluster = planned.roots[0].data.args[0]
+    assert type(cluster).__name__ == "_RowCluster" and cluster.n_stages == 2
+    last = cluster.program[-1]
+    assert last["kind"] == 7 and last.get("flags") == 1          # the program ends in the value per row
+    assert [ins["kind"] for ins in cluster.program].count(7) == 2
+    assert_bits_equal(planned(x), log_sum_exp(x), "log-sum-exp, step by step on a backend without the kernel")
+
+    def mean_and_squeeze(t):  # one stage: the sum and its division; the squeeze stays outside
+        return Nx.squeeze(Nx.mean(t, axes=[-1], keep_axes=True), axes=[1])
+
+    planned = defn.compile(mean_and_squeeze, x, fuse="compiled")
+    assert_bits_equal(planned(x), mean_and_squeeze(x), "mean")
+
+    def plain_sum(t):         # a lone reduction is left as it is
+        return Nx.sum(t, axes=[-1], keep_axes=True)
+
+    assert defn.compile(plain_sum, x, fuse="compiled").roots[0].data.op == "sum"

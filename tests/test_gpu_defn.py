@@ -679,3 +679,49 @@ def test_configuration_3_softmax_in_one_kernel(hip):
     planned = defn.compile(CHAINS["softmax"], *args, fuse="compiled")
     assert type(planned.roots[0].data.args[0]).__name__ == "_RowCluster"
     assert_bits_equal(planned(*args), defn.compile(CHAINS["softmax"], *args)(*args), "softmax of the scores")
+
+
+def log_sum_exp_rows(x):
+    m = Nx.reduce_max(x, axes=[-1], keep_axes=True)
+    return Nx.add(Nx.log(Nx.sum(Nx.exp(Nx.subtract(x, m)), axes=[-1], keep_axes=True)), m)
+
+
+def mean_rows(x):
+    return Nx.mean(x, axes=[-1], keep_axes=True)
+
+
+def root_mean_square_rows(x):
+    return Nx.sqrt(Nx.divide(Nx.sum(Nx.multiply(x, x), axes=[-1], keep_axes=True), float(x.shape[-1])))
+
+
+def spread_rows(x):               # the result reads two other statistics
+    lo = Nx.reduce_min(x, axes=[-1], keep_axes=True)
+    hi = Nx.reduce_max(x, axes=[-1], keep_axes=True)
+    return Nx.divide(Nx.sum(Nx.subtract(x, lo), axes=[-1], keep_axes=True), hi)
+
+
+@pytest.mark.parametrize("ty", ["f32", "bf16"])
+@pytest.mark.parametrize("shape", [(32, 512, 512), (100, 64), (7, 4096), (3, 5, 8), (1, 1024), (2049, 40)])
+@pytest.mark.parametrize("name", ["log_sum_exp_rows", "mean_rows", "root_mean_square_rows", "spread_rows"])
+def test_per_row_results_from_one_kernel_are_bit_identical(name, shape, ty, hip):
+    rng = np.random.default_rng(seed_of(name, shape, ty))
+    x = rand_float(rng, ty, shape, hip)
+    fun = {"log_sum_exp_rows": log_sum_exp_rows, "mean_rows": mean_rows, "root_mean_square_rows": root_mean_square_rows,
+           "spread_rows": spread_rows}[name]
+    want = defn.compile(fun, x)(x)
+    planned = defn.compile(fun, x, fuse="compiled")
+    cluster = planned.roots[0].data.args[0]
+    assert type(cluster).__name__ == "_RowCluster" and cluster.program[-1].get("flags") == 1
+    calls = []
+    original = hip.fused_elementwise.__func__
+
+    def counting(cls, *a, **k):
+        if "mode" in k:
+            calls.append(1)
+        return original(cls, *a, **k)
+    hip.fused_elementwise = classmethod(counting)
+    try:
+        assert_bits_equal(planned(x), want, f"{name} {shape} {ty}")
+    finally:
+        hip.fused_elementwise = classmethod(original)
+    assert calls == [1]
