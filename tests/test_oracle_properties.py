@@ -197,3 +197,25 @@ def test_mixed_integer_float_operands_promote_like_erlang(oracle):
     assert out.type == ("f", 32) and values(out).tolist() == [16777218.0, 3.5]
     d = Nx.divide(t(np.array([1, 2], dtype=np.int32), "s32", oracle), t(np.array([3, 3], dtype=np.int32), "s32", oracle))
     assert d.type == ("f", 32) and raw(d).tolist() == [np.float32(1 / 3), np.float32(2 / 3)]
+
+
+def test_f16_codec_against_the_reference_table_of_shortest_decimals(oracle):
+    """nx/test/fixtures/f16_table.txt (sampled, tests/golden/make_f16_sample.py) gives each f16 bit pattern
+    the shortest decimal that reads back as it: encoding that decimal must give the pattern, and
+    decoding the pattern must give the f16 nearest to the decimal -- on the oracle's own codec."""
+    import os
+    path = os.path.join(os.path.dirname(__file__), "golden", "f16_shortest_decimals_sample.txt")
+    bits, text = zip(*(line.strip().split(":") for line in open(path) if line.strip()))
+    bits = np.array([int(b, 16) for b in bits], dtype=np.uint16)
+    finite = np.array([t not in ("NaN", "-NaN", "Infinity", "-Infinity") for t in text])
+    decimals = np.array([float(t) if ok else 0.0 for t, ok in zip(text, finite)], dtype=np.float64)
+    # encode: the decimal, held as f64, written as f16 (binary_backend.ex:2031-2076 through the write path)
+    as_f64 = from_numpy(decimals[finite], "f64", oracle)
+    encoded = np.frombuffer(Nx.to_binary(Nx.as_type(as_f64, "f16")), dtype=np.uint16)
+    assert np.array_equal(encoded, bits[finite])
+    # decode: the pattern read as a number is the f16 value (and that value is what the decimal encodes to, above)
+    as_f16 = from_numpy(bits.view(np.float16), "f16", oracle)
+    decoded = np.frombuffer(Nx.to_binary(Nx.as_type(as_f16, "f64")), dtype=np.float64)
+    assert np.array_equal(decoded[finite], bits[finite].view(np.float16).astype(np.float64))
+    for t, d in zip(np.array(text)[~finite], decoded[~finite]):
+        assert (np.isnan(d) and "NaN" in t) or (np.isinf(d) and (d < 0) == t.startswith("-"))
