@@ -279,7 +279,8 @@ int hipnx_threefry2x32(hipnx_ctx *ctx, const hipnx_buf *key, int64_t n, hipnx_bu
  * The result of the last instruction is the output.  Types: bf16 / f16 / f32 values, u8 truth
  * values; inputs of at most 4 bytes per element.  The index space is [rows, cols]; col strides
  * are 1 or 0; cols, and with more than one row the row strides of dense inputs, are multiples
- * of 8 (otherwise HIPNX_EUNSUPPORTED: run the nodes one by one).
+ * of 8 (otherwise HIPNX_EUNSUPPORTED: run the nodes one by one) -- except that with rows = 1 a compiled
+ * kernel (HIPNX_FUSED_COMPILED) takes any cols: its last vector is partial.
  * reduce_op: -1, or HIPNX_RED_SUM / MAX / MIN to reduce the result along its rows without storing it
  * (sum/4, reduce_max/4, reduce_min/4 over the last axis, nx/lib/nx/backend.ex:89-92): `out` then has
  * `rows` elements, and equals the separate reduction kernel applied to the stored result. */

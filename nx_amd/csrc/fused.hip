@@ -128,8 +128,8 @@ __device__ __forceinline__ void run_program(KernArgs a, int n_instr, const int64
 
 template <bool FULL>
 struct RunInterpreted {
-  static __device__ __forceinline__ void run(KernArgs a, const int64_t (&row)[FV], const int64_t (&col)[FV], Vecs &acc) {
-    run_program<FULL>(a, a->n_instr, row, col, acc);
+  static __device__ __forceinline__ void run(KernArgs a, const int64_t (&row)[FV], const int64_t (&col)[FV], Vecs &acc, int = FE) {
+    run_program<FULL>(a, a->n_instr, row, col, acc);  // (whole vectors only: the host sees to it)
   }
   static __device__ __forceinline__ int out_dt(KernArgs a) { return a->out_dt; }
   static constexpr bool raw_out = false;
@@ -290,7 +290,12 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
   if (n_stats && (reduce_op != -1 || cols > 4096 || cols == 0))
     return set_error(HIPNX_EUNSUPPORTED, "fused: stages take rows of 1 .. 4096 elements and no reduction of the result");
   const int64_t n = rows * cols;
-  if (cols % 8 != 0) return set_error(HIPNX_EUNSUPPORTED, "fused: the row length is not a multiple of 8");
+  if (cols % 8 != 0) {
+    // a flat index space (one row) may end in a partial vector -- in a compiled kernel, which handles it
+    if (rows != 1 || reduce_op != -1 || n_stats || ctx->fused_mode != HIPNX_FUSED_COMPILED)
+      return set_error(HIPNX_EUNSUPPORTED, "fused: the row length is not a multiple of 8");
+    needs_compiled = true;
+  }
   for (int k = 0; k < n_inputs; k++) {
     const int dt = in_dts[k];
     const int sz = dtype_size(dt);
@@ -323,7 +328,7 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
   a.out_dt = out_dt;
   a.rows = rows;
   a.cols = cols;
-  a.vecs_per_row = cols / FE;
+  a.vecs_per_row = (cols + FE - 1) / FE;
   a.nvec = rows * a.vecs_per_row;
   if (ctx->fused_mode == HIPNX_FUSED_COMPILED) {
     // the same grids as the interpreting kernels below

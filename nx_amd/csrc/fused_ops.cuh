@@ -127,6 +127,26 @@ __device__ __forceinline__ void load_input_as(KernArgs a, int k, int dt, int cs,
   }
 }
 
+// the last, partial vector of a flat index space: only its first `valid` elements exist in memory
+__device__ __forceinline__ void load_input_tail(KernArgs a, int k, int dt, int cs, const int64_t (&row)[FV],
+                                                const int64_t (&col)[FV], int valid, Vecs &dst) {
+  if (cs == 0) {
+    load_input_as(a, k, dt, cs, row, col, dst);
+    return;
+  }
+  const int esz = (dt == HIPNX_U8 || dt == HIPNX_S8) ? 1 : (dt == HIPNX_U32 || dt == HIPNX_S32 || dt == HIPNX_F32) ? 4 : 2;
+  const char *p = (const char *)a->in[k] + (row[0] * a->in_rs[k] + col[0]) * esz;
+#pragma unroll
+  for (int e = 0; e < FE; e++) {
+    uint32_t w = 0;
+    if (e < valid)
+      w = esz == 4 ? *reinterpret_cast<const uint32_t *>(p + 4 * e)
+          : esz == 2 ? (uint32_t)*reinterpret_cast<const uint16_t *>(p + 2 * e)
+                     : (uint32_t)*reinterpret_cast<const uint8_t *>(p + e);
+    dst[0][e] = element_to_f32(w, dt);
+  }
+}
+
 __device__ __forceinline__ void copy_vecs(Vecs &dst, const Vecs &src) {
 #pragma unroll
   for (int u = 0; u < FV; u++)
@@ -148,7 +168,7 @@ typedef float RowStats[HIPNX_FUSED_STATS];  // results of the row reductions of 
 
 template <typename P, int SRC, int ARG, unsigned IMM, bool RAW>
 __device__ __forceinline__ void fetch_static(KernArgs a, const Saved &S, const RowStats &stats, const int64_t (&row)[FV],
-                                             const int64_t (&col)[FV], Vecs &dst) {
+                                             const int64_t (&col)[FV], int valid, Vecs &dst) {
   if constexpr (SRC == HIPNX_FUSED_SRC_ROWSTAT) {
 #pragma unroll
     for (int u = 0; u < FV; u++)
@@ -156,7 +176,8 @@ __device__ __forceinline__ void fetch_static(KernArgs a, const Saved &S, const R
       for (int e = 0; e < FE; e++) dst[u][e] = stats[ARG];
   } else if constexpr (SRC == HIPNX_FUSED_SRC_INPUT) {
     // RAW: the words of a 4-byte input as they are (what the f32 path does with its bits)
-    load_input_as(a, ARG, RAW ? (int)HIPNX_F32 : P::in_dt[ARG], P::in_cs[ARG], row, col, dst);
+    if (valid == FE) load_input_as(a, ARG, RAW ? (int)HIPNX_F32 : P::in_dt[ARG], P::in_cs[ARG], row, col, dst);
+    else load_input_tail(a, ARG, RAW ? (int)HIPNX_F32 : P::in_dt[ARG], P::in_cs[ARG], row, col, valid, dst);
   } else if constexpr (SRC == HIPNX_FUSED_SRC_SAVED) {
     copy_vecs(dst, S.s[ARG]);
   } else {
@@ -185,14 +206,14 @@ __device__ __forceinline__ float int_unary(float x) {
 // instructions PC .. END-1
 template <typename P, int PC, int END>
 __device__ __forceinline__ void static_steps(KernArgs a, const int64_t (&row)[FV], const int64_t (&col)[FV], Vecs &acc, Saved &S,
-                                             const RowStats &stats) {
+                                             const RowStats &stats, int valid = FE) {
   if constexpr (PC < END) {
     constexpr int kind = P::kind[PC], op = P::op[PC], src = P::src[PC], arg = P::arg[PC];
     constexpr int src2 = P::src2[PC], arg2 = P::arg2[PC], flags = P::flags[PC], dt = P::dt[PC];
     constexpr unsigned imm = P::imm[PC], imm2 = P::imm2[PC];
     constexpr bool ints = (flags & HIPNX_FUSED_FLAG_INT) != 0, uns = dt == HIPNX_U32;
     if constexpr (kind == HIPNX_FUSED_SET) {
-      fetch_static<P, src, arg, imm, ints>(a, S, stats, row, col, acc);
+      fetch_static<P, src, arg, imm, ints>(a, S, stats, row, col, valid, acc);
     } else if constexpr (kind == HIPNX_FUSED_UNARY) {
       if constexpr (ints) {
 #pragma unroll
@@ -204,7 +225,7 @@ __device__ __forceinline__ void static_steps(KernArgs a, const int64_t (&row)[FV
       }
     } else if constexpr (kind == HIPNX_FUSED_BINARY) {
       Vecs y;
-      fetch_static<P, src, arg, imm, ints>(a, S, stats, row, col, y);
+      fetch_static<P, src, arg, imm, ints>(a, S, stats, row, col, valid, y);
       if constexpr (ints) {
 #pragma unroll
         for (int u = 0; u < FV; u++)
@@ -215,8 +236,8 @@ __device__ __forceinline__ void static_steps(KernArgs a, const int64_t (&row)[FV
       }
     } else if constexpr (kind == HIPNX_FUSED_SELECT) {
       Vecs y, z;
-      fetch_static<P, src, arg, imm, false>(a, S, stats, row, col, y);
-      fetch_static<P, src2, arg2, imm2, false>(a, S, stats, row, col, z);
+      fetch_static<P, src, arg, imm, false>(a, S, stats, row, col, valid, y);
+      fetch_static<P, src2, arg2, imm2, false>(a, S, stats, row, col, valid, z);
 #pragma unroll
       for (int u = 0; u < FV; u++)
 #pragma unroll
@@ -234,16 +255,16 @@ __device__ __forceinline__ void static_steps(KernArgs a, const int64_t (&row)[FV
         for (int e = 0; e < FE; e++) acc[u][e] = round_to(acc[u][e], dt);
     }
     if constexpr ((flags >> 4) != 0) copy_vecs(S.s[(flags >> 4) - 1], acc);
-    static_steps<P, PC + 1, END>(a, row, col, acc, S, stats);
+    static_steps<P, PC + 1, END>(a, row, col, acc, S, stats, valid);
   }
 }
 
 template <typename P>
 struct RunStatic {
-  static __device__ __forceinline__ void run(KernArgs a, const int64_t (&row)[FV], const int64_t (&col)[FV], Vecs &acc) {
+  static __device__ __forceinline__ void run(KernArgs a, const int64_t (&row)[FV], const int64_t (&col)[FV], Vecs &acc, int valid = FE) {
     Saved S;
     const RowStats none = {};
-    static_steps<P, 0, P::n_instr>(a, row, col, acc, S, none);
+    static_steps<P, 0, P::n_instr>(a, row, col, acc, S, none, valid);
   }
   // a u32 / s32 result leaves as the bits it is held as
   static __device__ __forceinline__ int out_dt(KernArgs) { return P::out_dt; }
@@ -271,19 +292,30 @@ __device__ __forceinline__ void fused_elementwise_body() {
         col[u] = (v - row[u] * vecs_per_row) * FE;
       }
     }
+    static_assert(FV == 1, "the partial last vector is written for one vector per lane");
+    // a flat index space need not be a whole number of vectors: the last one is partial
+    const int64_t left = a->rows * cols - (row[0] * cols + col[0]);
+    const int valid = left < FE ? (int)left : FE;
     Vecs acc;
-    RUN::run(a, row, col, acc);
+    if (valid == FE) RUN::run(a, row, col, acc);
+    else RUN::run(a, row, col, acc, valid);
     void *out = (void *)a->out;
     const int odt = RUN::out_dt(a);
 #pragma unroll
     for (int u = 0; u < FV; u++) {
       if (!live[u]) continue;
-      if constexpr (RUN::raw_out) {
-        uint4 *p = reinterpret_cast<uint4 *>((uint32_t *)out + row[u] * cols + col[u]);
+      const int64_t at = row[u] * cols + col[u];
+      if (valid < FE) {
+        for (int e = 0; e < valid; e++) {
+          if constexpr (RUN::raw_out) ((uint32_t *)out)[at + e] = __float_as_uint(acc[u][e]);
+          else store_one<float>(out, odt, at + e, acc[u][e]);
+        }
+      } else if constexpr (RUN::raw_out) {
+        uint4 *p = reinterpret_cast<uint4 *>((uint32_t *)out + at);
         p[0] = make_uint4(__float_as_uint(acc[u][0]), __float_as_uint(acc[u][1]), __float_as_uint(acc[u][2]), __float_as_uint(acc[u][3]));
         p[1] = make_uint4(__float_as_uint(acc[u][4]), __float_as_uint(acc[u][5]), __float_as_uint(acc[u][6]), __float_as_uint(acc[u][7]));
       } else {
-        store_vec<float, FE>(out, odt, row[u] * cols + col[u], acc[u]);
+        store_vec<float, FE>(out, odt, at, acc[u]);
       }
     }
   }

@@ -516,8 +516,8 @@ def _layout(out_shape, in_shapes, split=None):
     padded = [(1,) * (rank - len(s)) + tuple(s) for s in in_shapes]
     for p in (range(rank + 1) if split is None else [split]):
         rows, cols = prod(out_shape[:p]), prod(out_shape[p:])
-        if cols % 8:  # the kernel works on whole vectors of 8 along a row
-            continue
+        if cols % 8 and not (_plan["ints"] and split is None and p == 0):
+            continue  # whole vectors of 8 along a row; a compiled kernel over a flat index space takes a partial last one
         strides = []
         for s in padded:
             outer, inner = s[:p], s[p:]

@@ -725,3 +725,43 @@ def test_per_row_results_from_one_kernel_are_bit_identical(name, shape, ty, hip)
     finally:
         hip.fused_elementwise = classmethod(original)
     assert calls == [1]
+
+
+# ---- a flat index space that is no whole number of vectors (compiled groups take the partial last one) ----
+
+@pytest.mark.parametrize("ty", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("shape", [(1,), (7,), (9,), (37, 11), (3, 5, 7), (1000003,), (255, 257)])
+def test_ragged_sizes_in_compiled_groups(shape, ty, hip):
+    rng = np.random.default_rng(seed_of(shape, ty))
+    x, y = rand_float(rng, ty, shape, hip), rand_float(rng, ty, shape, hip)
+    guard = rand_float(rng, ty, (64,), hip)   # a neighbour in memory that must stay as it is
+
+    def fun(a, b):
+        h = Nx.add(Nx.multiply(a, 0.5), b)
+        return Nx.select(Nx.greater(h, 0.0), Nx.tanh(h), Nx.multiply(h, 0.01))
+
+    want = defn.compile(fun, x, y)(x, y)
+    before = hip.to_numpy(guard).copy()
+    planned = defn.compile(fun, x, y, fuse="compiled")
+    assert planned.roots[0].data.op == "fused" and planned.roots[0].data.args[0].layout is not None
+    assert_bits_equal(planned(x, y), want, f"ragged {shape} {ty}")
+    np.testing.assert_array_equal(hip.to_numpy(guard), before)
+    # planned without the compiled kernels in mind, such a shape is left to the separate callbacks
+    assert_bits_equal(defn.compile(fun, x, y, fuse=True)(x, y), want, f"ragged {shape} {ty}, mode-agnostic plan")
+
+
+def test_ragged_integer_words(hip):
+    x = rand_words(np.random.default_rng(12), "u32", (1001,), hip)
+    planned = defn.compile(bits_to_unit_floats, x, fuse="compiled")
+    assert planned.roots[0].data.op == "fused"
+    assert_bits_equal(planned(x), defn.compile(bits_to_unit_floats, x)(x), "ragged u32 -> f32")
+
+
+def test_ragged_rows_still_fall_back(hip):
+    rng = np.random.default_rng(13)
+    x, bias = rand_float(rng, "f32", (37, 11), hip), rand_float(rng, "f32", (11,), hip)   # a row operand: no flat index space
+
+    def fun(a, b):
+        return Nx.exp(Nx.add(a, b))
+    planned = defn.compile(fun, x, bias, fuse="compiled")
+    assert_bits_equal(planned(x, bias), defn.compile(fun, x, bias)(x, bias), "row operand, ragged rows")
