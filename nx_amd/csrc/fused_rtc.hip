@@ -59,7 +59,7 @@ static std::string make_key(const FusedArgs &a, int reduce_op, bool block_per_ro
 }
 
 // the whole translation unit for one program
-static std::string make_source(const FusedArgs &a, int reduce_op, bool block_per_row) {
+static std::string make_source(const FusedArgs &a, int reduce_op, bool block_per_row, const std::string &name) {
   std::string s = RTC_PREAMBLE;
   s += "namespace hipnx {\nstruct P {\n  static constexpr int n_instr = " + std::to_string(a.n_instr) + ", out_dt = " + std::to_string(a.out_dt) + ";\n";
   const hipnx_fused_instr *q = a.ins;
@@ -88,7 +88,7 @@ static std::string make_source(const FusedArgs &a, int reduce_op, bool block_per
   }
   list_of(s, "seg_red", "int", (int)seg_red.size(), [&](int k) { return std::to_string(seg_red[k]); });
   list_of(s, "seg_save", "int", (int)seg_save.size(), [&](int k) { return std::to_string(seg_save[k]); });
-  s += "};\n}\nusing namespace hipnx;\nextern \"C\" __global__ void __launch_bounds__(FBLOCK) fused_group(FusedArgs by_value) {\n  (void)by_value;\n";
+  s += "};\n}\nusing namespace hipnx;\nextern \"C\" __global__ void __launch_bounds__(FBLOCK) " + name + "(FusedArgs by_value) {\n  (void)by_value;\n";
   const char *tpr = block_per_row ? "FBLOCK" : "WAVE";
   if (stages) s += "  fused_row_stages_body<P>();\n";
   else switch (reduce_op) {
@@ -101,7 +101,7 @@ static std::string make_source(const FusedArgs &a, int reduce_op, bool block_per
   return s;
 }
 
-static int compile(hipnx_ctx *ctx, const std::string &src, std::pair<hipModule_t, hipFunction_t> *out) {
+static int compile(hipnx_ctx *ctx, const std::string &src, const std::string &name, std::pair<hipModule_t, hipFunction_t> *out) {
   hipDeviceProp_t prop;
   HIPNX_HIP(hipGetDeviceProperties(&prop, ctx->device));
   const std::string arch = std::string("--offload-arch=") + prop.gcnArchName;
@@ -124,10 +124,10 @@ static int compile(hipnx_ctx *ctx, const std::string &src, std::pair<hipModule_t
   hiprtcGetCode(prog, &code[0]);
   hiprtcDestroyProgram(&prog);
   HIPNX_HIP(hipModuleLoadData(&out->first, code.data()));
-  hipError_t e = hipModuleGetFunction(&out->second, out->first, "fused_group");
+  hipError_t e = hipModuleGetFunction(&out->second, out->first, name.c_str());
   if (e != hipSuccess) {
     (void)hipModuleUnload(out->first);
-    return hip_fail(e, "hipModuleGetFunction(fused_group)");
+    return hip_fail(e, "hipModuleGetFunction(fused group)");
   }
   return HIPNX_OK;
 }
@@ -141,8 +141,15 @@ int fused_launch_compiled(hipnx_ctx *ctx, const FusedArgs &a, int reduce_op, boo
   auto it = ctx->fused_kernels.find(key);
   if (it == ctx->fused_kernels.end()) {
     if (ctx->capture) return HIPNX_OK;
+    // a name a profile can tell apart: what the kernel is (a map, a map with its row reduction, stages over rows),
+    // how long its program is, and a hash of what it is specialised on
+    int stages = 0;
+    for (int i = 0; i < a.n_instr; i++) stages += a.ins[i].kind == HIPNX_FUSED_ROW_REDUCE;
+    char name[96];
+    snprintf(name, sizeof(name), "fused_%s_%dinstr_%08zx", stages ? "stages" : reduce_op != -1 ? "map_reduce" : "map", a.n_instr,
+             std::hash<std::string>{}(key) & 0xFFFFFFFFu);
     std::pair<hipModule_t, hipFunction_t> k{};
-    if (int st = compile(ctx, make_source(a, reduce_op, block_per_row), &k)) return st;
+    if (int st = compile(ctx, make_source(a, reduce_op, block_per_row, name), name, &k)) return st;
     it = ctx->fused_kernels.emplace(key, k).first;
   }
   // the argument block is the kernel's one by-value parameter: hand it over as the packed buffer it is
