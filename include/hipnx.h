@@ -292,7 +292,8 @@ enum { HIPNX_FUSED_SET = 0, HIPNX_FUSED_UNARY, HIPNX_FUSED_BINARY, HIPNX_FUSED_S
  * element-type code) to the float dt; BITCAST (nx/lib/nx/backend.ex:69) relabels the bits.  These need
  * HIPNX_FUSED_COMPILED: the interpreting kernels return HIPNX_EUNSUPPORTED for them. */
 enum { HIPNX_FUSED_FLAG_SWAP = 1, HIPNX_FUSED_FLAG_INT = 2, HIPNX_FUSED_FLAG_RESULT = 1 /* on a ROW_STAT */ };
-enum { HIPNX_FUSED_SRC_CONST = 0, HIPNX_FUSED_SRC_INPUT, HIPNX_FUSED_SRC_SAVED, HIPNX_FUSED_SRC_ROWSTAT };
+enum { HIPNX_FUSED_SRC_CONST = 0, HIPNX_FUSED_SRC_INPUT, HIPNX_FUSED_SRC_SAVED, HIPNX_FUSED_SRC_ROWSTAT,
+       HIPNX_FUSED_SRC_CARRY };
 /* Stages over the same rows.  HIPNX_FUSED_ROW_REDUCE reduces the accumulator along the row (op =
  * HIPNX_RED_SUM / MAX / MIN, exactly as the reduction of the separate entry point would, the result stored
  * in type dt) and leaves that one value per row in the accumulator; the instructions that follow work on
@@ -300,7 +301,9 @@ enum { HIPNX_FUSED_SRC_CONST = 0, HIPNX_FUSED_SRC_INPUT, HIPNX_FUSED_SRC_SAVED, 
  * statistics) until HIPNX_FUSED_ROW_STAT ends the stage: the accumulator becomes row statistic number `arg`
  * (counted from 0 in program order), which later instructions read with source HIPNX_FUSED_SRC_ROWSTAT.
  * The next stage starts with a SET and empty slots; the last stage's value is the result.  Softmax over
- * rows is three stages of one program, a layer normalisation three as well.  A ROW_STAT with flags bit 0
+ * rows is three stages of one program, a layer normalisation three as well.  In a stage that follows a
+ * reducing one, source HIPNX_FUSED_SRC_CARRY is the value that stage reduced, element for element (it stays
+ * in the lanes' registers): the softmax's division reads the exponentials its sum was taken over.  A ROW_STAT with flags bit 0
  * (HIPNX_FUSED_FLAG_RESULT) ends the program instead: that one value per row is the result (`out` has
  * `rows` elements) -- a log-sum-exp is two such stages.  Rows of at most 4096
  * elements, reduce_op = -1, HIPNX_FUSED_COMPILED only (HIPNX_EUNSUPPORTED otherwise). */

@@ -198,6 +198,10 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
       if (arg >= n_stats) { *why = "reads a row statistic that no stage has produced yet"; return false; }
       return true;
     }
+    if (src == HIPNX_FUSED_SRC_CARRY) {
+      if (n_stats < 1 || on_stat) { *why = "reads the previous stage's values where there are none"; return false; }
+      return true;
+    }
     if (src != HIPNX_FUSED_SRC_INPUT && src != HIPNX_FUSED_SRC_SAVED && src != HIPNX_FUSED_SRC_CONST) { *why = "has an unknown operand source"; return false; }
     return true;
   };

@@ -168,8 +168,11 @@ typedef float RowStats[HIPNX_FUSED_STATS];  // results of the row reductions of 
 
 template <typename P, int SRC, int ARG, unsigned IMM, bool RAW>
 __device__ __forceinline__ void fetch_static(KernArgs a, const Saved &S, const RowStats &stats, const int64_t (&row)[FV],
-                                             const int64_t (&col)[FV], int valid, Vecs &dst) {
-  if constexpr (SRC == HIPNX_FUSED_SRC_ROWSTAT) {
+                                             const int64_t (&col)[FV], int valid, const float (*carry)[FE], Vecs &dst) {
+  if constexpr (SRC == HIPNX_FUSED_SRC_CARRY) {  // what the previous stage reduced, at this vector
+#pragma unroll
+    for (int e = 0; e < FE; e++) dst[0][e] = (*carry)[e];
+  } else if constexpr (SRC == HIPNX_FUSED_SRC_ROWSTAT) {
 #pragma unroll
     for (int u = 0; u < FV; u++)
 #pragma unroll
@@ -206,14 +209,14 @@ __device__ __forceinline__ float int_unary(float x) {
 // instructions PC .. END-1
 template <typename P, int PC, int END>
 __device__ __forceinline__ void static_steps(KernArgs a, const int64_t (&row)[FV], const int64_t (&col)[FV], Vecs &acc, Saved &S,
-                                             const RowStats &stats, int valid = FE) {
+                                             const RowStats &stats, int valid = FE, const float (*carry)[FE] = nullptr) {
   if constexpr (PC < END) {
     constexpr int kind = P::kind[PC], op = P::op[PC], src = P::src[PC], arg = P::arg[PC];
     constexpr int src2 = P::src2[PC], arg2 = P::arg2[PC], flags = P::flags[PC], dt = P::dt[PC];
     constexpr unsigned imm = P::imm[PC], imm2 = P::imm2[PC];
     constexpr bool ints = (flags & HIPNX_FUSED_FLAG_INT) != 0, uns = dt == HIPNX_U32;
     if constexpr (kind == HIPNX_FUSED_SET) {
-      fetch_static<P, src, arg, imm, ints>(a, S, stats, row, col, valid, acc);
+      fetch_static<P, src, arg, imm, ints>(a, S, stats, row, col, valid, carry, acc);
     } else if constexpr (kind == HIPNX_FUSED_UNARY) {
       if constexpr (ints) {
 #pragma unroll
@@ -225,7 +228,7 @@ __device__ __forceinline__ void static_steps(KernArgs a, const int64_t (&row)[FV
       }
     } else if constexpr (kind == HIPNX_FUSED_BINARY) {
       Vecs y;
-      fetch_static<P, src, arg, imm, ints>(a, S, stats, row, col, valid, y);
+      fetch_static<P, src, arg, imm, ints>(a, S, stats, row, col, valid, carry, y);
       if constexpr (ints) {
 #pragma unroll
         for (int u = 0; u < FV; u++)
@@ -236,8 +239,8 @@ __device__ __forceinline__ void static_steps(KernArgs a, const int64_t (&row)[FV
       }
     } else if constexpr (kind == HIPNX_FUSED_SELECT) {
       Vecs y, z;
-      fetch_static<P, src, arg, imm, false>(a, S, stats, row, col, valid, y);
-      fetch_static<P, src2, arg2, imm2, false>(a, S, stats, row, col, valid, z);
+      fetch_static<P, src, arg, imm, false>(a, S, stats, row, col, valid, carry, y);
+      fetch_static<P, src2, arg2, imm2, false>(a, S, stats, row, col, valid, carry, z);
 #pragma unroll
       for (int u = 0; u < FV; u++)
 #pragma unroll
@@ -255,7 +258,7 @@ __device__ __forceinline__ void static_steps(KernArgs a, const int64_t (&row)[FV
         for (int e = 0; e < FE; e++) acc[u][e] = round_to(acc[u][e], dt);
     }
     if constexpr ((flags >> 4) != 0) copy_vecs(S.s[(flags >> 4) - 1], acc);
-    static_steps<P, PC + 1, END>(a, row, col, acc, S, stats, valid);
+    static_steps<P, PC + 1, END>(a, row, col, acc, S, stats, valid, carry);
   }
 }
 
@@ -375,20 +378,36 @@ __device__ __forceinline__ float as_stored(CT v, int dt) {
   }
 }
 
-template <typename P, int SEG>
-__device__ __forceinline__ void row_stage(KernArgs a, int64_t r, int lane, RowStats &stats) {
+// The walk of a row: lane l takes the vectors l, l + WAVE, ... -- at most P::nv of them when the program
+// carries element values from one stage to the next (their registers are indexed by the trip), any
+// number otherwise.
+template <typename P, typename F>
+__device__ __forceinline__ void for_each_vector(int lane, int64_t cols, F &&body) {
+  if constexpr (P::nv > 0) {
+#pragma unroll
+    for (int it = 0; it < P::nv; it++) {
+      const int64_t k = ((int64_t)lane + (int64_t)it * WAVE) * FE;
+      if (k < cols) body(k, it);
+    }
+  } else {
+    for (int64_t k = (int64_t)lane * FE; k < cols; k += (int64_t)WAVE * FE) body(k, 0);
+  }
+}
+
+template <typename P, int SEG, typename CARRY>
+__device__ __forceinline__ void row_stage(KernArgs a, int64_t r, int lane, RowStats &stats, CARRY &carry) {
   // stage SEG: instructions [begin, red) on the row's elements, the reduction at `red`, instructions
   // (red, save) on the statistic, which is kept at `save`; the last stage is [begin, n_instr)
   constexpr int begin = SEG == 0 ? 0 : P::seg_save[SEG - 1] + 1;
   constexpr int red = P::seg_red[SEG], save = P::seg_save[SEG];
-  const int64_t cols = a->cols, step = (int64_t)WAVE * FE;
+  const int64_t cols = a->cols;
   if constexpr (red < 0) {  // the last stage: its value is the result
     void *out = (void *)a->out;
-    for (int64_t k = (int64_t)lane * FE; k < cols; k += step) {
+    for_each_vector<P>(lane, cols, [&](int64_t k, int it) {
       const int64_t row[FV] = {r}, col[FV] = {k};
       Vecs x;
       Saved S;
-      static_steps<P, begin, P::n_instr>(a, row, col, x, S, stats);
+      static_steps<P, begin, P::n_instr>(a, row, col, x, S, stats, FE, &carry[it]);
       if constexpr (P::out_dt == HIPNX_U32 || P::out_dt == HIPNX_S32) {
         uint4 *p = reinterpret_cast<uint4 *>((uint32_t *)out + r * cols + k);
         p[0] = make_uint4(__float_as_uint(x[0][0]), __float_as_uint(x[0][1]), __float_as_uint(x[0][2]), __float_as_uint(x[0][3]));
@@ -396,20 +415,24 @@ __device__ __forceinline__ void row_stage(KernArgs a, int64_t r, int lane, RowSt
       } else {
         store_vec<float, FE>(out, P::out_dt, r * cols + k, x[0]);
       }
-    }
+    });
   } else {
     constexpr int op = P::op[red];
     typedef typename std::conditional<op == HIPNX_RED_SUM, double, float>::type CT;
     typedef PlainReducer<CT, op, false> R;
     typename R::acc_t acc = R::init();
-    for (int64_t k = (int64_t)lane * FE; k < cols; k += step) {
+    for_each_vector<P>(lane, cols, [&](int64_t k, int it) {
       const int64_t row[FV] = {r}, col[FV] = {k};
       Vecs x;
       Saved S;
-      static_steps<P, begin, red>(a, row, col, x, S, stats);
+      static_steps<P, begin, red>(a, row, col, x, S, stats, FE, &carry[it]);
 #pragma unroll
       for (int e = 0; e < FE; e++) acc = R::accumulate(acc, (CT)x[0][e], k + e);
-    }
+      if constexpr (P::nv > 0) {  // kept for the next stage (after this stage's own reads of the previous one's)
+#pragma unroll
+        for (int e = 0; e < FE; e++) carry[it][e] = x[0][e];
+      }
+    });
     acc = wave_reduce<R>(acc);  // the butterfly leaves the same value in every lane
     // the work on the statistic: the same instructions on a vector that holds it eight times
     const int64_t row[FV] = {r}, col[FV] = {0};
@@ -422,7 +445,7 @@ __device__ __forceinline__ void row_stage(KernArgs a, int64_t r, int lane, RowSt
       if (lane == 0) store_one<float>((void *)a->out, P::out_dt, r, x[0][0]);
     } else {
       stats[P::arg[save]] = x[0][0];
-      row_stage<P, SEG + 1>(a, r, lane, stats);
+      row_stage<P, SEG + 1>(a, r, lane, stats, carry);
     }
   }
 }
@@ -434,7 +457,8 @@ __device__ __forceinline__ void fused_row_stages_body() {
   const int64_t r = (int64_t)blockIdx.x * (FBLOCK / WAVE) + threadIdx.x / WAVE;
   if (r >= a->rows) return;
   RowStats stats = {};
-  row_stage<P, 0>(a, r, threadIdx.x % WAVE, stats);
+  float carry[P::nv > 0 ? P::nv : 1][FE];  // (indexed by compile-time trip numbers only: registers)
+  row_stage<P, 0>(a, r, threadIdx.x % WAVE, stats, carry);
 }
 
 }  // namespace hipnx

@@ -46,11 +46,23 @@ static void list_of(std::string &s, const char *name, const char *type, int n, c
   s += "};\n";
 }
 
+// Trips of a lane along a row (of at most 4096 elements), when the program carries element values from
+// stage to stage and so indexes their registers by the trip; 0 when it does not.
+static int carry_trips(const FusedArgs &a) {
+  for (int i = 0; i < a.n_instr; i++) {
+    const hipnx_fused_instr &q = a.ins[i];
+    const bool reads = q.kind == HIPNX_FUSED_SET || q.kind == HIPNX_FUSED_BINARY || q.kind == HIPNX_FUSED_SELECT;
+    if (reads && (q.src == HIPNX_FUSED_SRC_CARRY || (q.kind == HIPNX_FUSED_SELECT && q.src2 == HIPNX_FUSED_SRC_CARRY)))
+      return (int)((a.cols + WAVE * FE - 1) / (WAVE * FE));
+  }
+  return 0;
+}
+
 // everything a compiled kernel is specialised on, as bytes: the cache key
 static std::string make_key(const FusedArgs &a, int reduce_op, bool block_per_row) {
   std::string k;
   k.reserve(16 + 16 * a.n_instr + 8 * a.n_inputs);
-  const int head[4] = {a.n_instr, a.n_inputs, a.out_dt, reduce_op * 2 + (block_per_row ? 1 : 0)};
+  const int head[5] = {a.n_instr, a.n_inputs, a.out_dt, reduce_op * 2 + (block_per_row ? 1 : 0), carry_trips(a)};
   k.append((const char *)head, sizeof(head));
   k.append((const char *)a.ins, sizeof(hipnx_fused_instr) * a.n_instr);
   k.append((const char *)a.in_dt, sizeof(int) * a.n_inputs);
@@ -61,7 +73,8 @@ static std::string make_key(const FusedArgs &a, int reduce_op, bool block_per_ro
 // the whole translation unit for one program
 static std::string make_source(const FusedArgs &a, int reduce_op, bool block_per_row, const std::string &name) {
   std::string s = RTC_PREAMBLE;
-  s += "namespace hipnx {\nstruct P {\n  static constexpr int n_instr = " + std::to_string(a.n_instr) + ", out_dt = " + std::to_string(a.out_dt) + ";\n";
+  s += "namespace hipnx {\nstruct P {\n  static constexpr int n_instr = " + std::to_string(a.n_instr) + ", out_dt = " + std::to_string(a.out_dt) +
+       ", nv = " + std::to_string(carry_trips(a)) + ";\n";
   const hipnx_fused_instr *q = a.ins;
   list_of(s, "kind", "int", a.n_instr, [&](int i) { return std::to_string((int)q[i].kind); });
   list_of(s, "op", "int", a.n_instr, [&](int i) { return std::to_string((int)q[i].op); });

@@ -1131,8 +1131,20 @@ def _cluster_rows(roots: List[Tensor]) -> int:
                 program.append(ins)
 
         program, steps, fits = _Program(), [], True
+        reduced = None  # the element-wise program of the stage before (what its reduction was taken over)
+
+        def start_from_carry(at):
+            """A stage whose program begins with the whole element-wise program of the stage before it
+            (the softmax's division begins with the exponentials its sum was taken over) reads those
+            values where they still are -- the lanes' registers -- instead of computing them again."""
+            mine = program[at:]
+            if (reduced and len(mine) >= len(reduced) and mine[:len(reduced)] == reduced
+                    and not any(ins.get("flags", 0) >> 4 for ins in reduced)):
+                program[at:] = [{"kind": 0, "src": 4, "dt": reduced[-1]["dt"]}] + mine[len(reduced):]
+
         for i in kept:
             base, links = stages[i]
+            at = len(program)
             if base.data.op == "fused":
                 group_program(base)
                 code = _REDUCE_CODES[base.data.args[0].reduce[0]]
@@ -1140,6 +1152,9 @@ def _cluster_rows(roots: List[Tensor]) -> int:
                 x = base.data.args[0]
                 program.append({"kind": 0, "src": 1, "arg": external(x), "dt": x.type})
                 code = _REDUCE_CODES[base.data.op]
+            mine = [dict(ins) for ins in program[at:]]
+            start_from_carry(at)
+            reduced = mine
             program.append({"kind": 6, "op": code, "dt": base.type})
             steps.append(base)
             chain = base
@@ -1168,7 +1183,9 @@ def _cluster_rows(roots: List[Tensor]) -> int:
             else:
                 program.append({"kind": 7, "arg": 0, "flags": 1, "dt": chain.type})  # the value per row is the result
         if not row_valued:
+            at = len(program)
             group_program(final)
+            start_from_carry(at)
         layout = _layout(full_shape, [t.shape for t in union], split=rank - 1)
         if not fits or layout is None or len(program) > _MAX_INSTR or len(union) > _MAX_INPUTS:
             return False
