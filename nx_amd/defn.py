@@ -1051,10 +1051,19 @@ def _cluster_rows(roots: List[Tensor]) -> int:
             links, cur = [], t
             while base_of(cur) is None:
                 d = cur.data
+                if d.op in ("reshape", "squeeze") and isinstance(d.args[0], Tensor) and d.args[0].size == cur.size:
+                    # the same values under another shape (a statistic taken without keep_axes, then given its axis back)
+                    chain = d.args[0]
+                    if (not is_per_row(chain, flat_too=True) or chain.data.id in stages or chain.data.id in absorbed
+                            or readers.get(chain.data.id, set()) != {d.id}):
+                        return False
+                    links.append(cur)
+                    cur = chain
+                    continue
                 if (d.op not in UNARY_OPS and d.op not in BINARY_OPS and d.op != "as_type") or not _fusable(cur):
                     return False
                 operands = [a for a in d.args if isinstance(a, Tensor) and _const(a) is None]
-                if not operands or not all(is_per_row(a, flat_too=is_final) for a in operands):
+                if not operands or not all(is_per_row(a, flat_too=True) for a in operands):
                     return False
                 # the chain continues through the operand computed last; any other one is a kept value of another stage
                 chain = max(operands, key=lambda a: position.get(a.data.id, -1))
@@ -1161,6 +1170,10 @@ def _cluster_rows(roots: List[Tensor]) -> int:
             for l in links:
                 d = l.data
                 ins = {"dt": l.type}
+                if d.op in ("reshape", "squeeze"):  # nothing happens to the value
+                    steps.append(l)
+                    chain = l
+                    continue
                 if d.op in UNARY_OPS:
                     ins.update(kind=1, op=UNARY_OPS.index(d.op))
                 elif d.op == "as_type":

@@ -423,3 +423,17 @@ def test_a_per_row_result_is_a_cluster_too(on_oracle):
         return Nx.sum(t, axes=[-1], keep_axes=True)
 
     assert defn.compile(plain_sum, x, fuse="compiled").roots[0].data.op == "sum"
+
+
+def test_statistic_taken_without_its_axis_and_given_it_back(on_oracle):
+    x = f32(np.random.default_rng(9).standard_normal((12, 64)), on_oracle)
+
+    def softmax_new_axis(t):
+        m = Nx.new_axis(Nx.reduce_max(t, axes=[-1]), -1)
+        e = Nx.exp(Nx.subtract(t, m))
+        return Nx.divide(e, Nx.new_axis(Nx.sum(e, axes=[-1]), -1))
+
+    planned = defn.compile(softmax_new_axis, x, fuse="compiled")
+    cluster = planned.roots[0].data.args[0]
+    assert type(cluster).__name__ == "_RowCluster" and cluster.n_stages == 2
+    assert_bits_equal(planned(x), softmax_new_axis(x), "softmax with new_axis")

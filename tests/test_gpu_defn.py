@@ -625,6 +625,12 @@ def range_normalised(x):          # three statistics: minimum, maximum, and the 
     return Nx.divide(u, Nx.sum(u, axes=[-1], keep_axes=True))
 
 
+def softmax_new_axis(x):          # statistics taken without keep_axes, then given their axis back
+    m = Nx.new_axis(Nx.reduce_max(x, axes=[-1]), -1)
+    e = Nx.exp(Nx.subtract(x, m))
+    return Nx.divide(e, Nx.new_axis(Nx.sum(e, axes=[-1]), -1))
+
+
 def log_softmax_rows(x):
     z = Nx.subtract(x, Nx.reduce_max(x, axes=[-1], keep_axes=True))
     return Nx.subtract(z, Nx.log(Nx.sum(Nx.exp(z), axes=[-1], keep_axes=True)))
@@ -638,13 +644,14 @@ def rms_scaled(x):                # one statistic, worked on with two constants 
 
 @pytest.mark.parametrize("ty", ["f32", "bf16"])
 @pytest.mark.parametrize("shape", [(32, 512, 512), (100, 64), (7, 4096), (3, 5, 8), (1, 1024), (2049, 40)])
-@pytest.mark.parametrize("name", ["softmax_rows", "centred_and_scaled", "range_normalised", "log_softmax_rows", "rms_scaled"])
+@pytest.mark.parametrize("name", ["softmax_rows", "centred_and_scaled", "range_normalised", "log_softmax_rows", "rms_scaled",
+                                  "softmax_new_axis"])
 def test_row_stages_are_bit_identical_to_node_by_node(name, shape, ty, hip):
     rng = np.random.default_rng(seed_of(name, shape, ty))
     x = rand_float(rng, ty, shape, hip)
     args = (x, rand_float(rng, ty, (shape[-1],), hip)) if name == "centred_and_scaled" else (x,)
     fun = {"softmax_rows": softmax_rows, "centred_and_scaled": centred_and_scaled, "range_normalised": range_normalised,
-           "log_softmax_rows": log_softmax_rows, "rms_scaled": rms_scaled}[name]
+           "log_softmax_rows": log_softmax_rows, "rms_scaled": rms_scaled, "softmax_new_axis": softmax_new_axis}[name]
     want = defn.compile(fun, *args)(*args)
     planned = defn.compile(fun, *args, fuse="compiled")
     # work on a statistic before it is used (the mean and the variance of the second function are divided by n,
