@@ -305,8 +305,10 @@ enum { HIPNX_FUSED_SRC_CONST = 0, HIPNX_FUSED_SRC_INPUT, HIPNX_FUSED_SRC_SAVED, 
  * reducing one, source HIPNX_FUSED_SRC_CARRY is the value that stage reduced, element for element (it stays
  * in the lanes' registers): the softmax's division reads the exponentials its sum was taken over.  A ROW_STAT with flags bit 0
  * (HIPNX_FUSED_FLAG_RESULT) ends the program instead: that one value per row is the result (`out` has
- * `rows` elements) -- a log-sum-exp is two such stages.  Rows of at most 4096
- * elements, reduce_op = -1, HIPNX_FUSED_COMPILED only (HIPNX_EUNSUPPORTED otherwise). */
+ * `rows` elements) -- a log-sum-exp is two such stages.  Rows of more than 4096 elements
+ * take a block each, as in the separate reduction; values are carried in registers for rows of up to 32768 elements
+ * (HIPNX_EUNSUPPORTED for a program that reads them over longer rows).
+ * reduce_op = -1, HIPNX_FUSED_COMPILED only (HIPNX_EUNSUPPORTED otherwise). */
 enum { HIPNX_FUSED_SAVED = 3, HIPNX_FUSED_MAX_INSTR = 32, HIPNX_FUSED_MAX_INPUTS = 8, HIPNX_FUSED_STATS = 3 };
 typedef struct {
   uint8_t kind, op, src, arg;

@@ -190,6 +190,7 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
   int n_stats = 0;       // row statistics kept so far (HIPNX_FUSED_ROW_STAT)
   bool on_stat = false;  // between a stage's reduction and its ROW_STAT
   bool row_result = false;  // the program ends in a ROW_STAT that is the result: one value per row
+  bool uses_carry = false;  // some instruction reads the previous stage's element values
   auto int32 = [](int dt) { return dt == HIPNX_U32 || dt == HIPNX_S32; };
   auto source_ok = [&](int src, int arg, const char **why) {
     if (src == HIPNX_FUSED_SRC_INPUT && arg >= n_inputs) { *why = "reads an input that is not there"; return false; }
@@ -200,6 +201,7 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
     }
     if (src == HIPNX_FUSED_SRC_CARRY) {
       if (n_stats < 1 || on_stat) { *why = "reads the previous stage's values where there are none"; return false; }
+      uses_carry = true;
       return true;
     }
     if (src != HIPNX_FUSED_SRC_INPUT && src != HIPNX_FUSED_SRC_SAVED && src != HIPNX_FUSED_SRC_CONST) { *why = "has an unknown operand source"; return false; }
@@ -291,8 +293,13 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
   if (needs_compiled && ctx->fused_mode != HIPNX_FUSED_COMPILED)
     return set_error(HIPNX_EUNSUPPORTED, "fused: 32-bit integer instructions and stages need the compiled mode");
   if (on_stat) return set_error(HIPNX_EINVAL, "fused: the program ends inside a stage's work on its statistic");
-  if (n_stats && (reduce_op != -1 || cols > 4096 || cols == 0))
-    return set_error(HIPNX_EUNSUPPORTED, "fused: stages take rows of 1 .. 4096 elements and no reduction of the result");
+  if (n_stats && (reduce_op != -1 || cols == 0))
+    return set_error(HIPNX_EUNSUPPORTED, "fused: stages take non-empty rows and no reduction of the result");
+  // a few very long rows are split into segments by the separate reduction, whose order the stages follow: not here
+  if (n_stats && rows < (int64_t)ctx->num_cus * 8 && cols >= 2 * 16384)
+    return set_error(HIPNX_EUNSUPPORTED, "fused: stages over rows that the reduction would split");
+  if (uses_carry && cols > 16 * (cols > 4096 ? 256 : 64) * 8)
+    return set_error(HIPNX_EUNSUPPORTED, "fused: rows too long to keep a stage's values in registers");
   const int64_t n = rows * cols;
   if (cols % 8 != 0) {
     // a flat index space (one row) may end in a partial vector -- in a compiled kernel, which handles it
@@ -336,8 +343,8 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
   a.nvec = rows * a.vecs_per_row;
   if (ctx->fused_mode == HIPNX_FUSED_COMPILED) {
     // the same grids as the interpreting kernels below
-    const bool block_per_row = reduce_op != -1 && a.cols > 4096;
-    int64_t grid = n_stats ? (a.rows + FBLOCK / WAVE - 1) / (FBLOCK / WAVE)  // a wave per row
+    const bool block_per_row = (reduce_op != -1 || n_stats) && a.cols > 4096;
+    int64_t grid = n_stats ? (block_per_row ? a.rows : (a.rows + FBLOCK / WAVE - 1) / (FBLOCK / WAVE))  // a wave or a block per row
                    : reduce_op == -1 ? (a.nvec + (int64_t)FBLOCK * FV - 1) / ((int64_t)FBLOCK * FV)
                    : block_per_row ? a.rows : (a.rows + FBLOCK / WAVE - 1) / (FBLOCK / WAVE);
     if (grid > (1ll << 30)) grid = 1ll << 30;

@@ -386,12 +386,29 @@ __device__ __forceinline__ void for_each_vector(int lane, int64_t cols, F &&body
   if constexpr (P::nv > 0) {
 #pragma unroll
     for (int it = 0; it < P::nv; it++) {
-      const int64_t k = ((int64_t)lane + (int64_t)it * WAVE) * FE;
+      const int64_t k = ((int64_t)lane + (int64_t)it * P::tpr) * FE;
       if (k < cols) body(k, it);
     }
   } else {
-    for (int64_t k = (int64_t)lane * FE; k < cols; k += (int64_t)WAVE * FE) body(k, 0);
+    for (int64_t k = (int64_t)lane * FE; k < cols; k += (int64_t)P::tpr * FE) body(k, 0);
   }
+}
+
+// the reduction of a stage over the P::tpr lanes of a row, left in every lane: within a wave by the
+// butterfly, across the waves of a block through LDS in the order of fused_reduce_rows_body
+template <typename P, typename R>
+__device__ __forceinline__ typename R::acc_t row_reduce(typename R::acc_t acc) {
+  acc = wave_reduce<R>(acc);
+  if constexpr (P::tpr > WAVE) {
+    __shared__ typename R::acc_t sm[FBLOCK / WAVE];
+    __syncthreads();  // the previous stage's readers are done with sm
+    if (threadIdx.x % WAVE == 0) sm[threadIdx.x / WAVE] = acc;
+    __syncthreads();
+    acc = sm[0];
+#pragma unroll
+    for (int w = 1; w < FBLOCK / WAVE; w++) acc = R::combine(acc, sm[w]);
+  }
+  return acc;
 }
 
 template <typename P, int SEG, typename CARRY>
@@ -433,7 +450,7 @@ __device__ __forceinline__ void row_stage(KernArgs a, int64_t r, int lane, RowSt
         for (int e = 0; e < FE; e++) carry[it][e] = x[0][e];
       }
     });
-    acc = wave_reduce<R>(acc);  // the butterfly leaves the same value in every lane
+    acc = row_reduce<P, R>(acc);  // the same value in every lane of the row
     // the work on the statistic: the same instructions on a vector that holds it eight times
     const int64_t row[FV] = {r}, col[FV] = {0};
     Vecs x;
@@ -442,7 +459,7 @@ __device__ __forceinline__ void row_stage(KernArgs a, int64_t r, int lane, RowSt
     for (int e = 0; e < FE; e++) x[0][e] = as_stored<CT>(acc, P::dt[red]);
     static_steps<P, red + 1, save>(a, row, col, x, S, stats);
     if constexpr ((P::flags[save] & HIPNX_FUSED_FLAG_RESULT) != 0) {  // this one value per row is the result
-      if (lane == 0) store_one<float>((void *)a->out, P::out_dt, r, x[0][0]);
+      if (lane == 0) store_one<float>((void *)a->out, P::out_dt, r, x[0][0]);  // lane 0 of the row
     } else {
       stats[P::arg[save]] = x[0][0];
       row_stage<P, SEG + 1>(a, r, lane, stats, carry);
@@ -454,11 +471,12 @@ template <typename P>
 __device__ __forceinline__ void fused_row_stages_body() {
   static_assert(FV == 1, "one vector per lane and step");
   KernArgs a = (KernArgs)__builtin_amdgcn_kernarg_segment_ptr();
-  const int64_t r = (int64_t)blockIdx.x * (FBLOCK / WAVE) + threadIdx.x / WAVE;
-  if (r >= a->rows) return;
+  // P::tpr lanes per row: a wave (rows of at most 4096 elements) or the whole block, as the separate reduction has it
+  const int64_t r = (int64_t)blockIdx.x * (FBLOCK / P::tpr) + threadIdx.x / P::tpr;
+  if (r >= a->rows) return;  // (a whole wave, or with a block per row nobody: no barrier is left waiting)
   RowStats stats = {};
   float carry[P::nv > 0 ? P::nv : 1][FE];  // (indexed by compile-time trip numbers only: registers)
-  row_stage<P, 0>(a, r, threadIdx.x % WAVE, stats, carry);
+  row_stage<P, 0>(a, r, threadIdx.x % P::tpr, stats, carry);
 }
 
 }  // namespace hipnx

@@ -53,7 +53,11 @@ static int carry_trips(const FusedArgs &a) {
     const hipnx_fused_instr &q = a.ins[i];
     const bool reads = q.kind == HIPNX_FUSED_SET || q.kind == HIPNX_FUSED_BINARY || q.kind == HIPNX_FUSED_SELECT;
     if (reads && (q.src == HIPNX_FUSED_SRC_CARRY || (q.kind == HIPNX_FUSED_SELECT && q.src2 == HIPNX_FUSED_SRC_CARRY)))
-      return (int)((a.cols + WAVE * FE - 1) / (WAVE * FE));
+      {
+        const int tpr = a.cols > 4096 ? FBLOCK : WAVE;
+        const int64_t trips = (a.cols + tpr * FE - 1) / (tpr * FE);
+        return trips <= 16 ? (int)trips : 0;  // (the host refuses longer rows for such programs)
+      }
   }
   return 0;
 }
@@ -74,7 +78,7 @@ static std::string make_key(const FusedArgs &a, int reduce_op, bool block_per_ro
 static std::string make_source(const FusedArgs &a, int reduce_op, bool block_per_row, const std::string &name) {
   std::string s = RTC_PREAMBLE;
   s += "namespace hipnx {\nstruct P {\n  static constexpr int n_instr = " + std::to_string(a.n_instr) + ", out_dt = " + std::to_string(a.out_dt) +
-       ", nv = " + std::to_string(carry_trips(a)) + ";\n";
+       ", nv = " + std::to_string(carry_trips(a)) + ", tpr = " + (block_per_row ? "FBLOCK" : "WAVE") + ";\n";
   const hipnx_fused_instr *q = a.ins;
   list_of(s, "kind", "int", a.n_instr, [&](int i) { return std::to_string((int)q[i].kind); });
   list_of(s, "op", "int", a.n_instr, [&](int i) { return std::to_string((int)q[i].op); });

@@ -978,8 +978,8 @@ def _cluster_rows(roots: List[Tensor]) -> int:
     last axis -- of a fused group's value or of a tensor as it is -- followed by a chain of
     element-wise nodes on the one value per row.  The node that is rewritten is an element-wise fused
     group over the full shape (a softmax, a layer normalisation), or itself such a per-row value
-    (a log-sum-exp).  Rows of at most 4096 elements: the width at which the separate reduction
-    gives a row to one wave, whose order the stages keep."""
+    (a log-sum-exp).  A row is walked by a wave, or by a block when it has more than 4096 elements: as the
+    separate reduction walks it, whose order the stages keep."""
     order, readers, seen = [], {}, set()
 
     def walk(t):
@@ -1018,9 +1018,10 @@ def _cluster_rows(roots: List[Tensor]) -> int:
         if rank == 0:
             return False
         cols, rows = full_shape[-1], prod(full_shape[:-1])
-        if cols > 4096 or cols % 8:
+        if cols % 8:
             return False
         per_row = tuple(full_shape[:-1]) + (1,)
+        carry_fits = cols <= 32768  # at most sixteen vectors per lane with a block per row (eight with a wave, <= 4096)
 
         def is_per_row(t, flat_too=False):
             if not (isinstance(t, Tensor) and isinstance(t.data, Expr) and _const(t) is None and t.type in _NARROW):
@@ -1147,7 +1148,7 @@ def _cluster_rows(roots: List[Tensor]) -> int:
             (the softmax's division begins with the exponentials its sum was taken over) reads those
             values where they still are -- the lanes' registers -- instead of computing them again."""
             mine = program[at:]
-            if (reduced and len(mine) >= len(reduced) and mine[:len(reduced)] == reduced
+            if (carry_fits and reduced and len(mine) >= len(reduced) and mine[:len(reduced)] == reduced
                     and not any(ins.get("flags", 0) >> 4 for ins in reduced)):
                 program[at:] = [{"kind": 0, "src": 4, "dt": reduced[-1]["dt"]}] + mine[len(reduced):]
 

@@ -674,11 +674,44 @@ def test_row_stages_are_bit_identical_to_node_by_node(name, shape, ty, hip):
         assert calls == [1]  # one launch for all stages
 
 
-def test_rows_longer_than_a_wave_takes_stay_separate_groups(hip):
-    x = rand_float(np.random.default_rng(6), "f32", (8, 8192), hip)
+@pytest.mark.parametrize("ty", ["f32", "bf16"])
+@pytest.mark.parametrize("shape", [(8, 8192), (64, 4104), (16, 32000), (3, 16384), (5, 16392)])
+@pytest.mark.parametrize("name", ["softmax_rows", "centred_and_scaled", "log_sum_exp_rows"])
+def test_long_rows_take_a_block_each(name, shape, ty, hip):
+    rng = np.random.default_rng(seed_of(name, shape, ty))
+    x = rand_float(rng, ty, shape, hip)
+    args = (x, rand_float(rng, ty, (shape[-1],), hip)) if name == "centred_and_scaled" else (x,)
+    fun = {"softmax_rows": softmax_rows, "centred_and_scaled": centred_and_scaled, "log_sum_exp_rows": log_sum_exp_rows}[name]
+    want = defn.compile(fun, *args)(*args)
+    planned = defn.compile(fun, *args, fuse="compiled")
+    assert type(planned.roots[0].data.args[0]).__name__ == "_RowCluster"
+    calls = []
+    original = hip.fused_elementwise.__func__
+
+    def counting(cls, *a, **k):
+        if "mode" in k:
+            calls.append(1)
+        return original(cls, *a, **k)
+    hip.fused_elementwise = classmethod(counting)
+    try:
+        assert_bits_equal(planned(*args), want, f"{name} {shape} {ty}")
+    finally:
+        hip.fused_elementwise = classmethod(original)
+    assert calls == [1]
+
+
+def test_rows_too_long_for_carried_values_are_read_again(hip):
+    x = rand_float(np.random.default_rng(7), "f32", (2048, 32776), hip)
     planned = defn.compile(softmax_rows, x, fuse="compiled")
-    assert type(planned.roots[0].data.args[0]).__name__ != "_RowCluster"
-    assert_bits_equal(planned(x), defn.compile(softmax_rows, x)(x), "long rows")
+    cluster = planned.roots[0].data.args[0]
+    assert type(cluster).__name__ == "_RowCluster" and not any(ins.get("src") == 4 for ins in cluster.program)
+    assert_bits_equal(planned(x), defn.compile(softmax_rows, x)(x), "rows of 32776")
+
+
+def test_rows_that_the_reduction_would_split_run_stage_by_stage(hip):
+    x = rand_float(np.random.default_rng(6), "f32", (4, 65536), hip)   # few rows, very long: the separate sum works in segments
+    planned = defn.compile(softmax_rows, x, fuse="compiled")
+    assert_bits_equal(planned(x), defn.compile(softmax_rows, x)(x), "split rows")
 
 
 def test_configuration_3_softmax_in_one_kernel(hip):
