@@ -205,7 +205,18 @@ class HipNxBackend:
             number_to_binary(number, out.type)  # the reference's argument checks
             elem = wrap_to_type(np.array([int(number)]), out.type).tobytes()
         else:
-            elem = number_to_binary(number, out.type)
+            # the same few numbers come back all the time (the 0.5 of `multiply(t, 0.5)`): their encodings are kept
+            # (a float by its sign and hex digits: 0.0 and -0.0 are equal as dictionary keys, and so are 1 and 1.0)
+            if number.__class__ in (int, float, bool):
+                memo = (out.type, number.hex() if number.__class__ is float else number, number.__class__)
+                elem = _encoded.get(memo)
+                if elem is None:
+                    elem = number_to_binary(number, out.type)
+                    if len(_encoded) > 4096:
+                        _encoded.clear()
+                    _encoded[memo] = elem
+            else:
+                elem = number_to_binary(number, out.type)
         if out.shape == ():
             key = (opts["device"], out.type, elem)
             ref = cls._scalar_cache.get(key)
@@ -946,6 +957,7 @@ def fused_mode(mode: str, device: int = 0) -> None:
     _fused_modes[device] = mode
 
 
+_encoded = {}  # (type, class of the number, number) -> its encoding (constant/3)
 _fused_modes = {}  # device -> the mode last set here
 _fused_arrays = {}  # (id of a layout, input types) -> (the layout itself, so the id stays its own; C arrays of types and strides)
 
