@@ -37,8 +37,8 @@ HEADLINE_TRAFFIC_BYTES = 235345715  # 98467 KiB x 2.0 fetched + 32895 KiB x 1.0 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=30)  # the clocks settle over the first tens of launches
     ap.add_argument("--no-suite", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--calibrate", action="store_true")
