@@ -397,7 +397,56 @@ __device__ __forceinline__ void gemm_epilogue(typename Mma16<DT>::acc_t (&acc)[T
       }
     }
   } else if constexpr (int_acc != int_out) return;  // the host never pairs them
-  else {
+  else if constexpr (!int_acc && (ODT == HIPNX_BF16 || ODT == HIPNX_F16) && TN % 2 == 0) {
+    // 2-byte outputs: a lane's 4 outputs of a tile are only 8 bytes, and a store instruction made of
+    // 32-byte runs per row is slow (measured on the 4096^3 bf16 case: 11 us of the kernel, twice the
+    // time the s32 epilogue takes for twice the bytes).  Two neighbouring column tiles are written
+    // together instead: lanes 16 apart hold adjacent groups of 4 columns, so they trade halves --
+    // the lane of the even group keeps tile j and receives its neighbour's 4 columns of tile j, the
+    // other keeps tile j+1 -- and every lane stores 16 bytes, 64 contiguous bytes per row.
+    const bool odd = (lane >> 4) & 1;
+    const int64_t gc = col0 + 4 * ((lane >> 4) & 2);  // first of this lane's 8 columns within its tile
+    auto pack = [](float lo, float hi) -> uint32_t {
+      if constexpr (ODT == HIPNX_BF16) return (uint32_t)f32_to_bf16_bits_trunc(lo) | ((uint32_t)f32_to_bf16_bits_trunc(hi) << 16);
+      else return (uint32_t)f32_to_f16_bits(lo) | ((uint32_t)f32_to_f16_bits(hi) << 16);
+    };
+    // N % 8 == 0: a group of 8 columns lies wholly inside or outside, and row starts keep the 16-byte alignment
+    const bool paired = (N % 8) == 0 && ((uintptr_t)out & 15) == 0;
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+      const int64_t gm = row0 + 16 * i + (lane & 15);
+#pragma unroll
+      for (int j = 0; j < TN; j += 2) {
+        if (paired) {
+          const uint32_t a0 = pack(acc[i][j][0], acc[i][j][1]), a1 = pack(acc[i][j][2], acc[i][j][3]);
+          const uint32_t b0 = pack(acc[i][j + 1][0], acc[i][j + 1][1]), b1 = pack(acc[i][j + 1][2], acc[i][j + 1][3]);
+          const uint32_t r0 = (uint32_t)__shfl_xor((int)(odd ? a0 : b0), 16, 64);
+          const uint32_t r1 = (uint32_t)__shfl_xor((int)(odd ? a1 : b1), 16, 64);
+          v4i v;
+          v[0] = (int)(odd ? r0 : a0); v[1] = (int)(odd ? r1 : a1); v[2] = (int)(odd ? b0 : r0); v[3] = (int)(odd ? b1 : r1);
+          const int64_t gn = gc + 16 * (j + (odd ? 1 : 0));
+          if (gm < M && gn < N) *reinterpret_cast<v4i *>((unsigned char *)out + (obase + gm * N + gn) * 2) = v;
+        } else {
+#pragma unroll
+          for (int jj = j; jj < j + 2; jj++) {
+            const int64_t gn = col0 + 16 * jj + 4 * (lane >> 4);
+            float v[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] = acc[i][jj][e];
+            const int64_t idx = obase + gm * N + gn;
+            if (gm < M) {
+              if ((N % 4) == 0 && gn + 4 <= N) store_vec<float, 4>(out, ODT, idx, v);
+              else {
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                  if (gn + e < N) store_one<float>(out, ODT, idx + e, v[e]);
+              }
+            }
+          }
+        }
+      }
+    }
+  } else {
     typedef typename std::conditional<int_acc, int64_t, float>::type S;
     const bool vec_ok = (N % 4) == 0;
 #pragma unroll

@@ -221,3 +221,21 @@ def test_large_ragged_dot_on_the_big_tile(ty, layout, hip, oracle):
         assert_bits_equal(got_rows, want, f"big tile s8 {layout}")
     else:
         check_float_dot(got_rows, want, values(oa), values(ob), "mk,kn->mn", K, f"big tile {ty} {layout}")
+
+
+@pytest.mark.parametrize("ty,M,N,K", [("bf16", 512, 520, 256), ("bf16", 300, 528, 128), ("f16", 264, 344, 128),
+                                      ("bf16", 130, 76, 64), ("f16", 64, 40, 128)])
+def test_two_byte_outputs_land_in_their_own_columns(ty, M, N, K, hip):
+    """The MFMA kernel writes bf16 / f16 results two column tiles at a time, lanes trading halves
+    so that each stores 16 bytes.  A selection matrix (one 1.0 per column) makes every output a
+    copy of one input element, so any mix-up of lanes, tiles or columns shows as a wrong value
+    -- exact, no tolerance."""
+    rng = np.random.default_rng(seed_of(ty, M, N, K))
+    a = rand_raw(rng, ty, (M, K), lo=-1, hi=1)
+    pick = (7 * np.arange(N) + 3) % K
+    b = np.zeros((K, N), dtype=a.dtype)
+    b[pick, np.arange(N)] = np.uint16(0x3F80) if ty == "bf16" else np.float16(1.0)
+    got = values(Nx.dot(from_numpy(a, ty, hip), from_numpy(b, ty, hip)))
+    want = values(from_numpy(np.ascontiguousarray(a[:, pick]), ty, hip))
+    assert got.shape == (M, N)
+    assert np.array_equal(got, want)  # (-0.0 == 0.0: a lone product plus zeros may lose the sign of a zero)
