@@ -1,0 +1,241 @@
+// hipnx_ceilings: what this MI355X sustains on the two rooflines the library is judged against,
+// measured the way the library's own kernels are timed (back-to-back launches on one stream, HIP
+// events), so that a kernel's fraction of the published peak can be read beside the fraction of what
+// the part actually delivers under its power management.
+//
+//   hipnx_ceilings mfma <bf16|f16|s8|f32> <random|normal|zero> [ms]
+//       an MFMA-only loop (the 16x16 forms the contraction kernel uses, 8 waves per CU, 32
+//       independent accumulator tiles per wave, operands in registers, no memory traffic) launched
+//       back to back for `ms` milliseconds; throughput is reported for the first 2 ms, for each fifth
+//       of the run and for the last fifth (the sustained figure: the clock the part settles at
+//       under this load depends on the operand bits and takes tens of milliseconds to settle)
+//   hipnx_ceilings stream <read|write|copy> [MiB] [ms]
+//       16-byte-per-lane streaming kernels over a buffer larger than the 256 MB last-level cache
+//
+// Each run prints one JSON line.  Built by the Makefile into nx_amd/lib/hipnx_ceilings; bench.py runs
+// it when present and copies the sustained figures into its `measured_ceiling` fields.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#define CK(x)                                                                          \
+  do {                                                                                 \
+    hipError_t e__ = (x);                                                              \
+    if (e__ != hipSuccess) {                                                           \
+      fprintf(stderr, "HIP error %s at line %d\n", hipGetErrorString(e__), __LINE__);  \
+      return 1;                                                                        \
+    }                                                                                  \
+  } while (0)
+
+typedef __attribute__((ext_vector_type(8))) __bf16 v8bf;
+typedef __attribute__((ext_vector_type(8))) _Float16 v8h;
+typedef __attribute__((ext_vector_type(4))) float v4f;
+typedef __attribute__((ext_vector_type(4))) int v4i;
+
+__device__ unsigned long long g_clk[2];
+
+enum { K_BF16 = 0, K_F16 = 1, K_S8 = 2, K_F32 = 3 };
+
+// 4 x 8 accumulator tiles of 16 x 16 per wave (the contraction kernel's wave tile); one trip of the
+// loop = 2 K steps x 32 tiles = 64 MFMA instructions (f32: 4 x 64, one per 4 k)
+template <int KIND>
+__global__ void __launch_bounds__(512) mfma_loop(const v4i *src, float *out, int iters) {
+  const int tid = threadIdx.x;
+  v4i pa[4], pb[8];
+  for (int q = 0; q < 4; q++) pa[q] = src[(blockIdx.x * 512 + tid) * 12 + q];
+  for (int q = 0; q < 8; q++) pb[q] = src[(blockIdx.x * 512 + tid) * 12 + 4 + q];
+  const unsigned long long c0 = clock64(), w0 = wall_clock64();
+  float sum = 0;
+  if constexpr (KIND == K_S8) {
+    v4i acc[4][8];
+    for (int i = 0; i < 4; i++) for (int j = 0; j < 8; j++) for (int q = 0; q < 4; q++) acc[i][j][q] = 0;
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+      for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+          for (int j = 0; j < 8; j++)
+            acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(pb[(ks + j) & 7], pa[(ks + i) & 3], acc[i][j], 0, 0, 0);
+    }
+    for (int i = 0; i < 4; i++) for (int j = 0; j < 8; j++) for (int q = 0; q < 4; q++) sum += acc[i][j][q];
+  } else {
+    v4f acc[4][8];
+    for (int i = 0; i < 4; i++) for (int j = 0; j < 8; j++) for (int q = 0; q < 4; q++) acc[i][j][q] = 0;
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+      for (int ks = 0; ks < (KIND == K_F32 ? 8 : 2); ks++)
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+          for (int j = 0; j < 8; j++) {
+            if constexpr (KIND == K_BF16)
+              acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, pb[(ks + j) & 7]), __builtin_bit_cast(v8bf, pa[(ks + i) & 3]), acc[i][j], 0, 0, 0);
+            else if constexpr (KIND == K_F16)
+              acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, pb[(ks + j) & 7]), __builtin_bit_cast(v8h, pa[(ks + i) & 3]), acc[i][j], 0, 0, 0);
+            else
+              acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(__int_as_float(pb[j][ks & 3]), __int_as_float(pa[i][ks & 3]), acc[i][j], 0, 0, 0);
+          }
+    }
+    for (int i = 0; i < 4; i++) for (int j = 0; j < 8; j++) for (int q = 0; q < 4; q++) sum += acc[i][j][q];
+  }
+  out[blockIdx.x * 512 + tid] = sum;
+  if (blockIdx.x == 8 && tid == 0) {
+    g_clk[0] = clock64() - c0;
+    g_clk[1] = wall_clock64() - w0;
+  }
+}
+
+__global__ void __launch_bounds__(256) stream_read(const v4i *__restrict__ in, v4i *__restrict__ out, size_t n) {
+  v4i acc = {0, 0, 0, 0};
+  const size_t stride = (size_t)gridDim.x * 256;
+  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  for (; i + 3 * stride < n; i += 4 * stride) {
+    const v4i a = in[i], b = in[i + stride], c = in[i + 2 * stride], d = in[i + 3 * stride];
+    acc ^= a ^ b ^ c ^ d;
+  }
+  for (; i < n; i += stride) acc ^= in[i];
+  if (acc[0] == 0x12345678 && acc[1] == 0x0BADF00D) out[0] = acc;  // keeps the loads alive; practically never taken
+}
+__global__ void __launch_bounds__(256) stream_write(v4i *__restrict__ out, size_t n, int v) {
+  const v4i x = {v, v + 1, v + 2, v + 3};
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) out[i] = x;
+}
+__global__ void __launch_bounds__(256) stream_copy(const v4i *__restrict__ in, v4i *__restrict__ out, size_t n) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  for (; i + stride < n; i += 2 * stride) {
+    const v4i a = in[i], b = in[i + stride];
+    out[i] = a;
+    out[i + stride] = b;
+  }
+  for (; i < n; i += stride) out[i] = in[i];
+}
+
+static void launch_mfma(int kind, const v4i *d, float *o, int iters) {
+  switch (kind) {
+    case K_BF16: hipLaunchKernelGGL(mfma_loop<K_BF16>, dim3(256), dim3(512), 0, 0, d, o, iters); break;
+    case K_F16: hipLaunchKernelGGL(mfma_loop<K_F16>, dim3(256), dim3(512), 0, 0, d, o, iters); break;
+    case K_S8: hipLaunchKernelGGL(mfma_loop<K_S8>, dim3(256), dim3(512), 0, 0, d, o, iters); break;
+    default: hipLaunchKernelGGL(mfma_loop<K_F32>, dim3(256), dim3(512), 0, 0, d, o, iters); break;
+  }
+}
+
+// times `chunks` chunks of back-to-back launches with one event pair each; returns ms per chunk
+template <typename F>
+static int timed_chunks(F &&launch, int chunks, int per_chunk, std::vector<float> &ms) {
+  std::vector<hipEvent_t> ev(chunks + 1);
+  for (int i = 0; i <= chunks; i++) {
+    hipEvent_t x;
+    CK(hipEventCreate(&x));
+    ev[i] = x;
+  }
+  CK(hipEventRecord(ev[0]));
+  for (int c = 0; c < chunks; c++) {
+    for (int i = 0; i < per_chunk; i++) launch();
+    CK(hipEventRecord(ev[c + 1]));
+  }
+  CK(hipEventSynchronize(ev[chunks]));
+  ms.resize(chunks);
+  for (int c = 0; c < chunks; c++) CK(hipEventElapsedTime(&ms[c], ev[c], ev[c + 1]));
+  CK(hipGetLastError());
+  return 0;
+}
+
+static int run_mfma(const char *type, const char *data, double want_ms) {
+  const int kind = !strcmp(type, "bf16") ? K_BF16 : !strcmp(type, "f16") ? K_F16 : !strcmp(type, "s8") ? K_S8 : !strcmp(type, "f32") ? K_F32 : -1;
+  if (kind < 0) { fprintf(stderr, "unknown type %s\n", type); return 2; }
+  const size_t nwords = (size_t)256 * 512 * 12 * 4;  // v4i per lane x 12
+  std::vector<uint32_t> h(nwords);
+  srand(1);
+  auto uni = [] { return rand() / (float)RAND_MAX; };
+  for (size_t w = 0; w < nwords; w++) {
+    uint32_t word = 0;
+    const int per = kind == K_S8 ? 4 : kind == K_F32 ? 1 : 2;
+    for (int e = 0; e < per; e++) {
+      float f = 0;
+      if (!strcmp(data, "random")) f = uni() * 2 - 1;
+      else if (!strcmp(data, "normal")) f = sqrtf(-2 * logf((float)((rand() + 1.0) / (RAND_MAX + 2.0)))) * cosf(6.2831853f * uni()) / 64;  // the benchmark's operands
+      uint32_t bits;
+      std::memcpy(&bits, &f, 4);
+      if (kind == K_S8) word |= (uint32_t)(uint8_t)(int8_t)(strcmp(data, "zero") ? (rand() % 255) - 127 : 0) << (8 * e);
+      else if (kind == K_F32) word = bits;
+      else if (kind == K_BF16) word |= (bits >> 16) << (16 * e);
+      else { _Float16 hf = (_Float16)f; uint16_t hb; std::memcpy(&hb, &hf, 2); word |= (uint32_t)hb << (16 * e); }
+    }
+    h[w] = word;
+  }
+  v4i *d;
+  float *o;
+  CK(hipMalloc(&d, nwords * 4));
+  CK(hipMalloc(&o, 256 * 512 * 4));
+  CK(hipMemcpy(d, h.data(), nwords * 4, hipMemcpyHostToDevice));
+  const int iters = kind == K_F32 ? 24 : 96;  // about 100 us per launch
+  // flop per launch: 256 groups x 8 waves x iters x instructions x flop per instruction
+  const double per_instr = kind == K_S8 ? 2.0 * 16 * 16 * 64 : kind == K_F32 ? 2.0 * 16 * 16 * 4 : 2.0 * 16 * 16 * 32;
+  const double flop = 256.0 * 8 * iters * (kind == K_F32 ? 256 : 64) * per_instr;
+  std::vector<float> probe;
+  if (timed_chunks([&] { launch_mfma(kind, d, o, iters); }, 1, 5, probe)) return 1;
+  const double launch_ms = probe[0] / 5;
+  const int per_chunk = std::max(1, (int)(2.0 / launch_ms));               // about 2 ms per chunk
+  const int chunks = std::max(5, (int)(want_ms / (per_chunk * launch_ms)));
+  CK(hipDeviceSynchronize());
+  std::vector<float> ms;
+  if (timed_chunks([&] { launch_mfma(kind, d, o, iters); }, chunks, per_chunk, ms)) return 1;
+  unsigned long long c[2];
+  CK(hipMemcpyFromSymbol(c, HIP_SYMBOL(g_clk), sizeof(c)));
+  auto rate = [&](int a, int b) { double t = 0; for (int i = a; i < b; i++) t += ms[i]; return flop * per_chunk * (b - a) / t / 1e9; };
+  printf("{\"kind\": \"mfma\", \"dtype\": \"%s\", \"operands\": \"%s\", \"unit\": \"%s\", \"first_2ms\": %.1f, \"fifths\": [", type, data,
+         kind == K_S8 ? "TOP/s" : "TFLOP/s", rate(0, 1));
+  for (int q = 0; q < 5; q++) printf("%s%.1f", q ? ", " : "", rate(chunks * q / 5, chunks * (q + 1) / 5));
+  printf("], \"sustained\": %.1f, \"run_ms\": %.1f, \"launch_us\": %.1f, \"clock_mhz_last_launch\": %.0f, \"clocks_per_instruction\": %.2f}\n",
+         rate(chunks * 4 / 5, chunks), [&] { double t = 0; for (float x : ms) t += x; return t; }(), 1000 * ms[chunks - 1] / per_chunk,
+         c[0] / (c[1] / 100.0), (double)c[0] / ((double)iters * (kind == K_F32 ? 256 : 64)));
+  return 0;
+}
+
+static int run_stream(const char *mode, size_t mib, double want_ms) {
+  const size_t bytes = mib << 20, n = bytes / 16;
+  v4i *a, *b;
+  CK(hipMalloc(&a, bytes));
+  CK(hipMalloc(&b, bytes));
+  CK(hipMemset(a, 1, bytes));
+  CK(hipMemset(b, 2, bytes));
+  const int m = !strcmp(mode, "read") ? 0 : !strcmp(mode, "write") ? 1 : !strcmp(mode, "copy") ? 2 : -1;
+  if (m < 0) { fprintf(stderr, "unknown mode %s\n", mode); return 2; }
+  const unsigned grid = 256 * 32;
+  auto launch = [&] {
+    if (m == 0) hipLaunchKernelGGL(stream_read, dim3(grid), dim3(256), 0, 0, a, b, n);
+    else if (m == 1) hipLaunchKernelGGL(stream_write, dim3(grid), dim3(256), 0, 0, b, n, 7);
+    else hipLaunchKernelGGL(stream_copy, dim3(grid), dim3(256), 0, 0, a, b, n);
+  };
+  std::vector<float> probe;
+  if (timed_chunks(launch, 1, 3, probe)) return 1;
+  const double launch_ms = probe[0] / 3;
+  const int per_chunk = std::max(1, (int)(2.0 / launch_ms));
+  const int chunks = std::max(5, (int)(want_ms / (per_chunk * launch_ms)));
+  std::vector<float> ms;
+  if (timed_chunks(launch, chunks, per_chunk, ms)) return 1;
+  const double moved = (m == 2 ? 2.0 : 1.0) * bytes;
+  auto rate = [&](int x, int y) { double t = 0; for (int i = x; i < y; i++) t += ms[i]; return moved * per_chunk * (y - x) / t / 1e6; };
+  std::vector<float> sorted(ms);
+  std::sort(sorted.begin(), sorted.end());
+  printf("{\"kind\": \"stream\", \"mode\": \"%s\", \"MiB\": %zu, \"unit\": \"GB/s\", \"bytes_counted\": \"%s\", \"sustained\": %.0f, \"best_chunk\": %.0f, \"launch_us\": %.1f}\n",
+         mode, mib, m == 2 ? "read + written" : "one direction", rate(chunks * 4 / 5, chunks), moved * per_chunk / sorted[0] / 1e6,
+         1000 * ms[chunks - 1] / per_chunk);
+  return 0;
+}
+
+int main(int argc, char **argv) {
+  if (argc >= 4 && !strcmp(argv[1], "mfma")) return run_mfma(argv[2], argv[3], argc > 4 ? atof(argv[4]) : 300.0);
+  if (argc >= 3 && !strcmp(argv[1], "stream")) return run_stream(argv[2], argc > 3 ? (size_t)atol(argv[3]) : 2048, argc > 4 ? atof(argv[4]) : 100.0);
+  fprintf(stderr, "usage: hipnx_ceilings mfma <bf16|f16|s8|f32> <random|normal|zero> [ms]\n       hipnx_ceilings stream <read|write|copy> [MiB] [ms]\n");
+  return 2;
+}

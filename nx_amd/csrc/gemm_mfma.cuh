@@ -488,7 +488,7 @@ __device__ __forceinline__ void wait_vmcnt() {  // s_waitcnt vmcnt(N), other cou
   __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
 }
 
-template <int DT, int WM, int WN, int TM, int TN, bool L_KIN, bool R_KIN, int NSTAGE = 2>
+template <int DT, int WM, int WN, int TM, int TN, bool L_KIN, bool R_KIN, int NSTAGE = 2, bool EARLY = false>
 __global__ void __launch_bounds__(WM *WN * 64)
 gemm_pipelined_kernel(GemmArgs a) {
   typedef typename Mma16<DT>::acc_t acc_t;
@@ -611,6 +611,20 @@ gemm_pipelined_kernel(GemmArgs a) {
 
   constexpr bool ALL_DMA = (L_KIN || L_TR) && (R_KIN || R_TR);
   static_assert(NSTAGE == 2 || ALL_DMA, "register-staged operands need the two-stage walk");
+  // EARLY (two stages, every operand by direct-to-LDS loads): the requests of a slab start right
+  // behind the barrier that frees its stage -- in the POST steps that follow the barrier of the slab
+  // before the previous one's successor -- instead of at the next slab's first step, one
+  // instruction per step (l in even, r in odd virtual steps u = 0, 1, ..): the last request then
+  // has POST more steps to land before the barrier that publishes the slab.
+  constexpr int POST = STEPS - 1 - BAR;
+  static_assert(!EARLY || (NSTAGE == 2 && ALL_DMA), "early requests need two stages of direct-to-LDS operands");
+  auto issue_early = [&](int u, int stage, int64_t kbyte0) {
+    unsigned char *sA = smem + stage * STAGE, *sB = sA + BM * SLAB;
+    if constexpr (L_KIN) lload.issue_at(u, 2 * KInnerLoader<BM, NW>::PER, 0, 0, kbyte0, sA);
+    else if constexpr (L_TR) ltr.issue_at(u, 2 * KOuterDmaLoader<TR_ES, L_TR ? BM : 256 * NW, NW>::PER, 0, 0, kbyte0 / ES, a.ld_l, sA);
+    if constexpr (R_KIN) rload.issue_at(u, 2 * KInnerLoader<BN, NW>::PER, 1, 0, kbyte0, sB);
+    else if constexpr (R_TR) rtr.issue_at(u, 2 * KOuterDmaLoader<TR_ES, R_TR ? BN : 256 * NW, NW>::PER, 1, 0, kbyte0 / ES, a.ld_r, sB);
+  };
   constexpr int OPS = (L_KIN ? KInnerLoader<BM, NW>::PER : L_TR ? KOuterDmaLoader<TR_ES, L_TR ? BM : 256 * NW, NW>::PER : 0) +
                       (R_KIN ? KInnerLoader<BN, NW>::PER : R_TR ? KOuterDmaLoader<TR_ES, R_TR ? BN : 256 * NW, NW>::PER : 0);
   constexpr int INFLIGHT = OPS * (NSTAGE - 2);  // requests of younger slabs that may stay outstanding
@@ -623,6 +637,12 @@ gemm_pipelined_kernel(GemmArgs a) {
   if (nslab >= NSTAGE - 1) wait_vmcnt<INFLIGHT>();
   else wait_vmcnt<0>();
   __syncthreads();
+  if constexpr (EARLY) {  // the first requests of slab 1 (what the steps behind a barrier would have issued)
+    if (1 < nslab) {
+#pragma unroll
+      for (int u = 0; u < POST; u++) issue_early(u, 1, SLAB);
+    }
+  }
   v4i fa[2][TM16], fb[RING];
 #pragma unroll
   for (int i = 0; i < TM16; i++) fa[0][i] = read_l(smem, 0, i);
@@ -657,7 +677,11 @@ gemm_pipelined_kernel(GemmArgs a) {
         for (int i = 0; i < TM16; i++)
           if (i >= d * TM16 / DIST && i < (d + 1) * TM16 / DIST) fa[0][i] = read_l(nxt, 0, i);
       }
-      if (request && t <= BAR) issue_step(t, req_stage, req_kbyte);
+      if constexpr (EARLY) {
+        if (t > BAR) {
+          if (s + 2 < nslab) issue_early(t - BAR - 1, s % NSTAGE, (int64_t)(s + 2) * SLAB);
+        } else if (request) issue_early(t + POST, req_stage, req_kbyte);
+      } else if (request && t <= BAR) issue_step(t, req_stage, req_kbyte);
 #pragma unroll
       for (int i = 0; i < TM16; i++) Mma16<DT>::step(acc[i][j], fb[t % RING], fa[ks & 1][i]);
       __builtin_amdgcn_s_setprio(0);
