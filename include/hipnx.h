@@ -164,6 +164,17 @@ int hipnx_as_type(hipnx_ctx *ctx, int in_dt, int out_dt, int64_t n, const hipnx_
 int hipnx_reduce(hipnx_ctx *ctx, int op, int in_dt, int out_dt, int64_t outer, int64_t red,
                  int64_t inner, const hipnx_buf *in, hipnx_buf *out);
 
+/* No counterpart in the reference: hipnx_reduce for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  Same
+ * arguments, same kernels, same results bit for bit; the partial results of a split reduction go
+ * to a static device array of HIPNX_REDUCE_STATIC_SCRATCH_BYTES (held by every GPU the library runs
+ * on until the process ends) instead of a pool block, and the call performs no hipMalloc / hipFree.
+ * A shape whose partials do not fit fails with HIPNX_EUNSUPPORTED and launches nothing.  All calls
+ * on one GPU share that array: calls that overlap on one GPU (two contexts, i.e. two streams) race. */
+#define HIPNX_REDUCE_STATIC_SCRATCH_BYTES (1u << 20)
+int hipnx_reduce_static(hipnx_ctx *ctx, int op, int in_dt, int out_dt, int64_t outer, int64_t red,
+                        int64_t inner, const hipnx_buf *in, hipnx_buf *out);
+
 /* replaces: argmax / argmin (nx/lib/nx/backend.ex:93-94; oracle binary_backend.ex:1393-1431).
  * Same view.  tie LOW = first index of the extreme, HIGH = last; any NaN wins and the last
  * NaN's index is returned.  out_dt is an integer type. */

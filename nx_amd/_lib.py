@@ -81,6 +81,7 @@ PROTOTYPES = {
     "hipnx_unary": [_ctx_p, C.c_int, C.c_int, C.c_int, C.c_int64, _buf_p, _buf_p],
     "hipnx_as_type": [_ctx_p, C.c_int, C.c_int, C.c_int64, _buf_p, _buf_p],
     "hipnx_reduce": [_ctx_p, C.c_int, C.c_int, C.c_int, C.c_int64, C.c_int64, C.c_int64, _buf_p, _buf_p],
+    "hipnx_reduce_static": [_ctx_p, C.c_int, C.c_int, C.c_int, C.c_int64, C.c_int64, C.c_int64, _buf_p, _buf_p],
     "hipnx_argreduce": [_ctx_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int64, C.c_int64, C.c_int64, _buf_p, _buf_p],
     "hipnx_dot": [_ctx_p, C.c_int, C.c_int, C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_int,
                   _buf_p, _buf_p, _buf_p],

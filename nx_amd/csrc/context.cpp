@@ -178,6 +178,10 @@ int hipnx_ctx_create(int device, hipnx_ctx **out) {
     return hip_fail(e1 != hipSuccess ? e1 : e2 != hipSuccess ? e2 : e3 != hipSuccess ? e3 : e4 != hipSuccess ? e4 : e5,
                     "context set-up");
   }
+  if (int st = reduce_static_init(ctx)) {
+    hipnx_ctx_destroy(ctx);
+    return st;
+  }
   *out = ctx;
   return HIPNX_OK;
 }

@@ -41,6 +41,7 @@ struct hipnx_ctx {
   void *flag = nullptr;       // 32-byte device scratch for the gather bounds report
   void *flag_host = nullptr;  // pinned host word, mapped into the device: non-zero once a kernel saw a bad index
   void *flag_host_dev = nullptr;  // its device address
+  void *reduce_scratch = nullptr;  // this device's address of the static partial-result array of reduce.hip
   hipnx_graph *capture = nullptr;                        // non-null while the stream is capturing
   std::unordered_map<void *, hipnx_graph *> graph_blocks;  // block -> the live graph that owns it
   std::vector<hipnx_graph *> graphs;                     // live graphs of this context
@@ -85,6 +86,10 @@ int check_buf(const hipnx_ctx *ctx, const hipnx_buf *b, uint64_t need_bytes, con
 // pooled device memory; both expect the context mutex to be held (i.e. inside an Enter scope)
 int pool_alloc(hipnx_ctx *ctx, size_t bytes, void **ptr_out, size_t *cap_out);
 int pool_free(hipnx_ctx *ctx, void *ptr, size_t cap);
+
+// looks up this device's address of the static scratch array of hipnx_reduce_static (the device of
+// `ctx` must be current); defined beside the array in reduce.hip
+int reduce_static_init(hipnx_ctx *ctx);
 
 // entry points that wait for the device cannot run while the stream is capturing
 #define HIPNX_NOT_CAPTURING(ctx, what)                                                                 \

@@ -165,9 +165,26 @@ combine_cols_kernel(const typename R::acc_t *__restrict__ partial, void *__restr
 
 static int64_t round_up(int64_t a, int64_t b) { return (a + b - 1) / b * b; }
 
+// Partial results of a split reduction live either in a block of the context's pool (handed back
+// right after the launches: later work on this stream is ordered behind them) or, for the entry
+// point that allocates nothing, in this file's static device array.
+static int partials_acquire(hipnx_ctx *ctx, bool static_ws, size_t bytes, void **ws, size_t *ws_cap) {
+  if (!static_ws) return pool_alloc(ctx, bytes, ws, ws_cap);
+  *ws_cap = 0;
+  if (bytes > HIPNX_REDUCE_STATIC_SCRATCH_BYTES)
+    return set_error(HIPNX_EUNSUPPORTED, "reduce_static: this shape needs %zu bytes of partial results, the static scratch holds %zu",
+                     bytes, (size_t)HIPNX_REDUCE_STATIC_SCRATCH_BYTES);
+  if (!ctx->reduce_scratch) return set_error(HIPNX_EHIP, "reduce_static: the static scratch of this device was not resolved");
+  *ws = ctx->reduce_scratch;
+  return HIPNX_OK;
+}
+static void partials_release(hipnx_ctx *ctx, bool static_ws, void *ws, size_t ws_cap) {
+  if (ws && !static_ws) pool_free(ctx, ws, ws_cap);
+}
+
 template <typename R, typename CT>
-static int run_reduce(hipnx_ctx *ctx, int idt, int odt, int64_t outer, int64_t red, int64_t inner, const void *in,
-                      void *out) {
+static int run_reduce(hipnx_ctx *ctx, bool static_ws, int idt, int odt, int64_t outer, int64_t red, int64_t inner,
+                      const void *in, void *out) {
   typedef typename R::acc_t acc_t;
   const int64_t target_units = (int64_t)ctx->num_cus * 8;  // units of parallel work wanted
   if (inner == 1) {
@@ -190,9 +207,7 @@ static int run_reduce(hipnx_ctx *ctx, int idt, int odt, int64_t outer, int64_t r
     void *ws = nullptr;
     size_t ws_cap = 0;
     if (nseg > 1) {
-      // workspace from the context pool; handed back right after the launches, which is safe
-      // because later work on this stream is ordered behind them
-      if (int st = pool_alloc(ctx, sizeof(acc_t) * (size_t)(rows * nseg), &ws, &ws_cap)) return st;
+      if (int st = partials_acquire(ctx, static_ws, sizeof(acc_t) * (size_t)(rows * nseg), &ws, &ws_cap)) return st;
       partial = (acc_t *)ws;
     }
     const int rpb = BLOCK / tpr;
@@ -210,7 +225,7 @@ static int run_reduce(hipnx_ctx *ctx, int idt, int odt, int64_t outer, int64_t r
         hipLaunchKernelGGL((combine_partials_kernel<R>), g2, block, 0, ctx->stream, partial, out, odt, rows, nseg);
       }
     }
-    if (ws) pool_free(ctx, ws, ws_cap);
+    partials_release(ctx, static_ws, ws, ws_cap);
   } else {
     const bool vec = inner % E == 0;
     const int64_t lanes = outer * (inner / (vec ? E : 1));
@@ -229,7 +244,7 @@ static int run_reduce(hipnx_ctx *ctx, int idt, int odt, int64_t outer, int64_t r
     void *ws = nullptr;
     size_t ws_cap = 0;
     if (nseg > 1) {
-      if (int st = pool_alloc(ctx, sizeof(acc_t) * (size_t)(outer * nseg * inner), &ws, &ws_cap)) return st;
+      if (int st = partials_acquire(ctx, static_ws, sizeof(acc_t) * (size_t)(outer * nseg * inner), &ws, &ws_cap)) return st;
       partial = (acc_t *)ws;
     }
     int64_t total = lanes * nseg;
@@ -245,32 +260,32 @@ static int run_reduce(hipnx_ctx *ctx, int idt, int odt, int64_t outer, int64_t r
         hipLaunchKernelGGL((combine_cols_kernel<R>), g2, block, 0, ctx->stream, partial, out, odt, outer, inner, nseg);
       }
     }
-    if (ws) pool_free(ctx, ws, ws_cap);
+    partials_release(ctx, static_ws, ws, ws_cap);
   }
   HIPNX_HIP(hipGetLastError());
   return HIPNX_OK;
 }
 
 template <int OP>
-static int reduce_op(hipnx_ctx *ctx, int idt, int odt, int64_t outer, int64_t red, int64_t inner, const void *in,
+static int reduce_op(hipnx_ctx *ctx, bool static_ws, int idt, int odt, int64_t outer, int64_t red, int64_t inner, const void *in,
                      void *out) {
   // selection (max / min) is exact in the element's own precision: f32 covers f32, bf16 and f16
   if (is_float(idt) && idt != HIPNX_F64 && (OP == HIPNX_RED_MAX || OP == HIPNX_RED_MIN || OP == HIPNX_RED_ALL || OP == HIPNX_RED_ANY))
-    return run_reduce<PlainReducer<float, OP, false>, float>(ctx, idt, odt, outer, red, inner, in, out);
-  if (is_float(idt)) return run_reduce<PlainReducer<double, OP, false>, double>(ctx, idt, odt, outer, red, inner, in, out);
+    return run_reduce<PlainReducer<float, OP, false>, float>(ctx, static_ws, idt, odt, outer, red, inner, in, out);
+  if (is_float(idt)) return run_reduce<PlainReducer<double, OP, false>, double>(ctx, static_ws, idt, odt, outer, red, inner, in, out);
   if (idt == HIPNX_U64 && (OP == HIPNX_RED_MAX || OP == HIPNX_RED_MIN))
-    return run_reduce<PlainReducer<int64_t, OP, true>, int64_t>(ctx, idt, odt, outer, red, inner, in, out);
-  return run_reduce<PlainReducer<int64_t, OP, false>, int64_t>(ctx, idt, odt, outer, red, inner, in, out);
+    return run_reduce<PlainReducer<int64_t, OP, true>, int64_t>(ctx, static_ws, idt, odt, outer, red, inner, in, out);
+  return run_reduce<PlainReducer<int64_t, OP, false>, int64_t>(ctx, static_ws, idt, odt, outer, red, inner, in, out);
 }
 
 template <int OP, int TIE>
 static int argreduce_op(hipnx_ctx *ctx, int idt, int odt, int64_t outer, int64_t red, int64_t inner, const void *in,
                         void *out) {
   if (is_float(idt) && idt != HIPNX_F64)
-    return run_reduce<ArgReducer<float, OP, TIE, false>, float>(ctx, idt, odt, outer, red, inner, in, out);
-  if (is_float(idt)) return run_reduce<ArgReducer<double, OP, TIE, false>, double>(ctx, idt, odt, outer, red, inner, in, out);
-  if (idt == HIPNX_U64) return run_reduce<ArgReducer<int64_t, OP, TIE, true>, int64_t>(ctx, idt, odt, outer, red, inner, in, out);
-  return run_reduce<ArgReducer<int64_t, OP, TIE, false>, int64_t>(ctx, idt, odt, outer, red, inner, in, out);
+    return run_reduce<ArgReducer<float, OP, TIE, false>, float>(ctx, false, idt, odt, outer, red, inner, in, out);
+  if (is_float(idt)) return run_reduce<ArgReducer<double, OP, TIE, false>, double>(ctx, false, idt, odt, outer, red, inner, in, out);
+  if (idt == HIPNX_U64) return run_reduce<ArgReducer<int64_t, OP, TIE, true>, int64_t>(ctx, false, idt, odt, outer, red, inner, in, out);
+  return run_reduce<ArgReducer<int64_t, OP, TIE, false>, int64_t>(ctx, false, idt, odt, outer, red, inner, in, out);
 }
 
 }  // namespace hipnx
@@ -282,8 +297,8 @@ static int check_view(int64_t outer, int64_t red, int64_t inner) {
   return HIPNX_OK;
 }
 
-extern "C" int hipnx_reduce(hipnx_ctx *ctx, int op, int in_dt, int out_dt, int64_t outer, int64_t red,
-                            int64_t inner, const hipnx_buf *inb, hipnx_buf *out) {
+static int reduce_entry(hipnx_ctx *ctx, bool static_ws, int op, int in_dt, int out_dt, int64_t outer, int64_t red,
+                        int64_t inner, const hipnx_buf *inb, hipnx_buf *out) {
   Enter in(ctx);
   if (in.status) return in.status;
   if (op < 0 || op > HIPNX_RED_ANY) return set_error(HIPNX_EINVAL, "reduce: unknown op %d", op);
@@ -295,13 +310,40 @@ extern "C" int hipnx_reduce(hipnx_ctx *ctx, int op, int in_dt, int out_dt, int64
   if (int st = check_buf(ctx, out, (uint64_t)outer * inner * dtype_size(out_dt), "reduce out")) return st;
   if (outer * inner == 0) return HIPNX_OK;
   switch (op) {
-    case HIPNX_RED_SUM: return reduce_op<HIPNX_RED_SUM>(ctx, in_dt, out_dt, outer, red, inner, inb->ptr, out->ptr);
-    case HIPNX_RED_MAX: return reduce_op<HIPNX_RED_MAX>(ctx, in_dt, out_dt, outer, red, inner, inb->ptr, out->ptr);
-    case HIPNX_RED_MIN: return reduce_op<HIPNX_RED_MIN>(ctx, in_dt, out_dt, outer, red, inner, inb->ptr, out->ptr);
-    case HIPNX_RED_PRODUCT: return reduce_op<HIPNX_RED_PRODUCT>(ctx, in_dt, out_dt, outer, red, inner, inb->ptr, out->ptr);
-    case HIPNX_RED_ALL: return reduce_op<HIPNX_RED_ALL>(ctx, in_dt, out_dt, outer, red, inner, inb->ptr, out->ptr);
-    default: return reduce_op<HIPNX_RED_ANY>(ctx, in_dt, out_dt, outer, red, inner, inb->ptr, out->ptr);
+    case HIPNX_RED_SUM: return reduce_op<HIPNX_RED_SUM>(ctx, static_ws, in_dt, out_dt, outer, red, inner, inb->ptr, out->ptr);
+    case HIPNX_RED_MAX: return reduce_op<HIPNX_RED_MAX>(ctx, static_ws, in_dt, out_dt, outer, red, inner, inb->ptr, out->ptr);
+    case HIPNX_RED_MIN: return reduce_op<HIPNX_RED_MIN>(ctx, static_ws, in_dt, out_dt, outer, red, inner, inb->ptr, out->ptr);
+    case HIPNX_RED_PRODUCT: return reduce_op<HIPNX_RED_PRODUCT>(ctx, static_ws, in_dt, out_dt, outer, red, inner, inb->ptr, out->ptr);
+    case HIPNX_RED_ALL: return reduce_op<HIPNX_RED_ALL>(ctx, static_ws, in_dt, out_dt, outer, red, inner, inb->ptr, out->ptr);
+    default: return reduce_op<HIPNX_RED_ANY>(ctx, static_ws, in_dt, out_dt, outer, red, inner, inb->ptr, out->ptr);
   }
+}
+
+extern "C" int hipnx_reduce(hipnx_ctx *ctx, int op, int in_dt, int out_dt, int64_t outer, int64_t red,
+                            int64_t inner, const hipnx_buf *inb, hipnx_buf *out) {
+  return reduce_entry(ctx, false, op, in_dt, out_dt, outer, red, inner, inb, out);
+}
+
+// ---- the reduction that allocates nothing ------------------------------------------------------
+// The partial results of a split reduction (few rows x a long axis, or few columns under a long
+// axis) go to this array instead of a pool block.  In host code its name is only a stand-in for the
+// symbol: the device address is looked up once per context (hipnx_ctx_create calls
+// reduce_static_init with the device current; every device holds its own copy at its own address)
+// and only that address is ever handed to a kernel.  Nothing in it has to start at zero -- every
+// partial a combine kernel reads was written by the launch before it -- so a call leaves the last
+// call's partials behind and clears nothing.
+static __device__ __align__(256) unsigned char scratch[HIPNX_REDUCE_STATIC_SCRATCH_BYTES];
+
+int hipnx::reduce_static_init(hipnx_ctx *ctx) {
+  void *ptr = nullptr;
+  HIPNX_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+  ctx->reduce_scratch = ptr;
+  return HIPNX_OK;
+}
+
+extern "C" int hipnx_reduce_static(hipnx_ctx *ctx, int op, int in_dt, int out_dt, int64_t outer, int64_t red,
+                                   int64_t inner, const hipnx_buf *inb, hipnx_buf *out) {
+  return reduce_entry(ctx, true, op, in_dt, out_dt, outer, red, inner, inb, out);
 }
 
 extern "C" int hipnx_argreduce(hipnx_ctx *ctx, int op, int tie, int in_dt, int out_dt, int64_t outer, int64_t red,
