@@ -240,6 +240,11 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
   if (!st) {
     Enter in(ctx);
     st = in.status;
+    // the lock was dropped for the re-layout above: the operands may have been freed meanwhile
+    if (!st) st = check_buf(ctx, l, (uint64_t)batch * M * K * dtype_size(l_dt), "dot lhs");
+    if (!st) st = check_buf(ctx, r, (uint64_t)batch * N * K * dtype_size(r_dt), "dot rhs");
+    if (!st) st = check_buf(ctx, out, (uint64_t)batch * M * N * dtype_size(out_dt), "dot out");
+    if (!st && scale_mode != HIPNX_SCALE_NONE) st = check_buf(ctx, scale, 4, "dot_scaled scale");
     if (!st) {
       const void *lp = lt ? lt->ptr : l->ptr, *rp = rt ? rt->ptr : r->ptr;
       if (pipelined) {

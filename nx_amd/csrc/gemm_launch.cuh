@@ -2,6 +2,7 @@
 // operand type keeps the build parallel).
 #pragma once
 #include "gemm_mfma.cuh"
+#include "gemm_pingpong.cuh"
 #include "internal.h"
 
 namespace hipnx {
@@ -39,10 +40,36 @@ static int launch_one(const hipnx_ctx *ctx, GemmArgs a, int64_t batch) {
   return HIPNX_OK;
 }
 
+// the two-group 256 x 256 kernel (gemm_pingpong.cuh): bf16 / f16 in every layout, s8 with a K-inner
+// left operand; its request offsets are 32 bits from the tile's first row or column
+template <int DT, bool LK, bool RK>
+static int launch_pingpong(const hipnx_ctx *ctx, GemmArgs a, int64_t batch) {
+  constexpr bool TALL = LK && !RK;  // the operand read by transposing loads gets the fewer fragments
+  constexpr int smem = 2 * 512 * SLAB;
+  auto kern = gemm_pingpong_kernel<DT, LK, RK, TALL>;
+  static bool configured = false;
+  if (!configured) {
+    HIPNX_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
+    configured = true;
+  }
+  a.tiles_m = (int)((a.M + 255) / 256);
+  a.tiles_n = (int)((a.N + 255) / 256);
+  a.group_m = gemm_group_m(a.tiles_m, a.tiles_n);
+  dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)batch), block(512);
+  hipLaunchKernelGGL(kern, grid, block, smem, ctx->stream, a);
+  HIPNX_HIP(hipGetLastError());
+  return HIPNX_OK;
+}
+
 template <int DT, bool LK, bool RK>
 static int launch_cfg(const hipnx_ctx *ctx, int cfg, const GemmArgs &a, int64_t batch) {
   switch (cfg) {
-    case GEMM_CFG_256: return launch_one<DT, 4, 2, 2, 4, LK, RK>(ctx, a, batch);
+    case GEMM_CFG_256:
+      if constexpr (DT == HIPNX_BF16 || DT == HIPNX_F16 || (DT == HIPNX_S8 && LK)) {
+        // 256 rows (or 128 k-rows) times the row pitch must fit the 32-bit request offsets
+        if (a.ld_l < (1ll << 23) && a.ld_r < (1ll << 23)) return launch_pingpong<DT, LK, RK>(ctx, a, batch);
+      }
+      return launch_one<DT, 4, 2, 2, 4, LK, RK>(ctx, a, batch);
     case GEMM_CFG_128: return launch_one<DT, 2, 2, 2, 2, LK, RK>(ctx, a, batch);
     default:
       // streaming a long weight matrix past a few rows is bound by the bytes in flight: six

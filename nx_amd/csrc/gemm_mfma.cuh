@@ -482,6 +482,22 @@ inline int gemm_group_m(int tiles_m, int tiles_n) {
   return g;
 }
 
+// Tile order: consecutive work-group ids go to different XCDs (id % 8), so each XCD takes a run of
+// total/8 consecutive positions of the order below; the order walks groups of `group_m` tile rows
+// column by column, which makes such a run a compact rectangle of tiles whose operand panels are
+// shared through the XCD's own L2.
+__device__ __forceinline__ void gemm_tile_position(const GemmArgs &a, int block, int &tm, int &tn) {
+  int tile = block;
+  const int total = a.tiles_m * a.tiles_n;
+  if (total % 8 == 0) tile = (block % 8) * (total / 8) + block / 8;
+  const int per_group = a.group_m * a.tiles_n;
+  const int first = (tile / per_group) * a.group_m;
+  const int rows = min(a.group_m, a.tiles_m - first);
+  const int in = tile % per_group;
+  tm = first + in % rows;
+  tn = in / rows;
+}
+
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {  // s_waitcnt vmcnt(N), other counters untouched
   static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
@@ -499,24 +515,8 @@ gemm_pipelined_kernel(GemmArgs a) {
   constexpr int KSTEPS = SLAB / 64;
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
-  // tile order: consecutive block ids go to different XCDs (id % 8), so each XCD takes a run of
-  // total/8 consecutive positions of the order below; the order walks groups of `group_m` tile
-  // rows column by column, which makes such a run a compact rectangle of tiles whose operand
-  // panels are shared through the XCD's own L2
-  int tile = blockIdx.x;
-  {
-    const int total = a.tiles_m * a.tiles_n;
-    if (total % 8 == 0) tile = (blockIdx.x % 8) * (total / 8) + blockIdx.x / 8;
-  }
   int tm, tn;
-  {
-    const int per_group = a.group_m * a.tiles_n;
-    const int first = (tile / per_group) * a.group_m;
-    const int rows = min(a.group_m, a.tiles_m - first);
-    const int in = tile % per_group;
-    tm = first + in % rows;
-    tn = in / rows;
-  }
+  gemm_tile_position(a, blockIdx.x, tm, tn);
   const int64_t b = blockIdx.y;
   const unsigned char *lb = a.l + b * a.bs_l;
   const unsigned char *rb = a.r + b * a.bs_r;

@@ -1,0 +1,262 @@
+// The 256 x 256 tile of the MFMA contraction as a two-group walk: the eight waves of a work-group
+// form two groups of four (one wave of each group per SIMD), and in every phase one group only
+// issues MFMAs while the other only moves data -- fragment reads out of LDS and the direct-to-LDS
+// requests of later slabs -- then they trade places at a work-group barrier.  The matrix pipe of a
+// SIMD is fed by one wave at a time from registers that are already loaded, and whatever a memory
+// instruction costs in the issue stage (a direct-to-LDS request sits there until the address unit
+// has taken it) is paid by a wave that has no MFMA to issue anyway.
+//
+// Wave tile 64 x 128 as in gemm_pipelined_kernel (4 x 8 MFMA tiles of 16 x 16, accumulators in
+// registers); K in slabs of 128 bytes per row, two LDS stages of one slab each.  A phase is one
+// K step (64 bytes of K): 12 fragment reads + 4 requests for the memory group, 32 MFMAs for the
+// other.  With p the phase number, group 0 (waves 0-3, the upper 128 rows of the tile) reads K step
+// q in phase 2q and multiplies in 2q+1; group 1 (waves 4-7, the lower rows) runs one phase behind.
+//
+// Requests (64 per slab, 16 per phase, 4 per wave and memory phase; s = slab being read):
+//   phase 4s   group 0: its share of the right operand of slab s+1
+//   phase 4s+1 group 1: its share of the right operand of slab s+1
+//   phase 4s+2 group 0: left rows 128..255 of slab s+1      (read by group 1 only: free since 4s)
+//   phase 4s+3 group 1: left rows   0..127 of slab s+2      (read by group 0 only: free since 4s+3)
+// Every request has two and a half phases to land: the wave that issued it waits for it at the end
+// of its next memory phase (vmcnt(4): everything but what it has just issued), the barrier behind
+// that wait publishes it, and the first reader comes a phase later or more.
+#pragma once
+#include "gemm_mfma.cuh"
+
+namespace hipnx {
+
+// Swizzle of the [row][k] LDS layout of this kernel: the 16-byte chunk index XOR the part of
+// lds_slot() that depends on the low four row bits only (the part that makes a fragment read of 16
+// consecutive rows conflict-free).  A fragment's address is then one per-lane base per K step plus
+// a compile-time multiple of 16 rows, which the LDS instruction carries as its immediate offset:
+// two address registers per operand instead of one per fragment.
+__device__ __forceinline__ int lds_slot16(int row, int chunk) {
+  return chunk ^ (((row ^ (row >> 2)) & 1) | ((((row >> 1) ^ (row >> 2)) & 1) << 1) | ((((row >> 2) ^ (row >> 3)) & 1) << 2));
+}
+
+// a pointer every lane of the wave holds the same value of, moved to scalar registers
+__device__ __forceinline__ const unsigned char *wave_uniform(const unsigned char *p) {
+  const uint64_t u = (uint64_t)p;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)u), hi = __builtin_amdgcn_readfirstlane((uint32_t)(u >> 32));
+  return (const unsigned char *)(((uint64_t)hi << 32) | lo);
+}
+
+// direct-to-LDS load with a wave-uniform 64-bit base and a 32-bit byte offset per lane
+__device__ __forceinline__ void lds_dma16_at(const unsigned char *base, unsigned off, unsigned char *lds) {
+  const unsigned dst = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(lptr_t)lds);
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(dst) : "memory", "m0");
+#pragma clang diagnostic pop
+}
+
+// K-inner rows [row0, row0 + ROWS) of an operand, ROWS x 128 B per slab, shared by NWAVES waves:
+// PER instructions per wave, each filling 1 KiB of LDS (8 rows x 8 chunks).  Offsets are relative
+// to the operand's first tile row (clamped into the matrix), so they fit 32 bits whenever
+// 2 * ROWS * ld does (the host checks).
+template <int ROWS, int NWAVES>
+struct PPKInnerLoader {
+  static constexpr int PER = ROWS / 8 / NWAVES;
+  const unsigned char *base;
+  unsigned off[PER];
+  __device__ __forceinline__ void init(const unsigned char *g, int64_t ld, int64_t row0, int64_t rows_valid, int wave, int lane) {
+    const int64_t first = row0 < rows_valid ? row0 : rows_valid - 1;
+    base = wave_uniform(g + first * ld);
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+      const int r = (wave + NWAVES * i) * 8 + (lane >> 3);
+      int64_t gr = row0 + r;
+      gr = gr < rows_valid ? gr : rows_valid - 1;
+      off[i] = (unsigned)((gr - first) * ld) + lds_slot16(r, lane & 7) * 16;
+    }
+  }
+  __device__ __forceinline__ void issue(int64_t kbyte0, unsigned char *lds, int wave) const {
+    const unsigned char *b = base + kbyte0;
+#pragma unroll
+    for (int i = 0; i < PER; i++) lds_dma16_at(b, off[i], lds + (wave + NWAVES * i) * 1024);
+  }
+};
+
+// K-outer columns [col0, col0 + ROWS) of an operand copied k-major ([k][ROWS * ES bytes]) for the
+// transposing fragment reads (tr_slot layout of gemm_mfma.cuh), with 32-bit offsets from the tile's
+// first column (clamped).
+template <int ES, int ROWS, int NWAVES>
+struct PPKOuterLoader {
+  static constexpr int RBYTES = ROWS * ES;
+  static constexpr int PER = ROWS / 8 / NWAVES;
+  static_assert(RBYTES >= 256, "a k-row must span all LDS banks");
+  const unsigned char *base;
+  unsigned off[PER];
+  __device__ __forceinline__ void init(const unsigned char *g, int64_t ld, int64_t col0, int64_t cols_valid, int wave, int lane) {
+    const int64_t last = cols_valid * ES - 16;
+    const int64_t first = col0 * ES <= last ? col0 * ES : last;
+    base = wave_uniform(g + first);
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+      const int o = (wave + NWAVES * i) * 1024 + lane * 16;
+      const int k = o / RBYTES, slot = (o % RBYTES) / 16;
+      int64_t byte = col0 * ES + tr_slot<ES>(k, slot) * 16;
+      byte = byte <= last ? byte : last;
+      off[i] = (unsigned)((int64_t)k * ld + (byte - first));
+    }
+  }
+  __device__ __forceinline__ void issue(int64_t k0, int64_t ld, unsigned char *lds, int wave) const {
+    const unsigned char *b = base + k0 * ld;
+#pragma unroll
+    for (int i = 0; i < PER; i++) lds_dma16_at(b, off[i], lds + (wave + NWAVES * i) * 1024);
+  }
+};
+
+// TALL = false: wave tile 64 x 128 (waves 4 x 2); TALL = true: 128 x 64 (waves 2 x 4).  Either way
+// waves 0-3 own the upper 128 rows.  A transposing fragment read moves 8 bytes per lane, a plain one
+// 16, so the operand that needs the transposing reads should be the one with fewer fragments per
+// wave: a K-outer right operand wants TALL, a K-outer left operand the other shape.
+template <int DT, bool L_KIN, bool R_KIN, bool TALL = false, bool PRIO = true>
+__global__ void __launch_bounds__(512)
+gemm_pingpong_kernel(GemmArgs a) {
+  typedef typename Mma16<DT>::acc_t acc_t;
+  constexpr int NW = 8, TM16 = TALL ? 8 : 4, TN16 = TALL ? 4 : 8, BM = 256, BN = 256, HALF = 128;
+  constexpr int STAGE = (BM + BN) * SLAB;
+  constexpr int ES = (DT == HIPNX_S8) ? 1 : 2;
+  static_assert(DT == HIPNX_BF16 || DT == HIPNX_F16 || DT == HIPNX_S8, "2-byte and 1-byte MFMA types");
+  static_assert(L_KIN || ES == 2, "a K-outer left operand is split into two 128-row halves: 2-byte types only");
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+
+  int tm, tn;
+  gemm_tile_position(a, blockIdx.x, tm, tn);
+  const int64_t b = blockIdx.y;
+  const unsigned char *lb = a.l + b * a.bs_l;
+  const unsigned char *rb = a.r + b * a.bs_r;
+  const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int grp = wave >> 2;                     // waves w and w + 4 share a SIMD
+  const int wm = TALL ? (wave >> 2) * 128 : (wave >> 1) * 64;  // group 0: rows 0..127, group 1: 128..255
+  const int wn = TALL ? (wave & 3) * 64 : (wave & 1) * 128;
+
+  acc_t acc[TM16][TN16];
+#pragma unroll
+  for (int i = 0; i < TM16; i++)
+#pragma unroll
+    for (int j = 0; j < TN16; j++)
+#pragma unroll
+      for (int q = 0; q < 4; q++) acc[i][j][q] = 0;
+
+  // right operand: the eight waves share its 32 instructions per slab (any split will do)
+  PPKInnerLoader<BN, NW> rload;
+  PPKOuterLoader<ES, BN, NW> rtr;
+  if constexpr (R_KIN) rload.init(rb, a.ld_r, n0, a.N, wave, lane);
+  else rtr.init(rb, a.ld_r, n0, a.N, wave, lane);
+  // left operand: a group requests the half the OTHER group reads (it is the half that is free in
+  // the group's own memory phase): group 0 rows 128..255, group 1 rows 0..127
+  const int lhalf = grp ^ 1;
+  constexpr int TR_ES = 2;
+  PPKInnerLoader<HALF, 4> lload;
+  PPKOuterLoader<TR_ES, HALF, 4> ltr;
+  if constexpr (L_KIN) lload.init(lb, a.ld_l, m0 + lhalf * HALF, a.M, wave & 3, lane);
+  else ltr.init(lb, a.ld_l, m0 + lhalf * HALF, a.M, wave & 3, lane);
+
+  auto issue_r = [&](int stage, int64_t kbyte0) {
+    unsigned char *sB = smem + stage * STAGE + BM * SLAB;
+    if constexpr (R_KIN) rload.issue(kbyte0, sB, wave);
+    else rtr.issue(kbyte0 / ES, a.ld_r, sB, wave);
+  };
+  auto issue_l = [&](int stage, int64_t kbyte0) {  // a half is HALF rows x 128 bytes in either layout
+    unsigned char *sA = smem + stage * STAGE + lhalf * (HALF * SLAB);
+    if constexpr (L_KIN) lload.issue(kbyte0, sA, wave & 3);
+    else ltr.issue(kbyte0 / ES, a.ld_l, sA, wave & 3);
+  };
+
+  // fragment addresses within a stage: one per-lane base per operand and K step; the tile index
+  // (16 rows = 2 KiB apart in the [row][k] layout) is a compile-time offset
+  int a_rd[2], b_rd[2];
+  if constexpr (L_KIN) {
+    const int row = wm + (lane & 15);
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) a_rd[ks] = row * SLAB + lds_slot16(row, 4 * ks + (lane >> 4)) * 16;
+  }
+  if constexpr (R_KIN) {
+    const int row = wn + (lane & 15);
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) b_rd[ks] = BM * SLAB + row * SLAB + lds_slot16(row, 4 * ks + (lane >> 4)) * 16;
+  }
+  auto read_l = [&](const unsigned char *st, int ks, int i) -> v4i {
+    if constexpr (L_KIN) return *reinterpret_cast<const v4i *>(st + a_rd[ks] + i * (16 * SLAB));
+    else return read_fragment_tr<TR_ES, HALF>(st + grp * (HALF * SLAB), (wm & (HALF - 1)) + 16 * i, ks, lane);  // two k-major halves
+  };
+  auto read_r = [&](const unsigned char *st, int ks, int j) -> v4i {
+    if constexpr (R_KIN) return *reinterpret_cast<const v4i *>(st + b_rd[ks] + j * (16 * SLAB));
+    else return read_fragment_tr<ES, BN>(st + BM * SLAB, wn + 16 * j, ks, lane);
+  };
+
+  const int nslab = (int)(a.Kb / SLAB);
+  // prologue: slabs 0 and 1 into the two stages; slab 0 must have landed before the first phase
+  issue_r(0, 0);
+  issue_l(0, 0);
+  if (nslab > 1) {
+    issue_r(1, SLAB);
+    issue_l(1, SLAB);
+    wait_vmcnt<8>();
+  } else {
+    wait_vmcnt<0>();
+  }
+  __builtin_amdgcn_s_barrier();
+  if (grp) __builtin_amdgcn_s_barrier();  // group 1 runs one phase behind
+
+  v4i fa[TM16], fb[TN16];
+  for (int s = 0; s < nslab; s++) {
+    const unsigned char *cur = smem + (s & 1) * STAGE;
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) {
+      // ---- memory phase: fragments of K step ks, then this phase's requests
+#pragma unroll
+      for (int i = 0; i < TM16; i++) fa[i] = read_l(cur, ks, i);
+#pragma unroll
+      for (int j = 0; j < TN16; j++) fb[j] = read_r(cur, ks, j);
+      bool issued = false;
+      if (ks == 0) {
+        if (s >= 1 && s + 1 < nslab) {
+          issue_r((s + 1) & 1, (int64_t)(s + 1) * SLAB);
+          issued = true;
+        }
+      } else if (grp == 0) {
+        if (s >= 1 && s + 1 < nslab) {
+          issue_l((s + 1) & 1, (int64_t)(s + 1) * SLAB);
+          issued = true;
+        }
+      } else if (s + 2 < nslab) {
+        issue_l(s & 1, (int64_t)(s + 2) * SLAB);
+        issued = true;
+      }
+      // what I requested a memory phase ago (or in the prologue) has to be in LDS before the barrier
+      // that publishes it; in the very first phase nothing is due yet (slab 1 is first read in phase 4)
+      if (issued) wait_vmcnt<4>();
+      else if (!(s == 0 && ks == 0)) wait_vmcnt<0>();
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): my fragments are in registers
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      // ---- compute phase: 32 MFMAs from registers
+      if constexpr (PRIO) __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+      for (int j = 0; j < TN16; j++)
+#pragma unroll
+        for (int i = 0; i < TM16; i++) Mma16<DT>::step(acc[i][j], fb[j], fa[i]);
+      if constexpr (PRIO) __builtin_amdgcn_s_setprio(0);
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  if (!grp) __builtin_amdgcn_s_barrier();  // group 0 finishes one phase ahead
+
+  const int64_t obase = b * a.M * a.N;
+  switch (a.odt) {
+#define HIPNX_EPI(T) case T: gemm_epilogue<DT, T, TM16, TN16>(acc, a.out, obase, a.M, a.N, m0 + wm, n0 + wn, lane, a.scale, a.scale_mode); break;
+    HIPNX_EPI(HIPNX_BF16) HIPNX_EPI(HIPNX_F16) HIPNX_EPI(HIPNX_F32) HIPNX_EPI(HIPNX_F64)
+    HIPNX_EPI(HIPNX_S8) HIPNX_EPI(HIPNX_U8) HIPNX_EPI(HIPNX_S16) HIPNX_EPI(HIPNX_U16)
+    HIPNX_EPI(HIPNX_S32) HIPNX_EPI(HIPNX_U32) HIPNX_EPI(HIPNX_S64) HIPNX_EPI(HIPNX_U64)
+#undef HIPNX_EPI
+  }
+}
+
+}  // namespace hipnx
