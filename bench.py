@@ -27,18 +27,59 @@ sys.path.insert(0, ROOT)
 PEAK_HBM_GBS = 8000.0
 PEAK = {"bf16": 2500.0, "f16": 2500.0, "s8": 5000.0, "f32": 157.3}  # dense MFMA TFLOP/s (TOP/s)
 
-# HBM bytes per launch of the headline dot kernel, from two counter runs of this file
-# (`rocprofv3 --pmc FETCH_SIZE`, then `--pmc WRITE_SIZE`, with --calibrate): KiB per dispatch of the
-# gemm kernel, each scaled by what the same counter read for the 1 GiB + 1 GiB calibration kernel.
-# The figures and the commands are in profiles/dot_bf16_4096_hbm_traffic.md.
-HEADLINE_TRAFFIC_BYTES = 235345715  # 98467 KiB x 2.0 fetched + 32895 KiB x 1.0 written; algorithmic 100663296
+# HBM bytes per launch of the headline dot kernel come from two counter runs of this file
+# (`rocprofv3 --pmc FETCH_SIZE`, then `--pmc WRITE_SIZE`, with --calibrate); the summary of those runs
+# carries the figure in a line `TRAFFIC_BYTES_PER_LAUNCH = <n>`, which is what is reported here.
+TRAFFIC_PROFILE = os.path.join("profiles", "dot_bf16_4096_hbm_traffic.md")
+CEILINGS_BIN = os.path.join(ROOT, "nx_amd", "lib", "hipnx_ceilings")
+
+
+def headline_traffic():
+    """(bytes per launch, source) from the committed counter summary; (None, reason) without it."""
+    try:
+        with open(os.path.join(ROOT, TRAFFIC_PROFILE)) as f:
+            for line in f:
+                if line.startswith("TRAFFIC_BYTES_PER_LAUNCH"):
+                    return int(line.split("=")[1].split()[0]), TRAFFIC_PROFILE
+    except OSError:
+        pass
+    return None, "no counter summary found"
+
+
+def measured_ceilings(ms=250):
+    """What this part sustains: MFMA-only loops (the kernel's own MFMA forms, operands drawn like the
+    benchmark's) and streaming kernels, each run by the stand-alone program for `ms` milliseconds."""
+    import subprocess
+    out = {}
+    if not os.path.exists(CEILINGS_BIN):
+        return out
+    runs = [("mfma_bf16", ["mfma", "bf16", "normal", str(ms)]), ("mfma_f16", ["mfma", "f16", "normal", str(ms)]),
+            ("mfma_s8", ["mfma", "s8", "normal", str(ms)]), ("mfma_f32", ["mfma", "f32", "normal", str(ms)]),
+            ("stream_read", ["stream", "read", "2048", "100"]), ("stream_write", ["stream", "write", "2048", "100"]),
+            ("stream_copy", ["stream", "copy", "2048", "100"])]
+    for name, argv in runs:
+        try:
+            res = subprocess.run([CEILINGS_BIN] + argv, capture_output=True, text=True, timeout=120)
+            line = json.loads(res.stdout.strip().splitlines()[-1])
+            line["command"] = "nx_amd/lib/hipnx_ceilings " + " ".join(argv)
+            out[name] = line
+        except Exception as exc:  # an extra: the published peaks stay the denominators of `frac`
+            out[name] = {"error": str(exc)[:200]}
+    return out
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=100)
-    ap.add_argument("--warmup", type=int, default=30)  # the clocks settle over the first tens of launches
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=30)
+    # The clock this part runs a kernel at settles over tens of milliseconds of the same load (a 4096^3
+    # dot starts near 112 us, drops to 130-140 us after 2 ms and recovers to ~100 us within 50 ms), so a
+    # short run measures the power controller's transient.  Before the warm-up steps of the headline the
+    # same call is therefore repeated untimed for this long; `cold_start` in the output is the figure
+    # without it.
+    ap.add_argument("--settle-ms", type=float, default=400.0)
+    ap.add_argument("--no-ceilings", action="store_true")
     ap.add_argument("--no-suite", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--calibrate", action="store_true")
@@ -74,6 +115,31 @@ def main():
         wall_ms = (time.perf_counter() - t0) * 1e3
         return wall_ms / steps, dev_ms / steps
 
+    def laps(fn, steps, warmup):
+        """Device ms per step from lap marks on the launch stream: (mean, median, min).  A mark costs a few
+        microseconds on the stream, so one is recorded per chunk of steps (at most 20 chunks) and the
+        median and the minimum are those of the chunks' per-step means."""
+        chunk = max(1, steps // 20)
+        chunks = max(1, steps // chunk)
+        for _ in range(warmup):
+            keep = fn()
+        B.timer_mark(0)
+        for c in range(chunks):
+            for _ in range(chunk):
+                keep = fn()  # noqa: F841
+            B.timer_mark(c + 1)
+        per = sorted(B.timer_between(c, c + 1) / chunk for c in range(chunks))
+        return B.timer_between(0, chunks) / (chunks * chunk), per[len(per) // 2], per[0]
+
+    def settle(fn, ms):
+        t0 = time.perf_counter()
+        while (time.perf_counter() - t0) * 1e3 < ms:
+            for _ in range(50):
+                keep = fn()  # noqa: F841
+            B.sync()
+
+    ceilings = {} if args.no_ceilings else measured_ceilings()
+
     if args.calibrate:
         big = put(np.ones((16384, 16384), dtype=np.float32), "f32")
         for _ in range(5):
@@ -86,9 +152,13 @@ def main():
     a_np, b_np = W.dense_gemm_bf16(n=n)
     a, b = put(a_np, "bf16"), put(b_np, "bf16")
     flop = 2.0 * n * n * n
+    _, cold_ms = timed(lambda: Nx.dot(a, b), 20, 5)  # an idle part's first 25 launches
+    settle(lambda: Nx.dot(a, b), args.settle_ms)
     wall_ms, dev_ms = timed(lambda: Nx.dot(a, b), args.steps, args.warmup)
     value = flop / (wall_ms * 1e-3) / 1e12
     achieved = flop / (dev_ms * 1e-3) / 1e12
+    lap_mean, lap_median, lap_min = laps(lambda: Nx.dot(a, b), args.steps, 0)
+    traffic, traffic_source = headline_traffic()
 
     result = {
         "metric": "Nx.dot TFLOP/s (bf16, s8->s32) + elementwise/reduce GB/s, % of MI355X peak",
@@ -98,9 +168,21 @@ def main():
         "config": {"workload": "dense GEMM: Nx.dot bf16 {4096,4096} x {4096,4096}, f32 accumulate, bf16 output "
                                "(BASELINE configs[1])", "seed": 2},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK["bf16"], "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK["bf16"], 4), "traffic": HEADLINE_TRAFFIC_BYTES,
-                     "kernel": "dot callback (gemm kernel + operand re-layout, if any), HIP events on the launch stream"},
+                     "frac": round(achieved / PEAK["bf16"], 4), "traffic": traffic, "traffic_source": traffic_source,
+                     "kernel": "dot callback (gemm kernel + operand re-layout, if any), HIP events on the launch stream",
+                     "per_step_us": {"mean": round(dev_ms * 1e3, 2), "median": round(lap_median * 1e3, 2),
+                                     "min": round(lap_min * 1e3, 2),
+                                     "note": "median / min over 20 chunks of a second pass of K steps (one lap mark per chunk)"}},
+        "settle_ms": args.settle_ms,
+        "cold_start": {"tflops": round(flop / (cold_ms * 1e-3) / 1e12, 1), "steps": 20, "warmup": 5,
+                       "note": "the same call on the idle part, before the settling phase"},
     }
+    if "sustained" in ceilings.get("mfma_bf16", {}):
+        top = ceilings["mfma_bf16"]["sustained"]
+        result["roofline"]["measured_ceiling"] = {"value": top, "unit": "TFLOP/s", "frac_of_ceiling": round(achieved / top, 4),
+                                                  "source": ceilings["mfma_bf16"]["command"]}
+    if ceilings:
+        result["ceilings"] = ceilings
 
     # ---- the other configurations -----------------------------------------------------------
     # Entries are timed "cache-hot" (the same operands every step).  Where the operands are smaller
@@ -121,94 +203,145 @@ def main():
                 return ring[state[0]]
             return nxt
 
-        def entry(name, work, unit, ms, peak, bound):
-            rate = work / (ms * 1e-3) / (1e12 if unit == "TFLOP/s" or unit == "TOP/s" else 1e9)
-            suite[name] = {"ms": round(ms, 5), "achieved": round(rate, 2), "unit": unit, "bound": bound,
-                           "peak": peak, "frac": round(rate / peak, 4)}
+        class Ms(float):
+            """Mean device ms per step, carrying the median and the minimum of the per-step times."""
+
+        def tstat(fn, steps, warmup, settle_ms=0.0):
+            if settle_ms:
+                settle(fn, settle_ms)
+            mean, median, least = laps(fn, steps, warmup)
+            ms = Ms(mean)
+            ms.median, ms.least = median, least
+            return None, ms
+
+        def entry(name, work, unit, ms, peak, bound, ceil=None, vs=None):
+            """`work` = the entry's own algorithmic bytes or flop per step; `ceil` names the measured ceiling
+            it is also compared with; `vs` = (label, ms of the formulation it replaces)."""
+            scale = 1e12 if unit in ("TFLOP/s", "TOP/s") else 1e9
+            rate = work / (ms * 1e-3) / scale
+            e = {"ms": round(ms, 5), "ms_median": round(ms.median, 5), "ms_min": round(ms.least, 5),
+                 "achieved": round(rate, 2), "unit": unit, "bound": bound, "peak": peak, "frac": round(rate / peak, 4)}
+            if ceil is None and bound == "hbm":
+                ceil = "stream_copy"
+            top = ceilings.get(ceil, {}).get("sustained") if ceil else None
+            if top:
+                e["measured_ceiling"] = {"value": top, "source": ceilings[ceil]["command"], "frac_of_ceiling": round(rate / top, 4)}
+            if vs:
+                e["vs_" + vs[0]] = round(vs[1] / ms, 2)
+            suite[name] = e
 
         # K-inner operands: the gemm kernel alone (no re-layout pass)
         bt = Nx.transpose(b)
-        _, ms = timed(lambda: Nx.dot(a, [1], bt, [1]), steps, warm)
-        entry("dot_bf16_4096_kinner", flop, "TFLOP/s", ms, PEAK["bf16"], "mfma")
+        msettle = min(args.settle_ms, 150.0)
+        _, ms = tstat(lambda: Nx.dot(a, [1], bt, [1]), steps, warm, msettle)
+        entry("dot_bf16_4096_kinner", flop, "TFLOP/s", ms, PEAK["bf16"], "mfma", "mfma_bf16")
         nxt = rotating(lambda: (put(a_np, "bf16"), put(b_np, "bf16")), 2 * n * n * 2)
 
         def dot_rot():
             x, y = nxt()
             return Nx.dot(x, y)
-        _, ms = timed(dot_rot, steps, warm)
-        entry("dot_bf16_4096_rotated", flop, "TFLOP/s", ms, PEAK["bf16"], "mfma")
+        _, ms = tstat(dot_rot, steps, warm, msettle)
+        entry("dot_bf16_4096_rotated", flop, "TFLOP/s", ms, PEAK["bf16"], "mfma", "mfma_bf16")
         del nxt
         fa, fb = W.dense_gemm_f32()
         fa, fb = put(fa, "f32"), put(fb, "f32")
-        _, ms = timed(lambda: Nx.dot(fa, fb), steps, warm)
-        entry("dot_f32_2048", 2.0 * 2048 ** 3, "TFLOP/s", ms, PEAK["f32"], "mfma")
+        _, ms = tstat(lambda: Nx.dot(fa, fb), steps, warm, msettle)
+        entry("dot_f32_2048", 2.0 * 2048 ** 3, "TFLOP/s", ms, PEAK["f32"], "mfma", "mfma_f32")
         sa, sb = W.dense_gemm_s8()
         sa, sb = put(sa, "s8"), put(sb, "s8")
-        _, ms = timed(lambda: Nx.dot(sa, sb, out_type="s32"), steps, warm)
-        entry("dot_s8_4096_s32", flop, "TOP/s", ms, PEAK["s8"], "mfma")
-        del fa, fb, sa, sb, bt
+        _, ms = tstat(lambda: Nx.dot(sa, sb, out_type="s32"), steps, warm, msettle)
+        entry("dot_s8_4096_s32", flop, "TOP/s", ms, PEAK["s8"], "mfma", "mfma_s8")
+        sbt = Nx.transpose(sb)
+        _, ms = tstat(lambda: Nx.dot(sa, [1], sbt, [1], out_type="s32"), steps, warm, msettle)
+        entry("dot_s8_4096_s32_kinner", flop, "TOP/s", ms, PEAK["s8"], "mfma", "mfma_s8")
+        ha, hb = put(W.bf16_to_f32(a_np).astype(np.float16), "f16"), put(W.bf16_to_f32(b_np).astype(np.float16), "f16")
+        _, ms = tstat(lambda: Nx.dot(ha, hb), steps, warm, msettle)
+        entry("dot_f16_4096", flop, "TFLOP/s", ms, PEAK["f16"], "mfma", "mfma_f16")
+        del fa, fb, sa, sb, bt, sbt, ha, hb
 
         # config 1 (and a HBM-resident scale of it)
         for nn in (1024, 16384):
             x, y = W.elementwise_reduce(n=nn)
             x, y = put(x, "f32"), put(y, "f32")
             N = nn * nn
-            _, ms = timed(lambda: Nx.add(x, y), steps, warm)
+            _, ms = tstat(lambda: Nx.add(x, y), steps, warm)
             entry(f"add_f32_{nn}", 12.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-            _, ms = timed(lambda: Nx.multiply(x, 0.5), steps, warm)
+            _, ms = tstat(lambda: Nx.multiply(x, 0.5), steps, warm)
             entry(f"multiply_scalar_f32_{nn}", 8.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-            _, ms = timed(lambda: Nx.exp(x), steps, warm)
+            _, ms = tstat(lambda: Nx.exp(x), steps, warm)
             entry(f"exp_f32_{nn}", 8.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-            _, ms = timed(lambda: Nx.sum(x, axes=[1]), steps, warm)
-            entry(f"sum_rows_f32_{nn}", 4.0 * N + 4.0 * nn, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+            _, ms = tstat(lambda: Nx.sum(x, axes=[1]), steps, warm)
+            entry(f"sum_rows_f32_{nn}", 4.0 * N + 4.0 * nn, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read")
             # the whole unfused chain of config 1: add -> multiply 0.5 -> exp -> sum over axis 1
-            _, ms = timed(lambda: Nx.sum(Nx.exp(Nx.multiply(Nx.add(x, y), 0.5)), axes=[1]), steps, warm)
+            _, ms = tstat(lambda: Nx.sum(Nx.exp(Nx.multiply(Nx.add(x, y), 0.5)), axes=[1]), steps, warm)
             entry(f"config1_chain_f32_{nn}", 32.0 * N + 4.0 * nn, "GB/s", ms, PEAK_HBM_GBS, "hbm")
             del x, y
 
         # config 3: attention scores + softmax chain
         q, k = W.attention_scores()
         q, k = put(q, "bf16"), put(k, "bf16")
-        _, ms = timed(lambda: Nx.dot(q, [2], [0], k, [2], [0]), steps, warm)
-        entry("dot_qk_bf16_32x512x64", 20971520.0, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+        _, ms = tstat(lambda: Nx.dot(q, [2], [0], k, [2], [0]), steps, warm)
+        entry("dot_qk_bf16_32x512x64", 20971520.0, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_write")
+        q_np, k_np = W.attention_scores()
+        nxt = rotating(lambda: (put(q_np, "bf16"), put(k_np, "bf16")), q_np.nbytes + k_np.nbytes)
+
+        def qk_rot():
+            qq, kk = nxt()
+            return Nx.dot(qq, [2], [0], kk, [2], [0])
+        _, ms = tstat(qk_rot, steps, warm)
+        entry("dot_qk_bf16_32x512x64_rotated", 20971520.0, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_write")
+        del nxt
         s = Nx.dot(q, [2], [0], k, [2], [0])
 
         def softmax():
             z = Nx.multiply(Nx.as_type(s, "f32"), 0.125)
             e = Nx.exp(Nx.subtract(z, Nx.reduce_max(z, axes=[2], keep_axes=True)))
             return Nx.divide(e, Nx.sum(e, axes=[2], keep_axes=True))
-        _, ms = timed(softmax, steps, warm)
+        _, ms = tstat(softmax, steps, warm)
         entry("softmax_chain_32x512x512", 386138112.0, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-        del q, k, s
+        nxt = rotating(lambda: Nx.dot(q, [2], [0], k, [2], [0]), 32 * 512 * 512 * 2)
+
+        def softmax_rot():
+            z = Nx.multiply(Nx.as_type(nxt(), "f32"), 0.125)
+            e = Nx.exp(Nx.subtract(z, Nx.reduce_max(z, axes=[2], keep_axes=True)))
+            return Nx.divide(e, Nx.sum(e, axes=[2], keep_axes=True))
+        _, ms = tstat(softmax_rot, steps, warm)
+        entry("softmax_chain_32x512x512_rotated", 386138112.0, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+        del q, k, s, nxt
 
         # config 4: int8 weight-only linear
         w, xq, sc = W.int8_linear()
         w, xq, sc = put(w, "s8"), put(xq, "s8"), put(sc, "f32")
-        _, ms = timed(lambda: Nx.dot(xq, [1], w, [1], out_type="s32"), steps, warm)
-        entry("dot_s8_w8_64x11008x4096", 48168960.0, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+        _, ms = tstat(lambda: Nx.dot(xq, [1], w, [1], out_type="s32"), steps, warm)
+        entry("dot_s8_w8_64x11008x4096", 48168960.0, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read")
         suite["dot_s8_w8_64x11008x4096"]["tops"] = round(5771362304.0 / (ms * 1e-3) / 1e12, 2)
         w_np = W.int8_linear()[0]
         nxt = rotating(lambda: put(w_np, "s8"), w_np.nbytes)
-        _, ms = timed(lambda: Nx.dot(xq, [1], nxt(), [1], out_type="s32"), steps, warm)
-        entry("dot_s8_w8_64x11008x4096_rotated", 48168960.0, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+        _, ms = tstat(lambda: Nx.dot(xq, [1], nxt(), [1], out_type="s32"), steps, warm)
+        entry("dot_s8_w8_64x11008x4096_rotated", 48168960.0, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read")
         # the whole config: dot -> as_type f32 -> multiply by the per-column scales
-        _, ms = timed(lambda: Nx.multiply(Nx.as_type(Nx.dot(xq, [1], nxt(), [1], out_type="s32"), "f32"), sc), steps, warm)
+        _, ms = tstat(lambda: Nx.multiply(Nx.as_type(Nx.dot(xq, [1], nxt(), [1], out_type="s32"), "f32"), sc), steps, warm)
         entry("config4_chain_rotated", 48168960.0 + 5636096.0 + 5680128.0, "GB/s", ms, PEAK_HBM_GBS, "hbm")
         del w, xq, sc, nxt
 
         # config 5: argmax + take
         logits, table, _ = W.logits_and_table()
         logits, table = put(logits, "f32"), put(table, "bf16")
-        _, ms = timed(lambda: Nx.argmax(logits, axis=1, type="u32"), steps, warm)
-        entry("argmax_f32_8192x32000", 1048608768.0, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+        _, ms = tstat(lambda: Nx.argmax(logits, axis=1, type="u32"), steps, warm)
+        entry("argmax_f32_8192x32000", 1048608768.0, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read")
         idx = Nx.argmax(logits, axis=1, type="u32")
-        _, ms = timed(lambda: Nx.take(table, idx), steps, warm)
+        _, ms = tstat(lambda: Nx.take(table, idx), steps, warm)
         entry("take_bf16_8192_of_32000x4096", 134250496.0, "GB/s", ms, PEAK_HBM_GBS, "hbm")
         suite["take_bf16_8192_of_32000x4096"]["note"] = (
             "per call, not per kernel: with the reference's raising bounds policy every take waits for its "
             "kernel before returning (an out-of-range index must raise from this call), so launch and wait "
             "latencies are inside; the kernel itself runs ~22 us = ~6.1 TB/s (rocprofv3 kernel trace)")
-        del logits, table, idx
+        # other rows every step (eight index sets, 537 MB of table rows in all): nothing comes from the cache
+        rng = np.random.default_rng(5)
+        nxt = rotating(lambda: put(rng.integers(0, 32000, size=8192, dtype=np.uint32), "u32"), 40e6)
+        _, ms = tstat(lambda: Nx.take(table, nxt()), steps, warm)
+        entry("take_bf16_8192_of_32000x4096_rotated", 134250496.0, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+        del logits, table, idx, nxt
 
         # selection, windows and creation at the HBM-resident size of config 1
         nn = 16384
@@ -216,19 +349,19 @@ def main():
         x, y = W.elementwise_reduce(n=nn)
         x, y = put(x, "f32"), put(y, "f32")
         pred = Nx.greater(x, y)
-        _, ms = timed(lambda: Nx.select(pred, x, y), steps, warm)
+        _, ms = tstat(lambda: Nx.select(pred, x, y), steps, warm)
         entry(f"select_f32_{nn}", 13.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-        _, ms = timed(lambda: Nx.clip(x, -0.5, 0.5), steps, warm)
+        _, ms = tstat(lambda: Nx.clip(x, -0.5, 0.5), steps, warm)
         entry(f"clip_f32_{nn}", 8.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-        _, ms = timed(lambda: Nx.slice(x, [64, 128], [nn - 128, nn - 256]), steps, warm)
+        _, ms = tstat(lambda: Nx.slice(x, [64, 128], [nn - 128, nn - 256]), steps, warm)
         entry(f"slice_f32_{nn}", 8.0 * (nn - 128) * (nn - 256), "GB/s", ms, PEAK_HBM_GBS, "hbm")
         del pred
-        _, ms = timed(lambda: Nx.concatenate([x, y], axis=1), steps, warm)
+        _, ms = tstat(lambda: Nx.concatenate([x, y], axis=1), steps, warm)
         entry(f"concatenate_axis1_f32_{nn}", 16.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-        _, ms = timed(lambda: Nx.all(x, axes=[1]), steps, warm)
-        entry(f"all_rows_f32_{nn}", 4.0 * N + nn, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-        _, ms = timed(lambda: Nx.iota((nn, nn), type="f32", axis=1, backend=H), steps, warm)
-        entry(f"iota_f32_{nn}", 4.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+        _, ms = tstat(lambda: Nx.all(x, axes=[1]), steps, warm)
+        entry(f"all_rows_f32_{nn}", 4.0 * N + nn, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read")
+        _, ms = tstat(lambda: Nx.iota((nn, nn), type="f32", axis=1, backend=H), steps, warm)
+        entry(f"iota_f32_{nn}", 4.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_write")
         del x, y
 
         # Nx.Random on the device: 2^28 u32 words from one key (counter-based, write-only), and
@@ -236,18 +369,19 @@ def main():
         from nx_amd import random as Random
         key = Random.key(1701, backend=H)
         nw = 1 << 28
-        _, ms = timed(lambda: Random.random_bits(key, shape=(nw,)), steps, warm)
-        entry("random_bits_u32_2p28", 4.0 * nw, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-        _, ms = timed(lambda: Random.uniform_split(key, 0.0, 1.0, shape=(nw,)), steps, warm)
+        _, ms = tstat(lambda: Random.random_bits(key, shape=(nw,)), steps, warm)
+        entry("random_bits_u32_2p28", 4.0 * nw, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_write")
+        _, ms = tstat(lambda: Random.uniform_split(key, 0.0, 1.0, shape=(nw,)), steps, warm)
+        unfused_ms = float(ms)
         # bits out; shift, or, subtract, multiply, add, max each read and write the array once
         entry("uniform_f32_2p28_unfused", 4.0 * nw * 13, "GB/s", ms, PEAK_HBM_GBS, "hbm")
         # the same function traced, its bits-to-floats chain (shift, or, bitcast, subtract, ..., max) planned as
         # one group compiled for the device: the cipher writes the words, one more pass reads them and writes floats
         from nx_amd import defn as _defn
         uniform = _defn.compile(lambda k: Random.uniform_split(k, 0.0, 1.0, shape=(nw,)), key, fuse="compiled")
-        _, ms = timed(lambda: uniform(key), steps, warm)
-        entry("uniform_f32_2p28_fused_compiled", 4.0 * nw * 13, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-        entry("uniform_f32_2p28_fused_compiled_two_passes", 4.0 * nw * 3, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+        _, ms = tstat(lambda: uniform(key), steps, warm)
+        # priced at what it moves: the words written, then read once and the floats written
+        entry("uniform_f32_2p28_fused_compiled", 4.0 * nw * 3, "GB/s", ms, PEAK_HBM_GBS, "hbm", vs=("unfused", unfused_ms))
         del key, uniform
 
         # traced chains: one callback per node (the evaluator), and the same chain captured once and
@@ -269,44 +403,47 @@ def main():
         q, k = W.attention_scores()
         w, xq, sc = W.int8_linear()
         q, k = put(q, "bf16"), put(k, "bf16")
-        cases = {"config1_chain_f32_1024": (chain1, (put(x, "f32"), put(y, "f32")), 32.0 * 1024 * 1024 + 4096.0),
-                 "softmax_chain_32x512x512": (chain3, (Nx.dot(q, [2], [0], k, [2], [0]),), 386138112.0),
-                 "config4_chain": (chain4, (put(xq, "s8"), put(w, "s8"), put(sc, "f32")), 48168960.0 + 5636096.0 + 5680128.0)}
-        for name, (fun, targs, nbytes) in cases.items():
+        n1, ns = 1024 * 1024, 32 * 512 * 512
+        # name -> (function, arguments, bytes node by node, bytes as fused groups, bytes planned as one kernel)
+        cases = {"config1_chain_f32_1024": (chain1, (put(x, "f32"), put(y, "f32")), 32.0 * n1 + 4096.0, 8.0 * n1 + 4096.0, 8.0 * n1 + 4096.0),
+                 "softmax_chain_32x512x512": (chain3, (Nx.dot(q, [2], [0], k, [2], [0]),), 386138112.0, 10.0 * ns + 8.0 * 16384, 6.0 * ns),
+                 "config4_chain": (chain4, (put(xq, "s8"), put(w, "s8"), put(sc, "f32")), 48168960.0 + 5636096.0 + 5680128.0, 48212992.0, 48212992.0)}
+        for name, (fun, targs, nbytes, fbytes, pbytes) in cases.items():
             compiled = defn.compile(fun, *targs)
-            _, ms = timed(lambda: compiled(*targs), steps, warm)
+            _, ms = tstat(lambda: compiled(*targs), steps, warm)
+            traced_ms = float(ms)
             entry(name + "_traced", nbytes, "GB/s", ms, PEAK_HBM_GBS, "hbm")
             captured = compiled.capture(*targs)
             held = captured.inputs  # arguments already in the captured buffers: no copies in
-            _, ms = timed(lambda: captured(*held), steps, warm)
-            entry(name + "_graph", nbytes, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+            _, ms = tstat(lambda: captured(*held), steps, warm)
+            entry(name + "_graph", nbytes, "GB/s", ms, PEAK_HBM_GBS, "hbm", vs=("traced", traced_ms))
             captured.destroy()
             # (for configuration 4 the planner also finishes the layer on the dot's accumulators: dot, as_type and
             # the multiplication by the scales are one kernel)
             # element-wise groups (with the row reduction that follows them) as one kernel each: decoded by
-            # the interpreting kernels, then with each group's program compiled for the device on first use
+            # the interpreting kernels, then with each group's program compiled for the device on first use.
+            # A fused entry is priced at the bytes IT moves; `vs_traced` is its speed-up over node by node.
             fused = defn.compile(fun, *targs, fuse=True)
             for mode, tag in (("interpreted", "_fused"), ("compiled", "_fused_compiled")):
                 fused_mode(mode)
-                _, ms = timed(lambda: fused(*targs), steps, warm)
-                entry(name + tag, nbytes, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+                _, ms = tstat(lambda: fused(*targs), steps, warm)
+                entry(name + tag, fbytes, "GB/s", ms, PEAK_HBM_GBS, "hbm", vs=("traced", traced_ms))
             fused_mode("interpreted")
             # planned for compiled kernels from the start: groups over the same rows become stages of one program
             # (the softmax: row maximum, sum of exponentials and division in one kernel)
             staged = defn.compile(fun, *targs, fuse="compiled")
-            _, ms = timed(lambda: staged(*targs), steps, warm)
-            entry(name + "_planned_compiled", nbytes, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+            _, ms = tstat(lambda: staged(*targs), steps, warm)
+            entry(name + "_planned_compiled", pbytes, "GB/s", ms, PEAK_HBM_GBS, "hbm", vs=("traced", traced_ms))
         x, y = W.elementwise_reduce(n=16384)
         big = (put(x, "f32"), put(y, "f32"))
+        node_ms = suite["config1_chain_f32_16384"]["ms"]
         fused = defn.compile(chain1, *big, fuse=True)
-        # priced at the bytes of the node-by-node chain, like the unfused entry: above 1.0 means the fused
-        # pass beats what the reference's formulation can reach at all; `_one_pass` prices the compiled
-        # kernel at what it really moves (both operands once, one value per row)
+        # priced at what the one pass moves (both operands once, one value per row)
         for mode, tag in (("interpreted", "_fused"), ("compiled", "_fused_compiled")):
             fused_mode(mode)
-            _, ms = timed(lambda: fused(*big), steps, warm)
-            entry("config1_chain_f32_16384" + tag, 32.0 * 16384 * 16384 + 4.0 * 16384, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-        entry("config1_chain_f32_16384_fused_compiled_one_pass", 8.0 * 16384 * 16384 + 4.0 * 16384, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+            _, ms = tstat(lambda: fused(*big), steps, warm)
+            entry("config1_chain_f32_16384" + tag, 8.0 * 16384 * 16384 + 4.0 * 16384, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read",
+                  vs=("node_by_node", node_ms))
         fused_mode("interpreted")
         del big, x, y
         del cases, q, k

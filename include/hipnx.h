@@ -108,6 +108,11 @@ int hipnx_trim(hipnx_ctx *ctx);
 /* HIP-event stopwatch on the context's stream (device-side timing for benchmarks) */
 int hipnx_timer_start(hipnx_ctx *ctx);
 int hipnx_timer_stop(hipnx_ctx *ctx, float *elapsed_ms);
+/* lap marks of the same stopwatch: `mark` records event number `index` (0 .. 65535) on the stream
+ * and returns at once; `between` waits for mark `to` and gives the device time from mark `from` to
+ * it.  One mark per step gives per-step times (median, minimum) without a host wait per step. */
+int hipnx_timer_mark(hipnx_ctx *ctx, int index);
+int hipnx_timer_between(hipnx_ctx *ctx, int from, int to, float *elapsed_ms);
 
 /* ---- buffers -------------------------------------------------------------------------------
  * replaces: from_binary / to_binary / backend_copy / backend_transfer / backend_deallocate

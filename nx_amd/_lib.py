@@ -67,6 +67,8 @@ PROTOTYPES = {
     "hipnx_trim": [_ctx_p],
     "hipnx_timer_start": [_ctx_p],
     "hipnx_timer_stop": [_ctx_p, C.POINTER(C.c_float)],
+    "hipnx_timer_mark": [_ctx_p, C.c_int],
+    "hipnx_timer_between": [_ctx_p, C.c_int, C.c_int, C.POINTER(C.c_float)],
     "hipnx_buf_alloc": [_ctx_p, C.c_size_t, C.POINTER(_buf_p)],
     "hipnx_buf_free": [_buf_p],
     "hipnx_buf_destroy": [_buf_p],

@@ -893,6 +893,18 @@ def timer_stop(device: int = 0) -> float:
     return ms.value
 
 
+def timer_mark(index: int, device: int = 0) -> None:
+    """Records lap mark `index` of the stopwatch on the stream (returns at once)."""
+    L.check(L.lib.hipnx_timer_mark(_Context.get(device), index))
+
+
+def timer_between(start: int, stop: int, device: int = 0) -> float:
+    """Device milliseconds from lap mark `start` to lap mark `stop` (waits for `stop`)."""
+    ms = C.c_float()
+    L.check(L.lib.hipnx_timer_between(_Context.get(device), start, stop, C.byref(ms)))
+    return ms.value
+
+
 _capturing = set()  # devices whose context is recording instead of running
 
 

@@ -92,31 +92,34 @@ __global__ void __launch_bounds__(512) mfma_loop(const v4i *src, float *out, int
   }
 }
 
+// Streaming kernels with a grid that covers the buffer (no grid-stride loop): a work-group owns
+// UNROLL * 4 KiB of contiguous memory, every lane has UNROLL independent 16-byte accesses in flight.
+constexpr int UNROLL = 8;
 __global__ void __launch_bounds__(256) stream_read(const v4i *__restrict__ in, v4i *__restrict__ out, size_t n) {
-  v4i acc = {0, 0, 0, 0};
-  const size_t stride = (size_t)gridDim.x * 256;
-  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-  for (; i + 3 * stride < n; i += 4 * stride) {
-    const v4i a = in[i], b = in[i + stride], c = in[i + 2 * stride], d = in[i + 3 * stride];
-    acc ^= a ^ b ^ c ^ d;
-  }
-  for (; i < n; i += stride) acc ^= in[i];
+  const size_t base = (size_t)blockIdx.x * (256 * UNROLL) + threadIdx.x;
+  v4i v[UNROLL];
+#pragma unroll
+  for (int u = 0; u < UNROLL; u++) v[u] = base + u * 256 < n ? in[base + u * 256] : v4i{0, 0, 0, 0};
+  v4i acc = v[0];
+#pragma unroll
+  for (int u = 1; u < UNROLL; u++) acc ^= v[u];
   if (acc[0] == 0x12345678 && acc[1] == 0x0BADF00D) out[0] = acc;  // keeps the loads alive; practically never taken
 }
 __global__ void __launch_bounds__(256) stream_write(v4i *__restrict__ out, size_t n, int v) {
   const v4i x = {v, v + 1, v + 2, v + 3};
-  const size_t stride = (size_t)gridDim.x * 256;
-  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) out[i] = x;
+  const size_t base = (size_t)blockIdx.x * (256 * UNROLL) + threadIdx.x;
+#pragma unroll
+  for (int u = 0; u < UNROLL; u++)
+    if (base + u * 256 < n) out[base + u * 256] = x;
 }
 __global__ void __launch_bounds__(256) stream_copy(const v4i *__restrict__ in, v4i *__restrict__ out, size_t n) {
-  const size_t stride = (size_t)gridDim.x * 256;
-  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-  for (; i + stride < n; i += 2 * stride) {
-    const v4i a = in[i], b = in[i + stride];
-    out[i] = a;
-    out[i + stride] = b;
-  }
-  for (; i < n; i += stride) out[i] = in[i];
+  const size_t base = (size_t)blockIdx.x * (256 * UNROLL) + threadIdx.x;
+  v4i v[UNROLL];
+#pragma unroll
+  for (int u = 0; u < UNROLL; u++) v[u] = base + u * 256 < n ? in[base + u * 256] : v4i{0, 0, 0, 0};
+#pragma unroll
+  for (int u = 0; u < UNROLL; u++)
+    if (base + u * 256 < n) out[base + u * 256] = v[u];
 }
 
 static void launch_mfma(int kind, const v4i *d, float *o, int iters) {
@@ -210,7 +213,7 @@ static int run_stream(const char *mode, size_t mib, double want_ms) {
   CK(hipMemset(b, 2, bytes));
   const int m = !strcmp(mode, "read") ? 0 : !strcmp(mode, "write") ? 1 : !strcmp(mode, "copy") ? 2 : -1;
   if (m < 0) { fprintf(stderr, "unknown mode %s\n", mode); return 2; }
-  const unsigned grid = 256 * 32;
+  const unsigned grid = (unsigned)((n + 256 * UNROLL - 1) / (256 * UNROLL));
   auto launch = [&] {
     if (m == 0) hipLaunchKernelGGL(stream_read, dim3(grid), dim3(256), 0, 0, a, b, n);
     else if (m == 1) hipLaunchKernelGGL(stream_write, dim3(grid), dim3(256), 0, 0, b, n, 7);

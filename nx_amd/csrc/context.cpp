@@ -205,6 +205,8 @@ int hipnx_ctx_destroy(hipnx_ctx *ctx) {
   if (ctx->flag_host) (void)hipHostFree(ctx->flag_host);
   if (ctx->ev_start) (void)hipEventDestroy(ctx->ev_start);
   if (ctx->ev_stop) (void)hipEventDestroy(ctx->ev_stop);
+  for (hipEvent_t m : ctx->marks)
+    if (m) (void)hipEventDestroy(m);
   if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
   delete ctx;
   return HIPNX_OK;
@@ -254,6 +256,30 @@ int hipnx_timer_stop(hipnx_ctx *ctx, float *elapsed_ms) {
   HIPNX_HIP(hipEventRecord(ctx->ev_stop, ctx->stream));
   HIPNX_HIP(hipEventSynchronize(ctx->ev_stop));
   HIPNX_HIP(hipEventElapsedTime(elapsed_ms, ctx->ev_start, ctx->ev_stop));
+  return HIPNX_OK;
+}
+
+int hipnx_timer_mark(hipnx_ctx *ctx, int index) {
+  Enter in(ctx);
+  if (in.status) return in.status;
+  if (index < 0 || index > 65535) return set_error(HIPNX_EINVAL, "timer mark %d out of range (0..65535)", index);
+  HIPNX_NOT_CAPTURING(ctx, "timer");
+  if ((size_t)index >= ctx->marks.size()) ctx->marks.resize((size_t)index + 1, nullptr);
+  if (!ctx->marks[index]) HIPNX_HIP(hipEventCreate(&ctx->marks[index]));
+  HIPNX_HIP(hipEventRecord(ctx->marks[index], ctx->stream));
+  return HIPNX_OK;
+}
+
+int hipnx_timer_between(hipnx_ctx *ctx, int from, int to, float *elapsed_ms) {
+  Enter in(ctx);
+  if (in.status) return in.status;
+  if (!elapsed_ms) return set_error(HIPNX_EINVAL, "null elapsed_ms");
+  const int n = (int)ctx->marks.size();
+  if (from < 0 || to < 0 || from >= n || to >= n || !ctx->marks[from] || !ctx->marks[to])
+    return set_error(HIPNX_EINVAL, "timer marks %d / %d were never recorded", from, to);
+  HIPNX_NOT_CAPTURING(ctx, "timer");
+  HIPNX_HIP(hipEventSynchronize(ctx->marks[to]));
+  HIPNX_HIP(hipEventElapsedTime(elapsed_ms, ctx->marks[from], ctx->marks[to]));
   return HIPNX_OK;
 }
 

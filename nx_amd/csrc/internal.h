@@ -32,6 +32,7 @@ struct hipnx_ctx {
   int device = 0;
   hipStream_t stream = nullptr;
   hipEvent_t ev_start = nullptr, ev_stop = nullptr;
+  std::vector<hipEvent_t> marks;  // lap marks of the stopwatch, created on first use
   std::mutex mu;  // serialises enqueueing and the pool
   // size-bucketed cache of freed device blocks; reuse is safe without a device wait because
   // every kernel of this context runs on the one stream, in order
