@@ -32,6 +32,22 @@ PEAK = {"bf16": 2500.0, "f16": 2500.0, "s8": 5000.0, "f32": 157.3}  # dense MFMA
 # carries the figure in a line `TRAFFIC_BYTES_PER_LAUNCH = <n>`, which is what is reported here.
 TRAFFIC_PROFILE = os.path.join("profiles", "dot_bf16_4096_hbm_traffic.md")
 CEILINGS_BIN = os.path.join(ROOT, "nx_amd", "lib", "hipnx_ceilings")
+ABI_DRIVER_BIN = os.path.join(ROOT, "nx_amd", "lib", "hipnx_abi_driver")
+
+
+def c_abi_figures():
+    """Configuration 1's callbacks and `take` issued from plain C through libhipnx.so (what a NIF would
+    see): host microseconds per call and per chain, without Python or ctypes in the path."""
+    import subprocess
+    if not os.path.exists(ABI_DRIVER_BIN):
+        return None
+    try:
+        res = subprocess.run([ABI_DRIVER_BIN, "2000"], capture_output=True, text=True, timeout=180)
+        out = json.loads(res.stdout.strip().splitlines()[-1])
+        out["command"] = "nx_amd/lib/hipnx_abi_driver 2000 (tests/c_abi/abi_driver.c)"
+        return out
+    except Exception as exc:
+        return {"error": str(exc)[:200]}
 
 
 def headline_traffic():
@@ -448,6 +464,15 @@ def main():
         del big, x, y
         del cases, q, k
         result["suite"] = suite
+        c_abi = c_abi_figures()
+        if c_abi:
+            result["c_abi"] = c_abi
+            if "config1_chain_f32_1024_us" in c_abi:
+                us = c_abi["config1_chain_f32_1024_us"]
+                suite["config1_chain_f32_1024_c_abi"] = {
+                    "ms": round(us / 1e3, 5), "achieved": round((32.0 * 1024 * 1024 + 4096.0) / (us * 1e-6) / 1e9, 2), "unit": "GB/s",
+                    "bound": "hbm", "peak": PEAK_HBM_GBS, "frac": round((32.0 * 1024 * 1024 + 4096.0) / (us * 1e-6) / 1e9 / PEAK_HBM_GBS, 4),
+                    "note": "the same four callbacks issued from plain C (no Python): per chain, device kept busy"}
 
     # ---- CPU baseline: the reference-semantics restatement on a bounded sample -----------------
     if not args.no_cpu:

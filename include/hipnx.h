@@ -44,7 +44,16 @@ enum {
   HIPNX_ENOMEM = 4,        /* device allocation failed */
   HIPNX_EHIP = 5,          /* a HIP runtime call failed */
   HIPNX_EINDEX = 6,        /* gather/take index out of bounds (-> ArgumentError, reference text) */
-  HIPNX_EUNSUPPORTED = 7   /* type combination not implemented natively */
+  HIPNX_EUNSUPPORTED = 7,  /* type combination not implemented natively */
+  HIPNX_ERAISED = 8        /* a kernel issued EARLIER on this context met operands the reference raises for
+                            * (integer quotient / remainder by zero, a negative shift count, a negative
+                            * integer exponent, float remainder by zero or of a non-finite value:
+                            * binary_backend.ex:711-750; a deferred gather index).  Kernels cannot raise:
+                            * they record the first case in a pinned host word and write 0 (or skip the
+                            * slice); the next call that waits for the device -- hipnx_sync, hipnx_d2h,
+                            * hipnx_timer_stop / between, a raising gather -- returns this status once with
+                            * the reference's exception text ("ArithmeticError: ..." / "ArgumentError: ...")
+                            * and re-arms the word.  The data of that call is still delivered. */
 };
 
 /* element types, Nx.Type tuples {:u,8} .. {:f,64} (nx/lib/nx/type.ex:27-48) */
@@ -87,7 +96,10 @@ enum {
 /* out-of-bounds index policy of hipnx_gather */
 enum {
   HIPNX_OOB_RAISE = 0, /* Nx.BinaryBackend: raise (binary_backend.ex:1949-1952); waits for the kernel */
-  HIPNX_OOB_CLAMP = 1  /* EXLA / Torchx behaviour: clamp into range; stays asynchronous */
+  HIPNX_OOB_CLAMP = 1, /* EXLA / Torchx behaviour: clamp into range; stays asynchronous */
+  HIPNX_OOB_DEFER = 2  /* raise, but late: the kernel records the first bad index it meets and the next
+                        * waiting call on the context (hipnx_sync, hipnx_d2h, ...) fails with HIPNX_ERAISED;
+                        * the slices of bad tuples are left unwritten; stays asynchronous */
 };
 
 /* ---- context, errors ---------------------------------------------------------------------

@@ -13,7 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("HIPNX_LIB", os.path.join(_HERE, "lib", "libhipnx.so"))
 
 # status codes of include/hipnx.h
-OK, ALREADY_FREED, EINVAL, EFREED, ENOMEM, EHIP, EINDEX, EUNSUPPORTED = range(8)
+OK, ALREADY_FREED, EINVAL, EFREED, ENOMEM, EHIP, EINDEX, EUNSUPPORTED, ERAISED = range(9)
 
 
 class HipNxError(RuntimeError):
@@ -26,6 +26,10 @@ class HipNxError(RuntimeError):
 
 class HipNxArgumentError(HipNxError, ValueError):
     """Status codes the Elixir side maps to ArgumentError (EINVAL, EINDEX)."""
+
+
+class HipNxArithmeticError(HipNxError, ArithmeticError):
+    """ERAISED with the reference's ArithmeticError text (div / rem by zero, negative integer exponent)."""
 
 
 if not os.path.exists(LIB_PATH):
@@ -126,8 +130,12 @@ def check(status: int) -> int:
     """Raises on every status except OK and ALREADY_FREED (which the caller interprets)."""
     if status in (OK, ALREADY_FREED):
         return status
-    cls = HipNxArgumentError if status in (EINVAL, EINDEX) else HipNxError
-    raise cls(status, last_error())
+    message = last_error()
+    if status == ERAISED:  # the reference's exception, surfaced late (include/hipnx.h HIPNX_ERAISED)
+        cls = HipNxArithmeticError if message.startswith("ArithmeticError") else HipNxArgumentError
+    else:
+        cls = HipNxArgumentError if status in (EINVAL, EINDEX) else HipNxError
+    raise cls(status, message)
 
 
 @functools.lru_cache(maxsize=4096)

@@ -30,7 +30,8 @@ _BIT_COUNTS = (UNARY_OPS.index("count_leading_zeros"), UNARY_OPS.index("populati
 
 RED_SUM, RED_MAX, RED_MIN, RED_PRODUCT, RED_ALL, RED_ANY = 0, 1, 2, 3, 4, 5
 K_INNER, K_OUTER = 0, 1
-OOB_RAISE, OOB_CLAMP = 0, 1
+OOB_RAISE, OOB_CLAMP, OOB_DEFER = 0, 1, 2
+_bounds = {"policy": OOB_RAISE}
 
 # callbacks of the behaviour that are not on the device path (nx/lib/nx/backend.ex:58-144)
 UNSUPPORTED = ["conv", "window_sum", "window_product",
@@ -536,7 +537,7 @@ class HipNxBackend:
         n_tuples = prod(indices.shape[:-1])
         res = cls._alloc(out, dev)
         L.check(L.lib.hipnx_gather(res.data.ref.ctx, T.size_bytes(t.type), rank, L.i64_array(t.shape),
-                                   T.code(indices.type), n_tuples, depth, opts.get("oob_policy", OOB_RAISE),
+                                   T.code(indices.type), n_tuples, depth, opts.get("oob_policy", _bounds["policy"]),
                                    cls._handle(t), cls._handle(indices), res.data.ref.handle))
         return res
 
@@ -956,6 +957,20 @@ def mem_stats(device: int = 0):
     live, peak, pooled = C.c_uint64(), C.c_uint64(), C.c_uint64()
     L.check(L.lib.hipnx_mem_stats(_Context.get(device), C.byref(live), C.byref(peak), C.byref(pooled)))
     return {"live": live.value, "peak": peak.value, "pooled": pooled.value}
+
+
+def bounds_policy(policy: str) -> str:
+    """What `gather` / `take` do with an out-of-range index from now on; returns the previous setting.
+    "raise" (the default, `Nx.BinaryBackend`'s behaviour: the call waits for its kernel and raises with
+    the reference's message), "clamp" (EXLA's and Torchx's behaviour, asynchronous) or "defer" (raises,
+    but late: the kernel records the bad index and the next call that waits for the device -- `to_binary`,
+    `sync` -- raises; asynchronous, so a take costs a launch instead of a launch and a wait)."""
+    names = {"raise": OOB_RAISE, "clamp": OOB_CLAMP, "defer": OOB_DEFER}
+    if policy not in names:
+        raise ValueError(f"expected one of {sorted(names)!r}, got: {policy!r}")
+    previous = next(k for k, v in names.items() if v == _bounds["policy"])
+    _bounds["policy"] = names[policy]
+    return previous
 
 
 def fused_mode(mode: str, device: int = 0) -> None:

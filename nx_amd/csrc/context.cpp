@@ -125,6 +125,25 @@ int pool_free(hipnx_ctx *ctx, void *ptr, size_t cap) {
   return HIPNX_OK;
 }
 
+// codes: HIPNX_RAISE_* of elementwise_ops.cuh (kept in step by value)
+int deferred_error(hipnx_ctx *ctx) {
+  volatile unsigned long long *word = (volatile unsigned long long *)((char *)ctx->flag_host + 16);
+  const unsigned long long w = *word;
+  if (w == 0) return HIPNX_OK;
+  *word = 0;
+  const int code = (int)(w >> 56);
+  long long operand = (long long)(w << 8) >> 8;  // sign-extend the low 56 bits
+  switch (code) {
+    case 1: return set_error(HIPNX_ERAISED, "ArithmeticError: bad argument in arithmetic expression (raised late: an earlier quotient / remainder on this context divided by zero)");
+    case 2: return set_error(HIPNX_ERAISED, "ArgumentError: cannot left shift by %lld (raised late: an earlier left_shift on this context)", operand);
+    case 3: return set_error(HIPNX_ERAISED, "ArgumentError: cannot right shift by %lld (raised late: an earlier right_shift on this context)", operand);
+    case 4: return set_error(HIPNX_ERAISED, "ArithmeticError: bad argument in arithmetic expression (raised late: an earlier integer pow on this context had the negative exponent %lld)", operand);
+    case 5: return set_error(HIPNX_ERAISED, "ArgumentError: errors were found at the given arguments: not a number (raised late: an earlier float remainder on this context met a non-finite element)");
+    case 6: return set_error(HIPNX_ERAISED, "ArgumentError: index %lld is out of bounds (raised late: an earlier gather / take on this context with the deferred bounds policy)", operand);
+  }
+  return set_error(HIPNX_ERAISED, "an earlier kernel on this context recorded error code %d", code);
+}
+
 }  // namespace hipnx
 
 using namespace hipnx;
@@ -217,7 +236,7 @@ int hipnx_sync(hipnx_ctx *ctx) {
   if (in.status) return in.status;
   HIPNX_NOT_CAPTURING(ctx, "sync");
   HIPNX_HIP(hipStreamSynchronize(ctx->stream));
-  return HIPNX_OK;
+  return deferred_error(ctx);
 }
 
 int hipnx_mem_stats(hipnx_ctx *ctx, uint64_t *live, uint64_t *peak, uint64_t *pooled) {
@@ -256,7 +275,7 @@ int hipnx_timer_stop(hipnx_ctx *ctx, float *elapsed_ms) {
   HIPNX_HIP(hipEventRecord(ctx->ev_stop, ctx->stream));
   HIPNX_HIP(hipEventSynchronize(ctx->ev_stop));
   HIPNX_HIP(hipEventElapsedTime(elapsed_ms, ctx->ev_start, ctx->ev_stop));
-  return HIPNX_OK;
+  return deferred_error(ctx);
 }
 
 int hipnx_timer_mark(hipnx_ctx *ctx, int index) {
@@ -280,7 +299,7 @@ int hipnx_timer_between(hipnx_ctx *ctx, int from, int to, float *elapsed_ms) {
   HIPNX_NOT_CAPTURING(ctx, "timer");
   HIPNX_HIP(hipEventSynchronize(ctx->marks[to]));
   HIPNX_HIP(hipEventElapsedTime(elapsed_ms, ctx->marks[from], ctx->marks[to]));
-  return HIPNX_OK;
+  return deferred_error(ctx);
 }
 
 // ---- captured graphs -------------------------------------------------------------------------
@@ -442,12 +461,12 @@ int hipnx_d2h(hipnx_ctx *ctx, const hipnx_buf *src, size_t src_offset, void *dst
   HIPNX_NOT_CAPTURING(ctx, "d2h");
   if (bytes == 0) {
     HIPNX_HIP(hipStreamSynchronize(ctx->stream));
-    return HIPNX_OK;
+    return deferred_error(ctx);
   }
   if (!dst) return set_error(HIPNX_EINVAL, "d2h: null destination");
   HIPNX_HIP(hipMemcpyAsync(dst, (const char *)src->ptr + src_offset, bytes, hipMemcpyDeviceToHost, ctx->stream));
   HIPNX_HIP(hipStreamSynchronize(ctx->stream));
-  return HIPNX_OK;
+  return deferred_error(ctx);  // the bytes have been delivered either way
 }
 
 int hipnx_d2d(hipnx_ctx *ctx, hipnx_buf *dst, size_t dst_offset, const hipnx_buf *src, size_t src_offset,

@@ -24,7 +24,8 @@ template <int OP, typename CT, bool UNS>
 __global__ void __launch_bounds__(BLOCK)
 binary_vec_kernel(const void *__restrict__ l, const void *__restrict__ r, void *__restrict__ out, int ldt, int rdt,
                   int odt, int64_t cols, int64_t vecs_per_row, int64_t nvec, int64_t ls0, int ls1, int64_t rs0,
-                  int rs1) {
+                  int rs1, unsigned long long *__restrict__ err) {
+  constexpr bool RAISES = binary_can_raise(OP, is_fp<CT>::value);
   for (int64_t v = (int64_t)blockIdx.x * BLOCK + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * BLOCK) {
     int64_t row = v / vecs_per_row;
     int64_t col = (v - row * vecs_per_row) * E;
@@ -45,10 +46,20 @@ binary_vec_kernel(const void *__restrict__ l, const void *__restrict__ r, void *
       }
 #pragma unroll
       for (int i = 0; i < E; i++) c[i] = binary_apply<OP, CT, UNS>(a[i], b[i]);
+      if constexpr (RAISES) {
+        long long operand = 0;
+#pragma unroll
+        for (int i = 0; i < E; i++)
+          if (int code = binary_raises<OP, CT, UNS>(a[i], b[i], &operand)) report_raise(err, code, operand);
+      }
       store_vec<CT, E>(out, odt, oo, c);
     } else {  // ragged tail of a row
       for (int i = 0; col + i < cols; i++) {
         CT x = load_one<CT>(l, ldt, lo + i * ls1), y = load_one<CT>(r, rdt, ro + i * rs1);
+        if constexpr (RAISES) {
+          long long operand = 0;
+          if (int code = binary_raises<OP, CT, UNS>(x, y, &operand)) report_raise(err, code, operand);
+        }
         store_one<CT>(out, odt, oo + i, binary_apply<OP, CT, UNS>(x, y));
       }
     }
@@ -66,11 +77,24 @@ __device__ __forceinline__ CT binary_switch(int op, CT a, CT b) {
   return (CT)0;
 }
 
+template <typename CT, bool UNS>
+__device__ __forceinline__ int binary_raises_switch(int op, CT a, CT b, long long *operand) {
+  switch (op) {
+    case HIPNX_QUOTIENT: return binary_raises<HIPNX_QUOTIENT, CT, UNS>(a, b, operand);
+    case HIPNX_REMAINDER: return binary_raises<HIPNX_REMAINDER, CT, UNS>(a, b, operand);
+    case HIPNX_LEFT_SHIFT: return binary_raises<HIPNX_LEFT_SHIFT, CT, UNS>(a, b, operand);
+    case HIPNX_RIGHT_SHIFT: return binary_raises<HIPNX_RIGHT_SHIFT, CT, UNS>(a, b, operand);
+    case HIPNX_POW: return binary_raises<HIPNX_POW, CT, UNS>(a, b, operand);
+  }
+  return HIPNX_RAISE_NONE;
+}
+
 // any rank, any strides: one element per lane per step
 template <typename CT, bool UNS>
 __global__ void __launch_bounds__(BLOCK)
 binary_nd_kernel(const void *__restrict__ l, const void *__restrict__ r, void *__restrict__ out, int op, int ldt,
-                 int rdt, int odt, int64_t n, NdIndex ix) {
+                 int rdt, int odt, int64_t n, NdIndex ix, unsigned long long *__restrict__ err) {
+  const bool raises = binary_can_raise(op, is_fp<CT>::value);
   for (int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x; i < n; i += (int64_t)gridDim.x * BLOCK) {
     int64_t rem = i, lo = 0, ro = 0;
     for (int a = ix.rank - 1; a >= 0; a--) {
@@ -80,6 +104,10 @@ binary_nd_kernel(const void *__restrict__ l, const void *__restrict__ r, void *_
       ro += c * ix.rs[a];
     }
     CT x = load_one<CT>(l, ldt, lo), y = load_one<CT>(r, rdt, ro);
+    if (raises) {
+      long long operand = 0;
+      if (int code = binary_raises_switch<CT, UNS>(op, x, y, &operand)) report_raise(err, code, operand);
+    }
     store_one<CT>(out, odt, i, binary_switch<CT, UNS>(op, x, y));
   }
 }
@@ -160,12 +188,13 @@ struct BinArgs {
   int ldt, rdt, odt;
   int64_t cols, vecs_per_row, nvec, ls0, rs0;
   int ls1, rs1;
+  unsigned long long *err;  // the context's deferred error word (device address of the pinned host word)
 };
 
 template <int OP, typename CT, bool UNS>
 static void launch_bvec(const hipnx_ctx *ctx, const BinArgs &a) {
   hipLaunchKernelGGL((binary_vec_kernel<OP, CT, UNS>), dim3(grid_for(ctx, a.nvec)), dim3(BLOCK), 0, ctx->stream, a.l,
-                     a.r, a.out, a.ldt, a.rdt, a.odt, a.cols, a.vecs_per_row, a.nvec, a.ls0, a.ls1, a.rs0, a.rs1);
+                     a.r, a.out, a.ldt, a.rdt, a.odt, a.cols, a.vecs_per_row, a.nvec, a.ls0, a.ls1, a.rs0, a.rs1, a.err);
 }
 
 template <int OP>
@@ -273,6 +302,7 @@ extern "C" int hipnx_binary(hipnx_ctx *ctx, int op, int l_dt, int r_dt, int out_
       a.vecs_per_row = (cols + E - 1) / E;
       a.nvec = rows * a.vecs_per_row;
       a.ls0 = l0; a.rs0 = r0; a.ls1 = (int)l1; a.rs1 = (int)r1;
+      a.err = deferred_error_word(ctx);
     }
   }
   if (vec_ok) {
@@ -287,19 +317,19 @@ extern "C" int hipnx_binary(hipnx_ctx *ctx, int op, int l_dt, int r_dt, int out_
     switch (cls) {
       case CLS_F32:
         hipLaunchKernelGGL((binary_nd_kernel<float, false>), grid, block, 0, ctx->stream, l->ptr, r->ptr, out->ptr, op,
-                           l_dt, r_dt, out_dt, n, ix);
+                           l_dt, r_dt, out_dt, n, ix, deferred_error_word(ctx));
         break;
       case CLS_F64:
         hipLaunchKernelGGL((binary_nd_kernel<double, false>), grid, block, 0, ctx->stream, l->ptr, r->ptr, out->ptr, op,
-                           l_dt, r_dt, out_dt, n, ix);
+                           l_dt, r_dt, out_dt, n, ix, deferred_error_word(ctx));
         break;
       case CLS_I64:
         hipLaunchKernelGGL((binary_nd_kernel<int64_t, false>), grid, block, 0, ctx->stream, l->ptr, r->ptr, out->ptr,
-                           op, l_dt, r_dt, out_dt, n, ix);
+                           op, l_dt, r_dt, out_dt, n, ix, deferred_error_word(ctx));
         break;
       default:
         hipLaunchKernelGGL((binary_nd_kernel<int64_t, true>), grid, block, 0, ctx->stream, l->ptr, r->ptr, out->ptr, op,
-                           l_dt, r_dt, out_dt, n, ix);
+                           l_dt, r_dt, out_dt, n, ix, deferred_error_word(ctx));
         break;
     }
   }

@@ -31,6 +31,48 @@ constexpr bool binary_sign_matters(int op) {
          op == HIPNX_RIGHT_SHIFT || (op >= HIPNX_GREATER && op <= HIPNX_LESS_EQUAL) || op == HIPNX_POW;
 }
 
+// Operand pairs the reference raises for instead of returning a value (binary_backend.ex:711-750):
+// codes of the deferred error word (the top byte; the low 56 bits carry the offending operand).
+enum {
+  HIPNX_RAISE_NONE = 0,
+  HIPNX_RAISE_BADARITH = 1,     // div/2, rem/2 by zero; :math.fmod/2 with a zero divisor
+  HIPNX_RAISE_LEFT_SHIFT = 2,   // "cannot left shift by <n>"
+  HIPNX_RAISE_RIGHT_SHIFT = 3,  // "cannot right shift by <n>"
+  HIPNX_RAISE_NEG_EXPONENT = 4, // Integer.pow/2 with a negative exponent
+  HIPNX_RAISE_NOT_A_NUMBER = 5, // :math.fmod/2 of a non-finite element
+  HIPNX_RAISE_INDEX = 6         // gather index out of bounds (deferred policy)
+};
+constexpr bool binary_can_raise(int op, bool fp) {
+  return fp ? op == HIPNX_REMAINDER
+            : (op == HIPNX_QUOTIENT || op == HIPNX_REMAINDER || op == HIPNX_LEFT_SHIFT || op == HIPNX_RIGHT_SHIFT || op == HIPNX_POW);
+}
+template <int OP, typename CT, bool UNS>
+__device__ __forceinline__ int binary_raises(CT a, CT b, long long *operand) {
+  if constexpr (is_fp<CT>::value) {
+    if constexpr (OP == HIPNX_REMAINDER) {
+      if (a != a || b != b || a - a != 0 || b - b != 0) return HIPNX_RAISE_NOT_A_NUMBER;
+      if (b == 0) return HIPNX_RAISE_BADARITH;
+    }
+  } else {
+    *operand = (long long)b;
+    if constexpr (OP == HIPNX_QUOTIENT || OP == HIPNX_REMAINDER) {
+      if (b == 0) return HIPNX_RAISE_BADARITH;
+    } else if constexpr (OP == HIPNX_LEFT_SHIFT) {
+      if (!UNS && b < 0) return HIPNX_RAISE_LEFT_SHIFT;
+    } else if constexpr (OP == HIPNX_RIGHT_SHIFT) {
+      if (!UNS && b < 0) return HIPNX_RAISE_RIGHT_SHIFT;
+    } else if constexpr (OP == HIPNX_POW) {
+      if (!UNS && b < 0) return HIPNX_RAISE_NEG_EXPONENT;
+    }
+  }
+  return HIPNX_RAISE_NONE;
+}
+// the report: one 8-byte store to the context's pinned host word (any of the offending lanes may win)
+__device__ __forceinline__ void report_raise(unsigned long long *err, int code, long long operand) {
+  __hip_atomic_store(err, ((unsigned long long)code << 56) | ((unsigned long long)operand & 0x00FFFFFFFFFFFFFFull),
+                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
 __device__ __forceinline__ int64_t ipow_wrap(int64_t base, uint64_t e) {
   uint64_t r = 1, b = (uint64_t)base;
   while (e) {
@@ -85,7 +127,7 @@ __device__ __forceinline__ CT binary_apply(CT a, CT b) {
     else if constexpr (OP == HIPNX_BITWISE_AND) return a & b;
     else if constexpr (OP == HIPNX_BITWISE_OR) return a | b;
     else if constexpr (OP == HIPNX_BITWISE_XOR) return a ^ b;
-    else if constexpr (OP == HIPNX_LEFT_SHIFT) return (b < 0 || b >= 64) ? 0 : (int64_t)(ua << b);
+    else if constexpr (OP == HIPNX_LEFT_SHIFT) return ((!UNS && b < 0) || ub >= 64) ? 0 : (int64_t)(ua << b);
     else if constexpr (OP == HIPNX_RIGHT_SHIFT) {
       if (b < 0) return 0;  // the reference raises ArgumentError
       if (b >= 64) return (!UNS && a < 0) ? -1 : 0;

@@ -88,6 +88,15 @@ int check_buf(const hipnx_ctx *ctx, const hipnx_buf *b, uint64_t need_bytes, con
 int pool_alloc(hipnx_ctx *ctx, size_t bytes, void **ptr_out, size_t *cap_out);
 int pool_free(hipnx_ctx *ctx, void *ptr, size_t cap);
 
+// The deferred error word: 8 bytes of the context's pinned, device-mapped host block (offset 16; the
+// first word belongs to the gather bounds report).  Kernels that meet operands the reference raises
+// for store (code << 56 | operand) there; deferred_error() is called by every entry point that has
+// just waited for the stream and turns a recorded case into HIPNX_ERAISED (once; the word is re-armed).
+inline unsigned long long *deferred_error_word(const hipnx_ctx *ctx) {
+  return (unsigned long long *)((char *)ctx->flag_host_dev + 16);
+}
+int deferred_error(hipnx_ctx *ctx);
+
 // looks up this device's address of the static scratch array of hipnx_reduce_static (the device of
 // `ctx` must be current); defined beside the array in reduce.hip
 int reduce_static_init(hipnx_ctx *ctx);

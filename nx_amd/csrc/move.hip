@@ -76,7 +76,7 @@ __global__ void __launch_bounds__(BLOCK)
 gather_kernel(const unsigned char *__restrict__ t, const void *__restrict__ idx, unsigned char *__restrict__ out,
               int idx_dt, int64_t n_tuples, int depth, Strided tdims /* dims = leading extents, strides = bytes */,
               int64_t slice_bytes, int lpr, int clamp, unsigned long long *__restrict__ flag,
-              unsigned int *__restrict__ host_seen) {
+              unsigned int *__restrict__ host_seen, unsigned long long *__restrict__ deferred) {
   constexpr int W = VEC ? 16 : 1;
   typedef raw_vec<W> vec_t;
   const int64_t chunks = slice_bytes / W;
@@ -94,8 +94,13 @@ gather_kernel(const unsigned char *__restrict__ t, const void *__restrict__ idx,
         else {
           ok = false;
           if (lane == 0) {
-            atomicMin(flag, (unsigned long long)(row * depth + a));
-            __hip_atomic_store(host_seen, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);  // pinned host word
+            if (deferred) {  // the policy that reports late: code 6 (HIPNX_RAISE_INDEX) and the offending index
+              __hip_atomic_store(deferred, (6ull << 56) | ((unsigned long long)v & 0x00FFFFFFFFFFFFFFull), __ATOMIC_RELAXED,
+                                 __HIP_MEMORY_SCOPE_SYSTEM);
+            } else {
+              atomicMin(flag, (unsigned long long)(row * depth + a));
+              __hip_atomic_store(host_seen, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);  // pinned host word
+            }
           }
           break;
         }
@@ -272,7 +277,8 @@ extern "C" int hipnx_gather(hipnx_ctx *ctx, int elem_bytes, int rank, const int6
     return set_error(HIPNX_EINVAL, "gather: bad rank / depth");
   if (elem_bytes <= 0 || dtype_size(idx_dt) < 0 || is_float(idx_dt))
     return set_error(HIPNX_EINVAL, "gather: indices must be an integer type");
-  if (oob_policy != HIPNX_OOB_RAISE && oob_policy != HIPNX_OOB_CLAMP) return set_error(HIPNX_EINVAL, "gather: bad policy");
+  if (oob_policy != HIPNX_OOB_RAISE && oob_policy != HIPNX_OOB_CLAMP && oob_policy != HIPNX_OOB_DEFER)
+    return set_error(HIPNX_EINVAL, "gather: bad policy");
   int64_t total = 1, slice = 1;
   for (int a = 0; a < rank; a++) {
     if (t_dims[a] < 0) return set_error(HIPNX_EINVAL, "gather: negative dimension");
@@ -305,16 +311,17 @@ extern "C" int hipnx_gather(hipnx_ctx *ctx, int elem_bytes, int rank, const int6
   dim3 grid(grid_for(ctx, n_tuples, BLOCK / lpr)), block(BLOCK);
   if (vec)
     hipLaunchKernelGGL((gather_kernel<true>), grid, block, 0, ctx->stream, (const unsigned char *)t->ptr, idx->ptr,
-                       (unsigned char *)out->ptr, idx_dt, n_tuples, depth, td, slice_bytes, lpr, (int)(oob_policy == HIPNX_OOB_CLAMP), flag, (unsigned int *)ctx->flag_host_dev);
+                       (unsigned char *)out->ptr, idx_dt, n_tuples, depth, td, slice_bytes, lpr, (int)(oob_policy == HIPNX_OOB_CLAMP), flag, (unsigned int *)ctx->flag_host_dev, oob_policy == HIPNX_OOB_DEFER ? deferred_error_word(ctx) : nullptr);
   else
     hipLaunchKernelGGL((gather_kernel<false>), grid, block, 0, ctx->stream, (const unsigned char *)t->ptr, idx->ptr,
-                       (unsigned char *)out->ptr, idx_dt, n_tuples, depth, td, slice_bytes, lpr, (int)(oob_policy == HIPNX_OOB_CLAMP), flag, (unsigned int *)ctx->flag_host_dev);
+                       (unsigned char *)out->ptr, idx_dt, n_tuples, depth, td, slice_bytes, lpr, (int)(oob_policy == HIPNX_OOB_CLAMP), flag, (unsigned int *)ctx->flag_host_dev, oob_policy == HIPNX_OOB_DEFER ? deferred_error_word(ctx) : nullptr);
   HIPNX_HIP(hipGetLastError());
   if (oob_policy == HIPNX_OOB_RAISE) {
     // the reference raises on the first offending index: wait, then report it the same way.
     // The kernel marks a pinned host word when it meets one, so the good path costs the wait only.
     volatile unsigned int *seen = (volatile unsigned int *)ctx->flag_host;
     HIPNX_HIP(hipStreamSynchronize(ctx->stream));
+    if (seen[0] == 0) return deferred_error(ctx);  // nothing of this call; something recorded earlier surfaces here
     if (seen[0] != 0) {
       unsigned long long first = ~0ull;
       HIPNX_HIP(hipMemcpy(&first, flag, 8, hipMemcpyDeviceToHost));

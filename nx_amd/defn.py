@@ -18,6 +18,7 @@ their own; outside a trace they run eagerly.
 """
 from __future__ import annotations
 
+import math
 import itertools
 import operator
 import threading
@@ -470,6 +471,8 @@ def _fusable(t: Tensor) -> bool:
     op, args = e.op, e.args
     if _plan["ints"]:
         if op in _INT_FUSED_BINARY and t.type in _INT32:
+            if op in ("left_shift", "right_shift") and (_const(args[1]) is None or _const(args[1]) < 0):
+                return False  # a negative count raises in the reference: only the separate kernel reports it
             def word_ok(a):
                 if _const(a) is None:
                     return a.type == t.type
@@ -493,6 +496,8 @@ def _fusable(t: Tensor) -> bool:
         out_ok = t.type == _TRUTH if op in ("is_nan", "is_infinity") else t.type in _NARROW
         return out_ok and value_ok(args[0])
     if op in BINARY_OPS and op not in _INT_ONLY_BINARY:
+        if op == "remainder" and not (_const(args[1]) is not None and _const(args[1]) != 0 and math.isfinite(_const(args[1]))):
+            return False  # :math.fmod raises for a zero divisor or a non-finite element: left to the separate kernel
         if op in _LOGICAL:
             return t.type == _TRUTH and all(a.type in _NARROW or a.type == _TRUTH for a in args)
         out_ok = t.type == _TRUTH if op in _COMPARE else t.type in _NARROW

@@ -498,6 +498,17 @@ def all_close(a, b, equal_nan=False, rtol=1.0e-5, atol=1.0e-8):
     return block(BlockAllClose(equal_nan, rtol, atol), [a, b], template(("u", 8), ()), compose)
 
 
+@dataclass(frozen=True)
+class BlockLogicalNot:
+    """%Nx.Block.LogicalNot{} (nx/lib/nx/block.ex)."""
+
+
+def logical_not(t):
+    """Nx.logical_not/1 (nx.ex:7345-7353): a block whose default body is `equal(t, 0)`; u8 output."""
+    t = to_tensor(t)
+    return block(BlockLogicalNot(), [t], template(("u", 8), t.shape), lambda _struct, x: equal(x, 0))
+
+
 def block(struct, args, out, fun):
     """Nx.block/4 (nx.ex:7370-7380): lets the backend replace a composite op."""
     return _impl(*args).block(struct, out, list(args), fun)

@@ -24,6 +24,7 @@
  */
 #include "hipnx_ref.h"
 #include <math.h>
+#include <stdarg.h>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
@@ -47,8 +48,11 @@ static int nthreads(void) {
 #endif
 }
 
-static int fail(int code, const char *msg) {
-  snprintf(g_err, sizeof g_err, "%s", msg);
+static int fail(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof g_err, fmt, ap);
+  va_end(ap);
   return code;
 }
 
@@ -243,7 +247,14 @@ static int bin_elem(int op, num a, num b, num *out) {
       if (both_int(a, b)) {
         if (b.i == 0) return fail(REF_ERAISE, "ArithmeticError: bad argument in arithmetic expression");
         *out = mk_int(a.i % b.i); /* C99 %: sign of the dividend, like rem/2 */
-      } else *out = from_double(fmod(to_double(a), to_double(b)));
+      } else {
+        /* :math.fmod/2 (binary_backend.ex:713): it takes numbers only -- the atoms of non-finite elements
+         * raise ArgumentError (nx/test/nx/non_finite_test.exs:257-267) -- and a zero divisor is badarith */
+        if (is_atom(a) || is_atom(b))
+          return fail(REF_ERAISE, "ArgumentError: errors were found at the given arguments: not a number");
+        if (to_double(b) == 0.0) return fail(REF_ERAISE, "ArithmeticError: bad argument in arithmetic expression");
+        *out = from_double(fmod(to_double(a), to_double(b)));
+      }
       return REF_OK;
     case REF_QUOTIENT:
       if (!both_int(a, b)) return fail(REF_ERAISE, "ArithmeticError: div/2 needs integers");
@@ -271,11 +282,11 @@ static int bin_elem(int op, num a, num b, num *out) {
     case REF_BITWISE_OR: *out = mk_int(a.i | b.i); return REF_OK;
     case REF_BITWISE_XOR: *out = mk_int(a.i ^ b.i); return REF_OK;
     case REF_LEFT_SHIFT:
-      if (b.i < 0) return fail(REF_ERAISE, "ArgumentError: cannot left shift by a negative count");
+      if (b.i < 0) return fail(REF_ERAISE, "ArgumentError: cannot left shift by %lld", (long long)b.i);
       *out = mk_int(b.i >= 127 ? 0 : (i128)((u128)a.i << (int)b.i));
       return REF_OK;
     case REF_RIGHT_SHIFT:
-      if (b.i < 0) return fail(REF_ERAISE, "ArgumentError: cannot right shift by a negative count");
+      if (b.i < 0) return fail(REF_ERAISE, "ArgumentError: cannot right shift by %lld", (long long)b.i);
       *out = mk_int(b.i >= 127 ? (a.i < 0 ? -1 : 0) : (a.i >> (int)b.i));
       return REF_OK;
     case REF_EQUAL:
