@@ -15,6 +15,7 @@
 #include <type_traits>
 
 #include <algorithm>
+#include <cstdlib>
 
 #include "gemm_launch.cuh"
 

@@ -24,11 +24,13 @@ int launch_gemm_rows(const hipnx_ctx *ctx, int dt, GemmArgs a, int64_t batch);
 template <int DT, int WM, int WN, int TM, int TN, bool LK, bool RK, int NSTAGE = 2>
 static int launch_one(const hipnx_ctx *ctx, GemmArgs a, int64_t batch) {
   constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
-  constexpr int smem = NSTAGE * (BM + BN) * SLAB;
+  constexpr int smem_max = NSTAGE * (BM + BN) * SLAB;
+  // a K of one slab only ever touches the first stage: the rest of the LDS stays with other work-groups
+  const int smem = a.Kb <= SLAB ? (BM + BN) * SLAB : smem_max;
   auto kern = gemm_pipelined_kernel<DT, WM, WN, TM, TN, LK, RK, NSTAGE>;
   static bool configured = false;  // per instantiation; racing writers store the same value
   if (!configured) {
-    HIPNX_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
+    HIPNX_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem_max));
     configured = true;
   }
   a.tiles_m = (int)((a.M + BM - 1) / BM);

@@ -412,20 +412,47 @@ __device__ __forceinline__ void gemm_epilogue(typename Mma16<DT>::acc_t (&acc)[T
     };
     // N % 8 == 0: a group of 8 columns lies wholly inside or outside, and row starts keep the 16-byte alignment
     const bool paired = (N % 8) == 0 && ((uintptr_t)out & 15) == 0;
+    // A second exchange makes the runs whole cache lines: of two neighbouring PAIRS of tiles the lanes of
+    // rows 8..15 hand their first pair's 16 bytes to the lane 8 rows up and take that lane's second pair, so
+    // that one store instruction covers rows 0..7 with 128 contiguous bytes each (four tiles wide) and the
+    // next one rows 8..15 -- instead of 16 rows of 64 bytes.
+    const bool hi = (lane >> 3) & 1;
+    auto pair16 = [&](int i, int j) -> v4i {  // this lane's 8 columns of tiles j, j+1 (see above)
+      const uint32_t a0 = pack(acc[i][j][0], acc[i][j][1]), a1 = pack(acc[i][j][2], acc[i][j][3]);
+      const uint32_t b0 = pack(acc[i][j + 1][0], acc[i][j + 1][1]), b1 = pack(acc[i][j + 1][2], acc[i][j + 1][3]);
+      const uint32_t r0 = (uint32_t)__shfl_xor((int)(odd ? a0 : b0), 16, 64);
+      const uint32_t r1 = (uint32_t)__shfl_xor((int)(odd ? a1 : b1), 16, 64);
+      v4i v;
+      v[0] = (int)(odd ? r0 : a0); v[1] = (int)(odd ? r1 : a1); v[2] = (int)(odd ? b0 : r0); v[3] = (int)(odd ? b1 : r1);
+      return v;
+    };
+    auto put16 = [&](int64_t gm, int64_t gn, const v4i &v) {
+      if (gm < M && gn < N) *reinterpret_cast<v4i *>((unsigned char *)out + (obase + gm * N + gn) * 2) = v;
+    };
 #pragma unroll
     for (int i = 0; i < TM; i++) {
       const int64_t gm = row0 + 16 * i + (lane & 15);
+      if constexpr (TN % 4 == 0) {
+        if (paired) {
+#pragma unroll
+          for (int j = 0; j < TN; j += 4) {
+            const v4i v = pair16(i, j), w = pair16(i, j + 2);
+            v4i got;  // the partner's other pair: rows 0..7 receive the second pair of rows 8..15 and vice versa
+#pragma unroll
+            for (int e = 0; e < 4; e++) got[e] = __shfl_xor(hi ? v[e] : w[e], 8, 64);
+            const int64_t gn0 = gc + 16 * (j + (odd ? 1 : 0)), gn1 = gn0 + 32;
+            // rows 0..7 of the 16: own first pair (rows < 8) | the partner's second pair, stored for row - 8
+            put16(hi ? gm - 8 : gm, hi ? gn1 : gn0, hi ? got : v);
+            // rows 8..15: own second pair stays with rows >= 8 | rows < 8 store the partner's first pair for row + 8
+            put16(hi ? gm : gm + 8, hi ? gn1 : gn0, hi ? w : got);
+          }
+          continue;
+        }
+      }
 #pragma unroll
       for (int j = 0; j < TN; j += 2) {
         if (paired) {
-          const uint32_t a0 = pack(acc[i][j][0], acc[i][j][1]), a1 = pack(acc[i][j][2], acc[i][j][3]);
-          const uint32_t b0 = pack(acc[i][j + 1][0], acc[i][j + 1][1]), b1 = pack(acc[i][j + 1][2], acc[i][j + 1][3]);
-          const uint32_t r0 = (uint32_t)__shfl_xor((int)(odd ? a0 : b0), 16, 64);
-          const uint32_t r1 = (uint32_t)__shfl_xor((int)(odd ? a1 : b1), 16, 64);
-          v4i v;
-          v[0] = (int)(odd ? r0 : a0); v[1] = (int)(odd ? r1 : a1); v[2] = (int)(odd ? b0 : r0); v[3] = (int)(odd ? b1 : r1);
-          const int64_t gn = gc + 16 * (j + (odd ? 1 : 0));
-          if (gm < M && gn < N) *reinterpret_cast<v4i *>((unsigned char *)out + (obase + gm * N + gn) * 2) = v;
+          put16(gm, gc + 16 * (j + (odd ? 1 : 0)), pair16(i, j));
         } else {
 #pragma unroll
           for (int jj = j; jj < j + 2; jj++) {
@@ -442,6 +469,45 @@ __device__ __forceinline__ void gemm_epilogue(typename Mma16<DT>::acc_t (&acc)[T
                   if (gn + e < N) store_one<float>(out, ODT, idx + e, v[e]);
               }
             }
+          }
+        }
+      }
+    }
+  } else if constexpr ((ODT == HIPNX_S32 || ODT == HIPNX_U32 || ODT == HIPNX_F32) && TN % 2 == 0) {
+    // 4-byte outputs: a lane's 4 outputs of a tile are 16 bytes, 64 contiguous bytes per row.  Of two
+    // neighbouring column tiles the lanes of rows 8..15 hand their first tile's values to the lane 8 rows up
+    // and take that lane's second tile, so that a store instruction writes 8 rows of 128 contiguous bytes
+    // (whole cache lines) instead of 16 rows of 64: the 64 MiB s32 result of the int8 kernel is the longest
+    // part of its epilogue, and nothing overlaps it when every CU holds one tile.
+    auto word = [](typename Mma16<DT>::acc_t const &c, int e) -> int {
+      if constexpr (int_acc) return (int)c[e];  // the low 32 bits: the wrap of shared.ex:190-194
+      else return (int)f32_canon_bits(c[e]);
+    };
+    const bool hi = (lane >> 3) & 1;
+    const bool lines = (N % 4) == 0 && ((uintptr_t)out & 15) == 0;
+    auto put16 = [&](int64_t gm, int64_t gn, const v4i &v) {
+      if (gm < M && gn < N) *reinterpret_cast<v4i *>((unsigned char *)out + (obase + gm * N + gn) * 4) = v;
+    };
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+      const int64_t gm = row0 + 16 * i + (lane & 15);
+#pragma unroll
+      for (int j = 0; j < TN; j += 2) {
+        const int64_t gn0 = col0 + 16 * j + 4 * (lane >> 4), gn1 = gn0 + 16;
+        v4i v, w;
+#pragma unroll
+        for (int e = 0; e < 4; e++) { v[e] = word(acc[i][j], e); w[e] = word(acc[i][j + 1], e); }
+        if (lines) {
+          v4i got;
+#pragma unroll
+          for (int e = 0; e < 4; e++) got[e] = __shfl_xor(hi ? v[e] : w[e], 8, 64);
+          put16(hi ? gm - 8 : gm, hi ? gn1 : gn0, hi ? got : v);  // rows 0..7 of the 16, both tiles
+          put16(hi ? gm : gm + 8, hi ? gn1 : gn0, hi ? w : got);  // rows 8..15
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            if (gm < M && gn0 + e < N) *reinterpret_cast<int *>((unsigned char *)out + (obase + gm * N + gn0 + e) * 4) = v[e];
+            if (gm < M && gn1 + e < N) *reinterpret_cast<int *>((unsigned char *)out + (obase + gm * N + gn1 + e) * 4) = w[e];
           }
         }
       }
