@@ -143,9 +143,20 @@ void *hipnx_buf_device_ptr(const hipnx_buf *buf);
 /* replaces: from_pointer/5 for a :local pointer (nx/lib/nx/backend.ex:59-65;
  * exla/lib/exla/backend.ex:133-181, exla/c_src/exla/exla.cc:387-437): a handle over `bytes` of
  * device memory of this context's device that someone else owns.  Freeing or destroying the
- * handle never frees the memory; the owner keeps it alive while the handle is used.  The :ipc
- * kind of pointer (a handle another process opens) is not built. */
+ * handle never frees the memory; the owner keeps it alive while the handle is used. */
 int hipnx_buf_wrap(hipnx_ctx *ctx, void *device_ptr, size_t bytes, hipnx_buf **out);
+/* replaces: to_pointer/2 with mode :ipc and from_pointer/5 for an :ipc pointer (nx/lib/nx/pointer.ex:8-15;
+ * exla/lib/exla/backend.ex:85-181; exla/c_src/exla/exla_cuda.cc:11-52 -- cudaIpcGetMemHandle /
+ * cudaIpcOpenMemHandle there, hipIpcGetMemHandle / hipIpcOpenMemHandle here).  `export` waits for the
+ * work enqueued so far and writes the HIPNX_IPC_HANDLE_BYTES bytes another PROCESS on the same machine
+ * opens with `import` (on the device with the same index); the buffer must own its memory (not a
+ * wrapped or imported one) and hold less than 2 GiB.  `import` gives a handle over the exporter's
+ * memory; destroying it closes the mapping and never frees the memory, which the exporter keeps alive
+ * while the importer uses it.  Opening a handle in the process that exported it is an error of the
+ * HIP runtime and is reported as such. */
+#define HIPNX_IPC_HANDLE_BYTES 64
+int hipnx_buf_ipc_export(hipnx_ctx *ctx, const hipnx_buf *buf, void *handle_out);
+int hipnx_buf_ipc_import(hipnx_ctx *ctx, const void *handle, size_t bytes, hipnx_buf **out);
 int hipnx_h2d(hipnx_ctx *ctx, hipnx_buf *dst, size_t dst_offset, const void *src, size_t bytes);
 /* waits for all work enqueued so far, then copies */
 int hipnx_d2h(hipnx_ctx *ctx, const hipnx_buf *src, size_t src_offset, void *dst, size_t bytes);

@@ -54,6 +54,7 @@ FUSED_FLAG_SWAP, FUSED_FLAG_INT = 1, 2
 FUSED_SRC_CONST, FUSED_SRC_INPUT, FUSED_SRC_SAVED = range(3)
 FUSED_SAVED, FUSED_MAX_INSTR, FUSED_MAX_INPUTS = 3, 32, 8
 FUSED_INTERPRETED, FUSED_COMPILED = 0, 1
+IPC_HANDLE_BYTES = 64
 SCALE_NONE, SCALE_PER_COLUMN, SCALE_PER_ROW, SCALE_ONE = range(4)
 
 _ctx_p, _buf_p = C.c_void_p, C.c_void_p
@@ -79,6 +80,8 @@ PROTOTYPES = {
     "hipnx_buf_size": [_buf_p, C.POINTER(C.c_size_t)],
     "hipnx_buf_device_ptr": [_buf_p],
     "hipnx_buf_wrap": [_ctx_p, C.c_void_p, C.c_size_t, C.POINTER(_buf_p)],
+    "hipnx_buf_ipc_export": [_ctx_p, _buf_p, C.c_void_p],
+    "hipnx_buf_ipc_import": [_ctx_p, C.c_void_p, C.c_size_t, C.POINTER(_buf_p)],
     "hipnx_h2d": [_ctx_p, _buf_p, C.c_size_t, C.c_void_p, C.c_size_t],
     "hipnx_d2h": [_ctx_p, _buf_p, C.c_size_t, C.c_void_p, C.c_size_t],
     "hipnx_d2d": [_ctx_p, _buf_p, C.c_size_t, _buf_p, C.c_size_t, C.c_size_t],

@@ -62,13 +62,16 @@ class _Ref:
     """Owns one device buffer.  Metadata-only callbacks (reshape / squeeze / bitcast) share it;
     it is deallocated when the last sharer is, or by the garbage collector."""
 
-    def __init__(self, ctx, nbytes: int, address=None, keep=None):
+    def __init__(self, ctx, nbytes: int, address=None, keep=None, ipc_handle=None):
         self.ctx = ctx
         self.handle = C.c_void_p()
         self.nbytes = nbytes
         self.sharers = 1
         self.keep = keep  # the owner of borrowed memory, kept alive with the handle
-        if address is None:
+        if ipc_handle is not None:  # another process's device memory, opened through its IPC handle
+            raw = C.create_string_buffer(bytes(ipc_handle), L.IPC_HANDLE_BYTES)
+            L.check(L.lib.hipnx_buf_ipc_import(ctx, raw, nbytes, C.byref(self.handle)))
+        elif address is None:
             L.check(L.lib.hipnx_buf_alloc(ctx, nbytes, C.byref(self.handle)))
         else:  # someone else's device memory: the handle never frees it
             L.check(L.lib.hipnx_buf_wrap(ctx, C.c_void_p(address), nbytes, C.byref(self.handle)))
@@ -755,17 +758,21 @@ class HipNxBackend:
     @classmethod
     def to_pointer(cls, t: Tensor, opts=None):
         """to_pointer/2 (backend.ex:66; semantics of exla/lib/exla/backend.ex:86-131): the device
-        address of the tensor's buffer as a `Pointer` of kind "local".  The "ipc" kind -- a handle
-        for another process -- is not built."""
+        address of the tensor's buffer as a `Pointer` of kind "local", or with `mode: :ipc` a handle
+        another process on the machine opens with `from_pointer` (kind "ipc": `handle` = the 64 bytes of
+        the HIP IPC handle, `address` = the device index, as EXLA's cuda client fills them)."""
         opts = dict(opts or {})
         mode = opts.pop("mode", "local")
+        opts.pop("permissions", None)  # host shared-memory permissions of EXLA's host client: nothing to set here
         if opts:
             raise ValueError(f"unknown options {sorted(opts)!r}")
-        if mode == "ipc":
-            raise NotImplementedError("HipNx.Backend.to_pointer: the :ipc mode is not built, only :local")
-        if mode != "local":
+        if mode not in ("local", "ipc"):
             raise ValueError(f"expected one of :local, :ipc, got: {mode!r}")
         from .nx import Pointer
+        if mode == "ipc":
+            raw = C.create_string_buffer(L.IPC_HANDLE_BYTES)
+            L.check(L.lib.hipnx_buf_ipc_export(t.data.ref.ctx, cls._handle(t), raw))
+            return Pointer(kind="ipc", address=t.data.device, data_size=t.size * T.size_bytes(t.type), handle=raw.raw)
         address = L.lib.hipnx_buf_device_ptr(cls._handle(t))
         return Pointer(kind="local", address=int(address), data_size=t.size * T.size_bytes(t.type))
 
@@ -779,8 +786,13 @@ class HipNxBackend:
         size = prod(shape) * T.size_bytes(ty)
         if pointer.data_size != size:
             raise ValueError(f"invalid pointer data_size for shape, expected: {size}, got: {pointer.data_size}")
+        if pointer.kind == "ipc":
+            if pointer.handle is None or len(pointer.handle) != L.IPC_HANDLE_BYTES:
+                raise ValueError(f"an :ipc pointer carries a handle of {L.IPC_HANDLE_BYTES} bytes")
+            ref = _Ref(_Context.get(backend_opts["device"]), size, ipc_handle=pointer.handle)
+            return Tensor(cls(ref, backend_opts["device"]), ty, tuple(shape), tuple(opts.get("names") or ()))
         if pointer.kind != "local":
-            raise NotImplementedError("HipNx.Backend.from_pointer: only pointers of kind :local are built")
+            raise ValueError(f"expected a pointer of kind :local or :ipc, got: {pointer.kind!r}")
         ref = _Ref(_Context.get(backend_opts["device"]), size, address=pointer.address, keep=opts.get("keep"))
         return Tensor(cls(ref, backend_opts["device"]), ty, tuple(shape), tuple(opts.get("names") or ()))
 

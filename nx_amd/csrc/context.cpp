@@ -395,7 +395,13 @@ int hipnx_buf_free(hipnx_buf *buf) {
   hipnx_ctx *ctx = buf->ctx;
   Enter in(ctx);
   if (in.status) return in.status;
-  int st = buf->borrowed ? HIPNX_OK : pool_free(ctx, buf->ptr, buf->capacity);
+  int st = HIPNX_OK;
+  if (buf->ipc) {  // work that uses the mapping may still be running: wait, then close it
+    (void)hipStreamSynchronize(ctx->stream);
+    if (hipIpcCloseMemHandle(buf->ptr) != hipSuccess) (void)hipGetLastError();
+  } else if (!buf->borrowed) {
+    st = pool_free(ctx, buf->ptr, buf->capacity);
+  }
   buf->ptr = nullptr;
   return st;
 }
@@ -418,6 +424,42 @@ int hipnx_buf_wrap(hipnx_ctx *ctx, void *device_ptr, size_t bytes, hipnx_buf **o
   b->bytes = bytes;
   b->capacity = bytes;
   b->borrowed = true;
+  *out = b;
+  return HIPNX_OK;
+}
+
+int hipnx_buf_ipc_export(hipnx_ctx *ctx, const hipnx_buf *buf, void *handle_out) {
+  Enter in(ctx);
+  if (in.status) return in.status;
+  if (!handle_out) return set_error(HIPNX_EINVAL, "ipc_export: null handle");
+  if (int st = check_buf(ctx, buf, 0, "ipc_export")) return st;
+  HIPNX_NOT_CAPTURING(ctx, "ipc_export");
+  if (buf->borrowed) return set_error(HIPNX_EUNSUPPORTED, "ipc_export: the buffer wraps memory it does not own");
+  if (buf->capacity >= (1ull << 31)) return set_error(HIPNX_EUNSUPPORTED, "ipc_export: allocations of 2 GiB or more are not shared");
+  static_assert(sizeof(hipIpcMemHandle_t) == HIPNX_IPC_HANDLE_BYTES, "handle size of the public header");
+  hipIpcMemHandle_t h;
+  HIPNX_HIP(hipIpcGetMemHandle(&h, buf->ptr));
+  HIPNX_HIP(hipStreamSynchronize(ctx->stream));  // the other process sees what has been written so far
+  std::memcpy(handle_out, &h, sizeof h);
+  return deferred_error(ctx);
+}
+
+int hipnx_buf_ipc_import(hipnx_ctx *ctx, const void *handle, size_t bytes, hipnx_buf **out) {
+  Enter in(ctx);
+  if (in.status) return in.status;
+  if (!handle || !out) return set_error(HIPNX_EINVAL, "ipc_import: null argument");
+  if (bytes >= (1ull << 31)) return set_error(HIPNX_EUNSUPPORTED, "ipc_import: allocations of 2 GiB or more are not shared");
+  hipIpcMemHandle_t h;
+  std::memcpy(&h, handle, sizeof h);
+  void *ptr = nullptr;
+  HIPNX_HIP(hipIpcOpenMemHandle(&ptr, h, hipIpcMemLazyEnablePeerAccess));
+  hipnx_buf *b = new hipnx_buf;
+  b->ctx = ctx;
+  b->ptr = ptr;
+  b->bytes = bytes;
+  b->capacity = bytes;
+  b->borrowed = true;
+  b->ipc = true;
   *out = b;
   return HIPNX_OK;
 }

@@ -58,6 +58,7 @@ struct hipnx_buf {
   size_t capacity = 0;  // what the pool block holds
   std::atomic<int> freed{0};
   bool borrowed = false;  // wraps memory owned by someone else: never returned to the pool
+  bool ipc = false;       // borrowed through an IPC handle of another process: closed on release
 };
 
 namespace hipnx {
