@@ -224,8 +224,12 @@ class HipNxBackend:
         if out.shape == ():
             key = (opts["device"], out.type, elem)
             ref = cls._scalar_cache.get(key)
-            if ref is None and opts["device"] in _capturing:
-                # written only when the captured graph replays: must not be shared with eager code
+            if opts["device"] in _capturing:
+                # While capturing, a constant is always the graph's own: allocated and filled inside the
+                # capture (the block belongs to the graph, the fill is replayed with it).  A cached block
+                # would be referenced by address only -- once the cache lets go of it (it is cleared after
+                # 1024 distinct numbers) the pool hands it to someone else and every later replay reads
+                # what they wrote.
                 res = cls._alloc(out, opts["device"])
                 L.check(L.lib.hipnx_fill(res.data.ref.ctx, res.data.ref.handle, len(elem), elem, 1))
                 return res

@@ -383,6 +383,30 @@ static ERL_NIF_TERM nif_wrap(ErlNifEnv *env, int argc, const ERL_NIF_TERM argv[]
   return ok(env, make_buf(env, buf));
 }
 
+/* ipc_export(ctx, buf) -> {:ok, handle_binary}: the :ipc pointer of to_pointer/2 (64 bytes another OS
+ * process opens with ipc_import) */
+static ERL_NIF_TERM nif_ipc_export(ErlNifEnv *env, int argc, const ERL_NIF_TERM argv[]) {
+  (void)argc;
+  GET_CTX(0, ctx); GET_BUF(1, buf);
+  ERL_NIF_TERM term;
+  unsigned char *dst = enif_make_new_binary(env, HIPNX_IPC_HANDLE_BYTES, &term);
+  CHECK(hipnx_buf_ipc_export(ctx, buf, dst));
+  return ok(env, term);
+}
+
+/* ipc_import(ctx, handle_binary, nbytes): from_pointer/5 for an :ipc pointer; the memory stays with the
+ * exporting process, destroying the buffer closes the mapping */
+static ERL_NIF_TERM nif_ipc_import(ErlNifEnv *env, int argc, const ERL_NIF_TERM argv[]) {
+  (void)argc;
+  GET_CTX(0, ctx);
+  ErlNifBinary handle;
+  if (!enif_inspect_binary(env, argv[1], &handle) || handle.size != HIPNX_IPC_HANDLE_BYTES) return enif_make_badarg(env);
+  GET_I64(2, nbytes);
+  hipnx_buf *buf;
+  CHECK(hipnx_buf_ipc_import(ctx, handle.data, (size_t)nbytes, &buf));
+  return ok(env, make_buf(env, buf));
+}
+
 static ERL_NIF_TERM nif_sync(ErlNifEnv *env, int argc, const ERL_NIF_TERM argv[]) {
   (void)argc;
   GET_CTX(0, ctx);
@@ -410,7 +434,8 @@ static ErlNifFunc funcs[] = {
     {"select", 13, nif_select, IO},             {"clip", 10, nif_clip, IO},
     {"strided_copy", 9, nif_strided_copy, IO},  {"iota", 6, nif_iota, IO},
     {"narrow_int", 5, nif_narrow_int, IO},      {"device_ptr", 1, nif_device_ptr, 0},
-    {"wrap", 3, nif_wrap, 0},
+    {"wrap", 3, nif_wrap, 0},                   {"ipc_export", 2, nif_ipc_export, IO},
+    {"ipc_import", 3, nif_ipc_import, IO},
     {"eye", 6, nif_eye, IO},                    {"threefry2x32", 4, nif_threefry2x32, IO},
     {"sync", 1, nif_sync, IO}};
 

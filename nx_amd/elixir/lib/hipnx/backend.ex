@@ -59,6 +59,16 @@ defmodule HipNx.Backend do
 
   defp unwrap!({:ok, value}), do: value
   defp unwrap!({:error, {status, msg}}) when status in [2, 6], do: raise(ArgumentError, List.to_string(msg))
+
+  # HIPNX_ERAISED: what a kernel issued earlier met (the reference raises for it at once; a device
+  # cannot, so the next call that waits for the device -- to_binary, inspect, backend_copy -- does)
+  defp unwrap!({:error, {8, msg}}) do
+    case List.to_string(msg) do
+      "ArithmeticError: " <> rest -> raise(ArithmeticError, rest)
+      "ArgumentError: " <> rest -> raise(ArgumentError, rest)
+      other -> raise(RuntimeError, "HipNx: " <> other)
+    end
+  end
   defp unwrap!({:error, {_status, msg}}), do: raise(RuntimeError, "HipNx: " <> List.to_string(msg))
 
   defp dt(type), do: Map.get(@dtypes, type) || raise(ArgumentError, "HipNx does not support type #{inspect(type)}")
@@ -648,16 +658,23 @@ defmodule HipNx.Backend do
     end
   end
 
-  ## Pointers (the :local kind; cf. EXLA.Backend.to_pointer/2 and from_pointer/5)
+  ## Pointers (cf. EXLA.Backend.to_pointer/2 and from_pointer/5, exla/lib/exla/backend.ex:85-181)
 
   @impl true
-  def to_pointer(%T{data: %__MODULE__{ref: ref}} = t, opts) do
-    opts = Keyword.validate!(opts, mode: :local)
+  def to_pointer(%T{data: %__MODULE__{ref: ref, device: device}} = t, opts) do
+    opts = Keyword.validate!(opts, mode: :local, permissions: 0o400)
 
     case opts[:mode] do
-      :local -> %Nx.Pointer{kind: :local, address: unwrap!(NIF.device_ptr(ref)), data_size: bytes(t)}
-      :ipc -> raise ArgumentError, "HipNx.Backend.to_pointer/2: the :ipc mode is not built, only :local"
-      mode -> raise ArgumentError, "expected one of :local, :ipc, got: #{inspect(mode)}"
+      :local ->
+        %Nx.Pointer{kind: :local, address: unwrap!(NIF.device_ptr(ref)), data_size: bytes(t)}
+
+      :ipc ->
+        # the 64 bytes of the HIP IPC handle; address carries the device index, as EXLA's cuda client does
+        handle = unwrap!(NIF.ipc_export(ctx(device), ref))
+        %Nx.Pointer{kind: :ipc, handle: handle, address: device, data_size: bytes(t)}
+
+      mode ->
+        raise ArgumentError, "expected one of :local, :ipc, got: #{inspect(mode)}"
     end
   end
 
@@ -676,8 +693,12 @@ defmodule HipNx.Backend do
         # the memory stays with its owner: deallocating this tensor never frees it
         to_nx(unwrap!(NIF.wrap(ctx(device), address, size)), device, template)
 
+      %Nx.Pointer{kind: :ipc, handle: handle} when is_binary(handle) and byte_size(handle) == 64 ->
+        # another OS process's buffer: deallocating this tensor closes the mapping, never frees the memory
+        to_nx(unwrap!(NIF.ipc_import(ctx(device), handle, size)), device, template)
+
       %Nx.Pointer{kind: :ipc} ->
-        raise ArgumentError, "HipNx.Backend.from_pointer/5: only pointers of kind :local are built"
+        raise ArgumentError, "an :ipc pointer carries a handle of 64 bytes"
     end
   end
 end

@@ -32,6 +32,8 @@ defmodule HipNx.NIF do
   def narrow_int(_ctx, _buf, _n, _bits, _signed), do: err()
   def device_ptr(_buf), do: err()
   def wrap(_ctx, _address, _nbytes), do: err()
+  def ipc_export(_ctx, _buf), do: err()
+  def ipc_import(_ctx, _handle, _nbytes), do: err()
   def threefry2x32(_ctx, _key, _n, _out_bytes), do: err()
   def sync(_ctx), do: err()
 

@@ -5,6 +5,8 @@ the tolerances of the per-op tests."""
 import numpy as np
 import pytest
 
+from nx_amd.tensor import template
+
 from nx_amd import defn
 from nx_amd import nx as Nx
 from nx_amd import random as Random
@@ -128,6 +130,29 @@ def test_captured_chain_replays_with_new_inputs(name, hip):
         want = hip.to_numpy(compiled(*fresh)).copy()
         np.testing.assert_array_equal(hip.to_numpy(captured(*fresh)), want, f"{name}: replay with new inputs")
         np.testing.assert_array_equal(hip.to_numpy(captured(*args)), eager, f"{name}: and back")
+    finally:
+        captured.destroy()
+
+
+def test_captured_constants_survive_the_scalar_cache(hip):
+    """A constant met while capturing is the graph's own block, filled inside the capture -- also when the
+    eager warm-up has left the same number in the backend's scalar cache.  After more than 1024 other
+    scalars have passed through that cache (it is cleared, its blocks go back to the pool and are
+    overwritten), a replay still multiplies by 0.5."""
+    x_np = np.linspace(-3, 3, 4096, dtype=np.float32)
+    x = from_numpy(x_np, "f32", hip)
+    compiled = defn.compile(lambda t: Nx.add(Nx.multiply(t, 0.5), 0.25), x)
+    want = hip.to_numpy(compiled(x)).copy()  # the warm-up: 0.5 and 0.25 are now cached scalars
+    captured = compiled.capture(x)
+    try:
+        np.testing.assert_array_equal(hip.to_numpy(captured(x)), want)
+        keep = []
+        for i in range(1100):  # distinct scalars: the cache overflows and is cleared
+            keep.append(Nx.multiply(x, 1.0 + i / 4096.0))
+        del keep
+        junk = [hip.constant(template("f32", ()), 1000.0 + i, {}) for i in range(64)]  # take the freed small blocks
+        np.testing.assert_array_equal(hip.to_numpy(captured(x)), want, "replay after the cache was cleared")
+        del junk
     finally:
         captured.destroy()
 
