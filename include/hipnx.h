@@ -60,7 +60,11 @@ enum {
 enum {
   HIPNX_U8 = 0, HIPNX_U16 = 1, HIPNX_U32 = 2, HIPNX_U64 = 3,
   HIPNX_S8 = 4, HIPNX_S16 = 5, HIPNX_S32 = 6, HIPNX_S64 = 7,
-  HIPNX_F16 = 8, HIPNX_BF16 = 9, HIPNX_F32 = 10, HIPNX_F64 = 11, HIPNX_NTYPES = 12
+  HIPNX_F16 = 8, HIPNX_BF16 = 9, HIPNX_F32 = 10, HIPNX_F64 = 11, HIPNX_NTYPES = 12,
+  /* OUTPUT ONLY, accepted as out_dt by hipnx_as_type and hipnx_dot: bf16 encoded with round-to-nearest-even,
+   * as Torchx and EXLA do (torchx/test/torchx/nx_test.exs:380-394 expects 1/5 -> 0.2001953125), instead of
+   * Nx.BinaryBackend's truncation (shared.ex:136-152).  The buffer holds ordinary bf16. */
+  HIPNX_BF16_RNE = 12
 };
 
 /* element-wise binary callbacks, in the order of nx/lib/nx/binary_backend.ex:649-653 */

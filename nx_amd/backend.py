@@ -32,6 +32,14 @@ RED_SUM, RED_MAX, RED_MIN, RED_PRODUCT, RED_ALL, RED_ANY = 0, 1, 2, 3, 4, 5
 K_INNER, K_OUTER = 0, 1
 OOB_RAISE, OOB_CLAMP, OOB_DEFER = 0, 1, 2
 _bounds = {"policy": OOB_RAISE}
+BF16_RNE = 12  # HIPNX_BF16_RNE: output-only type code of as_type and dot
+_bf16 = {"rounding": "truncate"}
+
+
+def _out_code(t) -> int:
+    """The type code `as_type` and `dot` pass for their result."""
+    c = T.code(t)
+    return BF16_RNE if c == T.BF16 and _bf16["rounding"] == "nearest_even" else c
 
 # callbacks of the behaviour that are not on the device path (nx/lib/nx/backend.ex:58-144)
 UNSUPPORTED = ["conv", "window_sum", "window_product",
@@ -351,7 +359,7 @@ class HipNxBackend:
         if t.type == out.type:
             return t
         res = cls._alloc(out, dev)
-        L.check(L.lib.hipnx_as_type(res.data.ref.ctx, T.code(t.type), T.code(out.type), out.size, cls._handle(t),
+        L.check(L.lib.hipnx_as_type(res.data.ref.ctx, T.code(t.type), _out_code(out.type), out.size, cls._handle(t),
                                     res.data.ref.handle))
         if out.type[1] < 8:
             res = cls._narrow(res)
@@ -474,7 +482,7 @@ class HipNxBackend:
         lt, l_layout, M = cls._dot_operand(l, c1s, nb)
         rt, r_layout, N = cls._dot_operand(r, c2s, nb)
         res = cls._alloc(out, dev)
-        L.check(L.lib.hipnx_dot(res.data.ref.ctx, T.code(l.type), T.code(r.type), T.code(out.type), batch, M, N, K,
+        L.check(L.lib.hipnx_dot(res.data.ref.ctx, T.code(l.type), T.code(r.type), _out_code(out.type), batch, M, N, K,
                                 l_layout, r_layout, cls._handle(lt), cls._handle(rt), res.data.ref.handle))
         return cls._narrow(res) if out.type[1] < 8 else res
 
@@ -986,6 +994,19 @@ def bounds_policy(policy: str) -> str:
         raise ValueError(f"expected one of {sorted(names)!r}, got: {policy!r}")
     previous = next(k for k, v in names.items() if v == _bounds["policy"])
     _bounds["policy"] = names[policy]
+    return previous
+
+
+def bf16_rounding(mode: str) -> str:
+    """How `as_type` and `dot` encode a bf16 result from now on; returns the previous setting.
+    "truncate" (the default) drops the low 16 bits of the f32 value as `Nx.BinaryBackend` does
+    (nx/lib/nx/shared.ex:136-152); "nearest_even" rounds as Torchx and EXLA do
+    (torchx/test/torchx/nx_test.exs:380-394 expects 1/5 -> 0.2001953125).  Element-wise results keep the
+    reference backend's truncation under either setting."""
+    if mode not in ("truncate", "nearest_even"):
+        raise ValueError(f'expected "truncate" or "nearest_even", got: {mode!r}')
+    previous = _bf16["rounding"]
+    _bf16["rounding"] = mode
     return previous
 
 

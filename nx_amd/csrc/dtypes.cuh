@@ -35,6 +35,11 @@ __device__ __forceinline__ uint16_t f32_to_bf16_bits_trunc(float f) {
   uint32_t b = __float_as_uint(f);
   return (f != f) ? (uint16_t)0x7FC0 : (uint16_t)(b >> 16);
 }
+// round-to-nearest-even to bf16 (the HIPNX_BF16_RNE output code)
+__device__ __forceinline__ uint16_t f32_to_bf16_bits_rne(float f) {
+  uint32_t b = __float_as_uint(f);
+  return (f != f) ? (uint16_t)0x7FC0 : (uint16_t)((b + 0x7FFFu + ((b >> 16) & 1u)) >> 16);
+}
 __device__ __forceinline__ uint32_t f32_canon_bits(float f) { return (f != f) ? 0x7FC00000u : __float_as_uint(f); }
 __device__ __forceinline__ uint64_t f64_canon_bits(double d) {
   return (d != d) ? 0x7FF8000000000000ull : (uint64_t)__double_as_longlong(d);
@@ -60,6 +65,9 @@ __device__ __forceinline__ float f64_to_f32_round_odd(double d) {
   if ((double)f != d && (b & 0x7F800000u) != 0x7F800000u) b |= 1u;
   return __uint_as_float(b);
 }
+// one rounding of the f64 value: round-to-odd keeps 24 significant bits, more than the 8 + 2 that make
+// the second rounding exact
+__device__ __forceinline__ uint16_t f64_to_bf16_bits_rne(double d) { return f32_to_bf16_bits_rne(f64_to_f32_round_odd(d)); }
 __device__ __forceinline__ uint16_t f64_to_f16_bits(double d) {
   return (d != d) ? (uint16_t)0x7E00 : f16_bits((f16_t)f64_to_f32_round_odd(d));
 }
@@ -75,6 +83,7 @@ struct conv<float> {
   static __device__ __forceinline__ float from_f64(double v) { return (float)v; }
   static __device__ __forceinline__ float from_f32(float v) { return v; }
   static __device__ __forceinline__ uint16_t to_bf16(float v) { return f32_to_bf16_bits_trunc(v); }
+  static __device__ __forceinline__ uint16_t to_bf16_rne(float v) { return f32_to_bf16_bits_rne(v); }
   static __device__ __forceinline__ uint16_t to_f16(float v) { return f32_to_f16_bits(v); }
   static __device__ __forceinline__ uint32_t to_f32(float v) { return f32_canon_bits(v); }
   static __device__ __forceinline__ uint64_t to_f64(float v) { return f64_canon_bits((double)v); }
@@ -87,6 +96,7 @@ struct conv<double> {
   static __device__ __forceinline__ double from_f64(double v) { return v; }
   static __device__ __forceinline__ double from_f32(float v) { return (double)v; }
   static __device__ __forceinline__ uint16_t to_bf16(double v) { return f32_to_bf16_bits_trunc((float)v); }
+  static __device__ __forceinline__ uint16_t to_bf16_rne(double v) { return f64_to_bf16_bits_rne(v); }
   static __device__ __forceinline__ uint16_t to_f16(double v) { return f64_to_f16_bits(v); }
   static __device__ __forceinline__ uint32_t to_f32(double v) { return f32_canon_bits((float)v); }
   static __device__ __forceinline__ uint64_t to_f64(double v) { return f64_canon_bits(v); }
@@ -98,6 +108,7 @@ struct conv<int64_t> {  // also carries u64 bit patterns
   static __device__ __forceinline__ int64_t from_f64(double v) { return (int64_t)v; }
   static __device__ __forceinline__ int64_t from_f32(float v) { return (int64_t)v; }
   static __device__ __forceinline__ uint16_t to_bf16(int64_t v) { return f32_to_bf16_bits_trunc((float)(double)v); }
+  static __device__ __forceinline__ uint16_t to_bf16_rne(int64_t v) { return f64_to_bf16_bits_rne((double)v); }
   static __device__ __forceinline__ uint16_t to_f16(int64_t v) { return f64_to_f16_bits((double)v); }
   static __device__ __forceinline__ uint32_t to_f32(int64_t v) { return __float_as_uint((float)(double)v); }
   static __device__ __forceinline__ uint64_t to_f64(int64_t v) { return (uint64_t)__double_as_longlong((double)v); }
@@ -193,13 +204,15 @@ __device__ __forceinline__ void store_vec(void *__restrict__ p, int dt, int64_t 
     case HIPNX_U16:
     case HIPNX_S16:
     case HIPNX_F16:
-    case HIPNX_BF16: {
+    case HIPNX_BF16:
+    case HIPNX_BF16_RNE: {
       raw_vec<2 * E> r;
       uint16_t *h = reinterpret_cast<uint16_t *>(r.b);
 #pragma unroll
       for (int i = 0; i < E; i++) {
         if (dt == HIPNX_F16) h[i] = conv<CT>::to_f16(v[i]);
         else if (dt == HIPNX_BF16) h[i] = conv<CT>::to_bf16(v[i]);
+        else if (dt == HIPNX_BF16_RNE) h[i] = conv<CT>::to_bf16_rne(v[i]);
         else h[i] = (uint16_t)conv<CT>::to_int(v[i]);
       }
       *reinterpret_cast<raw_vec<2 * E> *>((uint16_t *)p + idx) = r;

@@ -393,10 +393,10 @@ extern "C" int hipnx_as_type(hipnx_ctx *ctx, int in_dt, int out_dt, int64_t n, c
                              hipnx_buf *out) {
   Enter in(ctx);
   if (in.status) return in.status;
-  if (dtype_size(in_dt) < 0 || dtype_size(out_dt) < 0 || n < 0)
+  if (dtype_size(in_dt) < 0 || out_dtype_size(out_dt) < 0 || n < 0)
     return set_error(HIPNX_EINVAL, "as_type: unknown element type or negative size");
   if (int st = check_buf(ctx, inb, (uint64_t)n * dtype_size(in_dt), "as_type in")) return st;
-  if (int st = check_buf(ctx, out, (uint64_t)n * dtype_size(out_dt), "as_type out")) return st;
+  if (int st = check_buf(ctx, out, (uint64_t)n * out_dtype_size(out_dt), "as_type out")) return st;
   if (n == 0) return HIPNX_OK;
   static const int64_t tmax[8] = {0xFF, 0xFFFF, 0xFFFFFFFFll, -1ll /* u64 max */, 0x7F, 0x7FFF, 0x7FFFFFFFll,
                                   0x7FFFFFFFFFFFFFFFll};

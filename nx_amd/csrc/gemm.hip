@@ -175,14 +175,14 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
   {
     Enter in(ctx);
     if (in.status) return in.status;
-    if (dtype_size(l_dt) < 0 || dtype_size(r_dt) < 0 || dtype_size(out_dt) < 0)
+    if (dtype_size(l_dt) < 0 || dtype_size(r_dt) < 0 || out_dtype_size(out_dt) < 0)
       return set_error(HIPNX_EINVAL, "dot: unknown element type");
     if (batch < 0 || M < 0 || N < 0 || K < 0) return set_error(HIPNX_EINVAL, "dot: negative extent");
     if ((l_layout != HIPNX_K_INNER && l_layout != HIPNX_K_OUTER) || (r_layout != HIPNX_K_INNER && r_layout != HIPNX_K_OUTER))
       return set_error(HIPNX_EINVAL, "dot: unknown operand layout");
     if (int st = check_buf(ctx, l, (uint64_t)batch * M * K * dtype_size(l_dt), "dot lhs")) return st;
     if (int st = check_buf(ctx, r, (uint64_t)batch * N * K * dtype_size(r_dt), "dot rhs")) return st;
-    if (int st = check_buf(ctx, out, (uint64_t)batch * M * N * dtype_size(out_dt), "dot out")) return st;
+    if (int st = check_buf(ctx, out, (uint64_t)batch * M * N * out_dtype_size(out_dt), "dot out")) return st;
     if (batch * M * N == 0) return HIPNX_OK;
     if (batch > 65535) return set_error(HIPNX_EUNSUPPORTED, "dot: more than 65535 batch items");
 
@@ -244,7 +244,7 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
     // the lock was dropped for the re-layout above: the operands may have been freed meanwhile
     if (!st) st = check_buf(ctx, l, (uint64_t)batch * M * K * dtype_size(l_dt), "dot lhs");
     if (!st) st = check_buf(ctx, r, (uint64_t)batch * N * K * dtype_size(r_dt), "dot rhs");
-    if (!st) st = check_buf(ctx, out, (uint64_t)batch * M * N * dtype_size(out_dt), "dot out");
+    if (!st) st = check_buf(ctx, out, (uint64_t)batch * M * N * out_dtype_size(out_dt), "dot out");
     if (!st && scale_mode != HIPNX_SCALE_NONE) st = check_buf(ctx, scale, 4, "dot_scaled scale");
     if (!st) {
       const void *lp = lt ? lt->ptr : l->ptr, *rp = rt ? rt->ptr : r->ptr;

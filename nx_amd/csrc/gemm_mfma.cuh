@@ -397,7 +397,7 @@ __device__ __forceinline__ void gemm_epilogue(typename Mma16<DT>::acc_t (&acc)[T
       }
     }
   } else if constexpr (int_acc != int_out) return;  // the host never pairs them
-  else if constexpr (!int_acc && (ODT == HIPNX_BF16 || ODT == HIPNX_F16) && TN % 2 == 0) {
+  else if constexpr (!int_acc && (ODT == HIPNX_BF16 || ODT == HIPNX_BF16_RNE || ODT == HIPNX_F16) && TN % 2 == 0) {
     // 2-byte outputs: a lane's 4 outputs of a tile are only 8 bytes, and a store instruction made of
     // 32-byte runs per row is slow (measured on the 4096^3 bf16 case: 11 us of the kernel, twice the
     // time the s32 epilogue takes for twice the bytes).  Two neighbouring column tiles are written
@@ -408,6 +408,7 @@ __device__ __forceinline__ void gemm_epilogue(typename Mma16<DT>::acc_t (&acc)[T
     const int64_t gc = col0 + 4 * ((lane >> 4) & 2);  // first of this lane's 8 columns within its tile
     auto pack = [](float lo, float hi) -> uint32_t {
       if constexpr (ODT == HIPNX_BF16) return (uint32_t)f32_to_bf16_bits_trunc(lo) | ((uint32_t)f32_to_bf16_bits_trunc(hi) << 16);
+      else if constexpr (ODT == HIPNX_BF16_RNE) return (uint32_t)f32_to_bf16_bits_rne(lo) | ((uint32_t)f32_to_bf16_bits_rne(hi) << 16);
       else return (uint32_t)f32_to_f16_bits(lo) | ((uint32_t)f32_to_f16_bits(hi) << 16);
     };
     // N % 8 == 0: a group of 8 columns lies wholly inside or outside, and row starts keep the 16-byte alignment
@@ -766,7 +767,7 @@ gemm_pipelined_kernel(GemmArgs a) {
   const int64_t obase = b * a.M * a.N;
   switch (a.odt) {
 #define HIPNX_EPI(T) case T: gemm_epilogue<DT, T, TM16, TN16>(acc, a.out, obase, a.M, a.N, m0 + wm, n0 + wn, lane, a.scale, a.scale_mode); break;
-    HIPNX_EPI(HIPNX_BF16) HIPNX_EPI(HIPNX_F16) HIPNX_EPI(HIPNX_F32) HIPNX_EPI(HIPNX_F64)
+    HIPNX_EPI(HIPNX_BF16) HIPNX_EPI(HIPNX_F16) HIPNX_EPI(HIPNX_F32) HIPNX_EPI(HIPNX_F64) HIPNX_EPI(HIPNX_BF16_RNE)
     HIPNX_EPI(HIPNX_S8) HIPNX_EPI(HIPNX_U8) HIPNX_EPI(HIPNX_S16) HIPNX_EPI(HIPNX_U16)
     HIPNX_EPI(HIPNX_S32) HIPNX_EPI(HIPNX_U32) HIPNX_EPI(HIPNX_S64) HIPNX_EPI(HIPNX_U64)
 #undef HIPNX_EPI

@@ -77,6 +77,8 @@ inline int dtype_size(int dt) {
   return (dt >= 0 && dt < HIPNX_NTYPES) ? sz[dt] : -1;
 }
 inline bool is_float(int dt) { return dt >= HIPNX_F16; }
+// output type of as_type and dot: the twelve element types and the round-to-nearest-even bf16 encoding
+inline int out_dtype_size(int dt) { return dt == HIPNX_BF16_RNE ? 2 : dtype_size(dt); }
 inline bool is_unsigned(int dt) { return dt >= 0 && dt <= HIPNX_U64; }
 inline bool is_wide(int dt) {  // not exactly representable in f32
   return dt == HIPNX_U32 || dt == HIPNX_U64 || dt == HIPNX_S32 || dt == HIPNX_S64 || dt == HIPNX_F64;

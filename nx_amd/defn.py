@@ -504,6 +504,10 @@ def _fusable(t: Tensor) -> bool:
         return out_ok and all(value_ok(a, op) for a in args)
     if op == "as_type":
         src = args[0].type
+        if t.type == ("bf", 16):
+            from .backend import _bf16
+            if _bf16["rounding"] != "truncate":
+                return False  # only the separate kernel rounds to nearest even (the setting when the function is compiled counts)
         return t.type in _NARROW and (src in _NARROW or (T.is_integer(src) and src[1] <= 32)) and _const(args[0]) is None
     if op == "select":
         pred, on_true, on_false = args

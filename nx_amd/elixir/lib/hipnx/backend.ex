@@ -72,6 +72,14 @@ defmodule HipNx.Backend do
   defp unwrap!({:error, {_status, msg}}), do: raise(RuntimeError, "HipNx: " <> List.to_string(msg))
 
   defp dt(type), do: Map.get(@dtypes, type) || raise(ArgumentError, "HipNx does not support type #{inspect(type)}")
+
+  # The result type of as_type and dot.  `config :hipnx, bf16_rounding: :nearest_even` encodes bf16 results
+  # as Torchx and EXLA do (HIPNX_BF16_RNE = 12); the default truncates as Nx.BinaryBackend does.
+  defp out_dt({:bf, 16}) do
+    if Application.get_env(:hipnx, :bf16_rounding, :truncate) == :nearest_even, do: 12, else: dt({:bf, 16})
+  end
+
+  defp out_dt(type), do: dt(type)
   defp bytes(%T{type: {_, bits}, shape: shape}), do: max(div(bits, 8), 1) * Nx.size(shape)
 
   # a result of a sub-byte type was computed at 8 bits: keep its low bits (Nx.Shared's `<<x::size(bits)>>`)
@@ -240,7 +248,11 @@ defmodule HipNx.Backend do
 
   @impl true
   def as_type(%T{type: type}, %T{type: type} = t), do: t
-  def as_type(out, t), do: unary(-1, out, t)
+  def as_type(out, %T{} = t) do
+    device = device_of([t])
+    {ref, _} = from_nx(t, device)
+    to_nx(unwrap!(NIF.unary(ctx(device), -1, dt(t.type), out_dt(out.type), Nx.size(out), ref, bytes(out))), device, out)
+  end
 
   ## Reductions
 
@@ -321,7 +333,7 @@ defmodule HipNx.Backend do
     {rref, _} = from_nx(rt, device)
 
     ref =
-      NIF.dot(ctx(device), dt(l.type), dt(r.type), dt(out.type), batch, m, n, k, l_layout, r_layout, lref, rref, bytes(out))
+      NIF.dot(ctx(device), dt(l.type), dt(r.type), out_dt(out.type), batch, m, n, k, l_layout, r_layout, lref, rref, bytes(out))
 
     to_nx(unwrap!(ref), device, out)
   end

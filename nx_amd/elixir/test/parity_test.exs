@@ -124,6 +124,21 @@ defmodule HipNx.ParityTest do
     end
   end
 
+  describe "bf16 encodings" do
+    # torchx/test/torchx/nx_test.exs:380-394 expects the nearest value; Nx.BinaryBackend truncates
+    test "1/5 truncates by default and rounds to nearest even on request" do
+      t = Nx.tensor([0.2], type: :f32, backend: @hip)
+      assert Nx.to_binary(Nx.as_type(t, :bf16)) == <<0x3E4C::16-native>>
+      Application.put_env(:hipnx, :bf16_rounding, :nearest_even)
+
+      try do
+        assert Nx.to_binary(Nx.as_type(t, :bf16)) == <<0x3E4D::16-native>>
+      after
+        Application.delete_env(:hipnx, :bf16_rounding)
+      end
+    end
+  end
+
   describe "plumbing" do
     test "deallocation is idempotent" do
       t = Nx.tensor([1, 2, 3], backend: @hip)
