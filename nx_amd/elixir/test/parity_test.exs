@@ -2,7 +2,7 @@
 # type pairs on HipNx and on Nx.BinaryBackend, both brought to the host and compared; operands that
 # live on different backends; broadcasting scalars and columns on either side.
 defmodule HipNx.ParityTest do
-  use ExUnit.Case, async: true
+  use ExUnit.Case, async: false
 
   @types [{:s, 8}, {:u, 8}, {:s, 16}, {:u, 16}, {:s, 32}, {:u, 32}, {:s, 64}, {:u, 64}, {:bf, 16}, {:f, 16}, {:f, 32}, {:f, 64}]
   @ints [{:s, 8}, {:u, 8}, {:s, 16}, {:u, 16}, {:s, 32}, {:u, 32}, {:s, 64}, {:u, 64}]
