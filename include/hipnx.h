@@ -371,9 +371,14 @@ int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_fused_instr
  * hundred milliseconds) and kept with the context -- the role exla/lib/exla/defn.ex's compilation
  * cache plays for a whole function, here for one element-wise group.  Results are bit-identical in
  * both modes.  A program first met while the context is capturing runs interpreted in that capture.
- * hipnx_fused_compiled_count reports how many programs the context holds compiled. */
+ * A program's constants are part of what it is compiled for: one whose constant changes from call to
+ * call compiles again for each value.  The context keeps at most 512 programs (another limit, at least
+ * 4: hipnx_fused_set_cache_limit); when that many are held, the next new one first waits for the stream
+ * and unloads the least recently launched quarter (those recorded into a graph stay).
+ * hipnx_fused_compiled_count reports how many the context holds. */
 enum { HIPNX_FUSED_INTERPRETED = 0, HIPNX_FUSED_COMPILED = 1 };
 int hipnx_fused_set_mode(hipnx_ctx *ctx, int mode);
+int hipnx_fused_set_cache_limit(hipnx_ctx *ctx, int programs);
 int hipnx_fused_compiled_count(hipnx_ctx *ctx, int *count);
 
 /* ---- captured sequences ---------------------------------------------------------------------

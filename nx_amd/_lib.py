@@ -108,6 +108,7 @@ PROTOTYPES = {
     "hipnx_narrow_int": [_ctx_p, _buf_p, C.c_int64, C.c_int, C.c_int],
     "hipnx_fused_set_mode": [_ctx_p, C.c_int],
     "hipnx_fused_compiled_count": [_ctx_p, C.POINTER(C.c_int)],
+    "hipnx_fused_set_cache_limit": [_ctx_p, C.c_int],
     "hipnx_threefry2x32": [_ctx_p, _buf_p, C.c_int64, _buf_p],
     "hipnx_fused_elementwise": [_ctx_p, C.c_int, C.c_void_p, C.c_int, C.POINTER(C.c_void_p), _intp, _i64p, _intp, C.c_int64,
                                 C.c_int64, C.c_int, C.c_int, _buf_p],

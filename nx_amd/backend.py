@@ -1026,6 +1026,12 @@ _fused_modes = {}  # device -> the mode last set here
 _fused_arrays = {}  # (id of a layout, input types) -> (the layout itself, so the id stays its own; C arrays of types and strides)
 
 
+def fused_cache_limit(programs: int, device: int = 0) -> None:
+    """How many compiled programs the device's context keeps (512 unless set; at least 4).  A new program
+    that finds the table full first unloads the least recently launched quarter."""
+    L.check(L.lib.hipnx_fused_set_cache_limit(_Context.get(device), programs))
+
+
 def fused_compiled_count(device: int = 0) -> int:
     count = C.c_int()
     L.check(L.lib.hipnx_fused_compiled_count(_Context.get(device), C.byref(count)))

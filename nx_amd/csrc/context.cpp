@@ -216,7 +216,7 @@ int hipnx_ctx_destroy(hipnx_ctx *ctx) {
     delete g;
   }
   ctx->graphs.clear();
-  for (auto &kv : ctx->fused_kernels) (void)hipModuleUnload(kv.second.first);
+  for (auto &kv : ctx->fused_kernels) (void)hipModuleUnload(kv.second.module);
   ctx->fused_kernels.clear();
   for (auto &kv : ctx->pool) (void)hipFree(kv.second);
   ctx->pool.clear();

@@ -8,6 +8,7 @@
 // The device headers are embedded in the library as text, so nothing is read from disk.
 #include <hip/hiprtc.h>
 
+#include <algorithm>
 #include <cstring>
 #include <functional>
 #include <string>
@@ -118,7 +119,7 @@ static std::string make_source(const FusedArgs &a, int reduce_op, bool block_per
   return s;
 }
 
-static int compile(hipnx_ctx *ctx, const std::string &src, const std::string &name, std::pair<hipModule_t, hipFunction_t> *out) {
+static int compile(hipnx_ctx *ctx, const std::string &src, const std::string &name, hipnx_ctx::FusedKernel *out) {
   hipDeviceProp_t prop;
   HIPNX_HIP(hipGetDeviceProperties(&prop, ctx->device));
   const std::string arch = std::string("--offload-arch=") + prop.gcnArchName;
@@ -140,11 +141,34 @@ static int compile(hipnx_ctx *ctx, const std::string &src, const std::string &na
   std::string code(size, '\0');
   hiprtcGetCode(prog, &code[0]);
   hiprtcDestroyProgram(&prog);
-  HIPNX_HIP(hipModuleLoadData(&out->first, code.data()));
-  hipError_t e = hipModuleGetFunction(&out->second, out->first, name.c_str());
+  HIPNX_HIP(hipModuleLoadData(&out->module, code.data()));
+  hipError_t e = hipModuleGetFunction(&out->function, out->module, name.c_str());
   if (e != hipSuccess) {
-    (void)hipModuleUnload(out->first);
+    (void)hipModuleUnload(out->module);
     return hip_fail(e, "hipModuleGetFunction(fused group)");
+  }
+  return HIPNX_OK;
+}
+
+// Makes room in a full table: waits for the stream (a kernel may still be running), then unloads the least
+// recently launched quarter.  A program specialised on a constant that changes from call to call (a
+// temperature, a learning rate passed as a number) would otherwise grow the table, and the loaded
+// modules with it, without bound; each new value still costs one compilation (a few hundred ms).
+static int trim_cache(hipnx_ctx *ctx) {
+  HIPNX_HIP(hipStreamSynchronize(ctx->stream));
+  std::vector<std::pair<uint64_t, const std::string *>> by_age;
+  for (auto &kv : ctx->fused_kernels)
+    if (!kv.second.in_graph) by_age.emplace_back(kv.second.last_use, &kv.first);
+  std::sort(by_age.begin(), by_age.end());
+  // (a limit lowered below what is held: down to under the limit)
+  const size_t over = ctx->fused_kernels.size() - ctx->fused_cache_max + 1;
+  const size_t drop = std::min(by_age.size(), std::max<size_t>(over, ctx->fused_cache_max / 4));
+  std::vector<std::string> keys;
+  for (size_t i = 0; i < drop; i++) keys.push_back(*by_age[i].second);
+  for (const std::string &k : keys) {
+    auto it = ctx->fused_kernels.find(k);
+    (void)hipModuleUnload(it->second.module);
+    ctx->fused_kernels.erase(it);
   }
   return HIPNX_OK;
 }
@@ -165,14 +189,18 @@ int fused_launch_compiled(hipnx_ctx *ctx, const FusedArgs &a, int reduce_op, boo
     char name[96];
     snprintf(name, sizeof(name), "fused_%s_%dinstr_%08zx", stages ? "stages" : reduce_op != -1 ? "map_reduce" : "map", a.n_instr,
              std::hash<std::string>{}(key) & 0xFFFFFFFFu);
-    std::pair<hipModule_t, hipFunction_t> k{};
+    if (ctx->fused_kernels.size() >= ctx->fused_cache_max)
+      if (int st = trim_cache(ctx)) return st;
+    hipnx_ctx::FusedKernel k{};
     if (int st = compile(ctx, make_source(a, reduce_op, block_per_row, name), name, &k)) return st;
     it = ctx->fused_kernels.emplace(key, k).first;
   }
+  it->second.last_use = ++ctx->fused_clock;
+  if (ctx->capture) it->second.in_graph = true;  // a recorded launch refers to the loaded module for as long as the graph lives
   // the argument block is the kernel's one by-value parameter: hand it over as the packed buffer it is
   size_t size = sizeof(FusedArgs);
   void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, (void *)&a, HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
-  HIPNX_HIP(hipModuleLaunchKernel(it->second.second, grid, 1, 1, FBLOCK, 1, 1, 0, ctx->stream, nullptr, config));
+  HIPNX_HIP(hipModuleLaunchKernel(it->second.function, grid, 1, 1, FBLOCK, 1, 1, 0, ctx->stream, nullptr, config));
   *done = true;
   return HIPNX_OK;
 }
@@ -186,6 +214,14 @@ extern "C" int hipnx_fused_set_mode(hipnx_ctx *ctx, int mode) {
   if (in.status) return in.status;
   if (mode != HIPNX_FUSED_INTERPRETED && mode != HIPNX_FUSED_COMPILED) return set_error(HIPNX_EINVAL, "fused: mode %d", mode);
   ctx->fused_mode = mode;
+  return HIPNX_OK;
+}
+
+extern "C" int hipnx_fused_set_cache_limit(hipnx_ctx *ctx, int programs) {
+  Enter in(ctx);
+  if (in.status) return in.status;
+  if (programs < 4) return set_error(HIPNX_EINVAL, "fused: a cache limit of %d programs (at least 4)", programs);
+  ctx->fused_cache_max = (size_t)programs;
   return HIPNX_OK;
 }
 

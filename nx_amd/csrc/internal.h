@@ -48,7 +48,17 @@ struct hipnx_ctx {
   std::vector<hipnx_graph *> graphs;                     // live graphs of this context
   // fused groups compiled at run time for one program each: program bytes -> loaded kernel
   int fused_mode = 0;  // 0 = the interpreting kernels, 1 = compile each distinct program once
-  std::unordered_map<std::string, std::pair<hipModule_t, hipFunction_t>> fused_kernels;
+  // compiled fused groups, keyed by what each is specialised on; at most fused_cache_max are kept (the least
+  // recently launched quarter is unloaded when the table is full; kernels recorded into a graph stay)
+  struct FusedKernel {
+    hipModule_t module;
+    hipFunction_t function;
+    uint64_t last_use;
+    bool in_graph;
+  };
+  size_t fused_cache_max = 512;  // hipnx_fused_set_cache_limit
+  std::unordered_map<std::string, FusedKernel> fused_kernels;
+  uint64_t fused_clock = 0;
 };
 
 struct hipnx_buf {

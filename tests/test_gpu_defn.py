@@ -323,6 +323,35 @@ def test_each_distinct_program_is_compiled_once(hip):
         set_mode("interpreted")
 
 
+def test_compiled_programs_are_bounded_and_the_oldest_go_first(hip):
+    """A constant is part of what a program is compiled for, so a number that changes per call makes a new
+    program each time: the table stops at its limit, and a program unloaded meanwhile compiles again."""
+    from nx_amd import backend as B
+    from nx_amd._lib import HipNxError
+    x = rand_float(np.random.default_rng(12), "f32", (32, 64), hip)
+    xs = hip.to_numpy(x)
+
+    def scaled(c):
+        def fun(t):
+            return Nx.multiply(Nx.tanh(t), c)
+        return fun
+    consts = [1.0 + i / 16 for i in range(10)]
+    B.fused_mode("compiled")
+    B.fused_cache_limit(8)
+    pinned = 4  # programs that earlier tests recorded into graphs stay loaded
+    try:
+        for c in consts + consts[:2]:  # the first two have been unloaded by the time they come round again
+            got = hip.to_numpy(defn.compile(scaled(c), x, fuse=True)(x))
+            want = (np.tanh(xs.astype(np.float64)).astype(np.float32) * np.float32(c))
+            np.testing.assert_allclose(got, want, rtol=2e-6)
+            assert B.fused_compiled_count() <= 8 + pinned
+        with pytest.raises(HipNxError, match="at least 4"):
+            B.fused_cache_limit(1)
+    finally:
+        B.fused_cache_limit(512)
+        B.fused_mode("interpreted")
+
+
 def test_program_first_met_during_a_capture_runs_interpreted(hip):
     from nx_amd import backend as B
 
