@@ -31,6 +31,7 @@ PEAK = {"bf16": 2500.0, "f16": 2500.0, "s8": 5000.0, "f32": 157.3}  # dense MFMA
 # (`rocprofv3 --pmc FETCH_SIZE`, then `--pmc WRITE_SIZE`, with --calibrate); the summary of those runs
 # carries the figure in a line `TRAFFIC_BYTES_PER_LAUNCH = <n>`, which is what is reported here.
 TRAFFIC_PROFILE = os.path.join("profiles", "dot_bf16_4096_hbm_traffic.md")
+TRAFFIC_PROFILE_S8 = os.path.join("profiles", "dot_s8_4096_hbm_traffic.md")
 CEILINGS_BIN = os.path.join(ROOT, "nx_amd", "lib", "hipnx_ceilings")
 ABI_DRIVER_BIN = os.path.join(ROOT, "nx_amd", "lib", "hipnx_abi_driver")
 
@@ -50,13 +51,13 @@ def c_abi_figures():
         return {"error": str(exc)[:200]}
 
 
-def headline_traffic():
+def headline_traffic(profile):
     """(bytes per launch, source) from the committed counter summary; (None, reason) without it."""
     try:
-        with open(os.path.join(ROOT, TRAFFIC_PROFILE)) as f:
+        with open(os.path.join(ROOT, profile)) as f:
             for line in f:
                 if line.startswith("TRAFFIC_BYTES_PER_LAUNCH"):
-                    return int(line.split("=")[1].split()[0]), TRAFFIC_PROFILE
+                    return int(line.split("=")[1].split()[0]), profile
     except OSError:
         pass
     return None, "no counter summary found"
@@ -99,6 +100,9 @@ def main():
     ap.add_argument("--no-suite", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--calibrate", action="store_true")
+    # which 4096^3 contraction is timed as the headline: bf16 (the metric's configuration, the default) or the
+    # int8 one (s8 x s8 -> s32), so that the int8 kernel can be profiled by the same commands
+    ap.add_argument("--headline", choices=["bf16", "s8"], default="bf16")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (no sharding, no collectives); use --gpus 1")
@@ -168,23 +172,32 @@ def main():
     a_np, b_np = W.dense_gemm_bf16(n=n)
     a, b = put(a_np, "bf16"), put(b_np, "bf16")
     flop = 2.0 * n * n * n
-    _, cold_ms = timed(lambda: Nx.dot(a, b), 20, 5)  # an idle part's first 25 launches
-    settle(lambda: Nx.dot(a, b), args.settle_ms)
-    wall_ms, dev_ms = timed(lambda: Nx.dot(a, b), args.steps, args.warmup)
+    if args.headline == "s8":
+        qa, qb = W.dense_gemm_s8()
+        qa, qb = put(qa, "s8"), put(qb, "s8")
+        head = lambda: Nx.dot(qa, qb, out_type="s32")  # noqa: E731
+    else:
+        head = lambda: Nx.dot(a, b)  # noqa: E731
+    _, cold_ms = timed(head, 20, 5)  # an idle part's first 25 launches
+    settle(head, args.settle_ms)
+    wall_ms, dev_ms = timed(head, args.steps, args.warmup)
     value = flop / (wall_ms * 1e-3) / 1e12
     achieved = flop / (dev_ms * 1e-3) / 1e12
-    lap_mean, lap_median, lap_min = laps(lambda: Nx.dot(a, b), args.steps, 0)
-    traffic, traffic_source = headline_traffic()
+    lap_mean, lap_median, lap_min = laps(head, args.steps, 0)
+    traffic, traffic_source = headline_traffic(TRAFFIC_PROFILE if args.headline == "bf16" else TRAFFIC_PROFILE_S8)
 
+    hunit = "TFLOP/s" if args.headline == "bf16" else "TOP/s"
+    hwork = ("dense GEMM: Nx.dot bf16 {4096,4096} x {4096,4096}, f32 accumulate, bf16 output (BASELINE configs[1])"
+             if args.headline == "bf16" else
+             "dense GEMM: Nx.dot s8 {4096,4096} x {4096,4096}, s32 accumulate and output (the int8 leg of BASELINE configs[1])")
     result = {
         "metric": "Nx.dot TFLOP/s (bf16, s8->s32) + elementwise/reduce GB/s, % of MI355X peak",
-        "value": round(value, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "value": round(value, 3), "unit": hunit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(wall_ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "dense GEMM: Nx.dot bf16 {4096,4096} x {4096,4096}, f32 accumulate, bf16 output "
-                               "(BASELINE configs[1])", "seed": 2},
-        "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK["bf16"], "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK["bf16"], 4), "traffic": traffic, "traffic_source": traffic_source,
+        "dtype": args.headline, "data": "synthetic",
+        "config": {"workload": hwork, "seed": 2},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK[args.headline], "unit": hunit,
+                     "frac": round(achieved / PEAK[args.headline], 4), "traffic": traffic, "traffic_source": traffic_source,
                      "kernel": "dot callback (gemm kernel + operand re-layout, if any), HIP events on the launch stream",
                      "per_step_us": {"mean": round(dev_ms * 1e3, 2), "median": round(lap_median * 1e3, 2),
                                      "min": round(lap_min * 1e3, 2),
@@ -193,10 +206,11 @@ def main():
         "cold_start": {"tflops": round(flop / (cold_ms * 1e-3) / 1e12, 1), "steps": 20, "warmup": 5,
                        "note": "the same call on the idle part, before the settling phase"},
     }
-    if "sustained" in ceilings.get("mfma_bf16", {}):
-        top = ceilings["mfma_bf16"]["sustained"]
-        result["roofline"]["measured_ceiling"] = {"value": top, "unit": "TFLOP/s", "frac_of_ceiling": round(achieved / top, 4),
-                                                  "source": ceilings["mfma_bf16"]["command"]}
+    hceil = "mfma_" + args.headline
+    if "sustained" in ceilings.get(hceil, {}):
+        top = ceilings[hceil]["sustained"]
+        result["roofline"]["measured_ceiling"] = {"value": top, "unit": hunit, "frac_of_ceiling": round(achieved / top, 4),
+                                                  "source": ceilings[hceil]["command"]}
     if ceilings:
         result["ceilings"] = ceilings
 

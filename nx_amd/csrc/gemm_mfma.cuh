@@ -364,7 +364,8 @@ struct GemmArgs {
 template <int DT, int ODT, int TM, int TN>
 __device__ __forceinline__ void gemm_epilogue(typename Mma16<DT>::acc_t (&acc)[TM][TN], void *out, int64_t obase,
                                               int64_t M, int64_t N, int64_t row0, int64_t col0, int lane,
-                                              const float *scale = nullptr, int scale_mode = 0) {
+                                              const float *scale = nullptr, int scale_mode = 0,
+                                              unsigned char *wave_lds = nullptr) {
   constexpr bool int_acc = DT == HIPNX_S8;
   constexpr bool int_out = ODT < HIPNX_F16;
   if constexpr (int_acc && ODT == HIPNX_F32) {
@@ -430,6 +431,39 @@ __device__ __forceinline__ void gemm_epilogue(typename Mma16<DT>::acc_t (&acc)[T
     auto put16 = [&](int64_t gm, int64_t gn, const v4i &v) {
       if (gm < M && gn < N) *reinterpret_cast<v4i *>((unsigned char *)out + (obase + gm * N + gn) * 2) = v;
     };
+    if constexpr (TN % 4 == 0) {
+      if (wave_lds != nullptr && paired) {
+        // with LDS of its own the wave turns four tiles (16 rows x 128 bytes) around instead, as the 4-byte
+        // branch below describes: every cache line leaves as one run of eight neighbouring lanes
+        const int wr = lane & 15, wc = lane >> 4, rr = lane >> 3, rp = lane & 7;
+        const int w_off = wr * 128 + (wc & 1) * 8, w_swz = (wr >> 1) & 7;
+        const int r_off0 = rr * 128 + ((rp ^ ((rr >> 1) & 7)) * 16), r_off1 = (rr + 8) * 128 + ((rp ^ (((rr + 8) >> 1) & 7)) * 16);
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+#pragma unroll
+          for (int j = 0; j < TN; j += 4) {
+            unsigned char *half = wave_lds + (((i * TN + j) >> 2) & 1) * 2048;  // two halves in turn
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+              typedef __attribute__((ext_vector_type(2))) unsigned int v2u;
+              v2u pk;
+              pk[0] = pack(acc[i][j + t][0], acc[i][j + t][1]);
+              pk[1] = pack(acc[i][j + t][2], acc[i][j + t][3]);
+              *reinterpret_cast<v2u *>(half + w_off + (((2 * t + (wc >> 1)) ^ w_swz) * 16)) = pk;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            const v4i lo = *reinterpret_cast<const v4i *>(half + r_off0);
+            const v4i up = *reinterpret_cast<const v4i *>(half + r_off1);
+            const int64_t gm = row0 + 16 * i + rr, gn = col0 + 16 * j + 8 * rp;
+            put16(gm, gn, lo);
+            put16(gm + 8, gn, up);
+          }
+        }
+        return;
+      }
+    }
 #pragma unroll
     for (int i = 0; i < TM; i++) {
       const int64_t gm = row0 + 16 * i + (lane & 15);
@@ -489,6 +523,40 @@ __device__ __forceinline__ void gemm_epilogue(typename Mma16<DT>::acc_t (&acc)[T
     auto put16 = [&](int64_t gm, int64_t gn, const v4i &v) {
       if (gm < M && gn < N) *reinterpret_cast<v4i *>((unsigned char *)out + (obase + gm * N + gn) * 4) = v;
     };
+    if (wave_lds != nullptr && lines) {
+      // With 4 KiB of LDS of its own a wave turns each pair of tiles (16 rows x 128 bytes) around first:
+      // written as the accumulators hold it (lane = row, 16-byte piece c of either tile), read back with
+      // eight consecutive lanes along one row, so that every cache line of the result leaves as ONE
+      // contiguous 128-byte run of eight neighbouring lanes.  In the exchange-only form below a line is made
+      // of eight 16-byte pieces from four different quarters of the wave; when the result is larger than the
+      // L2s (the 64 MiB s32 result of a 4096^2 int8 contraction) lines are evicted between their pieces,
+      // and the counters show the cost: 94 MiB written and 30 MiB read back for 64 MiB of output.
+      // Piece index XOR (row / 2) % 8 keeps both the write and the read free of bank conflicts.
+      const int wr = lane & 15, wc = lane >> 4, rr = lane >> 3, rp = lane & 7;
+      const int w_off = wr * 128, w_swz = (wr >> 1) & 7;
+      const int r_off0 = rr * 128 + ((rp ^ ((rr >> 1) & 7)) * 16), r_off1 = (rr + 8) * 128 + ((rp ^ (((rr + 8) >> 1) & 7)) * 16);
+#pragma unroll
+      for (int i = 0; i < TM; i++) {
+#pragma unroll
+        for (int j = 0; j < TN; j += 2) {
+          unsigned char *half = wave_lds + (((i * TN + j) >> 1) & 1) * 2048;  // two halves in turn
+          v4i v, w;
+#pragma unroll
+          for (int e = 0; e < 4; e++) { v[e] = word(acc[i][j], e); w[e] = word(acc[i][j + 1], e); }
+          *reinterpret_cast<v4i *>(half + w_off + ((wc ^ w_swz) * 16)) = v;
+          *reinterpret_cast<v4i *>(half + w_off + (((4 + wc) ^ w_swz) * 16)) = w;
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+          const v4i lo = *reinterpret_cast<const v4i *>(half + r_off0);
+          const v4i up = *reinterpret_cast<const v4i *>(half + r_off1);
+          const int64_t gm = row0 + 16 * i + rr, gn = col0 + 16 * j + 4 * rp;
+          put16(gm, gn, lo);
+          put16(gm + 8, gn, up);
+        }
+      }
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < TM; i++) {
       const int64_t gm = row0 + 16 * i + (lane & 15);
@@ -765,8 +833,11 @@ gemm_pipelined_kernel(GemmArgs a) {
 
   // epilogue: the output type is wave-uniform; branch once, then every store is straight-line
   const int64_t obase = b * a.M * a.N;
+  // every wave has read its last fragments: the stages are free, and each wave takes 4 KiB of them to turn its
+  // result tiles into whole cache lines (a stage is at least (BM + BN) * 128 bytes = 6 KiB per wave)
+  __syncthreads();
   switch (a.odt) {
-#define HIPNX_EPI(T) case T: gemm_epilogue<DT, T, TM16, TN16>(acc, a.out, obase, a.M, a.N, m0 + wm, n0 + wn, lane, a.scale, a.scale_mode); break;
+#define HIPNX_EPI(T) case T: gemm_epilogue<DT, T, TM16, TN16>(acc, a.out, obase, a.M, a.N, m0 + wm, n0 + wn, lane, a.scale, a.scale_mode, smem + wave * 4096); break;
     HIPNX_EPI(HIPNX_BF16) HIPNX_EPI(HIPNX_F16) HIPNX_EPI(HIPNX_F32) HIPNX_EPI(HIPNX_F64) HIPNX_EPI(HIPNX_BF16_RNE)
     HIPNX_EPI(HIPNX_S8) HIPNX_EPI(HIPNX_U8) HIPNX_EPI(HIPNX_S16) HIPNX_EPI(HIPNX_U16)
     HIPNX_EPI(HIPNX_S32) HIPNX_EPI(HIPNX_U32) HIPNX_EPI(HIPNX_S64) HIPNX_EPI(HIPNX_U64)
