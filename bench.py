@@ -371,6 +371,14 @@ def main():
         nxt = rotating(lambda: put(rng.integers(0, 32000, size=8192, dtype=np.uint32), "u32"), 40e6)
         _, ms = tstat(lambda: Nx.take(table, nxt()), steps, warm)
         entry("take_bf16_8192_of_32000x4096_rotated", 134250496.0, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+        # the same with the bounds policy that raises late (the kernel records a bad index, the next wait
+        # reports it): the call no longer waits for its kernel, so this is the gather kernel's own rate
+        previous = B.bounds_policy("defer")
+        try:
+            _, ms = tstat(lambda: Nx.take(table, nxt()), steps, warm)
+        finally:
+            B.bounds_policy(previous)
+        entry("take_bf16_8192_of_32000x4096_rotated_deferred_bounds", 134250496.0, "GB/s", ms, PEAK_HBM_GBS, "hbm")
         del logits, table, idx, nxt
 
         # selection, windows and creation at the HBM-resident size of config 1
