@@ -10,7 +10,8 @@
 //       of the run and for the last fifth (the sustained figure: the clock the part settles at
 //       under this load depends on the operand bits and takes tens of milliseconds to settle)
 //   hipnx_ceilings stream <read|write|copy> [MiB] [ms]
-//       16-byte-per-lane streaming kernels over a buffer larger than the 256 MB last-level cache
+//       16-byte-per-lane streaming kernels over a buffer larger than the 256 MB last-level cache, the best of
+//       1, 2, 4 and 8 accesses in flight per lane
 //
 // Each run prints one JSON line.  Built by the Makefile into nx_amd/lib/hipnx_ceilings; bench.py runs
 // it when present and copies the sustained figures into its `measured_ceiling` fields.
@@ -92,34 +93,45 @@ __global__ void __launch_bounds__(512) mfma_loop(const v4i *src, float *out, int
   }
 }
 
-// Streaming kernels with a grid that covers the buffer (no grid-stride loop): a work-group owns
-// UNROLL * 4 KiB of contiguous memory, every lane has UNROLL independent 16-byte accesses in flight.
-constexpr int UNROLL = 8;
+// Streaming kernels with a grid that covers the buffer (no grid-stride loop; on this part a resident grid
+// that loops streams slower): a work-group of 256 lanes owns U * 4 KiB of contiguous memory, every lane has
+// U independent 16-byte accesses in flight.  Which U streams fastest depends on the direction, so each run
+// tries U = 1, 2, 4, 8 and reports the best.
+template <int U>
 __global__ void __launch_bounds__(256) stream_read(const v4i *__restrict__ in, v4i *__restrict__ out, size_t n) {
-  const size_t base = (size_t)blockIdx.x * (256 * UNROLL) + threadIdx.x;
-  v4i v[UNROLL];
+  const size_t base = (size_t)blockIdx.x * (256 * U) + threadIdx.x;
+  v4i v[U];
 #pragma unroll
-  for (int u = 0; u < UNROLL; u++) v[u] = base + u * 256 < n ? in[base + u * 256] : v4i{0, 0, 0, 0};
+  for (int u = 0; u < U; u++) v[u] = base + u * 256 < n ? in[base + u * 256] : v4i{0, 0, 0, 0};
   v4i acc = v[0];
 #pragma unroll
-  for (int u = 1; u < UNROLL; u++) acc ^= v[u];
+  for (int u = 1; u < U; u++) acc ^= v[u];
   if (acc[0] == 0x12345678 && acc[1] == 0x0BADF00D) out[0] = acc;  // keeps the loads alive; practically never taken
 }
+template <int U>
 __global__ void __launch_bounds__(256) stream_write(v4i *__restrict__ out, size_t n, int v) {
   const v4i x = {v, v + 1, v + 2, v + 3};
-  const size_t base = (size_t)blockIdx.x * (256 * UNROLL) + threadIdx.x;
+  const size_t base = (size_t)blockIdx.x * (256 * U) + threadIdx.x;
 #pragma unroll
-  for (int u = 0; u < UNROLL; u++)
+  for (int u = 0; u < U; u++)
     if (base + u * 256 < n) out[base + u * 256] = x;
 }
+template <int U>
 __global__ void __launch_bounds__(256) stream_copy(const v4i *__restrict__ in, v4i *__restrict__ out, size_t n) {
-  const size_t base = (size_t)blockIdx.x * (256 * UNROLL) + threadIdx.x;
-  v4i v[UNROLL];
+  const size_t base = (size_t)blockIdx.x * (256 * U) + threadIdx.x;
+  v4i v[U];
 #pragma unroll
-  for (int u = 0; u < UNROLL; u++) v[u] = base + u * 256 < n ? in[base + u * 256] : v4i{0, 0, 0, 0};
+  for (int u = 0; u < U; u++) v[u] = base + u * 256 < n ? in[base + u * 256] : v4i{0, 0, 0, 0};
 #pragma unroll
-  for (int u = 0; u < UNROLL; u++)
+  for (int u = 0; u < U; u++)
     if (base + u * 256 < n) out[base + u * 256] = v[u];
+}
+template <int U>
+static void launch_stream(int m, const v4i *a, v4i *b, size_t n) {
+  const unsigned grid = (unsigned)((n + 256 * U - 1) / (256 * U));
+  if (m == 0) hipLaunchKernelGGL(stream_read<U>, dim3(grid), dim3(256), 0, 0, a, b, n);
+  else if (m == 1) hipLaunchKernelGGL(stream_write<U>, dim3(grid), dim3(256), 0, 0, b, n, 7);
+  else hipLaunchKernelGGL(stream_copy<U>, dim3(grid), dim3(256), 0, 0, a, b, n);
 }
 
 static void launch_mfma(int kind, const v4i *d, float *o, int iters) {
@@ -213,26 +225,38 @@ static int run_stream(const char *mode, size_t mib, double want_ms) {
   CK(hipMemset(b, 2, bytes));
   const int m = !strcmp(mode, "read") ? 0 : !strcmp(mode, "write") ? 1 : !strcmp(mode, "copy") ? 2 : -1;
   if (m < 0) { fprintf(stderr, "unknown mode %s\n", mode); return 2; }
-  const unsigned grid = (unsigned)((n + 256 * UNROLL - 1) / (256 * UNROLL));
-  auto launch = [&] {
-    if (m == 0) hipLaunchKernelGGL(stream_read, dim3(grid), dim3(256), 0, 0, a, b, n);
-    else if (m == 1) hipLaunchKernelGGL(stream_write, dim3(grid), dim3(256), 0, 0, b, n, 7);
-    else hipLaunchKernelGGL(stream_copy, dim3(grid), dim3(256), 0, 0, a, b, n);
-  };
-  std::vector<float> probe;
-  if (timed_chunks(launch, 1, 3, probe)) return 1;
-  const double launch_ms = probe[0] / 3;
-  const int per_chunk = std::max(1, (int)(2.0 / launch_ms));
-  const int chunks = std::max(5, (int)(want_ms / (per_chunk * launch_ms)));
-  std::vector<float> ms;
-  if (timed_chunks(launch, chunks, per_chunk, ms)) return 1;
   const double moved = (m == 2 ? 2.0 : 1.0) * bytes;
-  auto rate = [&](int x, int y) { double t = 0; for (int i = x; i < y; i++) t += ms[i]; return moved * per_chunk * (y - x) / t / 1e6; };
-  std::vector<float> sorted(ms);
-  std::sort(sorted.begin(), sorted.end());
-  printf("{\"kind\": \"stream\", \"mode\": \"%s\", \"MiB\": %zu, \"unit\": \"GB/s\", \"bytes_counted\": \"%s\", \"sustained\": %.0f, \"best_chunk\": %.0f, \"launch_us\": %.1f}\n",
-         mode, mib, m == 2 ? "read + written" : "one direction", rate(chunks * 4 / 5, chunks), moved * per_chunk / sorted[0] / 1e6,
-         1000 * ms[chunks - 1] / per_chunk);
+  double best = 0, best_chunk = 0, best_us = 0;
+  int best_u = 0;
+  for (int u : {1, 2, 4, 8}) {
+    auto launch = [&] {
+      switch (u) {
+        case 1: launch_stream<1>(m, a, b, n); break;
+        case 2: launch_stream<2>(m, a, b, n); break;
+        case 4: launch_stream<4>(m, a, b, n); break;
+        default: launch_stream<8>(m, a, b, n); break;
+      }
+    };
+    std::vector<float> probe;
+    if (timed_chunks(launch, 1, 3, probe)) return 1;
+    const double launch_ms = probe[0] / 3;
+    const int per_chunk = std::max(1, (int)(2.0 / launch_ms));
+    const int chunks = std::max(5, (int)(want_ms / 4 / (per_chunk * launch_ms)));
+    std::vector<float> ms;
+    if (timed_chunks(launch, chunks, per_chunk, ms)) return 1;
+    auto rate = [&](int x, int y) { double t = 0; for (int i = x; i < y; i++) t += ms[i]; return moved * per_chunk * (y - x) / t / 1e6; };
+    std::vector<float> sorted(ms);
+    std::sort(sorted.begin(), sorted.end());
+    const double sustained = rate(chunks * 4 / 5, chunks);
+    if (sustained > best) {
+      best = sustained;
+      best_chunk = moved * per_chunk / sorted[0] / 1e6;
+      best_us = 1000 * ms[chunks - 1] / per_chunk;
+      best_u = u;
+    }
+  }
+  printf("{\"kind\": \"stream\", \"mode\": \"%s\", \"MiB\": %zu, \"unit\": \"GB/s\", \"bytes_counted\": \"%s\", \"sustained\": %.0f, \"best_chunk\": %.0f, \"launch_us\": %.1f, \"accesses_per_lane\": %d}\n",
+         mode, mib, m == 2 ? "read + written" : "one direction", best, best_chunk, best_us, best_u);
   return 0;
 }
 
