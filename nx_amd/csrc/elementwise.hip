@@ -6,6 +6,8 @@
 // with per-operand strides (row stride, column stride in {0, 1}) -- same shape, scalar operand,
 // trailing row vector, keep-dims column -- runs on the vector kernel, the rest on a generic
 // rank-N kernel.  Algorithmic traffic is exactly bytes(l) + bytes(r) + bytes(out).
+#include <type_traits>
+
 #include "elementwise_ops.cuh"
 #include "internal.h"
 
@@ -20,15 +22,44 @@ struct NdIndex {
   int64_t dims[MAXR], ls[MAXR], rs[MAXR];
 };
 
-template <int OP, typename CT, bool UNS>
+// Division of an index below 2^31 by an invariant divisor below 2^31 as one multiplication: the 64-bit
+// division the compiler emits costs every wave some hundred scalar and vector instructions, more than the
+// rest of an 8-element vector's work.
+struct FastDiv32 {
+  uint32_t mul, shr;
+};
+static FastDiv32 make_fastdiv(uint32_t d) {
+  uint32_t shr = 0;
+  while ((1ull << shr) < d) shr++;
+  return FastDiv32{(uint32_t)(((1ull << 32) * ((1ull << shr) - d)) / d + 1), shr};
+}
+__device__ __forceinline__ uint32_t fastdiv(uint32_t n, FastDiv32 f) { return (__umulhi(n, f.mul) + n) >> f.shr; }
+
+enum { ROWS_ONE = 0, ROWS_FAST = 1, ROWS_WIDE = 2 };  // how a vector index splits into (row, column)
+
+// FIX >= 0: both operands and the result have this element type, known when the kernel is compiled -- the
+// three run-time type switches (and the scalar bookkeeping the compiler builds around them, ~200 scalar
+// instructions per wave) fold away.  bf16 add on 16384^2: 388 -> 263 us (4.1 -> 6.1 TB/s), negate and exp 280 -> 175 us.
+template <int OP, typename CT, bool UNS, int FIX = -1>
 __global__ void __launch_bounds__(BLOCK)
-binary_vec_kernel(const void *__restrict__ l, const void *__restrict__ r, void *__restrict__ out, int ldt, int rdt,
-                  int odt, int64_t cols, int64_t vecs_per_row, int64_t nvec, int64_t ls0, int ls1, int64_t rs0,
-                  int rs1, unsigned long long *__restrict__ err) {
+binary_vec_kernel(const void *__restrict__ l, const void *__restrict__ r, void *__restrict__ out, int ldt_, int rdt_,
+                  int odt_, int64_t cols, int64_t vecs_per_row, int64_t nvec, int64_t ls0, int ls1, int64_t rs0,
+                  int rs1, unsigned long long *__restrict__ err, int rows_mode, FastDiv32 fd) {
   constexpr bool RAISES = binary_can_raise(OP, is_fp<CT>::value);
+  const int ldt = FIX >= 0 ? FIX : ldt_, rdt = FIX >= 0 ? FIX : rdt_, odt = FIX >= 0 ? FIX : odt_;
   for (int64_t v = (int64_t)blockIdx.x * BLOCK + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * BLOCK) {
-    int64_t row = v / vecs_per_row;
-    int64_t col = (v - row * vecs_per_row) * E;
+    int64_t row, col;
+    if (rows_mode == ROWS_ONE) {
+      row = 0;
+      col = v * E;
+    } else if (rows_mode == ROWS_FAST) {
+      const uint32_t q = fastdiv((uint32_t)v, fd);
+      row = q;
+      col = (int64_t)((uint32_t)v - q * (uint32_t)vecs_per_row) * E;
+    } else {
+      row = v / vecs_per_row;
+      col = (v - row * vecs_per_row) * E;
+    }
     int64_t lo = row * ls0 + col * ls1, ro = row * rs0 + col * rs1, oo = row * cols + col;
     CT a[E], b[E], c[E];
     if (col + E <= cols) {
@@ -112,9 +143,10 @@ binary_nd_kernel(const void *__restrict__ l, const void *__restrict__ r, void *_
   }
 }
 
-template <int OP, typename CT>
+template <int OP, typename CT, int FIX = -1>  // FIX: the one element type of input and result, as above
 __global__ void __launch_bounds__(BLOCK)
-unary_vec_kernel(const void *__restrict__ in, void *__restrict__ out, int idt, int odt, int bits, int64_t n) {
+unary_vec_kernel(const void *__restrict__ in, void *__restrict__ out, int idt_, int odt_, int bits, int64_t n) {
+  const int idt = FIX >= 0 ? FIX : idt_, odt = FIX >= 0 ? FIX : odt_;
   int64_t nvec = (n + E - 1) / E;
   for (int64_t v = (int64_t)blockIdx.x * BLOCK + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * BLOCK) {
     int64_t o = v * E;
@@ -191,10 +223,31 @@ struct BinArgs {
   unsigned long long *err;  // the context's deferred error word (device address of the pinned host word)
 };
 
+template <int OP, typename CT, bool UNS, int FIX>
+static void launch_bvec_fix(const hipnx_ctx *ctx, const BinArgs &a) {
+  const int mode = a.vecs_per_row >= a.nvec ? ROWS_ONE : a.nvec < (1ll << 31) ? ROWS_FAST : ROWS_WIDE;
+  const FastDiv32 fd = mode == ROWS_FAST ? make_fastdiv((uint32_t)a.vecs_per_row) : FastDiv32{0, 0};
+  hipLaunchKernelGGL((binary_vec_kernel<OP, CT, UNS, FIX>), dim3(grid_for(ctx, a.nvec)), dim3(BLOCK), 0, ctx->stream, a.l,
+                     a.r, a.out, a.ldt, a.rdt, a.odt, a.cols, a.vecs_per_row, a.nvec, a.ls0, a.ls1, a.rs0, a.rs1, a.err,
+                     mode, fd);
+}
+
+// the kernel compiled for one element type throughout, where there is one: the types of most tensor arithmetic
 template <int OP, typename CT, bool UNS>
 static void launch_bvec(const hipnx_ctx *ctx, const BinArgs &a) {
-  hipLaunchKernelGGL((binary_vec_kernel<OP, CT, UNS>), dim3(grid_for(ctx, a.nvec)), dim3(BLOCK), 0, ctx->stream, a.l,
-                     a.r, a.out, a.ldt, a.rdt, a.odt, a.cols, a.vecs_per_row, a.nvec, a.ls0, a.ls1, a.rs0, a.rs1, a.err);
+  if (a.ldt == a.rdt && a.ldt == a.odt) {
+    if constexpr (std::is_same<CT, float>::value) {
+      if (a.odt == HIPNX_F32) return launch_bvec_fix<OP, CT, UNS, HIPNX_F32>(ctx, a);
+      if (a.odt == HIPNX_BF16) return launch_bvec_fix<OP, CT, UNS, HIPNX_BF16>(ctx, a);
+      if (a.odt == HIPNX_F16) return launch_bvec_fix<OP, CT, UNS, HIPNX_F16>(ctx, a);
+    } else if constexpr (std::is_same<CT, double>::value) {
+      if (a.odt == HIPNX_F64) return launch_bvec_fix<OP, CT, UNS, HIPNX_F64>(ctx, a);
+    } else if constexpr (!UNS) {
+      if (a.odt == HIPNX_S32) return launch_bvec_fix<OP, CT, UNS, HIPNX_S32>(ctx, a);
+      if (a.odt == HIPNX_S64) return launch_bvec_fix<OP, CT, UNS, HIPNX_S64>(ctx, a);
+    }
+  }
+  launch_bvec_fix<OP, CT, UNS, -1>(ctx, a);
 }
 
 template <int OP>
@@ -339,10 +392,27 @@ extern "C" int hipnx_binary(hipnx_ctx *ctx, int op, int l_dt, int r_dt, int out_
 
 namespace hipnx {
 
+template <int OP, typename CT, int FIX>
+static void launch_uvec_fix(const hipnx_ctx *ctx, const void *in, void *out, int idt, int odt, int bits, int64_t n) {
+  hipLaunchKernelGGL((unary_vec_kernel<OP, CT, FIX>), dim3(grid_for(ctx, (n + E - 1) / E)), dim3(BLOCK), 0, ctx->stream, in,
+                     out, idt, odt, bits, n);
+}
+
 template <int OP, typename CT>
 static void launch_uvec(const hipnx_ctx *ctx, const void *in, void *out, int idt, int odt, int bits, int64_t n) {
-  hipLaunchKernelGGL((unary_vec_kernel<OP, CT>), dim3(grid_for(ctx, (n + E - 1) / E)), dim3(BLOCK), 0, ctx->stream, in,
-                     out, idt, odt, bits, n);
+  if (idt == odt) {
+    if constexpr (std::is_same<CT, float>::value) {
+      if (odt == HIPNX_F32) return launch_uvec_fix<OP, CT, HIPNX_F32>(ctx, in, out, idt, odt, bits, n);
+      if (odt == HIPNX_BF16) return launch_uvec_fix<OP, CT, HIPNX_BF16>(ctx, in, out, idt, odt, bits, n);
+      if (odt == HIPNX_F16) return launch_uvec_fix<OP, CT, HIPNX_F16>(ctx, in, out, idt, odt, bits, n);
+    } else if constexpr (std::is_same<CT, double>::value) {
+      if (odt == HIPNX_F64) return launch_uvec_fix<OP, CT, HIPNX_F64>(ctx, in, out, idt, odt, bits, n);
+    } else {
+      if (odt == HIPNX_S32) return launch_uvec_fix<OP, CT, HIPNX_S32>(ctx, in, out, idt, odt, bits, n);
+      if (odt == HIPNX_S64) return launch_uvec_fix<OP, CT, HIPNX_S64>(ctx, in, out, idt, odt, bits, n);
+    }
+  }
+  launch_uvec_fix<OP, CT, -1>(ctx, in, out, idt, odt, bits, n);
 }
 
 template <int OP>
