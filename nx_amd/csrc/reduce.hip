@@ -29,10 +29,13 @@ namespace hipnx {
 // TPR lanes per row (64 or 256); a block of 256 lanes covers 256/TPR rows.  Row `row` segment
 // `seg` covers elements [seg*seg_len, min(red, (seg+1)*seg_len)).  With nseg == 1 the result is
 // encoded into `out`; otherwise the raw accumulator goes to `partial[row*nseg + seg]`.
-template <typename R, typename CT, int TPR, bool VEC>
+// IDT >= 0: the input's element type, known when the kernel is compiled (the type switch inside every
+// vector load, and the scalar bookkeeping the compiler builds around it, fold away); -1: read from `idt_`.
+template <typename R, typename CT, int TPR, bool VEC, int IDT = -1>
 __global__ void __launch_bounds__(BLOCK)
 reduce_rows_kernel(const void *__restrict__ in, void *__restrict__ out, typename R::acc_t *__restrict__ partial,
-                   int idt, int odt, int64_t rows, int64_t red, int64_t seg_len, int nseg) {
+                   int idt_, int odt, int64_t rows, int64_t red, int64_t seg_len, int nseg) {
+  const int idt = IDT >= 0 ? IDT : idt_;
   constexpr int RPB = BLOCK / TPR;
   const int sub = threadIdx.x / TPR, lane = threadIdx.x % TPR;
   const int64_t unit = (int64_t)blockIdx.x * RPB + sub;  // (row, seg) pair
@@ -102,10 +105,11 @@ combine_partials_kernel(const typename R::acc_t *__restrict__ partial, void *__r
 // One lane per E adjacent inner positions (VEC) or per position; walks k in its segment.
 // With nseg == 1 results are encoded into out[outer, inner]; otherwise raw accumulators go to
 // partial[outer, nseg, inner].
-template <typename R, typename CT, bool VEC>
+template <typename R, typename CT, bool VEC, int IDT = -1>
 __global__ void __launch_bounds__(BLOCK)
 reduce_cols_kernel(const void *__restrict__ in, void *__restrict__ out, typename R::acc_t *__restrict__ partial,
-                   int idt, int odt, int64_t outer, int64_t red, int64_t inner, int64_t seg_len, int nseg) {
+                   int idt_, int odt, int64_t outer, int64_t red, int64_t inner, int64_t seg_len, int nseg) {
+  const int idt = IDT >= 0 ? IDT : idt_;
   constexpr int W = VEC ? E : 1;
   const int64_t ivecs = inner / W;
   const int64_t total = outer * nseg * ivecs;
@@ -182,9 +186,9 @@ static void partials_release(hipnx_ctx *ctx, bool static_ws, void *ws, size_t ws
   if (ws && !static_ws) pool_free(ctx, ws, ws_cap);
 }
 
-template <typename R, typename CT>
-static int run_reduce(hipnx_ctx *ctx, bool static_ws, int idt, int odt, int64_t outer, int64_t red, int64_t inner,
-                      const void *in, void *out) {
+template <typename R, typename CT, int IDT>
+static int run_reduce_t(hipnx_ctx *ctx, bool static_ws, int idt, int odt, int64_t outer, int64_t red, int64_t inner,
+                        const void *in, void *out) {
   typedef typename R::acc_t acc_t;
   const int64_t target_units = (int64_t)ctx->num_cus * 8;  // units of parallel work wanted
   if (inner == 1) {
@@ -214,10 +218,10 @@ static int run_reduce(hipnx_ctx *ctx, bool static_ws, int idt, int odt, int64_t 
     dim3 grid((unsigned)((rows * nseg + rpb - 1) / rpb)), block(BLOCK);
     if (rows * nseg > 0) {
       if (tpr == WAVE) {
-        if (vec) hipLaunchKernelGGL((reduce_rows_kernel<R, CT, WAVE, true>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
+        if (vec) hipLaunchKernelGGL((reduce_rows_kernel<R, CT, WAVE, true, IDT>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
         else hipLaunchKernelGGL((reduce_rows_kernel<R, CT, WAVE, false>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
       } else {
-        if (vec) hipLaunchKernelGGL((reduce_rows_kernel<R, CT, BLOCK, true>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
+        if (vec) hipLaunchKernelGGL((reduce_rows_kernel<R, CT, BLOCK, true, IDT>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
         else hipLaunchKernelGGL((reduce_rows_kernel<R, CT, BLOCK, false>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
       }
       if (nseg > 1) {
@@ -252,7 +256,7 @@ static int run_reduce(hipnx_ctx *ctx, bool static_ws, int idt, int odt, int64_t 
     int64_t cap = 1ll << 30;
     dim3 grid((unsigned)(blocks < 1 ? 1 : (blocks < cap ? blocks : cap))), block(BLOCK);
     if (total > 0) {
-      if (vec) hipLaunchKernelGGL((reduce_cols_kernel<R, CT, true>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, outer, red, inner, seg_len, nseg);
+      if (vec) hipLaunchKernelGGL((reduce_cols_kernel<R, CT, true, IDT>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, outer, red, inner, seg_len, nseg);
       else hipLaunchKernelGGL((reduce_cols_kernel<R, CT, false>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, outer, red, inner, seg_len, nseg);
       if (nseg > 1) {
         int64_t b2 = (outer * inner + BLOCK - 1) / BLOCK;
@@ -264,6 +268,21 @@ static int run_reduce(hipnx_ctx *ctx, bool static_ws, int idt, int odt, int64_t 
   }
   HIPNX_HIP(hipGetLastError());
   return HIPNX_OK;
+}
+
+// the vectorised kernels compiled for the input's element type where it is one of the common ones
+template <typename R, typename CT>
+static int run_reduce(hipnx_ctx *ctx, bool static_ws, int idt, int odt, int64_t outer, int64_t red, int64_t inner,
+                      const void *in, void *out) {
+#define HIPNX_RED_AS(T) if (idt == T) return run_reduce_t<R, CT, T>(ctx, static_ws, idt, odt, outer, red, inner, in, out);
+  if constexpr (std::is_floating_point<CT>::value) {
+    HIPNX_RED_AS(HIPNX_F32) HIPNX_RED_AS(HIPNX_BF16) HIPNX_RED_AS(HIPNX_F16)
+    if constexpr (std::is_same<CT, double>::value) { HIPNX_RED_AS(HIPNX_F64) }
+  } else {
+    HIPNX_RED_AS(HIPNX_S32) HIPNX_RED_AS(HIPNX_S64) HIPNX_RED_AS(HIPNX_U8)
+  }
+#undef HIPNX_RED_AS
+  return run_reduce_t<R, CT, -1>(ctx, static_ws, idt, odt, outer, red, inner, in, out);
 }
 
 template <int OP>
