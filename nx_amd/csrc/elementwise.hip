@@ -40,13 +40,14 @@ enum { ROWS_ONE = 0, ROWS_FAST = 1, ROWS_WIDE = 2 };  // how a vector index spli
 // FIX >= 0: both operands and the result have this element type, known when the kernel is compiled -- the
 // three run-time type switches (and the scalar bookkeeping the compiler builds around them, ~200 scalar
 // instructions per wave) fold away.  bf16 add on 16384^2: 388 -> 263 us (4.1 -> 6.1 TB/s), negate and exp 280 -> 175 us.
-template <int OP, typename CT, bool UNS, int FIX = -1>
+// (FIXO: the result's type when it differs -- u8 for comparisons and logical operations.)
+template <int OP, typename CT, bool UNS, int FIX = -1, int FIXO = FIX>
 __global__ void __launch_bounds__(BLOCK)
 binary_vec_kernel(const void *__restrict__ l, const void *__restrict__ r, void *__restrict__ out, int ldt_, int rdt_,
                   int odt_, int64_t cols, int64_t vecs_per_row, int64_t nvec, int64_t ls0, int ls1, int64_t rs0,
                   int rs1, unsigned long long *__restrict__ err, int rows_mode, FastDiv32 fd) {
   constexpr bool RAISES = binary_can_raise(OP, is_fp<CT>::value);
-  const int ldt = FIX >= 0 ? FIX : ldt_, rdt = FIX >= 0 ? FIX : rdt_, odt = FIX >= 0 ? FIX : odt_;
+  const int ldt = FIX >= 0 ? FIX : ldt_, rdt = FIX >= 0 ? FIX : rdt_, odt = FIX >= 0 ? FIXO : odt_;
   for (int64_t v = (int64_t)blockIdx.x * BLOCK + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * BLOCK) {
     int64_t row, col;
     if (rows_mode == ROWS_ONE) {
@@ -163,11 +164,13 @@ unary_vec_kernel(const void *__restrict__ in, void *__restrict__ out, int idt_, 
   }
 }
 
-// as_type: CT is the decode type of the input; float -> integer goes through the wrap rule
-template <typename CT>
+// as_type: CT is the decode type of the input; float -> integer goes through the wrap rule.
+// FIXI / FIXO >= 0: input and result type known when the kernel is compiled.
+template <typename CT, int FIXI = -1, int FIXO = -1>
 __global__ void __launch_bounds__(BLOCK)
-as_type_kernel(const void *__restrict__ in, void *__restrict__ out, int idt, int odt, int64_t n, int64_t tmax,
+as_type_kernel(const void *__restrict__ in, void *__restrict__ out, int idt_, int odt_, int64_t n, int64_t tmax,
                int64_t tmin) {
+  const int idt = FIXI >= 0 ? FIXI : idt_, odt = FIXO >= 0 ? FIXO : odt_;
   const bool to_int = odt < HIPNX_F16;
   int64_t nvec = (n + E - 1) / E;
   for (int64_t v = (int64_t)blockIdx.x * BLOCK + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * BLOCK) {
@@ -223,11 +226,11 @@ struct BinArgs {
   unsigned long long *err;  // the context's deferred error word (device address of the pinned host word)
 };
 
-template <int OP, typename CT, bool UNS, int FIX>
+template <int OP, typename CT, bool UNS, int FIX, int FIXO = FIX>
 static void launch_bvec_fix(const hipnx_ctx *ctx, const BinArgs &a) {
   const int mode = a.vecs_per_row >= a.nvec ? ROWS_ONE : a.nvec < (1ll << 31) ? ROWS_FAST : ROWS_WIDE;
   const FastDiv32 fd = mode == ROWS_FAST ? make_fastdiv((uint32_t)a.vecs_per_row) : FastDiv32{0, 0};
-  hipLaunchKernelGGL((binary_vec_kernel<OP, CT, UNS, FIX>), dim3(grid_for(ctx, a.nvec)), dim3(BLOCK), 0, ctx->stream, a.l,
+  hipLaunchKernelGGL((binary_vec_kernel<OP, CT, UNS, FIX, FIXO>), dim3(grid_for(ctx, a.nvec)), dim3(BLOCK), 0, ctx->stream, a.l,
                      a.r, a.out, a.ldt, a.rdt, a.odt, a.cols, a.vecs_per_row, a.nvec, a.ls0, a.ls1, a.rs0, a.rs1, a.err,
                      mode, fd);
 }
@@ -245,6 +248,16 @@ static void launch_bvec(const hipnx_ctx *ctx, const BinArgs &a) {
     } else if constexpr (!UNS) {
       if (a.odt == HIPNX_S32) return launch_bvec_fix<OP, CT, UNS, HIPNX_S32>(ctx, a);
       if (a.odt == HIPNX_S64) return launch_bvec_fix<OP, CT, UNS, HIPNX_S64>(ctx, a);
+    }
+  }
+  if (a.ldt == a.rdt && a.odt == HIPNX_U8) {  // what comparisons and logical operations produce
+    if constexpr (std::is_same<CT, float>::value) {
+      if (a.ldt == HIPNX_F32) return launch_bvec_fix<OP, CT, UNS, HIPNX_F32, HIPNX_U8>(ctx, a);
+      if (a.ldt == HIPNX_BF16) return launch_bvec_fix<OP, CT, UNS, HIPNX_BF16, HIPNX_U8>(ctx, a);
+      if (a.ldt == HIPNX_F16) return launch_bvec_fix<OP, CT, UNS, HIPNX_F16, HIPNX_U8>(ctx, a);
+    } else if constexpr (std::is_same<CT, int64_t>::value && !UNS) {
+      if (a.ldt == HIPNX_S32) return launch_bvec_fix<OP, CT, UNS, HIPNX_S32, HIPNX_U8>(ctx, a);
+      if (a.ldt == HIPNX_U8) return launch_bvec_fix<OP, CT, UNS, HIPNX_U8, HIPNX_U8>(ctx, a);
     }
   }
   launch_bvec_fix<OP, CT, UNS, -1>(ctx, a);
@@ -473,13 +486,25 @@ extern "C" int hipnx_as_type(hipnx_ctx *ctx, int in_dt, int out_dt, int64_t n, c
   static const int64_t tmin[8] = {0, 0, 0, 0, -0x80, -0x8000, -0x80000000ll, (int64_t)0x8000000000000000ull};
   int64_t mx = out_dt < HIPNX_F16 ? tmax[out_dt] : 0, mn = out_dt < HIPNX_F16 ? tmin[out_dt] : 0;
   dim3 grid(grid_for(ctx, (n + E - 1) / E)), block(BLOCK);
-  if (!is_float(in_dt) && !is_float(out_dt))  // integer -> integer: keep the low bits
-    hipLaunchKernelGGL((as_type_kernel<int64_t>), grid, block, 0, ctx->stream, inb->ptr, out->ptr, in_dt, out_dt, n, mx, mn);
+#define HIPNX_AS(CT, I, O) hipLaunchKernelGGL((as_type_kernel<CT, I, O>), grid, block, 0, ctx->stream, inb->ptr, out->ptr, in_dt, out_dt, n, mx, mn)
+  // the conversions of mixed-precision work, compiled for their two types
+  if (in_dt == HIPNX_F32 && out_dt == HIPNX_BF16) HIPNX_AS(float, HIPNX_F32, HIPNX_BF16);
+  else if (in_dt == HIPNX_BF16 && out_dt == HIPNX_F32) HIPNX_AS(float, HIPNX_BF16, HIPNX_F32);
+  else if (in_dt == HIPNX_F32 && out_dt == HIPNX_BF16_RNE) HIPNX_AS(float, HIPNX_F32, HIPNX_BF16_RNE);
+  else if (in_dt == HIPNX_F16 && out_dt == HIPNX_F32) HIPNX_AS(float, HIPNX_F16, HIPNX_F32);
+  else if (in_dt == HIPNX_F32 && out_dt == HIPNX_F16) HIPNX_AS(double, HIPNX_F32, HIPNX_F16);
+  else if (in_dt == HIPNX_S32 && out_dt == HIPNX_F32) HIPNX_AS(double, HIPNX_S32, HIPNX_F32);
+  else if (in_dt == HIPNX_U8 && out_dt == HIPNX_F32) HIPNX_AS(double, HIPNX_U8, HIPNX_F32);
+  else if (in_dt == HIPNX_F32 && out_dt == HIPNX_F64) HIPNX_AS(double, HIPNX_F32, HIPNX_F64);
+  else if (in_dt == HIPNX_F64 && out_dt == HIPNX_F32) HIPNX_AS(double, HIPNX_F64, HIPNX_F32);
+  else if (!is_float(in_dt) && !is_float(out_dt))  // integer -> integer: keep the low bits
+    HIPNX_AS(int64_t, -1, -1);
   else if (!is_float(in_dt) || in_dt == HIPNX_F64 || out_dt == HIPNX_F64 || out_dt == HIPNX_F16)
     // integer -> float decodes to f64 (exact below 2^53, u64 read as unsigned), then one rounding
-    hipLaunchKernelGGL((as_type_kernel<double>), grid, block, 0, ctx->stream, inb->ptr, out->ptr, in_dt, out_dt, n, mx, mn);
+    HIPNX_AS(double, -1, -1);
   else
-    hipLaunchKernelGGL((as_type_kernel<float>), grid, block, 0, ctx->stream, inb->ptr, out->ptr, in_dt, out_dt, n, mx, mn);
+    HIPNX_AS(float, -1, -1);
+#undef HIPNX_AS
   HIPNX_HIP(hipGetLastError());
   return HIPNX_OK;
 }

@@ -65,6 +65,80 @@ transpose2d_kernel(const T *__restrict__ in, T *__restrict__ out, int64_t R, int
   }
 }
 
+// The same with 16-byte accesses on both sides, for R and C that are multiples of 16 / sizeof(T) elements
+// and 16-byte aligned buffers: a lane loads V = 16 / sizeof(T) elements along C (a tile row is 128 bytes or
+// more: whole cache lines), the tile goes to LDS row by row with an odd pitch in words, and a lane then
+// collects V elements down a column -- V consecutive elements of an output row -- and stores them as one
+// 16-byte vector; lanes run along the output row, so a store instruction writes whole lines too.  The
+// one-element-per-lane kernel above moves 128 bytes (2-byte elements) per wave instruction.
+template <typename T>
+__global__ void __launch_bounds__(BLOCK)
+transpose2d_vec_kernel(const T *__restrict__ in, T *__restrict__ out, int64_t R, int64_t C, int64_t tiles_r,
+                       int64_t tiles_c) {
+  constexpr int S = sizeof(T), V = 16 / S, TILE = S <= 2 ? 128 : 64, CH = TILE / V;  // CH vectors per tile row
+  constexpr int PITCH = TILE * S / 4 + (S == 8 ? 2 : 1);                           // words per tile row in LDS
+  constexpr int RPP = BLOCK / CH;                                                    // tile rows per pass
+  __shared__ uint32_t lds[TILE * PITCH];
+  int64_t t = blockIdx.x;
+  const int64_t tc = t % tiles_c;
+  t /= tiles_c;
+  const int64_t tr = t % tiles_r, b = t / tiles_r;
+  const T *src = in + b * R * C;
+  T *dst = out + b * R * C;
+  const int q = threadIdx.x % CH, j0 = threadIdx.x / CH;
+#pragma unroll
+  for (int p = 0; p < TILE / RPP; p++) {
+    const int j = j0 + p * RPP;
+    const int64_t r = tr * TILE + j, c = tc * TILE + q * V;
+    if (r < R && c < C) {
+      const uint4 v = *reinterpret_cast<const uint4 *>(src + r * C + c);
+      uint32_t *w = lds + j * PITCH + q * 4;
+      w[0] = v.x; w[1] = v.y; w[2] = v.z; w[3] = v.w;
+    }
+  }
+  __syncthreads();
+  if constexpr (S >= 4) {
+    const T *cell = reinterpret_cast<const T *>(lds);
+#pragma unroll
+    for (int p = 0; p < TILE / RPP; p++) {
+      const int cc = j0 + p * RPP;  // tile column = output row
+      const int64_t c = tc * TILE + cc, r = tr * TILE + q * V;
+      if (c < C && r < R) {
+        T e[V];
+#pragma unroll
+        for (int k = 0; k < V; k++) e[k] = cell[(size_t)(q * V + k) * (PITCH * 4 / S) + cc];
+        *reinterpret_cast<uint4 *>(dst + c * R + r) = *reinterpret_cast<const uint4 *>(e);
+      }
+    }
+  } else {
+    // elements narrower than a word: a lane reads whole words down a group of G = 4 / S adjacent columns
+    // (V word reads instead of G * V element reads) and takes them apart into G output vectors
+    constexpr int G = 4 / S;
+#pragma unroll
+    for (int p = 0; p < TILE / (RPP * G); p++) {
+      const int cg = j0 + p * RPP;  // group of G tile columns = G output rows
+      const int64_t c = tc * TILE + (int64_t)cg * G, r = tr * TILE + q * V;
+      if (c < C && r < R) {
+        uint32_t w[V];
+#pragma unroll
+        for (int k = 0; k < V; k++) w[k] = lds[(q * V + k) * PITCH + cg];
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+          uint32_t o[4];
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            uint32_t x = 0;
+#pragma unroll
+            for (int e = 0; e < G; e++) x |= ((w[i * G + e] >> (8 * S * g)) & ((1u << (8 * S)) - 1u)) << (8 * S * e);
+            o[i] = x;
+          }
+          if (c + g < C) *reinterpret_cast<uint4 *>(dst + (c + g) * R + r) = *reinterpret_cast<const uint4 *>(o);
+        }
+      }
+    }
+  }
+}
+
 // gather: tuple i of `idx` ([n_tuples, depth]) selects a slice of `slice_bytes` bytes.
 // LPR lanes (a power of two, at most one wavefront) copy one slice with 16-byte (VEC) or 1-byte
 // accesses, four independent accesses in flight per lane; a 256-lane block works on 256/LPR
@@ -146,6 +220,13 @@ static int strided_copy(const hipnx_ctx *ctx, int elem_bytes, const void *in, vo
 
 template <typename T>
 static void launch_t2d(const hipnx_ctx *ctx, const void *in, void *out, int64_t B, int64_t R, int64_t C) {
+  constexpr int V = 16 / (int)sizeof(T), TILE = sizeof(T) <= 2 ? 128 : 64;
+  if (R % V == 0 && C % V == 0 && (((uintptr_t)in | (uintptr_t)out) & 15) == 0) {
+    const int64_t vr = (R + TILE - 1) / TILE, vc = (C + TILE - 1) / TILE;
+    hipLaunchKernelGGL((transpose2d_vec_kernel<T>), dim3((unsigned)(B * vr * vc)), dim3(BLOCK), 0, ctx->stream,
+                       (const T *)in, (T *)out, R, C, vr, vc);
+    return;
+  }
   int64_t tr = (R + 63) / 64, tc = (C + 63) / 64;
   hipLaunchKernelGGL((transpose2d_kernel<T>), dim3((unsigned)(B * tr * tc)), dim3(BLOCK), 0, ctx->stream,
                      (const T *)in, (T *)out, R, C, tr, tc);

@@ -55,11 +55,14 @@ select_nd_kernel(const void *__restrict__ p, const void *__restrict__ t, const v
   }
 }
 
-// all three operands dense (step 1) or a single element (step 0)
-template <typename CT>
+// all three operands dense (step 1) or a single element (step 0).  FIX >= 0: a u8 predicate and this
+// element type for both values and the result, known when the kernel is compiled (the run-time type
+// switches of the vector loads and the store fold away).
+template <typename CT, int FIX = -1>
 __global__ void __launch_bounds__(BLOCK)
 select_vec_kernel(const void *__restrict__ p, const void *__restrict__ t, const void *__restrict__ f, void *__restrict__ out,
-                  int pdt, int tdt, int fdt, int odt, int64_t n, int pstep, int tstep, int fstep) {
+                  int pdt_, int tdt_, int fdt_, int odt_, int64_t n, int pstep, int tstep, int fstep) {
+  const int pdt = FIX >= 0 ? HIPNX_U8 : pdt_, tdt = FIX >= 0 ? FIX : tdt_, fdt = FIX >= 0 ? FIX : fdt_, odt = FIX >= 0 ? FIX : odt_;
   const int64_t nvec = (n + E - 1) / E;
   for (int64_t v = (int64_t)blockIdx.x * BLOCK + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * BLOCK) {
     const int64_t i0 = v * E;
@@ -132,10 +135,11 @@ __device__ inline CT clip_one(CT x, CT lo, CT hi, bool xu, bool lou, bool hiu) {
   }
 }
 
-template <typename CT>
+template <typename CT, int FIX = -1>  // FIX >= 0: the element type of input and result, known at compile time
 __global__ void __launch_bounds__(BLOCK)
 clip_kernel(const void *__restrict__ in, const void *__restrict__ mn, const void *__restrict__ mx, void *__restrict__ out,
-            int idt, int mndt, int mxdt, int odt, int64_t n) {
+            int idt_, int mndt, int mxdt, int odt_, int64_t n) {
+  const int idt = FIX >= 0 ? FIX : idt_, odt = FIX >= 0 ? FIX : odt_;
   const CT lo = load_one<CT>(mn, mndt, 0), hi = load_one<CT>(mx, mxdt, 0);
   const bool xu = idt == HIPNX_U64, lou = mndt == HIPNX_U64, hiu = mxdt == HIPNX_U64;
   const int64_t nvec = (n + E - 1) / E;
@@ -286,12 +290,18 @@ extern "C" int hipnx_select(hipnx_ctx *ctx, int pred_dt, int true_dt, int false_
   const bool narrow = narrow_float(true_dt) && narrow_float(false_dt) && narrow_float(out_dt);
   if (m == 1 && s.ps[0] <= 1 && s.ts[0] <= 1 && s.fs[0] <= 1) {
     dim3 grid(grid_for((n + E - 1) / E)), block(BLOCK);
-    if (narrow) hipLaunchKernelGGL((select_vec_kernel<float>), grid, block, 0, ctx->stream, pred->ptr, on_true->ptr, on_false->ptr, out->ptr,
-                                   pred_dt, true_dt, false_dt, out_dt, n, (int)s.ps[0], (int)s.ts[0], (int)s.fs[0]);
-    else if (fl) hipLaunchKernelGGL((select_vec_kernel<double>), grid, block, 0, ctx->stream, pred->ptr, on_true->ptr, on_false->ptr, out->ptr,
-                               pred_dt, true_dt, false_dt, out_dt, n, (int)s.ps[0], (int)s.ts[0], (int)s.fs[0]);
-    else hipLaunchKernelGGL((select_vec_kernel<int64_t>), grid, block, 0, ctx->stream, pred->ptr, on_true->ptr, on_false->ptr, out->ptr,
-                            pred_dt, true_dt, false_dt, out_dt, n, (int)s.ps[0], (int)s.ts[0], (int)s.fs[0]);
+#define HIPNX_SELECT(CT, FIX) hipLaunchKernelGGL((select_vec_kernel<CT, FIX>), grid, block, 0, ctx->stream, pred->ptr, on_true->ptr, on_false->ptr, out->ptr, \
+                                               pred_dt, true_dt, false_dt, out_dt, n, (int)s.ps[0], (int)s.ts[0], (int)s.fs[0])
+    const bool one_type = pred_dt == HIPNX_U8 && true_dt == out_dt && false_dt == out_dt;
+    if (one_type && out_dt == HIPNX_F32) HIPNX_SELECT(float, HIPNX_F32);
+    else if (one_type && out_dt == HIPNX_BF16) HIPNX_SELECT(float, HIPNX_BF16);
+    else if (one_type && out_dt == HIPNX_F16) HIPNX_SELECT(float, HIPNX_F16);
+    else if (one_type && out_dt == HIPNX_S32) HIPNX_SELECT(int64_t, HIPNX_S32);
+    else if (one_type && out_dt == HIPNX_S64) HIPNX_SELECT(int64_t, HIPNX_S64);
+    else if (narrow) HIPNX_SELECT(float, -1);
+    else if (fl) HIPNX_SELECT(double, -1);
+    else HIPNX_SELECT(int64_t, -1);
+#undef HIPNX_SELECT
   } else {
     dim3 grid(grid_for(n)), block(BLOCK);
     if (fl) hipLaunchKernelGGL((select_nd_kernel<double>), grid, block, 0, ctx->stream, pred->ptr, on_true->ptr, on_false->ptr, out->ptr,
@@ -318,12 +328,16 @@ extern "C" int hipnx_clip(hipnx_ctx *ctx, int in_dt, int min_dt, int max_dt, int
   if (int st = check_buf(ctx, out, (uint64_t)n * dtype_size(out_dt), "clip out")) return st;
   if (n == 0) return HIPNX_OK;
   dim3 grid(grid_for((n + E - 1) / E)), block(BLOCK);
-  if (narrow_float(in_dt) && narrow_float(min_dt) && narrow_float(max_dt) && narrow_float(out_dt))
-    hipLaunchKernelGGL((clip_kernel<float>), grid, block, 0, ctx->stream, inb->ptr, min->ptr, max->ptr, out->ptr, in_dt, min_dt, max_dt, out_dt, n);
-  else if (is_float(out_dt))
-    hipLaunchKernelGGL((clip_kernel<double>), grid, block, 0, ctx->stream, inb->ptr, min->ptr, max->ptr, out->ptr, in_dt, min_dt, max_dt, out_dt, n);
-  else
-    hipLaunchKernelGGL((clip_kernel<int64_t>), grid, block, 0, ctx->stream, inb->ptr, min->ptr, max->ptr, out->ptr, in_dt, min_dt, max_dt, out_dt, n);
+#define HIPNX_CLIP(CT, FIX) hipLaunchKernelGGL((clip_kernel<CT, FIX>), grid, block, 0, ctx->stream, inb->ptr, min->ptr, max->ptr, out->ptr, in_dt, min_dt, max_dt, out_dt, n)
+  if (narrow_float(in_dt) && narrow_float(min_dt) && narrow_float(max_dt) && narrow_float(out_dt)) {
+    if (in_dt == out_dt && out_dt == HIPNX_F32) HIPNX_CLIP(float, HIPNX_F32);
+    else if (in_dt == out_dt && out_dt == HIPNX_BF16) HIPNX_CLIP(float, HIPNX_BF16);
+    else if (in_dt == out_dt && out_dt == HIPNX_F16) HIPNX_CLIP(float, HIPNX_F16);
+    else HIPNX_CLIP(float, -1);
+  } else if (is_float(out_dt)) HIPNX_CLIP(double, -1);
+  else if (in_dt == out_dt && out_dt == HIPNX_S32) HIPNX_CLIP(int64_t, HIPNX_S32);
+  else HIPNX_CLIP(int64_t, -1);
+#undef HIPNX_CLIP
   HIPNX_HIP(hipGetLastError());
   return HIPNX_OK;
 }
