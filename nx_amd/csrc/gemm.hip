@@ -167,6 +167,29 @@ extern "C" int hipnx_transpose(hipnx_ctx *ctx, int elem_bytes, int rank, const i
                                const hipnx_buf *inb, hipnx_buf *out);
 
 // scale_mode != NONE: the scaled form (out_dt is then f32 over an s32 sum)
+// Second pass of a contraction whose K was split over S work-groups per tile: out[i] = the S partial
+// results of element i added in split order (f32 adds for the float types, wrapping 32-bit adds -- exact --
+// for int8), then encoded once.
+template <typename AT>
+__global__ void __launch_bounds__(256)
+splitk_combine_kernel(const AT *__restrict__ part, void *__restrict__ out, int odt, int64_t mn, int splits) {
+  typedef typename std::conditional<std::is_same<AT, float>::value, float, int64_t>::type CT;
+  const int64_t nvec = mn / 4;
+  for (int64_t v = (int64_t)blockIdx.x * 256 + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * 256) {
+    typedef __attribute__((ext_vector_type(4))) AT vec_t;
+    vec_t acc = *reinterpret_cast<const vec_t *>(part + v * 4);
+    for (int s = 1; s < splits; s++) {
+      const vec_t p = *reinterpret_cast<const vec_t *>(part + s * mn + v * 4);
+#pragma unroll
+      for (int e = 0; e < 4; e++) acc[e] += p[e];
+    }
+    CT x[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) x[e] = (CT)acc[e];
+    store_vec<CT, 4>(out, odt, v * 4, x);
+  }
+}
+
 static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batch, int64_t M, int64_t N,
                     int64_t K, int l_layout, int r_layout, const hipnx_buf *l, const hipnx_buf *r,
                     hipnx_buf *out, int scale_mode, const hipnx_buf *scale) {
@@ -269,7 +292,45 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
         if (M <= 64) cfg = GEMM_CFG_64x32;
         else if (t256 * 4 >= (int64_t)ctx->num_cus * 3 && M >= 192 && N >= 192) cfg = GEMM_CFG_256;
         else cfg = GEMM_CFG_128;
-        if (M <= 64 && l_kin && r_kin && Kb % 4096 == 0 && N >= 256) {
+        // A grid of 128 x 128 tiles that leaves most CUs idle (a few hundred rows against a long weight
+        // matrix: 128 x 4096 x 4096 is 32 tiles walking 64 slabs each) splits K over S work-groups per tile:
+        // f32 (s32) partial results in pool workspace, then one pass that adds them in split order.
+        int splits = 1;
+        const int64_t t128 = ((M + 127) / 128) * ((N + 127) / 128);
+        const int64_t nslab = Kb / SLAB;
+        const bool splittable = cfg == GEMM_CFG_128 && batch == 1 && scale_mode == HIPNX_SCALE_NONE && (M * N) % 4 == 0 &&
+                                (l_dt == HIPNX_S8 ? !is_float(out_dt) : true);
+        // (the second pass and the partial results cost about 12 us: worth it from K = 32 slabs on, with at
+        // least 8 slabs left per split)
+        if (splittable && t128 * 2 <= ctx->num_cus && nslab >= 32)
+          for (int cand = 16; cand >= 2; cand /= 2)
+            if (t128 * cand <= 2 * (int64_t)ctx->num_cus && nslab % cand == 0 && nslab / cand >= 8) { splits = cand; break; }
+        void *ws = nullptr;
+        size_t ws_cap = 0;
+        if (splits > 1 && pool_alloc(ctx, (size_t)splits * M * N * 4, &ws, &ws_cap) != HIPNX_OK) splits = 1;
+        if (splits > 1) {
+          GemmArgs p = a;
+          p.Kb = Kb / splits;
+          p.bs_l = l_kin ? p.Kb : (p.Kb / esz) * a.ld_l;  // split s begins p.Kb bytes (or that many k-rows) further on
+          p.bs_r = r_kin ? p.Kb : (p.Kb / esz) * a.ld_r;
+          p.out = ws;
+          p.odt = l_dt == HIPNX_S8 ? HIPNX_S32 : HIPNX_F32;
+          switch (l_dt) {
+            case HIPNX_BF16: st = launch_gemm_bf16(ctx, cfg, l_kin, r_kin, p, splits); break;
+            case HIPNX_F16: st = launch_gemm_f16(ctx, cfg, l_kin, r_kin, p, splits); break;
+            case HIPNX_F32: st = launch_gemm_f32(ctx, cfg, l_kin, r_kin, p, splits); break;
+            default: st = launch_gemm_s8(ctx, cfg, l_kin, r_kin, p, splits); break;
+          }
+          if (!st) {
+            const int64_t mn = M * N;
+            dim3 grid((unsigned)std::min<int64_t>((mn / 4 + 255) / 256, 1 << 20)), block(256);
+            if (l_dt == HIPNX_S8) hipLaunchKernelGGL((splitk_combine_kernel<int>), grid, block, 0, ctx->stream, (const int *)ws, out->ptr, out_dt, mn, splits);
+            else hipLaunchKernelGGL((splitk_combine_kernel<float>), grid, block, 0, ctx->stream, (const float *)ws, out->ptr, out_dt, mn, splits);
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess) st = hip_fail(e, "split-K combine launch");
+          }
+          pool_free(ctx, ws, ws_cap);  // later work is ordered on the same stream
+        } else if (M <= 64 && l_kin && r_kin && Kb % 4096 == 0 && N >= 256) {
           st = launch_gemm_rows(ctx, l_dt, a, batch);  // weights streamed once, never through LDS
         } else
         switch (l_dt) {

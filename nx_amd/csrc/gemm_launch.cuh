@@ -72,7 +72,19 @@ static int launch_cfg(const hipnx_ctx *ctx, int cfg, const GemmArgs &a, int64_t 
         if (a.ld_l < (1ll << 23) && a.ld_r < (1ll << 23)) return launch_pingpong<DT, LK, RK>(ctx, a, batch);
       }
       return launch_one<DT, 4, 2, 2, 4, LK, RK>(ctx, a, batch);
-    case GEMM_CFG_128: return launch_one<DT, 2, 2, 2, 2, LK, RK>(ctx, a, batch);
+    case GEMM_CFG_128: {
+      // one wave per SIMD and 0.25 us of MFMA work per slab: two stages cannot cover the latency of the next
+      // slab's requests (measured 2100 clocks per slab, 1580 with four stages); four stages where every
+      // operand is copied straight into LDS (the condition of the kernel's L_TR / R_TR)
+      constexpr int ES = DT == HIPNX_S8 ? 1 : DT == HIPNX_F32 ? 4 : 2;
+      constexpr bool tr = ES <= 2 && 128 * ES >= 256;
+      if constexpr ((LK || tr) && (RK || tr)) {
+        // (128 KiB of LDS: one work-group per CU, so only where the grid has no second one to give it)
+        const int64_t groups = ((a.M + 127) / 128) * ((a.N + 127) / 128) * batch;
+        if (a.Kb >= 4 * SLAB && groups <= ctx->num_cus) return launch_one<DT, 2, 2, 2, 2, LK, RK, 4>(ctx, a, batch);
+      }
+      return launch_one<DT, 2, 2, 2, 2, LK, RK>(ctx, a, batch);
+    }
     default:
       // streaming a long weight matrix past a few rows is bound by the bytes in flight: six
       // stages (five slabs of 12 KiB requested ahead per work-group) when both operands are copied
