@@ -284,6 +284,15 @@ def main():
         sbt = Nx.transpose(sb)
         _, ms = tstat(lambda: Nx.dot(sa, [1], sbt, [1], out_type="s32"), steps, warm, msettle)
         entry("dot_s8_4096_s32_kinner", flop, "TOP/s", ms, PEAK["s8"], "mfma", "mfma_s8")
+        # a serving batch against one weight matrix (bound by the 33.5 MB of weights; K is split over the
+        # work-groups of the under-filled grid) and a mid-size square (one 128 x 128 tile per CU)
+        xa, wb = put(a_np[:128].copy(), "bf16"), bt
+        _, ms = tstat(lambda: Nx.dot(xa, [1], wb, [1]), steps, warm)
+        entry("dot_bf16_128x4096x4096", 2.0 * (128 * 4096 * 2) + 4096 * 4096 * 2.0, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read")
+        ma, mb = put(a_np[:2048, :2048].copy(), "bf16"), put(b_np[:2048, :2048].copy(), "bf16")
+        _, ms = tstat(lambda: Nx.dot(ma, mb), steps, warm)
+        entry("dot_bf16_2048", 2.0 * 2048 ** 3, "TFLOP/s", ms, PEAK["bf16"], "mfma", "mfma_bf16")
+        del xa, wb, ma, mb
         ha, hb = put(W.bf16_to_f32(a_np).astype(np.float16), "f16"), put(W.bf16_to_f32(b_np).astype(np.float16), "f16")
         _, ms = tstat(lambda: Nx.dot(ha, hb), steps, warm, msettle)
         entry("dot_f16_4096", flop, "TFLOP/s", ms, PEAK["f16"], "mfma", "mfma_f16")
