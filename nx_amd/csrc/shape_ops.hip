@@ -183,9 +183,13 @@ copy_nd_kernel(const T *__restrict__ in, T *__restrict__ out, int64_t n, Copy c)
 // IT is the type the coordinates are counted in: 32-bit when the tensor has fewer than 2^31 elements
 // (so the integer -> float conversion is one instruction and exact-or-nearest-even like the
 // reference's integer written as a float, nx/lib/nx/binary_backend.ex:49-75), 64-bit otherwise.
-template <typename CT, typename IT>
+// ODT >= 0: the result's element type, known when the kernel is compiled; EV elements per lane (4 for an
+// 8-byte type: 32 bytes per lane -- with 8 each of a lane's four stores would land in a quarter of a line).
+template <typename CT, typename IT, int ODT = -1, int EV = 8>
 __global__ void __launch_bounds__(BLOCK)
-iota_kernel(void *__restrict__ out, int odt, int64_t n, int64_t dim_, int64_t inner_, int mode) {
+iota_kernel(void *__restrict__ out, int odt_, int64_t n, int64_t dim_, int64_t inner_, int mode) {
+  constexpr int E = EV;
+  const int odt = ODT >= 0 ? ODT : odt_;
   const int64_t nvec = (n + E - 1) / E;
   const IT dim = (IT)dim_, inner = (IT)inner_;
   for (int64_t v = (int64_t)blockIdx.x * BLOCK + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * BLOCK) {
@@ -421,19 +425,22 @@ static int iota_like(hipnx_ctx *ctx, int out_dt, int64_t n, int64_t dim, int64_t
   if (n < 0 || dim < 1 || inner < 1) return set_error(HIPNX_EINVAL, "%s: bad extents", what);
   if (int st = check_buf(ctx, out, (uint64_t)n * dtype_size(out_dt), what)) return st;
   if (n == 0) return HIPNX_OK;
-  dim3 grid(grid_for((n + E - 1) / E)), block(BLOCK);
+  dim3 block(BLOCK);
   // an extent beyond the element count never wraps: clamp it so that it fits the counter type
   if (dim > n) dim = n;
   if (inner > n) inner = n;
   const bool small = n < (1ll << 31);
-  if (small && is_float(out_dt) && out_dt != HIPNX_F64)
-    hipLaunchKernelGGL((iota_kernel<float, int32_t>), grid, block, 0, ctx->stream, out->ptr, out_dt, n, dim, inner, mode);
-  else if (is_float(out_dt))
-    hipLaunchKernelGGL((iota_kernel<double, int64_t>), grid, block, 0, ctx->stream, out->ptr, out_dt, n, dim, inner, mode);
-  else if (small)
-    hipLaunchKernelGGL((iota_kernel<int64_t, int32_t>), grid, block, 0, ctx->stream, out->ptr, out_dt, n, dim, inner, mode);
-  else
-    hipLaunchKernelGGL((iota_kernel<int64_t, int64_t>), grid, block, 0, ctx->stream, out->ptr, out_dt, n, dim, inner, mode);
+#define HIPNX_IOTA(CT, IT, ODT, EV) hipLaunchKernelGGL((iota_kernel<CT, IT, ODT, EV>), dim3(grid_for((n + EV - 1) / EV)), block, 0, ctx->stream, out->ptr, out_dt, n, dim, inner, mode)
+  if (small && out_dt == HIPNX_F32) HIPNX_IOTA(float, int32_t, HIPNX_F32, 8);
+  else if (small && out_dt == HIPNX_BF16) HIPNX_IOTA(float, int32_t, HIPNX_BF16, 8);
+  else if (small && out_dt == HIPNX_S32) HIPNX_IOTA(int64_t, int32_t, HIPNX_S32, 8);
+  else if (small && out_dt == HIPNX_S64) HIPNX_IOTA(int64_t, int32_t, HIPNX_S64, 4);
+  else if (small && out_dt == HIPNX_U8) HIPNX_IOTA(int64_t, int32_t, HIPNX_U8, 8);
+  else if (small && is_float(out_dt) && out_dt != HIPNX_F64) HIPNX_IOTA(float, int32_t, -1, 8);
+  else if (is_float(out_dt)) HIPNX_IOTA(double, int64_t, -1, 8);
+  else if (small) HIPNX_IOTA(int64_t, int32_t, -1, 8);
+  else HIPNX_IOTA(int64_t, int64_t, -1, 8);
+#undef HIPNX_IOTA
   HIPNX_HIP(hipGetLastError());
   return HIPNX_OK;
 }
