@@ -193,6 +193,44 @@ gather_kernel(const unsigned char *__restrict__ t, const void *__restrict__ idx,
   }
 }
 
+// The same with one 16-byte vector of the OUTPUT per lane, for an innermost output axis that is a multiple of
+// V = 16 / sizeof(T) elements (`s.dims[rank - 1]` counts vectors here): the index is taken apart once per
+// vector, the V inputs are one 16-byte load (inner stride 1, aligned), one element repeated (inner stride 0:
+// a column or a scalar broadcast along rows) or V loads, and the store is whole.  One element per lane is
+// bound by instructions, not bytes: broadcasting to 16384^2 took 335-500 us whatever the element size.
+template <typename T>
+__global__ void __launch_bounds__(BLOCK)
+strided_copy_vec_kernel(const T *__restrict__ in, T *__restrict__ out, int64_t nvec, Strided s, int64_t inner_stride) {
+  constexpr int V = 16 / sizeof(T);
+  for (int64_t v = (int64_t)blockIdx.x * BLOCK + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * BLOCK) {
+    int64_t rem = v, off = 0;
+    for (int a = s.rank - 1; a >= 0; a--) {
+      int64_t q, c;
+      if (rem < (1ll << 31) && s.dims[a] < (1ll << 31)) { q = (uint32_t)rem / (uint32_t)s.dims[a]; c = (uint32_t)rem - (uint32_t)q * (uint32_t)s.dims[a]; }
+      else { q = rem / s.dims[a]; c = rem - q * s.dims[a]; }
+      off += c * s.strides[a] * (a == s.rank - 1 ? V : 1);
+      rem = q;
+    }
+    T e[V];
+    if (inner_stride == 1 && ((reinterpret_cast<uintptr_t>(in + off)) & 15) == 0) {
+      *reinterpret_cast<uint4 *>(e) = *reinterpret_cast<const uint4 *>(in + off);
+    } else if (inner_stride == 0) {
+      const T x = in[off];
+#pragma unroll
+      for (int k = 0; k < V; k++) e[k] = x;
+    } else {
+#pragma unroll
+      for (int k = 0; k < V; k++) e[k] = in[off + k * inner_stride];
+    }
+    *reinterpret_cast<uint4 *>(out + v * V) = *reinterpret_cast<const uint4 *>(e);
+  }
+}
+
+// 16 bytes of the repeated element per lane
+__global__ void __launch_bounds__(BLOCK) fill16_kernel(uint4 *__restrict__ out, uint4 pattern, int64_t nvec) {
+  for (int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * BLOCK) out[i] = pattern;
+}
+
 static int grid_for(const hipnx_ctx *ctx, int64_t items, int per_block) {
   int64_t blocks = (items + per_block - 1) / per_block;
   (void)ctx;
@@ -203,6 +241,14 @@ static int grid_for(const hipnx_ctx *ctx, int64_t items, int per_block) {
 
 template <typename T>
 static void launch_strided(const hipnx_ctx *ctx, const void *in, void *out, int64_t n, const Strided &s) {
+  constexpr int V = 16 / (int)sizeof(T);
+  if (s.rank >= 1 && s.dims[s.rank - 1] % V == 0 && ((uintptr_t)out & 15) == 0) {
+    Strided sv = s;
+    sv.dims[s.rank - 1] /= V;
+    hipLaunchKernelGGL((strided_copy_vec_kernel<T>), dim3(grid_for(ctx, n / V, BLOCK)), dim3(BLOCK), 0, ctx->stream,
+                       (const T *)in, (T *)out, n / V, sv, s.strides[s.rank - 1]);
+    return;
+  }
   hipLaunchKernelGGL((strided_copy_kernel<T>), dim3(grid_for(ctx, n, BLOCK)), dim3(BLOCK), 0, ctx->stream,
                      (const T *)in, (T *)out, n, s);
 }
@@ -244,6 +290,29 @@ extern "C" int hipnx_fill(hipnx_ctx *ctx, hipnx_buf *dst, int elem_bytes, const 
     return set_error(HIPNX_EINVAL, "fill: element size %d is not 1, 2, 4 or 8", elem_bytes);
   if (int st = check_buf(ctx, dst, (uint64_t)n * elem_bytes, "fill dst")) return st;
   if (n == 0) return HIPNX_OK;
+  // whole 16-byte vectors of the repeated element first, then what is left (fewer than 16 bytes) by element
+  const int64_t nvec = ((uintptr_t)dst->ptr & 15) == 0 ? n * elem_bytes / 16 : 0;
+  if (nvec > 0) {
+    unsigned char pat[16];
+    for (int i = 0; i < 16; i += elem_bytes) std::memcpy(pat + i, elem, (size_t)elem_bytes);
+    uint4 pattern;
+    std::memcpy(&pattern, pat, 16);
+    hipLaunchKernelGGL(fill16_kernel, dim3(grid_for(ctx, nvec, BLOCK)), dim3(BLOCK), 0, ctx->stream, (uint4 *)dst->ptr, pattern, nvec);
+    const int64_t done = nvec * 16 / elem_bytes;
+    if (done == n) { HIPNX_HIP(hipGetLastError()); return HIPNX_OK; }
+    // the tail: fewer than 16 / elem_bytes elements
+    unsigned char *tail = (unsigned char *)dst->ptr + nvec * 16;
+    const int64_t left = n - done;
+    dim3 g1(1), block1(BLOCK);
+    switch (elem_bytes) {
+      case 1: hipLaunchKernelGGL((fill_kernel<uint8_t>), g1, block1, 0, ctx->stream, (uint8_t *)tail, *(const uint8_t *)elem, left); break;
+      case 2: { uint16_t v; std::memcpy(&v, elem, 2); hipLaunchKernelGGL((fill_kernel<uint16_t>), g1, block1, 0, ctx->stream, (uint16_t *)tail, v, left); break; }
+      case 4: { uint32_t v; std::memcpy(&v, elem, 4); hipLaunchKernelGGL((fill_kernel<uint32_t>), g1, block1, 0, ctx->stream, (uint32_t *)tail, v, left); break; }
+      default: { uint64_t v; std::memcpy(&v, elem, 8); hipLaunchKernelGGL((fill_kernel<uint64_t>), g1, block1, 0, ctx->stream, (uint64_t *)tail, v, left); break; }
+    }
+    HIPNX_HIP(hipGetLastError());
+    return HIPNX_OK;
+  }
   dim3 grid(grid_for(ctx, n, BLOCK)), block(BLOCK);
   switch (elem_bytes) {
     case 1: hipLaunchKernelGGL((fill_kernel<uint8_t>), grid, block, 0, ctx->stream, (uint8_t *)dst->ptr, *(const uint8_t *)elem, n); break;

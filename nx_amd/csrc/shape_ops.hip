@@ -177,6 +177,46 @@ copy_nd_kernel(const T *__restrict__ in, T *__restrict__ out, int64_t n, Copy c)
   }
 }
 
+// The innermost axis dense on the output side and dense or reversed on the input side, but not on 16-byte
+// boundaries (a slice that starts at an odd column, a padded copy, a reverse): a lane still moves V = 16 /
+// sizeof(T) elements at once -- the hardware takes 16-byte accesses at element alignment -- and only the last,
+// partial vector of a row goes by element.  `c.dims[rank - 1]` counts vectors (the row's elements rounded up),
+// `row_len` elements.  One element per lane is bound by instructions: 1.4 TB/s on a bf16 slice of 16384^2.
+template <typename T>
+struct __attribute__((packed, aligned(sizeof(T)))) run_vec {
+  T e[16 / sizeof(T)];
+};
+template <typename T>
+__global__ void __launch_bounds__(BLOCK)
+copy_runs_kernel(const T *__restrict__ in, T *__restrict__ out, int64_t nvec, Copy c, int64_t row_len, int reversed) {
+  constexpr int V = 16 / sizeof(T);
+  for (int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * BLOCK) {
+    int64_t rem = i, io = 0, oo = 0, col = 0;
+    for (int a = c.rank - 1; a >= 0; a--) {
+      int64_t q, k;
+      if (rem < (1ll << 31) && c.dims[a] < (1ll << 31)) { q = (uint32_t)rem / (uint32_t)c.dims[a]; k = (uint32_t)rem - (uint32_t)q * (uint32_t)c.dims[a]; }
+      else { q = rem / c.dims[a]; k = rem - q * c.dims[a]; }
+      if (a == c.rank - 1) col = k * V;
+      else { io += k * c.is[a]; oo += k * c.os[a]; }
+      rem = q;
+    }
+    const T *src = in + io + (reversed ? -col : col);
+    T *dst = out + oo + col;
+    if (col + V <= row_len) {
+      run_vec<T> v;
+      if (!reversed) v = *reinterpret_cast<const run_vec<T> *>(src);
+      else {
+        const run_vec<T> w = *reinterpret_cast<const run_vec<T> *>(src - (V - 1));
+#pragma unroll
+        for (int k = 0; k < V; k++) v.e[k] = w.e[V - 1 - k];
+      }
+      *reinterpret_cast<run_vec<T> *>(dst) = v;
+    } else {
+      for (int k = 0; col + k < row_len; k++) dst[k] = reversed ? src[-k] : src[k];
+    }
+  }
+}
+
 // ---- iota / eye -----------------------------------------------------------------------------
 // mode 0: out[i] = (i / inner) % dim (iota along an axis; the flat iota is inner = 1, dim = n)
 // mode 1: out[i] = 1 where (i / inner) % dim == i % inner  (eye: dim = rows, inner = columns)
@@ -407,6 +447,21 @@ extern "C" int hipnx_strided_copy(hipnx_ctx *ctx, int elem_bytes, int rank, cons
   }
   const char *src = (const char *)inb->ptr + io * eb;
   char *dst = (char *)out->ptr + oo * eb;
+  if (eb < 8 && c.os[m - 1] == 1 && (c.is[m - 1] == 1 || c.is[m - 1] == -1) && c.dims[m - 1] >= 2 * (16 / eb)) {
+    const int V = 16 / eb;
+    const int64_t row_len = c.dims[m - 1];
+    const int reversed = c.is[m - 1] < 0;
+    c.dims[m - 1] = (row_len + V - 1) / V;
+    const int64_t nvec = n / row_len * c.dims[m - 1];
+    dim3 grid(grid_for(nvec)), block(BLOCK);
+    switch (eb) {
+      case 1: hipLaunchKernelGGL((copy_runs_kernel<uint8_t>), grid, block, 0, ctx->stream, (const uint8_t *)src, (uint8_t *)dst, nvec, c, row_len, reversed); break;
+      case 2: hipLaunchKernelGGL((copy_runs_kernel<uint16_t>), grid, block, 0, ctx->stream, (const uint16_t *)src, (uint16_t *)dst, nvec, c, row_len, reversed); break;
+      default: hipLaunchKernelGGL((copy_runs_kernel<uint32_t>), grid, block, 0, ctx->stream, (const uint32_t *)src, (uint32_t *)dst, nvec, c, row_len, reversed); break;
+    }
+    HIPNX_HIP(hipGetLastError());
+    return HIPNX_OK;
+  }
   switch (eb) {
     case 1: launch_copy<uint8_t>(ctx, src, dst, n, c); break;
     case 2: launch_copy<uint16_t>(ctx, src, dst, n, c); break;
