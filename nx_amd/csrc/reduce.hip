@@ -1,289 +1,9 @@
-// Axis reductions: sum / product / reduce_max / reduce_min and argmax / argmin.
-//
-// The input is viewed as [outer, red, inner].
-//   inner == 1  ("rows"):    the reduced axis is contiguous.  One wavefront (short rows) or one
-//                            256-lane block (long rows) per row streams it with 16-byte loads,
-//                            folds in registers, then combines across lanes with wave shuffles
-//                            and across the block's 4 waves through LDS.  A few very long rows
-//                            are split into segments and finished by a second tiny kernel.
-//   inner  > 1  ("columns"): lanes run along `inner` (coalesced), each walks `red` serially.
-// Accumulators: floats sum in f64 (the reference folds in f64 and rounds once,
-// nx/lib/nx/binary_backend.ex:1315-1324, 2342-2360; any f64 summation order rounds to the same
-// f32 except in rare half-ulp cases), integers in wrapping 64-bit (exact low bits).
-// Max/min keep NaN sticky (binary_backend.ex:1349-1375); arg-reductions carry (value, index)
-// pairs whose combine rule is associative and commutative, so the tree order cannot change the
-// answer: a NaN beats every number and the larger index wins among NaNs (the reference's
-// sequential scan lets every NaN replace the current extreme, binary_backend.ex:1419-1427);
-// otherwise the better value wins and equal values resolve to the smaller (tie LOW) or larger
-// (tie HIGH) index.
-// Algorithmic traffic: bytes(in) + bytes(out).
-#include <type_traits>
-#include <utility>
-
-#include "internal.h"
-#include "reduce_ops.cuh"
+// Axis reductions: the entry points of sum / product / reduce_max / reduce_min / all / any (kernels and their
+// launcher: reduce_kernels.cuh).  The operations are compiled in two units (this one: sum and product; the
+// selections in reduce_select.hip) so that the build runs in parallel.
+#include "reduce_kernels.cuh"
 
 namespace hipnx {
-
-// ---- rows: inner == 1 -----------------------------------------------------------------------
-// TPR lanes per row (64 or 256); a block of 256 lanes covers 256/TPR rows.  Row `row` segment
-// `seg` covers elements [seg*seg_len, min(red, (seg+1)*seg_len)).  With nseg == 1 the result is
-// encoded into `out`; otherwise the raw accumulator goes to `partial[row*nseg + seg]`.
-// IDT >= 0: the input's element type, known when the kernel is compiled (the type switch inside every
-// vector load, and the scalar bookkeeping the compiler builds around it, fold away); -1: read from `idt_`.
-template <typename R, typename CT, int TPR, bool VEC, int IDT = -1>
-__global__ void __launch_bounds__(BLOCK)
-reduce_rows_kernel(const void *__restrict__ in, void *__restrict__ out, typename R::acc_t *__restrict__ partial,
-                   int idt_, int odt, int64_t rows, int64_t red, int64_t seg_len, int nseg) {
-  const int idt = IDT >= 0 ? IDT : idt_;
-  constexpr int RPB = BLOCK / TPR;
-  const int sub = threadIdx.x / TPR, lane = threadIdx.x % TPR;
-  const int64_t unit = (int64_t)blockIdx.x * RPB + sub;  // (row, seg) pair
-  const int64_t row = unit / nseg;
-  const int seg = (int)(unit - row * nseg);
-  typename R::acc_t acc = R::init();
-  if (row < rows) {
-    const int64_t k0 = (int64_t)seg * seg_len;
-    const int64_t k1 = k0 + seg_len < red ? k0 + seg_len : red;
-    const int64_t base = row * red;
-    if constexpr (VEC) {  // red % E == 0 and seg_len % E == 0: every vector is aligned
-      // two (then one) 8-element vectors per step: both loads are issued before either is folded
-      int64_t k = k0 + (int64_t)lane * E;
-      if (k < k1) acc = R::seed(acc, k);
-      const int64_t step = (int64_t)TPR * E;
-      for (; k + step < k1; k += 2 * step) {
-        CT v[E], w[E];
-        load_vec<CT, E>(in, idt, base + k, v);
-        load_vec<CT, E>(in, idt, base + k + step, w);
-#pragma unroll
-        for (int i = 0; i < E; i++) acc = R::accumulate(acc, v[i], k + i);
-#pragma unroll
-        for (int i = 0; i < E; i++) acc = R::accumulate(acc, w[i], k + step + i);
-      }
-      for (; k < k1; k += step) {
-        CT v[E];
-        load_vec<CT, E>(in, idt, base + k, v);
-#pragma unroll
-        for (int i = 0; i < E; i++) acc = R::accumulate(acc, v[i], k + i);
-      }
-    } else {
-      if (k0 + lane < k1) acc = R::seed(acc, k0 + lane);
-      for (int64_t k = k0 + lane; k < k1; k += TPR) acc = R::accumulate(acc, load_one<CT>(in, idt, base + k), k);
-    }
-  }
-  acc = wave_reduce<R>(acc);
-  if constexpr (TPR > WAVE) {
-    __shared__ typename R::acc_t sm[BLOCK / WAVE];
-    if (threadIdx.x % WAVE == 0) sm[threadIdx.x / WAVE] = acc;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-#pragma unroll
-      for (int w = 1; w < BLOCK / WAVE; w++) acc = R::combine(acc, sm[w]);
-    }
-  }
-  if (lane == 0 && row < rows) {
-    if (nseg == 1) finalize(out, odt, row, acc);
-    else partial[row * nseg + seg] = acc;
-  }
-}
-
-// second pass of a split row reduction: one wave per row folds its nseg partials
-template <typename R>
-__global__ void __launch_bounds__(BLOCK)
-combine_partials_kernel(const typename R::acc_t *__restrict__ partial, void *__restrict__ out, int odt, int64_t rows,
-                        int nseg) {
-  const int64_t row = (int64_t)blockIdx.x * (BLOCK / WAVE) + threadIdx.x / WAVE;
-  const int lane = threadIdx.x % WAVE;
-  typename R::acc_t acc = R::init();
-  if (row < rows)
-    for (int s = lane; s < nseg; s += WAVE) acc = R::combine(acc, partial[row * nseg + s]);
-  acc = wave_reduce<R>(acc);
-  if (lane == 0 && row < rows) finalize(out, odt, row, acc);
-}
-
-// ---- columns: inner > 1 ---------------------------------------------------------------------
-// One lane per E adjacent inner positions (VEC) or per position; walks k in its segment.
-// With nseg == 1 results are encoded into out[outer, inner]; otherwise raw accumulators go to
-// partial[outer, nseg, inner].
-template <typename R, typename CT, bool VEC, int IDT = -1>
-__global__ void __launch_bounds__(BLOCK)
-reduce_cols_kernel(const void *__restrict__ in, void *__restrict__ out, typename R::acc_t *__restrict__ partial,
-                   int idt_, int odt, int64_t outer, int64_t red, int64_t inner, int64_t seg_len, int nseg) {
-  const int idt = IDT >= 0 ? IDT : idt_;
-  constexpr int W = VEC ? E : 1;
-  const int64_t ivecs = inner / W;
-  const int64_t total = outer * nseg * ivecs;
-  for (int64_t t = (int64_t)blockIdx.x * BLOCK + threadIdx.x; t < total; t += (int64_t)gridDim.x * BLOCK) {
-    const int64_t iv = t % ivecs, os = t / ivecs;
-    const int64_t o = os / nseg;
-    const int seg = (int)(os - o * nseg);
-    const int64_t k0 = (int64_t)seg * seg_len, k1 = k0 + seg_len < red ? k0 + seg_len : red;
-    typename R::acc_t acc[W];
-#pragma unroll
-    for (int i = 0; i < W; i++) acc[i] = k0 < k1 ? R::seed(R::init(), k0) : R::init();
-    const int64_t base = o * red * inner + iv * W;
-    int64_t k = k0;
-    for (; k + 3 < k1; k += 4) {  // four independent row loads in flight per lane
-      CT v0[W], v1[W], v2[W], v3[W];
-      load_vec<CT, W>(in, idt, base + k * inner, v0);
-      load_vec<CT, W>(in, idt, base + (k + 1) * inner, v1);
-      load_vec<CT, W>(in, idt, base + (k + 2) * inner, v2);
-      load_vec<CT, W>(in, idt, base + (k + 3) * inner, v3);
-#pragma unroll
-      for (int i = 0; i < W; i++) {
-        acc[i] = R::accumulate(acc[i], v0[i], k);
-        acc[i] = R::accumulate(acc[i], v1[i], k + 1);
-        acc[i] = R::accumulate(acc[i], v2[i], k + 2);
-        acc[i] = R::accumulate(acc[i], v3[i], k + 3);
-      }
-    }
-    for (; k < k1; k++) {
-      CT v[W];
-      load_vec<CT, W>(in, idt, base + k * inner, v);
-#pragma unroll
-      for (int i = 0; i < W; i++) acc[i] = R::accumulate(acc[i], v[i], k);
-    }
-#pragma unroll
-    for (int i = 0; i < W; i++) {
-      if (nseg == 1) finalize(out, odt, o * inner + iv * W + i, acc[i]);
-      else partial[(o * nseg + seg) * inner + iv * W + i] = acc[i];
-    }
-  }
-}
-
-// fold partial[outer, nseg, inner] -> out[outer, inner]
-template <typename R>
-__global__ void __launch_bounds__(BLOCK)
-combine_cols_kernel(const typename R::acc_t *__restrict__ partial, void *__restrict__ out, int odt, int64_t outer,
-                    int64_t inner, int nseg) {
-  const int64_t total = outer * inner;
-  for (int64_t t = (int64_t)blockIdx.x * BLOCK + threadIdx.x; t < total; t += (int64_t)gridDim.x * BLOCK) {
-    const int64_t o = t / inner, i = t - o * inner;
-    typename R::acc_t acc = R::init();
-    for (int s = 0; s < nseg; s++) acc = R::combine(acc, partial[(o * nseg + s) * inner + i]);
-    finalize(out, odt, t, acc);
-  }
-}
-
-// ---- host side ------------------------------------------------------------------------------
-
-static int64_t round_up(int64_t a, int64_t b) { return (a + b - 1) / b * b; }
-
-// Partial results of a split reduction live either in a block of the context's pool (handed back
-// right after the launches: later work on this stream is ordered behind them) or, for the entry
-// point that allocates nothing, in this file's static device array.
-static int partials_acquire(hipnx_ctx *ctx, bool static_ws, size_t bytes, void **ws, size_t *ws_cap) {
-  if (!static_ws) return pool_alloc(ctx, bytes, ws, ws_cap);
-  *ws_cap = 0;
-  if (bytes > HIPNX_REDUCE_STATIC_SCRATCH_BYTES)
-    return set_error(HIPNX_EUNSUPPORTED, "reduce_static: this shape needs %zu bytes of partial results, the static scratch holds %zu",
-                     bytes, (size_t)HIPNX_REDUCE_STATIC_SCRATCH_BYTES);
-  if (!ctx->reduce_scratch) return set_error(HIPNX_EHIP, "reduce_static: the static scratch of this device was not resolved");
-  *ws = ctx->reduce_scratch;
-  return HIPNX_OK;
-}
-static void partials_release(hipnx_ctx *ctx, bool static_ws, void *ws, size_t ws_cap) {
-  if (ws && !static_ws) pool_free(ctx, ws, ws_cap);
-}
-
-template <typename R, typename CT, int IDT>
-static int run_reduce_t(hipnx_ctx *ctx, bool static_ws, int idt, int odt, int64_t outer, int64_t red, int64_t inner,
-                        const void *in, void *out) {
-  typedef typename R::acc_t acc_t;
-  const int64_t target_units = (int64_t)ctx->num_cus * 8;  // units of parallel work wanted
-  if (inner == 1) {
-    const int64_t rows = outer;
-    const bool vec = red % E == 0;
-    int tpr = red <= 4096 ? WAVE : BLOCK;
-    int nseg = 1;
-    int64_t seg_len = red;
-    const int64_t min_seg = 16384;  // elements per segment worth a block
-    if (rows < target_units && red >= 2 * min_seg) {
-      int64_t want = target_units / (rows > 0 ? rows : 1);
-      int64_t maxs = red / min_seg;
-      nseg = (int)(want < maxs ? want : maxs);
-      if (nseg > 1024) nseg = 1024;
-      if (nseg < 1) nseg = 1;
-      seg_len = round_up((red + nseg - 1) / nseg, E);
-      nseg = (int)((red + seg_len - 1) / seg_len);
-    }
-    acc_t *partial = nullptr;
-    void *ws = nullptr;
-    size_t ws_cap = 0;
-    if (nseg > 1) {
-      if (int st = partials_acquire(ctx, static_ws, sizeof(acc_t) * (size_t)(rows * nseg), &ws, &ws_cap)) return st;
-      partial = (acc_t *)ws;
-    }
-    const int rpb = BLOCK / tpr;
-    dim3 grid((unsigned)((rows * nseg + rpb - 1) / rpb)), block(BLOCK);
-    if (rows * nseg > 0) {
-      if (tpr == WAVE) {
-        if (vec) hipLaunchKernelGGL((reduce_rows_kernel<R, CT, WAVE, true, IDT>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
-        else hipLaunchKernelGGL((reduce_rows_kernel<R, CT, WAVE, false>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
-      } else {
-        if (vec) hipLaunchKernelGGL((reduce_rows_kernel<R, CT, BLOCK, true, IDT>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
-        else hipLaunchKernelGGL((reduce_rows_kernel<R, CT, BLOCK, false>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
-      }
-      if (nseg > 1) {
-        dim3 g2((unsigned)((rows + BLOCK / WAVE - 1) / (BLOCK / WAVE)));
-        hipLaunchKernelGGL((combine_partials_kernel<R>), g2, block, 0, ctx->stream, partial, out, odt, rows, nseg);
-      }
-    }
-    partials_release(ctx, static_ws, ws, ws_cap);
-  } else {
-    const bool vec = inner % E == 0;
-    const int64_t lanes = outer * (inner / (vec ? E : 1));
-    int nseg = 1;
-    int64_t seg_len = red;
-    const int64_t want_lanes = target_units * BLOCK / 4;
-    if (lanes < want_lanes && red >= 64) {
-      int64_t want = want_lanes / (lanes > 0 ? lanes : 1), maxs = red / 32;
-      nseg = (int)(want < maxs ? want : maxs);
-      if (nseg > 1024) nseg = 1024;
-      if (nseg < 1) nseg = 1;
-      seg_len = (red + nseg - 1) / nseg;
-      nseg = (int)((red + seg_len - 1) / seg_len);
-    }
-    acc_t *partial = nullptr;
-    void *ws = nullptr;
-    size_t ws_cap = 0;
-    if (nseg > 1) {
-      if (int st = partials_acquire(ctx, static_ws, sizeof(acc_t) * (size_t)(outer * nseg * inner), &ws, &ws_cap)) return st;
-      partial = (acc_t *)ws;
-    }
-    int64_t total = lanes * nseg;
-    int64_t blocks = (total + BLOCK - 1) / BLOCK;
-    int64_t cap = 1ll << 30;
-    dim3 grid((unsigned)(blocks < 1 ? 1 : (blocks < cap ? blocks : cap))), block(BLOCK);
-    if (total > 0) {
-      if (vec) hipLaunchKernelGGL((reduce_cols_kernel<R, CT, true, IDT>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, outer, red, inner, seg_len, nseg);
-      else hipLaunchKernelGGL((reduce_cols_kernel<R, CT, false>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, outer, red, inner, seg_len, nseg);
-      if (nseg > 1) {
-        int64_t b2 = (outer * inner + BLOCK - 1) / BLOCK;
-        dim3 g2((unsigned)(b2 < cap ? b2 : cap));
-        hipLaunchKernelGGL((combine_cols_kernel<R>), g2, block, 0, ctx->stream, partial, out, odt, outer, inner, nseg);
-      }
-    }
-    partials_release(ctx, static_ws, ws, ws_cap);
-  }
-  HIPNX_HIP(hipGetLastError());
-  return HIPNX_OK;
-}
-
-// the vectorised kernels compiled for the input's element type where it is one of the common ones
-template <typename R, typename CT>
-static int run_reduce(hipnx_ctx *ctx, bool static_ws, int idt, int odt, int64_t outer, int64_t red, int64_t inner,
-                      const void *in, void *out) {
-#define HIPNX_RED_AS(T) if (idt == T) return run_reduce_t<R, CT, T>(ctx, static_ws, idt, odt, outer, red, inner, in, out);
-  if constexpr (std::is_floating_point<CT>::value) {
-    HIPNX_RED_AS(HIPNX_F32) HIPNX_RED_AS(HIPNX_BF16) HIPNX_RED_AS(HIPNX_F16)
-    if constexpr (std::is_same<CT, double>::value) { HIPNX_RED_AS(HIPNX_F64) }
-  } else {
-    HIPNX_RED_AS(HIPNX_S32) HIPNX_RED_AS(HIPNX_S64) HIPNX_RED_AS(HIPNX_U8)
-  }
-#undef HIPNX_RED_AS
-  return run_reduce_t<R, CT, -1>(ctx, static_ws, idt, odt, outer, red, inner, in, out);
-}
 
 template <int OP>
 static int reduce_op(hipnx_ctx *ctx, bool static_ws, int idt, int odt, int64_t outer, int64_t red, int64_t inner, const void *in,
@@ -297,19 +17,15 @@ static int reduce_op(hipnx_ctx *ctx, bool static_ws, int idt, int odt, int64_t o
   return run_reduce<PlainReducer<int64_t, OP, false>, int64_t>(ctx, static_ws, idt, odt, outer, red, inner, in, out);
 }
 
-template <int OP, int TIE>
-static int argreduce_op(hipnx_ctx *ctx, int idt, int odt, int64_t outer, int64_t red, int64_t inner, const void *in,
-                        void *out) {
-  if (is_float(idt) && idt != HIPNX_F64)
-    return run_reduce<ArgReducer<float, OP, TIE, false>, float>(ctx, false, idt, odt, outer, red, inner, in, out);
-  if (is_float(idt)) return run_reduce<ArgReducer<double, OP, TIE, false>, double>(ctx, false, idt, odt, outer, red, inner, in, out);
-  if (idt == HIPNX_U64) return run_reduce<ArgReducer<int64_t, OP, TIE, true>, int64_t>(ctx, false, idt, odt, outer, red, inner, in, out);
-  return run_reduce<ArgReducer<int64_t, OP, TIE, false>, int64_t>(ctx, false, idt, odt, outer, red, inner, in, out);
-}
+
+// max / min / all / any: reduce_select.hip
+int reduce_select(hipnx_ctx *ctx, bool static_ws, int op, int idt, int odt, int64_t outer, int64_t red, int64_t inner,
+                  const void *in, void *out);
 
 }  // namespace hipnx
 
 using namespace hipnx;
+
 
 static int check_view(int64_t outer, int64_t red, int64_t inner) {
   if (outer < 0 || red < 0 || inner < 0) return set_error(HIPNX_EINVAL, "reduce: negative extent");
@@ -330,11 +46,8 @@ static int reduce_entry(hipnx_ctx *ctx, bool static_ws, int op, int in_dt, int o
   if (outer * inner == 0) return HIPNX_OK;
   switch (op) {
     case HIPNX_RED_SUM: return reduce_op<HIPNX_RED_SUM>(ctx, static_ws, in_dt, out_dt, outer, red, inner, inb->ptr, out->ptr);
-    case HIPNX_RED_MAX: return reduce_op<HIPNX_RED_MAX>(ctx, static_ws, in_dt, out_dt, outer, red, inner, inb->ptr, out->ptr);
-    case HIPNX_RED_MIN: return reduce_op<HIPNX_RED_MIN>(ctx, static_ws, in_dt, out_dt, outer, red, inner, inb->ptr, out->ptr);
     case HIPNX_RED_PRODUCT: return reduce_op<HIPNX_RED_PRODUCT>(ctx, static_ws, in_dt, out_dt, outer, red, inner, inb->ptr, out->ptr);
-    case HIPNX_RED_ALL: return reduce_op<HIPNX_RED_ALL>(ctx, static_ws, in_dt, out_dt, outer, red, inner, inb->ptr, out->ptr);
-    default: return reduce_op<HIPNX_RED_ANY>(ctx, static_ws, in_dt, out_dt, outer, red, inner, inb->ptr, out->ptr);
+    default: return reduce_select(ctx, static_ws, op, in_dt, out_dt, outer, red, inner, inb->ptr, out->ptr);
   }
 }
 
@@ -365,25 +78,3 @@ extern "C" int hipnx_reduce_static(hipnx_ctx *ctx, int op, int in_dt, int out_dt
   return reduce_entry(ctx, true, op, in_dt, out_dt, outer, red, inner, inb, out);
 }
 
-extern "C" int hipnx_argreduce(hipnx_ctx *ctx, int op, int tie, int in_dt, int out_dt, int64_t outer, int64_t red,
-                               int64_t inner, const hipnx_buf *inb, hipnx_buf *out) {
-  Enter in(ctx);
-  if (in.status) return in.status;
-  if (op < 0 || op > HIPNX_ARGMIN || tie < 0 || tie > HIPNX_TIE_HIGH)
-    return set_error(HIPNX_EINVAL, "argreduce: unknown op / tie_break");
-  if (dtype_size(in_dt) < 0 || dtype_size(out_dt) < 0 || is_float(out_dt))
-    return set_error(HIPNX_EINVAL, "argreduce: bad element type (the output must be an integer type)");
-  if (int st = check_view(outer, red, inner)) return st;
-  if (red == 0 && outer * inner > 0) return set_error(HIPNX_EINVAL, "argreduce: empty axis");
-  if (red > 0x7FFFFFFF) return set_error(HIPNX_EUNSUPPORTED, "argreduce: more than 2^31 - 1 elements along the reduced axis");
-  if (int st = check_buf(ctx, inb, (uint64_t)outer * red * inner * dtype_size(in_dt), "argreduce in")) return st;
-  if (int st = check_buf(ctx, out, (uint64_t)outer * inner * dtype_size(out_dt), "argreduce out")) return st;
-  if (outer * inner == 0) return HIPNX_OK;
-  const void *ip = inb->ptr;
-  void *op_ = out->ptr;
-  if (op == HIPNX_ARGMAX)
-    return tie == HIPNX_TIE_LOW ? argreduce_op<HIPNX_ARGMAX, HIPNX_TIE_LOW>(ctx, in_dt, out_dt, outer, red, inner, ip, op_)
-                                : argreduce_op<HIPNX_ARGMAX, HIPNX_TIE_HIGH>(ctx, in_dt, out_dt, outer, red, inner, ip, op_);
-  return tie == HIPNX_TIE_LOW ? argreduce_op<HIPNX_ARGMIN, HIPNX_TIE_LOW>(ctx, in_dt, out_dt, outer, red, inner, ip, op_)
-                              : argreduce_op<HIPNX_ARGMIN, HIPNX_TIE_HIGH>(ctx, in_dt, out_dt, outer, red, inner, ip, op_);
-}

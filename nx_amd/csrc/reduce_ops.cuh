@@ -115,10 +115,12 @@ struct ArgReducer {
   }
 };
 
-template <typename R>
+// combines across the aligned groups of WIDTH lanes (a power of two, the whole wave by default); lane 0 of a
+// group ends with its result.  The steps for a narrower group are the last steps of the wave's.
+template <typename R, int WIDTH = WAVE>
 __device__ __forceinline__ typename R::acc_t wave_reduce(typename R::acc_t a) {
 #pragma unroll
-  for (int m = WAVE / 2; m >= 1; m >>= 1) a = R::combine(a, R::shfl_xor(a, m));
+  for (int m = WIDTH / 2; m >= 1; m >>= 1) a = R::combine(a, R::shfl_xor(a, m));
   return a;
 }
 
