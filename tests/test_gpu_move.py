@@ -116,3 +116,63 @@ def test_to_batched_against_the_oracle(ty, shape, batch, hip, oracle):
         assert len(got) == len(want)
         for g, w in zip(got, want):
             assert g.type == w.type and g.shape == w.shape and Nx.to_binary(g) == Nx.to_binary(w)
+
+
+# ---- the vectorised forms: 16-byte lanes on shapes that sit on, next to and across their boundaries ---------
+
+@pytest.mark.parametrize("ty", ["u8", "s16", "bf16", "f32", "s64"])
+@pytest.mark.parametrize("shape,new,axes", [((1,), (1031, 64), None), ((64,), (1031, 64), None), ((1031, 1), (1031, 64), None),
+                                             ((), (257, 48), None), ((48,), (9, 48), None), ((9, 1), (9, 48), None),
+                                             ((5, 1, 16), (5, 7, 16), None), ((1, 7, 1), (3, 7, 32), None), ((33,), (130, 33), None),
+                                             ((130, 1), (130, 33), None), ((16,), (16, 40), [0])])
+def test_broadcast_vector_lanes(ty, shape, new, axes, hip, oracle):
+    """Rows, columns and single values repeated into outputs whose innermost axis is a whole number of 16-byte
+    vectors (the vector kernel: one load, one repeated element, or gathered elements per vector) and into ones
+    where it is not (one element per lane)."""
+    rng = np.random.default_rng(seed_of(ty, shape, new, "vec"))
+    x = rand_raw(rng, ty, shape)
+    hx, ox = both(x, ty, hip, oracle)
+    assert_bits_equal(Nx.broadcast(hx, new, axes), Nx.broadcast(ox, new, axes), f"broadcast {ty} {shape}->{new}")
+
+
+@pytest.mark.parametrize("ty", ["u8", "bf16", "f32", "s64"])
+@pytest.mark.parametrize("n", [1, 7, 15, 16, 17, 64, 1000, 4097, 65536 + 3])
+def test_constant_fill_counts(ty, n, hip, oracle):
+    """A constant is written as 16-byte vectors of the repeated element plus a tail of fewer than 16 bytes."""
+    value = 3 if ty != "f32" else 2.5
+    got = Nx.broadcast(Nx.tensor(value, type=ty, backend=hip), (n,))
+    want = Nx.broadcast(Nx.tensor(value, type=ty, backend=oracle), (n,))
+    assert_bits_equal(got, want, f"fill {ty} {n}")
+
+
+@pytest.mark.parametrize("ty", ["u8", "bf16", "f32", "s64"])
+@pytest.mark.parametrize("shape", [(64, 64), (128, 128), (256, 64), (64, 256), (8, 8), (16, 48), (2, 192, 320), (3, 64, 72),
+                                   (130, 66), (136, 72), (1000, 24)])
+def test_transpose_tiles(ty, shape, hip, oracle):
+    """Swaps of the last two axes on whole tiles, ragged tiles, row counts that are and are not a multiple of a
+    16-byte vector (the vector kernel and the element kernel)."""
+    rng = np.random.default_rng(seed_of(ty, shape, "tiles"))
+    x = rand_raw(rng, ty, shape)
+    hx, ox = both(x, ty, hip, oracle)
+    perm = list(range(len(shape) - 2)) + [len(shape) - 1, len(shape) - 2]
+    assert_bits_equal(Nx.transpose(hx, perm), Nx.transpose(ox, perm), f"transpose {ty} {shape}")
+
+
+@pytest.mark.parametrize("ty", ["u8", "s16", "bf16", "f32"])
+@pytest.mark.parametrize("shape,starts,lengths", [((40, 100), [1, 1], [39, 99]), ((40, 100), [0, 3], [40, 64]), ((40, 100), [5, 7], [30, 33]),
+                                                   ((9, 257), [0, 1], [9, 256]), ((3, 4, 50), [1, 1, 5], [2, 3, 41]), ((300,), [13], [270]),
+                                                   ((64, 31), [0, 0], [64, 31]), ((64, 32), [1, 0], [63, 32])])
+def test_slices_off_the_vector_grid(ty, shape, starts, lengths, hip, oracle):
+    """Dense rows that start or end off a 16-byte boundary: whole vectors at element alignment, the last,
+    partial vector of a row by element."""
+    rng = np.random.default_rng(seed_of(ty, shape, starts, "runs"))
+    x = rand_raw(rng, ty, shape)
+    hx, ox = both(x, ty, hip, oracle)
+    assert_bits_equal(Nx.slice(hx, starts, lengths), Nx.slice(ox, starts, lengths), f"slice {ty} {shape} {starts}")
+    axes = [len(shape) - 1]
+    assert_bits_equal(Nx.reverse(hx, axes=axes), Nx.reverse(ox, axes=axes), f"reverse {ty} {shape}")
+    sl_h, sl_o = Nx.slice(hx, starts, lengths), Nx.slice(ox, starts, lengths)
+    assert_bits_equal(Nx.reverse(sl_h, axes=axes), Nx.reverse(sl_o, axes=axes), f"reverse of a slice {ty} {shape}")
+    cfg = [(1, 2, 0)] * len(shape)
+    pad_h, pad_o = Nx.tensor(0, type=ty, backend=hip), Nx.tensor(0, type=ty, backend=oracle)
+    assert_bits_equal(Nx.pad(hx, pad_h, cfg), Nx.pad(ox, pad_o, cfg), f"pad {ty} {shape}")

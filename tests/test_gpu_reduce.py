@@ -119,3 +119,29 @@ def test_argreduce_nan_and_infinities(op, hip, oracle):
         assert_bits_equal(getattr(Nx, op)(hx, axis=1, tie_break=tie), getattr(Nx, op)(ox, axis=1, tie_break=tie), op)
         assert_bits_equal(getattr(Nx, op)(hx, axis=0, tie_break=tie), getattr(Nx, op)(ox, axis=0, tie_break=tie), op)
     assert_bits_equal(getattr(Nx, op)(hx), getattr(Nx, op)(ox), f"{op} flat")
+
+
+@pytest.mark.parametrize("ty", ["f32", "bf16", "f16", "s32", "u8", "s16"])
+@pytest.mark.parametrize("red", [8, 16, 24, 64, 72, 128, 200, 256, 264, 512])
+@pytest.mark.parametrize("op", ["sum", "reduce_max", "argmax"])
+def test_short_rows_take_part_of_a_wave(ty, red, op, hip, oracle):
+    """Rows of up to 256 elements are reduced by 8 / 16 / 32 lanes, several rows per wave; the result must be the
+    oracle's (and the whole-wave kernel's: same combine steps)."""
+    rng = np.random.default_rng(seed_of(ty, red, op, "short"))
+    x = rand_raw(rng, ty, (37, red), lo=-4, hi=4)
+    hx, ox = both(x, ty, hip, oracle)
+    if op == "argmax":
+        assert_bits_equal(Nx.argmax(hx, axis=1), Nx.argmax(ox, axis=1), f"argmax {ty} {red}")
+    elif op == "reduce_max":
+        assert_bits_equal(Nx.reduce_max(hx, axes=[1]), Nx.reduce_max(ox, axes=[1]), f"max {ty} {red}")
+    else:
+        got, want = Nx.sum(hx, axes=[1]), Nx.sum(ox, axes=[1])
+        if ty in ("s32", "u8", "s16"):
+            assert_bits_equal(got, want, f"sum {ty} {red}")
+        else:
+            x64 = values(ox)
+            bits = got.type[1] if ty == "f32" else (16 if ty == "bf16" else 10)
+            eps = {32: 2.0 ** -23, 16: 2.0 ** -7, 10: 2.0 ** -10}[bits]
+            bound = red * 2.0 ** -24 * np.abs(x64).sum(axis=1) + eps * np.abs(x64.sum(axis=1)) + 1e-30
+            err = np.abs(values(got) - values(want))
+            assert (err <= bound).all(), f"sum {ty} {red}: max err {err.max():.3e}"
