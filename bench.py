@@ -316,6 +316,26 @@ def main():
             entry(f"config1_chain_f32_{nn}", 32.0 * N + 4.0 * nn, "GB/s", ms, PEAK_HBM_GBS, "hbm")
             del x, y
 
+        # the same callbacks on the 2-byte type of most model tensors (bf16, 16384^2), a column sum and a transpose
+        rng16 = np.random.default_rng(16)
+        bx = put((rng16.standard_normal((16384, 16384)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16), "bf16")
+        N = 16384 * 16384
+        _, ms = tstat(lambda: Nx.add(bx, bx), steps, warm)
+        entry("add_bf16_16384", 6.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+        _, ms = tstat(lambda: Nx.exp(bx), steps, warm)
+        entry("exp_bf16_16384", 4.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+        _, ms = tstat(lambda: Nx.sum(bx, axes=[1]), steps, warm)
+        entry("sum_rows_bf16_16384", 2.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read")
+        _, ms = tstat(lambda: Nx.sum(bx, axes=[0]), steps, warm)
+        entry("sum_columns_bf16_16384", 2.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read")
+        _, ms = tstat(lambda: Nx.argmax(bx, axis=1), steps, warm)
+        entry("argmax_rows_bf16_16384", 2.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read")
+        _, ms = tstat(lambda: Nx.transpose(bx), steps, warm)
+        entry("transpose_bf16_16384", 4.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+        _, ms = tstat(lambda: Nx.as_type(bx, "f32"), steps, warm)
+        entry("as_type_bf16_f32_16384", 6.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+        del bx
+
         # config 3: attention scores + softmax chain
         q, k = W.attention_scores()
         q, k = put(q, "bf16"), put(k, "bf16")
