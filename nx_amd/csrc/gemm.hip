@@ -192,7 +192,49 @@ splitk_combine_kernel(const AT *__restrict__ part, void *__restrict__ out, int o
 
 static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batch, int64_t M, int64_t N,
                     int64_t K, int l_layout, int r_layout, const hipnx_buf *l, const hipnx_buf *r,
+                    hipnx_buf *out, int scale_mode, const hipnx_buf *scale);
+
+// A copy of a dot operand ([batch, rows, K] or [batch, K, rows]) with K extended to Kp by zeros.
+static int pad_k(hipnx_ctx *ctx, int esz, int64_t batch, int64_t rows, int64_t K, int64_t Kp, int layout,
+                 const hipnx_buf *in, hipnx_buf **out) {
+  int st = hipnx_buf_alloc(ctx, (size_t)(batch * rows * Kp * esz), out);
+  if (st) return st;
+  const unsigned char zero = 0;
+  st = hipnx_fill(ctx, *out, 1, &zero, batch * rows * Kp * esz);
+  if (st) return st;
+  if (layout == HIPNX_K_INNER) {
+    const int64_t dims[2] = {batch * rows, K}, is[2] = {K, 1}, os[2] = {Kp, 1};
+    return hipnx_strided_copy(ctx, esz, 2, dims, is, 0, os, 0, in, *out);
+  }
+  const int64_t dims[2] = {batch, K * rows}, is[2] = {K * rows, 1}, os[2] = {Kp * rows, 1};
+  return hipnx_strided_copy(ctx, esz, 2, dims, is, 0, os, 0, in, *out);
+}
+
+static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batch, int64_t M, int64_t N,
+                    int64_t K, int l_layout, int r_layout, const hipnx_buf *l, const hipnx_buf *r,
                     hipnx_buf *out, int scale_mode, const hipnx_buf *scale) {
+  // A contraction length that is not a whole number of 128-byte slabs keeps a large MFMA-typed problem off the
+  // tiled kernels (K not a multiple of 16 bytes even sends it to the generic kernel: a few TFLOP/s).  Both
+  // operands are then copied with K extended by zeros -- products of two zeros, which add nothing -- and the
+  // contraction runs on the copies.
+  {
+    const int esz = dtype_size(l_dt);
+    const bool typed = l_dt == r_dt && esz > 0 && out_dtype_size(out_dt) > 0 &&
+                       (((l_dt == HIPNX_BF16 || l_dt == HIPNX_F16 || l_dt == HIPNX_F32) && is_float(out_dt)) ||
+                        (l_dt == HIPNX_S8 && !is_float(out_dt) && K <= (1ll << 16)));
+    if (typed && scale_mode == HIPNX_SCALE_NONE && K > 0 && batch > 0 && M > 0 && N > 0 && (K * esz) % SLAB != 0 && M * N >= 256 &&
+        (double)M * (double)N * (double)K * (double)batch >= 16777216.0 && l && r &&
+        (l_layout == HIPNX_K_INNER || l_layout == HIPNX_K_OUTER) && (r_layout == HIPNX_K_INNER || r_layout == HIPNX_K_OUTER)) {
+      const int64_t per = SLAB / esz, Kp = (K + per - 1) / per * per;
+      hipnx_buf *lp = nullptr, *rp = nullptr;
+      int st = pad_k(ctx, esz, batch, M, K, Kp, l_layout, l, &lp);
+      if (!st) st = pad_k(ctx, esz, batch, N, K, Kp, r_layout, r, &rp);
+      if (!st) st = dot_impl(ctx, l_dt, r_dt, out_dt, batch, M, N, Kp, l_layout, r_layout, lp, rp, out, scale_mode, scale);
+      if (lp) hipnx_buf_destroy(lp);
+      if (rp) hipnx_buf_destroy(rp);
+      return st;
+    }
+  }
   int64_t Kb = 0;
   bool mfma = false;
   {

@@ -223,6 +223,35 @@ def test_large_ragged_dot_on_the_big_tile(ty, layout, hip, oracle):
         check_float_dot(got_rows, want, values(oa), values(ob), "mk,kn->mn", K, f"big tile {ty} {layout}")
 
 
+@pytest.mark.parametrize("ty,M,N,K", [("bf16", 333, 777, 555), ("f16", 256, 512, 1000), ("f32", 300, 260, 250), ("s8", 384, 320, 1001),
+                                      ("bf16", 2, 4100, 2050)])
+@pytest.mark.parametrize("layout", ["nn", "nt", "tn", "tt"])
+def test_contraction_lengths_off_the_slab_grid_are_padded(ty, M, N, K, layout, hip, oracle):
+    """A K that is not a whole number of 128-byte slabs: large problems run on zero-extended copies of the
+    operands (products of two zeros add nothing), so int8 stays exact and floats stay within the bound."""
+    rng = np.random.default_rng(seed_of(ty, M, N, K, layout, "pad"))
+    if ty == "s8":
+        a = rng.integers(-127, 128, size=(M, K)).astype(np.int8)
+        b = rng.integers(-127, 128, size=(K, N)).astype(np.int8)
+    else:
+        a, b = rand_raw(rng, ty, (M, K), lo=-1, hi=1), rand_raw(rng, ty, (K, N), lo=-1, hi=1)
+    la = a if layout[0] == "n" else np.ascontiguousarray(a.T)
+    lb = b if layout[1] == "n" else np.ascontiguousarray(b.T)
+    c1 = [1] if layout[0] == "n" else [0]
+    c2 = [0] if layout[1] == "n" else [1]
+    kw = {"out_type": "s32"} if ty == "s8" else {}
+    got = Nx.dot(from_numpy(la, ty, hip), c1, from_numpy(lb, ty, hip), c2, **kw)
+    assert got.shape == (M, N)
+    rows = np.unique(np.concatenate([[0, M - 1], rng.integers(0, M, size=10)]))
+    oa, ob = from_numpy(np.ascontiguousarray(a[rows]), ty, oracle), from_numpy(b, ty, oracle)
+    want = Nx.dot(oa, ob, **kw)
+    got_rows = from_numpy(np.ascontiguousarray(hip.to_numpy(got)[rows]), "s32" if ty == "s8" else ty, oracle)
+    if ty == "s8":
+        assert_bits_equal(got_rows, want, f"padded K s8 {layout}")
+    else:
+        check_float_dot(got_rows, want, values(oa), values(ob), "mk,kn->mn", K, f"padded K {ty} {layout}")
+
+
 @pytest.mark.parametrize("ty,M,N,K", [("bf16", 128, 1024, 4096), ("s8", 128, 1024, 4096), ("f16", 200, 520, 2048), ("f32", 132, 384, 2048),
                                       ("s8", 384, 512, 8192), ("bf16", 512, 1024, 2048)])
 @pytest.mark.parametrize("layout", ["nn", "nt", "tn", "tt"])
