@@ -333,6 +333,9 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
         int cfg;
         if (M <= 64) cfg = GEMM_CFG_64x32;
         else if (t256 * 4 >= (int64_t)ctx->num_cus * 3 && M >= 192 && N >= 192) cfg = GEMM_CFG_256;
+        else if ((l_dt == HIPNX_BF16 || l_dt == HIPNX_F16) && M >= 192 && N >= 128 &&
+                 ((M + 255) / 256) * ((N + 127) / 128) * batch * 4 >= (int64_t)ctx->num_cus * 3)
+          cfg = GEMM_CFG_256x128;  // half-width tiles of the two-group kernel fill the CUs where 256 x 256 ones do not
         else cfg = GEMM_CFG_128;
         // A grid of 128 x 128 tiles that leaves most CUs idle (a few hundred rows against a long weight
         // matrix: 128 x 4096 x 4096 is 32 tiles walking 64 slabs each) splits K over S work-groups per tile:

@@ -9,6 +9,7 @@ namespace hipnx {
 
 // tile configurations of gemm_pipelined_kernel<DT, WM, WN, TM, TN, ...>
 enum {
+  GEMM_CFG_256x128 = 3,  // 256 x 128, the two-group kernel with half-width wave tiles: 2-byte types whose 256 x 256 grid is too small
   GEMM_CFG_256 = 0,  // 256 x 256, 8 waves (4 x 2, each 64 x 128): large square-ish problems
   GEMM_CFG_128 = 1,  // 128 x 128, 4 waves (2 x 2, each 64 x 64): mid-size and batched problems
   GEMM_CFG_64x32 = 2 // 64 x 32, 2 waves: few rows against a long weight matrix (HBM streaming)
@@ -44,18 +45,18 @@ static int launch_one(const hipnx_ctx *ctx, GemmArgs a, int64_t batch) {
 
 // the two-group 256 x 256 kernel (gemm_pingpong.cuh): bf16 / f16 in every layout, s8 with a K-inner
 // left operand; its request offsets are 32 bits from the tile's first row or column
-template <int DT, bool LK, bool RK>
+template <int DT, bool LK, bool RK, int BN = 256>
 static int launch_pingpong(const hipnx_ctx *ctx, GemmArgs a, int64_t batch) {
   constexpr bool TALL = LK && !RK;  // the operand read by transposing loads gets the fewer fragments
-  constexpr int smem = 2 * 512 * SLAB;
-  auto kern = gemm_pingpong_kernel<DT, LK, RK, TALL>;
+  constexpr int smem = 2 * (256 + BN) * SLAB;
+  auto kern = gemm_pingpong_kernel<DT, LK, RK, TALL, true, BN>;
   static bool configured = false;
   if (!configured) {
     HIPNX_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
     configured = true;
   }
   a.tiles_m = (int)((a.M + 255) / 256);
-  a.tiles_n = (int)((a.N + 255) / 256);
+  a.tiles_n = (int)((a.N + BN - 1) / BN);
   a.group_m = gemm_group_m(a.tiles_m, a.tiles_n);
   dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)batch), block(512);
   hipLaunchKernelGGL(kern, grid, block, smem, ctx->stream, a);
@@ -72,6 +73,11 @@ static int launch_cfg(const hipnx_ctx *ctx, int cfg, const GemmArgs &a, int64_t 
         if (a.ld_l < (1ll << 23) && a.ld_r < (1ll << 23)) return launch_pingpong<DT, LK, RK>(ctx, a, batch);
       }
       return launch_one<DT, 4, 2, 2, 4, LK, RK>(ctx, a, batch);
+    case GEMM_CFG_256x128:
+      if constexpr (DT == HIPNX_BF16 || DT == HIPNX_F16) {
+        if (a.ld_l < (1ll << 23) && a.ld_r < (1ll << 23)) return launch_pingpong<DT, LK, RK, 128>(ctx, a, batch);
+      }
+      return launch_one<DT, 2, 2, 2, 2, LK, RK>(ctx, a, batch);
     case GEMM_CFG_128: {
       // one wave per SIMD and 0.25 us of MFMA work per slab: two stages cannot cover the latency of the next
       // slab's requests (measured 2100 clocks per slab, 1580 with four stages); four stages where every

@@ -111,11 +111,15 @@ struct PPKOuterLoader {
 // waves 0-3 own the upper 128 rows.  A transposing fragment read moves 8 bytes per lane, a plain one
 // 16, so the operand that needs the transposing reads should be the one with fewer fragments per
 // wave: a K-outer right operand wants TALL, a K-outer left operand the other shape.
-template <int DT, bool L_KIN, bool R_KIN, bool TALL = false, bool PRIO = true>
+// BN = 128 halves the tile along N (wave tiles 64 x 64 or 128 x 32, 16 MFMAs per phase): twice the tiles for
+// problems whose 256 x 256 grid leaves CUs idle, at a somewhat lower rate per tile.
+template <int DT, bool L_KIN, bool R_KIN, bool TALL = false, bool PRIO = true, int BN_ = 256>
 __global__ void __launch_bounds__(512)
 gemm_pingpong_kernel(GemmArgs a) {
   typedef typename Mma16<DT>::acc_t acc_t;
-  constexpr int NW = 8, TM16 = TALL ? 8 : 4, TN16 = TALL ? 4 : 8, BM = 256, BN = 256, HALF = 128;
+  constexpr int NW = 8, BM = 256, BN = BN_, HALF = 128, TM16 = TALL ? 8 : 4, TN16 = TALL ? BN / 64 : BN / 32;
+  constexpr int RPER = BN / 8 / NW;  // requests of the right operand per wave and memory phase (the left one's: 4)
+  static_assert(BN == 256 || BN == 128, "tile widths of the two-group kernel");
   constexpr int STAGE = (BM + BN) * SLAB;
   constexpr int ES = (DT == HIPNX_S8) ? 1 : 2;
   static_assert(DT == HIPNX_BF16 || DT == HIPNX_F16 || DT == HIPNX_S8, "2-byte and 1-byte MFMA types");
@@ -132,7 +136,7 @@ gemm_pingpong_kernel(GemmArgs a) {
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int grp = wave >> 2;                     // waves w and w + 4 share a SIMD
   const int wm = TALL ? (wave >> 2) * 128 : (wave >> 1) * 64;  // group 0: rows 0..127, group 1: 128..255
-  const int wn = TALL ? (wave & 3) * 64 : (wave & 1) * 128;
+  const int wn = TALL ? (wave & 3) * (BN / 4) : (wave & 1) * (BN / 2);
 
   acc_t acc[TM16][TN16];
 #pragma unroll
@@ -196,7 +200,7 @@ gemm_pingpong_kernel(GemmArgs a) {
   if (nslab > 1) {
     issue_r(1, SLAB);
     issue_l(1, SLAB);
-    wait_vmcnt<8>();
+    wait_vmcnt<RPER + 4>();
   } else {
     wait_vmcnt<0>();
   }
@@ -213,11 +217,11 @@ gemm_pingpong_kernel(GemmArgs a) {
       for (int i = 0; i < TM16; i++) fa[i] = read_l(cur, ks, i);
 #pragma unroll
       for (int j = 0; j < TN16; j++) fb[j] = read_r(cur, ks, j);
-      bool issued = false;
+      bool issued = false, issued_r = false;
       if (ks == 0) {
         if (s >= 1 && s + 1 < nslab) {
           issue_r((s + 1) & 1, (int64_t)(s + 1) * SLAB);
-          issued = true;
+          issued_r = true;
         }
       } else if (grp == 0) {
         if (s >= 1 && s + 1 < nslab) {
@@ -231,6 +235,7 @@ gemm_pingpong_kernel(GemmArgs a) {
       // what I requested a memory phase ago (or in the prologue) has to be in LDS before the barrier
       // that publishes it; in the very first phase nothing is due yet (slab 1 is first read in phase 4)
       if (issued) wait_vmcnt<4>();
+      else if (issued_r) wait_vmcnt<RPER>();
       else if (!(s == 0 && ks == 0)) wait_vmcnt<0>();
       __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): my fragments are in registers
       __builtin_amdgcn_s_barrier();

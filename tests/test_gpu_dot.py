@@ -223,6 +223,27 @@ def test_large_ragged_dot_on_the_big_tile(ty, layout, hip, oracle):
         check_float_dot(got_rows, want, values(oa), values(ob), "mk,kn->mn", K, f"big tile {ty} {layout}")
 
 
+@pytest.mark.parametrize("ty", ["bf16", "f16"])
+@pytest.mark.parametrize("M,N,K", [(1024, 6144, 256), (1000, 6200, 384), (2048, 3080, 128)])
+@pytest.mark.parametrize("layout", ["nn", "nt", "tn", "tt"])
+def test_half_width_tiles_of_the_two_group_kernel(ty, M, N, K, layout, hip, oracle):
+    """Problems whose grid of 256 x 256 tiles would leave CUs idle take 256 x 128 tiles (wave tiles 64 x 64 or
+    128 x 32): whole and ragged grids, all four operand layouts."""
+    rng = np.random.default_rng(seed_of(ty, M, N, K, layout, "w128"))
+    a, b = rand_raw(rng, ty, (M, K), lo=-1, hi=1), rand_raw(rng, ty, (K, N), lo=-1, hi=1)
+    la = a if layout[0] == "n" else np.ascontiguousarray(a.T)
+    lb = b if layout[1] == "n" else np.ascontiguousarray(b.T)
+    c1 = [1] if layout[0] == "n" else [0]
+    c2 = [0] if layout[1] == "n" else [1]
+    got = Nx.dot(from_numpy(la, ty, hip), c1, from_numpy(lb, ty, hip), c2)
+    assert got.shape == (M, N)
+    rows = np.unique(np.concatenate([[0, 127, 128, 255, 256, M - 1], rng.integers(0, M, size=18)]))
+    oa, ob = from_numpy(np.ascontiguousarray(a[rows]), ty, oracle), from_numpy(b, ty, oracle)
+    want = Nx.dot(oa, ob)
+    got_rows = from_numpy(np.ascontiguousarray(hip.to_numpy(got)[rows]), ty, oracle)
+    check_float_dot(got_rows, want, values(oa), values(ob), "mk,kn->mn", K, f"256x128 tiles {ty} {layout}")
+
+
 @pytest.mark.parametrize("ty,M,N,K", [("bf16", 333, 777, 555), ("f16", 256, 512, 1000), ("f32", 300, 260, 250), ("s8", 384, 320, 1001),
                                       ("bf16", 2, 4100, 2050)])
 @pytest.mark.parametrize("layout", ["nn", "nt", "tn", "tt"])
@@ -282,7 +303,7 @@ def test_long_k_on_an_under_filled_grid_is_split(ty, M, N, K, layout, hip, oracl
         check_float_dot(got_rows, want, values(oa), values(ob), "mk,kn->mn", K, f"split K {ty} {layout}")
 
 
-@pytest.mark.parametrize("ty,M,N,K", [("bf16", 512, 520, 256), ("bf16", 300, 528, 128), ("f16", 264, 344, 128),
+@pytest.mark.parametrize("ty,M,N,K", [("bf16", 512, 520, 256), ("bf16", 300, 528, 128), ("f16", 264, 344, 128), ("bf16", 1024, 6152, 64),
                                       ("bf16", 130, 76, 64), ("f16", 64, 40, 128)])
 def test_two_byte_outputs_land_in_their_own_columns(ty, M, N, K, hip):
     """The MFMA kernel writes bf16 / f16 results two column tiles at a time, lanes trading halves
