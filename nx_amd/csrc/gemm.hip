@@ -350,6 +350,15 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
         if (splittable && t128 * 2 <= ctx->num_cus && nslab >= 32)
           for (int cand = 16; cand >= 2; cand /= 2)
             if (t128 * cand <= 2 * (int64_t)ctx->num_cus && nslab % cand == 0 && nslab / cand >= 8) { splits = cand; break; }
+        // Between the two: a half-width grid of the two-group kernel that covers 3/8 to 3/4 of the CUs, walked in
+        // two halves of K when K is long (64 slabs or more; 768 x 4096 x 4096: 51 -> 45 us, 1024 x 4096 x 4096: 53 -> 50 us)
+        const int64_t tw = ((M + 255) / 256) * ((N + 127) / 128);
+        if (splits == 1 && cfg == GEMM_CFG_128 && (l_dt == HIPNX_BF16 || l_dt == HIPNX_F16) && batch == 1 && M >= 192 && N >= 128 &&
+            scale_mode == HIPNX_SCALE_NONE && (M * N) % 4 == 0 && nslab >= 64 && nslab % 2 == 0 &&
+            tw * 8 >= (int64_t)ctx->num_cus * 3 && tw * 2 <= (int64_t)ctx->num_cus + ctx->num_cus / 4) {
+          cfg = GEMM_CFG_256x128;
+          splits = 2;
+        }
         void *ws = nullptr;
         size_t ws_cap = 0;
         if (splits > 1 && pool_alloc(ctx, (size_t)splits * M * N * 4, &ws, &ws_cap) != HIPNX_OK) splits = 1;
