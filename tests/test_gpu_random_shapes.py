@@ -1,0 +1,111 @@
+"""Seeded sweeps over random shapes: the vector paths of the streaming kernels change with divisibility and
+alignment (whole 16-byte vectors or ragged tails, one row or many, operands broadcast along rows or columns,
+windows that start off a vector boundary), so every case draws its shape, its broadcast pattern and its
+window at random, runs the callback on the device and on the CPU oracle, and compares bits."""
+import numpy as np
+import pytest
+
+from nx_amd import nx as Nx
+from nx_amd import types as T
+from support import assert_bits_equal, seed_of
+from test_gpu_elementwise import both, rand_raw
+
+pytestmark = pytest.mark.gpu
+
+SIZES = [1, 2, 3, 4, 5, 7, 8, 9, 15, 16, 17, 24, 31, 32, 33, 40, 63, 64, 65, 96, 127, 128, 130, 255, 256, 264]
+
+
+def draw_shape(rng, rank, limit=70000):
+    while True:
+        shape = tuple(int(rng.choice(SIZES)) for _ in range(rank))
+        if np.prod(shape) <= limit:
+            return shape
+
+
+def broadcastable(rng, shape):
+    """A shape that broadcasts to `shape`: some axes set to 1, some leading axes dropped."""
+    s = [d if rng.random() < 0.6 else 1 for d in shape]
+    drop = int(rng.integers(0, len(s)))
+    return tuple(s[drop:]) if rng.random() < 0.4 else tuple(s)
+
+
+@pytest.mark.parametrize("case", range(300))
+def test_exact_binary_ops_on_random_broadcasts(case, hip, oracle):
+    rng = np.random.default_rng(seed_of("binary", case))
+    rank = int(rng.integers(1, 4))
+    shape = draw_shape(rng, rank)
+    ls, rs = broadcastable(rng, shape), broadcastable(rng, shape)
+    if rng.random() < 0.5:
+        ls = shape
+    lt, rt = [("f32", "f32"), ("bf16", "bf16"), ("f16", "f16"), ("s32", "s32"), ("s64", "s64"), ("u8", "u8"), ("f32", "bf16"),
+              ("s16", "s16"), ("f64", "f64"), ("bf16", "f32"), ("s32", "s64")][int(rng.integers(0, 11))]
+    op = ["add", "subtract", "multiply", "max", "min", "less", "equal", "greater_equal", "logical_and"][int(rng.integers(0, 9))]
+    a, b = rand_raw(rng, lt, ls), rand_raw(rng, rt, rs)
+    ha, oa = both(a, lt, hip, oracle)
+    hb, ob = both(b, rt, hip, oracle)
+    assert_bits_equal(getattr(Nx, op)(ha, hb), getattr(Nx, op)(oa, ob), f"{op} {lt}{ls} {rt}{rs}")
+
+
+@pytest.mark.parametrize("case", range(250))
+def test_unary_conversions_and_selections_on_random_shapes(case, hip, oracle):
+    rng = np.random.default_rng(seed_of("unary", case))
+    shape = draw_shape(rng, int(rng.integers(1, 4)))
+    ty = ["f32", "bf16", "f16", "s32", "s64", "u8", "f64", "s16"][int(rng.integers(0, 8))]
+    x = rand_raw(rng, ty, shape)
+    hx, ox = both(x, ty, hip, oracle)
+    assert_bits_equal(Nx.negate(hx), Nx.negate(ox), f"negate {ty}{shape}")
+    assert_bits_equal(Nx.abs(hx), Nx.abs(ox), f"abs {ty}{shape}")
+    to = ["f32", "bf16", "f16", "s32", "s64", "u8", "f64"][int(rng.integers(0, 7))]
+    try:
+        want = Nx.as_type(ox, to)
+    except Exception as e:  # the reference raises where a finite value overflows f16: the device writes infinity
+        assert "overflows" in str(e)
+    else:
+        assert_bits_equal(Nx.as_type(hx, to), want, f"as_type {ty}->{to} {shape}")
+    y = rand_raw(rng, ty, shape)
+    hy, oy = both(y, ty, hip, oracle)
+    hp, op_ = Nx.less(hx, hy), Nx.less(ox, oy)
+    assert_bits_equal(Nx.select(hp, hx, hy), Nx.select(op_, ox, oy), f"select {ty}{shape}")
+
+
+@pytest.mark.parametrize("case", range(250))
+def test_exact_reductions_on_random_axes(case, hip, oracle):
+    rng = np.random.default_rng(seed_of("reduce", case))
+    rank = int(rng.integers(1, 4))
+    shape = draw_shape(rng, rank)
+    axes = sorted(rng.choice(rank, size=int(rng.integers(1, rank + 1)), replace=False).tolist())
+    ty = ["s32", "u8", "s16", "s64", "f32", "bf16", "f16"][int(rng.integers(0, 7))]
+    x = rand_raw(rng, ty, shape)
+    hx, ox = both(x, ty, hip, oracle)
+    assert_bits_equal(Nx.reduce_max(hx, axes=axes), Nx.reduce_max(ox, axes=axes), f"reduce_max {ty}{shape}{axes}")
+    assert_bits_equal(Nx.reduce_min(hx, axes=axes), Nx.reduce_min(ox, axes=axes), f"reduce_min {ty}{shape}{axes}")
+    if T.is_integer(T.normalize(ty)):
+        assert_bits_equal(Nx.sum(hx, axes=axes), Nx.sum(ox, axes=axes), f"sum {ty}{shape}{axes}")
+    axis = int(axes[0])
+    assert_bits_equal(Nx.argmax(hx, axis=axis), Nx.argmax(ox, axis=axis), f"argmax {ty}{shape}{axis}")
+    assert_bits_equal(Nx.argmin(hx, axis=axis, tie_break="high"), Nx.argmin(ox, axis=axis, tie_break="high"), f"argmin {ty}{shape}{axis}")
+
+
+@pytest.mark.parametrize("case", range(250))
+def test_copies_on_random_windows(case, hip, oracle):
+    rng = np.random.default_rng(seed_of("copy", case))
+    rank = int(rng.integers(1, 4))
+    shape = draw_shape(rng, rank)
+    ty = ["u8", "s16", "bf16", "f32", "s64"][int(rng.integers(0, 5))]
+    x = rand_raw(rng, ty, shape)
+    hx, ox = both(x, ty, hip, oracle)
+    starts = [int(rng.integers(0, d)) for d in shape]
+    lengths = [int(rng.integers(1, d - s + 1)) for d, s in zip(shape, starts)]
+    strides = [int(rng.integers(1, 3)) if rng.random() < 0.25 else 1 for _ in shape]
+    assert_bits_equal(Nx.slice(hx, starts, lengths, strides=strides), Nx.slice(ox, starts, lengths, strides=strides), f"slice {ty}{shape}")
+    rev = sorted(rng.choice(rank, size=int(rng.integers(1, rank + 1)), replace=False).tolist())
+    assert_bits_equal(Nx.reverse(hx, axes=rev), Nx.reverse(ox, axes=rev), f"reverse {ty}{shape}{rev}")
+    perm = rng.permutation(rank).tolist()
+    assert_bits_equal(Nx.transpose(hx, perm), Nx.transpose(ox, perm), f"transpose {ty}{shape}{perm}")
+    new = tuple(int(rng.choice([2, 3, 8])) for _ in range(int(rng.integers(0, 2)))) + shape
+    assert_bits_equal(Nx.broadcast(hx, new), Nx.broadcast(ox, new), f"broadcast {ty}{shape}->{new}")
+    cfg = [(int(rng.integers(-1, 3)), int(rng.integers(-1, 3)), int(rng.integers(0, 2))) for _ in shape]
+    if all(d + lo + hi + (d - 1) * it > 0 for d, (lo, hi, it) in zip(shape, cfg)):
+        pv_h, pv_o = Nx.tensor(1, type=ty, backend=hip), Nx.tensor(1, type=ty, backend=oracle)
+        assert_bits_equal(Nx.pad(hx, pv_h, cfg), Nx.pad(ox, pv_o, cfg), f"pad {ty}{shape}{cfg}")
+    assert_bits_equal(Nx.concatenate([hx, hx], axis=rank - 1), Nx.concatenate([ox, ox], axis=rank - 1), f"concatenate {ty}{shape}")
