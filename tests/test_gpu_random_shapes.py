@@ -109,3 +109,43 @@ def test_copies_on_random_windows(case, hip, oracle):
         pv_h, pv_o = Nx.tensor(1, type=ty, backend=hip), Nx.tensor(1, type=ty, backend=oracle)
         assert_bits_equal(Nx.pad(hx, pv_h, cfg), Nx.pad(ox, pv_o, cfg), f"pad {ty}{shape}{cfg}")
     assert_bits_equal(Nx.concatenate([hx, hx], axis=rank - 1), Nx.concatenate([ox, ox], axis=rank - 1), f"concatenate {ty}{shape}")
+
+
+DOT_M = [1, 3, 16, 33, 64, 65, 100, 128, 130, 192, 200, 256, 264, 300, 513]
+DOT_N = [1, 8, 16, 40, 64, 72, 128, 136, 256, 264, 320, 520]
+DOT_K = [1, 7, 8, 16, 24, 64, 72, 128, 136, 192, 256, 512, 1000, 1024, 4096]
+
+
+@pytest.mark.parametrize("case", range(200))
+def test_dot_on_random_shapes_types_and_layouts(case, hip, oracle):
+    """The contraction picks its kernel from the shape (generic, K-inner MFMA, the tiled kernels in four tile
+    sizes, the few-rows stream, K in splits, K extended by zeros): random extents, operand layouts, batch counts
+    and types against the oracle -- int8 exactly, floats within the accumulation bound."""
+    from test_gpu_dot import check_float_dot
+    from support import values
+    rng = np.random.default_rng(seed_of("dot", case))
+    M, N, K = int(rng.choice(DOT_M)), int(rng.choice(DOT_N)), int(rng.choice(DOT_K))
+    while M * N * K > 40_000_000:
+        M, N, K = int(rng.choice(DOT_M)), int(rng.choice(DOT_N)), int(rng.choice(DOT_K))
+    batch = int(rng.choice([1, 1, 1, 2, 3]))
+    ty = ["bf16", "f16", "f32", "s8"][int(rng.integers(0, 4))]
+    lk, rk = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))  # K-inner (True) or K-outer operand
+    if ty == "s8":
+        a = rng.integers(-127, 128, size=(batch, M, K)).astype(np.int8)
+        b = rng.integers(-127, 128, size=(batch, K, N)).astype(np.int8)
+    else:
+        a, b = rand_raw(rng, ty, (batch, M, K), lo=-1, hi=1), rand_raw(rng, ty, (batch, K, N), lo=-1, hi=1)
+    la = a if lk else np.ascontiguousarray(a.transpose(0, 2, 1))
+    lb = b if not rk else np.ascontiguousarray(b.transpose(0, 2, 1))
+    c1, c2 = [2] if lk else [1], [2] if rk else [1]
+    kw = {"out_type": "s32"} if ty == "s8" else {}
+    hla, ola = both(la, ty, hip, oracle)
+    hlb, olb = both(lb, ty, hip, oracle)
+    got = Nx.dot(hla, c1, [0], hlb, c2, [0], **kw)
+    want = Nx.dot(ola, c1, [0], olb, c2, [0], **kw)
+    what = f"dot {ty} batch {batch} {M}x{N}x{K} {'k-inner' if lk else 'k-outer'} {'k-inner' if rk else 'k-outer'}"
+    if ty == "s8":
+        assert_bits_equal(got, want, what)
+    else:
+        oa, ob = both(a, ty, hip, oracle)[1], both(b, ty, hip, oracle)[1]
+        check_float_dot(got, want, values(oa), values(ob), "bmk,bkn->bmn", K, what)
