@@ -283,8 +283,14 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
   const bool pipelined = Kb % SLAB == 0;
   // the pipelined kernel transposes K-outer operands itself when the rows come in whole blocks
   const int row_block = esz == 1 ? 16 : (esz == 2 ? 8 : 4);
-  const bool l_relay = l_layout == HIPNX_K_OUTER && !(pipelined && M % row_block == 0);
-  const bool r_relay = r_layout == HIPNX_K_OUTER && !(pipelined && N % row_block == 0);
+  // int8 on 128 x 128 tiles: a K-outer operand keeps the one-group kernel and its register-staged transposes
+  // (1024 x 2048 x 4096: 44 us against 18 us with both operands K-inner), so from 2^32 multiply-adds and K = 2048
+  // on the operand is laid out K-inner first, which costs 6-8 us
+  const bool s8_mid = l_dt == HIPNX_S8 && r_dt == HIPNX_S8 && pipelined && M > 64 && Kb >= 16 * SLAB &&
+                      (double)M * (double)N * (double)K * (double)batch >= 4294967296.0 &&
+                      !(((M + 255) / 256) * ((N + 255) / 256) * batch * 4 >= (int64_t)ctx->num_cus * 3 && M >= 192 && N >= 192);
+  const bool l_relay = l_layout == HIPNX_K_OUTER && (!(pipelined && M % row_block == 0) || s8_mid);
+  const bool r_relay = r_layout == HIPNX_K_OUTER && (!(pipelined && N % row_block == 0) || s8_mid);
   hipnx_buf *lt = nullptr, *rt = nullptr;
   int st = HIPNX_OK;
   if (l_relay) {
@@ -330,35 +336,29 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
         // tile choice: the largest tile that still gives every CU work; few rows against a long
         // weight matrix stream the weights with many small tiles
         const int64_t t256 = ((M + 255) / 256) * ((N + 255) / 256) * batch;
+        const int64_t t128 = ((M + 127) / 128) * ((N + 127) / 128);
+        const bool two_byte = l_dt == HIPNX_BF16 || l_dt == HIPNX_F16;
         int cfg;
         if (M <= 64) cfg = GEMM_CFG_64x32;
         else if (t256 * 4 >= (int64_t)ctx->num_cus * 3 && M >= 192 && N >= 192) cfg = GEMM_CFG_256;
-        else if ((l_dt == HIPNX_BF16 || l_dt == HIPNX_F16) && M >= 192 && N >= 128 &&
-                 ((M + 255) / 256) * ((N + 127) / 128) * batch * 4 >= (int64_t)ctx->num_cus * 3)
-          cfg = GEMM_CFG_256x128;  // half-width tiles of the two-group kernel fill the CUs where 256 x 256 ones do not
+        else if (two_byte && M >= 192 && N >= 128 && t128 * batch > ctx->num_cus)
+          // More 128 x 128 tiles than CUs: half-width tiles of the two-group kernel, even where they leave CUs
+          // idle (1280 x 4096 x 4096, 160 tiles: 66 us; as 320 tiles of 128 x 128 in two rounds: 76 us)
+          cfg = GEMM_CFG_256x128;
         else cfg = GEMM_CFG_128;
-        // A grid of 128 x 128 tiles that leaves most CUs idle (a few hundred rows against a long weight
-        // matrix: 128 x 4096 x 4096 is 32 tiles walking 64 slabs each) splits K over S work-groups per tile:
+        // A grid of 128 x 128 tiles that leaves three quarters of the CUs idle (a few hundred rows against a long
+        // weight matrix: 128 x 4096 x 4096 is 32 tiles walking 64 slabs each) splits K over S work-groups per tile:
         // f32 (s32) partial results in pool workspace, then one pass that adds them in split order.
         int splits = 1;
-        const int64_t t128 = ((M + 127) / 128) * ((N + 127) / 128);
         const int64_t nslab = Kb / SLAB;
         const bool splittable = cfg == GEMM_CFG_128 && batch == 1 && scale_mode == HIPNX_SCALE_NONE && (M * N) % 4 == 0 &&
                                 (l_dt == HIPNX_S8 ? !is_float(out_dt) : true);
-        // (the second pass and the partial results cost about 12 us: worth it from K = 32 slabs on, with at
-        // least 8 slabs left per split)
-        if (splittable && t128 * 2 <= ctx->num_cus && nslab >= 32)
+        // (the second pass and the partial results cost about 10 us: worth it from K = 32 slabs on, with at least
+        // 8 slabs left per split and no more work-groups than CUs; 1024 x 2048 x 2048, 128 tiles, is faster whole:
+        // 21 us against 22 us in two halves and 27 us in four quarters)
+        if (splittable && t128 * 2 <= ctx->num_cus && nslab >= (t128 * 4 <= ctx->num_cus ? 32 : 64))
           for (int cand = 16; cand >= 2; cand /= 2)
-            if (t128 * cand <= 2 * (int64_t)ctx->num_cus && nslab % cand == 0 && nslab / cand >= 8) { splits = cand; break; }
-        // Between the two: a half-width grid of the two-group kernel that covers 3/8 to 3/4 of the CUs, walked in
-        // two halves of K when K is long (64 slabs or more; 768 x 4096 x 4096: 51 -> 45 us, 1024 x 4096 x 4096: 53 -> 50 us)
-        const int64_t tw = ((M + 255) / 256) * ((N + 127) / 128);
-        if (splits == 1 && cfg == GEMM_CFG_128 && (l_dt == HIPNX_BF16 || l_dt == HIPNX_F16) && batch == 1 && M >= 192 && N >= 128 &&
-            scale_mode == HIPNX_SCALE_NONE && (M * N) % 4 == 0 && nslab >= 64 && nslab % 2 == 0 &&
-            tw * 8 >= (int64_t)ctx->num_cus * 3 && tw * 2 <= (int64_t)ctx->num_cus + ctx->num_cus / 4) {
-          cfg = GEMM_CFG_256x128;
-          splits = 2;
-        }
+            if (t128 * cand <= (int64_t)ctx->num_cus && nslab % cand == 0 && nslab / cand >= 8) { splits = cand; break; }
         void *ws = nullptr;
         size_t ws_cap = 0;
         if (splits > 1 && pool_alloc(ctx, (size_t)splits * M * N * 4, &ws, &ws_cap) != HIPNX_OK) splits = 1;

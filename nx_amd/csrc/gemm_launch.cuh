@@ -11,7 +11,7 @@ namespace hipnx {
 enum {
   GEMM_CFG_256x128 = 3,  // 256 x 128, the two-group kernel with half-width wave tiles: 2-byte types whose 256 x 256 grid is too small
   GEMM_CFG_256 = 0,  // 256 x 256, 8 waves (4 x 2, each 64 x 128): large square-ish problems
-  GEMM_CFG_128 = 1,  // 128 x 128, 4 waves (2 x 2, each 64 x 64): mid-size and batched problems
+  GEMM_CFG_128 = 1,  // 128 x 128: mid-size and batched problems; 4 waves (2 x 2, each 64 x 64), or two such groups sharing K
   GEMM_CFG_64x32 = 2 // 64 x 32, 2 waves: few rows against a long weight matrix (HBM streaming)
 };
 
@@ -64,6 +64,25 @@ static int launch_pingpong(const hipnx_ctx *ctx, GemmArgs a, int64_t batch) {
   return HIPNX_OK;
 }
 
+// the two-group 128 x 128 kernel: four LDS stages of 32 KiB, one work-group per CU
+template <int DT, bool LK, bool RK>
+static int launch_pingpong128(const hipnx_ctx *ctx, GemmArgs a, int64_t batch) {
+  constexpr int smem = 4 * 256 * SLAB;
+  auto kern = gemm_pingpong128_kernel<DT, LK, RK>;
+  static bool configured = false;
+  if (!configured) {
+    HIPNX_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
+    configured = true;
+  }
+  a.tiles_m = (int)((a.M + 127) / 128);
+  a.tiles_n = (int)((a.N + 127) / 128);
+  a.group_m = gemm_group_m(a.tiles_m, a.tiles_n);
+  dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)batch), block(512);
+  hipLaunchKernelGGL(kern, grid, block, smem, ctx->stream, a);
+  HIPNX_HIP(hipGetLastError());
+  return HIPNX_OK;
+}
+
 template <int DT, bool LK, bool RK>
 static int launch_cfg(const hipnx_ctx *ctx, int cfg, const GemmArgs &a, int64_t batch) {
   switch (cfg) {
@@ -84,6 +103,15 @@ static int launch_cfg(const hipnx_ctx *ctx, int cfg, const GemmArgs &a, int64_t 
       // operand is copied straight into LDS (the condition of the kernel's L_TR / R_TR)
       constexpr int ES = DT == HIPNX_S8 ? 1 : DT == HIPNX_F32 ? 4 : 2;
       constexpr bool tr = ES <= 2 && 128 * ES >= 256;
+      // From 8 slabs of K on, the two-group kernel (2-byte types; int8 with both operands K-inner): 730 clocks per
+      // slab against the 1600-2100 below.  It holds a CU's LDS alone, so for the 2-byte types only where no
+      // second work-group would share the CU; int8 has no wider two-group tile to fall back on and takes it
+      // for every grid (2048 x 4096 x 4096, 512 tiles: 52 -> 42 us).
+      if constexpr (DT == HIPNX_BF16 || DT == HIPNX_F16 || (DT == HIPNX_S8 && LK && RK)) {
+        const int64_t groups = ((a.M + 127) / 128) * ((a.N + 127) / 128) * batch;
+        if (a.Kb >= 8 * SLAB && a.ld_l < (1ll << 23) && a.ld_r < (1ll << 23) && (DT == HIPNX_S8 || groups <= ctx->num_cus))
+          return launch_pingpong128<DT, LK, RK>(ctx, a, batch);
+      }
       if constexpr ((LK || tr) && (RK || tr)) {
         // (128 KiB of LDS: one work-group per CU, so only where the grid has no second one to give it)
         const int64_t groups = ((a.M + 127) / 128) * ((a.N + 127) / 128) * batch;

@@ -264,4 +264,195 @@ gemm_pingpong_kernel(GemmArgs a) {
   }
 }
 
+// ---- the two-group walk on a 128 x 128 tile ----------------------------------------------------------
+//
+// Problems with fewer than a few hundred tiles of 256 x 128 take 128 x 128 tiles, one per CU.  The one-group
+// kernel (gemm_pipelined_kernel) has a single wave per SIMD there, which reads its fragments and issues its
+// MFMAs in turn: 1600-2100 clocks per slab for 512 clocks of MFMA work.  Here two groups of four waves walk
+// the same tile, each with the one-group kernel's wave tiles of 64 x 64 (so no more LDS traffic than there),
+// and share K: group 0 takes the even slabs, group 1 the odd ones.  In phase p the group p % 2 reads the 16
+// fragments of slab p and requests slab p + 3 while the other group issues the 32 MFMAs of slab p - 1; the
+// two partial sums meet in LDS at the end, where each group takes over the finished half (32 rows of every
+// wave tile) it then scales, converts and stores.
+//
+// A slab (both operands) is 32 KiB, the four LDS stages hold slabs p .. p + 3.  Slab p + 3 lands in the stage
+// of slab p - 1, whose last reader waited for its fragments before the barrier that opened phase p.  The
+// waves that requested a slab wait for it at the end of their next memory phase (vmcnt(8): all but the slab
+// requested just now), two phases later, and the barrier behind that wait opens the phase that reads it.
+template <int DT, bool L_KIN, bool R_KIN>
+__global__ void __launch_bounds__(512)
+gemm_pingpong128_kernel(GemmArgs a) {
+  typedef typename Mma16<DT>::acc_t acc_t;
+  constexpr int BM = 128, BN = 128, TM16 = 4, TN16 = 4, NSTAGE = 4, AHEAD = NSTAGE - 1;
+  constexpr int STAGE = (BM + BN) * SLAB;
+  constexpr int ES = (DT == HIPNX_S8) ? 1 : 2;
+  static_assert(DT == HIPNX_BF16 || DT == HIPNX_F16 || (DT == HIPNX_S8 && L_KIN && R_KIN), "2-byte MFMA types; int8 with K-inner operands");
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+
+  int tm, tn;
+  gemm_tile_position(a, blockIdx.x, tm, tn);
+  const int64_t b = blockIdx.y;
+  const unsigned char *lb = a.l + b * a.bs_l;
+  const unsigned char *rb = a.r + b * a.bs_r;
+  const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int grp = wave >> 2, w4 = wave & 3;  // waves w and w + 4 share a SIMD and a wave tile
+  const int wm = (w4 >> 1) * 64, wn = (w4 & 1) * 64;
+
+  acc_t acc[TM16][TN16];
+#pragma unroll
+  for (int i = 0; i < TM16; i++)
+#pragma unroll
+    for (int j = 0; j < TN16; j++)
+#pragma unroll
+      for (int q = 0; q < 4; q++) acc[i][j][q] = 0;
+
+  // the four waves of the memory group request a whole slab: 4 + 4 instructions per wave
+  PPKInnerLoader<128, 4> lkin, rkin;
+  PPKOuterLoader<2, 128, 4> lkout, rkout;
+  if constexpr (L_KIN) lkin.init(lb, a.ld_l, m0, a.M, w4, lane);
+  else lkout.init(lb, a.ld_l, m0, a.M, w4, lane);
+  if constexpr (R_KIN) rkin.init(rb, a.ld_r, n0, a.N, w4, lane);
+  else rkout.init(rb, a.ld_r, n0, a.N, w4, lane);
+  auto issue = [&](int slab) __attribute__((always_inline)) {
+    unsigned char *dst = smem + (slab % NSTAGE) * STAGE;
+    const int64_t kbyte0 = (int64_t)slab * SLAB;
+    if constexpr (L_KIN) lkin.issue(kbyte0, dst, w4);
+    else lkout.issue(kbyte0 / ES, a.ld_l, dst, w4);
+    if constexpr (R_KIN) rkin.issue(kbyte0, dst + BM * SLAB, w4);
+    else rkout.issue(kbyte0 / ES, a.ld_r, dst + BM * SLAB, w4);
+  };
+
+  int a_rd[2], b_rd[2];
+  if constexpr (L_KIN) {
+    const int row = wm + (lane & 15);
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) a_rd[ks] = row * SLAB + lds_slot16(row, 4 * ks + (lane >> 4)) * 16;
+  }
+  if constexpr (R_KIN) {
+    const int row = wn + (lane & 15);
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) b_rd[ks] = BM * SLAB + row * SLAB + lds_slot16(row, 4 * ks + (lane >> 4)) * 16;
+  }
+
+  const int nslab = (int)(a.Kb / SLAB);
+  v4i fa[2][TM16], fb[2][TN16];
+  auto mem_phase = [&](int p) __attribute__((always_inline)) {
+    const unsigned char *cur = smem + (p % NSTAGE) * STAGE;
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) {
+#pragma unroll
+      for (int i = 0; i < TM16; i++) {
+        if constexpr (L_KIN) fa[ks][i] = *reinterpret_cast<const v4i *>(cur + a_rd[ks] + i * (16 * SLAB));
+        else fa[ks][i] = read_fragment_tr<2, BM>(cur, wm + 16 * i, ks, lane);
+      }
+#pragma unroll
+      for (int j = 0; j < TN16; j++) {
+        if constexpr (R_KIN) fb[ks][j] = *reinterpret_cast<const v4i *>(cur + b_rd[ks] + j * (16 * SLAB));
+        else fb[ks][j] = read_fragment_tr<2, BN>(cur + BM * SLAB, wn + 16 * j, ks, lane);
+      }
+    }
+    if (p + AHEAD < nslab) {
+      issue(p + AHEAD);
+      wait_vmcnt<8>();
+    } else {
+      wait_vmcnt<0>();
+    }
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the fragments are in registers
+  };
+  auto compute_phase = [&]() __attribute__((always_inline)) {
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+      for (int j = 0; j < TN16; j++)
+#pragma unroll
+        for (int i = 0; i < TM16; i++) Mma16<DT>::step(acc[i][j], fb[ks][j], fa[ks][i]);
+    __builtin_amdgcn_s_setprio(0);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  // prologue: group 0 requests slabs 0 and 2, group 1 slab 1; slab 0 is awaited here, slab 1 by group 1
+  // before the barrier that ends phase 0, slab 2 by group 0 at the end of its first memory phase
+  if (grp == 0) {
+    issue(0);
+    if (2 < nslab) {
+      issue(2);
+      wait_vmcnt<8>();
+    } else {
+      wait_vmcnt<0>();
+    }
+  } else if (1 < nslab) {
+    issue(1);
+  }
+  __builtin_amdgcn_s_barrier();
+
+  // phases 0 .. nslab, every wave passes the barrier that ends each of them
+  if (grp == 0) {
+    for (int p = 0; p <= nslab; p += 2) {
+      if (p < nslab) mem_phase(p);
+      __builtin_amdgcn_s_barrier();
+      if (p + 1 > nslab) break;
+      compute_phase();
+      __builtin_amdgcn_s_barrier();
+    }
+  } else {
+    wait_vmcnt<0>();
+    for (int p = 0; p <= nslab; p += 2) {
+      __builtin_amdgcn_s_barrier();
+      if (p + 1 > nslab) break;
+      if (p + 1 < nslab) mem_phase(p + 1);
+      __builtin_amdgcn_s_barrier();
+      if (p + 1 < nslab) compute_phase();
+    }
+  }
+
+  // the two partial sums: every wave hands the half of its tile the other group finishes to that group
+  // (2 x 4 accumulator tiles, 8 KiB per wave, 64 KiB in all) and adds what it is handed
+  {
+    unsigned char *mine = smem + wave * 8192, *theirs = smem + (wave ^ 4) * 8192;
+    // (a branch per group rather than a selection per tile: the accumulators must keep constant indices)
+    if (grp == 0) {
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < TN16; j++) *reinterpret_cast<acc_t *>(mine + (i * TN16 + j) * 1024 + lane * 16) = acc[i + 2][j];
+    } else {
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < TN16; j++) *reinterpret_cast<acc_t *>(mine + (i * TN16 + j) * 1024 + lane * 16) = acc[i][j];
+    }
+    __syncthreads();
+    acc_t fin[2][TN16];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+      for (int j = 0; j < TN16; j++) fin[i][j] = *reinterpret_cast<const acc_t *>(theirs + (i * TN16 + j) * 1024 + lane * 16);
+    // the even slabs' sum first, as a single walk over K would have it
+    if (grp == 0) {
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < TN16; j++) fin[i][j] = acc[i][j] + fin[i][j];
+    } else {
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < TN16; j++) fin[i][j] = fin[i][j] + acc[i + 2][j];
+    }
+    const int64_t obase = b * a.M * a.N;
+    unsigned char *turn = smem + 65536 + wave * 4096;  // past the exchanged halves, which the other group may still be reading
+    switch (a.odt) {
+#define HIPNX_EPI(T) case T: gemm_epilogue<DT, T, 2, TN16>(fin, a.out, obase, a.M, a.N, m0 + wm + grp * 32, n0 + wn, lane, a.scale, a.scale_mode, turn); break;
+      HIPNX_EPI(HIPNX_BF16) HIPNX_EPI(HIPNX_F16) HIPNX_EPI(HIPNX_F32) HIPNX_EPI(HIPNX_F64) HIPNX_EPI(HIPNX_BF16_RNE)
+      HIPNX_EPI(HIPNX_S8) HIPNX_EPI(HIPNX_U8) HIPNX_EPI(HIPNX_S16) HIPNX_EPI(HIPNX_U16)
+      HIPNX_EPI(HIPNX_S32) HIPNX_EPI(HIPNX_U32) HIPNX_EPI(HIPNX_S64) HIPNX_EPI(HIPNX_U64)
+#undef HIPNX_EPI
+    }
+  }
+}
+
 }  // namespace hipnx

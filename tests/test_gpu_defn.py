@@ -2,6 +2,8 @@
 (nx/lib/nx/defn/evaluator.ex:363-388).  The device runs the traced function, the oracle runs the
 same function eagerly and traced; exact ops are compared bit for bit, transcendental chains within
 the tolerances of the per-op tests."""
+import gc
+
 import numpy as np
 import pytest
 
@@ -66,6 +68,7 @@ def test_intermediates_go_back_to_the_pool_during_the_walk(hip):
             t = Nx.exp(Nx.negate(t))
         return t
     defn.jit(chain)(x)  # warm the pool
+    gc.collect()  # tensors earlier tests left behind must not be freed in the middle of the walk
     before = mem_stats()["live"]
     seen = []
     original = defn._Run.apply

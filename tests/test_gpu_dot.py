@@ -320,3 +320,58 @@ def test_two_byte_outputs_land_in_their_own_columns(ty, M, N, K, hip):
     want = values(from_numpy(np.ascontiguousarray(a[:, pick]), ty, hip))
     assert got.shape == (M, N)
     assert np.array_equal(got, want)  # (-0.0 == 0.0: a lone product plus zeros may lose the sign of a zero)
+
+
+@pytest.mark.parametrize("ty,M,N,K", [("bf16", 1024, 1024, 1024), ("bf16", 1000, 904, 576), ("f16", 520, 1288, 640), ("bf16", 200, 136, 512),
+                                      ("s8", 1024, 1024, 1024), ("s8", 2056, 3080, 1152), ("f16", 2048, 2048, 1088)])
+@pytest.mark.parametrize("layout", ["nn", "nt", "tn", "tt"])
+def test_two_groups_sharing_k_on_128_tiles(ty, M, N, K, layout, hip, oracle):
+    """Grids of 128 x 128 tiles that fit the CUs once (for int8: any grid, both operands K-inner) are walked by two
+    groups of waves that take the even and the odd slabs of K and add their partial sums at the end: even and odd
+    numbers of slabs, whole and ragged grids, all four layouts.  int8 exact, floats within the bound."""
+    rng = np.random.default_rng(seed_of(ty, M, N, K, layout, "pp128"))
+    if ty == "s8":
+        a = rng.integers(-127, 128, size=(M, K)).astype(np.int8)
+        b = rng.integers(-127, 128, size=(K, N)).astype(np.int8)
+    else:
+        a, b = rand_raw(rng, ty, (M, K), lo=-1, hi=1), rand_raw(rng, ty, (K, N), lo=-1, hi=1)
+    la = a if layout[0] == "n" else np.ascontiguousarray(a.T)
+    lb = b if layout[1] == "n" else np.ascontiguousarray(b.T)
+    c1 = [1] if layout[0] == "n" else [0]
+    c2 = [0] if layout[1] == "n" else [1]
+    kw = {"out_type": "s32"} if ty == "s8" else {}
+    got = Nx.dot(from_numpy(la, ty, hip), c1, from_numpy(lb, ty, hip), c2, **kw)
+    assert got.shape == (M, N)
+    rows = np.unique(np.concatenate([[0, 31, 32, 63, 64, 127, 128, M - 1], rng.integers(0, M, size=16)]))
+    oa, ob = from_numpy(np.ascontiguousarray(a[rows]), ty, oracle), from_numpy(b, ty, oracle)
+    want = Nx.dot(oa, ob, **kw)
+    got_rows = from_numpy(np.ascontiguousarray(hip.to_numpy(got)[rows]), "s32" if ty == "s8" else ty, oracle)
+    if ty == "s8":
+        assert_bits_equal(got_rows, want, f"128 tiles, two groups, s8 {layout}")
+    else:
+        check_float_dot(got_rows, want, values(oa), values(ob), "mk,kn->mn", K, f"128 tiles, two groups, {ty} {layout}")
+
+
+@pytest.mark.parametrize("ty,M,N,K,out_type", [("bf16", 1024, 1032, 1024, None), ("f16", 520, 776, 576, None), ("bf16", 768, 512, 640, "f32"),
+                                               ("s8", 1024, 520, 1152, "s32"), ("s8", 264, 392, 1024, "s8")])
+def test_two_groups_sharing_k_put_every_output_in_its_place(ty, M, N, K, out_type, hip):
+    """A selection matrix (a single 1 per column, spread over even and odd slabs) makes every output a copy of one
+    input element: a tile half, row or column that ends up with the wrong group shows as a wrong value -- exact."""
+    rng = np.random.default_rng(seed_of(ty, M, N, K, "pp128 pick"))
+    pick = (37 * np.arange(N) + 11) % K
+    if ty == "s8":
+        a = rng.integers(-127, 128, size=(M, K)).astype(np.int8)
+        b = np.zeros((N, K), dtype=np.int8)
+        b[np.arange(N), pick] = 1
+        got = hip.to_numpy(Nx.dot(from_numpy(a, ty, hip), [1], from_numpy(b, ty, hip), [1], out_type=out_type))
+        assert got.shape == (M, N)
+        assert np.array_equal(got.astype(np.int64), a[:, pick].astype(np.int64))
+        return
+    a = rand_raw(rng, ty, (M, K), lo=-1, hi=1)
+    b = np.zeros((K, N), dtype=a.dtype)
+    b[pick, np.arange(N)] = np.uint16(0x3F80) if ty == "bf16" else np.float16(1.0)
+    kw = {"out_type": out_type} if out_type else {}
+    got = values(Nx.dot(from_numpy(a, ty, hip), from_numpy(b, ty, hip), **kw))
+    want = values(from_numpy(np.ascontiguousarray(a[:, pick]), ty, hip))
+    assert got.shape == (M, N)
+    assert np.array_equal(got, want)
