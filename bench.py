@@ -294,7 +294,18 @@ def main():
         ma, mb = put(a_np[:2048, :2048].copy(), "bf16"), put(b_np[:2048, :2048].copy(), "bf16")
         _, ms = tstat(lambda: Nx.dot(ma, mb), steps, warm)
         entry("dot_bf16_2048", 2.0 * 2048 ** 3, "TFLOP/s", ms, PEAK["bf16"], "mfma", "mfma_bf16")
-        del xa, wb, ma, mb
+        # a prefill-sized batch against the weight matrix (256 tiles of 128 x 128, 64 slabs of K each)
+        pa = put(a_np[:1024].copy(), "bf16")
+        _, ms = tstat(lambda: Nx.dot(pa, b), steps, warm)
+        entry("dot_bf16_1024x4096x4096", 2.0 * 1024 * 4096 * 4096, "TFLOP/s", ms, PEAK["bf16"], "mfma", "mfma_bf16")
+        # mid-size int8: both operands K-inner, and the plain layout (right operand K-outer, laid out K-inner first)
+        qa, qb = (put(q, "s8") for q in W.dense_gemm_s8(n=2048))
+        qbt = Nx.transpose(qb)
+        _, ms = tstat(lambda: Nx.dot(qa, [1], qbt, [1], out_type="s32"), steps, warm)
+        entry("dot_s8_2048_s32_kinner", 2.0 * 2048 ** 3, "TOP/s", ms, PEAK["s8"], "mfma", "mfma_s8")
+        _, ms = tstat(lambda: Nx.dot(qa, qb, out_type="s32"), steps, warm)
+        entry("dot_s8_2048_s32", 2.0 * 2048 ** 3, "TOP/s", ms, PEAK["s8"], "mfma", "mfma_s8")
+        del xa, wb, ma, mb, pa, qa, qb, qbt
         ha, hb = put(W.bf16_to_f32(a_np).astype(np.float16), "f16"), put(W.bf16_to_f32(b_np).astype(np.float16), "f16")
         _, ms = tstat(lambda: Nx.dot(ha, hb), steps, warm, msettle)
         entry("dot_f16_4096", flop, "TFLOP/s", ms, PEAK["f16"], "mfma", "mfma_f16")
