@@ -152,17 +152,42 @@ reduce_cols_kernel(const void *__restrict__ in, void *__restrict__ out, typename
   }
 }
 
-// fold partial[outer, nseg, inner] -> out[outer, inner]
+// fold partial[outer, nseg, inner] -> out[outer, inner].  A work-group takes 32 adjacent outputs; its eight rows
+// of 32 lanes each fold a slice of the segments (four loads in flight per lane), and the first row folds the eight
+// slices in segment order.  (One lane per output walking all segments is a chain of up to 1024 dependent
+// round trips to L2: 30-50 us on a 4096 x 4096 input, more than the first pass.)
+constexpr int COMBINE_COLS_X = 32, COMBINE_COLS_Y = BLOCK / COMBINE_COLS_X;
 template <typename R>
 __global__ void __launch_bounds__(BLOCK)
 combine_cols_kernel(const typename R::acc_t *__restrict__ partial, void *__restrict__ out, int odt, int64_t outer,
                     int64_t inner, int nseg) {
+  typedef typename R::acc_t acc_t;
+  __shared__ acc_t sm[COMBINE_COLS_Y][COMBINE_COLS_X];
+  const int tx = threadIdx.x % COMBINE_COLS_X, ty = threadIdx.x / COMBINE_COLS_X;
   const int64_t total = outer * inner;
-  for (int64_t t = (int64_t)blockIdx.x * BLOCK + threadIdx.x; t < total; t += (int64_t)gridDim.x * BLOCK) {
-    const int64_t o = t / inner, i = t - o * inner;
-    typename R::acc_t acc = R::init();
-    for (int s = 0; s < nseg; s++) acc = R::combine(acc, partial[(o * nseg + s) * inner + i]);
-    finalize(out, odt, t, acc);
+  const int per = (nseg + COMBINE_COLS_Y - 1) / COMBINE_COLS_Y;
+  const int s0 = ty * per, s1 = s0 + per < nseg ? s0 + per : nseg;
+  for (int64_t t0 = (int64_t)blockIdx.x * COMBINE_COLS_X; t0 < total; t0 += (int64_t)gridDim.x * COMBINE_COLS_X) {
+    const int64_t t = t0 + tx;
+    acc_t acc = R::init();
+    if (t < total) {
+      const int64_t o = t / inner, i = t - o * inner;
+      const acc_t *p = partial + o * nseg * inner + i;
+      int sgm = s0;
+      for (; sgm + 3 < s1; sgm += 4) {
+        const acc_t a0 = p[(int64_t)sgm * inner], a1 = p[(int64_t)(sgm + 1) * inner], a2 = p[(int64_t)(sgm + 2) * inner], a3 = p[(int64_t)(sgm + 3) * inner];
+        acc = R::combine(R::combine(R::combine(R::combine(acc, a0), a1), a2), a3);
+      }
+      for (; sgm < s1; sgm++) acc = R::combine(acc, p[(int64_t)sgm * inner]);
+    }
+    sm[ty][tx] = acc;
+    __syncthreads();
+    if (ty == 0 && t < total) {
+#pragma unroll
+      for (int y = 1; y < COMBINE_COLS_Y; y++) acc = R::combine(acc, sm[y][tx]);
+      finalize(out, odt, t, acc);
+    }
+    __syncthreads();
   }
 }
 
@@ -248,7 +273,13 @@ static int run_reduce_t(hipnx_ctx *ctx, bool static_ws, int idt, int odt, int64_
     const int64_t lanes = outer * (inner / (vec ? E : 1));
     int nseg = 1;
     int64_t seg_len = red;
-    const int64_t want_lanes = target_units * BLOCK / 4;
+    // Waves wanted per CU: what keeps about 128 bytes per lane-row times 64 lanes in flight -- 4 for f32 (32 bytes
+    // per lane and row), 8 for 2-byte types, 16 for bytes (measured on 16384 x 16384: f32 6.3 TB/s with 4 against
+    // 6.0 with 8 and 5.0 with 16; bf16 5.3 / 5.7 / 5.0; u8 2.5 / 3.6 / 4.7).  More segments than that only add
+    // partial results.
+    const int lane_bytes = (vec ? E : 1) * dtype_size(idt);
+    const int colw = lane_bytes >= 64 ? 2 : lane_bytes <= 8 ? 16 : 128 / lane_bytes;
+    const int64_t want_lanes = (int64_t)ctx->num_cus * colw * WAVE;
     if (lanes < want_lanes && red >= 64) {
       int64_t want = want_lanes / (lanes > 0 ? lanes : 1), maxs = red / 32;
       nseg = (int)(want < maxs ? want : maxs);
@@ -272,7 +303,7 @@ static int run_reduce_t(hipnx_ctx *ctx, bool static_ws, int idt, int odt, int64_
       if (vec) hipLaunchKernelGGL((reduce_cols_kernel<R, CT, true, IDT>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, outer, red, inner, seg_len, nseg);
       else hipLaunchKernelGGL((reduce_cols_kernel<R, CT, false>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, outer, red, inner, seg_len, nseg);
       if (nseg > 1) {
-        int64_t b2 = (outer * inner + BLOCK - 1) / BLOCK;
+        int64_t b2 = (outer * inner + COMBINE_COLS_X - 1) / COMBINE_COLS_X;
         dim3 g2((unsigned)(b2 < cap ? b2 : cap));
         hipLaunchKernelGGL((combine_cols_kernel<R>), g2, block, 0, ctx->stream, partial, out, odt, outer, inner, nseg);
       }
