@@ -356,7 +356,26 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
         // (the second pass and the partial results cost about 10 us: worth it from K = 32 slabs on, with at least
         // 8 slabs left per split and no more work-groups than CUs; 1024 x 2048 x 2048, 128 tiles, is faster whole:
         // 21 us against 22 us in two halves and 27 us in four quarters)
-        if (splittable && t128 * 2 <= ctx->num_cus && nslab >= (t128 * 4 <= ctx->num_cus ? 32 : 64))
+        if (l_dt == HIPNX_F32) {
+          // An f32 slab is eight times the MFMA work of a 2-byte one (2.6 us per slab of a 128 x 128 tile, 0.55 us
+          // for a 64 x 32 tile, the second pass of a split about 8 us), so a grid that leaves CUs idle is cut much
+          // earlier: the cheapest, by those figures, of whole 128 x 128 tiles, K split up to 64 ways (2 slabs or
+          // more each) and 64 x 32 tiles.  512^3: 41 -> 18 us; 256 x 256 x 16384: 84 -> 40 us.
+          if (cfg == GEMM_CFG_128) {
+            const int64_t cus = ctx->num_cus;
+            auto rounds = [&](int64_t groups) { return (double)((groups + cus - 1) / cus); };
+            double best = 10.0 + rounds(t128 * batch) * (double)nslab * 2.6;
+            if (splittable)
+              for (int cand = 2; cand <= 64; cand *= 2) {
+                if (t128 * cand > cus || nslab % cand != 0 || nslab / cand < 2) continue;
+                // second launch, then the partial results written and read once (mostly from cache: ~8 MB per us)
+                const double t = 15.0 + (double)(nslab / cand) * 2.6 + 2.0 * (double)cand * (double)(M * N) * 4.0 / 8.0e6;
+                if (t < best) { best = t; splits = cand; }
+              }
+            const int64_t t64 = ((M + 63) / 64) * ((N + 31) / 32) * batch;
+            if (10.0 + rounds(t64) * (double)nslab * 0.55 < best) { cfg = GEMM_CFG_64x32; splits = 1; }
+          }
+        } else if (splittable && t128 * 2 <= ctx->num_cus && nslab >= (t128 * 4 <= ctx->num_cus ? 32 : 64))
           for (int cand = 16; cand >= 2; cand /= 2)
             if (t128 * cand <= (int64_t)ctx->num_cus && nslab % cand == 0 && nslab / cand >= 8) { splits = cand; break; }
         void *ws = nullptr;

@@ -275,7 +275,9 @@ def test_contraction_lengths_off_the_slab_grid_are_padded(ty, M, N, K, layout, h
 
 @pytest.mark.parametrize("ty,M,N,K", [("bf16", 128, 1024, 4096), ("s8", 128, 1024, 4096), ("f16", 200, 520, 2048), ("f32", 132, 384, 2048),
                                       ("bf16", 768, 4096, 4096), ("f16", 1000, 4100, 4096),
-                                      ("s8", 384, 512, 8192), ("bf16", 512, 1024, 2048)])
+                                      ("s8", 384, 512, 8192), ("bf16", 512, 1024, 2048),
+                                      # f32 is cut much earlier: 64 ways, two ways with two slabs each, 64 x 32 tiles
+                                      ("f32", 256, 264, 4096), ("f32", 128, 128, 128), ("f32", 520, 512, 512), ("f32", 1024, 1024, 1024)])
 @pytest.mark.parametrize("layout", ["nn", "nt", "tn", "tt"])
 def test_long_k_on_an_under_filled_grid_is_split(ty, M, N, K, layout, hip, oracle):
     """A few hundred rows against a long K leave most CUs without a 128 x 128 tile; K is then split over
