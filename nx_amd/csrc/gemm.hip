@@ -194,6 +194,10 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
                     int64_t K, int l_layout, int r_layout, const hipnx_buf *l, const hipnx_buf *r,
                     hipnx_buf *out, int scale_mode, const hipnx_buf *scale);
 
+static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batch, int64_t M, int64_t N,
+                    int64_t K, int l_layout, int r_layout, const hipnx_buf *l, const hipnx_buf *r,
+                    hipnx_buf *out, int scale_mode, const hipnx_buf *scale);
+
 // A copy of a dot operand ([batch, rows, K] or [batch, K, rows]) with K extended to Kp by zeros.
 static int pad_k(hipnx_ctx *ctx, int esz, int64_t batch, int64_t rows, int64_t K, int64_t Kp, int layout,
                  const hipnx_buf *in, hipnx_buf **out) {
@@ -288,7 +292,7 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
   // on the operand is laid out K-inner first, which costs 6-8 us
   const bool s8_mid = l_dt == HIPNX_S8 && r_dt == HIPNX_S8 && pipelined && M > 64 && Kb >= 16 * SLAB &&
                       (double)M * (double)N * (double)K * (double)batch >= 4294967296.0 &&
-                      !(((M + 255) / 256) * ((N + 255) / 256) * batch * 4 >= (int64_t)ctx->num_cus * 3 && M >= 192 && N >= 192);
+                      !(((M + 255) / 256) * ((N + 255) / 256) * batch * 2 >= (int64_t)ctx->num_cus && M >= 192 && N >= 192);  // (those take 256 x 256 tiles)
   const bool l_relay = l_layout == HIPNX_K_OUTER && (!(pipelined && M % row_block == 0) || s8_mid);
   const bool r_relay = r_layout == HIPNX_K_OUTER && (!(pipelined && N % row_block == 0) || s8_mid);
   hipnx_buf *lt = nullptr, *rt = nullptr;
@@ -339,12 +343,18 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
         const int64_t t128 = ((M + 127) / 128) * ((N + 127) / 128);
         const bool two_byte = l_dt == HIPNX_BF16 || l_dt == HIPNX_F16;
         int cfg;
+        const bool big_ok = M >= 192 && N >= 192;
+        const int64_t tw = ((M + 255) / 256) * ((N + 127) / 128) * batch;
         if (M <= 64) cfg = GEMM_CFG_64x32;
-        else if (t256 * 4 >= (int64_t)ctx->num_cus * 3 && M >= 192 && N >= 192) cfg = GEMM_CFG_256;
+        else if (t256 * 4 >= (int64_t)ctx->num_cus * 3 && big_ok) cfg = GEMM_CFG_256;
         else if (two_byte && M >= 192 && N >= 128 && t128 * batch > ctx->num_cus)
-          // More 128 x 128 tiles than CUs: half-width tiles of the two-group kernel, even where they leave CUs
-          // idle (1280 x 4096 x 4096, 160 tiles: 66 us; as 320 tiles of 128 x 128 in two rounds: 76 us)
-          cfg = GEMM_CFG_256x128;
+          // More 128 x 128 tiles than CUs: half-width tiles of the two-group kernel while they fit the CUs in one
+          // round, even where they leave some idle (1280 x 4096 x 4096, 160 tiles: 66 us; as 320 tiles of
+          // 128 x 128 in two rounds: 76 us); where they would need a second round, full tiles on what is then more
+          // than half of the CUs (3072^3: 144 tiles of 256 x 256 72 us, 288 half-width tiles 100 us)
+          cfg = tw <= ctx->num_cus || !big_ok ? GEMM_CFG_256x128 : GEMM_CFG_256;
+        else if (l_dt == HIPNX_S8 && big_ok && t256 * 2 >= ctx->num_cus)
+          cfg = GEMM_CFG_256;  // int8 has no half-width tile: full tiles from half of the CUs on (3072^3: 46 us against 57 us)
         else cfg = GEMM_CFG_128;
         // A grid of 128 x 128 tiles that leaves three quarters of the CUs idle (a few hundred rows against a long
         // weight matrix: 128 x 4096 x 4096 is 32 tiles walking 64 slabs each) splits K over S work-groups per tile:
