@@ -345,7 +345,9 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
         int cfg;
         const bool big_ok = M >= 192 && N >= 192;
         const int64_t tw = ((M + 255) / 256) * ((N + 127) / 128) * batch;
-        if (M <= 64) cfg = GEMM_CFG_64x32;
+        // few rows: 64-row tiles, except for a 2-byte K-outer operand (x . W with W stored [K, N]), which only the
+        // 128-row kernels read by transposing loads (64 x 4096 x 4096 bf16: 72 us on 64 x 32 tiles, 19 us here)
+        if (M <= 64 && !(two_byte && !(l_kin && r_kin) && N >= 128)) cfg = GEMM_CFG_64x32;
         else if (t256 * 4 >= (int64_t)ctx->num_cus * 3 && big_ok) cfg = GEMM_CFG_256;
         else if (two_byte && M >= 192 && N >= 128 && t128 * batch > ctx->num_cus)
           // More 128 x 128 tiles than CUs: half-width tiles of the two-group kernel while they fit the CUs in one
@@ -413,8 +415,6 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
             if (e != hipSuccess) st = hip_fail(e, "split-K combine launch");
           }
           pool_free(ctx, ws, ws_cap);  // later work is ordered on the same stream
-        } else if (M <= 64 && l_kin && r_kin && Kb % 4096 == 0 && N >= 256) {
-          st = launch_gemm_rows(ctx, l_dt, a, batch);  // weights streamed once, never through LDS
         } else
         switch (l_dt) {
           case HIPNX_BF16: st = launch_gemm_bf16(ctx, cfg, l_kin, r_kin, a, batch); break;

@@ -19,8 +19,6 @@ int launch_gemm_bf16(const hipnx_ctx *ctx, int cfg, bool l_kin, bool r_kin, Gemm
 int launch_gemm_f16(const hipnx_ctx *ctx, int cfg, bool l_kin, bool r_kin, GemmArgs a, int64_t batch);
 int launch_gemm_f32(const hipnx_ctx *ctx, int cfg, bool l_kin, bool r_kin, GemmArgs a, int64_t batch);
 int launch_gemm_s8(const hipnx_ctx *ctx, int cfg, bool l_kin, bool r_kin, GemmArgs a, int64_t batch);
-// few rows (M <= 64) against a long K-inner matrix, Kb a multiple of 4096: gemm_rows.hip
-int launch_gemm_rows(const hipnx_ctx *ctx, int dt, GemmArgs a, int64_t batch);
 
 template <int DT, int WM, int WN, int TM, int TN, bool LK, bool RK, int NSTAGE = 2>
 static int launch_one(const hipnx_ctx *ctx, GemmArgs a, int64_t batch) {
@@ -64,18 +62,19 @@ static int launch_pingpong(const hipnx_ctx *ctx, GemmArgs a, int64_t batch) {
   return HIPNX_OK;
 }
 
-// the two-group 128 x 128 kernel: four LDS stages of 32 KiB, one work-group per CU
-template <int DT, bool LK, bool RK>
+// the two-group kernel on 128 x 128 tiles (four LDS stages of 32 KiB) or 64 x 64 tiles (eight of 16 KiB):
+// one work-group per CU
+template <int DT, bool LK, bool RK, int BM = 128, int BN = 128, int NSTAGE = 4, int SPP = 1>
 static int launch_pingpong128(const hipnx_ctx *ctx, GemmArgs a, int64_t batch) {
-  constexpr int smem = 4 * 256 * SLAB;
-  auto kern = gemm_pingpong128_kernel<DT, LK, RK>;
+  constexpr int smem = NSTAGE * SPP * (BM + BN) * SLAB;
+  auto kern = gemm_pingpong128_kernel<DT, LK, RK, BM, BN, NSTAGE, SPP>;
   static bool configured = false;
   if (!configured) {
     HIPNX_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
     configured = true;
   }
-  a.tiles_m = (int)((a.M + 127) / 128);
-  a.tiles_n = (int)((a.N + 127) / 128);
+  a.tiles_m = (int)((a.M + BM - 1) / BM);
+  a.tiles_n = (int)((a.N + BN - 1) / BN);
   a.group_m = gemm_group_m(a.tiles_m, a.tiles_n);
   dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)batch), block(512);
   hipLaunchKernelGGL(kern, grid, block, smem, ctx->stream, a);
@@ -120,6 +119,15 @@ static int launch_cfg(const hipnx_ctx *ctx, int cfg, const GemmArgs &a, int64_t 
       return launch_one<DT, 2, 2, 2, 2, LK, RK>(ctx, a, batch);
     }
     default:
+      // K-inner 2-byte and int8 operands: the two-group kernel on 64 x 64 tiles -- 64 rows of the weights per
+      // work-group, their slabs requested three phases (six slabs) ahead, two slabs per phase where K allows
+      // (int8 64 x 11008 x 4096: kernel 13.0 us; the 64 x 32 tiles below 18.7 us)
+      if constexpr (LK && RK && (DT == HIPNX_BF16 || DT == HIPNX_F16 || DT == HIPNX_S8)) {
+        if (a.Kb >= 8 * SLAB && a.ld_l < (1ll << 24) && a.ld_r < (1ll << 24)) {
+          if (a.Kb % (2 * SLAB) == 0) return launch_pingpong128<DT, LK, RK, 64, 64, 4, 2>(ctx, a, batch);
+          return launch_pingpong128<DT, LK, RK, 64, 64, 8, 1>(ctx, a, batch);
+        }
+      }
       // streaming a long weight matrix past a few rows is bound by the bytes in flight: six
       // stages (five slabs of 12 KiB requested ahead per work-group) when both operands are copied
       // straight into LDS

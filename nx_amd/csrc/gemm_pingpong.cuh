@@ -275,16 +275,24 @@ gemm_pingpong_kernel(GemmArgs a) {
 // two partial sums meet in LDS at the end, where each group takes over the finished half (32 rows of every
 // wave tile) it then scales, converts and stores.
 //
-// A slab (both operands) is 32 KiB, the four LDS stages hold slabs p .. p + 3.  Slab p + 3 lands in the stage
-// of slab p - 1, whose last reader waited for its fragments before the barrier that opened phase p.  The
-// waves that requested a slab wait for it at the end of their next memory phase (vmcnt(8): all but the slab
-// requested just now), two phases later, and the barrier behind that wait opens the phase that reads it.
-template <int DT, bool L_KIN, bool R_KIN>
+// A slab (both operands) is 32 KiB, the NSTAGE LDS stages hold slabs p .. p + NSTAGE - 1.  Slab p + NSTAGE - 1
+// lands in the stage of slab p - 1, whose last reader waited for its fragments before the barrier that opened
+// phase p.  The waves that requested a slab wait for it at the end of the memory phase before the one that
+// reads it (vmcnt: all but their (NSTAGE - 2) / 2 younger slabs), and the barrier behind that wait publishes it.
+//
+// BM_ = BN_ = 64 with eight stages is the shape for a few rows against a long K-inner weight matrix: 64 rows of
+// the weights per work-group (a slab of them is 8 KiB), seven slabs requested ahead -- 56 KiB in flight per CU,
+// which is what a stream from HBM at the part's rate needs -- while the rows' own slabs come from L2.
+template <int DT, bool L_KIN, bool R_KIN, int BM_ = 128, int BN_ = 128, int NSTAGE_ = 4, int SPP = 1>
 __global__ void __launch_bounds__(512)
 gemm_pingpong128_kernel(GemmArgs a) {
   typedef typename Mma16<DT>::acc_t acc_t;
-  constexpr int BM = 128, BN = 128, TM16 = 4, TN16 = 4, NSTAGE = 4, AHEAD = NSTAGE - 1;
-  constexpr int STAGE = (BM + BN) * SLAB;
+  constexpr int BM = BM_, BN = BN_, TM16 = BM / 32, TN16 = BN / 32, NSTAGE = NSTAGE_, AHEAD = NSTAGE - 1;
+  static_assert((BM == 128 || BM == 64) && (BN == 128 || BN == 64) && NSTAGE % 2 == 0 && NSTAGE >= 4, "tile extents of 64 or 128, an even number of stages");
+  static_assert((BM == 128 || L_KIN) && (BN == 128 || R_KIN), "a 64-row operand is K-inner (a k-row of a K-outer one must span all LDS banks)");
+  constexpr int LREQ = BM / 32, RREQ = BN / 32, REQ = SPP * (LREQ + RREQ);  // requests per wave and phase
+  // a stage holds the SPP slabs of one phase, each as [left rows | right rows]
+  constexpr int SLAB1 = (BM + BN) * SLAB, STAGE = SPP * SLAB1, KS = 2 * SPP;
   constexpr int ES = (DT == HIPNX_S8) ? 1 : 2;
   static_assert(DT == HIPNX_BF16 || DT == HIPNX_F16 || (DT == HIPNX_S8 && L_KIN && R_KIN), "2-byte MFMA types; int8 with K-inner operands");
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
@@ -298,7 +306,7 @@ gemm_pingpong128_kernel(GemmArgs a) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int grp = wave >> 2, w4 = wave & 3;  // waves w and w + 4 share a SIMD and a wave tile
-  const int wm = (w4 >> 1) * 64, wn = (w4 & 1) * 64;
+  const int wm = (w4 >> 1) * (BM / 2), wn = (w4 & 1) * (BN / 2);
 
   acc_t acc[TM16][TN16];
 #pragma unroll
@@ -308,20 +316,25 @@ gemm_pingpong128_kernel(GemmArgs a) {
 #pragma unroll
       for (int q = 0; q < 4; q++) acc[i][j][q] = 0;
 
-  // the four waves of the memory group request a whole slab: 4 + 4 instructions per wave
-  PPKInnerLoader<128, 4> lkin, rkin;
+  // the four waves of the memory group request a whole slab: LREQ + RREQ instructions per wave
+  PPKInnerLoader<BM, 4> lkin;
+  PPKInnerLoader<BN, 4> rkin;
   PPKOuterLoader<2, 128, 4> lkout, rkout;
   if constexpr (L_KIN) lkin.init(lb, a.ld_l, m0, a.M, w4, lane);
   else lkout.init(lb, a.ld_l, m0, a.M, w4, lane);
   if constexpr (R_KIN) rkin.init(rb, a.ld_r, n0, a.N, w4, lane);
   else rkout.init(rb, a.ld_r, n0, a.N, w4, lane);
+  // (below, "slab" stands for the SPP slabs of one phase)
   auto issue = [&](int slab) __attribute__((always_inline)) {
-    unsigned char *dst = smem + (slab % NSTAGE) * STAGE;
-    const int64_t kbyte0 = (int64_t)slab * SLAB;
-    if constexpr (L_KIN) lkin.issue(kbyte0, dst, w4);
-    else lkout.issue(kbyte0 / ES, a.ld_l, dst, w4);
-    if constexpr (R_KIN) rkin.issue(kbyte0, dst + BM * SLAB, w4);
-    else rkout.issue(kbyte0 / ES, a.ld_r, dst + BM * SLAB, w4);
+#pragma unroll
+    for (int u = 0; u < SPP; u++) {
+      unsigned char *dst = smem + (slab % NSTAGE) * STAGE + u * SLAB1;
+      const int64_t kbyte0 = ((int64_t)slab * SPP + u) * SLAB;
+      if constexpr (L_KIN) lkin.issue(kbyte0, dst, w4);
+      else lkout.issue(kbyte0 / ES, a.ld_l, dst, w4);
+      if constexpr (R_KIN) rkin.issue(kbyte0, dst + BM * SLAB, w4);
+      else rkout.issue(kbyte0 / ES, a.ld_r, dst + BM * SLAB, w4);
+    }
   };
 
   int a_rd[2], b_rd[2];
@@ -336,26 +349,28 @@ gemm_pingpong128_kernel(GemmArgs a) {
     for (int ks = 0; ks < 2; ks++) b_rd[ks] = BM * SLAB + row * SLAB + lds_slot16(row, 4 * ks + (lane >> 4)) * 16;
   }
 
-  const int nslab = (int)(a.Kb / SLAB);
-  v4i fa[2][TM16], fb[2][TN16];
+  const int nslab = (int)(a.Kb / (SPP * SLAB));  // the host sends whole phases only
+  v4i fa[KS][TM16], fb[KS][TN16];
   auto mem_phase = [&](int p) __attribute__((always_inline)) {
     const unsigned char *cur = smem + (p % NSTAGE) * STAGE;
 #pragma unroll
-    for (int ks = 0; ks < 2; ks++) {
+    for (int ks = 0; ks < KS; ks++) {
+      const unsigned char *sl = cur + (ks >> 1) * SLAB1;
 #pragma unroll
       for (int i = 0; i < TM16; i++) {
-        if constexpr (L_KIN) fa[ks][i] = *reinterpret_cast<const v4i *>(cur + a_rd[ks] + i * (16 * SLAB));
-        else fa[ks][i] = read_fragment_tr<2, BM>(cur, wm + 16 * i, ks, lane);
+        if constexpr (L_KIN) fa[ks][i] = *reinterpret_cast<const v4i *>(sl + a_rd[ks & 1] + i * (16 * SLAB));
+        else fa[ks][i] = read_fragment_tr<2, BM>(sl, wm + 16 * i, ks & 1, lane);
       }
 #pragma unroll
       for (int j = 0; j < TN16; j++) {
-        if constexpr (R_KIN) fb[ks][j] = *reinterpret_cast<const v4i *>(cur + b_rd[ks] + j * (16 * SLAB));
-        else fb[ks][j] = read_fragment_tr<2, BN>(cur + BM * SLAB, wn + 16 * j, ks, lane);
+        if constexpr (R_KIN) fb[ks][j] = *reinterpret_cast<const v4i *>(sl + b_rd[ks & 1] + j * (16 * SLAB));
+        else fb[ks][j] = read_fragment_tr<2, BN>(sl + BM * SLAB, wn + 16 * j, ks & 1, lane);
       }
     }
+    // this group's requests in flight, oldest first: slabs p + 1, p + 3, .. p + AHEAD; slab p + 1 is read next phase
     if (p + AHEAD < nslab) {
       issue(p + AHEAD);
-      wait_vmcnt<8>();
+      wait_vmcnt<(AHEAD - 1) / 2 * REQ>();
     } else {
       wait_vmcnt<0>();
     }
@@ -365,7 +380,7 @@ gemm_pingpong128_kernel(GemmArgs a) {
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_setprio(1);
 #pragma unroll
-    for (int ks = 0; ks < 2; ks++)
+    for (int ks = 0; ks < KS; ks++)
 #pragma unroll
       for (int j = 0; j < TN16; j++)
 #pragma unroll
@@ -374,18 +389,14 @@ gemm_pingpong128_kernel(GemmArgs a) {
     __builtin_amdgcn_sched_barrier(0);
   };
 
-  // prologue: group 0 requests slabs 0 and 2, group 1 slab 1; slab 0 is awaited here, slab 1 by group 1
-  // before the barrier that ends phase 0, slab 2 by group 0 at the end of its first memory phase
-  if (grp == 0) {
-    issue(0);
-    if (2 < nslab) {
-      issue(2);
-      wait_vmcnt<8>();
-    } else {
-      wait_vmcnt<0>();
-    }
-  } else if (1 < nslab) {
-    issue(1);
+  // prologue: slabs 0 .. AHEAD - 1, slab q by the group (q + 1) % 2 as in the walk (a group requests what the
+  // other one reads); group 1 holds slab 0 and waits for it here, slab 1 is awaited by group 0 in phase 0
+#pragma unroll
+  for (int q = 0; q < AHEAD; q++)
+    if (q < nslab && ((q + 1) & 1) == grp) issue(q);
+  if (grp == 1) {
+    if (nslab >= AHEAD) wait_vmcnt<(AHEAD - 1) / 2 * REQ>();
+    else wait_vmcnt<0>();
   }
   __builtin_amdgcn_s_barrier();
 
@@ -399,7 +410,6 @@ gemm_pingpong128_kernel(GemmArgs a) {
       __builtin_amdgcn_s_barrier();
     }
   } else {
-    wait_vmcnt<0>();
     for (int p = 0; p <= nslab; p += 2) {
       __builtin_amdgcn_s_barrier();
       if (p + 1 > nslab) break;
@@ -410,43 +420,45 @@ gemm_pingpong128_kernel(GemmArgs a) {
   }
 
   // the two partial sums: every wave hands the half of its tile the other group finishes to that group
-  // (2 x 4 accumulator tiles, 8 KiB per wave, 64 KiB in all) and adds what it is handed
+  // (TM16 / 2 x TN16 accumulator tiles of 1 KiB) and adds what it is handed
   {
-    unsigned char *mine = smem + wave * 8192, *theirs = smem + (wave ^ 4) * 8192;
+    constexpr int HM = TM16 / 2, XBYTES = HM * TN16 * 1024;
+    unsigned char *mine = smem + wave * XBYTES, *theirs = smem + (wave ^ 4) * XBYTES;
     // (a branch per group rather than a selection per tile: the accumulators must keep constant indices)
     if (grp == 0) {
 #pragma unroll
-      for (int i = 0; i < 2; i++)
+      for (int i = 0; i < HM; i++)
 #pragma unroll
-        for (int j = 0; j < TN16; j++) *reinterpret_cast<acc_t *>(mine + (i * TN16 + j) * 1024 + lane * 16) = acc[i + 2][j];
+        for (int j = 0; j < TN16; j++) *reinterpret_cast<acc_t *>(mine + (i * TN16 + j) * 1024 + lane * 16) = acc[i + HM][j];
     } else {
 #pragma unroll
-      for (int i = 0; i < 2; i++)
+      for (int i = 0; i < HM; i++)
 #pragma unroll
         for (int j = 0; j < TN16; j++) *reinterpret_cast<acc_t *>(mine + (i * TN16 + j) * 1024 + lane * 16) = acc[i][j];
     }
     __syncthreads();
-    acc_t fin[2][TN16];
+    acc_t fin[HM][TN16];
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < HM; i++)
 #pragma unroll
       for (int j = 0; j < TN16; j++) fin[i][j] = *reinterpret_cast<const acc_t *>(theirs + (i * TN16 + j) * 1024 + lane * 16);
     // the even slabs' sum first, as a single walk over K would have it
     if (grp == 0) {
 #pragma unroll
-      for (int i = 0; i < 2; i++)
+      for (int i = 0; i < HM; i++)
 #pragma unroll
         for (int j = 0; j < TN16; j++) fin[i][j] = acc[i][j] + fin[i][j];
     } else {
 #pragma unroll
-      for (int i = 0; i < 2; i++)
+      for (int i = 0; i < HM; i++)
 #pragma unroll
-        for (int j = 0; j < TN16; j++) fin[i][j] = fin[i][j] + acc[i + 2][j];
+        for (int j = 0; j < TN16; j++) fin[i][j] = fin[i][j] + acc[i + HM][j];
     }
     const int64_t obase = b * a.M * a.N;
-    unsigned char *turn = smem + 65536 + wave * 4096;  // past the exchanged halves, which the other group may still be reading
+    unsigned char *turn = smem + 8 * XBYTES + wave * 4096;  // past the exchanged halves, which the other group may still be reading
+    static_assert(8 * XBYTES + 8 * 4096 <= NSTAGE * STAGE, "the exchange and the epilogue's turn buffers fit the stages");
     switch (a.odt) {
-#define HIPNX_EPI(T) case T: gemm_epilogue<DT, T, 2, TN16>(fin, a.out, obase, a.M, a.N, m0 + wm + grp * 32, n0 + wn, lane, a.scale, a.scale_mode, turn); break;
+#define HIPNX_EPI(T) case T: gemm_epilogue<DT, T, HM, TN16>(fin, a.out, obase, a.M, a.N, m0 + wm + grp * (16 * HM), n0 + wn, lane, a.scale, a.scale_mode, turn); break;
       HIPNX_EPI(HIPNX_BF16) HIPNX_EPI(HIPNX_F16) HIPNX_EPI(HIPNX_F32) HIPNX_EPI(HIPNX_F64) HIPNX_EPI(HIPNX_BF16_RNE)
       HIPNX_EPI(HIPNX_S8) HIPNX_EPI(HIPNX_U8) HIPNX_EPI(HIPNX_S16) HIPNX_EPI(HIPNX_U16)
       HIPNX_EPI(HIPNX_S32) HIPNX_EPI(HIPNX_U32) HIPNX_EPI(HIPNX_S64) HIPNX_EPI(HIPNX_U64)

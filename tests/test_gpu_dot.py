@@ -182,6 +182,43 @@ def test_few_rows_against_long_matrix(M, ty, N, K, hip, oracle):
         check_float_dot(got, want, values(ox), values(ow), "mk,nk->mn", K, f"few rows {ty} {M}x{N}x{K}")
 
 
+@pytest.mark.parametrize("M", [1, 24, 64])
+@pytest.mark.parametrize("ty,N,K", [("bf16", 264, 2048), ("f16", 1024, 1056), ("s8", 400, 4096), ("bf16", 120, 640), ("bf16", 328, 192)])
+def test_few_rows_against_weights_stored_k_outer(M, ty, N, K, hip, oracle):
+    """x . W with W stored [K, N], the plain Nx.dot(x, w): a few rows of a 2-byte type take the 128-row kernels
+    (which read a K-outer operand by transposing loads, K split over work-groups when long), int8 and narrow
+    outputs the 64-row tiles; a contraction length that is an odd number of slabs takes one slab per phase."""
+    rng = np.random.default_rng(seed_of(M, ty, N, K, "k-outer weights"))
+    if ty == "s8":
+        x = rng.integers(-127, 128, size=(M, K)).astype(np.int8)
+        w = rng.integers(-127, 128, size=(K, N)).astype(np.int8)
+        hx, ox = both(x, ty, hip, oracle)
+        hw, ow = both(w, ty, hip, oracle)
+        assert_bits_equal(Nx.dot(hx, hw, out_type="s32"), Nx.dot(ox, ow, out_type="s32"), f"few rows s8 {M}x{N}x{K} NN")
+    else:
+        x, w = rand_raw(rng, ty, (M, K), lo=-1, hi=1), rand_raw(rng, ty, (K, N), lo=-1, hi=1)
+        hx, ox = both(x, ty, hip, oracle)
+        hw, ow = both(w, ty, hip, oracle)
+        check_float_dot(Nx.dot(hx, hw), Nx.dot(ox, ow), values(ox), values(ow), "mk,kn->mn", K, f"few rows {ty} {M}x{N}x{K} NN")
+
+
+@pytest.mark.parametrize("ty,M,N,K", [("bf16", 64, 1024, 1152), ("s8", 33, 520, 1152), ("f16", 7, 300, 4224), ("s8", 64, 11008, 4096)])
+def test_few_rows_one_and_two_slabs_per_phase(ty, M, N, K, hip, oracle):
+    """K-inner operands on 64 x 64 tiles of the two-group kernel: K of an odd number of slabs walks one slab per
+    phase through eight stages, an even number two per phase through four."""
+    rng = np.random.default_rng(seed_of(ty, M, N, K, "rows phases"))
+    if ty == "s8":
+        x = rng.integers(-127, 128, size=(M, K)).astype(np.int8)
+        w = rng.integers(-127, 128, size=(N, K)).astype(np.int8)
+        got = hip.to_numpy(Nx.dot(from_numpy(x, ty, hip), [1], from_numpy(w, ty, hip), [1], out_type="s32"))
+        assert np.array_equal(got, x.astype(np.int32) @ w.astype(np.int32).T)
+    else:
+        x, w = rand_raw(rng, ty, (M, K), lo=-1, hi=1), rand_raw(rng, ty, (N, K), lo=-1, hi=1)
+        hx, ox = both(x, ty, hip, oracle)
+        hw, ow = both(w, ty, hip, oracle)
+        check_float_dot(Nx.dot(hx, [1], hw, [1]), Nx.dot(ox, [1], ow, [1]), values(ox), values(ow), "mk,nk->mn", K, f"few rows {ty} {M}x{N}x{K}")
+
+
 def test_few_rows_against_long_matrix_batched(hip, oracle):
     rng = np.random.default_rng(7)
     x = rng.integers(-127, 128, size=(3, 20, 4096)).astype(np.int8)
