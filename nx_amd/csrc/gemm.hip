@@ -288,9 +288,10 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
   // the pipelined kernel transposes K-outer operands itself when the rows come in whole blocks
   const int row_block = esz == 1 ? 16 : (esz == 2 ? 8 : 4);
   // int8 on 128 x 128 tiles: a K-outer operand keeps the one-group kernel and its register-staged transposes
-  // (1024 x 2048 x 4096: 44 us against 18 us with both operands K-inner), so from 2^32 multiply-adds and K = 2048
-  // on the operand is laid out K-inner first, which costs 6-8 us
-  const bool s8_mid = l_dt == HIPNX_S8 && r_dt == HIPNX_S8 && pipelined && M > 64 && Kb >= 16 * SLAB &&
+  // (1024 x 2048 x 4096: 44 us against 18 us with both operands K-inner), so from 512 rows, 2^32 multiply-adds
+  // and K = 2048 on the operand is laid out K-inner first, which costs 6-12 us (with fewer rows the copy of the
+  // other operand costs more than it saves: 256 x 4096 x 4096 29 us with it)
+  const bool s8_mid = l_dt == HIPNX_S8 && r_dt == HIPNX_S8 && pipelined && M >= 512 && Kb >= 16 * SLAB &&
                       (double)M * (double)N * (double)K * (double)batch >= 4294967296.0 &&
                       !(((M + 255) / 256) * ((N + 255) / 256) * batch * 2 >= (int64_t)ctx->num_cus && M >= 192 && N >= 192);  // (those take 256 x 256 tiles)
   const bool l_relay = l_layout == HIPNX_K_OUTER && (!(pipelined && M % row_block == 0) || s8_mid);
@@ -345,9 +346,9 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
         int cfg;
         const bool big_ok = M >= 192 && N >= 192;
         const int64_t tw = ((M + 255) / 256) * ((N + 127) / 128) * batch;
-        // few rows: 64-row tiles, except for a 2-byte K-outer operand (x . W with W stored [K, N]), which only the
+        // few rows: 64-row tiles (f32: whatever its cost model below picks), except for a 2-byte K-outer operand (x . W with W stored [K, N]), which only the
         // 128-row kernels read by transposing loads (64 x 4096 x 4096 bf16: 72 us on 64 x 32 tiles, 19 us here)
-        if (M <= 64 && !(two_byte && !(l_kin && r_kin) && N >= 128)) cfg = GEMM_CFG_64x32;
+        if (M <= 64 && l_dt != HIPNX_F32 && !(two_byte && !(l_kin && r_kin) && N >= 128)) cfg = GEMM_CFG_64x32;
         else if (t256 * 4 >= (int64_t)ctx->num_cus * 3 && big_ok) cfg = GEMM_CFG_256;
         else if (two_byte && M >= 192 && N >= 128 && t128 * batch > ctx->num_cus)
           // More 128 x 128 tiles than CUs: half-width tiles of the two-group kernel while they fit the CUs in one
@@ -377,13 +378,26 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
             const int64_t cus = ctx->num_cus;
             auto rounds = [&](int64_t groups) { return (double)((groups + cus - 1) / cus); };
             double best = 10.0 + rounds(t128 * batch) * (double)nslab * 2.6;
+            // second launch, then the partial results written and read once (mostly from cache: ~8 MB per us)
+            auto split_cost = [&](int cand) { return 5.0 + 2.0 * (double)cand * (double)(M * N) * 4.0 / 8.0e6; };
             if (splittable)
               for (int cand = 2; cand <= 64; cand *= 2) {
                 if (t128 * cand > cus || nslab % cand != 0 || nslab / cand < 2) continue;
-                // second launch, then the partial results written and read once (mostly from cache: ~8 MB per us)
-                const double t = 15.0 + (double)(nslab / cand) * 2.6 + 2.0 * (double)cand * (double)(M * N) * 4.0 / 8.0e6;
+                const double t = 10.0 + (double)(nslab / cand) * 2.6 + split_cost(cand);
                 if (t < best) { best = t; splits = cand; }
               }
+            // up to 64 rows: tiles of 64 x 128, half the MFMA work per slab of a tile that would be half empty
+            if (M <= 64) {
+              const int64_t tn = (N + 127) / 128 * batch;
+              const double whole = 10.0 + rounds(tn) * (double)nslab * 1.3;
+              if (whole < best) { best = whole; cfg = GEMM_CFG_64x128; splits = 1; }
+              if (splittable)
+                for (int cand = 2; cand <= 64; cand *= 2) {
+                  if (tn * cand > cus || nslab % cand != 0 || nslab / cand < 2) continue;
+                  const double t = 10.0 + (double)(nslab / cand) * 1.3 + split_cost(cand);
+                  if (t < best) { best = t; cfg = GEMM_CFG_64x128; splits = cand; }
+                }
+            }
             const int64_t t64 = ((M + 63) / 64) * ((N + 31) / 32) * batch;
             if (10.0 + rounds(t64) * (double)nslab * 0.55 < best) { cfg = GEMM_CFG_64x32; splits = 1; }
           }
