@@ -398,7 +398,36 @@ class HipNxBackend:
     def _reduce(cls, op: int, out: Tensor, t: Tensor, opts) -> Tensor:
         dev = cls._device_of(t)
         t = cls._from_nx(t, dev)
-        view, outer, red, inner = cls._view_for_axes(t, opts.get("axes"))
+        axes = opts.get("axes")
+        if axes is not None and t.type[1] >= 8:
+            axes = sorted(a % len(t.shape) for a in axes)
+            runs = [[a] for a in axes[:1]]
+            for a in axes[1:]:
+                if a == runs[-1][-1] + 1:
+                    runs[-1].append(a)
+                else:
+                    runs.append([a])
+            if len(runs) > 1:
+                # Reduced axes that are not neighbours: one pass per run of neighbouring axes, innermost run
+                # first, instead of a transposed copy of the whole tensor.  Sums and products pass through
+                # f64 / 64-bit integers (the accumulators' own types), so the result is still rounded or
+                # wrapped once; among equal extremes the first in row-major order of the reduced axes still wins.
+                if op in (RED_SUM, RED_PRODUCT):
+                    mid = ("f", 64) if T.is_float(out.type) else (out.type[0] if out.type[0] in ("s", "u") else "s", 64)
+                else:
+                    mid = out.type
+                cur, shape = t, list(t.shape)
+                for i, run in enumerate(reversed(runs)):
+                    last = i == len(runs) - 1
+                    outer, red, inner = prod(shape[:run[0]]), prod(shape[run[0]:run[-1] + 1]), prod(shape[run[-1] + 1:])
+                    shape = shape[:run[0]] + shape[run[-1] + 1:]
+                    step = out if last else out.with_(data=None, type=mid, shape=tuple(shape))
+                    res = cls._alloc(step, dev)
+                    L.check(L.lib.hipnx_reduce(res.data.ref.ctx, op, T.code(cur.type), T.code(step.type), outer, red, inner,
+                                               cls._handle(cur), res.data.ref.handle))
+                    cur = res
+                return cur
+        view, outer, red, inner = cls._view_for_axes(t, axes)
         res = cls._alloc(out, dev)
         L.check(L.lib.hipnx_reduce(res.data.ref.ctx, op, T.code(t.type), T.code(out.type), outer, red, inner,
                                    cls._handle(view), res.data.ref.handle))

@@ -43,6 +43,17 @@ __device__ __forceinline__ uint32_t fastdiv(uint32_t n, FastDiv32 f) { return (_
 
 enum { ROWS_ONE = 0, ROWS_FAST = 1, ROWS_WIDE = 2 };  // how a vector index splits into (row, column)
 
+// Rows that are themselves two or three collapsed axes with their own strides per operand (a mask [b, 1, 1, s]
+// against scores [b, h, s, s] collapses to [b, h * s | s]: the mask's row offset is b's index times s, not a
+// multiple of the row number).  n = 0 or 1: a row's offset is row * stride, as without this; else the row
+// number is taken apart from the innermost of its axes outwards (d[k] = extent, fd[k] its reciprocal, k >= 1).
+struct RowAxes {
+  int n;
+  uint32_t d[3];
+  FastDiv32 fd[3];
+  int64_t ls[3], rs[3];
+};
+
 // FIX >= 0: both operands and the result have this element type, known when the kernel is compiled -- the
 // three run-time type switches (and the scalar bookkeeping the compiler builds around them, ~200 scalar
 // instructions per wave) fold away.  bf16 add on 16384^2: 388 -> 263 us (4.1 -> 6.1 TB/s), negate and exp 280 -> 175 us.
@@ -51,7 +62,7 @@ template <int OP, typename CT, bool UNS, int FIX = -1, int FIXO = FIX>
 __global__ void __launch_bounds__(BLOCK)
 binary_vec_kernel(const void *__restrict__ l, const void *__restrict__ r, void *__restrict__ out, int ldt_, int rdt_,
                   int odt_, int64_t cols, int64_t vecs_per_row, int64_t nvec, int64_t ls0, int ls1, int64_t rs0,
-                  int rs1, unsigned long long *__restrict__ err, int rows_mode, FastDiv32 fd) {
+                  int rs1, unsigned long long *__restrict__ err, int rows_mode, FastDiv32 fd, RowAxes ax) {
   constexpr bool RAISES = binary_can_raise(OP, is_fp<CT>::value);
   constexpr int E = vec_elems(FIX, FIXO);  // (vecs_per_row and nvec are counted in these by the launcher)
   const int ldt = FIX >= 0 ? FIX : ldt_, rdt = FIX >= 0 ? FIX : rdt_, odt = FIX >= 0 ? FIXO : odt_;
@@ -68,7 +79,24 @@ binary_vec_kernel(const void *__restrict__ l, const void *__restrict__ r, void *
       row = v / vecs_per_row;
       col = (v - row * vecs_per_row) * E;
     }
-    int64_t lo = row * ls0 + col * ls1, ro = row * rs0 + col * rs1, oo = row * cols + col;
+    int64_t lo, ro;
+    const int64_t oo = row * cols + col;
+    if (ax.n <= 1) {
+      lo = row * ls0 + col * ls1;
+      ro = row * rs0 + col * rs1;
+    } else {
+      uint32_t rem = (uint32_t)row;  // (the launcher takes this form only with fewer than 2^31 rows)
+      lo = col * ls1;
+      ro = col * rs1;
+      for (int k = ax.n - 1; k >= 1; k--) {
+        const uint32_t q = fastdiv(rem, ax.fd[k]), i = rem - q * ax.d[k];
+        lo += (int64_t)i * ax.ls[k];
+        ro += (int64_t)i * ax.rs[k];
+        rem = q;
+      }
+      lo += (int64_t)rem * ax.ls[0];
+      ro += (int64_t)rem * ax.rs[0];
+    }
     CT a[E], b[E], c[E];
     if (col + E <= cols) {
       if (ls1) load_vec<CT, E>(l, ldt, lo, a);
@@ -233,6 +261,7 @@ struct BinArgs {
   int64_t cols, vecs_per_row, nvec, ls0, rs0;
   int ls1, rs1;
   unsigned long long *err;  // the context's deferred error word (device address of the pinned host word)
+  RowAxes ax;
 };
 
 template <int OP, typename CT, bool UNS, int FIX, int FIXO = FIX>
@@ -248,7 +277,7 @@ static void launch_bvec_fix(const hipnx_ctx *ctx, const BinArgs &a_) {
   const FastDiv32 fd = mode == ROWS_FAST ? make_fastdiv((uint32_t)a.vecs_per_row) : FastDiv32{0, 0};
   hipLaunchKernelGGL((binary_vec_kernel<OP, CT, UNS, FIX, FIXO>), dim3(grid_for(ctx, a.nvec)), dim3(BLOCK), 0, ctx->stream, a.l,
                      a.r, a.out, a.ldt, a.rdt, a.odt, a.cols, a.vecs_per_row, a.nvec, a.ls0, a.ls1, a.rs0, a.rs1, a.err,
-                     mode, fd);
+                     mode, fd, a.ax);
 }
 
 // the kernel compiled for one element type throughout, where there is one: the types of most tensor arithmetic
@@ -371,6 +400,33 @@ extern "C" int hipnx_binary(hipnx_ctx *ctx, int op, int l_dt, int r_dt, int out_
 
   bool vec_ok = false;
   BinArgs a{};
+  if (m == 3 || m == 4) {
+    // two or three outer axes and a dense (or broadcast) inner one: the vector kernel with the row number taken apart
+    const int64_t cols = dims[m - 1], l1 = ls[m - 1], r1 = rs[m - 1];
+    int64_t rows = 1;
+    bool aligned = cols % E == 0;
+    for (int q = 0; q < m - 1; q++) {
+      rows *= dims[q];
+      aligned = aligned && (l1 == 0 || ls[q] % E == 0) && (r1 == 0 || rs[q] % E == 0);
+    }
+    if ((l1 == 0 || l1 == 1) && (r1 == 0 || r1 == 1) && aligned && rows * ((cols + 3) / 4) < (1ll << 31)) {
+      vec_ok = true;
+      a.l = l->ptr; a.r = r->ptr; a.out = out->ptr;
+      a.ldt = l_dt; a.rdt = r_dt; a.odt = out_dt;
+      a.cols = cols;
+      a.vecs_per_row = (cols + E - 1) / E;
+      a.nvec = rows * a.vecs_per_row;
+      a.ls0 = 0; a.rs0 = 0; a.ls1 = (int)l1; a.rs1 = (int)r1;
+      a.err = deferred_error_word(ctx);
+      a.ax.n = m - 1;
+      for (int q = 0; q < m - 1; q++) {
+        a.ax.d[q] = (uint32_t)dims[q];
+        a.ax.fd[q] = make_fastdiv((uint32_t)dims[q]);
+        a.ax.ls[q] = ls[q];
+        a.ax.rs[q] = rs[q];
+      }
+    }
+  }
   if (m <= 2) {
     int64_t rows = m == 2 ? dims[0] : 1, cols = dims[m - 1];
     int64_t l0 = m == 2 ? ls[0] : 0, r0 = m == 2 ? rs[0] : 0, l1 = ls[m - 1], r1 = rs[m - 1];

@@ -271,9 +271,63 @@ defmodule HipNx.Backend do
 
   defp reduce_op(code, out, %T{} = t, opts) do
     device = device_of([t])
-    {view, outer, red, inner} = view_for_axes(t, opts[:axes], device)
-    {ref, _} = from_nx(view, device)
-    to_nx(unwrap!(NIF.reduce(ctx(device), code, dt(t.type), dt(out.type), outer, red, inner, ref, bytes(out))), device, out)
+
+    # (sub-byte integers keep the single pass: their intermediates would have to be packed and unpacked)
+    case if(elem(t.type, 1) >= 8, do: axis_runs(opts[:axes]), else: []) do
+      [_, _ | _] = runs ->
+        # reduced axes that are not neighbours: one pass per run of neighbouring axes, innermost run first,
+        # instead of a transposed copy; sums and products pass through f64 / 64-bit integers (the
+        # accumulators' own types), so the result is still rounded or wrapped once
+        mid =
+          cond do
+            code not in [0, 3] -> out.type
+            Nx.Type.float?(out.type) -> {:f, 64}
+            true -> {elem(out.type, 0), 64}
+          end
+
+        last_run = hd(runs)
+
+        runs
+        |> Enum.reverse()
+        |> Enum.reduce(t, fn run, cur ->
+          dims = Tuple.to_list(cur.shape)
+          first = hd(run)
+          last = List.last(run)
+          shape = List.to_tuple(Enum.take(dims, first) ++ Enum.drop(dims, last + 1))
+          step = if run == last_run, do: out, else: %{out | type: mid, shape: shape, names: List.duplicate(nil, tuple_size(shape))}
+          {ref, _} = from_nx(cur, device)
+          outer = prod(Enum.take(dims, first))
+          red = prod(Enum.slice(dims, first..last))
+          inner = prod(Enum.drop(dims, last + 1))
+          to_nx(unwrap!(NIF.reduce(ctx(device), code, dt(cur.type), dt(step.type), outer, red, inner, ref, bytes(step))), device, step)
+        end)
+
+      _ ->
+        {view, outer, red, inner} = view_for_axes(t, opts[:axes], device)
+        {ref, _} = from_nx(view, device)
+        to_nx(unwrap!(NIF.reduce(ctx(device), code, dt(t.type), dt(out.type), outer, red, inner, ref, bytes(out))), device, out)
+    end
+  end
+
+  # the sorted axes as runs of neighbours: [1, 3, 4] -> [[1], [3, 4]]
+  defp axis_runs(nil), do: []
+
+  defp axis_runs(axes) do
+    axes
+    |> Enum.sort()
+    |> Enum.chunk_while(
+      [],
+      fn a, acc ->
+        case acc do
+          [prev | _] when a != prev + 1 -> {:cont, Enum.reverse(acc), [a]}
+          _ -> {:cont, [a | acc]}
+        end
+      end,
+      fn
+        [] -> {:cont, []}
+        acc -> {:cont, Enum.reverse(acc), []}
+      end
+    )
   end
 
   @impl true

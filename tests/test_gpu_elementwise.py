@@ -229,3 +229,24 @@ def test_nan_is_written_canonically(hip, oracle):
         assert_bits_equal(getattr(Nx, op)(hx), getattr(Nx, op)(ox), op)
     assert_bits_equal(Nx.add(hx, 1.0), Nx.add(ox, 1.0), "add")
     assert_bits_equal(Nx.as_type(hx, "bf16"), Nx.as_type(ox, "bf16"), "as_type bf16")
+
+
+DEEP = [((2, 3, 8, 16), (2, 1, 1, 16)), ((2, 3, 8, 16), (2, 1, 8, 1)), ((2, 3, 8, 16), (3, 1, 1)), ((2, 3, 8, 16), (1, 3, 1, 16)),
+        ((4, 5, 24), (4, 1, 24)), ((4, 5, 24), (1, 5, 1)), ((3, 2, 4, 2, 16), (3, 1, 4, 1, 16)), ((2, 3, 8, 12), (2, 1, 1, 12)),
+        ((6, 1, 7, 40), (1, 5, 1, 40)), ((2, 3, 5, 64), (2, 3, 1, 1))]
+
+
+@pytest.mark.parametrize("ls,rs", DEEP, ids=[f"{a}-{b}" for a, b in DEEP])
+@pytest.mark.parametrize("ty", ["f32", "bf16", "s32", "u8", "f64"])
+@pytest.mark.parametrize("op", ["add", "multiply", "less", "max"])
+def test_broadcasts_over_separated_axes(ls, rs, ty, op, hip, oracle):
+    """A mask [b, 1, 1, s] against scores [b, h, s, s], a per-head scale [h, 1, 1], a per-row term [b, 1, s, 1]: the
+    index space collapses to three or four axes, not to [rows, columns]; the vector kernel takes the row number
+    apart.  Both operand orders; shapes off the 8-element grid and rank 5 take the general kernel.  Bit for bit."""
+    rng = np.random.default_rng(seed_of(ls, rs, ty, op, "deep"))
+    a, b = rand_raw(rng, ty, ls, lo=-5, hi=5), rand_raw(rng, ty, rs, lo=-5, hi=5)
+    ha, oa = both(a, ty, hip, oracle)
+    hb, ob = both(b, ty, hip, oracle)
+    f = getattr(Nx, op)
+    assert_bits_equal(f(ha, hb), f(oa, ob), f"{op} {ty} {ls} {rs}")
+    assert_bits_equal(f(hb, ha), f(ob, oa), f"{op} {ty} {rs} {ls}")

@@ -145,3 +145,39 @@ def test_short_rows_take_part_of_a_wave(ty, red, op, hip, oracle):
             bound = red * 2.0 ** -24 * np.abs(x64).sum(axis=1) + eps * np.abs(x64.sum(axis=1)) + 1e-30
             err = np.abs(values(got) - values(want))
             assert (err <= bound).all(), f"sum {ty} {red}: max err {err.max():.3e}"
+
+
+@pytest.mark.parametrize("shape,axes", [((4, 6, 5, 8), [1, 3]), ((4, 6, 5, 8), [0, 2]), ((3, 4, 5, 6, 7), [0, 2, 4]), ((3, 4, 5, 6, 7), [0, 1, 3]),
+                                        ((2, 33, 3, 130), [0, 3]), ((5, 7, 9), [0, 2])])
+@pytest.mark.parametrize("ty", ["f32", "bf16", "s32", "u8", "s64", "f64"])
+@pytest.mark.parametrize("op", ["sum", "product", "reduce_max", "reduce_min", "all", "any"])
+def test_reduced_axes_that_are_not_neighbours(shape, axes, ty, op, hip, oracle):
+    """Reduced axes with kept axes between them go one run of neighbouring axes at a time (innermost first, sums
+    through f64 / 64-bit integers) instead of through a transposed copy: integers and selections bit for bit --
+    signed zeros and NaN included: the first extreme in row-major order of the reduced axes wins -- float sums
+    and products within the accumulation bound."""
+    rng = np.random.default_rng(seed_of(shape, axes, ty, op, "runs"))
+    if op == "product":
+        x = rand_raw(rng, ty, shape, lo=0.9, hi=1.1) if ty in ("f32", "bf16", "f64") else rng.integers(1, 3, size=shape).astype(T.numpy_dtype(T.normalize(ty)))
+    elif op in ("all", "any"):
+        x = (rng.random(shape) < (0.97 if op == "all" else 0.03)).astype(np.float64)
+        x = (x.astype(np.float32).view(np.uint32) >> 16).astype(np.uint16) if ty == "bf16" else x.astype(T.numpy_dtype(T.normalize(ty)))
+    else:
+        x = rand_raw(rng, ty, shape, lo=-3, hi=3)
+        if ty == "f32":
+            flat = x.reshape(-1)
+            flat[rng.integers(0, flat.size, 6)] = 0.0
+            flat[rng.integers(0, flat.size, 6)] = -0.0
+            if op != "sum":
+                flat[rng.integers(0, flat.size, 2)] = np.nan
+    hx, ox = both(x, ty, hip, oracle)
+    for keep in (False, True):
+        got, want = getattr(Nx, op)(hx, axes=axes, keep_axes=keep), getattr(Nx, op)(ox, axes=axes, keep_axes=keep)
+        if op in ("sum", "product") and T.is_float(T.normalize(ty)):
+            assert got.type == want.type and got.shape == want.shape
+            g, w = values(got), values(want)
+            k = int(np.prod([shape[a] for a in axes]))
+            eps = {"f64": 2.0 ** -52, "f32": 2.0 ** -23, "bf16": 2.0 ** -7}[ty]
+            assert np.allclose(g, w, rtol=eps + k * 2.0 ** -50, atol=(k * 2.0 ** -24 * np.abs(values(ox)).sum(axis=tuple(axes), keepdims=keep)) if op == "sum" else 0), f"{op} {ty} {shape} {axes}"
+        else:
+            assert_bits_equal(got, want, f"{op} {ty} {shape} {axes} keep={keep}")
