@@ -88,12 +88,13 @@ select_vec_kernel(const void *__restrict__ p, const void *__restrict__ t, const 
 #pragma unroll
         for (int e = 0; e < E; e++) pt[e] = pi[e] != 0;
       }
+      // (an operand that is one element for all -- a number -- keeps its own type also in the typed form)
       if (tstep) load_vec<CT, E>(t, tdt, i0, a);
-      else { const CT x = load_one<CT>(t, tdt, 0);
+      else { const CT x = load_one<CT>(t, tdt_, 0);
 #pragma unroll
         for (int e = 0; e < E; e++) a[e] = x; }
       if (fstep) load_vec<CT, E>(f, fdt, i0, b);
-      else { const CT x = load_one<CT>(f, fdt, 0);
+      else { const CT x = load_one<CT>(f, fdt_, 0);
 #pragma unroll
         for (int e = 0; e < E; e++) b[e] = x; }
 #pragma unroll
@@ -101,7 +102,7 @@ select_vec_kernel(const void *__restrict__ p, const void *__restrict__ t, const 
       store_vec<CT, E>(out, odt, i0, c);
     } else {
       for (int64_t i = i0; i < n; i++) {
-        const CT x = truthy<CT>(p, pdt, i * pstep) ? load_one<CT>(t, tdt, i * tstep) : load_one<CT>(f, fdt, i * fstep);
+        const CT x = truthy<CT>(p, pdt, i * pstep) ? load_one<CT>(t, tstep ? tdt : tdt_, i * tstep) : load_one<CT>(f, fstep ? fdt : fdt_, i * fstep);
         store_one<CT>(out, odt, i, x);
       }
     }
@@ -336,7 +337,14 @@ extern "C" int hipnx_select(hipnx_ctx *ctx, int pred_dt, int true_dt, int false_
     dim3 grid(grid_for((n + E - 1) / E)), block(BLOCK);
 #define HIPNX_SELECT(CT, FIX) hipLaunchKernelGGL((select_vec_kernel<CT, FIX>), grid, block, 0, ctx->stream, pred->ptr, on_true->ptr, on_false->ptr, out->ptr, \
                                                pred_dt, true_dt, false_dt, out_dt, n, (int)s.ps[0], (int)s.ts[0], (int)s.fs[0])
-    const bool one_type = pred_dt == HIPNX_U8 && true_dt == out_dt && false_dt == out_dt;
+    // one element type throughout, where a lone element (a number) may have another one that the kernel's
+    // arithmetic type holds exactly: select(mask, scores_bf16, -1.0e9) arrives with an f32 number
+    auto fits = [&](int dt, int64_t step) {
+      if (dt == out_dt) return true;
+      if (step != 0) return false;
+      return is_float(out_dt) ? narrow_float(dt) && narrow_float(out_dt) : !is_float(dt);
+    };
+    const bool one_type = pred_dt == HIPNX_U8 && fits(true_dt, s.ts[0]) && fits(false_dt, s.fs[0]) && (s.ts[0] != 0 || s.fs[0] != 0 || true_dt == false_dt);
     if (one_type && out_dt == HIPNX_F32) HIPNX_SELECT(float, HIPNX_F32);
     else if (one_type && out_dt == HIPNX_BF16) HIPNX_SELECT(float, HIPNX_BF16);
     else if (one_type && out_dt == HIPNX_F16) HIPNX_SELECT(float, HIPNX_F16);

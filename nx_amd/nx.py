@@ -602,8 +602,10 @@ def clip(t, min, max):  # noqa: A002 - Nx.clip/3 (nx.ex:13973-14000)
 def pad(t, pad_value, padding_config):
     """Nx.pad/3 (nx.ex:4233-4250; shape rule shape.ex:1038-1071): (low, high, interior) per axis;
     negative edges crop, interior padding must be non-negative."""
-    t, pad_value = to_tensor(t), to_tensor(pad_value)
-    out_type = T.binary_type(t.type, pad_value.type)
+    t = to_tensor(t)
+    # the type is merged before the number becomes a tensor (nx.ex:4237-4238): a bf16 tensor padded with 0.0 stays bf16
+    out_type = T.binary_type(t.type, pad_value if isinstance(pad_value, (int, float)) and not isinstance(pad_value, bool) else to_tensor(pad_value).type)
+    pad_value = to_tensor(pad_value)
     if pad_value.shape != ():
         raise ValueError("padding value must be a scalar and non-vectorized")
     padding_config = [tuple(c) for c in padding_config]

@@ -140,3 +140,13 @@ def test_to_batched_known_answers_on_the_host_backend_and_the_oracle(oracle):
     for backend in (HostBinary, oracle):
         check_known_answers(backend)
         check_counts(backend)
+
+
+def test_pad_merges_its_type_before_the_number_becomes_a_tensor(oracle):
+    """nx.ex:4237-4238: binary_type(tensor, pad_value) sees the number, so a bf16 tensor padded with 0.0 stays
+    bf16 and an s32 tensor padded with 0 stays s32."""
+    Nx.default_backend(oracle)
+    bf = Nx.as_type(Nx.tensor([1.0, 2.0]), "bf16")
+    assert Nx.pad(bf, 0.0, [(1, 1, 0)]).type == ("bf", 16)
+    assert Nx.pad(Nx.tensor([1, 2]), 0, [(1, 1, 0)]).type == ("s", 32)
+    assert Nx.to_flat_list(Nx.pad(bf, 0.0, [(1, 2, 0)])) == [0.0, 1.0, 2.0, 0.0, 0.0]
