@@ -107,9 +107,9 @@ static int launch_cfg(const hipnx_ctx *ctx, int cfg, const GemmArgs &a, int64_t 
       // slab against the 1600-2100 below.  It holds a CU's LDS alone, so for the 2-byte types only where no
       // second work-group would share the CU; int8 has no wider two-group tile to fall back on and takes it
       // for every grid (2048 x 4096 x 4096, 512 tiles: 52 -> 42 us).
-      if constexpr (DT == HIPNX_BF16 || DT == HIPNX_F16 || (DT == HIPNX_S8 && LK && RK)) {
+      if constexpr (DT == HIPNX_BF16 || DT == HIPNX_F16 || ((DT == HIPNX_S8 || DT == HIPNX_F32) && LK && RK)) {
         const int64_t groups = ((a.M + 127) / 128) * ((a.N + 127) / 128) * batch;
-        if (a.Kb >= 8 * SLAB && a.ld_l < (1ll << 23) && a.ld_r < (1ll << 23) && (DT == HIPNX_S8 || groups <= ctx->num_cus))
+        if (a.Kb >= 8 * SLAB && a.ld_l < (1ll << 23) && a.ld_r < (1ll << 23) && (DT == HIPNX_S8 || DT == HIPNX_F32 || groups <= ctx->num_cus))
           return launch_pingpong128<DT, LK, RK>(ctx, a, batch);
       }
       if constexpr ((LK || tr) && (RK || tr)) {

@@ -294,7 +294,8 @@ gemm_pingpong128_kernel(GemmArgs a) {
   // a stage holds the SPP slabs of one phase, each as [left rows | right rows]
   constexpr int SLAB1 = (BM + BN) * SLAB, STAGE = SPP * SLAB1, KS = 2 * SPP;
   constexpr int ES = (DT == HIPNX_S8) ? 1 : 2;
-  static_assert(DT == HIPNX_BF16 || DT == HIPNX_F16 || (DT == HIPNX_S8 && L_KIN && R_KIN), "2-byte MFMA types; int8 with K-inner operands");
+  static_assert(DT == HIPNX_BF16 || DT == HIPNX_F16 || ((DT == HIPNX_S8 || DT == HIPNX_F32) && L_KIN && R_KIN),
+                "2-byte MFMA types; int8 and f32 with K-inner operands");
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
   int tm, tn;
