@@ -152,6 +152,13 @@ def i64_array(values):
     return _i64_array_cached(tuple(values))
 
 
+@functools.lru_cache(maxsize=4096)
+def broadcast_stride_array(shape: tuple, out_shape: tuple):
+    """The element strides of `shape` viewed in `out_shape` (0 on broadcast axes) as a C array."""
+    from . import shape as S
+    return _i64_array_cached(S._broadcast_strides(shape, out_shape))
+
+
 def int_array(values):
     values = list(values)
     return (C.c_int * max(len(values), 1))(*values)

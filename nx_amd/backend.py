@@ -57,6 +57,9 @@ class _Context:
 
     @classmethod
     def get(cls, device: int):
+        ctx = cls._by_device.get(device)  # (a dict read is atomic; the lock is for the first use only)
+        if ctx is not None:
+            return ctx
         with cls._lock:
             ctx = cls._by_device.get(device)
             if ctx is None:
@@ -330,11 +333,13 @@ class HipNxBackend:
         dev = cls._device_of(l, r)
         l, r = cls._from_nx(l, dev), cls._from_nx(r, dev)
         res = cls._alloc(out, dev)
-        rank = len(out.shape)
-        L.check(L.lib.hipnx_binary(
-            res.data.ref.ctx, op, T.code(l.type), T.code(r.type), T.code(out.type), rank, L.i64_array(out.shape),
-            L.i64_array(S.broadcast_strides(l.shape, out.shape)), L.i64_array(S.broadcast_strides(r.shape, out.shape)),
-            cls._handle(l), cls._handle(r), res.data.ref.handle))
+        shape = out.shape
+        status = L.lib.hipnx_binary(
+            res.data.ref.ctx, op, T.code(l.type), T.code(r.type), T.code(out.type), len(shape), L.i64_array(shape),
+            L.broadcast_stride_array(l.shape, shape), L.broadcast_stride_array(r.shape, shape),
+            cls._handle(l), cls._handle(r), res.data.ref.handle)
+        if status:
+            L.check(status)
         return cls._narrow(res) if out.type[1] < 8 else res
 
     @classmethod
@@ -503,17 +508,39 @@ class HipNxBackend:
         operand needs no copy whenever its contracted axes are adjacent."""
         dev = cls._device_of(l, r)
         l, r = cls._from_nx(l, dev), cls._from_nx(r, dev)
-        pairs = sorted(zip(c1, c2))
-        c1s, c2s = [p[0] for p in pairs], [p[1] for p in pairs]
-        nb = len(b1)
-        K = prod(l.shape[a] for a in c1s)
-        batch = prod(l.shape[a] for a in b1)
-        lt, l_layout, M = cls._dot_operand(l, c1s, nb)
-        rt, r_layout, N = cls._dot_operand(r, c2s, nb)
+        # operands that already sit as [batch, rows, K] or [batch, K, rows] need no copy: that, and the
+        # extents, follow from the shapes and axes alone and are worked out once per signature
+        key = (l.shape, tuple(c1), len(b1), r.shape, tuple(c2))
+        plan = cls._dot_plans.get(key)
+        if plan is None:
+            pairs = sorted(zip(c1, c2))
+            c1s, c2s = [p[0] for p in pairs], [p[1] for p in pairs]
+            nb = len(b1)
+            direct = []
+            for t, cs in ((l, c1s), (r, c2s)):
+                rank = len(t.shape)
+                kept = [a for a in range(nb, rank) if a not in cs]
+                head = list(range(nb))
+                layout = K_INNER if head + kept + cs == list(range(rank)) else K_OUTER if head + cs + kept == list(range(rank)) else None
+                direct.append((layout, prod(t.shape[a] for a in kept)))
+            plan = (c1s, c2s, nb, prod(l.shape[a] for a in c1s), prod(l.shape[a] for a in b1), direct)
+            if len(cls._dot_plans) >= 4096:
+                cls._dot_plans.clear()
+            cls._dot_plans[key] = plan
+        c1s, c2s, nb, K, batch, ((l_layout, M), (r_layout, N)) = plan
+        lt, rt = l, r
+        if l_layout is None:
+            lt, l_layout, M = cls._dot_operand(l, c1s, nb)
+        if r_layout is None:
+            rt, r_layout, N = cls._dot_operand(r, c2s, nb)
         res = cls._alloc(out, dev)
-        L.check(L.lib.hipnx_dot(res.data.ref.ctx, T.code(l.type), T.code(r.type), _out_code(out.type), batch, M, N, K,
-                                l_layout, r_layout, cls._handle(lt), cls._handle(rt), res.data.ref.handle))
+        status = L.lib.hipnx_dot(res.data.ref.ctx, T.code(l.type), T.code(r.type), _out_code(out.type), batch, M, N, K,
+                                 l_layout, r_layout, cls._handle(lt), cls._handle(rt), res.data.ref.handle)
+        if status:
+            L.check(status)
         return cls._narrow(res) if out.type[1] < 8 else res
+
+    _dot_plans = {}
 
     # ---- data movement ---------------------------------------------------------------------
     @classmethod

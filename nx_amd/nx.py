@@ -202,9 +202,13 @@ def _number_or_type(x):
 
 
 def _binary(name, left, right, out_type_fun):
-    ty = T.binary_type(_number_or_type(left), _number_or_type(right))
-    l, r = to_tensor(left), to_tensor(right)
-    out = template(out_type_fun(ty), S.binary_broadcast(l.shape, r.shape))
+    if left.__class__ is Tensor and right.__class__ is Tensor:  # the common case: no number to look at
+        ty = left.type if left.type == right.type else T.merge(left.type, right.type)
+        l, r = left, right
+    else:
+        ty = T.binary_type(_number_or_type(left), _number_or_type(right))
+        l, r = to_tensor(left), to_tensor(right)
+    out = template(out_type_fun(ty), l.shape if l.shape == r.shape else S.binary_broadcast(l.shape, r.shape))
     return getattr(_impl(l, r), name)(out, l, r)
 
 
@@ -365,10 +369,21 @@ def dot(t1, *args, out_type=None):
     c1, b1, t2, c2, b2 = args
     t1, t2 = to_tensor(t1), to_tensor(t2)
     ty = T.normalize(out_type) if out_type is not None else T.binary_type(t1.type, t2.type)
-    c1, c2 = S.normalize_axes(t1.shape, c1), S.normalize_axes(t2.shape, c2)
-    b1, b2 = S.normalize_axes(t1.shape, b1), S.normalize_axes(t2.shape, b2)
-    out = template(ty, S.dot(t1.shape, c1, b1, t2.shape, c2, b2))
-    return _impl(t1, t2).dot(out, t1, c1, b1, t2, c2, b2)
+    # the axes and the output shape depend on the shapes and the axes given only: worked out once per signature
+    key = (t1.shape, tuple(c1), tuple(b1), t2.shape, tuple(c2), tuple(b2))
+    plan = _DOT_PLANS.get(key)
+    if plan is None:
+        n1, n2 = S.normalize_axes(t1.shape, c1), S.normalize_axes(t2.shape, c2)
+        m1, m2 = S.normalize_axes(t1.shape, b1), S.normalize_axes(t2.shape, b2)
+        plan = (n1, m1, n2, m2, S.dot(t1.shape, n1, m1, t2.shape, n2, m2))
+        if len(_DOT_PLANS) >= 4096:
+            _DOT_PLANS.clear()
+        _DOT_PLANS[key] = plan
+    c1, b1, c2, b2, shape = plan
+    return _impl(t1, t2).dot(template(ty, shape), t1, c1, b1, t2, c2, b2)
+
+
+_DOT_PLANS = {}
 
 
 # ---- shape / data movement -----------------------------------------------------------------

@@ -5,6 +5,8 @@ backend callback's arithmetic.
 """
 from __future__ import annotations
 
+import functools
+
 from math import prod
 
 
@@ -52,13 +54,18 @@ def binary_broadcast(left, right):
 def broadcast_strides(shape, out_shape):
     """Element strides of `shape` viewed in `out_shape` (right-aligned), 0 on broadcast axes --
     the index arithmetic behind broadcast_data/2 (binary_backend.ex:228-276)."""
+    return list(_broadcast_strides(tuple(shape), tuple(out_shape)))
+
+
+@functools.lru_cache(maxsize=4096)
+def _broadcast_strides(shape, out_shape):
     rank = len(out_shape)
-    padded = (1,) * (rank - len(shape)) + tuple(shape)
+    padded = (1,) * (rank - len(shape)) + shape
     strides, s = [0] * rank, 1
     for a in range(rank - 1, -1, -1):
         strides[a] = 0 if padded[a] == 1 else s
         s *= padded[a]
-    return strides
+    return tuple(strides)
 
 
 def broadcast_axes(shape, new_shape):

@@ -57,7 +57,14 @@ class Tensor:
 
 def template(type, shape) -> Tensor:
     """An output template: a tensor without data, as passed as the first callback argument."""
-    return Tensor(None, T.normalize(type), tuple(shape))
+    t = object.__new__(Tensor)  # (the hot path of every front-end call: no dataclass machinery)
+    set_ = object.__setattr__
+    shape = tuple(shape) if shape.__class__ is not tuple else shape
+    set_(t, "data", None)
+    set_(t, "type", T.normalize(type))
+    set_(t, "shape", shape if all(d.__class__ is int for d in shape) else tuple(int(d) for d in shape))
+    set_(t, "names", (None,) * len(shape))
+    return t
 
 
 # ---- number -> binary, following the reference's write path ---------------------------------

@@ -57,6 +57,9 @@ def is_sub_byte(t) -> bool:
 
 def code(t) -> int:
     """The element type a kernel is told: sub-byte integers are held one per byte."""
+    c = _CODES.get(t) if t.__class__ is tuple else None
+    if c is not None:
+        return c
     t = normalize(t)
     return _CODES[t] if t in _CODES else _SUB_BYTE[t]
 

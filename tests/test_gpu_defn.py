@@ -12,7 +12,8 @@ from nx_amd.tensor import template
 from nx_amd import defn
 from nx_amd import nx as Nx
 from nx_amd import random as Random
-from nx_amd.backend import mem_stats
+from nx_amd import _lib as L
+from nx_amd.backend import _Context, mem_stats
 from random_support import CASES, check_random_case
 from support import assert_all_close, assert_bits_equal, from_numpy, seed_of
 from test_defn import CHAINS, build_args, f32
@@ -67,8 +68,9 @@ def test_intermediates_go_back_to_the_pool_during_the_walk(hip):
         for _ in range(12):
             t = Nx.exp(Nx.negate(t))
         return t
+    gc.collect()  # tensors earlier tests left behind must not be freed in the middle of the walk,
+    L.check(L.lib.hipnx_trim(_Context.get(0)))  # nor their larger pooled blocks be handed out for these 16 MiB
     defn.jit(chain)(x)  # warm the pool
-    gc.collect()  # tensors earlier tests left behind must not be freed in the middle of the walk
     before = mem_stats()["live"]
     seen = []
     original = defn._Run.apply
