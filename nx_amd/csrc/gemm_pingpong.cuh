@@ -280,9 +280,11 @@ gemm_pingpong_kernel(GemmArgs a) {
 // phase p.  The waves that requested a slab wait for it at the end of the memory phase before the one that
 // reads it (vmcnt: all but their (NSTAGE - 2) / 2 younger slabs), and the barrier behind that wait publishes it.
 //
-// BM_ = BN_ = 64 with eight stages is the shape for a few rows against a long K-inner weight matrix: 64 rows of
-// the weights per work-group (a slab of them is 8 KiB), seven slabs requested ahead -- 56 KiB in flight per CU,
-// which is what a stream from HBM at the part's rate needs -- while the rows' own slabs come from L2.
+// BM_ = BN_ = 64 is the shape for a few rows against a long K-inner weight matrix: 64 rows of the weights per
+// work-group (a slab of them is 8 KiB, as is a slab of the rows, which comes from L2), either eight stages of one
+// slab or, with SPP = 2, four stages of two slabs -- a phase then covers 256 bytes of K and there are half as
+// many barriers.  The ring's depth hardly matters there (four, six and eight stages measured alike): a
+// work-group takes in as many bytes of the rows as of the weights, and a CU's intake is what bounds it.
 template <int DT, bool L_KIN, bool R_KIN, int BM_ = 128, int BN_ = 128, int NSTAGE_ = 4, int SPP = 1>
 __global__ void __launch_bounds__(512)
 gemm_pingpong128_kernel(GemmArgs a) {
