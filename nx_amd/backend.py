@@ -404,7 +404,7 @@ class HipNxBackend:
         dev = cls._device_of(t)
         t = cls._from_nx(t, dev)
         axes = opts.get("axes")
-        if axes is not None and t.type[1] >= 8:
+        if axes is not None and len(axes) > 1 and t.type[1] >= 8:
             axes = sorted(a % len(t.shape) for a in axes)
             runs = [[a] for a in axes[:1]]
             for a in axes[1:]:
