@@ -342,12 +342,13 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
         // weight matrix stream the weights with many small tiles
         const int64_t t256 = ((M + 255) / 256) * ((N + 255) / 256) * batch;
         const int64_t t128 = ((M + 127) / 128) * ((N + 127) / 128);
-        const bool two_byte = l_dt == HIPNX_BF16 || l_dt == HIPNX_F16;
-        int cfg;
-        const bool big_ok = M >= 192 && N >= 192;
         const int64_t tw = ((M + 255) / 256) * ((N + 127) / 128) * batch;
-        // few rows: 64-row tiles (f32: whatever its cost model below picks), except for a 2-byte K-outer operand (x . W with W stored [K, N]), which only the
-        // 128-row kernels read by transposing loads (64 x 4096 x 4096 bf16: 72 us on 64 x 32 tiles, 19 us here)
+        const bool two_byte = l_dt == HIPNX_BF16 || l_dt == HIPNX_F16;
+        const bool big_ok = M >= 192 && N >= 192;
+        int cfg;
+        // few rows: 64-row tiles (f32: whatever its cost model below picks), except for a 2-byte K-outer operand
+        // (x . W with W stored [K, N]), which only the 128-row kernels read by transposing loads
+        // (64 x 4096 x 4096 bf16: 72 us on 64 x 32 tiles, 16.5 us there)
         if (M <= 64 && l_dt != HIPNX_F32 && !(two_byte && !(l_kin && r_kin) && N >= 128)) cfg = GEMM_CFG_64x32;
         else if (t256 * 4 >= (int64_t)ctx->num_cus * 3 && big_ok) cfg = GEMM_CFG_256;
         else if (two_byte && M >= 192 && N >= 128 && t128 * batch > ctx->num_cus)
@@ -366,9 +367,6 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
         const int64_t nslab = Kb / SLAB;
         const bool splittable = cfg == GEMM_CFG_128 && batch == 1 && scale_mode == HIPNX_SCALE_NONE && (M * N) % 4 == 0 &&
                                 (l_dt == HIPNX_S8 ? !is_float(out_dt) : true);
-        // (the second pass and the partial results cost about 10 us: worth it from K = 32 slabs on, with at least
-        // 8 slabs left per split and no more work-groups than CUs; 1024 x 2048 x 2048, 128 tiles, is faster whole:
-        // 21 us against 22 us in two halves and 27 us in four quarters)
         if (l_dt == HIPNX_F32) {
           // An f32 slab is eight times the MFMA work of a 2-byte one (2.6 us per slab of a 128 x 128 tile, 0.55 us
           // for a 64 x 32 tile, the second pass of a split about 8 us), so a grid that leaves CUs idle is cut much
@@ -402,6 +400,10 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
             if (10.0 + rounds(t64) * (double)nslab * 0.55 < best) { cfg = GEMM_CFG_64x32; splits = 1; }
           }
         } else if (splittable && t128 * 2 <= ctx->num_cus && nslab >= (t128 * 4 <= ctx->num_cus ? 32 : 64))
+          // (the second pass and the partial results cost about 10 us: worth it from K = 32 slabs on -- 64 where
+          // the grid already covers more than a quarter of the CUs -- with at least 8 slabs left per split and no
+          // more work-groups than CUs; 1024 x 2048 x 2048, 128 tiles of 32 slabs, is faster whole: 21 us against
+          // 22 us in two halves and 27 us in four quarters)
           for (int cand = 16; cand >= 2; cand /= 2)
             if (t128 * cand <= (int64_t)ctx->num_cus && nslab % cand == 0 && nslab / cand >= 8) { splits = cand; break; }
         void *ws = nullptr;
