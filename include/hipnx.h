@@ -221,7 +221,7 @@ int hipnx_argreduce(hipnx_ctx *ctx, int op, int tie, int in_dt, int out_dt, int6
  * out_dt (f32 accumulation for f16/bf16/f32 operands, exact s32 for s8, then one encode).
  * out_dt may be HIPNX_BF16_RNE (bf16 rounded to nearest even).  The call may take workspace from the
  * context's pool and return it before it ends: a re-laid operand whose K-outer rows are not whole
- * 16-byte blocks (or, for mid-size int8 problems, any K-outer operand), zero-extended copies of both operands when K is not a whole number of 128-byte slabs,
+ * 16-byte blocks, zero-extended copies of both operands when K is not a whole number of 128-byte slabs,
  * the partial results of a contraction whose K is split over several work-groups per tile. */
 int hipnx_dot(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batch, int64_t M, int64_t N,
               int64_t K, int l_layout, int r_layout, const hipnx_buf *l, const hipnx_buf *r,

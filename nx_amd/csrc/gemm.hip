@@ -287,15 +287,8 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
   const bool pipelined = Kb % SLAB == 0;
   // the pipelined kernel transposes K-outer operands itself when the rows come in whole blocks
   const int row_block = esz == 1 ? 16 : (esz == 2 ? 8 : 4);
-  // int8 on 128 x 128 tiles: a K-outer operand keeps the one-group kernel and its register-staged transposes
-  // (1024 x 2048 x 4096: 44 us against 18 us with both operands K-inner), so from 512 rows, 2^32 multiply-adds
-  // and K = 2048 on the operand is laid out K-inner first, which costs 6-12 us (with fewer rows the copy of the
-  // other operand costs more than it saves: 256 x 4096 x 4096 29 us with it)
-  const bool s8_mid = l_dt == HIPNX_S8 && r_dt == HIPNX_S8 && pipelined && M >= 512 && Kb >= 16 * SLAB &&
-                      (double)M * (double)N * (double)K * (double)batch >= 4294967296.0 &&
-                      !(((M + 255) / 256) * ((N + 255) / 256) * batch * 2 >= (int64_t)ctx->num_cus && M >= 192 && N >= 192);  // (those take 256 x 256 tiles)
-  const bool l_relay = l_layout == HIPNX_K_OUTER && (!(pipelined && M % row_block == 0) || s8_mid);
-  const bool r_relay = r_layout == HIPNX_K_OUTER && (!(pipelined && N % row_block == 0) || s8_mid);
+  const bool l_relay = l_layout == HIPNX_K_OUTER && !(pipelined && M % row_block == 0);
+  const bool r_relay = r_layout == HIPNX_K_OUTER && !(pipelined && N % row_block == 0);
   hipnx_buf *lt = nullptr, *rt = nullptr;
   int st = HIPNX_OK;
   if (l_relay) {

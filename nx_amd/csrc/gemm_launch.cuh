@@ -103,11 +103,11 @@ static int launch_cfg(const hipnx_ctx *ctx, int cfg, const GemmArgs &a, int64_t 
       // operand is copied straight into LDS (the condition of the kernel's L_TR / R_TR)
       constexpr int ES = DT == HIPNX_S8 ? 1 : DT == HIPNX_F32 ? 4 : 2;
       constexpr bool tr = ES <= 2 && 128 * ES >= 256;
-      // From 8 slabs of K on, the two-group kernel (2-byte types; int8 with both operands K-inner): 730 clocks per
+      // From 8 slabs of K on, the two-group kernel (2-byte types and int8; f32 with both operands K-inner): 730 clocks per
       // slab against the 1600-2100 below.  It holds a CU's LDS alone, so for the 2-byte types only where no
       // second work-group would share the CU; int8 has no wider two-group tile to fall back on and takes it
       // for every grid (2048 x 4096 x 4096, 512 tiles: 52 -> 42 us).
-      if constexpr (DT == HIPNX_BF16 || DT == HIPNX_F16 || ((DT == HIPNX_S8 || DT == HIPNX_F32) && LK && RK)) {
+      if constexpr (DT == HIPNX_BF16 || DT == HIPNX_F16 || DT == HIPNX_S8 || (DT == HIPNX_F32 && LK && RK)) {
         const int64_t groups = ((a.M + 127) / 128) * ((a.N + 127) / 128) * batch;
         if (a.Kb >= 8 * SLAB && a.ld_l < (1ll << 23) && a.ld_r < (1ll << 23) && (DT == HIPNX_S8 || DT == HIPNX_F32 || groups <= ctx->num_cus))
           return launch_pingpong128<DT, LK, RK>(ctx, a, batch);
@@ -123,11 +123,17 @@ static int launch_cfg(const hipnx_ctx *ctx, int cfg, const GemmArgs &a, int64_t 
       if constexpr (DT == HIPNX_F32) return launch_one<DT, 2, 2, 1, 2, LK, RK>(ctx, a, batch);
       return launch_one<DT, 2, 2, 2, 2, LK, RK>(ctx, a, batch);
     default:
-      // K-inner 2-byte and int8 operands: the two-group kernel on 64 x 64 tiles -- 64 rows of the weights per
+      // K-inner 2-byte operands and int8 in either layout: the two-group kernel on 64 x 64 tiles -- 64 rows of the weights per
       // work-group, their slabs requested three phases (six slabs) ahead, two slabs per phase where K allows
       // (int8 64 x 11008 x 4096: kernel 13.0 us; the 64 x 32 tiles below 18.7 us)
-      if constexpr (LK && RK && (DT == HIPNX_BF16 || DT == HIPNX_F16 || DT == HIPNX_S8)) {
+      if constexpr ((LK && RK && (DT == HIPNX_BF16 || DT == HIPNX_F16)) || DT == HIPNX_S8) {
         if (a.Kb >= 8 * SLAB && a.ld_l < (1ll << 24) && a.ld_r < (1ll << 24)) {
+          if constexpr (DT == HIPNX_S8 && !RK) {
+            // int8 weights stored [K, N]: a k-row of a 64-column tile is half a cache line; where 128-column tiles
+            // still give 3/8 of the CUs work they stream the weights as fast as the K-inner layout
+            // (64 x 32000 x 4096: 50 -> 28 us; with 32 such tiles, 64 x 4096 x 4096, they are slower: 12 -> 18 us)
+            if (((a.N + 127) / 128) * batch * 8 >= (int64_t)ctx->num_cus * 3) return launch_pingpong128<DT, LK, RK, 64, 128, 6, 1>(ctx, a, batch);
+          }
           if (a.Kb % (2 * SLAB) == 0) return launch_pingpong128<DT, LK, RK, 64, 64, 4, 2>(ctx, a, batch);
           return launch_pingpong128<DT, LK, RK, 64, 64, 8, 1>(ctx, a, batch);
         }

@@ -272,6 +272,17 @@ __device__ __forceinline__ int tr_slot(int k, int chunk) {
   else return chunk ^ (k & 7) ^ (((k >> 4) & 1) << 3);
 }
 
+// the same for k-rows narrower than the 256 bytes that span all LDS banks (int8 tiles of 64 or 128 columns): the
+// chunk index XOR as many low bits of k as the row has chunk bits
+template <int ES, int RBYTES>
+__device__ __forceinline__ int tr_slot_w(int k, int chunk) {
+  if constexpr (RBYTES >= 256) return tr_slot<ES>(k, chunk);
+  else {
+    static_assert(ES == 1 && (RBYTES == 128 || RBYTES == 64), "narrow k-rows: int8 tiles of 64 or 128 columns");
+    return chunk ^ (k & (RBYTES / 16 - 1));
+  }
+}
+
 template <int ES, int ROWS, int NWAVES>
 struct KOuterDmaLoader {
   static constexpr int RBYTES = ROWS * ES;     // bytes per k-row of the slab
@@ -333,7 +344,7 @@ __device__ __forceinline__ v4i read_fragment_tr(const unsigned char *slab, int r
 #pragma unroll
     for (int h = 0; h < 2; h++) {
       const int k = kbase + 8 * h;
-      const unsigned char *p = slab + k * ROWS + tr_slot<1>(k, n >> 4) * 16 + (n & 15);
+      const unsigned char *p = slab + k * ROWS + tr_slot_w<1, ROWS>(k, n >> 4) * 16 + (n & 15);
       const v2i r = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i *)p);
       out[2 * h] = r[0];
       out[2 * h + 1] = r[1];

@@ -84,7 +84,7 @@ template <int ES, int ROWS, int NWAVES>
 struct PPKOuterLoader {
   static constexpr int RBYTES = ROWS * ES;
   static constexpr int PER = ROWS / 8 / NWAVES;
-  static_assert(RBYTES >= 256, "a k-row must span all LDS banks");
+  static_assert(RBYTES >= 256 || ES == 1, "a 2-byte k-row must span all LDS banks");
   const unsigned char *base;
   unsigned off[PER];
   __device__ __forceinline__ void init(const unsigned char *g, int64_t ld, int64_t col0, int64_t cols_valid, int wave, int lane) {
@@ -95,7 +95,7 @@ struct PPKOuterLoader {
     for (int i = 0; i < PER; i++) {
       const int o = (wave + NWAVES * i) * 1024 + lane * 16;
       const int k = o / RBYTES, slot = (o % RBYTES) / 16;
-      int64_t byte = col0 * ES + tr_slot<ES>(k, slot) * 16;
+      int64_t byte = col0 * ES + tr_slot_w<ES, RBYTES>(k, slot) * 16;
       byte = byte <= last ? byte : last;
       off[i] = (unsigned)((int64_t)k * ld + (byte - first));
     }
@@ -291,13 +291,14 @@ gemm_pingpong128_kernel(GemmArgs a) {
   typedef typename Mma16<DT>::acc_t acc_t;
   constexpr int BM = BM_, BN = BN_, TM16 = BM / 32, TN16 = BN / 32, NSTAGE = NSTAGE_, AHEAD = NSTAGE - 1;
   static_assert((BM == 128 || BM == 64) && (BN == 128 || BN == 64) && NSTAGE % 2 == 0 && NSTAGE >= 4, "tile extents of 64 or 128, an even number of stages");
-  static_assert((BM == 128 || L_KIN) && (BN == 128 || R_KIN), "a 64-row operand is K-inner (a k-row of a K-outer one must span all LDS banks)");
+  static_assert((BM == 128 || L_KIN || DT == HIPNX_S8) && (BN == 128 || R_KIN || DT == HIPNX_S8),
+                "a 64-row 2-byte operand is K-inner (a k-row of a K-outer one must span all LDS banks)");
   constexpr int LREQ = BM / 32, RREQ = BN / 32, REQ = SPP * (LREQ + RREQ);  // requests per wave and phase
   // a stage holds the SPP slabs of one phase, each as [left rows | right rows]
   constexpr int SLAB1 = (BM + BN) * SLAB, STAGE = SPP * SLAB1, KS = 2 * SPP;
   constexpr int ES = (DT == HIPNX_S8) ? 1 : 2;
-  static_assert(DT == HIPNX_BF16 || DT == HIPNX_F16 || ((DT == HIPNX_S8 || DT == HIPNX_F32) && L_KIN && R_KIN),
-                "2-byte MFMA types; int8 and f32 with K-inner operands");
+  static_assert(DT == HIPNX_BF16 || DT == HIPNX_F16 || DT == HIPNX_S8 || (DT == HIPNX_F32 && L_KIN && R_KIN),
+                "2-byte MFMA types and int8; f32 with K-inner operands");
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
   int tm, tn;
@@ -320,9 +321,11 @@ gemm_pingpong128_kernel(GemmArgs a) {
       for (int q = 0; q < 4; q++) acc[i][j][q] = 0;
 
   // the four waves of the memory group request a whole slab: LREQ + RREQ instructions per wave
-  PPKInnerLoader<BM, 4> lkin;
-  PPKInnerLoader<BN, 4> rkin;
-  PPKOuterLoader<2, 128, 4> lkout, rkout;
+  struct Unused {};  // (only the loader of an operand's own layout is instantiated)
+  std::conditional_t<L_KIN, PPKInnerLoader<BM, 4>, Unused> lkin;
+  std::conditional_t<R_KIN, PPKInnerLoader<BN, 4>, Unused> rkin;
+  std::conditional_t<L_KIN, Unused, PPKOuterLoader<ES, BM, 4>> lkout;
+  std::conditional_t<R_KIN, Unused, PPKOuterLoader<ES, BN, 4>> rkout;
   if constexpr (L_KIN) lkin.init(lb, a.ld_l, m0, a.M, w4, lane);
   else lkout.init(lb, a.ld_l, m0, a.M, w4, lane);
   if constexpr (R_KIN) rkin.init(rb, a.ld_r, n0, a.N, w4, lane);
@@ -362,12 +365,12 @@ gemm_pingpong128_kernel(GemmArgs a) {
 #pragma unroll
       for (int i = 0; i < TM16; i++) {
         if constexpr (L_KIN) fa[ks][i] = *reinterpret_cast<const v4i *>(sl + a_rd[ks & 1] + i * (16 * SLAB));
-        else fa[ks][i] = read_fragment_tr<2, BM>(sl, wm + 16 * i, ks & 1, lane);
+        else fa[ks][i] = read_fragment_tr<ES, BM>(sl, wm + 16 * i, ks & 1, lane);
       }
 #pragma unroll
       for (int j = 0; j < TN16; j++) {
         if constexpr (R_KIN) fb[ks][j] = *reinterpret_cast<const v4i *>(sl + b_rd[ks & 1] + j * (16 * SLAB));
-        else fb[ks][j] = read_fragment_tr<2, BN>(sl + BM * SLAB, wn + 16 * j, ks & 1, lane);
+        else fb[ks][j] = read_fragment_tr<ES, BN>(sl + BM * SLAB, wn + 16 * j, ks & 1, lane);
       }
     }
     // this group's requests in flight, oldest first: slabs p + 1, p + 3, .. p + AHEAD; slab p + 1 is read next phase

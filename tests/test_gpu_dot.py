@@ -183,11 +183,13 @@ def test_few_rows_against_long_matrix(M, ty, N, K, hip, oracle):
 
 
 @pytest.mark.parametrize("M", [1, 24, 64])
-@pytest.mark.parametrize("ty,N,K", [("bf16", 264, 2048), ("f16", 1024, 1056), ("s8", 400, 4096), ("bf16", 120, 640), ("bf16", 328, 192)])
+@pytest.mark.parametrize("ty,N,K", [("bf16", 264, 2048), ("f16", 1024, 1056), ("s8", 400, 4096), ("bf16", 120, 640), ("bf16", 328, 192),
+                                    ("s8", 12304, 1152), ("s8", 1040, 1024), ("s8", 48, 2048)])
 def test_few_rows_against_weights_stored_k_outer(M, ty, N, K, hip, oracle):
     """x . W with W stored [K, N], the plain Nx.dot(x, w): a few rows of a 2-byte type take the 128-row kernels
-    (which read a K-outer operand by transposing loads, K split over work-groups when long), int8 and narrow
-    outputs the 64-row tiles; a contraction length that is an odd number of slabs takes one slab per phase."""
+    (which read a K-outer operand by transposing loads, K split over work-groups when long), int8 the 64-row tiles
+    with 64 or -- for many columns -- 128 columns of the weights, read by the byte-transposing loads; a contraction
+    length that is an odd number of slabs takes one slab per phase."""
     rng = np.random.default_rng(seed_of(M, ty, N, K, "k-outer weights"))
     if ty == "s8":
         x = rng.integers(-127, 128, size=(M, K)).astype(np.int8)
