@@ -394,8 +394,9 @@ def main():
         _, ms = tstat(lambda: Nx.dot(xq, [1], nxt(), [1], out_type="s32"), steps, warm)
         entry("dot_s8_w8_64x11008x4096_rotated", 48168960.0, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read")
         # the same layer with its weights stored [K, N], the plain Nx.dot(x, w) of a dense layer (K-outer weights)
-        nxt = rotating(lambda: put(np.ascontiguousarray(w_np.T), "s8"), w_np.nbytes)
-        _, ms = tstat(lambda: Nx.dot(xq, nxt(), out_type="s32"), steps, warm)
+        nxt_t = rotating(lambda: put(np.ascontiguousarray(w_np.T), "s8"), w_np.nbytes)
+        _, ms = tstat(lambda: Nx.dot(xq, nxt_t(), out_type="s32"), steps, warm)
+        del nxt_t
         entry("dot_s8_w8_64x11008x4096_weights_k_outer_rotated", 48168960.0, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read")
         # the whole config: dot -> as_type f32 -> multiply by the per-column scales
         _, ms = tstat(lambda: Nx.multiply(Nx.as_type(Nx.dot(xq, [1], nxt(), [1], out_type="s32"), "f32"), sc), steps, warm)
