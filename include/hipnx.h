@@ -259,6 +259,15 @@ int hipnx_gather(hipnx_ctx *ctx, int elem_bytes, int rank, const int64_t *t_dims
                  int64_t n_tuples, int depth, int oob_policy, const hipnx_buf *t,
                  const hipnx_buf *idx, hipnx_buf *out);
 
+/* replaces: block(%Nx.Block.Take{axis}) for any axis (nx/lib/nx/backend.ex:144; nx/lib/nx/block.ex:57-59;
+ * nx/lib/nx.ex:14807-14819, whose default is gather + transpose).  The tensor is viewed as
+ * [outer, axis_len, inner]; out[o, j, :] = t[o, idx[j], :] for the n_idx indices of integer type idx_dt,
+ * out is [outer, n_idx, inner].  `msg_dims[rank]` is the shape an out-of-range index is reported against:
+ * the tensor's with the taken axis moved to the front, as the reference's transposing default reports it. */
+int hipnx_take(hipnx_ctx *ctx, int elem_bytes, int64_t outer, int64_t axis_len, int64_t inner, int idx_dt,
+               int64_t n_idx, int oob_policy, int rank, const int64_t *msg_dims, const hipnx_buf *t,
+               const hipnx_buf *idx, hipnx_buf *out);
+
 /* ---- callbacks one step off the hot path (callers: Nx.LinAlg, Nx.Random, grad code) ----------
  * replaces: select/4 (nx/lib/nx/backend.ex:84; oracle binary_backend.ex:604-648).
  * out[i] = pred[i] != 0 ? on_true[i] : on_false[i]; the three operands are broadcast to out_dims

@@ -99,6 +99,8 @@ PROTOTYPES = {
     "hipnx_transpose": [_ctx_p, C.c_int, C.c_int, _i64p, _intp, _buf_p, _buf_p],
     "hipnx_broadcast": [_ctx_p, C.c_int, C.c_int, _i64p, _i64p, _buf_p, _buf_p],
     "hipnx_gather": [_ctx_p, C.c_int, C.c_int, _i64p, C.c_int, C.c_int64, C.c_int, C.c_int, _buf_p, _buf_p, _buf_p],
+    "hipnx_take": [_ctx_p, C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_int64, C.c_int, C.c_int, _i64p, _buf_p, _buf_p,
+                   _buf_p],
     "hipnx_select": [_ctx_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _i64p, _i64p, _i64p, _i64p, _buf_p, _buf_p,
                      _buf_p, _buf_p],
     "hipnx_clip": [_ctx_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int64, _buf_p, _buf_p, _buf_p, _buf_p],

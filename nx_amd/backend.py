@@ -594,6 +594,23 @@ class HipNxBackend:
         return res
 
     @classmethod
+    def _take_along(cls, out: Tensor, t: Tensor, indices: Tensor, axis: int) -> Tensor:
+        """block(%Nx.Block.Take{axis}) along an axis that is not the first (backend.ex:144; nx.ex:14807-14819): one
+        kernel over the tensor viewed as [outer, axis_len, inner] instead of the default's transpose, gather and
+        transpose back.  An out-of-range index is reported as the default reports it: against the shape with the
+        taken axis moved to the front (binary_backend.ex:1906-1912, 1949-1952)."""
+        dev = cls._device_of(t, indices)
+        t, indices = cls._from_nx(t, dev), cls._from_nx(indices, dev)
+        shape = t.shape
+        outer, axis_len, inner = prod(shape[:axis]), shape[axis], prod(shape[axis + 1:])
+        moved = (axis_len,) + shape[:axis] + shape[axis + 1:]
+        res = cls._alloc(out, dev)
+        L.check(L.lib.hipnx_take(res.data.ref.ctx, T.size_bytes(t.type), outer, axis_len, inner, T.code(indices.type),
+                                 indices.size, _bounds["policy"], len(moved), L.i64_array(moved), cls._handle(t),
+                                 cls._handle(indices), res.data.ref.handle))
+        return res
+
+    @classmethod
     def gather(cls, out: Tensor, t: Tensor, indices: Tensor, opts) -> Tensor:
         """gather/4 (backend.ex:81; oracle binary_backend.ex:1902-1959): out-of-bounds indices
         raise, with the reference's message."""
@@ -932,6 +949,8 @@ class HipNxBackend:
             t, indices = args
             idx = indices.with_(shape=(indices.size, 1))
             return cls.gather(out, t, idx, {"axes": [0]})
+        if isinstance(struct, BlockTake) and T.storage(args[0].type) == args[0].type:
+            return cls._take_along(out, args[0], args[1], struct.axis)
         if isinstance(struct, BlockThreefry):
             return cls.threefry2x32(out, args[0])
         return fun(struct, *args)

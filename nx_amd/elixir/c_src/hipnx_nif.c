@@ -265,6 +265,22 @@ static ERL_NIF_TERM nif_gather(ErlNifEnv *env, int argc, const ERL_NIF_TERM argv
   return ok(env, make_buf(env, out));
 }
 
+/* take(ctx, elem_bytes, outer, axis_len, inner, idx_dt, n_idx, oob_policy, msg_dims, t, idx, out_bytes) */
+static ERL_NIF_TERM nif_take(ErlNifEnv *env, int argc, const ERL_NIF_TERM argv[]) {
+  (void)argc;
+  GET_CTX(0, ctx); GET_INT(1, esz); GET_I64(2, outer); GET_I64(3, axis_len); GET_I64(4, inner); GET_INT(5, idt); GET_I64(6, n_idx);
+  GET_INT(7, policy);
+  int64_t dims[64];
+  int rank;
+  if (!get_i64_list(env, argv[8], dims, 64, &rank)) return enif_make_badarg(env);
+  GET_BUF(9, t); GET_BUF(10, idx); GET_I64(11, out_bytes);
+  hipnx_buf *out;
+  CHECK(hipnx_buf_alloc(ctx, (size_t)out_bytes, &out));
+  int st = hipnx_take(ctx, esz, outer, axis_len, inner, idt, n_idx, policy, rank, dims, t, idx, out);
+  if (st != HIPNX_OK) { hipnx_buf_destroy(out); return error_from_status(env, st); }
+  return ok(env, make_buf(env, out));
+}
+
 /* select(ctx, pred_dt, true_dt, false_dt, out_dt, out_dims, pred_strides, true_strides, false_strides, pred, on_true, on_false, out_bytes) */
 static ERL_NIF_TERM nif_select(ErlNifEnv *env, int argc, const ERL_NIF_TERM argv[]) {
   (void)argc;
@@ -436,6 +452,7 @@ static ErlNifFunc funcs[] = {
     {"narrow_int", 5, nif_narrow_int, IO},      {"device_ptr", 1, nif_device_ptr, 0},
     {"wrap", 3, nif_wrap, 0},                   {"ipc_export", 2, nif_ipc_export, IO},
     {"ipc_import", 3, nif_ipc_import, IO},
+    {"take", 12, nif_take, IO},
     {"eye", 6, nif_eye, IO},                    {"threefry2x32", 4, nif_threefry2x32, IO},
     {"sync", 1, nif_sync, IO}};
 

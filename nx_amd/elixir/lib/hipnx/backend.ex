@@ -465,6 +465,23 @@ defmodule HipNx.Backend do
     gather(out, t, %{indices | shape: {Nx.size(indices), 1}, names: [nil, nil]}, axes: [0])
   end
 
+  # along any other axis: one kernel over the tensor viewed as [outer, axis, inner] instead of the default's
+  # transpose, gather and transpose back (nx.ex:14807-14819); a bad index is reported against the shape
+  # with the taken axis moved to the front, as the default reports it (binary_backend.ex:1906-1912)
+  def block(%Nx.Block.Take{axis: axis}, %T{type: {_, bits}} = out, [t, indices], _fun) when bits >= 8 do
+    device = device_of([t, indices])
+    {tref, _} = from_nx(t, device)
+    {iref, _} = from_nx(indices, device)
+    dims = Tuple.to_list(t.shape)
+    {before, [axis_len | rest]} = Enum.split(dims, axis)
+
+    ref =
+      NIF.take(ctx(device), div(bits, 8), Enum.product(before), axis_len, Enum.product(rest), dt(indices.type),
+        Nx.size(indices), 0, [axis_len | before ++ rest], tref, iref, bytes(out))
+
+    to_nx(unwrap!(ref), device, out)
+  end
+
   def block(struct, _out, args, fun), do: apply(fun, [struct | args])
 
   ## Selection, windows and creation

@@ -24,6 +24,7 @@ defmodule HipNx.NIF do
   def transpose(_ctx, _elem_bytes, _dims, _perm, _in, _out_bytes), do: err()
   def broadcast(_ctx, _elem_bytes, _dims, _strides, _in, _out_bytes), do: err()
   def gather(_ctx, _elem_bytes, _dims, _idx_dt, _n_tuples, _depth, _policy, _t, _idx, _out_bytes), do: err()
+  def take(_ctx, _elem_bytes, _outer, _axis_len, _inner, _idx_dt, _n_idx, _policy, _msg_dims, _t, _idx, _out_bytes), do: err()
   def select(_ctx, _p_dt, _t_dt, _f_dt, _out_dt, _dims, _p_strides, _t_strides, _f_strides, _p, _t, _f, _out_bytes), do: err()
   def clip(_ctx, _in_dt, _min_dt, _max_dt, _out_dt, _n, _in, _min, _max, _out_bytes), do: err()
   def strided_copy(_ctx, _elem_bytes, _dims, _in_strides, _in_offset, _out_strides, _out_offset, _in, _out_or_bytes), do: err()

@@ -176,3 +176,88 @@ def test_slices_off_the_vector_grid(ty, shape, starts, lengths, hip, oracle):
     cfg = [(1, 2, 0)] * len(shape)
     pad_h, pad_o = Nx.tensor(0, type=ty, backend=hip), Nx.tensor(0, type=ty, backend=oracle)
     assert_bits_equal(Nx.pad(hx, pad_h, cfg), Nx.pad(ox, pad_o, cfg), f"pad {ty} {shape}")
+
+
+TAKE_ALONG = [((40, 300, 16), 1, "bf16"), ((40, 300, 16), 2, "bf16"), ((7, 129, 5), 1, "f32"), ((7, 129, 5), 2, "f32"), ((513, 1000), 1, "u8"),
+              ((513, 1000), 1, "f32"), ((3, 4, 50, 6), 2, "s64"), ((3, 4, 50, 6), 3, "s16"), ((2, 3, 64, 24), 2, "bf16"), ((1, 9, 4096), 2, "f32")]
+
+
+@pytest.mark.parametrize("shape,axis,ty", TAKE_ALONG, ids=[f"{s}-{a}-{t}" for s, a, t in TAKE_ALONG])
+@pytest.mark.parametrize("idx_ty", ["s32", "u8", "s64"])
+def test_take_along_an_inner_axis_is_one_kernel(shape, axis, ty, idx_ty, hip, oracle):
+    """take along an axis that is not the first: the tensor viewed as [outer, axis, inner], slices of every width
+    (a single element along the last axis, 2 to 16 bytes, whole vectors) -- against the oracle's gather +
+    transpose and against numpy."""
+    rng = np.random.default_rng(seed_of(shape, axis, ty, idx_ty, "along"))
+    t = rand_raw(rng, ty, shape)
+    hi = min(shape[axis], 256 if idx_ty == "u8" else shape[axis])
+    idx = rng.integers(0, hi, size=(5, 21)).astype(np.dtype({"s32": np.int32, "u8": np.uint8, "s64": np.int64}[idx_ty]))
+    ht, ot = both(t, ty, hip, oracle)
+    hi_, oi = both(idx, idx_ty, hip, oracle)
+    got = Nx.take(ht, hi_, axis=axis)
+    assert_bits_equal(got, Nx.take(ot, oi, axis=axis), f"take {shape} axis {axis} {ty}")
+    assert np.array_equal(hip.to_numpy(got), np.take(t, idx.astype(np.int64), axis=axis))
+
+
+def test_take_along_an_inner_axis_reports_a_bad_index_like_the_reference(hip, oracle):
+    """The reference's take is gather on the tensor with the taken axis moved to the front, and its message names
+    that shape and axis 0 (binary_backend.ex:1906-1912, 1949-1952)."""
+    from nx_amd._lib import HipNxArgumentError
+    from oracle.binary_backend import ReferenceRaises
+    t = np.arange(3 * 4 * 5, dtype=np.float32).reshape(3, 4, 5)
+    idx = np.array([1, 9, 0, -2], dtype=np.int32)
+    ht, ot = both(t, "f32", hip, oracle)
+    hi_, oi = both(idx, "s32", hip, oracle)
+    with pytest.raises((ReferenceRaises, ValueError)) as ref:
+        Nx.take(ot, oi, axis=2)
+    assert "index 9 is out of bounds for axis 0 in shape {5, 3, 4}" in str(ref.value)
+    with pytest.raises(HipNxArgumentError, match="index 9 is out of bounds for axis 0 in shape \\{5, 3, 4\\}"):
+        Nx.take(ht, hi_, axis=2)
+    with pytest.raises(HipNxArgumentError, match="index 9 is out of bounds for axis 0 in shape \\{4, 3, 5\\}"):
+        Nx.take(ht, hi_, axis=1)
+    # and the device is usable afterwards
+    assert np.array_equal(hip.to_numpy(Nx.take(ht, from_numpy(np.array([4, 0], dtype=np.int32), "s32", hip), axis=2)), t[:, :, [4, 0]])
+
+
+@pytest.mark.parametrize("rows,cols,ty", [(300, 1024, "f32"), (260, 4096, "bf16"), (512, 2048, "u8"), (256, 512, "s64"),
+                                           (700, 16384, "f64"), (300, 2056, "bf16")])
+@pytest.mark.parametrize("idx_ty,picks", [("s32", 1024), ("s64", 2048), ("u32", 4104), ("u8", 8192)])
+def test_take_along_the_last_axis_of_long_rows(rows, cols, ty, idx_ty, picks, hip, oracle):
+    """Rows of 2 KB and more with at least half as many picks as the row has elements are staged in local memory;
+    fewer picks, rows of other sizes and index types of other widths take the kernel that reads through the
+    caches.  Both against numpy (the oracle's loop takes minutes at these sizes) and, on a corner, the oracle."""
+    rng = np.random.default_rng(seed_of(rows, cols, ty, idx_ty, picks, "long rows"))
+    t = rand_raw(rng, ty, (rows, cols))
+    hi = min(cols, 256 if idx_ty == "u8" else cols)
+    np_idx = {"s32": np.int32, "u32": np.uint32, "s64": np.int64, "u8": np.uint8}[idx_ty]
+    idx = rng.integers(0, hi, size=(picks,)).astype(np_idx)
+    got = Nx.take(from_numpy(t, ty, hip), from_numpy(idx, idx_ty, hip), axis=1)
+    assert np.array_equal(hip.to_numpy(got).view(np.uint8), np.take(t, idx.astype(np.int64), axis=1).view(np.uint8))
+    ot, oi = from_numpy(t[:3, :], ty, oracle), from_numpy(idx[:64], idx_ty, oracle)
+    assert_bits_equal(Nx.slice(got, [0, 0], [3, 64]), Nx.take(ot, oi, axis=1), f"take last axis {ty} {idx_ty}")
+
+
+def test_take_along_the_last_axis_of_long_rows_reports_and_clamps(hip):
+    """The three bounds policies on the kernel that stages rows: the raising one names the first bad index in index
+    order, the clamping one pins it to the ends of the axis, the deferring one reports at the next wait."""
+    from nx_amd import backend as B
+    from nx_amd._lib import HipNxArgumentError
+    rng = np.random.default_rng(5)
+    t = rng.standard_normal((300, 1024)).astype(np.float32)
+    idx = rng.integers(0, 1024, size=(1024,)).astype(np.int32)
+    idx[700], idx[333], idx[1000] = 1024, -7, 5000
+    ht, hi_ = from_numpy(t, "f32", hip), from_numpy(idx, "s32", hip)
+    with pytest.raises(HipNxArgumentError, match="index -7 is out of bounds for axis 0 in shape \\{1024, 300\\}"):
+        Nx.take(ht, hi_, axis=1)
+    good = np.clip(idx, 0, 1023)
+    assert np.array_equal(hip.to_numpy(Nx.take(ht, from_numpy(good, "s32", hip), axis=1)), t[:, good])
+    previous = B.bounds_policy("clamp")
+    try:
+        assert np.array_equal(hip.to_numpy(Nx.take(ht, hi_, axis=1)), t[:, good])
+        B.bounds_policy("defer")
+        late = Nx.take(ht, hi_, axis=1)
+        with pytest.raises(HipNxArgumentError, match="is out of bounds"):
+            Nx.to_binary(late)
+        B.sync()
+    finally:
+        B.bounds_policy(previous)
