@@ -438,6 +438,15 @@ def main():
         pred = Nx.greater(x, y)
         _, ms = tstat(lambda: Nx.select(pred, x, y), steps, warm)
         entry(f"select_f32_{nn}", 13.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+        # take along the last axis (picks within each row: the row goes through LDS), late-raising bounds policy
+        cols_idx = put(np.random.default_rng(6).integers(0, nn, size=nn, dtype=np.int32), "s32")
+        previous = B.bounds_policy("defer")
+        try:
+            _, ms = tstat(lambda: Nx.take(x, cols_idx, axis=1), steps, warm)
+        finally:
+            B.bounds_policy(previous)
+        entry(f"take_last_axis_f32_{nn}_deferred_bounds", 8.0 * N + 4.0 * nn, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+        del cols_idx
         _, ms = tstat(lambda: Nx.clip(x, -0.5, 0.5), steps, warm)
         entry(f"clip_f32_{nn}", 8.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
         _, ms = tstat(lambda: Nx.slice(x, [64, 128], [nn - 128, nn - 256]), steps, warm)
