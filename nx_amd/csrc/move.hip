@@ -201,11 +201,11 @@ gather_kernel(const unsigned char *__restrict__ t, const void *__restrict__ idx,
   }
 }
 
-// gather of slices of SB = 1, 2, 4 or 8 bytes (single elements: take along the innermost axis, gather with a
-// full tuple): one lane per 16-byte vector of the OUTPUT (8 bytes for SB = 1), i.e. S = 16 / SB slices, so that the row number
-// is taken apart once per S slices, the S reads are in flight together and the store is whole.  With one
-// slice per lane, take along the last axis of 4096^2 f32 ran at 1.4 TB/s although every read hits a
-// line its neighbours fetched.  The slices of one vector are walked by incrementing (o, j), which also
+// gather of slices of SB = 1, 2, 4 or 8 bytes (single elements), launched for take along the innermost axis with
+// rows before it (`period` > 0), whose reads stay within a row: one lane per 16-byte vector of the OUTPUT (8
+// bytes for SB = 1), i.e. S = 16 / SB slices, so that the row number is taken apart once per S slices, the
+// S reads are in flight together and the store is whole.  With one slice per lane, take along the last axis
+// of 4096^2 f32 ran at 1.4 TB/s although every read hits a line its neighbours fetched.  The slices of one vector are walked by incrementing (o, j), which also
 // covers a vector that crosses into the next `o`.  A vector with a rejected index (or the partial last
 // one) is stored slice by slice.
 template <int SB>
