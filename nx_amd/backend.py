@@ -195,11 +195,16 @@ class HipNxBackend:
     def to_binary(cls, t: Tensor, limit: int) -> bytes:
         """to_binary/2 (backend.ex:57): `limit` counts elements."""
         n = min(int(limit), t.size) * T.size_bytes(t.type)
-        buf = C.create_string_buffer(max(n, 1))
-        L.check(L.lib.hipnx_d2h(t.data.ref.ctx, cls._handle(t), 0, buf, n))
+        # the device writes straight into the bytes object that is returned (allocated unfilled, as the C API
+        # provides for a buffer that is filled before anyone sees it): a zeroed staging buffer and the copy out
+        # of it cost four times the transfer itself (256 MiB: 124 ms against 26 ms)
+        raw = _new_bytes(None, n)
+        address = _bytes_address(raw)
+        _advise_huge_pages(address, n)
+        L.check(L.lib.hipnx_d2h(t.data.ref.ctx, cls._handle(t), 0, address, n))
         if T.is_sub_byte(t.type):  # packed again on the way out (exla/lib/exla/device_buffer.ex:65-75)
-            return pack_sub_byte(np.frombuffer(buf.raw[:n], dtype=np.uint8), t.type)
-        return buf.raw[:n]
+            return pack_sub_byte(np.frombuffer(raw, dtype=np.uint8), t.type)
+        return raw
 
     @classmethod
     def to_numpy(cls, t: Tensor) -> np.ndarray:
@@ -1097,6 +1102,24 @@ def fused_mode(mode: str, device: int = 0) -> None:
 
 
 _encoded = {}  # (type, class of the number, number) -> its encoding (constant/3)
+
+_new_bytes = C.pythonapi.PyBytes_FromStringAndSize  # (NULL, n): a bytes object of n bytes whose content is the caller's to fill
+_new_bytes.restype, _new_bytes.argtypes = C.py_object, [C.c_char_p, C.c_ssize_t]
+_bytes_address = C.pythonapi.PyBytes_AsString
+_bytes_address.restype, _bytes_address.argtypes = C.c_void_p, [C.py_object]
+_libc = C.CDLL(None)
+_libc.madvise.restype, _libc.madvise.argtypes = C.c_int, [C.c_void_p, C.c_size_t, C.c_int]
+
+
+def _advise_huge_pages(address: int, n: int) -> None:
+    """A large, fresh destination is first touched by the copy: with 4 KiB pages the page faults cost more than the
+    transfer (256 MiB: 70 ms against 16 ms).  Asks for 2 MiB pages on the aligned interior, as numpy does for its
+    arrays; advice only, a kernel without transparent huge pages ignores it."""
+    if n >= 8 << 20:
+        huge = 2 << 20
+        lo, hi = (address + huge - 1) & ~(huge - 1), (address + n) & ~(huge - 1)
+        if hi > lo:
+            _libc.madvise(C.c_void_p(lo), hi - lo, 14)  # MADV_HUGEPAGE
 _fused_modes = {}  # device -> the mode last set here
 _fused_arrays = {}  # (id of a layout, input types) -> (the layout itself, so the id stays its own; C arrays of types and strides)
 

@@ -222,6 +222,10 @@ int hipnx_ctx_destroy(hipnx_ctx *ctx) {
   ctx->pool.clear();
   if (ctx->flag) (void)hipFree(ctx->flag);
   if (ctx->flag_host) (void)hipHostFree(ctx->flag_host);
+  for (int i = 0; i < 2; i++) {
+    if (ctx->stage[i]) (void)hipHostFree(ctx->stage[i]);
+    if (ctx->stage_ev[i]) (void)hipEventDestroy(ctx->stage_ev[i]);
+  }
   if (ctx->ev_start) (void)hipEventDestroy(ctx->ev_start);
   if (ctx->ev_stop) (void)hipEventDestroy(ctx->ev_stop);
   for (hipEvent_t m : ctx->marks)
@@ -483,6 +487,33 @@ void *hipnx_buf_device_ptr(const hipnx_buf *buf) {
   return buf->ptr;
 }
 
+// Host memory of callers is pageable (an Erlang binary, a numpy array).  The runtime's own path for it costs 35 us for
+// 64 KiB and delivers 17 GB/s device-to-host on large copies, against 10 us and 57 GB/s for pinned memory, so transfers
+// go through two pinned staging buffers of the context: the calling thread copies (30 GB/s) while the link fills or
+// drains the other buffer.
+static constexpr size_t STAGE_BYTES = 4u << 20;       // one staging buffer
+static constexpr size_t H2D_STAGED_MAX = 2u << 20;    // larger uploads: the runtime's path is as fast (one copy by the thread either way)
+static constexpr size_t H2D_CHUNK = 512u << 10;
+static constexpr size_t PINNED_CHECK_MIN = 256u << 10;  // from here on it pays to ask whether the host memory is pinned already
+
+static bool is_pinned(const void *p) {
+  hipPointerAttribute_t at;
+  const bool yes = hipPointerGetAttributes(&at, p) == hipSuccess && at.type == hipMemoryTypeHost;
+  (void)hipGetLastError();  // "not a registered pointer" is the expected answer
+  return yes;
+}
+
+// makes stage `i` exist and waits for the transfer that last used it
+static int stage_ready(hipnx_ctx *ctx, int i) {
+  if (!ctx->stage[i]) HIPNX_HIP(hipHostMalloc(&ctx->stage[i], STAGE_BYTES, hipHostMallocDefault));
+  if (!ctx->stage_ev[i]) HIPNX_HIP(hipEventCreateWithFlags(&ctx->stage_ev[i], hipEventDisableTiming));
+  if (ctx->stage_busy[i]) {
+    HIPNX_HIP(hipEventSynchronize(ctx->stage_ev[i]));
+    ctx->stage_busy[i] = false;
+  }
+  return HIPNX_OK;
+}
+
 int hipnx_h2d(hipnx_ctx *ctx, hipnx_buf *dst, size_t dst_offset, const void *src, size_t bytes) {
   Enter in(ctx);
   if (in.status) return in.status;
@@ -490,8 +521,22 @@ int hipnx_h2d(hipnx_ctx *ctx, hipnx_buf *dst, size_t dst_offset, const void *src
   HIPNX_NOT_CAPTURING(ctx, "h2d");
   if (bytes == 0) return HIPNX_OK;
   if (!src) return set_error(HIPNX_EINVAL, "h2d: null source");
+  if (bytes <= H2D_STAGED_MAX && !(bytes > PINNED_CHECK_MIN && is_pinned(src))) {
+    // the source (caller-owned: it must be consumed on return) is copied into a staging buffer, 512 KiB at a time, and
+    // the transfers out of it are left in flight: the call returns without waiting for the device
+    for (size_t done = 0; done < bytes; done += H2D_CHUNK) {
+      const size_t n = bytes - done < H2D_CHUNK ? bytes - done : H2D_CHUNK;
+      const int i = ctx->stage_next;
+      ctx->stage_next ^= 1;
+      if (int st = stage_ready(ctx, i)) return st;
+      std::memcpy(ctx->stage[i], (const char *)src + done, n);
+      HIPNX_HIP(hipMemcpyAsync((char *)dst->ptr + dst_offset + done, ctx->stage[i], n, hipMemcpyHostToDevice, ctx->stream));
+      HIPNX_HIP(hipEventRecord(ctx->stage_ev[i], ctx->stream));
+      ctx->stage_busy[i] = true;
+    }
+    return HIPNX_OK;
+  }
   HIPNX_HIP(hipMemcpyAsync((char *)dst->ptr + dst_offset, src, bytes, hipMemcpyHostToDevice, ctx->stream));
-  // the source is caller-owned host memory (an Erlang binary): it must be consumed on return
   HIPNX_HIP(hipStreamSynchronize(ctx->stream));
   return HIPNX_OK;
 }
@@ -506,8 +551,32 @@ int hipnx_d2h(hipnx_ctx *ctx, const hipnx_buf *src, size_t src_offset, void *dst
     return deferred_error(ctx);
   }
   if (!dst) return set_error(HIPNX_EINVAL, "d2h: null destination");
-  HIPNX_HIP(hipMemcpyAsync(dst, (const char *)src->ptr + src_offset, bytes, hipMemcpyDeviceToHost, ctx->stream));
-  HIPNX_HIP(hipStreamSynchronize(ctx->stream));
+  const char *from = (const char *)src->ptr + src_offset;
+  if (bytes > PINNED_CHECK_MIN && is_pinned(dst)) {  // a destination that is pinned already takes the transfer directly
+    HIPNX_HIP(hipMemcpyAsync(dst, from, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    HIPNX_HIP(hipStreamSynchronize(ctx->stream));
+    return deferred_error(ctx);
+  }
+  // up to 1 MiB in one piece (a piece costs ~15 us beside its bytes); beyond, quarters of the copy (512 KiB ... 4 MiB):
+  // piece k is on the link while piece k - 1 is copied out
+  size_t chunk = bytes;
+  if (bytes > (1u << 20)) {
+    chunk = bytes / 4;
+    chunk = chunk < (512u << 10) ? (512u << 10) : chunk > STAGE_BYTES ? STAGE_BYTES : (chunk + 4095) & ~(size_t)4095;
+  }
+  const size_t chunks = (bytes + chunk - 1) / chunk;
+  auto len = [&](size_t k) { return k + 1 < chunks ? chunk : bytes - k * chunk; };
+  for (size_t k = 0; k <= chunks; k++) {
+    if (k < chunks) {  // (chunk k - 2 has left this buffer in the pass before)
+      if (int st = stage_ready(ctx, (int)(k & 1))) return st;
+      HIPNX_HIP(hipMemcpyAsync(ctx->stage[k & 1], from + k * chunk, len(k), hipMemcpyDeviceToHost, ctx->stream));
+      HIPNX_HIP(hipEventRecord(ctx->stage_ev[k & 1], ctx->stream));
+    }
+    if (k >= 1) {
+      HIPNX_HIP(hipEventSynchronize(ctx->stage_ev[(k - 1) & 1]));
+      std::memcpy((char *)dst + (k - 1) * chunk, ctx->stage[(k - 1) & 1], len(k - 1));
+    }
+  }
   return deferred_error(ctx);  // the bytes have been delivered either way
 }
 

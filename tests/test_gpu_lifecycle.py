@@ -116,3 +116,30 @@ def test_memory_statistics_track_allocations(hip):
     assert mem_stats()["live"] >= before + 4 * 1024 * 1024
     Nx.backend_deallocate(t)
     assert mem_stats()["live"] == before
+
+
+@pytest.mark.parametrize("nbytes", [1, 4095, 256 << 10, (256 << 10) + 1, (512 << 10) + 7, 1 << 20, (1 << 20) + 1, (2 << 20) - 3,
+                                    (2 << 20) + 5, (4 << 20) + 1, (16 << 20) + 12289, (33 << 20) + 3])
+def test_host_transfers_of_every_staging_shape(nbytes, hip):
+    """Uploads and downloads go through the context's two pinned staging buffers in pieces (uploads up to 2 MiB, in flight
+    when the call returns; downloads of any size): sizes on and beside every piece boundary come back as they went,
+    through to_binary, into an array, at an offset through the C ABI, and after the source array has been overwritten."""
+    import ctypes as C
+    from nx_amd import _lib as L
+    rng = np.random.default_rng(nbytes)
+    a = rng.integers(0, 256, size=nbytes, dtype=np.uint8)
+    want = a.copy()
+    t = from_numpy(a, "u8", hip)
+    a[:] = 0  # the upload has consumed its source
+    assert Nx.to_binary(t) == want.tobytes()
+    assert np.array_equal(hip.to_numpy(t), want)
+    off = min(nbytes - 1, 4097)
+    part = np.empty(nbytes - off, dtype=np.uint8)
+    L.check(L.lib.hipnx_d2h(t.data.ref.ctx, hip._handle(t), off, part.ctypes.data_as(C.c_void_p), part.nbytes))
+    assert np.array_equal(part, want[off:])
+    # several small uploads in a row reuse the two buffers while earlier ones are still in flight
+    if nbytes <= 1 << 20:
+        parts = [rng.integers(0, 256, size=nbytes, dtype=np.uint8) for _ in range(5)]
+        tensors = [from_numpy(p, "u8", hip) for p in parts]
+        for p, x in zip(parts, tensors):
+            assert np.array_equal(hip.to_numpy(x), p)
