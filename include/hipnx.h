@@ -161,12 +161,13 @@ int hipnx_buf_wrap(hipnx_ctx *ctx, void *device_ptr, size_t bytes, hipnx_buf **o
 #define HIPNX_IPC_HANDLE_BYTES 64
 int hipnx_buf_ipc_export(hipnx_ctx *ctx, const hipnx_buf *buf, void *handle_out);
 int hipnx_buf_ipc_import(hipnx_ctx *ctx, const void *handle, size_t bytes, hipnx_buf **out);
-/* `src` is consumed on return (it may be an Erlang binary).  Up to 2 MiB the bytes are copied into pinned staging
- * buffers of the context and the transfer is left in flight on the stream, so the call does not wait for the device;
- * larger uploads (and uploads from memory that is pinned already) wait.  Later work on the context is ordered after the upload either way. */
+/* `src` is consumed on return (it may be an Erlang binary): the bytes are copied into pinned staging buffers of the
+ * context (from 32 MiB on by the calling thread and a helper thread, half each) and the transfers out of them are left
+ * in flight on the stream, so the call does not wait for the device.  Uploads from memory that is pinned already go
+ * straight over the link and wait.  Later work on the context is ordered after the upload either way. */
 int hipnx_h2d(hipnx_ctx *ctx, hipnx_buf *dst, size_t dst_offset, const void *src, size_t bytes);
-/* waits for all work enqueued so far, then copies: through the context's two pinned staging buffers (the link
- * fills one while the calling thread empties the other) unless `dst` is pinned memory itself */
+/* waits for all work enqueued so far, then copies: through the context's pinned staging buffers (the link fills one
+ * while a thread empties the other; from 32 MiB on two threads, half each) unless `dst` is pinned memory itself */
 int hipnx_d2h(hipnx_ctx *ctx, const hipnx_buf *src, size_t src_offset, void *dst, size_t bytes);
 int hipnx_d2d(hipnx_ctx *ctx, hipnx_buf *dst, size_t dst_offset, const hipnx_buf *src,
               size_t src_offset, size_t bytes);

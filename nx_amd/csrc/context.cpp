@@ -6,6 +6,8 @@
 // use-after-free that is an error, not a crash (exla/test/exla/backend_test.exs:48-50).
 #include <cstdlib>
 #include <cstring>
+#include <functional>
+#include <thread>
 
 #include "internal.h"
 
@@ -222,7 +224,7 @@ int hipnx_ctx_destroy(hipnx_ctx *ctx) {
   ctx->pool.clear();
   if (ctx->flag) (void)hipFree(ctx->flag);
   if (ctx->flag_host) (void)hipHostFree(ctx->flag_host);
-  for (int i = 0; i < 2; i++) {
+  for (int i = 0; i < 4; i++) {
     if (ctx->stage[i]) (void)hipHostFree(ctx->stage[i]);
     if (ctx->stage_ev[i]) (void)hipEventDestroy(ctx->stage_ev[i]);
   }
@@ -489,11 +491,11 @@ void *hipnx_buf_device_ptr(const hipnx_buf *buf) {
 
 // Host memory of callers is pageable (an Erlang binary, a numpy array).  The runtime's own path for it costs 35 us for
 // 64 KiB and delivers 17 GB/s device-to-host on large copies, against 10 us and 57 GB/s for pinned memory, so transfers
-// go through two pinned staging buffers of the context: the calling thread copies (30 GB/s) while the link fills or
-// drains the other buffer.
-static constexpr size_t STAGE_BYTES = 4u << 20;       // one staging buffer
-static constexpr size_t H2D_STAGED_MAX = 2u << 20;    // larger uploads: the runtime's path is as fast (one copy by the thread either way)
-static constexpr size_t H2D_CHUNK = 512u << 10;
+// go through pinned staging buffers of the context: a thread copies (28-30 GB/s) while the link fills or drains its
+// other buffer.  A lane is two buffers; copies of 32 MiB and more are halved between the calling thread on lane 0 and
+// a second thread on lane 1, since one thread's copy is what limits a lane.
+static constexpr size_t STAGE_BYTES = 4u << 20;        // one staging buffer
+static constexpr size_t TWO_LANES_MIN = 32u << 20;
 static constexpr size_t PINNED_CHECK_MIN = 256u << 10;  // from here on it pays to ask whether the host memory is pinned already
 
 static bool is_pinned(const void *p) {
@@ -503,15 +505,75 @@ static bool is_pinned(const void *p) {
   return yes;
 }
 
-// makes stage `i` exist and waits for the transfer that last used it
-static int stage_ready(hipnx_ctx *ctx, int i) {
-  if (!ctx->stage[i]) HIPNX_HIP(hipHostMalloc(&ctx->stage[i], STAGE_BYTES, hipHostMallocDefault));
-  if (!ctx->stage_ev[i]) HIPNX_HIP(hipEventCreateWithFlags(&ctx->stage_ev[i], hipEventDisableTiming));
+#define STAGE_TRY(call)               \
+  do {                                \
+    hipError_t e__ = (call);          \
+    if (e__ != hipSuccess) return e__; \
+  } while (0)
+
+// makes staging buffer `i` exist and waits for the transfer that last used it
+static hipError_t stage_ready(hipnx_ctx *ctx, int i) {
+  if (!ctx->stage[i]) STAGE_TRY(hipHostMalloc(&ctx->stage[i], STAGE_BYTES, hipHostMallocDefault));
+  if (!ctx->stage_ev[i]) STAGE_TRY(hipEventCreateWithFlags(&ctx->stage_ev[i], hipEventDisableTiming));
   if (ctx->stage_busy[i]) {
-    HIPNX_HIP(hipEventSynchronize(ctx->stage_ev[i]));
+    STAGE_TRY(hipEventSynchronize(ctx->stage_ev[i]));
     ctx->stage_busy[i] = false;
   }
-  return HIPNX_OK;
+  return hipSuccess;
+}
+
+// host -> device through lane `lane`, `chunk` bytes at a time; returns with the last transfers in flight
+static hipError_t upload_range(hipnx_ctx *ctx, int lane, char *dev, const char *src, size_t bytes, size_t chunk) {
+  STAGE_TRY(hipSetDevice(ctx->device));
+  for (size_t done = 0; done < bytes; done += chunk) {
+    const size_t n = bytes - done < chunk ? bytes - done : chunk;
+    const int i = 2 * lane + ctx->stage_next[lane];
+    ctx->stage_next[lane] ^= 1;
+    STAGE_TRY(stage_ready(ctx, i));
+    std::memcpy(ctx->stage[i], src + done, n);
+    STAGE_TRY(hipMemcpyAsync(dev + done, ctx->stage[i], n, hipMemcpyHostToDevice, ctx->stream));
+    STAGE_TRY(hipEventRecord(ctx->stage_ev[i], ctx->stream));
+    ctx->stage_busy[i] = true;
+  }
+  return hipSuccess;
+}
+
+// device -> host through lane `lane`: piece k is on the link while piece k - 1 is copied out
+static hipError_t download_range(hipnx_ctx *ctx, int lane, char *dst, const char *dev, size_t bytes, size_t chunk) {
+  STAGE_TRY(hipSetDevice(ctx->device));
+  const size_t chunks = (bytes + chunk - 1) / chunk;
+  auto len = [&](size_t k) { return k + 1 < chunks ? chunk : bytes - k * chunk; };
+  for (size_t k = 0; k <= chunks; k++) {
+    if (k < chunks) {  // (piece k - 2 has left this buffer in the pass before)
+      const int i = 2 * lane + (int)(k & 1);
+      STAGE_TRY(stage_ready(ctx, i));
+      STAGE_TRY(hipMemcpyAsync(ctx->stage[i], dev + k * chunk, len(k), hipMemcpyDeviceToHost, ctx->stream));
+      STAGE_TRY(hipEventRecord(ctx->stage_ev[i], ctx->stream));
+    }
+    if (k >= 1) {
+      const int i = 2 * lane + (int)((k - 1) & 1);
+      STAGE_TRY(hipEventSynchronize(ctx->stage_ev[i]));
+      std::memcpy(dst + (k - 1) * chunk, ctx->stage[i], len(k - 1));
+    }
+  }
+  return hipSuccess;
+}
+#undef STAGE_TRY
+
+// the two halves of a large copy on the two lanes; `half` is a multiple of the staging size
+// pieces of a copy on one lane: a quarter of it, 512 KiB ... 4 MiB (a piece costs ~15 us beside its bytes)
+static size_t piece_size(size_t bytes) {
+  const size_t q = (bytes / 4 + 4095) & ~(size_t)4095;
+  return q < (512u << 10) ? (512u << 10) : q > STAGE_BYTES ? STAGE_BYTES : q;
+}
+
+static hipError_t on_two_lanes(size_t bytes, const std::function<hipError_t(int, size_t, size_t)> &range) {
+  const size_t half = (bytes / 2 + STAGE_BYTES - 1) / STAGE_BYTES * STAGE_BYTES;
+  hipError_t second = hipSuccess;
+  std::thread helper([&] { second = range(1, half, bytes - half); });
+  const hipError_t first = range(0, (size_t)0, half);
+  helper.join();
+  return first != hipSuccess ? first : second;
 }
 
 int hipnx_h2d(hipnx_ctx *ctx, hipnx_buf *dst, size_t dst_offset, const void *src, size_t bytes) {
@@ -521,23 +583,21 @@ int hipnx_h2d(hipnx_ctx *ctx, hipnx_buf *dst, size_t dst_offset, const void *src
   HIPNX_NOT_CAPTURING(ctx, "h2d");
   if (bytes == 0) return HIPNX_OK;
   if (!src) return set_error(HIPNX_EINVAL, "h2d: null source");
-  if (bytes <= H2D_STAGED_MAX && !(bytes > PINNED_CHECK_MIN && is_pinned(src))) {
-    // the source (caller-owned: it must be consumed on return) is copied into a staging buffer, 512 KiB at a time, and
-    // the transfers out of it are left in flight: the call returns without waiting for the device
-    for (size_t done = 0; done < bytes; done += H2D_CHUNK) {
-      const size_t n = bytes - done < H2D_CHUNK ? bytes - done : H2D_CHUNK;
-      const int i = ctx->stage_next;
-      ctx->stage_next ^= 1;
-      if (int st = stage_ready(ctx, i)) return st;
-      std::memcpy(ctx->stage[i], (const char *)src + done, n);
-      HIPNX_HIP(hipMemcpyAsync((char *)dst->ptr + dst_offset + done, ctx->stage[i], n, hipMemcpyHostToDevice, ctx->stream));
-      HIPNX_HIP(hipEventRecord(ctx->stage_ev[i], ctx->stream));
-      ctx->stage_busy[i] = true;
-    }
+  char *to = (char *)dst->ptr + dst_offset;
+  if (bytes > PINNED_CHECK_MIN && is_pinned(src)) {  // pinned already: straight over the link
+    HIPNX_HIP(hipMemcpyAsync(to, src, bytes, hipMemcpyHostToDevice, ctx->stream));
+    HIPNX_HIP(hipStreamSynchronize(ctx->stream));
     return HIPNX_OK;
   }
-  HIPNX_HIP(hipMemcpyAsync((char *)dst->ptr + dst_offset, src, bytes, hipMemcpyHostToDevice, ctx->stream));
-  HIPNX_HIP(hipStreamSynchronize(ctx->stream));
+  // The source (caller-owned: it must be consumed on return) is copied into staging buffers and the transfers out
+  // of them are left in flight: the call returns without waiting for the device.
+  if (bytes >= TWO_LANES_MIN) {
+    HIPNX_HIP(on_two_lanes(bytes, [&](int lane, size_t at, size_t n) {
+      return upload_range(ctx, lane, to + at, (const char *)src + at, n, STAGE_BYTES);
+    }));
+    return HIPNX_OK;
+  }
+  HIPNX_HIP(upload_range(ctx, 0, to, (const char *)src, bytes, piece_size(bytes)));
   return HIPNX_OK;
 }
 
@@ -557,26 +617,13 @@ int hipnx_d2h(hipnx_ctx *ctx, const hipnx_buf *src, size_t src_offset, void *dst
     HIPNX_HIP(hipStreamSynchronize(ctx->stream));
     return deferred_error(ctx);
   }
-  // up to 1 MiB in one piece (a piece costs ~15 us beside its bytes); beyond, quarters of the copy (512 KiB ... 4 MiB):
-  // piece k is on the link while piece k - 1 is copied out
-  size_t chunk = bytes;
-  if (bytes > (1u << 20)) {
-    chunk = bytes / 4;
-    chunk = chunk < (512u << 10) ? (512u << 10) : chunk > STAGE_BYTES ? STAGE_BYTES : (chunk + 4095) & ~(size_t)4095;
+  if (bytes >= TWO_LANES_MIN) {
+    HIPNX_HIP(on_two_lanes(bytes, [&](int lane, size_t at, size_t n) {
+      return download_range(ctx, lane, (char *)dst + at, from + at, n, STAGE_BYTES);
+    }));
+    return deferred_error(ctx);
   }
-  const size_t chunks = (bytes + chunk - 1) / chunk;
-  auto len = [&](size_t k) { return k + 1 < chunks ? chunk : bytes - k * chunk; };
-  for (size_t k = 0; k <= chunks; k++) {
-    if (k < chunks) {  // (chunk k - 2 has left this buffer in the pass before)
-      if (int st = stage_ready(ctx, (int)(k & 1))) return st;
-      HIPNX_HIP(hipMemcpyAsync(ctx->stage[k & 1], from + k * chunk, len(k), hipMemcpyDeviceToHost, ctx->stream));
-      HIPNX_HIP(hipEventRecord(ctx->stage_ev[k & 1], ctx->stream));
-    }
-    if (k >= 1) {
-      HIPNX_HIP(hipEventSynchronize(ctx->stage_ev[(k - 1) & 1]));
-      std::memcpy((char *)dst + (k - 1) * chunk, ctx->stage[(k - 1) & 1], len(k - 1));
-    }
-  }
+  HIPNX_HIP(download_range(ctx, 0, (char *)dst, from, bytes, bytes <= (1u << 20) ? bytes : piece_size(bytes)));
   return deferred_error(ctx);  // the bytes have been delivered either way
 }
 

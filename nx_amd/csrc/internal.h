@@ -42,13 +42,13 @@ struct hipnx_ctx {
   void *flag = nullptr;       // 32-byte device scratch for the gather bounds report
   void *flag_host = nullptr;  // pinned host word, mapped into the device: non-zero once a kernel saw a bad index
   void *flag_host_dev = nullptr;  // its device address
-  // two pinned staging buffers for host transfers (created on first use): the link fills or drains one while the
-  // calling thread copies the other; `stage_busy[i]`: an upload out of buffer i may still be in flight (its end is
-  // `stage_ev[i]`)
-  void *stage[2] = {nullptr, nullptr};
-  hipEvent_t stage_ev[2] = {nullptr, nullptr};
-  bool stage_busy[2] = {false, false};
-  int stage_next = 0;
+  // pinned staging buffers for host transfers (created on first use), two per lane: the link fills or drains one while
+  // a thread copies the other; large copies run on both lanes (buffers 0-1: the calling thread, 2-3: a helper thread).
+  // `stage_busy[i]`: an upload out of buffer i may still be in flight (its end is `stage_ev[i]`)
+  void *stage[4] = {nullptr, nullptr, nullptr, nullptr};
+  hipEvent_t stage_ev[4] = {nullptr, nullptr, nullptr, nullptr};
+  bool stage_busy[4] = {false, false, false, false};
+  int stage_next[2] = {0, 0};  // per lane: the buffer its next upload piece takes
   void *reduce_scratch = nullptr;  // this device's address of the static partial-result array of reduce.hip
   hipnx_graph *capture = nullptr;                        // non-null while the stream is capturing
   std::unordered_map<void *, hipnx_graph *> graph_blocks;  // block -> the live graph that owns it
