@@ -36,6 +36,37 @@ CEILINGS_BIN = os.path.join(ROOT, "nx_amd", "lib", "hipnx_ceilings")
 ABI_DRIVER_BIN = os.path.join(ROOT, "nx_amd", "lib", "hipnx_abi_driver")
 
 
+def host_transfer_figures(H, B, Nx, template):
+    """from_binary / to_binary through the host link (pageable host memory, as a caller has it): never part of
+    `value`, reported so that the PCIe-inclusive cost of a round trip is on record."""
+    import ctypes
+    from nx_amd import _lib as L
+    out = {"note": "pageable host memory; uploads return once the source is consumed, downloads wait for the device"}
+    for label, nbytes in (("64KiB", 64 << 10), ("256MiB", 256 << 20)):
+        host = np.random.default_rng(3).integers(0, 256, size=nbytes, dtype=np.uint8)
+        dev = H.from_numpy(template("u8", host.shape), host)
+        back = np.zeros(nbytes, dtype=np.uint8)
+        B.sync()
+        up, down, binary = [], [], []
+        for _ in range(5):
+            t0 = time.perf_counter()
+            dev = H.from_numpy(template("u8", host.shape), host)
+            B.sync()
+            up.append(time.perf_counter() - t0)
+            t0 = time.perf_counter()
+            L.check(L.lib.hipnx_d2h(dev.data.ref.ctx, H._handle(dev), 0, back.ctypes.data_as(ctypes.c_void_p), nbytes))
+            down.append(time.perf_counter() - t0)
+            t0 = time.perf_counter()
+            raw = Nx.to_binary(dev)
+            binary.append(time.perf_counter() - t0)
+            del raw
+        assert np.array_equal(back, host)
+        out[label] = {"from_binary_us": round(min(up) * 1e6, 1), "from_binary_GBps": round(nbytes / min(up) / 1e9, 2),
+                      "d2h_into_touched_memory_us": round(min(down) * 1e6, 1), "d2h_GBps": round(nbytes / min(down) / 1e9, 2),
+                      "to_binary_us": round(min(binary) * 1e6, 1), "to_binary_GBps": round(nbytes / min(binary) / 1e9, 2)}
+    return out
+
+
 def c_abi_figures():
     """Configuration 1's callbacks and `take` issued from plain C through libhipnx.so (what a NIF would
     see): host microseconds per call and per chain, without Python or ctypes in the path."""
@@ -544,6 +575,7 @@ def main():
         del big, x, y
         del cases, q, k
         result["suite"] = suite
+        result["host_transfers"] = host_transfer_figures(H, B, Nx, template)
         c_abi = c_abi_figures()
         if c_abi:
             result["c_abi"] = c_abi
