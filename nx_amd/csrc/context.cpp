@@ -7,6 +7,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <functional>
+#include <system_error>
 #include <thread>
 
 #include "internal.h"
@@ -570,7 +571,13 @@ static size_t piece_size(size_t bytes) {
 static hipError_t on_two_lanes(size_t bytes, const std::function<hipError_t(int, size_t, size_t)> &range) {
   const size_t half = (bytes / 2 + STAGE_BYTES - 1) / STAGE_BYTES * STAGE_BYTES;
   hipError_t second = hipSuccess;
-  std::thread helper([&] { second = range(1, half, bytes - half); });
+  std::thread helper;
+  try {
+    helper = std::thread([&] { second = range(1, half, bytes - half); });
+  } catch (const std::system_error &) {  // no thread to be had: the calling thread does both halves
+    const hipError_t first = range(0, (size_t)0, half);
+    return first != hipSuccess ? first : range(0, half, bytes - half);
+  }
   const hipError_t first = range(0, (size_t)0, half);
   helper.join();
   return first != hipSuccess ? first : second;
