@@ -249,7 +249,7 @@ static int grid_for(const hipnx_ctx *ctx, int64_t work_items) {
   // one 8-element vector per lane: on this part a grid that covers the whole tensor streams
   // faster than a resident grid looping over it (5.8 vs 5.1 TB/s on a 1 GiB add)
   (void)ctx;
-  int64_t cap = 1ll << 30;
+  int64_t cap = ((1ll << 32) - 1) / BLOCK;  // a launch may hold at most 2^32 - 1 lanes: the kernels loop over the rest
   if (blocks < 1) blocks = 1;
   return (int)(blocks < cap ? blocks : cap);
 }

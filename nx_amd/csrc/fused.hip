@@ -347,13 +347,20 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
     int64_t grid = n_stats ? (block_per_row ? a.rows : (a.rows + FBLOCK / WAVE - 1) / (FBLOCK / WAVE))  // a wave or a block per row
                    : reduce_op == -1 ? (a.nvec + (int64_t)FBLOCK * FV - 1) / ((int64_t)FBLOCK * FV)
                    : block_per_row ? a.rows : (a.rows + FBLOCK / WAVE - 1) / (FBLOCK / WAVE);
-    if (grid > (1ll << 30)) grid = 1ll << 30;
+    // a launch may hold at most 2^32 - 1 lanes: the element-wise kernel loops over what a capped grid leaves, the row
+    // kernels take one row (or wave of rows) per work-group and leave larger inputs to the separate callbacks
+    const int64_t max_grid = ((1ll << 32) - 1) / FBLOCK;
+    if (grid > max_grid) {
+      if (n_stats || reduce_op != -1) return set_error(HIPNX_EUNSUPPORTED, "fused: more rows than one launch holds");
+      grid = max_grid;
+    }
     bool done = false;
     if (int st = fused_launch_compiled(ctx, a, reduce_op, block_per_row, (unsigned)grid, &done)) return st;
     if (done) return HIPNX_OK;
   }
   if (needs_compiled || (full && reduce_op != -1))
     return set_error(HIPNX_EUNSUPPORTED, "fused: a program that exists only compiled, first met while capturing");
+  if (reduce_op != -1 && a.rows > ((1ll << 32) - 1) / FBLOCK) return set_error(HIPNX_EUNSUPPORTED, "fused: more rows than one launch holds");
   if (reduce_op == HIPNX_RED_SUM) launch_fused_reduce<PlainReducer<double, HIPNX_RED_SUM, false>, double>(ctx, a);
   else if (reduce_op == HIPNX_RED_MAX) launch_fused_reduce<PlainReducer<float, HIPNX_RED_MAX, false>, float>(ctx, a);
   else if (reduce_op == HIPNX_RED_MIN) launch_fused_reduce<PlainReducer<float, HIPNX_RED_MIN, false>, float>(ctx, a);
@@ -362,7 +369,7 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
     return HIPNX_OK;
   }
   int64_t blocks = (a.nvec + (int64_t)FBLOCK * FV - 1) / ((int64_t)FBLOCK * FV);
-  if (blocks > (1ll << 30)) blocks = 1ll << 30;
+  if (blocks > ((1ll << 32) - 1) / FBLOCK) blocks = ((1ll << 32) - 1) / FBLOCK;
   if (full) hipLaunchKernelGGL((fused_elementwise_kernel<true>), dim3((unsigned)blocks), dim3(FBLOCK), 0, ctx->stream, a);
   else hipLaunchKernelGGL((fused_elementwise_kernel<false>), dim3((unsigned)blocks), dim3(FBLOCK), 0, ctx->stream, a);
   HIPNX_HIP(hipGetLastError());

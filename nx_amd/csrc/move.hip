@@ -391,7 +391,7 @@ __global__ void __launch_bounds__(BLOCK) fill16_kernel(uint4 *__restrict__ out, 
 static int grid_for(const hipnx_ctx *ctx, int64_t items, int per_block) {
   int64_t blocks = (items + per_block - 1) / per_block;
   (void)ctx;
-  int64_t cap = 1ll << 30;  // cover the whole index space: faster here than a resident grid that loops
+  int64_t cap = ((1ll << 32) - 1) / BLOCK;  // cover the whole index space (faster here than a resident grid that loops) up to the 2^32 - 1 lanes a launch may hold
   if (blocks < 1) blocks = 1;
   return (int)(blocks < cap ? blocks : cap);
 }

@@ -75,7 +75,7 @@ extern "C" int hipnx_threefry2x32(hipnx_ctx *ctx, const hipnx_buf *key, int64_t 
   const int64_t half = (n + 1) / 2;
   const int64_t per_block = (int64_t)RBLOCK * RPAIRS;
   int64_t blocks = (half + per_block - 1) / per_block;
-  if (blocks > (1ll << 30)) blocks = 1ll << 30;
+  if (blocks > ((1ll << 32) - 1) / RBLOCK) blocks = ((1ll << 32) - 1) / RBLOCK;  // a launch may hold at most 2^32 - 1 lanes
   hipLaunchKernelGGL(threefry2x32_kernel, dim3((unsigned)blocks), dim3(RBLOCK), 0, ctx->stream,
                      (const uint32_t *)key->ptr, (uint32_t *)out->ptr, n, half, (int)(half % RPAIRS == 0 && (uintptr_t)out->ptr % 16 == 0));
   HIPNX_HIP(hipGetLastError());

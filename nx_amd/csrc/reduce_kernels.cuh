@@ -39,7 +39,9 @@ reduce_rows_kernel(const void *__restrict__ in, void *__restrict__ out, typename
   const int idt = IDT >= 0 ? IDT : idt_;
   constexpr int RPB = BLOCK / TPR;
   const int sub = threadIdx.x / TPR, lane = threadIdx.x % TPR;
-  const int64_t unit = (int64_t)blockIdx.x * RPB + sub;  // (row, seg) pair
+  // (the grid is capped: a launch may not hold 2^32 lanes, and rows * nseg has no such bound)
+  for (int64_t first = (int64_t)blockIdx.x * RPB; first < rows * nseg; first += (int64_t)gridDim.x * RPB) {
+  const int64_t unit = first + sub;  // (row, seg) pair
   const int64_t row = unit / nseg;
   const int seg = (int)(unit - row * nseg);
   typename R::acc_t acc = R::init();
@@ -81,10 +83,36 @@ reduce_rows_kernel(const void *__restrict__ in, void *__restrict__ out, typename
 #pragma unroll
       for (int w = 1; w < BLOCK / WAVE; w++) acc = R::combine(acc, sm[w]);
     }
+    __syncthreads();  // before the next pass writes sm again
   }
   if (lane == 0 && row < rows) {
     if (nseg == 1) finalize(out, odt, row, acc);
     else partial[row * nseg + seg] = acc;
+  }
+  }
+}
+
+// rows of up to 16 elements: one lane per row, walking it in order.  A group of 8 lanes (the narrowest above) would
+// leave most of its lanes without an element (f32 rows of 8: 1.3 TB/s; rows of 2, which are not whole vectors and took
+// a wave each: 0.06 TB/s).  Adjacent lanes read adjacent rows, so a wave's loads stay within `red` neighbouring lines.
+template <typename R, typename CT, int IDT = -1>
+__global__ void __launch_bounds__(BLOCK)
+reduce_rows_short_kernel(const void *__restrict__ in, void *__restrict__ out, int idt_, int odt, int64_t rows, int red) {
+  const int idt = IDT >= 0 ? IDT : idt_;
+  for (int64_t row = (int64_t)blockIdx.x * BLOCK + threadIdx.x; row < rows; row += (int64_t)gridDim.x * BLOCK) {
+    typename R::acc_t acc = red > 0 ? R::seed(R::init(), 0) : R::init();
+    const int64_t base = row * red;
+    if (red % E == 0) {  // whole vectors (rows of 8 or 16 elements)
+      for (int k = 0; k < red; k += E) {
+        CT v[E];
+        load_vec<CT, E>(in, idt, base + k, v);
+#pragma unroll
+        for (int i = 0; i < E; i++) acc = R::accumulate(acc, v[i], k + i);
+      }
+    } else {
+      for (int k = 0; k < red; k++) acc = R::accumulate(acc, load_one<CT>(in, idt, base + k), k);
+    }
+    finalize(out, odt, row, acc);
   }
 }
 
@@ -195,6 +223,9 @@ combine_cols_kernel(const typename R::acc_t *__restrict__ partial, void *__restr
 
 static int64_t round_up(int64_t a, int64_t b) { return (a + b - 1) / b * b; }
 
+// a launch may hold at most 2^32 - 1 lanes along x: the kernels loop over what a capped grid leaves
+constexpr int64_t MAX_BLOCKS = ((1ll << 32) - 1) / BLOCK;
+
 // Partial results of a split reduction live either in a block of the context's pool (handed back
 // right after the launches: later work on this stream is ordered behind them) or, for the entry
 // point that allocates nothing, in this file's static device array.
@@ -246,10 +277,23 @@ static int run_reduce_t(hipnx_ctx *ctx, bool static_ws, int idt, int odt, int64_
     // up to 64 / 128 / 256 elements take 8 / 16 / 32 lanes, eight to two rows per wave, with the same bits.
     // (compiled for the common element types only: IDT >= 0)
     if (IDT >= 0 && vec && nseg == 1 && red <= 32 * E) tpr = red <= 8 * E ? 8 : red <= 16 * E ? 16 : 32;
+    // rows that are not whole vectors are read element by element, a lane group per row: 8 / 16 / 32 lanes for up to
+    // 64 / 128 / 256 elements instead of a wave (f32 rows of 33: 0.6 TB/s with a wave per row)
+    const bool narrow_scalar = !vec && nseg == 1 && red <= 256;
+    if (narrow_scalar) tpr = red <= 64 ? 8 : red <= 128 ? 16 : 32;
     const int rpb = BLOCK / tpr;
-    dim3 grid((unsigned)((rows * nseg + rpb - 1) / rpb)), block(BLOCK);
-    if (rows * nseg > 0) {
-      if (tpr < WAVE) {
+    const int64_t blocks = (rows * nseg + rpb - 1) / rpb;
+    dim3 grid((unsigned)(blocks < MAX_BLOCKS ? blocks : MAX_BLOCKS)), block(BLOCK);
+    if (rows * nseg > 0 && red <= 16) {
+      const int64_t b1 = (rows + BLOCK - 1) / BLOCK;
+      hipLaunchKernelGGL((reduce_rows_short_kernel<R, CT, IDT>), dim3((unsigned)(b1 < MAX_BLOCKS ? b1 : MAX_BLOCKS)), block, 0, ctx->stream, in, out,
+                         idt, odt, rows, (int)red);
+    } else if (rows * nseg > 0) {
+      if (narrow_scalar) {
+        if (tpr == 8) hipLaunchKernelGGL((reduce_rows_kernel<R, CT, 8, false>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
+        else if (tpr == 16) hipLaunchKernelGGL((reduce_rows_kernel<R, CT, 16, false>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
+        else hipLaunchKernelGGL((reduce_rows_kernel<R, CT, 32, false>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
+      } else if (tpr < WAVE) {
         if constexpr (IDT >= 0) {
           if (tpr == 8) hipLaunchKernelGGL((reduce_rows_kernel<R, CT, 8, true, IDT>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
           else if (tpr == 16) hipLaunchKernelGGL((reduce_rows_kernel<R, CT, 16, true, IDT>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
@@ -263,7 +307,7 @@ static int run_reduce_t(hipnx_ctx *ctx, bool static_ws, int idt, int odt, int64_
         else hipLaunchKernelGGL((reduce_rows_kernel<R, CT, BLOCK, false>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
       }
       if (nseg > 1) {
-        dim3 g2((unsigned)((rows + BLOCK / WAVE - 1) / (BLOCK / WAVE)));
+        dim3 g2((unsigned)((rows + BLOCK / WAVE - 1) / (BLOCK / WAVE)));  // (rows < 8 * CUs here)
         hipLaunchKernelGGL((combine_partials_kernel<R>), g2, block, 0, ctx->stream, partial, out, odt, rows, nseg);
       }
     }
@@ -297,7 +341,7 @@ static int run_reduce_t(hipnx_ctx *ctx, bool static_ws, int idt, int odt, int64_
     }
     int64_t total = lanes * nseg;
     int64_t blocks = (total + BLOCK - 1) / BLOCK;
-    int64_t cap = 1ll << 30;
+    const int64_t cap = MAX_BLOCKS;
     dim3 grid((unsigned)(blocks < 1 ? 1 : (blocks < cap ? blocks : cap))), block(BLOCK);
     if (total > 0) {
       if (vec) hipLaunchKernelGGL((reduce_cols_kernel<R, CT, true, IDT>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, outer, red, inner, seg_len, nseg);

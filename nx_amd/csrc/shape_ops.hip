@@ -18,7 +18,8 @@ static bool narrow_float(int dt) { return dt == HIPNX_BF16 || dt == HIPNX_F16 ||
 static int grid_for(int64_t items) {
   int64_t blocks = (items + BLOCK - 1) / BLOCK;
   if (blocks < 1) blocks = 1;
-  return (int)(blocks < (1ll << 30) ? blocks : (1ll << 30));
+  const int64_t cap = ((1ll << 32) - 1) / BLOCK;  // a launch may hold at most 2^32 - 1 lanes: the kernels loop over the rest
+  return (int)(blocks < cap ? blocks : cap);
 }
 
 // ---- select ---------------------------------------------------------------------------------

@@ -181,3 +181,50 @@ def test_reduced_axes_that_are_not_neighbours(shape, axes, ty, op, hip, oracle):
             assert np.allclose(g, w, rtol=eps + k * 2.0 ** -50, atol=(k * 2.0 ** -24 * np.abs(values(ox)).sum(axis=tuple(axes), keepdims=keep)) if op == "sum" else 0), f"{op} {ty} {shape} {axes}"
         else:
             assert_bits_equal(got, want, f"{op} {ty} {shape} {axes} keep={keep}")
+
+
+FEW = [((5000, c), 1) for c in (1, 2, 3, 5, 8, 13, 16, 17, 33, 100, 255)] + \
+      [((8192, 3), 0), ((12288, 2), 0), ((3, 4096, 7), 1), ((20000, 33), 0), ((2, 8190, 5), 1), ((4099, 3), 0), ((65536, 1, 2), 0)]
+
+
+@pytest.mark.parametrize("shape,axis", FEW, ids=[f"{s}-{a}" for s, a in FEW])
+@pytest.mark.parametrize("ty", ["f32", "bf16", "s32", "u8", "f64"])
+@pytest.mark.parametrize("op", ["sum", "product", "reduce_max", "reduce_min", "argmax", "argmin", "all", "any"])
+def test_few_elements_per_row_and_few_columns(shape, axis, ty, op, hip, oracle):
+    """Rows of up to 16 elements are walked by one lane each, unaligned rows of up to 256 by 8 to 32 lanes, and a few
+    columns under a long axis are reduced in two steps (a divisor of the axis folded into the columns first, sums and
+    products through f64 / 64-bit integers): integers, selections and indices bit for bit (NaN and signed zeros
+    included), float sums and products within the accumulation bound."""
+    rng = np.random.default_rng(seed_of(shape, axis, ty, op, "few"))
+    floating = ty in ("f32", "bf16", "f64")
+    if op == "product":
+        x = rand_raw(rng, ty, shape, lo=0.999, hi=1.001) if floating else rng.integers(1, 3, size=shape).astype(T.numpy_dtype(T.normalize(ty)))
+    elif op in ("all", "any"):
+        x = (rng.random(shape) < (0.9997 if op == "all" else 0.0003)).astype(np.float64)
+        x = (x.astype(np.float32).view(np.uint32) >> 16).astype(np.uint16) if ty == "bf16" else x.astype(T.numpy_dtype(T.normalize(ty)))
+    else:
+        x = rand_raw(rng, ty, shape, lo=-3, hi=3)
+        if ty == "f32":
+            flat = x.reshape(-1)
+            flat[rng.integers(0, flat.size, 40)] = 0.0
+            flat[rng.integers(0, flat.size, 40)] = -0.0
+            if op != "sum":
+                flat[rng.integers(0, flat.size, 5)] = np.nan
+    hx, ox = both(x, ty, hip, oracle)
+    if op in ("argmax", "argmin"):
+        for tie in ("low", "high"):
+            assert_bits_equal(getattr(Nx, op)(hx, axis=axis, tie_break=tie), getattr(Nx, op)(ox, axis=axis, tie_break=tie), f"{op} {ty} {shape}")
+        return
+    got, want = getattr(Nx, op)(hx, axes=[axis]), getattr(Nx, op)(ox, axes=[axis])
+    if op in ("sum", "product") and floating:
+        assert got.type == want.type and got.shape == want.shape
+        k = shape[axis]
+        eps = {"f64": 2.0 ** -52, "f32": 2.0 ** -23, "bf16": 2.0 ** -7}[ty]
+        atol = k * 2.0 ** -24 * np.abs(values(ox)).sum(axis=axis) if op == "sum" else 0
+        assert np.allclose(values(got), values(want), rtol=eps + k * 2.0 ** -50, atol=atol), f"{op} {ty} {shape} axis {axis}"
+    elif op in ("reduce_max", "reduce_min") and ty == "f32":
+        # equal extremes of both signs of zero: the device may keep the other zero (selected by value)
+        g, w = values(got), values(want)
+        assert np.array_equal(np.isnan(g), np.isnan(w)) and np.array_equal(g[~np.isnan(g)], w[~np.isnan(w)]), f"{op} {shape}"
+    else:
+        assert_bits_equal(got, want, f"{op} {ty} {shape} axis {axis}")
