@@ -41,7 +41,9 @@ static FastDiv32 make_fastdiv(uint32_t d) {
 }
 __device__ __forceinline__ uint32_t fastdiv(uint32_t n, FastDiv32 f) { return (__umulhi(n, f.mul) + n) >> f.shr; }
 
-enum { ROWS_ONE = 0, ROWS_FAST = 1, ROWS_WIDE = 2 };  // how a vector index splits into (row, column)
+// how a vector index splits into (row, column); the FLAT modes cut the flat output into vectors that may run across
+// row ends (rows whose length is not a whole number of vectors) and count `vecs_per_row` as the element count
+enum { ROWS_ONE = 0, ROWS_FAST = 1, ROWS_WIDE = 2, ROWS_FLAT = 3, ROWS_FLAT_WIDE = 4 };
 
 // Rows that are themselves two or three collapsed axes with their own strides per operand (a mask [b, 1, 1, s]
 // against scores [b, h, s, s] collapses to [b, h * s | s]: the mask's row offset is b's index times s, not a
@@ -68,6 +70,49 @@ binary_vec_kernel(const void *__restrict__ l, const void *__restrict__ r, void *
   const int ldt = FIX >= 0 ? FIX : ldt_, rdt = FIX >= 0 ? FIX : rdt_, odt = FIX >= 0 ? FIXO : odt_;
   for (int64_t v = (int64_t)blockIdx.x * BLOCK + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * BLOCK) {
     int64_t row, col;
+    if (rows_mode >= ROWS_FLAT) {
+      // [rows, cols] with cols not a whole number of vectors (x[N, 3] * w[3], x[N, 5] + b[N, 1]): a lane takes E
+      // consecutive outputs anyway -- an operand as dense as the output is one vector load, a broadcast one is read
+      // element by element (from a row or a column that the cache holds) -- instead of one output per lane with
+      // its index divisions (1.5 TB/s whatever the element type)
+      const int64_t total = vecs_per_row, f0 = v * E;
+      if (rows_mode == ROWS_FLAT) {
+        const uint32_t q = fastdiv((uint32_t)f0, fd);
+        row = q;
+        col = (int64_t)((uint32_t)f0 - q * (uint32_t)cols);
+      } else {
+        row = f0 / cols;
+        col = f0 - row * cols;
+      }
+      const int nel = f0 + E <= total ? E : (int)(total - f0);
+      const bool l_dense = ls1 == 1 && ls0 == cols && nel == E, r_dense = rs1 == 1 && rs0 == cols && nel == E;
+      CT a[E], b[E], c[E];
+      if (l_dense) load_vec<CT, E>(l, ldt, f0, a);
+      if (r_dense) load_vec<CT, E>(r, rdt, f0, b);
+#pragma unroll
+      for (int i = 0; i < E; i++) {
+        if (i < nel) {
+          if (!l_dense) a[i] = load_one<CT>(l, ldt, row * ls0 + col * ls1);
+          if (!r_dense) b[i] = load_one<CT>(r, rdt, row * rs0 + col * rs1);
+        } else {
+          a[i] = (CT)1;
+          b[i] = (CT)1;
+        }
+        if (++col == cols) { col = 0; row++; }
+      }
+#pragma unroll
+      for (int i = 0; i < E; i++) c[i] = binary_apply<OP, CT, UNS>(a[i], b[i]);
+      if constexpr (RAISES) {
+        long long operand = 0;
+#pragma unroll
+        for (int i = 0; i < E; i++)
+          if (int code = binary_raises<OP, CT, UNS>(a[i], b[i], &operand)) report_raise(err, code, operand);
+      }
+      if (nel == E) store_vec<CT, E>(out, odt, f0, c);
+      else
+        for (int i = 0; i < nel; i++) store_one<CT>(out, odt, f0 + i, c[i]);
+      continue;
+    }
     if (rows_mode == ROWS_ONE) {
       row = 0;
       col = v * E;
@@ -262,6 +307,7 @@ struct BinArgs {
   int ls1, rs1;
   unsigned long long *err;  // the context's deferred error word (device address of the pinned host word)
   RowAxes ax;
+  int64_t flat_total;  // > 0: the FLAT modes over this many outputs (rows * cols)
 };
 
 template <int OP, typename CT, bool UNS, int FIX, int FIXO = FIX>
@@ -273,8 +319,14 @@ static void launch_bvec_fix(const hipnx_ctx *ctx, const BinArgs &a_) {
     a.vecs_per_row = (a.cols + EV - 1) / EV;
     a.nvec = rows * a.vecs_per_row;
   }
-  const int mode = a.vecs_per_row >= a.nvec ? ROWS_ONE : a.nvec < (1ll << 31) ? ROWS_FAST : ROWS_WIDE;
-  const FastDiv32 fd = mode == ROWS_FAST ? make_fastdiv((uint32_t)a.vecs_per_row) : FastDiv32{0, 0};
+  int mode = a.vecs_per_row >= a.nvec ? ROWS_ONE : a.nvec < (1ll << 31) ? ROWS_FAST : ROWS_WIDE;
+  FastDiv32 fd = mode == ROWS_FAST ? make_fastdiv((uint32_t)a.vecs_per_row) : FastDiv32{0, 0};
+  if (a.flat_total > 0) {
+    a.vecs_per_row = a.flat_total;
+    a.nvec = (a.flat_total + EV - 1) / EV;
+    mode = a.flat_total < (1ll << 31) ? ROWS_FLAT : ROWS_FLAT_WIDE;
+    if (mode == ROWS_FLAT) fd = make_fastdiv((uint32_t)a.cols);
+  }
   hipLaunchKernelGGL((binary_vec_kernel<OP, CT, UNS, FIX, FIXO>), dim3(grid_for(ctx, a.nvec)), dim3(BLOCK), 0, ctx->stream, a.l,
                      a.r, a.out, a.ldt, a.rdt, a.odt, a.cols, a.vecs_per_row, a.nvec, a.ls0, a.ls1, a.rs0, a.rs1, a.err,
                      mode, fd, a.ax);
@@ -441,6 +493,16 @@ extern "C" int hipnx_binary(hipnx_ctx *ctx, int op, int l_dt, int r_dt, int out_
       a.nvec = rows * a.vecs_per_row;
       a.ls0 = l0; a.rs0 = r0; a.ls1 = (int)l1; a.rs1 = (int)r1;
       a.err = deferred_error_word(ctx);
+    } else if (m == 2 && (l1 == 0 || l1 == 1) && (r1 == 0 || r1 == 1) && cols < (1ll << 31)) {
+      // rows that are not whole vectors: vectors of the flat output
+      vec_ok = true;
+      a.l = l->ptr; a.r = r->ptr; a.out = out->ptr;
+      a.ldt = l_dt; a.rdt = r_dt; a.odt = out_dt;
+      a.cols = cols;
+      a.vecs_per_row = 1; a.nvec = 1;  // (set by the launcher from flat_total)
+      a.ls0 = l0; a.rs0 = r0; a.ls1 = (int)l1; a.rs1 = (int)r1;
+      a.err = deferred_error_word(ctx);
+      a.flat_total = n;
     }
   }
   if (vec_ok) {

@@ -250,3 +250,29 @@ def test_broadcasts_over_separated_axes(ls, rs, ty, op, hip, oracle):
     f = getattr(Nx, op)
     assert_bits_equal(f(ha, hb), f(oa, ob), f"{op} {ty} {ls} {rs}")
     assert_bits_equal(f(hb, ha), f(ob, oa), f"{op} {ty} {rs} {ls}")
+
+
+RAGGED = [((301, c), (c,)) for c in (2, 3, 5, 7, 12, 17, 33, 100)] + [((301, c), (301, 1)) for c in (2, 3, 7, 33)] + \
+         [((1, 13), (77, 1)), ((4, 25, 3), (3,)), ((9, 10, 5), (9, 10, 1)), ((2, 3), (3,))]
+
+
+@pytest.mark.parametrize("ls,rs", RAGGED, ids=[f"{a}-{b}" for a, b in RAGGED])
+@pytest.mark.parametrize("ty", ["f32", "bf16", "s32", "u8", "f64", "s64"])
+@pytest.mark.parametrize("op", ["add", "multiply", "less", "max", "quotient"])
+def test_rows_that_are_not_whole_vectors(ls, rs, ty, op, hip, oracle):
+    """x[N, 3] * w[3], x[N, 5] + b[N, 1], a column against a row: rows whose length is not a whole number of vectors are
+    cut into vectors of the flat output (vectors run across row ends, the last one is partial).  Both operand orders,
+    bit for bit; an integer quotient by non-zero divisors reports nothing for the lanes beyond the end."""
+    rng = np.random.default_rng(seed_of(ls, rs, ty, op, "ragged"))
+    a, b = rand_raw(rng, ty, ls, lo=1, hi=9), rand_raw(rng, ty, rs, lo=1, hi=9)
+    if op == "quotient":
+        if ty in ("f32", "bf16", "f64"):
+            pytest.skip("quotient is an integer operation")
+        a, b = np.where(a == 0, 1, a).astype(a.dtype), np.where(b == 0, 1, b).astype(b.dtype)
+    ha, oa = both(a, ty, hip, oracle)
+    hb, ob = both(b, ty, hip, oracle)
+    f = getattr(Nx, op)
+    assert_bits_equal(f(ha, hb), f(oa, ob), f"{op} {ty} {ls} {rs}")
+    assert_bits_equal(f(hb, ha), f(ob, oa), f"{op} {ty} {rs} {ls}")
+    from nx_amd import backend as B
+    B.sync()  # nothing was recorded for a later wait to raise
