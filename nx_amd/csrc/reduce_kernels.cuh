@@ -69,9 +69,37 @@ reduce_rows_kernel(const void *__restrict__ in, void *__restrict__ out, typename
 #pragma unroll
         for (int i = 0; i < E; i++) acc = R::accumulate(acc, v[i], k + i);
       }
-    } else {
+    } else if constexpr (TPR < WAVE) {
       if (k0 + lane < k1) acc = R::seed(acc, k0 + lane);
       for (int64_t k = k0 + lane; k < k1; k += TPR) acc = R::accumulate(acc, load_one<CT>(in, idt, base + k), k);
+    } else {
+      // a row that is not whole vectors (a vocabulary of 50257 entries): its first elements up to a vector boundary of
+      // the BUFFER one per lane, then whole aligned vectors, then the last few elements one per lane.  A lane still
+      // meets its elements in rising order, as the index reducers expect.  (One element per lane and step moved
+      // 256 bytes per wave instruction: f32 rows of 16381 ran at 2.5 TB/s.)
+      const int64_t head0 = (E - (base + k0) % E) % E, head = head0 < k1 - k0 ? head0 : k1 - k0;
+      const int64_t kb = k0 + head, nv = (k1 - kb) / E, kt = kb + nv * E;
+      if (lane < head) acc = R::seed(acc, k0 + lane);
+      else if (lane < nv) acc = R::seed(acc, kb + (int64_t)lane * E);
+      else if (kt + lane < k1) acc = R::seed(acc, kt + lane);
+      if (lane < head) acc = R::accumulate(acc, load_one<CT>(in, idt, base + k0 + lane), k0 + lane);
+      int64_t v = lane;
+      for (; v + TPR < nv; v += 2 * TPR) {
+        CT x[E], y[E];
+        load_vec<CT, E>(in, idt, base + kb + v * E, x);
+        load_vec<CT, E>(in, idt, base + kb + (v + TPR) * E, y);
+#pragma unroll
+        for (int i = 0; i < E; i++) acc = R::accumulate(acc, x[i], kb + v * E + i);
+#pragma unroll
+        for (int i = 0; i < E; i++) acc = R::accumulate(acc, y[i], kb + (v + TPR) * E + i);
+      }
+      for (; v < nv; v += TPR) {
+        CT x[E];
+        load_vec<CT, E>(in, idt, base + kb + v * E, x);
+#pragma unroll
+        for (int i = 0; i < E; i++) acc = R::accumulate(acc, x[i], kb + v * E + i);
+      }
+      if (kt + lane < k1) acc = R::accumulate(acc, load_one<CT>(in, idt, base + kt + lane), kt + lane);
     }
   }
   acc = wave_reduce<R, (TPR < WAVE ? TPR : WAVE)>(acc);
@@ -301,10 +329,10 @@ static int run_reduce_t(hipnx_ctx *ctx, bool static_ws, int idt, int odt, int64_
         }
       } else if (tpr == WAVE) {
         if (vec) hipLaunchKernelGGL((reduce_rows_kernel<R, CT, WAVE, true, IDT>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
-        else hipLaunchKernelGGL((reduce_rows_kernel<R, CT, WAVE, false>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
+        else hipLaunchKernelGGL((reduce_rows_kernel<R, CT, WAVE, false, IDT>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
       } else {
         if (vec) hipLaunchKernelGGL((reduce_rows_kernel<R, CT, BLOCK, true, IDT>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
-        else hipLaunchKernelGGL((reduce_rows_kernel<R, CT, BLOCK, false>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
+        else hipLaunchKernelGGL((reduce_rows_kernel<R, CT, BLOCK, false, IDT>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
       }
       if (nseg > 1) {
         dim3 g2((unsigned)((rows + BLOCK / WAVE - 1) / (BLOCK / WAVE)));  // (rows < 8 * CUs here)

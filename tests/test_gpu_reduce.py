@@ -228,3 +228,35 @@ def test_few_elements_per_row_and_few_columns(shape, axis, ty, op, hip, oracle):
         assert np.array_equal(np.isnan(g), np.isnan(w)) and np.array_equal(g[~np.isnan(g)], w[~np.isnan(w)]), f"{op} {shape}"
     else:
         assert_bits_equal(got, want, f"{op} {ty} {shape} axis {axis}")
+
+
+@pytest.mark.parametrize("shape", [(37, 50257), (5, 16381), (3, 4097), (2, 300001), (9, 261), (4, 1023)])
+@pytest.mark.parametrize("ty", ["f32", "bf16", "s32", "u8", "f64"])
+@pytest.mark.parametrize("op", ["sum", "reduce_max", "reduce_min", "argmax", "argmin"])
+def test_long_rows_that_are_not_whole_vectors(shape, ty, op, hip, oracle):
+    """Rows of 50257 elements (a vocabulary): every row starts at another offset from a vector boundary; the kernel
+    reads a row's first elements up to the boundary and its last ones singly and the rest as aligned vectors.  With
+    equal extremes in the head, the body and the tail of a row, and NaN, for the index reducers."""
+    rng = np.random.default_rng(seed_of(shape, ty, op, "ragged rows"))
+    x = rand_raw(rng, ty, shape, lo=-3, hi=3)
+    rows, cols = shape
+    if op != "sum":
+        top = {"f32": 7.0, "bf16": None, "s32": 100, "u8": 250, "f64": 7.0}[ty]
+        if top is not None:
+            for r in range(rows):  # the same extreme near the start, in the middle and at the very end
+                for c in (r % 7, cols // 2 + r, cols - 1 - (r % 5)):
+                    x[r, c] = top if op in ("reduce_max", "argmax") else (-top if ty not in ("u8",) else 0)
+        if ty == "f32" and rows > 2:
+            x[1, cols - 2] = np.nan
+            x[2, 3] = np.nan
+            x[2, cols // 3] = np.nan
+    hx, ox = both(x, ty, hip, oracle)
+    if op in ("argmax", "argmin"):
+        for tie in ("low", "high"):
+            assert_bits_equal(getattr(Nx, op)(hx, axis=1, tie_break=tie), getattr(Nx, op)(ox, axis=1, tie_break=tie), f"{op} {ty} {shape} {tie}")
+    elif op == "sum" and ty in ("f32", "bf16", "f64"):
+        got, want = Nx.sum(hx, axes=[1]), Nx.sum(ox, axes=[1])
+        eps = {"f64": 2.0 ** -52, "f32": 2.0 ** -23, "bf16": 2.0 ** -7}[ty]
+        assert np.allclose(values(got), values(want), rtol=eps + cols * 2.0 ** -50, atol=cols * 2.0 ** -24 * np.abs(values(ox)).sum(axis=1))
+    else:
+        assert_bits_equal(getattr(Nx, op)(hx, axes=[1]), getattr(Nx, op)(ox, axes=[1]), f"{op} {ty} {shape}")
