@@ -383,6 +383,46 @@ strided_copy_vec_kernel(const T *__restrict__ in, T *__restrict__ out, int64_t n
   }
 }
 
+// The same for an innermost output axis that is NOT a multiple of V (broadcasting a column along rows of 50257
+// elements): vectors of the flat output, which may run across row ends.  A lane takes its first element's index
+// apart, walks along the innermost axis and takes the index apart again only where a row ends.  The last vector
+// may be partial.  (One element per lane: 2.0 TB/s on that broadcast.)
+template <typename T>
+__global__ void __launch_bounds__(BLOCK)
+strided_copy_flat_kernel(const T *__restrict__ in, T *__restrict__ out, int64_t n, Strided s) {
+  constexpr int V = 16 / sizeof(T);
+  const int64_t nvec = (n + V - 1) / V, inner = s.dims[s.rank - 1], istride = s.strides[s.rank - 1];
+  for (int64_t v = (int64_t)blockIdx.x * BLOCK + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * BLOCK) {
+    const int64_t i0 = v * V;
+    int64_t base = 0, c = 0;
+    auto locate = [&](int64_t i) {  // base = offset of the outer coordinates of flat index i, c = its innermost one
+      int64_t rem = i;
+      base = 0;
+      for (int a = s.rank - 1; a >= 0; a--) {
+        int64_t q, r;
+        if (rem < (1ll << 31) && s.dims[a] < (1ll << 31)) { q = (uint32_t)rem / (uint32_t)s.dims[a]; r = (uint32_t)rem - (uint32_t)q * (uint32_t)s.dims[a]; }
+        else { q = rem / s.dims[a]; r = rem - q * s.dims[a]; }
+        if (a == s.rank - 1) c = r;
+        else base += r * s.strides[a];
+        rem = q;
+      }
+    };
+    locate(i0);
+    T e[V];
+    const int nel = i0 + V <= n ? V : (int)(n - i0);
+#pragma unroll
+    for (int k = 0; k < V; k++) {
+      if (k < nel) {
+        e[k] = in[base + c * istride];
+        if (++c == inner && k + 1 < nel) locate(i0 + k + 1);
+      }
+    }
+    if (nel == V) *reinterpret_cast<uint4 *>(out + i0) = *reinterpret_cast<const uint4 *>(e);
+    else
+      for (int k = 0; k < nel; k++) out[i0 + k] = e[k];
+  }
+}
+
 // 16 bytes of the repeated element per lane
 __global__ void __launch_bounds__(BLOCK) fill16_kernel(uint4 *__restrict__ out, uint4 pattern, int64_t nvec) {
   for (int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * BLOCK) out[i] = pattern;
@@ -404,6 +444,11 @@ static void launch_strided(const hipnx_ctx *ctx, const void *in, void *out, int6
     sv.dims[s.rank - 1] /= V;
     hipLaunchKernelGGL((strided_copy_vec_kernel<T>), dim3(grid_for(ctx, n / V, BLOCK)), dim3(BLOCK), 0, ctx->stream,
                        (const T *)in, (T *)out, n / V, sv, s.strides[s.rank - 1]);
+    return;
+  }
+  if (s.rank >= 1 && n >= 4 * V && ((uintptr_t)out & 15) == 0) {
+    hipLaunchKernelGGL((strided_copy_flat_kernel<T>), dim3(grid_for(ctx, (n + V - 1) / V, BLOCK)), dim3(BLOCK), 0, ctx->stream,
+                       (const T *)in, (T *)out, n, s);
     return;
   }
   hipLaunchKernelGGL((strided_copy_kernel<T>), dim3(grid_for(ctx, n, BLOCK)), dim3(BLOCK), 0, ctx->stream,

@@ -261,3 +261,29 @@ def test_take_along_the_last_axis_of_long_rows_reports_and_clamps(hip):
         B.sync()
     finally:
         B.bounds_policy(previous)
+
+
+@pytest.mark.parametrize("shape,new,axes", [((300,), (300, 1001), [0]), ((1001,), (300, 1001), None), ((), (7, 33), None), ((5, 1, 3), (5, 77, 3), None),
+                                             ((9, 1), (4, 9, 13), None), ((2, 3), (2, 50257, 3), [0, 2])])
+@pytest.mark.parametrize("ty", ["u8", "bf16", "f32", "s64"])
+def test_broadcast_to_rows_that_are_not_whole_vectors(shape, new, axes, ty, hip, oracle):
+    """An innermost output axis that is not a multiple of 16 bytes: vectors of the flat output that run across row ends,
+    the last one partial."""
+    rng = np.random.default_rng(seed_of(shape, new, ty, "flat"))
+    x = rand_raw(rng, ty, shape)
+    got = Nx.broadcast(from_numpy(x, ty, hip), new, axes)
+    if int(np.prod(new)) <= 50000:
+        assert_bits_equal(got, Nx.broadcast(from_numpy(x, ty, oracle), new, axes), f"broadcast {shape}->{new}")
+    ax = axes if axes is not None else list(range(len(new) - len(shape), len(new)))
+    lifted = x.reshape([new[a] if a in ax and x.shape[ax.index(a)] != 1 else 1 for a in range(len(new))]) if x.ndim else x
+    assert np.array_equal(hip.to_numpy(got).view(np.uint8), np.broadcast_to(lifted, new).copy().view(np.uint8))
+
+
+@pytest.mark.parametrize("shape,perm", [((5, 7, 9), [2, 0, 1]), ((5, 7, 9), [1, 2, 0]), ((3, 11, 2, 13), [3, 1, 0, 2]), ((6, 50257), [1, 0]),
+                                         ((4, 3, 1001), [1, 0, 2])])
+@pytest.mark.parametrize("ty", ["u8", "bf16", "f32", "s64"])
+def test_transposes_with_odd_extents(shape, perm, ty, hip):
+    rng = np.random.default_rng(seed_of(shape, perm, ty, "odd"))
+    x = rand_raw(rng, ty, shape)
+    got = hip.to_numpy(Nx.transpose(from_numpy(x, ty, hip), perm))
+    assert np.array_equal(got.view(np.uint8), np.ascontiguousarray(np.transpose(x, perm)).view(np.uint8))
