@@ -149,6 +149,66 @@ dot_generic_kernel(const void *__restrict__ l, const void *__restrict__ r, void 
   if (m < M && n < N) store_one<CT>(out, odt, b * M * N + m * N + n, acc);
 }
 
+// A handful of outputs over a long contraction (the dot of two vectors, a [16, K] . [K, 16] Gram block): a work-group per
+// output and segment of K, lanes along k, partial sums in f64 (wrapping 64-bit integers), then one small pass that adds
+// an output's segments in order and encodes it.  The tiled kernels give such a problem one tile -- one work-group,
+// or below 256 outputs one lane of the kernel above walking all of K (4M-element vectors: 0.26 s).
+// l element (m, k) = l[m * l_sm + k * l_sk], r element (n, k) = r[n * r_sn + k * r_sk].
+template <typename CT>
+__global__ void __launch_bounds__(256)
+dot_reduce_kernel(const void *__restrict__ l, const void *__restrict__ r, CT *__restrict__ partial, void *__restrict__ out, int ldt,
+                  int rdt, int odt, int64_t M, int64_t N, int64_t K, int64_t l_sm, int64_t l_sk, int64_t r_sn, int64_t r_sk,
+                  int64_t seg_len, int nseg, int vec) {
+  constexpr int V = 8;
+  const int64_t mn = blockIdx.y, b = blockIdx.z, m = mn / N, n = mn - m * N;
+  const int seg = blockIdx.x;
+  const int64_t k0 = (int64_t)seg * seg_len, k1 = k0 + seg_len < K ? k0 + seg_len : K;
+  const int64_t lb = b * M * K + m * l_sm, rb = b * N * K + n * r_sn;
+  CT acc = 0;
+  auto mac = [&](CT x, CT y) {
+    if constexpr (std::is_same<CT, double>::value) acc = x * y + acc;
+    else acc = (int64_t)((uint64_t)x * (uint64_t)y + (uint64_t)acc);
+  };
+  if (vec) {  // both operands contiguous along k, every row and segment on a vector boundary
+    for (int64_t k = k0 + (int64_t)threadIdx.x * V; k < k1; k += 256 * V) {
+      CT x[V], y[V];
+      load_vec<CT, V>(l, ldt, lb + k, x);
+      load_vec<CT, V>(r, rdt, rb + k, y);
+#pragma unroll
+      for (int i = 0; i < V; i++) mac(x[i], y[i]);
+    }
+  } else {
+    for (int64_t k = k0 + threadIdx.x; k < k1; k += 256) mac(load_one<CT>(l, ldt, lb + k * l_sk), load_one<CT>(r, rdt, rb + k * r_sk));
+  }
+  __shared__ CT sm[256];
+  sm[threadIdx.x] = acc;
+  __syncthreads();
+  for (int w = 128; w > 0; w >>= 1) {
+    if ((int)threadIdx.x < w) {
+      if constexpr (std::is_same<CT, double>::value) sm[threadIdx.x] = sm[threadIdx.x] + sm[threadIdx.x + w];
+      else sm[threadIdx.x] = (int64_t)((uint64_t)sm[threadIdx.x] + (uint64_t)sm[threadIdx.x + w]);
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    if (nseg == 1) store_one<CT>(out, odt, b * M * N + mn, sm[0]);
+    else partial[(b * M * N + mn) * nseg + seg] = sm[0];
+  }
+}
+
+template <typename CT>
+__global__ void __launch_bounds__(256)
+dot_reduce_finish_kernel(const CT *__restrict__ partial, void *__restrict__ out, int odt, int64_t outputs, int nseg) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < outputs; i += (int64_t)gridDim.x * 256) {
+    CT acc = partial[i * nseg];
+    for (int s = 1; s < nseg; s++) {
+      if constexpr (std::is_same<CT, double>::value) acc = acc + partial[i * nseg + s];
+      else acc = (int64_t)((uint64_t)acc + (uint64_t)partial[i * nseg + s]);
+    }
+    store_one<CT>(out, odt, i, acc);
+  }
+}
+
 template <int DT>
 static void launch_mfma(const hipnx_ctx *ctx, const void *l, const void *r, void *out, int odt, int64_t batch,
                         int64_t M, int64_t N, int64_t Kb) {
@@ -265,6 +325,42 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
       if (scale_mode == HIPNX_SCALE_PER_ROW && batch != 1) return set_error(HIPNX_EUNSUPPORTED, "dot_scaled: a scale per row with more than one batch item");
       const int64_t need = scale_mode == HIPNX_SCALE_PER_COLUMN ? N : scale_mode == HIPNX_SCALE_PER_ROW ? M : 1;
       if (int st = check_buf(ctx, scale, (uint64_t)need * 4, "dot_scaled scale")) return st;
+    }
+
+    // at most 32 x 32 outputs over a contraction of 4096 elements or more: the reduction kernels
+    if (!scaled && M <= 32 && N <= 32 && K >= 4096 && batch * M * N <= 65535 && !(!is_float(l_dt) && !is_float(r_dt) && is_float(out_dt))) {
+      const bool any_float = is_float(l_dt) || is_float(r_dt);
+      const int lk = l_layout == HIPNX_K_INNER, rk = r_layout == HIPNX_K_INNER;
+      const int64_t l_sm = lk ? K : 1, l_sk = lk ? 1 : M, r_sn = rk ? K : 1, r_sk = rk ? 1 : N;
+      const int64_t outputs = batch * M * N;
+      int64_t nseg = (2 * (int64_t)ctx->num_cus + outputs - 1) / outputs;
+      if (nseg > K / 2048) nseg = K / 2048;
+      if (nseg > 1024) nseg = 1024;
+      if (nseg < 1) nseg = 1;
+      int64_t seg_len = ((K + nseg - 1) / nseg + 7) / 8 * 8;
+      nseg = (K + seg_len - 1) / seg_len;
+      const int vec = l_sk == 1 && r_sk == 1 && K % 8 == 0 && ((uintptr_t)l->ptr % 32 == 0) && ((uintptr_t)r->ptr % 32 == 0);
+      void *ws = nullptr;
+      size_t ws_cap = 0;
+      if (nseg > 1)
+        if (int st = pool_alloc(ctx, (size_t)(outputs * nseg) * 8, &ws, &ws_cap)) return st;
+      dim3 grid((unsigned)nseg, (unsigned)(M * N), (unsigned)batch), block(256);
+      if (any_float) {
+        hipLaunchKernelGGL((dot_reduce_kernel<double>), grid, block, 0, ctx->stream, l->ptr, r->ptr, (double *)ws, out->ptr, l_dt, r_dt, out_dt, M, N, K,
+                           l_sm, l_sk, r_sn, r_sk, seg_len, (int)nseg, vec);
+        if (nseg > 1)
+          hipLaunchKernelGGL((dot_reduce_finish_kernel<double>), dim3((unsigned)((outputs + 255) / 256)), block, 0, ctx->stream, (const double *)ws,
+                             out->ptr, out_dt, outputs, (int)nseg);
+      } else {
+        hipLaunchKernelGGL((dot_reduce_kernel<int64_t>), grid, block, 0, ctx->stream, l->ptr, r->ptr, (int64_t *)ws, out->ptr, l_dt, r_dt, out_dt, M, N, K,
+                           l_sm, l_sk, r_sn, r_sk, seg_len, (int)nseg, vec);
+        if (nseg > 1)
+          hipLaunchKernelGGL((dot_reduce_finish_kernel<int64_t>), dim3((unsigned)((outputs + 255) / 256)), block, 0, ctx->stream, (const int64_t *)ws,
+                             out->ptr, out_dt, outputs, (int)nseg);
+      }
+      if (ws) pool_free(ctx, ws, ws_cap);  // later work is ordered on the same stream
+      HIPNX_HIP(hipGetLastError());
+      return HIPNX_OK;
     }
 
     if (!mfma) {
