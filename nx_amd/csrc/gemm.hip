@@ -250,13 +250,10 @@ splitk_combine_kernel(const AT *__restrict__ part, void *__restrict__ out, int o
   }
 }
 
+// k_use > 0: contract only the first k_use of the K elements (a whole number of slabs); the operands keep their shapes
 static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batch, int64_t M, int64_t N,
                     int64_t K, int l_layout, int r_layout, const hipnx_buf *l, const hipnx_buf *r,
-                    hipnx_buf *out, int scale_mode, const hipnx_buf *scale);
-
-static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batch, int64_t M, int64_t N,
-                    int64_t K, int l_layout, int r_layout, const hipnx_buf *l, const hipnx_buf *r,
-                    hipnx_buf *out, int scale_mode, const hipnx_buf *scale);
+                    hipnx_buf *out, int scale_mode, const hipnx_buf *scale, int64_t k_use = 0);
 
 // A copy of a dot operand ([batch, rows, K] or [batch, K, rows]) with K extended to Kp by zeros.
 static int pad_k(hipnx_ctx *ctx, int esz, int64_t batch, int64_t rows, int64_t K, int64_t Kp, int layout,
@@ -276,7 +273,7 @@ static int pad_k(hipnx_ctx *ctx, int esz, int64_t batch, int64_t rows, int64_t K
 
 static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batch, int64_t M, int64_t N,
                     int64_t K, int l_layout, int r_layout, const hipnx_buf *l, const hipnx_buf *r,
-                    hipnx_buf *out, int scale_mode, const hipnx_buf *scale) {
+                    hipnx_buf *out, int scale_mode, const hipnx_buf *scale, int64_t k_use) {
   // A contraction length that is not a whole number of 128-byte slabs keeps a large MFMA-typed problem off the
   // tiled kernels (K not a multiple of 16 bytes even sends it to the generic kernel: a few TFLOP/s).  Both
   // operands are then copied with K extended by zeros -- products of two zeros, which add nothing -- and the
@@ -286,10 +283,58 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
     const bool typed = l_dt == r_dt && esz > 0 && out_dtype_size(out_dt) > 0 &&
                        (((l_dt == HIPNX_BF16 || l_dt == HIPNX_F16 || l_dt == HIPNX_F32) && is_float(out_dt)) ||
                         (l_dt == HIPNX_S8 && !is_float(out_dt) && K <= (1ll << 16)));
-    if (typed && scale_mode == HIPNX_SCALE_NONE && K > 0 && batch > 0 && M > 0 && N > 0 && (K * esz) % SLAB != 0 && M * N >= 256 &&
+    if (!k_use && typed && scale_mode == HIPNX_SCALE_NONE && K > 0 && batch > 0 && M > 0 && N > 0 && (K * esz) % SLAB != 0 && M * N >= 256 &&
         (double)M * (double)N * (double)K * (double)batch >= 16777216.0 && l && r &&
         (l_layout == HIPNX_K_INNER || l_layout == HIPNX_K_OUTER) && (r_layout == HIPNX_K_INNER || r_layout == HIPNX_K_OUTER)) {
       const int64_t per = SLAB / esz, Kp = (K + per - 1) / per * per;
+      const int64_t Kmain = K / per * per, Ktail = K - Kmain;
+      if (!k_use && batch == 1 && (K * esz) % 16 == 0 && Kmain >= 8 * per && (M * N) % 4 == 0) {
+        // Rows that are whole 16-byte blocks need no copy of the operands: the whole slabs of K are contracted in
+        // place (the kernels take a row pitch), the last part of K from two small zero-extended copies of one slab
+        // per row, and the two f32 (s32) results are added and encoded by the pass that finishes a split K.  (A copy
+        // of both operands extended to whole slabs: f32 [60000, 784] . [784, 10] 172 us for a 35 us contraction.)
+        const int ws_dt = l_dt == HIPNX_S8 ? HIPNX_S32 : HIPNX_F32;
+        const int64_t mn = M * N;
+        hipnx_buf *ws = nullptr, *ws2 = nullptr, *lt = nullptr, *rt = nullptr;
+        int st = hipnx_buf_alloc(ctx, (size_t)(2 * mn * 4), &ws);
+        if (!st) st = hipnx_buf_wrap(ctx, (char *)ws->ptr + mn * 4, (size_t)(mn * 4), &ws2);
+        if (!st) st = dot_impl(ctx, l_dt, r_dt, ws_dt, 1, M, N, K, l_layout, r_layout, l, r, ws, scale_mode, scale, Kmain);
+        const unsigned char zero = 0;
+        if (!st) st = hipnx_buf_alloc(ctx, (size_t)(M * SLAB), &lt);
+        if (!st) st = hipnx_buf_alloc(ctx, (size_t)(N * SLAB), &rt);
+        if (!st) st = hipnx_fill(ctx, lt, 1, &zero, M * SLAB);
+        if (!st) st = hipnx_fill(ctx, rt, 1, &zero, N * SLAB);
+        if (!st) {
+          const int64_t dims[2] = {M, Ktail}, os[2] = {per, 1};
+          const int64_t is_in[2] = {K, 1}, is_out[2] = {1, M};
+          st = hipnx_strided_copy(ctx, esz, 2, dims, l_layout == HIPNX_K_INNER ? is_in : is_out,
+                                  l_layout == HIPNX_K_INNER ? Kmain : Kmain * M, os, 0, l, lt);
+        }
+        if (!st) {
+          const int64_t dims[2] = {N, Ktail}, os[2] = {per, 1};
+          const int64_t is_in[2] = {K, 1}, is_out[2] = {1, N};
+          st = hipnx_strided_copy(ctx, esz, 2, dims, r_layout == HIPNX_K_INNER ? is_in : is_out,
+                                  r_layout == HIPNX_K_INNER ? Kmain : Kmain * N, os, 0, r, rt);
+        }
+        if (!st) st = dot_impl(ctx, l_dt, r_dt, ws_dt, 1, M, N, per, HIPNX_K_INNER, HIPNX_K_INNER, lt, rt, ws2, scale_mode, scale);
+        if (!st) {
+          Enter in(ctx);
+          st = in.status;
+          if (!st) st = check_buf(ctx, out, (uint64_t)mn * out_dtype_size(out_dt), "dot out");
+          if (!st) {
+            dim3 grid((unsigned)std::min<int64_t>((mn / 4 + 255) / 256, 1 << 20)), block(256);
+            if (ws_dt == HIPNX_S32) hipLaunchKernelGGL((splitk_combine_kernel<int>), grid, block, 0, ctx->stream, (const int *)ws->ptr, out->ptr, out_dt, mn, 2);
+            else hipLaunchKernelGGL((splitk_combine_kernel<float>), grid, block, 0, ctx->stream, (const float *)ws->ptr, out->ptr, out_dt, mn, 2);
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess) st = hip_fail(e, "combine launch");
+          }
+        }
+        if (lt) hipnx_buf_destroy(lt);
+        if (rt) hipnx_buf_destroy(rt);
+        if (ws2) hipnx_buf_destroy(ws2);
+        if (ws) hipnx_buf_destroy(ws);
+        return st;
+      }
       hipnx_buf *lp = nullptr, *rp = nullptr;
       int st = pad_k(ctx, esz, batch, M, K, Kp, l_layout, l, &lp);
       if (!st) st = pad_k(ctx, esz, batch, N, K, Kp, r_layout, r, &rp);
@@ -315,7 +360,7 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
     if (batch * M * N == 0) return HIPNX_OK;
     if (batch > 65535) return set_error(HIPNX_EUNSUPPORTED, "dot: more than 65535 batch items");
 
-    Kb = K * dtype_size(l_dt);
+    Kb = (k_use ? k_use : K) * dtype_size(l_dt);  // what is contracted; the rows keep their pitch of K elements
     const bool float_pair = l_dt == r_dt && (l_dt == HIPNX_BF16 || l_dt == HIPNX_F16 || l_dt == HIPNX_F32) && is_float(out_dt);
     const bool scaled = scale_mode != HIPNX_SCALE_NONE;
     const bool int8_pair = l_dt == HIPNX_S8 && r_dt == HIPNX_S8 && (scaled || !is_float(out_dt)) && K <= (1ll << 16);
@@ -328,7 +373,7 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
     }
 
     // at most 32 x 32 outputs over a contraction of 4096 elements or more: the reduction kernels
-    if (!scaled && M <= 32 && N <= 32 && K >= 4096 && batch * M * N <= 65535 && !(!is_float(l_dt) && !is_float(r_dt) && is_float(out_dt))) {
+    if (!k_use && !scaled && M <= 32 && N <= 32 && K >= 4096 && batch * M * N <= 65535 && !(!is_float(l_dt) && !is_float(r_dt) && is_float(out_dt))) {
       const bool any_float = is_float(l_dt) || is_float(r_dt);
       const int lk = l_layout == HIPNX_K_INNER, rk = r_layout == HIPNX_K_INNER;
       const int64_t l_sm = lk ? K : 1, l_sk = lk ? 1 : M, r_sn = rk ? K : 1, r_sk = rk ? 1 : N;
@@ -421,10 +466,10 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
         a.out = out->ptr;
         a.odt = out_dt;
         a.M = M; a.N = N; a.Kb = Kb;
-        a.ld_l = l_kin ? Kb : M * esz;
-        a.ld_r = r_kin ? Kb : N * esz;
-        a.bs_l = M * Kb;
-        a.bs_r = N * Kb;
+        a.ld_l = l_kin ? K * esz : M * esz;
+        a.ld_r = r_kin ? K * esz : N * esz;
+        a.bs_l = M * K * esz;
+        a.bs_r = N * K * esz;
         a.scale = scale_mode != HIPNX_SCALE_NONE ? (const float *)scale->ptr : nullptr;
         a.scale_mode = scale_mode;
         // tile choice: the largest tile that still gives every CU work; few rows against a long
