@@ -494,14 +494,27 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
         else if (l_dt == HIPNX_S8 && big_ok && t256 * 2 >= ctx->num_cus)
           cfg = GEMM_CFG_256;  // int8 has no half-width tile: full tiles from half of the CUs on (3072^3: 46 us against 57 us)
         else cfg = GEMM_CFG_128;
+        // many rows against at most 32 columns (a layer with a few outputs): a 128-column tile would be three
+        // quarters empty or more, and its MFMA work is what bounds f32
+        if (N <= 32 && M > 64 && cfg == GEMM_CFG_128) cfg = GEMM_CFG_128x32;
         // A grid of 128 x 128 tiles that leaves three quarters of the CUs idle (a few hundred rows against a long
         // weight matrix: 128 x 4096 x 4096 is 32 tiles walking 64 slabs each) splits K over S work-groups per tile:
         // f32 (s32) partial results in pool workspace, then one pass that adds them in split order.
         int splits = 1;
         const int64_t nslab = Kb / SLAB;
-        const bool splittable = cfg == GEMM_CFG_128 && batch == 1 && scale_mode == HIPNX_SCALE_NONE && (M * N) % 4 == 0 &&
+        const bool splittable = (cfg == GEMM_CFG_128 || cfg == GEMM_CFG_128x32) && batch == 1 && scale_mode == HIPNX_SCALE_NONE && (M * N) % 4 == 0 &&
                                 (l_dt == HIPNX_S8 ? !is_float(out_dt) : true);
-        if (l_dt == HIPNX_F32) {
+        if (l_dt == HIPNX_F32 && cfg == GEMM_CFG_128x32) {
+          // (0.6 us per slab of a 128 x 32 tile; the split as below)
+          const int64_t cus = ctx->num_cus, tiles = t128 * batch;
+          double best = 10.0 + (double)((tiles + cus - 1) / cus) * (double)nslab * 0.6;
+          if (splittable)
+            for (int cand = 2; cand <= 64; cand *= 2) {
+              if (tiles * cand > cus || nslab % cand != 0 || nslab / cand < 2) continue;
+              const double t = 10.0 + (double)(nslab / cand) * 0.6 + 5.0 + 2.0 * (double)cand * (double)(M * N) * 4.0 / 8.0e6;
+              if (t < best) { best = t; splits = cand; }
+            }
+        } else if (l_dt == HIPNX_F32) {
           // An f32 slab is eight times the MFMA work of a 2-byte one (2.6 us per slab of a 128 x 128 tile, 0.55 us
           // for a 64 x 32 tile, the second pass of a split about 8 us), so a grid that leaves CUs idle is cut much
           // earlier: the cheapest, by those figures, of whole 128 x 128 tiles, K split up to 64 ways (2 slabs or

@@ -13,7 +13,8 @@ enum {
   GEMM_CFG_256 = 0,  // 256 x 256, 8 waves (4 x 2, each 64 x 128): large square-ish problems
   GEMM_CFG_128 = 1,  // 128 x 128: mid-size and batched problems; 4 waves (2 x 2, each 64 x 64), or two such groups sharing K
   GEMM_CFG_64x32 = 2, // 64 x 32, 2 waves: few rows against a long weight matrix (HBM streaming)
-  GEMM_CFG_64x128 = 4 // 64 x 128, 4 waves (2 x 2, each 32 x 64): f32 with up to 64 rows
+  GEMM_CFG_64x128 = 4, // 64 x 128, 4 waves (2 x 2, each 32 x 64): f32 with up to 64 rows
+  GEMM_CFG_128x32 = 5  // 128 x 32, 4 waves (4 x 1, each 32 x 32): many rows against up to 32 columns (a layer with a few outputs)
 };
 
 int launch_gemm_bf16(const hipnx_ctx *ctx, int cfg, bool l_kin, bool r_kin, GemmArgs a, int64_t batch);
@@ -119,6 +120,9 @@ static int launch_cfg(const hipnx_ctx *ctx, int cfg, const GemmArgs &a, int64_t 
       }
       return launch_one<DT, 2, 2, 2, 2, LK, RK>(ctx, a, batch);
     }
+    case GEMM_CFG_128x32:
+      if constexpr (LK && RK) return launch_one<DT, 4, 1, 1, 1, LK, RK, 4>(ctx, a, batch);
+      else return launch_one<DT, 4, 1, 1, 1, LK, RK>(ctx, a, batch);
     case GEMM_CFG_64x128:
       if constexpr (DT == HIPNX_F32) return launch_one<DT, 2, 2, 1, 2, LK, RK>(ctx, a, batch);
       return launch_one<DT, 2, 2, 2, 2, LK, RK>(ctx, a, batch);

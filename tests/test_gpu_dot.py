@@ -459,3 +459,35 @@ def test_few_outputs_over_a_long_contraction_batched(hip, oracle):
     v = rng.integers(-100, 100, size=(1 << 20,)).astype(np.int32)
     hv, ov = both(v, "s32", hip, oracle)
     assert_bits_equal(Nx.dot(hv, hv), Nx.dot(ov, ov), "vector . vector s32")
+
+
+@pytest.mark.parametrize("M,N,K", [(300, 10, 784), (1000, 1, 512), (65, 32, 256), (2000, 17, 128), (4099, 3, 1152)])
+@pytest.mark.parametrize("ty", ["f32", "bf16", "f16", "s8"])
+@pytest.mark.parametrize("layout", ["nn", "nt", "tn", "tt"])
+def test_many_rows_against_a_few_columns(M, N, K, ty, layout, hip, oracle):
+    """A layer with a few outputs ([60000, 784] . [784, 10]): tiles of 128 x 32, and a K that is not whole slabs
+    contracted in place with its last part from padded copies.  int8 exact, floats within the accumulation bound,
+    and every output in its own place (rows and columns off every tile edge)."""
+    rng = np.random.default_rng(seed_of(M, N, K, ty, layout, "narrow"))
+    if ty == "s8":
+        a = rng.integers(-127, 128, size=(M, K)).astype(np.int8)
+        b = rng.integers(-127, 128, size=(K, N)).astype(np.int8)
+    else:
+        a, b = rand_raw(rng, ty, (M, K), lo=-1, hi=1), rand_raw(rng, ty, (K, N), lo=-1, hi=1)
+    la = a if layout[0] == "n" else np.ascontiguousarray(a.T)
+    lb = b if layout[1] == "n" else np.ascontiguousarray(b.T)
+    c1 = [1] if layout[0] == "n" else [0]
+    c2 = [0] if layout[1] == "n" else [1]
+    kw = {"out_type": "s32"} if ty == "s8" else {}
+    got = Nx.dot(from_numpy(la, ty, hip), c1, from_numpy(lb, ty, hip), c2, **kw)
+    assert got.shape == (M, N)
+    rows = np.unique(np.concatenate([[0, 63, 64, min(127, M - 1), min(128, M - 1), M - 1], rng.integers(0, M, size=20)]))
+    oa, ob = from_numpy(np.ascontiguousarray(a[rows]), ty, oracle), from_numpy(b, ty, oracle)
+    want = Nx.dot(oa, ob, **kw)
+    got_rows = from_numpy(np.ascontiguousarray(hip.to_numpy(got)[rows]), "s32" if ty == "s8" else ty, oracle)
+    if ty == "s8":
+        assert_bits_equal(got_rows, want, f"narrow s8 {layout}")
+        full = a.astype(np.int64) @ b.astype(np.int64)
+        assert np.array_equal(hip.to_numpy(got).astype(np.int64), full)
+    else:
+        check_float_dot(got_rows, want, values(oa), values(ob), "mk,kn->mn", K, f"narrow {ty} {layout}")
