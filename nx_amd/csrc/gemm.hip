@@ -274,6 +274,31 @@ static int pad_k(hipnx_ctx *ctx, int esz, int64_t batch, int64_t rows, int64_t K
 static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batch, int64_t M, int64_t N,
                     int64_t K, int l_layout, int r_layout, const hipnx_buf *l, const hipnx_buf *r,
                     hipnx_buf *out, int scale_mode, const hipnx_buf *scale, int64_t k_use) {
+  // More batch items than a grid's second dimension holds (100000 small matrices): runs of 65535 items, each over
+  // borrowed handles on its part of the three buffers.
+  if (batch > 65535 && M > 0 && N > 0 && l && r && out && dtype_size(l_dt) > 0 && dtype_size(r_dt) > 0 && out_dtype_size(out_dt) > 0 && K >= 0) {
+    {
+      Enter in(ctx);
+      if (in.status) return in.status;
+      if (int st = check_buf(ctx, l, (uint64_t)batch * M * K * dtype_size(l_dt), "dot lhs")) return st;
+      if (int st = check_buf(ctx, r, (uint64_t)batch * N * K * dtype_size(r_dt), "dot rhs")) return st;
+      if (int st = check_buf(ctx, out, (uint64_t)batch * M * N * out_dtype_size(out_dt), "dot out")) return st;
+    }
+    const size_t lb = (size_t)(M * K) * dtype_size(l_dt), rb = (size_t)(N * K) * dtype_size(r_dt), ob = (size_t)(M * N) * out_dtype_size(out_dt);
+    for (int64_t b0 = 0; b0 < batch; b0 += 65535) {
+      const int64_t nb = batch - b0 < 65535 ? batch - b0 : 65535;
+      hipnx_buf *lw = nullptr, *rw = nullptr, *ow = nullptr;
+      int st = hipnx_buf_wrap(ctx, (char *)l->ptr + b0 * lb, nb * lb > 0 ? nb * lb : 1, &lw);
+      if (!st) st = hipnx_buf_wrap(ctx, (char *)r->ptr + b0 * rb, nb * rb > 0 ? nb * rb : 1, &rw);
+      if (!st) st = hipnx_buf_wrap(ctx, (char *)out->ptr + b0 * ob, nb * ob, &ow);
+      if (!st) st = dot_impl(ctx, l_dt, r_dt, out_dt, nb, M, N, K, l_layout, r_layout, lw, rw, ow, scale_mode, scale, k_use);
+      if (lw) hipnx_buf_destroy(lw);
+      if (rw) hipnx_buf_destroy(rw);
+      if (ow) hipnx_buf_destroy(ow);
+      if (st) return st;
+    }
+    return HIPNX_OK;
+  }
   // A contraction length that is not a whole number of 128-byte slabs keeps a large MFMA-typed problem off the
   // tiled kernels (K not a multiple of 16 bytes even sends it to the generic kernel: a few TFLOP/s).  Both
   // operands are then copied with K extended by zeros -- products of two zeros, which add nothing -- and the
@@ -373,7 +398,7 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
     }
 
     // at most 32 x 32 outputs over a contraction of 4096 elements or more: the reduction kernels
-    if (!k_use && !scaled && M <= 32 && N <= 32 && K >= 4096 && batch * M * N <= 65535 && !(!is_float(l_dt) && !is_float(r_dt) && is_float(out_dt))) {
+    if (!k_use && !scaled && M <= 32 && N <= 32 && (K >= 4096 || (M * N <= 4 && K >= 128)) && batch * M * N <= 65535 && !(!is_float(l_dt) && !is_float(r_dt) && is_float(out_dt))) {
       const bool any_float = is_float(l_dt) || is_float(r_dt);
       const int lk = l_layout == HIPNX_K_INNER, rk = r_layout == HIPNX_K_INNER;
       const int64_t l_sm = lk ? K : 1, l_sk = lk ? 1 : M, r_sn = rk ? K : 1, r_sk = rk ? 1 : N;

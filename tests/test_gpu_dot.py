@@ -491,3 +491,34 @@ def test_many_rows_against_a_few_columns(M, N, K, ty, layout, hip, oracle):
         assert np.array_equal(hip.to_numpy(got).astype(np.int64), full)
     else:
         check_float_dot(got_rows, want, values(oa), values(ob), "mk,kn->mn", K, f"narrow {ty} {layout}")
+
+
+def test_more_batch_items_than_a_grid_dimension_holds(hip, oracle):
+    """100000 small matrices (a transform per point): the batch goes in runs of 65535 items.  Integer-valued f32, so
+    every product and sum is exact and numpy's einsum is the answer bit for bit; a few items against the oracle."""
+    rng = np.random.default_rng(31)
+    a = rng.integers(-8, 9, size=(70001, 3, 3)).astype(np.float32)
+    b = rng.integers(-8, 9, size=(70001, 3, 2)).astype(np.float32)
+    got = Nx.dot(from_numpy(a, "f32", hip), [2], [0], from_numpy(b, "f32", hip), [1], [0])
+    assert got.shape == (70001, 3, 2)
+    assert np.array_equal(hip.to_numpy(got), np.einsum("bmk,bkn->bmn", a, b))
+    pick = [0, 65534, 65535, 65536, 70000]
+    want = Nx.dot(from_numpy(a[pick], "f32", oracle), [2], [0], from_numpy(b[pick], "f32", oracle), [1], [0])
+    assert_bits_equal(from_numpy(hip.to_numpy(got)[pick], "f32", oracle), want, "batch of 70001")
+
+
+@pytest.mark.parametrize("ty", ["f32", "bf16", "s32"])
+def test_a_dot_product_per_batch_item(ty, hip, oracle):
+    """[B, 1, K] . [B, K, 1]: one output per item, each a work-group of the reduction kernel."""
+    rng = np.random.default_rng(seed_of(ty, "rowwise dot"))
+    if ty == "s32":
+        a, b = rng.integers(-100, 100, size=(3000, 1, 512)).astype(np.int32), rng.integers(-100, 100, size=(3000, 512, 1)).astype(np.int32)
+    else:
+        a, b = rand_raw(rng, ty, (3000, 1, 512), lo=-1, hi=1), rand_raw(rng, ty, (3000, 512, 1), lo=-1, hi=1)
+    ha, oa = both(a, ty, hip, oracle)
+    hb, ob = both(b, ty, hip, oracle)
+    got, want = Nx.dot(ha, [2], [0], hb, [1], [0]), Nx.dot(oa, [2], [0], ob, [1], [0])
+    if ty == "s32":
+        assert_bits_equal(got, want, "row-wise dot s32")
+    else:
+        check_float_dot(got, want, values(oa), values(ob), "bmk,bkn->bmn", 512, f"row-wise dot {ty}")
