@@ -127,14 +127,15 @@ dot_generic_kernel(const void *__restrict__ l, const void *__restrict__ r, void 
   constexpr int T = 16;
   __shared__ CT sA[T][T + 1], sB[T][T + 1];
   const int tx = threadIdx.x % T, ty = threadIdx.x / T;
+  // (tiles of M along x, which holds 2^31 - 1 groups: [2M, 3] . [3, 3] has 131072 of them; tiles of N along y)
   const int64_t b = blockIdx.z;
-  const int64_t m = (int64_t)blockIdx.y * T + ty, n = (int64_t)blockIdx.x * T + tx;
+  const int64_t m = (int64_t)blockIdx.x * T + ty, n = (int64_t)blockIdx.y * T + tx;
   const int64_t lbase = b * M * K, rbase = b * N * K;
   CT acc = 0;
   for (int64_t k0 = 0; k0 < K; k0 += T) {
     {  // sA[ty][tx] = l[m, k0 + tx]; sB[ty][tx] = r[n0 + ty, k0 + tx]
       const int64_t k = k0 + tx;
-      const int64_t mm = (int64_t)blockIdx.y * T + ty, nn = (int64_t)blockIdx.x * T + ty;
+      const int64_t mm = (int64_t)blockIdx.x * T + ty, nn = (int64_t)blockIdx.y * T + ty;
       sA[ty][tx] = (mm < M && k < K) ? load_one<CT>(l, ldt, lbase + (lk ? mm * K + k : k * M + mm)) : (CT)0;
       sB[ty][tx] = (nn < N && k < K) ? load_one<CT>(r, rdt, rbase + (rk ? nn * K + k : k * N + nn)) : (CT)0;
     }
@@ -436,8 +437,9 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
     if (!mfma) {
       const bool any_float = is_float(l_dt) || is_float(r_dt);
       if (!any_float && is_float(out_dt)) return set_error(HIPNX_EUNSUPPORTED, "dot: integer operands with a float output");
-      dim3 grid((unsigned)((N + 15) / 16), (unsigned)((M + 15) / 16), (unsigned)batch), block(256);
-      if (grid.y > 65535) return set_error(HIPNX_EUNSUPPORTED, "dot: M too large for the generic kernel");
+      dim3 grid((unsigned)((M + 15) / 16), (unsigned)((N + 15) / 16), (unsigned)batch), block(256);
+      if ((N + 15) / 16 > 65535 || (M + 15) / 16 >= (1ll << 31) / 256)
+        return set_error(HIPNX_EUNSUPPORTED, "dot: more than a million columns (or 134 million rows) on the plain kernel");
       const int lk = l_layout == HIPNX_K_INNER, rk = r_layout == HIPNX_K_INNER;
       if (any_float)
         hipLaunchKernelGGL((dot_generic_kernel<double>), grid, block, 0, ctx->stream, l->ptr, r->ptr, out->ptr, l_dt, r_dt, out_dt, M, N, K, lk, rk);

@@ -522,3 +522,13 @@ def test_a_dot_product_per_batch_item(ty, hip, oracle):
         assert_bits_equal(got, want, "row-wise dot s32")
     else:
         check_float_dot(got, want, values(oa), values(ob), "bmk,bkn->bmn", 512, f"row-wise dot {ty}")
+
+
+def test_millions_of_rows_against_a_tiny_matrix(hip):
+    """[2M, 3] . [3, 3] (points times a transform): K is not a multiple of 16 bytes, so the plain kernel runs, with
+    131072 tiles of rows along the grid's first dimension.  Integer-valued f32: exact."""
+    rng = np.random.default_rng(9)
+    a = rng.integers(-8, 9, size=(2_000_003, 3)).astype(np.float32)
+    b = rng.integers(-8, 9, size=(3, 3)).astype(np.float32)
+    got = hip.to_numpy(Nx.dot(from_numpy(a, "f32", hip), from_numpy(b, "f32", hip)))
+    assert np.array_equal(got, a @ b)
