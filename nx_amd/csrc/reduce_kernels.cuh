@@ -162,13 +162,16 @@ combine_partials_kernel(const typename R::acc_t *__restrict__ partial, void *__r
 // One lane per E adjacent inner positions (VEC) or per position; walks k in its segment.
 // With nseg == 1 results are encoded into out[outer, inner]; otherwise raw accumulators go to
 // partial[outer, nseg, inner].
-template <typename R, typename CT, bool VEC, int IDT = -1>
+// UNAL (with VEC): `inner` is not a multiple of E (a row of 50257 columns), so a row begins at any offset from a
+// vector boundary: whole vectors are fetched at whatever address they have, the last lane of a row takes its
+// remaining columns one by one (one column per lane moved 256 bytes per wave instruction: 1.6-1.9 TB/s).
+template <typename R, typename CT, bool VEC, int IDT = -1, bool UNAL = false>
 __global__ void __launch_bounds__(BLOCK)
 reduce_cols_kernel(const void *__restrict__ in, void *__restrict__ out, typename R::acc_t *__restrict__ partial,
                    int idt_, int odt, int64_t outer, int64_t red, int64_t inner, int64_t seg_len, int nseg) {
   const int idt = IDT >= 0 ? IDT : idt_;
   constexpr int W = VEC ? E : 1;
-  const int64_t ivecs = inner / W;
+  const int64_t ivecs = UNAL ? (inner + W - 1) / W : inner / W;
   const int64_t total = outer * nseg * ivecs;
   for (int64_t t = (int64_t)blockIdx.x * BLOCK + threadIdx.x; t < total; t += (int64_t)gridDim.x * BLOCK) {
     const int64_t iv = t % ivecs, os = t / ivecs;
@@ -179,13 +182,23 @@ reduce_cols_kernel(const void *__restrict__ in, void *__restrict__ out, typename
 #pragma unroll
     for (int i = 0; i < W; i++) acc[i] = k0 < k1 ? R::seed(R::init(), k0) : R::init();
     const int64_t base = o * red * inner + iv * W;
+    const int valid = UNAL && iv * W + W > inner ? (int)(inner - iv * W) : W;  // columns of this lane inside the row
+    if (UNAL && valid < W) {
+      for (int i = 0; i < valid; i++) {
+        typename R::acc_t a = k0 < k1 ? R::seed(R::init(), k0) : R::init();
+        for (int64_t k = k0; k < k1; k++) a = R::accumulate(a, load_one<CT>(in, idt, base + k * inner + i), k);
+        if (nseg == 1) finalize(out, odt, o * inner + iv * W + i, a);
+        else partial[(o * nseg + seg) * inner + iv * W + i] = a;
+      }
+      continue;
+    }
     int64_t k = k0;
     for (; k + 3 < k1; k += 4) {  // four independent row loads in flight per lane
       CT v0[W], v1[W], v2[W], v3[W];
-      load_vec<CT, W>(in, idt, base + k * inner, v0);
-      load_vec<CT, W>(in, idt, base + (k + 1) * inner, v1);
-      load_vec<CT, W>(in, idt, base + (k + 2) * inner, v2);
-      load_vec<CT, W>(in, idt, base + (k + 3) * inner, v3);
+      load_vec<CT, W, !UNAL>(in, idt, base + k * inner, v0);
+      load_vec<CT, W, !UNAL>(in, idt, base + (k + 1) * inner, v1);
+      load_vec<CT, W, !UNAL>(in, idt, base + (k + 2) * inner, v2);
+      load_vec<CT, W, !UNAL>(in, idt, base + (k + 3) * inner, v3);
 #pragma unroll
       for (int i = 0; i < W; i++) {
         acc[i] = R::accumulate(acc[i], v0[i], k);
@@ -196,7 +209,7 @@ reduce_cols_kernel(const void *__restrict__ in, void *__restrict__ out, typename
     }
     for (; k < k1; k++) {
       CT v[W];
-      load_vec<CT, W>(in, idt, base + k * inner, v);
+      load_vec<CT, W, !UNAL>(in, idt, base + k * inner, v);
 #pragma unroll
       for (int i = 0; i < W; i++) acc[i] = R::accumulate(acc[i], v[i], k);
     }
@@ -342,14 +355,15 @@ static int run_reduce_t(hipnx_ctx *ctx, bool static_ws, int idt, int odt, int64_
     partials_release(ctx, static_ws, ws, ws_cap);
   } else {
     const bool vec = inner % E == 0;
-    const int64_t lanes = outer * (inner / (vec ? E : 1));
+    const bool unal = !vec && inner >= 8 * E && IDT >= 0;  // long rows off the vector grid (compiled for the common element types)
+    const int64_t lanes = outer * (unal ? (inner + E - 1) / E : inner / (vec ? E : 1));
     int nseg = 1;
     int64_t seg_len = red;
     // Waves wanted per CU: what keeps about 128 bytes per lane-row times 64 lanes in flight -- 4 for f32 (32 bytes
     // per lane and row), 8 for 2-byte types, 16 for bytes (measured on 16384 x 16384: f32 6.3 TB/s with 4 against
     // 6.0 with 8 and 5.0 with 16; bf16 5.3 / 5.7 / 5.0; u8 2.5 / 3.6 / 4.7).  More segments than that only add
     // partial results.
-    const int lane_bytes = (vec ? E : 1) * dtype_size(idt);
+    const int lane_bytes = (vec || unal ? E : 1) * dtype_size(idt);
     const int colw = lane_bytes >= 64 ? 2 : lane_bytes <= 8 ? 16 : 128 / lane_bytes;
     const int64_t want_lanes = (int64_t)ctx->num_cus * colw * WAVE;
     if (lanes < want_lanes && red >= 64) {
@@ -373,6 +387,7 @@ static int run_reduce_t(hipnx_ctx *ctx, bool static_ws, int idt, int odt, int64_
     dim3 grid((unsigned)(blocks < 1 ? 1 : (blocks < cap ? blocks : cap))), block(BLOCK);
     if (total > 0) {
       if (vec) hipLaunchKernelGGL((reduce_cols_kernel<R, CT, true, IDT>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, outer, red, inner, seg_len, nseg);
+      else if (unal) hipLaunchKernelGGL((reduce_cols_kernel<R, CT, true, IDT, true>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, outer, red, inner, seg_len, nseg);
       else hipLaunchKernelGGL((reduce_cols_kernel<R, CT, false>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, outer, red, inner, seg_len, nseg);
       if (nseg > 1) {
         int64_t b2 = (outer * inner + COMBINE_COLS_X - 1) / COMBINE_COLS_X;

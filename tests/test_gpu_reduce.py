@@ -184,7 +184,8 @@ def test_reduced_axes_that_are_not_neighbours(shape, axes, ty, op, hip, oracle):
 
 
 FEW = [((5000, c), 1) for c in (1, 2, 3, 5, 8, 13, 16, 17, 33, 100, 255)] + \
-      [((8192, 3), 0), ((12288, 2), 0), ((3, 4096, 7), 1), ((20000, 33), 0), ((2, 8190, 5), 1), ((4099, 3), 0), ((65536, 1, 2), 0)]
+      [((8192, 3), 0), ((12288, 2), 0), ((3, 4096, 7), 1), ((20000, 33), 0), ((2, 8190, 5), 1), ((4099, 3), 0), ((65536, 1, 2), 0)] + \
+      [((300, 1001), 0), ((7, 50, 77), 1), ((64, 261), 0), ((5000, 69), 0), ((3, 700, 131), 1)]  # rows off the vector grid under the reduced axis
 
 
 @pytest.mark.parametrize("shape,axis", FEW, ids=[f"{s}-{a}" for s, a in FEW])
