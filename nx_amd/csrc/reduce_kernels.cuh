@@ -70,8 +70,18 @@ reduce_rows_kernel(const void *__restrict__ in, void *__restrict__ out, typename
         for (int i = 0; i < E; i++) acc = R::accumulate(acc, v[i], k + i);
       }
     } else if constexpr (TPR < WAVE) {
-      if (k0 + lane < k1) acc = R::seed(acc, k0 + lane);
-      for (int64_t k = k0 + lane; k < k1; k += TPR) acc = R::accumulate(acc, load_one<CT>(in, idt, base + k), k);
+      // a short row that is not whole vectors (33 elements): vectors fetched at whatever address they have, the
+      // last few elements one per lane; a lane meets its elements in rising order
+      const int64_t nv = (k1 - k0) / E, kt = k0 + nv * E;
+      if (lane < nv) acc = R::seed(acc, k0 + (int64_t)lane * E);
+      else if (kt + lane < k1) acc = R::seed(acc, kt + lane);
+      for (int64_t v = lane; v < nv; v += TPR) {
+        CT x[E];
+        load_vec<CT, E, false>(in, idt, base + k0 + v * E, x);
+#pragma unroll
+        for (int i = 0; i < E; i++) acc = R::accumulate(acc, x[i], k0 + v * E + i);
+      }
+      if (kt + lane < k1) acc = R::accumulate(acc, load_one<CT>(in, idt, base + kt + lane), kt + lane);
     } else {
       // a row that is not whole vectors (a vocabulary of 50257 entries): its first elements up to a vector boundary of
       // the BUFFER one per lane, then whole aligned vectors, then the last few elements one per lane.  A lane still
@@ -130,16 +140,14 @@ reduce_rows_short_kernel(const void *__restrict__ in, void *__restrict__ out, in
   for (int64_t row = (int64_t)blockIdx.x * BLOCK + threadIdx.x; row < rows; row += (int64_t)gridDim.x * BLOCK) {
     typename R::acc_t acc = red > 0 ? R::seed(R::init(), 0) : R::init();
     const int64_t base = row * red;
-    if (red % E == 0) {  // whole vectors (rows of 8 or 16 elements)
-      for (int k = 0; k < red; k += E) {
-        CT v[E];
-        load_vec<CT, E>(in, idt, base + k, v);
+    int k = 0;
+    for (; k + E <= red; k += E) {  // whole vectors at whatever address the row has (rows of 8 ... 16 elements)
+      CT v[E];
+      load_vec<CT, E, false>(in, idt, base + k, v);
 #pragma unroll
-        for (int i = 0; i < E; i++) acc = R::accumulate(acc, v[i], k + i);
-      }
-    } else {
-      for (int k = 0; k < red; k++) acc = R::accumulate(acc, load_one<CT>(in, idt, base + k), k);
+      for (int i = 0; i < E; i++) acc = R::accumulate(acc, v[i], k + i);
     }
+    for (; k < red; k++) acc = R::accumulate(acc, load_one<CT>(in, idt, base + k), k);
     finalize(out, odt, row, acc);
   }
 }
@@ -331,9 +339,9 @@ static int run_reduce_t(hipnx_ctx *ctx, bool static_ws, int idt, int odt, int64_
                          idt, odt, rows, (int)red);
     } else if (rows * nseg > 0) {
       if (narrow_scalar) {
-        if (tpr == 8) hipLaunchKernelGGL((reduce_rows_kernel<R, CT, 8, false>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
-        else if (tpr == 16) hipLaunchKernelGGL((reduce_rows_kernel<R, CT, 16, false>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
-        else hipLaunchKernelGGL((reduce_rows_kernel<R, CT, 32, false>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
+        if (tpr == 8) hipLaunchKernelGGL((reduce_rows_kernel<R, CT, 8, false, IDT>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
+        else if (tpr == 16) hipLaunchKernelGGL((reduce_rows_kernel<R, CT, 16, false, IDT>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
+        else hipLaunchKernelGGL((reduce_rows_kernel<R, CT, 32, false, IDT>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
       } else if (tpr < WAVE) {
         if constexpr (IDT >= 0) {
           if (tpr == 8) hipLaunchKernelGGL((reduce_rows_kernel<R, CT, 8, true, IDT>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
