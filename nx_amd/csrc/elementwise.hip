@@ -85,20 +85,45 @@ binary_vec_kernel(const void *__restrict__ l, const void *__restrict__ r, void *
         col = f0 - row * cols;
       }
       const int nel = f0 + E <= total ? E : (int)(total - f0);
+      // (with rows of several axes, ls0 / rs0 only say whether the operand is as dense as the output: cols if so)
       const bool l_dense = ls1 == 1 && ls0 == cols && nel == E, r_dense = rs1 == 1 && rs0 == cols && nel == E;
+      int64_t lrow = 0, rrow = 0;
+      auto row_offsets = [&]() {  // where row `row` begins in each operand
+        if (ax.n <= 1) {
+          lrow = row * ls0;
+          rrow = row * rs0;
+        } else {
+          uint32_t rem = (uint32_t)row;
+          lrow = 0;
+          rrow = 0;
+          for (int k = ax.n - 1; k >= 1; k--) {
+            const uint32_t q = fastdiv(rem, ax.fd[k]), i = rem - q * ax.d[k];
+            lrow += (int64_t)i * ax.ls[k];
+            rrow += (int64_t)i * ax.rs[k];
+            rem = q;
+          }
+          lrow += (int64_t)rem * ax.ls[0];
+          rrow += (int64_t)rem * ax.rs[0];
+        }
+      };
+      row_offsets();
       CT a[E], b[E], c[E];
       if (l_dense) load_vec<CT, E>(l, ldt, f0, a);
       if (r_dense) load_vec<CT, E>(r, rdt, f0, b);
 #pragma unroll
       for (int i = 0; i < E; i++) {
         if (i < nel) {
-          if (!l_dense) a[i] = load_one<CT>(l, ldt, row * ls0 + col * ls1);
-          if (!r_dense) b[i] = load_one<CT>(r, rdt, row * rs0 + col * rs1);
+          if (!l_dense) a[i] = load_one<CT>(l, ldt, lrow + col * ls1);
+          if (!r_dense) b[i] = load_one<CT>(r, rdt, rrow + col * rs1);
         } else {
           a[i] = (CT)1;
           b[i] = (CT)1;
         }
-        if (++col == cols) { col = 0; row++; }
+        if (++col == cols) {
+          col = 0;
+          row++;
+          if (i + 1 < nel) row_offsets();
+        }
       }
 #pragma unroll
       for (int i = 0; i < E; i++) c[i] = binary_apply<OP, CT, UNS>(a[i], b[i]);
@@ -461,7 +486,32 @@ extern "C" int hipnx_binary(hipnx_ctx *ctx, int op, int l_dt, int r_dt, int out_
       rows *= dims[q];
       aligned = aligned && (l1 == 0 || ls[q] % E == 0) && (r1 == 0 || rs[q] % E == 0);
     }
-    if ((l1 == 0 || l1 == 1) && (r1 == 0 || r1 == 1) && aligned && rows * ((cols + 3) / 4) < (1ll << 31)) {
+    if ((l1 == 0 || l1 == 1) && (r1 == 0 || r1 == 1) && !aligned && rows < (1ll << 31) && cols < (1ll << 31)) {
+      // rows of several axes whose length (or an operand's row starts) is off the vector grid -- a mask
+      // [b, 1, 1, 197] against scores [b, h, 197, 197] -- as vectors of the flat output
+      vec_ok = true;
+      a.l = l->ptr; a.r = r->ptr; a.out = out->ptr;
+      a.ldt = l_dt; a.rdt = r_dt; a.odt = out_dt;
+      a.cols = cols;
+      a.vecs_per_row = 1; a.nvec = 1;  // (set by the launcher from flat_total)
+      a.ls1 = (int)l1; a.rs1 = (int)r1;
+      a.err = deferred_error_word(ctx);
+      a.flat_total = n;
+      a.ax.n = m - 1;
+      bool l_dense = l1 == 1, r_dense = r1 == 1;
+      int64_t run = cols;
+      for (int q = m - 2; q >= 0; q--) {
+        a.ax.d[q] = (uint32_t)dims[q];
+        a.ax.fd[q] = make_fastdiv((uint32_t)dims[q]);
+        a.ax.ls[q] = ls[q];
+        a.ax.rs[q] = rs[q];
+        l_dense = l_dense && ls[q] == run;
+        r_dense = r_dense && rs[q] == run;
+        run *= dims[q];
+      }
+      a.ls0 = l_dense ? cols : 0;
+      a.rs0 = r_dense ? cols : 0;
+    } else if ((l1 == 0 || l1 == 1) && (r1 == 0 || r1 == 1) && aligned && rows * ((cols + 3) / 4) < (1ll << 31)) {
       vec_ok = true;
       a.l = l->ptr; a.r = r->ptr; a.out = out->ptr;
       a.ldt = l_dt; a.rdt = r_dt; a.odt = out_dt;

@@ -276,3 +276,35 @@ def test_rows_that_are_not_whole_vectors(ls, rs, ty, op, hip, oracle):
     assert_bits_equal(f(hb, ha), f(ob, oa), f"{op} {ty} {rs} {ls}")
     from nx_amd import backend as B
     B.sync()  # nothing was recorded for a later wait to raise
+
+
+DEEP_RAGGED = [((2, 3, 197, 197), (2, 1, 1, 197)), ((2, 3, 77, 77), (1, 3, 1, 1)), ((4, 7, 13), (4, 1, 13)), ((5, 9, 3), (1, 9, 1)),
+               ((3, 5, 7, 11), (3, 1, 7, 1)), ((2, 4, 6, 9), (1, 4, 1, 9))]
+
+
+@pytest.mark.parametrize("ls,rs", DEEP_RAGGED, ids=[f"{a}-{b}" for a, b in DEEP_RAGGED])
+@pytest.mark.parametrize("ty", ["f32", "bf16", "s32", "u8"])
+@pytest.mark.parametrize("op", ["add", "multiply", "less", "quotient"])
+def test_broadcasts_over_separated_axes_off_the_vector_grid(ls, rs, ty, op, hip, oracle):
+    """A mask [b, 1, 1, 197] against scores [b, h, 197, 197]: three or four collapsed axes AND rows that are not whole
+    vectors -- vectors of the flat output, the row's operand offsets taken apart again where a row ends."""
+    rng = np.random.default_rng(seed_of(ls, rs, ty, op, "deep ragged"))
+    a, b = rand_raw(rng, ty, ls, lo=1, hi=9), rand_raw(rng, ty, rs, lo=1, hi=9)
+    if op == "quotient":
+        if ty in ("f32", "bf16"):
+            pytest.skip("quotient is an integer operation")
+        a, b = np.where(a == 0, 1, a).astype(a.dtype), np.where(b == 0, 1, b).astype(b.dtype)
+    if int(np.prod(ls)) > 60000:  # the oracle's loops: a corner of the big case, numpy for the rest
+        got = hip.to_numpy(getattr(Nx, op)(from_numpy(a, ty, hip), from_numpy(b, ty, hip)))
+        sub = (slice(0, 1), slice(0, 2), slice(0, 50), slice(None))
+        bs = tuple(s_ if d != 1 else slice(None) for s_, d in zip(sub, rs))
+        want = getattr(Nx, op)(from_numpy(np.ascontiguousarray(a[sub]), ty, oracle), from_numpy(np.ascontiguousarray(b[bs]), ty, oracle))
+        assert np.array_equal(np.ascontiguousarray(got[sub]).view(np.uint8), oracle.to_numpy(want).view(np.uint8) if hasattr(oracle, "to_numpy") else np.frombuffer(Nx.to_binary(want), dtype=np.uint8).reshape(np.ascontiguousarray(got[sub]).view(np.uint8).shape))
+        if op in ("add", "multiply") and ty in ("f32", "s32"):
+            assert np.array_equal(got, (a + b) if op == "add" else (a * b))
+        return
+    ha, oa = both(a, ty, hip, oracle)
+    hb, ob = both(b, ty, hip, oracle)
+    f = getattr(Nx, op)
+    assert_bits_equal(f(ha, hb), f(oa, ob), f"{op} {ty} {ls} {rs}")
+    assert_bits_equal(f(hb, ha), f(ob, oa), f"{op} {ty} {rs} {ls}")
