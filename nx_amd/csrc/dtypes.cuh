@@ -120,27 +120,27 @@ struct conv<int64_t> {  // also carries u64 bit patterns
 
 // ALIGNED = false: `idx` is any element (the bytes are fetched through a copy whose source claims no alignment, which
 // the compiler still turns into whole-vector loads: global memory takes them at any address).
+// (Written into its destination, not returned: with the bytes returned by value the compiler took an f32 -> bf16
+// conversion's two 16-byte loads apart into sixteen 2-byte ones.)
 template <int N, bool ALIGNED>
-__device__ __forceinline__ raw_vec<N> fetch_raw(const void *q) {
-  if constexpr (ALIGNED) return *reinterpret_cast<const raw_vec<N> *>(q);
-  else {
-    raw_vec<N> r;
-    __builtin_memcpy(&r, q, N);
-    return r;
-  }
+__device__ __forceinline__ void fetch_raw(raw_vec<N> *dst, const void *q) {
+  if constexpr (ALIGNED) *dst = *reinterpret_cast<const raw_vec<N> *>(q);
+  else __builtin_memcpy(dst, q, N);
 }
 
 template <typename CT, int E, bool ALIGNED = true>
 __device__ __forceinline__ void load_vec(const void *__restrict__ p, int dt, int64_t idx, CT (&v)[E]) {
   switch (dt) {
     case HIPNX_U8: {
-      raw_vec<E> r = fetch_raw<E, ALIGNED>((const uint8_t *)p + idx);
+      raw_vec<E> r;
+      fetch_raw<E, ALIGNED>(&r, (const uint8_t *)p + idx);
 #pragma unroll
       for (int i = 0; i < E; i++) v[i] = conv<CT>::from_int((uint32_t)r.b[i]);
       break;
     }
     case HIPNX_S8: {
-      raw_vec<E> r = fetch_raw<E, ALIGNED>((const uint8_t *)p + idx);
+      raw_vec<E> r;
+      fetch_raw<E, ALIGNED>(&r, (const uint8_t *)p + idx);
 #pragma unroll
       for (int i = 0; i < E; i++) v[i] = conv<CT>::from_int((int32_t)(int8_t)r.b[i]);
       break;
@@ -149,7 +149,8 @@ __device__ __forceinline__ void load_vec(const void *__restrict__ p, int dt, int
     case HIPNX_S16:
     case HIPNX_F16:
     case HIPNX_BF16: {
-      raw_vec<2 * E> r = fetch_raw<2 * E, ALIGNED>((const uint16_t *)p + idx);
+      raw_vec<2 * E> r;
+      fetch_raw<2 * E, ALIGNED>(&r, (const uint16_t *)p + idx);
       const uint16_t *h = reinterpret_cast<const uint16_t *>(r.b);
 #pragma unroll
       for (int i = 0; i < E; i++) {
@@ -167,7 +168,7 @@ __device__ __forceinline__ void load_vec(const void *__restrict__ p, int dt, int
       uint32_t w[E];
 #pragma unroll
       for (int c = 0; c < B / CH; c++)
-        *reinterpret_cast<raw_vec<CH> *>(&w[c * CH / 4]) = fetch_raw<CH, ALIGNED>((const char *)p + idx * 4 + c * CH);
+        fetch_raw<CH, ALIGNED>(reinterpret_cast<raw_vec<CH> *>(&w[c * CH / 4]), (const char *)p + idx * 4 + c * CH);
 #pragma unroll
       for (int i = 0; i < E; i++) {
         if (dt == HIPNX_U32) v[i] = conv<CT>::from_int(w[i]);
@@ -181,7 +182,7 @@ __device__ __forceinline__ void load_vec(const void *__restrict__ p, int dt, int
       uint64_t w[E];
 #pragma unroll
       for (int c = 0; c < B / CH; c++)
-        *reinterpret_cast<raw_vec<CH> *>(reinterpret_cast<char *>(w) + c * CH) = fetch_raw<CH, ALIGNED>((const char *)p + idx * 8 + c * CH);
+        fetch_raw<CH, ALIGNED>(reinterpret_cast<raw_vec<CH> *>(reinterpret_cast<char *>(w) + c * CH), (const char *)p + idx * 8 + c * CH);
 #pragma unroll
       for (int i = 0; i < E; i++) {
         if (dt == HIPNX_F64) v[i] = conv<CT>::from_f64(__longlong_as_double((long long)w[i]));
