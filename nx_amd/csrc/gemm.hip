@@ -150,6 +150,61 @@ dot_generic_kernel(const void *__restrict__ l, const void *__restrict__ r, void 
   if (m < M && n < N) store_one<CT>(out, odt, b * M * N + m * N + n, acc);
 }
 
+// The same contraction on 64 x 64 tiles with 4 x 4 outputs per lane: eight LDS reads per sixteen multiply-adds
+// instead of two per one, each output still accumulated over k in order (the same bits as the kernel above).
+// f64 / s32 / mixed-type 4096^3: 8.4 TFLOP/s there.
+template <typename CT>
+__global__ void __launch_bounds__(256)
+dot_blocked_kernel(const void *__restrict__ l, const void *__restrict__ r, void *__restrict__ out, int ldt, int rdt,
+                   int odt, int64_t M, int64_t N, int64_t K, int lk, int rk) {
+  constexpr int TM = 64, TN = 64, TK = 16;
+  __shared__ CT sA[TK][TM + 4], sB[TK][TN + 4];
+  const int tid = threadIdx.x, tx = tid % 16, ty = tid / 16;
+  const int64_t b = blockIdx.z, m0 = (int64_t)blockIdx.x * TM, n0 = (int64_t)blockIdx.y * TN;
+  const int64_t lbase = b * M * K, rbase = b * N * K;
+  CT acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++) acc[i][j] = 0;
+  for (int64_t k0 = 0; k0 < K; k0 += TK) {
+#pragma unroll
+    for (int q = 0; q < TM * TK / 256; q++) {
+      const int e = tid + q * 256;
+      // consecutive lanes along the operand's contiguous axis
+      const int am = lk ? e / TK : e % TM, ak = lk ? e % TK : e / TM;
+      const int bn = rk ? e / TK : e % TN, bk = rk ? e % TK : e / TN;
+      const int64_t mm = m0 + am, nn = n0 + bn, ka = k0 + ak, kb = k0 + bk;
+      sA[ak][am] = (mm < M && ka < K) ? load_one<CT>(l, ldt, lbase + (lk ? mm * K + ka : ka * M + mm)) : (CT)0;
+      sB[bk][bn] = (nn < N && kb < K) ? load_one<CT>(r, rdt, rbase + (rk ? nn * K + kb : kb * N + nn)) : (CT)0;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < TK; kk++) {
+      CT a[4], c[4];
+#pragma unroll
+      for (int i = 0; i < 4; i++) a[i] = sA[kk][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; j++) c[j] = sB[kk][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          if constexpr (std::is_same<CT, double>::value) acc[i][j] = a[i] * c[j] + acc[i][j];
+          else acc[i][j] = (int64_t)((uint64_t)a[i] * (uint64_t)c[j] + (uint64_t)acc[i][j]);
+        }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const int64_t m = m0 + ty * 4 + i, n = n0 + tx * 4 + j;
+      if (m < M && n < N) store_one<CT>(out, odt, b * M * N + m * N + n, acc[i][j]);
+    }
+}
+
 // A handful of outputs over a long contraction (the dot of two vectors, a [16, K] . [K, 16] Gram block): a work-group per
 // output and segment of K, lanes along k, partial sums in f64 (wrapping 64-bit integers), then one small pass that adds
 // an output's segments in order and encodes it.  The tiled kernels give such a problem one tile -- one work-group,
@@ -441,6 +496,17 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
       if ((N + 15) / 16 > 65535 || (M + 15) / 16 >= (1ll << 31) / 256)
         return set_error(HIPNX_EUNSUPPORTED, "dot: more than a million columns (or 134 million rows) on the plain kernel");
       const int lk = l_layout == HIPNX_K_INNER, rk = r_layout == HIPNX_K_INNER;
+      // tiles of 64 x 64, sixteen outputs per lane, where they still give every CU two work-groups (512^3: 64 tiles, 143 us
+      // against 53 us on 16 x 16 tiles)
+      if (M >= 64 && N >= 64 && (N + 63) / 64 <= 65535 && ((M + 63) / 64) * ((N + 63) / 64) * batch >= 2 * (int64_t)ctx->num_cus) {
+        dim3 g64((unsigned)((M + 63) / 64), (unsigned)((N + 63) / 64), (unsigned)batch);
+        if (any_float)
+          hipLaunchKernelGGL((dot_blocked_kernel<double>), g64, block, 0, ctx->stream, l->ptr, r->ptr, out->ptr, l_dt, r_dt, out_dt, M, N, K, lk, rk);
+        else
+          hipLaunchKernelGGL((dot_blocked_kernel<int64_t>), g64, block, 0, ctx->stream, l->ptr, r->ptr, out->ptr, l_dt, r_dt, out_dt, M, N, K, lk, rk);
+        HIPNX_HIP(hipGetLastError());
+        return HIPNX_OK;
+      }
       if (any_float)
         hipLaunchKernelGGL((dot_generic_kernel<double>), grid, block, 0, ctx->stream, l->ptr, r->ptr, out->ptr, l_dt, r_dt, out_dt, M, N, K, lk, rk);
       else

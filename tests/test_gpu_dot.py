@@ -532,3 +532,30 @@ def test_millions_of_rows_against_a_tiny_matrix(hip):
     b = rng.integers(-8, 9, size=(3, 3)).astype(np.float32)
     got = hip.to_numpy(Nx.dot(from_numpy(a, "f32", hip), from_numpy(b, "f32", hip)))
     assert np.array_equal(got, a @ b)
+
+
+@pytest.mark.parametrize("ty", ["f64", "s32", "u8", "s64"])
+@pytest.mark.parametrize("layout", ["nn", "nt", "tn", "tt"])
+def test_plain_kernel_on_64_tiles(ty, layout, hip, oracle):
+    """Types without a matrix-core path (f64, wide integers) on tiles of 64 x 64 with sixteen outputs per lane, from 512
+    tiles on: every output is still accumulated over k in order, so integers are exact and f64 agrees with the oracle's
+    sequential f64 sum bit for bit.  Shapes off the tile and K-step grids."""
+    M, N, K = 1500, 1400, 37
+    rng = np.random.default_rng(seed_of(ty, layout, "plain 64"))
+    if ty == "f64":
+        a, b = rng.standard_normal((M, K)), rng.standard_normal((K, N))
+    else:
+        dt = T.numpy_dtype(T.normalize(ty))
+        lo, hi = (0, 200) if ty == "u8" else (-1000, 1000)
+        a, b = rng.integers(lo, hi, size=(M, K)).astype(dt), rng.integers(lo, hi, size=(K, N)).astype(dt)
+    la = a if layout[0] == "n" else np.ascontiguousarray(a.T)
+    lb = b if layout[1] == "n" else np.ascontiguousarray(b.T)
+    c1 = [1] if layout[0] == "n" else [0]
+    c2 = [0] if layout[1] == "n" else [1]
+    got = Nx.dot(from_numpy(la, ty, hip), c1, from_numpy(lb, ty, hip), c2)
+    rows = np.unique(np.concatenate([[0, 63, 64, M - 1], rng.integers(0, M, size=8)]))
+    want = Nx.dot(from_numpy(np.ascontiguousarray(a[rows]), ty, oracle), from_numpy(b, ty, oracle))
+    assert_bits_equal(from_numpy(np.ascontiguousarray(hip.to_numpy(got)[rows]), ty, oracle), want, f"plain 64 {ty} {layout}")
+    if ty != "f64":
+        wide = (a.astype(np.int64) @ b.astype(np.int64)).astype(T.numpy_dtype(T.normalize(ty)))
+        assert np.array_equal(hip.to_numpy(got), wide)
