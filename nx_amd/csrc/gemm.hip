@@ -150,6 +150,27 @@ dot_generic_kernel(const void *__restrict__ l, const void *__restrict__ r, void 
   if (m < M && n < N) store_one<CT>(out, odt, b * M * N + m * N + n, acc);
 }
 
+// Many small matrices (a 3 x 3 transform per point, a 4 x 4 block per item): one lane per output over the whole batch,
+// walking k in order -- the tiled kernel above spends a work-group of 256 lanes on each item's nine outputs.
+template <typename CT>
+__global__ void __launch_bounds__(256)
+dot_small_batched_kernel(const void *__restrict__ l, const void *__restrict__ r, void *__restrict__ out, int ldt, int rdt,
+                         int odt, int64_t batch, int M, int N, int K, int lk, int rk) {
+  const int64_t total = batch * M * N;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t b = i / (M * N);
+    const int mn = (int)(i - b * (M * N)), m = mn / N, n = mn - m * N;
+    const int64_t lbase = b * M * K, rbase = b * N * K;
+    CT acc = 0;
+    for (int k = 0; k < K; k++) {
+      const CT x = load_one<CT>(l, ldt, lbase + (lk ? m * K + k : k * M + m)), y = load_one<CT>(r, rdt, rbase + (rk ? n * K + k : k * N + n));
+      if constexpr (std::is_same<CT, double>::value) acc = x * y + acc;
+      else acc = (int64_t)((uint64_t)x * (uint64_t)y + (uint64_t)acc);
+    }
+    store_one<CT>(out, odt, i, acc);
+  }
+}
+
 // The same contraction on 64 x 64 tiles with 4 x 4 outputs per lane: eight LDS reads per sixteen multiply-adds
 // instead of two per one, each output still accumulated over k in order (the same bits as the kernel above).
 // f64 / s32 / mixed-type 4096^3: 8.4 TFLOP/s there.
@@ -496,6 +517,16 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
       if ((N + 15) / 16 > 65535 || (M + 15) / 16 >= (1ll << 31) / 256)
         return set_error(HIPNX_EUNSUPPORTED, "dot: more than a million columns (or 134 million rows) on the plain kernel");
       const int lk = l_layout == HIPNX_K_INNER, rk = r_layout == HIPNX_K_INNER;
+      if (M * N <= 64 && K <= 64 && batch >= 64) {  // many small matrices: a lane per output
+        const int64_t blocks = (batch * M * N + 255) / 256;
+        dim3 gs((unsigned)(blocks < (1ll << 24) - 1 ? blocks : (1ll << 24) - 1));
+        if (any_float)
+          hipLaunchKernelGGL((dot_small_batched_kernel<double>), gs, block, 0, ctx->stream, l->ptr, r->ptr, out->ptr, l_dt, r_dt, out_dt, batch, (int)M, (int)N, (int)K, lk, rk);
+        else
+          hipLaunchKernelGGL((dot_small_batched_kernel<int64_t>), gs, block, 0, ctx->stream, l->ptr, r->ptr, out->ptr, l_dt, r_dt, out_dt, batch, (int)M, (int)N, (int)K, lk, rk);
+        HIPNX_HIP(hipGetLastError());
+        return HIPNX_OK;
+      }
       // tiles of 64 x 64, sixteen outputs per lane, where they still give every CU two work-groups (512^3: 64 tiles, 143 us
       // against 53 us on 16 x 16 tiles)
       if (M >= 64 && N >= 64 && (N + 63) / 64 <= 65535 && ((M + 63) / 64) * ((N + 63) / 64) * batch >= 2 * (int64_t)ctx->num_cus) {

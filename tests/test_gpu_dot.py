@@ -559,3 +559,23 @@ def test_plain_kernel_on_64_tiles(ty, layout, hip, oracle):
     if ty != "f64":
         wide = (a.astype(np.int64) @ b.astype(np.int64)).astype(T.numpy_dtype(T.normalize(ty)))
         assert np.array_equal(hip.to_numpy(got), wide)
+
+
+@pytest.mark.parametrize("M,K,N", [(3, 3, 1), (4, 4, 4), (1, 7, 5), (8, 2, 8), (2, 64, 2)])
+@pytest.mark.parametrize("ty", ["f32", "bf16", "s32", "f64"])
+def test_many_small_matrices(M, K, N, ty, hip, oracle):
+    """A batch of small matrices takes one lane per output over the whole batch; k in order, so the oracle's bits."""
+    rng = np.random.default_rng(seed_of(M, K, N, ty, "small batched"))
+    Bn = 777
+    if ty == "s32":
+        a, b = rng.integers(-99, 99, size=(Bn, M, K)).astype(np.int32), rng.integers(-99, 99, size=(Bn, K, N)).astype(np.int32)
+    else:
+        a, b = rand_raw(rng, ty, (Bn, M, K), lo=-2, hi=2), rand_raw(rng, ty, (Bn, K, N), lo=-2, hi=2)
+    ha, oa = both(a, ty, hip, oracle)
+    hb, ob = both(b, ty, hip, oracle)
+    assert_bits_equal(Nx.dot(ha, [2], [0], hb, [1], [0]), Nx.dot(oa, [2], [0], ob, [1], [0]), f"small batched {ty} {M}x{K}x{N}")
+    # the other layouts: contract the first axis of the left operand, the last of the right
+    at, bt = np.ascontiguousarray(a.transpose(0, 2, 1)), np.ascontiguousarray(b.transpose(0, 2, 1))
+    hat, oat = both(at, ty, hip, oracle)
+    hbt, obt = both(bt, ty, hip, oracle)
+    assert_bits_equal(Nx.dot(hat, [1], [0], hbt, [2], [0]), Nx.dot(oat, [1], [0], obt, [2], [0]), f"small batched tt {ty}")
