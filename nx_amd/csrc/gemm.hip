@@ -475,7 +475,11 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
     }
 
     // at most 32 x 32 outputs over a contraction of 4096 elements or more: the reduction kernels
-    if (!k_use && !scaled && M <= 32 && N <= 32 && (K >= 4096 || (M * N <= 4 && K >= 128)) && batch * M * N <= 65535 && !(!is_float(l_dt) && !is_float(r_dt) && is_float(out_dt))) {
+    // (also a matrix against one to four vectors in f32 or wider types, where the matrix is contiguous along k: an MFMA
+    // tile would be all but empty, and its f32 work costs more than the bytes -- [1, 8192] . [8192, 8192]^T 105 us)
+    const bool few_vectors = dtype_size(l_dt) >= 4 && dtype_size(r_dt) >= 4 && K >= 1024 &&
+                             ((M <= 4 && r_layout == HIPNX_K_INNER) || (N <= 4 && l_layout == HIPNX_K_INNER));
+    if (!k_use && !scaled && ((M <= 32 && N <= 32 && (K >= 4096 || (M * N <= 4 && K >= 128))) || few_vectors) && M * N <= 65535 && batch * M * N <= 65535 && !(!is_float(l_dt) && !is_float(r_dt) && is_float(out_dt))) {
       const bool any_float = is_float(l_dt) || is_float(r_dt);
       const int lk = l_layout == HIPNX_K_INNER, rk = r_layout == HIPNX_K_INNER;
       const int64_t l_sm = lk ? K : 1, l_sk = lk ? 1 : M, r_sn = rk ? K : 1, r_sk = rk ? 1 : N;

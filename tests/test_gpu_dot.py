@@ -579,3 +579,33 @@ def test_many_small_matrices(M, K, N, ty, hip, oracle):
     hat, oat = both(at, ty, hip, oracle)
     hbt, obt = both(bt, ty, hip, oracle)
     assert_bits_equal(Nx.dot(hat, [1], [0], hbt, [2], [0]), Nx.dot(oat, [1], [0], obt, [2], [0]), f"small batched tt {ty}")
+
+
+@pytest.mark.parametrize("S,R,K", [(1, 4096, 1024), (4, 1000, 300), (2, 257, 5000), (3, 70000, 256)])
+@pytest.mark.parametrize("ty", ["f32", "f64", "s32"])
+@pytest.mark.parametrize("side", ["vectors_left", "vectors_right"])
+@pytest.mark.parametrize("small_layout", ["k_inner", "k_outer"])
+def test_a_few_vectors_against_a_matrix(S, R, K, ty, side, small_layout, hip, oracle):
+    """A few vectors against a matrix in f32 and wider types: with the matrix stored [N, K] (contiguous along k) the
+    reduction kernel, a work-group per output; stored [K, N] the tiled kernels.  Integers exact, floats in the bound."""
+    rng = np.random.default_rng(seed_of(S, R, K, ty, side, small_layout, "few vectors"))
+    if ty == "s32":
+        small, big = rng.integers(-99, 99, size=(S, K)).astype(np.int32), rng.integers(-99, 99, size=(K, R)).astype(np.int32)
+    else:
+        small, big = rand_raw(rng, ty, (S, K), lo=-1, hi=1), rand_raw(rng, ty, (K, R), lo=-1, hi=1)
+    for big_layout in ("k_outer", "k_inner"):
+        sm = small if small_layout == "k_inner" else np.ascontiguousarray(small.T)
+        bg = big if big_layout == "k_outer" else np.ascontiguousarray(big.T)
+        cs, cb = ([1] if small_layout == "k_inner" else [0]), ([0] if big_layout == "k_outer" else [1])
+        hs, os_ = both(sm, ty, hip, oracle)
+        hb, ob = both(bg, ty, hip, oracle)
+        if side == "vectors_left":
+            got, want, eq = Nx.dot(hs, cs, hb, cb), Nx.dot(os_, cs, ob, cb), "sk,kr->sr"
+            a64, b64 = values(from_numpy(small, ty, oracle)), values(from_numpy(big, ty, oracle))
+        else:
+            got, want, eq = Nx.dot(hb, cb, hs, cs), Nx.dot(ob, cb, os_, cs), "kr,sk->rs"
+            a64, b64 = values(from_numpy(big, ty, oracle)), values(from_numpy(small, ty, oracle))
+        if ty == "s32":
+            assert_bits_equal(got, want, f"few vectors s32 {side} {big_layout}")
+        else:
+            check_float_dot(got, want, a64, b64, eq, K, f"few vectors {ty} {side} {small_layout} {big_layout}")
