@@ -223,11 +223,14 @@ int hipnx_argreduce(hipnx_ctx *ctx, int op, int tie, int in_dt, int out_dt, int6
  * torchx/c_src/torchx.cpp:844-890 tensordot).
  * out[b, m, n] = sum_k l[b, m, k] * r[b, n, k]; l is [batch, M, K] (HIPNX_K_INNER) or
  * [batch, K, M] (HIPNX_K_OUTER), r is [batch, N, K] or [batch, K, N]; out is [batch, M, N] in
- * out_dt (f32 accumulation for f16/bf16/f32 operands, exact s32 for s8, then one encode).
- * out_dt may be HIPNX_BF16_RNE (bf16 rounded to nearest even).  The call may take workspace from the
- * context's pool and return it before it ends: a re-laid operand whose K-outer rows are not whole
- * 16-byte blocks, zero-extended copies of both operands when K is not a whole number of 128-byte slabs,
- * the partial results of a contraction whose K is split over several work-groups per tile. */
+ * out_dt (f32 accumulation for f16/bf16/f32 operands, exact s32 for s8, then one encode; f64, wider integers and
+ * mixed operand types accumulate in f64 / wrapping 64-bit integers over k in order, as do a handful of outputs over
+ * a long K -- the dot of two vectors -- whose segments of K are summed in f64).
+ * out_dt may be HIPNX_BF16_RNE (bf16 rounded to nearest even).  Any batch count is taken (beyond 65535 items in
+ * several launches).  The call may take workspace from the context's pool and return it before it ends: a re-laid
+ * operand whose K-outer rows are not whole 16-byte blocks, one-slab zero-extended copies of the last part of K when K
+ * is not a whole number of 128-byte slabs (copies of both operands where their rows are not whole 16-byte blocks
+ * either), the partial results of a contraction whose K is split over several work-groups per tile or output. */
 int hipnx_dot(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batch, int64_t M, int64_t N,
               int64_t K, int l_layout, int r_layout, const hipnx_buf *l, const hipnx_buf *r,
               hipnx_buf *out);
