@@ -514,6 +514,21 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
       return HIPNX_OK;
     }
 
+    // many small matrices (up to 64 outputs, K up to 64): a lane per output over the whole batch (16 x 16 x 16 items are
+    // faster on the tiled kernels: 51 us against 175 us for 8192 of them)
+    if (!scaled && !k_use && M * N <= 64 && K <= 64 && batch >= 64 && !(!is_float(l_dt) && !is_float(r_dt) && is_float(out_dt))) {
+      const bool any_float = is_float(l_dt) || is_float(r_dt);
+      const int lk = l_layout == HIPNX_K_INNER, rk = r_layout == HIPNX_K_INNER;
+      const int64_t blocks = (batch * M * N + 255) / 256;
+      dim3 gs((unsigned)(blocks < (1ll << 24) - 1 ? blocks : (1ll << 24) - 1)), block(256);
+      if (any_float)
+        hipLaunchKernelGGL((dot_small_batched_kernel<double>), gs, block, 0, ctx->stream, l->ptr, r->ptr, out->ptr, l_dt, r_dt, out_dt, batch, (int)M, (int)N, (int)K, lk, rk);
+      else
+        hipLaunchKernelGGL((dot_small_batched_kernel<int64_t>), gs, block, 0, ctx->stream, l->ptr, r->ptr, out->ptr, l_dt, r_dt, out_dt, batch, (int)M, (int)N, (int)K, lk, rk);
+      HIPNX_HIP(hipGetLastError());
+      return HIPNX_OK;
+    }
+
     if (!mfma) {
       const bool any_float = is_float(l_dt) || is_float(r_dt);
       if (!any_float && is_float(out_dt)) return set_error(HIPNX_EUNSUPPORTED, "dot: integer operands with a float output");
@@ -521,16 +536,6 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
       if ((N + 15) / 16 > 65535 || (M + 15) / 16 >= (1ll << 31) / 256)
         return set_error(HIPNX_EUNSUPPORTED, "dot: more than a million columns (or 134 million rows) on the plain kernel");
       const int lk = l_layout == HIPNX_K_INNER, rk = r_layout == HIPNX_K_INNER;
-      if (M * N <= 64 && K <= 64 && batch >= 64) {  // many small matrices: a lane per output
-        const int64_t blocks = (batch * M * N + 255) / 256;
-        dim3 gs((unsigned)(blocks < (1ll << 24) - 1 ? blocks : (1ll << 24) - 1));
-        if (any_float)
-          hipLaunchKernelGGL((dot_small_batched_kernel<double>), gs, block, 0, ctx->stream, l->ptr, r->ptr, out->ptr, l_dt, r_dt, out_dt, batch, (int)M, (int)N, (int)K, lk, rk);
-        else
-          hipLaunchKernelGGL((dot_small_batched_kernel<int64_t>), gs, block, 0, ctx->stream, l->ptr, r->ptr, out->ptr, l_dt, r_dt, out_dt, batch, (int)M, (int)N, (int)K, lk, rk);
-        HIPNX_HIP(hipGetLastError());
-        return HIPNX_OK;
-      }
       // tiles of 64 x 64, sixteen outputs per lane, where they still give every CU two work-groups (512^3: 64 tiles, 143 us
       // against 53 us on 16 x 16 tiles)
       if (M >= 64 && N >= 64 && (N + 63) / 64 <= 65535 && ((M + 63) / 64) * ((N + 63) / 64) * batch >= 2 * (int64_t)ctx->num_cus) {
