@@ -104,6 +104,7 @@ PROTOTYPES = {
     "hipnx_select": [_ctx_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _i64p, _i64p, _i64p, _i64p, _buf_p, _buf_p,
                      _buf_p, _buf_p],
     "hipnx_clip": [_ctx_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int64, _buf_p, _buf_p, _buf_p, _buf_p],
+    "hipnx_concat": [_ctx_p, C.c_int, C.c_int, C.POINTER(_buf_p), _i64p, C.c_int64, C.c_int64, _buf_p],
     "hipnx_strided_copy": [_ctx_p, C.c_int, C.c_int, _i64p, _i64p, C.c_int64, _i64p, C.c_int64, _buf_p, _buf_p],
     "hipnx_iota": [_ctx_p, C.c_int, C.c_int64, C.c_int64, C.c_int64, _buf_p],
     "hipnx_eye": [_ctx_p, C.c_int, C.c_int64, C.c_int64, C.c_int64, _buf_p],

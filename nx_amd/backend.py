@@ -825,6 +825,17 @@ class HipNxBackend:
         converted to the output type and copied into its window along `axis`."""
         dev = cls._device_of(*tensors)
         res = cls._alloc(out, dev)
+        if not T.is_sub_byte(out.type) and len(tensors) > 1:
+            # one launch per 64 operands: the tensors viewed as [outer, their extent along the axis, inner]
+            parts = []
+            for t in tensors:
+                t = cls._from_nx(t, dev)
+                parts.append(t if t.type == out.type else cls.as_type(t.with_(data=None, type=out.type), t))
+            handles = (L._buf_p * len(parts))(*[cls._handle(t) for t in parts])
+            L.check(L.lib.hipnx_concat(res.data.ref.ctx, T.size_bytes(out.type), len(parts), handles,
+                                       L.i64_array([t.shape[axis] for t in parts]), prod(out.shape[:axis]), prod(out.shape[axis + 1:]),
+                                       res.data.ref.handle))
+            return res
         out_strides = cls._dense_strides(out.shape)
         offset = 0
         for t in tensors:

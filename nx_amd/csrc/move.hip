@@ -776,6 +776,87 @@ extern "C" int hipnx_gather(hipnx_ctx *ctx, int elem_bytes, int rank, const int6
   return gather_run(ctx, idx_dt, n_tuples, depth, oob_policy, t, idx, out, td, slice_bytes, 0, 0, rank, t_dims);
 }
 
+// concatenate: parts [outer, a_i, inner] -> out [outer, sum a_i, inner], up to 64 parts per launch (their pointers
+// and where each begins within a row of the output travel as kernel arguments).  One launch per part cost 6 us of
+// host time each: 64 parts of 2 MiB 425 us, 256 small ones 1.5 ms.
+constexpr int CONCAT_PARTS = 64;
+struct ConcatArgs {
+  const unsigned char *src[CONCAT_PARTS];
+  int64_t begin[CONCAT_PARTS + 1];  // bytes from the start of an output row to the part (last entry: end of the last part)
+  int n;
+};
+
+template <int W>
+__global__ void __launch_bounds__(BLOCK)
+concat_kernel(ConcatArgs a, unsigned char *__restrict__ out, int64_t outer, int64_t row_bytes) {
+  typedef raw_vec<W> vec_t;
+  const int64_t first = a.begin[0], span = a.begin[a.n] - first;  // this launch's share of an output row
+  const int64_t per_row = span / W, total = outer * per_row;
+  for (int64_t v = (int64_t)blockIdx.x * BLOCK + threadIdx.x; v < total; v += (int64_t)gridDim.x * BLOCK) {
+    const int64_t o = v / per_row, within = first + (v - o * per_row) * W;
+    int lo = 0, hi = a.n - 1;  // the last part that begins at or before `within`
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (a.begin[mid] <= within) lo = mid;
+      else hi = mid - 1;
+    }
+    const int64_t len = a.begin[lo + 1] - a.begin[lo];
+    *reinterpret_cast<vec_t *>(out + o * row_bytes + within) =
+        *reinterpret_cast<const vec_t *>(a.src[lo] + o * len + (within - a.begin[lo]));
+  }
+}
+
+extern "C" int hipnx_concat(hipnx_ctx *ctx, int elem_bytes, int n_parts, const hipnx_buf *const *parts, const int64_t *extents,
+                            int64_t outer, int64_t inner, hipnx_buf *out) {
+  Enter in(ctx);
+  if (in.status) return in.status;
+  if (elem_bytes <= 0 || n_parts < 0 || outer < 0 || inner < 0 || (n_parts > 0 && (!parts || !extents)))
+    return set_error(HIPNX_EINVAL, "concat: bad argument");
+  int64_t sum = 0;
+  for (int p = 0; p < n_parts; p++) {
+    if (extents[p] < 0) return set_error(HIPNX_EINVAL, "concat: negative extent");
+    if (int st = check_buf(ctx, parts[p], (uint64_t)outer * extents[p] * inner * elem_bytes, "concat part")) return st;
+    sum += extents[p];
+  }
+  const int64_t row_bytes = sum * inner * elem_bytes;
+  if (int st = check_buf(ctx, out, (uint64_t)outer * row_bytes, "concat out")) return st;
+  if (outer * row_bytes == 0) return HIPNX_OK;
+  // the widest access that every part's row and address allows
+  int width = 16;
+  uintptr_t bits = reinterpret_cast<uintptr_t>(out->ptr) | (uintptr_t)row_bytes;
+  for (int p = 0; p < n_parts; p++)
+    if (extents[p] > 0) bits |= reinterpret_cast<uintptr_t>(parts[p]->ptr) | (uintptr_t)(extents[p] * inner * elem_bytes);
+  while (width > 1 && (bits & (uintptr_t)(width - 1))) width >>= 1;
+  int64_t begin = 0;
+  int p = 0;
+  while (p < n_parts) {
+    ConcatArgs a;
+    a.n = 0;
+    while (p < n_parts && a.n < CONCAT_PARTS) {
+      if (extents[p] > 0) {
+        a.src[a.n] = (const unsigned char *)parts[p]->ptr;
+        a.begin[a.n] = begin;
+        a.n++;
+        begin += extents[p] * inner * elem_bytes;
+      }
+      p++;
+    }
+    if (a.n == 0) break;
+    a.begin[a.n] = begin;
+    const int64_t total = outer * ((a.begin[a.n] - a.begin[0]) / width);
+    dim3 grid(grid_for(ctx, total, BLOCK)), block(BLOCK);
+    switch (width) {
+      case 16: hipLaunchKernelGGL((concat_kernel<16>), grid, block, 0, ctx->stream, a, (unsigned char *)out->ptr, outer, row_bytes); break;
+      case 8: hipLaunchKernelGGL((concat_kernel<8>), grid, block, 0, ctx->stream, a, (unsigned char *)out->ptr, outer, row_bytes); break;
+      case 4: hipLaunchKernelGGL((concat_kernel<4>), grid, block, 0, ctx->stream, a, (unsigned char *)out->ptr, outer, row_bytes); break;
+      case 2: hipLaunchKernelGGL((concat_kernel<2>), grid, block, 0, ctx->stream, a, (unsigned char *)out->ptr, outer, row_bytes); break;
+      default: hipLaunchKernelGGL((concat_kernel<1>), grid, block, 0, ctx->stream, a, (unsigned char *)out->ptr, outer, row_bytes); break;
+    }
+  }
+  HIPNX_HIP(hipGetLastError());
+  return HIPNX_OK;
+}
+
 extern "C" int hipnx_take(hipnx_ctx *ctx, int elem_bytes, int64_t outer, int64_t axis_len, int64_t inner, int idx_dt,
                           int64_t n_idx, int oob_policy, int rank, const int64_t *msg_dims, const hipnx_buf *t,
                           const hipnx_buf *idx, hipnx_buf *out) {

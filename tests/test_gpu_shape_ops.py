@@ -245,3 +245,31 @@ def test_iota_beyond_the_exact_integers_of_f32(ty, hip, oracle):
     tail = Nx.slice(got, [n - 4096], [4096])
     want = Nx.slice(Nx.iota((n,), type=ty, backend=oracle), [n - 4096], [4096])
     assert_bits_equal(tail, want, f"iota {ty} tail")
+
+
+@pytest.mark.parametrize("ty", ["u8", "bf16", "f32", "s64"])
+@pytest.mark.parametrize("axis", [0, 1, 2])
+def test_concatenate_of_many_operands_is_a_launch_per_64(ty, axis, hip):
+    """150 operands of different (some odd, one empty) extents along the axis go in three launches, each operand found by
+    where it begins within an output row; a stack of 70; an operand of another type is converted first.  Bit for bit
+    against numpy."""
+    import numpy as np
+    from nx_amd import nx as Nx
+    from nx_amd import types as T
+    from support import from_numpy
+    rng = np.random.default_rng(axis * 7 + len(ty))
+    dt = T.numpy_dtype(T.normalize(ty))
+    base = [3, 5, 4]
+    parts = []
+    for i in range(150):
+        shape = list(base)
+        shape[axis] = 0 if i == 17 else int(rng.integers(1, 9))
+        parts.append(rng.integers(0, 200, size=shape).astype(dt) if ty != "bf16" else rng.integers(0, 60000, size=shape).astype(np.uint16))
+    got = Nx.concatenate([from_numpy(p, ty, hip) for p in parts], axis=axis)
+    assert np.array_equal(hip.to_numpy(got).view(np.uint8), np.concatenate(parts, axis=axis).view(np.uint8))
+    same = [rng.integers(0, 200, size=(4, 7)).astype(dt) if ty != "bf16" else rng.integers(0, 60000, size=(4, 7)).astype(np.uint16) for _ in range(70)]
+    stacked = Nx.stack([from_numpy(p, ty, hip) for p in same], axis=1)
+    assert np.array_equal(hip.to_numpy(stacked).view(np.uint8), np.stack(same, axis=1).view(np.uint8))
+    if ty == "f32":
+        mixed = Nx.concatenate([from_numpy(np.arange(6, dtype=np.float32).reshape(2, 3), "f32", hip), from_numpy(np.arange(4, dtype=np.int32).reshape(2, 2), "s32", hip)], axis=1)
+        assert hip.to_numpy(mixed).tolist() == [[0.0, 1.0, 2.0, 0.0, 1.0], [3.0, 4.0, 5.0, 2.0, 3.0]]
