@@ -825,8 +825,9 @@ class HipNxBackend:
         converted to the output type and copied into its window along `axis`."""
         dev = cls._device_of(*tensors)
         res = cls._alloc(out, dev)
-        if not T.is_sub_byte(out.type) and len(tensors) > 1:
-            # one launch per 64 operands: the tensors viewed as [outer, their extent along the axis, inner]
+        if not T.is_sub_byte(out.type) and len(tensors) >= 4:
+            # one launch per 64 operands: the tensors viewed as [outer, their extent along the axis, inner] (two or three
+            # large operands are a little faster as a copy each: 16384^2 f32 twice 0.70 ms against 0.76 ms)
             parts = []
             for t in tensors:
                 t = cls._from_nx(t, dev)
