@@ -5,8 +5,9 @@
 
 Headline workload (the configuration the metric is quoted on): `Nx.dot` of bf16 {4096,4096} x
 {4096,4096}, f32 accumulation on MFMA, bf16 output -- one step = one `dot` callback through the
-C ABI, inputs resident in HBM.  Prints ONE JSON line; `value` is TFLOP/s over K timed steps
-(wall clock between two device synchronisations).  `roofline` is measured live with HIP events on
+C ABI, inputs resident in HBM.  The LAST stdout line is the headline as JSON (under 4 KB); a table of the
+suite precedes it and the full record is written to gpurun_out/bench_suite.json.  `value` is TFLOP/s over
+K timed steps (wall clock between two device synchronisations).  `roofline` is measured live with HIP events on
 the stream the kernels are launched on.  `suite` carries the other configurations (GB/s or
 TFLOP/s and their roofline fractions), `cpu_baseline` the CPU restatement of the reference on a
 bounded sample of the same workload.  `--calibrate` first launches a streaming kernel of known
@@ -34,6 +35,11 @@ TRAFFIC_PROFILE = os.path.join("profiles", "dot_bf16_4096_hbm_traffic.md")
 TRAFFIC_PROFILE_S8 = os.path.join("profiles", "dot_s8_4096_hbm_traffic.md")
 CEILINGS_BIN = os.path.join(ROOT, "nx_amd", "lib", "hipnx_ceilings")
 ABI_DRIVER_BIN = os.path.join(ROOT, "nx_amd", "lib", "hipnx_abi_driver")
+# suite entries whose roofline fraction is repeated in the headline line (the rest stay in the detail file)
+HEADLINE_ALSO = ("dot_s8_4096_s32", "dot_bf16_4096_kinner", "dot_f32_2048", "dot_s8_w8_64x11008x4096_rotated",
+                 "dot_qk_bf16_32x512x64_rotated", "softmax_chain_32x512x512_rotated", "config1_chain_f32_1024",
+                 "config1_chain_f32_16384", "add_f32_16384", "sum_rows_f32_16384", "argmax_f32_8192x32000",
+                 "take_bf16_8192_of_32000x4096_rotated", "config4_chain_rotated")
 
 
 def host_transfer_figures(H, B, Nx, template):
@@ -666,7 +672,46 @@ def main():
             "vectorised_library": vectorised,
             "other_configurations": per_config}
 
-    print(json.dumps(result))
+    emit(result)
+
+
+def emit(result):
+    """The full record (suite, ceilings, host transfers, plain-C figures, the CPU baseline's extras) goes to
+    `gpurun_out/bench_suite.json` and, as a short table, to stdout; the LAST stdout line is the headline
+    alone, a few hundred bytes of JSON that a reader of the output's tail can parse."""
+    detail_path = os.path.join(ROOT, "gpurun_out", "bench_suite.json")
+    try:
+        os.makedirs(os.path.dirname(detail_path), exist_ok=True)
+        with open(detail_path, "w") as f:
+            json.dump(result, f)
+    except OSError as exc:  # a read-only tree: the table below still carries the figures
+        detail_path = "not written: " + str(exc)[:80]
+    suite = result.get("suite", {})
+    if suite:
+        print("%-58s %10s %10s %9s %6s %6s" % ("suite entry (device time per call)", "us", "achieved", "unit", "frac", "bound"))
+        for name, e in suite.items():
+            print("%-58s %10.2f %10.1f %9s %6.3f %6s" % (name, e["ms"] * 1e3, e["achieved"], e["unit"], e["frac"], e["bound"]))
+    for name, c in result.get("ceilings", {}).items():
+        if "sustained" in c:
+            print("ceiling %-50s %10s sustained" % (name, c["sustained"]))
+    head = {k: result[k] for k in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better",
+                                   "scaling", "vs_baseline", "dtype", "data", "config", "roofline")}
+    cpu = result.get("cpu_baseline")
+    if cpu:
+        head["cpu_baseline"] = {k: cpu[k] for k in ("value", "unit", "cores", "kind", "sample")}
+    head["cold_start"] = result["cold_start"]["tflops"]
+    # the other figures the targets are stated on, one fraction each (full entries in the detail file)
+    also = {}
+    for name in HEADLINE_ALSO:
+        if name in suite:
+            also[name] = {"us": round(suite[name]["ms"] * 1e3, 2), "frac": suite[name]["frac"], "of": suite[name]["bound"]}
+    if also:
+        head["also"] = also
+    head["detail"] = "gpurun_out/bench_suite.json" if not detail_path.startswith("not written") else detail_path
+    line = json.dumps(head)
+    assert len(line) < 4096, "headline JSON line is %d bytes: keep it under 4 KB" % len(line)
+    sys.stdout.flush()
+    print(line, flush=True)
 
 
 if __name__ == "__main__":

@@ -13,11 +13,13 @@
  * nearest even and *raises* when a finite value overflows, bf16 is the f32 encoding with the
  * low 16 bits dropped, atoms become canonical bit patterns (type.ex:128-158).
  *
- * Parity pinning status of the pieces (what independent evidence fixes them) is recorded in
- * the test-suite next to the golden vectors; functions whose last-bit behaviour lives in the
- * un-vendored `complex` 0.7.0 package (erf, erfc, cbrt, erf_inv at and beyond +-1, pow/atan2/divide on
- * non-finite or zero operands, fmod corner cases) are "parity unpinned": they follow IEEE /
- * libm here.
+ * Parity pinning status: every function here is checked against answers the reference's own
+ * doctests and tests hold (tests/golden/, each with file:line; sum, product, reduce_max/min,
+ * argmax/argmin, dot, gather, as_type and the element-wise callbacks all have cases there) and
+ * against closed forms, arbitrary-precision values and brute force (tests/test_oracle_*.py).
+ * "Parity unpinned" remains only what the un-vendored `complex` 0.7.0 package alone could
+ * settle: the last bit of erf, erfc and cbrt, and erf_inv at and beyond +-1; they follow a
+ * correctly rounded routine / IEEE here.
  *
  * Build: gcc -O2 -ffp-contract=off -fopenmp -shared -fPIC hipnx_ref.c -lm
  * (-ffp-contract=off is required: the reference multiplies and adds in two roundings.)

@@ -219,3 +219,45 @@ def test_f16_codec_against_the_reference_table_of_shortest_decimals(oracle):
     assert np.array_equal(decoded[finite], bits[finite].view(np.float16).astype(np.float64))
     for t, d in zip(np.array(text)[~finite], decoded[~finite]):
         assert (np.isnan(d) and "NaN" in t) or (np.isinf(d) and (d < 0) == t.startswith("-"))
+
+
+def test_product_wraps_exact_integers_and_rounds_a_float_fold_once(oracle):
+    """`product` (nx/lib/nx/binary_backend.ex:1327-1335): fold `acc = x * acc` from integer 1 over unbounded
+    integers / f64 in row-major order of the reduced axes, encoded once to the aggregate type."""
+    import math
+    # s32 operands whose exact product exceeds 2^31: the low 32 bits of the unbounded product (no saturation,
+    # no early wrap that a narrower intermediate would show differently for a later zero-crossing factor)
+    x = np.array([65537, 65539, -3, 7, 11], dtype=np.int32)
+    exact = math.prod(int(v) for v in x)
+    want = ((exact + 2 ** 31) % 2 ** 32) - 2 ** 31
+    assert abs(exact) > 2 ** 31
+    assert raw(Nx.product(t(x, "s32", oracle))).item() == want
+    # u8 -> u32: 255^5 wraps modulo 2^32, it does not saturate
+    u = np.full(5, 255, dtype=np.uint8)
+    assert raw(Nx.product(t(u, "u8", oracle))).item() == 255 ** 5 % 2 ** 32
+    # per axis against exact arithmetic, brute force
+    rng = np.random.default_rng(12)
+    a = rng.integers(-50, 50, size=(3, 4, 5)).astype(np.int32)
+    for axis in range(3):
+        got = raw(Nx.product(t(a, "s32", oracle), axes=[axis])).astype(np.int64)
+        ex = np.empty(got.shape, dtype=object)
+        moved = np.moveaxis(a, axis, -1)
+        for idx in np.ndindex(*moved.shape[:-1]):
+            ex[idx] = ((math.prod(int(v) for v in moved[idx]) + 2 ** 31) % 2 ** 32) - 2 ** 31
+        assert np.array_equal(got, ex.astype(np.int64)), axis
+    # f32: the fold runs in f64 and is rounded to f32 ONCE: factors of 1 + 2^-12 keep bits in f64 that an f32
+    # fold loses (the f32 fold of these forty factors ends one f32 ulp below the f64 one)
+    f = np.full(40, 1.0 + 2.0 ** -12, dtype=np.float32)
+    acc64 = 1.0
+    acc32 = np.float32(1.0)
+    for v in f:
+        acc64 = float(v) * acc64
+        acc32 = np.float32(v) * acc32
+    want32 = np.float32(acc64)
+    assert want32 != acc32  # the case separates the two formulations
+    assert raw(Nx.product(t(f, "f32", oracle))).item() == want32
+    # sequential from index zero: 1e-200 * 1e-200 underflows to 0 first and stays 0; the reverse order never
+    # leaves the f64 range (1e300 * 1e-200 = 1e100, then * 1e-200)
+    g = np.array([1e-200, 1e-200, 1e300], dtype=np.float64)
+    assert values(Nx.product(t(g, "f64", oracle))).item() == 0.0
+    assert values(Nx.product(t(g[::-1].copy(), "f64", oracle))).item() == (1e300 * 1e-200) * 1e-200
