@@ -157,7 +157,9 @@ int hipnx_buf_wrap(hipnx_ctx *ctx, void *device_ptr, size_t bytes, hipnx_buf **o
  * wrapped or imported one) and hold less than 2 GiB.  `import` gives a handle over the exporter's
  * memory; destroying it closes the mapping and never frees the memory, which the exporter keeps alive
  * while the importer uses it.  Opening a handle in the process that exported it is an error of the
- * HIP runtime and is reported as such. */
+ * HIP runtime and is reported as such.  What an importer writes through the handle (hipnx_h2d, a
+ * kernel's output) is in flight on ITS context's stream when the call returns: the exporter may read it
+ * only after the writing process has called hipnx_sync (and told the exporter so). */
 #define HIPNX_IPC_HANDLE_BYTES 64
 int hipnx_buf_ipc_export(hipnx_ctx *ctx, const hipnx_buf *buf, void *handle_out);
 int hipnx_buf_ipc_import(hipnx_ctx *ctx, const void *handle, size_t bytes, hipnx_buf **out);
@@ -203,9 +205,15 @@ int hipnx_reduce(hipnx_ctx *ctx, int op, int in_dt, int out_dt, int64_t outer, i
 
 /* No counterpart in the reference: hipnx_reduce for callers that cannot allocate device memory
  * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  Same
- * arguments, same kernels, same results bit for bit; the partial results of a split reduction go
+ * arguments and kernels; the partial results of a split reduction go
  * to a static device array of HIPNX_REDUCE_STATIC_SCRATCH_BYTES (held by every GPU the library runs
  * on until the process ends) instead of a pool block, and the call performs no hipMalloc / hipFree.
+ * Results are those of hipnx_reduce bit for bit, with one exception: for a few columns under a long
+ * axis (inner > 1, inner * element size < 1024 bytes, red >= 4096) hipnx_reduce folds rows into the
+ * columns and reduces in two steps through a pool block, which this entry point does not -- integer
+ * results and selections (max, min, all, any) are still identical, float sums and products are
+ * accumulated in another order and agree within the accumulation bound (red * 2^-53 * sum|x| before the
+ * one rounding to the output type).
  * A shape whose partials do not fit fails with HIPNX_EUNSUPPORTED and launches nothing.  All calls
  * on one GPU share that array: calls that overlap on one GPU (two contexts, i.e. two streams) race. */
 #define HIPNX_REDUCE_STATIC_SCRATCH_BYTES (1u << 20)

@@ -29,11 +29,7 @@ static int launch_one(const hipnx_ctx *ctx, GemmArgs a, int64_t batch) {
   // a K of one slab only ever touches the first stage: the rest of the LDS stays with other work-groups
   const int smem = a.Kb <= SLAB ? (BM + BN) * SLAB : smem_max;
   auto kern = gemm_pipelined_kernel<DT, WM, WN, TM, TN, LK, RK, NSTAGE>;
-  static bool configured = false;  // per instantiation; racing writers store the same value
-  if (!configured) {
-    HIPNX_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem_max));
-    configured = true;
-  }
+  HIPNX_ALLOW_DYNAMIC_LDS(ctx, kern, smem_max);
   a.tiles_m = (int)((a.M + BM - 1) / BM);
   a.tiles_n = (int)((a.N + BN - 1) / BN);
   a.group_m = gemm_group_m(a.tiles_m, a.tiles_n);
@@ -50,11 +46,7 @@ static int launch_pingpong(const hipnx_ctx *ctx, GemmArgs a, int64_t batch) {
   constexpr bool TALL = LK && !RK;  // the operand read by transposing loads gets the fewer fragments
   constexpr int smem = 2 * (256 + BN) * SLAB;
   auto kern = gemm_pingpong_kernel<DT, LK, RK, TALL, true, BN>;
-  static bool configured = false;
-  if (!configured) {
-    HIPNX_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
-    configured = true;
-  }
+  HIPNX_ALLOW_DYNAMIC_LDS(ctx, kern, smem);
   a.tiles_m = (int)((a.M + 255) / 256);
   a.tiles_n = (int)((a.N + BN - 1) / BN);
   a.group_m = gemm_group_m(a.tiles_m, a.tiles_n);
@@ -70,11 +62,7 @@ template <int DT, bool LK, bool RK, int BM = 128, int BN = 128, int NSTAGE = 4, 
 static int launch_pingpong128(const hipnx_ctx *ctx, GemmArgs a, int64_t batch) {
   constexpr int smem = NSTAGE * SPP * (BM + BN) * SLAB;
   auto kern = gemm_pingpong128_kernel<DT, LK, RK, BM, BN, NSTAGE, SPP>;
-  static bool configured = false;
-  if (!configured) {
-    HIPNX_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
-    configured = true;
-  }
+  HIPNX_ALLOW_DYNAMIC_LDS(ctx, kern, smem);
   a.tiles_m = (int)((a.M + BM - 1) / BM);
   a.tiles_n = (int)((a.N + BN - 1) / BN);
   a.group_m = gemm_group_m(a.tiles_m, a.tiles_n);

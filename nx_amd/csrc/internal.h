@@ -89,6 +89,20 @@ int hip_fail(hipError_t e, const char *what);
     if (e__ != hipSuccess) return hipnx::hip_fail(e__, #call);  \
   } while (0)
 
+// hipFuncAttributeMaxDynamicSharedMemorySize is a property of a kernel ON A DEVICE.  Expanded where a kernel
+// that needs more than 64 KiB of LDS is launched (so the static below belongs to that kernel's launch site):
+// sets the attribute once per device (a bit per device index; devices beyond 63 set it on every launch), with
+// the context's device current -- the entry point's scope has selected it.
+#define HIPNX_ALLOW_DYNAMIC_LDS(ctx, kern, bytes)                                                              \
+  do {                                                                                                         \
+    static std::atomic<uint64_t> done__{0};                                                                    \
+    const uint64_t bit__ = (ctx)->device >= 0 && (ctx)->device < 64 ? 1ull << (ctx)->device : 0;               \
+    if (!bit__ || !(done__.load(std::memory_order_acquire) & bit__)) {                                         \
+      HIPNX_HIP(hipFuncSetAttribute((const void *)(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (bytes))); \
+      if (bit__) done__.fetch_or(bit__, std::memory_order_release);                                            \
+    }                                                                                                          \
+  } while (0)
+
 inline int dtype_size(int dt) {
   static const int sz[HIPNX_NTYPES] = {1, 2, 4, 8, 1, 2, 4, 8, 2, 2, 4, 8};
   return (dt >= 0 && dt < HIPNX_NTYPES) ? sz[dt] : -1;

@@ -657,11 +657,7 @@ static int gather_run(hipnx_ctx *ctx, int idx_dt, int64_t n_tuples, int depth, i
 #define HIPNX_TAKE_ROW(SB)                                                                                                        \
   do {                                                                                                                            \
     auto kern = take_row_lds_kernel<SB>;                                                                                          \
-    static bool configured = false;                                                                                               \
-    if (!configured) {                                                                                                            \
-      HIPNX_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024));                 \
-      configured = true;                                                                                                          \
-    }                                                                                                                             \
+    HIPNX_ALLOW_DYNAMIC_LDS(ctx, kern, 128 * 1024);                                                                               \
     hipLaunchKernelGGL(kern, dim3(blocks), dim3(TAKE_ROW_BLOCK), (size_t)row_bytes, ctx->stream, (const unsigned char *)t->ptr,   \
                        idx->ptr, (unsigned char *)out->ptr, idx_dt, outer, td.dims[0], period, (int)(oob_policy == HIPNX_OOB_CLAMP), \
                        flag, (unsigned int *)ctx->flag_host_dev, oob_policy == HIPNX_OOB_DEFER ? deferred_error_word(ctx) : nullptr); \

@@ -31,6 +31,8 @@ def main():
         return 4
     reply = np.ascontiguousarray(-want)
     L.check(L.lib.hipnx_h2d(t.data.ref.ctx, t.data.ref.handle, 0, reply.ctypes.data_as(C.c_void_p), reply.nbytes))
+    # the upload is left in flight on this process's stream: wait for it before telling the parent to look
+    L.check(L.lib.hipnx_sync(t.data.ref.ctx))
     print("child: ok")
     return 0
 

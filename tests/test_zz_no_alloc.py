@@ -84,6 +84,21 @@ def test_static_matches_pooled_twice(ctx, first, second, op, ty):
         assert np.array_equal(got, want), f"op {op} {ty} [{outer}, {red}, {inner}]: static result differs from hipnx_reduce"
 
 
+def test_float_sums_over_folded_shapes_agree_within_the_accumulation_bound(ctx):
+    """A few columns under a long axis: hipnx_reduce folds rows into the columns (two steps through a pool
+    block), the static entry point reduces the columns directly -- another order of the same f64 additions.
+    Twice in a row, the second smaller; f64 so that no final rounding hides the difference."""
+    rng = np.random.default_rng(9)
+    for outer, red, inner in ((1, 8192, 64), (1, 4096, 24)):
+        x = rng.uniform(-1, 1, size=outer * red * inner)
+        got, want = _both(ctx, RED_SUM, "f64", x, outer, red, inner)
+        got, want = got.view(np.float64), want.view(np.float64)
+        bound = red * 2.0 ** -53 * np.abs(x.reshape(outer, red, inner)).sum(axis=1).ravel()
+        assert (np.abs(got - want) <= bound).all(), f"[{outer}, {red}, {inner}]: beyond the accumulation bound"
+        exact = np.array([float(np.sum(x.reshape(outer, red, inner)[:, :, j].astype(np.longdouble))) for j in range(inner)])
+        assert (np.abs(got - exact) <= bound).all()
+
+
 def test_unsplit_shapes_need_no_scratch(ctx):
     rng = np.random.default_rng(8)
     x = rng.uniform(-1, 1, size=1024 * 1024).astype(np.float32)
