@@ -25,6 +25,24 @@
 
 namespace hipnx {
 
+// Only the stand-alone timeline program (gemm_timeline.hip) defines HIPNX_GEMM_TIMELINE: the 256-row kernel then
+// leaves, per work-group, the constant-rate clock at its start, at the first phase of the walk, at the end of the
+// walk and after its last store was issued, the shader clocks the walk took, and the XCD it ran on.  The same
+// program sets HIPNX_PP_EXP for timing-only builds of the walk (their results are wrong): 1 = no requests after
+// the prologue, 32 = no fragment reads after the first slab, 64 = no wait for the requests.  The library is built
+// without either.
+#ifdef HIPNX_GEMM_TIMELINE
+__device__ unsigned long long g_timeline[4096 * 8];
+#define HIPNX_TL_STAMP(var) const unsigned long long var = wall_clock64()
+#define HIPNX_TL_CLOCK(var) const unsigned long long var = clock64()
+#else
+#define HIPNX_TL_STAMP(var)
+#define HIPNX_TL_CLOCK(var)
+#endif
+#ifndef HIPNX_PP_EXP
+#define HIPNX_PP_EXP 0
+#endif
+
 // Swizzle of the [row][k] LDS layout of this kernel: the 16-byte chunk index XOR the part of
 // lds_slot() that depends on the low four row bits only (the part that makes a fragment read of 16
 // consecutive rows conflict-free).  A fragment's address is then one per-lane base per K step plus
@@ -125,6 +143,7 @@ gemm_pingpong_kernel(GemmArgs a) {
   static_assert(DT == HIPNX_BF16 || DT == HIPNX_F16 || DT == HIPNX_S8, "2-byte and 1-byte MFMA types");
   static_assert(L_KIN || ES == 2, "a K-outer left operand is split into two 128-row halves: 2-byte types only");
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  HIPNX_TL_STAMP(tl_start);
 
   int tm, tn;
   gemm_tile_position(a, blockIdx.x, tm, tn);
@@ -206,6 +225,8 @@ gemm_pingpong_kernel(GemmArgs a) {
   }
   __builtin_amdgcn_s_barrier();
   if (grp) __builtin_amdgcn_s_barrier();  // group 1 runs one phase behind
+  HIPNX_TL_STAMP(tl_walk);
+  HIPNX_TL_CLOCK(tl_c0);
 
   v4i fa[TM16], fb[TN16];
   for (int s = 0; s < nslab; s++) {
@@ -213,11 +234,18 @@ gemm_pingpong_kernel(GemmArgs a) {
 #pragma unroll
     for (int ks = 0; ks < 2; ks++) {
       // ---- memory phase: fragments of K step ks, then this phase's requests
+#if HIPNX_PP_EXP & 32
+      if (s == 0) {
+#endif
 #pragma unroll
       for (int i = 0; i < TM16; i++) fa[i] = read_l(cur, ks, i);
 #pragma unroll
       for (int j = 0; j < TN16; j++) fb[j] = read_r(cur, ks, j);
+#if HIPNX_PP_EXP & 32
+      }
+#endif
       bool issued = false, issued_r = false;
+#if !(HIPNX_PP_EXP & 1)
       if (ks == 0) {
         if (s >= 1 && s + 1 < nslab) {
           issue_r((s + 1) & 1, (int64_t)(s + 1) * SLAB);
@@ -232,11 +260,14 @@ gemm_pingpong_kernel(GemmArgs a) {
         issue_l(s & 1, (int64_t)(s + 2) * SLAB);
         issued = true;
       }
+#endif
       // what I requested a memory phase ago (or in the prologue) has to be in LDS before the barrier
       // that publishes it; in the very first phase nothing is due yet (slab 1 is first read in phase 4)
+#if !(HIPNX_PP_EXP & 64)
       if (issued) wait_vmcnt<4>();
       else if (issued_r) wait_vmcnt<RPER>();
       else if (!(s == 0 && ks == 0)) wait_vmcnt<0>();
+#endif
       __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): my fragments are in registers
       __builtin_amdgcn_s_barrier();
       __builtin_amdgcn_sched_barrier(0);
@@ -253,6 +284,8 @@ gemm_pingpong_kernel(GemmArgs a) {
     }
   }
   if (!grp) __builtin_amdgcn_s_barrier();  // group 0 finishes one phase ahead
+  HIPNX_TL_STAMP(tl_done);
+  HIPNX_TL_CLOCK(tl_c1);
 
   const int64_t obase = b * a.M * a.N;
   switch (a.odt) {
@@ -262,6 +295,13 @@ gemm_pingpong_kernel(GemmArgs a) {
     HIPNX_EPI(HIPNX_S32) HIPNX_EPI(HIPNX_U32) HIPNX_EPI(HIPNX_S64) HIPNX_EPI(HIPNX_U64)
 #undef HIPNX_EPI
   }
+#ifdef HIPNX_GEMM_TIMELINE
+  if (threadIdx.x == 0 && blockIdx.x < 4096) {
+    unsigned long long *p = g_timeline + (size_t)blockIdx.x * 8;
+    p[0] = tl_start; p[1] = tl_walk; p[2] = tl_done; p[3] = wall_clock64(); p[4] = tl_c1 - tl_c0;
+    p[5] = __builtin_amdgcn_s_getreg((31 << 11) | 20);  // XCC_ID
+  }
+#endif
 }
 
 // ---- the two-group walk on a 128 x 128 tile ----------------------------------------------------------
