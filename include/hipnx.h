@@ -144,6 +144,14 @@ int hipnx_buf_size(const hipnx_buf *buf, size_t *bytes);
 /* replaces: to_pointer/2 with mode :local (nx/lib/nx/backend.ex:66; exla/lib/exla/backend.ex:86-131,
  * exla/c_src/exla/exla.cc:327-385): the raw device address of a live buffer; NULL once freed */
 void *hipnx_buf_device_ptr(const hipnx_buf *buf);
+/* replaces: nothing in the reference (its backends check or clamp every index, nx/lib/nx/binary_backend.ex:1949-1952,
+ * exla/test/exla/defn/expr_test.exs:3478-3481).  0, or the length L of the axis along which hipnx_argreduce last
+ * wrote this buffer's values, every one of them in [0, L): such a buffer used as the indices of hipnx_take /
+ * hipnx_gather (one index per slice, same index type) along an axis of at least L entries cannot hold a bad index,
+ * and the HIPNX_OOB_RAISE policy then does not wait for the kernel (a violation, impossible by construction, would
+ * still be recorded and raised by the next wait).  The knowledge is dropped when the buffer is written again (any
+ * entry point that takes it as an output) or its address leaves the library (hipnx_buf_device_ptr, ipc_export). */
+int hipnx_buf_index_bound(const hipnx_buf *buf, int64_t *bound);
 /* replaces: from_pointer/5 for a :local pointer (nx/lib/nx/backend.ex:59-65;
  * exla/lib/exla/backend.ex:133-181, exla/c_src/exla/exla.cc:387-437): a handle over `bytes` of
  * device memory of this context's device that someone else owns.  Freeing or destroying the

@@ -79,6 +79,7 @@ PROTOTYPES = {
     "hipnx_buf_destroy": [_buf_p],
     "hipnx_buf_size": [_buf_p, C.POINTER(C.c_size_t)],
     "hipnx_buf_device_ptr": [_buf_p],
+    "hipnx_buf_index_bound": [_buf_p, _i64p],
     "hipnx_buf_wrap": [_ctx_p, C.c_void_p, C.c_size_t, C.POINTER(_buf_p)],
     "hipnx_buf_ipc_export": [_ctx_p, _buf_p, C.c_void_p],
     "hipnx_buf_ipc_import": [_ctx_p, C.c_void_p, C.c_size_t, C.POINTER(_buf_p)],

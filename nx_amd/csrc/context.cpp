@@ -445,6 +445,7 @@ int hipnx_buf_ipc_export(hipnx_ctx *ctx, const hipnx_buf *buf, void *handle_out)
   if (buf->capacity >= (1ull << 31)) return set_error(HIPNX_EUNSUPPORTED, "ipc_export: allocations of 2 GiB or more are not shared");
   static_assert(sizeof(hipIpcMemHandle_t) == HIPNX_IPC_HANDLE_BYTES, "handle size of the public header");
   hipIpcMemHandle_t h;
+  buf->index_bound = 0;  // another process may write here from now on
   HIPNX_HIP(hipIpcGetMemHandle(&h, buf->ptr));
   HIPNX_HIP(hipStreamSynchronize(ctx->stream));  // the other process sees what has been written so far
   std::memcpy(handle_out, &h, sizeof h);
@@ -487,7 +488,15 @@ int hipnx_buf_size(const hipnx_buf *buf, size_t *bytes) {
 
 void *hipnx_buf_device_ptr(const hipnx_buf *buf) {
   if (!buf || buf->freed.load()) return nullptr;
+  buf->index_bound = 0;  // the address leaves the library: what is written through it is not seen here
   return buf->ptr;
+}
+
+int hipnx_buf_index_bound(const hipnx_buf *buf, int64_t *bound) {
+  if (!buf || !bound) return set_error(HIPNX_EINVAL, "null argument");
+  if (buf->freed.load()) return set_error(HIPNX_EFREED, "buffer has been deallocated");
+  *bound = buf->index_bound;
+  return HIPNX_OK;
 }
 
 // Host memory of callers is pageable (an Erlang binary, a numpy array).  The runtime's own path for it costs 35 us for

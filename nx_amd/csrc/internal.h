@@ -76,6 +76,14 @@ struct hipnx_buf {
   std::atomic<int> freed{0};
   bool borrowed = false;  // wraps memory owned by someone else: never returned to the pool
   bool ipc = false;       // borrowed through an IPC handle of another process: closed on release
+  // What the library knows about the VALUES it last wrote here: the first index_bytes bytes hold indices of type
+  // index_dt that all lie in [0, index_bound) -- set by hipnx_argreduce on its result (an index along an axis of
+  // that length), cleared whenever the buffer is handed to an entry point as an output or its address leaves the
+  // library.  gather / take use it to skip the wait of the raising bounds policy for indices that cannot be out
+  // of range.  0 = nothing known.
+  mutable int64_t index_bound = 0;
+  uint64_t index_bytes = 0;
+  int index_dt = -1;
 };
 
 namespace hipnx {
@@ -117,6 +125,12 @@ inline bool is_wide(int dt) {  // not exactly representable in f32
 
 // operand checks shared by every entry point: live handle, same context, enough bytes
 int check_buf(const hipnx_ctx *ctx, const hipnx_buf *b, uint64_t need_bytes, const char *name);
+// the same for a buffer an entry point is about to write (outputs are the non-const handles of the C ABI): what was
+// known about its values is forgotten
+inline int check_buf(const hipnx_ctx *ctx, hipnx_buf *b, uint64_t need_bytes, const char *name) {
+  if (b) b->index_bound = 0;
+  return check_buf(ctx, static_cast<const hipnx_buf *>(b), need_bytes, name);
+}
 
 // pooled device memory; both expect the context mutex to be held (i.e. inside an Enter scope)
 int pool_alloc(hipnx_ctx *ctx, size_t bytes, void **ptr_out, size_t *cap_out);

@@ -736,12 +736,19 @@ static int gather_run(hipnx_ctx *ctx, int idx_dt, int64_t n_tuples, int depth, i
   return HIPNX_OK;
 }
 
+// Indices the library wrote itself as positions along an axis no longer than the one they now address (the result
+// of hipnx_argreduce, untouched since, read as the type it was written in) cannot be out of range: the raising
+// policy then has nothing to wait for.  The kernel still checks them and records a violation for the next wait
+// (the late-raising policy), so a wrong claim would surface instead of passing silently.
+static bool indices_known_in_range(const hipnx_buf *idx, int idx_dt, uint64_t idx_bytes, int depth, int64_t axis_len) {
+  return depth == 1 && idx->index_bound > 0 && idx->index_dt == idx_dt && idx->index_bytes >= idx_bytes && idx->index_bound <= axis_len;
+}
+
 extern "C" int hipnx_gather(hipnx_ctx *ctx, int elem_bytes, int rank, const int64_t *t_dims, int idx_dt,
                             int64_t n_tuples, int depth, int oob_policy, const hipnx_buf *t, const hipnx_buf *idx,
                             hipnx_buf *out) {
   Enter in(ctx);
   if (in.status) return in.status;
-  if (oob_policy == HIPNX_OOB_RAISE) HIPNX_NOT_CAPTURING(ctx, "gather with the raising bounds policy");
   if (rank < 0 || rank > 64 || depth < 0 || depth > rank || depth > MAXR || n_tuples < 0 || (rank > 0 && !t_dims))
     return set_error(HIPNX_EINVAL, "gather: bad rank / depth");
   if (elem_bytes <= 0 || dtype_size(idx_dt) < 0 || is_float(idx_dt))
@@ -758,6 +765,10 @@ extern "C" int hipnx_gather(hipnx_ctx *ctx, int elem_bytes, int rank, const int6
   if (int st = check_buf(ctx, t, (uint64_t)total * elem_bytes, "gather tensor")) return st;
   if (int st = check_buf(ctx, idx, (uint64_t)n_tuples * depth * dtype_size(idx_dt), "gather indices")) return st;
   if (int st = check_buf(ctx, out, (uint64_t)n_tuples * slice_bytes, "gather out")) return st;
+  if (oob_policy == HIPNX_OOB_RAISE && rank > 0 &&
+      indices_known_in_range(idx, idx_dt, (uint64_t)n_tuples * depth * dtype_size(idx_dt), depth, t_dims[0]))
+    oob_policy = HIPNX_OOB_DEFER;
+  if (oob_policy == HIPNX_OOB_RAISE) HIPNX_NOT_CAPTURING(ctx, "gather with the raising bounds policy");
   if (n_tuples == 0 || slice_bytes == 0) return HIPNX_OK;
   if (total == 0) {
     if (oob_policy == HIPNX_OOB_CLAMP) return set_error(HIPNX_EINVAL, "gather: cannot clamp into an empty tensor");
@@ -858,7 +869,6 @@ extern "C" int hipnx_take(hipnx_ctx *ctx, int elem_bytes, int64_t outer, int64_t
                           const hipnx_buf *idx, hipnx_buf *out) {
   Enter in(ctx);
   if (in.status) return in.status;
-  if (oob_policy == HIPNX_OOB_RAISE) HIPNX_NOT_CAPTURING(ctx, "take with the raising bounds policy");
   if (elem_bytes <= 0 || dtype_size(idx_dt) < 0 || is_float(idx_dt)) return set_error(HIPNX_EINVAL, "take: indices must be an integer type");
   if (outer < 0 || axis_len < 0 || inner < 0 || n_idx < 0 || rank < 0 || rank > 64 || (rank > 0 && !msg_dims))
     return set_error(HIPNX_EINVAL, "take: negative extent or bad rank");
@@ -868,6 +878,9 @@ extern "C" int hipnx_take(hipnx_ctx *ctx, int elem_bytes, int64_t outer, int64_t
   if (int st = check_buf(ctx, t, (uint64_t)outer * axis_len * slice_bytes, "take tensor")) return st;
   if (int st = check_buf(ctx, idx, (uint64_t)n_idx * dtype_size(idx_dt), "take indices")) return st;
   if (int st = check_buf(ctx, out, (uint64_t)outer * n_idx * slice_bytes, "take out")) return st;
+  if (oob_policy == HIPNX_OOB_RAISE && indices_known_in_range(idx, idx_dt, (uint64_t)n_idx * dtype_size(idx_dt), 1, axis_len))
+    oob_policy = HIPNX_OOB_DEFER;
+  if (oob_policy == HIPNX_OOB_RAISE) HIPNX_NOT_CAPTURING(ctx, "take with the raising bounds policy");
   if (outer * n_idx == 0 || slice_bytes == 0) return HIPNX_OK;
   if (axis_len == 0) {
     if (oob_policy == HIPNX_OOB_CLAMP) return set_error(HIPNX_EINVAL, "take: cannot clamp into an empty axis");

@@ -38,9 +38,20 @@ extern "C" int hipnx_argreduce(hipnx_ctx *ctx, int op, int tie, int in_dt, int o
   if (outer * inner == 0) return HIPNX_OK;
   const void *ip = inb->ptr;
   void *op_ = out->ptr;
+  int st;
   if (op == HIPNX_ARGMAX)
-    return tie == HIPNX_TIE_LOW ? argreduce_op<HIPNX_ARGMAX, HIPNX_TIE_LOW>(ctx, in_dt, out_dt, outer, red, inner, ip, op_)
-                                : argreduce_op<HIPNX_ARGMAX, HIPNX_TIE_HIGH>(ctx, in_dt, out_dt, outer, red, inner, ip, op_);
-  return tie == HIPNX_TIE_LOW ? argreduce_op<HIPNX_ARGMIN, HIPNX_TIE_LOW>(ctx, in_dt, out_dt, outer, red, inner, ip, op_)
+    st = tie == HIPNX_TIE_LOW ? argreduce_op<HIPNX_ARGMAX, HIPNX_TIE_LOW>(ctx, in_dt, out_dt, outer, red, inner, ip, op_)
+                              : argreduce_op<HIPNX_ARGMAX, HIPNX_TIE_HIGH>(ctx, in_dt, out_dt, outer, red, inner, ip, op_);
+  else
+    st = tie == HIPNX_TIE_LOW ? argreduce_op<HIPNX_ARGMIN, HIPNX_TIE_LOW>(ctx, in_dt, out_dt, outer, red, inner, ip, op_)
                               : argreduce_op<HIPNX_ARGMIN, HIPNX_TIE_HIGH>(ctx, in_dt, out_dt, outer, red, inner, ip, op_);
+  // every value written is an index along the reduced axis: in [0, red) unless the output type is too narrow
+  // to hold red - 1 (the index is then written wrapped, shared.ex:190-194, and nothing is claimed)
+  const int bits = 8 * dtype_size(out_dt) - (is_unsigned(out_dt) ? 0 : 1);
+  if (st == HIPNX_OK && !out->borrowed && (bits >= 63 || red - 1 < ((int64_t)1 << bits))) {
+    out->index_bound = red;
+    out->index_bytes = (uint64_t)outer * inner * dtype_size(out_dt);
+    out->index_dt = out_dt;
+  }
+  return st;
 }

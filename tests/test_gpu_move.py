@@ -287,3 +287,60 @@ def test_transposes_with_odd_extents(shape, perm, ty, hip):
     x = rand_raw(rng, ty, shape)
     got = hip.to_numpy(Nx.transpose(from_numpy(x, ty, hip), perm))
     assert np.array_equal(got.view(np.uint8), np.ascontiguousarray(np.transpose(x, perm)).view(np.uint8))
+
+
+def _index_bound(t):
+    import ctypes as C
+    from nx_amd import _lib as L
+    bound = C.c_int64(-1)
+    L.check(L.lib.hipnx_buf_index_bound(t.data.ref.handle, C.byref(bound)))
+    return bound.value
+
+
+def test_indices_written_by_argmax_need_no_bounds_wait(hip, oracle):
+    """`argmax` writes positions along an axis; `take` along an axis at least as long cannot meet a bad one, so
+    the raising policy has nothing to wait for (the reference checks every index, binary_backend.ex:1949-1952:
+    same results, same error for indices that CAN be out of range)."""
+    import ctypes as C
+    from nx_amd import _lib as L
+    from nx_amd import backend as B
+    from nx_amd._lib import HipNxArgumentError
+    rng = np.random.default_rng(11)
+    logits = rng.standard_normal((300, 1000)).astype(np.float32)
+    logits[7, 999] = 50.0  # one row points at the last entry
+    table = rand_raw(rng, "bf16", (1000, 64))
+    hl, ol = both(logits, "f32", hip, oracle)
+    ht, ot = both(table, "bf16", hip, oracle)
+    hidx, oidx = Nx.argmax(hl, axis=1, type="u32"), Nx.argmax(ol, axis=1, type="u32")
+    assert _index_bound(hidx) == 1000
+    assert_bits_equal(Nx.take(ht, hidx), Nx.take(ot, oidx), "take of argmax indices")
+    assert _index_bound(hidx) == 1000  # reading does not change what is known
+    # the same indices into a shorter axis CAN be out of range: checked at once, the reference's message
+    short = from_numpy(table[:500].copy(), "bf16", hip)
+    with pytest.raises(HipNxArgumentError, match="index 999 is out of bounds for axis 0 in shape \\{500, 64\\}"):
+        Nx.take(short, hidx)
+    # with the bound known, the raising policy runs inside a captured graph (it would have to wait otherwise)
+    B.capture_begin(0)
+    try:
+        inside = Nx.take(ht, hidx)
+    finally:
+        graph = B.capture_end(0)
+    graph.launch()
+    assert_bits_equal(inside, Nx.take(ot, oidx), "take of argmax indices in a captured graph")
+    del inside
+    graph.destroy()
+    assert _index_bound(Nx.argmax(hl, axis=1, type="s64")) == 1000
+    # an output type too narrow for the axis wraps the index: no claim
+    assert _index_bound(Nx.argmax(hl, axis=1, type="u8")) == 0
+    assert _index_bound(Nx.argmax(hl, axis=1, type="s8")) == 0
+    assert _index_bound(Nx.argmax(from_numpy(logits[:, :128].copy(), "f32", hip), axis=1, type="s8")) == 128
+    # written again, the buffer holds whatever was written
+    zero = np.zeros(1, dtype=np.uint32)
+    L.check(L.lib.hipnx_fill(hidx.data.ref.ctx, hidx.data.ref.handle, 4, zero.ctypes.data_as(C.c_void_p), 300))
+    assert _index_bound(hidx) == 0
+    # and indices from anywhere else are checked as ever
+    foreign = from_numpy(np.array([3, 1000, 2], dtype=np.uint32), "u32", hip)
+    assert _index_bound(foreign) == 0
+    with pytest.raises(HipNxArgumentError, match="index 1000 is out of bounds for axis 0 in shape \\{1000, 64\\}"):
+        Nx.take(ht, foreign)
+    assert B.bounds_policy("raise") == "raise"
