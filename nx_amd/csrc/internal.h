@@ -128,8 +128,9 @@ int check_buf(const hipnx_ctx *ctx, const hipnx_buf *b, uint64_t need_bytes, con
 // the same for a buffer an entry point is about to write (outputs are the non-const handles of the C ABI): what was
 // known about its values is forgotten
 inline int check_buf(const hipnx_ctx *ctx, hipnx_buf *b, uint64_t need_bytes, const char *name) {
-  if (b) b->index_bound = 0;
-  return check_buf(ctx, static_cast<const hipnx_buf *>(b), need_bytes, name);
+  const int st = check_buf(ctx, static_cast<const hipnx_buf *>(b), need_bytes, name);
+  if (st == HIPNX_OK) b->index_bound = 0;  // (only a live handle of this context is written to)
+  return st;
 }
 
 // pooled device memory; both expect the context mutex to be held (i.e. inside an Enter scope)
