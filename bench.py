@@ -140,6 +140,9 @@ def main():
     ap.add_argument("--no-suite", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--calibrate", action="store_true")
+    # parts of the suite to run (comma-separated: dots, config1, bf16, config3, config4, config5, misc, random, chains,
+    # softmax1m); default all
+    ap.add_argument("--only", default=None)
     # which 4096^3 contraction is timed as the headline: bf16 (the metric's configuration, the default) or the
     # int8 one (s8 x s8 -> s32), so that the int8 kernel can be profiled by the same commands
     ap.add_argument("--headline", choices=["bf16", "s8"], default="bf16")
@@ -261,6 +264,11 @@ def main():
     if not args.no_suite:
         suite = {}
         steps, warm = max(args.steps // 2, 10), 5
+        from nx_amd import defn
+
+        def section(name):
+            """`--only a,b` runs the named parts of the suite alone (for profiles of one configuration)."""
+            return args.only is None or name in args.only.split(",")
 
         def rotating(make, nbytes):
             """A ring of operand sets exceeding 320 MB in total; returns next()."""
@@ -300,337 +308,348 @@ def main():
                 e["vs_" + vs[0]] = round(vs[1] / ms, 2)
             suite[name] = e
 
-        # K-inner operands: the gemm kernel alone (no re-layout pass)
-        bt = Nx.transpose(b)
-        msettle = min(args.settle_ms, 150.0)
-        _, ms = tstat(lambda: Nx.dot(a, [1], bt, [1]), steps, warm, msettle)
-        entry("dot_bf16_4096_kinner", flop, "TFLOP/s", ms, PEAK["bf16"], "mfma", "mfma_bf16")
-        nxt = rotating(lambda: (put(a_np, "bf16"), put(b_np, "bf16")), 2 * n * n * 2)
+        if section("dots"):
+            # K-inner operands: the gemm kernel alone (no re-layout pass)
+            bt = Nx.transpose(b)
+            msettle = min(args.settle_ms, 150.0)
+            _, ms = tstat(lambda: Nx.dot(a, [1], bt, [1]), steps, warm, msettle)
+            entry("dot_bf16_4096_kinner", flop, "TFLOP/s", ms, PEAK["bf16"], "mfma", "mfma_bf16")
+            nxt = rotating(lambda: (put(a_np, "bf16"), put(b_np, "bf16")), 2 * n * n * 2)
 
-        def dot_rot():
-            x, y = nxt()
-            return Nx.dot(x, y)
-        _, ms = tstat(dot_rot, steps, warm, msettle)
-        entry("dot_bf16_4096_rotated", flop, "TFLOP/s", ms, PEAK["bf16"], "mfma", "mfma_bf16")
-        del nxt
-        fa, fb = W.dense_gemm_f32()
-        fa, fb = put(fa, "f32"), put(fb, "f32")
-        _, ms = tstat(lambda: Nx.dot(fa, fb), steps, warm, msettle)
-        entry("dot_f32_2048", 2.0 * 2048 ** 3, "TFLOP/s", ms, PEAK["f32"], "mfma", "mfma_f32")
-        sa, sb = W.dense_gemm_s8()
-        sa, sb = put(sa, "s8"), put(sb, "s8")
-        _, ms = tstat(lambda: Nx.dot(sa, sb, out_type="s32"), steps, warm, msettle)
-        entry("dot_s8_4096_s32", flop, "TOP/s", ms, PEAK["s8"], "mfma", "mfma_s8")
-        sbt = Nx.transpose(sb)
-        _, ms = tstat(lambda: Nx.dot(sa, [1], sbt, [1], out_type="s32"), steps, warm, msettle)
-        entry("dot_s8_4096_s32_kinner", flop, "TOP/s", ms, PEAK["s8"], "mfma", "mfma_s8")
-        # a serving batch against one weight matrix (bound by the 33.5 MB of weights; K is split over the
-        # work-groups of the under-filled grid) and a mid-size square (one 128 x 128 tile per CU)
-        xa, wb = put(a_np[:128].copy(), "bf16"), bt
-        _, ms = tstat(lambda: Nx.dot(xa, [1], wb, [1]), steps, warm)
-        entry("dot_bf16_128x4096x4096", 2.0 * (128 * 4096 * 2) + 4096 * 4096 * 2.0, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read")
-        ma, mb = put(a_np[:2048, :2048].copy(), "bf16"), put(b_np[:2048, :2048].copy(), "bf16")
-        _, ms = tstat(lambda: Nx.dot(ma, mb), steps, warm)
-        entry("dot_bf16_2048", 2.0 * 2048 ** 3, "TFLOP/s", ms, PEAK["bf16"], "mfma", "mfma_bf16")
-        # a prefill-sized batch against the weight matrix (256 tiles of 128 x 128, 64 slabs of K each)
-        pa = put(a_np[:1024].copy(), "bf16")
-        _, ms = tstat(lambda: Nx.dot(pa, b), steps, warm)
-        entry("dot_bf16_1024x4096x4096", 2.0 * 1024 * 4096 * 4096, "TFLOP/s", ms, PEAK["bf16"], "mfma", "mfma_bf16")
-        # mid-size int8: both operands K-inner, and the plain layout (right operand K-outer, laid out K-inner first)
-        qa, qb = (put(q, "s8") for q in W.dense_gemm_s8(n=2048))
-        qbt = Nx.transpose(qb)
-        _, ms = tstat(lambda: Nx.dot(qa, [1], qbt, [1], out_type="s32"), steps, warm)
-        entry("dot_s8_2048_s32_kinner", 2.0 * 2048 ** 3, "TOP/s", ms, PEAK["s8"], "mfma", "mfma_s8")
-        _, ms = tstat(lambda: Nx.dot(qa, qb, out_type="s32"), steps, warm)
-        entry("dot_s8_2048_s32", 2.0 * 2048 ** 3, "TOP/s", ms, PEAK["s8"], "mfma", "mfma_s8")
-        del xa, wb, ma, mb, pa, qa, qb, qbt
-        ha, hb = put(W.bf16_to_f32(a_np).astype(np.float16), "f16"), put(W.bf16_to_f32(b_np).astype(np.float16), "f16")
-        _, ms = tstat(lambda: Nx.dot(ha, hb), steps, warm, msettle)
-        entry("dot_f16_4096", flop, "TFLOP/s", ms, PEAK["f16"], "mfma", "mfma_f16")
-        del fa, fb, sa, sb, bt, sbt, ha, hb
+            def dot_rot():
+                x, y = nxt()
+                return Nx.dot(x, y)
+            _, ms = tstat(dot_rot, steps, warm, msettle)
+            entry("dot_bf16_4096_rotated", flop, "TFLOP/s", ms, PEAK["bf16"], "mfma", "mfma_bf16")
+            del nxt
+            fa, fb = W.dense_gemm_f32()
+            fa, fb = put(fa, "f32"), put(fb, "f32")
+            _, ms = tstat(lambda: Nx.dot(fa, fb), steps, warm, msettle)
+            entry("dot_f32_2048", 2.0 * 2048 ** 3, "TFLOP/s", ms, PEAK["f32"], "mfma", "mfma_f32")
+            sa, sb = W.dense_gemm_s8()
+            sa, sb = put(sa, "s8"), put(sb, "s8")
+            _, ms = tstat(lambda: Nx.dot(sa, sb, out_type="s32"), steps, warm, msettle)
+            entry("dot_s8_4096_s32", flop, "TOP/s", ms, PEAK["s8"], "mfma", "mfma_s8")
+            sbt = Nx.transpose(sb)
+            _, ms = tstat(lambda: Nx.dot(sa, [1], sbt, [1], out_type="s32"), steps, warm, msettle)
+            entry("dot_s8_4096_s32_kinner", flop, "TOP/s", ms, PEAK["s8"], "mfma", "mfma_s8")
+            # a serving batch against one weight matrix (bound by the 33.5 MB of weights; K is split over the
+            # work-groups of the under-filled grid) and a mid-size square (one 128 x 128 tile per CU)
+            xa, wb = put(a_np[:128].copy(), "bf16"), bt
+            _, ms = tstat(lambda: Nx.dot(xa, [1], wb, [1]), steps, warm)
+            entry("dot_bf16_128x4096x4096", 2.0 * (128 * 4096 * 2) + 4096 * 4096 * 2.0, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read")
+            ma, mb = put(a_np[:2048, :2048].copy(), "bf16"), put(b_np[:2048, :2048].copy(), "bf16")
+            _, ms = tstat(lambda: Nx.dot(ma, mb), steps, warm)
+            entry("dot_bf16_2048", 2.0 * 2048 ** 3, "TFLOP/s", ms, PEAK["bf16"], "mfma", "mfma_bf16")
+            # a prefill-sized batch against the weight matrix (256 tiles of 128 x 128, 64 slabs of K each)
+            pa = put(a_np[:1024].copy(), "bf16")
+            _, ms = tstat(lambda: Nx.dot(pa, b), steps, warm)
+            entry("dot_bf16_1024x4096x4096", 2.0 * 1024 * 4096 * 4096, "TFLOP/s", ms, PEAK["bf16"], "mfma", "mfma_bf16")
+            # mid-size int8: both operands K-inner, and the plain layout (right operand K-outer, laid out K-inner first)
+            qa, qb = (put(q, "s8") for q in W.dense_gemm_s8(n=2048))
+            qbt = Nx.transpose(qb)
+            _, ms = tstat(lambda: Nx.dot(qa, [1], qbt, [1], out_type="s32"), steps, warm)
+            entry("dot_s8_2048_s32_kinner", 2.0 * 2048 ** 3, "TOP/s", ms, PEAK["s8"], "mfma", "mfma_s8")
+            _, ms = tstat(lambda: Nx.dot(qa, qb, out_type="s32"), steps, warm)
+            entry("dot_s8_2048_s32", 2.0 * 2048 ** 3, "TOP/s", ms, PEAK["s8"], "mfma", "mfma_s8")
+            del xa, wb, ma, mb, pa, qa, qb, qbt
+            ha, hb = put(W.bf16_to_f32(a_np).astype(np.float16), "f16"), put(W.bf16_to_f32(b_np).astype(np.float16), "f16")
+            _, ms = tstat(lambda: Nx.dot(ha, hb), steps, warm, msettle)
+            entry("dot_f16_4096", flop, "TFLOP/s", ms, PEAK["f16"], "mfma", "mfma_f16")
+            del fa, fb, sa, sb, bt, sbt, ha, hb
 
-        # config 1 (and a HBM-resident scale of it)
-        for nn in (1024, 16384):
+        if section("config1"):
+            # config 1 (and a HBM-resident scale of it)
+            for nn in (1024, 16384):
+                x, y = W.elementwise_reduce(n=nn)
+                x, y = put(x, "f32"), put(y, "f32")
+                N = nn * nn
+                _, ms = tstat(lambda: Nx.add(x, y), steps, warm)
+                entry(f"add_f32_{nn}", 12.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+                _, ms = tstat(lambda: Nx.multiply(x, 0.5), steps, warm)
+                entry(f"multiply_scalar_f32_{nn}", 8.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+                _, ms = tstat(lambda: Nx.exp(x), steps, warm)
+                entry(f"exp_f32_{nn}", 8.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+                _, ms = tstat(lambda: Nx.sum(x, axes=[1]), steps, warm)
+                entry(f"sum_rows_f32_{nn}", 4.0 * N + 4.0 * nn, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read")
+                # the whole unfused chain of config 1: add -> multiply 0.5 -> exp -> sum over axis 1
+                _, ms = tstat(lambda: Nx.sum(Nx.exp(Nx.multiply(Nx.add(x, y), 0.5)), axes=[1]), steps, warm)
+                entry(f"config1_chain_f32_{nn}", 32.0 * N + 4.0 * nn, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+                del x, y
+
+        if section("bf16"):
+            # the same callbacks on the 2-byte type of most model tensors (bf16, 16384^2), a column sum and a transpose
+            rng16 = np.random.default_rng(16)
+            bx = put((rng16.standard_normal((16384, 16384)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16), "bf16")
+            N = 16384 * 16384
+            by = put((rng16.standard_normal((16384, 16384)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16), "bf16")
+            _, ms = tstat(lambda: Nx.add(bx, by), steps, warm)
+            entry("add_bf16_16384", 6.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+            del by
+            _, ms = tstat(lambda: Nx.exp(bx), steps, warm)
+            entry("exp_bf16_16384", 4.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+            _, ms = tstat(lambda: Nx.sum(bx, axes=[1]), steps, warm)
+            entry("sum_rows_bf16_16384", 2.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read")
+            _, ms = tstat(lambda: Nx.sum(bx, axes=[0]), steps, warm)
+            entry("sum_columns_bf16_16384", 2.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read")
+            _, ms = tstat(lambda: Nx.argmax(bx, axis=1), steps, warm)
+            entry("argmax_rows_bf16_16384", 2.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read")
+            _, ms = tstat(lambda: Nx.transpose(bx), steps, warm)
+            entry("transpose_bf16_16384", 4.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+            _, ms = tstat(lambda: Nx.as_type(bx, "f32"), steps, warm)
+            entry("as_type_bf16_f32_16384", 6.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+            del bx
+
+        if section("config3"):
+            # config 3: attention scores + softmax chain
+            q, k = W.attention_scores()
+            q, k = put(q, "bf16"), put(k, "bf16")
+            _, ms = tstat(lambda: Nx.dot(q, [2], [0], k, [2], [0]), steps, warm)
+            entry("dot_qk_bf16_32x512x64", 20971520.0, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_write")
+            q_np, k_np = W.attention_scores()
+            nxt = rotating(lambda: (put(q_np, "bf16"), put(k_np, "bf16")), q_np.nbytes + k_np.nbytes)
+
+            def qk_rot():
+                qq, kk = nxt()
+                return Nx.dot(qq, [2], [0], kk, [2], [0])
+            _, ms = tstat(qk_rot, steps, warm)
+            entry("dot_qk_bf16_32x512x64_rotated", 20971520.0, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_write")
+            del nxt
+            s = Nx.dot(q, [2], [0], k, [2], [0])
+
+            def softmax():
+                z = Nx.multiply(Nx.as_type(s, "f32"), 0.125)
+                e = Nx.exp(Nx.subtract(z, Nx.reduce_max(z, axes=[2], keep_axes=True)))
+                return Nx.divide(e, Nx.sum(e, axes=[2], keep_axes=True))
+            _, ms = tstat(softmax, steps, warm)
+            entry("softmax_chain_32x512x512", 386138112.0, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+            nxt = rotating(lambda: Nx.dot(q, [2], [0], k, [2], [0]), 32 * 512 * 512 * 2)
+
+            def softmax_rot():
+                z = Nx.multiply(Nx.as_type(nxt(), "f32"), 0.125)
+                e = Nx.exp(Nx.subtract(z, Nx.reduce_max(z, axes=[2], keep_axes=True)))
+                return Nx.divide(e, Nx.sum(e, axes=[2], keep_axes=True))
+            _, ms = tstat(softmax_rot, steps, warm)
+            entry("softmax_chain_32x512x512_rotated", 386138112.0, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+            del q, k, s, nxt
+
+        if section("config4"):
+            # config 4: int8 weight-only linear
+            w, xq, sc = W.int8_linear()
+            w, xq, sc = put(w, "s8"), put(xq, "s8"), put(sc, "f32")
+            _, ms = tstat(lambda: Nx.dot(xq, [1], w, [1], out_type="s32"), steps, warm)
+            entry("dot_s8_w8_64x11008x4096", 48168960.0, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read")
+            suite["dot_s8_w8_64x11008x4096"]["tops"] = round(5771362304.0 / (ms * 1e-3) / 1e12, 2)
+            w_np = W.int8_linear()[0]
+            nxt = rotating(lambda: put(w_np, "s8"), w_np.nbytes)
+            _, ms = tstat(lambda: Nx.dot(xq, [1], nxt(), [1], out_type="s32"), steps, warm)
+            entry("dot_s8_w8_64x11008x4096_rotated", 48168960.0, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read")
+            # the same layer with its weights stored [K, N], the plain Nx.dot(x, w) of a dense layer (K-outer weights)
+            nxt_t = rotating(lambda: put(np.ascontiguousarray(w_np.T), "s8"), w_np.nbytes)
+            _, ms = tstat(lambda: Nx.dot(xq, nxt_t(), out_type="s32"), steps, warm)
+            del nxt_t
+            entry("dot_s8_w8_64x11008x4096_weights_k_outer_rotated", 48168960.0, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read")
+            # the whole config: dot -> as_type f32 -> multiply by the per-column scales
+            _, ms = tstat(lambda: Nx.multiply(Nx.as_type(Nx.dot(xq, [1], nxt(), [1], out_type="s32"), "f32"), sc), steps, warm)
+            entry("config4_chain_rotated", 48168960.0 + 5636096.0 + 5680128.0, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+            del w, xq, sc, nxt
+
+        if section("config5"):
+            # config 5: argmax + take
+            logits, table, _ = W.logits_and_table()
+            logits, table = put(logits, "f32"), put(table, "bf16")
+            _, ms = tstat(lambda: Nx.argmax(logits, axis=1, type="u32"), steps, warm)
+            entry("argmax_f32_8192x32000", 1048608768.0, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read")
+            idx = Nx.argmax(logits, axis=1, type="u32")
+            _, ms = tstat(lambda: Nx.take(table, idx), steps, warm)
+            entry("take_bf16_8192_of_32000x4096", 134250496.0, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+            suite["take_bf16_8192_of_32000x4096"]["note"] = (
+                "per call, not per kernel; the indices are the argmax's own result, which the library knows to lie within "
+                "an axis of 32000 entries: the raising bounds policy does not wait for the kernel (the kernel itself "
+                "runs ~22 us = ~6.1 TB/s by the rocprofv3 kernel trace)")
+            # other rows every step (nine index sets, 600 MB of table rows in all: nothing comes from the cache), each set
+            # the argmax over its own {8192, 32000} tensor of random words as in the configuration (indices written by
+            # argmax are known to lie within an axis of that length, so the raising policy has nothing to wait for)
+            from nx_amd import random as Random
+            ring = []
+            for part in range(9):
+                ring.append(Nx.argmax(Random.random_bits(Random.key(505 + part, backend=H), shape=(8192, 32000)), axis=1, type="u32"))
+            pos = [0]
+
+            def next_argmax_indices():
+                pos[0] = (pos[0] + 1) % len(ring)
+                return ring[pos[0]]
+            _, ms = tstat(lambda: Nx.take(table, next_argmax_indices()), steps, warm)
+            entry("take_bf16_8192_of_32000x4096_rotated", 134250496.0, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+            del ring
+            # indices from anywhere else (uploaded from the host): every call waits for its kernel, as the reference's
+            # raising bounds check demands
+            rng = np.random.default_rng(5)
+            nxt = rotating(lambda: put(rng.integers(0, 32000, size=8192, dtype=np.uint32), "u32"), 40e6)
+            _, ms = tstat(lambda: Nx.take(table, nxt()), steps, warm)
+            entry("take_bf16_8192_of_32000x4096_rotated_foreign_indices", 134250496.0, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+            # the same with the bounds policy that raises late (the kernel records a bad index, the next wait
+            # reports it): the call no longer waits for its kernel, so this is the gather kernel's own rate
+            previous = B.bounds_policy("defer")
+            try:
+                _, ms = tstat(lambda: Nx.take(table, nxt()), steps, warm)
+            finally:
+                B.bounds_policy(previous)
+            entry("take_bf16_8192_of_32000x4096_rotated_deferred_bounds", 134250496.0, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+            del logits, table, idx, nxt
+
+        if section("misc"):
+            # selection, windows and creation at the HBM-resident size of config 1
+            nn = 16384
+            N = nn * nn
             x, y = W.elementwise_reduce(n=nn)
             x, y = put(x, "f32"), put(y, "f32")
-            N = nn * nn
-            _, ms = tstat(lambda: Nx.add(x, y), steps, warm)
-            entry(f"add_f32_{nn}", 12.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-            _, ms = tstat(lambda: Nx.multiply(x, 0.5), steps, warm)
-            entry(f"multiply_scalar_f32_{nn}", 8.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-            _, ms = tstat(lambda: Nx.exp(x), steps, warm)
-            entry(f"exp_f32_{nn}", 8.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-            _, ms = tstat(lambda: Nx.sum(x, axes=[1]), steps, warm)
-            entry(f"sum_rows_f32_{nn}", 4.0 * N + 4.0 * nn, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read")
-            # the whole unfused chain of config 1: add -> multiply 0.5 -> exp -> sum over axis 1
-            _, ms = tstat(lambda: Nx.sum(Nx.exp(Nx.multiply(Nx.add(x, y), 0.5)), axes=[1]), steps, warm)
-            entry(f"config1_chain_f32_{nn}", 32.0 * N + 4.0 * nn, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+            pred = Nx.greater(x, y)
+            _, ms = tstat(lambda: Nx.select(pred, x, y), steps, warm)
+            entry(f"select_f32_{nn}", 13.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+            # take along the last axis (picks within each row: the row goes through LDS), late-raising bounds policy
+            cols_idx = put(np.random.default_rng(6).integers(0, nn, size=nn, dtype=np.int32), "s32")
+            previous = B.bounds_policy("defer")
+            try:
+                _, ms = tstat(lambda: Nx.take(x, cols_idx, axis=1), steps, warm)
+            finally:
+                B.bounds_policy(previous)
+            entry(f"take_last_axis_f32_{nn}_deferred_bounds", 8.0 * N + 4.0 * nn, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+            del cols_idx
+            _, ms = tstat(lambda: Nx.clip(x, -0.5, 0.5), steps, warm)
+            entry(f"clip_f32_{nn}", 8.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+            _, ms = tstat(lambda: Nx.slice(x, [64, 128], [nn - 128, nn - 256]), steps, warm)
+            entry(f"slice_f32_{nn}", 8.0 * (nn - 128) * (nn - 256), "GB/s", ms, PEAK_HBM_GBS, "hbm")
+            del pred
+            _, ms = tstat(lambda: Nx.concatenate([x, y], axis=1), steps, warm)
+            entry(f"concatenate_axis1_f32_{nn}", 16.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+            _, ms = tstat(lambda: Nx.all(x, axes=[1]), steps, warm)
+            entry(f"all_rows_f32_{nn}", 4.0 * N + nn, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read")
+            _, ms = tstat(lambda: Nx.iota((nn, nn), type="f32", axis=1, backend=H), steps, warm)
+            entry(f"iota_f32_{nn}", 4.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_write")
             del x, y
 
-        # the same callbacks on the 2-byte type of most model tensors (bf16, 16384^2), a column sum and a transpose
-        rng16 = np.random.default_rng(16)
-        bx = put((rng16.standard_normal((16384, 16384)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16), "bf16")
-        N = 16384 * 16384
-        by = put((rng16.standard_normal((16384, 16384)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16), "bf16")
-        _, ms = tstat(lambda: Nx.add(bx, by), steps, warm)
-        entry("add_bf16_16384", 6.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-        del by
-        _, ms = tstat(lambda: Nx.exp(bx), steps, warm)
-        entry("exp_bf16_16384", 4.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-        _, ms = tstat(lambda: Nx.sum(bx, axes=[1]), steps, warm)
-        entry("sum_rows_bf16_16384", 2.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read")
-        _, ms = tstat(lambda: Nx.sum(bx, axes=[0]), steps, warm)
-        entry("sum_columns_bf16_16384", 2.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read")
-        _, ms = tstat(lambda: Nx.argmax(bx, axis=1), steps, warm)
-        entry("argmax_rows_bf16_16384", 2.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read")
-        _, ms = tstat(lambda: Nx.transpose(bx), steps, warm)
-        entry("transpose_bf16_16384", 4.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-        _, ms = tstat(lambda: Nx.as_type(bx, "f32"), steps, warm)
-        entry("as_type_bf16_f32_16384", 6.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-        del bx
+        if section("random"):
+            # Nx.Random on the device: 2^28 u32 words from one key (counter-based, write-only), and
+            # uniform f32 samples built on them by the reference's chain of element-wise callbacks
+            from nx_amd import random as Random
+            key = Random.key(1701, backend=H)
+            nw = 1 << 28
+            _, ms = tstat(lambda: Random.random_bits(key, shape=(nw,)), steps, warm)
+            entry("random_bits_u32_2p28", 4.0 * nw, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_write")
+            _, ms = tstat(lambda: Random.uniform_split(key, 0.0, 1.0, shape=(nw,)), steps, warm)
+            unfused_ms = float(ms)
+            # bits out; shift, or, subtract, multiply, add, max each read and write the array once
+            entry("uniform_f32_2p28_unfused", 4.0 * nw * 13, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+            # the same function traced, its bits-to-floats chain (shift, or, bitcast, subtract, ..., max) planned as
+            # one group compiled for the device: the cipher writes the words, one more pass reads them and writes floats
+            from nx_amd import defn as _defn
+            uniform = _defn.compile(lambda k: Random.uniform_split(k, 0.0, 1.0, shape=(nw,)), key, fuse="compiled")
+            _, ms = tstat(lambda: uniform(key), steps, warm)
+            # priced at what it moves: the words written, then read once and the floats written
+            entry("uniform_f32_2p28_fused_compiled", 4.0 * nw * 3, "GB/s", ms, PEAK_HBM_GBS, "hbm", vs=("unfused", unfused_ms))
+            del key, uniform
 
-        # config 3: attention scores + softmax chain
-        q, k = W.attention_scores()
-        q, k = put(q, "bf16"), put(k, "bf16")
-        _, ms = tstat(lambda: Nx.dot(q, [2], [0], k, [2], [0]), steps, warm)
-        entry("dot_qk_bf16_32x512x64", 20971520.0, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_write")
-        q_np, k_np = W.attention_scores()
-        nxt = rotating(lambda: (put(q_np, "bf16"), put(k_np, "bf16")), q_np.nbytes + k_np.nbytes)
+        if section("chains"):
+            # traced chains: one callback per node (the evaluator), and the same chain captured once and
+            # replayed as a device graph (one submission for all its kernels)
+            from nx_amd import defn
+            from nx_amd.backend import fused_mode
 
-        def qk_rot():
-            qq, kk = nxt()
-            return Nx.dot(qq, [2], [0], kk, [2], [0])
-        _, ms = tstat(qk_rot, steps, warm)
-        entry("dot_qk_bf16_32x512x64_rotated", 20971520.0, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_write")
-        del nxt
-        s = Nx.dot(q, [2], [0], k, [2], [0])
+            def chain1(a, b):
+                return Nx.sum(Nx.exp(Nx.multiply(Nx.add(a, b), 0.5)), axes=[1])
 
-        def softmax():
-            z = Nx.multiply(Nx.as_type(s, "f32"), 0.125)
-            e = Nx.exp(Nx.subtract(z, Nx.reduce_max(z, axes=[2], keep_axes=True)))
-            return Nx.divide(e, Nx.sum(e, axes=[2], keep_axes=True))
-        _, ms = tstat(softmax, steps, warm)
-        entry("softmax_chain_32x512x512", 386138112.0, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-        nxt = rotating(lambda: Nx.dot(q, [2], [0], k, [2], [0]), 32 * 512 * 512 * 2)
+            def chain3(scores):
+                z = Nx.multiply(Nx.as_type(scores, "f32"), 0.125)
+                e = Nx.exp(Nx.subtract(z, Nx.reduce_max(z, axes=[2], keep_axes=True)))
+                return Nx.divide(e, Nx.sum(e, axes=[2], keep_axes=True))
 
-        def softmax_rot():
-            z = Nx.multiply(Nx.as_type(nxt(), "f32"), 0.125)
-            e = Nx.exp(Nx.subtract(z, Nx.reduce_max(z, axes=[2], keep_axes=True)))
-            return Nx.divide(e, Nx.sum(e, axes=[2], keep_axes=True))
-        _, ms = tstat(softmax_rot, steps, warm)
-        entry("softmax_chain_32x512x512_rotated", 386138112.0, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-        del q, k, s, nxt
-
-        # config 4: int8 weight-only linear
-        w, xq, sc = W.int8_linear()
-        w, xq, sc = put(w, "s8"), put(xq, "s8"), put(sc, "f32")
-        _, ms = tstat(lambda: Nx.dot(xq, [1], w, [1], out_type="s32"), steps, warm)
-        entry("dot_s8_w8_64x11008x4096", 48168960.0, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read")
-        suite["dot_s8_w8_64x11008x4096"]["tops"] = round(5771362304.0 / (ms * 1e-3) / 1e12, 2)
-        w_np = W.int8_linear()[0]
-        nxt = rotating(lambda: put(w_np, "s8"), w_np.nbytes)
-        _, ms = tstat(lambda: Nx.dot(xq, [1], nxt(), [1], out_type="s32"), steps, warm)
-        entry("dot_s8_w8_64x11008x4096_rotated", 48168960.0, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read")
-        # the same layer with its weights stored [K, N], the plain Nx.dot(x, w) of a dense layer (K-outer weights)
-        nxt_t = rotating(lambda: put(np.ascontiguousarray(w_np.T), "s8"), w_np.nbytes)
-        _, ms = tstat(lambda: Nx.dot(xq, nxt_t(), out_type="s32"), steps, warm)
-        del nxt_t
-        entry("dot_s8_w8_64x11008x4096_weights_k_outer_rotated", 48168960.0, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read")
-        # the whole config: dot -> as_type f32 -> multiply by the per-column scales
-        _, ms = tstat(lambda: Nx.multiply(Nx.as_type(Nx.dot(xq, [1], nxt(), [1], out_type="s32"), "f32"), sc), steps, warm)
-        entry("config4_chain_rotated", 48168960.0 + 5636096.0 + 5680128.0, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-        del w, xq, sc, nxt
-
-        # config 5: argmax + take
-        logits, table, _ = W.logits_and_table()
-        logits, table = put(logits, "f32"), put(table, "bf16")
-        _, ms = tstat(lambda: Nx.argmax(logits, axis=1, type="u32"), steps, warm)
-        entry("argmax_f32_8192x32000", 1048608768.0, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read")
-        idx = Nx.argmax(logits, axis=1, type="u32")
-        _, ms = tstat(lambda: Nx.take(table, idx), steps, warm)
-        entry("take_bf16_8192_of_32000x4096", 134250496.0, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-        suite["take_bf16_8192_of_32000x4096"]["note"] = (
-            "per call, not per kernel; the indices are the argmax's own result, which the library knows to lie within "
-            "an axis of 32000 entries: the raising bounds policy does not wait for the kernel (the kernel itself "
-            "runs ~22 us = ~6.1 TB/s by the rocprofv3 kernel trace)")
-        # other rows every step (nine index sets, 600 MB of table rows in all: nothing comes from the cache), each set
-        # the argmax over its own {8192, 32000} tensor of random words as in the configuration (indices written by
-        # argmax are known to lie within an axis of that length, so the raising policy has nothing to wait for)
-        from nx_amd import random as Random
-        ring = []
-        for part in range(9):
-            ring.append(Nx.argmax(Random.random_bits(Random.key(505 + part, backend=H), shape=(8192, 32000)), axis=1, type="u32"))
-        pos = [0]
-
-        def next_argmax_indices():
-            pos[0] = (pos[0] + 1) % len(ring)
-            return ring[pos[0]]
-        _, ms = tstat(lambda: Nx.take(table, next_argmax_indices()), steps, warm)
-        entry("take_bf16_8192_of_32000x4096_rotated", 134250496.0, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-        del ring
-        # indices from anywhere else (uploaded from the host): every call waits for its kernel, as the reference's
-        # raising bounds check demands
-        rng = np.random.default_rng(5)
-        nxt = rotating(lambda: put(rng.integers(0, 32000, size=8192, dtype=np.uint32), "u32"), 40e6)
-        _, ms = tstat(lambda: Nx.take(table, nxt()), steps, warm)
-        entry("take_bf16_8192_of_32000x4096_rotated_foreign_indices", 134250496.0, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-        # the same with the bounds policy that raises late (the kernel records a bad index, the next wait
-        # reports it): the call no longer waits for its kernel, so this is the gather kernel's own rate
-        previous = B.bounds_policy("defer")
-        try:
-            _, ms = tstat(lambda: Nx.take(table, nxt()), steps, warm)
-        finally:
-            B.bounds_policy(previous)
-        entry("take_bf16_8192_of_32000x4096_rotated_deferred_bounds", 134250496.0, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-        del logits, table, idx, nxt
-
-        # selection, windows and creation at the HBM-resident size of config 1
-        nn = 16384
-        N = nn * nn
-        x, y = W.elementwise_reduce(n=nn)
-        x, y = put(x, "f32"), put(y, "f32")
-        pred = Nx.greater(x, y)
-        _, ms = tstat(lambda: Nx.select(pred, x, y), steps, warm)
-        entry(f"select_f32_{nn}", 13.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-        # take along the last axis (picks within each row: the row goes through LDS), late-raising bounds policy
-        cols_idx = put(np.random.default_rng(6).integers(0, nn, size=nn, dtype=np.int32), "s32")
-        previous = B.bounds_policy("defer")
-        try:
-            _, ms = tstat(lambda: Nx.take(x, cols_idx, axis=1), steps, warm)
-        finally:
-            B.bounds_policy(previous)
-        entry(f"take_last_axis_f32_{nn}_deferred_bounds", 8.0 * N + 4.0 * nn, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-        del cols_idx
-        _, ms = tstat(lambda: Nx.clip(x, -0.5, 0.5), steps, warm)
-        entry(f"clip_f32_{nn}", 8.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-        _, ms = tstat(lambda: Nx.slice(x, [64, 128], [nn - 128, nn - 256]), steps, warm)
-        entry(f"slice_f32_{nn}", 8.0 * (nn - 128) * (nn - 256), "GB/s", ms, PEAK_HBM_GBS, "hbm")
-        del pred
-        _, ms = tstat(lambda: Nx.concatenate([x, y], axis=1), steps, warm)
-        entry(f"concatenate_axis1_f32_{nn}", 16.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-        _, ms = tstat(lambda: Nx.all(x, axes=[1]), steps, warm)
-        entry(f"all_rows_f32_{nn}", 4.0 * N + nn, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read")
-        _, ms = tstat(lambda: Nx.iota((nn, nn), type="f32", axis=1, backend=H), steps, warm)
-        entry(f"iota_f32_{nn}", 4.0 * N, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_write")
-        del x, y
-
-        # Nx.Random on the device: 2^28 u32 words from one key (counter-based, write-only), and
-        # uniform f32 samples built on them by the reference's chain of element-wise callbacks
-        from nx_amd import random as Random
-        key = Random.key(1701, backend=H)
-        nw = 1 << 28
-        _, ms = tstat(lambda: Random.random_bits(key, shape=(nw,)), steps, warm)
-        entry("random_bits_u32_2p28", 4.0 * nw, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_write")
-        _, ms = tstat(lambda: Random.uniform_split(key, 0.0, 1.0, shape=(nw,)), steps, warm)
-        unfused_ms = float(ms)
-        # bits out; shift, or, subtract, multiply, add, max each read and write the array once
-        entry("uniform_f32_2p28_unfused", 4.0 * nw * 13, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-        # the same function traced, its bits-to-floats chain (shift, or, bitcast, subtract, ..., max) planned as
-        # one group compiled for the device: the cipher writes the words, one more pass reads them and writes floats
-        from nx_amd import defn as _defn
-        uniform = _defn.compile(lambda k: Random.uniform_split(k, 0.0, 1.0, shape=(nw,)), key, fuse="compiled")
-        _, ms = tstat(lambda: uniform(key), steps, warm)
-        # priced at what it moves: the words written, then read once and the floats written
-        entry("uniform_f32_2p28_fused_compiled", 4.0 * nw * 3, "GB/s", ms, PEAK_HBM_GBS, "hbm", vs=("unfused", unfused_ms))
-        del key, uniform
-
-        # traced chains: one callback per node (the evaluator), and the same chain captured once and
-        # replayed as a device graph (one submission for all its kernels)
-        from nx_amd import defn
-        from nx_amd.backend import fused_mode
-
-        def chain1(a, b):
-            return Nx.sum(Nx.exp(Nx.multiply(Nx.add(a, b), 0.5)), axes=[1])
-
-        def chain3(scores):
-            z = Nx.multiply(Nx.as_type(scores, "f32"), 0.125)
-            e = Nx.exp(Nx.subtract(z, Nx.reduce_max(z, axes=[2], keep_axes=True)))
-            return Nx.divide(e, Nx.sum(e, axes=[2], keep_axes=True))
-
-        def chain4(xq_, w_, sc_):
-            return Nx.multiply(Nx.as_type(Nx.dot(xq_, [1], w_, [1], out_type="s32"), "f32"), sc_)
-        x, y = W.elementwise_reduce(n=1024)
-        q, k = W.attention_scores()
-        w, xq, sc = W.int8_linear()
-        q, k = put(q, "bf16"), put(k, "bf16")
-        n1, ns = 1024 * 1024, 32 * 512 * 512
-        # name -> (function, arguments, bytes node by node, bytes as fused groups, bytes planned as one kernel)
-        cases = {"config1_chain_f32_1024": (chain1, (put(x, "f32"), put(y, "f32")), 32.0 * n1 + 4096.0, 8.0 * n1 + 4096.0, 8.0 * n1 + 4096.0),
-                 "softmax_chain_32x512x512": (chain3, (Nx.dot(q, [2], [0], k, [2], [0]),), 386138112.0, 10.0 * ns + 8.0 * 16384, 6.0 * ns),
-                 "config4_chain": (chain4, (put(xq, "s8"), put(w, "s8"), put(sc, "f32")), 48168960.0 + 5636096.0 + 5680128.0, 48212992.0, 48212992.0)}
-        for name, (fun, targs, nbytes, fbytes, pbytes) in cases.items():
-            compiled = defn.compile(fun, *targs)
-            _, ms = tstat(lambda: compiled(*targs), steps, warm)
-            traced_ms = float(ms)
-            entry(name + "_traced", nbytes, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-            captured = compiled.capture(*targs)
-            held = captured.inputs  # arguments already in the captured buffers: no copies in
-            _, ms = tstat(lambda: captured(*held), steps, warm)
-            entry(name + "_graph", nbytes, "GB/s", ms, PEAK_HBM_GBS, "hbm", vs=("traced", traced_ms))
-            captured.destroy()
-            # (for configuration 4 the planner also finishes the layer on the dot's accumulators: dot, as_type and
-            # the multiplication by the scales are one kernel)
-            # element-wise groups (with the row reduction that follows them) as one kernel each: decoded by
-            # the interpreting kernels, then with each group's program compiled for the device on first use.
-            # A fused entry is priced at the bytes IT moves; `vs_traced` is its speed-up over node by node.
-            fused = defn.compile(fun, *targs, fuse=True)
+            def chain4(xq_, w_, sc_):
+                return Nx.multiply(Nx.as_type(Nx.dot(xq_, [1], w_, [1], out_type="s32"), "f32"), sc_)
+            x, y = W.elementwise_reduce(n=1024)
+            q, k = W.attention_scores()
+            w, xq, sc = W.int8_linear()
+            q, k = put(q, "bf16"), put(k, "bf16")
+            n1, ns = 1024 * 1024, 32 * 512 * 512
+            # name -> (function, arguments, bytes node by node, bytes as fused groups, bytes planned as one kernel)
+            cases = {"config1_chain_f32_1024": (chain1, (put(x, "f32"), put(y, "f32")), 32.0 * n1 + 4096.0, 8.0 * n1 + 4096.0, 8.0 * n1 + 4096.0),
+                     "softmax_chain_32x512x512": (chain3, (Nx.dot(q, [2], [0], k, [2], [0]),), 386138112.0, 10.0 * ns + 8.0 * 16384, 6.0 * ns),
+                     "config4_chain": (chain4, (put(xq, "s8"), put(w, "s8"), put(sc, "f32")), 48168960.0 + 5636096.0 + 5680128.0, 48212992.0, 48212992.0)}
+            for name, (fun, targs, nbytes, fbytes, pbytes) in cases.items():
+                compiled = defn.compile(fun, *targs)
+                _, ms = tstat(lambda: compiled(*targs), steps, warm)
+                traced_ms = float(ms)
+                entry(name + "_traced", nbytes, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+                captured = compiled.capture(*targs)
+                held = captured.inputs  # arguments already in the captured buffers: no copies in
+                _, ms = tstat(lambda: captured(*held), steps, warm)
+                entry(name + "_graph", nbytes, "GB/s", ms, PEAK_HBM_GBS, "hbm", vs=("traced", traced_ms))
+                captured.destroy()
+                # (for configuration 4 the planner also finishes the layer on the dot's accumulators: dot, as_type and
+                # the multiplication by the scales are one kernel)
+                # element-wise groups (with the row reduction that follows them) as one kernel each: decoded by
+                # the interpreting kernels, then with each group's program compiled for the device on first use.
+                # A fused entry is priced at the bytes IT moves; `vs_traced` is its speed-up over node by node.
+                fused = defn.compile(fun, *targs, fuse=True)
+                for mode, tag in (("interpreted", "_fused"), ("compiled", "_fused_compiled")):
+                    fused_mode(mode)
+                    _, ms = tstat(lambda: fused(*targs), steps, warm)
+                    entry(name + tag, fbytes, "GB/s", ms, PEAK_HBM_GBS, "hbm", vs=("traced", traced_ms))
+                fused_mode("interpreted")
+                # planned for compiled kernels from the start: groups over the same rows become stages of one program
+                # (the softmax: row maximum, sum of exponentials and division in one kernel)
+                staged = defn.compile(fun, *targs, fuse="compiled")
+                _, ms = tstat(lambda: staged(*targs), steps, warm)
+                entry(name + "_planned_compiled", pbytes, "GB/s", ms, PEAK_HBM_GBS, "hbm", vs=("traced", traced_ms))
+            x, y = W.elementwise_reduce(n=16384)
+            big = (put(x, "f32"), put(y, "f32"))
+            node_ms = suite["config1_chain_f32_16384"]["ms"] if "config1_chain_f32_16384" in suite else None
+            fused = defn.compile(chain1, *big, fuse=True)
+            # priced at what the one pass moves (both operands once, one value per row)
             for mode, tag in (("interpreted", "_fused"), ("compiled", "_fused_compiled")):
                 fused_mode(mode)
-                _, ms = tstat(lambda: fused(*targs), steps, warm)
-                entry(name + tag, fbytes, "GB/s", ms, PEAK_HBM_GBS, "hbm", vs=("traced", traced_ms))
+                _, ms = tstat(lambda: fused(*big), steps, warm)
+                entry("config1_chain_f32_16384" + tag, 8.0 * 16384 * 16384 + 4.0 * 16384, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read",
+                      vs=("node_by_node", node_ms) if node_ms else None)
             fused_mode("interpreted")
-            # planned for compiled kernels from the start: groups over the same rows become stages of one program
-            # (the softmax: row maximum, sum of exponentials and division in one kernel)
-            staged = defn.compile(fun, *targs, fuse="compiled")
-            _, ms = tstat(lambda: staged(*targs), steps, warm)
-            entry(name + "_planned_compiled", pbytes, "GB/s", ms, PEAK_HBM_GBS, "hbm", vs=("traced", traced_ms))
-        x, y = W.elementwise_reduce(n=16384)
-        big = (put(x, "f32"), put(y, "f32"))
-        node_ms = suite["config1_chain_f32_16384"]["ms"]
-        fused = defn.compile(chain1, *big, fuse=True)
-        # priced at what the one pass moves (both operands once, one value per row)
-        for mode, tag in (("interpreted", "_fused"), ("compiled", "_fused_compiled")):
-            fused_mode(mode)
-            _, ms = tstat(lambda: fused(*big), steps, warm)
-            entry("config1_chain_f32_16384" + tag, 8.0 * 16384 * 16384 + 4.0 * 16384, "GB/s", ms, PEAK_HBM_GBS, "hbm", "stream_read",
-                  vs=("node_by_node", node_ms))
-        fused_mode("interpreted")
-        del big, x, y
-        del cases, q, k
+            del big, x, y
+            del cases, q, k
 
-        # the one benchmark the reference publishes (nx/README.md:135-146, exla/bench/softmax.exs:1-41):
-        # softmax(n) = exp(n) / sum(exp(n)) on 1,000,000 uniform values kept on the device, f32 and f64 --
-        # node by node (four callbacks: exp, exp, sum over all axes, divide by the rank-0 sum) and traced with
-        # its groups planned for compiled kernels.  Its published figures (hardware unstated) ride along as context.
-        published = {"f32": {"exla_gpu_kept_on_device_us": 65.3, "exla_host_jit_us": 2300.0, "binary_backend_us": 311010.0},
-                     "f64": {"exla_gpu_kept_on_device_us": 220.0, "exla_host_jit_us": 5940.0, "binary_backend_us": 321700.0}}
-        rng1m = np.random.default_rng(1000000)
-        vals = rng1m.random(1000000)
+        if section("softmax1m"):
+            # the one benchmark the reference publishes (nx/README.md:135-146, exla/bench/softmax.exs:1-41):
+            # softmax(n) = exp(n) / sum(exp(n)) on 1,000,000 uniform values kept on the device, f32 and f64 --
+            # node by node (four callbacks: exp, exp, sum over all axes, divide by the rank-0 sum) and traced with
+            # its groups planned for compiled kernels.  Its published figures (hardware unstated) ride along as context.
+            published = {"f32": {"exla_gpu_kept_on_device_us": 65.3, "exla_host_jit_us": 2300.0, "binary_backend_us": 311010.0},
+                         "f64": {"exla_gpu_kept_on_device_us": 220.0, "exla_host_jit_us": 5940.0, "binary_backend_us": 321700.0}}
+            rng1m = np.random.default_rng(1000000)
+            vals = rng1m.random(1000000)
 
-        def softmax1m(n_):
-            return Nx.divide(Nx.exp(n_), Nx.sum(Nx.exp(n_)))
-        for ty, npt, esz in (("f32", np.float32, 4), ("f64", np.float64, 8)):
-            t1m = put(vals.astype(npt), ty)
-            nel = 1000000.0
-            _, ms = tstat(lambda: softmax1m(t1m), steps, warm)
-            eager_ms = float(ms)
-            # exp, exp: 2 x (read + write); sum: read + one element; divide: read + read of one element + write
-            entry(f"softmax_1M_{ty}", esz * nel * 7 + 3 * esz, "GB/s", ms, PEAK_HBM_GBS, "hbm")
-            suite[f"softmax_1M_{ty}"]["reference_published_us"] = published[ty]
-            suite[f"softmax_1M_{ty}"]["note"] = ("4 MB (8 MB) tensors: launch-bound, not bandwidth-bound; the reference's figures are for unstated "
-                                                 "hardware (nx/README.md:135-146)")
-            try:
-                planned = defn.compile(softmax1m, t1m, fuse="compiled")
-                _, ms = tstat(lambda: planned(t1m), steps, warm)
-                # priced at what it has to move: the values read (twice: once for the sum, once for the quotient) and written
-                entry(f"softmax_1M_{ty}_planned_compiled", esz * nel * 3, "GB/s", ms, PEAK_HBM_GBS, "hbm", vs=("unfused", eager_ms))
-                del planned
-            except Exception as exc:  # a type the planner does not group: the node-by-node figure stands
-                suite[f"softmax_1M_{ty}_planned_compiled"] = {"error": str(exc)[:160]}
-            del t1m
+            def softmax1m(n_):
+                return Nx.divide(Nx.exp(n_), Nx.sum(Nx.exp(n_)))
+            for ty, npt, esz in (("f32", np.float32, 4), ("f64", np.float64, 8)):
+                t1m = put(vals.astype(npt), ty)
+                nel = 1000000.0
+                _, ms = tstat(lambda: softmax1m(t1m), steps, warm)
+                eager_ms = float(ms)
+                # exp, exp: 2 x (read + write); sum: read + one element; divide: read + read of one element + write
+                entry(f"softmax_1M_{ty}", esz * nel * 7 + 3 * esz, "GB/s", ms, PEAK_HBM_GBS, "hbm")
+                suite[f"softmax_1M_{ty}"]["reference_published_us"] = published[ty]
+                suite[f"softmax_1M_{ty}"]["note"] = ("4 MB (8 MB) tensors: launch-bound, not bandwidth-bound; the reference's figures are for unstated "
+                                                     "hardware (nx/README.md:135-146)")
+                try:
+                    planned = defn.compile(softmax1m, t1m, fuse="compiled")
+                    _, ms = tstat(lambda: planned(t1m), steps, warm)
+                    # priced at what it has to move: the values read (twice: once for the sum, once for the quotient) and written
+                    entry(f"softmax_1M_{ty}_planned_compiled", esz * nel * 3, "GB/s", ms, PEAK_HBM_GBS, "hbm", vs=("unfused", eager_ms))
+                    del planned
+                except Exception as exc:  # a type the planner does not group: the node-by-node figure stands
+                    suite[f"softmax_1M_{ty}_planned_compiled"] = {"error": str(exc)[:160]}
+                del t1m
         result["suite"] = suite
-        result["host_transfers"] = host_transfer_figures(H, B, Nx, template)
-        c_abi = c_abi_figures()
+        if args.only is None:
+            result["host_transfers"] = host_transfer_figures(H, B, Nx, template)
+        c_abi = c_abi_figures() if args.only is None else None
         if c_abi:
             result["c_abi"] = c_abi
             if "config1_chain_f32_1024_us" in c_abi:
