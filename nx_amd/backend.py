@@ -908,13 +908,11 @@ class HipNxBackend:
         EUNSUPPORTED when the shapes do not fit the kernel: the caller then runs the nodes one by one.
         `mode` ("interpreted" / "compiled") runs this call in that mode whatever the device is set to."""
         dev = cls._device_of(*inputs) if inputs else 0
-        previous = _fused_modes.get(dev, "interpreted")
-        if mode is not None and previous != mode:
-            fused_mode(mode, dev)
-            try:
-                return cls.fused_elementwise(out, program, inputs, layout, reduce_op)
-            finally:
-                fused_mode(previous, dev)
+        # the library is switched when a call wants another mode than the last call had, not around every call:
+        # the groups of a traced function all want the same one
+        wanted = mode if mode is not None else _fused_modes.get(dev, "interpreted")
+        if _fused_set.get(dev, "interpreted") != wanted:
+            _set_fused_mode(wanted, dev)
         inputs = [cls._from_nx(t, dev) for t in inputs]
         rows, cols, strides = layout
         prog = getattr(program, "packed", None)
@@ -1106,11 +1104,16 @@ def fused_mode(mode: str, device: int = 0) -> None:
     """How fused groups run on the device from now on: "interpreted" (one pair of kernels decodes any
     program; the default) or "compiled" (each distinct program is compiled for the device once, on
     first use, and kept).  Results are bit-identical."""
+    _set_fused_mode(mode, device)
+    _fused_modes[device] = mode
+
+
+def _set_fused_mode(mode: str, device: int) -> None:
     codes = {"interpreted": L.FUSED_INTERPRETED, "compiled": L.FUSED_COMPILED}
     if mode not in codes:
         raise ValueError(f"expected one of {sorted(codes)!r}, got: {mode!r}")
     L.check(L.lib.hipnx_fused_set_mode(_Context.get(device), codes[mode]))
-    _fused_modes[device] = mode
+    _fused_set[device] = mode
 
 
 _encoded = {}  # (type, class of the number, number) -> its encoding (constant/3)
@@ -1132,7 +1135,8 @@ def _advise_huge_pages(address: int, n: int) -> None:
         lo, hi = (address + huge - 1) & ~(huge - 1), (address + n) & ~(huge - 1)
         if hi > lo:
             _libc.madvise(C.c_void_p(lo), hi - lo, 14)  # MADV_HUGEPAGE
-_fused_modes = {}  # device -> the mode last set here
+_fused_modes = {}  # device -> the mode chosen with fused_mode/2: what a call that names none runs in
+_fused_set = {}    # device -> the mode the library is in at this moment (a call that names one leaves it there)
 _fused_arrays = {}  # (id of a layout, input types) -> (the layout itself, so the id stays its own; C arrays of types and strides)
 
 

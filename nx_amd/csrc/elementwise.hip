@@ -213,6 +213,58 @@ binary_vec_kernel(const void *__restrict__ l, const void *__restrict__ r, void *
   }
 }
 
+// The common case of the above as a kernel of its own: element types known when it is compiled, an operation that
+// cannot raise, rows that are whole vectors and one stride pair per operand -- [rows, cols] against itself, a row
+// [cols], one value per row or one value.  Every wave of the general kernel spends some 0.4 us on eleven scalar
+// loads of its arguments and the branches that choose its path before it asks for data; a wave lives for about
+// 2.5 us, and at 4 to 64 MiB the grid is few waves deep, so that time shows: 8.4 M f32 elements, x * scalar
+// 11.7 -> 10.6 us, x - value per row 10.7 -> 9.7 us, x + y 16.1 -> 14.7 us.
+//   LM / RM: how an operand is met: 0 one value (read through the scalar cache: one address asked for by every
+//   wave at once is a hot spot in the vector path), 1 one value per row, 2 whole vectors (row * s0 + col).
+//   U vectors per lane, lanes side by side (v, v + 256, ...), every load issued before the first result is formed:
+//   two for x + y of 1 to 64 MiB a side (32 MiB: 15.3 -> 14.7 us); beyond the last-level cache one streams faster
+//   (1 GiB a side: 534 against 562 us).
+template <int OP, typename CT, bool UNS, int FIX, int FIXO, int LM, int RM, int U>
+__global__ void __launch_bounds__(BLOCK)
+binary_rows_kernel(const void *__restrict__ l, const void *__restrict__ r, void *__restrict__ out, uint32_t nvec,
+                   uint32_t vecs_per_row, FastDiv32 fd, int64_t ls0, int64_t rs0) {
+  constexpr int E = vec_elems(FIX, FIXO);
+  const uint32_t v0 = blockIdx.x * (uint32_t)(BLOCK * U) + threadIdx.x;
+  CT a[U][E], b[U][E];
+  CT l_one = (CT)0, r_one = (CT)0;
+  if constexpr (LM == 0) l_one = load_one<CT>(l, FIX, 0);
+  if constexpr (RM == 0) r_one = load_one<CT>(r, FIX, 0);
+#pragma unroll
+  for (int u = 0; u < U; u++) {
+    const uint32_t v = v0 + u * BLOCK;
+    if (v < nvec) {
+      const uint32_t row = fastdiv(v, fd), col = (v - row * vecs_per_row) * E;
+      if constexpr (LM == 2) load_vec<CT, E>(l, FIX, (int64_t)row * ls0 + col, a[u]);
+      else {
+        const CT s = LM == 0 ? l_one : load_one<CT>(l, FIX, (int64_t)row * ls0);
+#pragma unroll
+        for (int i = 0; i < E; i++) a[u][i] = s;
+      }
+      if constexpr (RM == 2) load_vec<CT, E>(r, FIX, (int64_t)row * rs0 + col, b[u]);
+      else {
+        const CT s = RM == 0 ? r_one : load_one<CT>(r, FIX, (int64_t)row * rs0);
+#pragma unroll
+        for (int i = 0; i < E; i++) b[u][i] = s;
+      }
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < U; u++) {
+    const uint32_t v = v0 + u * BLOCK;
+    if (v < nvec) {
+      CT c[E];
+#pragma unroll
+      for (int i = 0; i < E; i++) c[i] = binary_apply<OP, CT, UNS>(a[u][i], b[u][i]);
+      store_vec<CT, E>(out, FIXO, (int64_t)v * E, c);
+    }
+  }
+}
+
 template <typename CT, bool UNS>
 __device__ __forceinline__ CT binary_switch(int op, CT a, CT b) {
   switch (op) {
@@ -361,6 +413,29 @@ static void launch_bvec_fix(const hipnx_ctx *ctx, const BinArgs &a_) {
     a.nvec = (a.flat_total + EV - 1) / EV;
     mode = a.flat_total < (1ll << 31) ? ROWS_FLAT : ROWS_FLAT_WIDE;
     if (mode == ROWS_FLAT) fd = make_fastdiv((uint32_t)a.cols);
+  }
+  if constexpr (FIX >= 0 && !binary_can_raise(OP, is_fp<CT>::value)) {
+    if (a.flat_total <= 0 && a.ax.n <= 1 && a.cols % EV == 0 && a.nvec < (1ll << 31)) {
+      const bool one_row = mode == ROWS_ONE;
+      const uint32_t nvec = (uint32_t)a.nvec, vpr = one_row ? nvec : (uint32_t)a.vecs_per_row;
+      const FastDiv32 fdr = make_fastdiv(vpr);
+      // how each operand is met (an operand of one row has no row stride to speak of)
+      const int64_t l0 = one_row ? 0 : a.ls0, r0 = one_row ? 0 : a.rs0;
+      const int lm = a.ls1 ? 2 : l0 ? 1 : 0, rm = a.rs1 ? 2 : r0 ? 1 : 0;
+#define HIPNX_ROWS(LM, RM, U)                                                                                         \
+  hipLaunchKernelGGL((binary_rows_kernel<OP, CT, UNS, FIX, FIXO, LM, RM, U>),                                         \
+                     dim3((unsigned)((a.nvec + BLOCK * U - 1) / (BLOCK * U))), dim3(BLOCK), 0, ctx->stream, a.l, a.r, \
+                     a.out, nvec, vpr, fdr, l0, r0)
+      const int how = lm * 3 + rm;
+      if (how == 8 && a.nvec >= (1 << 16) && a.nvec <= (1 << 22)) HIPNX_ROWS(2, 2, 2);  // (1 to 64 MiB a side)
+      else if (how == 8) HIPNX_ROWS(2, 2, 1);
+      else if (how == 7) HIPNX_ROWS(2, 1, 1);
+      else if (how == 6) HIPNX_ROWS(2, 0, 1);
+      else if (how == 5) HIPNX_ROWS(1, 2, 1);
+      else if (how == 2) HIPNX_ROWS(0, 2, 1);
+#undef HIPNX_ROWS
+      if (how == 2 || how >= 5) return;
+    }
   }
   hipLaunchKernelGGL((binary_vec_kernel<OP, CT, UNS, FIX, FIXO>), dim3(grid_for(ctx, a.nvec)), dim3(BLOCK), 0, ctx->stream, a.l,
                      a.r, a.out, a.ldt, a.rdt, a.odt, a.cols, a.vecs_per_row, a.nvec, a.ls0, a.ls1, a.rs0, a.rs1, a.err,

@@ -23,6 +23,7 @@
 // Bound by HBM: bytes(inputs) + bytes(out).
 #include "fused_ops.cuh"
 #include "internal.h"
+#include "reduce_kernels.cuh"
 
 namespace hipnx {
 
@@ -153,8 +154,22 @@ static void launch_fused_reduce(const hipnx_ctx *ctx, const FusedArgs &a) {
     const int rpb = FBLOCK / WAVE;
     hipLaunchKernelGGL((fused_reduce_rows_kernel<R, CT, WAVE>), dim3((unsigned)((a.rows + rpb - 1) / rpb)), dim3(FBLOCK), 0, ctx->stream, a);
   } else {
-    hipLaunchKernelGGL((fused_reduce_rows_kernel<R, CT, FBLOCK>), dim3((unsigned)a.rows), dim3(FBLOCK), 0, ctx->stream, a);
+    hipLaunchKernelGGL((fused_reduce_rows_kernel<R, CT, FBLOCK>), dim3((unsigned)(a.rows * a.nseg)), dim3(FBLOCK), 0, ctx->stream, a);
   }
+}
+
+// the second kernel of a reduction whose rows were cut into segments: the separate reduction's own
+static void launch_fused_combine(const hipnx_ctx *ctx, const FusedArgs &a, int reduce_op) {
+  const dim3 grid((unsigned)((a.rows + BLOCK / WAVE - 1) / (BLOCK / WAVE))), block(BLOCK);
+  if (reduce_op == HIPNX_RED_SUM)
+    hipLaunchKernelGGL((combine_partials_kernel<PlainReducer<double, HIPNX_RED_SUM, false>>), grid, block, 0, ctx->stream,
+                       (const double *)a.partial, a.out, a.out_dt, a.rows, a.nseg);
+  else if (reduce_op == HIPNX_RED_MAX)
+    hipLaunchKernelGGL((combine_partials_kernel<PlainReducer<float, HIPNX_RED_MAX, false>>), grid, block, 0, ctx->stream,
+                       (const float *)a.partial, a.out, a.out_dt, a.rows, a.nseg);
+  else
+    hipLaunchKernelGGL((combine_partials_kernel<PlainReducer<float, HIPNX_RED_MIN, false>>), grid, block, 0, ctx->stream,
+                       (const float *)a.partial, a.out, a.out_dt, a.rows, a.nseg);
 }
 
 static bool narrow(int dt) { return dt == HIPNX_BF16 || dt == HIPNX_F16 || dt == HIPNX_F32; }
@@ -330,8 +345,6 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
       return set_error(HIPNX_EUNSUPPORTED, "fused: a reduction after a program with pow, atan2, remainder, trigonometric or erf functions");
     if (!narrow(prog[n_instr - 1].dt) || !narrow(out_dt)) return set_error(HIPNX_EUNSUPPORTED, "fused: a reduction of a non-float value");
     if (cols == 0) return set_error(HIPNX_EUNSUPPORTED, "fused: a reduction over an empty axis");
-    // a few very long rows are split into segments by the separate reduction: not here
-    if (rows < (int64_t)ctx->num_cus * 8 && cols >= 2 * 16384) return set_error(HIPNX_EUNSUPPORTED, "fused: rows that the reduction would split");
   }
   if (int st = check_buf(ctx, out, (uint64_t)(reduce_op == -1 && !row_result ? n : rows) * dtype_size(out_dt), "fused out")) return st;
   if (n == 0) return HIPNX_OK;
@@ -341,12 +354,29 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
   a.cols = cols;
   a.vecs_per_row = (cols + FE - 1) / FE;
   a.nvec = rows * a.vecs_per_row;
+  a.nseg = 1;
+  a.seg_len = cols;
+  // a few very long rows are cut into segments as the separate reduction cuts them, so that the sums add in its order
+  void *partials = nullptr;
+  size_t partials_cap = 0;
+  if (reduce_op != -1) {
+    plan_row_segments(ctx, rows, cols, &a.nseg, &a.seg_len);
+    if (a.nseg > 1) {
+      if (int st = pool_alloc(ctx, (size_t)(rows * a.nseg) * sizeof(double), &partials, &partials_cap)) return st;
+      a.partial = partials;
+    }
+  }
+  // (the pool hands the memory to later work on this stream only: it may go back right after the launches)
+  struct Release {
+    hipnx_ctx *ctx; void *&p; size_t &cap;
+    ~Release() { if (p) pool_free(ctx, p, cap); }
+  } release{ctx, partials, partials_cap};
   if (ctx->fused_mode == HIPNX_FUSED_COMPILED) {
     // the same grids as the interpreting kernels below
     const bool block_per_row = (reduce_op != -1 || n_stats) && a.cols > 4096;
     int64_t grid = n_stats ? (block_per_row ? a.rows : (a.rows + FBLOCK / WAVE - 1) / (FBLOCK / WAVE))  // a wave or a block per row
                    : reduce_op == -1 ? (a.nvec + (int64_t)FBLOCK * FV - 1) / ((int64_t)FBLOCK * FV)
-                   : block_per_row ? a.rows : (a.rows + FBLOCK / WAVE - 1) / (FBLOCK / WAVE);
+                   : block_per_row ? a.rows * a.nseg : (a.rows + FBLOCK / WAVE - 1) / (FBLOCK / WAVE);
     // a launch may hold at most 2^32 - 1 lanes: the element-wise kernel loops over what a capped grid leaves, the row
     // kernels take one row (or wave of rows) per work-group and leave larger inputs to the separate callbacks
     const int64_t max_grid = ((1ll << 32) - 1) / FBLOCK;
@@ -356,15 +386,22 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
     }
     bool done = false;
     if (int st = fused_launch_compiled(ctx, a, reduce_op, block_per_row, (unsigned)grid, &done)) return st;
-    if (done) return HIPNX_OK;
+    if (done) {
+      if (a.nseg > 1) {
+        launch_fused_combine(ctx, a, reduce_op);
+        HIPNX_HIP(hipGetLastError());
+      }
+      return HIPNX_OK;
+    }
   }
   if (needs_compiled || (full && reduce_op != -1))
     return set_error(HIPNX_EUNSUPPORTED, "fused: a program that exists only compiled, first met while capturing");
-  if (reduce_op != -1 && a.rows > ((1ll << 32) - 1) / FBLOCK) return set_error(HIPNX_EUNSUPPORTED, "fused: more rows than one launch holds");
+  if (reduce_op != -1 && a.rows * a.nseg > ((1ll << 32) - 1) / FBLOCK) return set_error(HIPNX_EUNSUPPORTED, "fused: more rows than one launch holds");
   if (reduce_op == HIPNX_RED_SUM) launch_fused_reduce<PlainReducer<double, HIPNX_RED_SUM, false>, double>(ctx, a);
   else if (reduce_op == HIPNX_RED_MAX) launch_fused_reduce<PlainReducer<float, HIPNX_RED_MAX, false>, float>(ctx, a);
   else if (reduce_op == HIPNX_RED_MIN) launch_fused_reduce<PlainReducer<float, HIPNX_RED_MIN, false>, float>(ctx, a);
   if (reduce_op != -1) {
+    if (a.nseg > 1) launch_fused_combine(ctx, a, reduce_op);
     HIPNX_HIP(hipGetLastError());
     return HIPNX_OK;
   }

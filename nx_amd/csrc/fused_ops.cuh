@@ -30,6 +30,11 @@ struct FusedArgs {
   void *out;
   int out_dt, unused;
   int64_t rows, cols, vecs_per_row, nvec;
+  // a reduction of the result along rows that are cut into segments (nseg > 1): segment `seg` of a row covers the
+  // columns [seg * seg_len, min(cols, (seg + 1) * seg_len)) and leaves its raw accumulator in partial[row * nseg + seg]
+  int64_t seg_len;
+  void *partial;
+  int nseg, unused2;
 };
 
 // The argument block is read where the launch put it (the kernel-argument segment, constant address
@@ -328,7 +333,8 @@ __device__ __forceinline__ void fused_elementwise_body() {
 // in the order of reduce_rows_kernel (lane l takes the vectors l, l + TPR, ... and folds their
 // elements in turn, then lanes combine by wave shuffles and the block's waves through LDS) with the
 // same reducer policy, so the value equals what the element-wise group followed by the separate
-// reduction kernel gives, bit for bit.
+// reduction kernel gives, bit for bit.  A few very long rows are cut into segments exactly as that
+// kernel cuts them (plan_row_segments), a work-group each, and the same second kernel folds them.
 template <typename RUN, typename R, typename CT, int TPR>
 __device__ __forceinline__ void fused_reduce_rows_body() {
   static_assert(FV == 1, "one vector per lane and step");
@@ -336,11 +342,16 @@ __device__ __forceinline__ void fused_reduce_rows_body() {
   constexpr int RPB = FBLOCK / TPR;
   const int sub = threadIdx.x / TPR, lane = threadIdx.x % TPR;
   const int64_t rows = a->rows, red = a->cols;
-  const int64_t r = (int64_t)blockIdx.x * RPB + sub;
+  const int nseg = a->nseg;
+  const int64_t unit = (int64_t)blockIdx.x * RPB + sub;  // (row, segment): whole rows unless nseg > 1
+  const int64_t r = nseg > 1 ? unit / nseg : unit;
+  const int seg = nseg > 1 ? (int)(unit - r * nseg) : 0;
+  const int64_t k0 = nseg > 1 ? (int64_t)seg * a->seg_len : 0;
+  const int64_t k1 = nseg > 1 && k0 + a->seg_len < red ? k0 + a->seg_len : red;
   typename R::acc_t acc = R::init();
   if (r < rows) {
     const int64_t step = (int64_t)TPR * FE;
-    for (int64_t k = (int64_t)lane * FE; k < red; k += step) {
+    for (int64_t k = k0 + (int64_t)lane * FE; k < k1; k += step) {
       const int64_t row[FV] = {r}, col[FV] = {k};
       Vecs x;
       RUN::run(a, row, col, x);
@@ -358,7 +369,10 @@ __device__ __forceinline__ void fused_reduce_rows_body() {
       for (int w = 1; w < FBLOCK / WAVE; w++) acc = R::combine(acc, sm[w]);
     }
   }
-  if (lane == 0 && r < rows) finalize((void *)a->out, a->out_dt, r, acc);
+  if (lane == 0 && r < rows) {
+    if (nseg > 1) ((typename R::acc_t *)a->partial)[r * nseg + seg] = acc;
+    else finalize((void *)a->out, a->out_dt, r, acc);
+  }
 }
 
 // ---- several stages over the same rows in one kernel ------------------------------------------------

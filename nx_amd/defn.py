@@ -807,7 +807,7 @@ def _fuse_planned(roots: List[Tensor]) -> int:
         if len(readers) != 1 or uses.get(t.data.id) != 1 or len(t.shape) == 0:
             return False
         r = readers[0].data
-        return (r.op in _REDUCE_CODES and isinstance(r.args[0], Tensor) and r.args[0].data.id == t.data.id and list(r.args[1].get("axes") or []) == [len(t.shape) - 1])
+        return (r.op in _REDUCE_CODES and isinstance(r.args[0], Tensor) and r.args[0].data.id == t.data.id and _over_last_axis(r.args[1], len(t.shape)))
 
     for r in roots:
         walk(r)
@@ -935,7 +935,7 @@ def _fuse_planned(roots: List[Tensor]) -> int:
         if not isinstance(inner, Expr) or inner.op != "fused" or uses.get(inner.id) != 1:
             continue
         rank = len(operand.shape)
-        if list(opts.get("axes") or []) != [rank - 1]:
+        if not _over_last_axis(opts, rank):
             continue
         both = inner.args[0].with_reduction(e.op, opts)
         if both is None:
@@ -944,6 +944,13 @@ def _fuse_planned(roots: List[Tensor]) -> int:
     if _plan["ints"]:  # planned for compiled kernels: groups over the same rows become stages of one
         _cluster_rows(roots)
     return formed
+
+
+def _over_last_axis(opts, rank: int) -> bool:
+    """Whether a reduction with these options folds exactly the last axis -- of a vector, its only one, also when
+    no axis is named (the softmax of a vector: exp(t) / sum(exp(t)))."""
+    axes = opts.get("axes")
+    return (rank == 1 and axes is None) or list(axes or []) == [rank - 1]
 
 
 class _RowCluster:
@@ -955,6 +962,7 @@ class _RowCluster:
 
     reduce = None
     how = {"mode": "compiled"}
+    split_rows = False
 
     def __init__(self, steps, inputs, program, layout, n_stages):
         self.steps, self.inputs, self.program, self.layout, self.n_stages = steps, inputs, program, layout, n_stages
@@ -962,12 +970,15 @@ class _RowCluster:
 
     def run(self, run: "_Run", out: Tensor, values: List[Tensor]):
         fused = getattr(run.pick(values), "fused_elementwise", None)
-        if fused is not None:
+        if fused is not None and not self.split_rows:
             try:
                 return fused(out, self.program, values, self.layout, **self.how)
             except Exception as e:
                 if getattr(e, "status", None) != _EUNSUPPORTED:
                     raise
+                # a refusal that the shape alone decides (a few very long rows, which the reductions cut into
+                # segments) holds for every later call: the steps run at once from then on
+                self.split_rows = "the reduction would split" in str(e)
         known = {t.data.id: v for t, v in zip(self.inputs, values)}
         for node in self.steps:
             e = node.data
@@ -1017,7 +1028,7 @@ def _cluster_rows(roots: List[Tensor]) -> int:
             return tuple(d.args[0].root.shape)
         if d.op in _REDUCE_CODES and isinstance(d.args[0], Tensor):
             x, opts = d.args[0], d.args[1]
-            if x.type in _NARROW and _const(x) is None and list(opts.get("axes") or []) == [len(x.shape) - 1]:
+            if x.type in _NARROW and _const(x) is None and _over_last_axis(opts, len(x.shape)):
                 return tuple(x.shape)
         return None
 

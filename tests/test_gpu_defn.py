@@ -439,7 +439,8 @@ def test_compiled_reduction_takes_any_float_program(hip):
 
 
 @pytest.mark.parametrize("name", sorted(REDUCED))
-@pytest.mark.parametrize("shape", [(64, 256), (300, 4096), (16, 8192), (5, 40000), (4, 65536), (2049, 8), (3, 7, 512)])
+@pytest.mark.parametrize("shape", [(64, 256), (300, 4096), (16, 8192), (5, 40000), (4, 65536), (1, 1000000), (2, 131080), (2049, 8),
+                                   (3, 7, 512)])
 def test_group_with_its_row_reduction_is_bit_identical(name, shape, hip, fused_mode):
     rng = np.random.default_rng(seed_of(name, shape))
     if len(shape) == 3 and name == "sum_of_exp":
@@ -777,6 +778,37 @@ def test_rows_that_the_reduction_would_split_run_stage_by_stage(hip):
     x = rand_float(np.random.default_rng(6), "f32", (4, 65536), hip)   # few rows, very long: the separate sum works in segments
     planned = defn.compile(softmax_rows, x, fuse="compiled")
     assert_bits_equal(planned(x), defn.compile(softmax_rows, x)(x), "split rows")
+
+
+def test_a_few_very_long_rows_keep_their_reduction_in_the_group(hip):
+    """exp(t) / sum(exp(t)) over a million values (exla/bench/softmax.exs:1-41): the sum is cut into segments as the
+    separate reduction cuts it, so the group that feeds it still holds it -- one call, the same bits -- and the
+    refusal of the stage program, which the shape alone decides, is asked for once."""
+    from nx_amd.backend import fused_mode as set_mode
+    t = rand_float(np.random.default_rng(1000000), "f32", (1000000,), hip)
+
+    def softmax(n):
+        return Nx.divide(Nx.exp(n), Nx.sum(Nx.exp(n)))
+    want = defn.compile(softmax, t)(t)
+    planned = defn.compile(softmax, t, fuse="compiled")
+    calls = []
+    original = hip.fused_elementwise.__func__
+
+    def counting(cls, *a, **k):
+        calls.append(a[4] if len(a) > 4 else k.get("reduce_op", -1))
+        return original(cls, *a, **k)
+    hip.fused_elementwise = classmethod(counting)
+    try:
+        set_mode("compiled")
+        assert_bits_equal(planned(t), want, "first call")
+        first = list(calls)
+        del calls[:]
+        assert_bits_equal(planned(t), want, "second call")
+        assert calls == [0, -1], calls            # the sum inside its group, then the quotient
+        assert first in ([-1, 0, -1], [0, -1])    # (with the stage program offered and refused once, where one was planned)
+    finally:
+        set_mode("interpreted")
+        hip.fused_elementwise = classmethod(original)
 
 
 def test_configuration_3_softmax_in_one_kernel(hip):
