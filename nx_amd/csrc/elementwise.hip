@@ -426,7 +426,9 @@ static void launch_bvec_fix(const hipnx_ctx *ctx, const BinArgs &a_) {
   hipLaunchKernelGGL((binary_rows_kernel<OP, CT, UNS, FIX, FIXO, LM, RM, U>),                                         \
                      dim3((unsigned)((a.nvec + BLOCK * U - 1) / (BLOCK * U))), dim3(BLOCK), 0, ctx->stream, a.l, a.r, \
                      a.out, nvec, vpr, fdr, l0, r0)
-      const int how = lm * 3 + rm;
+      // (two streams in and one out, each beyond 128 MiB: the general kernel is as fast, and with the three buffers
+      // half a GiB apart this one lost 7 % -- bf16 x + y of 2^28 elements 260 against 279 us)
+      const int how = lm == 2 && rm == 2 && a.nvec > (1 << 23) ? -1 : lm * 3 + rm;
       if (how == 8 && a.nvec >= (1 << 16) && a.nvec <= (1 << 22)) HIPNX_ROWS(2, 2, 2);  // (1 to 64 MiB a side)
       else if (how == 8) HIPNX_ROWS(2, 2, 1);
       else if (how == 7) HIPNX_ROWS(2, 1, 1);
