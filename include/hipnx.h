@@ -368,7 +368,9 @@ int hipnx_threefry2x32(hipnx_ctx *ctx, const hipnx_buf *key, int64_t n, hipnx_bu
  * kernel (HIPNX_FUSED_COMPILED) takes any cols: its last vector is partial.
  * reduce_op: -1, or HIPNX_RED_SUM / MAX / MIN to reduce the result along its rows without storing it
  * (sum/4, reduce_max/4, reduce_min/4 over the last axis, nx/lib/nx/backend.ex:89-92): `out` then has
- * `rows` elements, and equals the separate reduction kernel applied to the stored result. */
+ * `rows` elements, and equals the separate reduction kernel applied to the stored result (a few very long rows are
+ * cut into segments by that kernel's own rule, their partial results kept in pool workspace and folded by its
+ * second kernel: the same order of additions). */
 enum { HIPNX_FUSED_SET = 0, HIPNX_FUSED_UNARY, HIPNX_FUSED_BINARY, HIPNX_FUSED_SELECT, HIPNX_FUSED_AS_TYPE,
        HIPNX_FUSED_BITCAST, HIPNX_FUSED_ROW_REDUCE, HIPNX_FUSED_ROW_STAT };
 /* flags bit 1: the instruction works on 32-bit integers (dt u32 / s32) kept as raw bits -- a SET loads the
@@ -392,7 +394,8 @@ enum { HIPNX_FUSED_SRC_CONST = 0, HIPNX_FUSED_SRC_INPUT, HIPNX_FUSED_SRC_SAVED, 
  * (HIPNX_FUSED_FLAG_RESULT) ends the program instead: that one value per row is the result (`out` has
  * `rows` elements) -- a log-sum-exp is two such stages.  Rows of more than 4096 elements
  * take a block each, as in the separate reduction; values are carried in registers for rows of up to 32768 elements
- * (HIPNX_EUNSUPPORTED for a program that reads them over longer rows).
+ * (HIPNX_EUNSUPPORTED for a program that reads them over longer rows, and for stages over the few very long rows
+ * that the separate reduction cuts into segments: fewer than 8 rows per compute unit, 32768 elements or more each).
  * reduce_op = -1, HIPNX_FUSED_COMPILED only (HIPNX_EUNSUPPORTED otherwise). */
 enum { HIPNX_FUSED_SAVED = 3, HIPNX_FUSED_MAX_INSTR = 32, HIPNX_FUSED_MAX_INPUTS = 8, HIPNX_FUSED_STATS = 3 };
 typedef struct {
