@@ -73,6 +73,8 @@ class _Ref:
     """Owns one device buffer.  Metadata-only callbacks (reshape / squeeze / bitcast) share it;
     it is deallocated when the last sharer is, or by the garbage collector."""
 
+    __slots__ = ("ctx", "handle", "nbytes", "sharers", "keep")
+
     def __init__(self, ctx, nbytes: int, address=None, keep=None, ipc_handle=None):
         self.ctx = ctx
         self.handle = C.c_void_p()
@@ -87,17 +89,38 @@ class _Ref:
         else:  # someone else's device memory: the handle never frees it
             L.check(L.lib.hipnx_buf_wrap(ctx, C.c_void_p(address), nbytes, C.byref(self.handle)))
 
-    def __del__(self):
-        if getattr(self, "handle", None) and self.handle.value:
+    def __del__(self, _destroy=L.lib.hipnx_buf_destroy):
+        try:
+            handle = self.handle
+        except AttributeError:  # the constructor raised before it had one
+            return
+        if handle is not None and handle.value:
             try:
-                L.lib.hipnx_buf_destroy(self.handle)
+                _destroy(handle)
             except Exception:  # interpreter shutdown
                 pass
             self.handle = None
 
 
+def _fresh_ref(ctx, nbytes: int, _new=object.__new__, _alloc=L.lib.hipnx_buf_alloc, _byref=C.byref, _handle=C.c_void_p) -> _Ref:
+    """A buffer of the pool for a callback's result: `_Ref(ctx, nbytes)` without the argument handling of the
+    general constructor (every callback allocates one)."""
+    ref = _new(_Ref)
+    ref.ctx = ctx
+    ref.handle = handle = _handle()
+    ref.nbytes = nbytes
+    ref.sharers = 1
+    ref.keep = None
+    status = _alloc(ctx, nbytes, _byref(handle))
+    if status:
+        L.check(status)
+    return ref
+
+
 class HipNxBackend:
     """Backend struct: `%HipNx.Backend{ref, device}`."""
+
+    __slots__ = ("ref", "device", "released")
 
     def __init__(self, ref: _Ref, device: int):
         self.ref = ref
@@ -125,7 +148,7 @@ class HipNxBackend:
     @classmethod
     def _alloc(cls, out: Tensor, device: int) -> Tensor:
         nbytes = out.size * T.size_bytes(out.type)
-        return out.with_(data=cls(_Ref(cls._ctx(device), nbytes), device))
+        return out.with_(data=cls(_fresh_ref(_Context.get(device), nbytes), device))
 
     @classmethod
     def _narrow(cls, res: Tensor) -> Tensor:
@@ -213,6 +236,7 @@ class HipNxBackend:
         return arr
 
     _scalar_cache = {}  # (device, type, encoded element) -> _Ref of a rank-0 constant
+    _scalar_refs = {}   # (device, type, number, its class) -> the same _Ref, found without encoding the number
 
     @classmethod
     def constant(cls, out: Tensor, number, opts=None) -> Tensor:
@@ -220,6 +244,16 @@ class HipNxBackend:
         `Nx.multiply(t, 0.5)` turns its number into -- are kept per device and shared: tensors are
         immutable, and the cache holds its own share of the buffer, so deallocating one user
         never frees it."""
+        if out.shape == () and number.__class__ in (int, float) and (not opts or (len(opts) == 1 and "device" in opts)):
+            # the number met before, on this device, in this type: its buffer at once
+            device = opts["device"] if opts else 0
+            memo = (device, out.type, number.hex() if number.__class__ is float else number, number.__class__)
+            ref = cls._scalar_refs.get(memo)
+            if ref is not None and device not in _capturing:
+                ref.sharers += 1
+                return out.with_(data=HipNxBackend(ref, device))
+        else:
+            memo = None
         opts = cls.init(opts)
         if T.is_sub_byte(out.type):
             number_to_binary(number, out.type)  # the reference's argument checks
@@ -252,9 +286,14 @@ class HipNxBackend:
             if ref is None:
                 if len(cls._scalar_cache) >= 1024:
                     cls._scalar_cache.clear()
+                    cls._scalar_refs.clear()
                 res = cls._alloc(out, opts["device"])
                 L.check(L.lib.hipnx_fill(res.data.ref.ctx, res.data.ref.handle, len(elem), elem, 1))
                 ref = cls._scalar_cache[key] = res.data.ref
+            if memo is not None:
+                if len(cls._scalar_refs) >= 4096:
+                    cls._scalar_refs.clear()
+                cls._scalar_refs[memo] = ref
             ref.sharers += 1
             return out.with_(data=cls(ref, opts["device"]))
         res = cls._alloc(out, opts["device"])
@@ -335,20 +374,48 @@ class HipNxBackend:
     # ---- element-wise ----------------------------------------------------------------------
     @classmethod
     def _binary(cls, op: int, out: Tensor, l: Tensor, r: Tensor) -> Tensor:
-        dev = cls._device_of(l, r)
-        l, r = cls._from_nx(l, dev), cls._from_nx(r, dev)
-        res = cls._alloc(out, dev)
-        shape = out.shape
-        status = L.lib.hipnx_binary(
-            res.data.ref.ctx, op, T.code(l.type), T.code(r.type), T.code(out.type), len(shape), L.i64_array(shape),
-            L.broadcast_stride_array(l.shape, shape), L.broadcast_stride_array(r.shape, shape),
-            cls._handle(l), cls._handle(r), res.data.ref.handle)
+        ld, rd = l.data, r.data
+        if ld.__class__ is HipNxBackend and rd.__class__ is HipNxBackend:
+            dev = ld.device
+        else:
+            dev = cls._device_of(l, r)
+            l, r = cls._from_nx(l, dev), cls._from_nx(r, dev)
+            ld, rd = l.data, r.data
+        if ld.released or rd.released:
+            raise L.HipNxError(L.EFREED, "tensor has been deallocated")
+        # what the call needs of types and shapes repeats from call to call: worked out once per signature
+        key = (l.type, l.shape, r.type, r.shape, out.type, out.shape)
+        plan = _binary_plans.get(key)
+        if plan is None:
+            if len(_binary_plans) > 4096:
+                _binary_plans.clear()
+            shape = out.shape
+            plan = _binary_plans[key] = (T.code(l.type), T.code(r.type), T.code(out.type), len(shape), L.i64_array(shape),
+                                         L.broadcast_stride_array(l.shape, shape), L.broadcast_stride_array(r.shape, shape),
+                                         out.size * T.size_bytes(out.type), out.type[1] < 8)
+        lc, rc, oc, rank, dims, ls, rs, nbytes, narrow = plan
+        ctx = _Context.get(dev)
+        ref = _fresh_ref(ctx, nbytes)
+        res = out.with_(data=HipNxBackend(ref, dev))
+        status = L.lib.hipnx_binary(ctx, op, lc, rc, oc, rank, dims, ls, rs, ld.ref.handle, rd.ref.handle, ref.handle)
         if status:
             L.check(status)
-        return cls._narrow(res) if out.type[1] < 8 else res
+        return cls._narrow(res) if narrow else res
 
     @classmethod
     def _unary(cls, op: int, out: Tensor, t: Tensor) -> Tensor:
+        td = t.data
+        if td.__class__ is HipNxBackend and t.type[1] >= 8 and out.type[1] >= 8:  # the usual call, without the detours below
+            if td.released:
+                raise L.HipNxError(L.EFREED, "tensor has been deallocated")
+            dev = td.device
+            ctx = _Context.get(dev)
+            n = out.size
+            ref = _fresh_ref(ctx, n * T.size_bytes(out.type))
+            status = L.lib.hipnx_unary(ctx, op, T.code(t.type), T.code(out.type), n, td.ref.handle, ref.handle)
+            if status:
+                L.check(status)
+            return out.with_(data=HipNxBackend(ref, dev))
         dev = cls._device_of(t)
         t = cls._from_nx(t, dev)
         if t.type[1] < 8 and op in _BIT_COUNTS:
@@ -406,9 +473,33 @@ class HipNxBackend:
 
     @classmethod
     def _reduce(cls, op: int, out: Tensor, t: Tensor, opts) -> Tensor:
+        axes = opts.get("axes")
+        td = t.data
+        if td.__class__ is HipNxBackend:
+            # the usual call -- one run of neighbouring axes (or all of them) of a tensor that is here -- by its
+            # signature: the view [outer, red, inner], the type codes and the result's size are worked out once
+            key = (t.type, t.shape, out.type, None if axes is None else tuple(axes))
+            plan = _reduce_plans.get(key)
+            if plan is None and t.type[1] >= 8 and out.type[1] >= 8:
+                run = None if axes is None else sorted(a % len(t.shape) for a in axes)
+                if run is None or (run and run == list(range(run[0], run[-1] + 1))):
+                    _, outer, red, inner = cls._view_for_axes(t, run)
+                    if len(_reduce_plans) > 4096:
+                        _reduce_plans.clear()
+                    plan = _reduce_plans[key] = (T.code(t.type), T.code(out.type), outer, red, inner, out.size * T.size_bytes(out.type))
+            if plan is not None:
+                if td.released:
+                    raise L.HipNxError(L.EFREED, "tensor has been deallocated")
+                ic, oc, outer, red, inner, nbytes = plan
+                dev = td.device
+                ctx = _Context.get(dev)
+                ref = _fresh_ref(ctx, nbytes)
+                status = L.lib.hipnx_reduce(ctx, op, ic, oc, outer, red, inner, td.ref.handle, ref.handle)
+                if status:
+                    L.check(status)
+                return out.with_(data=HipNxBackend(ref, dev))
         dev = cls._device_of(t)
         t = cls._from_nx(t, dev)
-        axes = opts.get("axes")
         if axes is not None and len(axes) > 1 and t.type[1] >= 8:
             axes = sorted(a % len(t.shape) for a in axes)
             runs = [[a] for a in axes[:1]]
@@ -1135,6 +1226,8 @@ def _advise_huge_pages(address: int, n: int) -> None:
         lo, hi = (address + huge - 1) & ~(huge - 1), (address + n) & ~(huge - 1)
         if hi > lo:
             _libc.madvise(C.c_void_p(lo), hi - lo, 14)  # MADV_HUGEPAGE
+_reduce_plans = {}  # (types, shape and axes of a reduction callback) -> its type codes, [outer, red, inner] view, result bytes
+_binary_plans = {}  # (types and shapes of a binary callback) -> its type codes, shape and stride arrays, result bytes
 _fused_modes = {}  # device -> the mode chosen with fused_mode/2: what a call that names none runs in
 _fused_set = {}    # device -> the mode the library is in at this moment (a call that names one leaves it there)
 _fused_arrays = {}  # (id of a layout, input types) -> (the layout itself, so the id stays its own; C arrays of types and strides)

@@ -120,6 +120,12 @@ def byte_size(t: Tensor) -> int:
 
 def to_tensor(value) -> Tensor:
     """Nx.to_tensor/1 (nx.ex:2149-2157): numbers become rank-0 constants on the default backend."""
+    c = value.__class__
+    if c is Tensor:
+        return value
+    if c is float or c is int:  # (the number of `multiply(t, 0.5)`: the common case, without the checks below)
+        mod, opts = getattr(_state, "backend", None) or _global_default[0]
+        return mod.constant(_F32_SCALAR if c is float else _S32_SCALAR, value, opts)
     if isinstance(value, Tensor):
         return value
     if isinstance(value, (bool, int, float, np.integer, np.floating)):
@@ -127,6 +133,9 @@ def to_tensor(value) -> Tensor:
         v = value.item() if isinstance(value, np.generic) else value
         return mod.constant(template(T.infer(v), ()), v, opts)
     return tensor(value)
+
+
+_F32_SCALAR, _S32_SCALAR = template(("f", 32), ()), template(("s", 32), ())  # what Nx.Type.infer/1 gives a float / an integer
 
 
 def to_binary(t: Tensor, limit=None) -> bytes:
@@ -208,8 +217,10 @@ def _binary(name, left, right, out_type_fun):
     else:
         ty = T.binary_type(_number_or_type(left), _number_or_type(right))
         l, r = to_tensor(left), to_tensor(right)
-    out = template(out_type_fun(ty), l.shape if l.shape == r.shape else S.binary_broadcast(l.shape, r.shape))
-    return getattr(_impl(l, r), name)(out, l, r)
+    ls, rs = l.shape, r.shape
+    out = template(out_type_fun(ty), ls if ls == rs or rs == () else rs if ls == () else S.binary_broadcast(ls, rs))
+    lb, rb = l.data.__class__, r.data.__class__
+    return getattr(lb if lb is rb else _impl(l, r), name)(out, l, r)
 
 
 def _def_binary():
@@ -283,16 +294,32 @@ def as_type(t, type) -> Tensor:
 def _aggregate(t, op, out_type, axes=None, keep_axes=False):
     """aggregate_axes_op/4 (nx.ex:10594-10649)."""
     t = to_tensor(t)
-    if axes is not None:
-        axes = S.normalize_axes(t.shape, axes)
-        shape_ = S.contract(t.shape, axes, keep_axes)
-    elif keep_axes:
-        shape_, axes = (1,) * len(t.shape), list(range(len(t.shape)))
-    else:
-        shape_ = ()
+    # the axes and the result's shape depend on the shape and the options only: worked out once per signature
+    try:
+        key = (t.shape, axes if axes is None else tuple(axes), keep_axes)
+        known = _aggregate_shapes.get(key)
+    except TypeError:  # axes that are no list of integers: the checks below say so
+        key = known = None
+    if known is None:
+        if axes is not None:
+            axes = S.normalize_axes(t.shape, axes)
+            shape_ = S.contract(t.shape, axes, keep_axes)
+        elif keep_axes:
+            shape_, axes = (1,) * len(t.shape), list(range(len(t.shape)))
+        else:
+            shape_ = ()
+        known = (axes, shape_)
+        if key is not None:
+            if len(_aggregate_shapes) > 4096:
+                _aggregate_shapes.clear()
+            _aggregate_shapes[key] = known
+    axes, shape_ = known
     if axes == []:
         return as_type(t, out_type)
-    return getattr(_impl(t), op)(template(out_type, shape_), t, {"axes": axes, "keep_axes": keep_axes})
+    return getattr(t.data.__class__, op)(template(out_type, shape_), t, {"axes": None if axes is None else list(axes), "keep_axes": keep_axes})
+
+
+_aggregate_shapes = {}  # (shape, axes, keep_axes) -> (normalised axes, shape of the result)
 
 
 def sum(t, axes=None, keep_axes=False):  # noqa: A001 - Nx.sum/2 (nx.ex:9622-9626)
