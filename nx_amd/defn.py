@@ -1329,12 +1329,27 @@ class _Scope:
         self.results: Dict[Any, Any] = {}
 
 
+# nodes that `apply` does not evaluate as a callback on its evaluated operands
+_EVALUATED_APART = frozenset(["parameter", "elem", "while", "cond", "fused", "dot_scaled", "block"]) | frozenset(CREATION_OPS)
+
+
 class _Run:
     def __init__(self, plans, backend):
         self.plans, self.backend = plans, backend
 
     def eval(self, x, scope: _Scope):  # noqa: A003
-        e = _expr_of(x)
+        e = x.data if x.__class__ is Tensor else _expr_of(x)
+        counts = scope.counts if scope is not None else ()  # (no scope: a group's constant, evaluated by the group itself)
+        if e.id in counts and e.op not in ("tensor", "constant"):  # the usual node: one of this scope's own
+            results = scope.results
+            if e.id in results:
+                res = results[e.id]
+            else:
+                res = results[e.id] = self.apply(e, x, scope)
+            left = counts[e.id] = counts[e.id] - 1
+            if left == 0:
+                results.pop(e.id, None)
+            return res
         if e.op == "tensor":
             t = e.args[0]
             mod, opts = self.backend
@@ -1373,6 +1388,26 @@ class _Run:
         op = e.op
         if op == "parameter":
             return scope.params[e.args[0]]
+        if op not in _EVALUATED_APART:
+            # a callback on tensors and options (nearly every node): its operands, then the backend they are on
+            args, mod = [], None
+            for a in e.args:
+                if a.__class__ is Tensor:
+                    a = self.eval(a, scope)
+                    b = a.data.__class__
+                    if mod is None:
+                        mod = b
+                    elif mod is not b:
+                        mod = False  # operands on different backends: the general rule decides
+                elif a.__class__ is list and any(isinstance(v, Tensor) for v in a):
+                    mod = False
+                    a = [self.eval(v, scope) if isinstance(v, Tensor) else v for v in a]
+                args.append(a)
+            if not mod or mod is HostBinary:
+                mod = self.pick([a for a in args if isinstance(a, Tensor)]) if op not in LIST_OPS and op not in INDICES_OPS else None
+                if mod is None:
+                    mod = self.pick(args[0]) if op in LIST_OPS else self.pick([args[0]] + [i for i in args[1] if isinstance(i, Tensor)])
+            return getattr(mod, op)(x.with_(data=None), *args)
         if op == "elem":
             return self.eval(e.args[0], scope)[e.args[1]]
         if op == "while":
