@@ -1004,7 +1004,8 @@ class HipNxBackend:
         wanted = mode if mode is not None else _fused_modes.get(dev, "interpreted")
         if _fused_set.get(dev, "interpreted") != wanted:
             _set_fused_mode(wanted, dev)
-        inputs = [cls._from_nx(t, dev) for t in inputs]
+        if not all(t.data.__class__ is HipNxBackend for t in inputs):
+            inputs = [cls._from_nx(t, dev) for t in inputs]
         rows, cols, strides = layout
         prog = getattr(program, "packed", None)
         if prog is None:
@@ -1019,20 +1020,43 @@ class HipNxBackend:
                 program.packed = prog  # a caller's list type with room for the packed form keeps it
             except AttributeError:
                 pass
-        res = cls._alloc(out, dev)
         n = max(len(inputs), 1)
-        handles = (C.c_void_p * n)(*[cls._handle(t) for t in inputs])
         # types and strides repeat from call to call of a traced function: kept with the layout they belong to
-        key = (id(layout), tuple(t.type for t in inputs))
+        if getattr(program, "packed", None) is not prog:  # a plain list: its packed form lives for this call only
+            return cls._fused_call(out, prog, len(program), inputs, layout, reduce_op, dev)
+        key = (id(layout), id(prog), out.type, out.shape, *[t.type for t in inputs])
         cached = _fused_arrays.get(key)
-        if cached is None or cached[0] is not layout:
+        if cached is None or cached[0] is not layout or cached[1] is not prog:
             if len(_fused_arrays) > 4096:
                 _fused_arrays.clear()
-            cached = _fused_arrays[key] = (layout, (C.c_int * n)(*[T.code(t.type) for t in inputs]),
-                                           (C.c_int64 * n)(*[s[0] for s in strides]), (C.c_int * n)(*[s[1] for s in strides]))
-        _, dts, rs, cs = cached
-        L.check(L.lib.hipnx_fused_elementwise(res.data.ref.ctx, len(program), C.cast(prog, C.c_void_p), len(inputs), handles,
-                                              dts, rs, cs, rows, cols, reduce_op, T.code(out.type), res.data.ref.handle))
+            cached = _fused_arrays[key] = (layout, prog, (C.c_int * n)(*[T.code(t.type) for t in inputs]),
+                                           (C.c_int64 * n)(*[s[0] for s in strides]), (C.c_int * n)(*[s[1] for s in strides]),
+                                           C.cast(prog, C.c_void_p), (C.c_void_p * n), T.code(out.type),
+                                           out.size * T.size_bytes(out.type))
+        _, _, dts, rs, cs, prog_ptr, handle_array, out_code, nbytes = cached
+        for t in inputs:
+            if t.data.released:
+                raise L.HipNxError(L.EFREED, "tensor has been deallocated")
+        handles = handle_array(*[t.data.ref.handle.value for t in inputs])
+        ctx = _Context.get(dev)
+        ref = _fresh_ref(ctx, nbytes)
+        status = L.lib.hipnx_fused_elementwise(ctx, len(program), prog_ptr, len(inputs), handles, dts, rs, cs, rows, cols,
+                                               reduce_op, out_code, ref.handle)
+        if status:
+            L.check(status)
+        return out.with_(data=HipNxBackend(ref, dev))
+
+    @classmethod
+    def _fused_call(cls, out, prog, n_instr, inputs, layout, reduce_op, dev) -> Tensor:
+        """fused_elementwise for a program whose packed form nobody keeps: every argument array made for this call."""
+        rows, cols, strides = layout
+        n = max(len(inputs), 1)
+        res = cls._alloc(out, dev)
+        handles = (C.c_void_p * n)(*[cls._handle(t) for t in inputs])
+        L.check(L.lib.hipnx_fused_elementwise(res.data.ref.ctx, n_instr, C.cast(prog, C.c_void_p), len(inputs), handles,
+                                              (C.c_int * n)(*[T.code(t.type) for t in inputs]), (C.c_int64 * n)(*[s[0] for s in strides]),
+                                              (C.c_int * n)(*[s[1] for s in strides]), rows, cols, reduce_op, T.code(out.type),
+                                              res.data.ref.handle))
         return res
 
     @classmethod
