@@ -311,8 +311,12 @@ extern "C" int hipnx_fused_elementwise(hipnx_ctx *ctx, int n_instr, const hipnx_
   if (n_stats && (reduce_op != -1 || cols == 0))
     return set_error(HIPNX_EUNSUPPORTED, "fused: stages take non-empty rows and no reduction of the result");
   // a few very long rows are split into segments by the separate reduction, whose order the stages follow: not here
-  if (n_stats && rows < (int64_t)ctx->num_cus * 8 && cols >= 2 * 16384)
-    return set_error(HIPNX_EUNSUPPORTED, "fused: stages over rows that the reduction would split");
+  if (n_stats) {
+    int would_be = 1;
+    int64_t of_length = cols;
+    plan_row_segments(ctx, rows, cols, &would_be, &of_length);
+    if (would_be > 1) return set_error(HIPNX_EUNSUPPORTED, "fused: stages over rows that the reduction would split");
+  }
   if (uses_carry && cols > 16 * (cols > 4096 ? 256 : 64) * 8)
     return set_error(HIPNX_EUNSUPPORTED, "fused: rows too long to keep a stage's values in registers");
   const int64_t n = rows * cols;

@@ -319,10 +319,11 @@ static void partials_release(hipnx_ctx *ctx, bool static_ws, void *ws, size_t ws
 // must add in the same order (the reduction fused into an element-wise group follows it).
 static inline void plan_row_segments(const hipnx_ctx *ctx, int64_t rows, int64_t red, int *nseg, int64_t *seg_len) {
   const int64_t target_units = (int64_t)ctx->num_cus * 8;  // units of parallel work wanted
-  const int64_t min_seg = 16384;                           // elements per segment worth a block
+  const int64_t min_row = 32768;                           // a row shorter than this stays whole: the second kernel costs more
+  const int64_t min_seg = 4096;                            // elements per segment worth a block (sixteen per lane)
   *nseg = 1;
   *seg_len = red;
-  if (rows < target_units && red >= 2 * min_seg) {
+  if (rows < target_units && red >= min_row) {
     const int64_t want = target_units / (rows > 0 ? rows : 1), maxs = red / min_seg;
     int n = (int)(want < maxs ? want : maxs);
     if (n > 1024) n = 1024;
