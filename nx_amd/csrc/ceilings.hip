@@ -12,6 +12,12 @@
 //   hipnx_ceilings stream <read|write|copy> [MiB] [ms]
 //       16-byte-per-lane streaming kernels over a buffer larger than the 256 MB last-level cache, the best of
 //       1, 2, 4 and 8 accesses in flight per lane
+//   hipnx_ceilings ingest <l2|llc|hbm> [ms]
+//       what a compute unit takes in: 256 work-groups of 8 waves, one per CU, each pulling 4 MiB into LDS with
+//       direct-to-LDS loads of 16 bytes per lane (the contraction kernels' way; 4, 8 and 16 KiB in flight per wave,
+//       the best reported), from a region its XCD's L2 holds (`l2`: the work-groups of an XCD share 2 MiB), from
+//       the last-level cache (`llc`: 512 KiB per work-group, 128 MiB in all) or from HBM (`hbm`: 4 MiB per
+//       work-group, 1 GiB in all); bytes per clock of the shader clock measured in the last launch
 //
 // Each run prints one JSON line.  Built by the Makefile into nx_amd/lib/hipnx_ceilings; bench.py runs
 // it when present and copies the sustained figures into its `measured_ceiling` fields.
@@ -88,6 +94,40 @@ __global__ void __launch_bounds__(512) mfma_loop(const v4i *src, float *out, int
   }
   out[blockIdx.x * 512 + tid] = sum;
   if (blockIdx.x == 8 && tid == 0) {
+    g_clk[0] = clock64() - c0;
+    g_clk[1] = wall_clock64() - w0;
+  }
+}
+
+// One direct-to-LDS load as the contraction kernels issue it: every lane moves 16 bytes from its global address to
+// LDS[base + 16 * lane], the wave-uniform base carried in M0.
+typedef __attribute__((address_space(3))) void *lds_ptr_t;
+__device__ __forceinline__ void lds_dma16(const unsigned char *g, unsigned char *lds) {
+  const unsigned base = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(lds_ptr_t)lds);
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(base) : "memory", "m0");
+#pragma clang diagnostic pop
+}
+
+// A work-group pulls `bytes_per_wg` from its region into LDS, DEPTH KiB in flight per wave.  Consecutive work-group
+// ids go to different XCDs, so the groups with equal id % 8 share the regions of one XCD.
+template <int DEPTH>
+__global__ void __launch_bounds__(512) ingest_loop(const unsigned char *src, size_t region_bytes, int regions, size_t bytes_per_wg, unsigned *sink) {
+  extern __shared__ unsigned char ingest_lds[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int xcd = blockIdx.x % 8, within = blockIdx.x / 8, per_xcd = regions / 8;
+  const unsigned char *base = src + (size_t)(xcd * per_xcd + within % per_xcd) * region_bytes;
+  const size_t per_step = 8 * 1024, steps = bytes_per_wg / per_step;  // the 8 waves move 8 KiB per step
+  unsigned char *mine = ingest_lds + wave * DEPTH * 1024;
+  const unsigned long long c0 = clock64(), w0 = wall_clock64();
+  for (size_t s = 0; s < steps; s += DEPTH) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++) lds_dma16(base + ((s + d) * per_step + wave * 1024 + lane * 16) % region_bytes, mine + d * 1024);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  }
+  if (((unsigned *)mine)[lane] == 0x12345678u) sink[0] = 1;  // (keeps the loads alive)
+  if (blockIdx.x == 8 && threadIdx.x == 0) {
     g_clk[0] = clock64() - c0;
     g_clk[1] = wall_clock64() - w0;
   }
@@ -260,9 +300,56 @@ static int run_stream(const char *mode, size_t mib, double want_ms) {
   return 0;
 }
 
+static int run_ingest(const char *from, double want_ms) {
+  const int level = !strcmp(from, "l2") ? 0 : !strcmp(from, "llc") ? 1 : !strcmp(from, "hbm") ? 2 : -1;
+  if (level < 0) { fprintf(stderr, "unknown source %s\n", from); return 2; }
+  const size_t region = level == 0 ? (2u << 20) : level == 1 ? (512u << 10) : (4u << 20), per_wg = 4u << 20;
+  const int regions = level == 0 ? 8 : 256;
+  unsigned char *src;
+  unsigned *sink;
+  CK(hipMalloc(&src, region * regions));
+  CK(hipMalloc(&sink, 4));
+  CK(hipMemset(src, 1, region * regions));
+  double best = 0, best_us = 0, best_clk = 0;
+  int best_depth = 0;
+  for (int depth : {4, 8, 16}) {
+    const int lds = 8 * depth * 1024;
+    auto launch = [&] {
+      if (depth == 4) hipLaunchKernelGGL(ingest_loop<4>, dim3(256), dim3(512), lds, 0, src, region, regions, per_wg, sink);
+      else if (depth == 8) hipLaunchKernelGGL(ingest_loop<8>, dim3(256), dim3(512), lds, 0, src, region, regions, per_wg, sink);
+      else hipLaunchKernelGGL(ingest_loop<16>, dim3(256), dim3(512), lds, 0, src, region, regions, per_wg, sink);
+    };
+    if (depth == 16) CK(hipFuncSetAttribute((const void *)ingest_loop<16>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    std::vector<float> probe;
+    if (timed_chunks(launch, 1, 3, probe)) return 1;
+    const double launch_ms = probe[0] / 3;
+    const int per_chunk = std::max(1, (int)(2.0 / launch_ms));
+    const int chunks = std::max(5, (int)(want_ms / 3 / (per_chunk * launch_ms)));
+    std::vector<float> ms;
+    if (timed_chunks(launch, chunks, per_chunk, ms)) return 1;
+    unsigned long long c[2];
+    CK(hipMemcpyFromSymbol(c, HIP_SYMBOL(g_clk), sizeof(c)));
+    double t = 0;
+    for (int i = chunks * 4 / 5; i < chunks; i++) t += ms[i];
+    const double us = 1000 * t / ((chunks - chunks * 4 / 5) * per_chunk), rate = 256.0 * per_wg / us / 1e3;  // GB/s
+    if (rate > best) {
+      best = rate;
+      best_us = us;
+      best_clk = c[0] / (c[1] / 100.0);
+      best_depth = depth;
+    }
+  }
+  printf("{\"kind\": \"ingest\", \"from\": \"%s\", \"unit\": \"GB/s\", \"sustained\": %.0f, \"per_cu\": %.1f, \"bytes_per_clock_per_cu\": %.1f, "
+         "\"clock_mhz_last_launch\": %.0f, \"launch_us\": %.1f, \"KiB_in_flight_per_wave\": %d}\n",
+         from, best, best / 256, best / 256 * 1e3 / best_clk, best_clk, best_us, best_depth);
+  return 0;
+}
+
 int main(int argc, char **argv) {
+  if (argc >= 3 && !strcmp(argv[1], "ingest")) return run_ingest(argv[2], argc > 3 ? atof(argv[3]) : 100.0);
   if (argc >= 4 && !strcmp(argv[1], "mfma")) return run_mfma(argv[2], argv[3], argc > 4 ? atof(argv[4]) : 300.0);
   if (argc >= 3 && !strcmp(argv[1], "stream")) return run_stream(argv[2], argc > 3 ? (size_t)atol(argv[3]) : 2048, argc > 4 ? atof(argv[4]) : 100.0);
-  fprintf(stderr, "usage: hipnx_ceilings mfma <bf16|f16|s8|f32> <random|normal|zero> [ms]\n       hipnx_ceilings stream <read|write|copy> [MiB] [ms]\n");
+  fprintf(stderr, "usage: hipnx_ceilings mfma <bf16|f16|s8|f32> <random|normal|zero> [ms]\n       hipnx_ceilings stream <read|write|copy> [MiB] [ms]\n"
+                  "       hipnx_ceilings ingest <l2|llc|hbm> [ms]\n");
   return 2;
 }
