@@ -118,12 +118,14 @@ __global__ void __launch_bounds__(512) ingest_loop(const unsigned char *src, siz
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int xcd = blockIdx.x % 8, within = blockIdx.x / 8, per_xcd = regions / 8;
   const unsigned char *base = src + (size_t)(xcd * per_xcd + within % per_xcd) * region_bytes;
-  const size_t per_step = 8 * 1024, steps = bytes_per_wg / per_step;  // the 8 waves move 8 KiB per step
+  const unsigned per_step = 8 * 1024, steps = (unsigned)(bytes_per_wg / per_step);  // the 8 waves move 8 KiB per step
+  const unsigned mask = (unsigned)region_bytes - 1, mine_at = wave * 1024 + lane * 16;  // (regions are powers of two: a 64-bit
+  // remainder per load costs a lane more instructions than the load and halves the rate measured)
   unsigned char *mine = ingest_lds + wave * DEPTH * 1024;
   const unsigned long long c0 = clock64(), w0 = wall_clock64();
-  for (size_t s = 0; s < steps; s += DEPTH) {
+  for (unsigned s = 0; s < steps; s += DEPTH) {
 #pragma unroll
-    for (int d = 0; d < DEPTH; d++) lds_dma16(base + ((s + d) * per_step + wave * 1024 + lane * 16) % region_bytes, mine + d * 1024);
+    for (int d = 0; d < DEPTH; d++) lds_dma16(base + (((s + d) * per_step + mine_at) & mask), mine + d * 1024);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   }
   if (((unsigned *)mine)[lane] == 0x12345678u) sink[0] = 1;  // (keeps the loads alive)
