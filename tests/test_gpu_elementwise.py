@@ -118,6 +118,18 @@ def test_broadcasting_shapes(ls, rs, ty, hip, oracle):
         assert_bits_equal(getattr(Nx, op)(ha, hb), getattr(Nx, op)(oa, ob), f"{op} {ls} {rs} {ty}")
 
 
+@pytest.mark.parametrize("ty,shape", [("f32", (1016, 264)), ("bf16", (2040, 264)), ("s32", (1016, 264))])
+def test_two_dense_operands_of_a_megabyte_take_two_vectors_per_lane(ty, shape, hip, oracle):
+    """From 65536 vectors on, x + y of two dense tensors gives a lane two vectors, 256 apart: the last work-group
+    here is partly filled, some of its lanes with a first vector and no second."""
+    rng = np.random.default_rng(seed_of(ty, shape, "two vectors"))
+    a, b = rand_raw(rng, ty, shape), rand_raw(rng, ty, shape)
+    ha, oa = both(a, ty, hip, oracle)
+    hb, ob = both(b, ty, hip, oracle)
+    for op in ("add", "subtract", "multiply", "max", "less"):
+        assert_bits_equal(getattr(Nx, op)(ha, hb), getattr(Nx, op)(oa, ob), f"{op} {ty} {shape}")
+
+
 def test_scalar_number_operand(hip, oracle):
     rng = np.random.default_rng(5)
     a = rand_raw(rng, "f32", (33, 65))
