@@ -224,7 +224,10 @@ binary_vec_kernel(const void *__restrict__ l, const void *__restrict__ r, void *
 //   U vectors per lane, lanes side by side (v, v + 256, ...), every load issued before the first result is formed:
 //   two for x + y of 1 to 64 MiB a side (32 MiB: 15.3 -> 14.7 us); beyond the last-level cache one streams faster
 //   (1 GiB a side: 534 against 562 us).
-template <int OP, typename CT, bool UNS, int FIX, int FIXO, int LM, int RM, int U>
+//   NT: the tensors are far larger than the last-level cache and every access carries the non-temporal hint (a
+//   template parameter, not an argument: where a branch chooses between a hinted and a plain access the compiler
+//   merges the two and drops the hint).
+template <int OP, typename CT, bool UNS, int FIX, int FIXO, int LM, int RM, int U, bool NT = false>
 __global__ void __launch_bounds__(BLOCK)
 binary_rows_kernel(const void *__restrict__ l, const void *__restrict__ r, void *__restrict__ out, uint32_t nvec,
                    uint32_t vecs_per_row, FastDiv32 fd, int64_t ls0, int64_t rs0) {
@@ -239,13 +242,13 @@ binary_rows_kernel(const void *__restrict__ l, const void *__restrict__ r, void 
     const uint32_t v = v0 + u * BLOCK;
     if (v < nvec) {
       const uint32_t row = fastdiv(v, fd), col = (v - row * vecs_per_row) * E;
-      if constexpr (LM == 2) load_vec<CT, E>(l, FIX, (int64_t)row * ls0 + col, a[u]);
+      if constexpr (LM == 2) load_vec<CT, E, true, NT>(l, FIX, (int64_t)row * ls0 + col, a[u]);
       else {
         const CT s = LM == 0 ? l_one : load_one<CT>(l, FIX, (int64_t)row * ls0);
 #pragma unroll
         for (int i = 0; i < E; i++) a[u][i] = s;
       }
-      if constexpr (RM == 2) load_vec<CT, E>(r, FIX, (int64_t)row * rs0 + col, b[u]);
+      if constexpr (RM == 2) load_vec<CT, E, true, NT>(r, FIX, (int64_t)row * rs0 + col, b[u]);
       else {
         const CT s = RM == 0 ? r_one : load_one<CT>(r, FIX, (int64_t)row * rs0);
 #pragma unroll
@@ -260,7 +263,7 @@ binary_rows_kernel(const void *__restrict__ l, const void *__restrict__ r, void 
       CT c[E];
 #pragma unroll
       for (int i = 0; i < E; i++) c[i] = binary_apply<OP, CT, UNS>(a[u][i], b[u][i]);
-      store_vec<CT, E>(out, FIXO, (int64_t)v * E, c);
+      store_vec<CT, E, NT>(out, FIXO, (int64_t)v * E, c);
     }
   }
 }
@@ -311,7 +314,7 @@ binary_nd_kernel(const void *__restrict__ l, const void *__restrict__ r, void *_
   }
 }
 
-template <int OP, typename CT, int FIX = -1>  // FIX: the one element type of input and result, as above
+template <int OP, typename CT, int FIX = -1, bool NT = false>  // FIX: the one element type of input and result, as above; NT: as above
 __global__ void __launch_bounds__(BLOCK)
 unary_vec_kernel(const void *__restrict__ in, void *__restrict__ out, int idt_, int odt_, int bits, int64_t n) {
   const int idt = FIX >= 0 ? FIX : idt_, odt = FIX >= 0 ? FIX : odt_;
@@ -321,10 +324,10 @@ unary_vec_kernel(const void *__restrict__ in, void *__restrict__ out, int idt_, 
     int64_t o = v * E;
     if (o + E <= n) {
       CT a[E], c[E];
-      load_vec<CT, E>(in, idt, o, a);
+      load_vec<CT, E, true, NT>(in, idt, o, a);
 #pragma unroll
       for (int i = 0; i < E; i++) c[i] = unary_apply<OP, CT>(a[i], bits);
-      store_vec<CT, E>(out, odt, o, c);
+      store_vec<CT, E, NT>(out, odt, o, c);
     } else {
       for (int i = 0; o + i < n; i++)
         store_one<CT>(out, odt, o + i, unary_apply<OP, CT>(load_one<CT>(in, idt, o + i), bits));
@@ -334,7 +337,7 @@ unary_vec_kernel(const void *__restrict__ in, void *__restrict__ out, int idt_, 
 
 // as_type: CT is the decode type of the input; float -> integer goes through the wrap rule.
 // FIXI / FIXO >= 0: input and result type known when the kernel is compiled.
-template <typename CT, int FIXI = -1, int FIXO = -1>
+template <typename CT, int FIXI = -1, int FIXO = -1, bool NT = false>
 __global__ void __launch_bounds__(BLOCK)
 as_type_kernel(const void *__restrict__ in, void *__restrict__ out, int idt_, int odt_, int64_t n, int64_t tmax,
                int64_t tmin) {
@@ -346,17 +349,17 @@ as_type_kernel(const void *__restrict__ in, void *__restrict__ out, int idt_, in
     int64_t o = v * E;
     if (o + E <= n) {
       CT a[E];
-      load_vec<CT, E>(in, idt, o, a);
+      load_vec<CT, E, true, NT>(in, idt, o, a);
       if constexpr (is_fp<CT>::value) {
         if (to_int) {
           int64_t c[E];
 #pragma unroll
           for (int i = 0; i < E; i++) c[i] = float_to_int_wrap((double)a[i], tmax, tmin);
-          store_vec<int64_t, E>(out, odt, o, c);
+          store_vec<int64_t, E, NT>(out, odt, o, c);
           continue;
         }
       }
-      store_vec<CT, E>(out, odt, o, a);
+      store_vec<CT, E, NT>(out, odt, o, a);
     } else {
       for (int i = 0; o + i < n; i++) {
         CT x = load_one<CT>(in, idt, o + i);
@@ -375,6 +378,16 @@ as_type_kernel(const void *__restrict__ in, void *__restrict__ out, int idt_, in
 // ---- host side ------------------------------------------------------------------------------
 
 enum { CLS_F32 = 0, CLS_F64 = 1, CLS_I64 = 2, CLS_U64 = 3 };
+
+// Whether a launch over `n` elements moves tensors far larger than the 256 MB last-level cache (the widest of the
+// element types decides): its loads and stores then carry the non-temporal hint.  Smaller tensors are better left in
+// the cache for the callback that reads them next.
+static int streams_past_cache(int64_t n, int dt_a, int dt_b = -1, int dt_c = -1) {
+  int widest = dtype_size(dt_a);
+  if (dt_b >= 0 && dtype_size(dt_b) > widest) widest = dtype_size(dt_b);
+  if (dt_c >= 0 && dtype_size(dt_c) > widest) widest = dtype_size(dt_c);
+  return n * widest >= (256ll << 20);
+}
 
 static int grid_for(const hipnx_ctx *ctx, int64_t work_items) {
   int64_t blocks = (work_items + BLOCK - 1) / BLOCK;
@@ -395,6 +408,7 @@ struct BinArgs {
   unsigned long long *err;  // the context's deferred error word (device address of the pinned host word)
   RowAxes ax;
   int64_t flat_total;  // > 0: the FLAT modes over this many outputs (rows * cols)
+  int stream;          // the tensors are far larger than the last-level cache: loads and stores carry the non-temporal hint
 };
 
 template <int OP, typename CT, bool UNS, int FIX, int FIXO = FIX>
@@ -422,13 +436,19 @@ static void launch_bvec_fix(const hipnx_ctx *ctx, const BinArgs &a_) {
       // how each operand is met (an operand of one row has no row stride to speak of)
       const int64_t l0 = one_row ? 0 : a.ls0, r0 = one_row ? 0 : a.rs0;
       const int lm = a.ls1 ? 2 : l0 ? 1 : 0, rm = a.rs1 ? 2 : r0 ? 1 : 0;
-#define HIPNX_ROWS(LM, RM, U)                                                                                         \
-  hipLaunchKernelGGL((binary_rows_kernel<OP, CT, UNS, FIX, FIXO, LM, RM, U>),                                         \
-                     dim3((unsigned)((a.nvec + BLOCK * U - 1) / (BLOCK * U))), dim3(BLOCK), 0, ctx->stream, a.l, a.r, \
-                     a.out, nvec, vpr, fdr, l0, r0)
+#define HIPNX_ROWS(LM, RM, U)                                                                                           \
+  do {                                                                                                                  \
+    const dim3 g((unsigned)((a.nvec + BLOCK * U - 1) / (BLOCK * U)));                                                    \
+    if (U == 1 && a.stream)                                                                                             \
+      hipLaunchKernelGGL((binary_rows_kernel<OP, CT, UNS, FIX, FIXO, LM, RM, 1, true>), g, dim3(BLOCK), 0, ctx->stream, \
+                         a.l, a.r, a.out, nvec, vpr, fdr, l0, r0);                                                      \
+    else                                                                                                                \
+      hipLaunchKernelGGL((binary_rows_kernel<OP, CT, UNS, FIX, FIXO, LM, RM, U>), g, dim3(BLOCK), 0, ctx->stream, a.l,  \
+                         a.r, a.out, nvec, vpr, fdr, l0, r0);                                                           \
+  } while (0)
       // (two streams in and one out, each beyond 128 MiB: the general kernel is as fast, and with the three buffers
       // half a GiB apart this one lost 7 % -- bf16 x + y of 2^28 elements 260 against 279 us)
-      const int how = lm == 2 && rm == 2 && a.nvec > (1 << 23) ? -1 : lm * 3 + rm;
+      const int how = lm == 2 && rm == 2 && a.nvec > (1 << 23) && !a.stream ? -1 : lm * 3 + rm;
       if (how == 8 && a.nvec >= (1 << 16) && a.nvec <= (1 << 22)) HIPNX_ROWS(2, 2, 2);  // (1 to 64 MiB a side)
       else if (how == 8) HIPNX_ROWS(2, 2, 1);
       else if (how == 7) HIPNX_ROWS(2, 1, 1);
@@ -643,6 +663,7 @@ extern "C" int hipnx_binary(hipnx_ctx *ctx, int op, int l_dt, int r_dt, int out_
     }
   }
   if (vec_ok) {
+    a.stream = streams_past_cache(n, out_dt, l_dt, r_dt);
     int st = launch_bvec_op(std::make_integer_sequence<int, HIPNX_NBINARY>{}, ctx, op, cls, a);
     if (st) return st;
   } else {
@@ -678,8 +699,11 @@ namespace hipnx {
 
 template <int OP, typename CT, int FIX>
 static void launch_uvec_fix(const hipnx_ctx *ctx, const void *in, void *out, int idt, int odt, int bits, int64_t n) {
-  hipLaunchKernelGGL((unary_vec_kernel<OP, CT, FIX>), dim3(grid_for(ctx, (n + vec_elems(FIX, FIX) - 1) / vec_elems(FIX, FIX))), dim3(BLOCK), 0, ctx->stream, in,
-                     out, idt, odt, bits, n);
+  const dim3 grid(grid_for(ctx, (n + vec_elems(FIX, FIX) - 1) / vec_elems(FIX, FIX)));
+  if (FIX >= 0 && streams_past_cache(n, idt, odt))
+    hipLaunchKernelGGL((unary_vec_kernel<OP, CT, FIX, (FIX >= 0)>), grid, dim3(BLOCK), 0, ctx->stream, in, out, idt, odt, bits, n);
+  else
+    hipLaunchKernelGGL((unary_vec_kernel<OP, CT, FIX>), grid, dim3(BLOCK), 0, ctx->stream, in, out, idt, odt, bits, n);
 }
 
 template <int OP, typename CT>
@@ -757,7 +781,14 @@ extern "C" int hipnx_as_type(hipnx_ctx *ctx, int in_dt, int out_dt, int64_t n, c
   static const int64_t tmin[8] = {0, 0, 0, 0, -0x80, -0x8000, -0x80000000ll, (int64_t)0x8000000000000000ull};
   int64_t mx = out_dt < HIPNX_F16 ? tmax[out_dt] : 0, mn = out_dt < HIPNX_F16 ? tmin[out_dt] : 0;
   dim3 grid(grid_for(ctx, (n + E - 1) / E)), block(BLOCK);
-#define HIPNX_AS(CT, I, O) hipLaunchKernelGGL((as_type_kernel<CT, I, O>), dim3(grid_for(ctx, (n + vec_elems(I, O) - 1) / vec_elems(I, O))), block, 0, ctx->stream, inb->ptr, out->ptr, in_dt, out_dt, n, mx, mn)
+#define HIPNX_AS(CT, I, O)                                                                                                        \
+  do {                                                                                                                            \
+    const dim3 g(grid_for(ctx, (n + vec_elems(I, O) - 1) / vec_elems(I, O)));                                                      \
+    if (I >= 0 && streams_past_cache(n, in_dt, out_dt))                                                                           \
+      hipLaunchKernelGGL((as_type_kernel<CT, I, O, (I >= 0)>), g, block, 0, ctx->stream, inb->ptr, out->ptr, in_dt, out_dt, n, mx, mn); \
+    else                                                                                                                          \
+      hipLaunchKernelGGL((as_type_kernel<CT, I, O>), g, block, 0, ctx->stream, inb->ptr, out->ptr, in_dt, out_dt, n, mx, mn);      \
+  } while (0)
   // the conversions of mixed-precision work, compiled for their two types
   if (in_dt == HIPNX_F32 && out_dt == HIPNX_BF16) HIPNX_AS(float, HIPNX_F32, HIPNX_BF16);
   else if (in_dt == HIPNX_BF16 && out_dt == HIPNX_F32) HIPNX_AS(float, HIPNX_BF16, HIPNX_F32);

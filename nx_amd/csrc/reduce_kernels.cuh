@@ -32,7 +32,9 @@ namespace hipnx {
 // encoded into `out`; otherwise the raw accumulator goes to `partial[row*nseg + seg]`.
 // IDT >= 0: the input's element type, known when the kernel is compiled (the type switch inside every
 // vector load, and the scalar bookkeeping the compiler builds around it, fold away); -1: read from `idt_`.
-template <typename R, typename CT, int TPR, bool VEC, int IDT = -1>
+// NT: the input is far larger than the last-level cache and is read with the non-temporal hint (a template parameter:
+// where a branch chooses between a hinted and a plain load the compiler merges them and drops the hint).
+template <typename R, typename CT, int TPR, bool VEC, int IDT = -1, bool NT = false>
 __global__ void __launch_bounds__(BLOCK)
 reduce_rows_kernel(const void *__restrict__ in, void *__restrict__ out, typename R::acc_t *__restrict__ partial,
                    int idt_, int odt, int64_t rows, int64_t red, int64_t seg_len, int nseg) {
@@ -57,8 +59,8 @@ reduce_rows_kernel(const void *__restrict__ in, void *__restrict__ out, typename
       const int64_t step = (int64_t)TPR * E;
       for (; k + step < k1; k += 2 * step) {
         CT v[E], w[E];
-        load_vec<CT, E>(in, idt, base + k, v);
-        load_vec<CT, E>(in, idt, base + k + step, w);
+        load_vec<CT, E, true, NT>(in, idt, base + k, v);
+        load_vec<CT, E, true, NT>(in, idt, base + k + step, w);
 #pragma unroll
         for (int i = 0; i < E; i++) acc = R::accumulate(acc, v[i], k + i);
 #pragma unroll
@@ -66,7 +68,7 @@ reduce_rows_kernel(const void *__restrict__ in, void *__restrict__ out, typename
       }
       for (; k < k1; k += step) {
         CT v[E];
-        load_vec<CT, E>(in, idt, base + k, v);
+        load_vec<CT, E, true, NT>(in, idt, base + k, v);
 #pragma unroll
         for (int i = 0; i < E; i++) acc = R::accumulate(acc, v[i], k + i);
       }
@@ -195,7 +197,7 @@ combine_partials_kernel(const typename R::acc_t *__restrict__ partial, void *__r
 // UNAL (with VEC): `inner` is not a multiple of E (a row of 50257 columns), so a row begins at any offset from a
 // vector boundary: whole vectors are fetched at whatever address they have, the last lane of a row takes its
 // remaining columns one by one (one column per lane moved 256 bytes per wave instruction: 1.6-1.9 TB/s).
-template <typename R, typename CT, bool VEC, int IDT = -1, bool UNAL = false>
+template <typename R, typename CT, bool VEC, int IDT = -1, bool UNAL = false, bool NT = false>
 __global__ void __launch_bounds__(BLOCK)
 reduce_cols_kernel(const void *__restrict__ in, void *__restrict__ out, typename R::acc_t *__restrict__ partial,
                    int idt_, int odt, int64_t outer, int64_t red, int64_t inner, int64_t seg_len, int nseg) {
@@ -225,10 +227,10 @@ reduce_cols_kernel(const void *__restrict__ in, void *__restrict__ out, typename
     int64_t k = k0;
     for (; k + 3 < k1; k += 4) {  // four independent row loads in flight per lane
       CT v0[W], v1[W], v2[W], v3[W];
-      load_vec<CT, W, !UNAL>(in, idt, base + k * inner, v0);
-      load_vec<CT, W, !UNAL>(in, idt, base + (k + 1) * inner, v1);
-      load_vec<CT, W, !UNAL>(in, idt, base + (k + 2) * inner, v2);
-      load_vec<CT, W, !UNAL>(in, idt, base + (k + 3) * inner, v3);
+      load_vec<CT, W, !UNAL, NT>(in, idt, base + k * inner, v0);
+      load_vec<CT, W, !UNAL, NT>(in, idt, base + (k + 1) * inner, v1);
+      load_vec<CT, W, !UNAL, NT>(in, idt, base + (k + 2) * inner, v2);
+      load_vec<CT, W, !UNAL, NT>(in, idt, base + (k + 3) * inner, v3);
 #pragma unroll
       for (int i = 0; i < W; i++) {
         acc[i] = R::accumulate(acc[i], v0[i], k);
@@ -338,6 +340,10 @@ static int run_reduce_t(hipnx_ctx *ctx, bool static_ws, int idt, int odt, int64_
                         const void *in, void *out) {
   typedef typename R::acc_t acc_t;
   const int64_t target_units = (int64_t)ctx->num_cus * 8;  // units of parallel work wanted
+  // an input far larger than the 256 MB last-level cache is read with the non-temporal hint -- where a lane's vector is
+  // one access (elements of 1 or 2 bytes: bf16 row sums over 16384^2 88 -> 80 us): the two 16-byte accesses of eight
+  // f32 each take half of the same lines, and a line that is let go early is fetched twice (f32: 169 -> 180 us)
+  const int stream = outer * red * inner * (int64_t)dtype_size(idt) >= (256ll << 20) && dtype_size(idt) * E <= 16;
   if (inner == 1) {
     const int64_t rows = outer;
     const bool vec = red % E == 0;
@@ -390,10 +396,12 @@ static int run_reduce_t(hipnx_ctx *ctx, bool static_ws, int idt, int odt, int64_
           else hipLaunchKernelGGL((reduce_rows_kernel<R, CT, 32, true, IDT>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
         }
       } else if (tpr == WAVE) {
-        if (vec) hipLaunchKernelGGL((reduce_rows_kernel<R, CT, WAVE, true, IDT>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
+        if (vec && stream && IDT >= 0) hipLaunchKernelGGL((reduce_rows_kernel<R, CT, WAVE, true, IDT, (IDT >= 0)>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
+        else if (vec) hipLaunchKernelGGL((reduce_rows_kernel<R, CT, WAVE, true, IDT>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
         else hipLaunchKernelGGL((reduce_rows_kernel<R, CT, WAVE, false, IDT>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
       } else {
-        if (vec) hipLaunchKernelGGL((reduce_rows_kernel<R, CT, BLOCK, true, IDT>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
+        if (vec && stream && IDT >= 0) hipLaunchKernelGGL((reduce_rows_kernel<R, CT, BLOCK, true, IDT, (IDT >= 0)>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
+        else if (vec) hipLaunchKernelGGL((reduce_rows_kernel<R, CT, BLOCK, true, IDT>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
         else hipLaunchKernelGGL((reduce_rows_kernel<R, CT, BLOCK, false, IDT>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, rows, red, seg_len, nseg);
       }
       if (nseg > 1) {
@@ -435,7 +443,8 @@ static int run_reduce_t(hipnx_ctx *ctx, bool static_ws, int idt, int odt, int64_
     const int64_t cap = MAX_BLOCKS;
     dim3 grid((unsigned)(blocks < 1 ? 1 : (blocks < cap ? blocks : cap))), block(BLOCK);
     if (total > 0) {
-      if (vec) hipLaunchKernelGGL((reduce_cols_kernel<R, CT, true, IDT>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, outer, red, inner, seg_len, nseg);
+      if (vec && stream && IDT >= 0) hipLaunchKernelGGL((reduce_cols_kernel<R, CT, true, IDT, false, (IDT >= 0)>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, outer, red, inner, seg_len, nseg);
+      else if (vec) hipLaunchKernelGGL((reduce_cols_kernel<R, CT, true, IDT>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, outer, red, inner, seg_len, nseg);
       else if (unal) hipLaunchKernelGGL((reduce_cols_kernel<R, CT, true, IDT, true>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, outer, red, inner, seg_len, nseg);
       else hipLaunchKernelGGL((reduce_cols_kernel<R, CT, false>), grid, block, 0, ctx->stream, in, out, partial, idt, odt, outer, red, inner, seg_len, nseg);
       if (nseg > 1) {
