@@ -15,6 +15,9 @@ constexpr int E = 8;  // elements per lane per step of the vector kernels
 
 static bool narrow_float(int dt) { return dt == HIPNX_BF16 || dt == HIPNX_F16 || dt == HIPNX_F32; }
 
+// elements per lane of the select kernel compiled for one element type: 16 bytes of a 4-byte type, else 8
+constexpr int select_elems(int fix) { return fix == HIPNX_F32 || fix == HIPNX_S32 || fix == HIPNX_U32 ? 4 : 8; }
+
 static int grid_for(int64_t items) {
   int64_t blocks = (items + BLOCK - 1) / BLOCK;
   if (blocks < 1) blocks = 1;
@@ -59,10 +62,11 @@ select_nd_kernel(const void *__restrict__ p, const void *__restrict__ t, const v
 // all three operands dense (step 1) or a single element (step 0).  FIX >= 0: a u8 predicate and this
 // element type for both values and the result, known when the kernel is compiled (the run-time type
 // switches of the vector loads and the store fold away).
-template <typename CT, int FIX = -1>
+template <typename CT, int FIX = -1, bool NT = false>
 __global__ void __launch_bounds__(BLOCK)
 select_vec_kernel(const void *__restrict__ p, const void *__restrict__ t, const void *__restrict__ f, void *__restrict__ out,
                   int pdt_, int tdt_, int fdt_, int odt_, int64_t n, int pstep, int tstep, int fstep) {
+  constexpr int E = select_elems(FIX);
   const int pdt = FIX >= 0 ? HIPNX_U8 : pdt_, tdt = FIX >= 0 ? FIX : tdt_, fdt = FIX >= 0 ? FIX : fdt_, odt = FIX >= 0 ? FIX : odt_;
   const int64_t nvec = (n + E - 1) / E;
   for (int64_t v = (int64_t)blockIdx.x * BLOCK + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * BLOCK) {
@@ -75,9 +79,15 @@ select_vec_kernel(const void *__restrict__ p, const void *__restrict__ t, const 
 #pragma unroll
         for (int e = 0; e < E; e++) pt[e] = one;
       } else if (pdt == HIPNX_U8 || pdt == HIPNX_S8) {  // what comparisons and logical ops produce
-        const uint2 w = *reinterpret_cast<const uint2 *>(static_cast<const unsigned char *>(p) + i0);
+        if constexpr (E == 8) {
+          const uint2 w = *reinterpret_cast<const uint2 *>(static_cast<const unsigned char *>(p) + i0);
 #pragma unroll
-        for (int e = 0; e < E; e++) pt[e] = (((e < 4 ? w.x : w.y) >> (8 * (e & 3))) & 0xFF) != 0;
+          for (int e = 0; e < E; e++) pt[e] = (((e < 4 ? w.x : w.y) >> (8 * (e & 3))) & 0xFF) != 0;
+        } else {
+          const uint32_t w = *reinterpret_cast<const uint32_t *>(static_cast<const unsigned char *>(p) + i0);
+#pragma unroll
+          for (int e = 0; e < E; e++) pt[e] = ((w >> (8 * e)) & 0xFF) != 0;
+        }
       } else if (pdt >= HIPNX_F16) {
         double pd[E];
         load_vec<double, E>(p, pdt, i0, pd);
@@ -90,17 +100,17 @@ select_vec_kernel(const void *__restrict__ p, const void *__restrict__ t, const 
         for (int e = 0; e < E; e++) pt[e] = pi[e] != 0;
       }
       // (an operand that is one element for all -- a number -- keeps its own type also in the typed form)
-      if (tstep) load_vec<CT, E>(t, tdt, i0, a);
+      if (tstep) load_vec<CT, E, true, NT>(t, tdt, i0, a);
       else { const CT x = load_one<CT>(t, tdt_, 0);
 #pragma unroll
         for (int e = 0; e < E; e++) a[e] = x; }
-      if (fstep) load_vec<CT, E>(f, fdt, i0, b);
+      if (fstep) load_vec<CT, E, true, NT>(f, fdt, i0, b);
       else { const CT x = load_one<CT>(f, fdt_, 0);
 #pragma unroll
         for (int e = 0; e < E; e++) b[e] = x; }
 #pragma unroll
       for (int e = 0; e < E; e++) c[e] = pt[e] ? a[e] : b[e];
-      store_vec<CT, E>(out, odt, i0, c);
+      store_vec<CT, E, NT>(out, odt, i0, c);
     } else {
       for (int64_t i = i0; i < n; i++) {
         const CT x = truthy<CT>(p, pdt, i * pstep) ? load_one<CT>(t, tstep ? tdt : tdt_, i * tstep) : load_one<CT>(f, fstep ? fdt : fdt_, i * fstep);
@@ -137,22 +147,38 @@ __device__ inline CT clip_one(CT x, CT lo, CT hi, bool xu, bool lou, bool hiu) {
   }
 }
 
-template <typename CT, int FIX = -1>  // FIX >= 0: the element type of input and result, known at compile time
+// elements per lane where the element type is known at compile time: 16 bytes of a 4-byte type (one access per lane,
+// lanes side by side: a wave instruction covers whole lines), else the 8 of the general form
+constexpr int fixed_elems(int fix) { return fix == HIPNX_F32 || fix == HIPNX_S32 || fix == HIPNX_U32 ? 4 : 8; }
+
+// FIX >= 0: the element type of input and result, known at compile time; NT: tensors far larger than the last-level
+// cache, every access with the non-temporal hint
+template <typename CT, int FIX = -1, bool NT = false>
 __global__ void __launch_bounds__(BLOCK)
 clip_kernel(const void *__restrict__ in, const void *__restrict__ mn, const void *__restrict__ mx, void *__restrict__ out,
             int idt_, int mndt, int mxdt, int odt_, int64_t n) {
+  constexpr int E = fixed_elems(FIX);
   const int idt = FIX >= 0 ? FIX : idt_, odt = FIX >= 0 ? FIX : odt_;
-  const CT lo = load_one<CT>(mn, mndt, 0), hi = load_one<CT>(mx, mxdt, 0);
+  // (bounds of the tensor's own type, the usual case, are two scalar loads issued together; decoding a bound of any
+  // type is a chain of branches and waits that every wave would walk before it asks for its data)
+  CT lo, hi;
+  if (FIX >= 0 && mndt == FIX && mxdt == FIX) {
+    lo = load_one<CT>(mn, FIX, 0);
+    hi = load_one<CT>(mx, FIX, 0);
+  } else {
+    lo = load_one<CT>(mn, mndt, 0);
+    hi = load_one<CT>(mx, mxdt, 0);
+  }
   const bool xu = idt == HIPNX_U64, lou = mndt == HIPNX_U64, hiu = mxdt == HIPNX_U64;
   const int64_t nvec = (n + E - 1) / E;
   for (int64_t v = (int64_t)blockIdx.x * BLOCK + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * BLOCK) {
     const int64_t i0 = v * E;
     if (i0 + E <= n) {
       CT x[E];
-      load_vec<CT, E>(in, idt, i0, x);
+      load_vec<CT, E, true, NT>(in, idt, i0, x);
 #pragma unroll
       for (int e = 0; e < E; e++) x[e] = clip_one<CT>(x[e], lo, hi, xu, lou, hiu);
-      store_vec<CT, E>(out, odt, i0, x);
+      store_vec<CT, E, NT>(out, odt, i0, x);
     } else {
       for (int64_t i = i0; i < n; i++) store_one<CT>(out, odt, i, clip_one<CT>(load_one<CT>(in, idt, i), lo, hi, xu, lou, hiu));
     }
@@ -335,9 +361,18 @@ extern "C" int hipnx_select(hipnx_ctx *ctx, int pred_dt, int true_dt, int false_
   // values only pass through: f32 arithmetic holds every bf16 / f16 / f32 exactly
   const bool narrow = narrow_float(true_dt) && narrow_float(false_dt) && narrow_float(out_dt);
   if (m == 1 && s.ps[0] <= 1 && s.ts[0] <= 1 && s.fs[0] <= 1) {
-    dim3 grid(grid_for((n + E - 1) / E)), block(BLOCK);
-#define HIPNX_SELECT(CT, FIX) hipLaunchKernelGGL((select_vec_kernel<CT, FIX>), grid, block, 0, ctx->stream, pred->ptr, on_true->ptr, on_false->ptr, out->ptr, \
-                                               pred_dt, true_dt, false_dt, out_dt, n, (int)s.ps[0], (int)s.ts[0], (int)s.fs[0])
+    const dim3 block(BLOCK);
+    const bool past_cache = n * (int64_t)dtype_size(out_dt) >= (256ll << 20);
+#define HIPNX_SELECT(CT, FIX)                                                                                                       \
+  do {                                                                                                                              \
+    const dim3 grid(grid_for((n + select_elems(FIX) - 1) / select_elems(FIX)));                                                      \
+    if (FIX >= 0 && past_cache)                                                                                                     \
+      hipLaunchKernelGGL((select_vec_kernel<CT, FIX, (FIX >= 0)>), grid, block, 0, ctx->stream, pred->ptr, on_true->ptr, on_false->ptr, out->ptr, \
+                         pred_dt, true_dt, false_dt, out_dt, n, (int)s.ps[0], (int)s.ts[0], (int)s.fs[0]);                          \
+    else                                                                                                                            \
+      hipLaunchKernelGGL((select_vec_kernel<CT, FIX>), grid, block, 0, ctx->stream, pred->ptr, on_true->ptr, on_false->ptr, out->ptr, \
+                         pred_dt, true_dt, false_dt, out_dt, n, (int)s.ps[0], (int)s.ts[0], (int)s.fs[0]);                          \
+  } while (0)
     // one element type throughout, where a lone element (a number) may have another one that the kernel's
     // arithmetic type holds exactly: select(mask, scores_bf16, -1.0e9) arrives with an f32 number
     auto fits = [&](int dt, int64_t step) {
@@ -380,8 +415,16 @@ extern "C" int hipnx_clip(hipnx_ctx *ctx, int in_dt, int min_dt, int max_dt, int
   if (int st = check_buf(ctx, max, dtype_size(max_dt), "clip max")) return st;
   if (int st = check_buf(ctx, out, (uint64_t)n * dtype_size(out_dt), "clip out")) return st;
   if (n == 0) return HIPNX_OK;
-  dim3 grid(grid_for((n + E - 1) / E)), block(BLOCK);
-#define HIPNX_CLIP(CT, FIX) hipLaunchKernelGGL((clip_kernel<CT, FIX>), grid, block, 0, ctx->stream, inb->ptr, min->ptr, max->ptr, out->ptr, in_dt, min_dt, max_dt, out_dt, n)
+  const dim3 block(BLOCK);
+  const bool past_cache = n * (int64_t)dtype_size(out_dt) >= (256ll << 20);
+#define HIPNX_CLIP(CT, FIX)                                                                                                        \
+  do {                                                                                                                             \
+    const dim3 grid(grid_for((n + fixed_elems(FIX) - 1) / fixed_elems(FIX)));                                                       \
+    if (FIX >= 0 && past_cache)                                                                                                    \
+      hipLaunchKernelGGL((clip_kernel<CT, FIX, (FIX >= 0)>), grid, block, 0, ctx->stream, inb->ptr, min->ptr, max->ptr, out->ptr, in_dt, min_dt, max_dt, out_dt, n); \
+    else                                                                                                                           \
+      hipLaunchKernelGGL((clip_kernel<CT, FIX>), grid, block, 0, ctx->stream, inb->ptr, min->ptr, max->ptr, out->ptr, in_dt, min_dt, max_dt, out_dt, n); \
+  } while (0)
   if (narrow_float(in_dt) && narrow_float(min_dt) && narrow_float(max_dt) && narrow_float(out_dt)) {
     if (in_dt == out_dt && out_dt == HIPNX_F32) HIPNX_CLIP(float, HIPNX_F32);
     else if (in_dt == out_dt && out_dt == HIPNX_BF16) HIPNX_CLIP(float, HIPNX_BF16);
