@@ -32,6 +32,18 @@ namespace hipnx {
 // encoded into `out`; otherwise the raw accumulator goes to `partial[row*nseg + seg]`.
 // IDT >= 0: the input's element type, known when the kernel is compiled (the type switch inside every
 // vector load, and the scalar bookkeeping the compiler builds around it, fold away); -1: read from `idt_`.
+// Elements a lane takes per load where the reducer allows any assignment of elements to lanes and the element type is
+// known at compile time: 16 bytes (one access per lane, lanes side by side, so that a wave instruction covers whole
+// lines), instead of the eight elements whose order of folding a sum's bits depend on.
+constexpr int reduce_type_bytes(int dt) {
+  return dt < 0 ? 0 : (dt == HIPNX_U8 || dt == HIPNX_S8) ? 1 : (dt == HIPNX_U16 || dt == HIPNX_S16 || dt == HIPNX_F16 || dt == HIPNX_BF16) ? 2
+         : (dt == HIPNX_U32 || dt == HIPNX_S32 || dt == HIPNX_F32) ? 4 : 8;
+}
+template <typename R>
+constexpr int reduce_load_elems(int idt) {
+  return R::any_order && reduce_type_bytes(idt) >= 4 ? 16 / reduce_type_bytes(idt) : E;
+}
+
 // NT: the input is far larger than the last-level cache and is read with the non-temporal hint (a template parameter:
 // where a branch chooses between a hinted and a plain load the compiler merges them and drops the hint).
 template <typename R, typename CT, int TPR, bool VEC, int IDT = -1, bool NT = false>
@@ -53,24 +65,26 @@ reduce_rows_kernel(const void *__restrict__ in, void *__restrict__ out, typename
     const int64_t k1 = k0 + seg_len < red ? k0 + seg_len : red;
     const int64_t base = row * red;
     if constexpr (VEC) {  // red % E == 0 and seg_len % E == 0: every vector is aligned
-      // two (then one) 8-element vectors per step: both loads are issued before either is folded
-      int64_t k = k0 + (int64_t)lane * E;
+      // two (then one) vectors per step: both loads are issued before either is folded.  A vector is eight elements,
+      // or 16 bytes where the reducer lets the lanes share a row any way (EL: maxima, arg-reductions, all / any)
+      constexpr int EL = reduce_load_elems<R>(IDT);
+      int64_t k = k0 + (int64_t)lane * EL;
       if (k < k1) acc = R::seed(acc, k);
-      const int64_t step = (int64_t)TPR * E;
+      const int64_t step = (int64_t)TPR * EL;
       for (; k + step < k1; k += 2 * step) {
-        CT v[E], w[E];
-        load_vec<CT, E, true, NT>(in, idt, base + k, v);
-        load_vec<CT, E, true, NT>(in, idt, base + k + step, w);
+        CT v[EL], w[EL];
+        load_vec<CT, EL, true, NT>(in, idt, base + k, v);
+        load_vec<CT, EL, true, NT>(in, idt, base + k + step, w);
 #pragma unroll
-        for (int i = 0; i < E; i++) acc = R::accumulate(acc, v[i], k + i);
+        for (int i = 0; i < EL; i++) acc = R::accumulate(acc, v[i], k + i);
 #pragma unroll
-        for (int i = 0; i < E; i++) acc = R::accumulate(acc, w[i], k + step + i);
+        for (int i = 0; i < EL; i++) acc = R::accumulate(acc, w[i], k + step + i);
       }
       for (; k < k1; k += step) {
-        CT v[E];
-        load_vec<CT, E, true, NT>(in, idt, base + k, v);
+        CT v[EL];
+        load_vec<CT, EL, true, NT>(in, idt, base + k, v);
 #pragma unroll
-        for (int i = 0; i < E; i++) acc = R::accumulate(acc, v[i], k + i);
+        for (int i = 0; i < EL; i++) acc = R::accumulate(acc, v[i], k + i);
       }
     } else if constexpr (TPR < WAVE) {
       // a short row that is not whole vectors (33 elements): vectors fetched at whatever address they have, the
@@ -343,7 +357,9 @@ static int run_reduce_t(hipnx_ctx *ctx, bool static_ws, int idt, int odt, int64_
   // an input far larger than the 256 MB last-level cache is read with the non-temporal hint -- where a lane's vector is
   // one access (elements of 1 or 2 bytes: bf16 row sums over 16384^2 88 -> 80 us): the two 16-byte accesses of eight
   // f32 each take half of the same lines, and a line that is let go early is fetched twice (f32: 169 -> 180 us)
-  const int stream = outer * red * inner * (int64_t)dtype_size(idt) >= (256ll << 20) && dtype_size(idt) * E <= 16;
+  // (reducers that let a lane take 16 bytes at a time read any type that way)
+  const int stream = outer * red * inner * (int64_t)dtype_size(idt) >= (256ll << 20) &&
+                     (dtype_size(idt) * E <= 16 || (R::any_order && IDT >= 0));
   if (inner == 1) {
     const int64_t rows = outer;
     const bool vec = red % E == 0;

@@ -21,6 +21,9 @@ constexpr int WAVE = 64;
 template <typename CT, int OP, bool UNS>
 struct PlainReducer {
   typedef CT acc_t;
+  // whether the result is the same bits whichever elements a lane is given (sums and products of floats are not:
+  // their order of additions is part of the result)
+  static constexpr bool any_order = OP != HIPNX_RED_SUM && OP != HIPNX_RED_PRODUCT;
   static __device__ __forceinline__ acc_t init() {
     if constexpr (OP == HIPNX_RED_SUM || OP == HIPNX_RED_ANY) return (CT)0;
     else if constexpr (OP == HIPNX_RED_PRODUCT || OP == HIPNX_RED_ALL) return (CT)1;
@@ -65,6 +68,7 @@ struct ArgAcc {
 template <typename CT, int OP, int TIE, bool UNS>
 struct ArgReducer {
   typedef ArgAcc<CT> acc_t;
+  static constexpr bool any_order = true;  // (a lane must still meet its own elements in rising order)
   static constexpr bool FP = std::is_floating_point<CT>::value;
   // the worst possible value: nothing is worse, so a lane seeded with {worst, first index} is
   // already the right answer for "no better element seen yet"
