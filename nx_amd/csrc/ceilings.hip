@@ -18,6 +18,14 @@
 //       the best reported), from a region its XCD's L2 holds (`l2`: the work-groups of an XCD share 2 MiB), from
 //       the last-level cache (`llc`: 512 KiB per work-group, 128 MiB in all) or from HBM (`hbm`: 4 MiB per
 //       work-group, 1 GiB in all); bytes per clock of the shader clock measured in the last launch
+//   hipnx_ceilings weights <work-groups> <none|interleaved|first> [KiB of rows per work-group]
+//       the requests of a few rows against a long weight matrix (64 x 4096 int8 rows, 11008 x 4096 int8 weights: 45 MB
+//       streamed once) without the arithmetic: `work-groups` work-groups of 8 waves share the weights evenly and pull
+//       them into LDS with direct-to-LDS loads, 8 KiB in flight per wave, from one of ten copies in turn (nothing comes
+//       from the last-level cache); beside them no bytes of the rows (`none`), as many bytes of the rows as of the
+//       weights, request by request, from 256 KiB that L2 holds (`interleaved`: what a tile of the contraction kernels
+//       takes in), or a fixed share of the rows before the first weights (`first`: what a work-group with its share of
+//       the rows resident would take in).  Microseconds per launch over 400 launches back to back.
 //
 // Each run prints one JSON line.  Built by the Makefile into nx_amd/lib/hipnx_ceilings; bench.py runs
 // it when present and copies the sustained figures into its `measured_ceiling` fields.
@@ -133,6 +141,34 @@ __global__ void __launch_bounds__(512) ingest_loop(const unsigned char *src, siz
     g_clk[0] = clock64() - c0;
     g_clk[1] = wall_clock64() - w0;
   }
+}
+
+// The requests of the few-rows contraction without its arithmetic: a work-group pulls `w_per_wg` bytes of weights,
+// 8 KiB in flight per wave; x_mode 1: every request for weights is followed by one for the rows (a 256 KiB region
+// that L2 holds); x_mode 2: `xbytes` of the rows first.
+__global__ void __launch_bounds__(512) weights_requests(const unsigned char *w, size_t w_per_wg, const unsigned char *x, size_t xbytes, int x_mode, unsigned *sink) {
+  extern __shared__ unsigned char ingest_lds[];
+  constexpr int DEPTH = 8;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const unsigned char *wb = w + (size_t)blockIdx.x * w_per_wg;
+  unsigned char *mine = ingest_lds + wave * DEPTH * 1024;
+  const unsigned at = wave * 1024 + lane * 16, per_step = 8 * 1024, xmask = 256 * 1024 - 1;
+  const unsigned steps = (unsigned)(w_per_wg / per_step);
+  if (x_mode == 2)
+    for (unsigned s = 0; s < xbytes / per_step; s += DEPTH) {
+#pragma unroll
+      for (int d = 0; d < DEPTH; d++) lds_dma16(x + (((s + d) * per_step + at) & xmask), mine + d * 1024);
+    }
+  for (unsigned s = 0; s < steps; s += DEPTH) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++) {
+      const unsigned o = s + d < steps ? (s + d) * per_step + at : at;
+      lds_dma16(wb + o, mine + d * 1024);
+      if (x_mode == 1) lds_dma16(x + (o & xmask), mine + d * 1024);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  }
+  if (((unsigned *)mine)[lane] == 0x12345678u) sink[0] = 1;  // (keeps the loads alive)
 }
 
 // Streaming kernels with a grid that covers the buffer (no grid-stride loop; on this part a resident grid
@@ -347,11 +383,38 @@ static int run_ingest(const char *from, double want_ms) {
   return 0;
 }
 
+static int run_weights(int groups, const char *rows, size_t x_kib) {
+  const int x_mode = !strcmp(rows, "none") ? 0 : !strcmp(rows, "interleaved") ? 1 : !strcmp(rows, "first") ? 2 : -1;
+  if (x_mode < 0 || groups < 1 || groups > 4096) { fprintf(stderr, "weights <work-groups> <none|interleaved|first> [KiB]\n"); return 2; }
+  const size_t total = 11008ull * 4096, step = 8 * 1024, per = (total / groups + step - 1) / step * step, wbuf = per * groups;
+  const int copies = 10, lds = 8 * 8 * 1024, launches = 400;
+  unsigned char *w, *x;
+  unsigned *sink;
+  CK(hipMalloc(&w, wbuf * copies));
+  CK(hipMalloc(&x, 256 * 1024));
+  CK(hipMalloc(&sink, 4));
+  CK(hipMemset(w, 1, wbuf * copies));
+  CK(hipMemset(x, 1, 256 * 1024));
+  int turn = 0;
+  auto launch = [&] {
+    hipLaunchKernelGGL(weights_requests, dim3(groups), dim3(512), lds, 0, w + (size_t)(turn++ % copies) * wbuf, per, x, x_kib * 1024, x_mode, sink);
+  };
+  std::vector<float> ms;
+  if (timed_chunks(launch, 1, 50, ms)) return 1;
+  if (timed_chunks(launch, 1, launches, ms)) return 1;
+  const double us = 1000.0 * ms[0] / launches;
+  printf("{\"kind\": \"weights\", \"work_groups\": %d, \"rows\": \"%s\", \"KiB_of_weights_per_work_group\": %zu, \"KiB_of_rows_per_work_group\": %zu, "
+         "\"launch_us\": %.2f, \"GBps_of_weights\": %.0f}\n",
+         groups, rows, per / 1024, x_mode == 1 ? per / 1024 : x_mode == 2 ? x_kib : (size_t)0, us, (double)wbuf / us / 1e3);
+  return 0;
+}
+
 int main(int argc, char **argv) {
+  if (argc >= 4 && !strcmp(argv[1], "weights")) return run_weights(atoi(argv[2]), argv[3], argc > 4 ? (size_t)atol(argv[4]) : 64);
   if (argc >= 3 && !strcmp(argv[1], "ingest")) return run_ingest(argv[2], argc > 3 ? atof(argv[3]) : 100.0);
   if (argc >= 4 && !strcmp(argv[1], "mfma")) return run_mfma(argv[2], argv[3], argc > 4 ? atof(argv[4]) : 300.0);
   if (argc >= 3 && !strcmp(argv[1], "stream")) return run_stream(argv[2], argc > 3 ? (size_t)atol(argv[3]) : 2048, argc > 4 ? atof(argv[4]) : 100.0);
   fprintf(stderr, "usage: hipnx_ceilings mfma <bf16|f16|s8|f32> <random|normal|zero> [ms]\n       hipnx_ceilings stream <read|write|copy> [MiB] [ms]\n"
-                  "       hipnx_ceilings ingest <l2|llc|hbm> [ms]\n");
+                  "       hipnx_ceilings ingest <l2|llc|hbm> [ms]\n       hipnx_ceilings weights <work-groups> <none|interleaved|first> [KiB of rows]\n");
   return 2;
 }
