@@ -345,6 +345,7 @@ gemm_pingpong128_kernel(GemmArgs a) {
   static_assert(DT == HIPNX_BF16 || DT == HIPNX_F16 || DT == HIPNX_S8 || (DT == HIPNX_F32 && L_KIN && R_KIN),
                 "2-byte MFMA types and int8; f32 with K-inner operands");
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  HIPNX_TL_STAMP(tl_start);
 
   int tm, tn;
   gemm_tile_position(a, blockIdx.x, tm, tn);
@@ -453,6 +454,8 @@ gemm_pingpong128_kernel(GemmArgs a) {
     else wait_vmcnt<0>();
   }
   __builtin_amdgcn_s_barrier();
+  HIPNX_TL_STAMP(tl_walk);
+  HIPNX_TL_CLOCK(tl_c0);
 
   // phases 0 .. nslab, every wave passes the barrier that ends each of them
   if (grp == 0) {
@@ -473,6 +476,8 @@ gemm_pingpong128_kernel(GemmArgs a) {
     }
   }
 
+  HIPNX_TL_STAMP(tl_done);
+  HIPNX_TL_CLOCK(tl_c1);
   // the two partial sums: every wave hands the half of its tile the other group finishes to that group
   // (TM16 / 2 x TN16 accumulator tiles of 1 KiB) and adds what it is handed
   {
@@ -519,6 +524,13 @@ gemm_pingpong128_kernel(GemmArgs a) {
 #undef HIPNX_EPI
     }
   }
+#ifdef HIPNX_GEMM_TIMELINE
+  if (threadIdx.x == 0 && blockIdx.x < 4096) {
+    unsigned long long *p = g_timeline + (size_t)blockIdx.x * 8;
+    p[0] = tl_start; p[1] = tl_walk; p[2] = tl_done; p[3] = wall_clock64(); p[4] = tl_c1 - tl_c0;
+    p[5] = __builtin_amdgcn_s_getreg((31 << 11) | 20);  // XCC_ID
+  }
+#endif
 }
 
 }  // namespace hipnx

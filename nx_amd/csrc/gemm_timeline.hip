@@ -8,7 +8,8 @@
 //
 // Environment: HIPNX_TL_ZERO=1 fills the operands with zeros (the same instructions and traffic with the least
 // switching in the data paths: what the clock does to the figure); HIPNX_TL_HALF_WIDTH=1 runs 256 x 128 tiles
-// (two per compute unit at n = 4096); HIPNX_TL_GROUP_M sets the tile order's group height.  The Makefile also
+// (two per compute unit at n = 4096); HIPNX_TL_TILE_128=1 runs the two-group kernel on 128 x 128 tiles (the mid-size
+// problems' kernel: one tile per compute unit at n = 2048); HIPNX_TL_GROUP_M sets the tile order's group height.  The Makefile also
 // builds hipnx_gemm_timeline_exp1 / _exp32 / _exp64 from this file with -DHIPNX_PP_EXP=1 / 32 / 64: the walk
 // without its requests, without its fragment reads, without the wait for its requests (timing only, results
 // wrong -- "sampled_outputs_wrong" says so) -- what each of the three costs the walk.
@@ -60,11 +61,12 @@ __global__ void sample_rows(const unsigned char *l, const unsigned char *r, floa
   }
 }
 
-template <int DT, int BN = 256>
+// BM = 256: the 256-row two-group kernel (BN = 256 or 128); BM = 128: the two-group kernel on 128 x 128 tiles
+template <int DT, int BN = 256, int BM = 256>
 static int run(int n, double settle_ms, int launches) {
   constexpr int ES = DT == HIPNX_S8 ? 1 : 2, OS = DT == HIPNX_S8 ? 4 : 2;
   constexpr int MFMA_K = DT == HIPNX_S8 ? 64 : 32;  // k per 16 x 16 MFMA of 16 clocks
-  if (n % 256 != 0 || n <= 0 || (n / 256) * (n / BN) > 4096) {
+  if (n % 256 != 0 || n <= 0 || (n / BM) * (n / BN) > 4096) {
     fprintf(stderr, "n must be a multiple of 256 with at most 4096 tiles\n");
     return 2;
   }
@@ -108,11 +110,14 @@ static int run(int n, double settle_ms, int launches) {
   a.Kb = (int64_t)n * ES;
   a.ld_l = (int64_t)n * ES;  // [M, K], K contiguous
   a.ld_r = (int64_t)n * ES;  // [K, N], N contiguous
-  a.tiles_m = n / 256;
+  a.tiles_m = n / BM;
   a.tiles_n = n / BN;
   a.group_m = getenv("HIPNX_TL_GROUP_M") ? atoi(getenv("HIPNX_TL_GROUP_M")) : gemm_group_m(a.tiles_m, a.tiles_n);
-  auto kern = gemm_pingpong_kernel<DT, true, false, true, true, BN>;  // BN = 256: the instantiation the library launches for these layouts
-  const int smem = 2 * (256 + BN) * SLAB;
+  // (the instantiations the library launches for these layouts)
+  void (*kern)(GemmArgs);
+  if constexpr (BM == 256) kern = gemm_pingpong_kernel<DT, true, false, true, true, BN>;
+  else kern = gemm_pingpong128_kernel<DT, true, false, 128, 128, 4, 1>;
+  const int smem = BM == 256 ? 2 * (256 + BN) * SLAB : 4 * (128 + 128) * SLAB;
   CK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
   const dim3 grid(a.tiles_m * a.tiles_n), block(512);
 
@@ -194,16 +199,16 @@ static int run(int n, double settle_ms, int launches) {
   }
   start /= nb, walk0 /= nb, walk1 /= nb, stored /= nb, clocks /= nb, dur /= nb;
   // MFMA work of a work-group's walk: per SIMD two waves of 32 tiles each, 16 clocks per MFMA, K / MFMA_K steps
-  const double mfma_clocks = 2.0 * (32 * BN / 256) * 16 * ((double)n / MFMA_K);
+  const double mfma_clocks = BM == 256 ? 2.0 * (32 * BN / 256) * 16 * ((double)n / MFMA_K) : 16.0 * 16 * ((double)n / MFMA_K);
   const double ops = 2.0 * n * n * (double)n;
-  printf("{\"kernel\": \"gemm_pingpong_kernel<%s, K-inner x K-outer, 256 x %d>\", \"variant\": \"%s\", \"operands\": \"%s\", \"n\": %d, \"work_groups\": %d, \"launches\": %d, "
+  printf("{\"kernel\": \"%s<%s, K-inner x K-outer, %d x %d>\", \"variant\": \"%s\", \"operands\": \"%s\", \"n\": %d, \"work_groups\": %d, \"launches\": %d, "
          "\"launch_us\": %.2f, \"rate_T\": %.1f, \"sampled_outputs_wrong\": %d, "
          "\"timeline_us_from_first_start\": {\"group_start\": {\"avg\": %.2f, \"max\": %.2f}, \"walk_begins\": {\"avg\": %.2f, \"max\": %.2f}, "
          "\"walk_ends\": {\"avg\": %.2f, \"max\": %.2f}, \"last_store_issued\": {\"avg\": %.2f, \"max\": %.2f}, \"span\": %.2f}, "
          "\"walk_us\": {\"min\": %.2f, \"avg\": %.2f, \"max\": %.2f}, \"epilogue_us_avg\": %.2f, \"after_last_store_us\": %.2f, "
          "\"walk_shader_clocks\": %.0f, \"walk_shader_clock_MHz\": %.0f, \"mfma_clocks_needed\": %.0f, \"mfma_share_of_walk_clocks\": %.4f, "
          "\"walk_us_avg_per_xcc\": [",
-         DT == HIPNX_S8 ? "s8" : "bf16", BN, HIPNX_PP_EXP == 0 ? "the library's kernel" : HIPNX_PP_EXP == 1 ? "timing only: no requests after the prologue" : HIPNX_PP_EXP == 32 ? "timing only: no fragment reads after the first slab" : HIPNX_PP_EXP == 64 ? "timing only: no wait for the requests" : "timing only", getenv("HIPNX_TL_ZERO") ? "all zero" : "as the benchmark draws them", n, nb, launches, launch_us, ops / launch_us / 1e6, bad, start, start_max, walk0, walk0_max, walk1, walk1_max,
+         BM == 256 ? "gemm_pingpong_kernel" : "gemm_pingpong128_kernel", DT == HIPNX_S8 ? "s8" : "bf16", BM, BN, HIPNX_PP_EXP == 0 ? "the library's kernel" : HIPNX_PP_EXP == 1 ? "timing only: no requests after the prologue" : HIPNX_PP_EXP == 32 ? "timing only: no fragment reads after the first slab" : HIPNX_PP_EXP == 64 ? "timing only: no wait for the requests" : "timing only", getenv("HIPNX_TL_ZERO") ? "all zero" : "as the benchmark draws them", n, nb, launches, launch_us, ops / launch_us / 1e6, bad, start, start_max, walk0, walk0_max, walk1, walk1_max,
          stored, stored_max, (tend - t0) * tick, dur_min, dur, dur_max, stored - walk1, launch_us - stored_max, clocks, clocks / dur,
          mfma_clocks, mfma_clocks / clocks);
   for (int x = 0; x < 8; x++) printf("%s%.2f", x ? ", " : "", xcc_n[x] ? xcc_dur[x] / xcc_n[x] : 0.0);
@@ -219,6 +224,10 @@ int main(int argc, char **argv) {
   const double settle = argc > 3 ? atof(argv[3]) : 400.0;
   const int launches = argc > 4 ? atoi(argv[4]) : 100;
   const bool half = getenv("HIPNX_TL_HALF_WIDTH") != nullptr;  // 256 x 128 tiles: two per compute unit at n = 4096
+  if (getenv("HIPNX_TL_TILE_128")) {  // the two-group kernel on 128 x 128 tiles (what the library launches at n = 2048)
+    if (type == "bf16") return run<HIPNX_BF16, 128, 128>(n, settle, launches);
+    if (type == "s8") return run<HIPNX_S8, 128, 128>(n, settle, launches);
+  }
   if (type == "bf16") return half ? run<HIPNX_BF16, 128>(n, settle, launches) : run<HIPNX_BF16>(n, settle, launches);
   if (type == "s8") return half ? run<HIPNX_S8, 128>(n, settle, launches) : run<HIPNX_S8>(n, settle, launches);
   fprintf(stderr, "usage: hipnx_gemm_timeline <bf16|s8> [n] [settle ms] [launches]\n");
