@@ -93,7 +93,12 @@ __device__ __forceinline__ CT binary_apply(CT a, CT b) {
     else if constexpr (OP == HIPNX_DIVIDE) return a / b;
     else if constexpr (OP == HIPNX_POW) return pow(a, b);
     else if constexpr (OP == HIPNX_REMAINDER) return fmod(a, b);
-    else if constexpr (OP == HIPNX_ATAN2) return atan2(a, b);
+    else if constexpr (OP == HIPNX_ATAN2) {
+      // through f64, as the reference computes it (one rounding of the f64 result).  The f32 routine of the device
+      // library comes in two variants (one with a faster division), and the offline and the run-time compiler do not
+      // pick the same one: a fused group compiled at run time would differ from the same node run alone in the last bit.
+      return (CT)atan2((double)a, (double)b);
+    }
     else if constexpr (OP == HIPNX_MAX) return (a != a || b != b) ? (CT)NAN : (b > a ? b : a);
     else if constexpr (OP == HIPNX_MIN) return (a != a || b != b) ? (CT)NAN : (b < a ? b : a);
     else if constexpr (OP == HIPNX_EQUAL) return (CT)(a == b);

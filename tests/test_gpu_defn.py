@@ -346,7 +346,7 @@ def test_compiled_programs_are_bounded_and_the_oldest_go_first(hip):
         def fun(t):
             return Nx.multiply(Nx.tanh(t), c)
         return fun
-    consts = [1.0 + i / 16 for i in range(10)]
+    consts = [1.0 + i / 16 for i in range(1, 11)]  # (not 1.0: the tracer drops a multiplication by one, and the first call must compile)
     B.fused_mode("compiled")
     B.fused_cache_limit(8)
     pinned = 4  # programs that earlier tests recorded into graphs stay loaded
