@@ -127,7 +127,7 @@ def test_binary_ops_over_random_ranks_and_numbers(case, hip, oracle):
 
     f = getattr(Nx, op)
     check(lambda: f(ha, hb), lambda: f(oa, ob), what)
-    number = [2, -3, 0.5, 1.0, 7][int(rng.integers(0, 5))]
+    number = [2, -3, 0.5, 1.0, 7, 0.1, 0.044715, -1.0e-3, 3.0e9, 300][int(rng.integers(0, 10))]  # some inexact in every float type, some beyond the narrow integers
     check(lambda: f(ha, number), lambda: f(oa, number), f"{what} with the number {number} on the right")
     check(lambda: f(number, hb), lambda: f(number, ob), f"{what} with the number {number} on the left")
 
