@@ -155,3 +155,112 @@ def test_dot_on_random_shapes_types_and_layouts(case, hip, oracle):
     else:
         oa, ob = both(a, ty, hip, oracle)[1], both(b, ty, hip, oracle)[1]
         check_float_dot(got, want, values(oa), values(ob), "bmk,bkn->bmn", K, what)
+
+
+# ---- the same sweeps at sizes where the kernels change shape: rows longer than a work-group's share (split rows), more
+# vectors than one pass of the grid, column reductions under long axes, copies past 2^16 vectors ----------------------------
+
+BIG = [1, 2, 3, 8, 17, 64, 100, 257, 1000, 1024, 4096, 4100, 8191, 32768, 40000, 65536, 70001, 131080, 262144, 1000003]
+
+
+def draw_big_shape(rng, rank, lo=200_000, hi=5_000_000):
+    while True:
+        shape = tuple(int(rng.choice(BIG)) for _ in range(rank))
+        if lo <= int(np.prod(shape, dtype=np.int64)) <= hi:
+            return shape
+
+
+@pytest.mark.parametrize("case", range(40))
+def test_exact_callbacks_on_large_random_shapes(case, hip, oracle):
+    rng = np.random.default_rng(seed_of("large", case + OFFSET))
+    rank = int(rng.integers(1, 4))
+    shape = draw_big_shape(rng, rank)
+    ty = ["f32", "bf16", "s32", "u8", "f16", "s16", "s64", "f64"][int(rng.integers(0, 8))]
+    x = rand_raw(rng, ty, shape)
+    hx, ox = both(x, ty, hip, oracle)
+    what = f"{ty}{shape}"
+    # element-wise against a broadcast operand, and a conversion
+    bs = broadcastable(rng, shape)
+    y = rand_raw(rng, ty, bs)
+    hy, oy = both(y, ty, hip, oracle)
+    op = ["add", "subtract", "multiply", "max", "less", "equal"][int(rng.integers(0, 6))]
+    assert_bits_equal(getattr(Nx, op)(hx, hy), getattr(Nx, op)(ox, oy), f"{op} {what} {bs}")
+    to = ["f32", "bf16", "s32", "u8", "f64", "s64"][int(rng.integers(0, 6))]
+    try:
+        want = Nx.as_type(ox, to)
+    except Exception as e:
+        assert "overflows" in str(e)
+    else:
+        assert_bits_equal(Nx.as_type(hx, to), want, f"as_type {what} -> {to}")
+    # reductions over a random axis set
+    axes = sorted(rng.choice(rank, size=int(rng.integers(1, rank + 1)), replace=False).tolist())
+    assert_bits_equal(Nx.reduce_max(hx, axes=axes), Nx.reduce_max(ox, axes=axes), f"reduce_max {what}{axes}")
+    assert_bits_equal(Nx.reduce_min(hx, axes=axes, keep_axes=True), Nx.reduce_min(ox, axes=axes, keep_axes=True), f"reduce_min {what}{axes}")
+    if T.is_integer(T.normalize(ty)):
+        assert_bits_equal(Nx.sum(hx, axes=axes), Nx.sum(ox, axes=axes), f"sum {what}{axes}")
+    axis = int(axes[-1])
+    assert_bits_equal(Nx.argmax(hx, axis=axis), Nx.argmax(ox, axis=axis), f"argmax {what}{axis}")
+    assert_bits_equal(Nx.argmin(hx, axis=None, tie_break="high", type="s64"), Nx.argmin(ox, axis=None, tie_break="high", type="s64"), f"argmin {what} flat")
+    # copies
+    perm = rng.permutation(rank).tolist()
+    assert_bits_equal(Nx.transpose(hx, perm), Nx.transpose(ox, perm), f"transpose {what}{perm}")
+    starts = [int(rng.integers(0, d)) for d in shape]
+    lengths = [int(rng.integers(1, d - s + 1)) for d, s in zip(shape, starts)]
+    assert_bits_equal(Nx.slice(hx, starts, lengths), Nx.slice(ox, starts, lengths), f"slice {what}{starts}{lengths}")
+    n = shape[axis]
+    idx = rng.integers(0, n, size=(int(rng.choice([1, 7, 300])),)).astype(np.int64)
+    hi_, oi_ = both(idx, "s64", hip, oracle)
+    assert_bits_equal(Nx.take(hx, hi_, axis=axis), Nx.take(ox, oi_, axis=axis), f"take {what} axis {axis}")
+
+
+DOT_BIG_MN = [1, 16, 33, 64, 100, 128, 192, 256, 300, 512, 768, 1000, 1024, 1536, 2048, 3072, 4096, 11008]
+DOT_BIG_K = [64, 128, 136, 512, 784, 1000, 1024, 2048, 4096, 8192, 11008]
+
+
+@pytest.mark.parametrize("case", range(60))
+def test_dot_on_large_random_shapes_against_f64_blas(case, hip):
+    """The tile rules of the contraction (256 x 256, 256 x 128, 128 x 128 and 64 x 64 two-group tiles, K in splits, K
+    extended by zeros, few rows, few columns) at the sizes that select them.  Operands hold small integers, so every
+    partial sum is exact in f32 / s32 and in the f64 product the host's BLAS computes: the device must match it bit for
+    bit whatever the order of its additions (bf16 results by truncation, f16 to nearest)."""
+    from support import from_numpy
+    rng = np.random.default_rng(seed_of("dot-large", case + OFFSET))
+    while True:
+        M, N, K = int(rng.choice(DOT_BIG_MN)), int(rng.choice(DOT_BIG_MN)), int(rng.choice(DOT_BIG_K))
+        batch = int(rng.choice([1, 1, 1, 2, 4]))
+        if 50_000_000 <= batch * M * N * K <= 9_000_000_000 and batch * (M + N) * K <= 200_000_000 and batch * M * N <= 40_000_000:
+            break
+    ty, out = [("s8", "s32"), ("bf16", None), ("bf16", "f32"), ("f16", None), ("f32", None), ("s8", "s32"), ("bf16", None)][int(rng.integers(0, 7))]
+    lk, rk = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))  # K-inner (True) or K-outer operand
+    span = 127 if ty == "s8" else 3
+    a = rng.integers(-span, span + 1, size=(batch, M, K)).astype(np.int8)
+    b = rng.integers(-span, span + 1, size=(batch, K, N)).astype(np.int8)
+    want = np.matmul(a.astype(np.float64), b.astype(np.float64))  # exact: every sum is far below 2^53
+
+    def raw(v):
+        if ty == "s8":
+            return v
+        if ty == "bf16":
+            return (v.astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+        return v.astype(np.float16 if ty == "f16" else np.float32)
+
+    la = a if lk else np.ascontiguousarray(a.transpose(0, 2, 1))
+    lb = b if not rk else np.ascontiguousarray(b.transpose(0, 2, 1))
+    c1, c2 = [2] if lk else [1], [2] if rk else [1]
+    kw = {"out_type": out} if out else {}
+    got = Nx.dot(from_numpy(raw(la), ty, hip), c1, [0], from_numpy(raw(lb), ty, hip), c2, [0], **kw)
+    res = hip.to_numpy(got)
+    what = f"dot {ty}->{out or ty} batch {batch} {M}x{N}x{K} {'k-inner' if lk else 'k-outer'} {'k-inner' if rk else 'k-outer'}"
+    out_ty = out or ty
+    if out_ty == "s32":
+        expect = want.astype(np.int64).astype(np.int32)
+    elif out_ty == "bf16":
+        expect = (want.astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    elif out_ty == "f16":
+        with np.errstate(over="ignore"):
+            expect = want.astype(np.float32).astype(np.float16)
+    else:
+        expect = want.astype(np.float32)
+    assert res.shape == expect.shape, what
+    same = res.view(np.uint8) == expect.view(np.uint8)
+    assert same.all(), f"{what}: {int((~same).sum())} bytes differ"
