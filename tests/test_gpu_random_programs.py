@@ -113,3 +113,41 @@ def test_random_program_has_the_same_bits_however_it_is_grouped(case, hip):
             assert_bits_equal(g, w, f"planned; {what}")
     finally:
         set_mode("interpreted")
+
+
+@pytest.mark.parametrize("case", range(40))
+def test_random_program_replays_from_a_captured_graph(case, hip):
+    """The same programs recorded into a graph (node by node, or as compiled groups) and replayed: with the captured
+    tensors, with new values, and back, eager work and synchronisations in between; every replay against the function run
+    outside the graph."""
+    from nx_amd.backend import fused_mode as set_mode, sync
+    rng = np.random.default_rng(seed_of("program-graph", case + OFFSET))
+    full = LEAD[int(rng.integers(0, len(LEAD)))] + (int(rng.choice(LAST)),)
+    n_inputs = int(rng.integers(1, 4))
+    shapes_types = [(full if i == 0 else broadcastable(rng, full), ["f32", "f32", "bf16", "f16"][int(rng.integers(0, 4))]) for i in range(n_inputs)]
+    args = [operand(rng, ty, sh, hip) for sh, ty in shapes_types]
+    fresh = [operand(rng, ty, sh, hip) for sh, ty in shapes_types]
+    steps, fn = make_program(rng, n_inputs)
+    fuse = [False, True, "compiled"][int(rng.integers(0, 3))]
+    what = f"case {case + OFFSET}: fuse={fuse} {[(tuple(a.shape), a.type) for a in args]} {steps}"
+    try:
+        plain = defn.compile(fn, *args)
+        want_args, want_fresh = plain(*args), plain(*fresh)
+    except (ValueError, TypeError) as e:
+        pytest.skip(f"the program does not type-check: {e}")
+    set_mode("compiled")
+    captured = None
+    try:
+        compiled = defn.compile(fn, *args, fuse=fuse)
+        compiled(*args)  # (a program first met while capturing would run interpreted: compile it beforehand)
+        captured = compiled.capture(*args)
+        for given, want in ((args, want_args), (fresh, want_fresh), (args, want_args)):
+            got = captured(*given)
+            for g, w in zip(got, want):
+                assert_bits_equal(g, w, f"replay; {what}")
+            plain(*fresh)
+            sync()
+    finally:
+        if captured is not None:
+            captured.destroy()
+        set_mode("interpreted")
