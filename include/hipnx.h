@@ -230,7 +230,9 @@ int hipnx_reduce_static(hipnx_ctx *ctx, int op, int in_dt, int out_dt, int64_t o
 
 /* replaces: argmax / argmin (nx/lib/nx/backend.ex:93-94; oracle binary_backend.ex:1393-1431).
  * Same view.  tie LOW = first index of the extreme, HIGH = last; any NaN wins and the last
- * NaN's index is returned.  out_dt is an integer type. */
+ * NaN's index is returned.  out_dt is an integer type.  An axis of 2^31 positions or more is searched in
+ * chunks (outer == 1: the flattened tensor, or the first axis); under more than one outer index such an axis
+ * is refused with HIPNX_EUNSUPPORTED. */
 int hipnx_argreduce(hipnx_ctx *ctx, int op, int tie, int in_dt, int out_dt, int64_t outer,
                     int64_t red, int64_t inner, const hipnx_buf *in, hipnx_buf *out);
 
