@@ -140,3 +140,28 @@ def test_argmax_down_an_axis_of_more_than_2_to_the_31(hip):
         assert int(hip.to_numpy(Nx.argmin(f, tie_break=tie, type="s64"))) == 2 ** 31 + 12345
     del f
     _release()
+
+
+@pytest.mark.parametrize("layout", ["k-inner", "k-outer"])
+def test_dot_with_an_operand_past_32_bit_offsets(layout, hip):
+    """A bf16 operand of 4.3 GB (its last rows start past byte 2^32) against 256 columns: operands of small integers,
+    so every sum is exact; sampled rows of the result against the same rows computed on the host."""
+    from support import from_numpy
+    M, K, N = 2 ** 16 + 16, 2 ** 15 + 128, 256
+    shape = (M, K) if layout == "k-inner" else (K, M)
+    m_axis, k_axis = (0, 1) if layout == "k-inner" else (1, 0)
+    mk = Nx.add(Nx.iota(shape, type="s32", axis=m_axis, backend=hip), Nx.iota(shape, type="s32", axis=k_axis, backend=hip))
+    a = Nx.as_type(Nx.subtract(Nx.remainder(mk, 5), 2), "bf16")  # a[m, k] = (m + k) mod 5 - 2
+    del mk
+    _release()
+    k = np.arange(K, dtype=np.int64)
+    b_host = ((3 * k[:, None] + np.arange(N)[None, :]) % 7 - 3).astype(np.float32)  # b[k, n]
+    b = from_numpy((b_host.view(np.uint32) >> 16).astype(np.uint16), "bf16", hip)
+    got = Nx.dot(a, [k_axis], b, [0], out_type="f32")
+    assert got.shape == (M, N)
+    rows = [0, 1, 32767, 32768, 65535, 65536, M - 1]
+    for m in rows:
+        want = (((m + k) % 5 - 2).astype(np.float64) @ b_host.astype(np.float64)).astype(np.float32)
+        np.testing.assert_array_equal(hip.to_numpy(Nx.slice(got, [m, 0], [1, N]))[0], want, f"row {m}")
+    del a, b, got
+    _release()
