@@ -165,3 +165,36 @@ def test_dot_with_an_operand_past_32_bit_offsets(layout, hip):
         np.testing.assert_array_equal(hip.to_numpy(Nx.slice(got, [m, 0], [1, N]))[0], want, f"row {m}")
     del a, b, got
     _release()
+
+
+@pytest.mark.parametrize("mode", ["interpreted", "compiled"])
+def test_fused_group_past_32_bit_indices(mode, hip):
+    """A fused element-wise group over 2^32 + 4099 bf16 elements, and one with its row reduction over {65537, 65600}."""
+    from nx_amd import defn
+    from nx_amd.backend import fused_mode as set_mode
+    n = 2 ** 32 + 4099
+    x = Nx.as_type(Nx.iota((n,), type="u8", backend=hip), "bf16")  # i mod 256, exact in bf16
+    set_mode(mode)
+    try:
+        f = defn.compile(lambda t: Nx.multiply(Nx.add(t, 1.0), 0.5), x, fuse=True)
+        assert f.fused_groups == 1
+        y = f(x)
+        for start in (0, 2 ** 32 - 500, n - 1000):
+            idx = np.arange(start, start + 1000, dtype=np.int64)
+            want = (((idx % 256).astype(np.float32) + 1.0) * 0.5)
+            want = (want.view(np.uint32) >> 16).astype(np.uint16)  # bf16 by truncation (every value here is exact anyway)
+            np.testing.assert_array_equal(hip.to_numpy(Nx.slice(y, [start], [1000])), want, f"window at {start}")
+        del y, x
+        _release()
+        rows, cols = 65537, 65600
+        m = Nx.as_type(Nx.iota((rows, cols), type="u8", backend=hip), "f32")
+        g = defn.compile(lambda t: Nx.sum(Nx.multiply(t, 2.0), axes=[1]), m, fuse=True)
+        got = hip.to_numpy(g(m))
+        start = (np.arange(rows, dtype=np.int64) * cols) % 256
+        for r in (0, 1, 300, rows - 2, rows - 1):
+            want = 2.0 * (np.arange(start[r], start[r] + cols, dtype=np.int64) % 256).sum()
+            assert got[r] == np.float32(want), f"row {r}"
+        del m
+        _release()
+    finally:
+        set_mode("interpreted")
