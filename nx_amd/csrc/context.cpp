@@ -4,6 +4,7 @@
 // explicit, idempotent deallocation that reports :ok / :already_deallocated
 // (torchx/c_src/torchx_nif_util.h:66-111, torchx/test/torchx/device_test.exs:30-37) and a
 // use-after-free that is an error, not a crash (exla/test/exla/backend_test.exs:48-50).
+#include <chrono>
 #include <cstdlib>
 #include <cstring>
 #include <functional>
@@ -92,10 +93,32 @@ int pool_alloc(hipnx_ctx *ctx, size_t bytes, void **ptr_out, size_t *cap_out) {
       // give cached blocks back and retry once
       (void)hipGetLastError();
       (void)hipStreamSynchronize(ctx->stream);
-      for (auto &kv : ctx->pool) (void)hipFree(kv.second);
+      int refused = 0;
+      hipError_t first_refusal = hipSuccess;
+      for (auto &kv : ctx->pool) {
+        const hipError_t f = hipFree(kv.second);
+        if (f != hipSuccess) {
+          if (!refused++) first_refusal = f;
+          (void)hipGetLastError();
+        }
+      }
+      const size_t handed_back = ctx->pool.size();
       ctx->pool.clear();
       ctx->pooled = 0;
       e = hipMalloc(&ptr, cap);
+      // hipFree returns before the driver has the memory back (observed: a third of a second after freeing 30 GiB): give
+      // it up to a second, as long as what it reports free is short of the request
+      for (int spin = 0; e == hipErrorOutOfMemory && handed_back > 0 && spin < 50; spin++) {
+        (void)hipGetLastError();
+        std::this_thread::sleep_for(std::chrono::milliseconds(20));
+        e = hipMalloc(&ptr, cap);
+      }
+      if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return set_error(e == hipErrorOutOfMemory ? HIPNX_ENOMEM : HIPNX_EHIP,
+                         "HIP error %d (%s) in hipMalloc of %zu bytes, after %zu pooled blocks went back to the device (hipFree refused %d of them, first with error %d)",
+                         (int)e, hipGetErrorString(e), cap, handed_back, refused, (int)first_refusal);
+      }
     }
     if (e != hipSuccess) return hip_fail(e, "hipMalloc");
   }

@@ -143,3 +143,36 @@ def test_host_transfers_of_every_staging_shape(nbytes, hip):
         tensors = [from_numpy(p, "u8", hip) for p in parts]
         for p, x in zip(parts, tensors):
             assert np.array_equal(hip.to_numpy(x), p)
+
+
+def test_out_of_memory_is_an_error_and_the_pool_gives_way(hip):
+    """A request the device cannot meet fails with ENOMEM and leaves the context usable; blocks that the pool still
+    holds are handed back to the device before a large request is refused."""
+    import gc
+    from nx_amd import backend as B
+    from nx_amd._lib import ENOMEM, HipNxError
+
+    def device_memory():
+        free, total = C.c_size_t(), C.c_size_t()
+        assert C.CDLL("libamdhip64.so").hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+        return free.value, total.value
+
+    Nx.tensor([0], backend=hip)  # (the context exists)
+    _, total = device_memory()
+    with pytest.raises(HipNxError) as err:
+        Nx.iota((total + 100 * 2 ** 30,), type="u8", backend=hip)  # more than the part has
+    assert err.value.status == ENOMEM
+    assert Nx.to_flat_list(Nx.add(Nx.tensor([1, 2, 3], backend=hip), 1)) == [2, 3, 4]
+    # the pool keeps up to 32 GiB of freed blocks (HIPNX_POOL_MAX_MB): park 30 GiB there, then ask for 10 GiB more than
+    # the device has free beside them
+    held = [Nx.iota((10 * 2 ** 30,), type="u8", backend=hip) for _ in range(3)]
+    del held
+    gc.collect()
+    assert B.mem_stats()["pooled"] >= 30 * 2 ** 30
+    free, _ = device_memory()
+    n = free + 10 * 2 ** 30
+    c = Nx.iota((n,), type="u8", backend=hip)  # fits only once the pool has let go of its blocks
+    assert B.mem_stats()["pooled"] < 30 * 2 ** 30
+    assert int(hip.to_numpy(Nx.slice(c, [n - 1], [1]))[0]) == (n - 1) % 256
+    del c
+    gc.collect()
