@@ -26,7 +26,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_HBM_GBS = 8000.0
-PEAK = {"bf16": 2500.0, "f16": 2500.0, "s8": 5000.0, "f32": 157.3}  # dense MFMA TFLOP/s (TOP/s)
+PEAK = {"bf16": 2500.0, "f16": 2500.0, "s8": 5000.0, "f32": 157.3, "f64": 78.6}  # dense MFMA TFLOP/s (TOP/s)
 
 # HBM bytes per launch of the headline dot kernel come from two counter runs of this file
 # (`rocprofv3 --pmc FETCH_SIZE`, then `--pmc WRITE_SIZE`, with --calibrate); the summary of those runs
@@ -322,10 +322,14 @@ def main():
             _, ms = tstat(dot_rot, steps, warm, msettle)
             entry("dot_bf16_4096_rotated", flop, "TFLOP/s", ms, PEAK["bf16"], "mfma", "mfma_bf16")
             del nxt
-            fa, fb = W.dense_gemm_f32()
-            fa, fb = put(fa, "f32"), put(fb, "f32")
+            fa_np, fb_np = W.dense_gemm_f32()
+            fa, fb = put(fa_np, "f32"), put(fb_np, "f32")
             _, ms = tstat(lambda: Nx.dot(fa, fb), steps, warm, msettle)
             entry("dot_f32_2048", 2.0 * 2048 ** 3, "TFLOP/s", ms, PEAK["f32"], "mfma", "mfma_f32")
+            da, db = put(fa_np.astype(np.float64), "f64"), put(fb_np.astype(np.float64), "f64")
+            _, ms = tstat(lambda: Nx.dot(da, db), steps, warm, msettle)
+            entry("dot_f64_2048", 2.0 * 2048 ** 3, "TFLOP/s", ms, PEAK["f64"], "mfma")
+            del da, db
             sa, sb = W.dense_gemm_s8()
             sa, sb = put(sa, "s8"), put(sb, "s8")
             _, ms = tstat(lambda: Nx.dot(sa, sb, out_type="s32"), steps, warm, msettle)

@@ -241,9 +241,10 @@ int hipnx_argreduce(hipnx_ctx *ctx, int op, int tie, int in_dt, int out_dt, int6
  * torchx/c_src/torchx.cpp:844-890 tensordot).
  * out[b, m, n] = sum_k l[b, m, k] * r[b, n, k]; l is [batch, M, K] (HIPNX_K_INNER) or
  * [batch, K, M] (HIPNX_K_OUTER), r is [batch, N, K] or [batch, K, N]; out is [batch, M, N] in
- * out_dt (f32 accumulation for f16/bf16/f32 operands, exact s32 for s8, then one encode; f64, wider integers and
- * mixed operand types accumulate in f64 / wrapping 64-bit integers over k in order, as do a handful of outputs over
- * a long K -- the dot of two vectors -- whose segments of K are summed in f64).
+ * out_dt (f32 accumulation for f16/bf16/f32 operands, exact s32 for s8, f64 accumulation on the matrix cores for
+ * f64 operands whose K is a multiple of 16 and whose result has 256 elements or more, then one encode; other f64
+ * shapes, wider integers and mixed operand types accumulate in f64 / wrapping 64-bit integers over k in order, as do
+ * a handful of outputs over a long K -- the dot of two vectors -- whose segments of K are summed in f64).
  * out_dt may be HIPNX_BF16_RNE (bf16 rounded to nearest even).  Any batch count is taken (beyond 65535 items in
  * several launches).  The call may take workspace from the context's pool and return it before it ends: a re-laid
  * operand whose K-outer rows are not whole 16-byte blocks, one-slab zero-extended copies of the last part of K when K

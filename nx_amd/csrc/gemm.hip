@@ -463,10 +463,10 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
     if (batch > 65535) return set_error(HIPNX_EUNSUPPORTED, "dot: more than 65535 batch items");
 
     Kb = (k_use ? k_use : K) * dtype_size(l_dt);  // what is contracted; the rows keep their pitch of K elements
-    const bool float_pair = l_dt == r_dt && (l_dt == HIPNX_BF16 || l_dt == HIPNX_F16 || l_dt == HIPNX_F32) && is_float(out_dt);
+    const bool float_pair = l_dt == r_dt && (l_dt == HIPNX_BF16 || l_dt == HIPNX_F16 || l_dt == HIPNX_F32 || l_dt == HIPNX_F64) && is_float(out_dt);
     const bool scaled = scale_mode != HIPNX_SCALE_NONE;
     const bool int8_pair = l_dt == HIPNX_S8 && r_dt == HIPNX_S8 && (scaled || !is_float(out_dt)) && K <= (1ll << 16);
-    mfma = (float_pair || int8_pair) && K > 0 && Kb % 16 == 0 && M * N >= 256;
+    mfma = (float_pair || int8_pair) && K > 0 && Kb % 16 == 0 && M * N >= 256 && (l_dt != HIPNX_F64 || Kb % SLAB == 0);  // (f64: the slab kernels only)
     if (scaled) {
       if (!(int8_pair && mfma && Kb % SLAB == 0)) return set_error(HIPNX_EUNSUPPORTED, "dot_scaled: s8 x s8 with K a multiple of 128 and at most 65536, M * N >= 256");
       if (scale_mode == HIPNX_SCALE_PER_ROW && batch != 1) return set_error(HIPNX_EUNSUPPORTED, "dot_scaled: a scale per row with more than one batch item");
@@ -560,7 +560,7 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
   const int esz = dtype_size(l_dt);
   const bool pipelined = Kb % SLAB == 0;
   // the pipelined kernel transposes K-outer operands itself when the rows come in whole blocks
-  const int row_block = esz == 1 ? 16 : (esz == 2 ? 8 : 4);
+  const int row_block = esz == 1 ? 16 : (esz == 2 ? 8 : esz == 4 ? 4 : 2);
   const bool l_relay = l_layout == HIPNX_K_OUTER && !(pipelined && M % row_block == 0);
   const bool r_relay = r_layout == HIPNX_K_OUTER && !(pipelined && N % row_block == 0);
   hipnx_buf *lt = nullptr, *rt = nullptr;
@@ -616,7 +616,8 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
         // few rows: 64-row tiles (f32: whatever its cost model below picks), except for a 2-byte K-outer operand
         // (x . W with W stored [K, N]), which only the 128-row kernels read by transposing loads
         // (64 x 4096 x 4096 bf16: 72 us on 64 x 32 tiles, 16.5 us there)
-        if (M <= 64 && l_dt != HIPNX_F32 && !(two_byte && !(l_kin && r_kin) && N >= 128)) cfg = GEMM_CFG_64x32;
+        const bool wide = l_dt == HIPNX_F32 || l_dt == HIPNX_F64;  // (an f64 slab costs the matrix pipes what an f32 one does)
+        if (M <= 64 && !wide && !(two_byte && !(l_kin && r_kin) && N >= 128)) cfg = GEMM_CFG_64x32;
         else if (t256 * 4 >= (int64_t)ctx->num_cus * 3 && big_ok) cfg = GEMM_CFG_256;
         else if (two_byte && M >= 192 && N >= 128 && t128 * batch > ctx->num_cus)
           // More 128 x 128 tiles than CUs: half-width tiles of the two-group kernel while they fit the CUs in one
@@ -636,8 +637,8 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
         int splits = 1;
         const int64_t nslab = Kb / SLAB;
         const bool splittable = (cfg == GEMM_CFG_128 || cfg == GEMM_CFG_128x32) && batch == 1 && scale_mode == HIPNX_SCALE_NONE && (M * N) % 4 == 0 &&
-                                (l_dt == HIPNX_S8 ? !is_float(out_dt) : true);
-        if (l_dt == HIPNX_F32 && cfg == GEMM_CFG_128x32) {
+                                (l_dt == HIPNX_S8 ? !is_float(out_dt) : true) && l_dt != HIPNX_F64;  // (partial results are f32 / s32)
+        if (wide && cfg == GEMM_CFG_128x32) {
           // (0.6 us per slab of a 128 x 32 tile; the split as below)
           const int64_t cus = ctx->num_cus, tiles = t128 * batch;
           double best = 10.0 + (double)((tiles + cus - 1) / cus) * (double)nslab * 0.6;
@@ -647,7 +648,7 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
               const double t = 10.0 + (double)(nslab / cand) * 0.6 + 5.0 + 2.0 * (double)cand * (double)(M * N) * 4.0 / 8.0e6;
               if (t < best) { best = t; splits = cand; }
             }
-        } else if (l_dt == HIPNX_F32) {
+        } else if (wide) {
           // An f32 slab is eight times the MFMA work of a 2-byte one (2.6 us per slab of a 128 x 128 tile, 0.55 us
           // for a 64 x 32 tile, the second pass of a split about 8 us), so a grid that leaves CUs idle is cut much
           // earlier: the cheapest, by those figures, of whole 128 x 128 tiles, K split up to 64 ways (2 slabs or
@@ -700,6 +701,7 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
             case HIPNX_BF16: st = launch_gemm_bf16(ctx, cfg, l_kin, r_kin, p, splits); break;
             case HIPNX_F16: st = launch_gemm_f16(ctx, cfg, l_kin, r_kin, p, splits); break;
             case HIPNX_F32: st = launch_gemm_f32(ctx, cfg, l_kin, r_kin, p, splits); break;
+            case HIPNX_F64: st = launch_gemm_f64(ctx, cfg, l_kin, r_kin, p, splits); break;
             default: st = launch_gemm_s8(ctx, cfg, l_kin, r_kin, p, splits); break;
           }
           if (!st) {
@@ -716,6 +718,7 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
           case HIPNX_BF16: st = launch_gemm_bf16(ctx, cfg, l_kin, r_kin, a, batch); break;
           case HIPNX_F16: st = launch_gemm_f16(ctx, cfg, l_kin, r_kin, a, batch); break;
           case HIPNX_F32: st = launch_gemm_f32(ctx, cfg, l_kin, r_kin, a, batch); break;
+          case HIPNX_F64: st = launch_gemm_f64(ctx, cfg, l_kin, r_kin, a, batch); break;
           default: st = launch_gemm_s8(ctx, cfg, l_kin, r_kin, a, batch); break;
         }
       } else {

@@ -21,6 +21,7 @@ int launch_gemm_bf16(const hipnx_ctx *ctx, int cfg, bool l_kin, bool r_kin, Gemm
 int launch_gemm_f16(const hipnx_ctx *ctx, int cfg, bool l_kin, bool r_kin, GemmArgs a, int64_t batch);
 int launch_gemm_f32(const hipnx_ctx *ctx, int cfg, bool l_kin, bool r_kin, GemmArgs a, int64_t batch);
 int launch_gemm_s8(const hipnx_ctx *ctx, int cfg, bool l_kin, bool r_kin, GemmArgs a, int64_t batch);
+int launch_gemm_f64(const hipnx_ctx *ctx, int cfg, bool l_kin, bool r_kin, GemmArgs a, int64_t batch);  // (tiles of 128 rows or fewer)
 
 template <int DT, int WM, int WN, int TM, int TN, bool LK, bool RK, int NSTAGE = 2>
 static int launch_one(const hipnx_ctx *ctx, GemmArgs a, int64_t batch) {
@@ -74,6 +75,25 @@ static int launch_pingpong128(const hipnx_ctx *ctx, GemmArgs a, int64_t batch) {
 
 template <int DT, bool LK, bool RK>
 static int launch_cfg(const hipnx_ctx *ctx, int cfg, const GemmArgs &a, int64_t batch) {
+  if constexpr (DT == HIPNX_F64) {
+    // f64 accumulators take two registers an element: wave tiles of 64 x 64 at most, on the one-group kernel (an f64
+    // slab is 4096 clocks of MFMA work, as an f32 one: the data movement beside it is a few hundred)
+    switch (cfg) {
+      case GEMM_CFG_128x32:
+        if constexpr (LK && RK) return launch_one<DT, 4, 1, 1, 1, LK, RK, 4>(ctx, a, batch);
+        else return launch_one<DT, 4, 1, 1, 1, LK, RK>(ctx, a, batch);
+      case GEMM_CFG_64x128: return launch_one<DT, 2, 2, 1, 2, LK, RK>(ctx, a, batch);
+      case GEMM_CFG_64x32:
+        if constexpr (LK && RK) return launch_one<DT, 2, 1, 1, 1, LK, RK, 6>(ctx, a, batch);
+        else return launch_one<DT, 2, 1, 1, 1, LK, RK>(ctx, a, batch);
+      default: {
+        const int64_t groups = ((a.M + 127) / 128) * ((a.N + 127) / 128) * batch;
+        if constexpr (LK && RK)
+          if (a.Kb >= 4 * SLAB && groups <= ctx->num_cus) return launch_one<DT, 2, 2, 2, 2, LK, RK, 4>(ctx, a, batch);
+        return launch_one<DT, 2, 2, 2, 2, LK, RK>(ctx, a, batch);
+      }
+    }
+  } else
   switch (cfg) {
     case GEMM_CFG_256:
       if constexpr (DT == HIPNX_BF16 || DT == HIPNX_F16 || (DT == HIPNX_S8 && LK)) {

@@ -99,6 +99,20 @@ template <> struct Mma16<HIPNX_F32> {
   }
 };
 
+// f64: a lane's 16 bytes are two consecutive k; v_mfma_f64_16x16x4_f64 takes one value per lane (k = lane / 16), so the
+// two instructions contract k = {0, 2, 4, 6} and {1, 3, 5, 7} of the 8-k step.  Its result sits differently from the
+// other types' (measured on the part): register e of lane l is row 4 e + l / 16 of the first operand, column l % 16.
+typedef double v4d __attribute__((ext_vector_type(4)));
+typedef double v2d __attribute__((ext_vector_type(2)));
+template <> struct Mma16<HIPNX_F64> {
+  typedef v4d acc_t;
+  static __device__ __forceinline__ void step(acc_t &c, const v4i &a, const v4i &b) {
+    const v2d x = __builtin_bit_cast(v2d, a), y = __builtin_bit_cast(v2d, b);
+    c = __builtin_amdgcn_mfma_f64_16x16x4f64(x[0], y[0], c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f64_16x16x4f64(x[1], y[1], c, 0, 0, 0);
+  }
+};
+
 // Swizzle of the [row][k] LDS layout: 16-byte chunk index XOR a 3-bit function of the row.  Its
 // part in the low four row bits (bit0 = r0^r2, bit1 = r1^r2, bit2 = r2^r3) is one of the maps a
 // sweep over all linear maps of those bits measured as conflict-free for the fragment read
@@ -180,6 +194,7 @@ template <int ES> struct KOuterShape;
 template <> struct KOuterShape<2> { static constexpr int KB = 8, RB = 8; };
 template <> struct KOuterShape<4> { static constexpr int KB = 4, RB = 4; };
 template <> struct KOuterShape<1> { static constexpr int KB = 4, RB = 16; };
+template <> struct KOuterShape<8> { static constexpr int KB = 2, RB = 2; };
 
 template <int ES, int ROWS, int NTHREADS>
 struct KOuterStage {
@@ -228,6 +243,13 @@ struct KOuterStage {
         for (int i = 0; i < 4; i++) {
           const v4i t = {v[p][0][i], v[p][1][i], v[p][2][i], v[p][3][i]};
           const int r = rb * 4 + i;
+          *reinterpret_cast<v4i *>(lds + r * SLAB + lds_slot(r, kb) * 16) = t;
+        }
+      } else if constexpr (ES == 8) {
+#pragma unroll
+        for (int i = 0; i < 2; i++) {  // row i: its two k of this block, 8 bytes each
+          const v4i t = {v[p][0][2 * i], v[p][0][2 * i + 1], v[p][1][2 * i], v[p][1][2 * i + 1]};
+          const int r = rb * 2 + i;
           *reinterpret_cast<v4i *>(lds + r * SLAB + lds_slot(r, kb) * 16) = t;
         }
       } else {
@@ -379,7 +401,23 @@ __device__ __forceinline__ void gemm_epilogue(typename Mma16<DT>::acc_t (&acc)[T
                                               unsigned char *wave_lds = nullptr) {
   constexpr bool int_acc = DT == HIPNX_S8;
   constexpr bool int_out = ODT < HIPNX_F16;
-  if constexpr (int_acc && ODT == HIPNX_F32) {
+  if constexpr (DT == HIPNX_F64) {
+    // f64 accumulators: register e of a lane is n = 4 e + lane / 16 (Mma16<HIPNX_F64>), one rounding to the output type
+    if constexpr (int_out) return;  // the host never pairs them
+    else {
+#pragma unroll
+      for (int i = 0; i < TM; i++) {
+        const int64_t gm = row0 + 16 * i + (lane & 15);
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            const int64_t gn = col0 + 16 * j + 4 * e + (lane >> 4);
+            if (gm < M && gn < N) store_one<double>(out, ODT, obase + gm * N + gn, acc[i][j][e]);
+          }
+      }
+    }
+  } else if constexpr (int_acc && ODT == HIPNX_F32) {
     // as_type(s32 -> f32) then multiply, each rounding once, as the two separate kernels would
     if (scale_mode == HIPNX_SCALE_NONE) return;  // the host pairs them only with a scale
     const bool vec_ok = (N % 4) == 0;
@@ -683,7 +721,8 @@ gemm_pipelined_kernel(GemmArgs a) {
   KInnerLoader<BN, NW> rload;
   if constexpr (L_KIN) lload.init(lb, a.ld_l, m0, a.M, wave, lane);
   if constexpr (R_KIN) rload.init(rb, a.ld_r, n0, a.N, wave, lane);
-  constexpr int ES = (DT == HIPNX_S8) ? 1 : (DT == HIPNX_F32 ? 4 : 2);
+  constexpr int ES = (DT == HIPNX_S8) ? 1 : (DT == HIPNX_F32 ? 4 : DT == HIPNX_F64 ? 8 : 2);
+  static_assert(DT != HIPNX_F64 || TM16 * TN16 <= 16, "f64 accumulators are two registers an element: wave tiles up to 64 x 64");
   // K-outer 1- and 2-byte operands of tiles whose k-rows span all LDS banks: DMA + transposing reads
   constexpr bool L_TR = !L_KIN && ES <= 2 && BM * ES >= 256 && (BM / 8) % NW == 0;
   constexpr bool R_TR = !R_KIN && ES <= 2 && BN * ES >= 256 && (BN / 8) % NW == 0;

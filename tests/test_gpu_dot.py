@@ -609,3 +609,30 @@ def test_a_few_vectors_against_a_matrix(S, R, K, ty, side, small_layout, hip, or
             assert_bits_equal(got, want, f"few vectors s32 {side} {big_layout}")
         else:
             check_float_dot(got, want, a64, b64, eq, K, f"few vectors {ty} {side} {small_layout} {big_layout}")
+
+
+@pytest.mark.parametrize("layout", ["nn", "nt", "tn", "tt"])
+@pytest.mark.parametrize("M,N,K", [(128, 128, 64), (256, 384, 512), (130, 70, 144), (1024, 1024, 256), (64, 2048, 1024), (33, 40, 16), (2000, 16, 4096)])
+def test_f64_contraction_on_the_matrix_cores(M, N, K, layout, hip, oracle):
+    """f64 operands whose K is a whole number of 128-byte slabs (16 elements) and whose result has 256 elements or more
+    take the MFMA f64 path (`v_mfma_f64_16x16x4_f64`, f64 accumulators): within the accumulation bound of the oracle's
+    sequential f64 sum, and exact where every partial sum is (small integers).  Other f64 shapes stay on the plain
+    kernels, which add over k in order and so match the oracle bit for bit (test_plain_kernel_on_64_tiles)."""
+    rng = np.random.default_rng(seed_of(M, N, K, layout, "f64 mfma"))
+    a_shape = (M, K) if layout[0] == "n" else (K, M)
+    b_shape = (K, N) if layout[1] == "n" else (N, K)
+    c1, c2 = [1] if layout[0] == "n" else [0], [0] if layout[1] == "n" else [1]
+    a, b = rng.standard_normal(a_shape), rng.standard_normal(b_shape)
+    ha, oa = both(a, "f64", hip, oracle)
+    hb, ob = both(b, "f64", hip, oracle)
+    got, want = Nx.dot(ha, c1, hb, c2), Nx.dot(oa, c1, ob, c2)
+    am = a if layout[0] == "n" else a.T
+    bm = b if layout[1] == "n" else b.T
+    check_float_dot(got, want, am, bm, "mk,kn->mn", K, f"f64 {M}x{N}x{K} {layout}")
+    ai, bi = rng.integers(-50, 51, size=a_shape).astype(np.float64), rng.integers(-50, 51, size=b_shape).astype(np.float64)
+    exact = (ai if layout[0] == "n" else ai.T) @ (bi if layout[1] == "n" else bi.T)
+    res = hip.to_numpy(Nx.dot(from_numpy(ai, "f64", hip), c1, from_numpy(bi, "f64", hip), c2))
+    assert np.array_equal(res, exact)
+    # an f32 result from f64 operands: one rounding of the f64 sum
+    res32 = hip.to_numpy(Nx.dot(from_numpy(ai, "f64", hip), c1, from_numpy(bi, "f64", hip), c2, out_type="f32"))
+    assert np.array_equal(res32, exact.astype(np.float32))

@@ -134,7 +134,7 @@ def test_dot_on_random_shapes_types_and_layouts(case, hip, oracle):
     while M * N * K > 40_000_000:
         M, N, K = int(rng.choice(DOT_M)), int(rng.choice(DOT_N)), int(rng.choice(DOT_K))
     batch = int(rng.choice([1, 1, 1, 2, 3]))
-    ty = ["bf16", "f16", "f32", "s8"][int(rng.integers(0, 4))]
+    ty = ["bf16", "f16", "f32", "s8", "f64"][int(rng.integers(0, 5))]
     lk, rk = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))  # K-inner (True) or K-outer operand
     if ty == "s8":
         a = rng.integers(-127, 128, size=(batch, M, K)).astype(np.int8)
@@ -230,7 +230,8 @@ def test_dot_on_large_random_shapes_against_f64_blas(case, hip):
         batch = int(rng.choice([1, 1, 1, 2, 4]))
         if 50_000_000 <= batch * M * N * K <= 9_000_000_000 and batch * (M + N) * K <= 200_000_000 and batch * M * N <= 40_000_000:
             break
-    ty, out = [("s8", "s32"), ("bf16", None), ("bf16", "f32"), ("f16", None), ("f32", None), ("s8", "s32"), ("bf16", None)][int(rng.integers(0, 7))]
+    ty, out = [("s8", "s32"), ("bf16", None), ("bf16", "f32"), ("f16", None), ("f32", None), ("s8", "s32"), ("bf16", None), ("f64", None),
+               ("f64", "f32")][int(rng.integers(0, 9))]
     lk, rk = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))  # K-inner (True) or K-outer operand
     span = 127 if ty == "s8" else 3
     a = rng.integers(-span, span + 1, size=(batch, M, K)).astype(np.int8)
@@ -242,7 +243,7 @@ def test_dot_on_large_random_shapes_against_f64_blas(case, hip):
             return v
         if ty == "bf16":
             return (v.astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
-        return v.astype(np.float16 if ty == "f16" else np.float32)
+        return v.astype(np.float16 if ty == "f16" else np.float64 if ty == "f64" else np.float32)
 
     la = a if lk else np.ascontiguousarray(a.transpose(0, 2, 1))
     lb = b if not rk else np.ascontiguousarray(b.transpose(0, 2, 1))
@@ -260,7 +261,7 @@ def test_dot_on_large_random_shapes_against_f64_blas(case, hip):
         with np.errstate(over="ignore"):
             expect = want.astype(np.float32).astype(np.float16)
     else:
-        expect = want.astype(np.float32)
+        expect = want.astype(np.float64 if out_ty == "f64" else np.float32)
     assert res.shape == expect.shape, what
     same = res.view(np.uint8) == expect.view(np.uint8)
     assert same.all(), f"{what}: {int((~same).sum())} bytes differ"
