@@ -3,7 +3,7 @@
 // events), so that a kernel's fraction of the published peak can be read beside the fraction of what
 // the part actually delivers under its power management.
 //
-//   hipnx_ceilings mfma <bf16|f16|s8|f32> <random|normal|zero> [ms]
+//   hipnx_ceilings mfma <bf16|f16|s8|f32|f64> <random|normal|zero> [ms]
 //       an MFMA-only loop (the 16x16 forms the contraction kernel uses, 8 waves per CU, 32
 //       independent accumulator tiles per wave, operands in registers, no memory traffic) launched
 //       back to back for `ms` milliseconds; throughput is reported for the first 2 ms, for each fifth
@@ -100,6 +100,33 @@ __global__ void __launch_bounds__(512) mfma_loop(const v4i *src, float *out, int
     }
     for (int i = 0; i < 4; i++) for (int j = 0; j < 8; j++) for (int q = 0; q < 4; q++) sum += acc[i][j][q];
   }
+  out[blockIdx.x * 512 + tid] = sum;
+  if (blockIdx.x == 8 && tid == 0) {
+    g_clk[0] = clock64() - c0;
+    g_clk[1] = wall_clock64() - w0;
+  }
+}
+
+// The f64 form: 4 x 4 accumulator tiles per wave (the f64 contraction kernel's wave tile: f64 accumulators take two
+// registers an element), one trip = 8 k x 16 tiles = 128 v_mfma_f64_16x16x4_f64.
+typedef __attribute__((ext_vector_type(4))) double v4d;
+__global__ void __launch_bounds__(512) mfma_loop_f64(const double *src, double *out, int iters) {
+  const int tid = threadIdx.x;
+  double pa[8], pb[8];
+  for (int q = 0; q < 8; q++) pa[q] = src[(size_t)(blockIdx.x * 512 + tid) * 16 + q], pb[q] = src[(size_t)(blockIdx.x * 512 + tid) * 16 + 8 + q];
+  const unsigned long long c0 = clock64(), w0 = wall_clock64();
+  v4d acc[4][4];
+  for (int i = 0; i < 4; i++) for (int j = 0; j < 4; j++) for (int q = 0; q < 4; q++) acc[i][j][q] = 0;
+  for (int it = 0; it < iters; it++) {
+#pragma unroll
+    for (int ks = 0; ks < 8; ks++)
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(pb[(ks + j) & 7], pa[(ks + i) & 7], acc[i][j], 0, 0, 0);
+  }
+  double sum = 0;
+  for (int i = 0; i < 4; i++) for (int j = 0; j < 4; j++) for (int q = 0; q < 4; q++) sum += acc[i][j][q];
   out[blockIdx.x * 512 + tid] = sum;
   if (blockIdx.x == 8 && tid == 0) {
     g_clk[0] = clock64() - c0;
@@ -242,7 +269,40 @@ static int timed_chunks(F &&launch, int chunks, int per_chunk, std::vector<float
   return 0;
 }
 
+static int run_mfma_f64(const char *data, double want_ms) {
+  const size_t n = (size_t)256 * 512 * 16;
+  std::vector<double> h(n);
+  srand(1);
+  auto uni = [] { return rand() / (double)RAND_MAX; };
+  for (size_t i = 0; i < n; i++)
+    h[i] = !strcmp(data, "random") ? uni() * 2 - 1 : !strcmp(data, "normal") ? sqrt(-2 * log((rand() + 1.0) / (RAND_MAX + 2.0))) * cos(6.283185307179586 * uni()) / 64 : 0.0;
+  double *d, *o;
+  CK(hipMalloc(&d, n * 8));
+  CK(hipMalloc(&o, 256 * 512 * 8));
+  CK(hipMemcpy(d, h.data(), n * 8, hipMemcpyHostToDevice));
+  const int iters = 12;  // about 100 us per launch
+  const double flop = 256.0 * 8 * iters * 128 * (2.0 * 16 * 16 * 4);
+  auto launch = [&] { hipLaunchKernelGGL(mfma_loop_f64, dim3(256), dim3(512), 0, 0, d, o, iters); };
+  std::vector<float> probe;
+  if (timed_chunks(launch, 1, 5, probe)) return 1;
+  const double launch_ms = probe[0] / 5;
+  const int per_chunk = std::max(1, (int)(2.0 / launch_ms));
+  const int chunks = std::max(5, (int)(want_ms / (per_chunk * launch_ms)));
+  CK(hipDeviceSynchronize());
+  std::vector<float> ms;
+  if (timed_chunks(launch, chunks, per_chunk, ms)) return 1;
+  unsigned long long c[2];
+  CK(hipMemcpyFromSymbol(c, HIP_SYMBOL(g_clk), sizeof(c)));
+  auto rate = [&](int a, int b) { double t = 0; for (int i = a; i < b; i++) t += ms[i]; return flop * per_chunk * (b - a) / t / 1e9; };
+  printf("{\"kind\": \"mfma\", \"dtype\": \"f64\", \"operands\": \"%s\", \"unit\": \"TFLOP/s\", \"first_2ms\": %.1f, \"fifths\": [", data, rate(0, 1));
+  for (int q = 0; q < 5; q++) printf("%s%.1f", q ? ", " : "", rate(chunks * q / 5, chunks * (q + 1) / 5));
+  printf("], \"sustained\": %.1f, \"launch_us\": %.1f, \"clock_mhz_last_launch\": %.0f, \"clocks_per_instruction\": %.2f}\n", rate(chunks * 4 / 5, chunks),
+         1000 * ms[chunks - 1] / per_chunk, c[0] / (c[1] / 100.0), (double)c[0] / ((double)iters * 128));
+  return 0;
+}
+
 static int run_mfma(const char *type, const char *data, double want_ms) {
+  if (!strcmp(type, "f64")) return run_mfma_f64(data, want_ms);
   const int kind = !strcmp(type, "bf16") ? K_BF16 : !strcmp(type, "f16") ? K_F16 : !strcmp(type, "s8") ? K_S8 : !strcmp(type, "f32") ? K_F32 : -1;
   if (kind < 0) { fprintf(stderr, "unknown type %s\n", type); return 2; }
   const size_t nwords = (size_t)256 * 512 * 12 * 4;  // v4i per lane x 12
@@ -414,7 +474,7 @@ int main(int argc, char **argv) {
   if (argc >= 3 && !strcmp(argv[1], "ingest")) return run_ingest(argv[2], argc > 3 ? atof(argv[3]) : 100.0);
   if (argc >= 4 && !strcmp(argv[1], "mfma")) return run_mfma(argv[2], argv[3], argc > 4 ? atof(argv[4]) : 300.0);
   if (argc >= 3 && !strcmp(argv[1], "stream")) return run_stream(argv[2], argc > 3 ? (size_t)atol(argv[3]) : 2048, argc > 4 ? atof(argv[4]) : 100.0);
-  fprintf(stderr, "usage: hipnx_ceilings mfma <bf16|f16|s8|f32> <random|normal|zero> [ms]\n       hipnx_ceilings stream <read|write|copy> [MiB] [ms]\n"
+  fprintf(stderr, "usage: hipnx_ceilings mfma <bf16|f16|s8|f32|f64> <random|normal|zero> [ms]\n       hipnx_ceilings stream <read|write|copy> [MiB] [ms]\n"
                   "       hipnx_ceilings ingest <l2|llc|hbm> [ms]\n       hipnx_ceilings weights <work-groups> <none|interleaved|first> [KiB of rows]\n");
   return 2;
 }
