@@ -110,6 +110,7 @@ def measured_ceilings(ms=250):
         return out
     runs = [("mfma_bf16", ["mfma", "bf16", "normal", str(ms)]), ("mfma_f16", ["mfma", "f16", "normal", str(ms)]),
             ("mfma_s8", ["mfma", "s8", "normal", str(ms)]), ("mfma_f32", ["mfma", "f32", "normal", str(ms)]),
+            ("mfma_f64", ["mfma", "f64", "normal", str(ms)]),
             # 1 GiB per buffer: the size of the suite's 16384^2 f32 tensors (a 2 GiB stream keeps less of itself in
             # the 256 MB last-level cache and reads a few per cent lower)
             ("stream_read", ["stream", "read", "1024", "100"]), ("stream_write", ["stream", "write", "1024", "100"]),
@@ -328,7 +329,7 @@ def main():
             entry("dot_f32_2048", 2.0 * 2048 ** 3, "TFLOP/s", ms, PEAK["f32"], "mfma", "mfma_f32")
             da, db = put(fa_np.astype(np.float64), "f64"), put(fb_np.astype(np.float64), "f64")
             _, ms = tstat(lambda: Nx.dot(da, db), steps, warm, msettle)
-            entry("dot_f64_2048", 2.0 * 2048 ** 3, "TFLOP/s", ms, PEAK["f64"], "mfma")
+            entry("dot_f64_2048", 2.0 * 2048 ** 3, "TFLOP/s", ms, PEAK["f64"], "mfma", "mfma_f64")
             del da, db
             sa, sb = W.dense_gemm_s8()
             sa, sb = put(sa, "s8"), put(sb, "s8")
