@@ -689,7 +689,12 @@ __device__ __forceinline__ void wait_vmcnt() {  // s_waitcnt vmcnt(N), other cou
 }
 
 template <int DT, int WM, int WN, int TM, int TN, bool L_KIN, bool R_KIN, int NSTAGE = 2, bool EARLY = false>
-__global__ void __launch_bounds__(WM *WN * 64)
+// (f64: at least two waves per SIMD, i.e. at most 256 registers and all of them VGPRs.  With the 512 that a work-group
+// of four waves may have, the compiler keeps some accumulators in AGPRs and moves them to and fro inside the K loop --
+// 128 copies per slab beside 64 MFMAs, each waiting for the MFMA that last wrote its source: 2048^3 404 -> 329 us,
+// 4096^3 2.8 -> 2.0 ms.  f64 with both operands K-outer does not fit 256 registers and would spill; the f32 kernels
+// lose by the same limit, 2048^3 152 -> 167 us.)
+__global__ void __launch_bounds__(WM *WN * 64) __attribute__((amdgpu_waves_per_eu(DT == HIPNX_F64 && (L_KIN || R_KIN) ? 2 : 1)))
 gemm_pipelined_kernel(GemmArgs a) {
   typedef typename Mma16<DT>::acc_t acc_t;
   constexpr int NW = WM * WN, NT = NW * 64;
