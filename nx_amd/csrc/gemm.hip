@@ -665,9 +665,11 @@ static int dot_impl(hipnx_ctx *ctx, int l_dt, int r_dt, int out_dt, int64_t batc
                 const double t = 10.0 + (double)(nslab / cand) * 2.6 + split_cost(cand);
                 if (t < best) { best = t; splits = cand; }
               }
-            // up to 64 rows: tiles of 64 x 128, half the MFMA work per slab of a tile that would be half empty
-            if (M <= 64) {
-              const int64_t tn = (N + 127) / 128 * batch;
+            // tiles of 64 x 128, half the MFMA work per slab: up to 64 rows a 128-row tile would be half empty, and a grid
+            // of 128 x 128 tiles whose last round leaves most CUs idle ends sooner in halves (3072^3: 576 tiles in three
+            // rounds, 1152 in five of half the length)
+            {
+              const int64_t tn = ((M + 63) / 64) * ((N + 127) / 128) * batch;
               const double whole = 10.0 + rounds(tn) * (double)nslab * 1.3;
               if (whole < best) { best = whole; cfg = GEMM_CFG_64x128; splits = 1; }
               if (splittable)
