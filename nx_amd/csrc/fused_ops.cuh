@@ -211,6 +211,28 @@ __device__ __forceinline__ float int_unary(float x) {
   return __uint_as_float((uint32_t)unary_apply<OP, int64_t>(UNS ? (int64_t)a : (int64_t)(int32_t)a, 32));
 }
 
+// A program that relabels bits or computes on integers can look at the bits of a float it made.  The separate kernels
+// store every NaN they compute as the one quiet NaN (0x7FC00000), so such a program does the same after each float
+// instruction; bits that only pass through (an input, a BITCAST) stay as they are, there as here.
+template <typename P>
+constexpr bool bits_are_observed() {
+  for (int i = 0; i < P::n_instr; i++)
+    if (P::kind[i] == HIPNX_FUSED_BITCAST || (P::flags[i] & HIPNX_FUSED_FLAG_INT) != 0) return true;
+  return false;
+}
+// the result is the bits of the last instruction when that is a BITCAST to f32 (any NaN pattern leaves as it came)
+template <typename P>
+constexpr bool result_is_relabelled_bits() {
+  return P::out_dt == HIPNX_U32 || P::out_dt == HIPNX_S32 || (P::out_dt == HIPNX_F32 && P::kind[P::n_instr - 1] == HIPNX_FUSED_BITCAST);
+}
+
+// Where integer bits become a float (a BITCAST, a conversion of a computed integer) the compiler is made to forget how
+// the bits were computed.  Knowing it, this compiler (a) takes an integer with few significant bits for exactly
+// convertible to f16 whatever its size and drops the rounding to f16 -- (x << 24) as f16 then stays finite -- and (b) turns
+// an arithmetic shift by 24 whose result a float instruction reads into that instruction's byte select, which cannot
+// sign-extend: the bits of -3 relabelled as f32 (a NaN) minus 1.0 came out as -1.0.
+__device__ __forceinline__ void forget_provenance(float &x) { asm volatile("" : "+v"(x)); }
+
 // instructions PC .. END-1
 template <typename P, int PC, int END>
 __device__ __forceinline__ void static_steps(KernArgs a, const int64_t (&row)[FV], const int64_t (&col)[FV], Vecs &acc, Saved &S,
@@ -254,8 +276,27 @@ __device__ __forceinline__ void static_steps(KernArgs a, const int64_t (&row)[FV
 #pragma unroll
       for (int u = 0; u < FV; u++)
 #pragma unroll
-        for (int e = 0; e < FE; e++) acc[u][e] = element_to_f32(__float_as_uint(acc[u][e]), op);
-    }  // a float AS_TYPE is the rounding below; a BITCAST changes nothing in the registers
+        for (int e = 0; e < FE; e++) {
+          forget_provenance(acc[u][e]);
+          acc[u][e] = element_to_f32(__float_as_uint(acc[u][e]), op);
+        }
+    } else if constexpr (kind == HIPNX_FUSED_BITCAST) {  // changes nothing in the registers
+#pragma unroll
+      for (int u = 0; u < FV; u++)
+#pragma unroll
+        for (int e = 0; e < FE; e++) forget_provenance(acc[u][e]);
+    }  // a float AS_TYPE is the rounding below
+    constexpr bool computed = kind == HIPNX_FUSED_UNARY || kind == HIPNX_FUSED_BINARY || kind == HIPNX_FUSED_SELECT || kind == HIPNX_FUSED_AS_TYPE ||
+                              (kind == HIPNX_FUSED_SET && (src == HIPNX_FUSED_SRC_ROWSTAT || src == HIPNX_FUSED_SRC_CARRY));
+    if constexpr (dt == HIPNX_F32 && computed && bits_are_observed<P>()) {
+#pragma unroll
+      for (int u = 0; u < FV; u++)
+#pragma unroll
+        for (int e = 0; e < FE; e++) {  // (tested on the bits: a float comparison that selects between floats is folded away)
+          const uint32_t b = __float_as_uint(acc[u][e]);
+          acc[u][e] = __uint_as_float((b & 0x7FFFFFFFu) > 0x7F800000u ? 0x7FC00000u : b);
+        }
+    }
     if constexpr (dt == HIPNX_BF16 || dt == HIPNX_F16) {
 #pragma unroll
       for (int u = 0; u < FV; u++)
@@ -276,7 +317,7 @@ struct RunStatic {
   }
   // a u32 / s32 result leaves as the bits it is held as
   static __device__ __forceinline__ int out_dt(KernArgs) { return P::out_dt; }
-  static constexpr bool raw_out = P::out_dt == HIPNX_U32 || P::out_dt == HIPNX_S32;
+  static constexpr bool raw_out = result_is_relabelled_bits<P>();
 };
 
 // ---- kernel bodies: RUN is RunStatic<P> or the interpreter of fused.hip ---------------------------
@@ -439,7 +480,7 @@ __device__ __forceinline__ void row_stage(KernArgs a, int64_t r, int lane, RowSt
       Vecs x;
       Saved S;
       static_steps<P, begin, P::n_instr>(a, row, col, x, S, stats, FE, &carry[it]);
-      if constexpr (P::out_dt == HIPNX_U32 || P::out_dt == HIPNX_S32) {
+      if constexpr (result_is_relabelled_bits<P>()) {
         uint4 *p = reinterpret_cast<uint4 *>((uint32_t *)out + r * cols + k);
         p[0] = make_uint4(__float_as_uint(x[0][0]), __float_as_uint(x[0][1]), __float_as_uint(x[0][2]), __float_as_uint(x[0][3]));
         p[1] = make_uint4(__float_as_uint(x[0][4]), __float_as_uint(x[0][5]), __float_as_uint(x[0][6]), __float_as_uint(x[0][7]));

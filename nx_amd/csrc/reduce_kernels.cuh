@@ -353,7 +353,6 @@ template <typename R, typename CT, int IDT>
 static int run_reduce_t(hipnx_ctx *ctx, bool static_ws, int idt, int odt, int64_t outer, int64_t red, int64_t inner,
                         const void *in, void *out) {
   typedef typename R::acc_t acc_t;
-  const int64_t target_units = (int64_t)ctx->num_cus * 8;  // units of parallel work wanted
   // an input far larger than the 256 MB last-level cache is read with the non-temporal hint -- where a lane's vector is
   // one access (elements of 1 or 2 bytes: bf16 row sums over 16384^2 88 -> 80 us): the two 16-byte accesses of eight
   // f32 each take half of the same lines, and a line that is let go early is fetched twice (f32: 169 -> 180 us)

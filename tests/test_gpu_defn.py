@@ -15,7 +15,7 @@ from nx_amd import random as Random
 from nx_amd import _lib as L
 from nx_amd.backend import _Context, mem_stats
 from random_support import CASES, check_random_case
-from support import assert_all_close, assert_bits_equal, from_numpy, seed_of
+from support import assert_all_close, assert_bits_equal, from_numpy, raw, seed_of
 from test_defn import CHAINS, build_args, f32
 
 pytestmark = pytest.mark.gpu
@@ -530,6 +530,25 @@ def floats_to_bits_and_back(x):
     return Nx.sqrt(Nx.bitcast(sign_cleared, "f32"))
 
 
+# Where the bits of a float can be looked at, every NaN a node computes is the one quiet NaN its kernel would have stored
+# (0x7FC00000), bits that only pass through a relabelling stay as they are, and a conversion rounds however few significant
+# bits the compiler can see in the integer (each of these once came out differently from the compiled group):
+def bits_of_a_computed_nan(x):
+    return Nx.bitcast(Nx.sqrt(x), "s32")                       # sqrt of a negative number: the hardware's NaN has the sign set
+
+
+def relabelled_nan_bits(a):
+    return Nx.bitcast(Nx.negate(Nx.max(a, 0x7FFFFFFF)), "f32")  # NaN patterns with payloads: the result's last node relabels
+
+
+def shifted_integer_to_f16(a):
+    return Nx.sqrt(Nx.as_type(Nx.left_shift(a, 24), "f16"))     # eight significant bits, far beyond f16's range: infinity
+
+
+def sign_extended_byte_as_float(a):
+    return Nx.subtract(Nx.bitcast(Nx.right_shift(a, 24), "f32"), 1.0)   # negative a: the bits of a NaN
+
+
 def rand_words(rng, ty, shape, backend):
     info = np.iinfo(np.uint32 if ty == "u32" else np.int32)
     return from_numpy(rng.integers(info.min, info.max, size=shape, dtype=info.dtype, endpoint=True), ty, backend)
@@ -541,7 +560,27 @@ INT_CASES = {
     "integer_mix_s32": (integer_mix, lambda rng, b: (rand_words(rng, "s32", (8, 4096), b), rand_words(rng, "s32", (4096,), b))),
     "signed_shift_and_convert": (signed_shift_and_convert, lambda rng, b: (rand_words(rng, "s32", (40, 64), b), rand_words(rng, "s32", (40, 64), b))),
     "floats_to_bits_and_back": (floats_to_bits_and_back, lambda rng, b: (rand_float(rng, "f32", (1000, 8), b),)),
+    "bits_of_a_computed_nan": (bits_of_a_computed_nan, lambda rng, b: (rand_float(rng, "f32", (4, 64), b),)),
+    "relabelled_nan_bits": (relabelled_nan_bits, lambda rng, b: (rand_words(rng, "u32", (5, 8), b),)),
+    "shifted_integer_to_f16": (shifted_integer_to_f16, lambda rng, b: (rand_words(rng, "u32", (2, 520), b),)),
+    "sign_extended_byte_as_float": (sign_extended_byte_as_float, lambda rng, b: (rand_words(rng, "s32", (64, 8), b),)),
 }
+
+
+def test_what_a_compiled_group_sees_in_the_bits_of_a_nan(hip):
+    """The same four against what they must give, worked out here."""
+    x = from_numpy(np.array([-4.0, 4.0, -0.0, -1e-30] * 2, np.float32), "f32", hip)
+    got = raw(defn.compile(bits_of_a_computed_nan, x, fuse="compiled")(x))
+    assert got.view(np.uint32).tolist() == [0x7FC00000, 0x40000000, 0x80000000, 0x7FC00000] * 2
+    a = from_numpy(np.array([0x80000001, 0x7FFFFFFF, 5, 0xFFFFFFFF, 0x80000000, 0x80000002, 0, 9], np.uint32), "u32", hip)
+    got = raw(defn.compile(relabelled_nan_bits, a, fuse="compiled")(a))
+    assert got.view(np.uint32).tolist() == [0x7FFFFFFF, 0x80000001, 0x80000001, 1, 0x80000000, 0x7FFFFFFE, 0x80000001, 0x80000001]
+    a = from_numpy(np.array([0, 1, 2, 255, 256 + 4, 16, 64, 100], np.uint32), "u32", hip)
+    got = raw(defn.compile(shifted_integer_to_f16, a, fuse="compiled")(a))
+    assert got.view(np.uint16).tolist() == [0, 0x7C00, 0x7C00, 0x7C00, 0x7C00, 0x7C00, 0x7C00, 0x7C00]
+    a = from_numpy(np.array([-1 << 24, 3 << 24, -128 << 24, 0, 127 << 24, -5 << 24, 1 << 23, -(1 << 23)], np.int32), "s32", hip)
+    got = raw(defn.compile(sign_extended_byte_as_float, a, fuse="compiled")(a))
+    assert got.view(np.uint32).tolist() == [0x7FC00000, 0xBF800000, 0x7FC00000, 0xBF800000, 0xBF800000, 0x7FC00000, 0xBF800000, 0x7FC00000]
 
 
 @pytest.mark.parametrize("name", sorted(INT_CASES))

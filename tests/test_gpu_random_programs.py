@@ -151,3 +151,124 @@ def test_random_program_replays_from_a_captured_graph(case, hip):
         if captured is not None:
             captured.destroy()
         set_mode("interpreted")
+
+
+# ---- programs over 32-bit integers (what Nx.Random's bits-to-floats chains are made of) -------------------------
+INT_BINARY = ["add", "subtract", "multiply", "bitwise_and", "bitwise_or", "bitwise_xor", "min", "max"]
+INT_NUMBERS = [0, 1, 3, 9, 31, 255, 0x3F800000, 0x7FFFFFFF, 0x9E3779B9, -1, -7]
+
+
+def make_integer_program(rng, types):
+    """Steps over words: integer arithmetic (wrapping), shifts by constants, relabelling of bits between u32 / s32 / f32,
+    conversions to floats and float work after them.  `types` is the list of the inputs' types, extended as steps are added
+    (a step only picks operands of a type it is defined for, so every program type-checks)."""
+    steps, types = [], list(types)
+    n_inputs = len(types)
+
+    def pick(wanted):
+        at = [i for i, t in enumerate(types) if t in wanted]
+        return at[int(rng.integers(0, len(at)))] if at else None
+
+    for _ in range(int(rng.integers(3, 12))):
+        kind = rng.choice(["int2", "number", "shift", "unary", "bitcast", "as_type", "float", "select"],
+                          p=[0.22, 0.18, 0.14, 0.08, 0.14, 0.1, 0.1, 0.04])
+        a = pick(("u32", "s32"))
+        if kind == "int2" and a is not None:
+            b = pick((types[a],))
+            steps.append(("binary", INT_BINARY[int(rng.integers(0, len(INT_BINARY)))], a, b))
+            types.append(types[a])
+        elif kind == "number" and a is not None:
+            number = INT_NUMBERS[int(rng.integers(0, len(INT_NUMBERS)))]
+            if types[a] == "u32" and number < 0:
+                number = -number
+            if types[a] == "s32" and number > 0x7FFFFFFF:
+                number = 12345
+            steps.append(("number", INT_BINARY[int(rng.integers(0, len(INT_BINARY)))], a, number, bool(rng.integers(0, 2))))
+            types.append(types[a])
+        elif kind == "shift" and a is not None:
+            steps.append(("number", ["left_shift", "right_shift"][int(rng.integers(0, 2))], a, int(rng.integers(0, 32)), False))
+            types.append(types[a])
+        elif kind == "unary" and a is not None:
+            steps.append(("unary", ["negate", "bitwise_not"][int(rng.integers(0, 2))], a))
+            types.append(types[a])
+        elif kind == "bitcast":
+            a = int(rng.integers(0, len(types)))
+            if types[a] not in ("u32", "s32", "f32"):
+                continue
+            to = [t for t in ("u32", "s32", "f32") if t != types[a]][int(rng.integers(0, 2))]
+            steps.append(("bitcast", to, a))
+            types.append(to)
+        elif kind == "as_type":
+            a = int(rng.integers(0, len(types)))
+            to = ["f32", "bf16", "f16"][int(rng.integers(0, 3))]
+            steps.append(("as_type", to, a))
+            types.append(to)
+        elif kind == "float":
+            a = pick(("f32", "bf16", "f16"))
+            if a is None:
+                continue
+            if rng.random() < 0.5:
+                steps.append(("number", ["subtract", "multiply", "add"][int(rng.integers(0, 3))], a, [1.0, 0.5, 2.0][int(rng.integers(0, 3))], False))
+            else:
+                steps.append(("unary", ["abs", "sqrt", "negate", "floor"][int(rng.integers(0, 4))], a))
+            types.append(types[a])
+        elif kind == "select" and a is not None:
+            f = pick(("f32",))
+            if f is None:
+                continue
+            steps.append(("select_float", a, f))
+            types.append("f32")
+
+    def fn(*xs):
+        vals = list(xs)
+        for st in steps:
+            if st[0] == "unary":
+                v = getattr(Nx, st[1])(vals[st[2]])
+            elif st[0] == "binary":
+                v = getattr(Nx, st[1])(vals[st[2]], vals[st[3]])
+            elif st[0] == "number":
+                v = getattr(Nx, st[1])(st[3], vals[st[2]]) if st[4] else getattr(Nx, st[1])(vals[st[2]], st[3])
+            elif st[0] == "bitcast":
+                v = Nx.bitcast(vals[st[2]], st[1])
+            elif st[0] == "as_type":
+                v = Nx.as_type(vals[st[2]], st[1])
+            else:  # a float chosen by a comparison of floats made from the integers
+                as_float = Nx.as_type(vals[st[1]], "f32")
+                v = Nx.select(Nx.less(as_float, vals[st[2]]), as_float, vals[st[2]])
+            vals.append(v)
+        return vals[-1], vals[n_inputs + (len(vals) - n_inputs) // 2]
+
+    return steps, fn
+
+
+@pytest.mark.parametrize("case", range(80))
+def test_random_integer_program_has_the_same_bits_however_it_is_grouped(case, hip):
+    from nx_amd.backend import fused_mode as set_mode
+    rng = np.random.default_rng(seed_of("integer-program", case + OFFSET))
+    full = LEAD[int(rng.integers(0, len(LEAD)))] + (int(rng.choice(LAST)),)
+    types, args = [], []
+    for i in range(int(rng.integers(1, 4))):
+        ty = ["u32", "s32", "u32", "f32", "u8", "s16"][int(rng.integers(0, 6))] if i else ["u32", "s32"][int(rng.integers(0, 2))]
+        shape = full if i == 0 else broadcastable(rng, full)
+        if ty == "f32":
+            args.append(operand(rng, ty, shape, hip))
+        else:
+            bits = rng.integers(0, 1 << 32, size=shape, dtype=np.uint64).astype(np.uint32)
+            if rng.random() < 0.3:
+                bits >>= np.uint32(rng.integers(8, 30))  # small numbers: conversions to narrow floats stay finite
+            args.append(from_numpy(bits.astype({"u32": np.uint32, "s32": np.int32, "u8": np.uint8, "s16": np.int16}[ty]), ty, hip))
+        types.append(ty)
+    steps, fn = make_integer_program(rng, types)
+    what = f"case {case + OFFSET}: {[(tuple(a.shape), a.type) for a in args]} {steps}"
+    want = defn.compile(fn, *args)(*args)
+    try:
+        for mode in ("interpreted", "compiled"):
+            set_mode(mode)
+            got = defn.compile(fn, *args, fuse=True)(*args)
+            for g, w in zip(got, want):
+                assert_bits_equal(g, w, f"fused, {mode}; {what}")
+        got = defn.compile(fn, *args, fuse="compiled")(*args)
+        for g, w in zip(got, want):
+            assert_bits_equal(g, w, f"planned; {what}")
+    finally:
+        set_mode("interpreted")
