@@ -241,23 +241,30 @@ def make_integer_program(rng, types):
     return steps, fn
 
 
+def integer_operand(rng, ty, shape, hip):
+    if ty == "f32":
+        return operand(rng, ty, shape, hip)
+    bits = rng.integers(0, 1 << 32, size=shape, dtype=np.uint64).astype(np.uint32)
+    if rng.random() < 0.3:
+        bits >>= np.uint32(rng.integers(8, 30))  # small numbers: conversions to narrow floats stay finite
+    return from_numpy(bits.astype({"u32": np.uint32, "s32": np.int32, "u8": np.uint8, "s16": np.int16}[ty]), ty, hip)
+
+
+def integer_operand_types(rng):
+    full = LEAD[int(rng.integers(0, len(LEAD)))] + (int(rng.choice(LAST)),)
+    types, shapes = [], []
+    for i in range(int(rng.integers(1, 4))):
+        types.append(["u32", "s32", "u32", "f32", "u8", "s16"][int(rng.integers(0, 6))] if i else ["u32", "s32"][int(rng.integers(0, 2))])
+        shapes.append(full if i == 0 else broadcastable(rng, full))
+    return types, shapes
+
+
 @pytest.mark.parametrize("case", range(80))
 def test_random_integer_program_has_the_same_bits_however_it_is_grouped(case, hip):
     from nx_amd.backend import fused_mode as set_mode
     rng = np.random.default_rng(seed_of("integer-program", case + OFFSET))
-    full = LEAD[int(rng.integers(0, len(LEAD)))] + (int(rng.choice(LAST)),)
-    types, args = [], []
-    for i in range(int(rng.integers(1, 4))):
-        ty = ["u32", "s32", "u32", "f32", "u8", "s16"][int(rng.integers(0, 6))] if i else ["u32", "s32"][int(rng.integers(0, 2))]
-        shape = full if i == 0 else broadcastable(rng, full)
-        if ty == "f32":
-            args.append(operand(rng, ty, shape, hip))
-        else:
-            bits = rng.integers(0, 1 << 32, size=shape, dtype=np.uint64).astype(np.uint32)
-            if rng.random() < 0.3:
-                bits >>= np.uint32(rng.integers(8, 30))  # small numbers: conversions to narrow floats stay finite
-            args.append(from_numpy(bits.astype({"u32": np.uint32, "s32": np.int32, "u8": np.uint8, "s16": np.int16}[ty]), ty, hip))
-        types.append(ty)
+    types, shapes = integer_operand_types(rng)
+    args = [integer_operand(rng, ty, sh, hip) for ty, sh in zip(types, shapes)]
     steps, fn = make_integer_program(rng, types)
     what = f"case {case + OFFSET}: {[(tuple(a.shape), a.type) for a in args]} {steps}"
     want = defn.compile(fn, *args)(*args)
@@ -271,4 +278,34 @@ def test_random_integer_program_has_the_same_bits_however_it_is_grouped(case, hi
         for g, w in zip(got, want):
             assert_bits_equal(g, w, f"planned; {what}")
     finally:
+        set_mode("interpreted")
+
+
+@pytest.mark.parametrize("case", range(30))
+def test_random_integer_program_replays_from_a_captured_graph(case, hip):
+    """Planned for compilation, recorded, and replayed with the captured tensors, new ones, and the first again."""
+    from nx_amd.backend import fused_mode as set_mode, sync
+    rng = np.random.default_rng(seed_of("integer-program-graph", case + OFFSET))
+    types, shapes = integer_operand_types(rng)
+    args = [integer_operand(rng, ty, sh, hip) for ty, sh in zip(types, shapes)]
+    fresh = [integer_operand(rng, ty, sh, hip) for ty, sh in zip(types, shapes)]
+    steps, fn = make_integer_program(rng, types)
+    what = f"case {case + OFFSET}: {[(tuple(a.shape), a.type) for a in args]} {steps}"
+    plain = defn.compile(fn, *args)
+    want_args, want_fresh = plain(*args), plain(*fresh)
+    set_mode("compiled")
+    captured = None
+    try:
+        compiled = defn.compile(fn, *args, fuse="compiled")
+        compiled(*args)  # (compiled before the capture begins)
+        captured = compiled.capture(*args)
+        for given, want in ((args, want_args), (fresh, want_fresh), (args, want_args)):
+            got = captured(*given)
+            for g, w in zip(got, want):
+                assert_bits_equal(g, w, f"replay; {what}")
+            plain(*fresh)
+            sync()
+    finally:
+        if captured is not None:
+            captured.destroy()
         set_mode("interpreted")

@@ -265,3 +265,43 @@ def test_dot_on_large_random_shapes_against_f64_blas(case, hip):
     assert res.shape == expect.shape, what
     same = res.view(np.uint8) == expect.view(np.uint8)
     assert same.all(), f"{what}: {int((~same).sum())} bytes differ"
+
+
+@pytest.mark.parametrize("case", range(60))
+def test_scaled_int8_dot_on_random_shapes(case, hip):
+    """The quantised linear layer (dot to s32, as_type f32, multiply by scales) as one callback on the accumulators against
+    the three callbacks one after the other: rows from one to several tiles, ragged columns, K in steps of 128, weights
+    K-inner or K-outer, batches, every kind of scale; an integer check of the accumulators themselves on top
+    (small operands: the s32 sums are exact in numpy's int64)."""
+    from nx_amd import defn
+    from support import from_numpy, raw
+    rng = np.random.default_rng(seed_of("scaled-dot", case + OFFSET))
+    m = int(rng.choice([1, 2, 7, 16, 33, 64, 65, 128, 200, 300, 520]))
+    n = int(rng.choice([1, 8, 40, 64, 100, 256, 260, 512, 1000, 1100]))
+    k = 128 * int(rng.choice([1, 2, 3, 5, 8, 16, 33]))
+    batch = int(rng.choice([0, 0, 0, 2, 3]))
+    k_outer = bool(rng.integers(0, 2))
+    lead = (batch,) if batch else ()
+    x = from_numpy(rng.integers(-127, 128, size=lead + (m, k), dtype=np.int8), "s8", hip)
+    w = from_numpy(rng.integers(-127, 128, size=lead + ((k, n) if k_outer else (n, k)), dtype=np.int8), "s8", hip)
+    kind = ["per_column", "per_row", "one", "constant"][int(rng.integers(0, 4))]
+    r = len(lead)
+    bx = [0] if batch else []
+
+    def product(xq, wq):
+        return Nx.dot(xq, [r + 1], bx, wq, [r] if k_outer else [r + 1], bx, out_type="s32")
+    what = f"case {case + OFFSET}: {lead} {m}x{n}x{k} weights {'K-outer' if k_outer else 'K-inner'} scales {kind}"
+    if kind == "constant":
+        fun, args = (lambda xq, wq: Nx.multiply(Nx.as_type(product(xq, wq), "f32"), 0.0078125)), (x, w)
+    else:
+        shape = {"per_column": (n,), "per_row": (m, 1), "one": (1, 1)}[kind]
+        sc = from_numpy(rng.uniform(1e-3, 1e-2, size=shape).astype(np.float32), "f32", hip)
+        fun, args = (lambda xq, wq, s: Nx.multiply(Nx.as_type(product(xq, wq), "f32"), s)), (x, w, sc)
+    want = defn.compile(fun, *args)(*args)
+    planned = defn.compile(fun, *args, fuse=True)
+    assert_bits_equal(planned(*args), want, what)
+    # the accumulators, by int64 arithmetic on the host
+    xs, ws = raw(x).astype(np.int64), raw(w).astype(np.int64)
+    acc = np.matmul(xs, ws if k_outer else np.swapaxes(ws, -1, -2))
+    got = raw(defn.compile(product, x, w)(x, w))
+    assert np.array_equal(got, acc.astype(np.int32)), what
