@@ -25,12 +25,18 @@ LAST = [1, 3, 7, 8, 33, 64, 100, 256, 513, 1024, 4100]
 LEAD = [(), (1,), (5,), (64,), (3, 4), (2, 1), (300,)]
 
 
-def make_program(rng, n_inputs):
-    """A list of steps over a growing list of values; returns (steps, function)."""
+def make_program(rng, n_inputs, in_memory=False):
+    """A list of steps over a growing list of values; returns (steps, function).  `in_memory`: also nodes that are not
+    element-wise and keep the shape (a reversal, a clip, a reduction along the first axis, a transposition there and back
+    with work in between), whose operands must exist in memory: they cut the groups."""
     steps = []
     n = n_inputs
     reduced = False
     for _ in range(int(rng.integers(2, 10))):
+        if in_memory and rng.random() < 0.25:
+            steps.append((["reverse", "clip", "sum_first", "transposed_tanh"][int(rng.integers(0, 4))], int(rng.integers(0, n))))
+            n += 1
+            continue
         kind = rng.choice(["unary", "binary", "number", "reduce", "select", "as_type"], p=[0.3, 0.3, 0.15, 0.12, 0.08, 0.05])
         a, b, c = int(rng.integers(0, n)), int(rng.integers(0, n)), int(rng.integers(0, n))
         if kind == "unary":
@@ -65,8 +71,22 @@ def make_program(rng, n_inputs):
                 v = getattr(Nx, st[1])(t, axes=[len(t.shape) - 1], keep_axes=st[3]) if len(t.shape) else t
             elif st[0] == "select":
                 v = Nx.select(getattr(Nx, st[1])(vals[st[2]], vals[st[3]]), vals[st[3]], vals[st[4]])
-            else:
+            elif st[0] == "as_type":
                 v = Nx.as_type(vals[st[2]], st[1])
+            else:
+                t = vals[st[1]]
+                rank = len(t.shape)
+                if rank == 0:
+                    v = Nx.negate(t)
+                elif st[0] == "reverse":
+                    v = Nx.reverse(t, axes=[rank - 1])
+                elif st[0] == "clip":
+                    v = Nx.clip(t, -0.75, 1.5)
+                elif st[0] == "sum_first":
+                    v = Nx.subtract(t, Nx.sum(t, axes=[0], keep_axes=True))
+                else:
+                    back = list(range(rank - 1, -1, -1))
+                    v = Nx.transpose(Nx.tanh(Nx.transpose(t, axes=back)), axes=back)
             vals.append(v)
         # the last value, and an earlier one that something else may also have read
         return vals[-1], vals[n_inputs + (len(vals) - n_inputs) // 2]
@@ -101,6 +121,37 @@ def test_random_program_has_the_same_bits_however_it_is_grouped(case, hip):
     try:
         want = defn.compile(fn, *args)(*args)
     except (ValueError, TypeError) as e:  # a shape the front end refuses (a reduced value against a full one of another rank)
+        pytest.skip(f"the program does not type-check: {e}")
+    try:
+        for mode in ("interpreted", "compiled"):
+            set_mode(mode)
+            got = defn.compile(fn, *args, fuse=True)(*args)
+            for g, w in zip(got, want):
+                assert_bits_equal(g, w, f"fused, {mode}; {what}")
+        got = defn.compile(fn, *args, fuse="compiled")(*args)
+        for g, w in zip(got, want):
+            assert_bits_equal(g, w, f"planned; {what}")
+    finally:
+        set_mode("interpreted")
+
+
+@pytest.mark.parametrize("case", range(80))
+def test_random_program_with_nodes_that_cut_the_groups(case, hip):
+    """Reversals, clips, reductions along the first axis and transpositions between the element-wise nodes: what a group
+    reads from such a node, and what such a node reads from a group, has to be in memory at the right time."""
+    from nx_amd.backend import fused_mode as set_mode
+    rng = np.random.default_rng(seed_of("program-in-memory", case + OFFSET))
+    full = LEAD[int(rng.integers(0, len(LEAD)))] + (int(rng.choice(LAST)),)
+    n_inputs = int(rng.integers(1, 4))
+    args = []
+    for i in range(n_inputs):
+        ty = ["f32", "f32", "bf16", "f16"][int(rng.integers(0, 4))]
+        args.append(operand(rng, ty, full if i == 0 else broadcastable(rng, full), hip))
+    steps, fn = make_program(rng, n_inputs, in_memory=True)
+    what = f"case {case + OFFSET}: {[(tuple(a.shape), a.type) for a in args]} {steps}"
+    try:
+        want = defn.compile(fn, *args)(*args)
+    except (ValueError, TypeError) as e:
         pytest.skip(f"the program does not type-check: {e}")
     try:
         for mode in ("interpreted", "compiled"):
