@@ -54,7 +54,10 @@ __device__ __forceinline__ f16_t bits_f16(uint16_t u) {
   x.u = u;
   return x.h;
 }
+// The conversion is kept apart from the arithmetic that made `f` (the empty asm): the compiler otherwise turns a product
+// followed by this rounding into one mixed-precision fma with +0 as the addend, and (-x) * 0 = -0 comes out as +0.
 __device__ __forceinline__ uint16_t f32_to_f16_bits(float f) {
+  asm("" : "+v"(f));
   return (f != f) ? (uint16_t)0x7E00 : f16_bits((f16_t)f);
 }
 // f64 -> f32 with round-to-odd, so that a following round-to-nearest narrowing equals a single

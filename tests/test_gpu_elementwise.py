@@ -320,3 +320,25 @@ def test_broadcasts_over_separated_axes_off_the_vector_grid(ls, rs, ty, op, hip,
     f = getattr(Nx, op)
     assert_bits_equal(f(ha, hb), f(oa, ob), f"{op} {ty} {ls} {rs}")
     assert_bits_equal(f(hb, ha), f(ob, oa), f"{op} {ty} {rs} {ls}")
+
+
+@pytest.mark.parametrize("ty", ["f16", "bf16", "f32", "f64"])
+@pytest.mark.parametrize("op", ["multiply", "divide", "add", "subtract"])
+@pytest.mark.parametrize("form", ["same_shape", "one_per_row", "one_row", "a_number"])
+def test_signed_zeros_through_every_operand_form(ty, op, form, hip, oracle):
+    """The sign of a zero result: (-x) * 0 = -0, 0 / (-x) = -0, -0 + -0 = -0, x - x = +0, in the kernels for operands of
+    one shape and in those that spread one operand along or across the rows (a product followed by the rounding to f16
+    once came out of the compiler as one instruction that added +0 to it)."""
+    rng = np.random.default_rng(seed_of("signed zeros", ty, op, form))
+    dtype = np.float32 if ty == "bf16" else T.numpy_dtype(T.normalize(ty))
+    shape = {"same_shape": (64, 256), "one_per_row": (64, 1), "one_row": (256,), "a_number": ()}[form]
+    a = rng.choice(np.array([0.0, -0.0, 1.25, -1.25, 3.0, -0.5], dtype), size=(64, 256))
+    b = rng.choice(np.array([0.0, -0.0, 2.0, -2.0], dtype), size=shape)
+    if ty == "bf16":
+        a, b = [(np.asarray(v, np.float32).view(np.uint32) >> 16).astype(np.uint16) for v in (a, b)]
+    ha, oa = both(a, ty, hip, oracle)
+    hb, ob = both(b, ty, hip, oracle)
+    for flip in (False, True):  # (a float divided by zero is an infinity or a NaN in the reference, not an error)
+        got = getattr(Nx, op)(hb, ha) if flip else getattr(Nx, op)(ha, hb)
+        want = getattr(Nx, op)(ob, oa) if flip else getattr(Nx, op)(oa, ob)
+        assert_bits_equal(got, want, f"{op} {ty} {form} flipped={flip}")

@@ -270,6 +270,9 @@ def make_integer_program(rng, types):
             steps.append(("select_float", a, f))
             types.append("f32")
 
+    if not steps:  # every draw fell on a step its operands' types do not allow
+        steps.append(("unary", "bitwise_not", 0))
+
     def fn(*xs):
         vals = list(xs)
         for st in steps:
