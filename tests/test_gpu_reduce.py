@@ -261,3 +261,20 @@ def test_long_rows_that_are_not_whole_vectors(shape, ty, op, hip, oracle):
         assert np.allclose(values(got), values(want), rtol=eps + cols * 2.0 ** -50, atol=cols * 2.0 ** -24 * np.abs(values(ox)).sum(axis=1))
     else:
         assert_bits_equal(getattr(Nx, op)(hx, axes=[1]), getattr(Nx, op)(ox, axes=[1]), f"{op} {ty} {shape}")
+
+
+@pytest.mark.parametrize("ty", ["f16", "bf16", "f32", "f64"])
+@pytest.mark.parametrize("op", ["product", "sum", "reduce_max", "reduce_min"])
+@pytest.mark.parametrize("shape,axes", [((40, 64), [1]), ((64, 40), [0]), ((6, 5000), [1]), ((3000, 8), [0]), ((7, 9, 33), [0, 2])])
+def test_signed_zeros_in_reductions(ty, op, shape, axes, hip, oracle):
+    """Zeros of either sign among ones and minus ones: the product's zero carries the sign of the factors, a sum of
+    negative zeros is a negative zero (the reference folds from the first element; exact here, in any order, up to that sign)."""
+    rng = np.random.default_rng(seed_of("zeros in reductions", ty, op, shape))
+    dtype = np.float32 if ty == "bf16" else T.numpy_dtype(T.normalize(ty))
+    x = rng.choice(np.array([1.0, -1.0, 0.0, -0.0], dtype), size=shape, p=[0.49, 0.49, 0.01, 0.01])
+    if op == "sum":  # rows of zeros only, most of them all negative
+        x = np.where(rng.random(shape) < 0.002, 0.0, -0.0).astype(dtype)
+    if ty == "bf16":
+        x = (np.asarray(x, np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    hx, ox = both(x, ty, hip, oracle)
+    assert_bits_equal(getattr(Nx, op)(hx, axes=axes), getattr(Nx, op)(ox, axes=axes), f"{op} {ty} {shape} {axes}")
