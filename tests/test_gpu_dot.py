@@ -636,3 +636,21 @@ def test_f64_contraction_on_the_matrix_cores(M, N, K, layout, hip, oracle):
     # an f32 result from f64 operands: one rounding of the f64 sum
     res32 = hip.to_numpy(Nx.dot(from_numpy(ai, "f64", hip), c1, from_numpy(bi, "f64", hip), c2, out_type="f32"))
     assert np.array_equal(res32, exact.astype(np.float32))
+
+
+@pytest.mark.parametrize("ty", ["f16", "bf16", "f32", "f64"])
+@pytest.mark.parametrize("m,k,n", [(1, 1, 1), (5, 1, 7), (64, 1, 64), (3, 2, 4), (16, 16, 16), (33, 64, 40), (128, 128, 128), (1, 256, 1)])
+def test_zero_products_leave_a_positive_zero(ty, m, k, n, hip, oracle):
+    """The reference adds every product to a sum that starts at 0, so products that are all -0 (a negative factor
+    times +0) give +0, with one term (K = 1) as with many; outputs whose terms cancel are +0 as well."""
+    rng = np.random.default_rng(seed_of("zero products", ty, m, k, n))
+    dtype = np.float32 if ty == "bf16" else T.numpy_dtype(T.normalize(ty))
+    a = rng.choice(np.array([-1.0, -2.0, 1.0, 0.0, -0.0]), size=(m, k)).astype(dtype)
+    b = rng.choice(np.array([0.0, -0.0, 0.0, 1.0, -1.0]), size=(k, n), p=[0.4, 0.3, 0.1, 0.1, 0.1]).astype(dtype)
+    if ty == "bf16":
+        a, b = [(np.asarray(v, np.float32).view(np.uint32) >> 16).astype(np.uint16) for v in (a, b)]
+    ha, oa = both(a, ty, hip, oracle)
+    hb, ob = both(b, ty, hip, oracle)
+    assert_bits_equal(Nx.dot(ha, hb), Nx.dot(oa, ob), f"dot {ty} {m}x{k}x{n}")
+    assert_bits_equal(Nx.dot(ha, [0], hb, [1]) if m == n else Nx.dot(hb, [0], ha, [1]),
+                      Nx.dot(oa, [0], ob, [1]) if m == n else Nx.dot(ob, [0], oa, [1]), f"dot {ty} other axes")
