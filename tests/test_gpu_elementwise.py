@@ -8,7 +8,7 @@ import pytest
 
 from nx_amd import nx as Nx
 from nx_amd import types as T
-from support import assert_all_close, assert_bits_equal, from_numpy, seed_of
+from support import _uint, assert_all_close, assert_bits_equal, from_numpy, raw, seed_of, values
 
 pytestmark = pytest.mark.gpu
 
@@ -342,3 +342,35 @@ def test_signed_zeros_through_every_operand_form(ty, op, form, hip, oracle):
         got = getattr(Nx, op)(hb, ha) if flip else getattr(Nx, op)(ha, hb)
         want = getattr(Nx, op)(ob, oa) if flip else getattr(Nx, op)(oa, ob)
         assert_bits_equal(got, want, f"{op} {ty} {form} flipped={flip}")
+
+
+MATH = ["exp", "expm1", "log", "log1p", "sigmoid", "cos", "sin", "tan", "cosh", "sinh", "tanh", "acos", "asin", "atan", "acosh",
+        "asinh", "atanh", "sqrt", "rsqrt", "cbrt", "erf", "erfc", "erf_inv", "abs", "negate", "floor", "ceil", "round", "sign"]
+
+
+@pytest.mark.parametrize("ty", ["f16", "bf16", "f32", "f64"])
+@pytest.mark.parametrize("op", MATH)
+def test_unary_results_that_are_zero_or_not_finite_have_the_reference_bits(op, ty, hip, oracle):
+    """Zeros of either sign, the smallest numbers, ones, the ends of the domains, infinities and NaN: wherever the
+    reference's result is a zero, an infinity or NaN the device's is the same bits (sin(-0) = -0, tanh of a tiny negative
+    number that rounds to zero keeps its sign, log(0) = -inf, ...); elsewhere the tolerance of the other tests applies."""
+    tiny = {"f16": 6e-8, "bf16": 1e-38, "f32": 1e-45, "f64": 5e-324}[ty]
+    from oracle.binary_backend import ReferenceRaises
+    large = 8.0 if ty == "f16" else 30.0  # (a finite result beyond f16's range raises in the reference)
+    v = np.array([0.0, -0.0, tiny, -tiny, 1.0, -1.0, 0.5, -0.5, 2.0, -2.0, np.inf, -np.inf, np.nan, 1e-4, -1e-4, large, -large])
+    x = encode(v, ty)
+    hx, ox = both(x, ty, hip, oracle)
+    try:
+        want = getattr(Nx, op)(ox)
+    except ReferenceRaises as e:
+        pytest.skip(f"the reference raises: {e}")
+    got = getattr(Nx, op)(hx)
+    assert got.type == want.type and got.shape == want.shape
+    g, w = raw(got), raw(want)
+    gf, wf = values(got), values(want)
+    fixed = (wf == 0) | ~np.isfinite(wf)
+    gb, wb = g.view(_uint(g.dtype)), w.view(_uint(w.dtype))
+    assert np.array_equal(gb[fixed], wb[fixed]), f"{op} {ty}: inputs {v[fixed][gb[fixed] != wb[fixed]]} got {gf[fixed][gb[fixed] != wb[fixed]]} want {wf[fixed][gb[fixed] != wb[fixed]]}"
+    rest = ~fixed
+    tol = {"f16": 2e-3, "bf16": 1.6e-2, "f32": 2e-6, "f64": 1e-12}[ty]
+    assert np.all(np.abs(gf[rest] - wf[rest]) <= tol * np.abs(wf[rest])), f"{op} {ty}: {gf[rest]} vs {wf[rest]}"
