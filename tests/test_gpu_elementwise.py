@@ -374,3 +374,38 @@ def test_unary_results_that_are_zero_or_not_finite_have_the_reference_bits(op, t
     rest = ~fixed
     tol = {"f16": 2e-3, "bf16": 1.6e-2, "f32": 2e-6, "f64": 1e-12}[ty]
     assert np.all(np.abs(gf[rest] - wf[rest]) <= tol * np.abs(wf[rest])), f"{op} {ty}: {gf[rest]} vs {wf[rest]}"
+
+
+@pytest.mark.parametrize("ty", ["f16", "bf16", "f32", "f64"])
+@pytest.mark.parametrize("op", ["add", "subtract", "multiply", "divide", "pow", "atan2", "min", "max", "remainder"])
+def test_binary_results_that_are_zero_or_not_finite_have_the_reference_bits(op, ty, hip, oracle):
+    """Every pair from zeros of either sign, the smallest numbers, small integers (odd and even), a half, infinities and
+    NaN (the special cases of pow, atan2 and division among them), as operands of one shape and with a number on either
+    side; results that are a zero, an infinity or NaN must be the reference's bits."""
+    from oracle.binary_backend import ReferenceRaises
+    tiny = {"f16": 6e-8, "bf16": 1e-38, "f32": 1e-45, "f64": 5e-324}[ty]
+    s = np.array([0.0, -0.0, tiny, -tiny, 1.0, -1.0, 2.0, -2.0, 3.0, -3.0, 0.5, -0.5, np.inf, -np.inf, np.nan])
+    if op == "remainder":  # :math.fmod raises for a zero divisor and for operands that are not finite
+        s = s[np.isfinite(s) & (s != 0)]
+    a, b = [g.ravel() for g in np.meshgrid(s, s, indexing="ij")]
+    if op in ("divide", "pow") and ty != "f64":  # a finite result beyond the type's range raises in the reference: not asked
+        with np.errstate(all="ignore"):
+            exact = np.divide(a, b) if op == "divide" else np.power(a, b)
+        fits = ~(np.isfinite(exact) & (np.abs(exact) > (65504.0 if ty == "f16" else 3.4e38)))
+        a, b = a[fits], b[fits]
+    ha, oa = both(encode(a, ty), ty, hip, oracle)
+    hb, ob = both(encode(b, ty), ty, hip, oracle)
+    try:
+        want = getattr(Nx, op)(oa, ob)
+    except ReferenceRaises as e:
+        pytest.skip(f"the reference raises: {e}")
+    got = getattr(Nx, op)(ha, hb)
+    g, w = raw(got), raw(want)
+    gf, wf = values(got), values(want)
+    fixed = (wf == 0) | ~np.isfinite(wf)
+    gb, wb = g.view(_uint(g.dtype)), w.view(_uint(w.dtype))
+    bad = fixed & (gb != wb)
+    assert not bad.any(), f"{op} {ty}: a {a[bad]} b {b[bad]} got {gf[bad]} want {wf[bad]}"
+    rest = ~fixed
+    tol = {"f16": 2e-3, "bf16": 1.6e-2, "f32": 2e-6, "f64": 1e-12}[ty]
+    assert np.all(np.abs(gf[rest] - wf[rest]) <= tol * np.abs(wf[rest])), f"{op} {ty}"
