@@ -941,3 +941,32 @@ def test_ragged_rows_still_fall_back(hip):
         return Nx.exp(Nx.add(a, b))
     planned = defn.compile(fun, x, bias, fuse="compiled")
     assert_bits_equal(planned(x, bias), defn.compile(fun, x, bias)(x, bias), "row operand, ragged rows")
+
+
+@pytest.mark.parametrize("ty", ["f16", "bf16", "f32"])
+def test_fused_groups_on_special_values(ty, hip):
+    """Every unary and binary element-wise node a group can hold, on zeros of either sign, the smallest numbers, domain
+    ends, infinities and NaN: the group's bits are those of the nodes run one by one, interpreted and compiled."""
+    from nx_amd.backend import fused_mode as set_mode
+    from test_gpu_elementwise import MATH, encode
+    tiny = {"f16": 6e-8, "bf16": 1e-38, "f32": 1e-45}[ty]
+    large = 8.0 if ty == "f16" else 30.0
+    v = np.array([0.0, -0.0, tiny, -tiny, 1.0, -1.0, 0.5, -0.5, 2.0, -2.0, np.inf, -np.inf, np.nan, 1e-4, -1e-4, large, -large,
+                  3.0, -3.0, 0.25, -0.25, 1.5, -1.5, 7.0])
+    x = from_numpy(encode(v, ty), ty, hip)
+    a, b = [g.ravel() for g in np.meshgrid(v[:16], v[:16], indexing="ij")]
+    ha, hb = from_numpy(encode(a, ty), ty, hip), from_numpy(encode(b, ty), ty, hip)
+    programs = [(f"{op} then negate", (lambda t, op=op: Nx.negate(getattr(Nx, op)(t))), (x,)) for op in MATH]
+    programs += [(f"{op} plus its operand", (lambda t, op=op: Nx.add(getattr(Nx, op)(t), t)), (x,)) for op in MATH]
+    programs += [(f"{op} then negate", (lambda p, q, op=op: Nx.negate(getattr(Nx, op)(p, q))), (ha, hb))
+                 for op in ("add", "subtract", "multiply", "divide", "pow", "atan2", "min", "max")]
+    programs += [(f"{op} times its operand", (lambda p, q, op=op: Nx.multiply(getattr(Nx, op)(p, q), q)), (ha, hb))
+                 for op in ("add", "subtract", "multiply", "divide", "min", "max")]
+    try:
+        for name, fun, args in programs:
+            want = defn.compile(fun, *args)(*args)
+            for mode in ("interpreted", "compiled"):
+                set_mode(mode)
+                assert_bits_equal(defn.compile(fun, *args, fuse=True)(*args), want, f"{name}, {ty}, {mode}")
+    finally:
+        set_mode("interpreted")
