@@ -278,3 +278,31 @@ def test_signed_zeros_in_reductions(ty, op, shape, axes, hip, oracle):
         x = (np.asarray(x, np.float32).view(np.uint32) >> 16).astype(np.uint16)
     hx, ox = both(x, ty, hip, oracle)
     assert_bits_equal(getattr(Nx, op)(hx, axes=axes), getattr(Nx, op)(ox, axes=axes), f"{op} {ty} {shape} {axes}")
+
+
+@pytest.mark.parametrize("ty", ["f16", "bf16", "f32", "f64"])
+@pytest.mark.parametrize("op", ["sum", "product", "reduce_max", "reduce_min"])
+@pytest.mark.parametrize("shape,axes", [((48, 64), [1]), ((64, 48), [0]), ((5, 6000), [1]), ((2500, 8), [0])])
+def test_infinities_and_nan_in_reductions(ty, op, shape, axes, hip, oracle):
+    """Rows with an infinity, with infinities of both signs (their sum is NaN), with an infinity and a zero (their product is
+    NaN), with a NaN, and plain ones: the same bits as the reference in every float type."""
+    rng = np.random.default_rng(seed_of("not finite in reductions", ty, op, shape))
+    dtype = np.float32 if ty == "bf16" else T.numpy_dtype(T.normalize(ty))
+    x = rng.choice(np.array([1.0, -1.0] if op == "product" else [1.0, -1.0, 0.5, 2.0]), size=shape)  # (exact in any order)
+    lines = np.moveaxis(x, axes[0], -1)  # a view: one line per output
+    for i, line in enumerate(lines):
+        kind = i % 5
+        at = rng.choice(line.size, size=3, replace=False)
+        if kind == 0:
+            line[at[0]] = np.inf
+        elif kind == 1:
+            line[at[0]], line[at[1]] = np.inf, -np.inf
+        elif kind == 2:
+            line[at[0]], line[at[1]] = -np.inf, 0.0
+        elif kind == 3:
+            line[at[0]], line[at[1]] = np.nan, np.inf
+    x = x.astype(dtype)
+    if ty == "bf16":
+        x = (x.view(np.uint32) >> 16).astype(np.uint16)
+    hx, ox = both(x, ty, hip, oracle)
+    assert_bits_equal(getattr(Nx, op)(hx, axes=axes), getattr(Nx, op)(ox, axes=axes), f"{op} {ty} {shape} {axes}")
