@@ -188,7 +188,10 @@ int hipnx_fill(hipnx_ctx *ctx, hipnx_buf *dst, int elem_bytes, const void *elem,
  * replaces: the 24 binary callbacks (nx/lib/nx/backend.ex:115-123; oracle
  * nx/lib/nx/binary_backend.ex:649-823; torchx/c_src/torchx.cpp:737-769).
  * out[i] = op(l[bcast i], r[bcast i]) over the row-major index space `out_dims[rank]`;
- * strides are in elements, 0 marks a broadcast axis (numpy-style, nx/lib/nx/shape.ex:316-376). */
+ * strides are in elements, 0 marks a broadcast axis (numpy-style, nx/lib/nx/shape.ex:316-376).
+ * Known difference from the reference: with one operand u64 and the other a signed integer the pair is computed as s64,
+ * so u64 values of 2^63 and more read as negative in the comparisons, min, max, quotient, remainder and right_shift
+ * (add, subtract, multiply, bitwise and left_shift wrap to the same bits as the reference's unbounded integers). */
 int hipnx_binary(hipnx_ctx *ctx, int op, int l_dt, int r_dt, int out_dt, int rank,
                  const int64_t *out_dims, const int64_t *l_strides, const int64_t *r_strides,
                  const hipnx_buf *l, const hipnx_buf *r, hipnx_buf *out);

@@ -409,3 +409,36 @@ def test_binary_results_that_are_zero_or_not_finite_have_the_reference_bits(op, 
     rest = ~fixed
     tol = {"f16": 2e-3, "bf16": 1.6e-2, "f32": 2e-6, "f64": 1e-12}[ty]
     assert np.all(np.abs(gf[rest] - wf[rest]) <= tol * np.abs(wf[rest])), f"{op} {ty}"
+
+
+@pytest.mark.parametrize("lt", ["s8", "u8", "s16", "u16", "s32", "u32", "s64", "u64"])
+@pytest.mark.parametrize("rt", ["s8", "u8", "s32", "u32", "s64", "u64"])
+@pytest.mark.parametrize("op", ["add", "subtract", "multiply", "quotient", "remainder", "min", "max", "less", "equal",
+                                "bitwise_and", "bitwise_or", "bitwise_xor", "left_shift", "right_shift"])
+def test_integer_extremes_in_every_pair_of_types(op, lt, rt, hip, oracle):
+    """Every pair from the ends of each type, the values next to them, zero, one and minus one: the most negative number
+    divided by -1, products and sums that wrap, an unsigned operand beyond the signed range against a negative one, shift
+    counts up to the width and beyond (negative counts and zero divisors raise in the reference: left out)."""
+    order_matters = ("quotient", "remainder", "min", "max", "less", "equal", "right_shift")
+    if op in order_matters and "u64" in (lt, rt) and "s" in (lt[0], rt[0]):
+        # known difference: a u64 operand against a signed one is computed in the s64 class, where values of 2^63 and more
+        # read as negative; the reference keeps them positive (unbounded integers).  Sums, products and bitwise results
+        # wrap to the same bits either way and are checked below.
+        pytest.skip("u64 values of 2^63 and more against a signed operand: compared, divided and shifted as negative s64")
+
+    def ends(ty):
+        info = np.iinfo(T.numpy_dtype(T.normalize(ty)))
+        vals = {info.min, info.min + 1, info.max, info.max - 1, 0, 1, 2, 7}
+        if info.min < 0:
+            vals |= {-1, -2, -7}
+        return np.array(sorted(vals), dtype=T.numpy_dtype(T.normalize(ty)))
+    a, b = ends(lt), ends(rt)
+    if op in ("quotient", "remainder"):
+        b = b[b != 0]
+    if op in ("left_shift", "right_shift"):
+        b = np.array([0, 1, 7, 8, 31, 32, 63, 64, 65], dtype=np.int64).astype(b.dtype)
+        b = np.unique(b[b >= 0])
+    a, b = [g.ravel() for g in np.meshgrid(a, b, indexing="ij")]
+    ha, oa = both(a, lt, hip, oracle)
+    hb, ob = both(b, rt, hip, oracle)
+    assert_bits_equal(getattr(Nx, op)(ha, hb), getattr(Nx, op)(oa, ob), f"{op} {lt} {rt}")
